@@ -1,0 +1,170 @@
+"""Pins the oracle's block formats against what the reference's own tests hold
+(engine/quant.rs tests, cited per case).  CPU only."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import Q4_K, Q6_K, Q8_0
+
+# quant.rs:1389-1417 GOLDEN (the three types on the path)
+GOLDEN = [
+    (Q8_0, "q8_0", 256, 0xC5D58782F54E52E5),
+    (Q4_K, "q4_k", 512, 0x9A7268A432A5C5FA),
+    (Q6_K, "q6_k", 512, 0x61001D333CB0CFD1),
+]
+
+
+@pytest.mark.parametrize("ggml_type,name,count,expected", GOLDEN)
+def test_dequantizing_every_type_is_unchanged(ggml_type, name, count, expected):
+    """quant.rs:1451-1463: bit checksum of dequantize(fixture_bytes).  The Q4_K and Q6_K fixtures
+    contain NaN scale fields, so this also pins NaN payload propagation."""
+    n = oracle.tensor_byte_size(ggml_type, count)
+    data = oracle.fixture_bytes(n)
+    values = oracle.dequantize(ggml_type, data, count)
+    assert values.size == count
+    assert oracle.bit_checksum(values) == expected, name
+
+
+def test_fixture_bytes_is_xorshift64():
+    """Independent restatement of quant.rs:1427-1437 in Python integers."""
+    state = 0x2545F4914F6CDD1D
+    want = []
+    for _ in range(64):
+        state ^= (state << 13) & 0xFFFFFFFFFFFFFFFF
+        state ^= state >> 7
+        state ^= (state << 17) & 0xFFFFFFFFFFFFFFFF
+        want.append((state >> 33) & 0xFF)
+    assert oracle.fixture_bytes(64).tolist() == want
+
+
+def test_tensor_byte_size_and_block_layout():
+    """quant.rs:132-169, 344-357."""
+    assert oracle.tensor_byte_size(Q8_0, 256) == 8 * 34
+    assert oracle.tensor_byte_size(Q4_K, 512) == 2 * 144
+    assert oracle.tensor_byte_size(Q6_K, 512) == 2 * 210
+    assert oracle.tensor_byte_size(Q4_K, 100) == -2  # not a whole number of blocks
+    assert oracle.tensor_byte_size(99, 256) == -1  # unknown type
+
+
+def test_f16_conversion_matches_ieee_for_all_65536_inputs():
+    """quant.rs:1671-1690: every finite value, zero, subnormal and infinity equals IEEE binary16
+    (numpy's float16 is the independent implementation); a NaN stays a NaN with payload kept."""
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([oracle.f16_bits_to_f32(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    # payload: mantissa shifted left by 13, sign preserved (quant.rs:493-497).  The value comes
+    # back through a C float return and a Python float, which quiets a signalling NaN, so the
+    # quiet bit is masked on both sides; the golden checksums above pin the payload bits inside
+    # dequantize, where no such hop exists.
+    quiet = np.uint32(0x00400000)
+    gb = got[nan].view(np.uint32) | quiet
+    hb = bits[nan].astype(np.uint32)
+    assert np.array_equal(gb, ((hb & 0x8000) << 16) | 0x7F800000 | ((hb & 0x3FF) << 13) | quiet)
+
+
+def _f16(v):
+    return np.frombuffer(np.float16(v).tobytes(), np.uint8)
+
+
+def test_dequantize_q8_0_scales_signed_bytes():
+    """quant.rs:1818-1828."""
+    qs = np.zeros(32, np.int8)
+    qs[0], qs[1] = 1, -1
+    block = np.concatenate([_f16(2.0), qs.view(np.uint8)])
+    out = oracle.dequantize(Q8_0, block, 32)
+    assert out[0] == 2.0 and out[1] == -2.0
+    assert np.all(out[2:] == 0.0)
+
+
+def test_dequantize_q4_k_matches_the_reference_scale_unpacking():
+    """quant.rs:1846-1865: scale 1 / min 0 for all eight sub-blocks, nibble 5 -> 5.0."""
+    scales = np.array([1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1], np.uint8)
+    block = np.concatenate([_f16(1.0), _f16(0.0), scales, np.full(128, 0x55, np.uint8)])
+    out = oracle.dequantize(Q4_K, block, 256)
+    assert out.size == 256
+    assert np.all(np.abs(out - 5.0) < 1e-5)
+
+
+def test_get_scale_min_k4_against_bit_by_bit_decode():
+    """quant.rs:653-662 against ggml's published layout decoded field by field: sub-blocks 0..3
+    keep their 6 bits in bytes 0..3 (scale) and 4..7 (min); sub-blocks 4..7 keep the low 4 bits in
+    bytes 8..11 (scale low nibble, min high nibble) and the top 2 bits in the top 2 bits of bytes
+    0..3 (scale) and 4..7 (min).  A wrong index or shift fails for a random byte pattern."""
+    rng = np.random.default_rng(3)
+    for _ in range(50):
+        b = rng.integers(0, 256, 12, dtype=np.uint8)
+        for j in range(8):
+            if j < 4:
+                sc, m = b[j] % 64, b[j + 4] % 64
+            else:
+                sc = (b[j + 4] % 16) + 16 * (b[j - 4] // 64)
+                m = (b[j + 4] // 16) + 16 * (b[j] // 64)
+            assert oracle.get_scale_min_k4(j, b) == (int(sc), int(m))
+
+
+def test_dequantize_q4_k_sub_block_order_and_min():
+    """Distinct scale and min per sub-block, distinct nibbles per half: pins element order
+    (low nibbles of qs[32g..] are sub-block 2g, high nibbles 2g+1; quant.rs:679-690) and the
+    sign of the min term."""
+    sc = [3, 5, 7, 9, 11, 13, 15, 17]
+    mn = [1, 2, 3, 4, 21, 22, 23, 24]
+    scales = np.zeros(12, np.uint8)
+    for j in range(4):
+        scales[j] = sc[j] | ((sc[j + 4] >> 4) << 6)
+        scales[j + 4] = mn[j] | ((mn[j + 4] >> 4) << 6)
+        scales[j + 8] = (sc[j + 4] & 0xF) | ((mn[j + 4] & 0xF) << 4)
+    qs = np.zeros(128, np.uint8)
+    for g in range(4):
+        for l in range(32):
+            lo, hi = (l + g) % 16, (3 * l + g) % 16
+            qs[32 * g + l] = lo | (hi << 4)
+    block = np.concatenate([_f16(0.5), _f16(0.25), scales, qs])
+    out = oracle.dequantize(Q4_K, block, 256)
+    for g in range(4):
+        for l in range(32):
+            lo, hi = (l + g) % 16, (3 * l + g) % 16
+            assert out[64 * g + l] == 0.5 * sc[2 * g] * lo - 0.25 * mn[2 * g]
+            assert out[64 * g + 32 + l] == 0.5 * sc[2 * g + 1] * hi - 0.25 * mn[2 * g + 1]
+
+
+def test_dequantize_q6_k_zero_quant_gives_the_offset_scaled_value():
+    """quant.rs:1891-1903."""
+    block = np.concatenate([np.zeros(128, np.uint8), np.zeros(64, np.uint8),
+                            np.full(16, 2, np.uint8), _f16(1.0)])
+    out = oracle.dequantize(Q6_K, block, 256)
+    assert np.all(out == -64.0)
+
+
+def test_dequantize_q6_k_treats_scales_as_signed():
+    """quant.rs:1910-1921."""
+    block = np.concatenate([np.zeros(128, np.uint8), np.zeros(64, np.uint8),
+                            np.full(16, 0xFE, np.uint8), _f16(1.0)])
+    out = oracle.dequantize(Q6_K, block, 256)
+    assert np.all(out == 64.0)
+
+
+def test_dequantize_q6_k_element_order():
+    """Every element gets its own 6-bit value q = e % 64 and every 16-group its own scale; packs
+    them by ggml's published layout (element 128h+32r+l: nibble in ql[64h+32(r&1)+l] low for r<2
+    else high, top 2 bits at qh[32h+l] >> 2r, scale 8h+2r+l/16) and expects d*sc*(q-32)."""
+    ql = np.zeros(128, np.uint8)
+    qh = np.zeros(64, np.uint8)
+    sc = np.arange(-8, 8, dtype=np.int8)
+    for h in range(2):
+        for r in range(4):
+            for l in range(32):
+                e = 128 * h + 32 * r + l
+                q = (e * 7 + 3) % 64
+                nib, top = q & 0xF, q >> 4
+                idx = 64 * h + 32 * (r & 1) + l
+                ql[idx] |= nib if r < 2 else nib << 4
+                qh[32 * h + l] |= top << (2 * r)
+    block = np.concatenate([ql, qh, sc.view(np.uint8), _f16(0.5)])
+    out = oracle.dequantize(Q6_K, block, 256)
+    for e in range(256):
+        h, r, l = e // 128, (e % 128) // 32, e % 32
+        q = (e * 7 + 3) % 64
+        assert out[e] == 0.5 * float(sc[8 * h + 2 * r + l // 16]) * (q - 32), e
