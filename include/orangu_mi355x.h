@@ -1,0 +1,169 @@
+/*
+ * orangu_mi355x.h -- C ABI of the MI355X (gfx950) quantized matmul backend for orangu-server.
+ *
+ * This is the boundary a Rust `impl Backend` binds through FFI.  It replaces, for the GGUF types
+ * Q8_0, Q4_K and Q6_K, what `engine::backend::Backend` asks of a device
+ * (src/bin/orangu-server/engine/backend/mod.rs:309-496) and reproduces the arithmetic of
+ * `CpuBackend` (engine/backend/cpu.rs:55-317) over `engine::vecdot`:
+ *   - activation int8 quantization, per-block integer sums: bit-exact with the CPU path;
+ *   - f32 outputs: the per-block terms are combined in the CPU path's order, so they are
+ *     bit-identical as well (the contract asked for is 1e-3 relative / 1e-5 absolute).
+ *
+ * Conventions
+ *   - Every function returns OGM_OK (0) or a negative ogm_status.  Nothing aborts, throws or
+ *     exits across this boundary (the existing vendor backends panic on a HIP error,
+ *     engine/backend/rocm.rs:333-347; the shim decides what to do with a status).
+ *   - `x` is [n_tokens][in_dim] f32 row-major, `y` is [n_tokens][out_dim] f32 row-major
+ *     (backend/mod.rs:310-313).
+ *   - Host-pointer entry points copy in and out and return when `y` is complete.  `_dev` entry
+ *     points take device pointers, enqueue on `stream` (a hipStream_t, NULL = the context's own
+ *     stream) and return without synchronizing.
+ *   - A context is thread-safe: calls on one context serialize on an internal mutex, as
+ *     RocmBackend does (engine/backend/rocm.rs:30-41).
+ *   - There is no CPU fallback.  Without a usable gfx950 device ogm_init fails.
+ */
+#ifndef ORANGU_MI355X_H
+#define ORANGU_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ogm_ctx ogm_ctx;       /* one device + stream + weight cache */
+typedef struct ogm_weight ogm_weight; /* one uploaded, repacked QuantMatrix */
+
+typedef enum ogm_status {
+  OGM_OK = 0,
+  OGM_ERR_INVALID = -1,     /* bad argument (null pointer, zero dimension, size mismatch) */
+  OGM_ERR_UNSUPPORTED = -2, /* ggml type / in_dim without a kernel (vecdot.rs:274-283) */
+  OGM_ERR_NO_DEVICE = -3,   /* no HIP device, or not a gfx950 */
+  OGM_ERR_HIP = -4,         /* a HIP call failed; see ogm_last_error */
+  OGM_ERR_OOM = -5          /* host or device allocation failed */
+} ogm_status;
+
+/* ggml type ids (engine/quant.rs:50-61) */
+#define OGM_TYPE_Q8_0 8u
+#define OGM_TYPE_Q4_K 12u
+#define OGM_TYPE_Q6_K 14u
+
+/* Activation quantization modes */
+#define OGM_ACT_PER_32 0  /* vecdot::quantize_act,       vecdot.rs:79-126   (Q8_0 weights)   */
+#define OGM_ACT_PER_256 1 /* vecdot::quantize_act_k_row, vecdot.rs:3030-3053 (Q4_K, Q6_K)    */
+
+/* ---- lifetime -------------------------------------------------------------------------- */
+
+/* RocmBackend::try_init (engine/backend/rocm.rs:168-305): never aborts; a missing device is a
+ * status.  `device` is the HIP ordinal. */
+int ogm_init(int device, ogm_ctx **out);
+/* Frees every weight and buffer of the context.  Drop of the backend. */
+void ogm_destroy(ogm_ctx *ctx);
+/* Text of the last failure on this context (or of the last failed ogm_init when ctx is NULL).
+ * Valid until the next call on the same thread. */
+const char *ogm_last_error(ogm_ctx *ctx);
+/* RocmBackend::device_name (engine/backend/rocm.rs:307-316). */
+int ogm_device_name(ogm_ctx *ctx, char *buf, size_t buf_len);
+
+/* ---- capabilities ---------------------------------------------------------------------- */
+
+/* Backend::supports_type (backend/mod.rs:493): 1 for Q8_0, Q4_K, Q6_K, else 0. */
+int ogm_supports_type(uint32_t ggml_type);
+/* vecdot::supports (vecdot.rs:274-283) for those types: Q8_0 needs in_dim % 32 == 0, the
+ * K-quants in_dim % 256 == 0. */
+int ogm_supports(uint32_t ggml_type, uint32_t in_dim);
+/* quant::block_layout (quant.rs:132-169).  Returns OGM_ERR_UNSUPPORTED for other types. */
+int ogm_block_layout(uint32_t ggml_type, uint32_t *block_bytes, uint32_t *block_elems);
+
+/* ---- weights: the uploader --------------------------------------------------------------- */
+
+/* Bytes of the repacked ("tile-planar") form of a matrix: the raw GGUF blocks regrouped in tiles
+ * of 64 blocks so that every 16-byte piece of a block lies in a plane that 64 lanes read as one
+ * contiguous kilobyte; no bit of any block is altered and only the last tile is zero-padded. */
+size_t ogm_repacked_size(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim);
+/* Host-side repack and its exact inverse.  `raw` is QuantMatrix::raw_bytes()
+ * (engine/loader.rs:608-610): out_dim rows of row_bytes. */
+int ogm_repack_host(uint32_t ggml_type, const void *raw, size_t row_bytes, uint32_t in_dim,
+                    uint32_t out_dim, void *repacked);
+int ogm_unrepack_host(uint32_t ggml_type, const void *repacked, size_t row_bytes, uint32_t in_dim,
+                      uint32_t out_dim, void *raw);
+
+/* Uploads one QuantMatrix (engine/loader.rs:561-680): repacks `raw` and copies it to the device.
+ * Idempotent per (key_addr, key_len) = QuantMatrix::cache_key() (loader.rs:674-679): a second
+ * call with a known key returns the first handle and touches no memory, the way the vendor
+ * backends cache weights by key and never evict (engine/backend/rocm.rs:329-350).  key_len == 0
+ * disables caching. */
+int ogm_weight_upload(ogm_ctx *ctx, uint32_t ggml_type, const void *raw, size_t row_bytes,
+                      uint32_t in_dim, uint32_t out_dim, uint64_t key_addr, uint64_t key_len,
+                      ogm_weight **out);
+/* Copies the matrix back from the device and undoes the repack: `raw_out` receives exactly the
+ * bytes that were uploaded. */
+int ogm_weight_download(ogm_ctx *ctx, const ogm_weight *w, void *raw_out, size_t raw_len);
+/* Frees one weight (and its cache entry).  The reference never evicts; tests and long-running
+ * hosts may. */
+int ogm_weight_free(ogm_ctx *ctx, ogm_weight *w);
+int ogm_weight_info(const ogm_weight *w, uint32_t *ggml_type, uint32_t *in_dim, uint32_t *out_dim,
+                    size_t *device_bytes);
+
+/* ---- matmul: Backend ----------------------------------------------------------------------- */
+
+/* Backend::matmul / matmul_into (backend/mod.rs:313, 342) with CpuBackend's kernel choice
+ * (backend/cpu.rs:55-167): n_tokens == 1 -> the decode GEMV; n_tokens > 1 -> the prefill GEMM
+ * (K-quants: per-256 activations, min pass then dot pass; Q8_0: per-32 activations). */
+int ogm_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint32_t n_tokens, float *y);
+/* Backend::matmul_decode / matmul_decode_into (backend/mod.rs:386, 349; backend/cpu.rs:265-317):
+ * the n_tokens == 1 kernel once per (row, token), so row t equals decoding token t alone. */
+int ogm_matmul_decode(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint32_t n_tokens,
+                      float *y);
+
+/* MatmulOp (backend/mod.rs:121-125). */
+typedef struct ogm_op {
+  const ogm_weight *w;
+  const float *x;    /* [n_tokens][w.in_dim] */
+  uint32_t n_tokens;
+  float *y;          /* [n_tokens][w.out_dim] */
+} ogm_op;
+/* Backend::matmul_batch / matmul_batch_decode (backend/mod.rs:362, 405): independent ops, all
+ * launched before one synchronization.  Ops longer than `max_tokens_per_phase`
+ * (ORANGU_MAX_TOKENS_PER_SUBMISSION, default 256; backend/mod.rs:131-172) run in token stripes;
+ * 0 selects the default.  Striping never changes a value (vecdot.rs:4522-4549). */
+int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, int decode,
+                     uint32_t max_tokens_per_phase);
+
+/* Device-pointer forms: x and y already live in HBM.  Enqueues the activation quantize and the
+ * matmul kernels on `stream` and returns. */
+int ogm_matmul_dev(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
+                   float *y_dev, int decode, void *stream);
+
+/* ---- the integer stage, exposed for parity checks ------------------------------------------- */
+
+/* The fused activation quantizer on its own.  mode OGM_ACT_PER_32: d has n/32 entries
+ * (vecdot.rs:95-126); OGM_ACT_PER_256: n/256 (vecdot.rs:3030-3053).  q has n, sums n/16
+ * (per-16 sums of q, i32).  Host pointers; n % 32 (resp. 256) must be 0. */
+int ogm_quantize_act(ogm_ctx *ctx, int mode, const float *x, size_t n, int8_t *q, float *d,
+                     int32_t *sums);
+/* Per (token, row, block) integer sums the matmul kernels form before any float is touched:
+ * Q4_K: isum = sum_j sc_j * dot32_j and imin = sum_j m_j * bsum_j per super-block
+ * (vecdot.rs:3152-3178); Q6_K: isum per super-block (vecdot.rs:3215-3241), imin untouched;
+ * Q8_0: isum per 32-block (vecdot.rs:2829-2838).  Arrays are [n_tokens][out_dim][blocks per
+ * row]; imin may be NULL.  Runs the same kernels as ogm_matmul_decode with a dump switch. */
+int ogm_dump_block_sums(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint32_t n_tokens,
+                        int32_t *isum, int32_t *imin);
+
+/* f16 -> f32 as the kernels convert block scales, for all `n` inputs (host pointers).  Lets a
+ * test compare the device conversion with quant::f16_bits_to_f32 (quant.rs:511-528). */
+int ogm_f16_to_f32(ogm_ctx *ctx, const uint16_t *bits, size_t n, float *out);
+
+/* ---- tuning / introspection ------------------------------------------------------------------ */
+
+/* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.
+ * key: "gemv_rows" (output rows per workgroup; 0 = heuristic). */
+int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value);
+/* Name of the kernel the last matmul on this context launched (for profiles). */
+const char *ogm_last_kernel(ogm_ctx *ctx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,239 @@
+"""Host-side mirror of the reference's backend seam, over the C ABI.
+
+Same names and argument meaning as ``engine::backend::Backend``
+(src/bin/orangu-server/engine/backend/mod.rs:309-496), ``MatmulOp`` (mod.rs:121-125) and
+``QuantMatrix`` (engine/loader.rs:561-680), so the parity tests read like the reference's own
+(engine/backend/cpu.rs:509-651, engine/backend/rocm.rs:633-697).  Every method runs the HIP
+kernels through ``liborangu_mi355x.so``; there is no CPU path here.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import capi
+from .capi import OgmError, OgmOp
+
+BLOCK_LAYOUT = {8: (34, 32), 12: (144, 256), 14: (210, 256)}
+
+# backend/mod.rs:304-306
+MATMUL_ONLY_SURFACE = "matmul only - no fused layer chain, GPU attention or GPU sampling"
+# backend/mod.rs:131
+MAX_MULTI_TOKEN_PHASE_TOKENS_DEFAULT = 256
+
+
+class QuantMatrix:
+    """A quantized weight matrix as the loader hands it to a backend: ``out_dim`` contiguous rows
+    of ``row_bytes`` raw GGUF blocks (engine/loader.rs:561-680)."""
+
+    def __init__(self, data, ggml_type: int, in_dim: int, out_dim: int, start: int = 0):
+        self._bytes = np.ascontiguousarray(
+            np.frombuffer(data, dtype=np.uint8) if isinstance(data, (bytes, bytearray)) else data,
+            dtype=np.uint8)
+        if ggml_type not in BLOCK_LAYOUT:
+            raise ValueError(f"unsupported ggml_type {ggml_type}")
+        bb, be = BLOCK_LAYOUT[ggml_type]
+        if in_dim % be != 0:
+            raise ValueError(f"in_dim {in_dim} is not a multiple of the block size {be}")
+        self._ggml_type = ggml_type
+        self._start = start
+        self._row_bytes = in_dim // be * bb
+        self.in_dim = in_dim
+        self.out_dim = out_dim
+        if start + self._row_bytes * out_dim > self._bytes.size:
+            raise ValueError("byte range exceeds the tensor")  # loader.rs:1562-1570
+
+    def ggml_type(self) -> int:
+        return self._ggml_type
+
+    def row_bytes(self) -> int:
+        return self._row_bytes
+
+    def raw_bytes(self) -> np.ndarray:
+        return self._bytes[self._start:self._start + self._row_bytes * self.out_dim]
+
+    def rows(self, first: int, count: int) -> "QuantMatrix":
+        """loader.rs:627-646: a view of rows first..first+count sharing the same bytes."""
+        if first + count > self.out_dim:
+            raise ValueError(f"row range {first}..{first + count} exceeds out_dim {self.out_dim}")
+        return QuantMatrix(self._bytes, self._ggml_type, self.in_dim, count,
+                           self._start + first * self._row_bytes)
+
+    def cache_key(self) -> tuple[int, int]:
+        """loader.rs:674-679: (absolute address, byte length)."""
+        return (self._bytes.ctypes.data + self._start, self._row_bytes * self.out_dim)
+
+
+@dataclass
+class MatmulOp:
+    """backend/mod.rs:121-125."""
+    x: np.ndarray
+    n_tokens: int
+    w: QuantMatrix
+
+
+class Mi355xBackend:
+    """``impl Backend`` over the MI355X kernels."""
+
+    def __init__(self, device: int = 0):
+        self._lib = capi.load_library()
+        ctx = C.c_void_p()
+        rc = self._lib.ogm_init(device, C.byref(ctx))
+        if rc != 0:
+            raise OgmError(rc, "ogm_init", self._lib.ogm_last_error(None).decode())
+        self._ctx = ctx
+        self._keepalive: dict[tuple[int, int], np.ndarray] = {}
+
+    # ---- lifetime ----
+    @classmethod
+    def try_init(cls, device: int = 0):
+        """RocmBackend::try_init (rocm.rs:168-173): None when no usable device."""
+        try:
+            return cls(device)
+        except OgmError:
+            return None
+
+    def close(self):
+        if getattr(self, "_ctx", None):
+            self._lib.ogm_destroy(self._ctx)
+            self._ctx = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _check(self, rc: int, where: str):
+        if rc != 0:
+            raise OgmError(rc, where, self._lib.ogm_last_error(self._ctx).decode())
+
+    def device_name(self) -> str:
+        buf = C.create_string_buffer(256)
+        self._check(self._lib.ogm_device_name(self._ctx, buf, 256), "ogm_device_name")
+        return buf.value.decode()
+
+    # ---- Backend ----
+    def supports_type(self, ggml_type: int) -> bool:
+        return bool(self._lib.ogm_supports_type(ggml_type))
+
+    def reduced_surface(self):
+        return MATMUL_ONLY_SURFACE
+
+    def as_wgpu(self):
+        return None
+
+    def upload(self, w: QuantMatrix) -> int:
+        """Weight handle for ``w``, uploading (and repacking) on first sight of its cache key."""
+        key = w.cache_key()
+        raw = w.raw_bytes()
+        handle = C.c_void_p()
+        rc = self._lib.ogm_weight_upload(self._ctx, w.ggml_type(), raw.ctypes.data, w.row_bytes(),
+                                         w.in_dim, w.out_dim, key[0], key[1], C.byref(handle))
+        self._check(rc, "ogm_weight_upload")
+        self._keepalive[key] = w._bytes  # the key is an address: keep the bytes alive with it
+        return handle.value
+
+    def download(self, w: QuantMatrix) -> np.ndarray:
+        h = self.upload(w)
+        out = np.empty(w.row_bytes() * w.out_dim, np.uint8)
+        self._check(self._lib.ogm_weight_download(self._ctx, h, out.ctypes.data, out.size),
+                    "ogm_weight_download")
+        return out
+
+    def _x(self, x, n_tokens: int, w: QuantMatrix) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+        if x.size != n_tokens * w.in_dim:
+            raise ValueError(f"x has {x.size} elements, expected {n_tokens}*{w.in_dim}")
+        return x
+
+    def matmul(self, x, n_tokens: int, w: QuantMatrix) -> np.ndarray:
+        """y[t, o] = sum_i x[t, i] * w.row(o)[i]; returns [n_tokens * out_dim] (mod.rs:313)."""
+        out = np.empty(0, np.float32)
+        return self.matmul_into(out, x, n_tokens, w)
+
+    def matmul_into(self, out: np.ndarray, x, n_tokens: int, w: QuantMatrix) -> np.ndarray:
+        x = self._x(x, n_tokens, w)
+        y = np.empty(n_tokens * w.out_dim, np.float32)
+        h = self.upload(w)
+        self._check(self._lib.ogm_matmul(self._ctx, h, x.ctypes.data, n_tokens, y.ctypes.data), "ogm_matmul")
+        return y
+
+    def matmul_decode(self, x, n_tokens: int, w: QuantMatrix) -> np.ndarray:
+        """mod.rs:386: the single-token kernel per (row, token)."""
+        x = self._x(x, n_tokens, w)
+        y = np.empty(n_tokens * w.out_dim, np.float32)
+        h = self.upload(w)
+        self._check(self._lib.ogm_matmul_decode(self._ctx, h, x.ctypes.data, n_tokens, y.ctypes.data),
+                    "ogm_matmul_decode")
+        return y
+
+    def _batch(self, ops, decode: bool, max_tokens: int):
+        arr = (OgmOp * len(ops))()
+        xs, ys = [], []
+        for i, op in enumerate(ops):
+            x = self._x(op.x, op.n_tokens, op.w)
+            y = np.empty(op.n_tokens * op.w.out_dim, np.float32)
+            xs.append(x)
+            ys.append(y)
+            arr[i].w = self.upload(op.w)
+            arr[i].x = x.ctypes.data
+            arr[i].n_tokens = op.n_tokens
+            arr[i].y = y.ctypes.data
+        self._check(self._lib.ogm_matmul_batch(self._ctx, arr, len(ops), int(decode), max_tokens),
+                    "ogm_matmul_batch")
+        return ys
+
+    def matmul_batch(self, ops, max_tokens_per_phase: int = 0):
+        """mod.rs:362-366: independent ops; long ones run in token stripes (mod.rs:154-172)."""
+        return self._batch(ops, False, max_tokens_per_phase)
+
+    def matmul_batch_decode(self, ops):
+        """mod.rs:405."""
+        return self._batch(ops, True, 0)
+
+    # ---- integer stage, for parity checks ----
+    def quantize_act(self, x, per_256: bool):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        n = x.size
+        g = 256 if per_256 else 32
+        q = np.empty(n, np.int8)
+        d = np.empty(n // g, np.float32)
+        s = np.empty(n // 16, np.int32)
+        self._check(self._lib.ogm_quantize_act(self._ctx, int(per_256), x.ctypes.data, n,
+                                               q.ctypes.data, d.ctypes.data, s.ctypes.data),
+                    "ogm_quantize_act")
+        return q, d, s
+
+    def dump_block_sums(self, x, n_tokens: int, w: QuantMatrix):
+        x = self._x(x, n_tokens, w)
+        _, be = BLOCK_LAYOUT[w.ggml_type()]
+        shape = (n_tokens, w.out_dim, w.in_dim // be)
+        isum = np.zeros(shape, np.int32)
+        imin = np.zeros(shape, np.int32)
+        h = self.upload(w)
+        self._check(self._lib.ogm_dump_block_sums(self._ctx, h, x.ctypes.data, n_tokens,
+                                                  isum.ctypes.data, imin.ctypes.data),
+                    "ogm_dump_block_sums")
+        return isum, imin
+
+    def f16_to_f32(self, bits) -> np.ndarray:
+        bits = np.ascontiguousarray(bits, np.uint16)
+        out = np.empty(bits.size, np.float32)
+        self._check(self._lib.ogm_f16_to_f32(self._ctx, bits.ctypes.data, bits.size, out.ctypes.data),
+                    "ogm_f16_to_f32")
+        return out
+
+    # ---- device-resident path (torch tensors or raw device pointers) ----
+    def matmul_dev(self, w_handle: int, x_ptr: int, n_tokens: int, y_ptr: int, decode: bool = False,
+                   stream: int = 0):
+        self._check(self._lib.ogm_matmul_dev(self._ctx, w_handle, x_ptr, n_tokens, y_ptr,
+                                             int(decode), stream or None), "ogm_matmul_dev")
+
+    def set_tuning(self, key: str, value: int):
+        self._check(self._lib.ogm_set_tuning(self._ctx, key.encode(), value), "ogm_set_tuning")
+
+    def last_kernel(self) -> str:
+        return self._lib.ogm_last_kernel(self._ctx).decode()

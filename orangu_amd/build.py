@@ -1,0 +1,49 @@
+"""Builds the HIP library in-tree (``orangu_amd/liborangu_mi355x.so``) for gfx950.
+
+hipcc cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is installed.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_NAME = "liborangu_mi355x.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+
+SOURCES = ["ogm_kernels.hip", "ogm_gemm.hip", "ogm_api.cpp", "ogm_repack.cpp"]
+
+# -ffp-contract=off: the kernels reproduce the CPU path's f32 results bit for bit, which an FMA
+#   contraction would break.
+# -packed-fp32-ops off: keeps hipcc from forming packed FP32 instructions out of scalar code.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def build(verbose: bool = False) -> str:
+    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    cmd = [hipcc(), *HIPCC_FLAGS, "-shared", "-o", LIB_PATH, *srcs]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    log = "\n".join(l for l in (proc.stdout + proc.stderr).splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + log)
+    if verbose and log.strip():
+        print(log)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

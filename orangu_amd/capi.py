@@ -1,0 +1,79 @@
+"""ctypes declarations of ``include/orangu_mi355x.h``.
+
+Loads the in-tree ``liborangu_mi355x.so``.  There is no fallback: if the library is missing or a
+call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "liborangu_mi355x.so")
+
+OGM_OK = 0
+STATUS = {0: "OGM_OK", -1: "OGM_ERR_INVALID", -2: "OGM_ERR_UNSUPPORTED", -3: "OGM_ERR_NO_DEVICE",
+          -4: "OGM_ERR_HIP", -5: "OGM_ERR_OOM"}
+
+# every symbol the header declares
+SYMBOLS = [
+    "ogm_init", "ogm_destroy", "ogm_last_error", "ogm_device_name", "ogm_supports_type",
+    "ogm_supports", "ogm_block_layout", "ogm_repacked_size", "ogm_repack_host",
+    "ogm_unrepack_host", "ogm_weight_upload", "ogm_weight_download", "ogm_weight_free",
+    "ogm_weight_info", "ogm_matmul", "ogm_matmul_decode", "ogm_matmul_batch", "ogm_matmul_dev",
+    "ogm_quantize_act", "ogm_dump_block_sums", "ogm_f16_to_f32", "ogm_set_tuning",
+    "ogm_last_kernel",
+]
+
+
+class OgmError(RuntimeError):
+    def __init__(self, status: int, where: str, detail: str = ""):
+        self.status = status
+        super().__init__(f"{where}: {STATUS.get(status, status)}" + (f" ({detail})" if detail else ""))
+
+
+class OgmOp(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("x", C.c_void_p), ("n_tokens", C.c_uint32), ("y", C.c_void_p)]
+
+
+_lib = None
+
+
+def load_library() -> C.CDLL:
+    """Loads the built library, building nothing.  Raises if it is absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise OgmError(-3, "load_library", f"{LIB_PATH} is not built; run __graft_entry__.build()")
+    L = C.CDLL(LIB_PATH)
+    vp, sz, u32, u64 = C.c_void_p, C.c_size_t, C.c_uint32, C.c_uint64
+    L.ogm_init.argtypes = [C.c_int, C.POINTER(vp)]
+    L.ogm_destroy.argtypes = [vp]
+    L.ogm_destroy.restype = None
+    L.ogm_last_error.argtypes = [vp]
+    L.ogm_last_error.restype = C.c_char_p
+    L.ogm_device_name.argtypes = [vp, C.c_char_p, sz]
+    L.ogm_supports_type.argtypes = [u32]
+    L.ogm_supports.argtypes = [u32, u32]
+    L.ogm_block_layout.argtypes = [u32, C.POINTER(u32), C.POINTER(u32)]
+    L.ogm_repacked_size.argtypes = [u32, u32, u32]
+    L.ogm_repacked_size.restype = sz
+    L.ogm_repack_host.argtypes = [u32, vp, sz, u32, u32, vp]
+    L.ogm_unrepack_host.argtypes = [u32, vp, sz, u32, u32, vp]
+    L.ogm_weight_upload.argtypes = [vp, u32, vp, sz, u32, u32, u64, u64, C.POINTER(vp)]
+    L.ogm_weight_download.argtypes = [vp, vp, vp, sz]
+    L.ogm_weight_free.argtypes = [vp, vp]
+    L.ogm_weight_info.argtypes = [vp, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32), C.POINTER(sz)]
+    L.ogm_matmul.argtypes = [vp, vp, vp, u32, vp]
+    L.ogm_matmul_decode.argtypes = [vp, vp, vp, u32, vp]
+    L.ogm_matmul_batch.argtypes = [vp, C.POINTER(OgmOp), sz, C.c_int, u32]
+    L.ogm_matmul_dev.argtypes = [vp, vp, vp, u32, vp, C.c_int, vp]
+    L.ogm_quantize_act.argtypes = [vp, C.c_int, vp, sz, vp, vp, vp]
+    L.ogm_dump_block_sums.argtypes = [vp, vp, vp, u32, vp, vp]
+    L.ogm_f16_to_f32.argtypes = [vp, vp, sz, vp]
+    L.ogm_set_tuning.argtypes = [vp, C.c_char_p, C.c_int]
+    L.ogm_last_kernel.argtypes = [vp]
+    L.ogm_last_kernel.restype = C.c_char_p
+    _lib = L
+    return L

@@ -1,0 +1,520 @@
+// C ABI of the MI355X quantized matmul backend (include/orangu_mi355x.h): context, weight
+// uploader and the Backend::matmul family (engine/backend/mod.rs:309-496 of orangu-server),
+// over the kernels in ogm_kernels.hip.  No CPU fallback: every compute entry point runs the
+// HIP kernels or returns an error status.
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <new>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/orangu_mi355x.h"
+#include "ogm_kernels.h"
+#include "ogm_layout.h"
+
+// ------------------------------------------------------------------------------------------
+
+struct ogm_weight {
+  uint32_t ggml_type, in_dim, out_dim;
+  size_t row_bytes, device_bytes;
+  uint8_t *dev;  // tile-planar
+  uint64_t key_addr, key_len;
+};
+
+struct DevBuf {
+  void *p = nullptr;
+  size_t cap = 0;
+};
+
+struct ogm_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  std::mutex mu;
+  std::string err;
+  std::string name;
+  std::map<std::pair<uint64_t, uint64_t>, ogm_weight *> cache;
+  std::vector<ogm_weight *> weights;
+  // scratch, grown on demand and reused (the vendor backends allocate per call,
+  // engine/backend/rocm.rs:352-376; a pool is what the Vulkan op_cache does instead)
+  DevBuf x, y, q, d, sums, bsum, isum, imin;
+  DevBuf hx, hy;  // pinned host staging
+  int tune_gemv_rows = 0;
+  const char *last_kernel = "";
+};
+
+static thread_local std::string g_init_err;
+
+static int fail(ogm_ctx *ctx, int status, const std::string &msg) {
+  if (ctx)
+    ctx->err = msg;
+  else
+    g_init_err = msg;
+  return status;
+}
+
+#define HIPCHK(ctx, call)                                                              \
+  do {                                                                                 \
+    hipError_t e_ = (call);                                                            \
+    if (e_ != hipSuccess)                                                              \
+      return fail(ctx, e_ == hipErrorOutOfMemory ? OGM_ERR_OOM : OGM_ERR_HIP,          \
+                  std::string(#call) + ": " + hipGetErrorString(e_));                  \
+  } while (0)
+
+static int ensure_dev(ogm_ctx *ctx, DevBuf &b, size_t bytes) {
+  if (bytes <= b.cap) return OGM_OK;
+  // Kernels still in flight may read the old buffer.
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  if (b.p) HIPCHK(ctx, hipFree(b.p));
+  b.p = nullptr;
+  b.cap = 0;
+  size_t cap = (bytes + 255) & ~(size_t)255;
+  HIPCHK(ctx, hipMalloc(&b.p, cap));
+  b.cap = cap;
+  return OGM_OK;
+}
+
+static int ensure_host(ogm_ctx *ctx, DevBuf &b, size_t bytes) {
+  if (bytes <= b.cap) return OGM_OK;
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  if (b.p) HIPCHK(ctx, hipHostFree(b.p));
+  b.p = nullptr;
+  b.cap = 0;
+  size_t cap = (bytes + 4095) & ~(size_t)4095;
+  HIPCHK(ctx, hipHostMalloc(&b.p, cap, hipHostMallocDefault));
+  b.cap = cap;
+  return OGM_OK;
+}
+
+static int act_mode_for(uint32_t ggml_type) {
+  // backend/cpu.rs:100-116: K-quants take the per-256 quantizer, Q8_0 the per-32 one
+  return ggml_type == OGM_Q8_0 ? OGM_ACT_PER_32 : OGM_ACT_PER_256;
+}
+
+static int ensure_act(ogm_ctx *ctx, uint32_t in_dim, uint32_t n_tokens) {
+  int rc;
+  size_t n = (size_t)in_dim * n_tokens;
+  if ((rc = ensure_dev(ctx, ctx->q, n)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->d, n / 32 * 4)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->sums, n / 16 * 4)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->bsum, n / 32 * 2)) != OGM_OK) return rc;
+  return OGM_OK;
+}
+
+static OgmActDev act_view(ogm_ctx *ctx, uint32_t in_dim, int mode, uint32_t token0) {
+  OgmActDev a;
+  a.q = (int8_t *)ctx->q.p + (size_t)token0 * in_dim;
+  a.d = (float *)ctx->d.p + (size_t)token0 * (in_dim / (mode == OGM_ACT_PER_32 ? 32 : 256));
+  a.sums = (int32_t *)ctx->sums.p + (size_t)token0 * (in_dim / 16);
+  a.bsum = (int16_t *)ctx->bsum.p + (size_t)token0 * (in_dim / 32);
+  return a;
+}
+
+// ------------------------------------------------------------------------------------------
+// lifetime
+
+extern "C" int ogm_init(int device, ogm_ctx **out) {
+  if (!out) return fail(nullptr, OGM_ERR_INVALID, "ogm_init: out is null");
+  *out = nullptr;
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n <= 0)
+    return fail(nullptr, OGM_ERR_NO_DEVICE,
+                std::string("no HIP device: ") + (e != hipSuccess ? hipGetErrorString(e) : "count 0"));
+  if (device < 0 || device >= n)
+    return fail(nullptr, OGM_ERR_NO_DEVICE, "device ordinal out of range");
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess)
+    return fail(nullptr, OGM_ERR_HIP, std::string("hipGetDeviceProperties: ") + hipGetErrorString(e));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(nullptr, OGM_ERR_NO_DEVICE,
+                std::string("device is ") + prop.gcnArchName + ", these kernels are built for gfx950 only");
+  ogm_ctx *ctx = new (std::nothrow) ogm_ctx();
+  if (!ctx) return fail(nullptr, OGM_ERR_OOM, "out of host memory");
+  ctx->device = device;
+  ctx->name = std::string(prop.name) + " (" + prop.gcnArchName + ")";
+  e = hipSetDevice(device);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    std::string msg = std::string("stream creation: ") + hipGetErrorString(e);
+    delete ctx;
+    return fail(nullptr, OGM_ERR_HIP, msg);
+  }
+  *out = ctx;
+  return OGM_OK;
+}
+
+extern "C" void ogm_destroy(ogm_ctx *ctx) {
+  if (!ctx) return;
+  (void)hipSetDevice(ctx->device);
+  if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+  for (ogm_weight *w : ctx->weights) {
+    if (w->dev) (void)hipFree(w->dev);
+    delete w;
+  }
+  DevBuf *dev[] = {&ctx->x, &ctx->y, &ctx->q, &ctx->d, &ctx->sums, &ctx->bsum, &ctx->isum, &ctx->imin};
+  for (DevBuf *b : dev)
+    if (b->p) (void)hipFree(b->p);
+  if (ctx->hx.p) (void)hipHostFree(ctx->hx.p);
+  if (ctx->hy.p) (void)hipHostFree(ctx->hy.p);
+  if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+  delete ctx;
+}
+
+extern "C" const char *ogm_last_error(ogm_ctx *ctx) {
+  static thread_local std::string copy;
+  if (ctx) {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    copy = ctx->err;
+  } else {
+    copy = g_init_err;
+  }
+  return copy.c_str();
+}
+
+extern "C" int ogm_device_name(ogm_ctx *ctx, char *buf, size_t buf_len) {
+  if (!ctx || !buf || buf_len == 0) return OGM_ERR_INVALID;
+  snprintf(buf, buf_len, "%s", ctx->name.c_str());
+  return OGM_OK;
+}
+
+extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
+  if (!ctx || !key) return OGM_ERR_INVALID;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (strcmp(key, "gemv_rows") == 0) {
+    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemv_rows must be >= 0");
+    ctx->tune_gemv_rows = value;
+    return OGM_OK;
+  }
+  return fail(ctx, OGM_ERR_INVALID, std::string("unknown tuning key ") + key);
+}
+
+extern "C" const char *ogm_last_kernel(ogm_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
+
+// ------------------------------------------------------------------------------------------
+// weights
+
+extern "C" int ogm_weight_upload(ogm_ctx *ctx, uint32_t ggml_type, const void *raw,
+                                 size_t row_bytes, uint32_t in_dim, uint32_t out_dim,
+                                 uint64_t key_addr, uint64_t key_len, ogm_weight **out) {
+  if (!ctx || !out) return OGM_ERR_INVALID;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  *out = nullptr;
+  if (key_len != 0) {
+    auto it = ctx->cache.find({key_addr, key_len});
+    if (it != ctx->cache.end()) {
+      ogm_weight *w = it->second;
+      if (w->ggml_type != ggml_type || w->in_dim != in_dim || w->out_dim != out_dim)
+        return fail(ctx, OGM_ERR_INVALID, "cache key reused with a different shape or type");
+      *out = w;
+      return OGM_OK;
+    }
+  }
+  if (!raw) return fail(ctx, OGM_ERR_INVALID, "raw is null");
+  if (!ogm_supports_type(ggml_type)) return fail(ctx, OGM_ERR_UNSUPPORTED, "ggml type without a kernel");
+  if (in_dim == 0 || out_dim == 0) return fail(ctx, OGM_ERR_INVALID, "zero dimension");
+  if (!ogm_supports(ggml_type, in_dim))
+    return fail(ctx, OGM_ERR_UNSUPPORTED, "in_dim is not a whole number of blocks");
+  size_t bytes = ogm_repacked_size(ggml_type, in_dim, out_dim);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  void *staging = nullptr;
+  HIPCHK(ctx, hipHostMalloc(&staging, bytes, hipHostMallocDefault));
+  int rc = ogm_repack_host(ggml_type, raw, row_bytes, in_dim, out_dim, staging);
+  if (rc != OGM_OK) {
+    (void)hipHostFree(staging);
+    return fail(ctx, rc, "row_bytes does not match in_dim for this type");
+  }
+  ogm_weight *w = new (std::nothrow) ogm_weight();
+  if (!w) {
+    (void)hipHostFree(staging);
+    return fail(ctx, OGM_ERR_OOM, "out of host memory");
+  }
+  w->ggml_type = ggml_type;
+  w->in_dim = in_dim;
+  w->out_dim = out_dim;
+  w->row_bytes = row_bytes;
+  w->device_bytes = bytes;
+  w->key_addr = key_addr;
+  w->key_len = key_len;
+  w->dev = nullptr;
+  hipError_t e = hipMalloc((void **)&w->dev, bytes);
+  if (e == hipSuccess) e = hipMemcpyAsync(w->dev, staging, bytes, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  (void)hipHostFree(staging);
+  if (e != hipSuccess) {
+    if (w->dev) (void)hipFree(w->dev);
+    delete w;
+    return fail(ctx, e == hipErrorOutOfMemory ? OGM_ERR_OOM : OGM_ERR_HIP,
+                std::string("weight upload: ") + hipGetErrorString(e));
+  }
+  ctx->weights.push_back(w);
+  if (key_len != 0) ctx->cache[{key_addr, key_len}] = w;
+  *out = w;
+  return OGM_OK;
+}
+
+extern "C" int ogm_weight_download(ogm_ctx *ctx, const ogm_weight *w, void *raw_out, size_t raw_len) {
+  if (!ctx || !w || !raw_out) return OGM_ERR_INVALID;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (raw_len != w->row_bytes * w->out_dim) return fail(ctx, OGM_ERR_INVALID, "raw_len mismatch");
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  std::vector<uint8_t> tmp(w->device_bytes);
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  HIPCHK(ctx, hipMemcpy(tmp.data(), w->dev, w->device_bytes, hipMemcpyDeviceToHost));
+  return ogm_unrepack_host(w->ggml_type, tmp.data(), w->row_bytes, w->in_dim, w->out_dim, raw_out);
+}
+
+extern "C" int ogm_weight_free(ogm_ctx *ctx, ogm_weight *w) {
+  if (!ctx || !w) return OGM_ERR_INVALID;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  for (size_t i = 0; i < ctx->weights.size(); i++) {
+    if (ctx->weights[i] == w) {
+      ctx->weights.erase(ctx->weights.begin() + (long)i);
+      if (w->key_len != 0) ctx->cache.erase({w->key_addr, w->key_len});
+      if (w->dev) HIPCHK(ctx, hipFree(w->dev));
+      delete w;
+      return OGM_OK;
+    }
+  }
+  return fail(ctx, OGM_ERR_INVALID, "weight does not belong to this context");
+}
+
+extern "C" int ogm_weight_info(const ogm_weight *w, uint32_t *ggml_type, uint32_t *in_dim,
+                               uint32_t *out_dim, size_t *device_bytes) {
+  if (!w) return OGM_ERR_INVALID;
+  if (ggml_type) *ggml_type = w->ggml_type;
+  if (in_dim) *in_dim = w->in_dim;
+  if (out_dim) *out_dim = w->out_dim;
+  if (device_bytes) *device_bytes = w->device_bytes;
+  return OGM_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// matmul
+
+// Enqueues quantize + kernels for tokens of x_dev into y_dev.  Caller holds the lock.
+static int enqueue_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
+                          float *y_dev, int decode, hipStream_t stream, int32_t *dump_isum,
+                          int32_t *dump_imin) {
+  if (n_tokens == 0) return OGM_OK;
+  const int mode = act_mode_for(w->ggml_type);
+  int rc = ensure_act(ctx, w->in_dim, n_tokens);
+  if (rc != OGM_OK) return rc;
+  HIPCHK(ctx, ogm_launch_quantize(mode, x_dev, w->in_dim, n_tokens, act_view(ctx, w->in_dim, mode, 0),
+                                  stream));
+  // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
+  // n_tokens == 1 and every matmul_decode take the GEMV's.
+  const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
+  const uint32_t rows = (uint32_t)ctx->tune_gemv_rows;
+  const uint32_t chunk = ogm_gemv_max_tokens(w->ggml_type, w->in_dim, gemm_order, rows);
+  if (chunk == 0) return fail(ctx, OGM_ERR_UNSUPPORTED, "no kernel for this type");
+  const uint32_t blocks_per_row = w->in_dim / (w->ggml_type == OGM_Q8_0 ? 32 : 256);
+  for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
+    OgmGemvArgs a;
+    a.ggml_type = w->ggml_type;
+    a.wt = w->dev;
+    a.in_dim = w->in_dim;
+    a.out_dim = w->out_dim;
+    a.act = act_view(ctx, w->in_dim, mode, t0);
+    a.n_tokens = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
+    a.y = y_dev + (size_t)t0 * w->out_dim;
+    a.gemm_order = gemm_order;
+    a.rows_per_wg = rows;
+    a.dump_isum = dump_isum ? dump_isum + (size_t)t0 * w->out_dim * blocks_per_row : nullptr;
+    a.dump_imin = dump_imin ? dump_imin + (size_t)t0 * w->out_dim * blocks_per_row : nullptr;
+    HIPCHK(ctx, ogm_launch_gemv(a, stream, &ctx->last_kernel));
+  }
+  return OGM_OK;
+}
+
+static int check_matmul_args(ogm_ctx *ctx, const ogm_weight *w, const void *x, const void *y,
+                             uint32_t n_tokens) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!w) return fail(ctx, OGM_ERR_INVALID, "weight is null");
+  if (n_tokens != 0 && (!x || !y)) return fail(ctx, OGM_ERR_INVALID, "x or y is null");
+  return OGM_OK;
+}
+
+static int host_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint32_t n_tokens,
+                       float *y, int decode) {
+  int rc = check_matmul_args(ctx, w, x, y, n_tokens);
+  if (rc != OGM_OK) return rc;
+  if (n_tokens == 0) return OGM_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  const size_t xb = (size_t)n_tokens * w->in_dim * 4, yb = (size_t)n_tokens * w->out_dim * 4;
+  if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
+  if ((rc = ensure_host(ctx, ctx->hx, xb)) != OGM_OK) return rc;
+  if ((rc = ensure_host(ctx, ctx->hy, yb)) != OGM_OK) return rc;
+  memcpy(ctx->hx.p, x, xb);
+  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, ctx->hx.p, xb, hipMemcpyHostToDevice, ctx->stream));
+  rc = enqueue_matmul(ctx, w, (const float *)ctx->x.p, n_tokens, (float *)ctx->y.p, decode,
+                      ctx->stream, nullptr, nullptr);
+  if (rc != OGM_OK) return rc;
+  HIPCHK(ctx, hipMemcpyAsync(ctx->hy.p, ctx->y.p, yb, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  memcpy(y, ctx->hy.p, yb);
+  return OGM_OK;
+}
+
+extern "C" int ogm_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint32_t n_tokens,
+                          float *y) {
+  return host_matmul(ctx, w, x, n_tokens, y, 0);
+}
+
+extern "C" int ogm_matmul_decode(ogm_ctx *ctx, const ogm_weight *w, const float *x,
+                                 uint32_t n_tokens, float *y) {
+  return host_matmul(ctx, w, x, n_tokens, y, 1);
+}
+
+extern "C" int ogm_matmul_dev(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev,
+                              uint32_t n_tokens, float *y_dev, int decode, void *stream) {
+  int rc = check_matmul_args(ctx, w, x_dev, y_dev, n_tokens);
+  if (rc != OGM_OK) return rc;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
+  return enqueue_matmul(ctx, w, x_dev, n_tokens, y_dev, decode, s, nullptr, nullptr);
+}
+
+// Backend::matmul_batch (backend/mod.rs:362-366) with guarded_matmul_op's token stripes
+// (backend/mod.rs:154-172): every stripe of every op is enqueued, then one synchronization.
+extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, int decode,
+                                uint32_t max_tokens_per_phase) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (n_ops == 0) return OGM_OK;
+  if (!ops) return fail(ctx, OGM_ERR_INVALID, "ops is null");
+  const uint32_t cap = max_tokens_per_phase ? max_tokens_per_phase : 256;
+  for (size_t i = 0; i < n_ops; i++) {
+    int rc = check_matmul_args(ctx, ops[i].w, ops[i].x, ops[i].y, ops[i].n_tokens);
+    if (rc != OGM_OK) return rc;
+  }
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  // All ops share the activation scratch, so x / y of every op get their own slice of the
+  // transfer buffers but the quantized activations are consumed before the next op's quantize
+  // (same stream, in order).
+  size_t xb = 0, yb = 0;
+  for (size_t i = 0; i < n_ops; i++) {
+    xb += (size_t)ops[i].n_tokens * ops[i].w->in_dim * 4;
+    yb += (size_t)ops[i].n_tokens * ops[i].w->out_dim * 4;
+  }
+  if (xb == 0) return OGM_OK;
+  int rc;
+  if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
+  if ((rc = ensure_host(ctx, ctx->hx, xb)) != OGM_OK) return rc;
+  if ((rc = ensure_host(ctx, ctx->hy, yb)) != OGM_OK) return rc;
+  // Size the activation scratch for the largest stripe before anything is enqueued, so it is
+  // never reallocated under kernels in flight.
+  for (size_t i = 0; i < n_ops; i++) {
+    uint32_t t = ops[i].n_tokens < cap ? ops[i].n_tokens : cap;
+    if ((rc = ensure_act(ctx, ops[i].w->in_dim, t)) != OGM_OK) return rc;
+  }
+  size_t xo = 0, yo = 0;
+  for (size_t i = 0; i < n_ops; i++) {
+    const ogm_op &op = ops[i];
+    const size_t bytes = (size_t)op.n_tokens * op.w->in_dim * 4;
+    if (bytes) memcpy((uint8_t *)ctx->hx.p + xo, op.x, bytes);
+    xo += bytes;
+  }
+  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, ctx->hx.p, xb, hipMemcpyHostToDevice, ctx->stream));
+  xo = 0;
+  for (size_t i = 0; i < n_ops; i++) {
+    const ogm_op &op = ops[i];
+    const float *xd = (const float *)((uint8_t *)ctx->x.p + xo);
+    float *yd = (float *)((uint8_t *)ctx->y.p + yo);
+    for (uint32_t t0 = 0; t0 < op.n_tokens; t0 += cap) {
+      const uint32_t nt = op.n_tokens - t0 < cap ? op.n_tokens - t0 : cap;
+      rc = enqueue_matmul(ctx, op.w, xd + (size_t)t0 * op.w->in_dim, nt,
+                          yd + (size_t)t0 * op.w->out_dim, decode, ctx->stream, nullptr, nullptr);
+      if (rc != OGM_OK) return rc;
+    }
+    xo += (size_t)op.n_tokens * op.w->in_dim * 4;
+    yo += (size_t)op.n_tokens * op.w->out_dim * 4;
+  }
+  HIPCHK(ctx, hipMemcpyAsync(ctx->hy.p, ctx->y.p, yb, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  yo = 0;
+  for (size_t i = 0; i < n_ops; i++) {
+    const size_t bytes = (size_t)ops[i].n_tokens * ops[i].w->out_dim * 4;
+    if (bytes) memcpy(ops[i].y, (uint8_t *)ctx->hy.p + yo, bytes);
+    yo += bytes;
+  }
+  return OGM_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// integer stage, exposed
+
+extern "C" int ogm_quantize_act(ogm_ctx *ctx, int mode, const float *x, size_t n, int8_t *q,
+                                float *d, int32_t *sums) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (mode != OGM_ACT_PER_32 && mode != OGM_ACT_PER_256) return fail(ctx, OGM_ERR_INVALID, "bad mode");
+  const size_t group = mode == OGM_ACT_PER_32 ? 32 : 256;
+  if (n == 0) return OGM_OK;
+  if (!x || !q || !d) return fail(ctx, OGM_ERR_INVALID, "null pointer");
+  if (n % group != 0 || n > 0xFFFFFF00u) return fail(ctx, OGM_ERR_INVALID, "n is not a whole number of groups");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  int rc;
+  if ((rc = ensure_dev(ctx, ctx->x, n * 4)) != OGM_OK) return rc;
+  if ((rc = ensure_act(ctx, (uint32_t)n, 1)) != OGM_OK) return rc;
+  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, x, n * 4, hipMemcpyHostToDevice, ctx->stream));
+  HIPCHK(ctx, ogm_launch_quantize(mode, (const float *)ctx->x.p, (uint32_t)n, 1,
+                                  act_view(ctx, (uint32_t)n, mode, 0), ctx->stream));
+  HIPCHK(ctx, hipMemcpyAsync(q, ctx->q.p, n, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipMemcpyAsync(d, ctx->d.p, n / group * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (sums) HIPCHK(ctx, hipMemcpyAsync(sums, ctx->sums.p, n / 16 * 4, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return OGM_OK;
+}
+
+extern "C" int ogm_dump_block_sums(ogm_ctx *ctx, const ogm_weight *w, const float *x,
+                                   uint32_t n_tokens, int32_t *isum, int32_t *imin) {
+  int rc = check_matmul_args(ctx, w, x, isum, n_tokens);
+  if (rc != OGM_OK) return rc;
+  if (n_tokens == 0) return OGM_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  const size_t blocks = (size_t)w->in_dim / (w->ggml_type == OGM_Q8_0 ? 32 : 256);
+  const size_t nb = (size_t)n_tokens * w->out_dim * blocks * 4;
+  const size_t xb = (size_t)n_tokens * w->in_dim * 4, yb = (size_t)n_tokens * w->out_dim * 4;
+  const bool want_min = imin && w->ggml_type == OGM_Q4_K;
+  if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->isum, nb)) != OGM_OK) return rc;
+  if (want_min && (rc = ensure_dev(ctx, ctx->imin, nb)) != OGM_OK) return rc;
+  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, x, xb, hipMemcpyHostToDevice, ctx->stream));
+  rc = enqueue_matmul(ctx, w, (const float *)ctx->x.p, n_tokens, (float *)ctx->y.p, 1, ctx->stream,
+                      (int32_t *)ctx->isum.p, want_min ? (int32_t *)ctx->imin.p : nullptr);
+  if (rc != OGM_OK) return rc;
+  HIPCHK(ctx, hipMemcpyAsync(isum, ctx->isum.p, nb, hipMemcpyDeviceToHost, ctx->stream));
+  if (want_min) HIPCHK(ctx, hipMemcpyAsync(imin, ctx->imin.p, nb, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return OGM_OK;
+}
+
+extern "C" int ogm_f16_to_f32(ogm_ctx *ctx, const uint16_t *bits, size_t n, float *out) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (n == 0) return OGM_OK;
+  if (!bits || !out) return fail(ctx, OGM_ERR_INVALID, "null pointer");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  int rc;
+  if ((rc = ensure_dev(ctx, ctx->x, n * 2)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->y, n * 4)) != OGM_OK) return rc;
+  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, bits, n * 2, hipMemcpyHostToDevice, ctx->stream));
+  HIPCHK(ctx, ogm_launch_f16_to_f32((const uint16_t *)ctx->x.p, n, (float *)ctx->y.p, ctx->stream));
+  HIPCHK(ctx, hipMemcpyAsync(out, ctx->y.p, n * 4, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return OGM_OK;
+}

@@ -1,0 +1,40 @@
+// Launchers of the gfx950 kernels, called by the C ABI in ogm_api.cpp.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// Quantized activations of up to n_tokens tokens, token-major, on the device:
+//   q    int8 [T][in_dim]
+//   d    f32  [T][in_dim/32] (per-32 mode) or [T][in_dim/256] (per-256 mode)
+//   sums i32  [T][in_dim/16]   per-16 sums of q   (ActQ8 / ActQ8KRow .sums, vecdot.rs:66-75, 3020-3026)
+//   bsum i16  [T][in_dim/32]   per-32 sums of q   (ActQ8K .bsum, vecdot.rs:1849-1852)
+struct OgmActDev {
+  int8_t *q;
+  float *d;
+  int32_t *sums;
+  int16_t *bsum;
+};
+
+// mode 0: one scale per 32 (vecdot.rs:95-126); mode 1: one per 256 (vecdot.rs:3030-3053).
+hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,
+                               OgmActDev act, hipStream_t stream);
+
+struct OgmGemvArgs {
+  uint32_t ggml_type;
+  const uint8_t *wt;  // tile-planar weights
+  uint32_t in_dim, out_dim;
+  OgmActDev act;      // matching the type's activation mode
+  uint32_t n_tokens;  // tokens in this launch (<= ogm_gemv_max_tokens)
+  float *y;           // [n_tokens][out_dim], row stride out_dim
+  int gemm_order;     // 0: GEMV float order (cpu.rs T==1 / matmul_decode), 1: GEMM order (T>1)
+  uint32_t rows_per_wg;  // 0 = heuristic
+  int32_t *dump_isum;    // optional [n_tokens][out_dim][blocks/row]
+  int32_t *dump_imin;    // optional, Q4_K only
+};
+
+// Largest token count one launch can take for this shape (LDS budget), at least 1.
+uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order,
+                             uint32_t rows_per_wg);
+hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name);
+
+hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hipStream_t stream);

@@ -1,0 +1,549 @@
+// gfx950 kernels of the quantized matmul path: the fused activation quantizer and the
+// decode GEMV for Q8_0 / Q4_K / Q6_K weights in the tile-planar layout (ogm_layout.h).
+//
+// Arithmetic contract (engine/vecdot.rs of orangu-server):
+//   * the quantizer reproduces quantize_act / quantize_act_k_row bit for bit;
+//   * every per-block integer sum (isum, imin) is formed exactly, in i32;
+//   * the f32 stage evaluates the reference's expression per block and then adds the block
+//     terms in ascending block order with one accumulator, so the f32 result has the
+//     reference's bits as well.  Build with -ffp-contract=off: an FMA would change them.
+//
+// Work mapping: one lane owns one block ("unit") for the whole kernel.  A workgroup owns a run
+// of output rows, i.e. a contiguous run of units; lane l of a wave reads piece p of its unit at
+// tile*tile_bytes + p*1024 + l*16, so each load instruction of a wave covers one contiguous
+// kilobyte.  The int8 activations sit in LDS, laid out so that lanes owning neighbouring
+// blocks read neighbouring 16-byte chunks (no bank conflicts).  Each lane leaves its block's
+// f32 term in LDS; one lane per (row, token) then adds the row's terms in order.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "ogm_kernels.h"
+#include "ogm_layout.h"
+
+#define OGM_WG 256
+
+// ------------------------------------------------------------------------------------------
+// small helpers
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
+  // Block scales are IEEE binary16 (quant.rs:511-528); the hardware conversion is exact for every
+  // finite value, subnormal and infinity.
+  return __half2float(__ushort_as_half((unsigned short)bits16));
+}
+
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int acc) {
+  // v_dot4_i32_i8: four signed int8 products added to acc, exact (dot16/dot32 of vecdot.rs:471-707)
+  return __builtin_amdgcn_sdot4((int)a, (int)b, acc, false);
+}
+
+__device__ __forceinline__ int byte_of(uint32_t w, int i) { return (int)((w >> (8 * i)) & 0xFFu); }
+__device__ __forceinline__ int sbyte_of(uint32_t w, int i) { return (int)(int8_t)((w >> (8 * i)) & 0xFFu); }
+__device__ __forceinline__ int lo16(uint32_t w) { return (int)(int16_t)(w & 0xFFFFu); }
+__device__ __forceinline__ int hi16(uint32_t w) { return ((int)w) >> 16; }
+
+// ------------------------------------------------------------------------------------------
+// activation quantizer
+//
+// One wave per 256 activations of one token; lane l holds elements 4l..4l+3.
+//   amax  = fold(0, max(m, |v|)) ignoring NaN          (vecdot.rs:103, 3037)
+//   scale = amax / 127 ; inv = scale > 0 ? 1/scale : 0   (vecdot.rs:106-107)
+//   q     = clamp(round_half_away(v * inv), -127, 127), NaN -> 0   (vecdot.rs:117)
+// GROUP = 32: scale per 32 (quantize_act); GROUP = 256: per 256 (quantize_act_k_row).
+
+__device__ __forceinline__ float nan_blind_max(float m, float a) { return a > m ? a : m; }
+
+__device__ __forceinline__ int quantize_one(float v, float inv) {
+  float r = roundf(v * inv);
+  if (r != r) r = 0.0f;
+  r = fminf(fmaxf(r, -127.0f), 127.0f);
+  return (int)r;
+}
+
+template <int GROUP>
+__global__ __launch_bounds__(64) void ogm_quantize_kernel(const float *__restrict__ x,
+                                                          uint32_t in_dim, OgmActDev act) {
+  const uint32_t lane = threadIdx.x;
+  const uint32_t t = blockIdx.y;
+  const uint32_t e0 = blockIdx.x * 256u + lane * 4u;
+  const bool active = e0 < in_dim;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (active) v = *(const float4 *)(x + (size_t)t * in_dim + e0);
+
+  float amax = 0.0f;
+  amax = nan_blind_max(amax, fabsf(v.x));
+  amax = nan_blind_max(amax, fabsf(v.y));
+  amax = nan_blind_max(amax, fabsf(v.z));
+  amax = nan_blind_max(amax, fabsf(v.w));
+#pragma unroll
+  for (int m = 1; m < GROUP / 4; m <<= 1) amax = nan_blind_max(amax, __shfl_xor(amax, m, 64));
+
+  const float scale = amax / 127.0f;
+  const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+  const int q0 = quantize_one(v.x, inv), q1 = quantize_one(v.y, inv);
+  const int q2 = quantize_one(v.z, inv), q3 = quantize_one(v.w, inv);
+  const uint32_t packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) |
+                          ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
+  int s = q0 + q1 + q2 + q3;
+  s += __shfl_xor(s, 1, 64);
+  s += __shfl_xor(s, 2, 64);
+  const int s32 = s + __shfl_xor(s, 4, 64);
+  if (active) {
+    *(uint32_t *)(act.q + (size_t)t * in_dim + e0) = packed;
+    if ((lane & 3u) == 0) act.sums[(size_t)t * (in_dim / 16) + e0 / 16] = s;
+    if ((lane & 7u) == 0) act.bsum[(size_t)t * (in_dim / 32) + e0 / 32] = (int16_t)s32;
+    if ((lane & (GROUP / 4 - 1)) == 0) act.d[(size_t)t * (in_dim / GROUP) + e0 / GROUP] = scale;
+  }
+}
+
+hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,
+                               OgmActDev act, hipStream_t stream) {
+  if (n_tokens == 0) return hipSuccess;
+  dim3 grid((in_dim + 255) / 256, n_tokens);
+  if (mode == 0)
+    hipLaunchKernelGGL(ogm_quantize_kernel<32>, grid, dim3(64), 0, stream, x, in_dim, act);
+  else
+    hipLaunchKernelGGL(ogm_quantize_kernel<256>, grid, dim3(64), 0, stream, x, in_dim, act);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// formats: how one lane loads its block and forms the block's integer sums
+
+// LDS views of one token's activations, as the formats read them.
+struct ActLds {
+  const uint4 *xq;   // 16-byte chunks of q; chunk c of block `col` at [c * upr + col]
+  const float *d;    // activation scale per scale group
+  const uint4 *aux;  // per-block integer side sums (AUX16 chunks per block, [k * upr + col])
+  uint32_t upr;      // blocks per row
+};
+
+// Q4_K: d:f16 | dmin:f16 | scales:u8[12] | qs:u8[128]            (quant.rs:664-697)
+struct FmtQ4K {
+  static constexpr uint32_t TYPE = OGM_Q4_K;
+  static constexpr int PIECES = 9, TILE_BYTES = 64 * 144, ELEMS = 256;
+  static constexpr int XPIECES = 16;   // 16-byte activation chunks per block
+  static constexpr int AUX16 = 1;      // bsum: 8 x i16 per block
+  static constexpr int ACT_GROUP = 256;
+  static constexpr bool HAS_MIN = true;
+  struct Regs {
+    uint4 p[PIECES];
+  };
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, uint32_t u) {
+    const uint8_t *base = wt + (size_t)(u >> 6) * TILE_BYTES + (u & 63u) * 16u;
+#pragma unroll
+    for (int i = 0; i < PIECES; i++) r.p[i] = *(const uint4 *)(base + i * 1024);
+  }
+  // isum = sum_j sc_j * dot32(nibbles_j, x_j), imin = sum_j m_j * bsum_j     (vecdot.rs:3152-3178)
+  __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
+                                              int &isum, int &imin) {
+    // get_scale_min_k4 (quant.rs:653-662) for all eight sub-blocks at once, four bytes a word
+    const uint32_t w0 = r.p[0].y, w1 = r.p[0].z, w2 = r.p[0].w;
+    const uint32_t sca = w0 & 0x3F3F3F3Fu;                                   // sc 0..3
+    const uint32_t mna = w1 & 0x3F3F3F3Fu;                                   // m  0..3
+    const uint32_t scb = (w2 & 0x0F0F0F0Fu) | ((w0 >> 2) & 0x30303030u);     // sc 4..7
+    const uint32_t mnb = ((w2 >> 4) & 0x0F0F0F0Fu) | ((w1 >> 2) & 0x30303030u);  // m 4..7
+    isum = 0;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      // qs[32g .. 32g+32): low nibbles are sub-block 2g, high nibbles sub-block 2g+1
+      int dlo = 0, dhi = 0;
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const uint4 w = r.p[1 + 2 * g + h];
+        const uint4 xa = a.xq[(4 * g + h) * a.upr + col];      // elements 64g + 16h ..
+        const uint4 xb = a.xq[(4 * g + 2 + h) * a.upr + col];  // elements 64g + 32 + 16h ..
+        dlo = dot4(w.x & 0x0F0F0F0Fu, xa.x, dlo);
+        dlo = dot4(w.y & 0x0F0F0F0Fu, xa.y, dlo);
+        dlo = dot4(w.z & 0x0F0F0F0Fu, xa.z, dlo);
+        dlo = dot4(w.w & 0x0F0F0F0Fu, xa.w, dlo);
+        dhi = dot4((w.x >> 4) & 0x0F0F0F0Fu, xb.x, dhi);
+        dhi = dot4((w.y >> 4) & 0x0F0F0F0Fu, xb.y, dhi);
+        dhi = dot4((w.z >> 4) & 0x0F0F0F0Fu, xb.z, dhi);
+        dhi = dot4((w.w >> 4) & 0x0F0F0F0Fu, xb.w, dhi);
+      }
+      const int j = 2 * g;
+      const int sc_lo = j < 4 ? byte_of(sca, j) : byte_of(scb, j - 4);
+      const int sc_hi = j + 1 < 4 ? byte_of(sca, j + 1) : byte_of(scb, j - 3);
+      isum += sc_lo * dlo + sc_hi * dhi;
+    }
+    const uint4 b = a.aux[col];  // bsum_0..7 as i16
+    imin = byte_of(mna, 0) * lo16(b.x) + byte_of(mna, 1) * hi16(b.x) +
+           byte_of(mna, 2) * lo16(b.y) + byte_of(mna, 3) * hi16(b.y) +
+           byte_of(mnb, 0) * lo16(b.z) + byte_of(mnb, 1) * hi16(b.z) +
+           byte_of(mnb, 2) * lo16(b.w) + byte_of(mnb, 3) * hi16(b.w);
+  }
+  // GEMV: total += act.d[s] * (d*isum - dmin*imin)                           (vecdot.rs:3175)
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int imin) {
+    const float d = f16_bits_to_f32(r.p[0].x & 0xFFFFu), dmin = f16_bits_to_f32(r.p[0].x >> 16);
+    return ad * (d * (float)isum - dmin * (float)imin);
+  }
+  // GEMM: acc -= (ad*dmin)*imin [all blocks first]; acc += ad*(d*isum)       (vecdot.rs:2229-2303)
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int imin,
+                                                   float &tmin, float &tdot) {
+    const float d = f16_bits_to_f32(r.p[0].x & 0xFFFFu), dmin = f16_bits_to_f32(r.p[0].x >> 16);
+    tmin = ad * dmin * (float)imin;
+    tdot = ad * (d * (float)isum);
+  }
+};
+
+// Q6_K: ql:u8[128] | qh:u8[64] | scales:i8[16] | d:f16                      (quant.rs:744-787)
+struct FmtQ6K {
+  static constexpr uint32_t TYPE = OGM_Q6_K;
+  static constexpr int PIECES = 13, TILE_BYTES = 64 * 210, ELEMS = 256;
+  static constexpr int XPIECES = 16;
+  static constexpr int AUX16 = 2;  // per-16 sums of q: 16 x i16 per block
+  static constexpr int ACT_GROUP = 256;
+  static constexpr bool HAS_MIN = false;
+  struct Regs {
+    uint4 p[PIECES];
+    uint32_t d16;
+  };
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, uint32_t u) {
+    const uint8_t *tile = wt + (size_t)(u >> 6) * TILE_BYTES;
+    const uint8_t *base = tile + (u & 63u) * 16u;
+#pragma unroll
+    for (int i = 0; i < PIECES; i++) r.p[i] = *(const uint4 *)(base + i * 1024);
+    r.d16 = *(const uint16_t *)(tile + PIECES * 1024 + (u & 63u) * 2u);
+  }
+  __device__ static __forceinline__ int run_dot(uint4 ql, uint4 qh, uint4 x, int r) {
+    // 6-bit value = nibble | (two bits of qh) << 4, still carrying the +32 bias (0..63)
+    const uint32_t m4 = 0x0F0F0F0Fu, m2 = 0x30303030u;
+    uint32_t v0, v1, v2, v3;
+    if (r < 2) {
+      v0 = ql.x & m4; v1 = ql.y & m4; v2 = ql.z & m4; v3 = ql.w & m4;
+    } else {
+      v0 = (ql.x >> 4) & m4; v1 = (ql.y >> 4) & m4; v2 = (ql.z >> 4) & m4; v3 = (ql.w >> 4) & m4;
+    }
+    // ((qh >> 2r) & 3) << 4
+    if (r == 0) { v0 |= (qh.x << 4) & m2; v1 |= (qh.y << 4) & m2; v2 |= (qh.z << 4) & m2; v3 |= (qh.w << 4) & m2; }
+    if (r == 1) { v0 |= (qh.x << 2) & m2; v1 |= (qh.y << 2) & m2; v2 |= (qh.z << 2) & m2; v3 |= (qh.w << 2) & m2; }
+    if (r == 2) { v0 |= qh.x & m2; v1 |= qh.y & m2; v2 |= qh.z & m2; v3 |= qh.w & m2; }
+    if (r == 3) { v0 |= (qh.x >> 2) & m2; v1 |= (qh.y >> 2) & m2; v2 |= (qh.z >> 2) & m2; v3 |= (qh.w >> 2) & m2; }
+    int acc = 0;
+    acc = dot4(v0, x.x, acc);
+    acc = dot4(v1, x.y, acc);
+    acc = dot4(v2, x.z, acc);
+    acc = dot4(v3, x.w, acc);
+    return acc;
+  }
+  // isum = sum over 16 groups of sc_g * dot16(q_g - 32, x_g)                (vecdot.rs:3215-3241)
+  // with dot16(q - 32, x) = dot16(q, x) - 32 * sum16(x), exact in integers.
+  __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
+                                              int &isum, int &imin) {
+    const uint4 s_lo = a.aux[col], s_hi = a.aux[a.upr + col];  // sum16 of groups 0..7, 8..15
+    const uint32_t sw[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+    const uint32_t scw[4] = {r.p[12].x, r.p[12].y, r.p[12].z, r.p[12].w};
+    isum = 0;
+    imin = 0;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+      for (int rr = 0; rr < 4; rr++) {
+        const int R = 4 * h + rr;  // run of 32 elements: 128h + 32rr ..
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+          const int g = 2 * R + k;  // group of 16
+          const uint4 ql = r.p[4 * h + 2 * (rr & 1) + k];
+          const uint4 qh = r.p[8 + 2 * h + k];
+          const uint4 x = a.xq[g * a.upr + col];
+          const int dot = run_dot(ql, qh, x, rr);
+          const int s16 = (g & 1) ? hi16(sw[g >> 1]) : lo16(sw[g >> 1]);
+          isum += sbyte_of(scw[g >> 2], g & 3) * (dot - 32 * s16);
+        }
+      }
+    }
+  }
+  // GEMV: total += act.d[s] * d * isum                                       (vecdot.rs:3238)
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int) {
+    return ad * f16_bits_to_f32(r.d16) * (float)isum;
+  }
+  // GEMM: acc += ad * (d * isum)                                              (vecdot.rs:2389-2390)
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int,
+                                                   float &tmin, float &tdot) {
+    tmin = 0.0f;
+    tdot = ad * (f16_bits_to_f32(r.d16) * (float)isum);
+  }
+};
+
+// Q8_0: d:f16 | qs:i8[32]                                                     (quant.rs:638-649)
+struct FmtQ80 {
+  static constexpr uint32_t TYPE = OGM_Q8_0;
+  static constexpr int PIECES = 2, TILE_BYTES = 64 * 34, ELEMS = 32;
+  static constexpr int XPIECES = 2;
+  static constexpr int AUX16 = 0;
+  static constexpr int ACT_GROUP = 32;
+  static constexpr bool HAS_MIN = false;
+  struct Regs {
+    uint4 p[PIECES];
+    uint32_t d16;
+  };
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, uint32_t u) {
+    const uint8_t *tile = wt + (size_t)(u >> 6) * TILE_BYTES;
+    const uint8_t *base = tile + (u & 63u) * 16u;
+    r.p[0] = *(const uint4 *)(base);
+    r.p[1] = *(const uint4 *)(base + 1024);
+    r.d16 = *(const uint16_t *)(tile + PIECES * 1024 + (u & 63u) * 2u);
+  }
+  __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
+                                              int &isum, int &imin) {
+    const uint4 x0 = a.xq[col], x1 = a.xq[a.upr + col];
+    int acc = 0;
+    acc = dot4(r.p[0].x, x0.x, acc);
+    acc = dot4(r.p[0].y, x0.y, acc);
+    acc = dot4(r.p[0].z, x0.z, acc);
+    acc = dot4(r.p[0].w, x0.w, acc);
+    acc = dot4(r.p[1].x, x1.x, acc);
+    acc = dot4(r.p[1].y, x1.y, acc);
+    acc = dot4(r.p[1].z, x1.z, acc);
+    acc = dot4(r.p[1].w, x1.w, acc);
+    isum = acc;
+    imin = 0;
+  }
+  // GEMV: total += dw * act.d[b] * isum (vecdot.rs:2835); the flat GEMM's ad*dw*isum
+  // (vecdot.rs:2623) is the same product, so one form serves both orders.
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int) {
+    return f16_bits_to_f32(r.d16) * ad * (float)isum;
+  }
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int,
+                                                   float &tmin, float &tdot) {
+    tmin = 0.0f;
+    tdot = ad * f16_bits_to_f32(r.d16) * (float)isum;
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// GEMV kernel
+
+struct GemvParams {
+  const uint8_t *wt;
+  OgmActDev act;
+  float *y;
+  int32_t *dump_isum, *dump_imin;
+  uint32_t in_dim, out_dim, upr;  // upr = blocks per row
+  uint32_t n_tokens, rows_per_wg;
+};
+
+template <class F, bool GEMM_ORDER>
+__host__ __device__ constexpr int n_term_arrays() {
+  return (GEMM_ORDER && F::HAS_MIN) ? 2 : 1;
+}
+
+// Dynamic LDS bytes of one workgroup.
+template <class F, bool GEMM_ORDER>
+static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rows_per_wg) {
+  const size_t upr = in_dim / F::ELEMS;
+  const size_t n_scale = in_dim / F::ACT_GROUP;
+  size_t b = (size_t)n_tokens * in_dim;                     // xq
+  b += (size_t)n_tokens * upr * F::AUX16 * 16;              // aux
+  b += (size_t)n_tokens * n_scale * 4;                      // act.d
+  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * rows_per_wg * upr * 4;  // terms
+  return b;
+}
+
+template <class F, bool GEMM_ORDER, bool DUMP>
+__global__ __launch_bounds__(OGM_WG) void ogm_gemv_kernel(GemvParams p) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t tid = threadIdx.x;
+  const uint32_t T = p.n_tokens;
+  const uint32_t upr = p.upr;
+  const uint32_t xch = p.in_dim / 16;              // 16-byte chunks of q per token
+  const uint32_t n_scale = p.in_dim / F::ACT_GROUP;
+  const uint32_t r0 = blockIdx.x * p.rows_per_wg;
+  const uint32_t rows = min(p.rows_per_wg, p.out_dim - r0);
+  const uint32_t u0 = r0 * upr, uw = rows * upr;   // this workgroup's units: [u0, u0 + uw)
+  constexpr int NT = n_term_arrays<F, GEMM_ORDER>();
+
+  uint4 *l_xq = (uint4 *)lds;                                   // [T][xch]
+  uint4 *l_aux = l_xq + (size_t)T * xch;                        // [T][AUX16][upr]
+  float *l_d = (float *)(l_aux + (size_t)T * upr * F::AUX16);   // [T][n_scale]
+  float *l_term = l_d + (size_t)T * n_scale;                    // [NT][T][rows_per_wg * upr]
+  const uint32_t term_stride = p.rows_per_wg * upr;
+
+  // The first block's weight loads go out before anything else: they are the long pole.
+  typename F::Regs cur;
+  uint32_t u = tid;
+  bool have = u < uw;
+  if (have) F::load(cur, p.wt, u0 + u);
+
+  // Stage the activations: q permuted so that chunk c of block `col` lands at [c*upr + col].
+  for (uint32_t i = tid; i < T * xch; i += OGM_WG) {
+    const uint32_t t = i / xch, ch = i - t * xch;
+    const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
+    l_xq[(size_t)t * xch + c * upr + col] = ((const uint4 *)(p.act.q + (size_t)t * p.in_dim))[ch];
+  }
+  if (F::AUX16 == 1) {  // Q4_K: bsum, 8 x i16 per super-block, already in that form
+    for (uint32_t i = tid; i < T * upr; i += OGM_WG)
+      l_aux[i] = ((const uint4 *)p.act.bsum)[i];
+  } else if (F::AUX16 == 2) {  // Q6_K: per-16 sums as i16, groups 0..7 then 8..15
+    for (uint32_t i = tid; i < T * upr * 2; i += OGM_WG) {
+      const uint32_t t = i / (upr * 2), rem = i - t * upr * 2;
+      const uint32_t col = rem >> 1, k = rem & 1u;
+      const int4 *src = (const int4 *)(p.act.sums + ((size_t)t * upr + col) * 16 + k * 8);
+      const int4 a = src[0], b = src[1];
+      uint4 o;
+      o.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
+      o.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
+      o.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
+      o.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
+      l_aux[(size_t)t * upr * 2 + k * upr + col] = o;
+    }
+  }
+  for (uint32_t i = tid; i < T * n_scale; i += OGM_WG) l_d[i] = p.act.d[i];
+  __syncthreads();
+
+  while (have) {
+    const uint32_t un = u + OGM_WG;
+    const bool have_next = un < uw;
+    typename F::Regs nxt;
+    if (have_next) F::load(nxt, p.wt, u0 + un);
+
+    const uint32_t row = u / upr, col = u - row * upr;
+    for (uint32_t t = 0; t < T; t++) {
+      ActLds a;
+      a.xq = l_xq + (size_t)t * xch;
+      a.aux = l_aux + (size_t)t * upr * F::AUX16;
+      a.d = l_d + (size_t)t * n_scale;
+      a.upr = upr;
+      int isum, imin;
+      F::sums(cur, a, col, isum, imin);
+      const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
+      if (GEMM_ORDER) {
+        float tmin, tdot;
+        F::term_gemm(cur, ad, isum, imin, tmin, tdot);
+        l_term[(size_t)t * term_stride + u] = tdot;
+        if (NT == 2) l_term[(size_t)(T + t) * term_stride + u] = tmin;
+      } else {
+        l_term[(size_t)t * term_stride + u] = F::term_gemv(cur, ad, isum, imin);
+      }
+      if (DUMP) {
+        const size_t o = ((size_t)t * p.out_dim + r0) * upr + u;
+        if (p.dump_isum) p.dump_isum[o] = isum;
+        if (F::HAS_MIN && p.dump_imin) p.dump_imin[o] = imin;
+      }
+    }
+    if (have_next) cur = nxt;
+    u = un;
+    have = have_next;
+  }
+  __syncthreads();
+
+  // One lane per (row, token): the row's block terms in ascending order, one accumulator.
+  for (uint32_t i = tid; i < rows * T; i += OGM_WG) {
+    const uint32_t t = i / rows, row = i - t * rows;
+    const float *td = l_term + (size_t)t * term_stride + row * upr;
+    float acc = 0.0f;
+    if (NT == 2) {
+      const float *tm = l_term + (size_t)(T + t) * term_stride + row * upr;
+      for (uint32_t s = 0; s < upr; s++) acc -= tm[s];
+    }
+    for (uint32_t s = 0; s < upr; s++) acc += td[s];
+    p.y[(size_t)t * p.out_dim + r0 + row] = acc;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// host side of the launch
+
+static const size_t OGM_LDS_BUDGET = 64 * 1024;
+
+static uint32_t default_rows_per_wg(uint32_t upr, uint32_t out_dim) {
+  // About one block per lane and per pass; at least one row.
+  uint32_t r = (OGM_WG + upr - 1) / upr;
+  if (r == 0) r = 1;
+  if (r > out_dim) r = out_dim;
+  return r;
+}
+
+template <class F, bool GEMM_ORDER>
+static uint32_t max_tokens_t(uint32_t in_dim, uint32_t rows_per_wg) {
+  uint32_t t = 8;
+  while (t > 1 && gemv_lds_bytes<F, GEMM_ORDER>(in_dim, t, rows_per_wg) > OGM_LDS_BUDGET) t--;
+  return t;
+}
+
+template <class F>
+static uint32_t resolve_rows(uint32_t in_dim, uint32_t out_dim, uint32_t rows_per_wg) {
+  const uint32_t upr = in_dim / F::ELEMS;
+  uint32_t r = rows_per_wg ? rows_per_wg : default_rows_per_wg(upr, out_dim);
+  if (r > out_dim) r = out_dim;
+  // one token must fit
+  while (r > 1 && gemv_lds_bytes<F, true>(in_dim, 1, r) > OGM_LDS_BUDGET) r--;
+  return r;
+}
+
+uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order,
+                             uint32_t rows_per_wg) {
+  switch (ggml_type) {
+    case OGM_Q4_K: {
+      uint32_t r = resolve_rows<FmtQ4K>(in_dim, 0xFFFFFFFFu, rows_per_wg);
+      return gemm_order ? max_tokens_t<FmtQ4K, true>(in_dim, r) : max_tokens_t<FmtQ4K, false>(in_dim, r);
+    }
+    case OGM_Q6_K: {
+      uint32_t r = resolve_rows<FmtQ6K>(in_dim, 0xFFFFFFFFu, rows_per_wg);
+      return gemm_order ? max_tokens_t<FmtQ6K, true>(in_dim, r) : max_tokens_t<FmtQ6K, false>(in_dim, r);
+    }
+    case OGM_Q8_0: {
+      uint32_t r = resolve_rows<FmtQ80>(in_dim, 0xFFFFFFFFu, rows_per_wg);
+      return gemm_order ? max_tokens_t<FmtQ80, true>(in_dim, r) : max_tokens_t<FmtQ80, false>(in_dim, r);
+    }
+    default:
+      return 0;
+  }
+}
+
+template <class F, bool GEMM_ORDER>
+static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
+  GemvParams p;
+  p.wt = a.wt;
+  p.act = a.act;
+  p.y = a.y;
+  p.dump_isum = a.dump_isum;
+  p.dump_imin = a.dump_imin;
+  p.in_dim = a.in_dim;
+  p.out_dim = a.out_dim;
+  p.upr = a.in_dim / F::ELEMS;
+  p.n_tokens = a.n_tokens;
+  p.rows_per_wg = resolve_rows<F>(a.in_dim, a.out_dim, a.rows_per_wg);
+  const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, p.rows_per_wg);
+  if (lds > OGM_LDS_BUDGET) return hipErrorInvalidValue;
+  const uint32_t grid = (a.out_dim + p.rows_per_wg - 1) / p.rows_per_wg;
+  if (a.dump_isum || a.dump_imin)
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, GEMM_ORDER, true>), dim3(grid), dim3(OGM_WG), lds,
+                       stream, p);
+  else
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, GEMM_ORDER, false>), dim3(grid), dim3(OGM_WG), lds,
+                       stream, p);
+  return hipGetLastError();
+}
+
+hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name) {
+  if (a.n_tokens == 0 || a.out_dim == 0) return hipSuccess;
+  switch (a.ggml_type) {
+    case OGM_Q4_K:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ4K,gemm>" : "ogm_gemv_kernel<FmtQ4K,gemv>";
+      return a.gemm_order ? launch_t<FmtQ4K, true>(a, stream) : launch_t<FmtQ4K, false>(a, stream);
+    case OGM_Q6_K:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ6K,gemm>" : "ogm_gemv_kernel<FmtQ6K,gemv>";
+      return a.gemm_order ? launch_t<FmtQ6K, true>(a, stream) : launch_t<FmtQ6K, false>(a, stream);
+    case OGM_Q8_0:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ80,gemm>" : "ogm_gemv_kernel<FmtQ80,gemv>";
+      return a.gemm_order ? launch_t<FmtQ80, true>(a, stream) : launch_t<FmtQ80, false>(a, stream);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// f16 -> f32 as the kernels do it, exposed for a parity check
+
+__global__ void ogm_f16_kernel(const uint16_t *bits, size_t n, float *out) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = f16_bits_to_f32(bits[i]);
+}
+
+hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(ogm_f16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, bits,
+                     n, out);
+  return hipGetLastError();
+}
