@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized matmul hot path on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): batch-1 decode GEMVs of a
+Llama-3-8B feed-forward block in Q4_K -- gate and up 4096 -> 14336 and down 14336 -> 4096 --
+on seeded synthetic weights and N(0,1) activations.  One step is one pass over that block: the
+activation quantizer plus the GEMV for each of the three matrices, through the library's C ABI
+with inputs and outputs resident in HBM.  Steps rotate over enough distinct weight copies that
+every pass streams from HBM rather than from the last-level cache.
+
+Prints ONE JSON line: whole-step throughput in algorithmic GB/s, a roofline object for the
+dominant kernel (the Q4_K GEMV at 4096 -> 14336, timed with HIP events over back-to-back
+launches) and the CPU path (the C oracle, all host cores) timed on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import numpy as np  # noqa: E402
+
+Q4_K = 12
+HIDDEN, FFN = 4096, 14336
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def gemv_bytes(in_dim: int, out_dim: int, t: int = 1) -> int:
+    """Algorithmic bytes of one Q4_K GEMV: raw GGUF rows + f32 x + f32 y."""
+    return out_dim * (in_dim // 256 * 144) + 4 * in_dim * t + 4 * out_dim * t
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--copies", type=int, default=12,
+                    help="distinct copies of the three matrices (12 x 99 MB = 1.2 GB > 256 MB cache)")
+    ap.add_argument("--roofline-launches", type=int, default=600)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
+    ap.add_argument("--wg-waves", type=int, default=0, help="waves per workgroup override (0 = heuristic)")
+    ap.add_argument("--max-waves", type=int, default=0, help="cap on waves per launch (0 = heuristic)")
+    ap.add_argument("--only-roofline", action="store_true",
+                    help="run only the dominant-kernel leg (for rocprofv3 --kernel-trace --stats)")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only; --gpus N with N > 1 is not supported "
+              "(the path has no collectives; see DESIGN.md for how it would shard).", file=sys.stderr)
+        return 2
+
+    import helpers
+    from orangu_amd import Mi355xBackend
+    from orangu_amd import hiprt
+
+    be = Mi355xBackend()  # raises without the HIP library or a gfx950 device
+    if args.wg_waves:
+        be.set_tuning("gemv_wg_waves", args.wg_waves)
+    if args.max_waves:
+        be.set_tuning("gemv_max_waves", args.max_waves)
+    stream = hiprt.Stream()
+
+    # ---- synthetic inputs -------------------------------------------------------------------
+    seed = 20240607
+    shapes = {"gate": (HIDDEN, FFN), "up": (HIDDEN, FFN), "down": (FFN, HIDDEN)}
+    raw = {k: helpers.synth_weights(Q4_K, i, o, seed + n) for n, (k, (i, o)) in enumerate(shapes.items())}
+    x_h = helpers.synth_x(1, HIDDEN, seed)[0]
+    h_h = helpers.synth_x(1, FFN, seed + 1)[0]
+    copies = max(1, args.copies)
+    handles = {k: [be.upload_raw(raw[k], Q4_K, *shapes[k]) for _ in range(copies)] for k in shapes}
+    x_d = hiprt.DeviceBuffer.from_numpy(x_h)
+    h_d = hiprt.DeviceBuffer.from_numpy(h_h)
+    y_gate, y_up, y_down = (hiprt.DeviceBuffer(4 * FFN), hiprt.DeviceBuffer(4 * FFN),
+                            hiprt.DeviceBuffer(4 * HIDDEN))
+
+    def step(i: int):
+        c = i % copies
+        be.matmul_dev(handles["gate"][c], x_d.ptr, 1, y_gate.ptr, False, stream.ptr)
+        be.matmul_dev(handles["up"][c], x_d.ptr, 1, y_up.ptr, False, stream.ptr)
+        be.matmul_dev(handles["down"][c], h_d.ptr, 1, y_down.ptr, False, stream.ptr)
+
+    step_bytes = 2 * gemv_bytes(HIDDEN, FFN) + gemv_bytes(FFN, HIDDEN)
+    result = {}
+
+    if not args.only_roofline:
+        for i in range(args.warmup):
+            step(i)
+        stream.synchronize()
+        hiprt.device_synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(args.warmup + i)
+        stream.synchronize()
+        hiprt.device_synchronize()
+        t1 = time.perf_counter()
+        ms_per_step = (t1 - t0) * 1e3 / args.steps
+        result["ms_per_step"] = ms_per_step
+        result["value"] = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- dominant kernel: Q4_K GEMV 4096 -> 14336, back-to-back, HIP events on its stream -----
+    mats = handles["gate"] + handles["up"]
+    be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr)
+    for i in range(50):
+        be.matmul_act_dev(mats[i % len(mats)], 1, y_gate.ptr, False, stream.ptr)
+    stream.synchronize()
+    e0, e1 = hiprt.Event(), hiprt.Event()
+    n_launch = args.roofline_launches
+    e0.record(stream)
+    for i in range(n_launch):
+        be.matmul_act_dev(mats[i % len(mats)], 1, y_gate.ptr, False, stream.ptr)
+    e1.record(stream)
+    e1.synchronize()
+    us_per_launch = e0.elapsed_ms(e1) * 1e3 / n_launch
+    kbytes = gemv_bytes(HIDDEN, FFN)
+    achieved = kbytes / (us_per_launch * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": be.last_kernel(), "us_per_launch": round(us_per_launch, 3),
+                "bytes_per_launch": kbytes, "launches": n_launch}
+
+    # ---- parity of what was just timed + CPU baseline (the oracle, all host cores) -------------
+    cpu = None
+    parity = None
+    if not args.only_roofline and args.cpu_seconds > 0:
+        import oracle
+        step(0)
+        stream.synchronize()
+        got = {"gate": y_gate.to_numpy(np.float32, FFN), "up": y_up.to_numpy(np.float32, FFN),
+               "down": y_down.to_numpy(np.float32, HIDDEN)}
+        xin = {"gate": x_h, "up": x_h, "down": h_h}
+        cores = oracle.host_threads()
+
+        def cpu_step():
+            return {k: oracle.matmul(Q4_K, raw[k], shapes[k][0], shapes[k][1], xin[k], 1, threads=0)[0]
+                    for k in shapes}
+
+        want = cpu_step()  # warm-up and the parity reference
+        ok = all(np.all(np.abs(got[k].astype(np.float64) - want[k]) <= 1e-3 * np.abs(want[k]) + 1e-5)
+                 for k in shapes)
+        bits = all(np.array_equal(got[k].view(np.uint32), want[k].view(np.uint32)) for k in shapes)
+        parity = "bit-exact" if bits else ("within 1e-3/1e-5" if ok else "FAILED")
+        times = []
+        t_end = time.perf_counter() + args.cpu_seconds
+        while time.perf_counter() < t_end or len(times) < 5:
+            a = time.perf_counter()
+            cpu_step()
+            times.append(time.perf_counter() - a)
+        best, med = min(times), sorted(times)[len(times) // 2]
+        # one thread, a few repetitions of one GEMV, scaled to the step
+        t1s = []
+        for _ in range(3):
+            a = time.perf_counter()
+            oracle.matmul(Q4_K, raw["gate"], HIDDEN, FFN, x_h, 1, threads=1)
+            t1s.append(time.perf_counter() - a)
+        cpu = {"value": round(step_bytes / med / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+               "sample": f"{len(times)} repetitions of the same 3-GEMV step ({step_bytes} B each), "
+                         f"median; best {step_bytes / best / 1e9:.2f} GB/s; "
+                         f"1 thread {gemv_bytes(HIDDEN, FFN) / min(t1s) / 1e9:.2f} GB/s; "
+                         f"integer dots on {oracle.isa_name()}"}
+        if parity == "FAILED":
+            print("bench.py: GPU output differs from the CPU oracle beyond 1e-3/1e-5", file=sys.stderr)
+
+    out = {
+        "metric": "Q4_K GEMV HBM GB/s (batch-1 decode, Llama-3-8B FFN shapes)",
+        "value": round(result.get("value", achieved), 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps if not args.only_roofline else n_launch,
+        "warmup": args.warmup,
+        "ms_per_step": round(result.get("ms_per_step", us_per_launch * 1e-3), 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8 dot / i32 block sums / f32 combine",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: Q4_K decode GEMV batch 1, gate+up 4096->14336 and down "
+                               "14336->4096; step = 3 x (activation quantize + GEMV)",
+                   "algorithmic_bytes_per_step": step_bytes, "weight_copies": copies,
+                   "frac_of_hbm_peak": round(result.get("value", achieved) / HBM_PEAK_GBS, 4),
+                   "parity_vs_cpu": parity, "device": be.device_name()},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+    be.close()
+    return 0 if parity != "FAILED" else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -136,6 +136,16 @@ int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, int decode,
 int ogm_matmul_dev(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
                    float *y_dev, int decode, void *stream);
 
+/* The same path in two steps, so that ops reading one input (a layer's q/k/v, or gate/up:
+ * engine/arch/mod.rs:1082-1096) quantize it once.  ogm_act_quantize_dev quantizes x_dev
+ * ([n_tokens][in_dim]) into the context's activation buffer with the mode `ggml_type` needs
+ * (backend/cpu.rs:100-116); ogm_matmul_act_dev then multiplies any weight of the same in_dim and
+ * activation mode by it.  Values equal ogm_matmul_dev's: the quantizer is a pure function of x. */
+int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev, uint32_t in_dim,
+                         uint32_t n_tokens, void *stream);
+int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, float *y_dev,
+                       int decode, void *stream);
+
 /* ---- the integer stage, exposed for parity checks ------------------------------------------- */
 
 /* The fused activation quantizer on its own.  mode OGM_ACT_PER_32: d has n/32 entries
@@ -158,7 +168,8 @@ int ogm_f16_to_f32(ogm_ctx *ctx, const uint16_t *bits, size_t n, float *out);
 /* ---- tuning / introspection ------------------------------------------------------------------ */
 
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.
- * key: "gemv_rows" (output rows per workgroup; 0 = heuristic). */
+ * keys: "gemv_wg_waves" (waves per workgroup, 1..16), "gemv_max_waves" (cap on the waves of one
+ * launch; more row segments than that are looped over); 0 = heuristic. */
 int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value);
 /* Name of the kernel the last matmul on this context launched (for profiles). */
 const char *ogm_last_kernel(ogm_ctx *ctx);

@@ -232,6 +232,25 @@ class Mi355xBackend:
         self._check(self._lib.ogm_matmul_dev(self._ctx, w_handle, x_ptr, n_tokens, y_ptr,
                                              int(decode), stream or None), "ogm_matmul_dev")
 
+    def act_quantize_dev(self, ggml_type: int, x_ptr: int, in_dim: int, n_tokens: int, stream: int = 0):
+        self._check(self._lib.ogm_act_quantize_dev(self._ctx, ggml_type, x_ptr, in_dim, n_tokens,
+                                                   stream or None), "ogm_act_quantize_dev")
+
+    def matmul_act_dev(self, w_handle: int, n_tokens: int, y_ptr: int, decode: bool = False,
+                       stream: int = 0):
+        self._check(self._lib.ogm_matmul_act_dev(self._ctx, w_handle, n_tokens, y_ptr, int(decode),
+                                                 stream or None), "ogm_matmul_act_dev")
+
+    def upload_raw(self, raw: np.ndarray, ggml_type: int, in_dim: int, out_dim: int) -> int:
+        """Uploads without a cache key: every call makes a new device copy."""
+        raw = np.ascontiguousarray(raw, np.uint8)
+        bb, be = BLOCK_LAYOUT[ggml_type]
+        handle = C.c_void_p()
+        rc = self._lib.ogm_weight_upload(self._ctx, ggml_type, raw.ctypes.data, in_dim // be * bb,
+                                         in_dim, out_dim, 0, 0, C.byref(handle))
+        self._check(rc, "ogm_weight_upload")
+        return handle.value
+
     def set_tuning(self, key: str, value: int):
         self._check(self._lib.ogm_set_tuning(self._ctx, key.encode(), value), "ogm_set_tuning")
 

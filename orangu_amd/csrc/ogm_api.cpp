@@ -43,8 +43,11 @@ struct ogm_ctx {
   // engine/backend/rocm.rs:352-376; a pool is what the Vulkan op_cache does instead)
   DevBuf x, y, q, d, sums, bsum, isum, imin;
   DevBuf hx, hy;  // pinned host staging
-  int tune_gemv_rows = 0;
+  int tune_wg_waves = 0, tune_max_waves = 0;
   const char *last_kernel = "";
+  // what the activation buffer currently holds (ogm_act_quantize_dev)
+  int act_mode = -1;
+  uint32_t act_in_dim = 0, act_tokens = 0;
 };
 
 static thread_local std::string g_init_err;
@@ -186,9 +189,14 @@ extern "C" int ogm_device_name(ogm_ctx *ctx, char *buf, size_t buf_len) {
 extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (!ctx || !key) return OGM_ERR_INVALID;
   std::lock_guard<std::mutex> lock(ctx->mu);
-  if (strcmp(key, "gemv_rows") == 0) {
-    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemv_rows must be >= 0");
-    ctx->tune_gemv_rows = value;
+  if (strcmp(key, "gemv_wg_waves") == 0) {
+    if (value < 0 || value > 16) return fail(ctx, OGM_ERR_INVALID, "gemv_wg_waves must be 0..16");
+    ctx->tune_wg_waves = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemv_max_waves") == 0) {
+    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemv_max_waves must be >= 0");
+    ctx->tune_max_waves = value;
     return OGM_OK;
   }
   return fail(ctx, OGM_ERR_INVALID, std::string("unknown tuning key ") + key);
@@ -299,21 +307,40 @@ extern "C" int ogm_weight_info(const ogm_weight *w, uint32_t *ggml_type, uint32_
 // ------------------------------------------------------------------------------------------
 // matmul
 
+// Enqueues the activation quantizer.  Caller holds the lock.
+static int enqueue_quantize(ogm_ctx *ctx, int mode, const float *x_dev, uint32_t in_dim,
+                            uint32_t n_tokens, hipStream_t stream) {
+  int rc = ensure_act(ctx, in_dim, n_tokens);
+  if (rc != OGM_OK) return rc;
+  HIPCHK(ctx, ogm_launch_quantize(mode, x_dev, in_dim, n_tokens, act_view(ctx, in_dim, mode, 0), stream));
+  ctx->act_mode = mode;
+  ctx->act_in_dim = in_dim;
+  ctx->act_tokens = n_tokens;
+  return OGM_OK;
+}
+
+static int enqueue_gemv(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, float *y_dev,
+                        int decode, hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin);
+
 // Enqueues quantize + kernels for tokens of x_dev into y_dev.  Caller holds the lock.
 static int enqueue_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
                           float *y_dev, int decode, hipStream_t stream, int32_t *dump_isum,
                           int32_t *dump_imin) {
   if (n_tokens == 0) return OGM_OK;
-  const int mode = act_mode_for(w->ggml_type);
-  int rc = ensure_act(ctx, w->in_dim, n_tokens);
+  int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type), x_dev, w->in_dim, n_tokens, stream);
   if (rc != OGM_OK) return rc;
-  HIPCHK(ctx, ogm_launch_quantize(mode, x_dev, w->in_dim, n_tokens, act_view(ctx, w->in_dim, mode, 0),
-                                  stream));
+  return enqueue_gemv(ctx, w, n_tokens, y_dev, decode, stream, dump_isum, dump_imin);
+}
+
+// Enqueues the matmul kernels over the context's quantized activations.  Caller holds the lock.
+static int enqueue_gemv(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, float *y_dev,
+                        int decode, hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin) {
+  const int mode = act_mode_for(w->ggml_type);
   // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
   // n_tokens == 1 and every matmul_decode take the GEMV's.
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
-  const uint32_t rows = (uint32_t)ctx->tune_gemv_rows;
-  const uint32_t chunk = ogm_gemv_max_tokens(w->ggml_type, w->in_dim, gemm_order, rows);
+  const uint32_t wg_waves = (uint32_t)ctx->tune_wg_waves;
+  const uint32_t chunk = ogm_gemv_max_tokens(w->ggml_type, w->in_dim, gemm_order, wg_waves);
   if (chunk == 0) return fail(ctx, OGM_ERR_UNSUPPORTED, "no kernel for this type");
   const uint32_t blocks_per_row = w->in_dim / (w->ggml_type == OGM_Q8_0 ? 32 : 256);
   for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
@@ -326,7 +353,8 @@ static int enqueue_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev,
     a.n_tokens = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
     a.y = y_dev + (size_t)t0 * w->out_dim;
     a.gemm_order = gemm_order;
-    a.rows_per_wg = rows;
+    a.wg_waves = wg_waves;
+    a.max_waves = (uint32_t)ctx->tune_max_waves;
     a.dump_isum = dump_isum ? dump_isum + (size_t)t0 * w->out_dim * blocks_per_row : nullptr;
     a.dump_imin = dump_imin ? dump_imin + (size_t)t0 * w->out_dim * blocks_per_row : nullptr;
     HIPCHK(ctx, ogm_launch_gemv(a, stream, &ctx->last_kernel));
@@ -383,6 +411,34 @@ extern "C" int ogm_matmul_dev(ogm_ctx *ctx, const ogm_weight *w, const float *x_
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
   return enqueue_matmul(ctx, w, x_dev, n_tokens, y_dev, decode, s, nullptr, nullptr);
+}
+
+extern "C" int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev,
+                                    uint32_t in_dim, uint32_t n_tokens, void *stream) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!ogm_supports(ggml_type, in_dim)) return fail(ctx, OGM_ERR_UNSUPPORTED, "type / in_dim without a kernel");
+  if (n_tokens == 0) return OGM_OK;
+  if (!x_dev) return fail(ctx, OGM_ERR_INVALID, "x is null");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
+  return enqueue_quantize(ctx, act_mode_for(ggml_type), x_dev, in_dim, n_tokens, s);
+}
+
+extern "C" int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens,
+                                  float *y_dev, int decode, void *stream) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!w) return fail(ctx, OGM_ERR_INVALID, "weight is null");
+  if (n_tokens == 0) return OGM_OK;
+  if (!y_dev) return fail(ctx, OGM_ERR_INVALID, "y is null");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (ctx->act_mode != act_mode_for(w->ggml_type) || ctx->act_in_dim != w->in_dim ||
+      ctx->act_tokens < n_tokens)
+    return fail(ctx, OGM_ERR_INVALID, "the quantized activations do not fit this weight "
+                "(call ogm_act_quantize_dev with its type, in_dim and token count first)");
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
+  return enqueue_gemv(ctx, w, n_tokens, y_dev, decode, s, nullptr, nullptr);
 }
 
 // Backend::matmul_batch (backend/mod.rs:362-366) with guarded_matmul_op's token stripes

@@ -20,7 +20,6 @@
 #include "ogm_kernels.h"
 #include "ogm_layout.h"
 
-#define OGM_WG 256
 
 // ------------------------------------------------------------------------------------------
 // small helpers
@@ -125,6 +124,7 @@ struct FmtQ4K {
   static constexpr int AUX16 = 1;      // bsum: 8 x i16 per block
   static constexpr int ACT_GROUP = 256;
   static constexpr bool HAS_MIN = true;
+  static constexpr int MAX_THREADS = 1024;  // 16 waves share one staged activation vector
   struct Regs {
     uint4 p[PIECES];
   };
@@ -134,6 +134,7 @@ struct FmtQ4K {
     for (int i = 0; i < PIECES; i++) r.p[i] = *(const uint4 *)(base + i * 1024);
   }
   // isum = sum_j sc_j * dot32(nibbles_j, x_j), imin = sum_j m_j * bsum_j     (vecdot.rs:3152-3178)
+  template <int UPR>
   __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
                                               int &isum, int &imin) {
     // get_scale_min_k4 (quant.rs:653-662) for all eight sub-blocks at once, four bytes a word
@@ -142,31 +143,52 @@ struct FmtQ4K {
     const uint32_t mna = w1 & 0x3F3F3F3Fu;                                   // m  0..3
     const uint32_t scb = (w2 & 0x0F0F0F0Fu) | ((w0 >> 2) & 0x30303030u);     // sc 4..7
     const uint32_t mnb = ((w2 >> 4) & 0x0F0F0F0Fu) | ((w1 >> 2) & 0x30303030u);  // m 4..7
+    const uint32_t m4 = 0x0F0F0F0Fu;
+    const uint4 *xp = a.xq + col;
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;  // compile-time: LDS offsets become immediates
+    // The four activation chunks of group g+1 are requested before group g is consumed.
+    uint4 xa0 = xp[0], xa1 = xp[st], xb0 = xp[2 * st], xb1 = xp[3 * st];
+    const uint4 b = a.aux[col];  // bsum_0..7 as i16
     isum = 0;
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-      // qs[32g .. 32g+32): low nibbles are sub-block 2g, high nibbles sub-block 2g+1
-      int dlo = 0, dhi = 0;
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const uint4 w = r.p[1 + 2 * g + h];
-        const uint4 xa = a.xq[(4 * g + h) * a.upr + col];      // elements 64g + 16h ..
-        const uint4 xb = a.xq[(4 * g + 2 + h) * a.upr + col];  // elements 64g + 32 + 16h ..
-        dlo = dot4(w.x & 0x0F0F0F0Fu, xa.x, dlo);
-        dlo = dot4(w.y & 0x0F0F0F0Fu, xa.y, dlo);
-        dlo = dot4(w.z & 0x0F0F0F0Fu, xa.z, dlo);
-        dlo = dot4(w.w & 0x0F0F0F0Fu, xa.w, dlo);
-        dhi = dot4((w.x >> 4) & 0x0F0F0F0Fu, xb.x, dhi);
-        dhi = dot4((w.y >> 4) & 0x0F0F0F0Fu, xb.y, dhi);
-        dhi = dot4((w.z >> 4) & 0x0F0F0F0Fu, xb.z, dhi);
-        dhi = dot4((w.w >> 4) & 0x0F0F0F0Fu, xb.w, dhi);
+      // qs[32g .. 32g+32): low nibbles are sub-block 2g (elements 64g..), high nibbles sub-block
+      // 2g+1 (elements 64g+32..); piece 1+2g holds bytes 0..15 of the run, piece 2+2g bytes 16..31
+      uint4 na0 = xa0, na1 = xa1, nb0 = xb0, nb1 = xb1;
+      if (g < 3) {
+        const uint4 *q = xp + 4 * (g + 1) * st;
+        na0 = q[0];
+        na1 = q[st];
+        nb0 = q[2 * st];
+        nb1 = q[3 * st];
       }
+      const uint4 wa = r.p[1 + 2 * g], wb = r.p[2 + 2 * g];
+      int dlo = 0, dhi = 0;
+      dlo = dot4(wa.x & m4, xa0.x, dlo);
+      dlo = dot4(wa.y & m4, xa0.y, dlo);
+      dlo = dot4(wa.z & m4, xa0.z, dlo);
+      dlo = dot4(wa.w & m4, xa0.w, dlo);
+      dlo = dot4(wb.x & m4, xa1.x, dlo);
+      dlo = dot4(wb.y & m4, xa1.y, dlo);
+      dlo = dot4(wb.z & m4, xa1.z, dlo);
+      dlo = dot4(wb.w & m4, xa1.w, dlo);
+      dhi = dot4((wa.x >> 4) & m4, xb0.x, dhi);
+      dhi = dot4((wa.y >> 4) & m4, xb0.y, dhi);
+      dhi = dot4((wa.z >> 4) & m4, xb0.z, dhi);
+      dhi = dot4((wa.w >> 4) & m4, xb0.w, dhi);
+      dhi = dot4((wb.x >> 4) & m4, xb1.x, dhi);
+      dhi = dot4((wb.y >> 4) & m4, xb1.y, dhi);
+      dhi = dot4((wb.z >> 4) & m4, xb1.z, dhi);
+      dhi = dot4((wb.w >> 4) & m4, xb1.w, dhi);
       const int j = 2 * g;
       const int sc_lo = j < 4 ? byte_of(sca, j) : byte_of(scb, j - 4);
       const int sc_hi = j + 1 < 4 ? byte_of(sca, j + 1) : byte_of(scb, j - 3);
       isum += sc_lo * dlo + sc_hi * dhi;
+      xa0 = na0;
+      xa1 = na1;
+      xb0 = nb0;
+      xb1 = nb1;
     }
-    const uint4 b = a.aux[col];  // bsum_0..7 as i16
     imin = byte_of(mna, 0) * lo16(b.x) + byte_of(mna, 1) * hi16(b.x) +
            byte_of(mna, 2) * lo16(b.y) + byte_of(mna, 3) * hi16(b.y) +
            byte_of(mnb, 0) * lo16(b.z) + byte_of(mnb, 1) * hi16(b.z) +
@@ -194,6 +216,7 @@ struct FmtQ6K {
   static constexpr int AUX16 = 2;  // per-16 sums of q: 16 x i16 per block
   static constexpr int ACT_GROUP = 256;
   static constexpr bool HAS_MIN = false;
+  static constexpr int MAX_THREADS = 512;  // 13 pieces a lane: needs more than 128 registers
   struct Regs {
     uint4 p[PIECES];
     uint32_t d16;
@@ -228,9 +251,11 @@ struct FmtQ6K {
   }
   // isum = sum over 16 groups of sc_g * dot16(q_g - 32, x_g)                (vecdot.rs:3215-3241)
   // with dot16(q - 32, x) = dot16(q, x) - 32 * sum16(x), exact in integers.
+  template <int UPR>
   __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
                                               int &isum, int &imin) {
-    const uint4 s_lo = a.aux[col], s_hi = a.aux[a.upr + col];  // sum16 of groups 0..7, 8..15
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;
+    const uint4 s_lo = a.aux[col], s_hi = a.aux[st + col];  // sum16 of groups 0..7, 8..15
     const uint32_t sw[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
     const uint32_t scw[4] = {r.p[12].x, r.p[12].y, r.p[12].z, r.p[12].w};
     isum = 0;
@@ -245,7 +270,7 @@ struct FmtQ6K {
           const int g = 2 * R + k;  // group of 16
           const uint4 ql = r.p[4 * h + 2 * (rr & 1) + k];
           const uint4 qh = r.p[8 + 2 * h + k];
-          const uint4 x = a.xq[g * a.upr + col];
+          const uint4 x = a.xq[g * st + col];
           const int dot = run_dot(ql, qh, x, rr);
           const int s16 = (g & 1) ? hi16(sw[g >> 1]) : lo16(sw[g >> 1]);
           isum += sbyte_of(scw[g >> 2], g & 3) * (dot - 32 * s16);
@@ -273,6 +298,7 @@ struct FmtQ80 {
   static constexpr int AUX16 = 0;
   static constexpr int ACT_GROUP = 32;
   static constexpr bool HAS_MIN = false;
+  static constexpr int MAX_THREADS = 1024;
   struct Regs {
     uint4 p[PIECES];
     uint32_t d16;
@@ -284,9 +310,10 @@ struct FmtQ80 {
     r.p[1] = *(const uint4 *)(base + 1024);
     r.d16 = *(const uint16_t *)(tile + PIECES * 1024 + (u & 63u) * 2u);
   }
+  template <int UPR>
   __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
                                               int &isum, int &imin) {
-    const uint4 x0 = a.xq[col], x1 = a.xq[a.upr + col];
+    const uint4 x0 = a.xq[col], x1 = a.xq[(UPR ? (uint32_t)UPR : a.upr) + col];
     int acc = 0;
     acc = dot4(r.p[0].x, x0.x, acc);
     acc = dot4(r.p[0].y, x0.y, acc);
@@ -313,6 +340,14 @@ struct FmtQ80 {
 
 // ------------------------------------------------------------------------------------------
 // GEMV kernel
+//
+// A wave owns whole output rows.  With `upr` blocks per row, a "segment" is RW = max(1, 64/upr)
+// consecutive rows; lane i of the wave owns block i of the segment (blocks i, i+64, ... when a
+// row has more than 64 blocks).  Waves never wait for each other after the activations are
+// staged: each one loads its blocks, forms the per-block f32 terms, leaves them in its own
+// slice of LDS and adds every row's terms in ascending block order with one lane per row.
+// The only workgroup barrier follows the activation staging, whose loads are issued before the
+// weight loads and therefore complete long before them.
 
 struct GemvParams {
   const uint8_t *wt;
@@ -320,7 +355,12 @@ struct GemvParams {
   float *y;
   int32_t *dump_isum, *dump_imin;
   uint32_t in_dim, out_dim, upr;  // upr = blocks per row
-  uint32_t n_tokens, rows_per_wg;
+  uint32_t n_tokens;
+  uint32_t rows_per_seg;          // RW
+  uint32_t n_seg;                 // ceil(out_dim / RW)
+  uint32_t seg_units;             // RW * upr
+  uint32_t term_stride;           // floats per token in a wave's term slice (>= seg_units)
+  uint32_t n_units;               // out_dim * upr
 };
 
 template <class F, bool GEMM_ORDER>
@@ -328,57 +368,132 @@ __host__ __device__ constexpr int n_term_arrays() {
   return (GEMM_ORDER && F::HAS_MIN) ? 2 : 1;
 }
 
-// Dynamic LDS bytes of one workgroup.
+static uint32_t rows_per_seg_for(uint32_t upr) { return upr >= 64 ? 1u : 64u / upr; }
+
+// Dynamic LDS bytes of one workgroup of `waves` waves.
 template <class F, bool GEMM_ORDER>
-static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rows_per_wg) {
+static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t waves) {
   const size_t upr = in_dim / F::ELEMS;
   const size_t n_scale = in_dim / F::ACT_GROUP;
+  const size_t seg_units = rows_per_seg_for((uint32_t)upr) * upr;
   size_t b = (size_t)n_tokens * in_dim;                     // xq
   b += (size_t)n_tokens * upr * F::AUX16 * 16;              // aux
   b += (size_t)n_tokens * n_scale * 4;                      // act.d
-  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * rows_per_wg * upr * 4;  // terms
+  b = (b + 15) & ~(size_t)15;
+  b += (size_t)waves * n_term_arrays<F, GEMM_ORDER>() * n_tokens * ((seg_units + 3) & ~(size_t)3) * 4;
   return b;
 }
 
-template <class F, bool GEMM_ORDER, bool DUMP>
-__global__ __launch_bounds__(OGM_WG) void ogm_gemv_kernel(GemvParams p) {
+#define OGM_STAGE_PEEL 4
+
+// Sum of n floats at p in ascending order with one accumulator, sign +1 or -1.
+template <bool NEGATE>
+__device__ __forceinline__ float ordered_sum(float acc, const float *p, uint32_t n) {
+  uint32_t s = 0;
+  if ((n & 3u) == 0) {  // rows of whole float4s: few wide LDS reads, then the same adds
+    for (; s < n; s += 4) {
+      const float4 v = *(const float4 *)(p + s);
+      if (NEGATE) { acc -= v.x; acc -= v.y; acc -= v.z; acc -= v.w; }
+      else        { acc += v.x; acc += v.y; acc += v.z; acc += v.w; }
+    }
+  } else {
+    for (; s < n; s++) {
+      if (NEGATE) acc -= p[s];
+      else acc += p[s];
+    }
+  }
+  return acc;
+}
+
+// UPR: blocks per row when known at compile time (the hot shapes), 0 = read it from the params.
+template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP>
+__global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) {
   extern __shared__ __align__(16) uint8_t lds[];
-  const uint32_t tid = threadIdx.x;
-  const uint32_t T = p.n_tokens;
-  const uint32_t upr = p.upr;
-  const uint32_t xch = p.in_dim / 16;              // 16-byte chunks of q per token
-  const uint32_t n_scale = p.in_dim / F::ACT_GROUP;
-  const uint32_t r0 = blockIdx.x * p.rows_per_wg;
-  const uint32_t rows = min(p.rows_per_wg, p.out_dim - r0);
-  const uint32_t u0 = r0 * upr, uw = rows * upr;   // this workgroup's units: [u0, u0 + uw)
+  const uint32_t tid = threadIdx.x, nthr = blockDim.x;
+  const uint32_t lane = tid & 63u, wave = tid >> 6, n_wave = nthr >> 6;
+  const uint32_t T = SINGLE ? 1u : p.n_tokens;
+  const uint32_t upr = UPR ? (uint32_t)UPR : p.upr;
+  const uint32_t xch = upr * F::XPIECES;           // 16-byte chunks of q per token
+  const uint32_t n_scale = upr * (F::ELEMS / F::ACT_GROUP);
+  const uint32_t rows_per_seg = UPR ? (UPR >= 64 ? 1u : 64u / UPR) : p.rows_per_seg;
+  const uint32_t seg_units = rows_per_seg * upr;
+  const uint32_t term_stride = (seg_units + 3) & ~3u;
   constexpr int NT = n_term_arrays<F, GEMM_ORDER>();
 
   uint4 *l_xq = (uint4 *)lds;                                   // [T][xch]
   uint4 *l_aux = l_xq + (size_t)T * xch;                        // [T][AUX16][upr]
   float *l_d = (float *)(l_aux + (size_t)T * upr * F::AUX16);   // [T][n_scale]
-  float *l_term = l_d + (size_t)T * n_scale;                    // [NT][T][rows_per_wg * upr]
-  const uint32_t term_stride = p.rows_per_wg * upr;
+  const size_t head = ((size_t)T * (xch * 16 + upr * F::AUX16 * 16 + n_scale * 4) + 15) & ~(size_t)15;
+  float *l_term = (float *)(lds + head) + (size_t)wave * NT * T * term_stride;  // this wave's
 
-  // The first block's weight loads go out before anything else: they are the long pole.
+  // ---- issue the activation loads (few, L2-resident) ...
+  // Every load below is unconditional with a clamped index: straight-line code lets the
+  // compiler wait for exactly the staging loads (vmcnt) while the weight loads stay in flight.
+  const uint32_t n_xq = T * xch;
+  const uint4 *gq = (const uint4 *)p.act.q;
+  const uint4 st0 = gq[min(tid, n_xq - 1)];
+  const uint4 st1 = gq[min(tid + nthr, n_xq - 1)];
+  const uint4 st2 = gq[min(tid + 2 * nthr, n_xq - 1)];
+  const uint4 st3 = gq[min(tid + 3 * nthr, n_xq - 1)];
+  const uint32_t n_aux = T * upr * F::AUX16;
+  uint4 st_aux = make_uint4(0, 0, 0, 0);
+  if (F::AUX16 == 1) {
+    st_aux = ((const uint4 *)p.act.bsum)[min(tid, n_aux - 1)];  // Q4_K: bsum, 8 x i16 per block
+  } else if (F::AUX16 == 2) {
+    // Q6_K: per-16 sums narrowed to i16, groups 0..7 / 8..15 of a block
+    const uint32_t i = min(tid, n_aux - 1);
+    const int4 *src = (const int4 *)(p.act.sums + (size_t)(i >> 1) * 16 + (i & 1u) * 8);
+    const int4 a = src[0], b = src[1];
+    st_aux.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
+    st_aux.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
+    st_aux.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
+    st_aux.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
+  }
+  const uint32_t n_d = T * n_scale;
+  const float st_d = p.act.d[min(tid, n_d - 1)];
+
+  // ---- ... then this wave's first segment of weights (the long pole) ...
+  const uint32_t total_waves = gridDim.x * n_wave;
+  uint32_t seg = blockIdx.x * n_wave + wave;
   typename F::Regs cur;
-  uint32_t u = tid;
-  bool have = u < uw;
-  if (have) F::load(cur, p.wt, u0 + u);
+  F::load(cur, p.wt, min(seg * seg_units + lane, p.n_units - 1));
 
-  // Stage the activations: q permuted so that chunk c of block `col` lands at [c*upr + col].
-  for (uint32_t i = tid; i < T * xch; i += OGM_WG) {
+  // ---- ... and park the activations in LDS while the weights are in flight.
+  // q is permuted so that chunk c of block `col` lands at [c*upr + col].
+  auto park = [&](uint32_t i, const uint4 &v) {
+    if (i < n_xq) {
+      const uint32_t t = i / xch, ch = i - t * xch;
+      const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
+      l_xq[(size_t)t * xch + c * upr + col] = v;
+    }
+  };
+  park(tid, st0);
+  park(tid + nthr, st1);
+  park(tid + 2 * nthr, st2);
+  park(tid + 3 * nthr, st3);
+  if (F::AUX16 == 1) {
+    if (tid < n_aux) l_aux[tid] = st_aux;
+  } else if (F::AUX16 == 2) {
+    if (tid < n_aux) {
+      const uint32_t blk = tid >> 1, k = tid & 1u;
+      const uint32_t t = blk / upr, col = blk - t * upr;
+      l_aux[(size_t)t * upr * 2 + k * upr + col] = st_aux;
+    }
+  }
+  if (tid < n_d) l_d[tid] = st_d;
+  // Whatever the peeled loads did not cover (many tokens, or very long rows).
+  for (uint32_t i = tid + OGM_STAGE_PEEL * nthr; i < n_xq; i += nthr) {
     const uint32_t t = i / xch, ch = i - t * xch;
     const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
-    l_xq[(size_t)t * xch + c * upr + col] = ((const uint4 *)(p.act.q + (size_t)t * p.in_dim))[ch];
+    l_xq[(size_t)t * xch + c * upr + col] = gq[i];
   }
-  if (F::AUX16 == 1) {  // Q4_K: bsum, 8 x i16 per super-block, already in that form
-    for (uint32_t i = tid; i < T * upr; i += OGM_WG)
-      l_aux[i] = ((const uint4 *)p.act.bsum)[i];
-  } else if (F::AUX16 == 2) {  // Q6_K: per-16 sums as i16, groups 0..7 then 8..15
-    for (uint32_t i = tid; i < T * upr * 2; i += OGM_WG) {
-      const uint32_t t = i / (upr * 2), rem = i - t * upr * 2;
-      const uint32_t col = rem >> 1, k = rem & 1u;
-      const int4 *src = (const int4 *)(p.act.sums + ((size_t)t * upr + col) * 16 + k * 8);
+  if (F::AUX16 == 1) {
+    for (uint32_t i = tid + nthr; i < n_aux; i += nthr) l_aux[i] = ((const uint4 *)p.act.bsum)[i];
+  } else if (F::AUX16 == 2) {
+    for (uint32_t i = tid + nthr; i < n_aux; i += nthr) {
+      const uint32_t blk = i >> 1, k = i & 1u;
+      const uint32_t t = blk / upr, col = blk - t * upr;
+      const int4 *src = (const int4 *)(p.act.sums + (size_t)blk * 16 + k * 8);
       const int4 a = src[0], b = src[1];
       uint4 o;
       o.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
@@ -388,56 +503,59 @@ __global__ __launch_bounds__(OGM_WG) void ogm_gemv_kernel(GemvParams p) {
       l_aux[(size_t)t * upr * 2 + k * upr + col] = o;
     }
   }
-  for (uint32_t i = tid; i < T * n_scale; i += OGM_WG) l_d[i] = p.act.d[i];
+  for (uint32_t i = tid + nthr; i < n_d; i += nthr) l_d[i] = p.act.d[i];
   __syncthreads();
 
-  while (have) {
-    const uint32_t un = u + OGM_WG;
-    const bool have_next = un < uw;
-    typename F::Regs nxt;
-    if (have_next) F::load(nxt, p.wt, u0 + un);
-
-    const uint32_t row = u / upr, col = u - row * upr;
-    for (uint32_t t = 0; t < T; t++) {
-      ActLds a;
-      a.xq = l_xq + (size_t)t * xch;
-      a.aux = l_aux + (size_t)t * upr * F::AUX16;
-      a.d = l_d + (size_t)t * n_scale;
-      a.upr = upr;
-      int isum, imin;
-      F::sums(cur, a, col, isum, imin);
-      const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
-      if (GEMM_ORDER) {
-        float tmin, tdot;
-        F::term_gemm(cur, ad, isum, imin, tmin, tdot);
-        l_term[(size_t)t * term_stride + u] = tdot;
-        if (NT == 2) l_term[(size_t)(T + t) * term_stride + u] = tmin;
-      } else {
-        l_term[(size_t)t * term_stride + u] = F::term_gemv(cur, ad, isum, imin);
-      }
-      if (DUMP) {
-        const size_t o = ((size_t)t * p.out_dim + r0) * upr + u;
-        if (p.dump_isum) p.dump_isum[o] = isum;
-        if (F::HAS_MIN && p.dump_imin) p.dump_imin[o] = imin;
+  // ---- segments of this wave
+  for (; seg < p.n_seg; seg += total_waves) {
+    const uint32_t row0 = seg * rows_per_seg;
+    for (uint32_t i = lane; i < seg_units; i += 64) {
+      const uint32_t rl = i / upr, col = i - rl * upr;
+      const bool live = row0 + rl < p.out_dim;
+      if (i != lane) F::load(cur, p.wt, min(row0 * upr + i, p.n_units - 1));  // first block is loaded
+      if (live) {
+        for (uint32_t t = 0; t < T; t++) {
+          ActLds a;
+          a.xq = l_xq + (size_t)t * xch;
+          a.aux = l_aux + (size_t)t * upr * F::AUX16;
+          a.d = l_d + (size_t)t * n_scale;
+          a.upr = upr;
+          int isum, imin;
+          F::template sums<UPR>(cur, a, col, isum, imin);
+          const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
+          if (GEMM_ORDER) {
+            float tmin, tdot;
+            F::term_gemm(cur, ad, isum, imin, tmin, tdot);
+            l_term[(size_t)t * term_stride + i] = tdot;
+            if (NT == 2) l_term[(size_t)(T + t) * term_stride + i] = tmin;
+          } else {
+            l_term[(size_t)t * term_stride + i] = F::term_gemv(cur, ad, isum, imin);
+          }
+          if (DUMP) {
+            const size_t o = ((size_t)t * p.out_dim + row0) * upr + i;
+            if (p.dump_isum) p.dump_isum[o] = isum;
+            if (F::HAS_MIN && p.dump_imin) p.dump_imin[o] = imin;
+          }
+        }
       }
     }
-    if (have_next) cur = nxt;
-    u = un;
-    have = have_next;
-  }
-  __syncthreads();
-
-  // One lane per (row, token): the row's block terms in ascending order, one accumulator.
-  for (uint32_t i = tid; i < rows * T; i += OGM_WG) {
-    const uint32_t t = i / rows, row = i - t * rows;
-    const float *td = l_term + (size_t)t * term_stride + row * upr;
-    float acc = 0.0f;
-    if (NT == 2) {
-      const float *tm = l_term + (size_t)(T + t) * term_stride + row * upr;
-      for (uint32_t s = 0; s < upr; s++) acc -= tm[s];
+    // The registers are free again: request the next segment's first block now.
+    const uint32_t nseg = seg + total_waves;
+    if (nseg < p.n_seg) F::load(cur, p.wt, min(nseg * seg_units + lane, p.n_units - 1));
+    // One lane per (row, token): the row's block terms in ascending order, one accumulator.
+    // The same wave wrote them and a wave's LDS operations complete in order, so no workgroup
+    // barrier is needed; the wave barrier only pins the compiler's ordering.
+    __builtin_amdgcn_wave_barrier();
+    for (uint32_t i = lane; i < rows_per_seg * T; i += 64) {
+      const uint32_t t = i / rows_per_seg, rl = i - t * rows_per_seg;
+      if (row0 + rl < p.out_dim) {
+        float acc = 0.0f;
+        if (NT == 2) acc = ordered_sum<true>(acc, l_term + (size_t)(T + t) * term_stride + rl * upr, upr);
+        acc = ordered_sum<false>(acc, l_term + (size_t)t * term_stride + rl * upr, upr);
+        p.y[(size_t)t * p.out_dim + row0 + rl] = acc;
+      }
     }
-    for (uint32_t s = 0; s < upr; s++) acc += td[s];
-    p.y[(size_t)t * p.out_dim + r0 + row] = acc;
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -445,46 +563,47 @@ __global__ __launch_bounds__(OGM_WG) void ogm_gemv_kernel(GemvParams p) {
 // host side of the launch
 
 static const size_t OGM_LDS_BUDGET = 64 * 1024;
+static const uint32_t OGM_NUM_CU = 256;          // MI355X
+static const uint32_t OGM_WAVES_PER_CU = 16;     // at <= 128 VGPRs
 
-static uint32_t default_rows_per_wg(uint32_t upr, uint32_t out_dim) {
-  // About one block per lane and per pass; at least one row.
-  uint32_t r = (OGM_WG + upr - 1) / upr;
-  if (r == 0) r = 1;
-  if (r > out_dim) r = out_dim;
-  return r;
+static uint32_t default_wg_waves(uint32_t in_dim) {
+  // Longer rows mean more activation bytes per workgroup: share them among more waves.
+  if (in_dim <= 4096) return 4;
+  if (in_dim <= 8192) return 8;
+  return 16;
 }
 
 template <class F, bool GEMM_ORDER>
-static uint32_t max_tokens_t(uint32_t in_dim, uint32_t rows_per_wg) {
+static uint32_t max_tokens_t(uint32_t in_dim, uint32_t waves) {
   uint32_t t = 8;
-  while (t > 1 && gemv_lds_bytes<F, GEMM_ORDER>(in_dim, t, rows_per_wg) > OGM_LDS_BUDGET) t--;
+  while (t > 1 && gemv_lds_bytes<F, GEMM_ORDER>(in_dim, t, waves) > OGM_LDS_BUDGET) t--;
   return t;
 }
 
 template <class F>
-static uint32_t resolve_rows(uint32_t in_dim, uint32_t out_dim, uint32_t rows_per_wg) {
-  const uint32_t upr = in_dim / F::ELEMS;
-  uint32_t r = rows_per_wg ? rows_per_wg : default_rows_per_wg(upr, out_dim);
-  if (r > out_dim) r = out_dim;
+static uint32_t resolve_waves(uint32_t in_dim, uint32_t wg_waves) {
+  uint32_t w = wg_waves ? wg_waves : default_wg_waves(in_dim);
+  if (w > (uint32_t)F::MAX_THREADS / 64) w = F::MAX_THREADS / 64;
+  if (w < 1) w = 1;
   // one token must fit
-  while (r > 1 && gemv_lds_bytes<F, true>(in_dim, 1, r) > OGM_LDS_BUDGET) r--;
-  return r;
+  while (w > 1 && gemv_lds_bytes<F, true>(in_dim, 1, w) > OGM_LDS_BUDGET) w--;
+  return w;
 }
 
 uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order,
-                             uint32_t rows_per_wg) {
+                             uint32_t wg_waves) {
   switch (ggml_type) {
     case OGM_Q4_K: {
-      uint32_t r = resolve_rows<FmtQ4K>(in_dim, 0xFFFFFFFFu, rows_per_wg);
-      return gemm_order ? max_tokens_t<FmtQ4K, true>(in_dim, r) : max_tokens_t<FmtQ4K, false>(in_dim, r);
+      uint32_t w = resolve_waves<FmtQ4K>(in_dim, wg_waves);
+      return gemm_order ? max_tokens_t<FmtQ4K, true>(in_dim, w) : max_tokens_t<FmtQ4K, false>(in_dim, w);
     }
     case OGM_Q6_K: {
-      uint32_t r = resolve_rows<FmtQ6K>(in_dim, 0xFFFFFFFFu, rows_per_wg);
-      return gemm_order ? max_tokens_t<FmtQ6K, true>(in_dim, r) : max_tokens_t<FmtQ6K, false>(in_dim, r);
+      uint32_t w = resolve_waves<FmtQ6K>(in_dim, wg_waves);
+      return gemm_order ? max_tokens_t<FmtQ6K, true>(in_dim, w) : max_tokens_t<FmtQ6K, false>(in_dim, w);
     }
     case OGM_Q8_0: {
-      uint32_t r = resolve_rows<FmtQ80>(in_dim, 0xFFFFFFFFu, rows_per_wg);
-      return gemm_order ? max_tokens_t<FmtQ80, true>(in_dim, r) : max_tokens_t<FmtQ80, false>(in_dim, r);
+      uint32_t w = resolve_waves<FmtQ80>(in_dim, wg_waves);
+      return gemm_order ? max_tokens_t<FmtQ80, true>(in_dim, w) : max_tokens_t<FmtQ80, false>(in_dim, w);
     }
     default:
       return 0;
@@ -503,16 +622,35 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   p.out_dim = a.out_dim;
   p.upr = a.in_dim / F::ELEMS;
   p.n_tokens = a.n_tokens;
-  p.rows_per_wg = resolve_rows<F>(a.in_dim, a.out_dim, a.rows_per_wg);
-  const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, p.rows_per_wg);
+  p.rows_per_seg = rows_per_seg_for(p.upr);
+  p.n_seg = (a.out_dim + p.rows_per_seg - 1) / p.rows_per_seg;
+  p.seg_units = p.rows_per_seg * p.upr;
+  p.term_stride = (p.seg_units + 3) & ~3u;
+  p.n_units = a.out_dim * p.upr;
+  const uint32_t waves = resolve_waves<F>(a.in_dim, a.wg_waves);
+  const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, waves);
   if (lds > OGM_LDS_BUDGET) return hipErrorInvalidValue;
-  const uint32_t grid = (a.out_dim + p.rows_per_wg - 1) / p.rows_per_wg;
-  if (a.dump_isum || a.dump_imin)
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, GEMM_ORDER, true>), dim3(grid), dim3(OGM_WG), lds,
-                       stream, p);
-  else
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, GEMM_ORDER, false>), dim3(grid), dim3(OGM_WG), lds,
-                       stream, p);
+  // One segment per wave while the whole grid can be resident; beyond that waves loop.
+  const uint32_t max_waves = a.max_waves ? a.max_waves : OGM_NUM_CU * OGM_WAVES_PER_CU;
+  uint32_t want = p.n_seg < max_waves ? p.n_seg : max_waves;
+  uint32_t grid = (want + waves - 1) / waves;
+  if (grid == 0) grid = 1;
+  const dim3 g(grid), b(waves * 64);
+  if (a.dump_isum || a.dump_imin) {
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true>), g, b, lds, stream, p);
+  } else if (a.n_tokens == 1 && !GEMM_ORDER) {
+    // single-token decode: the hot shapes get their row length as a compile-time constant
+    if (F::ELEMS == 256 && p.upr == 16)
+      hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false>), g, b, lds, stream, p);
+    else if (F::ELEMS == 256 && p.upr == 56)
+      hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false>), g, b, lds, stream, p);
+    else if (F::ELEMS == 32 && p.upr == 128)
+      hipLaunchKernelGGL((ogm_gemv_kernel<F, 128, true, false, false>), g, b, lds, stream, p);
+    else
+      hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false>), g, b, lds, stream, p);
+  } else {
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false>), g, b, lds, stream, p);
+  }
   return hipGetLastError();
 }
 

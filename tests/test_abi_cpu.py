@@ -115,4 +115,4 @@ def test_init_without_a_device_is_a_status_not_a_crash(lib):
     assert Mi355xBackend.try_init() is None
     # null-context calls return a status
     assert lib.ogm_matmul(None, None, None, 1, None) == -1
-    assert lib.ogm_set_tuning(None, b"gemv_rows", 1) == -1
+    assert lib.ogm_set_tuning(None, b"gemv_wg_waves", 1) == -1
