@@ -120,6 +120,14 @@ def main() -> int:
     us_per_launch = e0.elapsed_ms(e1) * 1e3 / n_launch
     kbytes = gemv_bytes(HIDDEN, FFN)
     achieved = kbytes / (us_per_launch * 1e-6) / 1e9
+    if args.only_roofline:
+        # One plain device-to-device copy of known size: under `rocprofv3 --pmc FETCH_SIZE` /
+        # `WRITE_SIZE` its counter reading calibrates the GEMV's (bytes per counter unit).
+        cal = 64 << 20
+        src, dst = hiprt.DeviceBuffer(cal), hiprt.DeviceBuffer(cal)
+        src.fill(1)
+        hiprt.check(hiprt.hip().hipMemcpy(dst.ptr, src.ptr, cal, 3), "hipMemcpy D2D")
+        hiprt.device_synchronize()
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                 "kernel": be.last_kernel(), "us_per_launch": round(us_per_launch, 3),
