@@ -29,6 +29,9 @@ import numpy as np  # noqa: E402
 Q4_K = 12
 HIDDEN, FFN = 4096, 14336
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# runs of `bench.py --only-roofline`, calibrated on that run's 64 MiB copy (profiles/).
+GEMV_Q4K_4096x14336_TRAFFIC = 33175858
 
 
 def gemv_bytes(in_dim: int, out_dim: int, t: int = 1) -> int:
@@ -129,7 +132,7 @@ def main() -> int:
         hiprt.check(hiprt.hip().hipMemcpy(dst.ptr, src.ptr, cal, 3), "hipMemcpy D2D")
         hiprt.device_synchronize()
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_Q4K_4096x14336_TRAFFIC,
                 "kernel": be.last_kernel(), "us_per_launch": round(us_per_launch, 3),
                 "bytes_per_launch": kbytes, "launches": n_launch}
 
