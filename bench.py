@@ -49,7 +49,6 @@ def main() -> int:
     ap.add_argument("--roofline-launches", type=int, default=600)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--wg-waves", type=int, default=0, help="waves per workgroup override (0 = heuristic)")
-    ap.add_argument("--max-waves", type=int, default=0, help="cap on waves per launch (0 = heuristic)")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the dominant-kernel leg (for rocprofv3 --kernel-trace --stats)")
     args = ap.parse_args()
@@ -66,8 +65,6 @@ def main() -> int:
     be = Mi355xBackend()  # raises without the HIP library or a gfx950 device
     if args.wg_waves:
         be.set_tuning("gemv_wg_waves", args.wg_waves)
-    if args.max_waves:
-        be.set_tuning("gemv_max_waves", args.max_waves)
     stream = hiprt.Stream()
 
     # ---- synthetic inputs -------------------------------------------------------------------

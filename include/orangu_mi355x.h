@@ -79,8 +79,9 @@ int ogm_block_layout(uint32_t ggml_type, uint32_t *block_bytes, uint32_t *block_
 /* ---- weights: the uploader --------------------------------------------------------------- */
 
 /* Bytes of the repacked ("tile-planar") form of a matrix: the raw GGUF blocks regrouped in tiles
- * of 64 blocks so that every 16-byte piece of a block lies in a plane that 64 lanes read as one
- * contiguous kilobyte; no bit of any block is altered and only the last tile is zero-padded. */
+ * of 64 blocks (R rows x C blocks, C = 4, 2 or 1) so that every 16-byte piece of a block lies in
+ * a plane that 64 lanes read as one contiguous kilobyte; no bit of any block is altered and only
+ * the rows that pad the last row block to R are zero. */
 size_t ogm_repacked_size(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim);
 /* Host-side repack and its exact inverse.  `raw` is QuantMatrix::raw_bytes()
  * (engine/loader.rs:608-610): out_dim rows of row_bytes. */
@@ -168,8 +169,8 @@ int ogm_f16_to_f32(ogm_ctx *ctx, const uint16_t *bits, size_t n, float *out);
 /* ---- tuning / introspection ------------------------------------------------------------------ */
 
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.
- * keys: "gemv_wg_waves" (waves per workgroup, 1..16), "gemv_max_waves" (cap on the waves of one
- * launch; more row segments than that are looped over); 0 = heuristic. */
+ * key: "gemv_wg_waves" (waves per workgroup of the GEMV kernel, 1..16; 0 = one wave per column
+ * tile of a row block). */
 int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value);
 /* Name of the kernel the last matmul on this context launched (for profiles). */
 const char *ogm_last_kernel(ogm_ctx *ctx);

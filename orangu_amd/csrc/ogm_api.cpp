@@ -43,7 +43,7 @@ struct ogm_ctx {
   // engine/backend/rocm.rs:352-376; a pool is what the Vulkan op_cache does instead)
   DevBuf x, y, q, d, sums, bsum, isum, imin;
   DevBuf hx, hy;  // pinned host staging
-  int tune_wg_waves = 0, tune_max_waves = 0;
+  int tune_wg_waves = 0;
   const char *last_kernel = "";
   // what the activation buffer currently holds (ogm_act_quantize_dev)
   int act_mode = -1;
@@ -194,11 +194,6 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_wg_waves = value;
     return OGM_OK;
   }
-  if (strcmp(key, "gemv_max_waves") == 0) {
-    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemv_max_waves must be >= 0");
-    ctx->tune_max_waves = value;
-    return OGM_OK;
-  }
   return fail(ctx, OGM_ERR_INVALID, std::string("unknown tuning key ") + key);
 }
 
@@ -340,7 +335,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, fl
   // n_tokens == 1 and every matmul_decode take the GEMV's.
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
   const uint32_t wg_waves = (uint32_t)ctx->tune_wg_waves;
-  const uint32_t chunk = ogm_gemv_max_tokens(w->ggml_type, w->in_dim, gemm_order, wg_waves);
+  const uint32_t chunk = ogm_gemv_max_tokens(w->ggml_type, w->in_dim, gemm_order);
   if (chunk == 0) return fail(ctx, OGM_ERR_UNSUPPORTED, "no kernel for this type");
   const uint32_t blocks_per_row = w->in_dim / (w->ggml_type == OGM_Q8_0 ? 32 : 256);
   for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
@@ -354,7 +349,6 @@ static int enqueue_gemv(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, fl
     a.y = y_dev + (size_t)t0 * w->out_dim;
     a.gemm_order = gemm_order;
     a.wg_waves = wg_waves;
-    a.max_waves = (uint32_t)ctx->tune_max_waves;
     a.dump_isum = dump_isum ? dump_isum + (size_t)t0 * w->out_dim * blocks_per_row : nullptr;
     a.dump_imin = dump_imin ? dump_imin + (size_t)t0 * w->out_dim * blocks_per_row : nullptr;
     HIPCHK(ctx, ogm_launch_gemv(a, stream, &ctx->last_kernel));

@@ -27,15 +27,13 @@ struct OgmGemvArgs {
   uint32_t n_tokens;  // tokens in this launch (<= ogm_gemv_max_tokens)
   float *y;           // [n_tokens][out_dim], row stride out_dim
   int gemm_order;     // 0: GEMV float order (cpu.rs T==1 / matmul_decode), 1: GEMM order (T>1)
-  uint32_t wg_waves;     // waves per workgroup, 0 = heuristic
-  uint32_t max_waves;    // cap on resident waves of the launch, 0 = the whole chip
+  uint32_t wg_waves;     // waves per workgroup, 0 = one per column tile of a row block
   int32_t *dump_isum;    // optional [n_tokens][out_dim][blocks/row]
   int32_t *dump_imin;    // optional, Q4_K only
 };
 
 // Largest token count one launch can take for this shape (LDS budget), at least 1.
-uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order,
-                             uint32_t wg_waves);
+uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order);
 hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name);
 
 hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hipStream_t stream);

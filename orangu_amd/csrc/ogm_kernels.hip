@@ -8,12 +8,11 @@
 //     terms in ascending block order with one accumulator, so the f32 result has the
 //     reference's bits as well.  Build with -ffp-contract=off: an FMA would change them.
 //
-// Work mapping: one lane owns one block ("unit") for the whole kernel.  A workgroup owns a run
-// of output rows, i.e. a contiguous run of units; lane l of a wave reads piece p of its unit at
-// tile*tile_bytes + p*1024 + l*16, so each load instruction of a wave covers one contiguous
-// kilobyte.  The int8 activations sit in LDS, laid out so that lanes owning neighbouring
-// blocks read neighbouring 16-byte chunks (no bank conflicts).  Each lane leaves its block's
-// f32 term in LDS; one lane per (row, token) then adds the row's terms in order.
+// Work mapping: one lane owns one block ("unit").  A workgroup owns one row block of the
+// tile-planar layout (R rows); each of its waves takes one tile (R rows x C blocks) at a time and
+// lane l reads piece p of its unit at tile*tile_bytes + p*1024 + l*16, so each load instruction
+// of a wave covers one contiguous kilobyte.  The int8 activations sit in LDS.  Each lane leaves
+// its block's f32 term in LDS; one lane per (row, token) then adds the row's terms in order.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -128,8 +127,8 @@ struct FmtQ4K {
   struct Regs {
     uint4 p[PIECES];
   };
-  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, uint32_t u) {
-    const uint8_t *base = wt + (size_t)(u >> 6) * TILE_BYTES + (u & 63u) * 16u;
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
+    const uint8_t *base = wt + tile * TILE_BYTES + lane * 16u;
 #pragma unroll
     for (int i = 0; i < PIECES; i++) r.p[i] = *(const uint4 *)(base + i * 1024);
   }
@@ -221,12 +220,12 @@ struct FmtQ6K {
     uint4 p[PIECES];
     uint32_t d16;
   };
-  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, uint32_t u) {
-    const uint8_t *tile = wt + (size_t)(u >> 6) * TILE_BYTES;
-    const uint8_t *base = tile + (u & 63u) * 16u;
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
+    const uint8_t *tb = wt + tile * TILE_BYTES;
+    const uint8_t *base = tb + lane * 16u;
 #pragma unroll
     for (int i = 0; i < PIECES; i++) r.p[i] = *(const uint4 *)(base + i * 1024);
-    r.d16 = *(const uint16_t *)(tile + PIECES * 1024 + (u & 63u) * 2u);
+    r.d16 = *(const uint16_t *)(tb + PIECES * 1024 + lane * 2u);
   }
   __device__ static __forceinline__ int run_dot(uint4 ql, uint4 qh, uint4 x, int r) {
     // 6-bit value = nibble | (two bits of qh) << 4, still carrying the +32 bias (0..63)
@@ -303,12 +302,12 @@ struct FmtQ80 {
     uint4 p[PIECES];
     uint32_t d16;
   };
-  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, uint32_t u) {
-    const uint8_t *tile = wt + (size_t)(u >> 6) * TILE_BYTES;
-    const uint8_t *base = tile + (u & 63u) * 16u;
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
+    const uint8_t *tb = wt + tile * TILE_BYTES;
+    const uint8_t *base = tb + lane * 16u;
     r.p[0] = *(const uint4 *)(base);
     r.p[1] = *(const uint4 *)(base + 1024);
-    r.d16 = *(const uint16_t *)(tile + PIECES * 1024 + (u & 63u) * 2u);
+    r.d16 = *(const uint16_t *)(tb + PIECES * 1024 + lane * 2u);
   }
   template <int UPR>
   __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
@@ -341,13 +340,17 @@ struct FmtQ80 {
 // ------------------------------------------------------------------------------------------
 // GEMV kernel
 //
-// A wave owns whole output rows.  With `upr` blocks per row, a "segment" is RW = max(1, 64/upr)
-// consecutive rows; lane i of the wave owns block i of the segment (blocks i, i+64, ... when a
-// row has more than 64 blocks).  Waves never wait for each other after the activations are
-// staged: each one loads its blocks, forms the per-block f32 terms, leaves them in its own
-// slice of LDS and adds every row's terms in ascending block order with one lane per row.
-// The only workgroup barrier follows the activation staging, whose loads are issued before the
-// weight loads and therefore complete long before them.
+// One workgroup per row block (R rows of the tile-planar layout), one tile (R rows x C blocks)
+// per wave at a time; lane c*R + r of the wave owns block c of row r of its tile.  Every lane
+// forms its block's f32 term and leaves it in the workgroup's LDS table [block][row]; after one
+// barrier a lane per (row, token) adds the row's terms in ascending block order with one
+// accumulator, which is the reference's summation order.
+//
+// Vector-memory data returns in issue order, so the few activation loads are issued first and a
+// barrier (waiting for no data) keeps every one of them ahead of the workgroup's weight loads;
+// the code then waits with vmcnt for the activations only and the weights stay in flight across
+// the LDS hand-off.  All these loads use clamped indices instead of branches so that the
+// compiler can count them.
 
 struct GemvParams {
   const uint8_t *wt;
@@ -356,11 +359,7 @@ struct GemvParams {
   int32_t *dump_isum, *dump_imin;
   uint32_t in_dim, out_dim, upr;  // upr = blocks per row
   uint32_t n_tokens;
-  uint32_t rows_per_seg;          // RW
-  uint32_t n_seg;                 // ceil(out_dim / RW)
-  uint32_t seg_units;             // RW * upr
-  uint32_t term_stride;           // floats per token in a wave's term slice (>= seg_units)
-  uint32_t n_units;               // out_dim * upr
+  uint32_t C, nct;                // tile shape: C blocks x R rows, nct = upr / C column tiles
 };
 
 template <class F, bool GEMM_ORDER>
@@ -368,39 +367,35 @@ __host__ __device__ constexpr int n_term_arrays() {
   return (GEMM_ORDER && F::HAS_MIN) ? 2 : 1;
 }
 
-static uint32_t rows_per_seg_for(uint32_t upr) { return upr >= 64 ? 1u : 64u / upr; }
-
-// Dynamic LDS bytes of one workgroup of `waves` waves.
+// Dynamic LDS bytes of one workgroup.
 template <class F, bool GEMM_ORDER>
-static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t waves) {
+static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens) {
   const size_t upr = in_dim / F::ELEMS;
   const size_t n_scale = in_dim / F::ACT_GROUP;
-  const size_t seg_units = rows_per_seg_for((uint32_t)upr) * upr;
+  const OgmTiling tl = ogm_tiling_for((uint32_t)upr, 1);
   size_t b = (size_t)n_tokens * in_dim;                     // xq
   b += (size_t)n_tokens * upr * F::AUX16 * 16;              // aux
   b += (size_t)n_tokens * n_scale * 4;                      // act.d
   b = (b + 15) & ~(size_t)15;
-  b += (size_t)waves * n_term_arrays<F, GEMM_ORDER>() * n_tokens * ((seg_units + 3) & ~(size_t)3) * 4;
+  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * upr * tl.R * 4;  // terms [block][row]
   return b;
 }
 
 #define OGM_STAGE_PEEL 4
 
-// Sum of n floats at p in ascending order with one accumulator, sign +1 or -1.
+// acc (+|-)= p[0], p[stride], ... in ascending order, one accumulator.
 template <bool NEGATE>
-__device__ __forceinline__ float ordered_sum(float acc, const float *p, uint32_t n) {
+__device__ __forceinline__ float ordered_sum(float acc, const float *p, uint32_t n, uint32_t stride) {
   uint32_t s = 0;
-  if ((n & 3u) == 0) {  // rows of whole float4s: few wide LDS reads, then the same adds
-    for (; s < n; s += 4) {
-      const float4 v = *(const float4 *)(p + s);
-      if (NEGATE) { acc -= v.x; acc -= v.y; acc -= v.z; acc -= v.w; }
-      else        { acc += v.x; acc += v.y; acc += v.z; acc += v.w; }
-    }
-  } else {
-    for (; s < n; s++) {
-      if (NEGATE) acc -= p[s];
-      else acc += p[s];
-    }
+  for (; s + 4 <= n; s += 4) {  // four LDS reads in flight, then the same adds in the same order
+    const float a = p[(s + 0) * stride], b = p[(s + 1) * stride];
+    const float c = p[(s + 2) * stride], d = p[(s + 3) * stride];
+    if (NEGATE) { acc -= a; acc -= b; acc -= c; acc -= d; }
+    else        { acc += a; acc += b; acc += c; acc += d; }
+  }
+  for (; s < n; s++) {
+    if (NEGATE) acc -= p[s * stride];
+    else acc += p[s * stride];
   }
   return acc;
 }
@@ -413,22 +408,20 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
   const uint32_t lane = tid & 63u, wave = tid >> 6, n_wave = nthr >> 6;
   const uint32_t T = SINGLE ? 1u : p.n_tokens;
   const uint32_t upr = UPR ? (uint32_t)UPR : p.upr;
+  const uint32_t C = UPR ? ((UPR % 4 == 0) ? 4u : ((UPR % 2 == 0) ? 2u : 1u)) : p.C;
+  const uint32_t R = 64u / C, nct = upr / C;
   const uint32_t xch = upr * F::XPIECES;           // 16-byte chunks of q per token
   const uint32_t n_scale = upr * (F::ELEMS / F::ACT_GROUP);
-  const uint32_t rows_per_seg = UPR ? (UPR >= 64 ? 1u : 64u / UPR) : p.rows_per_seg;
-  const uint32_t seg_units = rows_per_seg * upr;
-  const uint32_t term_stride = (seg_units + 3) & ~3u;
+  const uint32_t term_stride = upr * R;            // floats per token in the term table
   constexpr int NT = n_term_arrays<F, GEMM_ORDER>();
 
   uint4 *l_xq = (uint4 *)lds;                                   // [T][xch]
   uint4 *l_aux = l_xq + (size_t)T * xch;                        // [T][AUX16][upr]
   float *l_d = (float *)(l_aux + (size_t)T * upr * F::AUX16);   // [T][n_scale]
   const size_t head = ((size_t)T * (xch * 16 + upr * F::AUX16 * 16 + n_scale * 4) + 15) & ~(size_t)15;
-  float *l_term = (float *)(lds + head) + (size_t)wave * NT * T * term_stride;  // this wave's
+  float *l_term = (float *)(lds + head);                        // [NT][T][upr][R]
 
   // ---- issue the activation loads (few, L2-resident) ...
-  // Every load below is unconditional with a clamped index: straight-line code lets the
-  // compiler wait for exactly the staging loads (vmcnt) while the weight loads stay in flight.
   const uint32_t n_xq = T * xch;
   const uint4 *gq = (const uint4 *)p.act.q;
   const uint4 st0 = gq[min(tid, n_xq - 1)];
@@ -452,16 +445,18 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
   const uint32_t n_d = T * n_scale;
   const float st_d = p.act.d[min(tid, n_d - 1)];
 
-  // Vector memory returns in issue order per CU, across waves.  This barrier (no data is waited
-  // for) keeps every staging load of the workgroup ahead of every weight load, so the small
-  // L2-resident activations are never queued behind another wave's HBM traffic.
+  // Keeps every staging load of the workgroup ahead of every weight load in the CU's
+  // memory pipeline (no data is waited for here).
   __syncthreads();
 
-  // ---- ... then this wave's first segment of weights (the long pole) ...
-  const uint32_t total_waves = gridDim.x * n_wave;
-  uint32_t seg = blockIdx.x * n_wave + wave;
+  // ---- ... then this wave's first tile of weights (the long pole) ...
+  const uint32_t rb = blockIdx.x;
+  const uint32_t r_local = lane & (R - 1), c_local = lane / R;
+  const uint32_t row = rb * R + r_local;
+  const bool live = row < p.out_dim;
+  uint32_t ct = wave;  // every wave has at least one tile: n_wave <= nct
   typename F::Regs cur;
-  F::load(cur, p.wt, min(seg * seg_units + lane, p.n_units - 1));
+  F::load(cur, p.wt, (size_t)rb * nct + ct, lane);
 
   // ---- ... and park the activations in LDS while the weights are in flight.
   // q is permuted so that chunk c of block `col` lands at [c*upr + col].
@@ -511,56 +506,47 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
   for (uint32_t i = tid + nthr; i < n_d; i += nthr) l_d[i] = p.act.d[i];
   __syncthreads();
 
-  // ---- segments of this wave
-  for (; seg < p.n_seg; seg += total_waves) {
-    const uint32_t row0 = seg * rows_per_seg;
-    for (uint32_t i = lane; i < seg_units; i += 64) {
-      const uint32_t rl = i / upr, col = i - rl * upr;
-      const bool live = row0 + rl < p.out_dim;
-      if (i != lane) F::load(cur, p.wt, min(row0 * upr + i, p.n_units - 1));  // first block is loaded
-      if (live) {
-        for (uint32_t t = 0; t < T; t++) {
-          ActLds a;
-          a.xq = l_xq + (size_t)t * xch;
-          a.aux = l_aux + (size_t)t * upr * F::AUX16;
-          a.d = l_d + (size_t)t * n_scale;
-          a.upr = upr;
-          int isum, imin;
-          F::template sums<UPR>(cur, a, col, isum, imin);
-          const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
-          if (GEMM_ORDER) {
-            float tmin, tdot;
-            F::term_gemm(cur, ad, isum, imin, tmin, tdot);
-            l_term[(size_t)t * term_stride + i] = tdot;
-            if (NT == 2) l_term[(size_t)(T + t) * term_stride + i] = tmin;
-          } else {
-            l_term[(size_t)t * term_stride + i] = F::term_gemv(cur, ad, isum, imin);
-          }
-          if (DUMP) {
-            const size_t o = ((size_t)t * p.out_dim + row0) * upr + i;
-            if (p.dump_isum) p.dump_isum[o] = isum;
-            if (F::HAS_MIN && p.dump_imin) p.dump_imin[o] = imin;
-          }
-        }
+  // ---- tiles of this wave
+  for (; ct < nct; ct += n_wave) {
+    const uint32_t col = ct * C + c_local;  // block index within the row
+    for (uint32_t t = 0; t < T; t++) {
+      ActLds a;
+      a.xq = l_xq + (size_t)t * xch;
+      a.aux = l_aux + (size_t)t * upr * F::AUX16;
+      a.d = l_d + (size_t)t * n_scale;
+      a.upr = upr;
+      int isum, imin;
+      F::template sums<UPR>(cur, a, col, isum, imin);
+      const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
+      const uint32_t slot = col * R + r_local;
+      if (GEMM_ORDER) {
+        float tmin, tdot;
+        F::term_gemm(cur, ad, isum, imin, tmin, tdot);
+        l_term[(size_t)t * term_stride + slot] = tdot;
+        if (NT == 2) l_term[(size_t)(T + t) * term_stride + slot] = tmin;
+      } else {
+        l_term[(size_t)t * term_stride + slot] = F::term_gemv(cur, ad, isum, imin);
+      }
+      if (DUMP && live) {
+        const size_t o = ((size_t)t * p.out_dim + row) * upr + col;
+        if (p.dump_isum) p.dump_isum[o] = isum;
+        if (F::HAS_MIN && p.dump_imin) p.dump_imin[o] = imin;
       }
     }
-    // The registers are free again: request the next segment's first block now.
-    const uint32_t nseg = seg + total_waves;
-    if (nseg < p.n_seg) F::load(cur, p.wt, min(nseg * seg_units + lane, p.n_units - 1));
-    // One lane per (row, token): the row's block terms in ascending order, one accumulator.
-    // The same wave wrote them and a wave's LDS operations complete in order, so no workgroup
-    // barrier is needed; the wave barrier only pins the compiler's ordering.
-    __builtin_amdgcn_wave_barrier();
-    for (uint32_t i = lane; i < rows_per_seg * T; i += 64) {
-      const uint32_t t = i / rows_per_seg, rl = i - t * rows_per_seg;
-      if (row0 + rl < p.out_dim) {
-        float acc = 0.0f;
-        if (NT == 2) acc = ordered_sum<true>(acc, l_term + (size_t)(T + t) * term_stride + rl * upr, upr);
-        acc = ordered_sum<false>(acc, l_term + (size_t)t * term_stride + rl * upr, upr);
-        p.y[(size_t)t * p.out_dim + row0 + rl] = acc;
-      }
+    if (ct + n_wave < nct) F::load(cur, p.wt, (size_t)rb * nct + ct + n_wave, lane);
+  }
+  __syncthreads();
+
+  // One lane per (row, token): the row's block terms in ascending order, one accumulator.
+  for (uint32_t i = tid; i < R * T; i += nthr) {
+    const uint32_t t = i / R, r = i - t * R;
+    const uint32_t orow = rb * R + r;
+    if (orow < p.out_dim) {
+      float acc = 0.0f;
+      if (NT == 2) acc = ordered_sum<true>(acc, l_term + (size_t)(T + t) * term_stride + r, upr, R);
+      acc = ordered_sum<false>(acc, l_term + (size_t)t * term_stride + r, upr, R);
+      p.y[(size_t)t * p.out_dim + orow] = acc;
     }
-    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -568,48 +554,22 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
 // host side of the launch
 
 static const size_t OGM_LDS_BUDGET = 64 * 1024;
-static const uint32_t OGM_NUM_CU = 256;          // MI355X
-static const uint32_t OGM_WAVES_PER_CU = 16;     // at <= 128 VGPRs
-
-static uint32_t default_wg_waves(uint32_t in_dim) {
-  // Measured on MI355X at 4096 -> 14336 and 14336 -> 4096: four waves per workgroup beat larger
-  // groups even though every group stages its own copy of the activations.
-  (void)in_dim;
-  return 4;
-}
 
 template <class F, bool GEMM_ORDER>
-static uint32_t max_tokens_t(uint32_t in_dim, uint32_t waves) {
+static uint32_t max_tokens_t(uint32_t in_dim) {
   uint32_t t = 8;
-  while (t > 1 && gemv_lds_bytes<F, GEMM_ORDER>(in_dim, t, waves) > OGM_LDS_BUDGET) t--;
+  while (t > 1 && gemv_lds_bytes<F, GEMM_ORDER>(in_dim, t) > OGM_LDS_BUDGET) t--;
   return t;
 }
 
-template <class F>
-static uint32_t resolve_waves(uint32_t in_dim, uint32_t wg_waves) {
-  uint32_t w = wg_waves ? wg_waves : default_wg_waves(in_dim);
-  if (w > (uint32_t)F::MAX_THREADS / 64) w = F::MAX_THREADS / 64;
-  if (w < 1) w = 1;
-  // one token must fit
-  while (w > 1 && gemv_lds_bytes<F, true>(in_dim, 1, w) > OGM_LDS_BUDGET) w--;
-  return w;
-}
-
-uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order,
-                             uint32_t wg_waves) {
+uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order) {
   switch (ggml_type) {
-    case OGM_Q4_K: {
-      uint32_t w = resolve_waves<FmtQ4K>(in_dim, wg_waves);
-      return gemm_order ? max_tokens_t<FmtQ4K, true>(in_dim, w) : max_tokens_t<FmtQ4K, false>(in_dim, w);
-    }
-    case OGM_Q6_K: {
-      uint32_t w = resolve_waves<FmtQ6K>(in_dim, wg_waves);
-      return gemm_order ? max_tokens_t<FmtQ6K, true>(in_dim, w) : max_tokens_t<FmtQ6K, false>(in_dim, w);
-    }
-    case OGM_Q8_0: {
-      uint32_t w = resolve_waves<FmtQ80>(in_dim, wg_waves);
-      return gemm_order ? max_tokens_t<FmtQ80, true>(in_dim, w) : max_tokens_t<FmtQ80, false>(in_dim, w);
-    }
+    case OGM_Q4_K:
+      return gemm_order ? max_tokens_t<FmtQ4K, true>(in_dim) : max_tokens_t<FmtQ4K, false>(in_dim);
+    case OGM_Q6_K:
+      return gemm_order ? max_tokens_t<FmtQ6K, true>(in_dim) : max_tokens_t<FmtQ6K, false>(in_dim);
+    case OGM_Q8_0:
+      return gemm_order ? max_tokens_t<FmtQ80, true>(in_dim) : max_tokens_t<FmtQ80, false>(in_dim);
     default:
       return 0;
   }
@@ -627,20 +587,23 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   p.out_dim = a.out_dim;
   p.upr = a.in_dim / F::ELEMS;
   p.n_tokens = a.n_tokens;
-  p.rows_per_seg = rows_per_seg_for(p.upr);
-  p.n_seg = (a.out_dim + p.rows_per_seg - 1) / p.rows_per_seg;
-  p.seg_units = p.rows_per_seg * p.upr;
-  p.term_stride = (p.seg_units + 3) & ~3u;
-  p.n_units = a.out_dim * p.upr;
-  const uint32_t waves = resolve_waves<F>(a.in_dim, a.wg_waves);
-  const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, waves);
+  const OgmTiling tl = ogm_tiling_for(p.upr, a.out_dim);
+  p.C = tl.C;
+  p.nct = tl.nct;
+  const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens);
   if (lds > OGM_LDS_BUDGET) return hipErrorInvalidValue;
-  // One segment per wave while the whole grid can be resident; beyond that waves loop.
-  const uint32_t max_waves = a.max_waves ? a.max_waves : OGM_NUM_CU * OGM_WAVES_PER_CU;
-  uint32_t want = p.n_seg < max_waves ? p.n_seg : max_waves;
-  uint32_t grid = (want + waves - 1) / waves;
-  if (grid == 0) grid = 1;
-  const dim3 g(grid), b(waves * 64);
+  // Waves per workgroup: the largest divisor of the row block's tile count up to 8 (measured on
+  // MI355X: 4 waves x 1 tile at 4096 -> 14336, 7 waves x 2 tiles at 14336 -> 4096 beat 14 x 1).
+  uint32_t waves = a.wg_waves;
+  if (waves == 0) {
+    waves = 1;
+    for (uint32_t w = 2; w <= 8 && w <= tl.nct; w++)
+      if (tl.nct % w == 0) waves = w;
+  }
+  if (waves > tl.nct) waves = tl.nct;
+  if (waves > (uint32_t)F::MAX_THREADS / 64) waves = F::MAX_THREADS / 64;
+  if (waves == 0) waves = 1;
+  const dim3 g(tl.nrb), b(waves * 64);
   if (a.dump_isum || a.dump_imin) {
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true>), g, b, lds, stream, p);
   } else if (a.n_tokens == 1 && !GEMM_ORDER) {

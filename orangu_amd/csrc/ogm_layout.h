@@ -1,12 +1,19 @@
 // Tile-planar weight layout shared by the host repacker and the device kernels.
 //
-// A matrix is a flat sequence of "units" in row-major order: one unit is one GGUF block
-// (Q8_0: 34 B / 32 weights; Q4_K: 144 B / 256; Q6_K: 210 B / 256; engine/quant.rs:638-787).
-// Units are grouped 64 to a tile.  A unit is cut into 16-byte pieces plus a short tail; inside
-// a tile, piece p of lane l sits at p*1024 + l*16 and the tails follow all pieces, lane after
-// lane.  A wave whose lane l owns unit (tile*64 + l) therefore reads each piece of its 64
-// units as one contiguous, 16-byte-aligned kilobyte, whatever the block size.  No byte of a
-// block is changed, dropped or reinterpreted; the last tile is zero-padded.
+// A matrix is out_dim rows of `upr` blocks ("units"; one unit is one GGUF block: Q8_0 34 B / 32
+// weights, Q4_K 144 B / 256, Q6_K 210 B / 256; engine/quant.rs:638-787).  A *tile* holds 64
+// units: R consecutive rows x C consecutive blocks, with C = 4 when a row has a multiple of four
+// blocks (else 2, else 1) and R = 64 / C.  Tiles are ordered [row block][column tile]; inside a
+// tile the unit of (row r, block c) is lane c*R + r.
+//
+// A unit is cut into 16-byte pieces plus a short tail; piece p of lane l sits at p*1024 + l*16
+// and the tails follow all pieces, lane after lane.  So
+//   * a wave whose lane l owns the tile's unit l reads every piece of its 64 units as one
+//     contiguous, 16-byte-aligned kilobyte, whatever the block size (decode GEMV);
+//   * the R rows of one block column are R consecutive lanes, i.e. a contiguous run of R*16
+//     bytes per piece, which is what a tiled GEMM over a row block fetches (prefill GEMM).
+// No byte of a block is changed, dropped or reinterpreted; rows beyond out_dim in the last row
+// block are zero units.
 //
 //   type   pieces                                   tail
 //   Q8_0   2  (qs[0..32))                           d      (2 B)
@@ -32,6 +39,15 @@ struct OgmLayout {
   uint32_t tile_bytes;    // 64 * block_bytes
 };
 
+// Shape of the tiling of one matrix.
+struct OgmTiling {
+  uint32_t upr;   // blocks per row
+  uint32_t C;     // blocks per tile row (1, 2 or 4)
+  uint32_t R;     // rows per tile (64 / C)
+  uint32_t nct;   // column tiles per row block (upr / C)
+  uint32_t nrb;   // row blocks (ceil(out_dim / R))
+};
+
 #if defined(__HIPCC__) || defined(__CUDACC__)
 #define OGM_HD __host__ __device__
 #else
@@ -52,4 +68,21 @@ OGM_HD inline bool ogm_layout_for(uint32_t ggml_type, OgmLayout *l) {
     default:
       return false;
   }
+}
+
+OGM_HD inline OgmTiling ogm_tiling_for(uint32_t upr, uint32_t out_dim) {
+  OgmTiling t;
+  t.upr = upr;
+  t.C = (upr % 4u == 0) ? 4u : ((upr % 2u == 0) ? 2u : 1u);
+  t.R = OGM_TILE_UNITS / t.C;
+  t.nct = upr / t.C;
+  t.nrb = (out_dim + t.R - 1) / t.R;
+  return t;
+}
+
+// Tile index and lane of the unit (row, block).
+OGM_HD inline void ogm_unit_place(const OgmTiling &t, uint32_t row, uint32_t block, size_t *tile,
+                                  uint32_t *lane) {
+  *tile = (size_t)(row / t.R) * t.nct + block / t.C;
+  *lane = (block % t.C) * t.R + row % t.R;
 }

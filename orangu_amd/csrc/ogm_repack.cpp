@@ -1,5 +1,5 @@
 // Host-side repack of raw GGUF rows into the tile-planar layout, and its exact inverse.
-// The layout itself is described in ogm_layout.h.  Input is QuantMatrix::raw_bytes()
+// The layout itself (64-unit tiles of R rows x C blocks) is described in ogm_layout.h.  Input is QuantMatrix::raw_bytes()
 // (engine/loader.rs:608-610): out_dim rows of row_bytes, rows contiguous.
 #include <string.h>
 
@@ -25,13 +25,13 @@ extern "C" int ogm_block_layout(uint32_t ggml_type, uint32_t *block_bytes, uint3
 }
 
 static size_t n_tiles_for(const OgmLayout &l, uint32_t in_dim, uint32_t out_dim) {
-  size_t units = (size_t)out_dim * (in_dim / l.block_elems);
-  return (units + OGM_TILE_UNITS - 1) / OGM_TILE_UNITS;
+  const OgmTiling t = ogm_tiling_for(in_dim / l.block_elems, out_dim);
+  return (size_t)t.nrb * t.nct;
 }
 
 extern "C" size_t ogm_repacked_size(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim) {
   OgmLayout l;
-  if (!ogm_layout_for(ggml_type, &l) || in_dim % l.block_elems != 0) return 0;
+  if (!ogm_layout_for(ggml_type, &l) || in_dim == 0 || in_dim % l.block_elems != 0) return 0;
   return n_tiles_for(l, in_dim, out_dim) * l.tile_bytes;
 }
 
@@ -53,20 +53,22 @@ extern "C" int ogm_repack_host(uint32_t ggml_type, const void *raw, size_t row_b
   if (!raw || !repacked) return OGM_ERR_INVALID;
   const uint8_t *src = (const uint8_t *)raw;
   uint8_t *dst = (uint8_t *)repacked;
-  // Rows are contiguous and a row is a whole number of blocks, so the matrix is one flat run
-  // of blocks.
-  size_t units = (size_t)out_dim * (in_dim / l.block_elems);
-  size_t tiles = n_tiles_for(l, in_dim, out_dim);
-  size_t last_full = units / OGM_TILE_UNITS;
-  if (last_full < tiles) memset(dst + last_full * l.tile_bytes, 0, l.tile_bytes);
-  for (size_t u = 0; u < units; u++) {
-    const uint8_t *b = src + u * l.block_bytes;
-    uint8_t *tile = dst + (u / OGM_TILE_UNITS) * l.tile_bytes;
-    size_t lane = u % OGM_TILE_UNITS;
-    for (uint32_t p = 0; p < l.pieces; p++)
-      memcpy(tile + p * 1024 + lane * 16, b + l.piece_off + p * 16, 16);
-    if (l.tail_bytes)
-      memcpy(tile + l.pieces * 1024 + lane * l.tail_bytes, b + l.tail_off, l.tail_bytes);
+  const OgmTiling t = ogm_tiling_for(in_dim / l.block_elems, out_dim);
+  // Only the last row block can hold rows beyond out_dim: zero it first.
+  if (out_dim % t.R != 0)
+    memset(dst + (size_t)(t.nrb - 1) * t.nct * l.tile_bytes, 0, (size_t)t.nct * l.tile_bytes);
+  for (uint32_t o = 0; o < out_dim; o++) {
+    for (uint32_t blk = 0; blk < t.upr; blk++) {
+      const uint8_t *b = src + (size_t)o * row_bytes + (size_t)blk * l.block_bytes;
+      size_t tile_index;
+      uint32_t lane;
+      ogm_unit_place(t, o, blk, &tile_index, &lane);
+      uint8_t *tile = dst + tile_index * l.tile_bytes;
+      for (uint32_t p = 0; p < l.pieces; p++)
+        memcpy(tile + p * 1024 + lane * 16, b + l.piece_off + p * 16, 16);
+      if (l.tail_bytes)
+        memcpy(tile + l.pieces * 1024 + lane * l.tail_bytes, b + l.tail_off, l.tail_bytes);
+    }
   }
   return OGM_OK;
 }
@@ -79,15 +81,19 @@ extern "C" int ogm_unrepack_host(uint32_t ggml_type, const void *repacked, size_
   if (!raw || !repacked) return OGM_ERR_INVALID;
   const uint8_t *src = (const uint8_t *)repacked;
   uint8_t *dst = (uint8_t *)raw;
-  size_t units = (size_t)out_dim * (in_dim / l.block_elems);
-  for (size_t u = 0; u < units; u++) {
-    uint8_t *b = dst + u * l.block_bytes;
-    const uint8_t *tile = src + (u / OGM_TILE_UNITS) * l.tile_bytes;
-    size_t lane = u % OGM_TILE_UNITS;
-    for (uint32_t p = 0; p < l.pieces; p++)
-      memcpy(b + l.piece_off + p * 16, tile + p * 1024 + lane * 16, 16);
-    if (l.tail_bytes)
-      memcpy(b + l.tail_off, tile + l.pieces * 1024 + lane * l.tail_bytes, l.tail_bytes);
+  const OgmTiling t = ogm_tiling_for(in_dim / l.block_elems, out_dim);
+  for (uint32_t o = 0; o < out_dim; o++) {
+    for (uint32_t blk = 0; blk < t.upr; blk++) {
+      uint8_t *b = dst + (size_t)o * row_bytes + (size_t)blk * l.block_bytes;
+      size_t tile_index;
+      uint32_t lane;
+      ogm_unit_place(t, o, blk, &tile_index, &lane);
+      const uint8_t *tile = src + tile_index * l.tile_bytes;
+      for (uint32_t p = 0; p < l.pieces; p++)
+        memcpy(b + l.piece_off + p * 16, tile + p * 1024 + lane * 16, 16);
+      if (l.tail_bytes)
+        memcpy(b + l.tail_off, tile + l.pieces * 1024 + lane * l.tail_bytes, l.tail_bytes);
+    }
   }
   return OGM_OK;
 }

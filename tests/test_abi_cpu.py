@@ -42,8 +42,15 @@ def test_supports_predicates_follow_vecdot(lib):
     assert lib.ogm_block_layout(2, None, None) == -2
 
 
+def tiling(upr, out_dim):
+    """ogm_layout.h: tiles of R rows x C blocks, C = 4 / 2 / 1 by divisibility of blocks per row."""
+    C_ = 4 if upr % 4 == 0 else (2 if upr % 2 == 0 else 1)
+    R = 64 // C_
+    return C_, R, upr // C_, (out_dim + R - 1) // R
+
+
 @pytest.mark.parametrize("ggml_type", [Q8_0, Q4_K, Q6_K])
-@pytest.mark.parametrize("in_blocks,out_dim", [(1, 1), (3, 11), (16, 64), (7, 130)])
+@pytest.mark.parametrize("in_blocks,out_dim", [(1, 1), (3, 11), (16, 64), (7, 130), (6, 33), (8, 70)])
 def test_repack_is_a_bijection_on_the_raw_bytes(lib, ggml_type, in_blocks, out_dim):
     bb, be = BLOCK[ggml_type]
     in_dim = in_blocks * be
@@ -51,46 +58,46 @@ def test_repack_is_a_bijection_on_the_raw_bytes(lib, ggml_type, in_blocks, out_d
     rng = np.random.default_rng(in_blocks * 1000 + out_dim)
     raw = rng.integers(0, 256, rb * out_dim, dtype=np.uint8)
     size = lib.ogm_repacked_size(ggml_type, in_dim, out_dim)
-    units = in_blocks * out_dim
-    assert size == (units + 63) // 64 * 64 * bb
+    C_, R, nct, nrb = tiling(in_blocks, out_dim)
+    assert size == nrb * nct * 64 * bb
     packed = np.full(size, 0xAA, np.uint8)
     assert lib.ogm_repack_host(ggml_type, raw.ctypes.data, rb, in_dim, out_dim, packed.ctypes.data) == 0
     back = np.zeros_like(raw)
     assert lib.ogm_unrepack_host(ggml_type, packed.ctypes.data, rb, in_dim, out_dim, back.ctypes.data) == 0
     assert np.array_equal(back, raw)
-    # same multiset of bytes plus zero padding: nothing altered, nothing dropped
-    assert np.array_equal(np.bincount(packed, minlength=256) - np.bincount(raw, minlength=256),
-                          np.eye(1, 256, 0, dtype=np.int64)[0] * (size - raw.size))
+    if out_dim % R == 0:
+        # no padding rows: the packed form is a permutation of the raw bytes
+        assert np.array_equal(np.bincount(packed, minlength=256), np.bincount(raw, minlength=256))
 
 
-def test_repack_places_pieces_in_planes(lib):
-    """Unit u of a Q4_K matrix: piece p at tile*9216 + p*1024 + (u%64)*16."""
-    in_dim, out_dim = 512, 70  # 140 units: 2 full tiles + 12
-    rb = row_bytes(Q4_K, in_dim)
-    raw = np.arange(rb * out_dim, dtype=np.uint32).astype(np.uint8)
-    raw = (np.arange(rb * out_dim) * 2654435761 >> 7).astype(np.uint8)
-    packed = np.zeros(lib.ogm_repacked_size(Q4_K, in_dim, out_dim), np.uint8)
-    lib.ogm_repack_host(Q4_K, raw.ctypes.data, rb, in_dim, out_dim, packed.ctypes.data)
-    for u in (0, 1, 63, 64, 100, 139):
-        for p in range(9):
-            off = (u // 64) * 9216 + p * 1024 + (u % 64) * 16
-            assert np.array_equal(packed[off:off + 16], raw[u * 144 + p * 16:u * 144 + p * 16 + 16])
-    # Q6_K tail (d) and Q8_0 tail (d) land after the planes
-    for t, npieces, tail_off, piece_off in ((Q6_K, 13, 208, 0), (Q8_0, 2, 0, 2)):
-        bb, be = BLOCK[t]
-        in_dim, out_dim = be * 5, 33
-        rb = row_bytes(t, in_dim)
-        raw = (np.arange(rb * out_dim) * 40503 >> 5).astype(np.uint8)
-        packed = np.zeros(lib.ogm_repacked_size(t, in_dim, out_dim), np.uint8)
-        lib.ogm_repack_host(t, raw.ctypes.data, rb, in_dim, out_dim, packed.ctypes.data)
-        for u in (0, 63, 64, 164):
-            base = (u // 64) * 64 * bb
+@pytest.mark.parametrize("t,npieces,piece_off,tail_off,tail", [(Q4_K, 9, 0, 0, 0), (Q6_K, 13, 0, 208, 2),
+                                                              (Q8_0, 2, 2, 0, 2)])
+@pytest.mark.parametrize("in_blocks,out_dim", [(8, 70), (6, 40), (3, 65)])
+def test_repack_places_pieces_in_planes(lib, t, npieces, piece_off, tail_off, tail, in_blocks, out_dim):
+    """Unit (row o, block b): tile (o / R) * nct + b / C, lane (b % C) * R + o % R; piece p at
+    tile * 64 * block_bytes + p * 1024 + lane * 16, tails after the pieces; padding rows zero."""
+    bb, be = BLOCK[t]
+    in_dim = in_blocks * be
+    rb = row_bytes(t, in_dim)
+    raw = ((np.arange(rb * out_dim, dtype=np.uint64) * 2654435761) >> 7).astype(np.uint8)
+    C_, R, nct, nrb = tiling(in_blocks, out_dim)
+    packed = np.full(lib.ogm_repacked_size(t, in_dim, out_dim), 0x5A, np.uint8)
+    assert lib.ogm_repack_host(t, raw.ctypes.data, rb, in_dim, out_dim, packed.ctypes.data) == 0
+    seen = np.zeros(packed.size, bool)
+    for o in range(out_dim):
+        for b in range(in_blocks):
+            base = ((o // R) * nct + b // C_) * 64 * bb
+            lane = (b % C_) * R + o % R
+            src = o * rb + b * bb
             for p in range(npieces):
-                off = base + p * 1024 + (u % 64) * 16
-                src = u * bb + piece_off + p * 16
-                assert np.array_equal(packed[off:off + 16], raw[src:src + 16])
-            off = base + npieces * 1024 + (u % 64) * 2
-            assert np.array_equal(packed[off:off + 2], raw[u * bb + tail_off:u * bb + tail_off + 2])
+                off = base + p * 1024 + lane * 16
+                assert np.array_equal(packed[off:off + 16], raw[src + piece_off + p * 16:src + piece_off + p * 16 + 16])
+                seen[off:off + 16] = True
+            if tail:
+                off = base + npieces * 1024 + lane * tail
+                assert np.array_equal(packed[off:off + tail], raw[src + tail_off:src + tail_off + tail])
+                seen[off:off + tail] = True
+    assert not packed[~seen].any()  # rows that pad the last row block are zero units
 
 
 def test_repack_rejects_bad_shapes(lib):
