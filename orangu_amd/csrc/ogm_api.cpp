@@ -41,9 +41,10 @@ struct ogm_ctx {
   std::vector<ogm_weight *> weights;
   // scratch, grown on demand and reused (the vendor backends allocate per call,
   // engine/backend/rocm.rs:352-376; a pool is what the Vulkan op_cache does instead)
-  DevBuf x, y, q, d, sums, bsum, isum, imin;
+  DevBuf x, y, q, d, sums, bsum, isum, imin, xh;
   DevBuf hx, hy;  // pinned host staging
   int tune_wg_waves = 0;
+  int tune_gemm_min_tokens = 9;  // matmul at n_tokens >= this takes the MFMA GEMM
   const char *last_kernel = "";
   // what the activation buffer currently holds (ogm_act_quantize_dev)
   int act_mode = -1;
@@ -160,7 +161,7 @@ extern "C" void ogm_destroy(ogm_ctx *ctx) {
     if (w->dev) (void)hipFree(w->dev);
     delete w;
   }
-  DevBuf *dev[] = {&ctx->x, &ctx->y, &ctx->q, &ctx->d, &ctx->sums, &ctx->bsum, &ctx->isum, &ctx->imin};
+  DevBuf *dev[] = {&ctx->x, &ctx->y, &ctx->q, &ctx->d, &ctx->sums, &ctx->bsum, &ctx->isum, &ctx->imin, &ctx->xh};
   for (DevBuf *b : dev)
     if (b->p) (void)hipFree(b->p);
   if (ctx->hx.p) (void)hipHostFree(ctx->hx.p);
@@ -192,6 +193,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemv_wg_waves") == 0) {
     if (value < 0 || value > 16) return fail(ctx, OGM_ERR_INVALID, "gemv_wg_waves must be 0..16");
     ctx->tune_wg_waves = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_min_tokens") == 0) {
+    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_min_tokens must be >= 0");
+    ctx->tune_gemm_min_tokens = value ? value : 9;
     return OGM_OK;
   }
   return fail(ctx, OGM_ERR_INVALID, std::string("unknown tuning key ") + key);
@@ -334,6 +340,23 @@ static int enqueue_gemv(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, fl
   // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
   // n_tokens == 1 and every matmul_decode take the GEMV's.
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
+  if (gemm_order && !dump_isum && !dump_imin && n_tokens >= (uint32_t)ctx->tune_gemm_min_tokens &&
+      ogm_gemm_supported(w->ggml_type, w->in_dim)) {
+    // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
+    int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w->in_dim, n_tokens));
+    if (rc != OGM_OK) return rc;
+    OgmGemmArgs g;
+    g.ggml_type = w->ggml_type;
+    g.wt = w->dev;
+    g.in_dim = w->in_dim;
+    g.out_dim = w->out_dim;
+    g.act = act_view(ctx, w->in_dim, mode, 0);
+    g.n_tokens = n_tokens;
+    g.y = y_dev;
+    g.xh = ctx->xh.p;
+    HIPCHK(ctx, ogm_launch_gemm(g, stream, &ctx->last_kernel));
+    return OGM_OK;
+  }
   const uint32_t wg_waves = (uint32_t)ctx->tune_wg_waves;
   const uint32_t chunk = ogm_gemv_max_tokens(w->ggml_type, w->in_dim, gemm_order);
   if (chunk == 0) return fail(ctx, OGM_ERR_UNSUPPORTED, "no kernel for this type");

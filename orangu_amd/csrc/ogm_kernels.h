@@ -36,4 +36,19 @@ struct OgmGemvArgs {
 uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order);
 hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name);
 
+// Prefill GEMM on MFMA (ogm_gemm.hip).  Same operands as the GEMV plus a scratch buffer `xh` of
+// ogm_gemm_xh_bytes() for the activations as f16.  Follows the CPU path's GEMM float order.
+struct OgmGemmArgs {
+  uint32_t ggml_type;
+  const uint8_t *wt;
+  uint32_t in_dim, out_dim;
+  OgmActDev act;       // per-256 quantized activations of all n_tokens
+  uint32_t n_tokens;
+  float *y;            // [n_tokens][out_dim]
+  void *xh;            // scratch
+};
+bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim);
+size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens);
+hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name);
+
 hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hipStream_t stream);

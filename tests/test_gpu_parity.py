@@ -309,3 +309,61 @@ def test_q6k_vocab_projection_batches_1_4_8(be):
     y1 = be.matmul(x[:1], 1, w)
     y2 = be.matmul(x[:1] * np.float32(4.0), 1, w)
     assert_bits(y2, y1 * np.float32(4.0), "scaling by 4")
+
+
+# ---------------------------------------------------------------- prefill GEMM on MFMA
+
+@pytest.mark.parametrize("in_dim,out_dim,T", [
+    (1024, 64, 9), (1024, 100, 64), (2048, 37, 128), (4096, 200, 130), (1024, 16, 300), (8192, 70, 33),
+])
+def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
+    """ogm_matmul at n_tokens >= 9 takes the MFMA kernel; values must equal CpuBackend's K-quant
+    GEMM (vecdot.rs:2213-2303): integer sums exact on the matrix cores, f32 order the reference's."""
+    raw = synth_weights(Q4_K, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T)
+    w = qm(raw, Q4_K, in_dim, out_dim)
+    say("gemm", in_dim, out_dim, T)
+    got = be.matmul(x, T, w)
+    assert be.last_kernel() == "ogm_gemm_q4k_kernel"
+    want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
+    assert_close(got, want, "mfma gemm")
+    assert_bits(got, want, "mfma gemm")
+
+
+def test_mfma_gemm_equals_small_batch_kernel_and_is_batch_independent(be):
+    """The two GPU kernels that serve ogm_matmul (multi-token GEMV below 9 tokens, MFMA GEMM above)
+    must agree bit for bit, and a token's result must not depend on the batch (vecdot.rs:4522-4549)."""
+    in_dim, out_dim = 2048, 48
+    raw, _ = k_fixture(Q4_K, in_dim, out_dim, 1, 77)
+    x = synth_x(40, in_dim, seed=5)
+    w = qm(raw, Q4_K, in_dim, out_dim)
+    full = be.matmul(x, 40, w).reshape(40, out_dim)
+    be.set_tuning("gemm_min_tokens", 1000)
+    try:
+        small = be.matmul(x, 40, w).reshape(40, out_dim)
+        assert be.last_kernel().startswith("ogm_gemv_kernel")
+    finally:
+        be.set_tuning("gemm_min_tokens", 0)
+    assert_bits(full, small, "mfma vs multi-token gemv")
+    for n in (9, 17, 33):
+        part = be.matmul(x[:n], n, w).reshape(n, out_dim)
+        assert_bits(part, full[:n], f"{n} of 40")
+
+
+def test_mfma_gemm_adversarial_integer_ranges(be):
+    """Largest magnitudes the integer stage can see: all nibbles 15, scales and mins 63, activations
+    +-127: the per-super-block sum (3.1e7) exceeds 2^24, so the two-half f32 add must round exactly
+    like `isum as f32`."""
+    in_dim, out_dim, T = 1024, 32, 16
+    blocks = np.zeros((out_dim * 4, 144), np.uint8)
+    blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    blocks[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
+    blocks[:, 4:16] = 0xFF
+    blocks[:, 16:] = 0xFF
+    x = np.full((T, in_dim), 127.0, np.float32)
+    x[1::2] *= -1
+    x[:, ::7] = 126.0
+    raw = blocks.reshape(-1)
+    got = be.matmul(x, T, qm(raw, Q4_K, in_dim, out_dim))
+    want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
+    assert_bits(got, want, "extreme ranges")
