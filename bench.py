@@ -4,12 +4,12 @@
 Workload (the configuration the headline metric is quoted on): batch-1 decode GEMVs of a
 Llama-3-8B feed-forward block in Q4_K -- gate and up 4096 -> 14336 and down 14336 -> 4096 --
 on seeded synthetic weights and N(0,1) activations.  One step is one pass over that block: the
-activation quantizer plus the GEMV for each of the three matrices, through the library's C ABI
-with inputs and outputs resident in HBM.  Steps rotate over enough distinct weight copies that
+activation quantizer and one GEMV launch over gate and up (they read the same input), then the
+quantizer and the GEMV for down, through the library's C ABI with inputs and outputs resident in HBM.  Steps rotate over enough distinct weight copies that
 every pass streams from HBM rather than from the last-level cache.
 
 Prints ONE JSON line: whole-step throughput in algorithmic GB/s, a roofline object for the
-dominant kernel (the Q4_K GEMV at 4096 -> 14336, timed with HIP events over back-to-back
+dominant kernel (the Q4_K GEMV over gate+up, timed with HIP events over back-to-back
 launches) and the CPU path (the C oracle, all host cores) timed on a bounded sample.
 """
 from __future__ import annotations
@@ -31,7 +31,7 @@ HIDDEN, FFN = 4096, 14336
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of `bench.py --only-roofline`, calibrated on that run's 64 MiB copy (profiles/).
-GEMV_Q4K_4096x14336_TRAFFIC = 33175858
+GEMV_Q4K_GATE_UP_TRAFFIC = 66243599
 
 
 def gemv_bytes(in_dim: int, out_dim: int, t: int = 1) -> int:
@@ -49,6 +49,11 @@ def main() -> int:
     ap.add_argument("--roofline-launches", type=int, default=600)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--wg-waves", type=int, default=0, help="waves per workgroup override (0 = heuristic)")
+    ap.add_argument("--fuse-quant", type=int, default=-1,
+                    help="quantize inside the GEMV: -1 library's choice, 0 never, 1 always")
+    ap.add_argument("--rb-per-wg", type=int, default=0, help="row blocks per GEMV workgroup (0 = heuristic)")
+    ap.add_argument("--separate", action="store_true",
+                    help="issue gate and up as two calls instead of one grouped call")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the dominant-kernel leg (for rocprofv3 --kernel-trace --stats)")
     args = ap.parse_args()
@@ -65,6 +70,10 @@ def main() -> int:
     be = Mi355xBackend()  # raises without the HIP library or a gfx950 device
     if args.wg_waves:
         be.set_tuning("gemv_wg_waves", args.wg_waves)
+    if args.rb_per_wg:
+        be.set_tuning("gemv_rb_per_wg", args.rb_per_wg)
+    if args.fuse_quant != -1:
+        be.set_tuning("gemv_fuse_quant", args.fuse_quant)
     stream = hiprt.Stream()
 
     # ---- synthetic inputs -------------------------------------------------------------------
@@ -81,9 +90,15 @@ def main() -> int:
                             hiprt.DeviceBuffer(4 * HIDDEN))
 
     def step(i: int):
+        # gate and up read the same input and go out as one call, as the forward pass batches
+        # them (engine/arch/mod.rs:1082-1096); down follows on its own input.
         c = i % copies
-        be.matmul_dev(handles["gate"][c], x_d.ptr, 1, y_gate.ptr, False, stream.ptr)
-        be.matmul_dev(handles["up"][c], x_d.ptr, 1, y_up.ptr, False, stream.ptr)
+        if args.separate:
+            be.matmul_dev(handles["gate"][c], x_d.ptr, 1, y_gate.ptr, False, stream.ptr)
+            be.matmul_dev(handles["up"][c], x_d.ptr, 1, y_up.ptr, False, stream.ptr)
+        else:
+            be.matmul_multi_dev([handles["gate"][c], handles["up"][c]], x_d.ptr, 1,
+                                [y_gate.ptr, y_up.ptr], False, stream.ptr)
         be.matmul_dev(handles["down"][c], h_d.ptr, 1, y_down.ptr, False, stream.ptr)
 
     step_bytes = 2 * gemv_bytes(HIDDEN, FFN) + gemv_bytes(FFN, HIDDEN)
@@ -104,22 +119,41 @@ def main() -> int:
         result["ms_per_step"] = ms_per_step
         result["value"] = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- dominant kernel: Q4_K GEMV 4096 -> 14336, back-to-back, HIP events on its stream -----
-    mats = handles["gate"] + handles["up"]
-    be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr)
-    for i in range(50):
-        be.matmul_act_dev(mats[i % len(mats)], 1, y_gate.ptr, False, stream.ptr)
-    stream.synchronize()
-    e0, e1 = hiprt.Event(), hiprt.Event()
+    # ---- dominant kernel: the Q4_K GEMV over gate+up (4096 -> 2 x 14336 in one launch), ---------
+    # back-to-back over pre-quantized activations, HIP events on its stream
+    def timed(launch, n):
+        for i in range(50):
+            launch(i)
+        stream.synchronize()
+        e0, e1 = hiprt.Event(), hiprt.Event()
+        e0.record(stream)
+        for i in range(n):
+            launch(i)
+        e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_ms(e1) * 1e3 / n
+
     n_launch = args.roofline_launches
-    e0.record(stream)
-    for i in range(n_launch):
-        be.matmul_act_dev(mats[i % len(mats)], 1, y_gate.ptr, False, stream.ptr)
-    e1.record(stream)
-    e1.synchronize()
-    us_per_launch = e0.elapsed_ms(e1) * 1e3 / n_launch
-    kbytes = gemv_bytes(HIDDEN, FFN)
+    be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr)
+    us_per_launch = timed(lambda i: be.matmul_multi_act_dev(
+        [handles["gate"][i % copies], handles["up"][i % copies]], 1, [y_gate.ptr, y_up.ptr], False,
+        stream.ptr), n_launch)
+    kernel_name = be.last_kernel()
+    kbytes = 2 * gemv_bytes(HIDDEN, FFN) - 4 * HIDDEN  # both matrices read the same x
     achieved = kbytes / (us_per_launch * 1e-6) / 1e9
+    others = None
+    if not args.only_roofline:
+        # the other launch shapes of the step, for the record (left out of the profiled run so
+        # that the trace's average for the GEMV kernel covers the gate+up launches only)
+        mats = handles["gate"] + handles["up"]
+        us_one = timed(lambda i: be.matmul_act_dev(mats[i % len(mats)], 1, y_gate.ptr, False, stream.ptr),
+                       n_launch)
+        be.act_quantize_dev(Q4_K, h_d.ptr, FFN, 1, stream.ptr)
+        us_down = timed(lambda i: be.matmul_act_dev(handles["down"][i % copies], 1, y_down.ptr, False,
+                                                    stream.ptr), n_launch)
+        us_quant = timed(lambda i: be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr), n_launch)
+        others = {"gemv 4096->14336 alone": round(us_one, 3), "gemv 14336->4096": round(us_down, 3),
+                  "activation quantize 4096": round(us_quant, 3)}
     if args.only_roofline:
         # One plain device-to-device copy of known size: under `rocprofv3 --pmc FETCH_SIZE` /
         # `WRITE_SIZE` its counter reading calibrates the GEMV's (bytes per counter unit).
@@ -129,9 +163,10 @@ def main() -> int:
         hiprt.check(hiprt.hip().hipMemcpy(dst.ptr, src.ptr, cal, 3), "hipMemcpy D2D")
         hiprt.device_synchronize()
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_Q4K_4096x14336_TRAFFIC,
-                "kernel": be.last_kernel(), "us_per_launch": round(us_per_launch, 3),
-                "bytes_per_launch": kbytes, "launches": n_launch}
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_Q4K_GATE_UP_TRAFFIC,
+                "kernel": kernel_name + " over gate+up", "us_per_launch": round(us_per_launch, 3),
+                "bytes_per_launch": kbytes, "launches": n_launch,
+                "other_launches_us": others}
 
     # ---- parity of what was just timed + CPU baseline (the oracle, all host cores) -------------
     cpu = None
@@ -189,7 +224,8 @@ def main() -> int:
         "dtype": "i8 dot / i32 block sums / f32 combine",
         "data": "synthetic",
         "config": {"workload": "configs[1]: Q4_K decode GEMV batch 1, gate+up 4096->14336 and down "
-                               "14336->4096; step = 3 x (activation quantize + GEMV)",
+                               "14336->4096; step = quantize(x) + GEMV over gate and up in one launch + "
+                               "quantize(h) + GEMV down",
                    "algorithmic_bytes_per_step": step_bytes, "weight_copies": copies,
                    "frac_of_hbm_peak": round(result.get("value", achieved) / HBM_PEAK_GBS, 4),
                    "parity_vs_cpu": parity, "device": be.device_name()},

@@ -147,6 +147,18 @@ int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev, u
 int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, float *y_dev,
                        int decode, void *stream);
 
+/* Several weights of one type and in_dim over the same device-resident input, as the forward pass
+ * issues them (q/k/v and gate/up: engine/arch/mod.rs:1082-1096, through Backend::matmul_batch,
+ * backend/mod.rs:362-366): the input is quantized once and, at one token, a single kernel launch
+ * covers all the weights.  ys_dev[i] is [n_tokens][ws[i].out_dim].  Values equal ogm_matmul_dev
+ * per weight. */
+int ogm_matmul_multi_dev(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n_ws, const float *x_dev,
+                         uint32_t n_tokens, float *const *ys_dev, int decode, void *stream);
+/* The same over activations already quantized by ogm_act_quantize_dev (the grouped form of
+ * ogm_matmul_act_dev). */
+int ogm_matmul_multi_act_dev(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n_ws,
+                             uint32_t n_tokens, float *const *ys_dev, int decode, void *stream);
+
 /* ---- the integer stage, exposed for parity checks ------------------------------------------- */
 
 /* The fused activation quantizer on its own.  mode OGM_ACT_PER_32: d has n/32 entries
@@ -171,7 +183,10 @@ int ogm_f16_to_f32(ogm_ctx *ctx, const uint16_t *bits, size_t n, float *out);
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.
  * keys: "gemv_wg_waves" (waves per workgroup of the GEMV kernel, 1..16; 0 = heuristic);
  * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default 9,
- * below it the multi-token GEMV kernel runs in the GEMM's float order). */
+ * below it the multi-token GEMV kernel runs in the GEMM's float order);
+ * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
+ * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
+ * the quantizer kernel first; 0 or -1 = default, off).  No setting changes a result bit. */
 int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value);
 /* Name of the kernel the last matmul on this context launched (for profiles). */
 const char *ogm_last_kernel(ogm_ctx *ctx);

@@ -241,6 +241,24 @@ class Mi355xBackend:
         self._check(self._lib.ogm_matmul_act_dev(self._ctx, w_handle, n_tokens, y_ptr, int(decode),
                                                  stream or None), "ogm_matmul_act_dev")
 
+    def matmul_multi_dev(self, w_handles, x_ptr: int, n_tokens: int, y_ptrs, decode: bool = False,
+                         stream: int = 0):
+        """Several weights over one device-resident input (q/k/v, gate/up): one quantize, and at
+        one token one launch."""
+        n = len(w_handles)
+        ws = (C.c_void_p * n)(*w_handles)
+        ys = (C.c_void_p * n)(*y_ptrs)
+        self._check(self._lib.ogm_matmul_multi_dev(self._ctx, ws, n, x_ptr, n_tokens, ys, int(decode),
+                                                   stream or None), "ogm_matmul_multi_dev")
+
+    def matmul_multi_act_dev(self, w_handles, n_tokens: int, y_ptrs, decode: bool = False, stream: int = 0):
+        """The grouped call over activations quantized by act_quantize_dev."""
+        n = len(w_handles)
+        ws = (C.c_void_p * n)(*w_handles)
+        ys = (C.c_void_p * n)(*y_ptrs)
+        self._check(self._lib.ogm_matmul_multi_act_dev(self._ctx, ws, n, n_tokens, ys, int(decode),
+                                                       stream or None), "ogm_matmul_multi_act_dev")
+
     def upload_raw(self, raw: np.ndarray, ggml_type: int, in_dim: int, out_dim: int) -> int:
         """Uploads without a cache key: every call makes a new device copy."""
         raw = np.ascontiguousarray(raw, np.uint8)

@@ -22,7 +22,7 @@ SYMBOLS = [
     "ogm_unrepack_host", "ogm_weight_upload", "ogm_weight_download", "ogm_weight_free",
     "ogm_weight_info", "ogm_matmul", "ogm_matmul_decode", "ogm_matmul_batch", "ogm_matmul_dev",
     "ogm_quantize_act", "ogm_dump_block_sums", "ogm_f16_to_f32", "ogm_set_tuning",
-    "ogm_last_kernel", "ogm_act_quantize_dev", "ogm_matmul_act_dev",
+    "ogm_last_kernel", "ogm_act_quantize_dev", "ogm_matmul_act_dev", "ogm_matmul_multi_dev", "ogm_matmul_multi_act_dev",
 ]
 
 
@@ -71,6 +71,8 @@ def load_library() -> C.CDLL:
     L.ogm_matmul_dev.argtypes = [vp, vp, vp, u32, vp, C.c_int, vp]
     L.ogm_act_quantize_dev.argtypes = [vp, u32, vp, u32, u32, vp]
     L.ogm_matmul_act_dev.argtypes = [vp, vp, u32, vp, C.c_int, vp]
+    L.ogm_matmul_multi_dev.argtypes = [vp, C.POINTER(vp), sz, vp, u32, C.POINTER(vp), C.c_int, vp]
+    L.ogm_matmul_multi_act_dev.argtypes = [vp, C.POINTER(vp), sz, u32, C.POINTER(vp), C.c_int, vp]
     L.ogm_quantize_act.argtypes = [vp, C.c_int, vp, sz, vp, vp, vp]
     L.ogm_dump_block_sums.argtypes = [vp, vp, vp, u32, vp, vp]
     L.ogm_f16_to_f32.argtypes = [vp, vp, sz, vp]

@@ -45,6 +45,8 @@ struct ogm_ctx {
   DevBuf hx, hy;  // pinned host staging
   int tune_wg_waves = 0;
   int tune_gemm_min_tokens = 9;  // matmul at n_tokens >= this takes the MFMA GEMM
+  int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
+  int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
   const char *last_kernel = "";
   // what the activation buffer currently holds (ogm_act_quantize_dev)
   int act_mode = -1;
@@ -200,6 +202,16 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_gemm_min_tokens = value ? value : 9;
     return OGM_OK;
   }
+  if (strcmp(key, "gemv_rb_per_wg") == 0) {
+    if (value < 0 || value > 64) return fail(ctx, OGM_ERR_INVALID, "gemv_rb_per_wg must be 0..64");
+    ctx->tune_rb_per_wg = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemv_fuse_quant") == 0) {
+    if (value < -1 || value > 1) return fail(ctx, OGM_ERR_INVALID, "gemv_fuse_quant must be -1, 0 or 1");
+    ctx->tune_fuse_quant = value < 0 ? 0 : value;  // -1 = the default
+    return OGM_OK;
+  }
   return fail(ctx, OGM_ERR_INVALID, std::string("unknown tuning key ") + key);
 }
 
@@ -320,61 +332,101 @@ static int enqueue_quantize(ogm_ctx *ctx, int mode, const float *x_dev, uint32_t
   return OGM_OK;
 }
 
-static int enqueue_gemv(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, float *y_dev,
-                        int decode, hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin);
+// One matrix and where its output goes; a group shares type, in_dim and the activations.
+struct Target {
+  const ogm_weight *w;
+  float *y;
+};
 
-// Enqueues quantize + kernels for tokens of x_dev into y_dev.  Caller holds the lock.
+static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
+                        hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
+                        const float *x_f32);
+
+// Whether a single-token launch quantizes inside the GEMV (every workgroup repeats the
+// quantizer on its way in) instead of running the quantizer kernel first.  Off unless asked
+// for: on MI355X the repeated work costs more than the launch it saves (Llama-8B FFN block:
+// 28.3 us per pass against 25.9 us).
+static bool fuse_quantize(ogm_ctx *ctx, const Target *, size_t) { return ctx->tune_fuse_quant > 0; }
+
+// Enqueues quantize + kernels for tokens of x_dev into the targets' outputs.  Caller holds the
+// lock and has checked that the targets share type and in_dim.
+static int enqueue_matmul(ogm_ctx *ctx, const Target *tg, size_t n_tg, const float *x_dev,
+                          uint32_t n_tokens, int decode, hipStream_t stream, int32_t *dump_isum,
+                          int32_t *dump_imin) {
+  if (n_tokens == 0 || n_tg == 0) return OGM_OK;
+  const ogm_weight *w = tg[0].w;
+  if (n_tokens == 1 && !dump_isum && !dump_imin && fuse_quantize(ctx, tg, n_tg))
+    return enqueue_gemv(ctx, tg, n_tg, 1, decode, stream, nullptr, nullptr, x_dev);
+  int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type), x_dev, w->in_dim, n_tokens, stream);
+  if (rc != OGM_OK) return rc;
+  return enqueue_gemv(ctx, tg, n_tg, n_tokens, decode, stream, dump_isum, dump_imin, nullptr);
+}
+
 static int enqueue_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
                           float *y_dev, int decode, hipStream_t stream, int32_t *dump_isum,
                           int32_t *dump_imin) {
-  if (n_tokens == 0) return OGM_OK;
-  int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type), x_dev, w->in_dim, n_tokens, stream);
-  if (rc != OGM_OK) return rc;
-  return enqueue_gemv(ctx, w, n_tokens, y_dev, decode, stream, dump_isum, dump_imin);
+  const Target t{w, y_dev};
+  return enqueue_matmul(ctx, &t, 1, x_dev, n_tokens, decode, stream, dump_isum, dump_imin);
 }
 
-// Enqueues the matmul kernels over the context's quantized activations.  Caller holds the lock.
-static int enqueue_gemv(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, float *y_dev,
-                        int decode, hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin) {
-  const int mode = act_mode_for(w->ggml_type);
+// Enqueues the matmul kernels over the context's quantized activations (or, with x_f32, over
+// one token of f32 activations that the kernel quantizes itself).  Caller holds the lock.
+static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
+                        hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
+                        const float *x_f32) {
+  const ogm_weight *w0 = tg[0].w;
+  const int mode = act_mode_for(w0->ggml_type);
   // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
   // n_tokens == 1 and every matmul_decode take the GEMV's.
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
   if (gemm_order && !dump_isum && !dump_imin && n_tokens >= (uint32_t)ctx->tune_gemm_min_tokens &&
-      ogm_gemm_supported(w->ggml_type, w->in_dim)) {
+      ogm_gemm_supported(w0->ggml_type, w0->in_dim)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
-    int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w->in_dim, n_tokens));
+    int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w0->in_dim, n_tokens));
     if (rc != OGM_OK) return rc;
-    OgmGemmArgs g;
-    g.ggml_type = w->ggml_type;
-    g.wt = w->dev;
-    g.in_dim = w->in_dim;
-    g.out_dim = w->out_dim;
-    g.act = act_view(ctx, w->in_dim, mode, 0);
-    g.n_tokens = n_tokens;
-    g.y = y_dev;
-    g.xh = ctx->xh.p;
-    HIPCHK(ctx, ogm_launch_gemm(g, stream, &ctx->last_kernel));
+    for (size_t i = 0; i < n_tg; i++) {
+      OgmGemmArgs g;
+      g.ggml_type = w0->ggml_type;
+      g.wt = tg[i].w->dev;
+      g.in_dim = w0->in_dim;
+      g.out_dim = tg[i].w->out_dim;
+      g.act = act_view(ctx, w0->in_dim, mode, 0);
+      g.n_tokens = n_tokens;
+      g.y = tg[i].y;
+      g.xh = ctx->xh.p;
+      HIPCHK(ctx, ogm_launch_gemm(g, stream, &ctx->last_kernel));
+    }
     return OGM_OK;
   }
   const uint32_t wg_waves = (uint32_t)ctx->tune_wg_waves;
-  const uint32_t chunk = ogm_gemv_max_tokens(w->ggml_type, w->in_dim, gemm_order);
+  const uint32_t chunk = ogm_gemv_max_tokens(w0->ggml_type, w0->in_dim, gemm_order);
   if (chunk == 0) return fail(ctx, OGM_ERR_UNSUPPORTED, "no kernel for this type");
-  const uint32_t blocks_per_row = w->in_dim / (w->ggml_type == OGM_Q8_0 ? 32 : 256);
-  for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
-    OgmGemvArgs a;
-    a.ggml_type = w->ggml_type;
-    a.wt = w->dev;
-    a.in_dim = w->in_dim;
-    a.out_dim = w->out_dim;
-    a.act = act_view(ctx, w->in_dim, mode, t0);
-    a.n_tokens = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
-    a.y = y_dev + (size_t)t0 * w->out_dim;
-    a.gemm_order = gemm_order;
-    a.wg_waves = wg_waves;
-    a.dump_isum = dump_isum ? dump_isum + (size_t)t0 * w->out_dim * blocks_per_row : nullptr;
-    a.dump_imin = dump_imin ? dump_imin + (size_t)t0 * w->out_dim * blocks_per_row : nullptr;
-    HIPCHK(ctx, ogm_launch_gemv(a, stream, &ctx->last_kernel));
+  const uint32_t blocks_per_row = w0->in_dim / (w0->ggml_type == OGM_Q8_0 ? 32 : 256);
+  for (size_t g0 = 0; g0 < n_tg; g0 += OGM_GEMV_MAX_MATS) {
+    const size_t ng = n_tg - g0 < OGM_GEMV_MAX_MATS ? n_tg - g0 : OGM_GEMV_MAX_MATS;
+    for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
+      OgmGemvArgs a;
+      a.ggml_type = w0->ggml_type;
+      a.wt = tg[g0].w->dev;
+      a.in_dim = w0->in_dim;
+      a.out_dim = tg[g0].w->out_dim;
+      a.act = act_view(ctx, w0->in_dim, mode, t0);
+      a.n_tokens = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
+      a.y = tg[g0].y + (size_t)t0 * a.out_dim;
+      a.gemm_order = gemm_order;
+      a.wg_waves = wg_waves;
+      a.rb_per_wg = (uint32_t)ctx->tune_rb_per_wg;
+      a.dump_isum = dump_isum ? dump_isum + (size_t)t0 * a.out_dim * blocks_per_row : nullptr;
+      a.dump_imin = dump_imin ? dump_imin + (size_t)t0 * a.out_dim * blocks_per_row : nullptr;
+      a.n_extra = (uint32_t)ng - 1;
+      for (size_t i = 1; i < ng; i++) {
+        a.extra_wt[i - 1] = tg[g0 + i].w->dev;
+        a.extra_out_dim[i - 1] = tg[g0 + i].w->out_dim;
+        a.extra_y[i - 1] = tg[g0 + i].y + (size_t)t0 * tg[g0 + i].w->out_dim;
+      }
+      a.x_f32 = x_f32;
+      HIPCHK(ctx, ogm_launch_gemv(a, stream, &ctx->last_kernel));
+    }
   }
   return OGM_OK;
 }
@@ -455,7 +507,55 @@ extern "C" int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_
                 "(call ogm_act_quantize_dev with its type, in_dim and token count first)");
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
-  return enqueue_gemv(ctx, w, n_tokens, y_dev, decode, s, nullptr, nullptr);
+  const Target t{w, y_dev};
+  return enqueue_gemv(ctx, &t, 1, n_tokens, decode, s, nullptr, nullptr, nullptr);
+}
+
+// Checks a group of weights and collects its targets.
+static int group_targets(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n_ws, const void *x,
+                         uint32_t n_tokens, float *const *ys_dev, std::vector<Target> &tg) {
+  if (!ws || !ys_dev) return fail(ctx, OGM_ERR_INVALID, "ws or ys is null");
+  tg.resize(n_ws);
+  for (size_t i = 0; i < n_ws; i++) {
+    int rc = check_matmul_args(ctx, ws[i], x, ys_dev[i], n_tokens);
+    if (rc != OGM_OK) return rc;
+    if (ws[i]->ggml_type != ws[0]->ggml_type || ws[i]->in_dim != ws[0]->in_dim)
+      return fail(ctx, OGM_ERR_INVALID, "weights of one call must share type and in_dim");
+    tg[i] = Target{ws[i], ys_dev[i]};
+  }
+  return OGM_OK;
+}
+
+extern "C" int ogm_matmul_multi_dev(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n_ws,
+                                    const float *x_dev, uint32_t n_tokens, float *const *ys_dev,
+                                    int decode, void *stream) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (n_ws == 0) return OGM_OK;
+  std::vector<Target> tg;
+  int rc = group_targets(ctx, ws, n_ws, x_dev, n_tokens, ys_dev, tg);
+  if (rc != OGM_OK) return rc;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
+  return enqueue_matmul(ctx, tg.data(), n_ws, x_dev, n_tokens, decode, s, nullptr, nullptr);
+}
+
+extern "C" int ogm_matmul_multi_act_dev(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n_ws,
+                                        uint32_t n_tokens, float *const *ys_dev, int decode,
+                                        void *stream) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (n_ws == 0 || n_tokens == 0) return OGM_OK;
+  std::vector<Target> tg;
+  int rc = group_targets(ctx, ws, n_ws, ys_dev /* stands in for x: only null-checked */, n_tokens, ys_dev, tg);
+  if (rc != OGM_OK) return rc;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (ctx->act_mode != act_mode_for(ws[0]->ggml_type) || ctx->act_in_dim != ws[0]->in_dim ||
+      ctx->act_tokens < n_tokens)
+    return fail(ctx, OGM_ERR_INVALID, "the quantized activations do not fit these weights "
+                "(call ogm_act_quantize_dev with their type, in_dim and token count first)");
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
+  return enqueue_gemv(ctx, tg.data(), n_ws, n_tokens, decode, s, nullptr, nullptr, nullptr);
 }
 
 // Backend::matmul_batch (backend/mod.rs:362-366) with guarded_matmul_op's token stripes
@@ -472,12 +572,23 @@ extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, i
   }
   std::lock_guard<std::mutex> lock(ctx->mu);
   HIPCHK(ctx, hipSetDevice(ctx->device));
-  // All ops share the activation scratch, so x / y of every op get their own slice of the
-  // transfer buffers but the quantized activations are consumed before the next op's quantize
-  // (same stream, in order).
+  // Every op gets its own slice of the transfer buffers; the activation scratch is shared,
+  // which is safe because one stream runs each quantize after the kernels that read the last.
+  // Ops that read the very same host slice (q/k/v, gate/up) share one device copy of it.
+  std::vector<size_t> xoff(n_ops), yoff(n_ops);
   size_t xb = 0, yb = 0;
   for (size_t i = 0; i < n_ops; i++) {
-    xb += (size_t)ops[i].n_tokens * ops[i].w->in_dim * 4;
+    size_t j = 0;
+    while (j < i && !(ops[j].x == ops[i].x && ops[j].n_tokens == ops[i].n_tokens &&
+                      ops[j].w->in_dim == ops[i].w->in_dim))
+      j++;
+    if (j < i) {
+      xoff[i] = xoff[j];
+    } else {
+      xoff[i] = xb;
+      xb += (size_t)ops[i].n_tokens * ops[i].w->in_dim * 4;
+    }
+    yoff[i] = yb;
     yb += (size_t)ops[i].n_tokens * ops[i].w->out_dim * 4;
   }
   if (xb == 0) return OGM_OK;
@@ -492,31 +603,37 @@ extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, i
     uint32_t t = ops[i].n_tokens < cap ? ops[i].n_tokens : cap;
     if ((rc = ensure_act(ctx, ops[i].w->in_dim, t)) != OGM_OK) return rc;
   }
-  size_t xo = 0, yo = 0;
   for (size_t i = 0; i < n_ops; i++) {
     const ogm_op &op = ops[i];
     const size_t bytes = (size_t)op.n_tokens * op.w->in_dim * 4;
-    if (bytes) memcpy((uint8_t *)ctx->hx.p + xo, op.x, bytes);
-    xo += bytes;
+    bool first = true;
+    for (size_t j = 0; j < i; j++) first = first && xoff[j] != xoff[i];
+    if (bytes && first) memcpy((uint8_t *)ctx->hx.p + xoff[i], op.x, bytes);
   }
   HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, ctx->hx.p, xb, hipMemcpyHostToDevice, ctx->stream));
-  xo = 0;
-  for (size_t i = 0; i < n_ops; i++) {
+  std::vector<Target> tg;
+  for (size_t i = 0; i < n_ops;) {
+    // a run of neighbouring ops over one input and one weight type: one group
+    size_t e = i + 1;
+    while (e < n_ops && xoff[e] == xoff[i] && ops[e].n_tokens == ops[i].n_tokens &&
+           ops[e].w->ggml_type == ops[i].w->ggml_type && ops[e].w->in_dim == ops[i].w->in_dim)
+      e++;
     const ogm_op &op = ops[i];
-    const float *xd = (const float *)((uint8_t *)ctx->x.p + xo);
-    float *yd = (float *)((uint8_t *)ctx->y.p + yo);
+    const float *xd = (const float *)((uint8_t *)ctx->x.p + xoff[i]);
     for (uint32_t t0 = 0; t0 < op.n_tokens; t0 += cap) {
       const uint32_t nt = op.n_tokens - t0 < cap ? op.n_tokens - t0 : cap;
-      rc = enqueue_matmul(ctx, op.w, xd + (size_t)t0 * op.w->in_dim, nt,
-                          yd + (size_t)t0 * op.w->out_dim, decode, ctx->stream, nullptr, nullptr);
+      tg.clear();
+      for (size_t k = i; k < e; k++)
+        tg.push_back(Target{ops[k].w, (float *)((uint8_t *)ctx->y.p + yoff[k]) + (size_t)t0 * ops[k].w->out_dim});
+      rc = enqueue_matmul(ctx, tg.data(), tg.size(), xd + (size_t)t0 * op.w->in_dim, nt, decode,
+                          ctx->stream, nullptr, nullptr);
       if (rc != OGM_OK) return rc;
     }
-    xo += (size_t)op.n_tokens * op.w->in_dim * 4;
-    yo += (size_t)op.n_tokens * op.w->out_dim * 4;
+    i = e;
   }
   HIPCHK(ctx, hipMemcpyAsync(ctx->hy.p, ctx->y.p, yb, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-  yo = 0;
+  size_t yo = 0;
   for (size_t i = 0; i < n_ops; i++) {
     const size_t bytes = (size_t)ops[i].n_tokens * ops[i].w->out_dim * 4;
     if (bytes) memcpy(ops[i].y, (uint8_t *)ctx->hy.p + yo, bytes);

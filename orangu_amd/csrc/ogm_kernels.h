@@ -19,6 +19,8 @@ struct OgmActDev {
 hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,
                                OgmActDev act, hipStream_t stream);
 
+#define OGM_GEMV_MAX_MATS 4
+
 struct OgmGemvArgs {
   uint32_t ggml_type;
   const uint8_t *wt;  // tile-planar weights
@@ -27,9 +29,19 @@ struct OgmGemvArgs {
   uint32_t n_tokens;  // tokens in this launch (<= ogm_gemv_max_tokens)
   float *y;           // [n_tokens][out_dim], row stride out_dim
   int gemm_order;     // 0: GEMV float order (cpu.rs T==1 / matmul_decode), 1: GEMM order (T>1)
-  uint32_t wg_waves;     // waves per workgroup, 0 = one per column tile of a row block
+  uint32_t wg_waves;     // waves per workgroup, 0 = by shape
+  uint32_t rb_per_wg;    // row blocks per workgroup, 0 = by shape
   int32_t *dump_isum;    // optional [n_tokens][out_dim][blocks/row]
   int32_t *dump_imin;    // optional, Q4_K only
+  // Further matrices of the same type and in_dim that read the same activations (q/k/v,
+  // gate/up): one launch covers all of them.  Not combined with the dumps.
+  uint32_t n_extra;
+  const uint8_t *extra_wt[OGM_GEMV_MAX_MATS - 1];
+  uint32_t extra_out_dim[OGM_GEMV_MAX_MATS - 1];
+  float *extra_y[OGM_GEMV_MAX_MATS - 1];
+  // When set (one token, GEMV order, no dumps): f32 activations [in_dim]; every workgroup
+  // quantizes them itself on its way in and `act` is not read.
+  const float *x_f32;
 };
 
 // Largest token count one launch can take for this shape (LDS budget), at least 1.

@@ -123,7 +123,7 @@ struct FmtQ4K {
   static constexpr int AUX16 = 1;      // bsum: 8 x i16 per block
   static constexpr int ACT_GROUP = 256;
   static constexpr bool HAS_MIN = true;
-  static constexpr int MAX_THREADS = 1024;  // 16 waves share one staged activation vector
+  static constexpr int MAX_THREADS = 512;   // launch bound: leaves 256 VGPRs to a lane
   struct Regs {
     uint4 p[PIECES];
   };
@@ -353,11 +353,17 @@ struct FmtQ80 {
 // compiler can count them.
 
 struct GemvParams {
-  const uint8_t *wt;
+  // Up to OGM_GEMV_MAX_MATS matrices of one type and in_dim read the same activations; the
+  // grid is the concatenation of their row blocks.
+  const uint8_t *wt[OGM_GEMV_MAX_MATS];
+  float *y[OGM_GEMV_MAX_MATS];
+  uint32_t out_dim[OGM_GEMV_MAX_MATS];
+  uint32_t wg_end[OGM_GEMV_MAX_MATS];  // workgroups of matrices 0..m, running total
+  uint32_t rb_per_wg;                  // consecutive row blocks one workgroup owns
   OgmActDev act;
-  float *y;
+  const float *x;                  // f32 activations of the kernels that quantize on the way in
   int32_t *dump_isum, *dump_imin;
-  uint32_t in_dim, out_dim, upr;  // upr = blocks per row
+  uint32_t in_dim, upr;            // upr = blocks per row
   uint32_t n_tokens;
   uint32_t C, nct;                // tile shape: C blocks x R rows, nct = upr / C column tiles
 };
@@ -369,7 +375,7 @@ __host__ __device__ constexpr int n_term_arrays() {
 
 // Dynamic LDS bytes of one workgroup.
 template <class F, bool GEMM_ORDER>
-static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens) {
+static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rb_per_wg = 1) {
   const size_t upr = in_dim / F::ELEMS;
   const size_t n_scale = in_dim / F::ACT_GROUP;
   const OgmTiling tl = ogm_tiling_for((uint32_t)upr, 1);
@@ -377,11 +383,47 @@ static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens) {
   b += (size_t)n_tokens * upr * F::AUX16 * 16;              // aux
   b += (size_t)n_tokens * n_scale * 4;                      // act.d
   b = (b + 15) & ~(size_t)15;
-  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * upr * tl.R * 4;  // terms [block][row]
+  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * rb_per_wg * upr * tl.R * 4;  // terms
   return b;
 }
 
 #define OGM_STAGE_PEEL 4
+
+// The activation quantizer inside the GEMV: quantizes the 256 activations of group g held four
+// per lane (lane l: elements 256g + 4l ..) exactly as ogm_quantize_kernel does and leaves q, the
+// scale and the side sums in LDS where the formats read them.  Every lane of the wave calls it.
+template <class F>
+__device__ __forceinline__ void quantize_park(const float4 &v, uint32_t g, bool active, uint32_t lane,
+                                              uint32_t upr, uint4 *l_xq, uint4 *l_aux, float *l_d) {
+  float amax = 0.0f;
+  amax = nan_blind_max(amax, fabsf(v.x));
+  amax = nan_blind_max(amax, fabsf(v.y));
+  amax = nan_blind_max(amax, fabsf(v.z));
+  amax = nan_blind_max(amax, fabsf(v.w));
+#pragma unroll
+  for (int m = 1; m < F::ACT_GROUP / 4; m <<= 1) amax = nan_blind_max(amax, __shfl_xor(amax, m, 64));
+  const float scale = amax / 127.0f;
+  const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+  const int q0 = quantize_one(v.x, inv), q1 = quantize_one(v.y, inv);
+  const int q2 = quantize_one(v.z, inv), q3 = quantize_one(v.w, inv);
+  const uint32_t packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) |
+                          ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
+  int s = q0 + q1 + q2 + q3;
+  s += __shfl_xor(s, 1, 64);
+  s += __shfl_xor(s, 2, 64);                    // sum of 16
+  const int s32 = s + __shfl_xor(s, 4, 64);     // sum of 32
+  if (!active) return;
+  const uint32_t ch = g * 16u + (lane >> 2);    // 16-byte chunk of the token
+  const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
+  ((uint32_t *)(l_xq + c * upr + col))[lane & 3u] = packed;
+  if (F::AUX16 == 1) {          // Q4_K: bsum, eight i16 per block
+    if ((lane & 7u) == 0) ((int16_t *)(l_aux + col))[lane >> 3] = (int16_t)s32;
+  } else if (F::AUX16 == 2) {   // Q6_K: per-16 sums as i16, groups 0..7 | 8..15 of a block
+    const uint32_t gi = lane >> 2;
+    if ((lane & 3u) == 0) ((int16_t *)(l_aux + (gi >> 3) * upr + col))[gi & 7u] = (int16_t)s;
+  }
+  if ((lane & (F::ACT_GROUP / 4 - 1)) == 0) l_d[(g * 256u + lane * 4u) / F::ACT_GROUP] = scale;
+}
 
 // acc (+|-)= p[0], p[stride], ... in ascending order, one accumulator.
 template <bool NEGATE>
@@ -401,7 +443,9 @@ __device__ __forceinline__ float ordered_sum(float acc, const float *p, uint32_t
 }
 
 // UPR: blocks per row when known at compile time (the hot shapes), 0 = read it from the params.
-template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP>
+// QUANT: the workgroup quantizes the f32 activations p.x itself (one token) instead of reading
+// the quantizer kernel's output.
+template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP, bool QUANT>
 __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t tid = threadIdx.x, nthr = blockDim.x;
@@ -419,95 +463,134 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
   uint4 *l_aux = l_xq + (size_t)T * xch;                        // [T][AUX16][upr]
   float *l_d = (float *)(l_aux + (size_t)T * upr * F::AUX16);   // [T][n_scale]
   const size_t head = ((size_t)T * (xch * 16 + upr * F::AUX16 * 16 + n_scale * 4) + 15) & ~(size_t)15;
-  float *l_term = (float *)(lds + head);                        // [NT][T][upr][R]
+  float *l_term = (float *)(lds + head);                        // [NT][T][K][upr][R]
+
+  // ---- which matrix of the launch this workgroup belongs to, and which of its row blocks
+  uint32_t m = 0;
+  if (blockIdx.x >= p.wg_end[0]) m = 1;
+  if (blockIdx.x >= p.wg_end[1]) m = 2;
+  if (blockIdx.x >= p.wg_end[2]) m = 3;
+  const uint32_t wg = blockIdx.x - (m == 0 ? 0u : m == 1 ? p.wg_end[0] : m == 2 ? p.wg_end[1] : p.wg_end[2]);
+  const uint32_t K = p.rb_per_wg;
+  const uint32_t rb0 = wg * K;
+  const uint8_t *wt = m == 0 ? p.wt[0] : m == 1 ? p.wt[1] : m == 2 ? p.wt[2] : p.wt[3];
+  float *y = m == 0 ? p.y[0] : m == 1 ? p.y[1] : m == 2 ? p.y[2] : p.y[3];
+  const uint32_t out_dim = m == 0 ? p.out_dim[0] : m == 1 ? p.out_dim[1] : m == 2 ? p.out_dim[2] : p.out_dim[3];
+  // The workgroup's tiles are consecutive in memory: item i is tile rb0 * nct + i, i.e. column
+  // tile i % nct of row block rb0 + i / nct.
+  const uint32_t n_items = min(K, (out_dim + R - 1) / R - rb0) * nct;
+  const size_t tile0 = (size_t)rb0 * nct;
 
   // ---- issue the activation loads (few, L2-resident) ...
-  const uint32_t n_xq = T * xch;
+  const uint32_t n_xq = T * xch, n_aux = T * upr * F::AUX16, n_d = T * n_scale;
   const uint4 *gq = (const uint4 *)p.act.q;
-  const uint4 st0 = gq[min(tid, n_xq - 1)];
-  const uint4 st1 = gq[min(tid + nthr, n_xq - 1)];
-  const uint4 st2 = gq[min(tid + 2 * nthr, n_xq - 1)];
-  const uint4 st3 = gq[min(tid + 3 * nthr, n_xq - 1)];
-  const uint32_t n_aux = T * upr * F::AUX16;
-  uint4 st_aux = make_uint4(0, 0, 0, 0);
-  if (F::AUX16 == 1) {
-    st_aux = ((const uint4 *)p.act.bsum)[min(tid, n_aux - 1)];  // Q4_K: bsum, 8 x i16 per block
-  } else if (F::AUX16 == 2) {
-    // Q6_K: per-16 sums narrowed to i16, groups 0..7 / 8..15 of a block
-    const uint32_t i = min(tid, n_aux - 1);
-    const int4 *src = (const int4 *)(p.act.sums + (size_t)(i >> 1) * 16 + (i & 1u) * 8);
-    const int4 a = src[0], b = src[1];
-    st_aux.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
-    st_aux.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
-    st_aux.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
-    st_aux.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
+  uint4 st0, st1, st2, st3, st_aux = make_uint4(0, 0, 0, 0);
+  float st_d = 0.0f;
+  // f32 activations of the quantizing kernels: group k of this wave is 256 * (wave + k * n_wave)
+  float4 xs0, xs1, xs2, xs3, xs4, xs5, xs6, xs7;
+  auto xload = [&](uint32_t k) -> float4 {
+    const uint32_t e0 = (wave + k * n_wave) * 256u + lane * 4u;
+    return *(const float4 *)(p.x + min(e0, p.in_dim - 4u));
+  };
+  constexpr int QPEEL = (UPR == 16) ? 4 : 8;  // 4096-wide rows: four groups for each of four waves
+  if constexpr (QUANT) {
+    xs0 = xload(0); xs1 = xload(1); xs2 = xload(2); xs3 = xload(3);
+    if constexpr (QPEEL == 8) { xs4 = xload(4); xs5 = xload(5); xs6 = xload(6); xs7 = xload(7); }
+  } else {
+    st0 = gq[min(tid, n_xq - 1)];
+    st1 = gq[min(tid + nthr, n_xq - 1)];
+    st2 = gq[min(tid + 2 * nthr, n_xq - 1)];
+    st3 = gq[min(tid + 3 * nthr, n_xq - 1)];
+    if (F::AUX16 == 1) {
+      st_aux = ((const uint4 *)p.act.bsum)[min(tid, n_aux - 1)];  // Q4_K: bsum, 8 x i16 per block
+    } else if (F::AUX16 == 2) {
+      // Q6_K: per-16 sums narrowed to i16, groups 0..7 / 8..15 of a block
+      const uint32_t i = min(tid, n_aux - 1);
+      const int4 *src = (const int4 *)(p.act.sums + (size_t)(i >> 1) * 16 + (i & 1u) * 8);
+      const int4 a = src[0], b = src[1];
+      st_aux.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
+      st_aux.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
+      st_aux.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
+      st_aux.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
+    }
+    st_d = p.act.d[min(tid, n_d - 1)];
   }
-  const uint32_t n_d = T * n_scale;
-  const float st_d = p.act.d[min(tid, n_d - 1)];
 
   // Keeps every staging load of the workgroup ahead of every weight load in the CU's
   // memory pipeline (no data is waited for here).
   __syncthreads();
 
   // ---- ... then this wave's first tile of weights (the long pole) ...
-  const uint32_t rb = blockIdx.x;
   const uint32_t r_local = lane & (R - 1), c_local = lane / R;
-  const uint32_t row = rb * R + r_local;
-  const bool live = row < p.out_dim;
-  uint32_t ct = wave;  // every wave has at least one tile: n_wave <= nct
+  uint32_t it = wave;  // every wave has at least one item: n_wave <= nct <= n_items
   typename F::Regs cur;
-  F::load(cur, p.wt, (size_t)rb * nct + ct, lane);
+  F::load(cur, wt, tile0 + it, lane);
+  // Nothing below may be scheduled above the weight loads: work on the activations would
+  // otherwise wait for them first and hold the weight loads back by a memory round trip.
+  __builtin_amdgcn_sched_barrier(0);
 
   // ---- ... and park the activations in LDS while the weights are in flight.
   // q is permuted so that chunk c of block `col` lands at [c*upr + col].
-  auto park = [&](uint32_t i, const uint4 &v) {
-    if (i < n_xq) {
+  if constexpr (QUANT) {
+    const uint32_t n_g = (p.in_dim + 255u) / 256u;
+    auto qpark = [&](uint32_t k, const float4 &v) {
+      const uint32_t g = wave + k * n_wave;
+      quantize_park<F>(v, g, g * 256u + lane * 4u < p.in_dim, lane, upr, l_xq, l_aux, l_d);
+    };
+    qpark(0, xs0); qpark(1, xs1); qpark(2, xs2); qpark(3, xs3);
+    if constexpr (QPEEL == 8) { qpark(4, xs4); qpark(5, xs5); qpark(6, xs6); qpark(7, xs7); }
+    for (uint32_t k = QPEEL; wave + k * n_wave < n_g; k++) qpark(k, xload(k));  // longer rows
+  } else {
+    auto park = [&](uint32_t i, const uint4 &v) {
+      if (i < n_xq) {
+        const uint32_t t = i / xch, ch = i - t * xch;
+        const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
+        l_xq[(size_t)t * xch + c * upr + col] = v;
+      }
+    };
+    park(tid, st0);
+    park(tid + nthr, st1);
+    park(tid + 2 * nthr, st2);
+    park(tid + 3 * nthr, st3);
+    if (F::AUX16 == 1) {
+      if (tid < n_aux) l_aux[tid] = st_aux;
+    } else if (F::AUX16 == 2) {
+      if (tid < n_aux) {
+        const uint32_t blk = tid >> 1, k = tid & 1u;
+        const uint32_t t = blk / upr, col = blk - t * upr;
+        l_aux[(size_t)t * upr * 2 + k * upr + col] = st_aux;
+      }
+    }
+    if (tid < n_d) l_d[tid] = st_d;
+    // Whatever the peeled loads did not cover (many tokens, or very long rows).
+    for (uint32_t i = tid + OGM_STAGE_PEEL * nthr; i < n_xq; i += nthr) {
       const uint32_t t = i / xch, ch = i - t * xch;
       const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
-      l_xq[(size_t)t * xch + c * upr + col] = v;
+      l_xq[(size_t)t * xch + c * upr + col] = gq[i];
     }
-  };
-  park(tid, st0);
-  park(tid + nthr, st1);
-  park(tid + 2 * nthr, st2);
-  park(tid + 3 * nthr, st3);
-  if (F::AUX16 == 1) {
-    if (tid < n_aux) l_aux[tid] = st_aux;
-  } else if (F::AUX16 == 2) {
-    if (tid < n_aux) {
-      const uint32_t blk = tid >> 1, k = tid & 1u;
-      const uint32_t t = blk / upr, col = blk - t * upr;
-      l_aux[(size_t)t * upr * 2 + k * upr + col] = st_aux;
+    if (F::AUX16 == 1) {
+      for (uint32_t i = tid + nthr; i < n_aux; i += nthr) l_aux[i] = ((const uint4 *)p.act.bsum)[i];
+    } else if (F::AUX16 == 2) {
+      for (uint32_t i = tid + nthr; i < n_aux; i += nthr) {
+        const uint32_t blk = i >> 1, k = i & 1u;
+        const uint32_t t = blk / upr, col = blk - t * upr;
+        const int4 *src = (const int4 *)(p.act.sums + (size_t)blk * 16 + k * 8);
+        const int4 a = src[0], b = src[1];
+        uint4 o;
+        o.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
+        o.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
+        o.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
+        o.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
+        l_aux[(size_t)t * upr * 2 + k * upr + col] = o;
+      }
     }
+    for (uint32_t i = tid + nthr; i < n_d; i += nthr) l_d[i] = p.act.d[i];
   }
-  if (tid < n_d) l_d[tid] = st_d;
-  // Whatever the peeled loads did not cover (many tokens, or very long rows).
-  for (uint32_t i = tid + OGM_STAGE_PEEL * nthr; i < n_xq; i += nthr) {
-    const uint32_t t = i / xch, ch = i - t * xch;
-    const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
-    l_xq[(size_t)t * xch + c * upr + col] = gq[i];
-  }
-  if (F::AUX16 == 1) {
-    for (uint32_t i = tid + nthr; i < n_aux; i += nthr) l_aux[i] = ((const uint4 *)p.act.bsum)[i];
-  } else if (F::AUX16 == 2) {
-    for (uint32_t i = tid + nthr; i < n_aux; i += nthr) {
-      const uint32_t blk = i >> 1, k = i & 1u;
-      const uint32_t t = blk / upr, col = blk - t * upr;
-      const int4 *src = (const int4 *)(p.act.sums + (size_t)blk * 16 + k * 8);
-      const int4 a = src[0], b = src[1];
-      uint4 o;
-      o.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
-      o.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
-      o.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
-      o.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
-      l_aux[(size_t)t * upr * 2 + k * upr + col] = o;
-    }
-  }
-  for (uint32_t i = tid + nthr; i < n_d; i += nthr) l_d[i] = p.act.d[i];
   __syncthreads();
 
   // ---- tiles of this wave
-  for (; ct < nct; ct += n_wave) {
+  for (; it < n_items; it += n_wave) {
+    const uint32_t rbk = it / nct, ct = it - rbk * nct;
     const uint32_t col = ct * C + c_local;  // block index within the row
     for (uint32_t t = 0; t < T; t++) {
       ActLds a;
@@ -518,34 +601,40 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
       int isum, imin;
       F::template sums<UPR>(cur, a, col, isum, imin);
       const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
-      const uint32_t slot = col * R + r_local;
+      const size_t slot = (size_t)(t * K + rbk) * term_stride + col * R + r_local;
       if (GEMM_ORDER) {
         float tmin, tdot;
         F::term_gemm(cur, ad, isum, imin, tmin, tdot);
-        l_term[(size_t)t * term_stride + slot] = tdot;
-        if (NT == 2) l_term[(size_t)(T + t) * term_stride + slot] = tmin;
+        l_term[slot] = tdot;
+        if (NT == 2) l_term[(size_t)T * K * term_stride + slot] = tmin;
       } else {
-        l_term[(size_t)t * term_stride + slot] = F::term_gemv(cur, ad, isum, imin);
+        l_term[slot] = F::term_gemv(cur, ad, isum, imin);
       }
-      if (DUMP && live) {
-        const size_t o = ((size_t)t * p.out_dim + row) * upr + col;
-        if (p.dump_isum) p.dump_isum[o] = isum;
-        if (F::HAS_MIN && p.dump_imin) p.dump_imin[o] = imin;
+      if (DUMP) {
+        const uint32_t row = (rb0 + rbk) * R + r_local;
+        if (row < out_dim) {
+          const size_t o = ((size_t)t * out_dim + row) * upr + col;
+          if (p.dump_isum) p.dump_isum[o] = isum;
+          if (F::HAS_MIN && p.dump_imin) p.dump_imin[o] = imin;
+        }
       }
     }
-    if (ct + n_wave < nct) F::load(cur, p.wt, (size_t)rb * nct + ct + n_wave, lane);
+    if (it + n_wave < n_items) F::load(cur, wt, tile0 + it + n_wave, lane);
   }
   __syncthreads();
 
-  // One lane per (row, token): the row's block terms in ascending order, one accumulator.
-  for (uint32_t i = tid; i < R * T; i += nthr) {
-    const uint32_t t = i / R, r = i - t * R;
-    const uint32_t orow = rb * R + r;
-    if (orow < p.out_dim) {
+  // One lane per (token, row): the row's block terms in ascending order, one accumulator.
+  const uint32_t KR = K * R;
+  for (uint32_t i = tid; i < KR * T; i += nthr) {
+    const uint32_t t = i / KR, rr = i - t * KR;
+    const uint32_t rbk = rr / R, r = rr - rbk * R;
+    const uint32_t orow = (rb0 + rbk) * R + r;
+    if (orow < out_dim) {
+      const float *terms = l_term + (size_t)(t * K + rbk) * term_stride + r;
       float acc = 0.0f;
-      if (NT == 2) acc = ordered_sum<true>(acc, l_term + (size_t)(T + t) * term_stride + r, upr, R);
-      acc = ordered_sum<false>(acc, l_term + (size_t)t * term_stride + r, upr, R);
-      p.y[(size_t)t * p.out_dim + orow] = acc;
+      if (NT == 2) acc = ordered_sum<true>(acc, terms + (size_t)T * K * term_stride, upr, R);
+      acc = ordered_sum<false>(acc, terms, upr, R);
+      y[(size_t)t * out_dim + orow] = acc;
     }
   }
 }
@@ -575,22 +664,61 @@ uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order
   }
 }
 
+template <class F, bool QUANT>
+static void launch_single(const GemvParams &p, dim3 g, dim3 b, size_t lds, hipStream_t stream) {
+  // single-token decode: the hot shapes get their row length as a compile-time constant
+  if (F::ELEMS == 256 && p.upr == 16)
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false, QUANT>), g, b, lds, stream, p);
+  else if (F::ELEMS == 256 && p.upr == 56)
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false, QUANT>), g, b, lds, stream, p);
+  else if (F::ELEMS == 32 && p.upr == 128)
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 128, true, false, false, QUANT>), g, b, lds, stream, p);
+  else
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false, QUANT>), g, b, lds, stream, p);
+}
+
 template <class F, bool GEMM_ORDER>
 static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
+  const bool dump = a.dump_isum || a.dump_imin;
+  if (a.n_extra > OGM_GEMV_MAX_MATS - 1 || (dump && a.n_extra)) return hipErrorInvalidValue;
+  if (a.x_f32 && (a.n_tokens != 1 || GEMM_ORDER || dump)) return hipErrorInvalidValue;
   GemvParams p;
-  p.wt = a.wt;
   p.act = a.act;
-  p.y = a.y;
+  p.x = a.x_f32;
   p.dump_isum = a.dump_isum;
   p.dump_imin = a.dump_imin;
   p.in_dim = a.in_dim;
-  p.out_dim = a.out_dim;
   p.upr = a.in_dim / F::ELEMS;
   p.n_tokens = a.n_tokens;
   const OgmTiling tl = ogm_tiling_for(p.upr, a.out_dim);
   p.C = tl.C;
   p.nct = tl.nct;
-  const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens);
+  uint32_t n_rb = 0;
+  for (uint32_t m = 0; m <= a.n_extra; m++)
+    n_rb += ((m ? a.extra_out_dim[m - 1] : a.out_dim) + tl.R - 1) / tl.R;
+  if (n_rb == 0) return hipSuccess;
+  // Row blocks per workgroup.  One is the measured optimum on MI355X at every shape tried
+  // (4096 -> 14336 x2: 2, 4 and 8 row blocks cost 7%, 25% and 60% more time): many small
+  // workgroups keep more loads in flight than the shared activation staging saves.
+  uint32_t K = a.rb_per_wg ? a.rb_per_wg : 1;
+  while (K > 1 && gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, K) > OGM_LDS_BUDGET) K--;
+  if (dump) K = 1;
+  p.rb_per_wg = K;
+  uint32_t n_wg = 0;
+  for (uint32_t m = 0; m < OGM_GEMV_MAX_MATS; m++) {
+    if (m <= a.n_extra) {
+      p.wt[m] = m ? a.extra_wt[m - 1] : a.wt;
+      p.y[m] = m ? a.extra_y[m - 1] : a.y;
+      p.out_dim[m] = m ? a.extra_out_dim[m - 1] : a.out_dim;
+      n_wg += ((p.out_dim[m] + tl.R - 1) / tl.R + K - 1) / K;
+    } else {
+      p.wt[m] = nullptr;
+      p.y[m] = nullptr;
+      p.out_dim[m] = 0;
+    }
+    p.wg_end[m] = n_wg;
+  }
+  const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, K);
   if (lds > OGM_LDS_BUDGET) return hipErrorInvalidValue;
   // Waves per workgroup: the largest divisor of the row block's tile count up to 8 (measured on
   // MI355X: 4 waves x 1 tile at 4096 -> 14336, 7 waves x 2 tiles at 14336 -> 4096 beat 14 x 1).
@@ -603,27 +731,20 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   if (waves > tl.nct) waves = tl.nct;
   if (waves > (uint32_t)F::MAX_THREADS / 64) waves = F::MAX_THREADS / 64;
   if (waves == 0) waves = 1;
-  const dim3 g(tl.nrb), b(waves * 64);
-  if (a.dump_isum || a.dump_imin) {
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true>), g, b, lds, stream, p);
+  const dim3 g(n_wg), b(waves * 64);
+  if (dump) {
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true, false>), g, b, lds, stream, p);
   } else if (a.n_tokens == 1 && !GEMM_ORDER) {
-    // single-token decode: the hot shapes get their row length as a compile-time constant
-    if (F::ELEMS == 256 && p.upr == 16)
-      hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false>), g, b, lds, stream, p);
-    else if (F::ELEMS == 256 && p.upr == 56)
-      hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false>), g, b, lds, stream, p);
-    else if (F::ELEMS == 32 && p.upr == 128)
-      hipLaunchKernelGGL((ogm_gemv_kernel<F, 128, true, false, false>), g, b, lds, stream, p);
-    else
-      hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false>), g, b, lds, stream, p);
+    if (a.x_f32) launch_single<F, true>(p, g, b, lds, stream);
+    else launch_single<F, false>(p, g, b, lds, stream);
   } else {
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false>), g, b, lds, stream, p);
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false>), g, b, lds, stream, p);
   }
   return hipGetLastError();
 }
 
 hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name) {
-  if (a.n_tokens == 0 || a.out_dim == 0) return hipSuccess;
+  if (a.n_tokens == 0) return hipSuccess;
   switch (a.ggml_type) {
     case OGM_Q4_K:
       if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ4K,gemm>" : "ogm_gemv_kernel<FmtQ4K,gemv>";

@@ -367,3 +367,136 @@ def test_mfma_gemm_adversarial_integer_ranges(be):
     got = be.matmul(x, T, qm(raw, Q4_K, in_dim, out_dim))
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     assert_bits(got, want, "extreme ranges")
+
+
+# ---------------------------------------------------------------- quantize inside the GEMV, grouped launches
+
+@pytest.mark.parametrize("t,in_dim,out_dim", [
+    (Q8_0, 32, 7), (Q8_0, 96, 33), (Q8_0, 4096, 130), (Q8_0, 4384, 64),
+    (Q4_K, 256, 5), (Q4_K, 768, 70), (Q4_K, 4096, 257), (Q4_K, 14336, 96), (Q4_K, 18432, 40),
+    (Q6_K, 256, 3), (Q6_K, 1280, 65), (Q6_K, 4096, 130), (Q6_K, 14336, 48), (Q6_K, 18432, 17),
+])
+def test_single_token_gemv_quantizes_in_kernel_or_before_with_the_same_bits(be, t, in_dim, out_dim):
+    """One token: the GEMV that quantizes its own activations and the quantizer kernel + GEMV
+    pair both reproduce backend/cpu.rs:445-458 bit for bit."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim * 3 + out_dim)
+    w = qm(raw, t, in_dim, out_dim)
+    for seed in (1, 2):
+        x = synth_x(1, in_dim, seed=seed).reshape(-1)
+        if seed == 2:  # adversarial activation groups: zeros, NaN, huge, denormal
+            x[:32] = 0.0
+            x[in_dim // 2] = np.nan
+            x[-1] = 3.0e38
+            x[1:in_dim:97] *= 1e-40
+        want = oracle.matmul(t, raw, in_dim, out_dim, x, 1).reshape(-1)
+        for mode in (1, 0, -1):
+            say("fuse", t, in_dim, out_dim, seed, mode)
+            be.set_tuning("gemv_fuse_quant", mode)
+            try:
+                got = be.matmul(x, 1, w)
+            finally:
+                be.set_tuning("gemv_fuse_quant", -1)
+            np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+            ok = ~np.isnan(want)
+            assert_bits(got[ok], want[ok], f"fuse mode {mode}")
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("T,decode", [(1, False), (1, True), (4, True), (3, False), (16, False), (11, True)])
+def test_grouped_weights_over_one_input_equal_single_calls(be, t, T, decode):
+    """q/k/v and gate/up read one input (engine/arch/mod.rs:1082-1096): the grouped call equals
+    matmul / matmul_decode per weight, also past four weights (two launches) and with ragged
+    out_dims."""
+    from orangu_amd.hiprt import DeviceBuffer, device_synchronize
+    in_dim = 1024
+    outs = [70, 16, 33, 128, 5]
+    raws = [synth_weights(t, in_dim, od, seed=40 + i) for i, od in enumerate(outs)]
+    ws = [qm(r, t, in_dim, od) for r, od in zip(raws, outs)]
+    x = synth_x(T, in_dim, seed=T)
+    xd = DeviceBuffer.from_numpy(x)
+    yds = [DeviceBuffer(T * od * 4) for od in outs]
+    for fuse in (-1, 0, 1):
+        be.set_tuning("gemv_fuse_quant", fuse)
+        say("grouped", t, T, decode, fuse)
+        for yd in yds:
+            yd.fill(0xFF)
+        try:
+            be.matmul_multi_dev([be.upload(w) for w in ws], xd.ptr, T, [yd.ptr for yd in yds], decode)
+        finally:
+            be.set_tuning("gemv_fuse_quant", -1)
+        device_synchronize()
+        for raw, od, yd in zip(raws, outs, yds):
+            got = yd.to_numpy(np.float32, T * od)
+            want = (oracle.matmul_decode if decode else oracle.matmul)(t, raw, in_dim, od, x, T)
+            assert_bits(got, want, f"out_dim {od}")
+    for b in [xd] + yds:
+        b.free()
+
+
+def test_grouped_call_rejects_mixed_weights(be):
+    from orangu_amd import OgmError
+    from orangu_amd.hiprt import DeviceBuffer
+    a = qm(synth_weights(Q4_K, 256, 4, seed=1), Q4_K, 256, 4)
+    b = qm(synth_weights(Q6_K, 256, 4, seed=2), Q6_K, 256, 4)
+    c = qm(synth_weights(Q4_K, 512, 4, seed=3), Q4_K, 512, 4)
+    xd, yd = DeviceBuffer(512 * 4), DeviceBuffer(64)
+    for pair in ((a, b), (a, c)):
+        with pytest.raises(OgmError):
+            be.matmul_multi_dev([be.upload(w) for w in pair], xd.ptr, 1, [yd.ptr, yd.ptr])
+    xd.free()
+    yd.free()
+
+
+def test_matmul_batch_groups_ops_that_share_their_input(be):
+    """Backend::matmul_batch over [wq, wk, wv] with one x (engine/arch/mod.rs:1082-1096): same
+    values as the ops one by one, whatever the grouping."""
+    from orangu_amd import MatmulOp
+    in_dim = 2048
+    x1, x4 = synth_x(1, in_dim, seed=5), synth_x(4, in_dim, seed=6)
+    mk = lambda t, od, s: qm(synth_weights(t, in_dim, od, seed=s), t, in_dim, od)
+    wq, wk, wv = mk(Q4_K, 96, 1), mk(Q4_K, 32, 2), mk(Q6_K, 32, 3)
+    gate, up = mk(Q4_K, 200, 4), mk(Q4_K, 200, 5)
+    ops = [MatmulOp(x1, 1, wq), MatmulOp(x1, 1, wk), MatmulOp(x1, 1, wv),
+           MatmulOp(x4, 4, gate), MatmulOp(x4, 4, up), MatmulOp(x1.copy(), 1, gate)]
+    for decode in (False, True):
+        outs = (be.matmul_batch_decode if decode else be.matmul_batch)(ops)
+        for op, y in zip(ops, outs):
+            one = (be.matmul_decode if decode else be.matmul)(op.x, op.n_tokens, op.w)
+            assert_bits(y, one, "grouped batch")
+            want = (oracle.matmul_decode if decode else oracle.matmul)(
+                op.w.ggml_type(), op.w.raw_bytes(), in_dim, op.w.out_dim, op.x, op.n_tokens)
+            assert_bits(y, want, "grouped batch vs cpu")
+
+
+@pytest.mark.parametrize("t,in_dim", [(Q8_0, 1056), (Q4_K, 1024), (Q4_K, 1536), (Q6_K, 1024), (Q6_K, 256)])
+def test_row_blocks_per_workgroup_do_not_change_a_bit(be, t, in_dim):
+    """A workgroup may own several row blocks (ragged last group, last row block partly beyond
+    out_dim, several matrices in one launch): every split gives the CPU path's bits."""
+    from orangu_amd.hiprt import DeviceBuffer, device_synchronize
+    outs = [150, 16, 33]
+    raws = [synth_weights(t, in_dim, od, seed=70 + i) for i, od in enumerate(outs)]
+    ws = [qm(r, t, in_dim, od) for r, od in zip(raws, outs)]
+    x = synth_x(3, in_dim, seed=9)
+    xd = DeviceBuffer.from_numpy(x)
+    yds = [DeviceBuffer(3 * od * 4) for od in outs]
+    try:
+        for K in (1, 2, 3, 4, 8, 64):
+            be.set_tuning("gemv_rb_per_wg", K)
+            for T, decode, fuse in ((1, False, 1), (1, False, 0), (3, True, -1), (3, False, -1)):
+                say("rb_per_wg", t, in_dim, K, T, decode, fuse)
+                be.set_tuning("gemv_fuse_quant", fuse)
+                want = (oracle.matmul_decode if decode else oracle.matmul)(t, raws[0], in_dim, outs[0], x[:T], T)
+                got = (be.matmul_decode if decode else be.matmul)(x[:T].reshape(-1), T, ws[0])
+                assert_bits(got, want, "single matrix")
+                for yd in yds:
+                    yd.fill(0xFF)
+                be.matmul_multi_dev([be.upload(w) for w in ws], xd.ptr, T, [yd.ptr for yd in yds], decode)
+                device_synchronize()
+                for raw, od, yd in zip(raws, outs, yds):
+                    want = (oracle.matmul_decode if decode else oracle.matmul)(t, raw, in_dim, od, x[:T], T)
+                    assert_bits(yd.to_numpy(np.float32, T * od), want, f"grouped out_dim {od}")
+    finally:
+        be.set_tuning("gemv_rb_per_wg", 0)
+        be.set_tuning("gemv_fuse_quant", -1)
+        for b in [xd] + yds:
+            b.free()
