@@ -369,6 +369,12 @@ static int enqueue_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev,
   return enqueue_matmul(ctx, &t, 1, x_dev, n_tokens, decode, stream, dump_isum, dump_imin);
 }
 
+static bool all_gemm_supported(const Target *tg, size_t n_tg, uint32_t n_tokens) {
+  for (size_t i = 0; i < n_tg; i++)
+    if (!ogm_gemm_supported(tg[i].w->ggml_type, tg[i].w->in_dim, tg[i].w->out_dim, n_tokens)) return false;
+  return true;
+}
+
 // Enqueues the matmul kernels over the context's quantized activations (or, with x_f32, over
 // one token of f32 activations that the kernel quantizes itself).  Caller holds the lock.
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
@@ -380,7 +386,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   // n_tokens == 1 and every matmul_decode take the GEMV's.
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
   if (gemm_order && !dump_isum && !dump_imin && n_tokens >= (uint32_t)ctx->tune_gemm_min_tokens &&
-      ogm_gemm_supported(w0->ggml_type, w0->in_dim)) {
+      all_gemm_supported(tg, n_tg, n_tokens)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
     int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w0->in_dim, n_tokens));
     if (rc != OGM_OK) return rc;

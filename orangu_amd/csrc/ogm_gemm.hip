@@ -2,21 +2,24 @@
 // (gemm_k_q4_k + accumulate_sym32, engine/vecdot.rs:2213-2303 of orangu-server).
 //
 // The integer stage stays exact on the matrix cores by keeping every operand an *integer-valued
-// f16*: a weight enters as sc_j * q (0..945, exact in f16: 11-bit significand), an activation as
-// its int8 value.  Products are exact in f32 and a chain of 128 of them stays below 2^24, so a
-// half super-block accumulates exactly in the MFMA's f32 accumulator; the two halves are added
-// with one f32 add, which rounds the exact integer sum once -- the same value as the
-// reference's `isum as f32`.  The min term sum_j m_j * bsum_j goes through one more MFMA per
-// super-block with bsum split as 64*bh + bl (both exact in f16).  The f32 epilogue then follows
-// the reference's order: first `acc -= (ad*dmin) * imin` over all super-blocks, then
+// f16*.  A weight enters centred and pre-scaled, sc_j * (q - 8) with |.| <= 504; an activation as
+// its int8 value.  Products are exact in f32 and a whole super-block (256 k) sums to at most
+// 63 * 8 * 127 * 256 = 16 386 048 < 2^24, so the MFMA's f32 accumulator holds
+//   c = sum_j sc_j * dot32(q_j - 8, x_j)
+// exactly.  The centring is undone by one more MFMA per super-block over the per-32 activation
+// sums, corr = 8 * sum_j sc_j * bsum_j (bsum split as 64*bh + bl so that every operand is exact in
+// f16; |corr| < 2^24), and `c + corr` is one f32 add of two exact integers: it rounds the exact
+// isum once, to nearest even -- the value of the reference's `isum as f32`.  The min term
+// sum_j m_j * bsum_j comes from the same kind of MFMA.  The f32 epilogue then follows the
+// reference's order: first `acc -= (ad*dmin) * imin` over all super-blocks, then
 // `acc += ad * (d * isum)` over all super-blocks.
 //
-// Tiling: a workgroup of four waves owns 64 rows (four row blocks of the tile-planar layout)
-// x 128 tokens; a wave owns 32 rows x 64 tokens = two 32x32 MFMA tiles.  Per half super-block
-// (128 k) the workgroup dequantizes its 64 x 128 weight tile to f16 in LDS (each thread one
-// 16-byte piece: v_perm nibble split, magic-number int->f16, one packed f16 fma per two
-// weights) and copies the 128 x 128 f16 activation tile, then runs 8 x v_mfma_f32_32x32x16_f16
-// per MFMA tile.
+// Tiling: a workgroup of eight waves owns 128 rows x 128 tokens; a wave owns 64 rows x 32 tokens
+// = two v_mfma_f32_32x32x16_f16 tiles.  The k loop advances 64 at a time (a quarter super-block:
+// one piece pair of qs, i.e. sub-blocks 2g and 2g+1): each thread dequantizes half a 16-byte piece
+// (v_perm byte spread, magic-number int->f16, packed f16 add and multiply) into LDS and copies
+// two 16-byte chunks of the f16 activations; LDS is double buffered and the next stage's global
+// loads are issued before the current stage's MFMAs, so there is one barrier per stage.
 #include <hip/hip_runtime.h>
 
 #include "ogm_kernels.h"
@@ -26,19 +29,19 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
-#define GM_BN 64    // rows per workgroup
+#define GM_BN 128   // rows per workgroup
 #define GM_BT 128   // tokens per workgroup
-#define GM_KH 128   // k per staging step: half a super-block
-#define GM_LD (GM_KH + 8)   // f16 per LDS row: 16 bytes of padding keep 16-byte row reads conflict-free
-#define GM_LD2 24           // f16 per LDS row of the min-term operands (16 + padding)
+#define GM_KS 64    // k per stage
+#define GM_STAGE_HALFS (128 * GM_KS)   // f16 per staged tile (A or B) of one stage
 
 struct GemmParams {
-  const uint8_t *wt;      // tile-planar Q4_K, C = 4 (16 rows x 4 blocks per tile)
+  const uint8_t *wt;      // tile-planar Q4_K
   const _Float16 *xh;     // [T][in_dim] int8 activations as f16
+  const _Float16 *bs16;   // [T][nsb][16]: floor(bsum_j / 64) for j = 0..7, then bsum_j mod 64
   const float *ad;        // [T][nsb] activation scales (per 256)
-  const int16_t *bsum;    // [T][in_dim/32] per-32 sums of q
   float *y;               // [T][out_dim]
-  uint32_t in_dim, out_dim, n_tokens, nsb, nct, nrb;
+  uint32_t in_dim, out_dim, n_tokens, nsb;
+  uint32_t c_shift, r_shift, nct;  // weight tiles of R = 1 << r_shift rows x C = 1 << c_shift blocks
 };
 
 __device__ __forceinline__ float gm_f16_bits_to_f32(uint32_t bits16) {
@@ -47,254 +50,404 @@ __device__ __forceinline__ float gm_f16_bits_to_f32(uint32_t bits16) {
   return (float)v.h;
 }
 
-// int8 activations -> f16, once per matmul.
-__global__ void ogm_q8_to_f16_kernel(const int8_t *__restrict__ q, _Float16 *__restrict__ xh, size_t n8) {
+// int8 activations -> f16 and per-32 sums -> (bh, bl) f16 pairs, once per matmul.
+__global__ void ogm_gemm_prep_kernel(const int8_t *__restrict__ q, const int16_t *__restrict__ bsum,
+                                     _Float16 *__restrict__ xh, _Float16 *__restrict__ bs16, size_t n8,
+                                     size_t n_sb) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n8) return;
-  const int2 v = ((const int2 *)q)[i];
-  half8 o;
-  o[0] = (_Float16)(float)(int8_t)(v.x);
-  o[1] = (_Float16)(float)(int8_t)(v.x >> 8);
-  o[2] = (_Float16)(float)(int8_t)(v.x >> 16);
-  o[3] = (_Float16)(float)(int8_t)(v.x >> 24);
-  o[4] = (_Float16)(float)(int8_t)(v.y);
-  o[5] = (_Float16)(float)(int8_t)(v.y >> 8);
-  o[6] = (_Float16)(float)(int8_t)(v.y >> 16);
-  o[7] = (_Float16)(float)(int8_t)(v.y >> 24);
-  ((half8 *)xh)[i] = o;
+  if (i < n8) {
+    const int2 v = ((const int2 *)q)[i];
+    half8 o;
+    o[0] = (_Float16)(float)(int8_t)(v.x);
+    o[1] = (_Float16)(float)(int8_t)(v.x >> 8);
+    o[2] = (_Float16)(float)(int8_t)(v.x >> 16);
+    o[3] = (_Float16)(float)(int8_t)(v.x >> 24);
+    o[4] = (_Float16)(float)(int8_t)(v.y);
+    o[5] = (_Float16)(float)(int8_t)(v.y >> 8);
+    o[6] = (_Float16)(float)(int8_t)(v.y >> 16);
+    o[7] = (_Float16)(float)(int8_t)(v.y >> 24);
+    ((half8 *)xh)[i] = o;
+  }
+  if (i < n_sb) {
+    const uint4 b = ((const uint4 *)bsum)[i];  // eight i16
+    const uint32_t w[4] = {b.x, b.y, b.z, b.w};
+    half8 bh, bl;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int b0 = (int)(int16_t)(w[j] & 0xFFFFu), b1 = ((int)w[j]) >> 16;
+      bh[2 * j] = (_Float16)(float)(b0 >> 6);  // floor(b / 64)
+      bl[2 * j] = (_Float16)(float)(b0 & 63);
+      bh[2 * j + 1] = (_Float16)(float)(b1 >> 6);
+      bl[2 * j + 1] = (_Float16)(float)(b1 & 63);
+    }
+    ((half8 *)bs16)[2 * i] = bh;
+    ((half8 *)bs16)[2 * i + 1] = bl;
+  }
 }
 
-// Four bytes b0..b3 of `w`, one nibble each (shift 0: low, 4: high), scaled by sc:
-// out = { sc*n(b0), sc*n(b1) }, { sc*n(b2), sc*n(b3) } as packed f16.
-__device__ __forceinline__ void dequant4(uint32_t w, int shift, half2v sc2, half2v nc2, uint32_t &o01,
-                                         uint32_t &o23) {
-  const uint32_t p01 = __builtin_amdgcn_perm(0u, w, 0x0c010c00u) >> shift;  // (b0, 0, b1, 0)
-  const uint32_t p23 = __builtin_amdgcn_perm(0u, w, 0x0c030c02u) >> shift;  // (b2, 0, b3, 0)
-  // 0x6400 | n is the f16 1024 + n; (1024 + n) * sc - 1024 * sc = n * sc exactly (one rounding
-  // of an exactly representable result)
-  union { uint32_t u; half2v h; } a, b;
+// Bytes b0..b3 of `w`: low nibbles (q - 8) * sl and high nibbles (q - 8) * sh as packed f16.
+// 0x6400 | n is the f16 1024 + n and 0x5400 | (n << 4) the f16 64 + n: subtracting 1032 or 72
+// leaves n - 8 exactly and the product with a scale <= 63 is an integer below 2^11, exact too.
+__device__ __forceinline__ void dequant8(uint32_t w, half2v sl2, half2v sh2, uint32_t &lo01,
+                                         uint32_t &lo23, uint32_t &hi01, uint32_t &hi23) {
+  const uint32_t p01 = __builtin_amdgcn_perm(0u, w, 0x0c010c00u);  // (b0, 0, b1, 0)
+  const uint32_t p23 = __builtin_amdgcn_perm(0u, w, 0x0c030c02u);  // (b2, 0, b3, 0)
+  union { uint32_t u; half2v h; } a, b, c, d;
+  const half2v k1032 = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+  const half2v k72 = {(_Float16)-72.0f, (_Float16)-72.0f};
   a.u = (p01 & 0x000F000Fu) | 0x64006400u;
   b.u = (p23 & 0x000F000Fu) | 0x64006400u;
-  a.h = __builtin_elementwise_fma(a.h, sc2, nc2);
-  b.h = __builtin_elementwise_fma(b.h, sc2, nc2);
-  o01 = a.u;
-  o23 = b.u;
+  c.u = (p01 & 0x00F000F0u) | 0x54005400u;
+  d.u = (p23 & 0x00F000F0u) | 0x54005400u;
+  a.h = (a.h + k1032) * sl2;
+  b.h = (b.h + k1032) * sl2;
+  c.h = (c.h + k72) * sh2;
+  d.h = (d.h + k72) * sh2;
+  lo01 = a.u;
+  lo23 = b.u;
+  hi01 = c.u;
+  hi23 = d.u;
 }
 
-__global__ __launch_bounds__(256) void ogm_gemm_q4k_kernel(GemmParams p) {
+// get_scale_min_k4 (quant.rs:653-662) for all eight sub-blocks: sc 0..3 | sc 4..7, one per byte.
+__device__ __forceinline__ void q4k_scales(const uint4 &hd, uint32_t &sca, uint32_t &scb) {
+  sca = hd.y & 0x3F3F3F3Fu;
+  scb = (hd.w & 0x0F0F0F0Fu) | ((hd.y >> 2) & 0x30303030u);
+}
+__device__ __forceinline__ void q4k_mins(const uint4 &hd, uint32_t &mna, uint32_t &mnb) {
+  mna = hd.z & 0x3F3F3F3Fu;
+  mnb = ((hd.w >> 4) & 0x0F0F0F0Fu) | ((hd.z >> 2) & 0x30303030u);
+}
+
+// The K = 16 operand of the side MFMAs for one row: k 0..7 pair with bh_j, k 8..15 with bl_j, so
+// a lane of the upper half (lh = 0) carries hi_scale * v_j and of the lower half v_j * lo_scale.
+__device__ __forceinline__ half8 side_operand(uint32_t va, uint32_t vb, float scale) {
+  half8 o;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    o[j] = (_Float16)(scale * (float)((va >> (8 * j)) & 0xFFu));
+    o[4 + j] = (_Float16)(scale * (float)((vb >> (8 * j)) & 0xFFu));
+  }
+  return o;
+}
+
+// LDS rows of the staged tiles are 128 bytes (64 f16) without padding; the 16-byte chunk c of row
+// r sits at chunk c ^ (r & 7) ^ ((r >> 3) & 1).  Eight consecutive rows then cover all eight chunk
+// positions (no conflict if a 128-bit access is served eight lanes at a time over 32 banks), and
+// in sixteen consecutive rows two rows with the same chunk position differ in row parity, i.e.
+// in the 128-byte half of a 256-byte bank line (no conflict with sixteen lanes over 64 banks).
+__device__ __forceinline__ uint32_t gm_swz(uint32_t row, uint32_t chunk) {
+  return row * 64u + ((chunk ^ (row & 7u) ^ ((row >> 3) & 1u)) << 3);  // in f16 units
+}
+
+__global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
   extern __shared__ __align__(16) uint8_t lds[];
-  _Float16 *A_l = (_Float16 *)lds;                    // [64][GM_LD]   (pass 1: [64][GM_LD2])
-  _Float16 *B_l = A_l + GM_BN * GM_LD;                // [128][GM_LD]  (pass 1: [128][GM_LD2])
-  float *d_l = (float *)(B_l + GM_BT * GM_LD);        // [64]
-  float *dmin_l = d_l + GM_BN;                        // [64]
-  float *ad_l = dmin_l + GM_BN;                       // [128]
+  _Float16 *A_l = (_Float16 *)lds;                  // [2][128][64]
+  _Float16 *B_l = A_l + 2 * GM_STAGE_HALFS;         // [2][128][64]
+  _Float16 *a2_l = B_l + 2 * GM_STAGE_HALFS;        // [128 rows][16]: 512*sc_j | 8*sc_j
+  _Float16 *b2_l = a2_l + 128 * 16;                 // [128 tokens][16]: bh_j | bl_j
+  float *d_l = (float *)(b2_l + 128 * 16);          // [128]
+  float *dmin_t = (float *)lds;                     // pass 1 only: [nsb][128], over A_l / B_l
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const uint32_t wr = wave & 1u, wt_ = wave >> 1;     // wave's row half and token half
-  const uint32_t r0 = blockIdx.x * GM_BN, t0 = blockIdx.y * GM_BT;
+  const uint32_t wr = wave & 1u, wt_ = wave >> 1;   // wave's row half (64 rows) and token quarter (32)
+  const uint32_t t0 = blockIdx.x * GM_BT, r0 = blockIdx.y * GM_BN;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
-  const uint32_t rb0 = r0 / 16u;
 
-  float16v y0 = {}, y1 = {};  // this wave's 32 rows x (2 x 32) tokens
+  // Address of block `s` of row `row` in the tile-planar layout (piece 0: d, dmin, scales).
+  // Rows past the matrix are clamped onto its last row; their results are never stored.
+  // Byte offsets stay below 4 GiB (checked by the launcher), so they are 32-bit: a row part
+  // that a thread computes once and a super-block part that is the same for every thread.
+  auto row_off = [&](uint32_t row) -> uint32_t {
+    row = min(row, p.out_dim - 1u);
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    return rb * p.nct * 9216u + r * 16u;
+  };
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    const uint32_t ct = s >> p.c_shift, cl = s & ((1u << p.c_shift) - 1u);
+    return ct * 9216u + (cl << p.r_shift) * 16u;
+  };
+  // token of this lane's column, clamped like the rows
+  const uint32_t tk = min(t0 + 32u * wt_ + l32, p.n_tokens - 1u);
+
+  float16v y0, y1;  // rows 64 wr + 0..31 and + 32..63, tokens 32 wt_ + 0..31
+#pragma unroll
+  for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
+  float16v zero;
+#pragma unroll
+  for (int r = 0; r < 16; r++) zero[r] = 0.0f;
 
   // ---------------- pass 1: acc -= (ad * dmin) * sum_j m_j * bsum_j, all super-blocks first
-  for (uint32_t s = 0; s < p.nsb; s++) {
-    if (tid < GM_BN) {
-      const uint32_t lr = tid;
-      // (row blocks past the matrix are clamped: their rows are never stored)
-      const size_t tile = (size_t)min(rb0 + lr / 16u, p.nrb - 1u) * p.nct + s / 4u;
-      const uint4 h = *(const uint4 *)(p.wt + tile * 9216u + ((s & 3u) * 16u + (lr & 15u)) * 16u);
-      const uint32_t mna = h.z & 0x3F3F3F3Fu;                                      // m 0..3
-      const uint32_t mnb = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);  // m 4..7
-      half8 hi, lo;
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const float ma = (float)((mna >> (8 * j)) & 0xFFu), mb = (float)((mnb >> (8 * j)) & 0xFFu);
-        lo[j] = (_Float16)ma;
-        lo[4 + j] = (_Float16)mb;
-        hi[j] = (_Float16)(64.0f * ma);
-        hi[4 + j] = (_Float16)(64.0f * mb);
-      }
-      *(half8 *)(A_l + lr * GM_LD2) = hi;       // k 0..7 : 64 * m_j  (pairs with bh_j)
-      *(half8 *)(A_l + lr * GM_LD2 + 8) = lo;   // k 8..15: m_j       (pairs with bl_j)
-      dmin_l[lr] = gm_f16_bits_to_f32(h.x >> 16);
-    } else if (tid < GM_BN + GM_BT) {
-      const uint32_t tt = tid - GM_BN, tk = t0 + tt;
-      half8 bh = {}, bl = {};
-      float adv = 0.0f;
-      if (tk < p.n_tokens) {
-        const uint4 b = *(const uint4 *)(p.bsum + ((size_t)tk * p.nsb + s) * 8u);
-        const uint32_t w[4] = {b.x, b.y, b.z, b.w};
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          const int b0 = (int)(int16_t)(w[j] & 0xFFFFu), b1 = ((int)w[j]) >> 16;
-          bh[2 * j] = (_Float16)(float)(b0 >> 6);      // floor(b / 64)
-          bl[2 * j] = (_Float16)(float)(b0 & 63);
-          bh[2 * j + 1] = (_Float16)(float)(b1 >> 6);
-          bl[2 * j + 1] = (_Float16)(float)(b1 & 63);
-        }
-        adv = p.ad[(size_t)tk * p.nsb + s];
-      }
-      *(half8 *)(B_l + tt * GM_LD2) = bh;
-      *(half8 *)(B_l + tt * GM_LD2 + 8) = bl;
-      ad_l[tt] = adv;
-    }
-    __syncthreads();
-    {
-      const half8 a = *(const half8 *)(A_l + (32u * wr + l32) * GM_LD2 + 8u * lh);
-      const half8 b0 = *(const half8 *)(B_l + (64u * wt_ + l32) * GM_LD2 + 8u * lh);
-      const half8 b1 = *(const half8 *)(B_l + (64u * wt_ + 32u + l32) * GM_LD2 + 8u * lh);
-      float16v z = {};
-      const float16v i0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, z, 0, 0, 0);
-      const float16v i1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, z, 0, 0, 0);
-      const float ad0 = ad_l[64u * wt_ + l32], ad1 = ad_l[64u * wt_ + 32u + l32];
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const uint32_t row_l = 32u * wr + 8u * (r / 4) + 4u * lh + (r % 4);
-        const float dm = dmin_l[row_l];
-        y0[r] -= ad0 * dm * i0[r];
-        y1[r] -= ad1 * dm * i1[r];
-      }
-    }
-    __syncthreads();
+  for (uint32_t i = tid; i < p.nsb * 128u; i += 512u) {
+    const uint32_t s = i >> 7, lr = i & 127u;
+    const uint32_t h = *(const uint32_t *)(p.wt + (row_off(r0 + lr) + sb_off(s)));
+    dmin_t[i] = gm_f16_bits_to_f32(h >> 16);
   }
+  __syncthreads();
+  const uint32_t ro0 = row_off(r0 + 64u * wr + l32), ro1 = row_off(r0 + 64u * wr + 32u + l32);
+  const uint32_t tko = tk * p.nsb;  // this token's first (token, super-block) index
+  {
+    const float side_scale = lh ? 1.0f : 64.0f;
+    // four super-blocks at a time, so that four sets of loads share one trip to memory
+#pragma unroll 1
+    for (uint32_t sg = 0; sg < p.nsb; sg += 4u) {
+      uint4 hd0[4], hd1[4];
+      half8 b2[4];
+      float adv[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const uint32_t su = min(sg + u, p.nsb - 1u);
+        hd0[u] = *(const uint4 *)(p.wt + (ro0 + sb_off(su)));
+        hd1[u] = *(const uint4 *)(p.wt + (ro1 + sb_off(su)));
+        b2[u] = *(const half8 *)(p.bs16 + ((tko + su) * 16u + 8u * lh));
+        adv[u] = p.ad[tko + su];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        if (sg + u < p.nsb) {
+          uint32_t mna, mnb;
+          q4k_mins(hd0[u], mna, mnb);
+          const half8 a10 = side_operand(mna, mnb, side_scale);
+          q4k_mins(hd1[u], mna, mnb);
+          const half8 a11 = side_operand(mna, mnb, side_scale);
+          const float16v im0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a10, b2[u], zero, 0, 0, 0);
+          const float16v im1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a11, b2[u], zero, 0, 0, 0);
+          const float *dm = dmin_t + (sg + u) * 128u + 64u * wr + 4u * lh;
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++) {
+            const float4 m0 = *(const float4 *)(dm + 8 * q4), m1 = *(const float4 *)(dm + 32 + 8 * q4);
+            y0[4 * q4 + 0] -= adv[u] * m0.x * im0[4 * q4 + 0];
+            y0[4 * q4 + 1] -= adv[u] * m0.y * im0[4 * q4 + 1];
+            y0[4 * q4 + 2] -= adv[u] * m0.z * im0[4 * q4 + 2];
+            y0[4 * q4 + 3] -= adv[u] * m0.w * im0[4 * q4 + 3];
+            y1[4 * q4 + 0] -= adv[u] * m1.x * im1[4 * q4 + 0];
+            y1[4 * q4 + 1] -= adv[u] * m1.y * im1[4 * q4 + 1];
+            y1[4 * q4 + 2] -= adv[u] * m1.z * im1[4 * q4 + 2];
+            y1[4 * q4 + 3] -= adv[u] * m1.w * im1[4 * q4 + 3];
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();  // dmin_t is about to be overwritten by the staging buffers
 
   // ---------------- pass 2: acc += ad * (d * sum_j sc_j * dot32_j)
-  for (uint32_t s = 0; s < p.nsb; s++) {
-    float16v c0 = {}, c1 = {};   // first half of the super-block
-    float16v e0 = {}, e1 = {};   // second half
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-      // ---- stage the weight tile: thread -> (row block rbl, piece pi of this half, row r)
-      {
-        const uint32_t rbl = tid >> 6, j = tid & 63u, pi = j >> 4, r = j & 15u;
-        const uint32_t lr = rbl * 16u + r;
-        const size_t tile = (size_t)min(rb0 + rbl, p.nrb - 1u) * p.nct + s / 4u;
-        const uint8_t *ub = p.wt + tile * 9216u + ((s & 3u) * 16u + r) * 16u;
-        const uint4 hd = *(const uint4 *)ub;
-        const uint4 qv = *(const uint4 *)(ub + (1u + 4u * h + pi) * 1024u);
-        // get_scale_min_k4 (quant.rs:653-662): scales of sub-blocks 2g (low nibbles), 2g+1 (high)
-        const uint32_t sca = hd.y & 0x3F3F3F3Fu;
-        const uint32_t scb = (hd.w & 0x0F0F0F0Fu) | ((hd.y >> 2) & 0x30303030u);
-        const uint32_t g = 2u * h + (pi >> 1);
-        const uint32_t scw = g < 2 ? sca : scb;
-        const uint32_t sh = (g & 1u) * 16u;
-        const float slo = (float)((scw >> sh) & 0xFFu), shi = (float)((scw >> (sh + 8u)) & 0xFFu);
-        half2v sl2, nl2, sh2, nh2;
-        sl2[0] = sl2[1] = (_Float16)slo;
-        nl2[0] = nl2[1] = (_Float16)(-1024.0f * slo);
-        sh2[0] = sh2[1] = (_Float16)shi;
-        nh2[0] = nh2[1] = (_Float16)(-1024.0f * shi);
-        uint4 lo_a, lo_b, hi_a, hi_b;  // 16 low-nibble weights, 16 high-nibble weights, as f16
-        dequant4(qv.x, 0, sl2, nl2, lo_a.x, lo_a.y);
-        dequant4(qv.y, 0, sl2, nl2, lo_a.z, lo_a.w);
-        dequant4(qv.z, 0, sl2, nl2, lo_b.x, lo_b.y);
-        dequant4(qv.w, 0, sl2, nl2, lo_b.z, lo_b.w);
-        dequant4(qv.x, 4, sh2, nh2, hi_a.x, hi_a.y);
-        dequant4(qv.y, 4, sh2, nh2, hi_a.z, hi_a.w);
-        dequant4(qv.z, 4, sh2, nh2, hi_b.x, hi_b.y);
-        dequant4(qv.w, 4, sh2, nh2, hi_b.z, hi_b.w);
-        // piece 1+2g+hh holds qs[32g+16hh ..]: low nibbles are elements 64g+16hh.., high +32
-        _Float16 *dst = A_l + lr * GM_LD + 64u * (pi >> 1) + 16u * (pi & 1u);
-        *(uint4 *)(dst) = lo_a;
-        *(uint4 *)(dst + 8) = lo_b;
-        *(uint4 *)(dst + 32) = hi_a;
-        *(uint4 *)(dst + 40) = hi_b;
-        if (h == 0 && pi == 0) d_l[lr] = gm_f16_bits_to_f32(hd.x & 0xFFFFu);
-      }
-      // ---- stage the activation tile: thread -> (token tt, 64 k)
-      {
-        const uint32_t tt = tid >> 1, kh = tid & 1u, tk = t0 + tt;
-        uint4 v[8];
-        if (tk < p.n_tokens) {
-          const uint4 *src = (const uint4 *)(p.xh + (size_t)tk * p.in_dim + (size_t)s * 256u + 128u * h + 64u * kh);
-#pragma unroll
-          for (int i = 0; i < 8; i++) v[i] = src[i];
-        } else {
-#pragma unroll
-          for (int i = 0; i < 8; i++) v[i] = make_uint4(0, 0, 0, 0);
-        }
-        uint4 *dst = (uint4 *)(B_l + tt * GM_LD + 64u * kh);
-#pragma unroll
-        for (int i = 0; i < 8; i++) dst[i] = v[i];
-        if (h == 0 && tid < GM_BT) {
-          const uint32_t tk2 = t0 + tid;
-          ad_l[tid] = tk2 < p.n_tokens ? p.ad[(size_t)tk2 * p.nsb + s] : 0.0f;
-        }
-      }
-      __syncthreads();
-      // ---- 8 k-steps of 16
-      const _Float16 *ap = A_l + (32u * wr + l32) * GM_LD + 8u * lh;
-      const _Float16 *bp0 = B_l + (64u * wt_ + l32) * GM_LD + 8u * lh;
-      const _Float16 *bp1 = bp0 + 32u * GM_LD;
-#pragma unroll
-      for (int kk = 0; kk < 8; kk++) {
-        const half8 a = *(const half8 *)(ap + 16 * kk);
-        const half8 b0 = *(const half8 *)(bp0 + 16 * kk);
-        const half8 b1 = *(const half8 *)(bp1 + 16 * kk);
-        if (h == 0) {
-          c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, c0, 0, 0, 0);
-          c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, c1, 0, 0, 0);
-        } else {
-          e0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, e0, 0, 0, 0);
-          e1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, e1, 0, 0, 0);
-        }
-      }
-      if (h == 1) {
-        const float ad0 = ad_l[64u * wt_ + l32], ad1 = ad_l[64u * wt_ + 32u + l32];
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const uint32_t row_l = 32u * wr + 8u * (r / 4) + 4u * lh + (r % 4);
-          const float d = d_l[row_l];
-          y0[r] += ad0 * (d * (c0[r] + e0[r]));
-          y1[r] += ad1 * (d * (c1[r] + e1[r]));
-        }
-      }
-      __syncthreads();
-    }
-  }
+  // Staging roles.  Weights: half a 16-byte piece of qs per thread (8 bytes = 8 low-nibble and 8
+  // high-nibble weights).  Activations: two 16-byte chunks per thread.  Once per super-block
+  // also the row's scales (side operand and d) and one chunk of bh | bl.
+  const uint32_t pid = tid >> 1, half = tid & 1u;
+  const uint32_t lr_a = (pid >> 5) * 16u + (pid & 15u), hh = (pid >> 4) & 1u;
+  const uint32_t btok = tid >> 3, bpart = tid & 7u;   // chunk i: token btok + 64 i, part bpart
+  const uint32_t bt0 = min(t0 + btok, p.n_tokens - 1u), bt1 = min(t0 + btok + 64u, p.n_tokens - 1u);
+  const uint32_t roa = row_off(r0 + lr_a) + hh * 1024u + 8u * half;   // this thread's half piece
+  const uint32_t bo0 = bt0 * p.in_dim + bpart * 8u, bo1 = bt1 * p.in_dim + bpart * 8u;  // in f16
+  // (the upper half of the workgroup repeats the lower half's bh | bl chunk: no branch needed)
+  const uint32_t b2o = min(t0 + ((tid & 255u) >> 1), p.n_tokens - 1u) * p.nsb * 16u + 8u * (tid & 1u);
+  // Loads run three stages ahead of the MFMAs through four rotating register sets (a stage is
+  // far shorter than a trip to memory); the header and bh | bl loads of a super-block have one
+  // set, which is consumed before the next super-block's are issued.
+  uint2 qv_0, qv_1, qv_2, qv_3;
+  uint4 bx0_0, bx0_1, bx0_2, bx0_3, bx1_0, bx1_1, bx1_2, bx1_3;
+  uint4 hdx = make_uint4(0, 0, 0, 0), b2x = make_uint4(0, 0, 0, 0);
+  uint32_t sca = 0, scb = 0;
+  float dnext = 0.0f;
 
-  // ---------------- store: lane holds token column l32 (+32), rows in runs of four
+#define GM_LOAD_STAGE(S, G, K)                                                                    \
+  do {                                                                                            \
+    const uint32_t so_ = sb_off(S);                                                               \
+    if ((G) == 0) hdx = *(const uint4 *)(p.wt + (roa - hh * 1024u - 8u * half + so_));            \
+    if ((G) == 1) b2x = *(const uint4 *)(p.bs16 + (b2o + (S) * 16u));                              \
+    qv_##K = *(const uint2 *)(p.wt + (roa + so_ + (1u + 2u * (G)) * 1024u));                      \
+    const uint32_t ko_ = (S) * 256u + (G) * 64u;                                                  \
+    bx0_##K = *(const uint4 *)(p.xh + (bo0 + ko_));                                               \
+    bx1_##K = *(const uint4 *)(p.xh + (bo1 + ko_));                                               \
+  } while (0)
+
+#define GM_STORE_STAGE(G, BUF, K)                                                                 \
+  do {                                                                                            \
+    if ((G) == 0) {                                                                               \
+      q4k_scales(hdx, sca, scb);                                                                  \
+      dnext = gm_f16_bits_to_f32(hdx.x & 0xFFFFu);                                                \
+    }                                                                                             \
+    const uint32_t scw_ = (G) < 2 ? sca : scb;                                                    \
+    const uint32_t sh_ = ((G) & 1u) * 16u;                                                        \
+    const _Float16 slo_ = (_Float16)(float)((scw_ >> sh_) & 0xFFu);                               \
+    const _Float16 shi_ = (_Float16)(float)((scw_ >> (sh_ + 8u)) & 0xFFu);                        \
+    const half2v sl2_ = {slo_, slo_}, sh2_ = {shi_, shi_};                                        \
+    uint4 lo_, hi_; /* 8 low-nibble weights, 8 high-nibble weights, as f16 */                     \
+    dequant8(qv_##K.x, sl2_, sh2_, lo_.x, lo_.y, hi_.x, hi_.y);                                   \
+    dequant8(qv_##K.y, sl2_, sh2_, lo_.z, lo_.w, hi_.z, hi_.w);                                   \
+    /* piece 1+2g+hh holds qs[32g+16hh ..]: low nibbles are k 16hh.. of the stage, high 32+16hh.. */ \
+    _Float16 *ab_ = A_l + (BUF) * GM_STAGE_HALFS;                                                 \
+    *(uint4 *)(ab_ + gm_swz(lr_a, 2u * hh + half)) = lo_;                                         \
+    *(uint4 *)(ab_ + gm_swz(lr_a, 4u + 2u * hh + half)) = hi_;                                    \
+    _Float16 *bb_ = B_l + (BUF) * GM_STAGE_HALFS;                                                 \
+    *(uint4 *)(bb_ + gm_swz(btok, bpart)) = bx0_##K;                                              \
+    *(uint4 *)(bb_ + gm_swz(btok + 64u, bpart)) = bx1_##K;                                        \
+    if ((G) == 1) {                                                                               \
+      /* Side tables of this super-block.  Their readers (after stage 3) of the last super-block \
+         are two barriers behind, their next readers two barriers ahead. */                      \
+      /* the four threads of a row write the same values */                                      \
+      *(half8 *)(a2_l + lr_a * 16u + 8u * half) = side_operand(sca, scb, half ? 8.0f : 512.0f);   \
+      d_l[lr_a] = dnext;                                                                          \
+      *(uint4 *)(b2_l + ((tid & 255u) >> 1) * 16u + 8u * (tid & 1u)) = b2x;                       \
+    }                                                                                             \
+  } while (0)
+
+  // One stage: issue the loads of the stage three ahead, then this stage's MFMAs with the
+  // dequantization of the next stage (into the other LDS buffer) in their shadow, then, after
+  // the super-block's last stage, its f32 step.
+#define GM_STAGE(G, KL, KS)                                                                       \
+  do {                                                                                            \
+    const uint32_t buf = (G) & 1u;                                                                \
+    if ((G) == 0) adv = p.ad[tko + s]; /* needed three stages from now */                         \
+    /* past the end the last super-block is loaded again and parked in the idle buffer */        \
+    GM_LOAD_STAGE(min((G) == 0 ? s : s + 1u, p.nsb - 1u), (uint32_t)(((G) + 3) & 3), KL);         \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+    const _Float16 *ab = A_l + buf * GM_STAGE_HALFS, *bb = B_l + buf * GM_STAGE_HALFS;            \
+    half8 a0 = *(const half8 *)(ab + gm_swz(ra, lh));                                             \
+    half8 a1 = *(const half8 *)(ab + gm_swz(ra + 32u, lh));                                       \
+    half8 b0 = *(const half8 *)(bb + gm_swz(rbk, lh));                                            \
+    _Pragma("unroll") for (int kk = 0; kk < 4; kk++) {                                            \
+      half8 na0 = a0, na1 = a1, nb0 = b0;                                                         \
+      if (kk < 3) {                                                                               \
+        na0 = *(const half8 *)(ab + gm_swz(ra, 2u * (kk + 1) + lh));                              \
+        na1 = *(const half8 *)(ab + gm_swz(ra + 32u, 2u * (kk + 1) + lh));                        \
+        nb0 = *(const half8 *)(bb + gm_swz(rbk, 2u * (kk + 1) + lh));                             \
+      }                                                                                           \
+      /* the super-block's first step starts a fresh accumulator */                              \
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b0, ((G) == 0 && kk == 0) ? zero : c0, 0, 0, 0); \
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, ((G) == 0 && kk == 0) ? zero : c1, 0, 0, 0); \
+      a0 = na0; a1 = na1; b0 = nb0;                                                               \
+    }                                                                                             \
+    GM_STORE_STAGE((uint32_t)(((G) + 1) & 3), buf ^ 1u, KS);                                      \
+    /* the dequantization of the next stage goes into the shadow of this stage's MFMAs */        \
+    _Pragma("unroll") for (int q_ = 0; q_ < 8; q_++) {                                            \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                          \
+      __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);                                          \
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                                          \
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                          \
+    }                                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+    if ((G) == 3) GM_SB_EPILOGUE();                                                               \
+    __syncthreads();                                                                              \
+  } while (0)
+
+  // isum = c + corr (one rounding of the exact integer), then the reference's f32 steps
+#define GM_SB_EPILOGUE()                                                                          \
+  do {                                                                                            \
+    const half8 b2 = *(const half8 *)(b2_l + rbk * 16u + 8u * lh);                                \
+    const half8 a20 = *(const half8 *)(a2_l + ra * 16u + 8u * lh);                                \
+    const half8 a21 = *(const half8 *)(a2_l + (ra + 32u) * 16u + 8u * lh);                        \
+    const float16v corr0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a20, b2, zero, 0, 0, 0);        \
+    const float16v corr1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a21, b2, zero, 0, 0, 0);        \
+    const float *dp = d_l + 64u * wr + 4u * lh;                                                   \
+    _Pragma("unroll") for (int q4 = 0; q4 < 4; q4++) {                                            \
+      const float4 d0 = *(const float4 *)(dp + 8 * q4), d1 = *(const float4 *)(dp + 32 + 8 * q4); \
+      y0[4 * q4 + 0] += adv * (d0.x * (c0[4 * q4 + 0] + corr0[4 * q4 + 0]));                      \
+      y0[4 * q4 + 1] += adv * (d0.y * (c0[4 * q4 + 1] + corr0[4 * q4 + 1]));                      \
+      y0[4 * q4 + 2] += adv * (d0.z * (c0[4 * q4 + 2] + corr0[4 * q4 + 2]));                      \
+      y0[4 * q4 + 3] += adv * (d0.w * (c0[4 * q4 + 3] + corr0[4 * q4 + 3]));                      \
+      y1[4 * q4 + 0] += adv * (d1.x * (c1[4 * q4 + 0] + corr1[4 * q4 + 0]));                      \
+      y1[4 * q4 + 1] += adv * (d1.y * (c1[4 * q4 + 1] + corr1[4 * q4 + 1]));                      \
+      y1[4 * q4 + 2] += adv * (d1.z * (c1[4 * q4 + 2] + corr1[4 * q4 + 2]));                      \
+      y1[4 * q4 + 3] += adv * (d1.w * (c1[4 * q4 + 3] + corr1[4 * q4 + 3]));                      \
+    }                                                                                             \
+  } while (0)
+
+  GM_LOAD_STAGE(0u, 0u, 0);
+  GM_LOAD_STAGE(0u, 1u, 1);
+  GM_LOAD_STAGE(0u, 2u, 2);
+  GM_STORE_STAGE(0u, 0u, 0);
+  __syncthreads();
+
+  const uint32_t ra = 64u * wr + l32, rbk = 32u * wt_ + l32;
+#pragma unroll 1
+  for (uint32_t s = 0; s < p.nsb; s++) {
+    float16v c0, c1;
+    float adv;
+    GM_STAGE(0, 3, 1);   // loads stage 4s+3 into set 3, parks stage 4s+1 from set 1
+    GM_STAGE(1, 0, 2);
+    GM_STAGE(2, 1, 3);
+    GM_STAGE(3, 2, 0);
+  }
+#undef GM_LOAD_STAGE
+#undef GM_STORE_STAGE
+#undef GM_STAGE
+#undef GM_SB_EPILOGUE
+
+  // ---------------- store: a lane holds one token column and its rows in runs of four
+  const uint32_t t = t0 + 32u * wt_ + l32;
+  if (t < p.n_tokens) {
+    const bool vec = (p.out_dim & 3u) == 0;
 #pragma unroll
-  for (int jt = 0; jt < 2; jt++) {
-    const uint32_t tk = t0 + 64u * wt_ + 32u * jt + l32;
-    if (tk >= p.n_tokens) continue;
-    const float16v &yy = jt ? y1 : y0;
+    for (int i = 0; i < 2; i++) {
+      const float16v &yy = i ? y1 : y0;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const uint32_t row = r0 + 32u * wr + 8u * (r / 4) + 4u * lh + (r % 4);
-      if (row < p.out_dim) p.y[(size_t)tk * p.out_dim + row] = yy[r];
+      for (int q4 = 0; q4 < 4; q4++) {
+        const uint32_t row = r0 + 64u * wr + 32u * i + 8u * q4 + 4u * lh;
+        float *dst = p.y + (size_t)t * p.out_dim + row;
+        if (vec && row + 3u < p.out_dim) {
+          *(float4 *)dst = make_float4(yy[4 * q4], yy[4 * q4 + 1], yy[4 * q4 + 2], yy[4 * q4 + 3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            if (row + e < p.out_dim) dst[e] = yy[4 * q4 + e];
+        }
+      }
     }
   }
 }
 
-size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens) { return (size_t)in_dim * n_tokens * 2; }
+static const uint32_t GM_LDS_BYTES = 4 * GM_STAGE_HALFS * 2 + 2 * 128 * 16 * 2 + 128 * 4;
+static const uint32_t GM_STAGING_BYTES = 4 * GM_STAGE_HALFS * 2;
 
-bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim) {
-  return ggml_type == OGM_Q4_K && in_dim % 1024u == 0;  // tiles of 16 rows x 4 super-blocks
+size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens) {
+  // f16 activations, then the (bh, bl) pairs: 16 f16 per (token, super-block)
+  return (size_t)in_dim * n_tokens * 2 + (size_t)(in_dim / 256) * n_tokens * 32;
+}
+
+bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
+  if (ggml_type != OGM_Q4_K || in_dim == 0 || in_dim % 256u != 0) return false;
+  // pass 1 keeps one f32 per (row, super-block) of the workgroup in the staging area of LDS
+  if ((size_t)(in_dim / 256u) * 512u > GM_STAGING_BYTES) return false;
+  // the kernel addresses weights and activations with 32-bit byte offsets
+  const uint64_t lim = 0xFFFFFFFFull;
+  return (uint64_t)ogm_tiling_for(in_dim / 256u, out_dim).nrb * 64u * (in_dim / 256u) * 144u <= lim &&
+         (uint64_t)in_dim * n_tokens * 2u <= lim;
 }
 
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name) {
   if (a.n_tokens == 0 || a.out_dim == 0) return hipSuccess;
-  if (!ogm_gemm_supported(a.ggml_type, a.in_dim)) return hipErrorInvalidValue;
-  const size_t n8 = (size_t)a.in_dim * a.n_tokens / 8;
-  hipLaunchKernelGGL(ogm_q8_to_f16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, stream,
-                     a.act.q, (_Float16 *)a.xh, n8);
+  if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return hipErrorInvalidValue;
+  const uint32_t nsb = a.in_dim / 256;
+  const size_t n8 = (size_t)a.in_dim * a.n_tokens / 8, n_sb = (size_t)nsb * a.n_tokens;
+  _Float16 *xh = (_Float16 *)a.xh;
+  _Float16 *bs16 = xh + (size_t)a.in_dim * a.n_tokens;
+  hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, stream,
+                     a.act.q, a.act.bsum, xh, bs16, n8, n_sb);
   GemmParams p;
   p.wt = a.wt;
-  p.xh = (const _Float16 *)a.xh;
+  p.xh = xh;
+  p.bs16 = bs16;
   p.ad = a.act.d;
-  p.bsum = a.act.bsum;
   p.y = a.y;
   p.in_dim = a.in_dim;
   p.out_dim = a.out_dim;
   p.n_tokens = a.n_tokens;
-  p.nsb = a.in_dim / 256;
-  p.nct = p.nsb / 4;
-  p.nrb = (a.out_dim + 15) / 16;
-  const size_t lds = (size_t)(GM_BN + GM_BT) * GM_LD * 2 + (GM_BN * 2 + GM_BT) * 4;
-  const dim3 grid((a.out_dim + GM_BN - 1) / GM_BN, (a.n_tokens + GM_BT - 1) / GM_BT);
-  hipLaunchKernelGGL(ogm_gemm_q4k_kernel, grid, dim3(256), lds, stream, p);
+  p.nsb = nsb;
+  const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
+  p.c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
+  p.r_shift = 6 - p.c_shift;
+  p.nct = tl.nct;
+  // token tiles vary fastest: workgroups that run together share weight rows, and with a
+  // power-of-two number of token tiles each XCD's L2 sees few distinct activation tiles
+  const dim3 grid((a.n_tokens + GM_BT - 1) / GM_BT, (a.out_dim + GM_BN - 1) / GM_BN);
+  // more dynamic LDS than the 64 KB a kernel gets without asking
+  hipError_t e = hipFuncSetAttribute((const void *)ogm_gemm_q4k_kernel,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)GM_LDS_BYTES);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(ogm_gemm_q4k_kernel, grid, dim3(512), GM_LDS_BYTES, stream, p);
   if (kernel_name) *kernel_name = "ogm_gemm_q4k_kernel";
   return hipGetLastError();
 }

@@ -59,7 +59,7 @@ struct OgmGemmArgs {
   float *y;            // [n_tokens][out_dim]
   void *xh;            // scratch
 };
-bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim);
+bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens);
 size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens);
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name);
 

@@ -315,6 +315,7 @@ def test_q6k_vocab_projection_batches_1_4_8(be):
 
 @pytest.mark.parametrize("in_dim,out_dim,T", [
     (1024, 64, 9), (1024, 100, 64), (2048, 37, 128), (4096, 200, 130), (1024, 16, 300), (8192, 70, 33),
+    (256, 5, 9), (512, 130, 17), (768, 64, 129), (1280, 257, 40), (14336, 96, 257), (4096, 1000, 512),
 ])
 def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     """ogm_matmul at n_tokens >= 9 takes the MFMA kernel; values must equal CpuBackend's K-quant
@@ -350,23 +351,36 @@ def test_mfma_gemm_equals_small_batch_kernel_and_is_batch_independent(be):
         assert_bits(part, full[:n], f"{n} of 40")
 
 
-def test_mfma_gemm_adversarial_integer_ranges(be):
-    """Largest magnitudes the integer stage can see: all nibbles 15, scales and mins 63, activations
-    +-127: the per-super-block sum (3.1e7) exceeds 2^24, so the two-half f32 add must round exactly
-    like `isum as f32`."""
+@pytest.mark.parametrize("qs_lo,qs_hi,sign", [(0xFF, 0xFF, "alt"), (0x00, 0x00, "alt"), (0x0F, 0xF0, "pos"),
+                                               (0xF0, 0x0F, "neg"), (0xFF, 0x00, "block")])
+def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign):
+    """Largest magnitudes the integer stage can see: nibbles 0 or 15, scales and mins 63, activations
+    +-127.  The per-super-block sum reaches 3.1e7 > 2^24 and the centred partial sums and their
+    correction reach +-1.64e7 each (and cancel when every nibble is 0), so the f32 add of the exact
+    parts must round exactly like `isum as f32`."""
     in_dim, out_dim, T = 1024, 32, 16
     blocks = np.zeros((out_dim * 4, 144), np.uint8)
     blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
     blocks[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
     blocks[:, 4:16] = 0xFF
-    blocks[:, 16:] = 0xFF
+    blocks[:, 16:80] = qs_lo
+    blocks[:, 80:] = qs_hi
     x = np.full((T, in_dim), 127.0, np.float32)
-    x[1::2] *= -1
-    x[:, ::7] = 126.0
+    if sign == "alt":
+        x[1::2] *= -1
+        x[:, ::7] = 126.0
+    elif sign == "neg":
+        x *= -1
+    elif sign == "block":
+        x[:, 128:256] *= -1
+        x[3] = -127.0
     raw = blocks.reshape(-1)
     got = be.matmul(x, T, qm(raw, Q4_K, in_dim, out_dim))
+    assert be.last_kernel() == "ogm_gemm_q4k_kernel"
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     assert_bits(got, want, "extreme ranges")
+    isum, imin = be.dump_block_sums(x[0], 1, qm(raw, Q4_K, in_dim, out_dim))
+    say("extreme isum", int(np.abs(isum).max()), "imin", int(np.abs(imin).max()))
 
 
 # ---------------------------------------------------------------- quantize inside the GEMV, grouped launches
