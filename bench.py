@@ -54,6 +54,9 @@ def main() -> int:
     ap.add_argument("--rb-per-wg", type=int, default=0, help="row blocks per GEMV workgroup (0 = heuristic)")
     ap.add_argument("--separate", action="store_true",
                     help="issue gate and up as two calls instead of one grouped call")
+    ap.add_argument("--gemm-tokens", type=int, default=512,
+                    help="tokens of the prefill GEMM leg (Q4_K 4096 -> 14336 on MFMA); 0 skips it")
+    ap.add_argument("--only-gemm", action="store_true", help="run only the prefill GEMM leg (for rocprofv3)")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the dominant-kernel leg (for rocprofv3 --kernel-trace --stats)")
     args = ap.parse_args()
@@ -104,7 +107,7 @@ def main() -> int:
     step_bytes = 2 * gemv_bytes(HIDDEN, FFN) + gemv_bytes(FFN, HIDDEN)
     result = {}
 
-    if not args.only_roofline:
+    if not args.only_roofline and not args.only_gemm:
         for i in range(args.warmup):
             step(i)
         stream.synchronize()
@@ -133,7 +136,7 @@ def main() -> int:
         e1.synchronize()
         return e0.elapsed_ms(e1) * 1e3 / n
 
-    n_launch = args.roofline_launches
+    n_launch = args.roofline_launches if not args.only_gemm else 1
     be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr)
     us_per_launch = timed(lambda i: be.matmul_multi_act_dev(
         [handles["gate"][i % copies], handles["up"][i % copies]], 1, [y_gate.ptr, y_up.ptr], False,
@@ -142,7 +145,7 @@ def main() -> int:
     kbytes = 2 * gemv_bytes(HIDDEN, FFN) - 4 * HIDDEN  # both matrices read the same x
     achieved = kbytes / (us_per_launch * 1e-6) / 1e9
     others = None
-    if not args.only_roofline:
+    if not args.only_roofline and not args.only_gemm:
         # the other launch shapes of the step, for the record (left out of the profiled run so
         # that the trace's average for the GEMV kernel covers the gate+up launches only)
         mats = handles["gate"] + handles["up"]
@@ -168,10 +171,41 @@ def main() -> int:
                 "bytes_per_launch": kbytes, "launches": n_launch,
                 "other_launches_us": others}
 
+    # ---- prefill GEMM on MFMA: Q4_K 4096 -> 14336 at --gemm-tokens tokens (quantize + f16 staging
+    # + GEMM kernel per call), checked against the CPU path on a sample of rows
+    gemm = None
+    if args.gemm_tokens > 0 and not args.only_roofline:
+        T = args.gemm_tokens
+        xg_h = helpers.synth_x(T, HIDDEN, seed + 7)
+        xg = hiprt.DeviceBuffer.from_numpy(xg_h)
+        yg = hiprt.DeviceBuffer(4 * T * FFN)
+        n_g = 20 if not args.only_gemm else 5
+        us_gemm = timed(lambda i: be.matmul_dev(handles["gate"][i % copies], xg.ptr, T, yg.ptr, False,
+                                                stream.ptr), n_g) if not args.only_gemm else None
+        if args.only_gemm:
+            for i in range(n_g):
+                be.matmul_dev(handles["gate"][i % copies], xg.ptr, T, yg.ptr, False, stream.ptr)
+            stream.synchronize()
+        gemm_kernel = be.last_kernel()
+        gemm = {"workload": f"Q4_K 4096->14336, {T} tokens (config a14 shape)", "kernel": gemm_kernel}
+        if us_gemm is not None:
+            flops = 2.0 * T * HIDDEN * FFN
+            gemm.update({"us_per_matmul": round(us_gemm, 1), "tflops": round(flops / us_gemm / 1e6, 1),
+                         "frac_of_f16_mfma_peak": round(flops / us_gemm / 1e6 / 2500.0, 4)})
+        if not args.only_gemm and args.cpu_seconds > 0:
+            import oracle
+            rows = np.r_[0:32, 7000:7032, FFN - 32:FFN]
+            rb = HIDDEN // 256 * 144
+            sub = np.concatenate([raw["gate"][r * rb:(r + 1) * rb] for r in rows])
+            want = oracle.matmul(Q4_K, sub, HIDDEN, rows.size, xg_h, T).reshape(T, rows.size)
+            got = yg.to_numpy(np.float32, T * FFN).reshape(T, FFN)[:, rows]
+            gemm["parity_vs_cpu"] = "bit-exact" if np.array_equal(got.view(np.uint32), want.view(np.uint32)) \
+                else ("within 1e-3/1e-5" if np.all(np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-5) else "FAILED")
+
     # ---- parity of what was just timed + CPU baseline (the oracle, all host cores) -------------
     cpu = None
     parity = None
-    if not args.only_roofline and args.cpu_seconds > 0:
+    if not args.only_roofline and not args.only_gemm and args.cpu_seconds > 0:
         import oracle
         step(0)
         stream.synchronize()
@@ -231,6 +265,7 @@ def main() -> int:
                    "parity_vs_cpu": parity, "device": be.device_name()},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "prefill_gemm": gemm,
     }
     print(json.dumps(out))
     be.close()
