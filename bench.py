@@ -39,6 +39,57 @@ def gemv_bytes(in_dim: int, out_dim: int, t: int = 1) -> int:
     return out_dim * (in_dim // 256 * 144) + 4 * in_dim * t + 4 * out_dim * t
 
 
+def sweep(be, helpers, hiprt) -> dict:
+    """Kernel timings at the full size of every benchmark configuration: device-resident inputs,
+    back-to-back calls over weight copies totalling more than the 256 MB last-level cache, HIP events
+    on the launch stream.  Each figure covers the whole call (activation quantizer + matmul kernels)."""
+    Q8_0, Q6_K = 8, 14
+    blk = {Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256)}
+    names = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+    stream = hiprt.Stream()
+    out = {"device": be.device_name(), "unit": "us per call; GB/s and TFLOP/s are algorithmic", "rows": []}
+
+    def run(t, in_dim, out_dim, T, decode, label, n=60):
+        w_bytes = out_dim * (in_dim // blk[t][1]) * blk[t][0]
+        copies = max(2, min(24, (300 << 20) // w_bytes + 1))
+        raw = helpers.synth_weights(t, in_dim, out_dim, 11)
+        hs = [be.upload_raw(raw, t, in_dim, out_dim) for _ in range(copies)]
+        x = hiprt.DeviceBuffer.from_numpy(helpers.synth_x(T, in_dim, 5))
+        y = hiprt.DeviceBuffer(4 * T * out_dim)
+        for i in range(5):
+            be.matmul_dev(hs[i % copies], x.ptr, T, y.ptr, decode, stream.ptr)
+        stream.synchronize()
+        e0, e1 = hiprt.Event(), hiprt.Event()
+        e0.record(stream)
+        for i in range(n):
+            be.matmul_dev(hs[i % copies], x.ptr, T, y.ptr, decode, stream.ptr)
+        e1.record(stream)
+        e1.synchronize()
+        us = e0.elapsed_ms(e1) * 1e3 / n
+        nbytes = w_bytes + 4 * T * (in_dim + out_dim)
+        flops = 2.0 * T * in_dim * out_dim
+        out["rows"].append({"config": label, "type": names[t], "in": in_dim, "out": out_dim, "tokens": T,
+                            "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                            "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                            "TFLOPs": round(flops / us / 1e6, 2), "kernel": be.last_kernel()})
+        for h in hs:
+            be.free_weight(h)
+        x.free()
+        y.free()
+
+    run(Q8_0, 4096, 4096, 1, False, "C1 GEMV")
+    run(Q4_K, HIDDEN, FFN, 1, False, "C2 gate/up GEMV")
+    run(Q4_K, FFN, HIDDEN, 1, False, "C2 down GEMV")
+    for T in (1, 4, 8):
+        run(Q6_K, 4096, 128256, T, False, f"C3 vocab batch {T}", n=20)
+        run(Q4_K, 4096, 4096, T, False, f"C3 q/o batch {T}")
+        run(Q4_K, 4096, 1024, T, False, f"C3 k/v batch {T}")
+    for T in (128, 512, 2048):
+        run(Q4_K, HIDDEN, FFN, T, False, f"C4 prefill GEMM M={T}", n=20)
+    run(Q6_K, FFN, HIDDEN, 1, False, "C5 ffn_down GEMV")
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -57,6 +108,9 @@ def main() -> int:
     ap.add_argument("--gemm-tokens", type=int, default=512,
                     help="tokens of the prefill GEMM leg (Q4_K 4096 -> 14336 on MFMA); 0 skips it")
     ap.add_argument("--only-gemm", action="store_true", help="run only the prefill GEMM leg (for rocprofv3)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="time every benchmark configuration's kernels instead (one JSON object, not the "
+                         "headline line)")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the dominant-kernel leg (for rocprofv3 --kernel-trace --stats)")
     args = ap.parse_args()
@@ -71,6 +125,10 @@ def main() -> int:
     from orangu_amd import hiprt
 
     be = Mi355xBackend()  # raises without the HIP library or a gfx950 device
+    if args.sweep:
+        print(json.dumps(sweep(be, helpers, hiprt)))
+        be.close()
+        return 0
     if args.wg_waves:
         be.set_tuning("gemv_wg_waves", args.wg_waves)
     if args.rb_per_wg:

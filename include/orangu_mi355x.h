@@ -178,6 +178,51 @@ int ogm_dump_block_sums(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint3
  * test compare the device conversion with quant::f16_bits_to_f32 (quant.rs:511-528). */
 int ogm_f16_to_f32(ogm_ctx *ctx, const uint16_t *bits, size_t n, float *out);
 
+/* ---- Llama-family decode step (the callers either side of the matmuls) ------------------------ */
+
+/* One token through every layer without returning to the host: what LlamaModel::run_layers +
+ * forward do at n_tokens == 1 (engine/arch/llama.rs:594-932, 1007-1032) -- RMSNorm
+ * (tensor.rs:732-757), q/k/v, NORM-paired RoPE (tensor.rs:1115-1177; freq_scale 1, no YaRN, no
+ * frequency factors), KV-cache append, causal grouped-query attention (attention.rs:426-549), wo,
+ * residual, RMSNorm, SwiGLU FFN (arch/mod.rs:1071-1106), residual; then the output norm and the
+ * vocabulary projection.  The matmuls are ogm_matmul's single-token path, bit for bit; the
+ * element-wise kernels use tree reductions and the KV cache is f16 (the reference's host cache is
+ * f32, kv_cache.rs:75-78), so logits agree with the CPU forward pass to tolerance, not to the bit. */
+typedef struct ogm_llama ogm_llama;
+typedef struct ogm_llama_config {
+  uint32_t n_layer, n_embd, n_head, n_head_kv, head_dim, n_ff, n_vocab;
+  uint32_t rope_dim;    /* rotated dimensions per head, <= head_dim */
+  uint32_t max_ctx;     /* KV-cache capacity in positions */
+  float rms_eps, rope_freq_base;
+} ogm_llama_config;
+typedef struct ogm_llama_layer {
+  const ogm_weight *wq, *wk, *wv, *wo, *w_gate, *w_up, *w_down;
+  const float *attn_norm, *ffn_norm;   /* host f32 [n_embd], copied */
+} ogm_llama_layer;
+
+/* Builds the device-side model over weights already uploaded with ogm_weight_upload (they must
+ * outlive it).  `layers` has cfg->n_layer entries; output_norm is host f32 [n_embd]. */
+int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const ogm_llama_layer *layers,
+                     const float *output_norm, const ogm_weight *output, ogm_llama **out);
+void ogm_llama_destroy(ogm_ctx *ctx, ogm_llama *m);
+
+/* Writes cache rows pos0 .. pos0+n_pos of one layer from host f32 [n_pos][n_head_kv*head_dim]
+ * (K already rotated), as a CPU prefill hands its cache over (LayerCache::push, kv_cache.rs:756-768). */
+int ogm_llama_kv_write(ogm_ctx *ctx, ogm_llama *m, uint32_t layer, uint32_t pos0, uint32_t n_pos,
+                       const float *k, const float *v);
+
+/* Decodes the token at position `pos` whose embedding row is x ([n_embd] f32; the caller looks it
+ * up as run_layers does, llama.rs:609-614).  Appends its K/V at `pos`, attends to 0..pos.
+ * logits ([n_vocab]) and argmax may each be null.  Host pointers; synchronizes. */
+int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos, float *logits,
+                     uint32_t *argmax);
+/* The same with device pointers, enqueued on `stream` (null = the context's) without waiting. */
+int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_t pos, float *logits_dev,
+                         uint32_t *argmax_dev, void *stream);
+/* The last decode's final hidden state, before the output norm ([n_embd] host f32; what
+ * run_layers returns), for parity checks. */
+int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out);
+
 /* ---- tuning / introspection ------------------------------------------------------------------ */
 
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.

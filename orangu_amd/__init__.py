@@ -5,7 +5,7 @@ The product is the C-ABI shared library (``include/orangu_mi355x.h``) built from
 reference's ``Backend`` trait used by tests and the benchmark.
 """
 from .capi import LIB_PATH, OgmError, load_library  # noqa: F401
-from .backend import Mi355xBackend, MatmulOp, QuantMatrix  # noqa: F401
+from .backend import LlamaDecoder, Mi355xBackend, MatmulOp, QuantMatrix  # noqa: F401
 
 GGML_TYPE_Q8_0 = 8
 GGML_TYPE_Q4_K = 12

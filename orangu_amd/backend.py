@@ -269,8 +269,75 @@ class Mi355xBackend:
         self._check(rc, "ogm_weight_upload")
         return handle.value
 
+    def free_weight(self, w_handle: int):
+        """Releases a device copy made by upload_raw (cached uploads live as long as the backend)."""
+        self._check(self._lib.ogm_weight_free(self._ctx, w_handle), "ogm_weight_free")
+
     def set_tuning(self, key: str, value: int):
         self._check(self._lib.ogm_set_tuning(self._ctx, key.encode(), value), "ogm_set_tuning")
 
     def last_kernel(self) -> str:
         return self._lib.ogm_last_kernel(self._ctx).decode()
+
+
+class LlamaDecoder:
+    """The device-resident decode step of a Llama-family model over a Mi355xBackend
+    (LlamaModel::forward at n_tokens == 1, engine/arch/llama.rs:1007-1032).
+
+    ``layers`` is a list of dicts with QuantMatrix entries wq, wk, wv, wo, w_gate, w_up, w_down and
+    f32 arrays attn_norm, ffn_norm; ``output`` a QuantMatrix; ``output_norm`` an f32 array."""
+
+    def __init__(self, be: "Mi355xBackend", *, n_embd: int, n_head: int, n_head_kv: int, head_dim: int,
+                 n_ff: int, n_vocab: int, layers, output_norm, output, max_ctx: int, rope_dim: int | None = None,
+                 rms_eps: float = 1e-5, rope_freq_base: float = 10000.0, upload=None):
+        self._be = be
+        up = upload or be.upload
+        cfg = capi.OgmLlamaConfig(len(layers), n_embd, n_head, n_head_kv, head_dim, n_ff, n_vocab,
+                                  head_dim if rope_dim is None else rope_dim, max_ctx, rms_eps, rope_freq_base)
+        arr = (capi.OgmLlamaLayer * len(layers))()
+        self._keep = []
+        for i, L in enumerate(layers):
+            for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
+                setattr(arr[i], name, up(L[name]))
+            for name in ("attn_norm", "ffn_norm"):
+                a = np.ascontiguousarray(L[name], np.float32)
+                self._keep.append(a)
+                setattr(arr[i], name, a.ctypes.data)
+        on = np.ascontiguousarray(output_norm, np.float32)
+        h = C.c_void_p()
+        be._check(be._lib.ogm_llama_create(be._ctx, C.byref(cfg), arr, on.ctypes.data, up(output), C.byref(h)),
+                  "ogm_llama_create")
+        self._h = h.value
+        self.n_embd, self.n_vocab, self.kv_dim = n_embd, n_vocab, n_head_kv * head_dim
+
+    def kv_write(self, layer: int, pos0: int, k, v):
+        k = np.ascontiguousarray(k, np.float32).reshape(-1, self.kv_dim)
+        v = np.ascontiguousarray(v, np.float32).reshape(-1, self.kv_dim)
+        self._be._check(self._be._lib.ogm_llama_kv_write(self._be._ctx, self._h, layer, pos0, k.shape[0],
+                                                         k.ctypes.data, v.ctypes.data), "ogm_llama_kv_write")
+
+    def decode(self, x, pos: int):
+        """Returns (logits, argmax) for the token whose embedding row is x, at position pos."""
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        if x.size != self.n_embd:
+            raise ValueError(f"x has {x.size} values, n_embd = {self.n_embd}")
+        logits = np.empty(self.n_vocab, np.float32)
+        am = C.c_uint32()
+        self._be._check(self._be._lib.ogm_llama_decode(self._be._ctx, self._h, x.ctypes.data, pos,
+                                                       logits.ctypes.data, C.byref(am)), "ogm_llama_decode")
+        return logits, am.value
+
+    def decode_dev(self, x_ptr: int, pos: int, logits_ptr: int = 0, argmax_ptr: int = 0, stream: int = 0):
+        self._be._check(self._be._lib.ogm_llama_decode_dev(self._be._ctx, self._h, x_ptr, pos, logits_ptr or None,
+                                                           argmax_ptr or None, stream or None), "ogm_llama_decode_dev")
+
+    def hidden(self) -> np.ndarray:
+        out = np.empty(self.n_embd, np.float32)
+        self._be._check(self._be._lib.ogm_llama_debug_hidden(self._be._ctx, self._h, out.ctypes.data),
+                        "ogm_llama_debug_hidden")
+        return out
+
+    def close(self):
+        if self._h:
+            self._be._lib.ogm_llama_destroy(self._be._ctx, self._h)
+            self._h = None

@@ -23,6 +23,8 @@ SYMBOLS = [
     "ogm_weight_info", "ogm_matmul", "ogm_matmul_decode", "ogm_matmul_batch", "ogm_matmul_dev",
     "ogm_quantize_act", "ogm_dump_block_sums", "ogm_f16_to_f32", "ogm_set_tuning",
     "ogm_last_kernel", "ogm_act_quantize_dev", "ogm_matmul_act_dev", "ogm_matmul_multi_dev", "ogm_matmul_multi_act_dev",
+    "ogm_llama_create", "ogm_llama_destroy", "ogm_llama_kv_write", "ogm_llama_decode", "ogm_llama_decode_dev",
+    "ogm_llama_debug_hidden",
 ]
 
 
@@ -30,6 +32,17 @@ class OgmError(RuntimeError):
     def __init__(self, status: int, where: str, detail: str = ""):
         self.status = status
         super().__init__(f"{where}: {STATUS.get(status, status)}" + (f" ({detail})" if detail else ""))
+
+
+class OgmLlamaConfig(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("n_layer", "n_embd", "n_head", "n_head_kv", "head_dim", "n_ff",
+                                          "n_vocab", "rope_dim", "max_ctx")] + \
+               [("rms_eps", C.c_float), ("rope_freq_base", C.c_float)]
+
+
+class OgmLlamaLayer(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down",
+                                          "attn_norm", "ffn_norm")]
 
 
 class OgmOp(C.Structure):
@@ -73,6 +86,13 @@ def load_library() -> C.CDLL:
     L.ogm_matmul_act_dev.argtypes = [vp, vp, u32, vp, C.c_int, vp]
     L.ogm_matmul_multi_dev.argtypes = [vp, C.POINTER(vp), sz, vp, u32, C.POINTER(vp), C.c_int, vp]
     L.ogm_matmul_multi_act_dev.argtypes = [vp, C.POINTER(vp), sz, u32, C.POINTER(vp), C.c_int, vp]
+    L.ogm_llama_create.argtypes = [vp, C.POINTER(OgmLlamaConfig), C.POINTER(OgmLlamaLayer), vp, vp, C.POINTER(vp)]
+    L.ogm_llama_destroy.argtypes = [vp, vp]
+    L.ogm_llama_destroy.restype = None
+    L.ogm_llama_kv_write.argtypes = [vp, vp, u32, u32, u32, vp, vp]
+    L.ogm_llama_decode.argtypes = [vp, vp, vp, u32, vp, vp]
+    L.ogm_llama_decode_dev.argtypes = [vp, vp, vp, u32, vp, vp, vp]
+    L.ogm_llama_debug_hidden.argtypes = [vp, vp, vp]
     L.ogm_quantize_act.argtypes = [vp, C.c_int, vp, sz, vp, vp, vp]
     L.ogm_dump_block_sums.argtypes = [vp, vp, vp, u32, vp, vp]
     L.ogm_f16_to_f32.argtypes = [vp, vp, sz, vp]

@@ -714,3 +714,282 @@ extern "C" int ogm_f16_to_f32(ogm_ctx *ctx, const uint16_t *bits, size_t n, floa
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   return OGM_OK;
 }
+
+// ------------------------------------------------------------------------------------------
+// Llama-family decode step
+
+#include <math.h>
+
+#include "ogm_llama.h"
+
+struct ogm_llama {
+  ogm_llama_config cfg;
+  std::vector<ogm_llama_layer> layers;  // weight handles; the norm pointers are unused after create
+  const ogm_weight *output = nullptr;
+  // device memory
+  float *norms = nullptr;     // [n_layer][2][n_embd] then output_norm [n_embd]
+  float *freq = nullptr;      // [rope_dim / 2]
+  void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
+  void *v_cache = nullptr;
+  float *x = nullptr;         // hidden state [n_embd]
+  float *q = nullptr, *k = nullptr, *v = nullptr;  // projections
+  float *proj = nullptr;      // wo / down output [n_embd]
+  float *gate = nullptr, *up = nullptr;            // [n_ff]
+  float *part_o = nullptr, *part_ml = nullptr;     // attention partials
+  float *logits = nullptr;    // [n_vocab]
+  uint32_t *amax_scratch = nullptr, *amax_out = nullptr;
+  float *stage = nullptr;     // host->device staging for ogm_llama_kv_write
+  size_t stage_cap = 0;
+  uint32_t max_splits = 0;
+  std::vector<void *> allocs;
+};
+
+static int llama_alloc(ogm_ctx *ctx, ogm_llama *m, void **p, size_t bytes) {
+  HIPCHK(ctx, hipMalloc(p, bytes ? bytes : 1));
+  m->allocs.push_back(*p);
+  return OGM_OK;
+}
+
+static void llama_free(ogm_llama *m) {
+  for (void *p : m->allocs) (void)hipFree(p);
+  if (m->stage) (void)hipFree(m->stage);
+  delete m;
+}
+
+static bool llama_weight_ok(const ogm_weight *w, uint32_t in_dim, uint32_t out_dim) {
+  return w && w->in_dim == in_dim && w->out_dim == out_dim;
+}
+
+extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const ogm_llama_layer *layers,
+                                const float *output_norm, const ogm_weight *output, ogm_llama **out) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!cfg || !layers || !output_norm || !output || !out) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  const ogm_llama_config c = *cfg;
+  if (c.n_layer == 0 || c.n_embd == 0 || c.n_head == 0 || c.n_head_kv == 0 || c.n_ff == 0 || c.max_ctx == 0)
+    return fail(ctx, OGM_ERR_INVALID, "empty model dimension");
+  if (c.n_head % c.n_head_kv != 0 || c.n_head / c.n_head_kv > 8)
+    return fail(ctx, OGM_ERR_UNSUPPORTED, "query heads per K/V head must divide evenly and be at most 8");
+  if (c.head_dim != 64 && c.head_dim != 128) return fail(ctx, OGM_ERR_UNSUPPORTED, "head_dim must be 64 or 128");
+  if (c.rope_dim > c.head_dim || c.rope_dim % 2 != 0) return fail(ctx, OGM_ERR_INVALID, "bad rope_dim");
+  if (c.n_embd > 16384 || c.n_embd % 32 != 0 || c.n_ff % 32 != 0)
+    return fail(ctx, OGM_ERR_UNSUPPORTED, "n_embd must be a multiple of 32 up to 16384, n_ff a multiple of 32");
+  const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
+  for (uint32_t l = 0; l < c.n_layer; l++) {
+    const ogm_llama_layer &L = layers[l];
+    if (!llama_weight_ok(L.wq, c.n_embd, qd) || !llama_weight_ok(L.wk, c.n_embd, kvd) ||
+        !llama_weight_ok(L.wv, c.n_embd, kvd) || !llama_weight_ok(L.wo, qd, c.n_embd) ||
+        !llama_weight_ok(L.w_gate, c.n_embd, c.n_ff) || !llama_weight_ok(L.w_up, c.n_embd, c.n_ff) ||
+        !llama_weight_ok(L.w_down, c.n_ff, c.n_embd) || !L.attn_norm || !L.ffn_norm)
+      return fail(ctx, OGM_ERR_INVALID, "layer " + std::to_string(l) + ": missing weight or wrong shape");
+  }
+  if (!llama_weight_ok(output, c.n_embd, c.n_vocab)) return fail(ctx, OGM_ERR_INVALID, "output weight shape");
+
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  ogm_llama *m = new (std::nothrow) ogm_llama();
+  if (!m) return fail(ctx, OGM_ERR_OOM, "out of host memory");
+  m->cfg = c;
+  m->layers.assign(layers, layers + c.n_layer);
+  m->output = output;
+  m->max_splits = (c.max_ctx + OGM_ATTN_CHUNK - 1) / OGM_ATTN_CHUNK;
+  const size_t cache_bytes = (size_t)c.n_layer * c.max_ctx * kvd * 2;
+  int rc = OGM_OK;
+  auto A = [&](void **p, size_t b) { if (rc == OGM_OK) rc = llama_alloc(ctx, m, p, b); };
+  A((void **)&m->norms, ((size_t)c.n_layer * 2 + 1) * c.n_embd * 4);
+  A((void **)&m->freq, (size_t)(c.rope_dim / 2 + 1) * 4);
+  A(&m->k_cache, cache_bytes);
+  A(&m->v_cache, cache_bytes);
+  A((void **)&m->x, (size_t)c.n_embd * 4);
+  A((void **)&m->q, (size_t)qd * 4);
+  A((void **)&m->k, (size_t)kvd * 4);
+  A((void **)&m->v, (size_t)kvd * 4);
+  A((void **)&m->proj, (size_t)c.n_embd * 4);
+  A((void **)&m->gate, (size_t)c.n_ff * 4);
+  A((void **)&m->up, (size_t)c.n_ff * 4);
+  A((void **)&m->part_o, (size_t)c.n_head * m->max_splits * c.head_dim * 4);
+  A((void **)&m->part_ml, (size_t)c.n_head * m->max_splits * 2 * 4);
+  A((void **)&m->logits, (size_t)c.n_vocab * 4);
+  A((void **)&m->amax_scratch, 512 * 4);
+  A((void **)&m->amax_out, 4);
+  if (rc != OGM_OK) { llama_free(m); return rc; }
+  // activation scratch for the widest matmul input
+  uint32_t widest = c.n_embd > c.n_ff ? c.n_embd : c.n_ff;
+  if (qd > widest) widest = qd;
+  if ((rc = ensure_act(ctx, widest, 1)) != OGM_OK) { llama_free(m); return rc; }
+
+  std::vector<float> host(((size_t)c.n_layer * 2 + 1) * c.n_embd);
+  for (uint32_t l = 0; l < c.n_layer; l++) {
+    memcpy(&host[((size_t)l * 2) * c.n_embd], layers[l].attn_norm, (size_t)c.n_embd * 4);
+    memcpy(&host[((size_t)l * 2 + 1) * c.n_embd], layers[l].ffn_norm, (size_t)c.n_embd * 4);
+  }
+  memcpy(&host[(size_t)c.n_layer * 2 * c.n_embd], output_norm, (size_t)c.n_embd * 4);
+  // freq_i = base^(-2i / rope_dim), in f32 as tensor.rs:1147 computes it
+  std::vector<float> freq(c.rope_dim / 2 + 1, 0.0f);
+  for (uint32_t i = 0; i < c.rope_dim / 2; i++)
+    freq[i] = powf(c.rope_freq_base, -2.0f * (float)i / (float)c.rope_dim);
+  hipError_t e = hipMemcpy(m->norms, host.data(), host.size() * 4, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
+  if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
+  if (e != hipSuccess) {
+    llama_free(m);
+    return fail(ctx, OGM_ERR_HIP, std::string("ogm_llama_create: ") + hipGetErrorString(e));
+  }
+  *out = m;
+  return OGM_OK;
+}
+
+extern "C" void ogm_llama_destroy(ogm_ctx *ctx, ogm_llama *m) {
+  if (!ctx || !m) return;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->stream);
+  llama_free(m);
+}
+
+extern "C" int ogm_llama_kv_write(ogm_ctx *ctx, ogm_llama *m, uint32_t layer, uint32_t pos0, uint32_t n_pos,
+                                  const float *k, const float *v) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !k || !v) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  const ogm_llama_config &c = m->cfg;
+  if (layer >= c.n_layer || (uint64_t)pos0 + n_pos > c.max_ctx)
+    return fail(ctx, OGM_ERR_INVALID, "layer or position range outside the cache");
+  if (n_pos == 0) return OGM_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  const size_t kvd = (size_t)c.n_head_kv * c.head_dim, n = (size_t)n_pos * kvd;
+  if (m->stage_cap < n * 4) {
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (m->stage) HIPCHK(ctx, hipFree(m->stage));
+    m->stage = nullptr;
+    m->stage_cap = 0;
+    HIPCHK(ctx, hipMalloc((void **)&m->stage, n * 4));
+    m->stage_cap = n * 4;
+  }
+  const size_t row0 = ((size_t)layer * c.max_ctx + pos0) * kvd;
+  const float *src[2] = {k, v};
+  void *dst[2] = {(uint8_t *)m->k_cache + row0 * 2, (uint8_t *)m->v_cache + row0 * 2};
+  for (int i = 0; i < 2; i++) {
+    HIPCHK(ctx, hipMemcpyAsync(m->stage, src[i], n * 4, hipMemcpyHostToDevice, ctx->stream));
+    HIPCHK(ctx, ogm_launch_f32_to_f16(m->stage, dst[i], n, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));  // the host buffer and the staging area are reused
+  }
+  return OGM_OK;
+}
+
+// One matmul group of the step over the activations the previous kernel quantized.
+static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, hipStream_t s) {
+  // weights of one type go out as one launch; a mixed group (Q4_K q/k with a Q6_K v) as several
+  size_t i = 0;
+  while (i < n) {
+    Target tg[OGM_GEMV_MAX_MATS];
+    size_t e = i;
+    while (e < n && e - i < OGM_GEMV_MAX_MATS && ws[e]->ggml_type == ws[i]->ggml_type) {
+      tg[e - i] = Target{ws[e], ys[e]};
+      e++;
+    }
+    int rc = enqueue_gemv(ctx, tg, e - i, 1, 0, s, nullptr, nullptr, nullptr);
+    if (rc != OGM_OK) return rc;
+    i = e;
+  }
+  return OGM_OK;
+}
+
+static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_t pos, float *logits_dev,
+                                uint32_t *argmax_dev, hipStream_t s) {
+  const ogm_llama_config &c = m->cfg;
+  if (pos >= c.max_ctx) return fail(ctx, OGM_ERR_INVALID, "position beyond the KV cache");
+  const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
+  const float scale = 1.0f / sqrtf((float)c.head_dim);
+  HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
+  const float *delta = nullptr;  // what the next norm adds to x first: the last block's output
+  for (uint32_t l = 0; l < c.n_layer; l++) {
+    const ogm_llama_layer &L = m->layers[l];
+    const float *attn_norm = m->norms + (size_t)l * 2 * c.n_embd, *ffn_norm = attn_norm + c.n_embd;
+    void *kc = (uint8_t *)m->k_cache + (size_t)l * c.max_ctx * kvd * 2;
+    void *vc = (uint8_t *)m->v_cache + (size_t)l * c.max_ctx * kvd * 2;
+    // q/k/v read one input; all supported types of a model share an activation mode only if they
+    // are all K-quants or all Q8_0, which create() cannot assume: quantize per consumer mode
+    const int mode_qkv = act_mode_for(L.wq->ggml_type);
+    if (act_mode_for(L.wk->ggml_type) != mode_qkv || act_mode_for(L.wv->ggml_type) != mode_qkv)
+      return fail(ctx, OGM_ERR_UNSUPPORTED, "wq, wk and wv must share an activation mode");
+    HIPCHK(ctx, ogm_launch_norm_quant(mode_qkv, m->x, delta, attn_norm, c.n_embd, c.rms_eps, nullptr,
+                                      act_view(ctx, c.n_embd, mode_qkv, 0), s));
+    const ogm_weight *w3[3] = {L.wq, L.wk, L.wv};
+    float *y3[3] = {m->q, m->k, m->v};
+    int rc = llama_matmul(ctx, w3, y3, 3, s);
+    if (rc != OGM_OK) return rc;
+    HIPCHK(ctx, ogm_launch_rope_kv(m->q, m->k, m->v, m->freq, pos, c.n_head, c.n_head_kv, c.head_dim,
+                                   c.rope_dim, kc, vc, s));
+    const int mode_o = act_mode_for(L.wo->ggml_type);
+    HIPCHK(ctx, ogm_launch_attn_decode(m->q, kc, vc, pos, m->max_splits, c.n_head, c.n_head_kv, c.head_dim,
+                                       scale, m->part_o, m->part_ml, mode_o, nullptr,
+                                       act_view(ctx, qd, mode_o, 0), s));
+    const ogm_weight *w1[1] = {L.wo};
+    float *y1[1] = {m->proj};
+    if ((rc = llama_matmul(ctx, w1, y1, 1, s)) != OGM_OK) return rc;
+    const int mode_ff = act_mode_for(L.w_gate->ggml_type);
+    if (act_mode_for(L.w_up->ggml_type) != mode_ff)
+      return fail(ctx, OGM_ERR_UNSUPPORTED, "w_gate and w_up must share an activation mode");
+    HIPCHK(ctx, ogm_launch_norm_quant(mode_ff, m->x, m->proj, ffn_norm, c.n_embd, c.rms_eps, nullptr,
+                                      act_view(ctx, c.n_embd, mode_ff, 0), s));
+    const ogm_weight *w2[2] = {L.w_gate, L.w_up};
+    float *y2[2] = {m->gate, m->up};
+    if ((rc = llama_matmul(ctx, w2, y2, 2, s)) != OGM_OK) return rc;
+    const int mode_d = act_mode_for(L.w_down->ggml_type);
+    HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr,
+                                        act_view(ctx, c.n_ff, mode_d, 0), s));
+    const ogm_weight *wd[1] = {L.w_down};
+    if ((rc = llama_matmul(ctx, wd, y1, 1, s)) != OGM_OK) return rc;
+    delta = m->proj;
+  }
+  const int mode_out = act_mode_for(m->output->ggml_type);
+  HIPCHK(ctx, ogm_launch_norm_quant(mode_out, m->x, delta, m->norms + (size_t)c.n_layer * 2 * c.n_embd,
+                                    c.n_embd, c.rms_eps, nullptr, act_view(ctx, c.n_embd, mode_out, 0), s));
+  float *lg = logits_dev ? logits_dev : m->logits;
+  const ogm_weight *wo_[1] = {m->output};
+  float *yo[1] = {lg};
+  int rc = llama_matmul(ctx, wo_, yo, 1, s);
+  if (rc != OGM_OK) return rc;
+  if (argmax_dev) HIPCHK(ctx, ogm_launch_argmax(lg, c.n_vocab, m->amax_scratch, argmax_dev, s));
+  // the activation scratch no longer holds what ogm_act_quantize_dev left there
+  ctx->act_mode = -1;
+  return OGM_OK;
+}
+
+extern "C" int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_t pos,
+                                    float *logits_dev, uint32_t *argmax_dev, void *stream) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !x_dev) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  return llama_decode_enqueue(ctx, m, x_dev, pos, logits_dev, argmax_dev, stream ? (hipStream_t)stream : ctx->stream);
+}
+
+extern "C" int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos, float *logits,
+                                uint32_t *argmax) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !x) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  const ogm_llama_config &c = m->cfg;
+  // gate is free until the first FFN: the embedding row is staged there
+  HIPCHK(ctx, hipMemcpyAsync(m->gate, x, (size_t)c.n_embd * 4, hipMemcpyHostToDevice, ctx->stream));
+  int rc = llama_decode_enqueue(ctx, m, m->gate, pos, nullptr, m->amax_out, ctx->stream);
+  if (rc != OGM_OK) return rc;
+  if (logits) HIPCHK(ctx, hipMemcpyAsync(logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (argmax) HIPCHK(ctx, hipMemcpyAsync(argmax, m->amax_out, 4, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return OGM_OK;
+}
+
+extern "C" int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !x_out) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  // the output norm added the last block's output to x in place before normalising
+  HIPCHK(ctx, hipMemcpy(x_out, m->x, (size_t)m->cfg.n_embd * 4, hipMemcpyDeviceToHost));
+  return OGM_OK;
+}

@@ -18,6 +18,7 @@
 
 #include "ogm_kernels.h"
 #include "ogm_layout.h"
+#include "ogm_quant_dev.h"
 
 
 // ------------------------------------------------------------------------------------------
@@ -48,15 +49,6 @@ __device__ __forceinline__ int hi16(uint32_t w) { return ((int)w) >> 16; }
 //   q     = clamp(round_half_away(v * inv), -127, 127), NaN -> 0   (vecdot.rs:117)
 // GROUP = 32: scale per 32 (quantize_act); GROUP = 256: per 256 (quantize_act_k_row).
 
-__device__ __forceinline__ float nan_blind_max(float m, float a) { return a > m ? a : m; }
-
-__device__ __forceinline__ int quantize_one(float v, float inv) {
-  float r = roundf(v * inv);
-  if (r != r) r = 0.0f;
-  r = fminf(fmaxf(r, -127.0f), 127.0f);
-  return (int)r;
-}
-
 template <int GROUP>
 __global__ __launch_bounds__(64) void ogm_quantize_kernel(const float *__restrict__ x,
                                                           uint32_t in_dim, OgmActDev act) {
@@ -66,31 +58,9 @@ __global__ __launch_bounds__(64) void ogm_quantize_kernel(const float *__restric
   const bool active = e0 < in_dim;
   float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
   if (active) v = *(const float4 *)(x + (size_t)t * in_dim + e0);
-
-  float amax = 0.0f;
-  amax = nan_blind_max(amax, fabsf(v.x));
-  amax = nan_blind_max(amax, fabsf(v.y));
-  amax = nan_blind_max(amax, fabsf(v.z));
-  amax = nan_blind_max(amax, fabsf(v.w));
-#pragma unroll
-  for (int m = 1; m < GROUP / 4; m <<= 1) amax = nan_blind_max(amax, __shfl_xor(amax, m, 64));
-
-  const float scale = amax / 127.0f;
-  const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
-  const int q0 = quantize_one(v.x, inv), q1 = quantize_one(v.y, inv);
-  const int q2 = quantize_one(v.z, inv), q3 = quantize_one(v.w, inv);
-  const uint32_t packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) |
-                          ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
-  int s = q0 + q1 + q2 + q3;
-  s += __shfl_xor(s, 1, 64);
-  s += __shfl_xor(s, 2, 64);
-  const int s32 = s + __shfl_xor(s, 4, 64);
-  if (active) {
-    *(uint32_t *)(act.q + (size_t)t * in_dim + e0) = packed;
-    if ((lane & 3u) == 0) act.sums[(size_t)t * (in_dim / 16) + e0 / 16] = s;
-    if ((lane & 7u) == 0) act.bsum[(size_t)t * (in_dim / 32) + e0 / 32] = (int16_t)s32;
-    if ((lane & (GROUP / 4 - 1)) == 0) act.d[(size_t)t * (in_dim / GROUP) + e0 / GROUP] = scale;
-  }
+  ogm_quantize_store<GROUP>(v, e0, active, lane, act.q + (size_t)t * in_dim,
+                            act.d + (size_t)t * (in_dim / GROUP), act.sums + (size_t)t * (in_dim / 16),
+                            act.bsum + (size_t)t * (in_dim / 32));
 }
 
 hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,
@@ -395,23 +365,9 @@ static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rb_per
 template <class F>
 __device__ __forceinline__ void quantize_park(const float4 &v, uint32_t g, bool active, uint32_t lane,
                                               uint32_t upr, uint4 *l_xq, uint4 *l_aux, float *l_d) {
-  float amax = 0.0f;
-  amax = nan_blind_max(amax, fabsf(v.x));
-  amax = nan_blind_max(amax, fabsf(v.y));
-  amax = nan_blind_max(amax, fabsf(v.z));
-  amax = nan_blind_max(amax, fabsf(v.w));
-#pragma unroll
-  for (int m = 1; m < F::ACT_GROUP / 4; m <<= 1) amax = nan_blind_max(amax, __shfl_xor(amax, m, 64));
-  const float scale = amax / 127.0f;
-  const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
-  const int q0 = quantize_one(v.x, inv), q1 = quantize_one(v.y, inv);
-  const int q2 = quantize_one(v.z, inv), q3 = quantize_one(v.w, inv);
-  const uint32_t packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) |
-                          ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
-  int s = q0 + q1 + q2 + q3;
-  s += __shfl_xor(s, 1, 64);
-  s += __shfl_xor(s, 2, 64);                    // sum of 16
-  const int s32 = s + __shfl_xor(s, 4, 64);     // sum of 32
+  float scale;
+  int s, s32;
+  const uint32_t packed = ogm_quantize4<F::ACT_GROUP>(v, scale, s, s32);
   if (!active) return;
   const uint32_t ch = g * 16u + (lane >> 2);    // 16-byte chunk of the token
   const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;

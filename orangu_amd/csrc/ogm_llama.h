@@ -1,0 +1,47 @@
+// Launchers of the decode-step kernels around the quantized matmuls (ogm_llama.hip): what a
+// Llama-family layer does between two matmuls at one token (engine/arch/llama.rs:594-932 of
+// orangu-server), with the activation quantizer of the next matmul fused into each producer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ogm_kernels.h"
+
+#define OGM_ATTN_CHUNK 128u   // cache positions per workgroup of the attention kernel
+
+// x += delta (when delta is given; x is updated in place), then
+// normed = x * (1 / sqrt(mean(x^2) + eps)) * weight        (tensor.rs:732-757)
+// quantized for the next matmul in `mode` (0: per 32, 1: per 256) into `act`; `normed` (f32) is
+// also stored when not null.  n <= 16384, n % 32 == 0.
+hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const float *weight, uint32_t n,
+                                 float eps, float *normed, OgmActDev act, hipStream_t stream);
+
+// NORM-paired RoPE (pairs 2i, 2i+1; tensor.rs:1115-1177 with freq_scale 1 and no YaRN) of q
+// (in place) and k at position `pos`, then k and v into the f16 cache rows of that position.
+// `freq` holds rope_dim / 2 frequencies.
+hipError_t ogm_launch_rope_kv(float *q, const float *k, const float *v, const float *freq, uint32_t pos,
+                              uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim, uint32_t rope_dim,
+                              void *k_cache_layer, void *v_cache_layer, hipStream_t stream);
+
+// Causal attention of one token over cache positions 0..pos (engine/attention.rs:426-549):
+// scores = (q . k) * scale, softmax over positions, out = sum w * v; grouped-query heads share
+// their K/V head.  Split over chunks of OGM_ATTN_CHUNK positions and combined; the combined
+// output is quantized for the next matmul in `mode` and stored as f32 when attn_out is not null.
+// part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch.
+hipError_t ogm_launch_attn_decode(const float *q, const void *k_cache_layer, const void *v_cache_layer,
+                                  uint32_t pos, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
+                                  uint32_t head_dim, float scale, float *part_o, float *part_ml, int mode,
+                                  float *attn_out, OgmActDev act, hipStream_t stream);
+
+// h = silu(gate) * up with silu(g) = g / (1 + exp(-g))     (tensor.rs:825-827, arch/mod.rs:1071-1106)
+// quantized for the down projection in `mode`; h (f32) is also stored when not null.
+hipError_t ogm_launch_swiglu_quant(int mode, const float *gate, const float *up, uint32_t n, float *h,
+                                   OgmActDev act, hipStream_t stream);
+
+// Index of the largest logit; of several equal ones the last (sampling.rs:336-343).  `scratch`
+// holds 2 * 256 words.
+hipError_t ogm_launch_argmax(const float *logits, uint32_t n, uint32_t *scratch, uint32_t *out,
+                             hipStream_t stream);
+
+// f32 -> f16 (round to nearest even) for cache rows handed over by the host.
+hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStream_t stream);

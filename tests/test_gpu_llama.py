@@ -1,0 +1,128 @@
+"""GPU parity of the decode step (ogm_llama_*, through the C ABI) against the CPU restatement
+oracle/llama_ref.py on the same seeded model.  The matmuls inside are bit-exact (tested in
+test_gpu_parity.py); the element-wise kernels use tree reductions and the device's exp / sin /
+cos, so the bar here is a tolerance: hidden state and logits within 2e-4 of the largest magnitude
+(stated in `close`), greedy token equal unless the CPU's top two logits are within that tolerance."""
+import sys
+
+import numpy as np
+import pytest
+
+from helpers import Q4_K, Q6_K, Q8_0, synth_weights
+from oracle import llama_ref as R
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+TOL = 2e-4
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def be():
+    from orangu_amd import Mi355xBackend
+    b = Mi355xBackend()
+    yield b
+    b.close()
+
+
+def close(got, want, what):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    scale = np.abs(want).max() + 1e-30
+    err = np.abs(got - want).max() / scale
+    assert np.isfinite(got).all(), what
+    assert err <= TOL, f"{what}: max error {err:.3e} of the largest magnitude {scale:.3e}"
+    return err
+
+
+def build(be, *, n_embd, n_head, n_kv, hd, n_ff, n_vocab, n_layer, types, max_ctx, seed, rope_dim=None,
+          base=10000.0):
+    from orangu_amd import LlamaDecoder, QuantMatrix
+    rng = np.random.default_rng(seed)
+    tq, tv, tdown, tout = types
+    mk = lambda t, i, o, s: (t, synth_weights(t, i, o, seed=s), i, o)
+    layers = []
+    for l in range(n_layer):
+        s = seed * 1000 + 10 * l
+        layers.append(R.Layer(mk(tq, n_embd, n_head * hd, s + 1), mk(tq, n_embd, n_kv * hd, s + 2),
+                              mk(tv, n_embd, n_kv * hd, s + 3), mk(tq, n_head * hd, n_embd, s + 4),
+                              mk(tq, n_embd, n_ff, s + 5), mk(tq, n_embd, n_ff, s + 6),
+                              mk(tdown, n_ff, n_embd, s + 7),
+                              (1 + 0.1 * rng.standard_normal(n_embd)).astype(f32),
+                              (1 + 0.1 * rng.standard_normal(n_embd)).astype(f32)))
+    out_norm = (1 + 0.1 * rng.standard_normal(n_embd)).astype(f32)
+    output = mk(tout, n_embd, n_vocab, seed * 1000 + 999)
+    ref = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd if rope_dim is None else rope_dim, 1e-5, base,
+                  layers, out_norm, output)
+    ref.reset()
+    qm = lambda w: QuantMatrix(np.ascontiguousarray(w[1]), w[0], w[2], w[3])
+    dev = LlamaDecoder(be, n_embd=n_embd, n_head=n_head, n_head_kv=n_kv, head_dim=hd, n_ff=n_ff,
+                       n_vocab=n_vocab, max_ctx=max_ctx, rope_dim=rope_dim, rms_eps=1e-5, rope_freq_base=base,
+                       layers=[{k: (qm(getattr(L, k)) if k.startswith("w") else getattr(L, k))
+                                for k in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down", "attn_norm", "ffn_norm")}
+                               for L in layers],
+                       output_norm=out_norm, output=qm(output))
+    return ref, dev, rng
+
+
+def step_both(ref, dev, x, pos, what):
+    want_logits, want_hidden = R.decode_step(ref, x, pos)
+    got_logits, got_tok = dev.decode(x, pos)
+    e1 = close(dev.hidden(), want_hidden, f"{what}: hidden state")
+    e2 = close(got_logits, want_logits, f"{what}: logits")
+    top = np.sort(want_logits)[-2:]
+    if top[1] - top[0] > TOL * np.abs(want_logits).max():
+        assert got_tok == R.argmax(want_logits), f"{what}: greedy token"
+    assert got_tok == R.argmax(got_logits), f"{what}: device argmax of its own logits"
+    say(what, "hidden err %.2e logits err %.2e token %d" % (e1, e2, got_tok))
+
+
+@pytest.mark.parametrize("types", [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q4_K, Q4_K, Q4_K, Q4_K)])
+def test_decode_steps_from_an_empty_cache(be, types):
+    """Positions 0..5 one after the other: RMSNorm, q/k/v, RoPE, cache append, attention over the
+    growing cache, wo, residual, SwiGLU FFN, output norm and vocabulary projection."""
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
+                          types=types, max_ctx=16, seed=5)
+    try:
+        for pos in range(6):
+            step_both(ref, dev, rng.standard_normal(256).astype(f32), pos, f"types {types} pos {pos}")
+    finally:
+        dev.close()
+
+
+def test_decode_over_a_prefilled_cache_with_several_attention_chunks(be):
+    """head_dim 128, four query heads per K/V head, 300 cached positions handed over from the host
+    (three attention chunks, the last one partial), partial rotary dimension."""
+    n_kv, hd = 2, 128
+    ref, dev, rng = build(be, n_embd=1024, n_head=8, n_kv=n_kv, hd=hd, n_ff=2816, n_vocab=1000, n_layer=3,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=512, seed=6, rope_dim=64, base=500000.0)
+    try:
+        n_pre = 300
+        for l in range(3):
+            k = rng.standard_normal((n_pre, n_kv * hd)).astype(f32)
+            v = rng.standard_normal((n_pre, n_kv * hd)).astype(f32)
+            dev.kv_write(l, 0, k, v)
+            ref.k_cache[l] = [r.astype(np.float16) for r in k]
+            ref.v_cache[l] = [r.astype(np.float16) for r in v]
+        for pos in (300, 301, 302):
+            step_both(ref, dev, rng.standard_normal(1024).astype(f32), pos, f"prefilled pos {pos}")
+    finally:
+        dev.close()
+
+
+def test_decode_rejects_bad_arguments(be):
+    from orangu_amd import OgmError
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=1,
+                          types=(Q4_K, Q4_K, Q4_K, Q4_K), max_ctx=4, seed=7)
+    try:
+        with pytest.raises(OgmError):
+            dev.decode(np.zeros(256, f32), 4)          # beyond the cache
+        with pytest.raises(ValueError):
+            dev.decode(np.zeros(100, f32), 0)
+        with pytest.raises(OgmError):
+            dev.kv_write(0, 3, np.zeros((2, 128), f32), np.zeros((2, 128), f32))
+    finally:
+        dev.close()

@@ -1,0 +1,135 @@
+"""Pins the CPU restatement of the decode step's element-wise functions (oracle/llama_ref.py)
+against the values the reference's own tests hold and against closed forms."""
+import math
+
+import numpy as np
+import pytest
+
+from oracle import llama_ref as R
+
+f32 = np.float32
+
+
+def test_rmsnorm_reference_case_and_closed_forms():
+    # tensor.rs:1450-1466: rows [3, 4] and [0, 0], weight ones, eps 1e-5
+    eps = 1e-5
+    rms = math.sqrt(12.5 + eps)
+    got = R.rmsnorm(np.array([3.0, 4.0], f32), np.ones(2, f32), eps)
+    assert abs(got[0] - 3.0 / rms) < 1e-6 and abs(got[1] - 4.0 / rms) < 1e-6
+    assert np.array_equal(R.rmsnorm(np.zeros(2, f32), np.ones(2, f32), eps), np.zeros(2, f32))
+    # a constant row c: out_i = c / sqrt(c^2 + eps) * w_i
+    w = np.linspace(0.5, 1.5, 64).astype(f32)
+    got = R.rmsnorm(np.full(64, 2.5, f32), w, 1e-6)
+    np.testing.assert_allclose(got, 2.5 / math.sqrt(6.25 + 1e-6) * w, rtol=2e-7)
+    # the weight multiplies after the scale: (v * scale) * w, and a sign flip of x flips the output
+    x = np.random.default_rng(1).standard_normal(256).astype(f32)
+    np.testing.assert_array_equal(R.rmsnorm(-x, w.repeat(4), 1e-5), -R.rmsnorm(x, w.repeat(4), 1e-5))
+    ref = x.astype(np.float64) / np.sqrt(np.mean(x.astype(np.float64) ** 2) + 1e-5) * w.repeat(4)
+    np.testing.assert_allclose(R.rmsnorm(x, w.repeat(4), 1e-5), ref, rtol=1e-6)
+
+
+def test_rope_reference_case_and_invariants():
+    # tensor.rs:1752-1769: [1..8], one head of 8, position 3, base 10000, NORM pairs
+    x = np.arange(1, 9, dtype=f32)
+    want = x.astype(np.float64).copy()
+    for p in range(4):
+        theta = 3.0 * float(f32(10000.0) ** f32(-2.0 * p / 8.0))
+        a, b = want[2 * p], want[2 * p + 1]
+        want[2 * p], want[2 * p + 1] = a * math.cos(theta) - b * math.sin(theta), a * math.sin(theta) + b * math.cos(theta)
+    np.testing.assert_allclose(R.rope_norm(x, 1, 8, 3, 8, 10000.0), want, atol=1e-6)
+    # position 0 is the identity (tensor.rs:1668); pair norms are preserved (:1676)
+    y = np.random.default_rng(2).standard_normal(4 * 16).astype(f32)
+    np.testing.assert_array_equal(R.rope_norm(y, 4, 16, 0, 16, 500000.0), y)
+    r = R.rope_norm(y, 4, 16, 77, 16, 500000.0).reshape(-1, 2)
+    np.testing.assert_allclose((r ** 2).sum(1), (y.reshape(-1, 2) ** 2).sum(1), rtol=1e-6)
+    # pair 0 has frequency 1: (1, 0) at position p becomes (cos p, sin p)
+    e = np.zeros(8, f32)
+    e[0] = 1.0
+    r = R.rope_norm(e, 1, 8, 2, 8, 10000.0)
+    assert abs(r[0] - math.cos(2.0)) < 1e-6 and abs(r[1] - math.sin(2.0)) < 1e-6
+    # dimensions past rope_dim are left alone; every head gets the same rotation
+    r = R.rope_norm(y, 4, 16, 5, 8, 10000.0).reshape(4, 16)
+    np.testing.assert_array_equal(r[:, 8:], y.reshape(4, 16)[:, 8:])
+    one = R.rope_norm(y.reshape(4, 16)[2], 1, 16, 5, 8, 10000.0)
+    np.testing.assert_array_equal(r[2], one)
+    # rotations compose: position a then position b equals position a + b (to rounding)
+    ab = R.rope_norm(R.rope_norm(y, 4, 16, 3, 16, 10000.0), 4, 16, 4, 16, 10000.0)
+    np.testing.assert_allclose(ab, R.rope_norm(y, 4, 16, 7, 16, 10000.0), atol=2e-6)
+
+
+def test_softmax_silu_argmax():
+    s = R.softmax(np.array([1.0, 2.0, 3.0], f32))           # tensor.rs:1612-1619
+    assert abs(float(s.sum()) - 1.0) < 1e-6 and s[0] < s[1] < s[2]
+    np.testing.assert_allclose(s, np.exp([-2.0, -1.0, 0.0]) / np.exp([-2.0, -1.0, 0.0]).sum(), rtol=1e-6)
+    assert abs(float(R.silu(f32(0.0)))) < 1e-6                 # tensor.rs:1621-1625
+    assert abs(float(R.silu(f32(1.0))) - 0.7310586) < 1e-6
+    assert abs(float(R.silu(f32(-1.0))) + 0.26894143) < 1e-6
+    assert R.argmax(np.array([1.0, 5.0, 2.0, 5.0, 0.0], f32)) == 3   # last of equal maxima
+    assert R.argmax(np.array([-3.0], f32)) == 0
+
+
+def test_attention_closed_forms_and_head_mapping():
+    rng = np.random.default_rng(3)
+    n_head, n_kv, hd = 4, 2, 8
+    q = rng.standard_normal(n_head * hd).astype(f32)
+    # a single cached position: out_h = v[kv head of h]
+    k1, v1 = rng.standard_normal((1, n_kv * hd)).astype(f32), rng.standard_normal((1, n_kv * hd)).astype(f32)
+    out = R.attention(q, k1, v1, n_head, n_kv, hd).reshape(n_head, hd)
+    for h in range(n_head):
+        np.testing.assert_allclose(out[h], v1.reshape(n_kv, hd)[h // 2], rtol=1e-6)
+    # equal scores (all keys the same): the mean of the values
+    k = np.tile(k1, (5, 1))
+    v = rng.standard_normal((5, n_kv * hd)).astype(f32)
+    out = R.attention(q, k, v, n_head, n_kv, hd).reshape(n_head, hd)
+    for h in range(n_head):
+        np.testing.assert_allclose(out[h], v.reshape(5, n_kv, hd)[:, h // 2].mean(0), rtol=1e-5, atol=1e-6)
+    # brute force in float64 with the explicit head mapping
+    k = rng.standard_normal((9, n_kv * hd)).astype(f32)
+    v = rng.standard_normal((9, n_kv * hd)).astype(f32)
+    out = R.attention(q, k, v, n_head, n_kv, hd).reshape(n_head, hd)
+    for h in range(n_head):
+        kh, vh = k.reshape(9, n_kv, hd)[:, h // 2].astype(np.float64), v.reshape(9, n_kv, hd)[:, h // 2].astype(np.float64)
+        sc = kh @ q.reshape(n_head, hd)[h].astype(np.float64) / math.sqrt(hd)
+        w = np.exp(sc - sc.max())
+        w /= w.sum()
+        np.testing.assert_allclose(out[h], w @ vh, rtol=1e-5, atol=1e-6)
+    # one overwhelming key: its value wins
+    k[4] = 50.0 * np.tile(q.reshape(n_head, hd)[:: 2].reshape(-1) / np.linalg.norm(q), 1)[: n_kv * hd]
+    out = R.attention(q, k, v, n_head, n_kv, hd).reshape(n_head, hd)
+    np.testing.assert_allclose(out[0], v.reshape(9, n_kv, hd)[4, 0], atol=1e-3)
+
+
+def test_decode_step_wiring_on_a_tiny_model():
+    """Two layers by hand: the residual stream, the cache growth and the f16 cache rounding."""
+    from helpers import Q4_K, Q6_K, synth_weights
+    rng = np.random.default_rng(4)
+    n_embd, n_head, n_kv, hd, n_ff, n_vocab = 256, 4, 2, 64, 512, 320
+    mk = lambda t, i, o, s: (t, synth_weights(t, i, o, seed=s), i, o)
+    layers = [R.Layer(mk(Q4_K, n_embd, n_head * hd, 1 + 10 * l), mk(Q4_K, n_embd, n_kv * hd, 2 + 10 * l),
+                      mk(Q6_K, n_embd, n_kv * hd, 3 + 10 * l), mk(Q4_K, n_head * hd, n_embd, 4 + 10 * l),
+                      mk(Q4_K, n_embd, n_ff, 5 + 10 * l), mk(Q4_K, n_embd, n_ff, 6 + 10 * l),
+                      mk(Q6_K, n_ff, n_embd, 7 + 10 * l),
+                      (1 + 0.1 * rng.standard_normal(n_embd)).astype(f32),
+                      (1 + 0.1 * rng.standard_normal(n_embd)).astype(f32)) for l in range(2)]
+    m = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 10000.0, layers,
+                np.ones(n_embd, f32), mk(Q6_K, n_embd, n_vocab, 99))
+    x0, x1 = rng.standard_normal(n_embd).astype(f32), rng.standard_normal(n_embd).astype(f32)
+    lg0, h0 = R.decode_step(m, x0, 0)
+    lg1, h1 = R.decode_step(m, x1, 1)
+    assert lg0.shape == (n_vocab,) and h1.shape == (n_embd,) and np.isfinite(lg1).all()
+    assert [len(c) for c in m.k_cache] == [2, 2] and m.k_cache[0][0].dtype == np.float16
+    # at position 0 attention returns the (f16-rounded) value row itself: rebuild layer 0 by hand
+    L = layers[0]
+    normed = R.rmsnorm(x0, L.attn_norm, 1e-5)
+    v = R._mm(L.wv, normed).astype(np.float16).astype(f32)
+    attn = np.repeat(v.reshape(n_kv, hd), n_head // n_kv, axis=0).reshape(-1)
+    x = x0 + R._mm(L.wo, attn)
+    n2 = R.rmsnorm(x, L.ffn_norm, 1e-5)
+    x = x + R._mm(L.w_down, R.silu(R._mm(L.w_gate, n2)) * R._mm(L.w_up, n2))
+    m1 = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 10000.0, layers[:1],
+                 np.ones(n_embd, f32), m.output)
+    _, h = R.decode_step(m1, x0, 0)
+    np.testing.assert_allclose(h, x, rtol=1e-5, atol=1e-6)
+    # a decode out of order is refused
+    with pytest.raises(AssertionError):
+        R.decode_step(m, x0, 5)
