@@ -90,6 +90,102 @@ def sweep(be, helpers, hiprt) -> dict:
     return out
 
 
+def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool) -> dict:
+    """Batch-1 decode of an 8B-shaped Llama (32 layers: wq, wo 4096x4096, wk, wv 4096->1024, gate, up
+    4096->14336 in Q4_K; down 14336->4096 and the 128256-row output in Q6_K; f16 KV cache holding `ctx`
+    random positions): tokens per second of ogm_llama_decode_dev with the embedding row, the logits and
+    the greedy token resident in HBM.  Every layer has its own device copy of the weights."""
+    from orangu_amd import LlamaDecoder, QuantMatrix
+    Q6_K = 14
+    n_layer, n_embd, n_head, n_kv, hd, n_ff, n_vocab = 32, 4096, 32, 8, 128, 14336, 128256
+    seed = 515
+    rng = np.random.default_rng(seed)
+    shapes = {"wq": (Q4_K, n_embd, n_embd), "wk": (Q4_K, n_embd, n_kv * hd), "wv": (Q4_K, n_embd, n_kv * hd),
+              "wo": (Q4_K, n_embd, n_embd), "w_gate": (Q4_K, n_embd, n_ff), "w_up": (Q4_K, n_embd, n_ff),
+              "w_down": (Q6_K, n_ff, n_embd)}
+    # two distinct byte patterns per matrix kind, alternating over layers; one device copy per layer
+    raws = {k: [helpers.synth_weights(t, i, o, seed + 17 * n + j) for j in range(2)]
+            for n, (k, (t, i, o)) in enumerate(shapes.items())}
+    out_raw = helpers.synth_weights(Q6_K, n_embd, n_vocab, seed + 999)
+    norms = [(1 + 0.05 * rng.standard_normal(n_embd)).astype(np.float32) for _ in range(2 * n_layer + 1)]
+    mats = {}
+
+    def up(key):  # key = (kind, layer) or "output"
+        if key not in mats:
+            if key == "output":
+                mats[key] = be.upload_raw(out_raw, Q6_K, n_embd, n_vocab)
+            else:
+                t, i, o = shapes[key[0]]
+                mats[key] = be.upload_raw(raws[key[0]][key[1] % 2], t, i, o)
+        return mats[key]
+
+    layers = [{**{k: (k, l) for k in shapes}, "attn_norm": norms[2 * l], "ffn_norm": norms[2 * l + 1]}
+              for l in range(n_layer)]
+    dec = LlamaDecoder(be, n_embd=n_embd, n_head=n_head, n_head_kv=n_kv, head_dim=hd, n_ff=n_ff, n_vocab=n_vocab,
+                       max_ctx=ctx + warmup + steps + 2, rms_eps=1e-5, rope_freq_base=500000.0, layers=layers,
+                       output_norm=norms[-1], output="output", upload=up)
+    kvs = []
+    for l in range(n_layer):
+        k = rng.standard_normal((ctx, n_kv * hd)).astype(np.float32)
+        v = rng.standard_normal((ctx, n_kv * hd)).astype(np.float32)
+        dec.kv_write(l, 0, k, v)
+        if check and l < 2:
+            kvs.append((k, v))
+    x_h = rng.standard_normal(n_embd).astype(np.float32)
+    x_d = hiprt.DeviceBuffer.from_numpy(x_h)
+    tok_d = hiprt.DeviceBuffer(4)
+    stream = hiprt.Stream()
+    pos = ctx
+    for _ in range(warmup):
+        dec.decode_dev(x_d.ptr, pos, 0, tok_d.ptr, stream.ptr)
+        pos += 1
+    stream.synchronize()
+    hiprt.device_synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        dec.decode_dev(x_d.ptr, pos, 0, tok_d.ptr, stream.ptr)
+        pos += 1
+    stream.synchronize()
+    hiprt.device_synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    weights = n_layer * sum(o * (i // 256) * (144 if t == Q4_K else 210) for t, i, o in shapes.values()) \
+        + n_vocab * (n_embd // 256) * 210
+    kv_bytes = 2 * n_layer * ctx * n_kv * hd * 2
+    res = {"workload": f"configs[4]: 8B-shaped Llama Q4_K_M-like, batch-1 greedy decode at context {ctx}",
+           "tok_per_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4),
+           "bytes_per_token": weights + kv_bytes,
+           "GBps": round((weights + kv_bytes) / dt / 1e9, 1),
+           "frac_of_hbm_peak": round((weights + kv_bytes) / dt / 1e9 / HBM_PEAK_GBS, 4)}
+    if check:
+        # the same two-layer prefix of the model on the CPU restatement, same cache rows, one token
+        from oracle import llama_ref as R
+        small = LlamaDecoder(be, n_embd=n_embd, n_head=n_head, n_head_kv=n_kv, head_dim=hd, n_ff=n_ff,
+                             n_vocab=n_vocab, max_ctx=ctx + 1, rms_eps=1e-5, rope_freq_base=500000.0,
+                             layers=layers[:2], output_norm=norms[-1], output="output", upload=up)
+        ref_layers = []
+        for l in range(2):
+            w = {k: (shapes[k][0], raws[k][l % 2], shapes[k][1], shapes[k][2]) for k in shapes}
+            ref_layers.append(R.Layer(w["wq"], w["wk"], w["wv"], w["wo"], w["w_gate"], w["w_up"], w["w_down"],
+                                      norms[2 * l], norms[2 * l + 1]))
+        ref = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 500000.0, ref_layers, norms[-1],
+                      (Q6_K, out_raw, n_embd, n_vocab))
+        ref.reset()
+        for l, (k, v) in enumerate(kvs):
+            small.kv_write(l, 0, k, v)
+            ref.k_cache[l] = list(k.astype(np.float16))
+            ref.v_cache[l] = list(v.astype(np.float16))
+        want, _ = R.decode_step(ref, x_h, ctx)
+        got, tok = small.decode(x_h, ctx)
+        err = float(np.abs(got.astype(np.float64) - want).max() / (np.abs(want).max() + 1e-30))
+        res["parity_vs_cpu"] = {"layers_checked": 2, "max_logit_error_over_max_logit": err,
+                                "greedy_token_equal": bool(tok == R.argmax(want)), "ok": bool(err <= 2e-4)}
+        small.close()
+    dec.close()
+    for h in mats.values():
+        be.free_weight(h)
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -108,6 +204,10 @@ def main() -> int:
     ap.add_argument("--gemm-tokens", type=int, default=512,
                     help="tokens of the prefill GEMM leg (Q4_K 4096 -> 14336 on MFMA); 0 skips it")
     ap.add_argument("--only-gemm", action="store_true", help="run only the prefill GEMM leg (for rocprofv3)")
+    ap.add_argument("--decode-steps", type=int, default=64,
+                    help="tokens of the 8B-shaped decode leg (config 5); 0 skips it")
+    ap.add_argument("--decode-ctx", type=int, default=2048, help="cached positions of the decode leg")
+    ap.add_argument("--only-decode", action="store_true", help="run only the decode leg (for rocprofv3)")
     ap.add_argument("--sweep", action="store_true",
                     help="time every benchmark configuration's kernels instead (one JSON object, not the "
                          "headline line)")
@@ -127,6 +227,10 @@ def main() -> int:
     be = Mi355xBackend()  # raises without the HIP library or a gfx950 device
     if args.sweep:
         print(json.dumps(sweep(be, helpers, hiprt)))
+        be.close()
+        return 0
+    if args.only_decode:
+        print(json.dumps(decode_leg(be, helpers, hiprt, max(1, args.decode_steps), 8, args.decode_ctx, False)))
         be.close()
         return 0
     if args.wg_waves:
@@ -302,6 +406,13 @@ def main() -> int:
         if parity == "FAILED":
             print("bench.py: GPU output differs from the CPU oracle beyond 1e-3/1e-5", file=sys.stderr)
 
+    decode = None
+    if args.decode_steps > 0 and not args.only_roofline and not args.only_gemm:
+        for k in handles:          # make room: the decode leg brings its own 4.8 GB of weights
+            for h in handles[k]:
+                be.free_weight(h)
+        decode = decode_leg(be, helpers, hiprt, args.decode_steps, 8, args.decode_ctx, args.cpu_seconds > 0)
+
     out = {
         "metric": "Q4_K GEMV HBM GB/s (batch-1 decode, Llama-3-8B FFN shapes)",
         "value": round(result.get("value", achieved), 1),
@@ -324,6 +435,7 @@ def main() -> int:
         "roofline": roofline,
         "cpu_baseline": cpu,
         "prefill_gemm": gemm,
+        "decode": decode,
     }
     print(json.dumps(out))
     be.close()

@@ -767,8 +767,9 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   const ogm_llama_config c = *cfg;
   if (c.n_layer == 0 || c.n_embd == 0 || c.n_head == 0 || c.n_head_kv == 0 || c.n_ff == 0 || c.max_ctx == 0)
     return fail(ctx, OGM_ERR_INVALID, "empty model dimension");
-  if (c.n_head % c.n_head_kv != 0 || c.n_head / c.n_head_kv > 8)
-    return fail(ctx, OGM_ERR_UNSUPPORTED, "query heads per K/V head must divide evenly and be at most 8");
+  const uint32_t gq = c.n_head % c.n_head_kv == 0 ? c.n_head / c.n_head_kv : 0;
+  if (gq != 1 && gq != 2 && gq != 4 && gq != 8)
+    return fail(ctx, OGM_ERR_UNSUPPORTED, "query heads per K/V head must be 1, 2, 4 or 8");
   if (c.head_dim != 64 && c.head_dim != 128) return fail(ctx, OGM_ERR_UNSUPPORTED, "head_dim must be 64 or 128");
   if (c.rope_dim > c.head_dim || c.rope_dim % 2 != 0) return fail(ctx, OGM_ERR_INVALID, "bad rope_dim");
   if (c.n_embd > 16384 || c.n_embd % 32 != 0 || c.n_ff % 32 != 0)

@@ -134,24 +134,27 @@ hipError_t ogm_launch_rope_kv(float *q, const float *k, const float *v, const fl
 // ------------------------------------------------------------------------------------------
 // attention: partial softmax per chunk of positions, then combine (+ quantize)
 
-#define ATT_MAXG 8   // query heads per K/V head
 
-// Workgroup (kvh, split): the query heads of K/V head kvh against positions
-// split * 128 .. + 128.  Phase 1: thread t scores position t for every query head (its K row
-// from HBM, q uniform).  Phase 2: thread t owns output dimension t and walks the positions.
-template <int HD>
+// Workgroup (kvh, split): the G query heads of K/V head kvh against positions
+// split * 128 .. + 128.  Every load of the workgroup is requested first (its K rows and its V
+// rows in one trip to memory).  Phase 1: thread t scores position t for every query head; q is
+// uniform (scalar loads).  Phase 2: sixteen threads share a V row (eight dimensions each), eight
+// rows per step, and LDS adds the eight partial sums.
+template <int HD, int G>
 __global__ __launch_bounds__(128) void ogm_attn_partial_kernel(const float *__restrict__ q,
                                                                const __half *__restrict__ kc,
                                                                const __half *__restrict__ vc, uint32_t pos,
-                                                               uint32_t max_splits, uint32_t n_head,
-                                                               uint32_t n_head_kv, float scale,
-                                                               float *__restrict__ part_o,
+                                                               uint32_t max_splits, uint32_t n_head_kv,
+                                                               float scale, float *__restrict__ part_o,
                                                                float *__restrict__ part_ml) {
-  __shared__ float sc[ATT_MAXG][OGM_ATTN_CHUNK];
-  __shared__ float red[ATT_MAXG][2];
+  constexpr int TPR = HD / 8;            // threads per V row
+  constexpr int ROWS = 128 / TPR;        // V rows in flight per step
+  constexpr int STEPS = OGM_ATTN_CHUNK / ROWS;
+  __shared__ float sc[G][OGM_ATTN_CHUNK];
+  __shared__ float red[2][G][2];
+  __shared__ float osum[ROWS][G][HD];
   const uint32_t kvh = blockIdx.x, split = blockIdx.y;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const uint32_t G = n_head / n_head_kv;
   const uint32_t kv_dim = n_head_kv * HD;
   const uint32_t n_pos = pos + 1u;
   const uint32_t p0 = split * OGM_ATTN_CHUNK;
@@ -159,17 +162,27 @@ __global__ __launch_bounds__(128) void ogm_attn_partial_kernel(const float *__re
   const uint32_t n_here = min(OGM_ATTN_CHUNK, n_pos - p0);
   const bool valid = tid < n_here;
 
-  // ---- phase 1: scores
-  float acc[ATT_MAXG];
+  const uint32_t rr = tid / TPR, dc = tid - rr * TPR;   // phase 2: row slot and 8-dimension chunk
+  // rows past the chunk's end read the last valid row; their scores are discarded (weight 0)
+  const __half *krow = kc + (size_t)(p0 + min(tid, n_here - 1u)) * kv_dim + kvh * HD;
+  uint4 kr[HD / 8];
 #pragma unroll
-  for (int g = 0; g < ATT_MAXG; g++) acc[g] = 0.0f;
-  if (valid) {
-    const __half *krow = kc + (size_t)(p0 + tid) * kv_dim + kvh * HD;
+  for (int c = 0; c < HD / 8; c++) kr[c] = *(const uint4 *)(krow + 8 * c);
+  const __half *vbase = vc + (size_t)p0 * kv_dim + kvh * HD + 8u * dc;
+  uint4 vr[STEPS];
+#pragma unroll
+  for (int st = 0; st < STEPS; st++)
+    vr[st] = *(const uint4 *)(vbase + (size_t)min((uint32_t)(st * ROWS) + rr, n_here - 1u) * kv_dim);
+
+  // ---- phase 1: scores
+  float acc[G];
+#pragma unroll
+  for (int g = 0; g < G; g++) acc[g] = 0.0f;
+  {
     const float *qb = q + (size_t)kvh * G * HD;
-#pragma unroll 2
-    for (int d = 0; d < HD; d += 8) {
-      const uint4 raw = *(const uint4 *)(krow + d);
-      const __half2 *h2 = (const __half2 *)&raw;
+#pragma unroll
+    for (int c = 0; c < HD / 8; c++) {
+      const __half2 *h2 = (const __half2 *)&kr[c];
       float kf[8];
 #pragma unroll
       for (int j = 0; j < 4; j++) {
@@ -178,121 +191,164 @@ __global__ __launch_bounds__(128) void ogm_attn_partial_kernel(const float *__re
         kf[2 * j + 1] = f.y;
       }
 #pragma unroll
-      for (int g = 0; g < ATT_MAXG; g++) {
-        if ((uint32_t)g < G) {
+      for (int g = 0; g < G; g++)
 #pragma unroll
-          for (int j = 0; j < 8; j++) acc[g] += qb[g * HD + d + j] * kf[j];
-        }
-      }
+        for (int j = 0; j < 8; j++) acc[g] = fmaf(qb[g * HD + 8 * c + j], kf[j], acc[g]);
     }
   }
-  // block max and sum per query head
+  // workgroup maximum and sum per query head: two barriers for all heads
+  float sv[G], mv[G];
 #pragma unroll
-  for (int g = 0; g < ATT_MAXG; g++) {
-    if ((uint32_t)g >= G) break;
-    const float s = valid ? acc[g] * scale : -INFINITY;
-    float m = s;
+  for (int g = 0; g < G; g++) {
+    sv[g] = valid ? acc[g] * scale : -INFINITY;
+    float m = sv[g];
 #pragma unroll
     for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
-    if (lane == 0) red[g][wave] = m;
-    __syncthreads();
-    m = fmaxf(red[g][0], red[g][1]);
-    __syncthreads();
-    const float e = valid ? expf(s - m) : 0.0f;
+    if (lane == 0) red[0][g][wave] = m;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < G; g++) {
+    mv[g] = fmaxf(red[0][g][0], red[0][g][1]);
+    const float e = valid ? expf(sv[g] - mv[g]) : 0.0f;
     sc[g][tid] = e;
     float l = e;
 #pragma unroll
     for (int k = 1; k < 64; k <<= 1) l += __shfl_xor(l, k, 64);
-    if (lane == 0) red[g][wave] = l;
-    __syncthreads();
-    if (tid == 0) {
-      const uint32_t h = kvh * G + g;
-      part_ml[((size_t)h * max_splits + split) * 2] = m;
-      part_ml[((size_t)h * max_splits + split) * 2 + 1] = red[g][0] + red[g][1];
-    }
-    __syncthreads();
+    if (lane == 0) red[1][g][wave] = l;
+  }
+  __syncthreads();
+  if (tid < G) {
+    const uint32_t h = kvh * G + tid;
+    part_ml[((size_t)h * max_splits + split) * 2] = fmaxf(red[0][tid][0], red[0][tid][1]);
+    part_ml[((size_t)h * max_splits + split) * 2 + 1] = red[1][tid][0] + red[1][tid][1];
   }
 
-  // ---- phase 2: weighted sum of V rows, one output dimension per thread
-  if (tid < HD) {
-    float o[ATT_MAXG];
+  // ---- phase 2: weighted sum of V rows
+  {
+    float o[G][8];
 #pragma unroll
-    for (int g = 0; g < ATT_MAXG; g++) o[g] = 0.0f;
-    const __half *vcol = vc + (size_t)p0 * kv_dim + kvh * HD + tid;
-    for (uint32_t p = 0; p < n_here; p++) {
-      const float vv = __half2float(vcol[(size_t)p * kv_dim]);
+    for (int g = 0; g < G; g++)
 #pragma unroll
-      for (int g = 0; g < ATT_MAXG; g++)
-        if ((uint32_t)g < G) o[g] += sc[g][p] * vv;
+      for (int j = 0; j < 8; j++) o[g][j] = 0.0f;
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) {
+      const uint32_t p = st * ROWS + rr;   // past the chunk's end the weight sc is 0
+      const __half2 *h2 = (const __half2 *)&vr[st];
+      float vf[8];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const float2 f = __half22float2(h2[j]);
+        vf[2 * j] = f.x;
+        vf[2 * j + 1] = f.y;
+      }
+#pragma unroll
+      for (int g = 0; g < G; g++) {
+        const float w = sc[g][p];
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[g][j] = fmaf(w, vf[j], o[g][j]);
+      }
     }
 #pragma unroll
-    for (int g = 0; g < ATT_MAXG; g++)
-      if ((uint32_t)g < G)
-        part_o[((size_t)(kvh * G + g) * max_splits + split) * HD + tid] = o[g];
+    for (int g = 0; g < G; g++) {
+      *(float4 *)&osum[rr][g][8 * dc] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
+      *(float4 *)&osum[rr][g][8 * dc + 4] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < G * HD; i += 128u) {
+      const uint32_t g = i / HD, d = i - g * HD;
+      float t = 0.0f;
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) t += osum[r][g][d];
+      part_o[((size_t)(kvh * G + g) * max_splits + split) * HD + d] = t;
+    }
   }
 }
 
-// One workgroup; wave w owns the 256-runs w, w + n_wave, ... of the output (n_head * HD values),
-// lane l their elements 4l..4l+3 (one head, four dimensions): merges the chunks' partial
-// softmaxes, stores and quantizes.
+// One wave per 256-run of the output (n_head * HD values), lane l its elements 4l..4l+3 (one
+// head, four dimensions): merges the chunks' partial softmaxes, stores and quantizes.
 template <int GROUP>
-__global__ __launch_bounds__(1024) void ogm_attn_combine_quant_kernel(const float *__restrict__ part_o,
-                                                                      const float *__restrict__ part_ml,
-                                                                      uint32_t n_splits, uint32_t max_splits,
-                                                                      uint32_t n, uint32_t head_dim,
-                                                                      float *__restrict__ attn_out,
-                                                                      OgmActDev act) {
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, n_wave = blockDim.x >> 6;
-  for (uint32_t run = wave; run * 256u < n; run += n_wave) {
-    const uint32_t e0 = run * 256u + 4u * lane;
-    const bool active = e0 < n;
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (active) {
-      const uint32_t h = e0 / head_dim, d = e0 - h * head_dim;
-      const float *ml = part_ml + (size_t)h * max_splits * 2;
-      float M = -INFINITY;
-      for (uint32_t s = 0; s < n_splits; s++) M = fmaxf(M, ml[2 * s]);
-      float den = 0.0f;
-      for (uint32_t s = 0; s < n_splits; s++) {
-        const float f = expf(ml[2 * s] - M);
-        const float4 po = *(const float4 *)(part_o + ((size_t)h * max_splits + s) * head_dim + d);
-        o.x += f * po.x; o.y += f * po.y; o.z += f * po.z; o.w += f * po.w;
-        den += f * ml[2 * s + 1];
+__global__ __launch_bounds__(64) void ogm_attn_combine_quant_kernel(const float *__restrict__ part_o,
+                                                                    const float *__restrict__ part_ml,
+                                                                    uint32_t n_splits, uint32_t max_splits,
+                                                                    uint32_t n, uint32_t head_dim,
+                                                                    float *__restrict__ attn_out,
+                                                                    OgmActDev act) {
+  const uint32_t lane = threadIdx.x;
+  const uint32_t e0 = blockIdx.x * 256u + 4u * lane;
+  const bool active = e0 < n;
+  float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (active) {
+    const uint32_t h = e0 / head_dim, d = e0 - h * head_dim;
+    const float2 *ml = (const float2 *)(part_ml + (size_t)h * max_splits * 2);
+    const float *po = part_o + (size_t)h * max_splits * head_dim + d;
+    // eight chunks at a time: their loads are independent of the running maximum
+    float M = -INFINITY, den = 0.0f;
+    for (uint32_t s0 = 0; s0 < n_splits; s0 += 8u) {
+      float2 mls[8];
+      float4 pos_[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const uint32_t s = min(s0 + u, n_splits - 1u);
+        mls[u] = ml[s];
+        pos_[u] = *(const float4 *)(po + (size_t)s * head_dim);
       }
-      o.x /= den; o.y /= den; o.z /= den; o.w /= den;
-      if (attn_out) *(float4 *)(attn_out + e0) = o;
+      float Mn = M;
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        if (s0 + u < n_splits) Mn = fmaxf(Mn, mls[u].x);
+      const float resc = expf(M - Mn);   // exp(-inf) = 0 on the first group
+      o.x *= resc; o.y *= resc; o.z *= resc; o.w *= resc;
+      den *= resc;
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        if (s0 + u < n_splits) {
+          const float f = expf(mls[u].x - Mn);
+          o.x += f * pos_[u].x; o.y += f * pos_[u].y; o.z += f * pos_[u].z; o.w += f * pos_[u].w;
+          den += f * mls[u].y;
+        }
+      }
+      M = Mn;
     }
-    ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum);
+    o.x /= den; o.y /= den; o.z /= den; o.w /= den;
+    if (attn_out) *(float4 *)(attn_out + e0) = o;
   }
+  ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum);
 }
 
 hipError_t ogm_launch_attn_decode(const float *q, const void *k_cache_layer, const void *v_cache_layer,
                                   uint32_t pos, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
                                   uint32_t head_dim, float scale, float *part_o, float *part_ml, int mode,
                                   float *attn_out, OgmActDev act, hipStream_t stream) {
-  if (n_head_kv == 0 || n_head % n_head_kv != 0 || n_head / n_head_kv > ATT_MAXG) return hipErrorInvalidValue;
+  if (n_head_kv == 0 || n_head % n_head_kv != 0) return hipErrorInvalidValue;
   const uint32_t n_splits = pos / OGM_ATTN_CHUNK + 1u;
   if (n_splits > max_splits) return hipErrorInvalidValue;
   const uint32_t n = n_head * head_dim;
   if (n % 32u != 0) return hipErrorInvalidValue;
   const dim3 grid(n_head_kv, n_splits);
-  if (head_dim == 128)
-    hipLaunchKernelGGL(ogm_attn_partial_kernel<128>, grid, dim3(128), 0, stream, q, (const __half *)k_cache_layer,
-                       (const __half *)v_cache_layer, pos, max_splits, n_head, n_head_kv, scale, part_o, part_ml);
-  else if (head_dim == 64)
-    hipLaunchKernelGGL(ogm_attn_partial_kernel<64>, grid, dim3(128), 0, stream, q, (const __half *)k_cache_layer,
-                       (const __half *)v_cache_layer, pos, max_splits, n_head, n_head_kv, scale, part_o, part_ml);
-  else
-    return hipErrorInvalidValue;
+  const uint32_t G = n_head / n_head_kv;
+#define OGM_ATTN_LAUNCH(HD_, G_)                                                                    \
+  hipLaunchKernelGGL((ogm_attn_partial_kernel<HD_, G_>), grid, dim3(128), 0, stream, q,              \
+                     (const __half *)k_cache_layer, (const __half *)v_cache_layer, pos, max_splits,   \
+                     n_head_kv, scale, part_o, part_ml)
+  if (head_dim == 128 && G == 1) OGM_ATTN_LAUNCH(128, 1);
+  else if (head_dim == 128 && G == 2) OGM_ATTN_LAUNCH(128, 2);
+  else if (head_dim == 128 && G == 4) OGM_ATTN_LAUNCH(128, 4);
+  else if (head_dim == 128 && G == 8) OGM_ATTN_LAUNCH(128, 8);
+  else if (head_dim == 64 && G == 1) OGM_ATTN_LAUNCH(64, 1);
+  else if (head_dim == 64 && G == 2) OGM_ATTN_LAUNCH(64, 2);
+  else if (head_dim == 64 && G == 4) OGM_ATTN_LAUNCH(64, 4);
+  else if (head_dim == 64 && G == 8) OGM_ATTN_LAUNCH(64, 8);
+  else return hipErrorInvalidValue;
+#undef OGM_ATTN_LAUNCH
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const uint32_t runs = (n + 255u) / 256u;
-  const uint32_t waves = runs < 16u ? runs : 16u;
+  const dim3 cgrid((n + 255u) / 256u);
   if (mode == 0)
-    hipLaunchKernelGGL(ogm_attn_combine_quant_kernel<32>, dim3(1), dim3(waves * 64), 0, stream, part_o, part_ml,
+    hipLaunchKernelGGL(ogm_attn_combine_quant_kernel<32>, cgrid, dim3(64), 0, stream, part_o, part_ml,
                        n_splits, max_splits, n, head_dim, attn_out, act);
   else
-    hipLaunchKernelGGL(ogm_attn_combine_quant_kernel<256>, dim3(1), dim3(waves * 64), 0, stream, part_o, part_ml,
+    hipLaunchKernelGGL(ogm_attn_combine_quant_kernel<256>, cgrid, dim3(64), 0, stream, part_o, part_ml,
                        n_splits, max_splits, n, head_dim, attn_out, act);
   return hipGetLastError();
 }
