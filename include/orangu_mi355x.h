@@ -223,6 +223,43 @@ int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_
  * run_layers returns), for parity checks. */
 int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out);
 
+/* ---- GGUF reader -> uploader -------------------------------------------------------------------- */
+
+/* Reads a GGUF file's header, metadata and tensor table (GgufFile::open_at / read, src/gguf.rs:149-280,
+ * value types :386-415) and views its 2-D tensors as matrices (LoadedModel::matrix,
+ * engine/loader.rs:1552-1580), so that a .gguf file loads without the Rust host.  `offset` is where
+ * the GGUF segment starts inside the file (0 for a plain .gguf).  The file is mapped read-only
+ * and stays mapped until ogm_gguf_close; weights uploaded from it do not refer to the mapping.
+ * On failure `err` (when given) receives a message.  GGUF v2+ only (gguf.rs:38). */
+typedef struct ogm_gguf ogm_gguf;
+int ogm_gguf_open(const char *path, uint64_t offset, ogm_gguf **out, char *err, size_t err_len);
+/* The same over bytes the caller holds (they must outlive the handle). */
+int ogm_gguf_parse(const void *bytes, size_t len, ogm_gguf **out, char *err, size_t err_len);
+void ogm_gguf_close(ogm_gguf *g);
+const char *ogm_gguf_last_error(const ogm_gguf *g);
+/* alignment = general.alignment when present and positive, else 32; data_offset = end of the
+ * tensor table rounded up to it, relative to the segment (gguf.rs:258-266). */
+int ogm_gguf_info(const ogm_gguf *g, uint32_t *version, uint64_t *alignment, uint64_t *data_offset,
+                  uint64_t *n_tensors, uint64_t *n_metadata);
+/* Metadata by key.  _u64 follows GgufValue::as_u64 (gguf.rs:70-83: unsigned, non-negative signed,
+ * bool); _f64 also takes the float types; _array reports element type and count. */
+int ogm_gguf_meta_u64(const ogm_gguf *g, const char *key, uint64_t *out);
+int ogm_gguf_meta_f64(const ogm_gguf *g, const char *key, double *out);
+int ogm_gguf_meta_string(const ogm_gguf *g, const char *key, const char **out, size_t *len);
+int ogm_gguf_meta_array(const ogm_gguf *g, const char *key, uint32_t *elem_type, uint64_t *count);
+/* Tensor table: index by name (-1 when absent), entry by index (dims has room for 8), and the
+ * tensor's bytes (size from the block layout, engine/quant.rs:344-357; bounds-checked). */
+int64_t ogm_gguf_find_tensor(const ogm_gguf *g, const char *name);
+int ogm_gguf_tensor(const ogm_gguf *g, uint64_t index, const char **name, uint32_t *n_dims, uint64_t dims[8],
+                    uint32_t *ggml_type, uint64_t *offset);
+int ogm_gguf_tensor_data(ogm_gguf *g, uint64_t index, const void **data, uint64_t *len);
+/* A 2-D tensor as a matrix: dims[0] = in_dim, dims[1] = out_dim, row_bytes * out_dim must equal the
+ * tensor's size (loader.rs:1565-1579). */
+int ogm_gguf_matrix(ogm_gguf *g, const char *name, uint32_t *ggml_type, uint32_t *in_dim, uint32_t *out_dim,
+                    size_t *row_bytes, const void **raw);
+/* ogm_gguf_matrix + ogm_weight_upload, keyed by the mapped bytes' address and length. */
+int ogm_gguf_upload_matrix(ogm_ctx *ctx, ogm_gguf *g, const char *name, ogm_weight **out);
+
 /* ---- tuning / introspection ------------------------------------------------------------------ */
 
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.

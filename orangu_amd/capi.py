@@ -25,6 +25,10 @@ SYMBOLS = [
     "ogm_last_kernel", "ogm_act_quantize_dev", "ogm_matmul_act_dev", "ogm_matmul_multi_dev", "ogm_matmul_multi_act_dev",
     "ogm_llama_create", "ogm_llama_destroy", "ogm_llama_kv_write", "ogm_llama_decode", "ogm_llama_decode_dev",
     "ogm_llama_debug_hidden",
+    "ogm_gguf_open", "ogm_gguf_parse", "ogm_gguf_close", "ogm_gguf_last_error", "ogm_gguf_info",
+    "ogm_gguf_meta_u64", "ogm_gguf_meta_f64", "ogm_gguf_meta_string", "ogm_gguf_meta_array",
+    "ogm_gguf_find_tensor", "ogm_gguf_tensor", "ogm_gguf_tensor_data", "ogm_gguf_matrix",
+    "ogm_gguf_upload_matrix",
 ]
 
 
@@ -93,6 +97,25 @@ def load_library() -> C.CDLL:
     L.ogm_llama_decode.argtypes = [vp, vp, vp, u32, vp, vp]
     L.ogm_llama_decode_dev.argtypes = [vp, vp, vp, u32, vp, vp, vp]
     L.ogm_llama_debug_hidden.argtypes = [vp, vp, vp]
+    L.ogm_gguf_open.argtypes = [C.c_char_p, u64, C.POINTER(vp), C.c_char_p, sz]
+    L.ogm_gguf_parse.argtypes = [vp, sz, C.POINTER(vp), C.c_char_p, sz]
+    L.ogm_gguf_close.argtypes = [vp]
+    L.ogm_gguf_close.restype = None
+    L.ogm_gguf_last_error.argtypes = [vp]
+    L.ogm_gguf_last_error.restype = C.c_char_p
+    L.ogm_gguf_info.argtypes = [vp, C.POINTER(u32), C.POINTER(u64), C.POINTER(u64), C.POINTER(u64), C.POINTER(u64)]
+    L.ogm_gguf_meta_u64.argtypes = [vp, C.c_char_p, C.POINTER(u64)]
+    L.ogm_gguf_meta_f64.argtypes = [vp, C.c_char_p, C.POINTER(C.c_double)]
+    L.ogm_gguf_meta_string.argtypes = [vp, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(sz)]
+    L.ogm_gguf_meta_array.argtypes = [vp, C.c_char_p, C.POINTER(u32), C.POINTER(u64)]
+    L.ogm_gguf_find_tensor.argtypes = [vp, C.c_char_p]
+    L.ogm_gguf_find_tensor.restype = C.c_int64
+    L.ogm_gguf_tensor.argtypes = [vp, u64, C.POINTER(C.c_char_p), C.POINTER(u32), C.POINTER(u64), C.POINTER(u32),
+                                  C.POINTER(u64)]
+    L.ogm_gguf_tensor_data.argtypes = [vp, u64, C.POINTER(vp), C.POINTER(u64)]
+    L.ogm_gguf_matrix.argtypes = [vp, C.c_char_p, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32), C.POINTER(sz),
+                                  C.POINTER(vp)]
+    L.ogm_gguf_upload_matrix.argtypes = [vp, vp, C.c_char_p, C.POINTER(vp)]
     L.ogm_quantize_act.argtypes = [vp, C.c_int, vp, sz, vp, vp, vp]
     L.ogm_dump_block_sums.argtypes = [vp, vp, vp, u32, vp, vp]
     L.ogm_f16_to_f32.argtypes = [vp, vp, sz, vp]

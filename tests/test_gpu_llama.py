@@ -126,3 +126,39 @@ def test_decode_rejects_bad_arguments(be):
             dev.kv_write(0, 3, np.zeros((2, 128), f32), np.zeros((2, 128), f32))
     finally:
         dev.close()
+
+
+def test_matrices_uploaded_from_a_gguf_file_multiply_like_direct_uploads(be, tmp_path):
+    """GGUF reader -> uploader: the same bytes reach the device as through QuantMatrix."""
+    import oracle
+    from orangu_amd import QuantMatrix
+    from orangu_amd.gguf import GgufFile
+    from orangu_amd.hiprt import DeviceBuffer, device_synchronize
+    from test_gguf_cpu import gguf, gstr, kv, tensor_info
+    specs = [("blk.0.ffn_gate.weight", Q4_K, 512, 70), ("blk.0.ffn_down.weight", Q6_K, 256, 33),
+             ("blk.0.attn_q.weight", Q8_0, 96, 17)]
+    blobs, infos, pos = [], [], 0
+    for i, (name, t, n_in, n_out) in enumerate(specs):
+        w = synth_weights(t, n_in, n_out, seed=20 + i)
+        infos.append(tensor_info(name, [n_in, n_out], t, pos))
+        blobs.append(w.tobytes() + b"\0" * ((-w.size) % 32))
+        pos += len(blobs[-1])
+    b, _ = gguf([kv("general.architecture", 8, gstr("llama"))], infos, data=b"".join(blobs))
+    path = tmp_path / "tiny.gguf"
+    path.write_bytes(b)
+    g = GgufFile(str(path))
+    for name, t, n_in, n_out in specs:
+        h = g.upload_matrix(be, name)
+        assert g.upload_matrix(be, name) == h          # same bytes, same key: one device copy
+        x = np.random.default_rng(n_in).standard_normal(n_in).astype(f32)
+        xd, yd = DeviceBuffer.from_numpy(x), DeviceBuffer(4 * n_out)
+        be.matmul_dev(h, xd.ptr, 1, yd.ptr)
+        device_synchronize()
+        raw = g.matrix(name)[4]
+        want = oracle.matmul(t, raw, n_in, n_out, x, 1).reshape(-1)
+        got = yd.to_numpy(f32, n_out)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), name
+        assert np.array_equal(got, be.matmul(x, 1, QuantMatrix(raw, t, n_in, n_out)))
+        xd.free()
+        yd.free()
+    g.close()
