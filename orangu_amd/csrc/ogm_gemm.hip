@@ -399,6 +399,232 @@ __global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Q6_K (gemm_k_q6_k, engine/vecdot.rs:2352-2398): acc += ad * (d * sum_g sc_g * dot16(q_g - 32, x_g))
+// over the 16 groups of a super-block, sc_g a signed byte.
+//
+// sc_g * (q - 32) reaches 4096 and is not exact in f16, so the scale is split in base 16,
+// sc = 16 a + b with a = sc >> 4 in [-8, 7] and b = sc & 15: the operands a*(q-32) (|.| <= 256)
+// and b*(q-32) (|.| <= 480) are exact, their 256-long chains stay below 2^24
+// (256*127*256 = 8.3e6, 480*127*256 = 1.56e7), and isum = 16 * c_hi + c_lo is an exact scaling
+// by a power of two followed by one f32 add of exact integers: the rounding of `isum as f32`.
+//
+// Same tiling as the Q4_K kernel: eight waves, 128 rows x 128 tokens, k in stages of 64.  A thread
+// stages one group of 16 weights (one ql piece, one qh piece, one scale) into both operand tiles.
+// Block layout (quant.rs:744-787): element 128h + 32r + 16k + j of a super-block has its low four
+// bits in ql[64h + 32(r&1) + 16k + j] (low nibble for r < 2, high for r >= 2), bits 4..5 in
+// qh[32h + 16k + j] >> 2r, and scale sc[8h + 2r + k].
+
+struct Gemm6Params {
+  const uint8_t *wt;      // tile-planar Q6_K
+  const _Float16 *xh;     // [T][in_dim] int8 activations as f16
+  const float *ad;        // [T][nsb] activation scales (per 256)
+  float *y;               // [T][out_dim]
+  uint32_t in_dim, out_dim, n_tokens, nsb;
+  uint32_t c_shift, r_shift, nct;
+};
+
+#define G6_TILE_BYTES 13440u   // 64 units of 210 bytes: 13 pieces of 1 KiB, then 64 two-byte tails
+
+__global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  _Float16 *Ah_l = (_Float16 *)lds;                 // [2][128][64]  a * (q - 32)
+  _Float16 *Al_l = Ah_l + 2 * GM_STAGE_HALFS;       // [2][128][64]  b * (q - 32)
+  _Float16 *B_l = Al_l + 2 * GM_STAGE_HALFS;        // [2][128][64]
+  float *d_l = (float *)(B_l + 2 * GM_STAGE_HALFS); // [2][128]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t wr = wave & 1u, wt_ = wave >> 1;   // wave's row half (64 rows) and token quarter (32)
+  const uint32_t t0 = blockIdx.x * GM_BT, r0 = blockIdx.y * GM_BN;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+
+  // staging role: row lr_a, group t16 (16 weights) of the stage
+  const uint32_t lr_a = (tid >> 6) * 16u + (tid & 15u), t16 = (tid >> 4) & 3u;
+  uint32_t unit_off, tail_off;   // the row's unit inside a tile: pieces at unit_off + 1024 p, d at tail_off
+  {
+    const uint32_t row = min(r0 + lr_a, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    unit_off = rb * p.nct * G6_TILE_BYTES + r * 16u;
+    tail_off = rb * p.nct * G6_TILE_BYTES + 13u * 1024u + r * 2u;
+  }
+  auto sb_tile = [&](uint32_t s) -> uint32_t { return (s >> p.c_shift) * G6_TILE_BYTES; };
+  auto sb_lane = [&](uint32_t s) -> uint32_t { return (s & ((1u << p.c_shift) - 1u)) << p.r_shift; };
+  const uint32_t btok = tid >> 3, bpart = tid & 7u;   // activation chunk i: token btok + 64 i, part bpart
+  const uint32_t bo0 = min(t0 + btok, p.n_tokens - 1u) * p.in_dim + bpart * 8u;
+  const uint32_t bo1 = min(t0 + btok + 64u, p.n_tokens - 1u) * p.in_dim + bpart * 8u;
+  const uint32_t tko = min(t0 + 32u * wt_ + l32, p.n_tokens - 1u) * p.nsb;
+
+  float16v y0, y1;
+  const float16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
+
+  // loads run two stages ahead through three rotating register sets
+  uint4 ql_0, ql_1, ql_2, qh_0, qh_1, qh_2, bx0_0, bx0_1, bx0_2, bx1_0, bx1_1, bx1_2;
+  uint4 scx = make_uint4(0, 0, 0, 0);   // the super-block's 16 scales
+  uint32_t d16 = 0;
+  uint32_t scw[4] = {0, 0, 0, 0};
+  float dnext = 0.0f;
+
+#define G6_LOAD_STAGE(S, G, K)                                                                    \
+  do {                                                                                            \
+    const uint32_t uo_ = unit_off + sb_tile(S) + sb_lane(S) * 16u;                                \
+    const uint32_t h_ = (G) >> 1;                                                                 \
+    if ((G) == 0) {                                                                               \
+      scx = *(const uint4 *)(p.wt + (uo_ + 12u * 1024u));                                         \
+      d16 = *(const uint16_t *)(p.wt + (tail_off + sb_tile(S) + sb_lane(S) * 2u));                \
+    }                                                                                             \
+    ql_##K = *(const uint4 *)(p.wt + (uo_ + (4u * h_ + t16) * 1024u));                            \
+    qh_##K = *(const uint4 *)(p.wt + (uo_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));                \
+    const uint32_t ko_ = (S) * 256u + (G) * 64u;                                                  \
+    bx0_##K = *(const uint4 *)(p.xh + (bo0 + ko_));                                               \
+    bx1_##K = *(const uint4 *)(p.xh + (bo1 + ko_));                                               \
+  } while (0)
+
+  // Four bytes of 6-bit values (still carrying the +32) -> (v - 32) * a and (v - 32) * b as f16
+#define G6_DEQ(V, HI01, HI23, LO01, LO23)                                                         \
+  do {                                                                                            \
+    union { uint32_t u; half2v h; } e_, f_;                                                       \
+    e_.u = __builtin_amdgcn_perm(0u, (V), 0x0c010c00u) | 0x64006400u; /* 1024 + v */              \
+    f_.u = __builtin_amdgcn_perm(0u, (V), 0x0c030c02u) | 0x64006400u;                             \
+    e_.h = e_.h + k1056_;                                                                         \
+    f_.h = f_.h + k1056_;                                                                         \
+    union { uint32_t u; half2v h; } o_;                                                           \
+    o_.h = e_.h * a2_; HI01 = o_.u;                                                               \
+    o_.h = f_.h * a2_; HI23 = o_.u;                                                               \
+    o_.h = e_.h * b2_; LO01 = o_.u;                                                               \
+    o_.h = f_.h * b2_; LO23 = o_.u;                                                               \
+  } while (0)
+
+#define G6_STORE_STAGE(S, G, BUF, K)                                                              \
+  do {                                                                                            \
+    if ((G) == 0) {                                                                               \
+      scw[0] = scx.x; scw[1] = scx.y; scw[2] = scx.z; scw[3] = scx.w;                             \
+      dnext = gm_f16_bits_to_f32(d16);                                                            \
+    }                                                                                             \
+    /* scale of group 4G + t16, split as 16 a + b */                                              \
+    const uint32_t sw_ = (G) == 0 ? scw[0] : (G) == 1 ? scw[1] : (G) == 2 ? scw[2] : scw[3];      \
+    const int sc_ = (int)(int8_t)((sw_ >> (8u * t16)) & 0xFFu);                                   \
+    const _Float16 af_ = (_Float16)(float)(sc_ >> 4), bf_ = (_Float16)(float)(sc_ & 15);          \
+    const half2v a2_ = {af_, af_}, b2_ = {bf_, bf_};                                              \
+    const half2v k1056_ = {(_Float16)-1056.0f, (_Float16)-1056.0f};                               \
+    const uint32_t m4_ = 0x0F0F0F0Fu, m2_ = 0x30303030u;                                          \
+    const uint32_t rr_ = 2u * ((G) & 1u) + (t16 >> 1);        /* run of 32 inside the half block */ \
+    const uint32_t qlw_[4] = {ql_##K.x, ql_##K.y, ql_##K.z, ql_##K.w};                            \
+    const uint32_t qhw_[4] = {qh_##K.x, qh_##K.y, qh_##K.z, qh_##K.w};                            \
+    uint32_t hi_[8], lo_[8];                                                                      \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      const uint32_t nib_ = (((G) & 1u) ? (qlw_[w_] >> 4) : qlw_[w_]) & m4_;                      \
+      const uint32_t v_ = nib_ | ((((qhw_[w_] >> (2u * rr_)) << 4)) & m2_);                       \
+      G6_DEQ(v_, hi_[2 * w_], hi_[2 * w_ + 1], lo_[2 * w_], lo_[2 * w_ + 1]);                     \
+    }                                                                                             \
+    _Float16 *ah_ = Ah_l + (BUF) * GM_STAGE_HALFS, *al_ = Al_l + (BUF) * GM_STAGE_HALFS;          \
+    *(uint4 *)(ah_ + gm_swz(lr_a, 2u * t16)) = make_uint4(hi_[0], hi_[1], hi_[2], hi_[3]);        \
+    *(uint4 *)(ah_ + gm_swz(lr_a, 2u * t16 + 1u)) = make_uint4(hi_[4], hi_[5], hi_[6], hi_[7]);   \
+    *(uint4 *)(al_ + gm_swz(lr_a, 2u * t16)) = make_uint4(lo_[0], lo_[1], lo_[2], lo_[3]);        \
+    *(uint4 *)(al_ + gm_swz(lr_a, 2u * t16 + 1u)) = make_uint4(lo_[4], lo_[5], lo_[6], lo_[7]);   \
+    _Float16 *bb_ = B_l + (BUF) * GM_STAGE_HALFS;                                                 \
+    *(uint4 *)(bb_ + gm_swz(btok, bpart)) = bx0_##K;                                              \
+    *(uint4 *)(bb_ + gm_swz(btok + 64u, bpart)) = bx1_##K;                                        \
+    if ((G) == 0) d_l[((S) & 1u) * 128u + lr_a] = dnext; /* the four threads of a row agree */    \
+  } while (0)
+
+  // One stage: loads of the stage two ahead, this stage's MFMAs with the next stage's
+  // dequantization in their shadow, then, after the super-block's last stage, its f32 step.
+#define G6_STAGE(G, KL, KS)                                                                       \
+  do {                                                                                            \
+    const uint32_t buf = (G) & 1u;                                                                \
+    if ((G) == 0) adv = p.ad[tko + s];                                                            \
+    /* past the end the last super-block is loaded again and parked in the idle buffer */        \
+    G6_LOAD_STAGE(min((G) < 2 ? s : s + 1u, p.nsb - 1u), (uint32_t)(((G) + 2) & 3), KL);          \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+    const _Float16 *ah = Ah_l + buf * GM_STAGE_HALFS, *al = Al_l + buf * GM_STAGE_HALFS;          \
+    const _Float16 *bb = B_l + buf * GM_STAGE_HALFS;                                              \
+    _Pragma("unroll") for (int kk = 0; kk < 4; kk++) {                                            \
+      const half8 ah0 = *(const half8 *)(ah + gm_swz(ra, 2u * kk + lh));                          \
+      const half8 ah1 = *(const half8 *)(ah + gm_swz(ra + 32u, 2u * kk + lh));                    \
+      const half8 al0 = *(const half8 *)(al + gm_swz(ra, 2u * kk + lh));                          \
+      const half8 al1 = *(const half8 *)(al + gm_swz(ra + 32u, 2u * kk + lh));                    \
+      const half8 b0 = *(const half8 *)(bb + gm_swz(rbk, 2u * kk + lh));                          \
+      const bool first_ = (G) == 0 && kk == 0;   /* the super-block starts fresh accumulators */  \
+      ch0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah0, b0, first_ ? zero : ch0, 0, 0, 0);        \
+      ch1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah1, b0, first_ ? zero : ch1, 0, 0, 0);        \
+      cl0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al0, b0, first_ ? zero : cl0, 0, 0, 0);        \
+      cl1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al1, b0, first_ ? zero : cl1, 0, 0, 0);        \
+    }                                                                                             \
+    G6_STORE_STAGE(((G) + 1) < 4 ? s : min(s + 1u, p.nsb - 1u), (uint32_t)(((G) + 1) & 3), buf ^ 1u, KS); \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+    if ((G) == 3) {                                                                               \
+      /* isum = 16 c_hi + c_lo (one rounding), then the reference's f32 steps */                  \
+      const float *dp = d_l + (s & 1u) * 128u + 64u * wr + 4u * lh;                               \
+      _Pragma("unroll") for (int q4 = 0; q4 < 4; q4++) {                                          \
+        const float4 d0 = *(const float4 *)(dp + 8 * q4), d1 = *(const float4 *)(dp + 32 + 8 * q4); \
+        const float d0v[4] = {d0.x, d0.y, d0.z, d0.w}, d1v[4] = {d1.x, d1.y, d1.z, d1.w};         \
+        _Pragma("unroll") for (int e = 0; e < 4; e++) {                                           \
+          y0[4 * q4 + e] += adv * (d0v[e] * (ch0[4 * q4 + e] * 16.0f + cl0[4 * q4 + e]));         \
+          y1[4 * q4 + e] += adv * (d1v[e] * (ch1[4 * q4 + e] * 16.0f + cl1[4 * q4 + e]));         \
+        }                                                                                         \
+      }                                                                                           \
+    }                                                                                             \
+    __syncthreads();                                                                              \
+  } while (0)
+
+  G6_LOAD_STAGE(0u, 0u, 0);
+  G6_LOAD_STAGE(0u, 1u, 1);
+  G6_STORE_STAGE(0u, 0u, 0u, 0);
+  __syncthreads();
+
+  const uint32_t ra = 64u * wr + l32, rbk = 32u * wt_ + l32;
+  // Stages rotate through three register sets while a super-block has four stages, so the set
+  // of a stage is (4 s + g) mod 3: three super-blocks make one period of the loop body.
+  uint32_t s = 0;
+  float16v ch0, ch1, cl0, cl1;
+  float adv = 0.0f;
+#define G6_SB(K0, K1, K2)            /* sets of stages g = 0, 1, 2; g = 3 uses K0 again */          \
+  do {                                                                                            \
+    G6_STAGE(0, K2, K1);   /* loads stage 4s+2 into the set two ahead, parks stage 4s+1 */        \
+    G6_STAGE(1, K0, K2);                                                                          \
+    G6_STAGE(2, K1, K0);                                                                          \
+    G6_STAGE(3, K2, K1);                                                                          \
+    s++;                                                                                          \
+  } while (0)
+  while (s < p.nsb) {
+    G6_SB(0, 1, 2);                 // stages 4s..4s+3 in sets 0 1 2 0
+    if (s >= p.nsb) break;
+    G6_SB(1, 2, 0);                 // 1 2 0 1
+    if (s >= p.nsb) break;
+    G6_SB(2, 0, 1);                 // 2 0 1 2
+  }
+#undef G6_SB
+#undef G6_STAGE
+#undef G6_STORE_STAGE
+#undef G6_LOAD_STAGE
+#undef G6_DEQ
+
+  const uint32_t t = t0 + 32u * wt_ + l32;
+  if (t < p.n_tokens) {
+    const bool vec = (p.out_dim & 3u) == 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const float16v &yy = i ? y1 : y0;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const uint32_t row = r0 + 64u * wr + 32u * i + 8u * q4 + 4u * lh;
+        float *dst = p.y + (size_t)t * p.out_dim + row;
+        if (vec && row + 3u < p.out_dim) {
+          *(float4 *)dst = make_float4(yy[4 * q4], yy[4 * q4 + 1], yy[4 * q4 + 2], yy[4 * q4 + 3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            if (row + e < p.out_dim) dst[e] = yy[4 * q4 + e];
+        }
+      }
+    }
+  }
+}
+
+static const uint32_t G6_LDS_BYTES = 6 * GM_STAGE_HALFS * 2 + 2 * 128 * 4;
+
 static const uint32_t GM_LDS_BYTES = 4 * GM_STAGE_HALFS * 2 + 2 * 128 * 16 * 2 + 128 * 4;
 static const uint32_t GM_STAGING_BYTES = 4 * GM_STAGE_HALFS * 2;
 
@@ -408,12 +634,13 @@ size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens) {
 }
 
 bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
-  if (ggml_type != OGM_Q4_K || in_dim == 0 || in_dim % 256u != 0) return false;
-  // pass 1 keeps one f32 per (row, super-block) of the workgroup in the staging area of LDS
-  if ((size_t)(in_dim / 256u) * 512u > GM_STAGING_BYTES) return false;
-  // the kernel addresses weights and activations with 32-bit byte offsets
+  if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K) || in_dim == 0 || in_dim % 256u != 0) return false;
+  // Q4_K's pass 1 keeps one f32 per (row, super-block) of the workgroup in the staging area of LDS
+  if (ggml_type == OGM_Q4_K && (size_t)(in_dim / 256u) * 512u > GM_STAGING_BYTES) return false;
+  // the kernels address weights and activations with 32-bit byte offsets
   const uint64_t lim = 0xFFFFFFFFull;
-  return (uint64_t)ogm_tiling_for(in_dim / 256u, out_dim).nrb * 64u * (in_dim / 256u) * 144u <= lim &&
+  const uint64_t block = ggml_type == OGM_Q4_K ? 144u : 210u;
+  return (uint64_t)ogm_tiling_for(in_dim / 256u, out_dim).nrb * 64u * (in_dim / 256u) * block <= lim &&
          (uint64_t)in_dim * n_tokens * 2u <= lim;
 }
 
@@ -426,6 +653,33 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   _Float16 *bs16 = xh + (size_t)a.in_dim * a.n_tokens;
   hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, stream,
                      a.act.q, a.act.bsum, xh, bs16, n8, n_sb);
+  const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
+  const uint32_t c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
+  // token tiles vary fastest: workgroups that run together share weight rows, and with a
+  // power-of-two number of token tiles each XCD's L2 sees few distinct activation tiles
+  const dim3 grid((a.n_tokens + GM_BT - 1) / GM_BT, (a.out_dim + GM_BN - 1) / GM_BN);
+  hipError_t e;
+  if (a.ggml_type == OGM_Q6_K) {
+    Gemm6Params p;
+    p.wt = a.wt;
+    p.xh = xh;
+    p.ad = a.act.d;
+    p.y = a.y;
+    p.in_dim = a.in_dim;
+    p.out_dim = a.out_dim;
+    p.n_tokens = a.n_tokens;
+    p.nsb = nsb;
+    p.c_shift = c_shift;
+    p.r_shift = 6 - c_shift;
+    p.nct = tl.nct;
+    // more dynamic LDS than the 64 KB a kernel gets without asking
+    e = hipFuncSetAttribute((const void *)ogm_gemm_q6k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)G6_LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(ogm_gemm_q6k_kernel, grid, dim3(512), G6_LDS_BYTES, stream, p);
+    if (kernel_name) *kernel_name = "ogm_gemm_q6k_kernel";
+    return hipGetLastError();
+  }
   GemmParams p;
   p.wt = a.wt;
   p.xh = xh;
@@ -436,16 +690,11 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   p.out_dim = a.out_dim;
   p.n_tokens = a.n_tokens;
   p.nsb = nsb;
-  const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
-  p.c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
-  p.r_shift = 6 - p.c_shift;
+  p.c_shift = c_shift;
+  p.r_shift = 6 - c_shift;
   p.nct = tl.nct;
-  // token tiles vary fastest: workgroups that run together share weight rows, and with a
-  // power-of-two number of token tiles each XCD's L2 sees few distinct activation tiles
-  const dim3 grid((a.n_tokens + GM_BT - 1) / GM_BT, (a.out_dim + GM_BN - 1) / GM_BN);
-  // more dynamic LDS than the 64 KB a kernel gets without asking
-  hipError_t e = hipFuncSetAttribute((const void *)ogm_gemm_q4k_kernel,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)GM_LDS_BYTES);
+  e = hipFuncSetAttribute((const void *)ogm_gemm_q4k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)GM_LDS_BYTES);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(ogm_gemm_q4k_kernel, grid, dim3(512), GM_LDS_BYTES, stream, p);
   if (kernel_name) *kernel_name = "ogm_gemm_q4k_kernel";

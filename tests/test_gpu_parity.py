@@ -383,6 +383,61 @@ def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign):
     say("extreme isum", int(np.abs(isum).max()), "imin", int(np.abs(imin).max()))
 
 
+@pytest.mark.parametrize("in_dim,out_dim,T", [
+    (256, 5, 9), (512, 130, 17), (768, 64, 129), (1024, 100, 64), (1280, 257, 40), (2048, 37, 128),
+    (4096, 200, 130), (14336, 96, 257), (4096, 1000, 512), (1792, 33, 10),
+])
+def test_mfma_gemm_q6k_matches_cpu_gemm(be, in_dim, out_dim, T):
+    """Q6_K at n_tokens >= 9 takes its MFMA kernel; values must equal gemm_k_q6_k
+    (vecdot.rs:2352-2398): the scale split 16a + b keeps both operand chains exact."""
+    raw = synth_weights(Q6_K, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T + 1)
+    w = qm(raw, Q6_K, in_dim, out_dim)
+    say("gemm q6k", in_dim, out_dim, T)
+    got = be.matmul(x, T, w)
+    assert be.last_kernel() == "ogm_gemm_q6k_kernel"
+    want = oracle.matmul(Q6_K, raw, in_dim, out_dim, x, T)
+    assert_close(got, want, "mfma gemm q6k")
+    assert_bits(got, want, "mfma gemm q6k")
+    be.set_tuning("gemm_min_tokens", 100000)
+    try:
+        small = be.matmul(x, T, w)
+        assert be.last_kernel().startswith("ogm_gemv_kernel")
+    finally:
+        be.set_tuning("gemm_min_tokens", 0)
+    assert_bits(got, small, "mfma vs multi-token gemv")
+
+
+@pytest.mark.parametrize("ql,qh,sc,sign", [(0xFF, 0xFF, 0x7F, "alt"), (0x00, 0x00, 0x80, "pos"), (0xFF, 0xFF, 0x80, "neg"),
+                                           (0x00, 0x00, 0x7F, "alt"), (0xF0, 0x0F, 0x8F, "block"), (0x0F, 0xF0, 0x70, "pos")])
+def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign):
+    """Extreme 6-bit values (0 -> -32, 63 -> +31), scales -128 / +127 / -113 / +112 and activations
+    +-127: |isum| reaches 1.3e8, far past 2^24; the high and low scale digits' chains reach their
+    bounds, and 16 * c_hi + c_lo must round exactly like `isum as f32`."""
+    in_dim, out_dim, T = 1024, 32, 16
+    blocks = np.zeros((out_dim * 4, 210), np.uint8)
+    blocks[:, 0:128] = ql
+    blocks[:, 128:192] = qh
+    blocks[:, 192:208] = sc
+    blocks[:, 208:210] = np.frombuffer(np.float16(0.003).tobytes(), np.uint8)
+    x = np.full((T, in_dim), 127.0, np.float32)
+    if sign == "alt":
+        x[1::2] *= -1
+        x[:, ::7] = 126.0
+    elif sign == "neg":
+        x *= -1
+    elif sign == "block":
+        x[:, 128:256] *= -1
+        x[3] = -127.0
+    raw = blocks.reshape(-1)
+    got = be.matmul(x, T, qm(raw, Q6_K, in_dim, out_dim))
+    assert be.last_kernel() == "ogm_gemm_q6k_kernel"
+    want = oracle.matmul(Q6_K, raw, in_dim, out_dim, x, T)
+    assert_bits(got, want, "extreme ranges")
+    isum, _ = be.dump_block_sums(x[0], 1, qm(raw, Q6_K, in_dim, out_dim))
+    say("extreme q6k isum", int(np.abs(isum).max()))
+
+
 # ---------------------------------------------------------------- quantize inside the GEMV, grouped launches
 
 @pytest.mark.parametrize("t,in_dim,out_dim", [
