@@ -14,12 +14,14 @@
 // reference's order: first `acc -= (ad*dmin) * imin` over all super-blocks, then
 // `acc += ad * (d * isum)` over all super-blocks.
 //
-// Tiling: a workgroup of eight waves owns 128 rows x 128 tokens; a wave owns 64 rows x 32 tokens
-// = two v_mfma_f32_32x32x16_f16 tiles.  The k loop advances 64 at a time (a quarter super-block:
-// one piece pair of qs, i.e. sub-blocks 2g and 2g+1): each thread dequantizes half a 16-byte piece
-// (v_perm byte spread, magic-number int->f16, packed f16 add and multiply) into LDS and copies
-// two 16-byte chunks of the f16 activations; LDS is double buffered and the next stage's global
-// loads are issued before the current stage's MFMAs, so there is one barrier per stage.
+// Tiling: a workgroup owns 128 rows x 128 tokens and has sixteen waves, four per SIMD.  Eight
+// "multiplying" waves own 64 rows x 32 tokens each = two v_mfma_f32_32x32x16_f16 tiles; eight
+// "feeding" waves do the global loads, the dequantization (v_perm byte spread, magic-number
+// int->f16, packed f16 add and multiply: half a 16-byte piece of qs per thread and stage) and the
+// LDS stores, so that on every SIMD the matrix pipe and the vector pipe are busy at the same time.
+// The k loop advances 64 at a time (a quarter super-block: one piece pair of qs, i.e. sub-blocks
+// 2g and 2g+1); LDS is double buffered, global loads run two stages ahead through three rotating
+// register sets, and there is one barrier per stage.
 #include <hip/hip_runtime.h>
 
 #include "ogm_kernels.h"
@@ -140,17 +142,22 @@ __device__ __forceinline__ uint32_t gm_swz(uint32_t row, uint32_t chunk) {
   return row * 64u + ((chunk ^ (row & 7u) ^ ((row >> 3) & 1u)) << 3);  // in f16 units
 }
 
-__global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
+__global__ __launch_bounds__(1024) void ogm_gemm_q4k_kernel(GemmParams p) {
   extern __shared__ __align__(16) uint8_t lds[];
   _Float16 *A_l = (_Float16 *)lds;                  // [2][128][64]
   _Float16 *B_l = A_l + 2 * GM_STAGE_HALFS;         // [2][128][64]
   _Float16 *a2_l = B_l + 2 * GM_STAGE_HALFS;        // [128 rows][16]: 512*sc_j | 8*sc_j
   _Float16 *b2_l = a2_l + 128 * 16;                 // [128 tokens][16]: bh_j | bl_j
   float *d_l = (float *)(b2_l + 128 * 16);          // [128]
-  float *dmin_t = (float *)lds;                     // pass 1 only: [nsb][128], over A_l / B_l
+  float *dmin_t = d_l + 128;                        // pass 1 only: [nsb][128]
 
+  // Sixteen waves, four per SIMD: waves 0..7 multiply (MFMA and the f32 steps), waves 8..15 feed
+  // them (global loads, dequantization, LDS stores), so that on every SIMD the matrix pipe and the
+  // vector pipe work at the same time.  Both halves run the same number of barriers.
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const uint32_t wr = wave & 1u, wt_ = wave >> 1;   // wave's row half (64 rows) and token quarter (32)
+  const bool producer = wave >= 8u;
+  const uint32_t rt = tid & 511u;                   // thread index within its half
+  const uint32_t wr = wave & 1u, wt_ = (wave & 7u) >> 1;   // multiplying wave: row half (64 rows), token quarter (32)
   const uint32_t t0 = blockIdx.x * GM_BT, r0 = blockIdx.y * GM_BN;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
@@ -178,7 +185,7 @@ __global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
   for (int r = 0; r < 16; r++) zero[r] = 0.0f;
 
   // ---------------- pass 1: acc -= (ad * dmin) * sum_j m_j * bsum_j, all super-blocks first
-  for (uint32_t i = tid; i < p.nsb * 128u; i += 512u) {
+  for (uint32_t i = tid; i < p.nsb * 128u; i += 1024u) {
     const uint32_t s = i >> 7, lr = i & 127u;
     const uint32_t h = *(const uint32_t *)(p.wt + (row_off(r0 + lr) + sb_off(s)));
     dmin_t[i] = gm_f16_bits_to_f32(h >> 16);
@@ -186,7 +193,7 @@ __global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
   __syncthreads();
   const uint32_t ro0 = row_off(r0 + 64u * wr + l32), ro1 = row_off(r0 + 64u * wr + 32u + l32);
   const uint32_t tko = tk * p.nsb;  // this token's first (token, super-block) index
-  {
+  if (!producer) {
     const float side_scale = lh ? 1.0f : 64.0f;
     // four super-blocks at a time, so that four sets of loads share one trip to memory
 #pragma unroll 1
@@ -229,25 +236,24 @@ __global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
       }
     }
   }
-  __syncthreads();  // dmin_t is about to be overwritten by the staging buffers
 
   // ---------------- pass 2: acc += ad * (d * sum_j sc_j * dot32_j)
   // Staging roles.  Weights: half a 16-byte piece of qs per thread (8 bytes = 8 low-nibble and 8
   // high-nibble weights).  Activations: two 16-byte chunks per thread.  Once per super-block
   // also the row's scales (side operand and d) and one chunk of bh | bl.
-  const uint32_t pid = tid >> 1, half = tid & 1u;
+  const uint32_t pid = rt >> 1, half = rt & 1u;
   const uint32_t lr_a = (pid >> 5) * 16u + (pid & 15u), hh = (pid >> 4) & 1u;
-  const uint32_t btok = tid >> 3, bpart = tid & 7u;   // chunk i: token btok + 64 i, part bpart
+  const uint32_t btok = rt >> 3, bpart = rt & 7u;   // chunk i: token btok + 64 i, part bpart
   const uint32_t bt0 = min(t0 + btok, p.n_tokens - 1u), bt1 = min(t0 + btok + 64u, p.n_tokens - 1u);
   const uint32_t roa = row_off(r0 + lr_a) + hh * 1024u + 8u * half;   // this thread's half piece
   const uint32_t bo0 = bt0 * p.in_dim + bpart * 8u, bo1 = bt1 * p.in_dim + bpart * 8u;  // in f16
   // (the upper half of the workgroup repeats the lower half's bh | bl chunk: no branch needed)
-  const uint32_t b2o = min(t0 + ((tid & 255u) >> 1), p.n_tokens - 1u) * p.nsb * 16u + 8u * (tid & 1u);
-  // Loads run three stages ahead of the MFMAs through four rotating register sets (a stage is
-  // far shorter than a trip to memory); the header and bh | bl loads of a super-block have one
+  const uint32_t b2o = min(t0 + ((rt & 255u) >> 1), p.n_tokens - 1u) * p.nsb * 16u + 8u * (rt & 1u);
+  // Loads run two stages ahead of the MFMAs through three rotating register sets (a stage is
+  // shorter than a trip to memory); the header and bh | bl loads of a super-block have one
   // set, which is consumed before the next super-block's are issued.
-  uint2 qv_0, qv_1, qv_2, qv_3;
-  uint4 bx0_0, bx0_1, bx0_2, bx0_3, bx1_0, bx1_1, bx1_2, bx1_3;
+  uint2 qv_0, qv_1, qv_2;
+  uint4 bx0_0, bx0_1, bx0_2, bx1_0, bx1_1, bx1_2;
   uint4 hdx = make_uint4(0, 0, 0, 0), b2x = make_uint4(0, 0, 0, 0);
   uint32_t sca = 0, scb = 0;
   float dnext = 0.0f;
@@ -290,20 +296,26 @@ __global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
       /* the four threads of a row write the same values */                                      \
       *(half8 *)(a2_l + lr_a * 16u + 8u * half) = side_operand(sca, scb, half ? 8.0f : 512.0f);   \
       d_l[lr_a] = dnext;                                                                          \
-      *(uint4 *)(b2_l + ((tid & 255u) >> 1) * 16u + 8u * (tid & 1u)) = b2x;                       \
+      *(uint4 *)(b2_l + ((rt & 255u) >> 1) * 16u + 8u * (rt & 1u)) = b2x;                         \
     }                                                                                             \
   } while (0)
 
-  // One stage: issue the loads of the stage three ahead, then this stage's MFMAs with the
-  // dequantization of the next stage (into the other LDS buffer) in their shadow, then, after
-  // the super-block's last stage, its f32 step.
-#define GM_STAGE(G, KL, KS)                                                                       \
+  // One stage of a feeding wave: issue the loads of the stage two ahead, dequantize and park
+  // the next stage in the LDS buffer the multiplying waves are not reading.
+#define GM_PRODUCE(G, KL, KS)                                                                     \
+  do {                                                                                            \
+    /* past the end the last super-block is loaded again and parked in the idle buffer */        \
+    GM_LOAD_STAGE(min((G) < 2 ? s : s + 1u, p.nsb - 1u), (uint32_t)(((G) + 2) & 3), KL);          \
+    GM_STORE_STAGE((uint32_t)(((G) + 1) & 3), ((G) & 1u) ^ 1u, KS);                               \
+    __syncthreads();                                                                              \
+  } while (0)
+
+  // One stage of a multiplying wave: this stage's MFMAs from LDS, then, after the super-block's
+  // last stage, its f32 step.
+#define GM_CONSUME(G)                                                                             \
   do {                                                                                            \
     const uint32_t buf = (G) & 1u;                                                                \
     if ((G) == 0) adv = p.ad[tko + s]; /* needed three stages from now */                         \
-    /* past the end the last super-block is loaded again and parked in the idle buffer */        \
-    GM_LOAD_STAGE(min((G) == 0 ? s : s + 1u, p.nsb - 1u), (uint32_t)(((G) + 3) & 3), KL);         \
-    __builtin_amdgcn_sched_barrier(0);                                                            \
     const _Float16 *ab = A_l + buf * GM_STAGE_HALFS, *bb = B_l + buf * GM_STAGE_HALFS;            \
     half8 a0 = *(const half8 *)(ab + gm_swz(ra, lh));                                             \
     half8 a1 = *(const half8 *)(ab + gm_swz(ra + 32u, lh));                                       \
@@ -320,15 +332,6 @@ __global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
       c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, ((G) == 0 && kk == 0) ? zero : c1, 0, 0, 0); \
       a0 = na0; a1 = na1; b0 = nb0;                                                               \
     }                                                                                             \
-    GM_STORE_STAGE((uint32_t)(((G) + 1) & 3), buf ^ 1u, KS);                                      \
-    /* the dequantization of the next stage goes into the shadow of this stage's MFMAs */        \
-    _Pragma("unroll") for (int q_ = 0; q_ < 8; q_++) {                                            \
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                          \
-      __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);                                          \
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                                          \
-      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                          \
-    }                                                                                             \
-    __builtin_amdgcn_sched_barrier(0);                                                            \
     if ((G) == 3) GM_SB_EPILOGUE();                                                               \
     __syncthreads();                                                                              \
   } while (0)
@@ -355,25 +358,48 @@ __global__ __launch_bounds__(512) void ogm_gemm_q4k_kernel(GemmParams p) {
     }                                                                                             \
   } while (0)
 
-  GM_LOAD_STAGE(0u, 0u, 0);
-  GM_LOAD_STAGE(0u, 1u, 1);
-  GM_LOAD_STAGE(0u, 2u, 2);
-  GM_STORE_STAGE(0u, 0u, 0);
+  if (producer) {   // while the multiplying waves run pass 1
+    GM_LOAD_STAGE(0u, 0u, 0);
+    GM_LOAD_STAGE(0u, 1u, 1);
+    GM_STORE_STAGE(0u, 0u, 0);
+  }
   __syncthreads();
 
   const uint32_t ra = 64u * wr + l32, rbk = 32u * wt_ + l32;
+  if (producer) {
+    // the set of stage n = 4 s + g is n mod 3, so three super-blocks make one period
+#define GM_PRODUCE_SB(K0, K1, K2)                                                                 \
+  do {                                                                                            \
+    GM_PRODUCE(0, K2, K1);   /* loads stage 4s+2, parks stage 4s+1 */                             \
+    GM_PRODUCE(1, K0, K2);                                                                        \
+    GM_PRODUCE(2, K1, K0);                                                                        \
+    GM_PRODUCE(3, K2, K1);                                                                        \
+    s++;                                                                                          \
+  } while (0)
+    uint32_t s = 0;
+    while (s < p.nsb) {
+      GM_PRODUCE_SB(0, 1, 2);
+      if (s >= p.nsb) break;
+      GM_PRODUCE_SB(1, 2, 0);
+      if (s >= p.nsb) break;
+      GM_PRODUCE_SB(2, 0, 1);
+    }
+#undef GM_PRODUCE_SB
+    return;
+  }
 #pragma unroll 1
   for (uint32_t s = 0; s < p.nsb; s++) {
     float16v c0, c1;
     float adv;
-    GM_STAGE(0, 3, 1);   // loads stage 4s+3 into set 3, parks stage 4s+1 from set 1
-    GM_STAGE(1, 0, 2);
-    GM_STAGE(2, 1, 3);
-    GM_STAGE(3, 2, 0);
+    GM_CONSUME(0);
+    GM_CONSUME(1);
+    GM_CONSUME(2);
+    GM_CONSUME(3);
   }
 #undef GM_LOAD_STAGE
 #undef GM_STORE_STAGE
-#undef GM_STAGE
+#undef GM_PRODUCE
+#undef GM_CONSUME
 #undef GM_SB_EPILOGUE
 
   // ---------------- store: a lane holds one token column and its rows in runs of four
@@ -626,7 +652,7 @@ __global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) {
 static const uint32_t G6_LDS_BYTES = 6 * GM_STAGE_HALFS * 2 + 2 * 128 * 4;
 
 static const uint32_t GM_LDS_BYTES = 4 * GM_STAGE_HALFS * 2 + 2 * 128 * 16 * 2 + 128 * 4;
-static const uint32_t GM_STAGING_BYTES = 4 * GM_STAGE_HALFS * 2;
+static const uint32_t GM_LDS_MAX = 160 * 1024;   // LDS of a CU
 
 size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens) {
   // f16 activations, then the (bh, bl) pairs: 16 f16 per (token, super-block)
@@ -635,8 +661,8 @@ size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens) {
 
 bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
   if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K) || in_dim == 0 || in_dim % 256u != 0) return false;
-  // Q4_K's pass 1 keeps one f32 per (row, super-block) of the workgroup in the staging area of LDS
-  if (ggml_type == OGM_Q4_K && (size_t)(in_dim / 256u) * 512u > GM_STAGING_BYTES) return false;
+  // Q4_K's pass 1 keeps one f32 per (row, super-block) of the workgroup in LDS
+  if (ggml_type == OGM_Q4_K && GM_LDS_BYTES + (size_t)(in_dim / 256u) * 512u > GM_LDS_MAX) return false;
   // the kernels address weights and activations with 32-bit byte offsets
   const uint64_t lim = 0xFFFFFFFFull;
   const uint64_t block = ggml_type == OGM_Q4_K ? 144u : 210u;
@@ -693,10 +719,11 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   p.c_shift = c_shift;
   p.r_shift = 6 - c_shift;
   p.nct = tl.nct;
+  const uint32_t lds4 = GM_LDS_BYTES + nsb * 512u;   // + pass 1's table of dmin
   e = hipFuncSetAttribute((const void *)ogm_gemm_q4k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                          (int)GM_LDS_BYTES);
+                          (int)GM_LDS_MAX);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(ogm_gemm_q4k_kernel, grid, dim3(512), GM_LDS_BYTES, stream, p);
+  hipLaunchKernelGGL(ogm_gemm_q4k_kernel, grid, dim3(1024), lds4, stream, p);
   if (kernel_name) *kernel_name = "ogm_gemm_q4k_kernel";
   return hipGetLastError();
 }

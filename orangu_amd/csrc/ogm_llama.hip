@@ -27,21 +27,25 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
                                                               OgmActDev act) {
   __shared__ float red[16];
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, n_wave = blockDim.x >> 6;
-  float4 v[4];
+  float4 v[4], wv[4];
   float ss = 0.0f;
+  // every load first (x, the residual delta and the norm weights share one trip to memory)
 #pragma unroll
   for (int k = 0; k < 4; k++) {
     const uint32_t e0 = (wave + k * n_wave) * 256u + 4u * lane;
     v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    wv[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
     if (e0 < n) {
       v[k] = *(const float4 *)(x + e0);
-      if (delta) {
-        const float4 d = *(const float4 *)(delta + e0);
-        v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
-        *(float4 *)(x + e0) = v[k];
-      }
-      ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+      wv[k] = *(const float4 *)(weight + e0);
+      if (delta) d = *(const float4 *)(delta + e0);
     }
+    if (e0 < n && delta) {
+      v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
+      *(float4 *)(x + e0) = v[k];
+    }
+    ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
   }
 #pragma unroll
   for (int m = 1; m < 64; m <<= 1) ss += __shfl_xor(ss, m, 64);
@@ -57,9 +61,8 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
     const bool active = e0 < n;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     if (active) {
-      const float4 w = *(const float4 *)(weight + e0);
-      o.x = v[k].x * scale * w.x; o.y = v[k].y * scale * w.y;
-      o.z = v[k].z * scale * w.z; o.w = v[k].w * scale * w.w;
+      o.x = v[k].x * scale * wv[k].x; o.y = v[k].y * scale * wv[k].y;
+      o.z = v[k].z * scale * wv[k].z; o.w = v[k].w * scale * wv[k].w;
       if (normed) *(float4 *)(normed + e0) = o;
     }
     if ((wave + k * n_wave) * 256u < n)  // wave-uniform: the run exists
