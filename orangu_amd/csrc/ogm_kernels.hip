@@ -94,6 +94,7 @@ struct FmtQ4K {
   static constexpr int ACT_GROUP = 256;
   static constexpr bool HAS_MIN = true;
   static constexpr int MAX_THREADS = 512;   // launch bound: leaves 256 VGPRs to a lane
+  static constexpr bool HAS_UNPACK = false;
   struct Regs {
     uint4 p[PIECES];
   };
@@ -247,6 +248,56 @@ struct FmtQ6K {
       }
     }
   }
+  // For several tokens per launch: the block's 6-bit values (still carrying the +32) unpacked
+  // once, four per word, group g of 16 at v[4g .. 4g+3]; every token then only runs the dots.
+  static constexpr bool HAS_UNPACK = true;
+  struct Unpacked {
+    uint32_t v[64];
+  };
+  __device__ static __forceinline__ void unpack(const Regs &r, Unpacked &u) {
+    const uint32_t m4 = 0x0F0F0F0Fu, m2 = 0x30303030u;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+      for (int rr = 0; rr < 4; rr++) {
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+          const int g = 2 * (4 * h + rr) + k;
+          const uint4 ql = r.p[4 * h + 2 * (rr & 1) + k];
+          const uint4 qh = r.p[8 + 2 * h + k];
+          const uint32_t qlw[4] = {ql.x, ql.y, ql.z, ql.w}, qhw[4] = {qh.x, qh.y, qh.z, qh.w};
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            const uint32_t nib = (rr < 2 ? qlw[w] : (qlw[w] >> 4)) & m4;
+            // ((qh >> 2 rr) & 3) << 4
+            const uint32_t hi = rr == 0 ? (qhw[w] << 4) : rr == 1 ? (qhw[w] << 2) : rr == 2 ? qhw[w] : (qhw[w] >> 2);
+            u.v[4 * g + w] = nib | (hi & m2);
+          }
+        }
+      }
+    }
+  }
+  template <int UPR>
+  __device__ static __forceinline__ void sums_unpacked(const Unpacked &u, const Regs &r, const ActLds &a,
+                                                       uint32_t col, int &isum, int &imin) {
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;
+    const uint4 s_lo = a.aux[col], s_hi = a.aux[st + col];  // sum16 of groups 0..7, 8..15
+    const uint32_t sw[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+    const uint32_t scw[4] = {r.p[12].x, r.p[12].y, r.p[12].z, r.p[12].w};
+    isum = 0;
+    imin = 0;
+#pragma unroll
+    for (int g = 0; g < 16; g++) {
+      const uint4 x = a.xq[g * st + col];
+      int dot = 0;
+      dot = dot4(u.v[4 * g + 0], x.x, dot);
+      dot = dot4(u.v[4 * g + 1], x.y, dot);
+      dot = dot4(u.v[4 * g + 2], x.z, dot);
+      dot = dot4(u.v[4 * g + 3], x.w, dot);
+      const int s16 = (g & 1) ? hi16(sw[g >> 1]) : lo16(sw[g >> 1]);
+      isum += sbyte_of(scw[g >> 2], g & 3) * (dot - 32 * s16);
+    }
+  }
   // GEMV: total += act.d[s] * d * isum                                       (vecdot.rs:3238)
   __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int) {
     return ad * f16_bits_to_f32(r.d16) * (float)isum;
@@ -268,6 +319,7 @@ struct FmtQ80 {
   static constexpr int ACT_GROUP = 32;
   static constexpr bool HAS_MIN = false;
   static constexpr int MAX_THREADS = 1024;
+  static constexpr bool HAS_UNPACK = false;
   struct Regs {
     uint4 p[PIECES];
     uint32_t d16;
@@ -398,10 +450,17 @@ __device__ __forceinline__ float ordered_sum(float acc, const float *p, uint32_t
   return acc;
 }
 
+struct NoUnpack {};
+template <class F, bool WANT, bool HAS = F::HAS_UNPACK>
+struct UnpackedOf { typedef NoUnpack type; };
+template <class F>
+struct UnpackedOf<F, true, true> { typedef typename F::Unpacked type; };
+
 // UPR: blocks per row when known at compile time (the hot shapes), 0 = read it from the params.
 // QUANT: the workgroup quantizes the f32 activations p.x itself (one token) instead of reading
 // the quantizer kernel's output.
-template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP, bool QUANT>
+// UNPACK: several tokens and a format whose block is expensive to unpack: unpack once per tile.
+template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP, bool QUANT, bool UNPACK = false>
 __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t tid = threadIdx.x, nthr = blockDim.x;
@@ -548,6 +607,10 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
   for (; it < n_items; it += n_wave) {
     const uint32_t rbk = it / nct, ct = it - rbk * nct;
     const uint32_t col = ct * C + c_local;  // block index within the row
+    // many tokens: unpack the block once where that is the expensive part (Q6_K; measured at
+    // 4096 -> 128256: 159 us against 182 us at 8 tokens, but 112 us against 97 us at 4)
+    [[maybe_unused]] typename UnpackedOf<F, UNPACK>::type unp;
+    if constexpr (UNPACK) F::unpack(cur, unp);
     for (uint32_t t = 0; t < T; t++) {
       ActLds a;
       a.xq = l_xq + (size_t)t * xch;
@@ -555,7 +618,8 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
       a.d = l_d + (size_t)t * n_scale;
       a.upr = upr;
       int isum, imin;
-      F::template sums<UPR>(cur, a, col, isum, imin);
+      if constexpr (UNPACK) F::template sums_unpacked<UPR>(unp, cur, a, col, isum, imin);
+      else F::template sums<UPR>(cur, a, col, isum, imin);
       const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
       const size_t slot = (size_t)(t * K + rbk) * term_stride + col * R + r_local;
       if (GEMM_ORDER) {
@@ -693,6 +757,8 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   } else if (a.n_tokens == 1 && !GEMM_ORDER) {
     if (a.x_f32) launch_single<F, true>(p, g, b, lds, stream);
     else launch_single<F, false>(p, g, b, lds, stream);
+  } else if (F::HAS_UNPACK && a.n_tokens >= 6) {
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false, F::HAS_UNPACK>), g, b, lds, stream, p);
   } else {
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false>), g, b, lds, stream, p);
   }
