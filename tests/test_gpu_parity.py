@@ -569,3 +569,36 @@ def test_row_blocks_per_workgroup_do_not_change_a_bit(be, t, in_dim):
         be.set_tuning("gemv_fuse_quant", -1)
         for b in [xd] + yds:
             b.free()
+
+
+def test_concurrent_callers_share_one_backend(be):
+    """The scheduler calls a backend from one blocking-pool thread per slot (scheduler.rs:16-22):
+    calls from several threads must serialise inside the library and each get their own result."""
+    import threading
+    in_dim = 1024
+    ws = [(t, synth_weights(t, in_dim, od, seed=200 + i), od) for i, (t, od) in
+          enumerate(((Q4_K, 300), (Q6_K, 130), (Q8_0, 257), (Q4_K, 64)))]
+    mats = [qm(raw, t, in_dim, od) for t, raw, od in ws]
+    xs = [synth_x(T, in_dim, seed=300 + i) for i, T in enumerate((1, 3, 12, 40))]
+    want = {(i, j): oracle.matmul(ws[i][0], ws[i][1], in_dim, ws[i][2], xs[j], xs[j].shape[0]).reshape(-1)
+            for i in range(4) for j in range(4)}
+    for m in mats:
+        be.upload(m)
+    errors = []
+
+    def worker(k):
+        try:
+            for rep in range(6):
+                i, j = (k + rep) % 4, (k * 3 + rep) % 4
+                got = be.matmul(xs[j].reshape(-1), xs[j].shape[0], mats[i])
+                if not np.array_equal(got.view(np.uint32), want[(i, j)].view(np.uint32)):
+                    errors.append((k, rep, i, j))
+        except Exception as e:  # noqa: BLE001
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(8)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
