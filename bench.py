@@ -122,7 +122,7 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     layers = [{**{k: (k, l) for k in shapes}, "attn_norm": norms[2 * l], "ffn_norm": norms[2 * l + 1]}
               for l in range(n_layer)]
     dec = LlamaDecoder(be, n_embd=n_embd, n_head=n_head, n_head_kv=n_kv, head_dim=hd, n_ff=n_ff, n_vocab=n_vocab,
-                       max_ctx=ctx + warmup + steps + 2, rms_eps=1e-5, rope_freq_base=500000.0, layers=layers,
+                       max_ctx=ctx + warmup + 2 * steps + 2, rms_eps=1e-5, rope_freq_base=500000.0, layers=layers,
                        output_norm=norms[-1], output="output", upload=up)
     kvs = []
     for l in range(n_layer):
@@ -148,11 +148,18 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     stream.synchronize()
     hiprt.device_synchronize()
     dt = (time.perf_counter() - t0) / steps
+    # the closed loop: each token's embedding row (tied to the output matrix) is read on the device
+    # from the previous step's argmax; one synchronization after `steps` tokens
+    t0 = time.perf_counter()
+    toks = dec.generate(up("output"), 1, pos, steps)
+    dt_gen = (time.perf_counter() - t0) / steps
+    pos += steps
     weights = n_layer * sum(o * (i // 256) * (144 if t == Q4_K else 210) for t, i, o in shapes.values()) \
         + n_vocab * (n_embd // 256) * 210
     kv_bytes = 2 * n_layer * ctx * n_kv * hd * 2
     res = {"workload": f"configs[4]: 8B-shaped Llama Q4_K_M-like, batch-1 greedy decode at context {ctx}",
            "tok_per_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4),
+           "generate_tok_per_s": round(1.0 / dt_gen, 1), "generated": [int(t) for t in toks[:4]],
            "bytes_per_token": weights + kv_bytes,
            "GBps": round((weights + kv_bytes) / dt / 1e9, 1),
            "frac_of_hbm_peak": round((weights + kv_bytes) / dt / 1e9 / HBM_PEAK_GBS, 4)}

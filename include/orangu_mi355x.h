@@ -219,6 +219,19 @@ int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos, f
 /* The same with device pointers, enqueued on `stream` (null = the context's) without waiting. */
 int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_t pos, float *logits_dev,
                          uint32_t *argmax_dev, void *stream);
+/* Rows row0 .. row0+n_rows of an uploaded matrix as f32 ([n_rows][in_dim], host memory), from the
+ * device copy: dequantize_q8_0 / _q4_k / _q6_k (engine/quant.rs:639-649, 666-697, 746-787), bit for
+ * bit.  This is the embedding lookup of run_layers (llama.rs:609-614). */
+int ogm_dequant_rows(ogm_ctx *ctx, const ogm_weight *w, uint32_t row0, uint32_t n_rows, float *out);
+
+/* Greedy generation without leaving the device: starting from `first_token` at position pos0,
+ * n_tokens times { embedding row of the current token from tok_embd (an uploaded [n_embd ->
+ * n_vocab] matrix); decode step; argmax (sampling.rs:336-343) becomes the next token }.
+ * tokens_out receives the n_tokens generated ids, last_logits (nullable) the final step's logits.
+ * One synchronization at the end. */
+int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *tok_embd, uint32_t first_token,
+                       uint32_t pos0, uint32_t n_tokens, uint32_t *tokens_out, float *last_logits);
+
 /* The last decode's final hidden state, before the output norm ([n_embd] host f32; what
  * run_layers returns), for parity checks. */
 int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out);

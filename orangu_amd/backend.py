@@ -273,6 +273,13 @@ class Mi355xBackend:
         """Releases a device copy made by upload_raw (cached uploads live as long as the backend)."""
         self._check(self._lib.ogm_weight_free(self._ctx, w_handle), "ogm_weight_free")
 
+    def dequant_rows(self, w: QuantMatrix, row0: int, n_rows: int) -> np.ndarray:
+        """Rows of an uploaded matrix as f32, from the device copy (quant.rs dequantize_*)."""
+        out = np.empty((n_rows, w.in_dim), np.float32)
+        self._check(self._lib.ogm_dequant_rows(self._ctx, self.upload(w), row0, n_rows, out.ctypes.data),
+                    "ogm_dequant_rows")
+        return out
+
     def set_tuning(self, key: str, value: int):
         self._check(self._lib.ogm_set_tuning(self._ctx, key.encode(), value), "ogm_set_tuning")
 
@@ -330,6 +337,16 @@ class LlamaDecoder:
     def decode_dev(self, x_ptr: int, pos: int, logits_ptr: int = 0, argmax_ptr: int = 0, stream: int = 0):
         self._be._check(self._be._lib.ogm_llama_decode_dev(self._be._ctx, self._h, x_ptr, pos, logits_ptr or None,
                                                            argmax_ptr or None, stream or None), "ogm_llama_decode_dev")
+
+    def generate(self, tok_embd, first_token: int, pos0: int, n_tokens: int, want_logits: bool = False):
+        """Greedy generation on the device; tok_embd is a QuantMatrix [n_embd -> n_vocab] or a handle."""
+        h = tok_embd if isinstance(tok_embd, int) else self._be.upload(tok_embd)
+        toks = np.empty(n_tokens, np.uint32)
+        logits = np.empty(self.n_vocab, np.float32) if want_logits else None
+        self._be._check(self._be._lib.ogm_llama_generate(self._be._ctx, self._h, h, first_token, pos0, n_tokens,
+                                                         toks.ctypes.data, logits.ctypes.data if want_logits else None),
+                        "ogm_llama_generate")
+        return (toks, logits) if want_logits else toks
 
     def hidden(self) -> np.ndarray:
         out = np.empty(self.n_embd, np.float32)

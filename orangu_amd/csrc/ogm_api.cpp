@@ -902,7 +902,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   if (pos >= c.max_ctx) return fail(ctx, OGM_ERR_INVALID, "position beyond the KV cache");
   const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
   const float scale = 1.0f / sqrtf((float)c.head_dim);
-  HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
+  if (x_dev != m->x) HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
   const float *delta = nullptr;  // what the next norm adds to x first: the last block's output
   for (uint32_t l = 0; l < c.n_layer; l++) {
     const ogm_llama_layer &L = m->layers[l];
@@ -992,5 +992,53 @@ extern "C" int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out) 
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   // the output norm added the last block's output to x in place before normalising
   HIPCHK(ctx, hipMemcpy(x_out, m->x, (size_t)m->cfg.n_embd * 4, hipMemcpyDeviceToHost));
+  return OGM_OK;
+}
+
+extern "C" int ogm_dequant_rows(ogm_ctx *ctx, const ogm_weight *w, uint32_t row0, uint32_t n_rows, float *out) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!w || !out) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  if ((uint64_t)row0 + n_rows > w->out_dim) return fail(ctx, OGM_ERR_INVALID, "rows outside the matrix");
+  if (n_rows == 0) return OGM_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  const size_t bytes = (size_t)n_rows * w->in_dim * 4;
+  int rc = ensure_dev(ctx, ctx->y, bytes);
+  if (rc != OGM_OK) return rc;
+  for (uint32_t r = 0; r < n_rows; r++)
+    HIPCHK(ctx, ogm_launch_dequant_row(w->dev, w->ggml_type, w->in_dim, w->out_dim, row0 + r, nullptr,
+                                       (float *)ctx->y.p + (size_t)r * w->in_dim, ctx->stream));
+  HIPCHK(ctx, hipMemcpyAsync(out, ctx->y.p, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return OGM_OK;
+}
+
+extern "C" int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *tok_embd, uint32_t first_token,
+                                  uint32_t pos0, uint32_t n_tokens, uint32_t *tokens_out, float *last_logits) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !tok_embd || !tokens_out) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  const ogm_llama_config &c = m->cfg;
+  if (tok_embd->in_dim != c.n_embd) return fail(ctx, OGM_ERR_INVALID, "embedding table row length != n_embd");
+  if (first_token >= tok_embd->out_dim) return fail(ctx, OGM_ERR_INVALID, "token id is out of vocab range");
+  if ((uint64_t)pos0 + n_tokens > c.max_ctx) return fail(ctx, OGM_ERR_INVALID, "positions beyond the KV cache");
+  if (n_tokens == 0) return OGM_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  // token ids live on the device: slot 0 is the prompt's last token, slot i + 1 the i-th generated
+  int rc = ensure_dev(ctx, ctx->isum, ((size_t)n_tokens + 1) * 4);
+  if (rc != OGM_OK) return rc;
+  uint32_t *toks = (uint32_t *)ctx->isum.p;
+  HIPCHK(ctx, hipMemcpyAsync(toks, &first_token, 4, hipMemcpyHostToDevice, ctx->stream));
+  for (uint32_t i = 0; i < n_tokens; i++) {
+    // the embedding row goes straight into the residual stream
+    HIPCHK(ctx, ogm_launch_dequant_row(tok_embd->dev, tok_embd->ggml_type, tok_embd->in_dim, tok_embd->out_dim, 0,
+                                       toks + i, m->x, ctx->stream));
+    rc = llama_decode_enqueue(ctx, m, m->x, pos0 + i, nullptr, toks + i + 1, ctx->stream);
+    if (rc != OGM_OK) return rc;
+  }
+  HIPCHK(ctx, hipMemcpyAsync(tokens_out, toks + 1, (size_t)n_tokens * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (last_logits)
+    HIPCHK(ctx, hipMemcpyAsync(last_logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   return OGM_OK;
 }

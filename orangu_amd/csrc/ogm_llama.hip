@@ -454,3 +454,78 @@ hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStrea
                      (__half *)dst, n);
   return hipGetLastError();
 }
+
+// ------------------------------------------------------------------------------------------
+// one row of a quantized matrix as f32: the embedding lookup (LlamaModel::run_layers,
+// llama.rs:609-614, over dequantize_q8_0 / _q4_k / _q6_k, quant.rs:639-649, 666-697, 746-787),
+// reading the tile-planar device copy.  One thread per element; the f32 expressions are the
+// reference's, so the values are bit-identical (built without FMA contraction).
+
+#include "ogm_layout.h"
+
+__device__ __forceinline__ float dq_f16(const uint8_t *p) {
+  return __half2float(__ushort_as_half((unsigned short)(p[0] | (p[1] << 8))));
+}
+
+__global__ __launch_bounds__(256) void ogm_dequant_row_kernel(const uint8_t *__restrict__ wt, uint32_t ggml_type,
+                                                              uint32_t in_dim, uint32_t out_dim, uint32_t row,
+                                                              const uint32_t *__restrict__ row_dev,
+                                                              float *__restrict__ out) {
+  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= in_dim) return;
+  if (row_dev) row = *row_dev;
+  if (row >= out_dim) row = out_dim - 1u;   // a token id beyond the table reads its last row
+  OgmLayout l;
+  ogm_layout_for(ggml_type, &l);
+  const OgmTiling t = ogm_tiling_for(in_dim / l.block_elems, out_dim);
+  const uint32_t s = e / l.block_elems, j = e - s * l.block_elems;
+  size_t tile;
+  uint32_t lane;
+  ogm_unit_place(t, row, s, &tile, &lane);
+  const uint8_t *tb = wt + tile * l.tile_bytes;
+  // byte `o` of the block's piece area (the raw block minus its tail)
+  auto piece_byte = [&](uint32_t o) -> uint32_t { return tb[(o >> 4) * 1024u + lane * 16u + (o & 15u)]; };
+  float v;
+  if (ggml_type == OGM_Q8_0) {
+    const float d = dq_f16(tb + l.pieces * 1024u + lane * 2u);
+    v = (float)(int8_t)piece_byte(j) * d;
+  } else if (ggml_type == OGM_Q4_K) {
+    const uint8_t *hd = tb + lane * 16u;   // piece 0: d, dmin, scales
+    const float d = dq_f16(hd), dmin = dq_f16(hd + 2);
+    const uint32_t g4 = j >> 6, hi = (j >> 5) & 1u, li = j & 31u;
+    const uint32_t is = 2u * g4 + hi;      // sub-block
+    // get_scale_min_k4 (quant.rs:653-662)
+    const uint8_t *q = hd + 4;
+    uint32_t sc, m;
+    if (is < 4) {
+      sc = q[is] & 63u;
+      m = q[is + 4] & 63u;
+    } else {
+      sc = (q[is + 4] & 0xFu) | ((q[is - 4] >> 6) << 4);
+      m = (q[is + 4] >> 4) | ((q[is] >> 6) << 4);
+    }
+    const uint32_t byte = piece_byte(16u + 32u * g4 + li);
+    const uint32_t nib = hi ? (byte >> 4) : (byte & 0xFu);
+    const float d1 = d * (float)sc, mm = dmin * (float)m;
+    v = d1 * (float)nib - mm;
+  } else {  // Q6_K
+    const float d = dq_f16(tb + l.pieces * 1024u + lane * 2u);
+    const uint32_t h = j >> 7, jj = j & 127u, qd = jj >> 5, li = jj & 31u;
+    const uint32_t qlb = piece_byte(64u * h + li + ((qd & 1u) ? 32u : 0u));
+    const uint32_t qhb = piece_byte(128u + 32u * h + li);
+    const int sc = (int)(int8_t)piece_byte(192u + 8u * h + (li >> 4) + 2u * qd);
+    const int qv = (int)(((qd < 2 ? qlb : (qlb >> 4)) & 0xFu) | (((qhb >> (2u * qd)) & 3u) << 4)) - 32;
+    v = d * (float)sc * (float)qv;
+  }
+  out[e] = v;
+}
+
+hipError_t ogm_launch_dequant_row(const uint8_t *wt, uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim,
+                                  uint32_t row, const uint32_t *row_dev, float *out, hipStream_t stream) {
+  OgmLayout l;
+  if (!ogm_layout_for(ggml_type, &l) || in_dim == 0 || in_dim % l.block_elems != 0 || out_dim == 0)
+    return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ogm_dequant_row_kernel, dim3((in_dim + 255u) / 256u), dim3(256), 0, stream, wt, ggml_type,
+                     in_dim, out_dim, row, row_dev, out);
+  return hipGetLastError();
+}

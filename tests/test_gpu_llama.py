@@ -162,3 +162,66 @@ def test_matrices_uploaded_from_a_gguf_file_multiply_like_direct_uploads(be, tmp
         xd.free()
         yd.free()
     g.close()
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim", [
+    (Q8_0, 64, 5), (Q8_0, 4096, 70),
+    (Q4_K, 256, 3), (Q4_K, 1024, 130), (Q4_K, 4096, 67),
+    (Q6_K, 256, 1), (Q6_K, 768, 65), (Q6_K, 4096, 129),
+])
+def test_dequant_rows_bits(be, t, in_dim, out_dim):
+    """Rows of the device copy equal dequantize_q8_0 / _q4_k / _q6_k (quant.rs:639-787) bit for bit."""
+    import oracle
+    from orangu_amd import OgmError, QuantMatrix
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + t)
+    want = oracle.dequantize(t, raw, in_dim * out_dim).reshape(out_dim, in_dim)
+    w = QuantMatrix(raw, t, in_dim, out_dim)
+    got = be.dequant_rows(w, 0, out_dim)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    if out_dim > 2:
+        got = be.dequant_rows(w, out_dim - 2, 2)
+        assert np.array_equal(got.view(np.uint32), want[-2:].view(np.uint32))
+    with pytest.raises(OgmError):
+        be.dequant_rows(w, out_dim, 1)
+
+
+@pytest.mark.parametrize("embd_t", [Q4_K, Q6_K, Q8_0])
+def test_generate_matches_stepwise(be, embd_t):
+    """Greedy generation on the device = the oracle's loop: embedding row of the token
+    (llama.rs:609-614), decode step, last-of-equal argmax (sampling.rs:336-343)."""
+    import oracle
+    from orangu_amd import OgmError, QuantMatrix
+    n_embd, n_vocab, max_ctx = 256, 320, 16
+    kw = dict(n_embd=n_embd, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=n_vocab, n_layer=2,
+              types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=max_ctx, seed=11)
+    ref, dev, _ = build(be, **kw)
+    _, dev2, _ = build(be, **kw)
+    embd_raw = synth_weights(embd_t, n_embd, n_vocab, seed=4242 + embd_t)
+    table = oracle.dequantize(embd_t, embd_raw, n_embd * n_vocab).reshape(n_vocab, n_embd)
+    embd = QuantMatrix(embd_raw, embd_t, n_embd, n_vocab)
+    first, steps = 17, 6
+    try:
+        tok, want, logits, sure = first, [], None, True
+        for pos in range(steps):
+            logits, _ = R.decode_step(ref, table[tok], pos)
+            top = np.sort(logits)[-2:]
+            sure = sure and top[1] - top[0] > TOL * np.abs(logits).max()
+            tok = R.argmax(logits)
+            want.append(tok)
+        assert sure, "pick another seed: the oracle's two best logits are within the tolerance"
+        got, got_logits = dev.generate(embd, first, 0, steps, want_logits=True)
+        say("generated", got.tolist(), "want", want)
+        assert got.tolist() == want
+        close(got_logits, logits, "logits of the last generated step")
+        # the same through single steps fed from the host
+        tok = first
+        for pos in range(steps):
+            _, tok = dev2.decode(table[tok], pos)
+            assert tok == want[pos]
+        with pytest.raises(OgmError):
+            dev.generate(embd, n_vocab, 0, 1)
+        with pytest.raises(OgmError):
+            dev.generate(embd, 0, max_ctx - 1, 2)
+    finally:
+        dev.close()
+        dev2.close()
