@@ -729,6 +729,8 @@ struct ogm_llama {
   // device memory
   float *norms = nullptr;     // [n_layer][2][n_embd] then output_norm [n_embd]
   float *freq = nullptr;      // [rope_dim / 2]
+  float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
+  uint32_t *attn_tickets = nullptr;   // [n_head_kv], zero between launches
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
   void *v_cache = nullptr;
   float *x = nullptr;         // hidden state [n_embd]
@@ -798,6 +800,8 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   auto A = [&](void **p, size_t b) { if (rc == OGM_OK) rc = llama_alloc(ctx, m, p, b); };
   A((void **)&m->norms, ((size_t)c.n_layer * 2 + 1) * c.n_embd * 4);
   A((void **)&m->freq, (size_t)(c.rope_dim / 2 + 1) * 4);
+  A((void **)&m->rope_cs, (size_t)(c.rope_dim / 2 + 1) * 8);
+  A((void **)&m->attn_tickets, (size_t)c.n_head_kv * 4);
   A(&m->k_cache, cache_bytes);
   A(&m->v_cache, cache_bytes);
   A((void **)&m->x, (size_t)c.n_embd * 4);
@@ -830,6 +834,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
     freq[i] = powf(c.rope_freq_base, -2.0f * (float)i / (float)c.rope_dim);
   hipError_t e = hipMemcpy(m->norms, host.data(), host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, (size_t)c.n_head_kv * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
   if (e != hipSuccess) {
@@ -903,6 +908,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
   const float scale = 1.0f / sqrtf((float)c.head_dim);
   if (x_dev != m->x) HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
+  HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos, c.rope_dim, m->rope_cs, s));
   const float *delta = nullptr;  // what the next norm adds to x first: the last block's output
   for (uint32_t l = 0; l < c.n_layer; l++) {
     const ogm_llama_layer &L = m->layers[l];
@@ -920,12 +926,10 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     float *y3[3] = {m->q, m->k, m->v};
     int rc = llama_matmul(ctx, w3, y3, 3, s);
     if (rc != OGM_OK) return rc;
-    HIPCHK(ctx, ogm_launch_rope_kv(m->q, m->k, m->v, m->freq, pos, c.n_head, c.n_head_kv, c.head_dim,
-                                   c.rope_dim, kc, vc, s));
     const int mode_o = act_mode_for(L.wo->ggml_type);
-    HIPCHK(ctx, ogm_launch_attn_decode(m->q, kc, vc, pos, m->max_splits, c.n_head, c.n_head_kv, c.head_dim,
-                                       scale, m->part_o, m->part_ml, mode_o, nullptr,
-                                       act_view(ctx, qd, mode_o, 0), s));
+    HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, m->rope_cs, c.rope_dim, kc, vc, pos, m->max_splits,
+                                       c.n_head, c.n_head_kv, c.head_dim, scale, m->part_o, m->part_ml,
+                                       m->attn_tickets, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s));
     const ogm_weight *w1[1] = {L.wo};
     float *y1[1] = {m->proj};
     if ((rc = llama_matmul(ctx, w1, y1, 1, s)) != OGM_OK) return rc;
@@ -974,9 +978,9 @@ extern "C" int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint
   std::lock_guard<std::mutex> lock(ctx->mu);
   HIPCHK(ctx, hipSetDevice(ctx->device));
   const ogm_llama_config &c = m->cfg;
-  // gate is free until the first FFN: the embedding row is staged there
-  HIPCHK(ctx, hipMemcpyAsync(m->gate, x, (size_t)c.n_embd * 4, hipMemcpyHostToDevice, ctx->stream));
-  int rc = llama_decode_enqueue(ctx, m, m->gate, pos, nullptr, m->amax_out, ctx->stream);
+  // the embedding row goes straight into the residual stream
+  HIPCHK(ctx, hipMemcpyAsync(m->x, x, (size_t)c.n_embd * 4, hipMemcpyHostToDevice, ctx->stream));
+  int rc = llama_decode_enqueue(ctx, m, m->x, pos, nullptr, m->amax_out, ctx->stream);
   if (rc != OGM_OK) return rc;
   if (logits) HIPCHK(ctx, hipMemcpyAsync(logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   if (argmax) HIPCHK(ctx, hipMemcpyAsync(argmax, m->amax_out, 4, hipMemcpyDeviceToHost, ctx->stream));

@@ -16,21 +16,25 @@
 hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const float *weight, uint32_t n,
                                  float eps, float *normed, OgmActDev act, hipStream_t stream);
 
-// NORM-paired RoPE (pairs 2i, 2i+1; tensor.rs:1115-1177 with freq_scale 1 and no YaRN) of q
-// (in place) and k at position `pos`, then k and v into the f16 cache rows of that position.
-// `freq` holds rope_dim / 2 frequencies.
-hipError_t ogm_launch_rope_kv(float *q, const float *k, const float *v, const float *freq, uint32_t pos,
-                              uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim, uint32_t rope_dim,
-                              void *k_cache_layer, void *v_cache_layer, hipStream_t stream);
+// cos / sin of pos * freq[p] for the rope_dim / 2 rotated pairs, as float2 (cos, sin): once per
+// token, every layer rotates by the same angles (tensor.rs:1147-1160, freq_scale 1, no YaRN).
+hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t rope_dim, void *cs, hipStream_t stream);
 
-// Causal attention of one token over cache positions 0..pos (engine/attention.rs:426-549):
-// scores = (q . k) * scale, softmax over positions, out = sum w * v; grouped-query heads share
-// their K/V head.  Split over chunks of OGM_ATTN_CHUNK positions and combined; the combined
-// output is quantized for the next matmul in `mode` and stored as f32 when attn_out is not null.
-// part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch.
-hipError_t ogm_launch_attn_decode(const float *q, const void *k_cache_layer, const void *v_cache_layer,
-                                  uint32_t pos, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
-                                  uint32_t head_dim, float scale, float *part_o, float *part_ml, int mode,
+// One token's attention, from the q / k / v the projections left (f32) to the quantized input of
+// the output projection:
+//   * NORM-paired RoPE (pairs 2i, 2i+1; tensor.rs:1115-1177) of q and k with the table `cs`,
+//     k and v rounded to f16 into the cache rows of position `pos`;
+//   * causal attention over cache positions 0..pos (engine/attention.rs:426-549): scores =
+//     (q . k) * scale, softmax over positions, out = sum w * v; grouped-query heads share their
+//     K/V head.  Split over chunks of OGM_ATTN_CHUNK positions and merged;
+//   * the merged output quantized for the next matmul in `mode`, and stored as f32 when attn_out
+//     is not null.
+// part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch;
+// counters: n_head_kv words, zero before the first launch (the kernel leaves them zero).
+hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
+                                  uint32_t rope_dim, void *k_cache_layer, void *v_cache_layer, uint32_t pos,
+                                  uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
+                                  float scale, float *part_o, float *part_ml, uint32_t *counters, int mode,
                                   float *attn_out, OgmActDev act, hipStream_t stream);
 
 // h = silu(gate) * up with silu(g) = g / (1 + exp(-g))     (tensor.rs:825-827, arch/mod.rs:1071-1106)

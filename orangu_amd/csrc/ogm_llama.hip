@@ -85,158 +85,291 @@ hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const f
 }
 
 // ------------------------------------------------------------------------------------------
-// RoPE + KV-cache write
+// RoPE table: cos and sin of pos * freq[p] for every rotated pair, once per token (all layers
+// rotate by the same angles)
 
-__global__ __launch_bounds__(256) void ogm_rope_kv_kernel(float *__restrict__ q, const float *__restrict__ k,
-                                                          const float *__restrict__ v,
-                                                          const float *__restrict__ freq, uint32_t pos,
-                                                          uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
-                                                          uint32_t rope_dim, __half *__restrict__ kc,
-                                                          __half *__restrict__ vc) {
-  const uint32_t half_dim = head_dim / 2, rope_half = rope_dim / 2;
-  const uint32_t kv_dim = n_head_kv * head_dim;
-  const uint32_t nq = n_head * half_dim, nk = n_head_kv * half_dim;
-  __half *krow = kc + (size_t)pos * kv_dim, *vrow = vc + (size_t)pos * kv_dim;
-  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < nq + nk; i += gridDim.x * blockDim.x) {
-    const bool is_q = i < nq;
-    const uint32_t j = is_q ? i : i - nq;
-    const uint32_t h = j / half_dim, p = j - h * half_dim;   // pair p of head h: elements 2p, 2p+1
-    const float *src = (is_q ? q : k) + h * head_dim + 2u * p;
-    float a = src[0], b = src[1];
-    if (p < rope_half) {
-      const float theta = (float)pos * freq[p];
-      float sn, cs;
-      sincosf(theta, &sn, &cs);
-      const float ra = a * cs - b * sn, rb = a * sn + b * cs;
-      a = ra;
-      b = rb;
-    }
-    if (is_q) {
-      float *dst = q + h * head_dim + 2u * p;
-      dst[0] = a;
-      dst[1] = b;
-    } else {
-      krow[h * head_dim + 2u * p] = __float2half_rn(a);
-      krow[h * head_dim + 2u * p + 1u] = __float2half_rn(b);
-      vrow[h * head_dim + 2u * p] = __float2half_rn(v[h * head_dim + 2u * p]);
-      vrow[h * head_dim + 2u * p + 1u] = __float2half_rn(v[h * head_dim + 2u * p + 1u]);
-    }
-  }
+__global__ __launch_bounds__(64) void ogm_rope_table_kernel(const float *__restrict__ freq, uint32_t pos,
+                                                            uint32_t rope_half, float2 *__restrict__ cs) {
+  const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= rope_half) return;
+  const float theta = (float)pos * freq[p];
+  float sn, c;
+  sincosf(theta, &sn, &c);
+  cs[p] = make_float2(c, sn);
 }
 
-hipError_t ogm_launch_rope_kv(float *q, const float *k, const float *v, const float *freq, uint32_t pos,
-                              uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim, uint32_t rope_dim,
-                              void *k_cache_layer, void *v_cache_layer, hipStream_t stream) {
-  if (head_dim % 2u != 0 || rope_dim > head_dim || rope_dim % 2u != 0) return hipErrorInvalidValue;
-  const uint32_t n = (n_head + n_head_kv) * head_dim / 2;
-  hipLaunchKernelGGL(ogm_rope_kv_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, q, k, v, freq, pos,
-                     n_head, n_head_kv, head_dim, rope_dim, (__half *)k_cache_layer, (__half *)v_cache_layer);
+hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t rope_dim, void *cs, hipStream_t stream) {
+  if (rope_dim % 2u != 0) return hipErrorInvalidValue;
+  if (rope_dim == 0) return hipSuccess;
+  hipLaunchKernelGGL(ogm_rope_table_kernel, dim3((rope_dim / 2u + 63u) / 64u), dim3(64), 0, stream, freq, pos,
+                     rope_dim / 2u, (float2 *)cs);
   return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------
-// attention: partial softmax per chunk of positions, then combine (+ quantize)
+// attention of one token: RoPE of q and of the new k, the cache write, a partial softmax per
+// chunk of positions, and (in the workgroup that finishes last) the merge of the chunks with the
+// quantizer of the next matmul
 
+__device__ __forceinline__ float2 rope_pair(float2 ab, float2 cs) {
+  return make_float2(ab.x * cs.x - ab.y * cs.y, ab.x * cs.y + ab.y * cs.x);
+}
 
-// Workgroup (kvh, split): the G query heads of K/V head kvh against positions
-// split * 128 .. + 128.  Every load of the workgroup is requested first (its K rows and its V
-// rows in one trip to memory).  Phase 1: thread t scores position t for every query head; q is
-// uniform (scalar loads).  Phase 2: sixteen threads share a V row (eight dimensions each), eight
-// rows per step, and LDS adds the eight partial sums.
-template <int HD, int G>
-__global__ __launch_bounds__(128) void ogm_attn_partial_kernel(const float *__restrict__ q,
-                                                               const __half *__restrict__ kc,
-                                                               const __half *__restrict__ vc, uint32_t pos,
-                                                               uint32_t max_splits, uint32_t n_head_kv,
-                                                               float scale, float *__restrict__ part_o,
-                                                               float *__restrict__ part_ml) {
-  constexpr int TPR = HD / 8;            // threads per V row
-  constexpr int ROWS = 128 / TPR;        // V rows in flight per step
+// Device-coherent accesses for results one workgroup hands to another inside a kernel: they go
+// through to the level all compute dies share, so no cache write-back or invalidate is needed.
+template <bool COHERENT>
+__device__ __forceinline__ float2 ld_pair(const float *p) {
+  if constexpr (COHERENT) {
+    const uint64_t u = __hip_atomic_load((const uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return make_float2(__uint_as_float((uint32_t)u), __uint_as_float((uint32_t)(u >> 32)));
+  } else {
+    return *(const float2 *)p;
+  }
+}
+template <bool COHERENT>
+__device__ __forceinline__ void st_one(float *p, float v) {
+  if constexpr (COHERENT) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *p = v;
+}
+
+// A partial softmax over some chunks of four neighbouring output elements: running maximum,
+// denominator and weighted sums relative to that maximum.
+struct AttnPart {
+  float m, den;
+  float4 o;
+};
+
+// Merges chunks s_first, s_first + s_step, ... (< n_splits) of the four output elements d .. d + 3
+// of query head h.
+template <bool COHERENT>
+__device__ __forceinline__ AttnPart attn_merge_chunks(const float *part_o, const float *part_ml, uint32_t h,
+                                                      uint32_t d, uint32_t s_first, uint32_t s_step,
+                                                      uint32_t n_splits, uint32_t max_splits, uint32_t head_dim) {
+  const float *ml = part_ml + (size_t)h * max_splits * 2;
+  const float *po = part_o + (size_t)h * max_splits * head_dim + d;
+  AttnPart r;
+  r.o = make_float4(0.f, 0.f, 0.f, 0.f);
+  r.m = -INFINITY;
+  r.den = 0.0f;
+  // eight chunks at a time: their loads are independent of the running maximum
+  for (uint32_t s0 = s_first; s0 < n_splits; s0 += 8u * s_step) {
+    float2 mls[8];
+    float4 pos_[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const uint32_t s = min(s0 + u * s_step, n_splits - 1u);
+      mls[u] = ld_pair<COHERENT>(ml + 2u * s);
+      const float2 lo = ld_pair<COHERENT>(po + (size_t)s * head_dim), hi = ld_pair<COHERENT>(po + (size_t)s * head_dim + 2);
+      pos_[u] = make_float4(lo.x, lo.y, hi.x, hi.y);
+    }
+    float Mn = r.m;
+#pragma unroll
+    for (int u = 0; u < 8; u++)
+      if (s0 + u * s_step < n_splits) Mn = fmaxf(Mn, mls[u].x);
+    const float resc = expf(r.m - Mn);   // exp(-inf) = 0 on the first group
+    r.o.x *= resc; r.o.y *= resc; r.o.z *= resc; r.o.w *= resc;
+    r.den *= resc;
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      if (s0 + u * s_step < n_splits) {
+        const float f = expf(mls[u].x - Mn);
+        r.o.x += f * pos_[u].x; r.o.y += f * pos_[u].y; r.o.z += f * pos_[u].z; r.o.w += f * pos_[u].w;
+        r.den += f * mls[u].y;
+      }
+    }
+    r.m = Mn;
+  }
+  return r;
+}
+
+// Workgroup (kvh, split), 512 threads: the G query heads of K/V head kvh against positions
+// split * 128 .. + 128.
+//   * Every cache load of the workgroup is requested first: four threads share a K row (each
+//     every fourth 16-byte piece), HD / 8 threads a V row.
+//   * q of the G heads is rotated into LDS (pairs 2i, 2i+1; tensor.rs:1115-1177).  The workgroup
+//     of the last chunk also rotates the token's k, rounds k and v to f16, writes both cache rows
+//     and uses the LDS copy for the row of the current position.
+//   * Phase 1: scores; the partial dot products of a row are exchanged so that each of its four
+//     lanes ends with the whole score of G / 4 heads.  Phase 2: weighted V sum, exchanged the
+//     same way across the rows a wave holds, then summed over the eight waves in LDS.
+//   * GROUP != 0 (G * HD is a multiple of the quantizer's group): the workgroup that takes the
+//     last ticket of its K/V head merges the chunks and quantizes the G * HD outputs; no other
+//     workgroup waits for anything.
+template <int HD, int G, int GROUP>
+__global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
+                                                       const float *__restrict__ v_new,
+                                                       const float2 *__restrict__ cs, uint32_t rope_half,
+                                                       __half *__restrict__ kc, __half *__restrict__ vc,
+                                                       uint32_t pos, uint32_t max_splits, uint32_t n_head_kv,
+                                                       float scale, float *part_o, float *part_ml,
+                                                       uint32_t *counters, float *__restrict__ attn_out,
+                                                       OgmActDev act) {
+  constexpr int NT = 512, NW = NT / 64;
+  constexpr int KU = HD / 32;             // 16-byte pieces of a K row per thread
+  constexpr int TPR = HD / 8;             // threads per V row
+  constexpr int ROWS = NT / TPR;          // V rows in flight per step
   constexpr int STEPS = OGM_ATTN_CHUNK / ROWS;
+  constexpr int NV = G * 8;               // phase-2 partial sums per lane
+  constexpr int NF = G >= 4 ? G / 4 : 1;  // scores a lane ends phase 1 with
+  static_assert(OGM_ATTN_CHUNK * 4 == NT, "four threads per cache position");
+  __shared__ __align__(16) float qs[G][HD];
+  __shared__ __align__(16) __half kcur[HD];
+  __shared__ __align__(16) __half vcur[HD];
   __shared__ float sc[G][OGM_ATTN_CHUNK];
-  __shared__ float red[2][G][2];
-  __shared__ float osum[ROWS][G][HD];
-  const uint32_t kvh = blockIdx.x, split = blockIdx.y;
+  __shared__ float red[2][G][NW];
+  __shared__ __align__(16) float osum[NW][G][HD];
+  __shared__ uint32_t s_last;
+  __shared__ float mrg[GROUP != 0 ? 6 : 1][GROUP != 0 ? NT : 1];   // the final merge's slices
+  const uint32_t kvh = blockIdx.x, split = blockIdx.y, n_splits = gridDim.y;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t kv_dim = n_head_kv * HD;
   const uint32_t n_pos = pos + 1u;
   const uint32_t p0 = split * OGM_ATTN_CHUNK;
-  if (p0 >= n_pos) return;
   const uint32_t n_here = min(OGM_ATTN_CHUNK, n_pos - p0);
-  const bool valid = tid < n_here;
+  const bool is_last = split == n_splits - 1u;   // holds the current position, not yet cached
+  const uint32_t cur = pos - p0;                 // meaningful in the last chunk only
 
-  const uint32_t rr = tid / TPR, dc = tid - rr * TPR;   // phase 2: row slot and 8-dimension chunk
-  // rows past the chunk's end read the last valid row; their scores are discarded (weight 0)
-  const __half *krow = kc + (size_t)(p0 + min(tid, n_here - 1u)) * kv_dim + kvh * HD;
-  uint4 kr[HD / 8];
+  const uint32_t r = tid >> 2, c = tid & 3u;              // phase 1: cache row and piece phase
+  const uint32_t rr = tid / TPR, dc = tid - rr * TPR;     // phase 2: row slot and 8-dimension chunk
+  // rows past the chunk's end read the last row; their scores are discarded (weight 0)
+  const __half *krow = kc + (size_t)(p0 + min(r, n_here - 1u)) * kv_dim + kvh * HD;
+  uint4 kr[KU];
 #pragma unroll
-  for (int c = 0; c < HD / 8; c++) kr[c] = *(const uint4 *)(krow + 8 * c);
+  for (int j = 0; j < KU; j++) kr[j] = *(const uint4 *)(krow + 8 * (c + 4 * j));
   const __half *vbase = vc + (size_t)p0 * kv_dim + kvh * HD + 8u * dc;
   uint4 vr[STEPS];
 #pragma unroll
   for (int st = 0; st < STEPS; st++)
     vr[st] = *(const uint4 *)(vbase + (size_t)min((uint32_t)(st * ROWS) + rr, n_here - 1u) * kv_dim);
 
+  // ---- RoPE of q (and of the new k), cache rows of the current position
+  for (uint32_t i = tid; i < (uint32_t)(G * HD / 2); i += NT) {
+    const uint32_t g = i / (HD / 2), p = i - g * (HD / 2);
+    float2 ab = *(const float2 *)(q + (size_t)(kvh * G + g) * HD + 2u * p);
+    if (p < rope_half) ab = rope_pair(ab, cs[p]);
+    *(float2 *)&qs[g][2u * p] = ab;
+  }
+  if (is_last) {
+    if (tid < HD / 2) {
+      float2 ab = *(const float2 *)(k_new + (size_t)kvh * HD + 2u * tid);
+      if (tid < rope_half) ab = rope_pair(ab, cs[tid]);
+      const __half2 h = __floats2half2_rn(ab.x, ab.y);
+      *(__half2 *)&kcur[2u * tid] = h;
+      *(__half2 *)(kc + (size_t)pos * kv_dim + kvh * HD + 2u * tid) = h;
+    } else if (tid >= 64u && tid < 64u + HD / 2) {
+      const uint32_t p = tid - 64u;
+      const float2 ab = *(const float2 *)(v_new + (size_t)kvh * HD + 2u * p);
+      const __half2 h = __floats2half2_rn(ab.x, ab.y);
+      *(__half2 *)&vcur[2u * p] = h;
+      *(__half2 *)(vc + (size_t)pos * kv_dim + kvh * HD + 2u * p) = h;
+    }
+  }
+  // The cache loads requested above must stay up there: without this the row substitutions
+  // below let the compiler move each load down to its use, one trip to memory after the other.
+#pragma unroll
+  for (int j = 0; j < KU; j++) asm volatile("" : "+v"(kr[j].x), "+v"(kr[j].y), "+v"(kr[j].z), "+v"(kr[j].w));
+#pragma unroll
+  for (int st = 0; st < STEPS; st++) asm volatile("" : "+v"(vr[st].x), "+v"(vr[st].y), "+v"(vr[st].z), "+v"(vr[st].w));
+  __syncthreads();
+
   // ---- phase 1: scores
+  if (is_last && r == cur) {
+#pragma unroll
+    for (int j = 0; j < KU; j++) kr[j] = *(const uint4 *)&kcur[8 * (c + 4 * j)];
+  }
   float acc[G];
 #pragma unroll
   for (int g = 0; g < G; g++) acc[g] = 0.0f;
-  {
-    const float *qb = q + (size_t)kvh * G * HD;
 #pragma unroll
-    for (int c = 0; c < HD / 8; c++) {
-      const __half2 *h2 = (const __half2 *)&kr[c];
-      float kf[8];
+  for (int j = 0; j < KU; j++) {
+    const __half2 *h2 = (const __half2 *)&kr[j];
+    float kf[8];
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const float2 f = __half22float2(h2[j]);
-        kf[2 * j] = f.x;
-        kf[2 * j + 1] = f.y;
-      }
+    for (int e = 0; e < 4; e++) {
+      const float2 f = __half22float2(h2[e]);
+      kf[2 * e] = f.x;
+      kf[2 * e + 1] = f.y;
+    }
 #pragma unroll
-      for (int g = 0; g < G; g++)
-#pragma unroll
-        for (int j = 0; j < 8; j++) acc[g] = fmaf(qb[g * HD + 8 * c + j], kf[j], acc[g]);
+    for (int g = 0; g < G; g++) {
+      const float4 qa = *(const float4 *)&qs[g][8 * (c + 4 * j)];
+      const float4 qb = *(const float4 *)&qs[g][8 * (c + 4 * j) + 4];
+      acc[g] = fmaf(qa.x, kf[0], acc[g]); acc[g] = fmaf(qa.y, kf[1], acc[g]);
+      acc[g] = fmaf(qa.z, kf[2], acc[g]); acc[g] = fmaf(qa.w, kf[3], acc[g]);
+      acc[g] = fmaf(qb.x, kf[4], acc[g]); acc[g] = fmaf(qb.y, kf[5], acc[g]);
+      acc[g] = fmaf(qb.z, kf[6], acc[g]); acc[g] = fmaf(qb.w, kf[7], acc[g]);
     }
   }
-  // workgroup maximum and sum per query head: two barriers for all heads
-  float sv[G], mv[G];
+  // sum over the row's four lanes: while a lane holds two or more heads it keeps one half and
+  // hands the other to its partner; afterwards plain butterflies
+  uint32_t g0 = 0;        // first head this lane holds
+  bool owner = true;      // of several lanes holding the same head, the one that stores
+  {
+    int n = G;
 #pragma unroll
-  for (int g = 0; g < G; g++) {
-    sv[g] = valid ? acc[g] * scale : -INFINITY;
-    float m = sv[g];
+    for (int b = 1; b < 4; b <<= 1) {
+      const bool up = (lane & b) != 0;
+      if (n >= 2) {
+        n >>= 1;
 #pragma unroll
-    for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
-    if (lane == 0) red[0][g][wave] = m;
+        for (int i = 0; i < n; i++) {
+          float lo = acc[i], hi = acc[n + i];
+          asm volatile("" : "+v"(lo), "+v"(hi));   // keeps the selects on values, not on array slots
+          acc[i] = (up ? hi : lo) + __shfl_xor(up ? lo : hi, b, 64);
+        }
+        g0 += up ? n : 0;
+      } else {
+        acc[0] += __shfl_xor(acc[0], b, 64);
+        owner = owner && !up;
+      }
+    }
+  }
+  const bool valid = r < n_here;
+  float sv[NF], mv[NF];
+#pragma unroll
+  for (int i = 0; i < NF; i++) {
+    sv[i] = valid ? acc[i] * scale : -INFINITY;
+    float m = sv[i];
+#pragma unroll
+    for (int k = 4; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
+    if (lane < 4u && owner) red[0][g0 + i][wave] = m;
   }
   __syncthreads();
 #pragma unroll
-  for (int g = 0; g < G; g++) {
-    mv[g] = fmaxf(red[0][g][0], red[0][g][1]);
-    const float e = valid ? expf(sv[g] - mv[g]) : 0.0f;
-    sc[g][tid] = e;
+  for (int i = 0; i < NF; i++) {
+    float m = red[0][g0 + i][0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) m = fmaxf(m, red[0][g0 + i][w]);
+    mv[i] = m;
+    const float e = valid ? expf(sv[i] - m) : 0.0f;
+    if (owner) sc[g0 + i][r] = e;
     float l = e;
 #pragma unroll
-    for (int k = 1; k < 64; k <<= 1) l += __shfl_xor(l, k, 64);
-    if (lane == 0) red[1][g][wave] = l;
+    for (int k = 4; k < 64; k <<= 1) l += __shfl_xor(l, k, 64);
+    if (lane < 4u && owner) red[1][g0 + i][wave] = l;
   }
   __syncthreads();
   if (tid < G) {
+    float m = red[0][tid][0], l = red[1][tid][0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) {
+      m = fmaxf(m, red[0][tid][w]);
+      l += red[1][tid][w];
+    }
     const uint32_t h = kvh * G + tid;
-    part_ml[((size_t)h * max_splits + split) * 2] = fmaxf(red[0][tid][0], red[0][tid][1]);
-    part_ml[((size_t)h * max_splits + split) * 2 + 1] = red[1][tid][0] + red[1][tid][1];
+    st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2], m);
+    st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2 + 1], l);
   }
 
   // ---- phase 2: weighted sum of V rows
   {
-    float o[G][8];
+    float o[NV];
 #pragma unroll
-    for (int g = 0; g < G; g++)
-#pragma unroll
-      for (int j = 0; j < 8; j++) o[g][j] = 0.0f;
+    for (int i = 0; i < NV; i++) o[i] = 0.0f;
 #pragma unroll
     for (int st = 0; st < STEPS; st++) {
       const uint32_t p = st * ROWS + rr;   // past the chunk's end the weight sc is 0
+      if (is_last && p >= cur) vr[st] = *(const uint4 *)&vcur[8u * dc];   // the cache row is not written yet
       const __half2 *h2 = (const __half2 *)&vr[st];
       float vf[8];
 #pragma unroll
@@ -249,21 +382,92 @@ __global__ __launch_bounds__(128) void ogm_attn_partial_kernel(const float *__re
       for (int g = 0; g < G; g++) {
         const float w = sc[g][p];
 #pragma unroll
-        for (int j = 0; j < 8; j++) o[g][j] = fmaf(w, vf[j], o[g][j]);
+        for (int j = 0; j < 8; j++) o[g * 8 + j] = fmaf(w, vf[j], o[g * 8 + j]);
       }
     }
+    // sum over the rows a wave holds (lanes that differ in the bits above the chunk index): each
+    // exchange halves what a lane keeps
+    uint32_t sel = 0;
+    int n = NV;
 #pragma unroll
-    for (int g = 0; g < G; g++) {
-      *(float4 *)&osum[rr][g][8 * dc] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
-      *(float4 *)&osum[rr][g][8 * dc + 4] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
+    for (int b = TPR; b < 64; b <<= 1) {
+      const bool up = (lane & b) != 0;
+      n >>= 1;
+#pragma unroll
+      for (int i = 0; i < n; i++) {
+        float lo = o[i], hi = o[n + i];
+        asm volatile("" : "+v"(lo), "+v"(hi));   // keeps the selects on values, not on array slots
+        o[i] = (up ? hi : lo) + __shfl_xor(up ? lo : hi, b, 64);
+      }
+      sel += up ? n : 0;
     }
+    // o[0 .. n) are the wave's sums of flattened (head, dimension-in-chunk) indices sel .. sel + n
+    // (sel is a multiple of n: the head and the dimension of index sel + i split into a lane part
+    // and a compile-time part)
+    float *dst = &osum[wave][0][0] + (sel >> 3) * HD + (sel & 7u) + 8u * dc;
+#pragma unroll
+    for (int i = 0; i < n; i++) dst[(i >> 3) * HD + (i & 7)] = o[i];
     __syncthreads();
-    for (uint32_t i = tid; i < G * HD; i += 128u) {
+    for (uint32_t i = tid; i < (uint32_t)(G * HD); i += NT) {
       const uint32_t g = i / HD, d = i - g * HD;
       float t = 0.0f;
 #pragma unroll
-      for (int r = 0; r < ROWS; r++) t += osum[r][g][d];
-      part_o[((size_t)(kvh * G + g) * max_splits + split) * HD + d] = t;
+      for (int w = 0; w < NW; w++) t += osum[w][g][d];
+      st_one<GROUP != 0>(&part_o[((size_t)(kvh * G + g) * max_splits + split) * HD + d], t);
+    }
+  }
+
+  // ---- the last workgroup of this K/V head merges the chunks and quantizes
+  if constexpr (GROUP != 0) {
+    // The partial results were stored device-coherently; once this wave's stores are acknowledged
+    // (vmcnt 0) and the workgroup has met, one ticket tells whether every chunk of the head is in.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (tid == 0) {
+      const uint32_t ticket =
+          __hip_atomic_fetch_add(&counters[kvh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = ticket == n_splits - 1u;
+      if (ticket == n_splits - 1u)
+        __hip_atomic_store(&counters[kvh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+    }
+    __syncthreads();
+    if (!s_last) return;
+    // every thread merges a slice of the chunks of one group of four outputs (one trip to memory
+    // up to 8 * NSL chunks), then the slices meet in LDS
+    constexpr int NG = G * HD / 4;    // groups of four outputs
+    constexpr int NSL = NT / NG;      // slices of chunks
+    static_assert(NG * NSL == NT, "the merge assumes whole slices");
+    {
+      const uint32_t eg = tid % NG, slice = tid / NG;
+      const uint32_t el = 4u * eg;
+      const AttnPart pt = attn_merge_chunks<true>(part_o, part_ml, kvh * G + el / HD, el % HD, slice, NSL, n_splits,
+                                                  max_splits, HD);
+      mrg[0][tid] = pt.m; mrg[1][tid] = pt.den;
+      mrg[2][tid] = pt.o.x; mrg[3][tid] = pt.o.y; mrg[4][tid] = pt.o.z; mrg[5][tid] = pt.o.w;
+    }
+    __syncthreads();
+    constexpr int RUNS = (NG + 63) / 64;
+    for (int run = wave; run < RUNS; run += NW) {
+      const uint32_t eg = run * 64u + lane;
+      const bool active = eg < (uint32_t)NG;
+      const uint32_t e0 = kvh * (uint32_t)(G * HD) + 4u * eg;
+      float4 ov = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (active) {
+        float M = mrg[0][eg];   // slice 0 always holds chunk 0
+#pragma unroll
+        for (int k = 1; k < NSL; k++) M = fmaxf(M, mrg[0][k * NG + eg]);
+        float den = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NSL; k++) {
+          const float f = expf(mrg[0][k * NG + eg] - M);   // a slice without chunks has m = -inf: f = 0
+          den += f * mrg[1][k * NG + eg];
+          ov.x += f * mrg[2][k * NG + eg]; ov.y += f * mrg[3][k * NG + eg];
+          ov.z += f * mrg[4][k * NG + eg]; ov.w += f * mrg[5][k * NG + eg];
+        }
+        ov.x /= den; ov.y /= den; ov.z /= den; ov.w /= den;
+        if (attn_out) *(float4 *)(attn_out + e0) = ov;
+      }
+      ogm_quantize_store<GROUP>(ov, e0, active, lane, act.q, act.d, act.sums, act.bsum);
     }
   }
 }
@@ -282,70 +486,53 @@ __global__ __launch_bounds__(64) void ogm_attn_combine_quant_kernel(const float 
   const bool active = e0 < n;
   float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
   if (active) {
-    const uint32_t h = e0 / head_dim, d = e0 - h * head_dim;
-    const float2 *ml = (const float2 *)(part_ml + (size_t)h * max_splits * 2);
-    const float *po = part_o + (size_t)h * max_splits * head_dim + d;
-    // eight chunks at a time: their loads are independent of the running maximum
-    float M = -INFINITY, den = 0.0f;
-    for (uint32_t s0 = 0; s0 < n_splits; s0 += 8u) {
-      float2 mls[8];
-      float4 pos_[8];
-#pragma unroll
-      for (int u = 0; u < 8; u++) {
-        const uint32_t s = min(s0 + u, n_splits - 1u);
-        mls[u] = ml[s];
-        pos_[u] = *(const float4 *)(po + (size_t)s * head_dim);
-      }
-      float Mn = M;
-#pragma unroll
-      for (int u = 0; u < 8; u++)
-        if (s0 + u < n_splits) Mn = fmaxf(Mn, mls[u].x);
-      const float resc = expf(M - Mn);   // exp(-inf) = 0 on the first group
-      o.x *= resc; o.y *= resc; o.z *= resc; o.w *= resc;
-      den *= resc;
-#pragma unroll
-      for (int u = 0; u < 8; u++) {
-        if (s0 + u < n_splits) {
-          const float f = expf(mls[u].x - Mn);
-          o.x += f * pos_[u].x; o.y += f * pos_[u].y; o.z += f * pos_[u].z; o.w += f * pos_[u].w;
-          den += f * mls[u].y;
-        }
-      }
-      M = Mn;
-    }
-    o.x /= den; o.y /= den; o.z /= den; o.w /= den;
+    const AttnPart pt = attn_merge_chunks<false>(part_o, part_ml, e0 / head_dim, e0 % head_dim, 0u, 1u, n_splits,
+                                                 max_splits, head_dim);
+    o = make_float4(pt.o.x / pt.den, pt.o.y / pt.den, pt.o.z / pt.den, pt.o.w / pt.den);
     if (attn_out) *(float4 *)(attn_out + e0) = o;
   }
   ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum);
 }
 
-hipError_t ogm_launch_attn_decode(const float *q, const void *k_cache_layer, const void *v_cache_layer,
-                                  uint32_t pos, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
-                                  uint32_t head_dim, float scale, float *part_o, float *part_ml, int mode,
+hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
+                                  uint32_t rope_dim, void *k_cache_layer, void *v_cache_layer, uint32_t pos,
+                                  uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
+                                  float scale, float *part_o, float *part_ml, uint32_t *counters, int mode,
                                   float *attn_out, OgmActDev act, hipStream_t stream) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0) return hipErrorInvalidValue;
+  if (rope_dim > head_dim || rope_dim % 2u != 0) return hipErrorInvalidValue;
   const uint32_t n_splits = pos / OGM_ATTN_CHUNK + 1u;
   if (n_splits > max_splits) return hipErrorInvalidValue;
   const uint32_t n = n_head * head_dim;
   if (n % 32u != 0) return hipErrorInvalidValue;
   const dim3 grid(n_head_kv, n_splits);
   const uint32_t G = n_head / n_head_kv;
-#define OGM_ATTN_LAUNCH(HD_, G_)                                                                    \
-  hipLaunchKernelGGL((ogm_attn_partial_kernel<HD_, G_>), grid, dim3(128), 0, stream, q,              \
-                     (const __half *)k_cache_layer, (const __half *)v_cache_layer, pos, max_splits,   \
-                     n_head_kv, scale, part_o, part_ml)
-  if (head_dim == 128 && G == 1) OGM_ATTN_LAUNCH(128, 1);
-  else if (head_dim == 128 && G == 2) OGM_ATTN_LAUNCH(128, 2);
-  else if (head_dim == 128 && G == 4) OGM_ATTN_LAUNCH(128, 4);
-  else if (head_dim == 128 && G == 8) OGM_ATTN_LAUNCH(128, 8);
-  else if (head_dim == 64 && G == 1) OGM_ATTN_LAUNCH(64, 1);
-  else if (head_dim == 64 && G == 2) OGM_ATTN_LAUNCH(64, 2);
-  else if (head_dim == 64 && G == 4) OGM_ATTN_LAUNCH(64, 4);
-  else if (head_dim == 64 && G == 8) OGM_ATTN_LAUNCH(64, 8);
+  const uint32_t group = mode == 0 ? 32u : 256u;
+  // the merge rides in the attention kernel when a K/V head's outputs are whole quantizer groups
+  const uint32_t fused = (G * head_dim) % group == 0 ? group : 0u;
+#define OGM_ATTN_LAUNCH(HD_, G_, GR_)                                                                  \
+  hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, GR_>), grid, dim3(512), 0, stream, q, k_new, v_new,      \
+                     (const float2 *)cs, rope_dim / 2u, (__half *)k_cache_layer, (__half *)v_cache_layer, \
+                     pos, max_splits, n_head_kv, scale, part_o, part_ml, counters, attn_out, act)
+#define OGM_ATTN_GROUPS(HD_, G_)                                \
+  do {                                                          \
+    if (fused == 32u) OGM_ATTN_LAUNCH(HD_, G_, 32);             \
+    else if (fused == 256u) OGM_ATTN_LAUNCH(HD_, G_, 256);      \
+    else OGM_ATTN_LAUNCH(HD_, G_, 0);                           \
+  } while (0)
+  if (head_dim == 128 && G == 1) OGM_ATTN_GROUPS(128, 1);
+  else if (head_dim == 128 && G == 2) OGM_ATTN_GROUPS(128, 2);
+  else if (head_dim == 128 && G == 4) OGM_ATTN_GROUPS(128, 4);
+  else if (head_dim == 128 && G == 8) OGM_ATTN_GROUPS(128, 8);
+  else if (head_dim == 64 && G == 1) OGM_ATTN_GROUPS(64, 1);
+  else if (head_dim == 64 && G == 2) OGM_ATTN_GROUPS(64, 2);
+  else if (head_dim == 64 && G == 4) OGM_ATTN_GROUPS(64, 4);
+  else if (head_dim == 64 && G == 8) OGM_ATTN_GROUPS(64, 8);
   else return hipErrorInvalidValue;
+#undef OGM_ATTN_GROUPS
 #undef OGM_ATTN_LAUNCH
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
+  if (e != hipSuccess || fused != 0u) return e;
   const dim3 cgrid((n + 255u) / 256u);
   if (mode == 0)
     hipLaunchKernelGGL(ogm_attn_combine_quant_kernel<32>, cgrid, dim3(64), 0, stream, part_o, part_ml,

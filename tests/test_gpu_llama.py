@@ -113,6 +113,30 @@ def test_decode_over_a_prefilled_cache_with_several_attention_chunks(be):
         dev.close()
 
 
+@pytest.mark.parametrize("hd,group,n_kv", [(128, 1, 2), (128, 2, 2), (128, 8, 1), (64, 1, 4), (64, 4, 2), (64, 8, 1)])
+@pytest.mark.parametrize("wtype", [Q4_K, Q8_0])
+def test_attention_head_shapes_across_a_chunk_boundary(be, hd, group, n_kv, wtype):
+    """Every (head_dim, query heads per K/V head) the attention kernel is built for, with per-256
+    and per-32 quantization of its output, over positions 126..130: the last row of a full chunk,
+    then a chunk that holds the current position only."""
+    n_head = group * n_kv
+    n_embd = n_head * hd
+    ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=2,
+                          types=(wtype, wtype, wtype, wtype), max_ctx=160, seed=hd + group, rope_dim=hd // 2)
+    try:
+        n_pre = 126
+        for l in range(2):
+            k = rng.standard_normal((n_pre, n_kv * hd)).astype(f32)
+            v = rng.standard_normal((n_pre, n_kv * hd)).astype(f32)
+            dev.kv_write(l, 0, k, v)
+            ref.k_cache[l] = [r.astype(np.float16) for r in k]
+            ref.v_cache[l] = [r.astype(np.float16) for r in v]
+        for pos in range(126, 131):
+            step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"hd {hd} group {group} pos {pos}")
+    finally:
+        dev.close()
+
+
 def test_decode_rejects_bad_arguments(be):
     from orangu_amd import OgmError
     ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=1,
