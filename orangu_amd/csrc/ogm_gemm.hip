@@ -39,6 +39,7 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 struct GemmParams {
   const uint8_t *wt;      // tile-planar Q4_K
   const _Float16 *xh;     // [T][in_dim] int8 activations as f16
+  const int8_t *xq;       // [T][in_dim] the int8 activations themselves (wide kernel)
   const _Float16 *bs16;   // [T][nsb][16]: floor(bsum_j / 64) for j = 0..7, then bsum_j mod 64
   const float *ad;        // [T][nsb] activation scales (per 256)
   float *y;               // [T][out_dim]
@@ -57,7 +58,7 @@ __global__ void ogm_gemm_prep_kernel(const int8_t *__restrict__ q, const int16_t
                                      _Float16 *__restrict__ xh, _Float16 *__restrict__ bs16, size_t n8,
                                      size_t n_sb) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n8) {
+  if (xh && i < n8) {
     const int2 v = ((const int2 *)q)[i];
     half8 o;
     o[0] = (_Float16)(float)(int8_t)(v.x);
@@ -426,6 +427,363 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q4k_kernel(GemmParams p) {
 }
 
 // ------------------------------------------------------------------------------------------
+// Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
+//
+// The 128 x 128 kernel above is bound by LDS bandwidth: a multiplying wave reads (64 + 32) k-rows
+// from LDS per pair of MFMAs.  Here a multiplying wave owns 64 rows x 64 tokens (four 32 x 32
+// tiles, so the same reads feed twice the MFMAs), the activations stay int8 in LDS (half the
+// bytes; the multiplying wave turns them into f16 with the 0x6400 | (x + 128) = 1024 + (x + 128)
+// trick, exact), and a workgroup has eight multiplying and four feeding waves, three per SIMD,
+// which leaves 168 registers per lane for the four integer-sum and four f32 accumulator tiles.
+//
+// k order inside a stage: MFMA step kk of the lane half lh covers k = 32 (kk >> 1) + 16 lh +
+// 8 (kk & 1) + 0..7, so that a lane's activations for two steps are 16 contiguous bytes.
+//
+// Pass 1 (the min terms of all super-blocks, first, as the reference orders them) takes its
+// operands from LDS tables that all twelve waves fill for eight super-blocks at a time: one trip
+// to memory per group instead of one per four super-blocks.  The tables alias the stage buffers.
+
+#define GW_BT 256u           // tokens per workgroup
+#define GW_PG 8u             // super-blocks per pass-1 group
+// Staged tiles are padded by one 16-byte chunk per row (weights: 64 f16 + 8, activations: 64 bytes
+// + 16).  Sixteen consecutive rows then start 36 (or 20) banks apart, which puts their 16-byte
+// accesses on sixteen disjoint groups of four banks, and a chunk's position is a compile-time
+// offset from the row's address: no swizzle arithmetic in the loop.
+#define GW_A_ROW 72u                     // f16 per staged weight row
+#define GW_B_ROW 80u                     // bytes per staged activation row
+#define GW_A_STAGE (128u * GW_A_ROW)     // f16 per staged weight tile (18 KB)
+#define GW_B_STAGE (256u * GW_B_ROW)     // bytes per staged activation tile (20 KB)
+// main loop: A [2] 36 KB | B [2] 40 KB | a2 4 KB | b2 8 KB | d 512 B
+// pass 1:    a1_t [8][128][16] f16 32 KB | b2_t [8][256][16] f16 64 KB | dm_t [8][128] f32 4 KB | ad_t [8][256] f32 8 KB
+#define GW_B_OFF (2u * GW_A_STAGE * 2u)              // bytes
+#define GW_SIDE_OFF (GW_B_OFF + 2u * GW_B_STAGE)     // bytes
+static const uint32_t GW_LDS_BYTES = 32768u + 65536u + 4096u + 8192u;
+
+// Eight activations (two dwords of x + 128, as the feeding waves store them) -> eight f16, exact:
+// 0x6400 | u is the f16 1024 + u, and 1024 + (x + 128) - 1152 = x.
+__device__ __forceinline__ half8 gw_u8_to_f16(uint32_t u0, uint32_t u1) {
+  union { uint32_t u[4]; half8 h; half2v p[4]; } r;
+  r.u[0] = __builtin_amdgcn_perm(0x64646464u, u0, 0x04010400u);  // (b0, 0x64, b1, 0x64)
+  r.u[1] = __builtin_amdgcn_perm(0x64646464u, u0, 0x04030402u);
+  r.u[2] = __builtin_amdgcn_perm(0x64646464u, u1, 0x04010400u);
+  r.u[3] = __builtin_amdgcn_perm(0x64646464u, u1, 0x04030402u);
+  const half2v k = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+#pragma unroll
+  for (int i = 0; i < 4; i++) r.p[i] = r.p[i] + k;
+  return r.h;
+}
+
+__device__ __forceinline__ uint4 gw_bias128(uint4 v) {
+  return make_uint4(v.x ^ 0x80808080u, v.y ^ 0x80808080u, v.z ^ 0x80808080u, v.w ^ 0x80808080u);
+}
+
+__global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  _Float16 *A_l = (_Float16 *)lds;                       // [2][128][72]
+  uint8_t *B_l = lds + GW_B_OFF;                         // [2][256][80]
+  _Float16 *a2_l = (_Float16 *)(lds + GW_SIDE_OFF);      // [128 rows][16]: 512*sc_j | 8*sc_j
+  _Float16 *b2_l = a2_l + 128 * 16;                      // [256 tokens][16]: bh_j | bl_j
+  float *d_l = (float *)(b2_l + 256 * 16);               // [128]
+  _Float16 *a1_t = (_Float16 *)lds;                      // pass 1: 64*m_j | m_j per (super-block, row)
+  _Float16 *b2_t = (_Float16 *)(lds + 32768);            //         bh_j | bl_j per (super-block, token)
+  float *dm_t = (float *)(lds + 32768 + 65536);          //         dmin per (super-block, row)
+  float *ad_t = dm_t + GW_PG * 128;                      //         activation scale per (super-block, token)
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const bool producer = wave >= 8u;
+  const uint32_t wr = wave & 1u, wt_ = (wave & 7u) >> 1;   // multiplying wave: row half, token quarter (64)
+  const uint32_t t0 = blockIdx.x * GW_BT, r0 = blockIdx.y * GM_BN;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+
+  auto row_off = [&](uint32_t row) -> uint32_t {
+    row = min(row, p.out_dim - 1u);
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    return rb * p.nct * 9216u + r * 16u;
+  };
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    const uint32_t ct = s >> p.c_shift, cl = s & ((1u << p.c_shift) - 1u);
+    return ct * 9216u + (cl << p.r_shift) * 16u;
+  };
+
+  // multiplying wave: rows ra (+32), local tokens tl (+32)
+  const uint32_t ra = 64u * wr + l32, tl = 64u * wt_ + l32;
+  float16v y00, y01, y10, y11;   // y<row tile><token tile>
+#pragma unroll
+  for (int r = 0; r < 16; r++) y00[r] = y01[r] = y10[r] = y11[r] = 0.0f;
+  const float16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  // ---------------- pass 1: acc -= (ad * dmin) * sum_j m_j * bsum_j, all super-blocks first
+#pragma unroll 1
+  for (uint32_t g0 = 0; g0 < p.nsb; g0 += GW_PG) {
+    const uint32_t ng = min(GW_PG, p.nsb - g0);
+    for (uint32_t i = tid; i < ng * 256u; i += 768u) {          // (super-block, row, half of the operand)
+      const uint32_t sb = i >> 8, row = (i >> 1) & 127u, hf = i & 1u;
+      const uint4 hd = *(const uint4 *)(p.wt + (row_off(r0 + row) + sb_off(g0 + sb)));
+      uint32_t mna, mnb;
+      q4k_mins(hd, mna, mnb);
+      *(half8 *)(a1_t + (sb * 128u + row) * 16u + 8u * hf) = side_operand(mna, mnb, hf ? 1.0f : 64.0f);
+      if (hf == 0) dm_t[sb * 128u + row] = gm_f16_bits_to_f32(hd.x >> 16);
+    }
+    for (uint32_t i = tid; i < ng * 512u; i += 768u) {          // (super-block, token, half)
+      const uint32_t sb = i >> 9, tok = (i >> 1) & 255u, hf = i & 1u;
+      const uint32_t t = min(t0 + tok, p.n_tokens - 1u);
+      *(uint4 *)(b2_t + (sb * 256u + tok) * 16u + 8u * hf) =
+          *(const uint4 *)(p.bs16 + ((t * p.nsb + g0 + sb) * 16u + 8u * hf));
+    }
+    for (uint32_t i = tid; i < ng * 256u; i += 768u) {
+      const uint32_t sb = i >> 8, tok = i & 255u;
+      ad_t[sb * 256u + tok] = p.ad[min(t0 + tok, p.n_tokens - 1u) * p.nsb + g0 + sb];
+    }
+    __syncthreads();
+    if (!producer) {
+#pragma unroll 1
+      for (uint32_t sb = 0; sb < ng; sb++) {
+        const half8 a10 = *(const half8 *)(a1_t + (sb * 128u + ra) * 16u + 8u * lh);
+        const half8 a11 = *(const half8 *)(a1_t + (sb * 128u + ra + 32u) * 16u + 8u * lh);
+        const half8 b20 = *(const half8 *)(b2_t + (sb * 256u + tl) * 16u + 8u * lh);
+        const half8 b21 = *(const half8 *)(b2_t + (sb * 256u + tl + 32u) * 16u + 8u * lh);
+        const float adv0 = ad_t[sb * 256u + tl], adv1 = ad_t[sb * 256u + tl + 32u];
+        const float *dm = dm_t + sb * 128u + 64u * wr + 4u * lh;
+#define GW_MIN_TILE(Y, A1, B2, ADV, DMO)                                                   \
+  do {                                                                                     \
+    const float16v im = __builtin_amdgcn_mfma_f32_32x32x16_f16(A1, B2, zero, 0, 0, 0);     \
+    _Pragma("unroll") for (int q4 = 0; q4 < 4; q4++) {                                     \
+      const float4 m = *(const float4 *)(dm + (DMO) + 8 * q4);                             \
+      Y[4 * q4 + 0] -= ADV * m.x * im[4 * q4 + 0];                                         \
+      Y[4 * q4 + 1] -= ADV * m.y * im[4 * q4 + 1];                                         \
+      Y[4 * q4 + 2] -= ADV * m.z * im[4 * q4 + 2];                                         \
+      Y[4 * q4 + 3] -= ADV * m.w * im[4 * q4 + 3];                                         \
+    }                                                                                      \
+  } while (0)
+        GW_MIN_TILE(y00, a10, b20, adv0, 0);
+        GW_MIN_TILE(y01, a10, b21, adv1, 0);
+        GW_MIN_TILE(y10, a11, b20, adv0, 32);
+        GW_MIN_TILE(y11, a11, b21, adv1, 32);
+#undef GW_MIN_TILE
+      }
+    }
+    __syncthreads();   // the tables are rewritten (next group) or become the stage buffers
+  }
+
+  // ---------------- pass 2: acc += ad * (d * sum_j sc_j * dot32_j)
+  // Feeding roles (256 threads).  Weights: one 16-byte piece of qs per thread and stage (16 low-
+  // nibble and 16 high-nibble weights of one row).  Activations: four 16-byte chunks per thread.
+  // Once per super-block also the row's header (scales, d) and two chunks of bh | bl.
+  const uint32_t rt = tid & 255u;
+  const uint32_t arow = rt & 127u, ah = rt >> 7;
+  const uint32_t hdo = row_off(r0 + arow), roa = hdo + (1u + ah) * 1024u;
+  const uint32_t btok = rt >> 2, bch = rt & 3u;
+  const uint32_t bo0 = min(t0 + btok, p.n_tokens - 1u) * p.in_dim + 16u * bch;
+  const uint32_t bo1 = min(t0 + btok + 64u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
+  const uint32_t bo2 = min(t0 + btok + 128u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
+  const uint32_t bo3 = min(t0 + btok + 192u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
+  const uint32_t bso = btok * GW_B_ROW + 16u * bch;       // byte offset in a staged activation tile
+  const uint32_t aso = arow * GW_A_ROW + 16u * ah;        // f16 offset of chunk 2 ah in a staged weight tile
+  const uint32_t tok2 = rt >> 1, hf2 = rt & 1u;
+  const uint32_t b2o0 = min(t0 + tok2, p.n_tokens - 1u) * p.nsb * 16u + 8u * hf2;
+  const uint32_t b2o1 = min(t0 + tok2 + 128u, p.n_tokens - 1u) * p.nsb * 16u + 8u * hf2;
+  // Loads run three stages ahead of the MFMAs (two ahead of their LDS store: a stage is shorter
+  // than a trip to memory) through three rotating register sets; stage m uses set m mod 3.
+  uint4 qv_0, qv_1, qv_2;
+  uint4 bxa_0, bxb_0, bxc_0, bxd_0, bxa_1, bxb_1, bxc_1, bxd_1, bxa_2, bxb_2, bxc_2, bxd_2;
+  uint4 hdx = make_uint4(0, 0, 0, 0), b2x0 = make_uint4(0, 0, 0, 0), b2x1 = make_uint4(0, 0, 0, 0);
+  uint32_t sca = 0, scb = 0;
+  float dnext = 0.0f;
+
+#define GW_LOAD_STAGE(S, G, K)                                                                    \
+  do {                                                                                            \
+    const uint32_t so_ = sb_off(S);                                                               \
+    if ((G) == 0) hdx = *(const uint4 *)(p.wt + (hdo + so_));                                     \
+    if ((G) == 1) {                                                                               \
+      b2x0 = *(const uint4 *)(p.bs16 + (b2o0 + (S) * 16u));                                        \
+      b2x1 = *(const uint4 *)(p.bs16 + (b2o1 + (S) * 16u));                                        \
+    }                                                                                             \
+    qv_##K = *(const uint4 *)(p.wt + (roa + so_ + 2u * (G) * 1024u));                             \
+    const uint32_t ko_ = (S) * 256u + (G) * 64u;                                                  \
+    bxa_##K = *(const uint4 *)(p.xq + (bo0 + ko_));                                               \
+    bxb_##K = *(const uint4 *)(p.xq + (bo1 + ko_));                                               \
+    bxc_##K = *(const uint4 *)(p.xq + (bo2 + ko_));                                               \
+    bxd_##K = *(const uint4 *)(p.xq + (bo3 + ko_));                                               \
+  } while (0)
+
+#define GW_STORE_STAGE(G, BUF, K)                                                                 \
+  do {                                                                                            \
+    if ((G) == 0) {                                                                               \
+      q4k_scales(hdx, sca, scb);                                                                  \
+      dnext = gm_f16_bits_to_f32(hdx.x & 0xFFFFu);                                                \
+    }                                                                                             \
+    const uint32_t scw_ = (G) < 2 ? sca : scb;                                                    \
+    const uint32_t sh_ = ((G) & 1u) * 16u;                                                        \
+    const _Float16 slo_ = (_Float16)(float)((scw_ >> sh_) & 0xFFu);                               \
+    const _Float16 shi_ = (_Float16)(float)((scw_ >> (sh_ + 8u)) & 0xFFu);                        \
+    const half2v sl2_ = {slo_, slo_}, sh2_ = {shi_, shi_};                                        \
+    uint4 la_, lb_, ha_, hb_; /* low nibbles of bytes 0..7 and 8..15, then the high nibbles */    \
+    dequant8(qv_##K.x, sl2_, sh2_, la_.x, la_.y, ha_.x, ha_.y);                                   \
+    dequant8(qv_##K.y, sl2_, sh2_, la_.z, la_.w, ha_.z, ha_.w);                                   \
+    dequant8(qv_##K.z, sl2_, sh2_, lb_.x, lb_.y, hb_.x, hb_.y);                                   \
+    dequant8(qv_##K.w, sl2_, sh2_, lb_.z, lb_.w, hb_.z, hb_.w);                                   \
+    /* piece 1+2g+ah holds qs[32g+16ah ..]: low nibbles are k 16ah.. of the stage, high 32+16ah.. */ \
+    _Float16 *ab_ = A_l + (BUF) * GW_A_STAGE;                                                     \
+    *(uint4 *)(ab_ + aso) = la_;              /* chunk 2 ah */                                    \
+    *(uint4 *)(ab_ + aso + 8u) = lb_;                                                             \
+    *(uint4 *)(ab_ + aso + 32u) = ha_;        /* chunk 4 + 2 ah */                                \
+    *(uint4 *)(ab_ + aso + 40u) = hb_;                                                            \
+    uint8_t *bb_ = B_l + (BUF) * GW_B_STAGE;                                                      \
+    /* stored as x + 128: the multiplying waves' conversion starts from unsigned bytes */         \
+    *(uint4 *)(bb_ + bso) = gw_bias128(bxa_##K);                                                  \
+    *(uint4 *)(bb_ + bso + 64u * GW_B_ROW) = gw_bias128(bxb_##K);                                 \
+    *(uint4 *)(bb_ + bso + 128u * GW_B_ROW) = gw_bias128(bxc_##K);                                \
+    *(uint4 *)(bb_ + bso + 192u * GW_B_ROW) = gw_bias128(bxd_##K);                                \
+    if ((G) == 1) {                                                                               \
+      /* side tables of this super-block: their last readers are two barriers behind, their      \
+         next readers two barriers ahead; the two threads of a row write the same d */           \
+      *(half8 *)(a2_l + arow * 16u + 8u * ah) = side_operand(sca, scb, ah ? 8.0f : 512.0f);       \
+      d_l[arow] = dnext;                                                                          \
+      *(uint4 *)(b2_l + tok2 * 16u + 8u * hf2) = b2x0;                                            \
+      *(uint4 *)(b2_l + (tok2 + 128u) * 16u + 8u * hf2) = b2x1;                                   \
+    }                                                                                             \
+  } while (0)
+
+#define GW_PRODUCE(G, KL, KS)                                                                     \
+  do {                                                                                            \
+    /* past the end the last super-block is loaded again and parked in the idle buffer */        \
+    GW_LOAD_STAGE(min((G) < 1 ? s : s + 1u, p.nsb - 1u), (uint32_t)(((G) + 3) & 3), KL);          \
+    GW_STORE_STAGE((uint32_t)(((G) + 1) & 3), ((G) & 1u) ^ 1u, KS);                               \
+    __syncthreads();                                                                              \
+  } while (0)
+
+  if (producer) {
+    // the feeding wave of a SIMD has little to do per stage but everybody waits for it at the
+    // barrier: let it go first
+    __builtin_amdgcn_s_setprio(3);
+    GW_LOAD_STAGE(0u, 0u, 0);
+    GW_LOAD_STAGE(0u, 1u, 1);
+    GW_LOAD_STAGE(0u, 2u, 2);
+    GW_STORE_STAGE(0u, 0u, 0);
+  }
+  __syncthreads();
+
+  if (producer) {
+#define GW_PRODUCE_SB(K0, K1, K2)                                                                 \
+  do {                                                                                            \
+    GW_PRODUCE(0, K0, K1);   /* loads stage 4s+3, parks stage 4s+1 */                             \
+    GW_PRODUCE(1, K1, K2);                                                                        \
+    GW_PRODUCE(2, K2, K0);                                                                        \
+    GW_PRODUCE(3, K0, K1);                                                                        \
+    s++;                                                                                          \
+  } while (0)
+    uint32_t s = 0;
+    while (s < p.nsb) {
+      GW_PRODUCE_SB(0, 1, 2);
+      if (s >= p.nsb) break;
+      GW_PRODUCE_SB(1, 2, 0);
+      if (s >= p.nsb) break;
+      GW_PRODUCE_SB(2, 0, 1);
+    }
+#undef GW_PRODUCE_SB
+    return;
+  }
+#undef GW_LOAD_STAGE
+#undef GW_STORE_STAGE
+#undef GW_PRODUCE
+
+  // ---- multiplying waves
+  const uint32_t tk0 = min(t0 + tl, p.n_tokens - 1u), tk1 = min(t0 + tl + 32u, p.n_tokens - 1u);
+  const uint32_t aro = ra * GW_A_ROW + 16u * lh;   // f16 offset of chunk 2 lh of row ra
+  const uint32_t bro = tl * GW_B_ROW + 16u * lh;   // byte offset of chunk lh of token tl
+  float16v c00, c01, c10, c11;
+  float adv0 = 0.0f, adv1 = 0.0f;
+
+#define GW_CONSUME(G)                                                                             \
+  do {                                                                                            \
+    const uint32_t buf = (G) & 1u;                                                                \
+    if ((G) == 0) {                                                                               \
+      adv0 = p.ad[tk0 * p.nsb + s];                                                               \
+      adv1 = p.ad[tk1 * p.nsb + s];                                                               \
+    }                                                                                             \
+    const _Float16 *ab = A_l + buf * GW_A_STAGE;                                                  \
+    const uint8_t *bb = B_l + buf * GW_B_STAGE;                                                   \
+    _Pragma("unroll") for (int m = 0; m < 2; m++) {                                               \
+      const uint4 bq0 = *(const uint4 *)(bb + bro + 32u * m);                                     \
+      const uint4 bq1 = *(const uint4 *)(bb + bro + 32u * GW_B_ROW + 32u * m);                    \
+      _Pragma("unroll") for (int e = 0; e < 2; e++) {                                             \
+        /* chunk 4 m + 2 lh + e of rows ra and ra + 32 */                                         \
+        const half8 a0 = *(const half8 *)(ab + aro + 32u * m + 8u * e);                           \
+        const half8 a1 = *(const half8 *)(ab + aro + 32u * GW_A_ROW + 32u * m + 8u * e);          \
+        /* the super-block's first step starts fresh accumulators */                             \
+        const bool first = (G) == 0 && m == 0 && e == 0;                                          \
+        const half8 b0 = e ? gw_u8_to_f16(bq0.z, bq0.w) : gw_u8_to_f16(bq0.x, bq0.y);             \
+        c00 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b0, first ? zero : c00, 0, 0, 0);        \
+        c10 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, first ? zero : c10, 0, 0, 0);        \
+        const half8 b1 = e ? gw_u8_to_f16(bq1.z, bq1.w) : gw_u8_to_f16(bq1.x, bq1.y);             \
+        c01 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b1, first ? zero : c01, 0, 0, 0);        \
+        c11 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, first ? zero : c11, 0, 0, 0);        \
+        /* 128 of the 168 registers are accumulators: keep the operands of later steps out */    \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+      }                                                                                           \
+    }                                                                                             \
+    if ((G) == 3) {                                                                               \
+      const float *dp = d_l + 64u * wr + 4u * lh;                                                 \
+      GW_SB_TILE(y00, c00, ra, tl, adv0, 0);                                                      \
+      GW_SB_TILE(y01, c01, ra, tl + 32u, adv1, 0);                                                \
+      GW_SB_TILE(y10, c10, ra + 32u, tl, adv0, 32);                                               \
+      GW_SB_TILE(y11, c11, ra + 32u, tl + 32u, adv1, 32);                                         \
+    }                                                                                             \
+    __syncthreads();                                                                              \
+  } while (0)
+
+  // isum = c + corr (one rounding of the exact integer), then the reference's f32 steps
+#define GW_SB_TILE(Y, C, ROW, TOK, ADV, DO)                                                       \
+  do {                                                                                            \
+    const half8 a2 = *(const half8 *)(a2_l + (ROW) * 16u + 8u * lh);                              \
+    const half8 b2 = *(const half8 *)(b2_l + (TOK) * 16u + 8u * lh);                              \
+    const float16v corr = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2, zero, 0, 0, 0);          \
+    _Pragma("unroll") for (int q4 = 0; q4 < 4; q4++) {                                            \
+      const float4 d = *(const float4 *)(dp + (DO) + 8 * q4);                                     \
+      Y[4 * q4 + 0] += ADV * (d.x * (C[4 * q4 + 0] + corr[4 * q4 + 0]));                          \
+      Y[4 * q4 + 1] += ADV * (d.y * (C[4 * q4 + 1] + corr[4 * q4 + 1]));                          \
+      Y[4 * q4 + 2] += ADV * (d.z * (C[4 * q4 + 2] + corr[4 * q4 + 2]));                          \
+      Y[4 * q4 + 3] += ADV * (d.w * (C[4 * q4 + 3] + corr[4 * q4 + 3]));                          \
+    }                                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+  } while (0)
+
+#pragma unroll 1
+  for (uint32_t s = 0; s < p.nsb; s++) {
+    GW_CONSUME(0);
+    GW_CONSUME(1);
+    GW_CONSUME(2);
+    GW_CONSUME(3);
+  }
+#undef GW_CONSUME
+#undef GW_SB_TILE
+
+  // ---------------- store: a lane holds one token column per token tile and its rows in runs of four
+  const bool vec = (p.out_dim & 3u) == 0;
+#define GW_STORE_TILE(Y, TI, RI)                                                                  \
+  do {                                                                                            \
+    const uint32_t t = t0 + tl + 32u * (TI);                                                      \
+    if (t < p.n_tokens) {                                                                         \
+      _Pragma("unroll") for (int q4 = 0; q4 < 4; q4++) {                                          \
+        const uint32_t row = r0 + 64u * wr + 32u * (RI) + 8u * q4 + 4u * lh;                      \
+        float *dst = p.y + (size_t)t * p.out_dim + row;                                           \
+        if (vec && row + 3u < p.out_dim) {                                                        \
+          *(float4 *)dst = make_float4(Y[4 * q4], Y[4 * q4 + 1], Y[4 * q4 + 2], Y[4 * q4 + 3]);   \
+        } else {                                                                                  \
+          _Pragma("unroll") for (int e = 0; e < 4; e++)                                           \
+            if (row + e < p.out_dim) dst[e] = Y[4 * q4 + e];                                      \
+        }                                                                                         \
+      }                                                                                           \
+    }                                                                                             \
+  } while (0)
+  GW_STORE_TILE(y00, 0, 0);
+  GW_STORE_TILE(y01, 1, 0);
+  GW_STORE_TILE(y10, 0, 1);
+  GW_STORE_TILE(y11, 1, 1);
+#undef GW_STORE_TILE
+}
+
+// ------------------------------------------------------------------------------------------
 // Q6_K (gemm_k_q6_k, engine/vecdot.rs:2352-2398): acc += ad * (d * sum_g sc_g * dot16(q_g - 32, x_g))
 // over the 16 groups of a super-block, sc_g a signed byte.
 //
@@ -677,8 +1035,11 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   const size_t n8 = (size_t)a.in_dim * a.n_tokens / 8, n_sb = (size_t)nsb * a.n_tokens;
   _Float16 *xh = (_Float16 *)a.xh;
   _Float16 *bs16 = xh + (size_t)a.in_dim * a.n_tokens;
-  hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, stream,
-                     a.act.q, a.act.bsum, xh, bs16, n8, n_sb);
+  // Q4_K beyond two token tiles of 128 runs the wide kernel, which reads the int8 activations as
+  // they are and needs only the (bh, bl) pairs prepared
+  const bool wide = a.ggml_type == OGM_Q4_K && a.n_tokens > 256u;
+  hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((wide ? n_sb : n8) + 255) / 256)), dim3(256), 0,
+                     stream, a.act.q, a.act.bsum, wide ? (_Float16 *)nullptr : xh, bs16, n8, n_sb);
   const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
   const uint32_t c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
   // token tiles vary fastest: workgroups that run together share weight rows, and with a
@@ -719,6 +1080,16 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   p.c_shift = c_shift;
   p.r_shift = 6 - c_shift;
   p.nct = tl.nct;
+  p.xq = a.act.q;
+  if (wide) {
+    const dim3 wgrid((a.n_tokens + GW_BT - 1) / GW_BT, (a.out_dim + GM_BN - 1) / GM_BN);
+    e = hipFuncSetAttribute((const void *)ogm_gemm_q4k_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)GW_LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(ogm_gemm_q4k_wide_kernel, wgrid, dim3(768), GW_LDS_BYTES, stream, p);
+    if (kernel_name) *kernel_name = "ogm_gemm_q4k_wide_kernel";
+    return hipGetLastError();
+  }
   const uint32_t lds4 = GM_LDS_BYTES + nsb * 512u;   // + pass 1's table of dmin
   e = hipFuncSetAttribute((const void *)ogm_gemm_q4k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)GM_LDS_MAX);

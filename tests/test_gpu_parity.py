@@ -316,6 +316,7 @@ def test_q6k_vocab_projection_batches_1_4_8(be):
 @pytest.mark.parametrize("in_dim,out_dim,T", [
     (1024, 64, 9), (1024, 100, 64), (2048, 37, 128), (4096, 200, 130), (1024, 16, 300), (8192, 70, 33),
     (256, 5, 9), (512, 130, 17), (768, 64, 129), (1280, 257, 40), (14336, 96, 257), (4096, 1000, 512),
+    (256, 5, 257), (2304, 130, 600), (4096, 257, 1030), (1024, 129, 256), (512, 64, 513),
 ])
 def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     """ogm_matmul at n_tokens >= 9 takes the MFMA kernel; values must equal CpuBackend's K-quant
@@ -325,7 +326,8 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     w = qm(raw, Q4_K, in_dim, out_dim)
     say("gemm", in_dim, out_dim, T)
     got = be.matmul(x, T, w)
-    assert be.last_kernel() == "ogm_gemm_q4k_kernel"
+    # beyond 256 tokens the 128 x 256 tile kernel runs
+    assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 else "ogm_gemm_q4k_kernel")
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     assert_close(got, want, "mfma gemm")
     assert_bits(got, want, "mfma gemm")
@@ -351,14 +353,15 @@ def test_mfma_gemm_equals_small_batch_kernel_and_is_batch_independent(be):
         assert_bits(part, full[:n], f"{n} of 40")
 
 
+@pytest.mark.parametrize("T", [16, 272])
 @pytest.mark.parametrize("qs_lo,qs_hi,sign", [(0xFF, 0xFF, "alt"), (0x00, 0x00, "alt"), (0x0F, 0xF0, "pos"),
                                                (0xF0, 0x0F, "neg"), (0xFF, 0x00, "block")])
-def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign):
+def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T):
     """Largest magnitudes the integer stage can see: nibbles 0 or 15, scales and mins 63, activations
     +-127.  The per-super-block sum reaches 3.1e7 > 2^24 and the centred partial sums and their
     correction reach +-1.64e7 each (and cancel when every nibble is 0), so the f32 add of the exact
     parts must round exactly like `isum as f32`."""
-    in_dim, out_dim, T = 1024, 32, 16
+    in_dim, out_dim = 1024, 32
     blocks = np.zeros((out_dim * 4, 144), np.uint8)
     blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
     blocks[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
@@ -376,7 +379,7 @@ def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign):
         x[3] = -127.0
     raw = blocks.reshape(-1)
     got = be.matmul(x, T, qm(raw, Q4_K, in_dim, out_dim))
-    assert be.last_kernel() == "ogm_gemm_q4k_kernel"
+    assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 else "ogm_gemm_q4k_kernel")
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     assert_bits(got, want, "extreme ranges")
     isum, imin = be.dump_block_sums(x[0], 1, qm(raw, Q4_K, in_dim, out_dim))
