@@ -445,12 +445,10 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q4k_kernel(GemmParams p) {
 
 #define GW_BT 256u           // tokens per workgroup
 #define GW_PG 8u             // super-blocks per pass-1 group
-// Staged tiles are padded by one 16-byte chunk per row (weights: 64 f16 + 8, activations: 64 bytes
-// + 16).  Sixteen consecutive rows then start 36 (or 20) banks apart, which puts their 16-byte
-// accesses on sixteen disjoint groups of four banks, and a chunk's position is a compile-time
-// offset from the row's address: no swizzle arithmetic in the loop.
-#define GW_A_ROW 72u                     // f16 per staged weight row
-#define GW_B_ROW 80u                     // bytes per staged activation row
+// Staged tiles are unpadded; the 16-byte chunk c of a weight row r sits at gm_swz(r, c), of an
+// activation row t (64 bytes) at chunk c ^ ((t >> 2) & 3).
+#define GW_A_ROW 64u                     // f16 per staged weight row
+#define GW_B_ROW 64u                     // bytes per staged activation row
 #define GW_A_STAGE (128u * GW_A_ROW)     // f16 per staged weight tile (18 KB)
 #define GW_B_STAGE (256u * GW_B_ROW)     // bytes per staged activation tile (20 KB)
 // main loop: A [2] 36 KB | B [2] 40 KB | a2 4 KB | b2 8 KB | d 512 B
@@ -461,8 +459,9 @@ static const uint32_t GW_LDS_BYTES = 32768u + 65536u + 4096u + 8192u;
 
 // Eight activations (two dwords of x + 128, as the feeding waves store them) -> eight f16, exact:
 // 0x6400 | u is the f16 1024 + u, and 1024 + (x + 128) - 1152 = x.
-__device__ __forceinline__ half8 gw_u8_to_f16(uint32_t u0, uint32_t u1) {
+__device__ __forceinline__ half8 gw_u8_to_f16(uint32_t w0, uint32_t w1) {
   union { uint32_t u[4]; half8 h; half2v p[4]; } r;
+  const uint32_t u0 = w0 ^ 0x80808080u, u1 = w1 ^ 0x80808080u;
   r.u[0] = __builtin_amdgcn_perm(0x64646464u, u0, 0x04010400u);  // (b0, 0x64, b1, 0x64)
   r.u[1] = __builtin_amdgcn_perm(0x64646464u, u0, 0x04030402u);
   r.u[2] = __builtin_amdgcn_perm(0x64646464u, u1, 0x04010400u);
@@ -577,8 +576,7 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
   const uint32_t bo1 = min(t0 + btok + 64u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
   const uint32_t bo2 = min(t0 + btok + 128u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
   const uint32_t bo3 = min(t0 + btok + 192u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
-  const uint32_t bso = btok * GW_B_ROW + 16u * bch;       // byte offset in a staged activation tile
-  const uint32_t aso = arow * GW_A_ROW + 16u * ah;        // f16 offset of chunk 2 ah in a staged weight tile
+  const uint32_t bso = btok * 64u + ((bch ^ ((btok >> 2) & 3u)) << 4);   // tokens 64 apart share the chunk swizzle
   const uint32_t tok2 = rt >> 1, hf2 = rt & 1u;
   const uint32_t b2o0 = min(t0 + tok2, p.n_tokens - 1u) * p.nsb * 16u + 8u * hf2;
   const uint32_t b2o1 = min(t0 + tok2 + 128u, p.n_tokens - 1u) * p.nsb * 16u + 8u * hf2;
@@ -624,16 +622,16 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
     dequant8(qv_##K.w, sl2_, sh2_, lb_.z, lb_.w, hb_.z, hb_.w);                                   \
     /* piece 1+2g+ah holds qs[32g+16ah ..]: low nibbles are k 16ah.. of the stage, high 32+16ah.. */ \
     _Float16 *ab_ = A_l + (BUF) * GW_A_STAGE;                                                     \
-    *(uint4 *)(ab_ + aso) = la_;              /* chunk 2 ah */                                    \
-    *(uint4 *)(ab_ + aso + 8u) = lb_;                                                             \
-    *(uint4 *)(ab_ + aso + 32u) = ha_;        /* chunk 4 + 2 ah */                                \
-    *(uint4 *)(ab_ + aso + 40u) = hb_;                                                            \
+    *(uint4 *)(ab_ + gm_swz(arow, 2u * ah)) = la_;                                                \
+    *(uint4 *)(ab_ + gm_swz(arow, 2u * ah + 1u)) = lb_;                                           \
+    *(uint4 *)(ab_ + gm_swz(arow, 4u + 2u * ah)) = ha_;                                           \
+    *(uint4 *)(ab_ + gm_swz(arow, 5u + 2u * ah)) = hb_;                                           \
     uint8_t *bb_ = B_l + (BUF) * GW_B_STAGE;                                                      \
     /* stored as x + 128: the multiplying waves' conversion starts from unsigned bytes */         \
-    *(uint4 *)(bb_ + bso) = gw_bias128(bxa_##K);                                                  \
-    *(uint4 *)(bb_ + bso + 64u * GW_B_ROW) = gw_bias128(bxb_##K);                                 \
-    *(uint4 *)(bb_ + bso + 128u * GW_B_ROW) = gw_bias128(bxc_##K);                                \
-    *(uint4 *)(bb_ + bso + 192u * GW_B_ROW) = gw_bias128(bxd_##K);                                \
+    *(uint4 *)(bb_ + bso) = bxa_##K;                                                  \
+    *(uint4 *)(bb_ + bso + 64u * GW_B_ROW) = bxb_##K;                                 \
+    *(uint4 *)(bb_ + bso + 128u * GW_B_ROW) = bxc_##K;                                \
+    *(uint4 *)(bb_ + bso + 192u * GW_B_ROW) = bxd_##K;                                \
     if ((G) == 1) {                                                                               \
       /* side tables of this super-block: their last readers are two barriers behind, their      \
          next readers two barriers ahead; the two threads of a row write the same d */           \
@@ -655,7 +653,6 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
   if (producer) {
     // the feeding wave of a SIMD has little to do per stage but everybody waits for it at the
     // barrier: let it go first
-    __builtin_amdgcn_s_setprio(3);
     GW_LOAD_STAGE(0u, 0u, 0);
     GW_LOAD_STAGE(0u, 1u, 1);
     GW_LOAD_STAGE(0u, 2u, 2);
@@ -689,8 +686,7 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
 
   // ---- multiplying waves
   const uint32_t tk0 = min(t0 + tl, p.n_tokens - 1u), tk1 = min(t0 + tl + 32u, p.n_tokens - 1u);
-  const uint32_t aro = ra * GW_A_ROW + 16u * lh;   // f16 offset of chunk 2 lh of row ra
-  const uint32_t bro = tl * GW_B_ROW + 16u * lh;   // byte offset of chunk lh of token tl
+  const uint32_t bsw = (tl >> 2) & 3u;   // chunk swizzle of this lane's tokens (the same for tl + 32)
   float16v c00, c01, c10, c11;
   float adv0 = 0.0f, adv1 = 0.0f;
 
@@ -704,12 +700,12 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
     const _Float16 *ab = A_l + buf * GW_A_STAGE;                                                  \
     const uint8_t *bb = B_l + buf * GW_B_STAGE;                                                   \
     _Pragma("unroll") for (int m = 0; m < 2; m++) {                                               \
-      const uint4 bq0 = *(const uint4 *)(bb + bro + 32u * m);                                     \
-      const uint4 bq1 = *(const uint4 *)(bb + bro + 32u * GW_B_ROW + 32u * m);                    \
+      const uint4 bq0 = *(const uint4 *)(bb + tl * 64u + (((2u * m + lh) ^ bsw) << 4));           \
+      const uint4 bq1 = *(const uint4 *)(bb + (tl + 32u) * 64u + (((2u * m + lh) ^ bsw) << 4));   \
       _Pragma("unroll") for (int e = 0; e < 2; e++) {                                             \
         /* chunk 4 m + 2 lh + e of rows ra and ra + 32 */                                         \
-        const half8 a0 = *(const half8 *)(ab + aro + 32u * m + 8u * e);                           \
-        const half8 a1 = *(const half8 *)(ab + aro + 32u * GW_A_ROW + 32u * m + 8u * e);          \
+        const half8 a0 = *(const half8 *)(ab + gm_swz(ra, 4u * m + 2u * lh + e));                 \
+        const half8 a1 = *(const half8 *)(ab + gm_swz(ra + 32u, 4u * m + 2u * lh + e));           \
         /* the super-block's first step starts fresh accumulators */                             \
         const bool first = (G) == 0 && m == 0 && e == 0;                                          \
         const half8 b0 = e ? gw_u8_to_f16(bq0.z, bq0.w) : gw_u8_to_f16(bq0.x, bq0.y);             \
@@ -718,26 +714,26 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
         const half8 b1 = e ? gw_u8_to_f16(bq1.z, bq1.w) : gw_u8_to_f16(bq1.x, bq1.y);             \
         c01 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b1, first ? zero : c01, 0, 0, 0);        \
         c11 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, first ? zero : c11, 0, 0, 0);        \
-        /* 128 of the 168 registers are accumulators: keep the operands of later steps out */    \
-        __builtin_amdgcn_sched_barrier(0);                                                        \
       }                                                                                           \
     }                                                                                             \
     if ((G) == 3) {                                                                               \
+      const half8 b20 = *(const half8 *)(b2_l + tl * 16u + 8u * lh);                              \
+      const half8 b21 = *(const half8 *)(b2_l + (tl + 32u) * 16u + 8u * lh);                      \
+      const half8 a20 = *(const half8 *)(a2_l + ra * 16u + 8u * lh);                              \
+      const half8 a21 = *(const half8 *)(a2_l + (ra + 32u) * 16u + 8u * lh);                      \
       const float *dp = d_l + 64u * wr + 4u * lh;                                                 \
-      GW_SB_TILE(y00, c00, ra, tl, adv0, 0);                                                      \
-      GW_SB_TILE(y01, c01, ra, tl + 32u, adv1, 0);                                                \
-      GW_SB_TILE(y10, c10, ra + 32u, tl, adv0, 32);                                               \
-      GW_SB_TILE(y11, c11, ra + 32u, tl + 32u, adv1, 32);                                         \
+      GW_SB_TILE(y00, c00, a20, b20, adv0, 0);                                                    \
+      GW_SB_TILE(y01, c01, a20, b21, adv1, 0);                                                    \
+      GW_SB_TILE(y10, c10, a21, b20, adv0, 32);                                                   \
+      GW_SB_TILE(y11, c11, a21, b21, adv1, 32);                                                   \
     }                                                                                             \
     __syncthreads();                                                                              \
   } while (0)
 
   // isum = c + corr (one rounding of the exact integer), then the reference's f32 steps
-#define GW_SB_TILE(Y, C, ROW, TOK, ADV, DO)                                                       \
+#define GW_SB_TILE(Y, C, A2, B2, ADV, DO)                                                         \
   do {                                                                                            \
-    const half8 a2 = *(const half8 *)(a2_l + (ROW) * 16u + 8u * lh);                              \
-    const half8 b2 = *(const half8 *)(b2_l + (TOK) * 16u + 8u * lh);                              \
-    const float16v corr = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2, zero, 0, 0, 0);          \
+    const float16v corr = __builtin_amdgcn_mfma_f32_32x32x16_f16(A2, B2, zero, 0, 0, 0);          \
     _Pragma("unroll") for (int q4 = 0; q4 < 4; q4++) {                                            \
       const float4 d = *(const float4 *)(dp + (DO) + 8 * q4);                                     \
       Y[4 * q4 + 0] += ADV * (d.x * (C[4 * q4 + 0] + corr[4 * q4 + 0]));                          \
@@ -745,7 +741,6 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
       Y[4 * q4 + 2] += ADV * (d.z * (C[4 * q4 + 2] + corr[4 * q4 + 2]));                          \
       Y[4 * q4 + 3] += ADV * (d.w * (C[4 * q4 + 3] + corr[4 * q4 + 3]));                          \
     }                                                                                             \
-    __builtin_amdgcn_sched_barrier(0);                                                            \
   } while (0)
 
 #pragma unroll 1
