@@ -434,7 +434,9 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q4k_kernel(GemmParams p) {
 // tiles, so the same reads feed twice the MFMAs), the activations stay int8 in LDS (half the
 // bytes; the multiplying wave turns them into f16 with the 0x6400 | (x + 128) = 1024 + (x + 128)
 // trick, exact), and a workgroup has eight multiplying and four feeding waves, three per SIMD,
-// which leaves 168 registers per lane for the four integer-sum and four f32 accumulator tiles.
+// which leaves 168 registers per lane.  The four integer-sum and four f32 accumulator tiles take
+// 128 of them, so the loop is written to keep little else alive (a fence after every MFMA step
+// keeps later steps' LDS reads from being hoisted; without it accumulators spill).
 //
 // k order inside a stage: MFMA step kk of the lane half lh covers k = 32 (kk >> 1) + 16 lh +
 // 8 (kk & 1) + 0..7, so that a lane's activations for two steps are 16 contiguous bytes.
@@ -445,10 +447,12 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q4k_kernel(GemmParams p) {
 
 #define GW_BT 256u           // tokens per workgroup
 #define GW_PG 8u             // super-blocks per pass-1 group
-// Staged tiles are unpadded; the 16-byte chunk c of a weight row r sits at gm_swz(r, c), of an
-// activation row t (64 bytes) at chunk c ^ ((t >> 2) & 3).
-#define GW_A_ROW 64u                     // f16 per staged weight row
-#define GW_B_ROW 64u                     // bytes per staged activation row
+// Staged tiles are padded by one 16-byte chunk per row (weights: 64 f16 + 8, activations: 64 bytes
+// + 16).  Sixteen consecutive rows then start 36 (or 20) banks apart, which puts their 16-byte
+// accesses on sixteen disjoint groups of four banks, and a chunk's position is a compile-time
+// offset from the row's address: no swizzle arithmetic in the loop.
+#define GW_A_ROW 72u                     // f16 per staged weight row
+#define GW_B_ROW 80u                     // bytes per staged activation row
 #define GW_A_STAGE (128u * GW_A_ROW)     // f16 per staged weight tile (18 KB)
 #define GW_B_STAGE (256u * GW_B_ROW)     // bytes per staged activation tile (20 KB)
 // main loop: A [2] 36 KB | B [2] 40 KB | a2 4 KB | b2 8 KB | d 512 B
@@ -457,9 +461,9 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q4k_kernel(GemmParams p) {
 #define GW_SIDE_OFF (GW_B_OFF + 2u * GW_B_STAGE)     // bytes
 static const uint32_t GW_LDS_BYTES = 32768u + 65536u + 4096u + 8192u;
 
-// Eight activations (two dwords of x + 128, as the feeding waves store them) -> eight f16, exact:
-// 0x6400 | u is the f16 1024 + u, and 1024 + (x + 128) - 1152 = x.
-__device__ __forceinline__ half8 gw_u8_to_f16(uint32_t w0, uint32_t w1) {
+// Eight int8 activations (two dwords) -> eight f16, exact: with u = x + 128 (the sign bit flipped),
+// 0x6400 | u is the f16 1024 + u, and 1024 + u - 1152 = x.
+__device__ __forceinline__ half8 gw_i8_to_f16(uint32_t w0, uint32_t w1) {
   union { uint32_t u[4]; half8 h; half2v p[4]; } r;
   const uint32_t u0 = w0 ^ 0x80808080u, u1 = w1 ^ 0x80808080u;
   r.u[0] = __builtin_amdgcn_perm(0x64646464u, u0, 0x04010400u);  // (b0, 0x64, b1, 0x64)
@@ -470,10 +474,6 @@ __device__ __forceinline__ half8 gw_u8_to_f16(uint32_t w0, uint32_t w1) {
 #pragma unroll
   for (int i = 0; i < 4; i++) r.p[i] = r.p[i] + k;
   return r.h;
-}
-
-__device__ __forceinline__ uint4 gw_bias128(uint4 v) {
-  return make_uint4(v.x ^ 0x80808080u, v.y ^ 0x80808080u, v.z ^ 0x80808080u, v.w ^ 0x80808080u);
 }
 
 __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
@@ -576,7 +576,8 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
   const uint32_t bo1 = min(t0 + btok + 64u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
   const uint32_t bo2 = min(t0 + btok + 128u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
   const uint32_t bo3 = min(t0 + btok + 192u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
-  const uint32_t bso = btok * 64u + ((bch ^ ((btok >> 2) & 3u)) << 4);   // tokens 64 apart share the chunk swizzle
+  const uint32_t bso = btok * GW_B_ROW + 16u * bch;       // byte offset in a staged activation tile
+  const uint32_t aso = arow * GW_A_ROW + 16u * ah;        // f16 offset of chunk 2 ah in a staged weight tile
   const uint32_t tok2 = rt >> 1, hf2 = rt & 1u;
   const uint32_t b2o0 = min(t0 + tok2, p.n_tokens - 1u) * p.nsb * 16u + 8u * hf2;
   const uint32_t b2o1 = min(t0 + tok2 + 128u, p.n_tokens - 1u) * p.nsb * 16u + 8u * hf2;
@@ -622,10 +623,10 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
     dequant8(qv_##K.w, sl2_, sh2_, lb_.z, lb_.w, hb_.z, hb_.w);                                   \
     /* piece 1+2g+ah holds qs[32g+16ah ..]: low nibbles are k 16ah.. of the stage, high 32+16ah.. */ \
     _Float16 *ab_ = A_l + (BUF) * GW_A_STAGE;                                                     \
-    *(uint4 *)(ab_ + gm_swz(arow, 2u * ah)) = la_;                                                \
-    *(uint4 *)(ab_ + gm_swz(arow, 2u * ah + 1u)) = lb_;                                           \
-    *(uint4 *)(ab_ + gm_swz(arow, 4u + 2u * ah)) = ha_;                                           \
-    *(uint4 *)(ab_ + gm_swz(arow, 5u + 2u * ah)) = hb_;                                           \
+    *(uint4 *)(ab_ + aso) = la_;              /* chunk 2 ah */                                    \
+    *(uint4 *)(ab_ + aso + 8u) = lb_;                                                             \
+    *(uint4 *)(ab_ + aso + 32u) = ha_;        /* chunk 4 + 2 ah */                                \
+    *(uint4 *)(ab_ + aso + 40u) = hb_;                                                            \
     uint8_t *bb_ = B_l + (BUF) * GW_B_STAGE;                                                      \
     /* stored as x + 128: the multiplying waves' conversion starts from unsigned bytes */         \
     *(uint4 *)(bb_ + bso) = bxa_##K;                                                  \
@@ -686,7 +687,8 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
 
   // ---- multiplying waves
   const uint32_t tk0 = min(t0 + tl, p.n_tokens - 1u), tk1 = min(t0 + tl + 32u, p.n_tokens - 1u);
-  const uint32_t bsw = (tl >> 2) & 3u;   // chunk swizzle of this lane's tokens (the same for tl + 32)
+  const uint32_t aro = ra * GW_A_ROW + 16u * lh;   // f16 offset of chunk 2 lh of row ra
+  const uint32_t bro = tl * GW_B_ROW + 16u * lh;   // byte offset of chunk lh of token tl
   float16v c00, c01, c10, c11;
   float adv0 = 0.0f, adv1 = 0.0f;
 
@@ -700,20 +702,21 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
     const _Float16 *ab = A_l + buf * GW_A_STAGE;                                                  \
     const uint8_t *bb = B_l + buf * GW_B_STAGE;                                                   \
     _Pragma("unroll") for (int m = 0; m < 2; m++) {                                               \
-      const uint4 bq0 = *(const uint4 *)(bb + tl * 64u + (((2u * m + lh) ^ bsw) << 4));           \
-      const uint4 bq1 = *(const uint4 *)(bb + (tl + 32u) * 64u + (((2u * m + lh) ^ bsw) << 4));   \
+      const uint4 bq0 = *(const uint4 *)(bb + bro + 32u * m);                                     \
+      const uint4 bq1 = *(const uint4 *)(bb + bro + 32u * GW_B_ROW + 32u * m);                    \
       _Pragma("unroll") for (int e = 0; e < 2; e++) {                                             \
         /* chunk 4 m + 2 lh + e of rows ra and ra + 32 */                                         \
-        const half8 a0 = *(const half8 *)(ab + gm_swz(ra, 4u * m + 2u * lh + e));                 \
-        const half8 a1 = *(const half8 *)(ab + gm_swz(ra + 32u, 4u * m + 2u * lh + e));           \
+        const half8 a0 = *(const half8 *)(ab + aro + 32u * m + 8u * e);                           \
+        const half8 a1 = *(const half8 *)(ab + aro + 32u * GW_A_ROW + 32u * m + 8u * e);          \
         /* the super-block's first step starts fresh accumulators */                             \
         const bool first = (G) == 0 && m == 0 && e == 0;                                          \
-        const half8 b0 = e ? gw_u8_to_f16(bq0.z, bq0.w) : gw_u8_to_f16(bq0.x, bq0.y);             \
+        const half8 b0 = e ? gw_i8_to_f16(bq0.z, bq0.w) : gw_i8_to_f16(bq0.x, bq0.y);             \
         c00 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b0, first ? zero : c00, 0, 0, 0);        \
         c10 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, first ? zero : c10, 0, 0, 0);        \
-        const half8 b1 = e ? gw_u8_to_f16(bq1.z, bq1.w) : gw_u8_to_f16(bq1.x, bq1.y);             \
+        const half8 b1 = e ? gw_i8_to_f16(bq1.z, bq1.w) : gw_i8_to_f16(bq1.x, bq1.y);             \
         c01 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b1, first ? zero : c01, 0, 0, 0);        \
         c11 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, first ? zero : c11, 0, 0, 0);        \
+        asm volatile("" ::: "memory");  /* later steps' LDS reads stay behind */                  \
       }                                                                                           \
     }                                                                                             \
     if ((G) == 3) {                                                                               \
