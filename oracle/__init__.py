@@ -16,8 +16,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liborangu_oracle.so")
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-BLOCK_LAYOUT = {Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256)}
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+BLOCK_LAYOUT = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
 
 
 def build() -> str:
@@ -65,6 +65,8 @@ def lib() -> C.CDLL:
         L.ogo_dot_q6_k.argtypes = [u8p, sz, i8p, f32p]
         L.ogo_dot_k_row_q4_k.restype = C.c_float
         L.ogo_dot_k_row_q4_k.argtypes = [u8p, sz, i8p, f32p, i32p, i32p, i32p]
+        L.ogo_dot_k_row_q5_k.restype = C.c_float
+        L.ogo_dot_k_row_q5_k.argtypes = [u8p, sz, i8p, f32p, i32p, i32p, i32p]
         L.ogo_dot_k_row_q6_k.restype = C.c_float
         L.ogo_dot_k_row_q6_k.argtypes = [u8p, sz, i8p, f32p, i32p]
         L.ogo_block_sums_q8_0.argtypes = [u8p, sz, i8p, i32p]
@@ -225,6 +227,8 @@ def dot_k_row(ggml_type: int, row, act, want_sums: bool = False):
     L = lib()
     if ggml_type == Q4_K:
         v = L.ogo_dot_k_row_q4_k(_p(r), n, _p(q), _p(d), _p(s), _p(isum), _p(imin))
+    elif ggml_type == Q5_K:
+        v = L.ogo_dot_k_row_q5_k(_p(r), n, _p(q), _p(d), _p(s), _p(isum), _p(imin))
     elif ggml_type == Q6_K:
         v = L.ogo_dot_k_row_q6_k(_p(r), n, _p(q), _p(d), _p(isum))
     else:
@@ -293,7 +297,7 @@ def k_gemm_t(ggml_type, raw, in_dim, out_dim, x, n_tokens) -> np.ndarray:
 
 
 def block_sums(ggml_type, raw, in_dim, out_dim, x, n_tokens=1):
-    """Integer stage only: isum (and imin for Q4_K) as [n_tokens][out_dim][n_blocks]."""
+    """Integer stage only: isum (and imin for Q4_K and Q5_K) as [n_tokens][out_dim][n_blocks]."""
     raw = _u8(raw)
     x = _f32(x)
     bb, be = BLOCK_LAYOUT[ggml_type]

@@ -67,6 +67,7 @@ int ogo_block_layout(uint32_t ggml_type, size_t *block_bytes, size_t *block_elem
     case OGO_TYPE_F16: bb = 2; be = 1; break;
     case OGO_TYPE_Q8_0: bb = 2 + 32; be = 32; break;
     case OGO_TYPE_Q4_K: bb = 2 + 2 + 12 + 128; be = 256; break;
+    case OGO_TYPE_Q5_K: bb = 2 + 2 + 12 + 32 + 128; be = 256; break;
     case OGO_TYPE_Q6_K: bb = 128 + 64 + 16 + 2; be = 256; break;
     default: return -1;
   }
@@ -116,6 +117,34 @@ static void dequantize_q4_k(const uint8_t *bytes, size_t n, float *out) {
   }
 }
 
+/* quant.rs:703-742: Q4_K plus a fifth bit; bit j of qh[l] belongs to element l of sub-block j */
+static void dequantize_q5_k(const uint8_t *bytes, size_t n, float *out) {
+  for (size_t s = 0; s < n / 256; s++) {
+    const uint8_t *block = bytes + s * 176;
+    float d = read_f16(block, 0);
+    float dmin = read_f16(block, 2);
+    const uint8_t *scales = block + 4;
+    const uint8_t *qh = block + 16;
+    const uint8_t *qs = block + 48;
+    float *o = out + s * 256;
+    int is = 0;
+    uint8_t u1 = 1, u2 = 2;
+    for (int q_offset = 0; q_offset < 256; q_offset += 64) {
+      uint8_t sc1, m1, sc2, m2;
+      ogo_get_scale_min_k4(is, scales, &sc1, &m1);
+      float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
+      ogo_get_scale_min_k4(is + 1, scales, &sc2, &m2);
+      float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
+      const uint8_t *ql = qs + q_offset / 2;
+      for (int l = 0; l < 32; l++) *o++ = d1 * (float)((int)(ql[l] & 0x0F) + ((qh[l] & u1) ? 16 : 0)) - mm1;
+      for (int l = 0; l < 32; l++) *o++ = d2 * (float)((int)(ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - mm2;
+      is += 2;
+      u1 = (uint8_t)(u1 << 2);
+      u2 = (uint8_t)(u2 << 2);
+    }
+  }
+}
+
 /* quant.rs:746-787 */
 static void dequantize_q6_k(const uint8_t *bytes, size_t n, float *out) {
   for (size_t s = 0; s < n / 256; s++) {
@@ -152,6 +181,7 @@ int ogo_dequantize(uint32_t ggml_type, const uint8_t *bytes, size_t element_coun
   switch (ggml_type) {
     case OGO_TYPE_Q8_0: dequantize_q8_0(bytes, element_count, out); return 0;
     case OGO_TYPE_Q4_K: dequantize_q4_k(bytes, element_count, out); return 0;
+    case OGO_TYPE_Q5_K: dequantize_q5_k(bytes, element_count, out); return 0;
     case OGO_TYPE_Q6_K: dequantize_q6_k(bytes, element_count, out); return 0;
     default: return -1;
   }
@@ -378,6 +408,34 @@ static void unpack_k_q4_k(const uint8_t *row, size_t in_dim, ogo_krow *out) {
   }
 }
 
+/* vecdot.rs:2064-2088 unpack_k_q5_k: unpack_k_q4_k with the high-bit plane applied */
+static void unpack_k_q5_k(const uint8_t *row, size_t in_dim, ogo_krow *out) {
+  size_t sb = 0;
+  for (size_t s = 0; s < in_dim / 256; s++) {
+    const uint8_t *block = row + s * 176;
+    out->d[s] = read_f16(block, 0);
+    out->dmin[s] = read_f16(block, 2);
+    const uint8_t *scales = block + 4;
+    const uint8_t *qh = block + 16;
+    const uint8_t *qs = block + 48;
+    for (int g = 0; g < 4; g++) {
+      const uint8_t *bytes = qs + g * 32;
+      for (int half = 0; half < 2; half++) {
+        int shift = half ? 4 : 0;
+        uint8_t sc, m;
+        ogo_get_scale_min_k4(g * 2 + half, scales, &sc, &m);
+        uint8_t hi_mask = (uint8_t)(1u << (g * 2 + half));
+        int8_t *w = out->q + (sb + (size_t)half) * 32;
+        for (int j = 0; j < 32; j++)
+          w[j] = (int8_t)(((bytes[j] >> shift) & 0x0F) + ((qh[j] & hi_mask) ? 16 : 0));
+        out->sc[sb + (size_t)half] = (int16_t)sc;
+        out->mins[sb + (size_t)half] = (int16_t)m;
+      }
+      sb += 2;
+    }
+  }
+}
+
 /* vecdot.rs:2119-2143 unpack_k_q6_k */
 static void unpack_k_q6_k(const uint8_t *row, size_t in_dim, ogo_krow *out) {
   for (size_t s = 0; s < in_dim / 256; s++) {
@@ -478,6 +536,10 @@ float ogo_dot_k_row_q4_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
                          const int32_t *sums, int32_t *isum_out, int32_t *imin_out) {
   return DISPATCH(dot_k_row_q4_k, row, in_dim, q, d, sums, isum_out, imin_out);
 }
+float ogo_dot_k_row_q5_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
+                         const int32_t *sums, int32_t *isum_out, int32_t *imin_out) {
+  return DISPATCH(dot_k_row_q5_k, row, in_dim, q, d, sums, isum_out, imin_out);
+}
 float ogo_dot_k_row_q6_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
                          int32_t *isum_out) {
   return DISPATCH(dot_k_row_q6_k, row, in_dim, q, d, isum_out);
@@ -485,19 +547,19 @@ float ogo_dot_k_row_q6_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
 
 /* ------------------------------------------------------------------ predicates */
 
-/* vecdot.rs:274-283, restricted to the three types on the path */
+/* vecdot.rs:274-283, restricted to the types on the path */
 int ogo_supports(uint32_t t, size_t in_dim) {
   if (t == OGO_TYPE_Q8_0) return in_dim % 32 == 0;
-  if (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q6_K) return in_dim % 256 == 0;
+  if (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) return in_dim % 256 == 0;
   return 0;
 }
 /* vecdot.rs:1821-1826 */
 int ogo_supports_k(uint32_t t, size_t in_dim) {
-  return (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
+  return (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
 }
 /* vecdot.rs:3083-3093 */
 int ogo_supports_k_row(uint32_t t, size_t in_dim) {
-  return (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
+  return (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
 }
 /* vecdot.rs:2456-2461 */
 int ogo_supports_flat(uint32_t t, size_t in_dim) { return t == OGO_TYPE_Q8_0 && in_dim % 32 == 0; }
@@ -531,7 +593,7 @@ static void finish_into(float *y, const float *yt, size_t n_tokens, size_t out_d
 /* vecdot.rs:2151-2172 dot_k_pair dispatch by kind */
 static void dot_k_pair(uint32_t ggml_type, const ogo_krow *w0, const ogo_krow *w1,
                        const ogo_actq8k *a, float *out0, float *out1) {
-  if (ggml_type == OGO_TYPE_Q4_K) {
+  if (ggml_type == OGO_TYPE_Q4_K || ggml_type == OGO_TYPE_Q5_K) {   /* both fill a KKind::Q4K row */
     DISPATCH(gemm_k_q4_k, w0, w1, a, out0, out1);
   } else {
     DISPATCH(gemm_k_q6_k, w0, w1, a, out0, out1);
@@ -541,6 +603,8 @@ static void dot_k_pair(uint32_t ggml_type, const ogo_krow *w0, const ogo_krow *w
 static void unpack_k_row(uint32_t ggml_type, const uint8_t *row, size_t in_dim, ogo_krow *out) {
   if (ggml_type == OGO_TYPE_Q4_K) {
     unpack_k_q4_k(row, in_dim, out);
+  } else if (ggml_type == OGO_TYPE_Q5_K) {
+    unpack_k_q5_k(row, in_dim, out);
   } else {
     unpack_k_q6_k(row, in_dim, out);
   }
@@ -682,6 +746,8 @@ static int gemv_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size
       float v;
       if (ggml_type == OGO_TYPE_Q4_K)
         v = DISPATCH(dot_k_row_q4_k, row, in_dim, qt, dt, st, io, mo);
+      else if (ggml_type == OGO_TYPE_Q5_K)
+        v = DISPATCH(dot_k_row_q5_k, row, in_dim, qt, dt, st, io, mo);
       else if (ggml_type == OGO_TYPE_Q6_K)
         v = DISPATCH(dot_k_row_q6_k, row, in_dim, qt, dt, io);
       else
@@ -737,7 +803,7 @@ int ogo_block_sums(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, siz
   float *yt = (float *)malloc(sizeof(float) * out_dim * n_tokens);
   if (!yt) return -3;
   int rc = gemv_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, pick_threads(0),
-                  isum, ggml_type == OGO_TYPE_Q4_K ? imin : NULL);
+                  isum, (ggml_type == OGO_TYPE_Q4_K || ggml_type == OGO_TYPE_Q5_K) ? imin : NULL);
   free(yt);
   return rc;
 }

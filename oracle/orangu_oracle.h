@@ -48,6 +48,7 @@ extern "C" {
 #define OGO_TYPE_F16 1u
 #define OGO_TYPE_Q8_0 8u
 #define OGO_TYPE_Q4_K 12u
+#define OGO_TYPE_Q5_K 13u
 #define OGO_TYPE_Q6_K 14u
 
 #define OGO_ACT_BLOCK 32   /* vecdot.rs ACT_BLOCK */
@@ -95,6 +96,8 @@ float ogo_dot_q6_k(const uint8_t *row, size_t in_dim, const int8_t *q, const flo
 /* per-256 forms; isum_out/imin_out (may be NULL) receive the per-super-block integer sums */
 float ogo_dot_k_row_q4_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
                          const int32_t *sums, int32_t *isum_out, int32_t *imin_out); /* :3152-3178 */
+float ogo_dot_k_row_q5_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
+                         const int32_t *sums, int32_t *isum_out, int32_t *imin_out); /* :3181-3213 */
 float ogo_dot_k_row_q6_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
                          int32_t *isum_out);                                          /* :3215-3241 */
 /* per-32 integer sums of a Q8_0 row (isum_out[in_dim/32]) */

@@ -9,4 +9,5 @@ from .backend import LlamaDecoder, Mi355xBackend, MatmulOp, QuantMatrix  # noqa:
 
 GGML_TYPE_Q8_0 = 8
 GGML_TYPE_Q4_K = 12
+GGML_TYPE_Q5_K = 13
 GGML_TYPE_Q6_K = 14

@@ -684,7 +684,7 @@ extern "C" int ogm_dump_block_sums(ogm_ctx *ctx, const ogm_weight *w, const floa
   const size_t blocks = (size_t)w->in_dim / (w->ggml_type == OGM_Q8_0 ? 32 : 256);
   const size_t nb = (size_t)n_tokens * w->out_dim * blocks * 4;
   const size_t xb = (size_t)n_tokens * w->in_dim * 4, yb = (size_t)n_tokens * w->out_dim * 4;
-  const bool want_min = imin && w->ggml_type == OGM_Q4_K;
+  const bool want_min = imin && (w->ggml_type == OGM_Q4_K || w->ggml_type == OGM_Q5_K);
   if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
   if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
   if ((rc = ensure_dev(ctx, ctx->isum, nb)) != OGM_OK) return rc;

@@ -178,6 +178,104 @@ struct FmtQ4K {
   }
 };
 
+// Q5_K: d:f16 | dmin:f16 | scales:u8[12] | qh:u8[32] | qs:u8[128]          (quant.rs:699-742)
+// Q4_K with a fifth bit: bit j of qh[l] belongs to element l of sub-block j.
+struct FmtQ5K {
+  static constexpr uint32_t TYPE = OGM_Q5_K;
+  static constexpr int PIECES = 11, TILE_BYTES = 64 * 176, ELEMS = 256;
+  static constexpr int XPIECES = 16;
+  static constexpr int AUX16 = 1;      // bsum: 8 x i16 per block
+  static constexpr int ACT_GROUP = 256;
+  static constexpr bool HAS_MIN = true;
+  static constexpr int MAX_THREADS = 512;
+  static constexpr bool HAS_UNPACK = false;
+  struct Regs {
+    uint4 p[PIECES];
+  };
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
+    const uint8_t *base = wt + tile * TILE_BYTES + lane * 16u;
+#pragma unroll
+    for (int i = 0; i < PIECES; i++) r.p[i] = *(const uint4 *)(base + i * 1024);
+  }
+  // Four weights of sub-block `bit`: nibbles n (already masked) plus 16 where the qh bytes have
+  // bit `bit` set.
+  __device__ static __forceinline__ uint32_t with_high(uint32_t n, uint32_t qh, int bit) {
+    return n | (((qh >> bit) & 0x01010101u) << 4);
+  }
+  // isum = sum_j sc_j * dot32(q5_j, x_j), imin = sum_j m_j * bsum_j          (vecdot.rs:3181-3213)
+  template <int UPR>
+  __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
+                                              int &isum, int &imin) {
+    const uint32_t w0 = r.p[0].y, w1 = r.p[0].z, w2 = r.p[0].w;
+    const uint32_t sca = w0 & 0x3F3F3F3Fu;                                   // sc 0..3
+    const uint32_t mna = w1 & 0x3F3F3F3Fu;                                   // m  0..3
+    const uint32_t scb = (w2 & 0x0F0F0F0Fu) | ((w0 >> 2) & 0x30303030u);     // sc 4..7
+    const uint32_t mnb = ((w2 >> 4) & 0x0F0F0F0Fu) | ((w1 >> 2) & 0x30303030u);  // m 4..7
+    const uint32_t m4 = 0x0F0F0F0Fu;
+    const uint4 ha = r.p[1], hb = r.p[2];   // qh[0..16), qh[16..32)
+    const uint4 *xp = a.xq + col;
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;
+    uint4 xa0 = xp[0], xa1 = xp[st], xb0 = xp[2 * st], xb1 = xp[3 * st];
+    const uint4 b = a.aux[col];  // bsum_0..7 as i16
+    isum = 0;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      // qs[32g .. 32g+32): low nibbles are sub-block 2g, high nibbles sub-block 2g+1; piece
+      // 3+2g holds bytes 0..15 of the run (qh bytes 0..15), piece 4+2g bytes 16..31
+      uint4 na0 = xa0, na1 = xa1, nb0 = xb0, nb1 = xb1;
+      if (g < 3) {
+        const uint4 *q = xp + 4 * (g + 1) * st;
+        na0 = q[0];
+        na1 = q[st];
+        nb0 = q[2 * st];
+        nb1 = q[3 * st];
+      }
+      const uint4 wa = r.p[3 + 2 * g], wb = r.p[4 + 2 * g];
+      const int lo = 2 * g, hi = 2 * g + 1;
+      int dlo = 0, dhi = 0;
+      dlo = dot4(with_high(wa.x & m4, ha.x, lo), xa0.x, dlo);
+      dlo = dot4(with_high(wa.y & m4, ha.y, lo), xa0.y, dlo);
+      dlo = dot4(with_high(wa.z & m4, ha.z, lo), xa0.z, dlo);
+      dlo = dot4(with_high(wa.w & m4, ha.w, lo), xa0.w, dlo);
+      dlo = dot4(with_high(wb.x & m4, hb.x, lo), xa1.x, dlo);
+      dlo = dot4(with_high(wb.y & m4, hb.y, lo), xa1.y, dlo);
+      dlo = dot4(with_high(wb.z & m4, hb.z, lo), xa1.z, dlo);
+      dlo = dot4(with_high(wb.w & m4, hb.w, lo), xa1.w, dlo);
+      dhi = dot4(with_high((wa.x >> 4) & m4, ha.x, hi), xb0.x, dhi);
+      dhi = dot4(with_high((wa.y >> 4) & m4, ha.y, hi), xb0.y, dhi);
+      dhi = dot4(with_high((wa.z >> 4) & m4, ha.z, hi), xb0.z, dhi);
+      dhi = dot4(with_high((wa.w >> 4) & m4, ha.w, hi), xb0.w, dhi);
+      dhi = dot4(with_high((wb.x >> 4) & m4, hb.x, hi), xb1.x, dhi);
+      dhi = dot4(with_high((wb.y >> 4) & m4, hb.y, hi), xb1.y, dhi);
+      dhi = dot4(with_high((wb.z >> 4) & m4, hb.z, hi), xb1.z, dhi);
+      dhi = dot4(with_high((wb.w >> 4) & m4, hb.w, hi), xb1.w, dhi);
+      const int sc_lo = lo < 4 ? byte_of(sca, lo) : byte_of(scb, lo - 4);
+      const int sc_hi = hi < 4 ? byte_of(sca, hi) : byte_of(scb, hi - 4);
+      isum += sc_lo * dlo + sc_hi * dhi;
+      xa0 = na0;
+      xa1 = na1;
+      xb0 = nb0;
+      xb1 = nb1;
+    }
+    imin = byte_of(mna, 0) * lo16(b.x) + byte_of(mna, 1) * hi16(b.x) +
+           byte_of(mna, 2) * lo16(b.y) + byte_of(mna, 3) * hi16(b.y) +
+           byte_of(mnb, 0) * lo16(b.z) + byte_of(mnb, 1) * hi16(b.z) +
+           byte_of(mnb, 2) * lo16(b.w) + byte_of(mnb, 3) * hi16(b.w);
+  }
+  // GEMV: total += act.d[s] * (d*isum - dmin*imin)                           (vecdot.rs:3210)
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int imin) {
+    const float d = f16_bits_to_f32(r.p[0].x & 0xFFFFu), dmin = f16_bits_to_f32(r.p[0].x >> 16);
+    return ad * (d * (float)isum - dmin * (float)imin);
+  }
+  // GEMM: the K-quant GEMM of Q4_K over a row unpacked with the fifth bit    (vecdot.rs:2010-2013, 2229-2303)
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int imin,
+                                                   float &tmin, float &tdot) {
+    const float d = f16_bits_to_f32(r.p[0].x & 0xFFFFu), dmin = f16_bits_to_f32(r.p[0].x >> 16);
+    tmin = ad * dmin * (float)imin;
+    tdot = ad * (d * (float)isum);
+  }
+};
+
 // Q6_K: ql:u8[128] | qh:u8[64] | scales:i8[16] | d:f16                      (quant.rs:744-787)
 struct FmtQ6K {
   static constexpr uint32_t TYPE = OGM_Q6_K;
@@ -675,6 +773,8 @@ uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order
   switch (ggml_type) {
     case OGM_Q4_K:
       return gemm_order ? max_tokens_t<FmtQ4K, true>(in_dim) : max_tokens_t<FmtQ4K, false>(in_dim);
+    case OGM_Q5_K:
+      return gemm_order ? max_tokens_t<FmtQ5K, true>(in_dim) : max_tokens_t<FmtQ5K, false>(in_dim);
     case OGM_Q6_K:
       return gemm_order ? max_tokens_t<FmtQ6K, true>(in_dim) : max_tokens_t<FmtQ6K, false>(in_dim);
     case OGM_Q8_0:
@@ -771,6 +871,9 @@ hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char 
     case OGM_Q4_K:
       if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ4K,gemm>" : "ogm_gemv_kernel<FmtQ4K,gemv>";
       return a.gemm_order ? launch_t<FmtQ4K, true>(a, stream) : launch_t<FmtQ4K, false>(a, stream);
+    case OGM_Q5_K:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ5K,gemm>" : "ogm_gemv_kernel<FmtQ5K,gemv>";
+      return a.gemm_order ? launch_t<FmtQ5K, true>(a, stream) : launch_t<FmtQ5K, false>(a, stream);
     case OGM_Q6_K:
       if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ6K,gemm>" : "ogm_gemv_kernel<FmtQ6K,gemv>";
       return a.gemm_order ? launch_t<FmtQ6K, true>(a, stream) : launch_t<FmtQ6K, false>(a, stream);

@@ -1,7 +1,7 @@
 // Tile-planar weight layout shared by the host repacker and the device kernels.
 //
 // A matrix is out_dim rows of `upr` blocks ("units"; one unit is one GGUF block: Q8_0 34 B / 32
-// weights, Q4_K 144 B / 256, Q6_K 210 B / 256; engine/quant.rs:638-787).  A *tile* holds 64
+// weights, Q4_K 144 B / 256, Q5_K 176 B / 256, Q6_K 210 B / 256; engine/quant.rs:638-787).  A *tile* holds 64
 // units: R consecutive rows x C consecutive blocks, with C = 4 when a row has a multiple of four
 // blocks (else 2, else 1) and R = 64 / C.  Tiles are ordered [row block][column tile]; inside a
 // tile the unit of (row r, block c) is lane c*R + r.
@@ -18,6 +18,7 @@
 //   type   pieces                                   tail
 //   Q8_0   2  (qs[0..32))                           d      (2 B)
 //   Q4_K   9  (d,dmin,scales | qs[0..128))          -
+//   Q5_K   11 (d,dmin,scales | qh[0..32) | qs)      -
 //   Q6_K   13 (ql[0..128) | qh[0..64) | scales)     d      (2 B)
 #pragma once
 #include <stddef.h>
@@ -25,6 +26,7 @@
 
 #define OGM_Q8_0 8u
 #define OGM_Q4_K 12u
+#define OGM_Q5_K 13u
 #define OGM_Q6_K 14u
 
 #define OGM_TILE_UNITS 64u
@@ -61,6 +63,9 @@ OGM_HD inline bool ogm_layout_for(uint32_t ggml_type, OgmLayout *l) {
       return true;
     case OGM_Q4_K:  // d:f16 | dmin:f16 | scales:u8[12] | qs:u8[128]
       *l = OgmLayout{144, 256, 9, 0, 0, 0, 64 * 144};
+      return true;
+    case OGM_Q5_K:  // d:f16 | dmin:f16 | scales:u8[12] | qh:u8[32] | qs:u8[128]
+      *l = OgmLayout{176, 256, 11, 0, 0, 0, 64 * 176};
       return true;
     case OGM_Q6_K:  // ql:u8[128] | qh:u8[64] | scales:i8[16] | d:f16
       *l = OgmLayout{210, 256, 13, 2, 0, 208, 64 * 210};

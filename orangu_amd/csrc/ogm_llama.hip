@@ -644,7 +644,7 @@ hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStrea
 
 // ------------------------------------------------------------------------------------------
 // one row of a quantized matrix as f32: the embedding lookup (LlamaModel::run_layers,
-// llama.rs:609-614, over dequantize_q8_0 / _q4_k / _q6_k, quant.rs:639-649, 666-697, 746-787),
+// llama.rs:609-614, over dequantize_q8_0 / _q4_k / _q5_k / _q6_k, quant.rs:639-649, 666-742, 746-787),
 // reading the tile-planar device copy.  One thread per element; the f32 expressions are the
 // reference's, so the values are bit-identical (built without FMA contraction).
 
@@ -695,6 +695,25 @@ __global__ __launch_bounds__(256) void ogm_dequant_row_kernel(const uint8_t *__r
     const uint32_t nib = hi ? (byte >> 4) : (byte & 0xFu);
     const float d1 = d * (float)sc, mm = dmin * (float)m;
     v = d1 * (float)nib - mm;
+  } else if (ggml_type == OGM_Q5_K) {
+    const uint8_t *hd = tb + lane * 16u;   // piece 0: d, dmin, scales; then qh[32], then qs
+    const float d = dq_f16(hd), dmin = dq_f16(hd + 2);
+    const uint32_t g4 = j >> 6, hi = (j >> 5) & 1u, li = j & 31u;
+    const uint32_t is = 2u * g4 + hi;
+    const uint8_t *q = hd + 4;
+    uint32_t sc, m;
+    if (is < 4) {
+      sc = q[is] & 63u;
+      m = q[is + 4] & 63u;
+    } else {
+      sc = (q[is + 4] & 0xFu) | ((q[is - 4] >> 6) << 4);
+      m = (q[is + 4] >> 4) | ((q[is] >> 6) << 4);
+    }
+    const uint32_t byte = piece_byte(48u + 32u * g4 + li);
+    const uint32_t high = (piece_byte(16u + li) >> is) & 1u;
+    const int qv = (int)(hi ? (byte >> 4) : (byte & 0xFu)) + (high ? 16 : 0);
+    const float d1 = d * (float)sc, mm = dmin * (float)m;
+    v = d1 * (float)qv - mm;
   } else {  // Q6_K
     const float d = dq_f16(tb + l.pieces * 1024u + lane * 2u);
     const uint32_t h = j >> 7, jj = j & 127u, qd = jj >> 5, li = jj & 31u;

@@ -8,9 +8,9 @@ from __future__ import annotations
 
 import numpy as np
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-BLOCK = {Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256)}
-TYPE_NAME = {Q8_0: "q8_0", Q4_K: "q4_k", Q6_K: "q6_k"}
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+BLOCK = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+TYPE_NAME = {Q8_0: "q8_0", Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k"}
 
 
 def row_bytes(ggml_type: int, in_dim: int) -> int:
@@ -57,7 +57,7 @@ def pin_scales(raw: np.ndarray, ggml_type: int) -> np.ndarray:
     blocks = raw.reshape(-1, bb)
     if ggml_type == Q8_0:
         blocks[:, 0:2] = (0x00, 0x30)
-    elif ggml_type == Q4_K:
+    elif ggml_type in (Q4_K, Q5_K):   # Q5_K shares Q4_K's leading d / dmin pair (vecdot.rs:3467)
         blocks[:, 0:2] = (0x00, 0x30)
         blocks[:, 2:4] = (0x00, 0x2C)
     elif ggml_type == Q6_K:
@@ -109,7 +109,7 @@ def cpu_rs_weights(ggml_type: int, in_dim: int, out_dim: int, nb: NextByte) -> n
         scale = np.float32(0.05) + (np.float32(nb()) / np.float32(255.0)) * np.float32(1.95)
         block[0:2] = np.frombuffer(np.float16(scale).tobytes(), np.uint8)
         qf = 2
-        if ggml_type == Q4_K:
+        if ggml_type in (Q4_K, Q5_K):
             dmin = np.float32(0.05) + (np.float32(nb()) / np.float32(255.0)) * np.float32(0.95)
             block[2:4] = np.frombuffer(np.float16(dmin).tobytes(), np.uint8)
             qf = 4
@@ -134,7 +134,7 @@ def synth_weights(ggml_type: int, in_dim: int, out_dim: int, seed: int) -> np.nd
         raw[:, 2:] = q.view(np.uint8)
         d = (np.abs(rng.normal(0, 0.02, nblk)) / 127).astype(np.float16)
         raw[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
-    elif ggml_type == Q4_K:
+    elif ggml_type in (Q4_K, Q5_K):
         d = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)
         dm = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)
         raw[:, 0:2] = d.view(np.uint8).reshape(-1, 2)

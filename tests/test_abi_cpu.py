@@ -29,9 +29,10 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_supports_predicates_follow_vecdot(lib):
-    """vecdot.rs:274-283 for the three types; Backend::supports_type (mod.rs:493)."""
+    """vecdot.rs:274-283 for the types built; Backend::supports_type (mod.rs:493)."""
     assert lib.ogm_supports_type(Q8_0) and lib.ogm_supports_type(Q4_K) and lib.ogm_supports_type(Q6_K)
-    assert not lib.ogm_supports_type(0) and not lib.ogm_supports_type(13)
+    assert lib.ogm_supports_type(13) and lib.ogm_supports(13, 256) and not lib.ogm_supports(13, 128)   # Q5_K
+    assert not lib.ogm_supports_type(0) and not lib.ogm_supports_type(11)
     assert lib.ogm_supports(Q8_0, 96) and not lib.ogm_supports(Q8_0, 100)
     assert lib.ogm_supports(Q4_K, 512) and not lib.ogm_supports(Q4_K, 896)
     assert lib.ogm_supports(Q6_K, 256) and not lib.ogm_supports(Q6_K, 0)

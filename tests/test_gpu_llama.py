@@ -8,7 +8,7 @@ import sys
 import numpy as np
 import pytest
 
-from helpers import Q4_K, Q6_K, Q8_0, synth_weights
+from helpers import Q4_K, Q5_K, Q6_K, Q8_0, synth_weights
 from oracle import llama_ref as R
 
 pytestmark = pytest.mark.gpu
@@ -80,7 +80,8 @@ def step_both(ref, dev, x, pos, what):
     say(what, "hidden err %.2e logits err %.2e token %d" % (e1, e2, got_tok))
 
 
-@pytest.mark.parametrize("types", [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q4_K, Q4_K, Q4_K, Q4_K)])
+@pytest.mark.parametrize("types", [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q4_K, Q4_K, Q4_K, Q4_K),
+                                   (Q5_K, Q5_K, Q6_K, Q5_K)])
 def test_decode_steps_from_an_empty_cache(be, types):
     """Positions 0..5 one after the other: RMSNorm, q/k/v, RoPE, cache append, attention over the
     growing cache, wo, residual, SwiGLU FFN, output norm and vocabulary projection."""
@@ -192,6 +193,7 @@ def test_matrices_uploaded_from_a_gguf_file_multiply_like_direct_uploads(be, tmp
     (Q8_0, 64, 5), (Q8_0, 4096, 70),
     (Q4_K, 256, 3), (Q4_K, 1024, 130), (Q4_K, 4096, 67),
     (Q6_K, 256, 1), (Q6_K, 768, 65), (Q6_K, 4096, 129),
+    (Q5_K, 256, 2), (Q5_K, 1280, 70), (Q5_K, 4096, 33),
 ])
 def test_dequant_rows_bits(be, t, in_dim, out_dim):
     """Rows of the device copy equal dequantize_q8_0 / _q4_k / _q6_k (quant.rs:639-787) bit for bit."""
@@ -209,7 +211,7 @@ def test_dequant_rows_bits(be, t, in_dim, out_dim):
         be.dequant_rows(w, out_dim, 1)
 
 
-@pytest.mark.parametrize("embd_t", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("embd_t", [Q4_K, Q5_K, Q6_K, Q8_0])
 def test_generate_matches_stepwise(be, embd_t):
     """Greedy generation on the device = the oracle's loop: embedding row of the token
     (llama.rs:609-614), decode step, last-of-equal argmax (sampling.rs:336-343)."""

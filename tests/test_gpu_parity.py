@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (BLOCK, Q4_K, Q6_K, Q8_0, NextByte, activations, activations_t, cpu_rs_weights,
+from helpers import (BLOCK, Q4_K, Q5_K, Q6_K, Q8_0, NextByte, activations, activations_t, cpu_rs_weights,
                      fixture_row, k_fixture, row_bytes, synth_weights, synth_x)
 from test_oracle_quantize import adversarial_blocks
 
@@ -67,7 +67,7 @@ def test_f16_scale_conversion_matches_quant_rs_for_all_inputs(be):
     assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q5_K, Q6_K])
 def test_upload_download_round_trip(be, t):
     """unrepack(repack(W)) == W through the device."""
     bb, bel = BLOCK[t]
@@ -113,6 +113,7 @@ def test_quantizer_ties_round_away_from_zero(be):
 
 @pytest.mark.parametrize("t,in_dim,out_dim,T", [
     (Q4_K, 256, 5, 1), (Q4_K, 2048, 37, 3), (Q4_K, 4864, 9, 1),
+    (Q5_K, 256, 5, 1), (Q5_K, 2048, 37, 3), (Q5_K, 4864, 9, 2),
     (Q6_K, 256, 5, 1), (Q6_K, 2048, 37, 3), (Q6_K, 4864, 9, 2),
     (Q8_0, 96, 11, 1), (Q8_0, 896, 19, 3), (Q8_0, 4864, 7, 1),
 ])
@@ -123,14 +124,14 @@ def test_block_integer_sums_bit_exact(be, t, in_dim, out_dim, T):
     isum, imin = be.dump_block_sums(x, T, w)
     wi, wm = oracle.block_sums(t, raw, in_dim, out_dim, x, T)
     assert np.array_equal(isum, wi)
-    if t == Q4_K:
+    if t in (Q4_K, Q5_K):
         assert np.array_equal(imin, wm)
 
 
 # ---------------------------------------------------------------- GEMV / matmul values
 
 CHECK = [(Q8_0, 896), (Q8_0, 4864), (Q4_K, 256), (Q4_K, 4864), (Q6_K, 256), (Q6_K, 4864),
-         (Q4_K, 2048), (Q6_K, 5632)]
+         (Q4_K, 2048), (Q6_K, 5632), (Q5_K, 256), (Q5_K, 3072), (Q5_K, 4864)]
 
 
 @pytest.mark.parametrize("t,in_dim", CHECK)
@@ -156,7 +157,7 @@ def test_gemv_matches_cpu_matmul_on_reference_fixtures(be, t, in_dim, seed):
         assert abs(float(got[o]) - float(ref[o])) <= budget * max(mag, 1e-6)
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("T", [1, 2, 5, 8, 13])
 def test_matmul_decode_matches_cpu_and_each_token_alone(be, t, T):
     """backend/cpu.rs:623-650: a decode batch's row t is what token t gives alone."""
@@ -177,7 +178,7 @@ def test_matmul_decode_matches_cpu_and_each_token_alone(be, t, T):
         assert_bits(got[k], alone, f"token {k} alone")
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q5_K, Q6_K])
 def test_matmul_multi_token_matches_cpu_gemm(be, t):
     """backend/cpu.rs:544-582 shapes: in = 3 blocks, out = 11 (odd), T in 1,2,5,77,3,1 from one
     reused backend; matmul at T > 1 follows the CPU GEMM kernels."""
@@ -196,7 +197,7 @@ def test_matmul_multi_token_matches_cpu_gemm(be, t):
         assert_bits(got, want, f"matmul T={T}")
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_dim", [256, 2048, 8192])
 def test_k_gemm_fixture(be, t, in_dim):
     """vecdot.rs:4479-4513: 5 rows x 7 tokens, seed 4242."""
@@ -207,7 +208,7 @@ def test_k_gemm_fixture(be, t, in_dim):
     assert_bits(got, want, "k_gemm")
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
 def test_gemm_result_is_independent_of_the_batch_size(be, t):
     """vecdot.rs:4522-4549: exact equality."""
     in_dim, out_dim = 512, 4
@@ -271,6 +272,7 @@ def test_error_statuses(be):
     (Q4_K, 14336, 4096),    # config 2 down
     (Q4_K, 4096, 1024),     # config 3 k/v
     (Q6_K, 14336, 4096),    # config 5 ffn_down
+    (Q5_K, 4096, 4096), (Q5_K, 14336, 4096),   # the same shapes in Q5_K
 ])
 def test_benchmark_shapes_match_cpu(be, t, in_dim, out_dim):
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim)
@@ -447,6 +449,7 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign):
     (Q8_0, 32, 7), (Q8_0, 96, 33), (Q8_0, 4096, 130), (Q8_0, 4384, 64),
     (Q4_K, 256, 5), (Q4_K, 768, 70), (Q4_K, 4096, 257), (Q4_K, 14336, 96), (Q4_K, 18432, 40),
     (Q6_K, 256, 3), (Q6_K, 1280, 65), (Q6_K, 4096, 130), (Q6_K, 14336, 48), (Q6_K, 18432, 17),
+    (Q5_K, 256, 5), (Q5_K, 768, 70), (Q5_K, 4096, 257), (Q5_K, 14336, 96), (Q5_K, 18432, 40),
 ])
 def test_single_token_gemv_quantizes_in_kernel_or_before_with_the_same_bits(be, t, in_dim, out_dim):
     """One token: the GEMV that quantizes its own activations and the quantizer kernel + GEMV
@@ -473,7 +476,7 @@ def test_single_token_gemv_quantizes_in_kernel_or_before_with_the_same_bits(be, 
             assert_bits(got[ok], want[ok], f"fuse mode {mode}")
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("T,decode", [(1, False), (1, True), (4, True), (3, False), (16, False), (11, True)])
 def test_grouped_weights_over_one_input_equal_single_calls(be, t, T, decode):
     """q/k/v and gate/up read one input (engine/arch/mod.rs:1082-1096): the grouped call equals
@@ -540,7 +543,8 @@ def test_matmul_batch_groups_ops_that_share_their_input(be):
             assert_bits(y, want, "grouped batch vs cpu")
 
 
-@pytest.mark.parametrize("t,in_dim", [(Q8_0, 1056), (Q4_K, 1024), (Q4_K, 1536), (Q6_K, 1024), (Q6_K, 256)])
+@pytest.mark.parametrize("t,in_dim", [(Q8_0, 1056), (Q4_K, 1024), (Q4_K, 1536), (Q6_K, 1024), (Q6_K, 256), (Q5_K, 1024),
+                                      (Q5_K, 768)])
 def test_row_blocks_per_workgroup_do_not_change_a_bit(be, t, in_dim):
     """A workgroup may own several row blocks (ragged last group, last row block partly beyond
     out_dim, several matrices in one launch): every split gives the CPU path's bits."""
@@ -605,3 +609,28 @@ def test_concurrent_callers_share_one_backend(be):
     for th in threads:
         th.join()
     assert not errors, errors
+
+
+@pytest.mark.parametrize("sign", ["pos", "alt"])
+def test_q5k_extreme_integer_ranges(be, sign):
+    """Q5_K's largest magnitudes: every weight 31, scales and mins 63, activations +-127: isum
+    reaches 6.3e7 per super-block (vecdot.rs:3077), inside i32; GEMV, decode batch and multi-token
+    matmul all give the CPU path's bits."""
+    in_dim, out_dim, T = 1024, 20, 12
+    blocks = np.zeros((out_dim * 4, 176), np.uint8)
+    blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    blocks[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
+    blocks[:, 4:] = 0xFF
+    x = np.full((T, in_dim), 127.0, np.float32)
+    if sign == "alt":
+        x[1::2] *= -1
+        x[:, ::7] = -126.0
+    raw = blocks.reshape(-1)
+    w = qm(raw, Q5_K, in_dim, out_dim)
+    isum, imin = be.dump_block_sums(x[0], 1, w)
+    wi, wm = oracle.block_sums(Q5_K, raw, in_dim, out_dim, x[0], 1)
+    assert np.array_equal(isum, wi) and np.array_equal(imin, wm)
+    say("extreme q5k isum", int(np.abs(isum).max()), "imin", int(np.abs(imin).max()))
+    assert_bits(be.matmul(x[0], 1, w), oracle.matmul(Q5_K, raw, in_dim, out_dim, x[0], 1), "gemv")
+    assert_bits(be.matmul(x, T, w), oracle.matmul(Q5_K, raw, in_dim, out_dim, x, T), "matmul")
+    assert_bits(be.matmul_decode(x, T, w), oracle.matmul_decode(Q5_K, raw, in_dim, out_dim, x, T), "decode")

@@ -4,12 +4,13 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Q4_K, Q6_K, Q8_0
+from helpers import Q4_K, Q5_K, Q6_K, Q8_0
 
-# quant.rs:1389-1417 GOLDEN (the three types on the path)
+# quant.rs:1389-1417 GOLDEN (the types on the path)
 GOLDEN = [
     (Q8_0, "q8_0", 256, 0xC5D58782F54E52E5),
     (Q4_K, "q4_k", 512, 0x9A7268A432A5C5FA),
+    (Q5_K, "q5_k", 512, 0x41C70B9BE1696E6D),
     (Q6_K, "q6_k", 512, 0x61001D333CB0CFD1),
 ]
 
@@ -42,6 +43,7 @@ def test_tensor_byte_size_and_block_layout():
     assert oracle.tensor_byte_size(Q8_0, 256) == 8 * 34
     assert oracle.tensor_byte_size(Q4_K, 512) == 2 * 144
     assert oracle.tensor_byte_size(Q6_K, 512) == 2 * 210
+    assert oracle.tensor_byte_size(Q5_K, 256) == 176  # quant.rs:1701
     assert oracle.tensor_byte_size(Q4_K, 100) == -2  # not a whole number of blocks
     assert oracle.tensor_byte_size(99, 256) == -1  # unknown type
 
@@ -168,3 +170,38 @@ def test_dequantize_q6_k_element_order():
         h, r, l = e // 128, (e % 128) // 32, e % 32
         q = (e * 7 + 3) % 64
         assert out[e] == 0.5 * float(sc[8 * h + 2 * r + l // 16]) * (q - 32), e
+
+
+def test_dequantize_q5_k_applies_the_high_bit_from_qh():
+    """quant.rs:1872-1888: d = 1, dmin = 0, every scale 1, every qh bit set, every nibble 0: all
+    256 elements are 1 * 1 * (0 + 16) - 0 = 16."""
+    block = np.zeros(176, np.uint8)
+    block[0:2] = _f16(1.0)
+    block[4:16] = [1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1]
+    block[16:48] = 0xFF
+    out = oracle.dequantize(Q5_K, block, 256)
+    assert out.size == 256 and np.all(out == 16.0)
+
+
+def test_dequantize_q5_k_bit_to_sub_block_mapping():
+    """Bit j of qh[l] is the fifth bit of element l of sub-block j (quant.rs:703-742): one qh bit
+    at a time lights exactly one element; with nibbles set, low nibbles are the even sub-blocks."""
+    for j in range(8):
+        for l in (0, 13, 31):
+            block = np.zeros(176, np.uint8)
+            block[0:2] = _f16(1.0)
+            block[4:16] = [1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1]
+            block[16 + l] = 1 << j
+            out = oracle.dequantize(Q5_K, block, 256)
+            want = np.zeros(256, np.float32)
+            want[32 * j + l] = 16.0
+            assert np.array_equal(out, want), (j, l)
+    block = np.zeros(176, np.uint8)
+    block[0:2] = _f16(1.0)
+    block[2:4] = _f16(0.5)
+    block[4:16] = [1, 2, 3, 4, 1, 1, 1, 1, 0x15, 0x16, 0x17, 0x18]   # sc 1..8, mins 1
+    block[48:] = 0x21                                                # low nibble 1, high nibble 2
+    out = oracle.dequantize(Q5_K, block, 256).reshape(8, 32)
+    for j in range(8):
+        nib = 1 if j % 2 == 0 else 2
+        assert np.all(out[j] == np.float32(j + 1) * nib - np.float32(0.5)), j

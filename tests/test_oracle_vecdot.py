@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (BLOCK, Q4_K, Q6_K, Q8_0, NextByte, activations, cpu_rs_weights, fixture_row,
+from helpers import (BLOCK, Q4_K, Q5_K, Q6_K, Q8_0, NextByte, activations, cpu_rs_weights, fixture_row,
                      k_fixture, row_bytes)
 
 
@@ -67,6 +67,12 @@ def np_unpack(ggml_type, row, in_dim):
         qs = blocks[:, 16:].astype(np.int64).reshape(nb, 4, 32)
         q = np.stack([qs & 15, qs >> 4], axis=2).reshape(-1)  # [nb][g][half][32]
         return q, np.repeat(sc, 32, axis=1).reshape(-1), np.repeat(mn, 32, axis=1).reshape(-1), d, dmin
+    if ggml_type == Q5_K:   # Q4_K with qh[32] between the scales and qs; bit j of qh[l]: sub-block j
+        q4, sce, mne, d, dmin = np_unpack(Q4_K, np.concatenate([blocks[:, :16], blocks[:, 48:]], axis=1).reshape(-1),
+                                          in_dim)
+        qh = blocks[:, 16:48].astype(np.int64)                                        # [nb][32]
+        hi = ((qh[:, None, :] >> np.arange(8)[None, :, None]) & 1) * 16              # [nb][8][32]
+        return q4 + hi.reshape(-1), sce, mne, d, dmin
     ql = blocks[:, 0:128].astype(np.int64).reshape(nb, 2, 2, 32)  # [h][r&1][l]
     qh = blocks[:, 128:192].astype(np.int64).reshape(nb, 2, 32)
     sc = blocks[:, 192:208].copy().view(np.int8).astype(np.int64)
@@ -88,7 +94,7 @@ def np_block_sums(ggml_type, row, in_dim, xq):
     return isum, imin
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_dim", [256, 2048])
 def test_k_row_integer_sums_equal_numpy_int64(ggml_type, in_dim):
     """Per-super-block isum / imin (vecdot.rs:3152-3178, 3215-3241) against int64 numpy over an
@@ -98,7 +104,7 @@ def test_k_row_integer_sums_equal_numpy_int64(ggml_type, in_dim):
     _, isum, imin = oracle.dot_k_row(ggml_type, row, act, want_sums=True)
     wi, wm = np_block_sums(ggml_type, row, in_dim, act[0])
     assert np.array_equal(isum, wi)
-    if ggml_type == Q4_K:
+    if ggml_type in (Q4_K, Q5_K):
         assert np.array_equal(imin, wm)
 
 
@@ -166,11 +172,11 @@ def test_fused_dot_row_matches_dequantize_reference(ggml_type, in_dim, seed):
     assert abs(float(got) - float(ref)) <= 0.01 * max(mag, 1e-6)
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q6_K])
-@pytest.mark.parametrize("in_dim", [256, 2048, 5632])
+@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("in_dim", [256, 2048, 3072, 5632])
 @pytest.mark.parametrize("seed", [1, 7, 99])
 def test_k_row_decode_matches_dequantize_reference(ggml_type, in_dim, seed):
-    """vecdot.rs:4011-4040: budget 0.02 * sum|w x| for the per-256 decode."""
+    """vecdot.rs:4011-4040 (and :4127-4133 for Q5_K): budget 0.02 * sum|w x| for the per-256 decode."""
     row = fixture_row(ggml_type, in_dim, seed)
     x = activations(in_dim)
     ref, mag = _reference(ggml_type, row, in_dim, x)
@@ -187,7 +193,7 @@ def test_integer_accumulators_stay_inside_i32_by_construction():
     assert 128 * 32 * 127 * 256 < 2**31
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_dim", [256, 2048, 8192])
 def test_k_gemm_matches_dequantize_reference(ggml_type, in_dim):
     """vecdot.rs:4479-4513: 5 rows x 7 tokens, seed 4242, budget 0.01 * sum|w x|."""
@@ -203,7 +209,7 @@ def test_k_gemm_matches_dequantize_reference(ggml_type, in_dim):
             assert abs(got[o, t] - ref) <= 0.01 * max(mag, 1e-6) + 1e-6 * mag
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
 def test_k_gemm_result_is_independent_of_the_batch_size(ggml_type):
     """vecdot.rs:4522-4549: exact equality."""
     in_dim, out_dim = 512, 4
@@ -214,7 +220,7 @@ def test_k_gemm_result_is_independent_of_the_batch_size(ggml_type):
         assert np.array_equal(part.view(np.uint32), full[:, :n].view(np.uint32))
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
 def test_k_gemm_float_order_rebuilt_from_integer_sums(ggml_type):
     """gemm_k_q4_k: acc -= (ad*dmin)*imin over all super-blocks first, then acc += ad*(d*isum)
     (vecdot.rs:2229-2303); gemm_k_q6_k: acc += ad*(d*isum) (vecdot.rs:2386-2391).  Rebuilt in
@@ -232,7 +238,7 @@ def test_k_gemm_float_order_rebuilt_from_integer_sums(ggml_type):
             xq, ad, _ = oracle.quantize_act_k_row(x[t * in_dim:(t + 1) * in_dim])
             isum, imin = np_block_sums(ggml_type, row, in_dim, xq)
             acc = f(0)
-            if ggml_type == Q4_K:
+            if ggml_type in (Q4_K, Q5_K):
                 for s in range(in_dim // 256):
                     acc = f(acc - f(f(ad[s] * dmin[s]) * f(imin[s])))
             for s in range(in_dim // 256):
@@ -309,6 +315,8 @@ def test_supports_predicates():
     """vecdot.rs:274-283, 1821-1826, 3083-3093, 2456-2461 for the three types."""
     assert oracle.supports(Q8_0, 96) and not oracle.supports(Q8_0, 100)
     assert oracle.supports(Q4_K, 512) and not oracle.supports(Q4_K, 896)
+    assert oracle.supports(Q5_K, 256) and oracle.supports_k(Q5_K, 512) and oracle.supports_k_row(Q5_K, 768)
+    assert not oracle.supports(Q5_K, 128) and not oracle.supports_flat(Q5_K, 256)
     assert oracle.supports_k(Q6_K, 256) and not oracle.supports_k(Q8_0, 256)
     assert oracle.supports_k_row(Q4_K, 256) and not oracle.supports_k_row(Q4_K, 128)
     assert oracle.supports_flat(Q8_0, 32) and not oracle.supports_flat(Q4_K, 256)
@@ -325,3 +333,20 @@ def test_block_sums_entry_matches_per_row_calls():
         for o in range(out_dim):
             _, a, b = oracle.dot_k_row(Q4_K, raw[o * rb:(o + 1) * rb], act, want_sums=True)
             assert np.array_equal(isum[t, o], a) and np.array_equal(imin[t, o], b)
+
+
+def test_q5_k_unpack_applies_the_high_bit_to_every_sub_block():
+    """vecdot.rs:4141-4165: every qh bit set and every nibble zero: every unpacked weight is exactly
+    16 on the decode path and on the K-GEMM path.  With all-one activations quantized to 127 each
+    sub-block's dot is 32 * 16 * 127 and the scales are 1."""
+    block = np.zeros(176, np.uint8)
+    block[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    block[4:16] = [1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1]
+    block[16:48] = 0xFF
+    x = np.ones(256, np.float32)
+    act = oracle.quantize_act_k_row(x)
+    v, isum, imin = oracle.dot_k_row(Q5_K, block, act, want_sums=True)
+    assert isum[0] == 8 * 32 * 16 * 127 and imin[0] == 0
+    assert v == np.float32(act[1][0] * np.float32(np.float32(1.0) * np.float32(isum[0])))
+    got = oracle.k_gemm_t(Q5_K, block, 256, 1, x, 1)
+    assert got[0, 0] == np.float32(act[1][0] * np.float32(isum[0]))
