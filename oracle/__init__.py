@@ -16,8 +16,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liborangu_oracle.so")
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
-BLOCK_LAYOUT = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+Q8_0, Q3_K, Q4_K, Q5_K, Q6_K = 8, 11, 12, 13, 14
+BLOCK_LAYOUT = {Q8_0: (34, 32), Q3_K: (110, 256), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
 
 
 def build() -> str:
@@ -69,6 +69,9 @@ def lib() -> C.CDLL:
         L.ogo_dot_k_row_q5_k.argtypes = [u8p, sz, i8p, f32p, i32p, i32p, i32p]
         L.ogo_dot_k_row_q6_k.restype = C.c_float
         L.ogo_dot_k_row_q6_k.argtypes = [u8p, sz, i8p, f32p, i32p]
+        L.ogo_dot_k_row_q3_k.restype = C.c_float
+        L.ogo_dot_k_row_q3_k.argtypes = [u8p, sz, i8p, f32p, i32p]
+        L.ogo_unpack_q3_k_scales.argtypes = [u8p, i32p]
         L.ogo_block_sums_q8_0.argtypes = [u8p, sz, i8p, i32p]
         for name in ("ogo_supports", "ogo_supports_k", "ogo_supports_k_row", "ogo_supports_flat"):
             getattr(L, name).argtypes = [C.c_uint32, sz]
@@ -217,6 +220,14 @@ def dot_row(ggml_type: int, row, act) -> np.float32:
     raise ValueError(ggml_type)
 
 
+def unpack_q3_k_scales(packed) -> np.ndarray:
+    """quant.rs:883-897."""
+    p = _u8(packed)
+    out = np.zeros(16, np.int32)
+    lib().ogo_unpack_q3_k_scales(_p(p), _p(out))
+    return out
+
+
 def dot_k_row(ggml_type: int, row, act, want_sums: bool = False):
     """vecdot.rs:3103 dot_k_row over a per-256 ActQ8KRow ``(q, d, sums)``."""
     r = _u8(row)
@@ -231,6 +242,8 @@ def dot_k_row(ggml_type: int, row, act, want_sums: bool = False):
         v = L.ogo_dot_k_row_q5_k(_p(r), n, _p(q), _p(d), _p(s), _p(isum), _p(imin))
     elif ggml_type == Q6_K:
         v = L.ogo_dot_k_row_q6_k(_p(r), n, _p(q), _p(d), _p(isum))
+    elif ggml_type == Q3_K:
+        v = L.ogo_dot_k_row_q3_k(_p(r), n, _p(q), _p(d), _p(isum))
     else:
         raise ValueError(ggml_type)
     return (np.float32(v), isum, imin) if want_sums else np.float32(v)

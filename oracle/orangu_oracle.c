@@ -66,6 +66,7 @@ int ogo_block_layout(uint32_t ggml_type, size_t *block_bytes, size_t *block_elem
     case OGO_TYPE_F32: bb = 4; be = 1; break;
     case OGO_TYPE_F16: bb = 2; be = 1; break;
     case OGO_TYPE_Q8_0: bb = 2 + 32; be = 32; break;
+    case OGO_TYPE_Q3_K: bb = 32 + 64 + 12 + 2; be = 256; break;
     case OGO_TYPE_Q4_K: bb = 2 + 2 + 12 + 128; be = 256; break;
     case OGO_TYPE_Q5_K: bb = 2 + 2 + 12 + 32 + 128; be = 256; break;
     case OGO_TYPE_Q6_K: bb = 128 + 64 + 16 + 2; be = 256; break;
@@ -145,6 +146,45 @@ static void dequantize_q5_k(const uint8_t *bytes, size_t n, float *out) {
   }
 }
 
+/* quant.rs:883-897 */
+void ogo_unpack_q3_k_scales(const uint8_t *packed, int32_t *scales) {
+  for (int i = 0; i < 16; i++) {
+    uint8_t low = i < 8 ? (uint8_t)(packed[i] & 0xF) : (uint8_t)(packed[i - 8] >> 4);
+    /* scale i's two high bits sit at bit 2 * (i / 4) of byte 8 + i % 4 */
+    uint8_t high = (uint8_t)((packed[8 + (i % 4)] >> (2 * (i / 4))) & 3);
+    scales[i] = (int32_t)(low | (high << 4));
+  }
+}
+
+/* quant.rs:841-871: hmask[32] | qs[64] | scales[12] | d; the third bit is stored inverted (clear
+ * means subtract 4), the mask bit advances once per 32 elements */
+static void dequantize_q3_k(const uint8_t *bytes, size_t n, float *out) {
+  for (size_t s = 0; s < n / 256; s++) {
+    const uint8_t *block = bytes + s * 110;
+    const uint8_t *hmask = block, *qs = block + 32;
+    int32_t scales[16];
+    ogo_unpack_q3_k_scales(block + 96, scales);
+    float d_all = read_f16(block, 108);
+    float *o = out + s * 256;
+    int is = 0;
+    uint8_t m = 1;
+    for (size_t q_off = 0; q_off < 64; q_off += 32) {
+      for (int shift = 0; shift < 8; shift += 2) {
+        for (int half = 0; half < 2; half++) {
+          float dl = d_all * (float)(scales[is] - 32);
+          is += 1;
+          for (int l = 0; l < 16; l++) {
+            int idx = half * 16 + l;
+            int hi = (hmask[idx] & m) ? 0 : 4;
+            *o++ = dl * (float)((int)((qs[q_off + (size_t)idx] >> shift) & 3) - hi);
+          }
+        }
+        m = (uint8_t)(m << 1);
+      }
+    }
+  }
+}
+
 /* quant.rs:746-787 */
 static void dequantize_q6_k(const uint8_t *bytes, size_t n, float *out) {
   for (size_t s = 0; s < n / 256; s++) {
@@ -180,6 +220,7 @@ int ogo_dequantize(uint32_t ggml_type, const uint8_t *bytes, size_t element_coun
   if (element_count % be != 0) return -2;
   switch (ggml_type) {
     case OGO_TYPE_Q8_0: dequantize_q8_0(bytes, element_count, out); return 0;
+    case OGO_TYPE_Q3_K: dequantize_q3_k(bytes, element_count, out); return 0;
     case OGO_TYPE_Q4_K: dequantize_q4_k(bytes, element_count, out); return 0;
     case OGO_TYPE_Q5_K: dequantize_q5_k(bytes, element_count, out); return 0;
     case OGO_TYPE_Q6_K: dequantize_q6_k(bytes, element_count, out); return 0;
@@ -436,6 +477,38 @@ static void unpack_k_q5_k(const uint8_t *row, size_t in_dim, ogo_krow *out) {
   }
 }
 
+/* vecdot.rs:1098-1107 Q2K_RUNS: (qs byte offset, low-bit shift) of the eight 32-element runs */
+static const struct { size_t off; int shift; } Q2K_RUNS[8] = {
+    {0, 0}, {0, 2}, {0, 4}, {0, 6}, {32, 0}, {32, 2}, {32, 4}, {32, 6}};
+
+/* vecdot.rs:1131-1136 unpack_q3k_run */
+static inline void unpack_q3k_run(const uint8_t *qs, const uint8_t *hmask, int shift, uint8_t bit,
+                                  int8_t *w) {
+  for (int j = 0; j < 32; j++) {
+    int8_t lo = (int8_t)((qs[j] >> shift) & 3);
+    w[j] = (int8_t)(lo - ((hmask[j] & bit) ? 0 : 4));
+  }
+}
+
+/* vecdot.rs:2100-2117 unpack_k_q3_k: a KKind::Q6K row (per-16 integer scales sc - 32) */
+static void unpack_k_q3_k(const uint8_t *row, size_t in_dim, ogo_krow *out) {
+  for (size_t s = 0; s < in_dim / 256; s++) {
+    const uint8_t *block = row + s * 110;
+    const uint8_t *hmask = block, *qs = block + 32;
+    int32_t sc[16];
+    ogo_unpack_q3_k_scales(block + 96, sc);
+    out->d[s] = read_f16(block, 108);
+    size_t base = s * 256;
+    for (int p = 0; p < 8; p++) {
+      size_t e0 = base + (size_t)p * 32;
+      unpack_q3k_run(qs + Q2K_RUNS[p].off, hmask, Q2K_RUNS[p].shift, (uint8_t)(1u << p), out->q + e0);
+      size_t gi = e0 / 16;
+      out->sc[gi] = (int16_t)(sc[2 * p] - 32);
+      out->sc[gi + 1] = (int16_t)(sc[2 * p + 1] - 32);
+    }
+  }
+}
+
 /* vecdot.rs:2119-2143 unpack_k_q6_k */
 static void unpack_k_q6_k(const uint8_t *row, size_t in_dim, ogo_krow *out) {
   for (size_t s = 0; s < in_dim / 256; s++) {
@@ -544,22 +617,26 @@ float ogo_dot_k_row_q6_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
                          int32_t *isum_out) {
   return DISPATCH(dot_k_row_q6_k, row, in_dim, q, d, isum_out);
 }
+float ogo_dot_k_row_q3_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
+                         int32_t *isum_out) {
+  return DISPATCH(dot_k_row_q3_k, row, in_dim, q, d, isum_out);
+}
 
 /* ------------------------------------------------------------------ predicates */
 
 /* vecdot.rs:274-283, restricted to the types on the path */
 int ogo_supports(uint32_t t, size_t in_dim) {
   if (t == OGO_TYPE_Q8_0) return in_dim % 32 == 0;
-  if (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) return in_dim % 256 == 0;
+  if (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) return in_dim % 256 == 0;
   return 0;
 }
 /* vecdot.rs:1821-1826 */
 int ogo_supports_k(uint32_t t, size_t in_dim) {
-  return (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
+  return (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
 }
 /* vecdot.rs:3083-3093 */
 int ogo_supports_k_row(uint32_t t, size_t in_dim) {
-  return (t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
+  return (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
 }
 /* vecdot.rs:2456-2461 */
 int ogo_supports_flat(uint32_t t, size_t in_dim) { return t == OGO_TYPE_Q8_0 && in_dim % 32 == 0; }
@@ -605,6 +682,8 @@ static void unpack_k_row(uint32_t ggml_type, const uint8_t *row, size_t in_dim, 
     unpack_k_q4_k(row, in_dim, out);
   } else if (ggml_type == OGO_TYPE_Q5_K) {
     unpack_k_q5_k(row, in_dim, out);
+  } else if (ggml_type == OGO_TYPE_Q3_K) {
+    unpack_k_q3_k(row, in_dim, out);
   } else {
     unpack_k_q6_k(row, in_dim, out);
   }
@@ -750,6 +829,8 @@ static int gemv_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size
         v = DISPATCH(dot_k_row_q5_k, row, in_dim, qt, dt, st, io, mo);
       else if (ggml_type == OGO_TYPE_Q6_K)
         v = DISPATCH(dot_k_row_q6_k, row, in_dim, qt, dt, io);
+      else if (ggml_type == OGO_TYPE_Q3_K)
+        v = DISPATCH(dot_k_row_q3_k, row, in_dim, qt, dt, io);
       else
         v = DISPATCH(dot_q8_0, row, in_dim, qt, dt, io);
       yt[o * n_tokens + t] = v;

@@ -47,6 +47,7 @@ extern "C" {
 #define OGO_TYPE_F32 0u
 #define OGO_TYPE_F16 1u
 #define OGO_TYPE_Q8_0 8u
+#define OGO_TYPE_Q3_K 11u
 #define OGO_TYPE_Q4_K 12u
 #define OGO_TYPE_Q5_K 13u
 #define OGO_TYPE_Q6_K 14u
@@ -100,6 +101,10 @@ float ogo_dot_k_row_q5_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
                          const int32_t *sums, int32_t *isum_out, int32_t *imin_out); /* :3181-3213 */
 float ogo_dot_k_row_q6_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
                          int32_t *isum_out);                                          /* :3215-3241 */
+float ogo_dot_k_row_q3_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
+                         int32_t *isum_out);                                          /* :3273-3292 */
+/* quant.rs:883-897: the 16 six-bit scales of a Q3_K block, still biased by 32 */
+void ogo_unpack_q3_k_scales(const uint8_t *packed, int32_t *scales);
 /* per-32 integer sums of a Q8_0 row (isum_out[in_dim/32]) */
 void ogo_block_sums_q8_0(const uint8_t *row, size_t in_dim, const int8_t *q, int32_t *isum_out);
 

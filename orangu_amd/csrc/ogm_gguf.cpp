@@ -1,6 +1,6 @@
 // GGUF reader and matrix uploader: header, metadata key/values, tensor table, alignment
 // (src/gguf.rs:149-280, 300-415 of orangu) and the 2-D matrix view with its shape / size
-// validation (engine/loader.rs:1552-1580), so that a .gguf file's Q8_0 / Q4_K / Q5_K / Q6_K matrices reach
+// validation (engine/loader.rs:1552-1580), so that a .gguf file's Q8_0 / Q3_K / Q4_K / Q5_K / Q6_K matrices reach
 // ogm_weight_upload without the Rust host.  The file is memory-mapped read-only; every read is
 // bounds-checked, so a malformed file gives an error, never an out-of-range access.
 #include <fcntl.h>

@@ -178,6 +178,80 @@ struct FmtQ4K {
   }
 };
 
+// Q3_K: hmask:u8[32] | qs:u8[64] | scales:u8[12] | d:f16                    (quant.rs:826-871)
+// Eight runs of 32 elements; run p takes qs[32 (p / 4) + j] >> 2 (p % 4) and bit p of hmask[j],
+// stored inverted: clear means subtract 4.  Sixteen six-bit scales, biased by 32, one per 16.
+// Repacked as seven pieces, the last one holding scales and d (and two bytes of padding).
+struct FmtQ3K {
+  static constexpr uint32_t TYPE = OGM_Q3_K;
+  static constexpr int PIECES = 7, TILE_BYTES = 64 * 112, ELEMS = 256;
+  static constexpr int XPIECES = 16;
+  static constexpr int AUX16 = 2;  // per-16 sums of q: 16 x i16 per block
+  static constexpr int ACT_GROUP = 256;
+  static constexpr bool HAS_MIN = false;
+  static constexpr int MAX_THREADS = 1024;
+  static constexpr bool HAS_UNPACK = false;
+  struct Regs {
+    uint4 p[PIECES];
+  };
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
+    const uint8_t *base = wt + tile * TILE_BYTES + lane * 16u;
+#pragma unroll
+    for (int i = 0; i < PIECES; i++) r.p[i] = *(const uint4 *)(base + i * 1024);
+  }
+  // unpack_q3_k_scales (quant.rs:883-897) for scale i, minus the bias
+  __device__ static __forceinline__ int scale(const uint4 &t, int i) {
+    const uint32_t w[3] = {t.x, t.y, t.z};
+    const int lowb = i < 8 ? i : i - 8;               // byte holding the low four bits
+    const uint32_t lb = (w[lowb >> 2] >> (8 * (lowb & 3))) & 0xFFu;
+    const uint32_t low = i < 8 ? (lb & 0xFu) : (lb >> 4);
+    const uint32_t hb = (w[2] >> (8 * (i & 3))) & 0xFFu;   // byte 8 + i % 4
+    const uint32_t high = (hb >> (2 * (i >> 2))) & 3u;
+    return (int)(low | (high << 4)) - 32;
+  }
+  // isum = sum over 16 groups of (sc_g - 32) * dot16(q_g, x_g), q = two bits | inverted third bit
+  // minus 4 (vecdot.rs:3273-3292); dot16(v - 4, x) = dot16(v, x) - 4 * sum16(x), exact.
+  template <int UPR>
+  __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
+                                              int &isum, int &imin) {
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;
+    const uint4 s_lo = a.aux[col], s_hi = a.aux[st + col];  // sum16 of groups 0..7, 8..15
+    const uint32_t sw[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+    isum = 0;
+    imin = 0;
+#pragma unroll
+    for (int p = 0; p < 8; p++) {
+#pragma unroll
+      for (int k = 0; k < 2; k++) {
+        const int g = 2 * p + k;                       // group of 16: elements 32p + 16k ..
+        const uint4 qs = r.p[2 + 2 * (p >> 2) + k];    // qs[32 (p / 4) + 16 k ..]
+        const uint4 hm = r.p[k];                       // hmask[16 k ..]
+        const uint4 x = a.xq[g * st + col];
+        const int sh = 2 * (p & 3);
+        const uint32_t m2 = 0x03030303u, m1 = 0x01010101u;
+        int dot = 0;
+        dot = dot4(((qs.x >> sh) & m2) | (((hm.x >> p) & m1) << 2), x.x, dot);
+        dot = dot4(((qs.y >> sh) & m2) | (((hm.y >> p) & m1) << 2), x.y, dot);
+        dot = dot4(((qs.z >> sh) & m2) | (((hm.z >> p) & m1) << 2), x.z, dot);
+        dot = dot4(((qs.w >> sh) & m2) | (((hm.w >> p) & m1) << 2), x.w, dot);
+        const int s16 = (g & 1) ? hi16(sw[g >> 1]) : lo16(sw[g >> 1]);
+        isum += scale(r.p[6], g) * (dot - 4 * s16);
+      }
+    }
+  }
+  // GEMV: total += act.d[s] * d * isum                                       (vecdot.rs:3289)
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int) {
+    return ad * f16_bits_to_f32(r.p[6].w & 0xFFFFu) * (float)isum;
+  }
+  // GEMM: the K-quant GEMM of Q6_K over a row unpacked by unpack_k_q3_k: acc += ad * (d * isum)
+  // (vecdot.rs:2018-2021, 2389-2390)
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int,
+                                                   float &tmin, float &tdot) {
+    tmin = 0.0f;
+    tdot = ad * (f16_bits_to_f32(r.p[6].w & 0xFFFFu) * (float)isum);
+  }
+};
+
 // Q5_K: d:f16 | dmin:f16 | scales:u8[12] | qh:u8[32] | qs:u8[128]          (quant.rs:699-742)
 // Q4_K with a fifth bit: bit j of qh[l] belongs to element l of sub-block j.
 struct FmtQ5K {
@@ -775,6 +849,8 @@ uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order
       return gemm_order ? max_tokens_t<FmtQ4K, true>(in_dim) : max_tokens_t<FmtQ4K, false>(in_dim);
     case OGM_Q5_K:
       return gemm_order ? max_tokens_t<FmtQ5K, true>(in_dim) : max_tokens_t<FmtQ5K, false>(in_dim);
+    case OGM_Q3_K:
+      return gemm_order ? max_tokens_t<FmtQ3K, true>(in_dim) : max_tokens_t<FmtQ3K, false>(in_dim);
     case OGM_Q6_K:
       return gemm_order ? max_tokens_t<FmtQ6K, true>(in_dim) : max_tokens_t<FmtQ6K, false>(in_dim);
     case OGM_Q8_0:
@@ -874,6 +950,9 @@ hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char 
     case OGM_Q5_K:
       if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ5K,gemm>" : "ogm_gemv_kernel<FmtQ5K,gemv>";
       return a.gemm_order ? launch_t<FmtQ5K, true>(a, stream) : launch_t<FmtQ5K, false>(a, stream);
+    case OGM_Q3_K:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ3K,gemm>" : "ogm_gemv_kernel<FmtQ3K,gemv>";
+      return a.gemm_order ? launch_t<FmtQ3K, true>(a, stream) : launch_t<FmtQ3K, false>(a, stream);
     case OGM_Q6_K:
       if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ6K,gemm>" : "ogm_gemv_kernel<FmtQ6K,gemv>";
       return a.gemm_order ? launch_t<FmtQ6K, true>(a, stream) : launch_t<FmtQ6K, false>(a, stream);

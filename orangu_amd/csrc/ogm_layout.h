@@ -1,7 +1,8 @@
 // Tile-planar weight layout shared by the host repacker and the device kernels.
 //
 // A matrix is out_dim rows of `upr` blocks ("units"; one unit is one GGUF block: Q8_0 34 B / 32
-// weights, Q4_K 144 B / 256, Q5_K 176 B / 256, Q6_K 210 B / 256; engine/quant.rs:638-787).  A *tile* holds 64
+// weights, Q3_K 110 B / 256, Q4_K 144 B / 256, Q5_K 176 B / 256, Q6_K 210 B / 256;
+// engine/quant.rs:638-871).  A *tile* holds 64
 // units: R consecutive rows x C consecutive blocks, with C = 4 when a row has a multiple of four
 // blocks (else 2, else 1) and R = 64 / C.  Tiles are ordered [row block][column tile]; inside a
 // tile the unit of (row r, block c) is lane c*R + r.
@@ -13,10 +14,12 @@
 //   * the R rows of one block column are R consecutive lanes, i.e. a contiguous run of R*16
 //     bytes per piece, which is what a tiled GEMM over a row block fetches (prefill GEMM).
 // No byte of a block is changed, dropped or reinterpreted; rows beyond out_dim in the last row
-// block are zero units.
+// block are zero units.  A block whose size is not piece-sized or piece-sized plus two (Q3_K: 110)
+// has its last piece zero-padded to 16 bytes: tile_bytes is then 64 * 16 * pieces.
 //
 //   type   pieces                                   tail
 //   Q8_0   2  (qs[0..32))                           d      (2 B)
+//   Q3_K   7  (hmask[0..32) | qs[0..64) | scales,d + 2 bytes of padding)   -
 //   Q4_K   9  (d,dmin,scales | qs[0..128))          -
 //   Q5_K   11 (d,dmin,scales | qh[0..32) | qs)      -
 //   Q6_K   13 (ql[0..128) | qh[0..64) | scales)     d      (2 B)
@@ -25,6 +28,7 @@
 #include <stdint.h>
 
 #define OGM_Q8_0 8u
+#define OGM_Q3_K 11u
 #define OGM_Q4_K 12u
 #define OGM_Q5_K 13u
 #define OGM_Q6_K 14u
@@ -60,6 +64,9 @@ OGM_HD inline bool ogm_layout_for(uint32_t ggml_type, OgmLayout *l) {
   switch (ggml_type) {
     case OGM_Q8_0:  // d:f16 | qs:i8[32]
       *l = OgmLayout{34, 32, 2, 2, 2, 0, 64 * 34};
+      return true;
+    case OGM_Q3_K:  // hmask:u8[32] | qs:u8[64] | scales:u8[12] | d:f16; the last piece holds 14 bytes
+      *l = OgmLayout{110, 256, 7, 0, 0, 0, 64 * 112};
       return true;
     case OGM_Q4_K:  // d:f16 | dmin:f16 | scales:u8[12] | qs:u8[128]
       *l = OgmLayout{144, 256, 9, 0, 0, 0, 64 * 144};

@@ -644,7 +644,7 @@ hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStrea
 
 // ------------------------------------------------------------------------------------------
 // one row of a quantized matrix as f32: the embedding lookup (LlamaModel::run_layers,
-// llama.rs:609-614, over dequantize_q8_0 / _q4_k / _q5_k / _q6_k, quant.rs:639-649, 666-742, 746-787),
+// llama.rs:609-614, over dequantize_q8_0 / _q3_k / _q4_k / _q5_k / _q6_k, quant.rs:639-649, 666-787, 841-871),
 // reading the tile-planar device copy.  One thread per element; the f32 expressions are the
 // reference's, so the values are bit-identical (built without FMA contraction).
 
@@ -714,6 +714,18 @@ __global__ __launch_bounds__(256) void ogm_dequant_row_kernel(const uint8_t *__r
     const int qv = (int)(hi ? (byte >> 4) : (byte & 0xFu)) + (high ? 16 : 0);
     const float d1 = d * (float)sc, mm = dmin * (float)m;
     v = d1 * (float)qv - mm;
+  } else if (ggml_type == OGM_Q3_K) {
+    // hmask[32] | qs[64] | scales[12] | d, all inside the pieces (quant.rs:841-871)
+    const uint32_t p = j >> 5, jj = j & 31u, g = j >> 4;
+    const uint32_t lo = (piece_byte(32u + 32u * (p >> 2) + jj) >> (2u * (p & 3u))) & 3u;
+    const int qv = (int)lo - (((piece_byte(jj) >> p) & 1u) ? 0 : 4);
+    const uint32_t lb = piece_byte(96u + (g & 7u));
+    const uint32_t low = g < 8 ? (lb & 0xFu) : (lb >> 4);
+    const uint32_t high = (piece_byte(104u + (g & 3u)) >> (2u * (g >> 2))) & 3u;
+    const int sc = (int)(low | (high << 4)) - 32;
+    const float d = __half2float(__ushort_as_half((unsigned short)(piece_byte(108u) | (piece_byte(109u) << 8))));
+    const float dl = d * (float)sc;
+    v = dl * (float)qv;
   } else {  // Q6_K
     const float d = dq_f16(tb + l.pieces * 1024u + lane * 2u);
     const uint32_t h = j >> 7, jj = j & 127u, qd = jj >> 5, li = jj & 31u;

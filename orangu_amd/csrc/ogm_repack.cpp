@@ -7,7 +7,8 @@
 #include "ogm_layout.h"
 
 extern "C" int ogm_supports_type(uint32_t ggml_type) {
-  return ggml_type == OGM_Q8_0 || ggml_type == OGM_Q4_K || ggml_type == OGM_Q5_K || ggml_type == OGM_Q6_K;
+  return ggml_type == OGM_Q8_0 || ggml_type == OGM_Q3_K || ggml_type == OGM_Q4_K || ggml_type == OGM_Q5_K ||
+         ggml_type == OGM_Q6_K;
 }
 
 extern "C" int ogm_supports(uint32_t ggml_type, uint32_t in_dim) {
@@ -22,6 +23,12 @@ extern "C" int ogm_block_layout(uint32_t ggml_type, uint32_t *block_bytes, uint3
   if (block_bytes) *block_bytes = l.block_bytes;
   if (block_elems) *block_elems = l.block_elems;
   return OGM_OK;
+}
+
+// Bytes of the raw block that piece p holds: 16, except a last piece that runs off the block.
+static uint32_t piece_bytes(const OgmLayout &l, uint32_t p) {
+  const uint32_t left = l.block_bytes - (l.piece_off + p * 16);
+  return left < 16 ? left : 16;
 }
 
 static size_t n_tiles_for(const OgmLayout &l, uint32_t in_dim, uint32_t out_dim) {
@@ -64,8 +71,12 @@ extern "C" int ogm_repack_host(uint32_t ggml_type, const void *raw, size_t row_b
       uint32_t lane;
       ogm_unit_place(t, o, blk, &tile_index, &lane);
       uint8_t *tile = dst + tile_index * l.tile_bytes;
-      for (uint32_t p = 0; p < l.pieces; p++)
-        memcpy(tile + p * 1024 + lane * 16, b + l.piece_off + p * 16, 16);
+      for (uint32_t p = 0; p < l.pieces; p++) {
+        const uint32_t have = piece_bytes(l, p);   // 16, or what is left of the block
+        uint8_t *dst_piece = tile + p * 1024 + lane * 16;
+        memcpy(dst_piece, b + l.piece_off + p * 16, have);
+        if (have < 16) memset(dst_piece + have, 0, 16 - have);
+      }
       if (l.tail_bytes)
         memcpy(tile + l.pieces * 1024 + lane * l.tail_bytes, b + l.tail_off, l.tail_bytes);
     }
@@ -90,7 +101,7 @@ extern "C" int ogm_unrepack_host(uint32_t ggml_type, const void *repacked, size_
       ogm_unit_place(t, o, blk, &tile_index, &lane);
       const uint8_t *tile = src + tile_index * l.tile_bytes;
       for (uint32_t p = 0; p < l.pieces; p++)
-        memcpy(b + l.piece_off + p * 16, tile + p * 1024 + lane * 16, 16);
+        memcpy(b + l.piece_off + p * 16, tile + p * 1024 + lane * 16, piece_bytes(l, p));
       if (l.tail_bytes)
         memcpy(b + l.tail_off, tile + l.pieces * 1024 + lane * l.tail_bytes, l.tail_bytes);
     }

@@ -8,9 +8,9 @@ from __future__ import annotations
 
 import numpy as np
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
-BLOCK = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
-TYPE_NAME = {Q8_0: "q8_0", Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k"}
+Q8_0, Q3_K, Q4_K, Q5_K, Q6_K = 8, 11, 12, 13, 14
+BLOCK = {Q8_0: (34, 32), Q3_K: (110, 256), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+TYPE_NAME = {Q8_0: "q8_0", Q3_K: "q3_k", Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k"}
 
 
 def row_bytes(ggml_type: int, in_dim: int) -> int:
@@ -62,6 +62,8 @@ def pin_scales(raw: np.ndarray, ggml_type: int) -> np.ndarray:
         blocks[:, 2:4] = (0x00, 0x2C)
     elif ggml_type == Q6_K:
         blocks[:, 208:210] = (0x00, 0x30)
+    elif ggml_type == Q3_K:   # vecdot.rs:3478
+        blocks[:, 108:110] = (0x00, 0x30)
     return raw
 
 
@@ -139,9 +141,9 @@ def synth_weights(ggml_type: int, in_dim: int, out_dim: int, seed: int) -> np.nd
         dm = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)
         raw[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
         raw[:, 2:4] = dm.view(np.uint8).reshape(-1, 2)
-    else:
+    else:   # Q6_K, Q3_K: d is the block's last field
         d = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)
-        raw[:, 208:210] = d.view(np.uint8).reshape(-1, 2)
+        raw[:, bb - 2:bb] = d.view(np.uint8).reshape(-1, 2)
     return raw.reshape(-1)
 
 

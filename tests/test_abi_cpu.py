@@ -7,7 +7,7 @@ import re
 import numpy as np
 import pytest
 
-from helpers import BLOCK, Q4_K, Q6_K, Q8_0, row_bytes
+from helpers import BLOCK, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, row_bytes
 from orangu_amd import capi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -32,7 +32,8 @@ def test_supports_predicates_follow_vecdot(lib):
     """vecdot.rs:274-283 for the types built; Backend::supports_type (mod.rs:493)."""
     assert lib.ogm_supports_type(Q8_0) and lib.ogm_supports_type(Q4_K) and lib.ogm_supports_type(Q6_K)
     assert lib.ogm_supports_type(13) and lib.ogm_supports(13, 256) and not lib.ogm_supports(13, 128)   # Q5_K
-    assert not lib.ogm_supports_type(0) and not lib.ogm_supports_type(11)
+    assert lib.ogm_supports_type(11) and lib.ogm_supports(11, 512) and not lib.ogm_supports(11, 896)   # Q3_K
+    assert not lib.ogm_supports_type(0) and not lib.ogm_supports_type(10)
     assert lib.ogm_supports(Q8_0, 96) and not lib.ogm_supports(Q8_0, 100)
     assert lib.ogm_supports(Q4_K, 512) and not lib.ogm_supports(Q4_K, 896)
     assert lib.ogm_supports(Q6_K, 256) and not lib.ogm_supports(Q6_K, 0)
@@ -50,7 +51,11 @@ def tiling(upr, out_dim):
     return C_, R, upr // C_, (out_dim + R - 1) // R
 
 
-@pytest.mark.parametrize("ggml_type", [Q8_0, Q4_K, Q6_K])
+# bytes a unit takes in the tile-planar form: the raw block, except Q3_K whose last piece is padded
+TILE_UNIT = {Q8_0: 34, Q3_K: 112, Q4_K: 144, Q5_K: 176, Q6_K: 210}
+
+
+@pytest.mark.parametrize("ggml_type", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_blocks,out_dim", [(1, 1), (3, 11), (16, 64), (7, 130), (6, 33), (8, 70)])
 def test_repack_is_a_bijection_on_the_raw_bytes(lib, ggml_type, in_blocks, out_dim):
     bb, be = BLOCK[ggml_type]
@@ -60,23 +65,25 @@ def test_repack_is_a_bijection_on_the_raw_bytes(lib, ggml_type, in_blocks, out_d
     raw = rng.integers(0, 256, rb * out_dim, dtype=np.uint8)
     size = lib.ogm_repacked_size(ggml_type, in_dim, out_dim)
     C_, R, nct, nrb = tiling(in_blocks, out_dim)
-    assert size == nrb * nct * 64 * bb
+    assert size == nrb * nct * 64 * TILE_UNIT[ggml_type]
     packed = np.full(size, 0xAA, np.uint8)
     assert lib.ogm_repack_host(ggml_type, raw.ctypes.data, rb, in_dim, out_dim, packed.ctypes.data) == 0
     back = np.zeros_like(raw)
     assert lib.ogm_unrepack_host(ggml_type, packed.ctypes.data, rb, in_dim, out_dim, back.ctypes.data) == 0
     assert np.array_equal(back, raw)
-    if out_dim % R == 0:
-        # no padding rows: the packed form is a permutation of the raw bytes
+    if out_dim % R == 0 and TILE_UNIT[ggml_type] == bb:
+        # no padding rows or bytes: the packed form is a permutation of the raw bytes
         assert np.array_equal(np.bincount(packed, minlength=256), np.bincount(raw, minlength=256))
 
 
 @pytest.mark.parametrize("t,npieces,piece_off,tail_off,tail", [(Q4_K, 9, 0, 0, 0), (Q6_K, 13, 0, 208, 2),
-                                                              (Q8_0, 2, 2, 0, 2)])
+                                                              (Q8_0, 2, 2, 0, 2), (Q5_K, 11, 0, 0, 0),
+                                                              (Q3_K, 7, 0, 0, 0)])
 @pytest.mark.parametrize("in_blocks,out_dim", [(8, 70), (6, 40), (3, 65)])
 def test_repack_places_pieces_in_planes(lib, t, npieces, piece_off, tail_off, tail, in_blocks, out_dim):
     """Unit (row o, block b): tile (o / R) * nct + b / C, lane (b % C) * R + o % R; piece p at
-    tile * 64 * block_bytes + p * 1024 + lane * 16, tails after the pieces; padding rows zero."""
+    tile * tile bytes + p * 1024 + lane * 16, tails after the pieces; padding rows zero, and so
+    are the two bytes that complete Q3_K's last piece."""
     bb, be = BLOCK[t]
     in_dim = in_blocks * be
     rb = row_bytes(t, in_dim)
@@ -87,13 +94,14 @@ def test_repack_places_pieces_in_planes(lib, t, npieces, piece_off, tail_off, ta
     seen = np.zeros(packed.size, bool)
     for o in range(out_dim):
         for b in range(in_blocks):
-            base = ((o // R) * nct + b // C_) * 64 * bb
+            base = ((o // R) * nct + b // C_) * 64 * TILE_UNIT[t]
             lane = (b % C_) * R + o % R
             src = o * rb + b * bb
             for p in range(npieces):
                 off = base + p * 1024 + lane * 16
-                assert np.array_equal(packed[off:off + 16], raw[src + piece_off + p * 16:src + piece_off + p * 16 + 16])
-                seen[off:off + 16] = True
+                have = min(16, bb - piece_off - p * 16)
+                assert np.array_equal(packed[off:off + have], raw[src + piece_off + p * 16:src + piece_off + p * 16 + have])
+                seen[off:off + have] = True
             if tail:
                 off = base + npieces * 1024 + lane * tail
                 assert np.array_equal(packed[off:off + tail], raw[src + tail_off:src + tail_off + tail])

@@ -8,7 +8,7 @@ import sys
 import numpy as np
 import pytest
 
-from helpers import Q4_K, Q5_K, Q6_K, Q8_0, synth_weights
+from helpers import Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, synth_weights
 from oracle import llama_ref as R
 
 pytestmark = pytest.mark.gpu
@@ -90,6 +90,19 @@ def test_decode_steps_from_an_empty_cache(be, types):
     try:
         for pos in range(6):
             step_both(ref, dev, rng.standard_normal(256).astype(f32), pos, f"types {types} pos {pos}")
+    finally:
+        dev.close()
+
+
+def test_decode_with_q3_k_value_and_down_projections(be):
+    """Q3_K in the v and down projections (what a Q3_K_M file does), one layer: the synthetic Q3_K
+    weights are large, and with two layers of them the final hidden state is a small difference of
+    huge terms whose f16 cache rounding dominates any tolerance relative to the result."""
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=1,
+                          types=(Q4_K, Q3_K, Q3_K, Q5_K), max_ctx=16, seed=5)
+    try:
+        for pos in range(5):
+            step_both(ref, dev, rng.standard_normal(256).astype(f32), pos, f"q3_k v/down pos {pos}")
     finally:
         dev.close()
 
@@ -194,6 +207,7 @@ def test_matrices_uploaded_from_a_gguf_file_multiply_like_direct_uploads(be, tmp
     (Q4_K, 256, 3), (Q4_K, 1024, 130), (Q4_K, 4096, 67),
     (Q6_K, 256, 1), (Q6_K, 768, 65), (Q6_K, 4096, 129),
     (Q5_K, 256, 2), (Q5_K, 1280, 70), (Q5_K, 4096, 33),
+    (Q3_K, 256, 2), (Q3_K, 1280, 70), (Q3_K, 4096, 33),
 ])
 def test_dequant_rows_bits(be, t, in_dim, out_dim):
     """Rows of the device copy equal dequantize_q8_0 / _q4_k / _q6_k (quant.rs:639-787) bit for bit."""
@@ -211,7 +225,7 @@ def test_dequant_rows_bits(be, t, in_dim, out_dim):
         be.dequant_rows(w, out_dim, 1)
 
 
-@pytest.mark.parametrize("embd_t", [Q4_K, Q5_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("embd_t", [Q3_K, Q4_K, Q5_K, Q6_K, Q8_0])
 def test_generate_matches_stepwise(be, embd_t):
     """Greedy generation on the device = the oracle's loop: embedding row of the token
     (llama.rs:609-614), decode step, last-of-equal argmax (sampling.rs:336-343)."""

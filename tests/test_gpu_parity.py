@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (BLOCK, Q4_K, Q5_K, Q6_K, Q8_0, NextByte, activations, activations_t, cpu_rs_weights,
+from helpers import (BLOCK, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, NextByte, activations, activations_t, cpu_rs_weights,
                      fixture_row, k_fixture, row_bytes, synth_weights, synth_x)
 from test_oracle_quantize import adversarial_blocks
 
@@ -67,7 +67,7 @@ def test_f16_scale_conversion_matches_quant_rs_for_all_inputs(be):
     assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
 def test_upload_download_round_trip(be, t):
     """unrepack(repack(W)) == W through the device."""
     bb, bel = BLOCK[t]
@@ -114,6 +114,7 @@ def test_quantizer_ties_round_away_from_zero(be):
 @pytest.mark.parametrize("t,in_dim,out_dim,T", [
     (Q4_K, 256, 5, 1), (Q4_K, 2048, 37, 3), (Q4_K, 4864, 9, 1),
     (Q5_K, 256, 5, 1), (Q5_K, 2048, 37, 3), (Q5_K, 4864, 9, 2),
+    (Q3_K, 256, 5, 1), (Q3_K, 2048, 37, 3), (Q3_K, 5632, 9, 2),
     (Q6_K, 256, 5, 1), (Q6_K, 2048, 37, 3), (Q6_K, 4864, 9, 2),
     (Q8_0, 96, 11, 1), (Q8_0, 896, 19, 3), (Q8_0, 4864, 7, 1),
 ])
@@ -131,7 +132,8 @@ def test_block_integer_sums_bit_exact(be, t, in_dim, out_dim, T):
 # ---------------------------------------------------------------- GEMV / matmul values
 
 CHECK = [(Q8_0, 896), (Q8_0, 4864), (Q4_K, 256), (Q4_K, 4864), (Q6_K, 256), (Q6_K, 4864),
-         (Q4_K, 2048), (Q6_K, 5632), (Q5_K, 256), (Q5_K, 3072), (Q5_K, 4864)]
+         (Q4_K, 2048), (Q6_K, 5632), (Q5_K, 256), (Q5_K, 3072), (Q5_K, 4864), (Q3_K, 256), (Q3_K, 2048),
+         (Q3_K, 5632)]
 
 
 @pytest.mark.parametrize("t,in_dim", CHECK)
@@ -157,14 +159,14 @@ def test_gemv_matches_cpu_matmul_on_reference_fixtures(be, t, in_dim, seed):
         assert abs(float(got[o]) - float(ref[o])) <= budget * max(mag, 1e-6)
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("T", [1, 2, 5, 8, 13])
 def test_matmul_decode_matches_cpu_and_each_token_alone(be, t, T):
     """backend/cpu.rs:623-650: a decode batch's row t is what token t gives alone."""
     in_dim = 128 if t == Q8_0 else 512
     out_dim = 7
     nb = NextByte(0x0051AB1E5EED)
-    raw = cpu_rs_weights(t, in_dim, out_dim, nb) if t != Q6_K else np.concatenate(
+    raw = cpu_rs_weights(t, in_dim, out_dim, nb) if t not in (Q6_K, Q3_K) else np.concatenate(
         [fixture_row(t, in_dim, 5 + o) for o in range(out_dim)])
     x = np.array([np.float32(nb()) / np.float32(255.0) * np.float32(2.0) - np.float32(1.0)
                   for _ in range(T * in_dim)], np.float32)
@@ -178,13 +180,13 @@ def test_matmul_decode_matches_cpu_and_each_token_alone(be, t, T):
         assert_bits(got[k], alone, f"token {k} alone")
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
 def test_matmul_multi_token_matches_cpu_gemm(be, t):
     """backend/cpu.rs:544-582 shapes: in = 3 blocks, out = 11 (odd), T in 1,2,5,77,3,1 from one
     reused backend; matmul at T > 1 follows the CPU GEMM kernels."""
     in_dim = BLOCK[t][1] * 3
     out_dim = 11
-    raw = cpu_rs_weights(t, in_dim, out_dim, NextByte(0x9E3779B97F4A7C15)) if t != Q6_K else \
+    raw = cpu_rs_weights(t, in_dim, out_dim, NextByte(0x9E3779B97F4A7C15)) if t not in (Q6_K, Q3_K) else \
         np.concatenate([fixture_row(t, in_dim, 50 + o) for o in range(out_dim)])
     w = qm(raw, t, in_dim, out_dim)
     for T in (1, 2, 5, 77, 3, 1):
@@ -197,7 +199,7 @@ def test_matmul_multi_token_matches_cpu_gemm(be, t):
         assert_bits(got, want, f"matmul T={T}")
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_dim", [256, 2048, 8192])
 def test_k_gemm_fixture(be, t, in_dim):
     """vecdot.rs:4479-4513: 5 rows x 7 tokens, seed 4242."""
@@ -208,7 +210,7 @@ def test_k_gemm_fixture(be, t, in_dim):
     assert_bits(got, want, "k_gemm")
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q3_K, Q4_K, Q5_K, Q6_K])
 def test_gemm_result_is_independent_of_the_batch_size(be, t):
     """vecdot.rs:4522-4549: exact equality."""
     in_dim, out_dim = 512, 4
@@ -273,6 +275,7 @@ def test_error_statuses(be):
     (Q4_K, 4096, 1024),     # config 3 k/v
     (Q6_K, 14336, 4096),    # config 5 ffn_down
     (Q5_K, 4096, 4096), (Q5_K, 14336, 4096),   # the same shapes in Q5_K
+    (Q3_K, 4096, 4096), (Q3_K, 14336, 4096),   # and in Q3_K
 ])
 def test_benchmark_shapes_match_cpu(be, t, in_dim, out_dim):
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim)
@@ -450,6 +453,7 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign):
     (Q4_K, 256, 5), (Q4_K, 768, 70), (Q4_K, 4096, 257), (Q4_K, 14336, 96), (Q4_K, 18432, 40),
     (Q6_K, 256, 3), (Q6_K, 1280, 65), (Q6_K, 4096, 130), (Q6_K, 14336, 48), (Q6_K, 18432, 17),
     (Q5_K, 256, 5), (Q5_K, 768, 70), (Q5_K, 4096, 257), (Q5_K, 14336, 96), (Q5_K, 18432, 40),
+    (Q3_K, 256, 5), (Q3_K, 768, 70), (Q3_K, 4096, 257), (Q3_K, 14336, 96), (Q3_K, 18432, 40),
 ])
 def test_single_token_gemv_quantizes_in_kernel_or_before_with_the_same_bits(be, t, in_dim, out_dim):
     """One token: the GEMV that quantizes its own activations and the quantizer kernel + GEMV
@@ -476,7 +480,7 @@ def test_single_token_gemv_quantizes_in_kernel_or_before_with_the_same_bits(be, 
             assert_bits(got[ok], want[ok], f"fuse mode {mode}")
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("T,decode", [(1, False), (1, True), (4, True), (3, False), (16, False), (11, True)])
 def test_grouped_weights_over_one_input_equal_single_calls(be, t, T, decode):
     """q/k/v and gate/up read one input (engine/arch/mod.rs:1082-1096): the grouped call equals
@@ -544,7 +548,7 @@ def test_matmul_batch_groups_ops_that_share_their_input(be):
 
 
 @pytest.mark.parametrize("t,in_dim", [(Q8_0, 1056), (Q4_K, 1024), (Q4_K, 1536), (Q6_K, 1024), (Q6_K, 256), (Q5_K, 1024),
-                                      (Q5_K, 768)])
+                                      (Q5_K, 768), (Q3_K, 1024), (Q3_K, 1280)])
 def test_row_blocks_per_workgroup_do_not_change_a_bit(be, t, in_dim):
     """A workgroup may own several row blocks (ragged last group, last row block partly beyond
     out_dim, several matrices in one launch): every split gives the CPU path's bits."""
@@ -634,3 +638,28 @@ def test_q5k_extreme_integer_ranges(be, sign):
     assert_bits(be.matmul(x[0], 1, w), oracle.matmul(Q5_K, raw, in_dim, out_dim, x[0], 1), "gemv")
     assert_bits(be.matmul(x, T, w), oracle.matmul(Q5_K, raw, in_dim, out_dim, x, T), "matmul")
     assert_bits(be.matmul_decode(x, T, w), oracle.matmul_decode(Q5_K, raw, in_dim, out_dim, x, T), "decode")
+
+
+@pytest.mark.parametrize("hmask,qs", [(0x00, 0x00), (0x00, 0xFF), (0xFF, 0xFF)])
+def test_q3k_extreme_integer_ranges(be, hmask, qs):
+    """Q3_K's poles: weights -4 (hmask clear, bits 0), -1 and 3, every scale byte 0xFF (scales
+    63 - 32 = 31) or 0x00 (-32), activations +-127: |isum| up to 4.2e6 (vecdot.rs:3271-3272)."""
+    in_dim, out_dim, T = 1024, 20, 12
+    for scb in (0xFF, 0x00):
+        blocks = np.zeros((out_dim * 4, 110), np.uint8)
+        blocks[:, 0:32] = hmask
+        blocks[:, 32:96] = qs
+        blocks[:, 96:108] = scb
+        blocks[:, 108:110] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+        x = np.full((T, in_dim), 127.0, np.float32)
+        x[1::2] *= -1
+        x[:, ::7] = -126.0
+        raw = blocks.reshape(-1)
+        w = qm(raw, Q3_K, in_dim, out_dim)
+        isum, _ = be.dump_block_sums(x[0], 1, w)
+        wi, _ = oracle.block_sums(Q3_K, raw, in_dim, out_dim, x[0], 1)
+        assert np.array_equal(isum, wi)
+        say("extreme q3k isum", int(np.abs(isum).max()))
+        assert_bits(be.matmul(x[0], 1, w), oracle.matmul(Q3_K, raw, in_dim, out_dim, x[0], 1), "gemv")
+        assert_bits(be.matmul(x, T, w), oracle.matmul(Q3_K, raw, in_dim, out_dim, x, T), "matmul")
+        assert_bits(be.matmul_decode(x, T, w), oracle.matmul_decode(Q3_K, raw, in_dim, out_dim, x, T), "decode")

@@ -4,11 +4,12 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Q4_K, Q5_K, Q6_K, Q8_0
+from helpers import Q3_K, Q4_K, Q5_K, Q6_K, Q8_0
 
 # quant.rs:1389-1417 GOLDEN (the types on the path)
 GOLDEN = [
     (Q8_0, "q8_0", 256, 0xC5D58782F54E52E5),
+    (Q3_K, "q3_k", 512, 0x2183E0B0538C6BE5),
     (Q4_K, "q4_k", 512, 0x9A7268A432A5C5FA),
     (Q5_K, "q5_k", 512, 0x41C70B9BE1696E6D),
     (Q6_K, "q6_k", 512, 0x61001D333CB0CFD1),
@@ -44,6 +45,7 @@ def test_tensor_byte_size_and_block_layout():
     assert oracle.tensor_byte_size(Q4_K, 512) == 2 * 144
     assert oracle.tensor_byte_size(Q6_K, 512) == 2 * 210
     assert oracle.tensor_byte_size(Q5_K, 256) == 176  # quant.rs:1701
+    assert oracle.tensor_byte_size(Q3_K, 512) == 2 * 110
     assert oracle.tensor_byte_size(Q4_K, 100) == -2  # not a whole number of blocks
     assert oracle.tensor_byte_size(99, 256) == -1  # unknown type
 
@@ -205,3 +207,67 @@ def test_dequantize_q5_k_bit_to_sub_block_mapping():
     for j in range(8):
         nib = 1 if j % 2 == 0 else 2
         assert np.all(out[j] == np.float32(j + 1) * nib - np.float32(0.5)), j
+
+
+def test_unpack_q3_k_scales_against_bit_by_bit_decode():
+    """quant.rs:883-897: low four bits of scales 0..8 in the low nibbles of bytes 0..8, of scales
+    8..16 in their high nibbles; the two high bits of scale i at bit 2 * (i / 4) of byte 8 + i % 4.
+    Also ggml's kmask shuffle on little-endian words, as a second formulation."""
+    rng = np.random.default_rng(3)
+    for _ in range(20):
+        packed = rng.integers(0, 256, 12, dtype=np.uint8)
+        got = oracle.unpack_q3_k_scales(packed)
+        want = np.zeros(16, np.int32)
+        for i in range(16):
+            low = packed[i] & 0xF if i < 8 else packed[i - 8] >> 4
+            high = (packed[8 + i % 4] >> (2 * (i // 4))) & 3
+            want[i] = int(low) | (int(high) << 4)
+        assert np.array_equal(got, want)
+        a = [int.from_bytes(packed[4 * k:4 * k + 4].tobytes(), "little") for k in range(3)]
+        k1, k2 = 0x03030303, 0x0F0F0F0F
+        tmp = a[2]
+        w = [(a[0] & k2) | (((tmp >> 0) & k1) << 4), (a[1] & k2) | (((tmp >> 2) & k1) << 4),
+             ((a[0] >> 4) & k2) | (((tmp >> 4) & k1) << 4), ((a[1] >> 4) & k2) | (((tmp >> 6) & k1) << 4)]
+        ggml = np.frombuffer(b"".join(x.to_bytes(4, "little") for x in w), np.uint8).astype(np.int32)
+        assert np.array_equal(got, ggml)
+
+
+def _q3k_block(hmask=0x00, qs=0x00, scales=0x20, d=1.0):
+    block = np.zeros(110, np.uint8)
+    block[0:32] = hmask
+    block[32:96] = qs
+    block[96:108] = scales
+    block[108:110] = _f16(d)
+    return block
+
+
+# scale bytes 0x20: low nibbles 0 (scales 0..8), high nibbles 2 (scales 8..16); the byte's bits 4..5
+# are also the high bits of scales 8..12: scales = 0 x 8, 34 x 4, 2 x 4, each minus 32
+Q3K_SC_0X20 = np.array([0] * 8 + [34] * 4 + [2] * 4, np.float32) - 32
+
+
+def test_dequantize_q3_k_inverted_high_bit_and_signed_scales():
+    """vecdot.rs:3938-3968 on the dequantizer: hmask clear subtracts 4, hmask set subtracts nothing;
+    the six-bit scales are biased by 32 (quant.rs:857)."""
+    per_elem = np.repeat(Q3K_SC_0X20, 16)
+    assert np.array_equal(oracle.dequantize(Q3_K, _q3k_block(hmask=0x00), 256), per_elem * -4)
+    assert np.all(oracle.dequantize(Q3_K, _q3k_block(hmask=0xFF), 256) == 0.0)
+    assert np.array_equal(oracle.dequantize(Q3_K, _q3k_block(hmask=0xFF, qs=0xFF), 256), per_elem * 3)
+
+
+def test_dequantize_q3_k_element_order():
+    """Run p (32 elements) takes qs[32 (p / 4) ..][j] >> 2 (p % 4) and hmask bit p; groups of 16
+    take scales 2p and 2p + 1 (quant.rs:851-868).  One qs bit, one hmask bit at a time."""
+    for p in range(8):
+        for j in (0, 15, 16, 31):
+            g = 2 * p + j // 16
+            block = _q3k_block(hmask=0xFF)
+            block[32 + 32 * (p // 4) + j] = 1 << (2 * (p % 4))
+            want = np.zeros(256, np.float32)
+            want[32 * p + j] = Q3K_SC_0X20[g] * 1
+            assert np.array_equal(oracle.dequantize(Q3_K, block, 256), want), (p, j)
+            block = _q3k_block(hmask=0xFF)
+            block[j] = 0xFF ^ (1 << p)          # clear hmask bit p of element j only
+            want = np.zeros(256, np.float32)
+            want[32 * p + j] = Q3K_SC_0X20[g] * -4
+            assert np.array_equal(oracle.dequantize(Q3_K, block, 256), want), (p, j)

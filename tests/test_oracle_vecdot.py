@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (BLOCK, Q4_K, Q5_K, Q6_K, Q8_0, NextByte, activations, cpu_rs_weights, fixture_row,
+from helpers import (BLOCK, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, NextByte, activations, cpu_rs_weights, fixture_row,
                      k_fixture, row_bytes)
 
 
@@ -73,6 +73,19 @@ def np_unpack(ggml_type, row, in_dim):
         qh = blocks[:, 16:48].astype(np.int64)                                        # [nb][32]
         hi = ((qh[:, None, :] >> np.arange(8)[None, :, None]) & 1) * 16              # [nb][8][32]
         return q4 + hi.reshape(-1), sce, mne, d, dmin
+    if ggml_type == Q3_K:   # hmask[32] | qs[64] | scales[12] | d; run p: qs[32 (p/4) + j] >> 2 (p%4), hmask bit p
+        hm = blocks[:, 0:32].astype(np.int64)
+        qs = blocks[:, 32:96].astype(np.int64).reshape(nb, 2, 32)
+        pk = blocks[:, 96:108].astype(np.int64)
+        d = blocks[:, 108:110].copy().view(np.float16).astype(np.float32).reshape(-1)
+        q = np.empty((nb, 8, 32), np.int64)
+        for p in range(8):
+            q[:, p, :] = ((qs[:, p // 4, :] >> (2 * (p % 4))) & 3) - np.where((hm >> p) & 1, 0, 4)
+        sc = np.empty((nb, 16), np.int64)
+        for i in range(16):
+            low = pk[:, i] & 15 if i < 8 else pk[:, i - 8] >> 4
+            sc[:, i] = (low | (((pk[:, 8 + i % 4] >> (2 * (i // 4))) & 3) << 4)) - 32
+        return q.reshape(-1), np.repeat(sc, 16, axis=1).reshape(-1), None, d, None
     ql = blocks[:, 0:128].astype(np.int64).reshape(nb, 2, 2, 32)  # [h][r&1][l]
     qh = blocks[:, 128:192].astype(np.int64).reshape(nb, 2, 32)
     sc = blocks[:, 192:208].copy().view(np.int8).astype(np.int64)
@@ -94,7 +107,7 @@ def np_block_sums(ggml_type, row, in_dim, xq):
     return isum, imin
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_dim", [256, 2048])
 def test_k_row_integer_sums_equal_numpy_int64(ggml_type, in_dim):
     """Per-super-block isum / imin (vecdot.rs:3152-3178, 3215-3241) against int64 numpy over an
@@ -172,7 +185,7 @@ def test_fused_dot_row_matches_dequantize_reference(ggml_type, in_dim, seed):
     assert abs(float(got) - float(ref)) <= 0.01 * max(mag, 1e-6)
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_dim", [256, 2048, 3072, 5632])
 @pytest.mark.parametrize("seed", [1, 7, 99])
 def test_k_row_decode_matches_dequantize_reference(ggml_type, in_dim, seed):
@@ -193,7 +206,7 @@ def test_integer_accumulators_stay_inside_i32_by_construction():
     assert 128 * 32 * 127 * 256 < 2**31
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_dim", [256, 2048, 8192])
 def test_k_gemm_matches_dequantize_reference(ggml_type, in_dim):
     """vecdot.rs:4479-4513: 5 rows x 7 tokens, seed 4242, budget 0.01 * sum|w x|."""
@@ -209,7 +222,7 @@ def test_k_gemm_matches_dequantize_reference(ggml_type, in_dim):
             assert abs(got[o, t] - ref) <= 0.01 * max(mag, 1e-6) + 1e-6 * mag
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q3_K, Q4_K, Q5_K, Q6_K])
 def test_k_gemm_result_is_independent_of_the_batch_size(ggml_type):
     """vecdot.rs:4522-4549: exact equality."""
     in_dim, out_dim = 512, 4
@@ -220,7 +233,7 @@ def test_k_gemm_result_is_independent_of_the_batch_size(ggml_type):
         assert np.array_equal(part.view(np.uint32), full[:, :n].view(np.uint32))
 
 
-@pytest.mark.parametrize("ggml_type", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q3_K, Q4_K, Q5_K, Q6_K])
 def test_k_gemm_float_order_rebuilt_from_integer_sums(ggml_type):
     """gemm_k_q4_k: acc -= (ad*dmin)*imin over all super-blocks first, then acc += ad*(d*isum)
     (vecdot.rs:2229-2303); gemm_k_q6_k: acc += ad*(d*isum) (vecdot.rs:2386-2391).  Rebuilt in
@@ -315,6 +328,8 @@ def test_supports_predicates():
     """vecdot.rs:274-283, 1821-1826, 3083-3093, 2456-2461 for the three types."""
     assert oracle.supports(Q8_0, 96) and not oracle.supports(Q8_0, 100)
     assert oracle.supports(Q4_K, 512) and not oracle.supports(Q4_K, 896)
+    assert oracle.supports(Q3_K, 256) and oracle.supports_k(Q3_K, 2048) and not oracle.supports_k_row(Q3_K, 896)
+    assert not oracle.supports_flat(Q3_K, 2048)   # vecdot.rs:4082, 4593-4594
     assert oracle.supports(Q5_K, 256) and oracle.supports_k(Q5_K, 512) and oracle.supports_k_row(Q5_K, 768)
     assert not oracle.supports(Q5_K, 128) and not oracle.supports_flat(Q5_K, 256)
     assert oracle.supports_k(Q6_K, 256) and not oracle.supports_k(Q8_0, 256)
@@ -350,3 +365,21 @@ def test_q5_k_unpack_applies_the_high_bit_to_every_sub_block():
     assert v == np.float32(act[1][0] * np.float32(np.float32(1.0) * np.float32(isum[0])))
     got = oracle.k_gemm_t(Q5_K, block, 256, 1, x, 1)
     assert got[0, 0] == np.float32(act[1][0] * np.float32(isum[0]))
+
+
+def test_q3_k_unpack_applies_the_inverted_high_bit():
+    """vecdot.rs:3938-3968 through the decode path and the K-GEMM path: with every 2-bit field 0,
+    hmask clear makes every weight -4 and hmask set makes it 0.  Scale bytes 0x20 unpack to
+    0 x 8, 34 x 4, 2 x 4 (minus 32); all-one activations quantize to 127."""
+    x = np.ones(256, np.float32)
+    act = oracle.quantize_act_k_row(x)
+    for hmask, w in ((0x00, -4), (0xFF, 0)):
+        block = np.zeros(110, np.uint8)
+        block[0:32] = hmask
+        block[96:108] = 0x20
+        block[108:110] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+        v, isum, _ = oracle.dot_k_row(Q3_K, block, act, want_sums=True)
+        assert isum[0] == (8 * (0 - 32) + 4 * (34 - 32) + 4 * (2 - 32)) * 16 * w * 127
+        assert v == np.float32(np.float32(act[1][0] * np.float32(1.0)) * np.float32(isum[0]))
+        got = oracle.k_gemm_t(Q3_K, block, 256, 1, x, 1)
+        assert got[0, 0] == np.float32(act[1][0] * np.float32(np.float32(1.0) * np.float32(isum[0])))
