@@ -2,7 +2,7 @@
  * orangu_mi355x.h -- C ABI of the MI355X (gfx950) quantized matmul backend for orangu-server.
  *
  * This is the boundary a Rust `impl Backend` binds through FFI.  It replaces, for the GGUF types
- * Q8_0, Q3_K, Q4_K, Q5_K and Q6_K, what `engine::backend::Backend` asks of a device
+ * Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K and Q6_K, what `engine::backend::Backend` asks of a device
  * (src/bin/orangu-server/engine/backend/mod.rs:309-496) and reproduces the arithmetic of
  * `CpuBackend` (engine/backend/cpu.rs:55-317) over `engine::vecdot`:
  *   - activation int8 quantization, per-block integer sums: bit-exact with the CPU path;
@@ -45,11 +45,14 @@ typedef enum ogm_status {
 } ogm_status;
 
 /* ggml type ids (engine/quant.rs:50-61) */
+#define OGM_TYPE_Q4_0 2u
+#define OGM_TYPE_Q5_0 6u
 #define OGM_TYPE_Q8_0 8u
 #define OGM_TYPE_Q3_K 11u
 #define OGM_TYPE_Q4_K 12u
 #define OGM_TYPE_Q5_K 13u
 #define OGM_TYPE_Q6_K 14u
+#define OGM_TYPE_IQ4_NL 20u
 
 /* Activation quantization modes */
 #define OGM_ACT_PER_32 0  /* vecdot::quantize_act,       vecdot.rs:79-126   (Q8_0 weights)   */
@@ -70,7 +73,8 @@ int ogm_device_name(ogm_ctx *ctx, char *buf, size_t buf_len);
 
 /* ---- capabilities ---------------------------------------------------------------------- */
 
-/* Backend::supports_type (backend/mod.rs:493): 1 for Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, else 0. */
+/* Backend::supports_type (backend/mod.rs:493): 1 for Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K,
+ * Q6_K, else 0. */
 int ogm_supports_type(uint32_t ggml_type);
 /* vecdot::supports (vecdot.rs:274-283) for those types: Q8_0 needs in_dim % 32 == 0, the
  * K-quants in_dim % 256 == 0. */
@@ -172,7 +176,7 @@ int ogm_quantize_act(ogm_ctx *ctx, int mode, const float *x, size_t n, int8_t *q
  * Q4_K and Q5_K: isum = sum_j sc_j * dot32_j and imin = sum_j m_j * bsum_j per super-block
  * (vecdot.rs:3152-3213); Q6_K and Q3_K: isum per super-block (vecdot.rs:3215-3241, 3273-3292),
  * imin untouched;
- * Q8_0: isum per 32-block (vecdot.rs:2829-2838).  Arrays are [n_tokens][out_dim][blocks per
+ * Q8_0, Q5_0, Q4_0, IQ4_NL: isum per 32-block (vecdot.rs:2829-2883).  Arrays are [n_tokens][out_dim][blocks per
  * row]; imin may be NULL.  Runs the same kernels as ogm_matmul_decode with a dump switch. */
 int ogm_dump_block_sums(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint32_t n_tokens,
                         int32_t *isum, int32_t *imin);

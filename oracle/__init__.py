@@ -16,8 +16,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liborangu_oracle.so")
 
-Q8_0, Q3_K, Q4_K, Q5_K, Q6_K = 8, 11, 12, 13, 14
-BLOCK_LAYOUT = {Q8_0: (34, 32), Q3_K: (110, 256), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+Q4_0, Q5_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL = 2, 6, 8, 11, 12, 13, 14, 20
+BLOCK_LAYOUT = {Q4_0: (18, 32), Q5_0: (22, 32), Q8_0: (34, 32), Q3_K: (110, 256), Q4_K: (144, 256), Q5_K: (176, 256),
+                Q6_K: (210, 256), IQ4_NL: (18, 32)}
 
 
 def build() -> str:
@@ -72,6 +73,10 @@ def lib() -> C.CDLL:
         L.ogo_dot_k_row_q3_k.restype = C.c_float
         L.ogo_dot_k_row_q3_k.argtypes = [u8p, sz, i8p, f32p, i32p]
         L.ogo_unpack_q3_k_scales.argtypes = [u8p, i32p]
+        L.ogo_dot_flat32.restype = C.c_float
+        L.ogo_dot_flat32.argtypes = [C.c_uint32, u8p, sz, i8p, f32p, i32p]
+        L.ogo_unpack_flat_block.restype = C.c_float
+        L.ogo_unpack_flat_block.argtypes = [C.c_uint32, u8p, i8p]
         L.ogo_block_sums_q8_0.argtypes = [u8p, sz, i8p, i32p]
         for name in ("ogo_supports", "ogo_supports_k", "ogo_supports_k_row", "ogo_supports_flat"):
             getattr(L, name).argtypes = [C.c_uint32, sz]
@@ -213,11 +218,21 @@ def dot_row(ggml_type: int, row, act) -> np.float32:
     L = lib()
     if ggml_type == Q8_0:
         return np.float32(L.ogo_dot_q8_0(_p(r), n, _p(q), _p(d)))
+    if ggml_type in (Q4_0, Q5_0, IQ4_NL):
+        return np.float32(L.ogo_dot_flat32(ggml_type, _p(r), n, _p(q), _p(d), None))
     if ggml_type == Q4_K:
         return np.float32(L.ogo_dot_q4_k(_p(r), n, _p(q), _p(d), _p(s)))
     if ggml_type == Q6_K:
         return np.float32(L.ogo_dot_q6_k(_p(r), n, _p(q), _p(d)))
     raise ValueError(ggml_type)
+
+
+def unpack_flat_block(ggml_type: int, block):
+    """One block of a symmetric per-32 type as (dw, int8[32]) (vecdot.rs:913-1039)."""
+    b = _u8(block)
+    w = np.zeros(32, np.int8)
+    dw = lib().ogo_unpack_flat_block(ggml_type, _p(b), _p(w))
+    return np.float32(dw), w
 
 
 def unpack_q3_k_scales(packed) -> np.ndarray:

@@ -65,7 +65,10 @@ int ogo_block_layout(uint32_t ggml_type, size_t *block_bytes, size_t *block_elem
   switch (ggml_type) {
     case OGO_TYPE_F32: bb = 4; be = 1; break;
     case OGO_TYPE_F16: bb = 2; be = 1; break;
+    case OGO_TYPE_Q4_0: bb = 2 + 16; be = 32; break;
+    case OGO_TYPE_Q5_0: bb = 2 + 4 + 16; be = 32; break;
     case OGO_TYPE_Q8_0: bb = 2 + 32; be = 32; break;
+    case OGO_TYPE_IQ4_NL: bb = 2 + 16; be = 32; break;
     case OGO_TYPE_Q3_K: bb = 32 + 64 + 12 + 2; be = 256; break;
     case OGO_TYPE_Q4_K: bb = 2 + 2 + 12 + 128; be = 256; break;
     case OGO_TYPE_Q5_K: bb = 2 + 2 + 12 + 32 + 128; be = 256; break;
@@ -146,6 +149,54 @@ static void dequantize_q5_k(const uint8_t *bytes, size_t n, float *out) {
   }
 }
 
+/* iq_grids.rs:5941-5943 */
+static const int8_t KVALUES_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10,
+                                          1,    13,   25,  38,  53,  69,  89,  113};
+
+/* unpack_block_q5_bits / unpack_block_q4_0 / _q5_0 / _iq4_nl (vecdot.rs:913-1039): elements 0..16
+ * from the low nibbles, 16..32 from the high nibbles; Q5_0 adds bit j (resp. j + 16) of qh as a
+ * fifth bit; Q4_0 and Q5_0 subtract their zero point (8, 16), IQ4_NL looks its nibble up. */
+float ogo_unpack_flat_block(uint32_t ggml_type, const uint8_t *block, int8_t *w) {
+  float dw = read_f16(block, 0);
+  if (ggml_type == OGO_TYPE_Q8_0) {
+    memcpy(w, block + 2, 32);
+  } else if (ggml_type == OGO_TYPE_IQ4_NL) {
+    const uint8_t *qs = block + 2;
+    for (int j = 0; j < 16; j++) {
+      w[j] = KVALUES_IQ4NL[qs[j] & 0x0F];
+      w[j + 16] = KVALUES_IQ4NL[qs[j] >> 4];
+    }
+  } else {
+    uint32_t qh = 0;
+    const uint8_t *qs = block + 2;
+    int bias = 8;
+    if (ggml_type == OGO_TYPE_Q5_0) {
+      qh = (uint32_t)block[2] | ((uint32_t)block[3] << 8) | ((uint32_t)block[4] << 16) | ((uint32_t)block[5] << 24);
+      qs = block + 6;
+      bias = 16;
+    }
+    for (int j = 0; j < 16; j++) {
+      uint32_t hi_lo = ((qh >> j) << 4) & 0x10;
+      uint32_t hi_hi = (qh >> (j + 12)) & 0x10;
+      w[j] = (int8_t)((int32_t)((uint32_t)(qs[j] & 0x0F) | hi_lo) - bias);
+      w[16 + j] = (int8_t)((int32_t)((uint32_t)(qs[j] >> 4) | hi_hi) - bias);
+    }
+  }
+  return dw;
+}
+
+/* quant.rs:537-554 (Q4_0), 560-580 (Q5_0), 1320-1337 (IQ4_NL).  Q4_0 and Q5_0 multiply
+ * (float)q * d, IQ4_NL d * (float)level: the products commute, the values are the same. */
+static void dequantize_flat32(uint32_t ggml_type, const uint8_t *bytes, size_t n, float *out) {
+  size_t bb, be;
+  ogo_block_layout(ggml_type, &bb, &be);
+  int8_t w[32];
+  for (size_t b = 0; b < n / 32; b++) {
+    float d = ogo_unpack_flat_block(ggml_type, bytes + b * bb, w);
+    for (int j = 0; j < 32; j++) out[b * 32 + (size_t)j] = (float)w[j] * d;
+  }
+}
+
 /* quant.rs:883-897 */
 void ogo_unpack_q3_k_scales(const uint8_t *packed, int32_t *scales) {
   for (int i = 0; i < 16; i++) {
@@ -220,6 +271,9 @@ int ogo_dequantize(uint32_t ggml_type, const uint8_t *bytes, size_t element_coun
   if (element_count % be != 0) return -2;
   switch (ggml_type) {
     case OGO_TYPE_Q8_0: dequantize_q8_0(bytes, element_count, out); return 0;
+    case OGO_TYPE_Q4_0:
+    case OGO_TYPE_Q5_0:
+    case OGO_TYPE_IQ4_NL: dequantize_flat32(ggml_type, bytes, element_count, out); return 0;
     case OGO_TYPE_Q3_K: dequantize_q3_k(bytes, element_count, out); return 0;
     case OGO_TYPE_Q4_K: dequantize_q4_k(bytes, element_count, out); return 0;
     case OGO_TYPE_Q5_K: dequantize_q5_k(bytes, element_count, out); return 0;
@@ -593,6 +647,10 @@ int32_t ogo_dot32(const int8_t *w, const int8_t *x) { return DISPATCH(dot32, w, 
 float ogo_dot_q8_0(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d) {
   return DISPATCH(dot_q8_0, row, in_dim, q, d, NULL);
 }
+float ogo_dot_flat32(uint32_t ggml_type, const uint8_t *row, size_t in_dim, const int8_t *q,
+                     const float *d, int32_t *isum_out) {
+  return DISPATCH(dot_flat32, ggml_type, row, in_dim, q, d, isum_out);
+}
 void ogo_block_sums_q8_0(const uint8_t *row, size_t in_dim, const int8_t *q, int32_t *isum_out) {
   float *d = (float *)calloc(in_dim / 32, sizeof(float));
   (void)DISPATCH(dot_q8_0, row, in_dim, q, d, isum_out);
@@ -626,7 +684,7 @@ float ogo_dot_k_row_q3_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
 
 /* vecdot.rs:274-283, restricted to the types on the path */
 int ogo_supports(uint32_t t, size_t in_dim) {
-  if (t == OGO_TYPE_Q8_0) return in_dim % 32 == 0;
+  if (t == OGO_TYPE_Q8_0 || t == OGO_TYPE_Q5_0 || t == OGO_TYPE_Q4_0 || t == OGO_TYPE_IQ4_NL) return in_dim % 32 == 0;
   if (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) return in_dim % 256 == 0;
   return 0;
 }
@@ -639,7 +697,9 @@ int ogo_supports_k_row(uint32_t t, size_t in_dim) {
   return (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
 }
 /* vecdot.rs:2456-2461 */
-int ogo_supports_flat(uint32_t t, size_t in_dim) { return t == OGO_TYPE_Q8_0 && in_dim % 32 == 0; }
+int ogo_supports_flat(uint32_t t, size_t in_dim) {
+  return (t == OGO_TYPE_Q8_0 || t == OGO_TYPE_Q5_0 || t == OGO_TYPE_Q4_0 || t == OGO_TYPE_IQ4_NL) && in_dim % 32 == 0;
+}
 
 /* ------------------------------------------------------------------ CpuBackend */
 
@@ -742,9 +802,9 @@ int ogo_k_gemm_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_
   return k_gemm_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, 1);
 }
 
-/* backend/cpu.rs:209-245 matmul_flat_gemm_into (Q8_0): unpack_q8_0 (vecdot.rs:1246-1255) then
- * dot_flat_pair */
-static int flat_gemm_t(const uint8_t *raw, size_t row_bytes, size_t in_dim, size_t out_dim,
+/* backend/cpu.rs:209-245 matmul_flat_gemm_into: unpack_q8_0 / _q5_0 / _q4_0 / _iq4_nl
+ * (vecdot.rs:1246-1296, 1351-1362) then dot_flat_pair */
+static int flat_gemm_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t in_dim, size_t out_dim,
                        const float *x, size_t n_tokens, float *yt, int threads) {
   ogo_actq8flat a;
   a.n_tokens = n_tokens;
@@ -756,6 +816,8 @@ static int flat_gemm_t(const uint8_t *raw, size_t row_bytes, size_t in_dim, size
   ogo_act_q8flat_quantize(x, in_dim, n_tokens, a.q, a.d);
   size_t n_pair = (out_dim + 1) / 2;
   size_t nb = in_dim / 32;
+  size_t bb, be;
+  ogo_block_layout(ggml_type, &bb, &be);
 #pragma omp parallel num_threads(threads)
   {
     int8_t *q0 = (int8_t *)malloc(in_dim), *q1 = (int8_t *)malloc(in_dim);
@@ -765,16 +827,10 @@ static int flat_gemm_t(const uint8_t *raw, size_t row_bytes, size_t in_dim, size
     for (size_t pair = 0; pair < n_pair; pair++) {
       size_t o0 = pair * 2;
       const uint8_t *r0 = raw + o0 * row_bytes;
-      for (size_t b = 0; b < nb; b++) {
-        s0[b] = read_f16(r0 + b * 34, 0);
-        memcpy(q0 + b * 32, r0 + b * 34 + 2, 32);
-      }
+      for (size_t b = 0; b < nb; b++) s0[b] = ogo_unpack_flat_block(ggml_type, r0 + b * bb, q0 + b * 32);
       if (o0 + 1 < out_dim) {
         const uint8_t *r1 = raw + (o0 + 1) * row_bytes;
-        for (size_t b = 0; b < nb; b++) {
-          s1[b] = read_f16(r1 + b * 34, 0);
-          memcpy(q1 + b * 32, r1 + b * 34 + 2, 32);
-        }
+        for (size_t b = 0; b < nb; b++) s1[b] = ogo_unpack_flat_block(ggml_type, r1 + b * bb, q1 + b * 32);
         DISPATCH(dot_flat_pair, q0, s0, q1, s1, &a, yt + o0 * n_tokens, yt + (o0 + 1) * n_tokens);
       } else {
         DISPATCH(dot_flat_pair, q0, s0, q0, s0, &a, yt + o0 * n_tokens, scratch);
@@ -831,8 +887,10 @@ static int gemv_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size
         v = DISPATCH(dot_k_row_q6_k, row, in_dim, qt, dt, io);
       else if (ggml_type == OGO_TYPE_Q3_K)
         v = DISPATCH(dot_k_row_q3_k, row, in_dim, qt, dt, io);
-      else
+      else if (ggml_type == OGO_TYPE_Q8_0)
         v = DISPATCH(dot_q8_0, row, in_dim, qt, dt, io);
+      else
+        v = DISPATCH(dot_flat32, ggml_type, row, in_dim, qt, dt, io);
       yt[o * n_tokens + t] = v;
     }
   }
@@ -854,7 +912,7 @@ int ogo_matmul(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t 
   if (n_tokens > 1 && ogo_supports_k(ggml_type, in_dim))
     rc = k_gemm_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads);
   else if (n_tokens > 1 && ogo_supports_flat(ggml_type, in_dim))
-    rc = flat_gemm_t(raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads);
+    rc = flat_gemm_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads);
   else
     rc = gemv_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads, NULL, NULL);
   if (rc == 0) finish_into(y, yt, n_tokens, out_dim);

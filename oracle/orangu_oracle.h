@@ -46,11 +46,14 @@ extern "C" {
 /* ggml type ids, quant.rs:50-61 */
 #define OGO_TYPE_F32 0u
 #define OGO_TYPE_F16 1u
+#define OGO_TYPE_Q4_0 2u
+#define OGO_TYPE_Q5_0 6u
 #define OGO_TYPE_Q8_0 8u
 #define OGO_TYPE_Q3_K 11u
 #define OGO_TYPE_Q4_K 12u
 #define OGO_TYPE_Q5_K 13u
 #define OGO_TYPE_Q6_K 14u
+#define OGO_TYPE_IQ4_NL 20u
 
 #define OGO_ACT_BLOCK 32   /* vecdot.rs ACT_BLOCK */
 #define OGO_GROUP 16       /* vecdot.rs:63 */
@@ -105,6 +108,12 @@ float ogo_dot_k_row_q3_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
                          int32_t *isum_out);                                          /* :3273-3292 */
 /* quant.rs:883-897: the 16 six-bit scales of a Q3_K block, still biased by 32 */
 void ogo_unpack_q3_k_scales(const uint8_t *packed, int32_t *scales);
+/* the other symmetric per-32 types (Q5_0, Q4_0, IQ4_NL): dot_q5_0 / dot_q4_0 / dot_iq4_nl,
+ * vecdot.rs:2842-2883; isum_out (may be NULL) receives the per-32 integer sums */
+float ogo_dot_flat32(uint32_t ggml_type, const uint8_t *row, size_t in_dim, const int8_t *q,
+                     const float *d, int32_t *isum_out);
+/* one block of such a type as 32 int8 weights (unpack_block_*, vecdot.rs:913-1039); returns dw */
+float ogo_unpack_flat_block(uint32_t ggml_type, const uint8_t *block, int8_t *w);
 /* per-32 integer sums of a Q8_0 row (isum_out[in_dim/32]) */
 void ogo_block_sums_q8_0(const uint8_t *row, size_t in_dim, const int8_t *q, int32_t *isum_out);
 

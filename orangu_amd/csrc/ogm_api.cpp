@@ -96,9 +96,14 @@ static int ensure_host(ogm_ctx *ctx, DevBuf &b, size_t bytes) {
   return OGM_OK;
 }
 
+static uint32_t block_elems_of(uint32_t ggml_type) {
+  OgmLayout l;
+  return ogm_layout_for(ggml_type, &l) ? l.block_elems : 256u;
+}
+
 static int act_mode_for(uint32_t ggml_type) {
-  // backend/cpu.rs:100-116: K-quants take the per-256 quantizer, Q8_0 the per-32 one
-  return ggml_type == OGM_Q8_0 ? OGM_ACT_PER_32 : OGM_ACT_PER_256;
+  // backend/cpu.rs:100-116: the K-quants take quantize_act_k_row (per 256), the per-32 types quantize_act
+  return block_elems_of(ggml_type) == 32 ? OGM_ACT_PER_32 : OGM_ACT_PER_256;
 }
 
 static int ensure_act(ogm_ctx *ctx, uint32_t in_dim, uint32_t n_tokens) {
@@ -407,7 +412,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   const uint32_t wg_waves = (uint32_t)ctx->tune_wg_waves;
   const uint32_t chunk = ogm_gemv_max_tokens(w0->ggml_type, w0->in_dim, gemm_order);
   if (chunk == 0) return fail(ctx, OGM_ERR_UNSUPPORTED, "no kernel for this type");
-  const uint32_t blocks_per_row = w0->in_dim / (w0->ggml_type == OGM_Q8_0 ? 32 : 256);
+  const uint32_t blocks_per_row = w0->in_dim / block_elems_of(w0->ggml_type);
   for (size_t g0 = 0; g0 < n_tg; g0 += OGM_GEMV_MAX_MATS) {
     const size_t ng = n_tg - g0 < OGM_GEMV_MAX_MATS ? n_tg - g0 : OGM_GEMV_MAX_MATS;
     for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
@@ -681,7 +686,7 @@ extern "C" int ogm_dump_block_sums(ogm_ctx *ctx, const ogm_weight *w, const floa
   if (n_tokens == 0) return OGM_OK;
   std::lock_guard<std::mutex> lock(ctx->mu);
   HIPCHK(ctx, hipSetDevice(ctx->device));
-  const size_t blocks = (size_t)w->in_dim / (w->ggml_type == OGM_Q8_0 ? 32 : 256);
+  const size_t blocks = (size_t)w->in_dim / block_elems_of(w->ggml_type);
   const size_t nb = (size_t)n_tokens * w->out_dim * blocks * 4;
   const size_t xb = (size_t)n_tokens * w->in_dim * 4, yb = (size_t)n_tokens * w->out_dim * 4;
   const bool want_min = imin && (w->ggml_type == OGM_Q4_K || w->ggml_type == OGM_Q5_K);

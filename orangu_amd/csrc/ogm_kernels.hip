@@ -531,6 +531,78 @@ struct FmtQ80 {
   }
 };
 
+// The other symmetric per-32 types (vecdot.rs:2842-2883): one 16-byte piece of nibbles per block,
+// elements 0..16 from the low nibbles, 16..32 from the high nibbles, total += dw * act.d[b] * isum
+// like Q8_0.  KIND 0: Q4_0 (nibble - 8); 1: Q5_0 (nibble | fifth bit from qh, - 16); 2: IQ4_NL
+// (nibble indexes the sixteen levels of iq_grids.rs:5941-5943).
+template <int KIND>
+struct FmtNib32 {
+  static constexpr uint32_t TYPE = KIND == 0 ? OGM_Q4_0 : (KIND == 1 ? OGM_Q5_0 : OGM_IQ4_NL);
+  static constexpr int TAIL = KIND == 1 ? 6 : 2;
+  static constexpr int PIECES = 1, TILE_BYTES = 64 * (16 + TAIL), ELEMS = 32;
+  static constexpr int XPIECES = 2;
+  static constexpr int AUX16 = 0;
+  static constexpr int ACT_GROUP = 32;
+  static constexpr bool HAS_MIN = false;
+  static constexpr int MAX_THREADS = 1024;
+  static constexpr bool HAS_UNPACK = false;
+  struct Regs {
+    uint4 p[PIECES];
+    uint32_t d16, qh;
+  };
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
+    const uint8_t *tb = wt + tile * TILE_BYTES;
+    r.p[0] = *(const uint4 *)(tb + lane * 16u);
+    const uint16_t *t = (const uint16_t *)(tb + 1024 + lane * TAIL);   // d, then qh (two-byte aligned)
+    r.d16 = t[0];
+    r.qh = KIND == 1 ? ((uint32_t)t[1] | ((uint32_t)t[2] << 16)) : 0u;
+  }
+  // Four nibbles (one per byte, 0..15), with four fifth bits `h4` for Q5_0, as signed weights.
+  __device__ static __forceinline__ uint32_t weights(uint32_t n, uint32_t h4) {
+    if (KIND == 2) {
+      // sixteen-entry byte table: two eight-entry v_perm lookups, chosen by bit 3 of the index
+      const uint32_t sel = n & 0x07070707u;
+      const uint32_t lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, sel);   // levels 0..7
+      const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, sel);   // levels 8..15
+      const uint32_t pick = ((n >> 3) & 0x01010101u) * 0xFFu;
+      return (lo & ~pick) | (hi & pick);
+    }
+    // v - bias per byte without borrows between bytes: set bit 7, subtract, flip bit 7 back
+    const uint32_t v = KIND == 1 ? (n | (((h4 * 0x00204081u) & 0x01010101u) << 4)) : n;
+    const uint32_t bias = KIND == 1 ? 0x10101010u : 0x08080808u;
+    return ((v | 0x80808080u) - bias) ^ 0x80808080u;
+  }
+  template <int UPR>
+  __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,
+                                              int &isum, int &imin) {
+    const uint4 x0 = a.xq[col], x1 = a.xq[(UPR ? (uint32_t)UPR : a.upr) + col];
+    const uint32_t m4 = 0x0F0F0F0Fu;
+    const uint32_t qw[4] = {r.p[0].x, r.p[0].y, r.p[0].z, r.p[0].w};
+    const uint32_t xl[4] = {x0.x, x0.y, x0.z, x0.w}, xh[4] = {x1.x, x1.y, x1.z, x1.w};
+    int acc = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      // bytes 4k .. 4k+3 of qs: elements 4k.. (bits 4k.. of qh) and 16+4k.. (bits 16+4k..)
+      acc = dot4(weights(qw[k] & m4, (r.qh >> (4 * k)) & 0xFu), xl[k], acc);
+      acc = dot4(weights((qw[k] >> 4) & m4, (r.qh >> (16 + 4 * k)) & 0xFu), xh[k], acc);
+    }
+    isum = acc;
+    imin = 0;
+  }
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int) {
+    return f16_bits_to_f32(r.d16) * ad * (float)isum;
+  }
+  // flat GEMM: acc += d * s * dot32 (vecdot.rs:2622-2623)
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int,
+                                                   float &tmin, float &tdot) {
+    tmin = 0.0f;
+    tdot = ad * f16_bits_to_f32(r.d16) * (float)isum;
+  }
+};
+typedef FmtNib32<0> FmtQ40;
+typedef FmtNib32<1> FmtQ50;
+typedef FmtNib32<2> FmtIQ4NL;
+
 // ------------------------------------------------------------------------------------------
 // GEMV kernel
 //
@@ -855,6 +927,12 @@ uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order
       return gemm_order ? max_tokens_t<FmtQ6K, true>(in_dim) : max_tokens_t<FmtQ6K, false>(in_dim);
     case OGM_Q8_0:
       return gemm_order ? max_tokens_t<FmtQ80, true>(in_dim) : max_tokens_t<FmtQ80, false>(in_dim);
+    case OGM_Q4_0:
+      return gemm_order ? max_tokens_t<FmtQ40, true>(in_dim) : max_tokens_t<FmtQ40, false>(in_dim);
+    case OGM_Q5_0:
+      return gemm_order ? max_tokens_t<FmtQ50, true>(in_dim) : max_tokens_t<FmtQ50, false>(in_dim);
+    case OGM_IQ4_NL:
+      return gemm_order ? max_tokens_t<FmtIQ4NL, true>(in_dim) : max_tokens_t<FmtIQ4NL, false>(in_dim);
     default:
       return 0;
   }
@@ -959,6 +1037,15 @@ hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char 
     case OGM_Q8_0:
       if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ80,gemm>" : "ogm_gemv_kernel<FmtQ80,gemv>";
       return a.gemm_order ? launch_t<FmtQ80, true>(a, stream) : launch_t<FmtQ80, false>(a, stream);
+    case OGM_Q4_0:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ40,gemm>" : "ogm_gemv_kernel<FmtQ40,gemv>";
+      return a.gemm_order ? launch_t<FmtQ40, true>(a, stream) : launch_t<FmtQ40, false>(a, stream);
+    case OGM_Q5_0:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ50,gemm>" : "ogm_gemv_kernel<FmtQ50,gemv>";
+      return a.gemm_order ? launch_t<FmtQ50, true>(a, stream) : launch_t<FmtQ50, false>(a, stream);
+    case OGM_IQ4_NL:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtIQ4NL,gemm>" : "ogm_gemv_kernel<FmtIQ4NL,gemv>";
+      return a.gemm_order ? launch_t<FmtIQ4NL, true>(a, stream) : launch_t<FmtIQ4NL, false>(a, stream);
     default:
       return hipErrorInvalidValue;
   }

@@ -1,7 +1,7 @@
 // Tile-planar weight layout shared by the host repacker and the device kernels.
 //
 // A matrix is out_dim rows of `upr` blocks ("units"; one unit is one GGUF block: Q8_0 34 B / 32
-// weights, Q3_K 110 B / 256, Q4_K 144 B / 256, Q5_K 176 B / 256, Q6_K 210 B / 256;
+// weights, Q4_0 and IQ4_NL 18 B / 32, Q5_0 22 B / 32, Q3_K 110 B / 256, Q4_K 144 B / 256, Q5_K 176 B / 256, Q6_K 210 B / 256;
 // engine/quant.rs:638-871).  A *tile* holds 64
 // units: R consecutive rows x C consecutive blocks, with C = 4 when a row has a multiple of four
 // blocks (else 2, else 1) and R = 64 / C.  Tiles are ordered [row block][column tile]; inside a
@@ -19,6 +19,8 @@
 //
 //   type   pieces                                   tail
 //   Q8_0   2  (qs[0..32))                           d      (2 B)
+//   Q4_0   1  (qs[0..16))                           d      (2 B)      (IQ4_NL the same)
+//   Q5_0   1  (qs[0..16))                           d, qh  (6 B)
 //   Q3_K   7  (hmask[0..32) | qs[0..64) | scales,d + 2 bytes of padding)   -
 //   Q4_K   9  (d,dmin,scales | qs[0..128))          -
 //   Q5_K   11 (d,dmin,scales | qh[0..32) | qs)      -
@@ -27,11 +29,14 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#define OGM_Q4_0 2u
+#define OGM_Q5_0 6u
 #define OGM_Q8_0 8u
 #define OGM_Q3_K 11u
 #define OGM_Q4_K 12u
 #define OGM_Q5_K 13u
 #define OGM_Q6_K 14u
+#define OGM_IQ4_NL 20u
 
 #define OGM_TILE_UNITS 64u
 
@@ -39,7 +44,7 @@ struct OgmLayout {
   uint32_t block_bytes;   // raw bytes per unit
   uint32_t block_elems;   // weights per unit
   uint32_t pieces;        // 16-byte pieces per unit
-  uint32_t tail_bytes;    // bytes after the pieces (0 or 2)
+  uint32_t tail_bytes;    // bytes kept after all pieces (0, 2 or 6), lane after lane
   uint32_t piece_off;     // raw offset of piece 0 inside the block
   uint32_t tail_off;      // raw offset of the tail inside the block
   uint32_t tile_bytes;    // 64 * block_bytes
@@ -62,6 +67,13 @@ struct OgmTiling {
 
 OGM_HD inline bool ogm_layout_for(uint32_t ggml_type, OgmLayout *l) {
   switch (ggml_type) {
+    case OGM_Q4_0:    // d:f16 | qs:u8[16]
+    case OGM_IQ4_NL:  // d:f16 | qs:u8[16] (codebook indices)
+      *l = OgmLayout{18, 32, 1, 2, 2, 0, 64 * 18};
+      return true;
+    case OGM_Q5_0:  // d:f16 | qh:u32 | qs:u8[16]
+      *l = OgmLayout{22, 32, 1, 6, 6, 0, 64 * 22};
+      return true;
     case OGM_Q8_0:  // d:f16 | qs:i8[32]
       *l = OgmLayout{34, 32, 2, 2, 2, 0, 64 * 34};
       return true;

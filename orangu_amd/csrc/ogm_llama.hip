@@ -644,7 +644,8 @@ hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStrea
 
 // ------------------------------------------------------------------------------------------
 // one row of a quantized matrix as f32: the embedding lookup (LlamaModel::run_layers,
-// llama.rs:609-614, over dequantize_q8_0 / _q3_k / _q4_k / _q5_k / _q6_k, quant.rs:639-649, 666-787, 841-871),
+// llama.rs:609-614, over dequantize_q8_0 / _q4_0 / _q5_0 / _iq4_nl / _q3_k / _q4_k / _q5_k / _q6_k,
+// quant.rs:537-580, 639-649, 666-787, 841-871, 1320-1337),
 // reading the tile-planar device copy.  One thread per element; the f32 expressions are the
 // reference's, so the values are bit-identical (built without FMA contraction).
 
@@ -676,6 +677,21 @@ __global__ __launch_bounds__(256) void ogm_dequant_row_kernel(const uint8_t *__r
   if (ggml_type == OGM_Q8_0) {
     const float d = dq_f16(tb + l.pieces * 1024u + lane * 2u);
     v = (float)(int8_t)piece_byte(j) * d;
+  } else if (ggml_type == OGM_Q4_0 || ggml_type == OGM_Q5_0 || ggml_type == OGM_IQ4_NL) {
+    // one piece of nibbles (elements 0..16 low, 16..32 high); the tail holds d, and qh for Q5_0
+    const uint8_t *tail = tb + 1024u + lane * l.tail_bytes;
+    const float d = dq_f16(tail);
+    const uint32_t byte = piece_byte(j & 15u);
+    const uint32_t nib = j < 16 ? (byte & 0xFu) : (byte >> 4);
+    if (ggml_type == OGM_IQ4_NL) {
+      const int8_t levels[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+      v = d * (float)levels[nib];
+    } else if (ggml_type == OGM_Q4_0) {
+      v = (float)((int)nib - 8) * d;
+    } else {
+      const uint32_t qh = tail[2] | (tail[3] << 8) | (tail[4] << 16) | ((uint32_t)tail[5] << 24);
+      v = (float)((int)(nib | (((qh >> j) & 1u) << 4)) - 16) * d;
+    }
   } else if (ggml_type == OGM_Q4_K) {
     const uint8_t *hd = tb + lane * 16u;   // piece 0: d, dmin, scales
     const float d = dq_f16(hd), dmin = dq_f16(hd + 2);

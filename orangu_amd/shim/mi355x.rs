@@ -193,7 +193,7 @@ impl Backend for Mi355xBackend {
         outs
     }
 
-    /// Q8_0, Q3_K, Q4_K, Q5_K, Q6_K; anything else is a start-up error through `unsupported_tensor_types`
+    /// Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K; anything else is a start-up error through `unsupported_tensor_types`
     /// (mod.rs:522-533).
     fn supports_type(&self, ggml_type: u32) -> bool {
         unsafe { ogm_supports_type(ggml_type) != 0 }

@@ -8,9 +8,12 @@ from __future__ import annotations
 
 import numpy as np
 
-Q8_0, Q3_K, Q4_K, Q5_K, Q6_K = 8, 11, 12, 13, 14
-BLOCK = {Q8_0: (34, 32), Q3_K: (110, 256), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
-TYPE_NAME = {Q8_0: "q8_0", Q3_K: "q3_k", Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k"}
+Q4_0, Q5_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL = 2, 6, 8, 11, 12, 13, 14, 20
+FLAT32 = (Q8_0, Q5_0, Q4_0, IQ4_NL)   # symmetric, one f16 scale per 32 (vecdot.rs:2456-2461)
+BLOCK = {Q4_0: (18, 32), Q5_0: (22, 32), Q8_0: (34, 32), Q3_K: (110, 256), Q4_K: (144, 256), Q5_K: (176, 256),
+         Q6_K: (210, 256), IQ4_NL: (18, 32)}
+TYPE_NAME = {Q4_0: "q4_0", Q5_0: "q5_0", Q8_0: "q8_0", Q3_K: "q3_k", Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k",
+             IQ4_NL: "iq4_nl"}
 
 
 def row_bytes(ggml_type: int, in_dim: int) -> int:
@@ -55,7 +58,7 @@ def pin_scales(raw: np.ndarray, ggml_type: int) -> np.ndarray:
     (d = 0x3000 = 0.125, dmin = 0x2c00 = 0.0625)."""
     bb, _ = BLOCK[ggml_type]
     blocks = raw.reshape(-1, bb)
-    if ggml_type == Q8_0:
+    if ggml_type in FLAT32:
         blocks[:, 0:2] = (0x00, 0x30)
     elif ggml_type in (Q4_K, Q5_K):   # Q5_K shares Q4_K's leading d / dmin pair (vecdot.rs:3467)
         blocks[:, 0:2] = (0x00, 0x30)
@@ -135,6 +138,9 @@ def synth_weights(ggml_type: int, in_dim: int, out_dim: int, seed: int) -> np.nd
         q = rng.integers(-127, 128, size=(nblk, 32), dtype=np.int8)
         raw[:, 2:] = q.view(np.uint8)
         d = (np.abs(rng.normal(0, 0.02, nblk)) / 127).astype(np.float16)
+        raw[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+    elif ggml_type in (Q4_0, Q5_0, IQ4_NL):
+        d = (np.abs(rng.normal(0, 0.02, nblk)) / (127 if ggml_type == IQ4_NL else 16)).astype(np.float16)
         raw[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
     elif ggml_type in (Q4_K, Q5_K):
         d = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)

@@ -7,7 +7,7 @@ import re
 import numpy as np
 import pytest
 
-from helpers import BLOCK, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, row_bytes
+from helpers import BLOCK, IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0, row_bytes
 from orangu_amd import capi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -33,7 +33,9 @@ def test_supports_predicates_follow_vecdot(lib):
     assert lib.ogm_supports_type(Q8_0) and lib.ogm_supports_type(Q4_K) and lib.ogm_supports_type(Q6_K)
     assert lib.ogm_supports_type(13) and lib.ogm_supports(13, 256) and not lib.ogm_supports(13, 128)   # Q5_K
     assert lib.ogm_supports_type(11) and lib.ogm_supports(11, 512) and not lib.ogm_supports(11, 896)   # Q3_K
-    assert not lib.ogm_supports_type(0) and not lib.ogm_supports_type(10)
+    for t in (2, 6, 20):   # Q4_0, Q5_0, IQ4_NL
+        assert lib.ogm_supports_type(t) and lib.ogm_supports(t, 896) and not lib.ogm_supports(t, 24)
+    assert not lib.ogm_supports_type(0) and not lib.ogm_supports_type(10) and not lib.ogm_supports_type(3)
     assert lib.ogm_supports(Q8_0, 96) and not lib.ogm_supports(Q8_0, 100)
     assert lib.ogm_supports(Q4_K, 512) and not lib.ogm_supports(Q4_K, 896)
     assert lib.ogm_supports(Q6_K, 256) and not lib.ogm_supports(Q6_K, 0)
@@ -41,7 +43,7 @@ def test_supports_predicates_follow_vecdot(lib):
         a, b = C.c_uint32(), C.c_uint32()
         assert lib.ogm_block_layout(t, C.byref(a), C.byref(b)) == 0
         assert (a.value, b.value) == (bb, be)
-    assert lib.ogm_block_layout(2, None, None) == -2
+    assert lib.ogm_block_layout(3, None, None) == -2   # Q4_1: not built
 
 
 def tiling(upr, out_dim):
@@ -52,10 +54,10 @@ def tiling(upr, out_dim):
 
 
 # bytes a unit takes in the tile-planar form: the raw block, except Q3_K whose last piece is padded
-TILE_UNIT = {Q8_0: 34, Q3_K: 112, Q4_K: 144, Q5_K: 176, Q6_K: 210}
+TILE_UNIT = {Q4_0: 18, Q5_0: 22, Q8_0: 34, IQ4_NL: 18, Q3_K: 112, Q4_K: 144, Q5_K: 176, Q6_K: 210}
 
 
-@pytest.mark.parametrize("ggml_type", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_blocks,out_dim", [(1, 1), (3, 11), (16, 64), (7, 130), (6, 33), (8, 70)])
 def test_repack_is_a_bijection_on_the_raw_bytes(lib, ggml_type, in_blocks, out_dim):
     bb, be = BLOCK[ggml_type]
@@ -78,7 +80,8 @@ def test_repack_is_a_bijection_on_the_raw_bytes(lib, ggml_type, in_blocks, out_d
 
 @pytest.mark.parametrize("t,npieces,piece_off,tail_off,tail", [(Q4_K, 9, 0, 0, 0), (Q6_K, 13, 0, 208, 2),
                                                               (Q8_0, 2, 2, 0, 2), (Q5_K, 11, 0, 0, 0),
-                                                              (Q3_K, 7, 0, 0, 0)])
+                                                              (Q3_K, 7, 0, 0, 0), (Q4_0, 1, 2, 0, 2),
+                                                              (Q5_0, 1, 6, 0, 6), (IQ4_NL, 1, 2, 0, 2)])
 @pytest.mark.parametrize("in_blocks,out_dim", [(8, 70), (6, 40), (3, 65)])
 def test_repack_places_pieces_in_planes(lib, t, npieces, piece_off, tail_off, tail, in_blocks, out_dim):
     """Unit (row o, block b): tile (o / R) * nct + b / C, lane (b % C) * R + o % R; piece p at
@@ -111,7 +114,7 @@ def test_repack_places_pieces_in_planes(lib, t, npieces, piece_off, tail_off, ta
 
 def test_repack_rejects_bad_shapes(lib):
     buf = np.zeros(4096, np.uint8)
-    assert lib.ogm_repack_host(2, buf.ctypes.data, 18, 32, 1, buf.ctypes.data) == -2  # Q4_0: no kernel
+    assert lib.ogm_repack_host(3, buf.ctypes.data, 20, 32, 1, buf.ctypes.data) == -2  # Q4_1: no kernel
     assert lib.ogm_repack_host(Q4_K, buf.ctypes.data, 144, 128, 1, buf.ctypes.data) == -2  # in_dim % 256
     assert lib.ogm_repack_host(Q4_K, buf.ctypes.data, 100, 256, 1, buf.ctypes.data) == -1  # row_bytes
     assert lib.ogm_repack_host(Q4_K, None, 144, 256, 1, buf.ctypes.data) == -1

@@ -8,7 +8,7 @@ import sys
 import numpy as np
 import pytest
 
-from helpers import Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, synth_weights
+from helpers import IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0, synth_weights
 from oracle import llama_ref as R
 
 pytestmark = pytest.mark.gpu
@@ -81,7 +81,7 @@ def step_both(ref, dev, x, pos, what):
 
 
 @pytest.mark.parametrize("types", [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q4_K, Q4_K, Q4_K, Q4_K),
-                                   (Q5_K, Q5_K, Q6_K, Q5_K)])
+                                   (Q5_K, Q5_K, Q6_K, Q5_K), (Q4_0, Q5_0, IQ4_NL, Q8_0)])
 def test_decode_steps_from_an_empty_cache(be, types):
     """Positions 0..5 one after the other: RMSNorm, q/k/v, RoPE, cache append, attention over the
     growing cache, wo, residual, SwiGLU FFN, output norm and vocabulary projection."""
@@ -208,6 +208,7 @@ def test_matrices_uploaded_from_a_gguf_file_multiply_like_direct_uploads(be, tmp
     (Q6_K, 256, 1), (Q6_K, 768, 65), (Q6_K, 4096, 129),
     (Q5_K, 256, 2), (Q5_K, 1280, 70), (Q5_K, 4096, 33),
     (Q3_K, 256, 2), (Q3_K, 1280, 70), (Q3_K, 4096, 33),
+    (Q4_0, 64, 5), (Q4_0, 4096, 70), (Q5_0, 96, 66), (Q5_0, 4096, 33), (IQ4_NL, 64, 5), (IQ4_NL, 896, 130),
 ])
 def test_dequant_rows_bits(be, t, in_dim, out_dim):
     """Rows of the device copy equal dequantize_q8_0 / _q4_k / _q6_k (quant.rs:639-787) bit for bit."""
@@ -225,7 +226,7 @@ def test_dequant_rows_bits(be, t, in_dim, out_dim):
         be.dequant_rows(w, out_dim, 1)
 
 
-@pytest.mark.parametrize("embd_t", [Q3_K, Q4_K, Q5_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("embd_t", [Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, Q4_0, Q5_0, IQ4_NL])
 def test_generate_matches_stepwise(be, embd_t):
     """Greedy generation on the device = the oracle's loop: embedding row of the token
     (llama.rs:609-614), decode step, last-of-equal argmax (sampling.rs:336-343)."""
@@ -236,19 +237,24 @@ def test_generate_matches_stepwise(be, embd_t):
               types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=max_ctx, seed=11)
     ref, dev, _ = build(be, **kw)
     _, dev2, _ = build(be, **kw)
-    embd_raw = synth_weights(embd_t, n_embd, n_vocab, seed=4242 + embd_t)
-    table = oracle.dequantize(embd_t, embd_raw, n_embd * n_vocab).reshape(n_vocab, n_embd)
-    embd = QuantMatrix(embd_raw, embd_t, n_embd, n_vocab)
     first, steps = 17, 6
     try:
-        tok, want, logits, sure = first, [], None, True
-        for pos in range(steps):
-            logits, _ = R.decode_step(ref, table[tok], pos)
-            top = np.sort(logits)[-2:]
-            sure = sure and top[1] - top[0] > TOL * np.abs(logits).max()
-            tok = R.argmax(logits)
-            want.append(tok)
-        assert sure, "pick another seed: the oracle's two best logits are within the tolerance"
+        # the first embedding seed whose greedy path is decided by more than the tolerance at every step
+        for embd_seed in range(4242 + embd_t, 4242 + embd_t + 400, 50):
+            embd_raw = synth_weights(embd_t, n_embd, n_vocab, seed=embd_seed)
+            table = oracle.dequantize(embd_t, embd_raw, n_embd * n_vocab).reshape(n_vocab, n_embd)
+            ref.reset()
+            tok, want, logits, sure = first, [], None, True
+            for pos in range(steps):
+                logits, _ = R.decode_step(ref, table[tok], pos)
+                top = np.sort(logits)[-2:]
+                sure = sure and top[1] - top[0] > TOL * np.abs(logits).max()
+                tok = R.argmax(logits)
+                want.append(tok)
+            if sure:
+                break
+        embd = QuantMatrix(embd_raw, embd_t, n_embd, n_vocab)
+        assert sure, "no seed found: the oracle's two best logits are within the tolerance"
         got, got_logits = dev.generate(embd, first, 0, steps, want_logits=True)
         say("generated", got.tolist(), "want", want)
         assert got.tolist() == want

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (BLOCK, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, NextByte, activations, activations_t, cpu_rs_weights,
+from helpers import (BLOCK, FLAT32, IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0, NextByte, activations, activations_t, cpu_rs_weights,
                      fixture_row, k_fixture, row_bytes, synth_weights, synth_x)
 from test_oracle_quantize import adversarial_blocks
 
@@ -67,7 +67,7 @@ def test_f16_scale_conversion_matches_quant_rs_for_all_inputs(be):
     assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K])
 def test_upload_download_round_trip(be, t):
     """unrepack(repack(W)) == W through the device."""
     bb, bel = BLOCK[t]
@@ -117,6 +117,7 @@ def test_quantizer_ties_round_away_from_zero(be):
     (Q3_K, 256, 5, 1), (Q3_K, 2048, 37, 3), (Q3_K, 5632, 9, 2),
     (Q6_K, 256, 5, 1), (Q6_K, 2048, 37, 3), (Q6_K, 4864, 9, 2),
     (Q8_0, 96, 11, 1), (Q8_0, 896, 19, 3), (Q8_0, 4864, 7, 1),
+    (Q5_0, 96, 11, 1), (Q5_0, 896, 19, 3), (Q4_0, 32, 5, 2), (Q4_0, 4864, 7, 1), (IQ4_NL, 896, 19, 3), (IQ4_NL, 4864, 7, 2),
 ])
 def test_block_integer_sums_bit_exact(be, t, in_dim, out_dim, T):
     raw = np.concatenate([fixture_row(t, in_dim, 100 + o) for o in range(out_dim)])
@@ -133,7 +134,7 @@ def test_block_integer_sums_bit_exact(be, t, in_dim, out_dim, T):
 
 CHECK = [(Q8_0, 896), (Q8_0, 4864), (Q4_K, 256), (Q4_K, 4864), (Q6_K, 256), (Q6_K, 4864),
          (Q4_K, 2048), (Q6_K, 5632), (Q5_K, 256), (Q5_K, 3072), (Q5_K, 4864), (Q3_K, 256), (Q3_K, 2048),
-         (Q3_K, 5632)]
+         (Q3_K, 5632), (Q5_0, 896), (Q5_0, 4864), (Q4_0, 32), (Q4_0, 896), (Q4_0, 4864), (IQ4_NL, 896), (IQ4_NL, 4864)]
 
 
 @pytest.mark.parametrize("t,in_dim", CHECK)
@@ -155,15 +156,15 @@ def test_gemv_matches_cpu_matmul_on_reference_fixtures(be, t, in_dim, seed):
     for o in range(out_dim):
         wrow = oracle.dequantize(t, raw[o * rb:(o + 1) * rb], in_dim).astype(np.float64)
         mag = np.abs(wrow * x).sum()
-        budget = 0.02 if t != Q8_0 else 0.01
+        budget = 0.01 if t in FLAT32 else 0.02
         assert abs(float(got[o]) - float(ref[o])) <= budget * max(mag, 1e-6)
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("T", [1, 2, 5, 8, 13])
 def test_matmul_decode_matches_cpu_and_each_token_alone(be, t, T):
     """backend/cpu.rs:623-650: a decode batch's row t is what token t gives alone."""
-    in_dim = 128 if t == Q8_0 else 512
+    in_dim = 128 if t in FLAT32 else 512
     out_dim = 7
     nb = NextByte(0x0051AB1E5EED)
     raw = cpu_rs_weights(t, in_dim, out_dim, nb) if t not in (Q6_K, Q3_K) else np.concatenate(
@@ -180,7 +181,7 @@ def test_matmul_decode_matches_cpu_and_each_token_alone(be, t, T):
         assert_bits(got[k], alone, f"token {k} alone")
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K])
 def test_matmul_multi_token_matches_cpu_gemm(be, t):
     """backend/cpu.rs:544-582 shapes: in = 3 blocks, out = 11 (odd), T in 1,2,5,77,3,1 from one
     reused backend; matmul at T > 1 follows the CPU GEMM kernels."""
@@ -276,6 +277,7 @@ def test_error_statuses(be):
     (Q6_K, 14336, 4096),    # config 5 ffn_down
     (Q5_K, 4096, 4096), (Q5_K, 14336, 4096),   # the same shapes in Q5_K
     (Q3_K, 4096, 4096), (Q3_K, 14336, 4096),   # and in Q3_K
+    (Q4_0, 4096, 4096), (Q5_0, 14336, 4096), (IQ4_NL, 4096, 14336),
 ])
 def test_benchmark_shapes_match_cpu(be, t, in_dim, out_dim):
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim)
@@ -454,6 +456,7 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign):
     (Q6_K, 256, 3), (Q6_K, 1280, 65), (Q6_K, 4096, 130), (Q6_K, 14336, 48), (Q6_K, 18432, 17),
     (Q5_K, 256, 5), (Q5_K, 768, 70), (Q5_K, 4096, 257), (Q5_K, 14336, 96), (Q5_K, 18432, 40),
     (Q3_K, 256, 5), (Q3_K, 768, 70), (Q3_K, 4096, 257), (Q3_K, 14336, 96), (Q3_K, 18432, 40),
+    (Q4_0, 32, 7), (Q4_0, 4096, 130), (Q5_0, 96, 33), (Q5_0, 4384, 64), (IQ4_NL, 896, 65), (IQ4_NL, 4096, 130),
 ])
 def test_single_token_gemv_quantizes_in_kernel_or_before_with_the_same_bits(be, t, in_dim, out_dim):
     """One token: the GEMV that quantizes its own activations and the quantizer kernel + GEMV
@@ -480,7 +483,7 @@ def test_single_token_gemv_quantizes_in_kernel_or_before_with_the_same_bits(be, 
             assert_bits(got[ok], want[ok], f"fuse mode {mode}")
 
 
-@pytest.mark.parametrize("t", [Q8_0, Q3_K, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("T,decode", [(1, False), (1, True), (4, True), (3, False), (16, False), (11, True)])
 def test_grouped_weights_over_one_input_equal_single_calls(be, t, T, decode):
     """q/k/v and gate/up read one input (engine/arch/mod.rs:1082-1096): the grouped call equals
@@ -548,7 +551,8 @@ def test_matmul_batch_groups_ops_that_share_their_input(be):
 
 
 @pytest.mark.parametrize("t,in_dim", [(Q8_0, 1056), (Q4_K, 1024), (Q4_K, 1536), (Q6_K, 1024), (Q6_K, 256), (Q5_K, 1024),
-                                      (Q5_K, 768), (Q3_K, 1024), (Q3_K, 1280)])
+                                      (Q5_K, 768), (Q3_K, 1024), (Q3_K, 1280), (Q4_0, 1056),
+                                      (Q5_0, 1056), (IQ4_NL, 1056)])
 def test_row_blocks_per_workgroup_do_not_change_a_bit(be, t, in_dim):
     """A workgroup may own several row blocks (ragged last group, last row block partly beyond
     out_dim, several matrices in one launch): every split gives the CPU path's bits."""
@@ -663,3 +667,33 @@ def test_q3k_extreme_integer_ranges(be, hmask, qs):
         assert_bits(be.matmul(x[0], 1, w), oracle.matmul(Q3_K, raw, in_dim, out_dim, x[0], 1), "gemv")
         assert_bits(be.matmul(x, T, w), oracle.matmul(Q3_K, raw, in_dim, out_dim, x, T), "matmul")
         assert_bits(be.matmul_decode(x, T, w), oracle.matmul_decode(Q3_K, raw, in_dim, out_dim, x, T), "decode")
+
+
+@pytest.mark.parametrize("t", [Q4_0, Q5_0, IQ4_NL])
+def test_per_32_nibble_types_every_byte_value_and_extreme_sums(be, t):
+    """Every nibble pair (and, for Q5_0, both values of every fifth bit) against activations of
+    +-127: the per-32 integer sums reach 32 * 127 * 127 (IQ4_NL), 32 * 16 * 127 (Q5_0)."""
+    bb = BLOCK[t][0]
+    in_dim, out_dim = 256, 64
+    blocks = np.zeros((out_dim * 8, bb), np.uint8)
+    blocks[:, 0:2] = np.frombuffer(np.float16(0.03125).tobytes(), np.uint8)
+    vals = np.arange(out_dim * 8 * 16, dtype=np.uint32)
+    blocks[:, bb - 16:] = ((vals * 37 + (vals >> 4) * 11) & 0xFF).reshape(-1, 16).astype(np.uint8)
+    blocks[::5, bb - 16:] = 0x00      # zero point / level 0 everywhere
+    blocks[1::5, bb - 16:] = 0xFF
+    if t == Q5_0:
+        blocks[:, 2:6] = ((vals[::16] * 2654435761) >> 3).astype(np.uint32).view(np.uint8).reshape(-1, 4)
+        blocks[::5, 2:6] = 0x00
+        blocks[1::5, 2:6] = 0xFF
+    raw = blocks.reshape(-1)
+    for sign in (1.0, -1.0):
+        x = np.full((3, in_dim), 127.0 * sign, np.float32)
+        x[1, ::2] *= -1
+        x[2, ::3] = 63.0
+        w = qm(raw, t, in_dim, out_dim)
+        isum, _ = be.dump_block_sums(x, 3, w)
+        wi, _ = oracle.block_sums(t, raw, in_dim, out_dim, x, 3)
+        assert np.array_equal(isum, wi)
+        say("per-32 extreme isum", t, int(np.abs(isum).max()))
+        assert_bits(be.matmul(x[0], 1, w), oracle.matmul(t, raw, in_dim, out_dim, x[0], 1), "gemv")
+        assert_bits(be.matmul(x, 3, w), oracle.matmul(t, raw, in_dim, out_dim, x, 3), "matmul")

@@ -4,11 +4,14 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Q3_K, Q4_K, Q5_K, Q6_K, Q8_0
+from helpers import IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0
 
 # quant.rs:1389-1417 GOLDEN (the types on the path)
 GOLDEN = [
+    (Q4_0, "q4_0", 256, 0x162325C968C10725),
+    (Q5_0, "q5_0", 256, 0x813F8949E12B3725),
     (Q8_0, "q8_0", 256, 0xC5D58782F54E52E5),
+    (IQ4_NL, "iq4_nl", 256, 0x7956C82FEBA12125),
     (Q3_K, "q3_k", 512, 0x2183E0B0538C6BE5),
     (Q4_K, "q4_k", 512, 0x9A7268A432A5C5FA),
     (Q5_K, "q5_k", 512, 0x41C70B9BE1696E6D),
@@ -46,6 +49,8 @@ def test_tensor_byte_size_and_block_layout():
     assert oracle.tensor_byte_size(Q6_K, 512) == 2 * 210
     assert oracle.tensor_byte_size(Q5_K, 256) == 176  # quant.rs:1701
     assert oracle.tensor_byte_size(Q3_K, 512) == 2 * 110
+    assert oracle.tensor_byte_size(Q4_0, 64) == 2 * 18 and oracle.tensor_byte_size(Q5_0, 64) == 2 * 22
+    assert oracle.tensor_byte_size(IQ4_NL, 64) == 2 * 18
     assert oracle.tensor_byte_size(Q4_K, 100) == -2  # not a whole number of blocks
     assert oracle.tensor_byte_size(99, 256) == -1  # unknown type
 
@@ -271,3 +276,43 @@ def test_dequantize_q3_k_element_order():
             want = np.zeros(256, np.float32)
             want[32 * p + j] = Q3K_SC_0X20[g] * -4
             assert np.array_equal(oracle.dequantize(Q3_K, block, 256), want), (p, j)
+
+
+KVALUES_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
+
+
+def test_dequantize_q4_0_and_q5_0_apply_their_fixed_offsets():
+    """quant.rs:1768-1775, 1807-1815: all-zero quants at d = 1 are -8 (Q4_0) and -16 (Q5_0)."""
+    block = np.zeros(18, np.uint8)
+    block[0:2] = _f16(1.0)
+    assert np.all(oracle.dequantize(Q4_0, block, 32) == -8.0)
+    block = np.zeros(22, np.uint8)
+    block[0:2] = _f16(1.0)
+    assert np.all(oracle.dequantize(Q5_0, block, 32) == -16.0)
+
+
+def test_dequantize_iq4_nl_uses_the_codebook_not_a_linear_offset():
+    """quant.rs:1785-1803: zero nibbles are level 0 = -127 (a linear Q4_0 decode would say -8);
+    byte j = j | j << 4 gives the sixteen levels in order in both halves."""
+    block = np.zeros(18, np.uint8)
+    block[0:2] = _f16(1.0)
+    assert np.all(oracle.dequantize(IQ4_NL, block, 32) == -127.0)
+    block[2:] = [j | (j << 4) for j in range(16)]
+    out = oracle.dequantize(IQ4_NL, block, 32)
+    assert np.array_equal(out[:16], KVALUES_IQ4NL) and np.array_equal(out[16:], KVALUES_IQ4NL)
+
+
+def test_per_32_nibble_types_element_order_and_fifth_bit():
+    """Element j < 16 is the low nibble of qs[j], element 16 + j the high nibble (quant.rs:546-551);
+    Q5_0's fifth bit of element e is bit e of the little-endian qh (quant.rs:571-574)."""
+    rng = np.random.default_rng(5)
+    for _ in range(10):
+        qs = rng.integers(0, 256, 16, dtype=np.uint8)
+        qh = rng.integers(0, 256, 4, dtype=np.uint8)
+        nib = np.concatenate([qs & 15, qs >> 4]).astype(np.int64)
+        b4 = np.concatenate([_f16(1.0), qs])
+        assert np.array_equal(oracle.dequantize(Q4_0, b4, 32), (nib - 8).astype(np.float32))
+        assert np.array_equal(oracle.dequantize(IQ4_NL, b4, 32), KVALUES_IQ4NL[nib])
+        bits = np.unpackbits(qh, bitorder="little").astype(np.int64)
+        b5 = np.concatenate([_f16(1.0), qh, qs])
+        assert np.array_equal(oracle.dequantize(Q5_0, b5, 32), (nib + 16 * bits - 16).astype(np.float32))

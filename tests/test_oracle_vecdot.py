@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (BLOCK, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, NextByte, activations, cpu_rs_weights, fixture_row,
+from helpers import (BLOCK, FLAT32, IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0, NextByte, activations, cpu_rs_weights, fixture_row,
                      k_fixture, row_bytes)
 
 
@@ -54,6 +54,17 @@ def np_unpack(ggml_type, row, in_dim):
         d = blocks[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)
         q = blocks[:, 2:].copy().view(np.int8).astype(np.int64).reshape(-1)
         return q, None, None, d, None
+    if ggml_type in (Q4_0, Q5_0, IQ4_NL):   # d | [qh u32] | qs[16]: low nibbles, then high nibbles
+        d = blocks[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)
+        qs = blocks[:, bb - 16:].astype(np.int64)
+        nib = np.concatenate([qs & 15, qs >> 4], axis=1)
+        if ggml_type == IQ4_NL:
+            q = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64)[nib]
+        elif ggml_type == Q4_0:
+            q = nib - 8
+        else:
+            q = nib + 16 * np.unpackbits(blocks[:, 2:6].copy(), axis=1, bitorder="little").astype(np.int64) - 16
+        return q.reshape(-1), None, None, d, None
     if ggml_type == Q4_K:
         d = blocks[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)
         dmin = blocks[:, 2:4].copy().view(np.float16).astype(np.float32).reshape(-1)
@@ -100,7 +111,7 @@ def np_unpack(ggml_type, row, in_dim):
 def np_block_sums(ggml_type, row, in_dim, xq):
     q, sce, mne, d, dmin = np_unpack(ggml_type, row, in_dim)
     xq = xq.astype(np.int64)
-    if ggml_type == Q8_0:
+    if ggml_type in FLAT32:
         return (q * xq).reshape(-1, 32).sum(axis=1), None
     isum = (q * sce * xq).reshape(-1, 256).sum(axis=1)
     imin = (mne * xq).reshape(-1, 256).sum(axis=1) if mne is not None else None
@@ -172,7 +183,9 @@ CHECK_CASES = [(Q8_0, 896), (Q8_0, 4864), (Q4_K, 256), (Q4_K, 4864 // 256 * 256)
 
 
 @pytest.mark.parametrize("ggml_type,in_dim", [(Q8_0, 896), (Q8_0, 4864), (Q4_K, 256), (Q4_K, 4864),
-                                              (Q6_K, 256), (Q6_K, 4864)])
+                                              (Q6_K, 256), (Q6_K, 4864), (Q5_0, 896), (Q5_0, 4864),
+                                              (Q4_0, 32), (Q4_0, 896), (Q4_0, 4864), (IQ4_NL, 896),
+                                              (IQ4_NL, 4864)])
 @pytest.mark.parametrize("seed", [1, 7, 99])
 def test_fused_dot_row_matches_dequantize_reference(ggml_type, in_dim, seed):
     """vecdot.rs:3436-3526 `check` via dot_row (per-32 activations): |got - ref| <= 0.01 * sum|w x|.
@@ -328,6 +341,9 @@ def test_supports_predicates():
     """vecdot.rs:274-283, 1821-1826, 3083-3093, 2456-2461 for the three types."""
     assert oracle.supports(Q8_0, 96) and not oracle.supports(Q8_0, 100)
     assert oracle.supports(Q4_K, 512) and not oracle.supports(Q4_K, 896)
+    for t in (Q5_0, Q4_0, IQ4_NL):   # vecdot.rs:4248-4262, 2456-2461
+        assert oracle.supports(t, 896) and not oracle.supports(t, 24) and oracle.supports_flat(t, 64)
+        assert not oracle.supports_k(t, 256) and not oracle.supports_k_row(t, 256)
     assert oracle.supports(Q3_K, 256) and oracle.supports_k(Q3_K, 2048) and not oracle.supports_k_row(Q3_K, 896)
     assert not oracle.supports_flat(Q3_K, 2048)   # vecdot.rs:4082, 4593-4594
     assert oracle.supports(Q5_K, 256) and oracle.supports_k(Q5_K, 512) and oracle.supports_k_row(Q5_K, 768)
@@ -383,3 +399,49 @@ def test_q3_k_unpack_applies_the_inverted_high_bit():
         assert v == np.float32(np.float32(act[1][0] * np.float32(1.0)) * np.float32(isum[0]))
         got = oracle.k_gemm_t(Q3_K, block, 256, 1, x, 1)
         assert got[0, 0] == np.float32(act[1][0] * np.float32(np.float32(1.0) * np.float32(isum[0])))
+
+
+def test_iq4_nl_block_unpack_is_exact_for_every_byte_value():
+    """vecdot.rs:3866-3887: all 256 byte values in every position against the table."""
+    table = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int8)
+    for base in range(256):
+        qs = ((base + 17 * np.arange(16)) % 256).astype(np.uint8)
+        _, w = oracle.unpack_flat_block(IQ4_NL, np.concatenate([np.zeros(2, np.uint8), qs]))
+        assert np.array_equal(w, np.concatenate([table[qs & 15], table[qs >> 4]])), base
+
+
+def test_q4_0_uses_its_own_zero_point_not_q5_0s():
+    """vecdot.rs:4226-4237: all-zero nibbles unpack to -8 for Q4_0 and to -16 for Q5_0."""
+    one = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    dw, w = oracle.unpack_flat_block(Q4_0, np.concatenate([one, np.zeros(16, np.uint8)]))
+    assert dw == 1.0 and np.all(w == -8)
+    dw, w = oracle.unpack_flat_block(Q5_0, np.concatenate([one, np.zeros(20, np.uint8)]))
+    assert dw == 1.0 and np.all(w == -16)
+    dw, w = oracle.unpack_flat_block(Q5_0, np.concatenate([one, np.full(4, 0xFF, np.uint8), np.full(16, 0xFF, np.uint8)]))
+    assert np.all(w == 15)
+
+
+@pytest.mark.parametrize("ggml_type", [Q5_0, Q4_0, IQ4_NL])
+def test_flat32_row_and_gemm_are_left_to_right_f32_over_independent_integer_sums(ggml_type):
+    """dot_q5_0 / _q4_0 / _iq4_nl: total += dw * act.d[b] * isum (vecdot.rs:2842-2883) and the flat
+    GEMM's acc += d * s * isum (vecdot.rs:2618-2624) rebuilt in numpy f32 from an independent decode;
+    matmul_decode rows equal single-token results."""
+    f = np.float32
+    in_dim, out_dim, T = 896, 5, 6
+    raw, x = k_fixture(ggml_type, in_dim, out_dim, T, 21)
+    rb = row_bytes(ggml_type, in_dim)
+    gemm = oracle.matmul(ggml_type, raw, in_dim, out_dim, x, T).reshape(T, out_dim)
+    dec = oracle.matmul_decode(ggml_type, raw, in_dim, out_dim, x, T).reshape(T, out_dim)
+    for o in range(out_dim):
+        row = raw[o * rb:(o + 1) * rb]
+        _, _, _, dw, _ = np_unpack(ggml_type, row, in_dim)
+        for t in range(T):
+            act = oracle.quantize_act(x[t * in_dim:(t + 1) * in_dim])
+            isum, _ = np_block_sums(ggml_type, row, in_dim, act[0])
+            a = b = f(0)
+            for blk in range(in_dim // 32):
+                a = f(a + f(f(dw[blk] * act[1][blk]) * f(isum[blk])))
+                b = f(b + f(f(act[1][blk] * dw[blk]) * f(isum[blk])))
+            assert oracle.dot_row(ggml_type, row, act).view(np.uint32) == a.view(np.uint32)
+            assert dec[t, o].view(np.uint32) == a.view(np.uint32)
+            assert gemm[t, o].view(np.uint32) == b.view(np.uint32)
