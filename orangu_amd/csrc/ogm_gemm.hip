@@ -26,6 +26,7 @@
 
 #include "ogm_kernels.h"
 #include "ogm_layout.h"
+#include "ogm_nib32_dev.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
@@ -782,6 +783,215 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
 }
 
 // ------------------------------------------------------------------------------------------
+// The symmetric per-32 types (Q8_0, Q5_0, Q4_0, IQ4_NL): the flat-activation GEMM
+// (dot_flat_pair, engine/vecdot.rs:2598-2629): acc += (ad * dw) * dot32 per 32-block.
+//
+// A block's integer dot is exact on the matrix cores: weights and activations are int8 values as
+// f16, a 32-long sum is at most 32 * 127 * 127 < 2^24.  Each block (two K = 16 MFMA steps) starts a
+// fresh accumulator and ends with the reference's f32 step, so the f32 work per MFMA is eight times
+// Q4_K's: this kernel is bound by the vector pipe, not by the matrix cores.
+//
+// Workgroup = 128 rows x 128 tokens, twelve waves: eight multiplying (64 rows x 32 tokens each),
+// four feeding.  A stage is 64 k = two blocks.  LDS rows are padded by one chunk (see the wide
+// Q4_K kernel); activations stay int8 in LDS.  Loads run three stages ahead of the MFMAs.
+
+struct GemmFlatParams {
+  const uint8_t *wt;      // tile-planar weights
+  const int8_t *xq;       // [T][in_dim] int8 activations
+  const float *ad;        // [T][in_dim / 32] activation scales
+  float *y;               // [T][out_dim]
+  uint32_t in_dim, out_dim, n_tokens, nblk;   // nblk = in_dim / 32 (even)
+  uint32_t c_shift, r_shift, nct;             // tiles of R = 1 << r_shift rows x C = 1 << c_shift blocks
+};
+
+#define GF_A_ROW 72u                       // f16 per staged weight row (64 + one chunk of padding)
+#define GF_B_ROW 80u                       // bytes per staged activation row
+#define GF_A_STAGE (128u * GF_A_ROW)       // f16
+#define GF_B_STAGE (128u * GF_B_ROW)       // bytes
+
+// KIND 0: Q4_0, 1: Q5_0, 2: IQ4_NL, 3: Q8_0
+template <int KIND>
+__global__ __launch_bounds__(768) void ogm_gemm_flat_kernel(GemmFlatParams p) {
+  constexpr uint32_t PIECES = KIND == 3 ? 2u : 1u;
+  constexpr uint32_t TAIL = KIND == 1 ? 6u : 2u;
+  constexpr uint32_t TILE = 64u * (16u * PIECES + TAIL);
+  __shared__ __align__(16) _Float16 A_l[2 * GF_A_STAGE];   // [2][128][72]
+  __shared__ __align__(16) uint8_t B_l[2 * GF_B_STAGE];    // [2][128][80]
+  __shared__ __align__(16) float dw_l[2 * 2 * 128];        // [2][block of the stage][128 rows]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const bool producer = wave >= 8u;
+  const uint32_t wr = wave & 1u, wt_ = (wave & 7u) >> 1;   // multiplying wave: row half, token quarter
+  const uint32_t t0 = blockIdx.x * 128u, r0 = blockIdx.y * 128u;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  const uint32_t n_st = p.nblk >> 1;
+
+  if (producer) {
+    // ---- feeding waves: one block of one row per thread and stage, two activation chunks
+    const uint32_t rt = tid & 255u;
+    const uint32_t arow = rt & 127u, abl = rt >> 7;
+    const uint32_t row = min(r0 + arow, p.out_dim - 1u);
+    const uint32_t rb = row >> p.r_shift, rr = row & ((1u << p.r_shift) - 1u);
+    const uint32_t tile_row = rb * p.nct * TILE;
+    // unit (row, block b): tile (b >> c_shift), lane ((b & (C - 1)) << r_shift) + rr
+    auto unit_off = [&](uint32_t b, uint32_t *tail) -> uint32_t {
+      const uint32_t to = tile_row + (b >> p.c_shift) * TILE;
+      const uint32_t ln = ((b & ((1u << p.c_shift) - 1u)) << p.r_shift) + rr;
+      *tail = to + PIECES * 1024u + ln * TAIL;
+      return to + ln * 16u;
+    };
+    const uint32_t btok0 = rt >> 2, bch = rt & 3u;   // chunk i: token btok0 + 64 i, 16-byte chunk bch
+    const uint32_t bo0 = min(t0 + btok0, p.n_tokens - 1u) * p.in_dim + 16u * bch;
+    const uint32_t bo1 = min(t0 + btok0 + 64u, p.n_tokens - 1u) * p.in_dim + 16u * bch;
+    const uint32_t bso = btok0 * GF_B_ROW + 16u * bch;
+    const uint32_t aso = arow * GF_A_ROW + 32u * abl;   // f16 offset of the block's first chunk
+
+    uint4 qa_0, qa_1, qa_2, qb_0, qb_1, qb_2;          // weight pieces (qb only for Q8_0)
+    uint32_t tl_0, tl_1, tl_2, th_0, th_1, th_2;       // tail: d16 (and qh for Q5_0)
+    uint4 bx_0, bx_1, bx_2, by_0, by_1, by_2;          // activation chunks
+
+#define GF_LOAD(ST, K)                                                                             \
+  do {                                                                                             \
+    const uint32_t st_ = min((uint32_t)(ST), n_st - 1u);                                           \
+    uint32_t tail_;                                                                                \
+    const uint32_t uo_ = unit_off(2u * st_ + abl, &tail_);                                         \
+    qa_##K = *(const uint4 *)(p.wt + uo_);                                                         \
+    if (KIND == 3) qb_##K = *(const uint4 *)(p.wt + uo_ + 1024u);                                  \
+    const uint16_t *tp_ = (const uint16_t *)(p.wt + tail_);                                        \
+    tl_##K = tp_[0];                                                                               \
+    th_##K = KIND == 1 ? ((uint32_t)tp_[1] | ((uint32_t)tp_[2] << 16)) : 0u;                       \
+    bx_##K = *(const uint4 *)(p.xq + (bo0 + st_ * 64u));                                           \
+    by_##K = *(const uint4 *)(p.xq + (bo1 + st_ * 64u));                                           \
+  } while (0)
+
+#define GF_STORE(BUF, K)                                                                           \
+  do {                                                                                             \
+    uint32_t w_[8]; /* the block's 32 int8 weights, k order */                                     \
+    if (KIND == 3) {                                                                               \
+      w_[0] = qa_##K.x; w_[1] = qa_##K.y; w_[2] = qa_##K.z; w_[3] = qa_##K.w;                      \
+      w_[4] = qb_##K.x; w_[5] = qb_##K.y; w_[6] = qb_##K.z; w_[7] = qb_##K.w;                      \
+    } else {                                                                                       \
+      const uint32_t q_[4] = {qa_##K.x, qa_##K.y, qa_##K.z, qa_##K.w};                             \
+      _Pragma("unroll") for (int k_ = 0; k_ < 4; k_++) {                                           \
+        w_[k_] = ogm_nib32_weights<KIND>(q_[k_] & 0x0F0F0F0Fu, (th_##K >> (4 * k_)) & 0xFu);       \
+        w_[4 + k_] = ogm_nib32_weights<KIND>((q_[k_] >> 4) & 0x0F0F0F0Fu,                          \
+                                             (th_##K >> (16 + 4 * k_)) & 0xFu);                    \
+      }                                                                                            \
+    }                                                                                              \
+    _Float16 *ab_ = A_l + (BUF) * GF_A_STAGE + aso;                                                \
+    _Pragma("unroll") for (int c_ = 0; c_ < 4; c_++)                                               \
+      *(half8 *)(ab_ + 8 * c_) = gw_i8_to_f16(w_[2 * c_], w_[2 * c_ + 1]);                         \
+    dw_l[(BUF) * 256u + abl * 128u + arow] = gm_f16_bits_to_f32(tl_##K);                           \
+    uint8_t *bb_ = B_l + (BUF) * GF_B_STAGE + bso;                                                 \
+    *(uint4 *)(bb_) = bx_##K;                                                                      \
+    *(uint4 *)(bb_ + 64u * GF_B_ROW) = by_##K;                                                     \
+  } while (0)
+
+    // stage m uses register set m mod 3; at the barrier of stage st the loads of st + 3 are
+    // requested and stage st + 1 is parked in the buffer the multiplying waves are not reading
+#define GF_PRODUCE(KL, KS)                                                                         \
+  do {                                                                                             \
+    GF_LOAD(st + 3u, KL);                                                                          \
+    GF_STORE((st + 1u) & 1u, KS);                                                                  \
+    __syncthreads();                                                                               \
+  } while (0)
+
+    GF_LOAD(0u, 0);
+    GF_LOAD(1u, 1);
+    GF_LOAD(2u, 2);
+    GF_STORE(0u, 0);
+    __syncthreads();
+    uint32_t st = 0;
+    while (true) {
+      GF_PRODUCE(0, 1);
+      if (++st == n_st) break;
+      GF_PRODUCE(1, 2);
+      if (++st == n_st) break;
+      GF_PRODUCE(2, 0);
+      if (++st == n_st) break;
+    }
+#undef GF_LOAD
+#undef GF_STORE
+#undef GF_PRODUCE
+    return;
+  }
+
+  // ---- multiplying waves: rows ra (+32), tokens tl
+  const uint32_t ra = 64u * wr + l32, tl = 32u * wt_ + l32;
+  const uint32_t tk = min(t0 + tl, p.n_tokens - 1u);
+  const uint32_t aro = ra * GF_A_ROW + 16u * lh;    // f16 offset of chunk 2 lh of row ra
+  const uint32_t bro = tl * GF_B_ROW + 16u * lh;    // byte offset of the lane half's 16 bytes
+  const float *adp = p.ad + (size_t)tk * p.nblk;
+  float16v y0, y1;
+#pragma unroll
+  for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
+  const float16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float2 adv = *(const float2 *)adp;   // the two blocks of stage 0
+  __syncthreads();
+#pragma unroll 1
+  for (uint32_t st = 0; st < n_st; st++) {
+    const uint32_t buf = st & 1u;
+    const float2 adn = *(const float2 *)(adp + 2u * min(st + 1u, n_st - 1u));
+    const _Float16 *ab = A_l + buf * GF_A_STAGE + aro;
+    const uint8_t *bb = B_l + buf * GF_B_STAGE + bro;
+    const float *dwp = dw_l + buf * 256u + 64u * wr + 4u * lh;
+#pragma unroll
+    for (int bl = 0; bl < 2; bl++) {
+      // the lane's 16 activations of this block: MFMA step kk takes bytes 8 kk .. 8 kk + 7
+      const uint4 bq = *(const uint4 *)(bb + 32u * bl);
+      float16v c0, c1;
+#pragma unroll
+      for (int kk = 0; kk < 2; kk++) {
+        const half8 a0 = *(const half8 *)(ab + 32u * bl + 8u * kk);
+        const half8 a1 = *(const half8 *)(ab + 32u * GF_A_ROW + 32u * bl + 8u * kk);
+        const half8 b = kk ? gw_i8_to_f16(bq.z, bq.w) : gw_i8_to_f16(bq.x, bq.y);
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b, kk ? c0 : zero, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b, kk ? c1 : zero, 0, 0, 0);
+      }
+      // acc += d * s * dot32 (vecdot.rs:2622): (ad * dw) * (f32)isum
+      const float ad = bl ? adv.y : adv.x;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const float4 d0 = *(const float4 *)(dwp + 128 * bl + 8 * q4);
+        const float4 d1 = *(const float4 *)(dwp + 128 * bl + 32 + 8 * q4);
+        y0[4 * q4 + 0] += ad * d0.x * c0[4 * q4 + 0];
+        y0[4 * q4 + 1] += ad * d0.y * c0[4 * q4 + 1];
+        y0[4 * q4 + 2] += ad * d0.z * c0[4 * q4 + 2];
+        y0[4 * q4 + 3] += ad * d0.w * c0[4 * q4 + 3];
+        y1[4 * q4 + 0] += ad * d1.x * c1[4 * q4 + 0];
+        y1[4 * q4 + 1] += ad * d1.y * c1[4 * q4 + 1];
+        y1[4 * q4 + 2] += ad * d1.z * c1[4 * q4 + 2];
+        y1[4 * q4 + 3] += ad * d1.w * c1[4 * q4 + 3];
+      }
+    }
+    adv = adn;
+    __syncthreads();
+  }
+
+  // ---------------- store: a lane holds one token column and its rows in runs of four
+  const uint32_t t = t0 + tl;
+  if (t < p.n_tokens) {
+    const bool vec = (p.out_dim & 3u) == 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const float16v &yy = i ? y1 : y0;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const uint32_t row = r0 + 64u * wr + 32u * i + 8u * q4 + 4u * lh;
+        float *dst = p.y + (size_t)t * p.out_dim + row;
+        if (vec && row + 3u < p.out_dim) {
+          *(float4 *)dst = make_float4(yy[4 * q4], yy[4 * q4 + 1], yy[4 * q4 + 2], yy[4 * q4 + 3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            if (row + e < p.out_dim) dst[e] = yy[4 * q4 + e];
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Q6_K (gemm_k_q6_k, engine/vecdot.rs:2352-2398): acc += ad * (d * sum_g sc_g * dot16(q_g - 32, x_g))
 // over the 16 groups of a super-block, sc_g a signed byte.
 //
@@ -1015,12 +1225,22 @@ size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens) {
   return (size_t)in_dim * n_tokens * 2 + (size_t)(in_dim / 256) * n_tokens * 32;
 }
 
+static bool is_flat32(uint32_t t) { return t == OGM_Q8_0 || t == OGM_Q5_0 || t == OGM_Q4_0 || t == OGM_IQ4_NL; }
+
 bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
+  // the kernels address weights and activations with 32-bit byte offsets
+  const uint64_t lim = 0xFFFFFFFFull;
+  if (is_flat32(ggml_type)) {
+    // two blocks per stage
+    if (in_dim == 0 || in_dim % 64u != 0) return false;
+    OgmLayout l;
+    ogm_layout_for(ggml_type, &l);
+    return (uint64_t)ogm_tiling_for(in_dim / 32u, out_dim).nrb * 64u * (in_dim / 32u) * l.block_bytes <= lim &&
+           (uint64_t)in_dim * n_tokens <= lim;
+  }
   if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K) || in_dim == 0 || in_dim % 256u != 0) return false;
   // Q4_K's pass 1 keeps one f32 per (row, super-block) of the workgroup in LDS
   if (ggml_type == OGM_Q4_K && GM_LDS_BYTES + (size_t)(in_dim / 256u) * 512u > GM_LDS_MAX) return false;
-  // the kernels address weights and activations with 32-bit byte offsets
-  const uint64_t lim = 0xFFFFFFFFull;
   const uint64_t block = ggml_type == OGM_Q4_K ? 144u : 210u;
   return (uint64_t)ogm_tiling_for(in_dim / 256u, out_dim).nrb * 64u * (in_dim / 256u) * block <= lim &&
          (uint64_t)in_dim * n_tokens * 2u <= lim;
@@ -1029,6 +1249,30 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name) {
   if (a.n_tokens == 0 || a.out_dim == 0) return hipSuccess;
   if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return hipErrorInvalidValue;
+  if (is_flat32(a.ggml_type)) {
+    GemmFlatParams p;
+    p.wt = a.wt;
+    p.xq = a.act.q;
+    p.ad = a.act.d;
+    p.y = a.y;
+    p.in_dim = a.in_dim;
+    p.out_dim = a.out_dim;
+    p.n_tokens = a.n_tokens;
+    p.nblk = a.in_dim / 32;
+    const OgmTiling tl = ogm_tiling_for(p.nblk, a.out_dim);
+    p.c_shift = tl.C == 4 ? 2 : 1;   // in_dim % 64 == 0: at least two blocks per tile row
+    p.r_shift = 6 - p.c_shift;
+    p.nct = tl.nct;
+    const dim3 grid((a.n_tokens + 127u) / 128u, (a.out_dim + 127u) / 128u);
+    switch (a.ggml_type) {
+      case OGM_Q4_0: hipLaunchKernelGGL(ogm_gemm_flat_kernel<0>, grid, dim3(768), 0, stream, p); break;
+      case OGM_Q5_0: hipLaunchKernelGGL(ogm_gemm_flat_kernel<1>, grid, dim3(768), 0, stream, p); break;
+      case OGM_IQ4_NL: hipLaunchKernelGGL(ogm_gemm_flat_kernel<2>, grid, dim3(768), 0, stream, p); break;
+      default: hipLaunchKernelGGL(ogm_gemm_flat_kernel<3>, grid, dim3(768), 0, stream, p); break;
+    }
+    if (kernel_name) *kernel_name = "ogm_gemm_flat_kernel";
+    return hipGetLastError();
+  }
   const uint32_t nsb = a.in_dim / 256;
   const size_t n8 = (size_t)a.in_dim * a.n_tokens / 8, n_sb = (size_t)nsb * a.n_tokens;
   _Float16 *xh = (_Float16 *)a.xh;

@@ -18,6 +18,7 @@
 
 #include "ogm_kernels.h"
 #include "ogm_layout.h"
+#include "ogm_nib32_dev.h"
 #include "ogm_quant_dev.h"
 
 
@@ -557,20 +558,8 @@ struct FmtNib32 {
     r.d16 = t[0];
     r.qh = KIND == 1 ? ((uint32_t)t[1] | ((uint32_t)t[2] << 16)) : 0u;
   }
-  // Four nibbles (one per byte, 0..15), with four fifth bits `h4` for Q5_0, as signed weights.
   __device__ static __forceinline__ uint32_t weights(uint32_t n, uint32_t h4) {
-    if (KIND == 2) {
-      // sixteen-entry byte table: two eight-entry v_perm lookups, chosen by bit 3 of the index
-      const uint32_t sel = n & 0x07070707u;
-      const uint32_t lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, sel);   // levels 0..7
-      const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, sel);   // levels 8..15
-      const uint32_t pick = ((n >> 3) & 0x01010101u) * 0xFFu;
-      return (lo & ~pick) | (hi & pick);
-    }
-    // v - bias per byte without borrows between bytes: set bit 7, subtract, flip bit 7 back
-    const uint32_t v = KIND == 1 ? (n | (((h4 * 0x00204081u) & 0x01010101u) << 4)) : n;
-    const uint32_t bias = KIND == 1 ? 0x10101010u : 0x08080808u;
-    return ((v | 0x80808080u) - bias) ^ 0x80808080u;
+    return ogm_nib32_weights<KIND>(n, h4);
   }
   template <int UPR>
   __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col,

@@ -697,3 +697,50 @@ def test_per_32_nibble_types_every_byte_value_and_extreme_sums(be, t):
         say("per-32 extreme isum", t, int(np.abs(isum).max()))
         assert_bits(be.matmul(x[0], 1, w), oracle.matmul(t, raw, in_dim, out_dim, x[0], 1), "gemv")
         assert_bits(be.matmul(x, 3, w), oracle.matmul(t, raw, in_dim, out_dim, x, 3), "matmul")
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL])
+@pytest.mark.parametrize("in_dim,out_dim,T", [(64, 5, 9), (128, 130, 17), (896, 64, 40), (4096, 257, 130),
+                                              (4864, 100, 300), (1024, 128, 128), (2048, 129, 513)])
+def test_mfma_gemm_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T):
+    """The symmetric per-32 types at n_tokens >= 9 and in_dim % 64 == 0 take the MFMA flat GEMM; values
+    must equal dot_flat_pair (vecdot.rs:2598-2629) bit for bit, and the small-batch kernel's."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T + t)
+    x = synth_x(T, in_dim, seed=T + 1)
+    w = qm(raw, t, in_dim, out_dim)
+    say("flat gemm", t, in_dim, out_dim, T)
+    got = be.matmul(x, T, w)
+    assert be.last_kernel() == "ogm_gemm_flat_kernel"
+    want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
+    assert_close(got, want, "flat mfma gemm")
+    assert_bits(got, want, "flat mfma gemm")
+    be.set_tuning("gemm_min_tokens", 100000)
+    try:
+        small = be.matmul(x, T, w)
+        assert be.last_kernel().startswith("ogm_gemv_kernel")
+    finally:
+        be.set_tuning("gemm_min_tokens", 0)
+    assert_bits(small, want, "multi-token gemv")
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL])
+def test_mfma_gemm_flat_extreme_block_sums(be, t):
+    """Largest per-32 sums: weights at their extremes against activations of +-127 (Q8_0 and IQ4_NL:
+    32 * 127 * 127 = 516 128, exact in the f32 accumulator)."""
+    bb = BLOCK[t][0]
+    in_dim, out_dim, T = 256, 40, 24
+    blocks = np.zeros((out_dim * 8, bb), np.uint8)
+    blocks[:, 0:2] = np.frombuffer(np.float16(0.0078125).tobytes(), np.uint8)
+    blocks[0::3, 2:] = 0x00 if t != Q8_0 else 0x81      # -127 / zero point / level 0
+    blocks[1::3, 2:] = 0xFF if t != Q8_0 else 0x7F      # +127 / top level
+    blocks[2::3, 2:] = 0xF0 if t != Q8_0 else 0x81
+    raw = blocks.reshape(-1)
+    x = np.full((T, in_dim), 127.0, np.float32)
+    x[1::2] *= -1
+    x[:, 5::11] = -127.0
+    w = qm(raw, t, in_dim, out_dim)
+    got = be.matmul(x, T, w)
+    assert be.last_kernel() == "ogm_gemm_flat_kernel"
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "extreme sums")
+    isum, _ = be.dump_block_sums(x[0], 1, w)
+    say("flat extreme isum", t, int(np.abs(isum).max()))
