@@ -17,8 +17,10 @@
  *   backend/cpu.rs  kernel choice per (type, n_tokens, entry point)
  *
  * Pinning (what each part is checked against, without running the reference):
- *   dequantize / f16 / get_scale_min_k4   golden bit checksums quant.rs:1389-1463 and the
- *                                         hand-built blocks quant.rs:1818-1921   -> PINNED
+ *   dequantize / f16 / get_scale_min_k4   golden bit checksums quant.rs:1389-1463 (q8_0, q4_0, q5_0,
+ *   / unpack_q3_k_scales / block unpacks  iq4_nl, q3_k, q4_k, q5_k, q6_k) and the hand-built blocks
+ *                                         quant.rs:1768-1921, vecdot.rs:3866-3968, 4141-4165,
+ *                                         4226-4237                              -> PINNED
  *   quantizers                            ties-away, zero block, adversarial blocks
  *                                         vecdot.rs:4259-4410 (expected bytes derived by hand
  *                                         from the stated rules)                 -> PINNED
