@@ -201,10 +201,20 @@ typedef struct ogm_llama_config {
   uint32_t rope_dim;    /* rotated dimensions per head, <= head_dim */
   uint32_t max_ctx;     /* KV-cache capacity in positions */
   float rms_eps, rope_freq_base;
+  /* RoPE pairing (rope_layout_for, llama.rs:115-120): 0 = NORM, pairs (2i, 2i+1), for "llama" and
+   * "mistral" files; 1 = NEOX, pairs (i, i + rope_dim/2), for qwen2 / qwen3 and the rest. */
+  uint32_t rope_neox;
+  /* rope_freqs.weight (llama.rs:186-201): host f32 [rope_dim/2] divisors of the pair frequencies,
+   * copied; null when the file has none. */
+  const float *rope_freq_factors;
 } ogm_llama_config;
 typedef struct ogm_llama_layer {
   const ogm_weight *wq, *wk, *wv, *wo, *w_gate, *w_up, *w_down;
   const float *attn_norm, *ffn_norm;   /* host f32 [n_embd], copied */
+  /* optional, host f32, copied, null when the file has no such tensor (llama.rs:174-178):
+   * projection biases [n_head*head_dim], [n_head_kv*head_dim] x 2 (added first, llama.rs:757-765)
+   * and per-head RMSNorm weights [head_dim] of q and k (applied before RoPE, llama.rs:770-787). */
+  const float *q_bias, *k_bias, *v_bias, *q_norm, *k_norm;
 } ogm_llama_layer;
 
 /* Builds the device-side model over weights already uploaded with ogm_weight_upload (they must
@@ -217,6 +227,12 @@ void ogm_llama_destroy(ogm_ctx *ctx, ogm_llama *m);
  * (K already rotated), as a CPU prefill hands its cache over (LayerCache::push, kv_cache.rs:756-768). */
 int ogm_llama_kv_write(ogm_ctx *ctx, ogm_llama *m, uint32_t layer, uint32_t pos0, uint32_t n_pos,
                        const float *k, const float *v);
+
+/* The reverse: cache rows pos0 .. pos0+n_pos of one layer as the f16 bit patterns the device holds
+ * ([n_pos][n_head_kv*head_dim] each, K rotated), e.g. to park a sequence on the host as the
+ * reference's slot store does with LayerCache rows (kv_cache.rs:756-768).  Waits for the stream. */
+int ogm_llama_kv_read(ogm_ctx *ctx, ogm_llama *m, uint32_t layer, uint32_t pos0, uint32_t n_pos,
+                      uint16_t *k_bits, uint16_t *v_bits);
 
 /* Decodes the token at position `pos` whose embedding row is x ([n_embd] f32; the caller looks it
  * up as run_layers does, llama.rs:609-614).  Appends its K/V at `pos`, attends to 0..pos.

@@ -5,8 +5,10 @@ legs, never by the product.
 
 Follows orangu-server's `LlamaModel::run_layers` + `forward` at n_tokens == 1
 (engine/arch/llama.rs:594-932, 1007-1032) with the element-wise definitions of engine/tensor.rs
-(rmsnorm_into :732-757, softmax_inplace :809-821, silu :825-827, rope_apply_params_inplace
-:1115-1177 with NORM pairing, freq_scale 1, no YaRN, no frequency factors), the CPU attention loop
+(rmsnorm_into :732-757, rmsnorm_inplace :691-706 per head, add_bias_per_row :1233-1240,
+softmax_inplace :809-821, silu :825-827, rope_apply_params_inplace :1115-1177 with NORM or NEOX
+pairing and frequency factors; freq_scale 1 and no YaRN, as llama.rs:203-208 sets them), the CPU
+attention loop
 (engine/attention.rs:426-549), swiglu_ffn_into (engine/arch/mod.rs:1071-1106) and the greedy
 argmax (engine/sampling.rs:336-343).  The quantized matmuls are the C oracle's (`oracle.matmul`,
 single-token path).
@@ -18,7 +20,8 @@ pinned to rounding, not to the bit.
 
 Pinned by tests/test_oracle_llama.py: the reference's own test values (rmsnorm of [3, 4]
 tensor.rs:1450-1466, silu(0) / silu(1) :1621-1625, the NORM rotation of [1..8] at position 3
-:1752-1769, position 0 = identity :1668, pair norms preserved :1676, softmax sums to one :1612),
+:1752-1769, the NEOX rotation of the same :1731-1749, frequency factors divide the angle
+:1785-1822, position 0 = identity :1668, pair norms preserved :1676, softmax sums to one :1612),
 closed forms (constant rows, a single cached position, equal scores = mean of V), the grouped-query
 head mapping by brute force, and last-of-equal argmax.  parity unpinned: none of these functions
 has a bit-level golden vector in the reference; they are pinned to 1e-6.
@@ -54,17 +57,36 @@ def rope_freqs(rope_dim: int, freq_base: float) -> np.ndarray:
     return np.power(f32(freq_base), (f32(-2.0) * i / f32(rope_dim)).astype(f32), dtype=f32)
 
 
-def rope_norm(x: np.ndarray, n_head: int, head_dim: int, pos: int, rope_dim: int, freq_base: float) -> np.ndarray:
-    """tensor.rs:1115-1177, RopeLayout::Norm: pair i is elements (2i, 2i+1) of every head."""
+def rope(x: np.ndarray, n_head: int, head_dim: int, pos: int, rope_dim: int, freq_base: float,
+         freq_factors=None, neox: bool = False) -> np.ndarray:
+    """tensor.rs:1115-1177 with freq_scale 1 and ext_factor 0: pair i turns by pos * freq_i, where
+    freq_i = base^(-2i / rope_dim) / factor_i (:1147-1150); RopeLayout::Norm pairs elements
+    (2i, 2i+1) of every head, RopeLayout::Neox pairs (i, i + rope_dim/2) (:1163-1168)."""
     x = np.array(x, f32).reshape(n_head, head_dim)
-    theta = (f32(pos) * rope_freqs(rope_dim, freq_base)).astype(f32)
+    freq = rope_freqs(rope_dim, freq_base)
+    if freq_factors is not None:
+        freq = (freq / np.asarray(freq_factors, f32)[:rope_dim // 2]).astype(f32)
+    theta = (f32(pos) * freq).astype(f32)
     sin, cos = np.sin(theta, dtype=f32), np.cos(theta, dtype=f32)
     half = rope_dim // 2
-    a = x[:, 0:2 * half:2].copy()
-    b = x[:, 1:2 * half:2].copy()
-    x[:, 0:2 * half:2] = a * cos - b * sin
-    x[:, 1:2 * half:2] = a * sin + b * cos
+    lo = slice(0, half) if neox else slice(0, 2 * half, 2)
+    hi = slice(half, 2 * half) if neox else slice(1, 2 * half, 2)
+    a = x[:, lo].copy()
+    b = x[:, hi].copy()
+    x[:, lo] = a * cos - b * sin
+    x[:, hi] = a * sin + b * cos
     return x.reshape(-1)
+
+
+def rope_norm(x: np.ndarray, n_head: int, head_dim: int, pos: int, rope_dim: int, freq_base: float) -> np.ndarray:
+    """RopeLayout::Norm without frequency factors."""
+    return rope(x, n_head, head_dim, pos, rope_dim, freq_base)
+
+
+def head_rmsnorm(x: np.ndarray, weight: np.ndarray, n_head: int, head_dim: int, eps: float) -> np.ndarray:
+    """llama.rs:770-787: rmsnorm_inplace over rows of head_dim, one weight vector for every head."""
+    x = np.asarray(x, f32).reshape(n_head, head_dim)
+    return np.concatenate([rmsnorm(x[h], weight, eps) for h in range(n_head)])
 
 
 def softmax(x: np.ndarray) -> np.ndarray:
@@ -119,6 +141,11 @@ class Layer:
     w_down: tuple
     attn_norm: np.ndarray
     ffn_norm: np.ndarray
+    q_bias: np.ndarray | None = None     # attn_q.bias etc. (Qwen2), llama.rs:174-176
+    k_bias: np.ndarray | None = None
+    v_bias: np.ndarray | None = None
+    q_norm: np.ndarray | None = None     # attn_q_norm.weight etc. (Qwen3), llama.rs:177-178
+    k_norm: np.ndarray | None = None
 
 
 @dataclass
@@ -135,7 +162,12 @@ class Model:
     layers: list
     output_norm: np.ndarray
     output: tuple
+    rope_neox: bool = False          # rope_layout_for, llama.rs:115-120
+    rope_freq_factors: np.ndarray | None = None   # rope_freqs.weight, llama.rs:186-201
     kv_dtype: type = np.float16      # the build keeps the cache in f16; np.float32 = the reference's host cache
+    # kv_hook(layer, pos, k_row, v_row) -> (k_row, v_row): lets a test look at the rows about to be
+    # cached and replace them (by a device's rows that differ in the last f16 bit, say)
+    kv_hook: object = None
     k_cache: list = field(default_factory=list)   # per layer: list of rows
     v_cache: list = field(default_factory=list)
 
@@ -158,12 +190,25 @@ def decode_step(m: Model, x: np.ndarray, pos: int):
     for li, L in enumerate(m.layers):
         normed = rmsnorm(x, L.attn_norm, m.rms_eps)
         q, k, v = _mm(L.wq, normed), _mm(L.wk, normed), _mm(L.wv, normed)
-        q = rope_norm(q, m.n_head, m.head_dim, pos, m.rope_dim, m.rope_freq_base)
-        k = rope_norm(k, m.n_head_kv, m.head_dim, pos, m.rope_dim, m.rope_freq_base)
+        if L.q_bias is not None:                       # llama.rs:757-765
+            q = (q + np.asarray(L.q_bias, f32)).astype(f32)
+        if L.k_bias is not None:
+            k = (k + np.asarray(L.k_bias, f32)).astype(f32)
+        if L.v_bias is not None:
+            v = (v + np.asarray(L.v_bias, f32)).astype(f32)
+        if L.q_norm is not None:                       # llama.rs:770-787, before RoPE
+            q = head_rmsnorm(q, L.q_norm, m.n_head, m.head_dim, m.rms_eps)
+        if L.k_norm is not None:
+            k = head_rmsnorm(k, L.k_norm, m.n_head_kv, m.head_dim, m.rms_eps)
+        q = rope(q, m.n_head, m.head_dim, pos, m.rope_dim, m.rope_freq_base, m.rope_freq_factors, m.rope_neox)
+        k = rope(k, m.n_head_kv, m.head_dim, pos, m.rope_dim, m.rope_freq_base, m.rope_freq_factors, m.rope_neox)
         kc, vc = m.k_cache[li], m.v_cache[li]
         assert len(kc) == pos, "decode positions must be appended in order"
-        kc.append(k.astype(m.kv_dtype))
-        vc.append(v.astype(m.kv_dtype))
+        k_row, v_row = k.astype(m.kv_dtype), v.astype(m.kv_dtype)
+        if m.kv_hook is not None:
+            k_row, v_row = m.kv_hook(li, pos, k_row, v_row)
+        kc.append(k_row)
+        vc.append(v_row)
         attn = attention(q, np.stack(kc).astype(f32), np.stack(vc).astype(f32), m.n_head, m.n_head_kv, m.head_dim)
         x = (x + _mm(L.wo, attn)).astype(f32)
         normed2 = rmsnorm(x, L.ffn_norm, m.rms_eps)

@@ -292,18 +292,32 @@ class LlamaDecoder:
     """The device-resident decode step of a Llama-family model over a Mi355xBackend
     (LlamaModel::forward at n_tokens == 1, engine/arch/llama.rs:1007-1032).
 
-    ``layers`` is a list of dicts with QuantMatrix entries wq, wk, wv, wo, w_gate, w_up, w_down and
-    f32 arrays attn_norm, ffn_norm; ``output`` a QuantMatrix; ``output_norm`` an f32 array."""
+    ``layers`` is a list of dicts with QuantMatrix entries wq, wk, wv, wo, w_gate, w_up, w_down,
+    f32 arrays attn_norm, ffn_norm and, where the file has them, q_bias, k_bias, v_bias (Qwen2) and
+    q_norm, k_norm (Qwen3; llama.rs:174-178); ``output`` a QuantMatrix; ``output_norm`` an f32 array.
+    ``rope_neox`` follows rope_layout_for (llama.rs:115-120): False for "llama" / "mistral" files;
+    ``rope_freq_factors`` is rope_freqs.weight (llama.rs:186-201) or None."""
 
     def __init__(self, be: "Mi355xBackend", *, n_embd: int, n_head: int, n_head_kv: int, head_dim: int,
                  n_ff: int, n_vocab: int, layers, output_norm, output, max_ctx: int, rope_dim: int | None = None,
-                 rms_eps: float = 1e-5, rope_freq_base: float = 10000.0, upload=None):
+                 rms_eps: float = 1e-5, rope_freq_base: float = 10000.0, rope_neox: bool = False,
+                 rope_freq_factors=None, upload=None):
         self._be = be
         up = upload or be.upload
-        cfg = capi.OgmLlamaConfig(len(layers), n_embd, n_head, n_head_kv, head_dim, n_ff, n_vocab,
-                                  head_dim if rope_dim is None else rope_dim, max_ctx, rms_eps, rope_freq_base)
-        arr = (capi.OgmLlamaLayer * len(layers))()
+        rope_dim = head_dim if rope_dim is None else rope_dim
         self._keep = []
+        ff = None
+        if rope_freq_factors is not None:
+            ff = np.ascontiguousarray(rope_freq_factors, np.float32).reshape(-1)
+            if ff.size < rope_dim // 2:   # llama.rs:189-195
+                raise ValueError(f"rope_freq_factors has {ff.size} entries, need {rope_dim // 2}")
+            self._keep.append(ff)
+        cfg = capi.OgmLlamaConfig(len(layers), n_embd, n_head, n_head_kv, head_dim, n_ff, n_vocab,
+                                  rope_dim, max_ctx, rms_eps, rope_freq_base, 1 if rope_neox else 0,
+                                  ff.ctypes.data if ff is not None else None)
+        arr = (capi.OgmLlamaLayer * len(layers))()
+        want = {"q_bias": n_head * head_dim, "k_bias": n_head_kv * head_dim, "v_bias": n_head_kv * head_dim,
+                "q_norm": head_dim, "k_norm": head_dim}
         for i, L in enumerate(layers):
             for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
                 setattr(arr[i], name, up(L[name]))
@@ -311,18 +325,34 @@ class LlamaDecoder:
                 a = np.ascontiguousarray(L[name], np.float32)
                 self._keep.append(a)
                 setattr(arr[i], name, a.ctypes.data)
+            for name, size in want.items():
+                if L.get(name) is None:
+                    continue
+                a = np.ascontiguousarray(L[name], np.float32).reshape(-1)
+                if a.size != size:
+                    raise ValueError(f"layer {i}: {name} has {a.size} values, expected {size}")
+                self._keep.append(a)
+                setattr(arr[i], name, a.ctypes.data)
         on = np.ascontiguousarray(output_norm, np.float32)
         h = C.c_void_p()
         be._check(be._lib.ogm_llama_create(be._ctx, C.byref(cfg), arr, on.ctypes.data, up(output), C.byref(h)),
                   "ogm_llama_create")
         self._h = h.value
-        self.n_embd, self.n_vocab, self.kv_dim = n_embd, n_vocab, n_head_kv * head_dim
+        self.n_embd, self.n_vocab, self.kv_dim, self.n_layer = n_embd, n_vocab, n_head_kv * head_dim, len(layers)
 
     def kv_write(self, layer: int, pos0: int, k, v):
         k = np.ascontiguousarray(k, np.float32).reshape(-1, self.kv_dim)
         v = np.ascontiguousarray(v, np.float32).reshape(-1, self.kv_dim)
         self._be._check(self._be._lib.ogm_llama_kv_write(self._be._ctx, self._h, layer, pos0, k.shape[0],
                                                          k.ctypes.data, v.ctypes.data), "ogm_llama_kv_write")
+
+    def kv_read(self, layer: int, pos0: int, n_pos: int):
+        """Cache rows pos0 .. pos0+n_pos of a layer as float16 arrays [n_pos][kv_dim] (k, v)."""
+        k = np.empty((n_pos, self.kv_dim), np.float16)
+        v = np.empty((n_pos, self.kv_dim), np.float16)
+        self._be._check(self._be._lib.ogm_llama_kv_read(self._be._ctx, self._h, layer, pos0, n_pos,
+                                                        k.ctypes.data, v.ctypes.data), "ogm_llama_kv_read")
+        return k, v
 
     def decode(self, x, pos: int):
         """Returns (logits, argmax) for the token whose embedding row is x, at position pos."""

@@ -23,7 +23,7 @@ SYMBOLS = [
     "ogm_weight_info", "ogm_matmul", "ogm_matmul_decode", "ogm_matmul_batch", "ogm_matmul_dev",
     "ogm_quantize_act", "ogm_dump_block_sums", "ogm_f16_to_f32", "ogm_set_tuning",
     "ogm_last_kernel", "ogm_act_quantize_dev", "ogm_matmul_act_dev", "ogm_matmul_multi_dev", "ogm_matmul_multi_act_dev",
-    "ogm_llama_create", "ogm_llama_destroy", "ogm_llama_kv_write", "ogm_llama_decode", "ogm_llama_decode_dev",
+    "ogm_llama_create", "ogm_llama_destroy", "ogm_llama_kv_write", "ogm_llama_kv_read", "ogm_llama_decode", "ogm_llama_decode_dev",
     "ogm_llama_debug_hidden", "ogm_dequant_rows", "ogm_llama_generate",
     "ogm_gguf_open", "ogm_gguf_parse", "ogm_gguf_close", "ogm_gguf_last_error", "ogm_gguf_info",
     "ogm_gguf_meta_u64", "ogm_gguf_meta_f64", "ogm_gguf_meta_string", "ogm_gguf_meta_array",
@@ -41,12 +41,14 @@ class OgmError(RuntimeError):
 class OgmLlamaConfig(C.Structure):
     _fields_ = [(n, C.c_uint32) for n in ("n_layer", "n_embd", "n_head", "n_head_kv", "head_dim", "n_ff",
                                           "n_vocab", "rope_dim", "max_ctx")] + \
-               [("rms_eps", C.c_float), ("rope_freq_base", C.c_float)]
+               [("rms_eps", C.c_float), ("rope_freq_base", C.c_float), ("rope_neox", C.c_uint32),
+                ("rope_freq_factors", C.c_void_p)]
 
 
 class OgmLlamaLayer(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down",
-                                          "attn_norm", "ffn_norm")]
+                                          "attn_norm", "ffn_norm", "q_bias", "k_bias", "v_bias",
+                                          "q_norm", "k_norm")]
 
 
 class OgmOp(C.Structure):
@@ -94,6 +96,7 @@ def load_library() -> C.CDLL:
     L.ogm_llama_destroy.argtypes = [vp, vp]
     L.ogm_llama_destroy.restype = None
     L.ogm_llama_kv_write.argtypes = [vp, vp, u32, u32, u32, vp, vp]
+    L.ogm_llama_kv_read.argtypes = [vp, vp, u32, u32, u32, vp, vp]
     L.ogm_llama_decode.argtypes = [vp, vp, vp, u32, vp, vp]
     L.ogm_llama_decode_dev.argtypes = [vp, vp, vp, u32, vp, vp, vp]
     L.ogm_llama_debug_hidden.argtypes = [vp, vp, vp]

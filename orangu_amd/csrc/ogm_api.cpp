@@ -729,11 +729,12 @@ extern "C" int ogm_f16_to_f32(ogm_ctx *ctx, const uint16_t *bits, size_t n, floa
 
 struct ogm_llama {
   ogm_llama_config cfg;
-  std::vector<ogm_llama_layer> layers;  // weight handles; the norm pointers are unused after create
+  std::vector<ogm_llama_layer> layers;  // weight handles; the optional vectors as device pointers
   const ogm_weight *output = nullptr;
   // device memory
   float *norms = nullptr;     // [n_layer][2][n_embd] then output_norm [n_embd]
-  float *freq = nullptr;      // [rope_dim / 2]
+  float *pre = nullptr;       // [n_layer][q_bias qd | k_bias kvd | v_bias kvd | q_norm hd | k_norm hd]
+  float *freq = nullptr;      // [rope_dim / 2], frequency factors applied
   float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
   uint32_t *attn_tickets = nullptr;   // [n_head_kv], zero between launches
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
@@ -775,8 +776,12 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   if (c.n_layer == 0 || c.n_embd == 0 || c.n_head == 0 || c.n_head_kv == 0 || c.n_ff == 0 || c.max_ctx == 0)
     return fail(ctx, OGM_ERR_INVALID, "empty model dimension");
   const uint32_t gq = c.n_head % c.n_head_kv == 0 ? c.n_head / c.n_head_kv : 0;
-  if (gq != 1 && gq != 2 && gq != 4 && gq != 8)
-    return fail(ctx, OGM_ERR_UNSUPPORTED, "query heads per K/V head must be 1, 2, 4 or 8");
+  if (gq < 1 || gq > 8)
+    return fail(ctx, OGM_ERR_UNSUPPORTED, "query heads per K/V head must be 1 to 8");
+  if (c.rope_neox > 1) return fail(ctx, OGM_ERR_INVALID, "rope_neox is 0 (NORM pairs) or 1 (NEOX pairs)");
+  if (c.rope_freq_factors)
+    for (uint32_t i = 0; i < c.rope_dim / 2; i++)
+      if (!(c.rope_freq_factors[i] != 0.0f)) return fail(ctx, OGM_ERR_INVALID, "rope frequency factor of zero");
   if (c.head_dim != 64 && c.head_dim != 128) return fail(ctx, OGM_ERR_UNSUPPORTED, "head_dim must be 64 or 128");
   if (c.rope_dim > c.head_dim || c.rope_dim % 2 != 0) return fail(ctx, OGM_ERR_INVALID, "bad rope_dim");
   if (c.n_embd > 16384 || c.n_embd % 32 != 0 || c.n_ff % 32 != 0)
@@ -797,6 +802,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   ogm_llama *m = new (std::nothrow) ogm_llama();
   if (!m) return fail(ctx, OGM_ERR_OOM, "out of host memory");
   m->cfg = c;
+  m->cfg.rope_freq_factors = nullptr;   // folded into the frequency table below; the caller's array is not kept
   m->layers.assign(layers, layers + c.n_layer);
   m->output = output;
   m->max_splits = (c.max_ctx + OGM_ATTN_CHUNK - 1) / OGM_ATTN_CHUNK;
@@ -804,6 +810,8 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   int rc = OGM_OK;
   auto A = [&](void **p, size_t b) { if (rc == OGM_OK) rc = llama_alloc(ctx, m, p, b); };
   A((void **)&m->norms, ((size_t)c.n_layer * 2 + 1) * c.n_embd * 4);
+  const size_t pre_stride = (size_t)qd + 2 * (size_t)kvd + 2 * (size_t)c.head_dim;
+  A((void **)&m->pre, (size_t)c.n_layer * pre_stride * 4);
   A((void **)&m->freq, (size_t)(c.rope_dim / 2 + 1) * 4);
   A((void **)&m->rope_cs, (size_t)(c.rope_dim / 2 + 1) * 8);
   A((void **)&m->attn_tickets, (size_t)c.n_head_kv * 4);
@@ -833,11 +841,31 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
     memcpy(&host[((size_t)l * 2 + 1) * c.n_embd], layers[l].ffn_norm, (size_t)c.n_embd * 4);
   }
   memcpy(&host[(size_t)c.n_layer * 2 * c.n_embd], output_norm, (size_t)c.n_embd * 4);
-  // freq_i = base^(-2i / rope_dim), in f32 as tensor.rs:1147 computes it
+  // freq_i = base^(-2i / rope_dim) [/ factor_i], in f32 as tensor.rs:1147-1150 computes it
   std::vector<float> freq(c.rope_dim / 2 + 1, 0.0f);
-  for (uint32_t i = 0; i < c.rope_dim / 2; i++)
+  for (uint32_t i = 0; i < c.rope_dim / 2; i++) {
     freq[i] = powf(c.rope_freq_base, -2.0f * (float)i / (float)c.rope_dim);
+    if (c.rope_freq_factors) freq[i] /= c.rope_freq_factors[i];
+  }
+  // the optional per-layer vectors, side by side; the layer keeps a device pointer or null
+  std::vector<float> pre_host((size_t)c.n_layer * pre_stride, 0.0f);
+  for (uint32_t l = 0; l < c.n_layer; l++) {
+    ogm_llama_layer &D = m->layers[l];
+    float *hb = &pre_host[(size_t)l * pre_stride], *db = m->pre + (size_t)l * pre_stride;
+    const float **slot[5] = {&D.q_bias, &D.k_bias, &D.v_bias, &D.q_norm, &D.k_norm};
+    const size_t len[5] = {qd, kvd, kvd, c.head_dim, c.head_dim};
+    size_t off = 0;
+    for (int i = 0; i < 5; i++) {
+      if (*slot[i]) {
+        memcpy(hb + off, *slot[i], len[i] * 4);
+        *slot[i] = db + off;
+      }
+      off += len[i];
+    }
+    D.attn_norm = D.ffn_norm = nullptr;   // copied into m->norms
+  }
   hipError_t e = hipMemcpy(m->norms, host.data(), host.size() * 4, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(m->pre, pre_host.data(), pre_host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, (size_t)c.n_head_kv * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
@@ -888,6 +916,24 @@ extern "C" int ogm_llama_kv_write(ogm_ctx *ctx, ogm_llama *m, uint32_t layer, ui
   return OGM_OK;
 }
 
+extern "C" int ogm_llama_kv_read(ogm_ctx *ctx, ogm_llama *m, uint32_t layer, uint32_t pos0, uint32_t n_pos,
+                                 uint16_t *k_bits, uint16_t *v_bits) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !k_bits || !v_bits) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  const ogm_llama_config &c = m->cfg;
+  if (layer >= c.n_layer || (uint64_t)pos0 + n_pos > c.max_ctx)
+    return fail(ctx, OGM_ERR_INVALID, "layer or position range outside the cache");
+  if (n_pos == 0) return OGM_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  const size_t kvd = (size_t)c.n_head_kv * c.head_dim, bytes = (size_t)n_pos * kvd * 2;
+  const size_t row0 = ((size_t)layer * c.max_ctx + pos0) * kvd;
+  HIPCHK(ctx, hipMemcpy(k_bits, (const uint8_t *)m->k_cache + row0 * 2, bytes, hipMemcpyDeviceToHost));
+  HIPCHK(ctx, hipMemcpy(v_bits, (const uint8_t *)m->v_cache + row0 * 2, bytes, hipMemcpyDeviceToHost));
+  return OGM_OK;
+}
+
 // One matmul group of the step over the activations the previous kernel quantized.
 static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, hipStream_t s) {
   // weights of one type go out as one launch; a mixed group (Q4_K q/k with a Q6_K v) as several
@@ -932,7 +978,8 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     int rc = llama_matmul(ctx, w3, y3, 3, s);
     if (rc != OGM_OK) return rc;
     const int mode_o = act_mode_for(L.wo->ggml_type);
-    HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, m->rope_cs, c.rope_dim, kc, vc, pos, m->max_splits,
+    const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
+    HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, m->rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
                                        c.n_head, c.n_head_kv, c.head_dim, scale, m->part_o, m->part_ml,
                                        m->attn_tickets, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s));
     const ogm_weight *w1[1] = {L.wo};

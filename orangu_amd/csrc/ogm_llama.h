@@ -17,25 +17,38 @@ hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const f
                                  float eps, float *normed, OgmActDev act, hipStream_t stream);
 
 // cos / sin of pos * freq[p] for the rope_dim / 2 rotated pairs, as float2 (cos, sin): once per
-// token, every layer rotates by the same angles (tensor.rs:1147-1160, freq_scale 1, no YaRN).
+// token, every layer rotates by the same angles (tensor.rs:1147-1160, freq_scale 1, no YaRN;
+// `freq` already holds base^(-2p / rope_dim) divided by the pair's frequency factor).
 hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t rope_dim, void *cs, hipStream_t stream);
+
+// What a layer applies to its projections before they meet (engine/arch/llama.rs:757-810): the
+// projection biases (Qwen2), then the per-head RMSNorm of q and k (Qwen3), then RoPE in the
+// architecture's pairing.  Null pointers mean "the file has no such tensor".
+struct OgmAttnPre {
+  const float *q_bias, *k_bias, *v_bias;   // [n_head * head_dim], [kv_dim], [kv_dim]
+  const float *q_norm, *k_norm;            // [head_dim] each
+  float eps;                               // of the per-head norms
+  uint32_t neox;                           // 0: pairs (2i, 2i+1); 1: pairs (i, i + rope_dim / 2)
+};
 
 // One token's attention, from the q / k / v the projections left (f32) to the quantized input of
 // the output projection:
-//   * NORM-paired RoPE (pairs 2i, 2i+1; tensor.rs:1115-1177) of q and k with the table `cs`,
-//     k and v rounded to f16 into the cache rows of position `pos`;
+//   * bias, per-head norm and RoPE (tensor.rs:1233-1240, 691-706, 1115-1177) of q and k with the
+//     table `cs`, k and v rounded to f16 into the cache rows of position `pos`;
 //   * causal attention over cache positions 0..pos (engine/attention.rs:426-549): scores =
 //     (q . k) * scale, softmax over positions, out = sum w * v; grouped-query heads share their
-//     K/V head.  Split over chunks of OGM_ATTN_CHUNK positions and merged;
+//     K/V head (1 to 8 query heads per K/V head).  Split over chunks of OGM_ATTN_CHUNK positions
+//     and merged;
 //   * the merged output quantized for the next matmul in `mode`, and stored as f32 when attn_out
 //     is not null.
 // part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch;
 // counters: n_head_kv words, zero before the first launch (the kernel leaves them zero).
 hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
-                                  uint32_t rope_dim, void *k_cache_layer, void *v_cache_layer, uint32_t pos,
-                                  uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
-                                  float scale, float *part_o, float *part_ml, uint32_t *counters, int mode,
-                                  float *attn_out, OgmActDev act, hipStream_t stream);
+                                  uint32_t rope_dim, const OgmAttnPre &pre, void *k_cache_layer,
+                                  void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
+                                  uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
+                                  float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
+                                  hipStream_t stream);
 
 // h = silu(gate) * up with silu(g) = g / (1 + exp(-g))     (tensor.rs:825-827, arch/mod.rs:1071-1106)
 // quantized for the down projection in `mode`; h (f32) is also stored when not null.

@@ -199,6 +199,7 @@ template <int HD, int G, int GROUP>
 __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
                                                        const float *__restrict__ v_new,
                                                        const float2 *__restrict__ cs, uint32_t rope_half,
+                                                       OgmAttnPre pre, uint32_t gq,
                                                        __half *__restrict__ kc, __half *__restrict__ vc,
                                                        uint32_t pos, uint32_t max_splits, uint32_t n_head_kv,
                                                        float scale, float *part_o, float *part_ml,
@@ -242,26 +243,70 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
   for (int st = 0; st < STEPS; st++)
     vr[st] = *(const uint4 *)(vbase + (size_t)min((uint32_t)(st * ROWS) + rr, n_here - 1u) * kv_dim);
 
-  // ---- RoPE of q (and of the new k), cache rows of the current position
-  for (uint32_t i = tid; i < (uint32_t)(G * HD / 2); i += NT) {
-    const uint32_t g = i / (HD / 2), p = i - g * (HD / 2);
-    float2 ab = *(const float2 *)(q + (size_t)(kvh * G + g) * HD + 2u * p);
-    if (p < rope_half) ab = rope_pair(ab, cs[p]);
-    *(float2 *)&qs[g][2u * p] = ab;
-  }
-  if (is_last) {
-    if (tid < HD / 2) {
-      float2 ab = *(const float2 *)(k_new + (size_t)kvh * HD + 2u * tid);
-      if (tid < rope_half) ab = rope_pair(ab, cs[tid]);
-      const __half2 h = __floats2half2_rn(ab.x, ab.y);
-      *(__half2 *)&kcur[2u * tid] = h;
-      *(__half2 *)(kc + (size_t)pos * kv_dim + kvh * HD + 2u * tid) = h;
-    } else if (tid >= 64u && tid < 64u + HD / 2) {
-      const uint32_t p = tid - 64u;
-      const float2 ab = *(const float2 *)(v_new + (size_t)kvh * HD + 2u * p);
-      const __half2 h = __floats2half2_rn(ab.x, ab.y);
-      *(__half2 *)&vcur[2u * p] = h;
-      *(__half2 *)(vc + (size_t)pos * kv_dim + kvh * HD + 2u * p) = h;
+  // ---- bias, per-head norm and RoPE: one wave per query head; in the workgroup of the last chunk
+  // two more take the new k and v rows, which also go to the cache.  G counts the head slots of the
+  // kernel, gq <= G the query heads the model has per K/V head: the other slots hold zeros and
+  // store nothing.
+  {
+    constexpr int PPL = (HD / 2 + 63) / 64;   // pairs per lane
+    const uint32_t n_units = (uint32_t)G + (is_last ? 2u : 0u);
+    for (uint32_t u = wave; u < n_units; u += NW) {
+      const bool is_q = u < (uint32_t)G, is_v = u == (uint32_t)G + 1u;
+      const bool live = !is_q || u < gq;
+      const size_t row = (is_q ? (size_t)kvh * gq + u : (size_t)kvh) * HD;
+      const float *src = (is_q ? q : is_v ? v_new : k_new) + row;
+      const float *bias = is_q ? pre.q_bias : is_v ? pre.v_bias : pre.k_bias;
+      const float *nw = is_q ? pre.q_norm : is_v ? nullptr : pre.k_norm;
+      float a[PPL], b[PPL];
+      uint32_t ia[PPL], ib[PPL];
+      float ss = 0.0f;
+#pragma unroll
+      for (int j = 0; j < PPL; j++) {
+        const uint32_t p = lane + 64u * j;
+        const bool have = p < (uint32_t)(HD / 2) && live;
+        const bool split_pair = pre.neox != 0u && !is_v && p < rope_half;
+        ia[j] = split_pair ? p : 2u * p;
+        ib[j] = split_pair ? p + rope_half : 2u * p + 1u;
+        a[j] = have ? src[ia[j]] : 0.0f;
+        b[j] = have ? src[ib[j]] : 0.0f;
+        if (bias != nullptr && have) {
+          a[j] += bias[row + ia[j]];
+          b[j] += bias[row + ib[j]];
+        }
+        ss += a[j] * a[j] + b[j] * b[j];
+      }
+      if (nw != nullptr) {
+#pragma unroll
+        for (int k = 1; k < 64; k <<= 1) ss += __shfl_xor(ss, k, 64);
+        const float sc_n = 1.0f / sqrtf(ss / (float)HD + pre.eps);
+#pragma unroll
+        for (int j = 0; j < PPL; j++) {
+          const uint32_t p = lane + 64u * j;
+          if (p < (uint32_t)(HD / 2)) {
+            a[j] = a[j] * sc_n * nw[ia[j]];
+            b[j] = b[j] * sc_n * nw[ib[j]];
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < PPL; j++) {
+        const uint32_t p = lane + 64u * j;
+        if (p >= (uint32_t)(HD / 2)) continue;
+        float2 ab = make_float2(a[j], b[j]);
+        if (!is_v && p < rope_half) ab = rope_pair(ab, cs[p]);
+        if (is_q) {
+          qs[u][ia[j]] = ab.x;
+          qs[u][ib[j]] = ab.y;
+        } else {
+          const __half ha = __float2half_rn(ab.x), hb = __float2half_rn(ab.y);
+          __half *lds = is_v ? vcur : kcur;
+          __half *cache = (is_v ? vc : kc) + (size_t)pos * kv_dim + kvh * HD;
+          lds[ia[j]] = ha;
+          lds[ib[j]] = hb;
+          cache[ia[j]] = ha;
+          cache[ib[j]] = hb;
+        }
+      }
     }
   }
   // The cache loads requested above must stay up there: without this the row substitutions
@@ -349,14 +394,14 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
     if (lane < 4u && owner) red[1][g0 + i][wave] = l;
   }
   __syncthreads();
-  if (tid < G) {
+  if (tid < gq) {
     float m = red[0][tid][0], l = red[1][tid][0];
 #pragma unroll
     for (int w = 1; w < NW; w++) {
       m = fmaxf(m, red[0][tid][w]);
       l += red[1][tid][w];
     }
-    const uint32_t h = kvh * G + tid;
+    const uint32_t h = kvh * gq + tid;
     st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2], m);
     st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2 + 1], l);
   }
@@ -413,7 +458,7 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
       float t = 0.0f;
 #pragma unroll
       for (int w = 0; w < NW; w++) t += osum[w][g][d];
-      st_one<GROUP != 0>(&part_o[((size_t)(kvh * G + g) * max_splits + split) * HD + d], t);
+      if (g < gq) st_one<GROUP != 0>(&part_o[((size_t)(kvh * gq + g) * max_splits + split) * HD + d], t);
     }
   }
 
@@ -495,10 +540,11 @@ __global__ __launch_bounds__(64) void ogm_attn_combine_quant_kernel(const float 
 }
 
 hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
-                                  uint32_t rope_dim, void *k_cache_layer, void *v_cache_layer, uint32_t pos,
-                                  uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
-                                  float scale, float *part_o, float *part_ml, uint32_t *counters, int mode,
-                                  float *attn_out, OgmActDev act, hipStream_t stream) {
+                                  uint32_t rope_dim, const OgmAttnPre &pre, void *k_cache_layer,
+                                  void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
+                                  uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
+                                  float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
+                                  hipStream_t stream) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0) return hipErrorInvalidValue;
   if (rope_dim > head_dim || rope_dim % 2u != 0) return hipErrorInvalidValue;
   const uint32_t n_splits = pos / OGM_ATTN_CHUNK + 1u;
@@ -506,14 +552,18 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
   const uint32_t n = n_head * head_dim;
   if (n % 32u != 0) return hipErrorInvalidValue;
   const dim3 grid(n_head_kv, n_splits);
-  const uint32_t G = n_head / n_head_kv;
+  const uint32_t gq = n_head / n_head_kv;
+  if (gq > 8u) return hipErrorInvalidValue;
+  const uint32_t G = gq <= 2u ? gq : (gq <= 4u ? 4u : 8u);   // head slots of the kernel
   const uint32_t group = mode == 0 ? 32u : 256u;
-  // the merge rides in the attention kernel when a K/V head's outputs are whole quantizer groups
-  const uint32_t fused = (G * head_dim) % group == 0 ? group : 0u;
+  // the merge rides in the attention kernel when every head slot is a head and a K/V head's
+  // outputs are whole quantizer groups
+  const uint32_t fused = (G == gq && (G * head_dim) % group == 0) ? group : 0u;
 #define OGM_ATTN_LAUNCH(HD_, G_, GR_)                                                                  \
   hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, GR_>), grid, dim3(512), 0, stream, q, k_new, v_new,      \
-                     (const float2 *)cs, rope_dim / 2u, (__half *)k_cache_layer, (__half *)v_cache_layer, \
-                     pos, max_splits, n_head_kv, scale, part_o, part_ml, counters, attn_out, act)
+                     (const float2 *)cs, rope_dim / 2u, pre, gq, (__half *)k_cache_layer,               \
+                     (__half *)v_cache_layer, pos, max_splits, n_head_kv, scale, part_o, part_ml,       \
+                     counters, attn_out, act)
 #define OGM_ATTN_GROUPS(HD_, G_)                                \
   do {                                                          \
     if (fused == 32u) OGM_ATTN_LAUNCH(HD_, G_, 32);             \

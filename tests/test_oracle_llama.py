@@ -57,6 +57,56 @@ def test_rope_reference_case_and_invariants():
     np.testing.assert_allclose(ab, R.rope_norm(y, 4, 16, 7, 16, 10000.0), atol=2e-6)
 
 
+def test_rope_neox_pairs_and_frequency_factors():
+    # tensor.rs:1731-1749: [1..8], one head of 8, position 3, NEOX: pair p is elements p and p + 4
+    x = np.arange(1, 9, dtype=f32)
+    want = x.astype(np.float64).copy()
+    for p in range(4):
+        theta = 3.0 * float(f32(10000.0) ** f32(-2.0 * p / 8.0))
+        a, b = want[p], want[p + 4]
+        want[p], want[p + 4] = a * math.cos(theta) - b * math.sin(theta), a * math.sin(theta) + b * math.cos(theta)
+    got = R.rope(x, 1, 8, 3, 8, 10000.0, neox=True)
+    np.testing.assert_allclose(got, want, atol=1e-6)
+    assert not np.array_equal(got, R.rope(x, 1, 8, 3, 8, 10000.0))        # :1771-1776: the layouts differ
+    # NEOX with rope_dim < head_dim: pairs (i, i + rope_dim/2), the tail is left alone
+    y = np.random.default_rng(5).standard_normal(2 * 16).astype(f32)
+    r = R.rope(y, 2, 16, 9, 8, 10000.0, neox=True).reshape(2, 16)
+    np.testing.assert_array_equal(r[:, 8:], y.reshape(2, 16)[:, 8:])
+    np.testing.assert_allclose(r[:, :4] ** 2 + r[:, 4:8] ** 2, y.reshape(2, 16)[:, :4] ** 2 + y.reshape(2, 16)[:, 4:8] ** 2,
+                               rtol=1e-5)
+    # tensor.rs:1785-1822: a factor of 32 turns pair 1 of a 4-wide rotation 32 times slower, in
+    # both layouts; a factor of 1 is the same bits as no factors
+    for neox, a_slot in ((True, 1), (False, 2)):
+        def angle(ff):
+            e = np.zeros(4, f32)
+            e[a_slot] = 1.0
+            return float(R.rope(e, 1, 4, 1, 4, 10000.0, ff, neox)[3])
+        plain, slowed = angle(None), angle(np.array([1.0, 32.0], f32))
+        assert plain > 0 and slowed > 0 and abs(plain / slowed - 32.0) < 1e-2
+        assert angle(np.array([1.0, 1.0], f32)) == plain
+    # both layouts keep the energy of the rotated block (:1825-1841)
+    z = np.array([1.0, -2.0, 3.0, 4.0, -5.0, 6.0, 7.0, -8.0], f32)
+    for neox in (False, True):
+        np.testing.assert_allclose((R.rope(z, 1, 8, 7, 8, 10000.0, neox=neox) ** 2).sum(), (z ** 2).sum(), rtol=1e-6)
+
+
+def test_head_rmsnorm_and_biases_in_the_step():
+    # per-head norm = rmsnorm of each head_dim row with one weight vector (llama.rs:770-787)
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal(3 * 8).astype(f32)
+    w = rng.uniform(0.5, 1.5, 8).astype(f32)
+    got = R.head_rmsnorm(x, w, 3, 8, 1e-6).reshape(3, 8)
+    for h in range(3):
+        row = x.reshape(3, 8)[h].astype(np.float64)
+        np.testing.assert_allclose(got[h], row / np.sqrt((row ** 2).mean() + 1e-6) * w, rtol=1e-6)
+    # scaling one head leaves the others' outputs alone and (eps aside) its own too
+    x2 = x.copy().reshape(3, 8)
+    x2[1] *= 7.0
+    got2 = R.head_rmsnorm(x2.reshape(-1), w, 3, 8, 1e-12).reshape(3, 8)
+    np.testing.assert_array_equal(got2[0], R.head_rmsnorm(x, w, 3, 8, 1e-12).reshape(3, 8)[0])
+    np.testing.assert_allclose(got2[1], R.head_rmsnorm(x, w, 3, 8, 1e-12).reshape(3, 8)[1], rtol=1e-5)
+
+
 def test_softmax_silu_argmax():
     s = R.softmax(np.array([1.0, 2.0, 3.0], f32))           # tensor.rs:1612-1619
     assert abs(float(s.sum()) - 1.0) < 1e-6 and s[0] < s[1] < s[2]
@@ -133,3 +183,33 @@ def test_decode_step_wiring_on_a_tiny_model():
     # a decode out of order is refused
     with pytest.raises(AssertionError):
         R.decode_step(m, x0, 5)
+
+
+def test_first_position_sees_only_v_and_its_bias():
+    """With one cached position the softmax weight is 1 whatever q and k are: the logits at
+    position 0 do not move with the q / k biases, the per-head norms, the pairing or the frequency
+    factors, and do move with the v bias; at position 1 the q / k side matters."""
+    from helpers import Q4_K, Q6_K, synth_weights
+    import dataclasses
+    rng = np.random.default_rng(8)
+    n_embd, n_head, n_kv, hd, n_ff, n_vocab = 256, 4, 2, 64, 256, 64
+    mk = lambda t, i, o, s: (t, synth_weights(t, i, o, seed=s), i, o)
+    base = R.Layer(mk(Q4_K, n_embd, n_head * hd, 1), mk(Q4_K, n_embd, n_kv * hd, 2), mk(Q6_K, n_embd, n_kv * hd, 3),
+                   mk(Q4_K, n_head * hd, n_embd, 4), mk(Q4_K, n_embd, n_ff, 5), mk(Q4_K, n_embd, n_ff, 6),
+                   mk(Q6_K, n_ff, n_embd, 7), np.ones(n_embd, f32), np.ones(n_embd, f32))
+    qk = dict(q_bias=rng.standard_normal(n_head * hd).astype(f32), k_bias=rng.standard_normal(n_kv * hd).astype(f32),
+              q_norm=rng.uniform(0.5, 2, hd).astype(f32), k_norm=rng.uniform(0.5, 2, hd).astype(f32))
+
+    def run(layer, **kw):
+        m = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 10000.0, [layer], np.ones(n_embd, f32),
+                    mk(Q6_K, n_embd, n_vocab, 9), **kw)
+        x0, x1 = np.random.default_rng(9).standard_normal((2, n_embd)).astype(f32)
+        return R.decode_step(m, x0, 0)[0], R.decode_step(m, x1, 1)[0]
+
+    plain0, plain1 = run(base)
+    other0, other1 = run(dataclasses.replace(base, **qk), rope_neox=True,
+                         rope_freq_factors=np.linspace(1, 8, hd // 2).astype(f32))
+    np.testing.assert_array_equal(other0, plain0)
+    assert not np.array_equal(other1, plain1)
+    vb0, _ = run(dataclasses.replace(base, v_bias=np.full(n_kv * hd, 0.5, f32)))
+    assert not np.array_equal(vb0, plain0)
