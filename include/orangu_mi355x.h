@@ -296,6 +296,19 @@ int ogm_gguf_matrix(ogm_gguf *g, const char *name, uint32_t *ggml_type, uint32_t
 /* ogm_gguf_matrix + ogm_weight_upload, keyed by the mapped bytes' address and length. */
 int ogm_gguf_upload_matrix(ogm_ctx *ctx, ogm_gguf *g, const char *name, ogm_weight **out);
 
+/* A Llama-style file (general.architecture llama, mistral, qwen2, qwen3 or qwen3vl: loader.rs:190) as a
+ * device-resident decoder: the hyperparameters as read_model_config derives them (loader.rs:1652-1714:
+ * head_count_kv defaults to head_count, key_length to embedding_length / head_count,
+ * rope.dimension_count to the head width, freq_base to 10000, the epsilon to 1e-5, vocab_size to the
+ * token list's length), the tensors LlamaModel::load_with_backend takes (llama.rs:123-220: output.weight
+ * falls back to token_embd.weight, the bias / per-head-norm / rope_freqs tensors are optional), the
+ * pairing rope_layout_for gives the architecture.  Every matrix goes through ogm_gguf_upload_matrix
+ * (the context keeps them); *tok_embd (nullable) receives the embedding matrix for
+ * ogm_llama_generate / ogm_dequant_rows, *cfg_out (nullable) the configuration used.  Errors are
+ * reported through ogm_gguf_last_error. */
+int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama **model,
+                        const ogm_weight **tok_embd, ogm_llama_config *cfg_out);
+
 /* ---- tuning / introspection ------------------------------------------------------------------ */
 
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.

@@ -274,10 +274,12 @@ class Mi355xBackend:
         """Releases a device copy made by upload_raw (cached uploads live as long as the backend)."""
         self._check(self._lib.ogm_weight_free(self._ctx, w_handle), "ogm_weight_free")
 
-    def dequant_rows(self, w: QuantMatrix, row0: int, n_rows: int) -> np.ndarray:
-        """Rows of an uploaded matrix as f32, from the device copy (quant.rs dequantize_*)."""
-        out = np.empty((n_rows, w.in_dim), np.float32)
-        self._check(self._lib.ogm_dequant_rows(self._ctx, self.upload(w), row0, n_rows, out.ctypes.data),
+    def dequant_rows(self, w, row0: int, n_rows: int, in_dim: int | None = None) -> np.ndarray:
+        """Rows of an uploaded matrix (a QuantMatrix, or a handle together with its in_dim) as f32,
+        from the device copy (quant.rs dequantize_*)."""
+        handle = w if isinstance(w, int) else self.upload(w)
+        out = np.empty((n_rows, in_dim if isinstance(w, int) else w.in_dim), np.float32)
+        self._check(self._lib.ogm_dequant_rows(self._ctx, handle, row0, n_rows, out.ctypes.data),
                     "ogm_dequant_rows")
         return out
 
@@ -339,6 +341,22 @@ class LlamaDecoder:
                   "ogm_llama_create")
         self._h = h.value
         self.n_embd, self.n_vocab, self.kv_dim, self.n_layer = n_embd, n_vocab, n_head_kv * head_dim, len(layers)
+
+    @classmethod
+    def from_gguf(cls, be: "Mi355xBackend", gguf, max_ctx: int) -> "LlamaDecoder":
+        """The decoder of a Llama-style GGUF file (a ``GgufFile``), built by the library as
+        LlamaModel::load_with_backend builds the model (llama.rs:123-220).  ``tok_embd`` is the
+        uploaded embedding matrix's handle, for ``generate`` and ``Mi355xBackend.dequant_rows``."""
+        self = cls.__new__(cls)
+        self._be, self._keep = be, [gguf]
+        h, embd, cfg = C.c_void_p(), C.c_void_p(), capi.OgmLlamaConfig()
+        rc = be._lib.ogm_llama_load_gguf(be._ctx, gguf._h, max_ctx, C.byref(h), C.byref(embd), C.byref(cfg))
+        if rc != 0:
+            gguf._fail(rc, "ogm_llama_load_gguf")
+        self._h, self.tok_embd, self.config = h.value, embd.value, cfg
+        self.n_embd, self.n_vocab, self.n_layer = cfg.n_embd, cfg.n_vocab, cfg.n_layer
+        self.kv_dim = cfg.n_head_kv * cfg.head_dim
+        return self
 
     def kv_write(self, layer: int, pos0: int, k, v):
         k = np.ascontiguousarray(k, np.float32).reshape(-1, self.kv_dim)

@@ -454,3 +454,208 @@ extern "C" int ogm_gguf_upload_matrix(ogm_ctx *ctx, ogm_gguf *g, const char *nam
   if (rc != OGM_OK) g->err = std::string("tensor '") + name + "': " + ogm_last_error(ctx);
   return rc;
 }
+
+// ---- a Llama-family file as a device-resident decoder ---------------------------------------
+
+namespace {
+
+// A small tensor (norm weights, biases, frequency factors) as f32, as LoadedModel::tensor hands
+// it out (loader.rs:1512-1550): F32 as is, F16 and BF16 widened.
+int small_tensor_f32(ogm_gguf *g, const std::string &name, uint64_t want, bool at_least, std::vector<float> *out) {
+  const int64_t idx = ogm_gguf_find_tensor(g, name.c_str());
+  if (idx < 0) {
+    g->err = "model is missing tensor '" + name + "'";
+    return OGM_ERR_INVALID;
+  }
+  const Tensor &t = g->tensors[(size_t)idx];
+  const uint8_t *p;
+  uint64_t len;
+  int rc = tensor_bytes(g, t, &p, &len);
+  if (rc != OGM_OK) return rc;
+  uint64_t n = 1;
+  for (uint64_t d : t.dims) n *= d;
+  if (at_least ? n < want : n != want) {
+    g->err = "tensor '" + name + "' has " + std::to_string(n) + " entries, need " + std::to_string(want);
+    return OGM_ERR_INVALID;
+  }
+  out->resize((size_t)n);
+  if (t.ggml_type == 0) {
+    memcpy(out->data(), p, (size_t)n * 4);
+  } else if (t.ggml_type == 1 || t.ggml_type == 30) {
+    for (uint64_t i = 0; i < n; i++) {
+      uint16_t h;
+      memcpy(&h, p + 2 * i, 2);
+      uint32_t bits;
+      if (t.ggml_type == 30) {
+        bits = (uint32_t)h << 16;
+      } else {   // IEEE binary16 -> binary32, subnormals included (quant.rs:511-528)
+        const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, ex = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+        if (ex == 0) {
+          if (man == 0) {
+            bits = sign;
+          } else {
+            int e = -1;
+            uint32_t m = man;
+            do { m <<= 1; e++; } while ((m & 0x400u) == 0);
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((m & 0x3FFu) << 13);
+          }
+        } else if (ex == 31) {
+          bits = sign | 0x7F800000u | (man << 13);
+        } else {
+          bits = sign | ((ex + 112u) << 23) | (man << 13);
+        }
+      }
+      memcpy(&(*out)[(size_t)i], &bits, 4);
+    }
+  } else {
+    g->err = "tensor '" + name + "': ggml_type " + std::to_string(t.ggml_type) + " is not read as a vector here";
+    return OGM_ERR_UNSUPPORTED;
+  }
+  return OGM_OK;
+}
+
+bool meta_u64_of(const ogm_gguf *g, const std::string &key, uint64_t *out) {
+  return ogm_gguf_meta_u64(g, key.c_str(), out) == OGM_OK;
+}
+
+// metadata_f32 (loader.rs:1634-1645): only the float types count
+bool meta_f32_of(const ogm_gguf *g, const std::string &key, float *out) {
+  const Value *v = find_meta(g, key.c_str());
+  if (!v || (v->type != 6 && v->type != 12)) return false;
+  *out = (float)v->f;
+  return true;
+}
+
+}  // namespace
+
+extern "C" int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama **model,
+                                   const ogm_weight **tok_embd, ogm_llama_config *cfg_out) {
+  if (!ctx || !g || !model) return OGM_ERR_INVALID;
+  const char *arch_c = nullptr;
+  if (ogm_gguf_meta_string(g, "general.architecture", &arch_c, nullptr) != OGM_OK) {
+    g->err = "GGUF file is missing general.architecture";
+    return OGM_ERR_INVALID;
+  }
+  const std::string arch(arch_c);
+  // LLAMA_STYLE_ARCHITECTURES (loader.rs:190): what LlamaModel runs
+  static const char *const kLlamaStyle[] = {"llama", "qwen2", "qwen3", "mistral", "qwen3vl"};
+  bool ours = false;
+  for (const char *a : kLlamaStyle) ours = ours || arch == a;
+  if (!ours) {
+    g->err = "architecture '" + arch + "' is not a Llama-style one";
+    return OGM_ERR_UNSUPPORTED;
+  }
+  // read_model_config (loader.rs:1652-1714)
+  uint64_t n_embd, n_layer, n_head, n_head_kv, n_vocab, head_dim, rope_dim;
+  struct { const char *suffix; uint64_t *dst; } required[] = {
+      {"embedding_length", &n_embd}, {"block_count", &n_layer}, {"attention.head_count", &n_head}};
+  for (auto &r : required)
+    if (!meta_u64_of(g, arch + "." + r.suffix, r.dst)) {
+      g->err = "GGUF file is missing " + arch + "." + r.suffix;
+      return OGM_ERR_INVALID;
+    }
+  if (!meta_u64_of(g, arch + ".attention.head_count_kv", &n_head_kv)) n_head_kv = n_head;
+  if (!meta_u64_of(g, arch + ".vocab_size", &n_vocab)) {
+    uint32_t et;
+    if (ogm_gguf_meta_array(g, "tokenizer.ggml.tokens", &et, &n_vocab) != OGM_OK) {
+      g->err = "GGUF file has no vocab_size and no tokenizer.ggml.tokens";
+      return OGM_ERR_INVALID;
+    }
+  }
+  if (n_head == 0 || n_head_kv == 0) {
+    g->err = arch + ".attention.head_count(_kv) must be nonzero";
+    return OGM_ERR_INVALID;
+  }
+  if (!meta_u64_of(g, arch + ".attention.key_length", &head_dim)) head_dim = n_embd / n_head;
+  if (head_dim == 0) {
+    g->err = arch + ".attention.key_length must be nonzero";
+    return OGM_ERR_INVALID;
+  }
+  if (!meta_u64_of(g, arch + ".rope.dimension_count", &rope_dim)) rope_dim = head_dim;
+  float freq_base = 10000.0f, rms_eps = 1e-5f;
+  (void)meta_f32_of(g, arch + ".rope.freq_base", &freq_base);
+  (void)meta_f32_of(g, arch + ".attention.layer_norm_rms_epsilon", &rms_eps);
+  if (n_layer == 0 || n_layer > 4096 || n_embd > UINT32_MAX || n_vocab > UINT32_MAX) {
+    g->err = "model dimensions out of range";
+    return OGM_ERR_INVALID;
+  }
+
+  // LlamaModel::load_with_backend (llama.rs:123-220)
+  ogm_weight *embd = nullptr, *output = nullptr;
+  int rc = ogm_gguf_upload_matrix(ctx, g, "token_embd.weight", &embd);
+  if (rc != OGM_OK) return rc;
+  if (ogm_gguf_find_tensor(g, "output.weight") >= 0) {
+    if ((rc = ogm_gguf_upload_matrix(ctx, g, "output.weight", &output)) != OGM_OK) return rc;
+  } else {
+    output = embd;   // tied embeddings: the file omits output.weight
+  }
+  std::vector<float> output_norm;
+  if ((rc = small_tensor_f32(g, "output_norm.weight", n_embd, false, &output_norm)) != OGM_OK) return rc;
+  const uint64_t qd = n_head * head_dim, kvd = n_head_kv * head_dim;
+  std::vector<ogm_llama_layer> layers((size_t)n_layer);
+  std::vector<std::vector<float>> keep;   // the vectors the layer structs point into
+  keep.reserve((size_t)n_layer * 7 + 2);
+  uint32_t n_ff = 0;
+  for (uint64_t i = 0; i < n_layer; i++) {
+    const std::string blk = "blk." + std::to_string(i) + ".";
+    ogm_llama_layer &L = layers[(size_t)i];
+    memset(&L, 0, sizeof(L));
+    struct { const char *name; const ogm_weight **dst; } mats[] = {
+        {"attn_q.weight", &L.wq}, {"attn_k.weight", &L.wk}, {"attn_v.weight", &L.wv},
+        {"attn_output.weight", &L.wo}, {"ffn_gate.weight", &L.w_gate}, {"ffn_up.weight", &L.w_up},
+        {"ffn_down.weight", &L.w_down}};
+    for (auto &mt : mats) {
+      ogm_weight *w = nullptr;
+      if ((rc = ogm_gguf_upload_matrix(ctx, g, (blk + mt.name).c_str(), &w)) != OGM_OK) return rc;
+      *mt.dst = w;
+    }
+    if (i == 0) {
+      uint32_t t, in_dim, out_dim;
+      if ((rc = ogm_gguf_matrix(g, (blk + "ffn_gate.weight").c_str(), &t, &in_dim, &out_dim, nullptr, nullptr)) != OGM_OK)
+        return rc;
+      n_ff = out_dim;
+    }
+    struct { const char *name; const float **dst; uint64_t n; bool optional; } vecs[] = {
+        {"attn_norm.weight", &L.attn_norm, n_embd, false}, {"ffn_norm.weight", &L.ffn_norm, n_embd, false},
+        {"attn_q.bias", &L.q_bias, qd, true},              {"attn_k.bias", &L.k_bias, kvd, true},
+        {"attn_v.bias", &L.v_bias, kvd, true},             {"attn_q_norm.weight", &L.q_norm, head_dim, true},
+        {"attn_k_norm.weight", &L.k_norm, head_dim, true}};
+    for (auto &v : vecs) {
+      if (v.optional && ogm_gguf_find_tensor(g, (blk + v.name).c_str()) < 0) continue;
+      keep.emplace_back();
+      if ((rc = small_tensor_f32(g, blk + v.name, v.n, false, &keep.back())) != OGM_OK) return rc;
+      *v.dst = keep.back().data();
+    }
+  }
+  // rope_freqs.weight (llama.rs:186-201): at least rope_dim / 2 entries
+  std::vector<float> factors;
+  const bool has_factors = ogm_gguf_find_tensor(g, "rope_freqs.weight") >= 0;
+  if (has_factors && (rc = small_tensor_f32(g, "rope_freqs.weight", rope_dim / 2, true, &factors)) != OGM_OK) return rc;
+
+  ogm_llama_config cfg;
+  memset(&cfg, 0, sizeof(cfg));
+  cfg.n_layer = (uint32_t)n_layer;
+  cfg.n_embd = (uint32_t)n_embd;
+  cfg.n_head = (uint32_t)n_head;
+  cfg.n_head_kv = (uint32_t)n_head_kv;
+  cfg.head_dim = (uint32_t)head_dim;
+  cfg.n_ff = n_ff;
+  cfg.n_vocab = (uint32_t)n_vocab;
+  cfg.rope_dim = (uint32_t)rope_dim;
+  cfg.max_ctx = max_ctx;
+  cfg.rms_eps = rms_eps;
+  cfg.rope_freq_base = freq_base;
+  cfg.rope_neox = (arch == "llama" || arch == "mistral") ? 0u : 1u;   // rope_layout_for, llama.rs:115-120
+  cfg.rope_freq_factors = has_factors ? factors.data() : nullptr;
+  rc = ogm_llama_create(ctx, &cfg, layers.data(), output_norm.data(), output, model);
+  if (rc != OGM_OK) {
+    g->err = std::string("ogm_llama_create: ") + ogm_last_error(ctx);
+    return rc;
+  }
+  if (tok_embd) *tok_embd = embd;
+  if (cfg_out) {
+    *cfg_out = cfg;
+    cfg_out->rope_freq_factors = nullptr;   // the array above does not outlive this call
+  }
+  return OGM_OK;
+}

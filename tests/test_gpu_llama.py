@@ -331,6 +331,145 @@ def test_matrices_uploaded_from_a_gguf_file_multiply_like_direct_uploads(be, tmp
     g.close()
 
 
+def model_gguf(ref, arch, *, n_ctx=4096, tok_embd=None, vec_type=0, omit=(), extra_kvs=(), explicit=True):
+    """A reference model as the bytes of a GGUF file with the tensor names and metadata keys
+    LlamaModel::load_with_backend and read_model_config read (llama.rs:123-220, loader.rs:1652-1714).
+    vec_type 0 stores the vectors as F32, 1 as F16."""
+    from test_gguf_cpu import gguf, gstr, kv, tensor_info, u32, u64
+    f32kv = lambda k, v: kv(f"{arch}.{k}", 6, np.float32(v).tobytes())
+    u32kv = lambda k, v: kv(f"{arch}.{k}", 4, u32(v))
+    kvs = [kv("general.architecture", 8, gstr(arch)), u32kv("embedding_length", ref.n_embd),
+           u32kv("block_count", len(ref.layers)), u32kv("attention.head_count", ref.n_head),
+           u32kv("context_length", n_ctx), f32kv("rope.freq_base", ref.rope_freq_base),
+           f32kv("attention.layer_norm_rms_epsilon", ref.rms_eps)]
+    if explicit:   # otherwise the loader's defaults must give the same model
+        kvs += [u32kv("attention.head_count_kv", ref.n_head_kv), u32kv("attention.key_length", ref.head_dim),
+                u32kv("rope.dimension_count", ref.rope_dim), u32kv("vocab_size", ref.n_vocab)]
+    else:
+        kvs.append(kv("tokenizer.ggml.tokens", 9, u32(8) + u64(ref.n_vocab) + b"".join(gstr("t%d" % i) for i in range(ref.n_vocab))))
+    kvs += list(extra_kvs)
+    tensors = []
+
+    def mat(name, w):
+        t, raw, n_in, n_out = w
+        tensors.append((name, [n_in, n_out], t, np.ascontiguousarray(raw).tobytes()))
+
+    def vec(name, a):
+        a = np.asarray(a, f32)
+        tensors.append((name, [a.size], vec_type, (a if vec_type == 0 else a.astype(np.float16)).tobytes()))
+
+    mat("token_embd.weight", tok_embd if tok_embd is not None else ref.output)
+    if tok_embd is not None:
+        mat("output.weight", ref.output)
+    vec("output_norm.weight", ref.output_norm)
+    if ref.rope_freq_factors is not None:
+        vec("rope_freqs.weight", ref.rope_freq_factors)
+    for i, L in enumerate(ref.layers):
+        for name, field in (("attn_q", "wq"), ("attn_k", "wk"), ("attn_v", "wv"), ("attn_output", "wo"),
+                            ("ffn_gate", "w_gate"), ("ffn_up", "w_up"), ("ffn_down", "w_down")):
+            mat(f"blk.{i}.{name}.weight", getattr(L, field))
+        for name, field in (("attn_norm.weight", "attn_norm"), ("ffn_norm.weight", "ffn_norm"), ("attn_q.bias", "q_bias"),
+                            ("attn_k.bias", "k_bias"), ("attn_v.bias", "v_bias"), ("attn_q_norm.weight", "q_norm"),
+                            ("attn_k_norm.weight", "k_norm")):
+            if getattr(L, field) is not None:
+                vec(f"blk.{i}.{name}", getattr(L, field))
+    tensors = [t for t in tensors if t[0] not in omit]
+    infos, blobs, pos = [], [], 0
+    for name, dims, t, data in tensors:
+        infos.append(tensor_info(name, dims, t, pos))
+        blobs.append(data + b"\0" * ((-len(data)) % 32))
+        pos += len(blobs[-1])
+    return gguf(kvs, infos, data=b"".join(blobs))[0]
+
+
+def f16_exact(ref):
+    """Rounds every vector of the model to f16 values, so that a file storing them as F16 holds
+    the same model."""
+    r16 = lambda a: None if a is None else np.asarray(a, f32).astype(np.float16).astype(f32)
+    ref.output_norm = r16(ref.output_norm)
+    ref.rope_freq_factors = r16(ref.rope_freq_factors)
+    for L in ref.layers:
+        for field in ("attn_norm", "ffn_norm", "q_bias", "k_bias", "v_bias", "q_norm", "k_norm"):
+            setattr(L, field, r16(getattr(L, field)))
+
+
+@pytest.mark.parametrize("arch,pre,ff,vec_type,explicit,tied", [
+    ("llama", (), True, 0, True, False),                                   # Llama-3.1-like: NORM pairs, rope_freqs
+    ("mistral", (), False, 1, False, True),                                # defaults, tied embeddings, F16 vectors
+    ("qwen2", ("q_bias", "k_bias", "v_bias"), False, 0, True, True),       # NEOX pairs, biases
+    ("qwen3", ("q_norm", "k_norm"), False, 1, True, False),                # per-head norms
+])
+def test_a_gguf_file_decodes_like_the_model_it_holds(be, tmp_path, arch, pre, ff, vec_type, explicit, tied):
+    """ogm_llama_load_gguf: hyperparameters, tensors, pairing and optional tensors as
+    read_model_config and LlamaModel::load_with_backend take them from the file."""
+    from orangu_amd import LlamaDecoder
+    from orangu_amd.gguf import GgufFile
+    n_head, n_kv, hd = (4, 4, 64) if not explicit else (8, 2, 64)   # the defaults: n_kv = n_head, head_dim = n_embd / n_head
+    n_embd = 256 if not explicit else 512
+    neox = arch not in ("llama", "mistral")
+    factors = np.linspace(1.0, 4.0, hd // 2).astype(f32) if ff else None
+    ref, dev0, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=320, n_layer=2,
+                           types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=8, seed=31 + len(pre), pre=pre, neox=neox,
+                           freq_factors=factors)
+    dev0.close()
+    if vec_type == 1:
+        f16_exact(ref)
+    embd = None if tied else (Q8_0, synth_weights(Q8_0, n_embd, 320, seed=77), n_embd, 320)
+    path = tmp_path / f"{arch}.gguf"
+    path.write_bytes(model_gguf(ref, arch, tok_embd=embd, vec_type=vec_type, explicit=explicit))
+    g = GgufFile(str(path))
+    dev = LlamaDecoder.from_gguf(be, g, max_ctx=8)
+    try:
+        c = dev.config
+        assert (c.n_layer, c.n_embd, c.n_head, c.n_head_kv, c.head_dim, c.n_ff, c.n_vocab, c.rope_dim, c.rope_neox) == \
+               (2, n_embd, n_head, n_kv, hd, 512, 320, hd, int(neox))
+        for pos in range(3):
+            step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"{arch} file pos {pos}")
+        # the embedding matrix handed back is the file's token_embd (the output matrix when tied)
+        import oracle
+        t, raw, _, _ = embd if embd is not None else ref.output
+        want = oracle.dequantize(t, raw, 320 * n_embd).reshape(320, n_embd)[5:7]
+        assert np.array_equal(be.dequant_rows(dev.tok_embd, 5, 2, in_dim=n_embd).view(np.uint32), want.view(np.uint32))
+    finally:
+        dev.close()
+        g.close()
+
+
+def test_gguf_model_loading_errors(be, tmp_path):
+    """The loader's refusals (loader.rs:312-380, 1647-1681; llama.rs:186-201) arrive as a status
+    and a message, not as a crash."""
+    from orangu_amd import LlamaDecoder, OgmError
+    from orangu_amd.gguf import GgufFile
+    from test_gguf_cpu import gstr, kv, u32
+    ref, dev0, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=1,
+                           types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=8, seed=41,
+                           freq_factors=np.ones(32, f32))
+    dev0.close()
+
+    def load(data):
+        g = GgufFile(data=data)
+        try:
+            LlamaDecoder.from_gguf(be, g, max_ctx=8).close()
+        finally:
+            g.close()
+
+    load(model_gguf(ref, "llama"))   # the file itself is fine
+    for what, data in [
+        ("not a Llama-style", model_gguf(ref, "gemma")),
+        ("missing tensor 'blk.0.ffn_up.weight'", model_gguf(ref, "llama", omit=("blk.0.ffn_up.weight",))),
+        ("missing tensor 'output_norm.weight'", model_gguf(ref, "llama", omit=("output_norm.weight",))),
+    ]:
+        with pytest.raises(OgmError, match=what):
+            load(data)
+    ref.rope_freq_factors = np.ones(8, f32)      # fewer than rope_dim / 2 entries
+    with pytest.raises(OgmError, match="rope_freqs.weight"):
+        load(model_gguf(ref, "llama"))
+    ref.rope_freq_factors = None
+    ref.n_head = 0                               # head_count must be nonzero
+    with pytest.raises(OgmError, match="nonzero"):
+        load(model_gguf(ref, "llama"))
+
+
 @pytest.mark.parametrize("t,in_dim,out_dim", [
     (Q8_0, 64, 5), (Q8_0, 4096, 70),
     (Q4_K, 256, 3), (Q4_K, 1024, 130), (Q4_K, 4096, 67),
