@@ -242,6 +242,18 @@ int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos, f
 /* The same with device pointers, enqueued on `stream` (null = the context's) without waiting. */
 int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_t pos, float *logits_dev,
                          uint32_t *argmax_dev, void *stream);
+/* Prefill: n_tokens embedding rows x ([n_tokens][n_embd], host f32) at positions pos0 .. pos0+n_tokens
+ * through run_layers at n_tokens > 1 (llama.rs:594-932): the matmuls in the GEMM kernels' float order
+ * (Backend::matmul, cpu.rs:445-458), K/V rows appended to the cache, causal attention; then the last
+ * row alone through the output norm and projection (forward, llama.rs:1007-1032).  last_logits
+ * ([n_vocab]) and argmax may each be null.  Runs in chunks of 512 tokens; synchronizes. */
+int ogm_llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos0, uint32_t n_tokens,
+                      float *last_logits, uint32_t *argmax);
+/* The same from token ids (host), their embedding rows read on the device from an uploaded
+ * [n_embd -> n_vocab] matrix (llama.rs:609-614). */
+int ogm_llama_prefill_tokens(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *tok_embd, const uint32_t *tokens,
+                             uint32_t pos0, uint32_t n_tokens, float *last_logits, uint32_t *argmax);
+
 /* Rows row0 .. row0+n_rows of an uploaded matrix as f32 ([n_rows][in_dim], host memory), from the
  * device copy: dequantize_q8_0 / _q4_k / _q6_k (engine/quant.rs:639-649, 666-697, 746-787), bit for
  * bit.  This is the embedding lookup of run_layers (llama.rs:609-614). */

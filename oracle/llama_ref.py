@@ -176,20 +176,28 @@ class Model:
         self.v_cache = [[] for _ in self.layers]
 
 
-def _mm(w: tuple, x: np.ndarray) -> np.ndarray:
+def _mm(w: tuple, x: np.ndarray, n_tokens: int = 1) -> np.ndarray:
+    """Backend::matmul (cpu.rs:445-458): the GEMV kernels at one token, the GEMM kernels above."""
     import oracle
     t, raw, in_dim, out_dim = w
-    return oracle.matmul(t, raw, in_dim, out_dim, np.ascontiguousarray(x, f32), 1).reshape(-1)
+    y = oracle.matmul(t, raw, in_dim, out_dim, np.ascontiguousarray(x, f32), n_tokens)
+    return y.reshape(-1) if n_tokens == 1 else y.reshape(n_tokens, out_dim)
 
 
-def decode_step(m: Model, x: np.ndarray, pos: int):
-    """llama.rs:594-932 + 1007-1032 for one token.  Returns (logits, final hidden state)."""
+def forward(m: Model, X: np.ndarray, pos0: int):
+    """llama.rs:594-932 + 1007-1032 for the tokens whose embedding rows are X [n_tokens][n_embd], at
+    positions pos0 ..: every matmul over all rows at once, K/V rows appended in order, token t
+    attending to cache rows 0 .. pos0 + t; the LAST row alone goes through the output norm and
+    projection.  Returns (logits of the last token, its final hidden state)."""
     if not m.k_cache:
         m.reset()
-    x = np.array(x, f32)
+    X = np.array(X, f32).reshape(-1, m.n_embd)
+    T = X.shape[0]
+    rows = lambda fn, A: np.stack([fn(A[t]) for t in range(T)])
+    mm = lambda w, A: _mm(w, A if T > 1 else A[0], T).reshape(T, -1)
     for li, L in enumerate(m.layers):
-        normed = rmsnorm(x, L.attn_norm, m.rms_eps)
-        q, k, v = _mm(L.wq, normed), _mm(L.wk, normed), _mm(L.wv, normed)
+        normed = rows(lambda r: rmsnorm(r, L.attn_norm, m.rms_eps), X)
+        q, k, v = mm(L.wq, normed), mm(L.wk, normed), mm(L.wv, normed)
         if L.q_bias is not None:                       # llama.rs:757-765
             q = (q + np.asarray(L.q_bias, f32)).astype(f32)
         if L.k_bias is not None:
@@ -197,23 +205,31 @@ def decode_step(m: Model, x: np.ndarray, pos: int):
         if L.v_bias is not None:
             v = (v + np.asarray(L.v_bias, f32)).astype(f32)
         if L.q_norm is not None:                       # llama.rs:770-787, before RoPE
-            q = head_rmsnorm(q, L.q_norm, m.n_head, m.head_dim, m.rms_eps)
+            q = rows(lambda r: head_rmsnorm(r, L.q_norm, m.n_head, m.head_dim, m.rms_eps), q)
         if L.k_norm is not None:
-            k = head_rmsnorm(k, L.k_norm, m.n_head_kv, m.head_dim, m.rms_eps)
-        q = rope(q, m.n_head, m.head_dim, pos, m.rope_dim, m.rope_freq_base, m.rope_freq_factors, m.rope_neox)
-        k = rope(k, m.n_head_kv, m.head_dim, pos, m.rope_dim, m.rope_freq_base, m.rope_freq_factors, m.rope_neox)
+            k = rows(lambda r: head_rmsnorm(r, L.k_norm, m.n_head_kv, m.head_dim, m.rms_eps), k)
         kc, vc = m.k_cache[li], m.v_cache[li]
-        assert len(kc) == pos, "decode positions must be appended in order"
-        k_row, v_row = k.astype(m.kv_dtype), v.astype(m.kv_dtype)
-        if m.kv_hook is not None:
-            k_row, v_row = m.kv_hook(li, pos, k_row, v_row)
-        kc.append(k_row)
-        vc.append(v_row)
-        attn = attention(q, np.stack(kc).astype(f32), np.stack(vc).astype(f32), m.n_head, m.n_head_kv, m.head_dim)
-        x = (x + _mm(L.wo, attn)).astype(f32)
-        normed2 = rmsnorm(x, L.ffn_norm, m.rms_eps)
-        gate, up = _mm(L.w_gate, normed2), _mm(L.w_up, normed2)
+        assert len(kc) == pos0, "positions must be appended in order"
+        attn = np.empty((T, m.n_head * m.head_dim), f32)
+        for t in range(T):                             # llama.rs:794-830: one row at a time, in order
+            pos = pos0 + t
+            qt = rope(q[t], m.n_head, m.head_dim, pos, m.rope_dim, m.rope_freq_base, m.rope_freq_factors, m.rope_neox)
+            kt = rope(k[t], m.n_head_kv, m.head_dim, pos, m.rope_dim, m.rope_freq_base, m.rope_freq_factors, m.rope_neox)
+            k_row, v_row = kt.astype(m.kv_dtype), v[t].astype(m.kv_dtype)
+            if m.kv_hook is not None:
+                k_row, v_row = m.kv_hook(li, pos, k_row, v_row)
+            kc.append(k_row)
+            vc.append(v_row)
+            attn[t] = attention(qt, np.stack(kc).astype(f32), np.stack(vc).astype(f32), m.n_head, m.n_head_kv, m.head_dim)
+        X = (X + mm(L.wo, attn)).astype(f32)
+        normed2 = rows(lambda r: rmsnorm(r, L.ffn_norm, m.rms_eps), X)
+        gate, up = mm(L.w_gate, normed2), mm(L.w_up, normed2)
         h = (silu(gate) * up).astype(f32)
-        x = (x + _mm(L.w_down, h)).astype(f32)
-    last = rmsnorm(x, m.output_norm, m.rms_eps)
-    return _mm(m.output, last), x
+        X = (X + mm(L.w_down, h)).astype(f32)
+    last = rmsnorm(X[-1], m.output_norm, m.rms_eps)
+    return _mm(m.output, last), X[-1]
+
+
+def decode_step(m: Model, x: np.ndarray, pos: int):
+    """One token: returns (logits, final hidden state)."""
+    return forward(m, np.asarray(x, f32).reshape(1, -1), pos)

@@ -383,6 +383,27 @@ class LlamaDecoder:
                                                        logits.ctypes.data, C.byref(am)), "ogm_llama_decode")
         return logits, am.value
 
+    def prefill(self, x, pos0: int = 0):
+        """Returns (logits, argmax) of the last of the tokens whose embedding rows are x
+        [n_tokens][n_embd], placed at positions pos0 .. (run_layers at n_tokens > 1)."""
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, self.n_embd)
+        logits = np.empty(self.n_vocab, np.float32)
+        am = C.c_uint32()
+        self._be._check(self._be._lib.ogm_llama_prefill(self._be._ctx, self._h, x.ctypes.data, pos0, x.shape[0],
+                                                        logits.ctypes.data, C.byref(am)), "ogm_llama_prefill")
+        return logits, am.value
+
+    def prefill_tokens(self, tok_embd, tokens, pos0: int = 0):
+        """The same from token ids; tok_embd is a QuantMatrix [n_embd -> n_vocab] or a handle."""
+        h = tok_embd if isinstance(tok_embd, int) else self._be.upload(tok_embd)
+        tokens = np.ascontiguousarray(tokens, np.uint32).reshape(-1)
+        logits = np.empty(self.n_vocab, np.float32)
+        am = C.c_uint32()
+        self._be._check(self._be._lib.ogm_llama_prefill_tokens(self._be._ctx, self._h, h, tokens.ctypes.data, pos0,
+                                                               tokens.size, logits.ctypes.data, C.byref(am)),
+                        "ogm_llama_prefill_tokens")
+        return logits, am.value
+
     def decode_dev(self, x_ptr: int, pos: int, logits_ptr: int = 0, argmax_ptr: int = 0, stream: int = 0):
         self._be._check(self._be._lib.ogm_llama_decode_dev(self._be._ctx, self._h, x_ptr, pos, logits_ptr or None,
                                                            argmax_ptr or None, stream or None), "ogm_llama_decode_dev")

@@ -45,6 +45,7 @@ struct ogm_ctx {
   DevBuf hx, hy;  // pinned host staging
   int tune_wg_waves = 0;
   int tune_gemm_min_tokens = 9;  // matmul at n_tokens >= this takes the MFMA GEMM
+  int tune_gemm_wide_min_wgs = 0;
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
   const char *last_kernel = "";
@@ -205,6 +206,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemm_min_tokens") == 0) {
     if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_min_tokens must be >= 0");
     ctx->tune_gemm_min_tokens = value ? value : 9;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_wide_min_wgs") == 0) {
+    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_wide_min_wgs must be >= 0");
+    ctx->tune_gemm_wide_min_wgs = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemv_rb_per_wg") == 0) {
@@ -395,7 +401,10 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
     int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w0->in_dim, n_tokens));
     if (rc != OGM_OK) return rc;
-    for (size_t i = 0; i < n_tg; i++) {
+    // Q4_K matrices over the same input (q, k, v; gate, up) share a launch, up to OGM_GEMM_MAX_MATS
+    const size_t per_launch = w0->ggml_type == OGM_TYPE_Q4_K ? OGM_GEMM_MAX_MATS : 1;
+    for (size_t i = 0; i < n_tg; i += per_launch) {
+      const size_t ng = n_tg - i < per_launch ? n_tg - i : per_launch;
       OgmGemmArgs g;
       g.ggml_type = w0->ggml_type;
       g.wt = tg[i].w->dev;
@@ -405,6 +414,13 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.n_tokens = n_tokens;
       g.y = tg[i].y;
       g.xh = ctx->xh.p;
+      g.wide_min_wgs = (uint32_t)ctx->tune_gemm_wide_min_wgs;
+      g.n_extra = (uint32_t)ng - 1;
+      for (size_t j = 1; j < ng; j++) {
+        g.extra_wt[j - 1] = tg[i + j].w->dev;
+        g.extra_out_dim[j - 1] = tg[i + j].w->out_dim;
+        g.extra_y[j - 1] = tg[i + j].y;
+      }
       HIPCHK(ctx, ogm_launch_gemm(g, stream, &ctx->last_kernel));
     }
     return OGM_OK;
@@ -748,6 +764,15 @@ struct ogm_llama {
   uint32_t *amax_scratch = nullptr, *amax_out = nullptr;
   float *stage = nullptr;     // host->device staging for ogm_llama_kv_write
   size_t stage_cap = 0;
+  // prefill rows, allocated at the first prefill for OGM_PREFILL_CHUNK tokens
+  struct Prefill {
+    float *x = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
+    float *proj = nullptr, *gate = nullptr, *up = nullptr, *h = nullptr, *cs = nullptr;
+    float *part_o = nullptr, *part_ml = nullptr;
+    uint32_t *tokens = nullptr;
+    uint32_t attn_tokens = 0;   // query rows one attention launch takes (bounded by part_o)
+    bool ready = false;
+  } pf;
   uint32_t max_splits = 0;
   std::vector<void *> allocs;
 };
@@ -959,7 +984,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
   const float scale = 1.0f / sqrtf((float)c.head_dim);
   if (x_dev != m->x) HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
-  HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos, c.rope_dim, m->rope_cs, s));
+  HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos, 1, c.rope_dim, m->rope_cs, s));
   const float *delta = nullptr;  // what the next norm adds to x first: the last block's output
   for (uint32_t l = 0; l < c.n_layer; l++) {
     const ogm_llama_layer &L = m->layers[l];
@@ -1097,4 +1122,170 @@ extern "C" int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
     HIPCHK(ctx, hipMemcpyAsync(last_logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   return OGM_OK;
+}
+
+// ---- prefill: run_layers at n_tokens > 1 (llama.rs:594-932) ------------------------------------
+
+static const uint32_t OGM_PREFILL_CHUNK = 512;             // tokens per pass over the layers
+static const size_t OGM_PREFILL_PART_BYTES = 256u << 20;   // attention partials per launch
+
+static int llama_prefill_buffers(ogm_ctx *ctx, ogm_llama *m) {
+  if (m->pf.ready) return OGM_OK;
+  const ogm_llama_config &c = m->cfg;
+  const size_t T = OGM_PREFILL_CHUNK, qd = (size_t)c.n_head * c.head_dim, kvd = (size_t)c.n_head_kv * c.head_dim;
+  // query rows per attention launch: as many as keep the partial results within their budget
+  const size_t per_token = (size_t)c.n_head * m->max_splits * c.head_dim * 4;
+  size_t at = OGM_PREFILL_PART_BYTES / per_token;
+  if (at < 1) at = 1;
+  if (at > T) at = T;
+  int rc = OGM_OK;
+  auto A = [&](float **p, size_t n) { if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)p, n * 4); };
+  A(&m->pf.x, T * c.n_embd);
+  A(&m->pf.normed, T * c.n_embd);
+  A(&m->pf.q, T * qd);
+  A(&m->pf.k, T * kvd);
+  A(&m->pf.v, T * kvd);
+  A(&m->pf.attn, T * qd);
+  A(&m->pf.proj, T * c.n_embd);
+  A(&m->pf.gate, T * c.n_ff);
+  A(&m->pf.up, T * c.n_ff);
+  A(&m->pf.h, T * c.n_ff);
+  A(&m->pf.cs, T * (c.rope_dim / 2 + 1) * 2);
+  A(&m->pf.part_o, at * per_token / 4);
+  A(&m->pf.part_ml, at * (size_t)c.n_head * m->max_splits * 2);
+  A((float **)&m->pf.tokens, T);
+  if (rc != OGM_OK) return rc;
+  m->pf.attn_tokens = (uint32_t)at;
+  m->pf.ready = true;
+  return OGM_OK;
+}
+
+// Matmuls over the same T input rows; weights of one type share the quantized activations.
+static int llama_matmul_rows(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, const float *x,
+                             uint32_t T, hipStream_t s) {
+  size_t i = 0;
+  while (i < n) {
+    Target tg[OGM_GEMV_MAX_MATS];
+    size_t e = i;
+    while (e < n && e - i < OGM_GEMV_MAX_MATS && ws[e]->ggml_type == ws[i]->ggml_type) {
+      tg[e - i] = Target{ws[e], ys[e]};
+      e++;
+    }
+    int rc = enqueue_matmul(ctx, tg, e - i, x, T, 0, s, nullptr, nullptr);
+    if (rc != OGM_OK) return rc;
+    i = e;
+  }
+  return OGM_OK;
+}
+
+// One chunk of T <= OGM_PREFILL_CHUNK tokens whose embedding rows sit in m->pf.x.  With `last`,
+// the final row's hidden state ends in m->x and its logits in m->logits.
+static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32_t T, bool last, hipStream_t s) {
+  const ogm_llama_config &c = m->cfg;
+  ogm_llama::Prefill &P = m->pf;
+  const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
+  const float scale = 1.0f / sqrtf((float)c.head_dim);
+  HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos0, T, c.rope_dim, P.cs, s));
+  const float *delta = nullptr;
+  for (uint32_t l = 0; l < c.n_layer; l++) {
+    const ogm_llama_layer &L = m->layers[l];
+    const float *attn_norm = m->norms + (size_t)l * 2 * c.n_embd, *ffn_norm = attn_norm + c.n_embd;
+    void *kc = (uint8_t *)m->k_cache + (size_t)l * c.max_ctx * kvd * 2;
+    void *vc = (uint8_t *)m->v_cache + (size_t)l * c.max_ctx * kvd * 2;
+    HIPCHK(ctx, ogm_launch_norm_rows(P.x, delta, attn_norm, c.n_embd, T, c.rms_eps, P.normed, s));
+    const ogm_weight *w3[3] = {L.wq, L.wk, L.wv};
+    float *y3[3] = {P.q, P.k, P.v};
+    int rc = llama_matmul_rows(ctx, w3, y3, 3, P.normed, T, s);
+    if (rc != OGM_OK) return rc;
+    const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
+    HIPCHK(ctx, ogm_launch_qkv_pre(P.q, P.k, P.v, P.cs, c.rope_dim, pre, c.n_head, c.n_head_kv, c.head_dim, kc, vc,
+                                   pos0, T, s));
+    for (uint32_t t0 = 0; t0 < T; t0 += P.attn_tokens) {
+      const uint32_t nt = T - t0 < P.attn_tokens ? T - t0 : P.attn_tokens;
+      HIPCHK(ctx, ogm_launch_attn_prefill(P.q + (size_t)t0 * qd, kc, vc, pos0 + t0, nt, m->max_splits, c.n_head,
+                                          c.n_head_kv, c.head_dim, scale, P.part_o, P.part_ml,
+                                          P.attn + (size_t)t0 * qd, s));
+    }
+    const ogm_weight *w1[1] = {L.wo};
+    float *y1[1] = {P.proj};
+    if ((rc = llama_matmul_rows(ctx, w1, y1, 1, P.attn, T, s)) != OGM_OK) return rc;
+    HIPCHK(ctx, ogm_launch_norm_rows(P.x, P.proj, ffn_norm, c.n_embd, T, c.rms_eps, P.normed, s));
+    const ogm_weight *w2[2] = {L.w_gate, L.w_up};
+    float *y2[2] = {P.gate, P.up};
+    if ((rc = llama_matmul_rows(ctx, w2, y2, 2, P.normed, T, s)) != OGM_OK) return rc;
+    HIPCHK(ctx, ogm_launch_swiglu_rows(P.gate, P.up, (size_t)T * c.n_ff, P.h, s));
+    const ogm_weight *wd[1] = {L.w_down};
+    if ((rc = llama_matmul_rows(ctx, wd, y1, 1, P.h, T, s)) != OGM_OK) return rc;
+    delta = P.proj;
+  }
+  ctx->act_mode = -1;   // the activation scratch was the matmuls'
+  if (!last) return OGM_OK;
+  // forward (llama.rs:1007-1032): the last row alone goes through the output norm and projection
+  float *x_last = P.x + (size_t)(T - 1) * c.n_embd;
+  const float *d_last = delta ? delta + (size_t)(T - 1) * c.n_embd : nullptr;
+  const int mode_out = act_mode_for(m->output->ggml_type);
+  int rc = ensure_act(ctx, c.n_embd, 1);
+  if (rc != OGM_OK) return rc;
+  HIPCHK(ctx, ogm_launch_norm_quant(mode_out, x_last, d_last, m->norms + (size_t)c.n_layer * 2 * c.n_embd, c.n_embd,
+                                    c.rms_eps, nullptr, act_view(ctx, c.n_embd, mode_out, 0), s));
+  HIPCHK(ctx, hipMemcpyAsync(m->x, x_last, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
+  const ogm_weight *wo_[1] = {m->output};
+  float *yo[1] = {m->logits};
+  if ((rc = llama_matmul(ctx, wo_, yo, 1, s)) != OGM_OK) return rc;
+  HIPCHK(ctx, ogm_launch_argmax(m->logits, c.n_vocab, m->amax_scratch, m->amax_out, s));
+  ctx->act_mode = -1;
+  return OGM_OK;
+}
+
+static int llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x_host, const ogm_weight *tok_embd,
+                         const uint32_t *tokens, uint32_t pos0, uint32_t n_tokens, float *last_logits,
+                         uint32_t *argmax) {
+  const ogm_llama_config &c = m->cfg;
+  if (n_tokens == 0) return fail(ctx, OGM_ERR_INVALID, "no tokens");
+  if ((uint64_t)pos0 + n_tokens > c.max_ctx) return fail(ctx, OGM_ERR_INVALID, "positions beyond the KV cache");
+  if (tok_embd) {
+    if (tok_embd->in_dim != c.n_embd) return fail(ctx, OGM_ERR_INVALID, "embedding matrix shape");
+    for (uint32_t i = 0; i < n_tokens; i++)
+      if (tokens[i] >= tok_embd->out_dim) return fail(ctx, OGM_ERR_INVALID, "token id outside the vocabulary");
+  }
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  int rc = llama_prefill_buffers(ctx, m);
+  if (rc != OGM_OK) return rc;
+  hipStream_t s = ctx->stream;
+  for (uint32_t t0 = 0; t0 < n_tokens; t0 += OGM_PREFILL_CHUNK) {
+    const uint32_t T = n_tokens - t0 < OGM_PREFILL_CHUNK ? n_tokens - t0 : OGM_PREFILL_CHUNK;
+    if (tok_embd) {
+      // the embedding rows (llama.rs:609-614), dequantized on the device
+      HIPCHK(ctx, hipMemcpyAsync(m->pf.tokens, tokens + t0, (size_t)T * 4, hipMemcpyHostToDevice, s));
+      for (uint32_t i = 0; i < T; i++)
+        HIPCHK(ctx, ogm_launch_dequant_row(tok_embd->dev, tok_embd->ggml_type, tok_embd->in_dim, tok_embd->out_dim, 0,
+                                           m->pf.tokens + i, m->pf.x + (size_t)i * c.n_embd, s));
+    } else {
+      HIPCHK(ctx, hipMemcpyAsync(m->pf.x, x_host + (size_t)t0 * c.n_embd, (size_t)T * c.n_embd * 4,
+                                 hipMemcpyHostToDevice, s));
+    }
+    rc = llama_prefill_chunk(ctx, m, pos0 + t0, T, t0 + T == n_tokens, s);
+    if (rc != OGM_OK) return rc;
+    // the staging copies above read caller memory and m->pf.tokens is reused: finish the chunk first
+    HIPCHK(ctx, hipStreamSynchronize(s));
+  }
+  if (last_logits) HIPCHK(ctx, hipMemcpy(last_logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost));
+  if (argmax) HIPCHK(ctx, hipMemcpy(argmax, m->amax_out, 4, hipMemcpyDeviceToHost));
+  return OGM_OK;
+}
+
+extern "C" int ogm_llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos0, uint32_t n_tokens,
+                                 float *last_logits, uint32_t *argmax) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !x) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  return llama_prefill(ctx, m, x, nullptr, nullptr, pos0, n_tokens, last_logits, argmax);
+}
+
+extern "C" int ogm_llama_prefill_tokens(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *tok_embd,
+                                        const uint32_t *tokens, uint32_t pos0, uint32_t n_tokens,
+                                        float *last_logits, uint32_t *argmax) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !tok_embd || !tokens) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  return llama_prefill(ctx, m, nullptr, tok_embd, tokens, pos0, n_tokens, last_logits, argmax);
 }

@@ -46,7 +46,30 @@ struct GemmParams {
   float *y;               // [T][out_dim]
   uint32_t in_dim, out_dim, n_tokens, nsb;
   uint32_t c_shift, r_shift, nct;  // weight tiles of R = 1 << r_shift rows x C = 1 << c_shift blocks
+  // further matrices over the same activations (q, k, v), their row tiles following in grid.y
+  uint32_t n_extra;
+  const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1];
+  float *extra_y[OGM_GEMM_MAX_MATS - 1];
+  uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
 };
+
+// The matrix a workgroup's row tile belongs to: rewrites p for it and returns the tile's index
+// within that matrix.
+__device__ __forceinline__ uint32_t gm_pick_matrix(GemmParams &p, uint32_t row_tile) {
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
+    const uint32_t tiles = (p.out_dim + 127u) / 128u;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  return row_tile;
+}
 
 __device__ __forceinline__ float gm_f16_bits_to_f32(uint32_t bits16) {
   union { unsigned short u; _Float16 h; } v;
@@ -160,7 +183,7 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q4k_kernel(GemmParams p) {
   const bool producer = wave >= 8u;
   const uint32_t rt = tid & 511u;                   // thread index within its half
   const uint32_t wr = wave & 1u, wt_ = (wave & 7u) >> 1;   // multiplying wave: row half (64 rows), token quarter (32)
-  const uint32_t t0 = blockIdx.x * GM_BT, r0 = blockIdx.y * GM_BN;
+  const uint32_t t0 = blockIdx.x * GM_BT, r0 = gm_pick_matrix(p, blockIdx.y) * GM_BN;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
   // Address of block `s` of row `row` in the tile-planar layout (piece 0: d, dmin, scales).
@@ -492,7 +515,7 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_wide_kernel(GemmParams p) {
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const bool producer = wave >= 8u;
   const uint32_t wr = wave & 1u, wt_ = (wave & 7u) >> 1;   // multiplying wave: row half, token quarter (64)
-  const uint32_t t0 = blockIdx.x * GW_BT, r0 = blockIdx.y * GM_BN;
+  const uint32_t t0 = blockIdx.x * GW_BT, r0 = gm_pick_matrix(p, blockIdx.y) * GM_BN;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
   auto row_off = [&](uint32_t row) -> uint32_t {
@@ -1279,14 +1302,24 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   _Float16 *bs16 = xh + (size_t)a.in_dim * a.n_tokens;
   // Q4_K beyond two token tiles of 128 runs the wide kernel, which reads the int8 activations as
   // they are and needs only the (bh, bl) pairs prepared
-  const bool wide = a.ggml_type == OGM_Q4_K && a.n_tokens > 256u;
+  // Q4_K beyond two token tiles of 128 runs the wide kernel (which reads the int8 activations as
+  // they are and needs only the (bh, bl) pairs prepared) once the 128 x 128 tiling would need more
+  // than one round of workgroups over the 256 compute units: within one round the smaller tile's
+  // shorter chain per workgroup wins (4096 -> 4096 at 512 tokens: 76 us against 103 us), beyond it
+  // the wide tile's halved weight traffic does (4096 -> 14336: 119 us against 166 us)
+  uint32_t row_tiles = (a.out_dim + GM_BN - 1) / GM_BN;
+  if (a.ggml_type != OGM_Q4_K && a.n_extra != 0) return hipErrorInvalidValue;
+  if (a.n_extra > OGM_GEMM_MAX_MATS - 1) return hipErrorInvalidValue;
+  for (uint32_t m = 0; m < a.n_extra; m++) row_tiles += (a.extra_out_dim[m] + GM_BN - 1) / GM_BN;
+  const uint32_t wgs128 = ((a.n_tokens + GM_BT - 1) / GM_BT) * row_tiles;
+  const bool wide = a.ggml_type == OGM_Q4_K && a.n_tokens > 256u && wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
   hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((wide ? n_sb : n8) + 255) / 256)), dim3(256), 0,
                      stream, a.act.q, a.act.bsum, wide ? (_Float16 *)nullptr : xh, bs16, n8, n_sb);
   const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
   const uint32_t c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
   // token tiles vary fastest: workgroups that run together share weight rows, and with a
   // power-of-two number of token tiles each XCD's L2 sees few distinct activation tiles
-  const dim3 grid((a.n_tokens + GM_BT - 1) / GM_BT, (a.out_dim + GM_BN - 1) / GM_BN);
+  const dim3 grid((a.n_tokens + GM_BT - 1) / GM_BT, row_tiles);
   hipError_t e;
   if (a.ggml_type == OGM_Q6_K) {
     Gemm6Params p;
@@ -1323,8 +1356,14 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   p.r_shift = 6 - c_shift;
   p.nct = tl.nct;
   p.xq = a.act.q;
+  p.n_extra = a.n_extra;
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
+    p.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
+    p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
+    p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
+  }
   if (wide) {
-    const dim3 wgrid((a.n_tokens + GW_BT - 1) / GW_BT, (a.out_dim + GM_BN - 1) / GM_BN);
+    const dim3 wgrid((a.n_tokens + GW_BT - 1) / GW_BT, row_tiles);
     e = hipFuncSetAttribute((const void *)ogm_gemm_q4k_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)GW_LDS_BYTES);
     if (e != hipSuccess) return e;

@@ -50,6 +50,7 @@ hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char 
 
 // Prefill GEMM on MFMA (ogm_gemm.hip).  Same operands as the GEMV plus a scratch buffer `xh` of
 // ogm_gemm_xh_bytes() for the activations as f16.  Follows the CPU path's GEMM float order.
+#define OGM_GEMM_MAX_MATS 3   // matrices one GEMM launch can take (q, k, v)
 struct OgmGemmArgs {
   uint32_t ggml_type;
   const uint8_t *wt;
@@ -58,6 +59,12 @@ struct OgmGemmArgs {
   uint32_t n_tokens;
   float *y;            // [n_tokens][out_dim]
   void *xh;            // scratch
+  uint32_t wide_min_wgs = 0;   // Q4_K: least 128x128 workgroups from which the wide tiling runs (0 = default)
+  // Q4_K only: further matrices of the same in_dim over the same activations, in the same launch
+  uint32_t n_extra = 0;
+  const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1] = {};
+  uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1] = {};
+  float *extra_y[OGM_GEMM_MAX_MATS - 1] = {};
 };
 bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens);
 size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens);

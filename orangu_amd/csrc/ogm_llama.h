@@ -19,7 +19,9 @@ hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const f
 // cos / sin of pos * freq[p] for the rope_dim / 2 rotated pairs, as float2 (cos, sin): once per
 // token, every layer rotates by the same angles (tensor.rs:1147-1160, freq_scale 1, no YaRN;
 // `freq` already holds base^(-2p / rope_dim) divided by the pair's frequency factor).
-hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t rope_dim, void *cs, hipStream_t stream);
+// Row t of `cs` (rope_dim / 2 pairs each) is the table of the token at position pos + t.
+hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t n_tokens, uint32_t rope_dim, void *cs,
+                                 hipStream_t stream);
 
 // What a layer applies to its projections before they meet (engine/arch/llama.rs:757-810): the
 // projection biases (Qwen2), then the per-head RMSNorm of q and k (Qwen3), then RoPE in the
@@ -67,3 +69,29 @@ hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStrea
 // embedding lookup (llama.rs:609-614 over quant.rs:639-649, 666-697, 746-787), bit-identical.
 hipError_t ogm_launch_dequant_row(const uint8_t *wt, uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim,
                                   uint32_t row, const uint32_t *row_dev, float *out, hipStream_t stream);
+
+// ---- the same layer over a batch of tokens (prefill, llama.rs:594-932 at n_tokens > 1) ----------
+// The matmuls between these are GEMMs that quantize their own input: plain f32 rows throughout.
+
+// Rows of n values: x += delta (when given, in place), normed = RMSNorm(x) * weight.  n % 4 == 0.
+hipError_t ogm_launch_norm_rows(float *x, const float *delta, const float *weight, uint32_t n, uint32_t n_rows,
+                                float eps, float *normed, hipStream_t stream);
+
+// q [n_tokens][n_head*head_dim] in place, k and v [n_tokens][n_head_kv*head_dim] into the cache
+// rows pos0 .. pos0 + n_tokens as f16: bias, per-head norm, RoPE (row t of `cs`) as in
+// ogm_launch_attn_decode.
+hipError_t ogm_launch_qkv_pre(float *q, const float *k, const float *v, const void *cs, uint32_t rope_dim,
+                              const OgmAttnPre &pre, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
+                              void *k_cache_layer, void *v_cache_layer, uint32_t pos0, uint32_t n_tokens,
+                              hipStream_t stream);
+
+// Causal attention of n_tokens query rows (already rotated) at positions pos0 .. over cache rows
+// 0 .. pos0 + t for token t; attn_out [n_tokens][n_head*head_dim].
+// part_o: [n_tokens][n_head][max_splits][head_dim], part_ml: [n_tokens][n_head][max_splits][2].
+hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_cache_layer, uint32_t pos0,
+                                   uint32_t n_tokens, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
+                                   uint32_t head_dim, float scale, float *part_o, float *part_ml, float *attn_out,
+                                   hipStream_t stream);
+
+// h = silu(gate) * up over n values.  n % 4 == 0.
+hipError_t ogm_launch_swiglu_rows(const float *gate, const float *up, size_t n, float *h, hipStream_t stream);

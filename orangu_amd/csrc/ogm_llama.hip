@@ -92,17 +92,18 @@ __global__ __launch_bounds__(64) void ogm_rope_table_kernel(const float *__restr
                                                             uint32_t rope_half, float2 *__restrict__ cs) {
   const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= rope_half) return;
-  const float theta = (float)pos * freq[p];
+  const float theta = (float)(pos + blockIdx.y) * freq[p];   // row blockIdx.y: the token at pos + blockIdx.y
   float sn, c;
   sincosf(theta, &sn, &c);
-  cs[p] = make_float2(c, sn);
+  cs[(size_t)blockIdx.y * rope_half + p] = make_float2(c, sn);
 }
 
-hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t rope_dim, void *cs, hipStream_t stream) {
-  if (rope_dim % 2u != 0) return hipErrorInvalidValue;
+hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t n_tokens, uint32_t rope_dim, void *cs,
+                                 hipStream_t stream) {
+  if (rope_dim % 2u != 0 || n_tokens == 0 || n_tokens > 65535u) return hipErrorInvalidValue;
   if (rope_dim == 0) return hipSuccess;
-  hipLaunchKernelGGL(ogm_rope_table_kernel, dim3((rope_dim / 2u + 63u) / 64u), dim3(64), 0, stream, freq, pos,
-                     rope_dim / 2u, (float2 *)cs);
+  hipLaunchKernelGGL(ogm_rope_table_kernel, dim3((rope_dim / 2u + 63u) / 64u, n_tokens), dim3(64), 0, stream, freq,
+                     pos, rope_dim / 2u, (float2 *)cs);
   return hipGetLastError();
 }
 
@@ -195,7 +196,12 @@ __device__ __forceinline__ AttnPart attn_merge_chunks(const float *part_o, const
 //   * GROUP != 0 (G * HD is a multiple of the quantizer's group): the workgroup that takes the
 //     last ticket of its K/V head merges the chunks and quantizes the G * HD outputs; no other
 //     workgroup waits for anything.
-template <int HD, int G, int GROUP>
+//
+// PREFILL: the same over a batch of query tokens (blockIdx.z; token t sits at position pos + t and
+// attends to positions 0 .. pos + t).  q arrives with bias, norm and RoPE applied and every K/V
+// row is in the cache already (ogm_qkv_pre_kernel), workgroups past a token's last chunk leave at
+// once, and nothing is quantized: the next matmul is a GEMM that quantizes its own input.
+template <int HD, int G, int GROUP, bool PREFILL = false>
 __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
                                                        const float *__restrict__ v_new,
                                                        const float2 *__restrict__ cs, uint32_t rope_half,
@@ -221,13 +227,24 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
   __shared__ __align__(16) float osum[NW][G][HD];
   __shared__ uint32_t s_last;
   __shared__ float mrg[GROUP != 0 ? 6 : 1][GROUP != 0 ? NT : 1];   // the final merge's slices
-  const uint32_t kvh = blockIdx.x, split = blockIdx.y, n_splits = gridDim.y;
+  static_assert(!PREFILL || GROUP == 0, "a prefill batch merges in its own launch");
+  const uint32_t kvh = blockIdx.x, split = blockIdx.y;
+  if constexpr (PREFILL) {
+    const uint32_t tok = blockIdx.z;
+    pos += tok;
+    if (split > pos / OGM_ATTN_CHUNK) return;   // the whole workgroup: this token has no such chunk
+    const size_t n_head = (size_t)n_head_kv * gq;
+    q += tok * n_head * HD;
+    part_o += tok * n_head * max_splits * HD;
+    part_ml += tok * n_head * max_splits * 2;
+  }
+  const uint32_t n_splits = PREFILL ? pos / OGM_ATTN_CHUNK + 1u : gridDim.y;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t kv_dim = n_head_kv * HD;
   const uint32_t n_pos = pos + 1u;
   const uint32_t p0 = split * OGM_ATTN_CHUNK;
   const uint32_t n_here = min(OGM_ATTN_CHUNK, n_pos - p0);
-  const bool is_last = split == n_splits - 1u;   // holds the current position, not yet cached
+  const bool is_last = !PREFILL && split == n_splits - 1u;   // holds the current position, not yet cached
   const uint32_t cur = pos - p0;                 // meaningful in the last chunk only
 
   const uint32_t r = tid >> 2, c = tid & 3u;              // phase 1: cache row and piece phase
@@ -247,7 +264,14 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
   // two more take the new k and v rows, which also go to the cache.  G counts the head slots of the
   // kernel, gq <= G the query heads the model has per K/V head: the other slots hold zeros and
   // store nothing.
-  {
+  if constexpr (PREFILL) {
+    for (uint32_t i = tid; i < (uint32_t)(G * HD / 4); i += NT) {
+      const uint32_t g = i / (HD / 4), d4 = i - g * (HD / 4);
+      float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (g < gq) v4 = *(const float4 *)(q + ((size_t)kvh * gq + g) * HD + 4u * d4);
+      *(float4 *)&qs[g][4u * d4] = v4;
+    }
+  } else {
     constexpr int PPL = (HD / 2 + 63) / 64;   // pairs per lane
     const uint32_t n_units = (uint32_t)G + (is_last ? 2u : 0u);
     for (uint32_t u = wave; u < n_units; u += NW) {
@@ -811,5 +835,208 @@ hipError_t ogm_launch_dequant_row(const uint8_t *wt, uint32_t ggml_type, uint32_
     return hipErrorInvalidValue;
   hipLaunchKernelGGL(ogm_dequant_row_kernel, dim3((in_dim + 255u) / 256u), dim3(256), 0, stream, wt, ggml_type,
                      in_dim, out_dim, row, row_dev, out);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// prefill: the same layer over a batch of tokens.  The matmuls are GEMMs that quantize their
+// own input, so these kernels leave plain f32 rows.
+
+// One workgroup per token row: x += delta (when given), normed = x * (1 / sqrt(mean(x^2) + eps)) * w.
+__global__ __launch_bounds__(256) void ogm_norm_rows_kernel(float *__restrict__ x, const float *__restrict__ delta,
+                                                            const float *__restrict__ weight, uint32_t n, float eps,
+                                                            float *__restrict__ normed) {
+  __shared__ float red[4];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const size_t row = (size_t)blockIdx.x * n;
+  float ss = 0.0f;
+  for (uint32_t e0 = 4u * tid; e0 < n; e0 += 1024u) {
+    float4 v = *(const float4 *)(x + row + e0);
+    if (delta) {
+      const float4 d = *(const float4 *)(delta + row + e0);
+      v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+      *(float4 *)(x + row + e0) = v;
+    }
+    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+  }
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) ss += __shfl_xor(ss, m, 64);
+  if (lane == 0) red[wave] = ss;
+  __syncthreads();
+  const float total = red[0] + red[1] + red[2] + red[3];
+  const float scale = 1.0f / sqrtf(total / (float)n + eps);
+  for (uint32_t e0 = 4u * tid; e0 < n; e0 += 1024u) {
+    const float4 v = *(const float4 *)(x + row + e0);   // this thread's own stores above
+    const float4 w = *(const float4 *)(weight + e0);
+    *(float4 *)(normed + row + e0) = make_float4(v.x * scale * w.x, v.y * scale * w.y, v.z * scale * w.z,
+                                                 v.w * scale * w.w);
+  }
+}
+
+hipError_t ogm_launch_norm_rows(float *x, const float *delta, const float *weight, uint32_t n, uint32_t n_rows,
+                                float eps, float *normed, hipStream_t stream) {
+  if (n == 0 || n % 4u != 0 || n_rows == 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ogm_norm_rows_kernel, dim3(n_rows), dim3(256), 0, stream, x, delta, weight, n, eps, normed);
+  return hipGetLastError();
+}
+
+// One wave per (token, head of q | k | v): bias, per-head norm and RoPE as the decode kernel's
+// first phase; q is rewritten in place, k and v go to their cache rows as f16.
+template <int HD>
+__global__ __launch_bounds__(256) void ogm_qkv_pre_kernel(float *__restrict__ q, const float *__restrict__ k,
+                                                          const float *__restrict__ v,
+                                                          const float2 *__restrict__ cs, uint32_t rope_half,
+                                                          OgmAttnPre pre, uint32_t n_head, uint32_t n_head_kv,
+                                                          __half *__restrict__ kc, __half *__restrict__ vc,
+                                                          uint32_t pos0) {
+  constexpr int PPL = (HD / 2 + 63) / 64;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t u = blockIdx.x * 4u + (threadIdx.x >> 6), tok = blockIdx.y;
+  if (u >= n_head + 2u * n_head_kv) return;
+  const bool is_q = u < n_head, is_v = u >= n_head + n_head_kv;
+  const uint32_t head = is_q ? u : (is_v ? u - n_head - n_head_kv : u - n_head);
+  const size_t kv_dim = (size_t)n_head_kv * HD;
+  const size_t row = (size_t)head * HD;   // within a token's vector and within the bias
+  float *qrow = q + (size_t)tok * n_head * HD + row;
+  const float *src = is_q ? qrow : (is_v ? v : k) + (size_t)tok * kv_dim + row;
+  const float *bias = is_q ? pre.q_bias : is_v ? pre.v_bias : pre.k_bias;
+  const float *nw = is_q ? pre.q_norm : is_v ? nullptr : pre.k_norm;
+  cs += (size_t)tok * rope_half;
+  float a[PPL], b[PPL];
+  uint32_t ia[PPL], ib[PPL];
+  float ss = 0.0f;
+#pragma unroll
+  for (int j = 0; j < PPL; j++) {
+    const uint32_t p = lane + 64u * j;
+    const bool have = p < (uint32_t)(HD / 2);
+    const bool split_pair = pre.neox != 0u && !is_v && p < rope_half;
+    ia[j] = split_pair ? p : 2u * p;
+    ib[j] = split_pair ? p + rope_half : 2u * p + 1u;
+    a[j] = have ? src[ia[j]] : 0.0f;
+    b[j] = have ? src[ib[j]] : 0.0f;
+    if (bias != nullptr && have) {
+      a[j] += bias[row + ia[j]];
+      b[j] += bias[row + ib[j]];
+    }
+    ss += a[j] * a[j] + b[j] * b[j];
+  }
+  if (nw != nullptr) {
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) ss += __shfl_xor(ss, m, 64);
+    const float sc_n = 1.0f / sqrtf(ss / (float)HD + pre.eps);
+#pragma unroll
+    for (int j = 0; j < PPL; j++) {
+      const uint32_t p = lane + 64u * j;
+      if (p < (uint32_t)(HD / 2)) {
+        a[j] = a[j] * sc_n * nw[ia[j]];
+        b[j] = b[j] * sc_n * nw[ib[j]];
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < PPL; j++) {
+    const uint32_t p = lane + 64u * j;
+    if (p >= (uint32_t)(HD / 2)) continue;
+    float2 ab = make_float2(a[j], b[j]);
+    if (!is_v && p < rope_half) ab = rope_pair(ab, cs[p]);
+    if (is_q) {
+      qrow[ia[j]] = ab.x;
+      qrow[ib[j]] = ab.y;
+    } else {
+      __half *cache = (is_v ? vc : kc) + (size_t)(pos0 + tok) * kv_dim + row;
+      cache[ia[j]] = __float2half_rn(ab.x);
+      cache[ib[j]] = __float2half_rn(ab.y);
+    }
+  }
+}
+
+hipError_t ogm_launch_qkv_pre(float *q, const float *k, const float *v, const void *cs, uint32_t rope_dim,
+                              const OgmAttnPre &pre, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
+                              void *k_cache_layer, void *v_cache_layer, uint32_t pos0, uint32_t n_tokens,
+                              hipStream_t stream) {
+  if (rope_dim > head_dim || rope_dim % 2u != 0 || n_tokens == 0 || n_tokens > 65535u) return hipErrorInvalidValue;
+  const dim3 grid((n_head + 2u * n_head_kv + 3u) / 4u, n_tokens);
+  if (head_dim == 128)
+    hipLaunchKernelGGL(ogm_qkv_pre_kernel<128>, grid, dim3(256), 0, stream, q, k, v, (const float2 *)cs,
+                       rope_dim / 2u, pre, n_head, n_head_kv, (__half *)k_cache_layer, (__half *)v_cache_layer, pos0);
+  else if (head_dim == 64)
+    hipLaunchKernelGGL(ogm_qkv_pre_kernel<64>, grid, dim3(256), 0, stream, q, k, v, (const float2 *)cs,
+                       rope_dim / 2u, pre, n_head, n_head_kv, (__half *)k_cache_layer, (__half *)v_cache_layer, pos0);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+// The chunks of every (token, head) merged: one wave per 256 outputs of a token.
+__global__ __launch_bounds__(64) void ogm_attn_combine_rows_kernel(const float *__restrict__ part_o,
+                                                                   const float *__restrict__ part_ml, uint32_t pos0,
+                                                                   uint32_t max_splits, uint32_t n, uint32_t head_dim,
+                                                                   float *__restrict__ attn_out) {
+  const uint32_t lane = threadIdx.x, tok = blockIdx.y;
+  const uint32_t e0 = blockIdx.x * 256u + 4u * lane;
+  if (e0 >= n) return;
+  const uint32_t n_head = n / head_dim;
+  const uint32_t n_splits = (pos0 + tok) / OGM_ATTN_CHUNK + 1u;
+  const AttnPart pt = attn_merge_chunks<false>(part_o + (size_t)tok * n_head * max_splits * head_dim,
+                                               part_ml + (size_t)tok * n_head * max_splits * 2, e0 / head_dim,
+                                               e0 % head_dim, 0u, 1u, n_splits, max_splits, head_dim);
+  *(float4 *)(attn_out + (size_t)tok * n + e0) =
+      make_float4(pt.o.x / pt.den, pt.o.y / pt.den, pt.o.z / pt.den, pt.o.w / pt.den);
+}
+
+hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_cache_layer, uint32_t pos0,
+                                   uint32_t n_tokens, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
+                                   uint32_t head_dim, float scale, float *part_o, float *part_ml, float *attn_out,
+                                   hipStream_t stream) {
+  if (n_head_kv == 0 || n_head % n_head_kv != 0 || n_tokens == 0 || n_tokens > 65535u) return hipErrorInvalidValue;
+  const uint32_t n_splits = (pos0 + n_tokens - 1u) / OGM_ATTN_CHUNK + 1u;   // of the last token
+  if (n_splits > max_splits) return hipErrorInvalidValue;
+  const uint32_t n = n_head * head_dim;
+  if (n % 4u != 0) return hipErrorInvalidValue;
+  const uint32_t gq = n_head / n_head_kv;
+  if (gq > 8u) return hipErrorInvalidValue;
+  const uint32_t G = gq <= 2u ? gq : (gq <= 4u ? 4u : 8u);
+  const dim3 grid(n_head_kv, n_splits, n_tokens);
+  const OgmAttnPre none{nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f, 0u};
+  const OgmActDev no_act{};
+#define OGM_ATTN_PREFILL(HD_, G_)                                                                           \
+  hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, 0, true>), grid, dim3(512), 0, stream, q, (const float *)nullptr, \
+                     (const float *)nullptr, (const float2 *)nullptr, 0u, none, gq, (__half *)k_cache_layer,  \
+                     (__half *)v_cache_layer, pos0, max_splits, n_head_kv, scale, part_o, part_ml,            \
+                     (uint32_t *)nullptr, (float *)nullptr, no_act)
+  if (head_dim == 128 && G == 1) OGM_ATTN_PREFILL(128, 1);
+  else if (head_dim == 128 && G == 2) OGM_ATTN_PREFILL(128, 2);
+  else if (head_dim == 128 && G == 4) OGM_ATTN_PREFILL(128, 4);
+  else if (head_dim == 128 && G == 8) OGM_ATTN_PREFILL(128, 8);
+  else if (head_dim == 64 && G == 1) OGM_ATTN_PREFILL(64, 1);
+  else if (head_dim == 64 && G == 2) OGM_ATTN_PREFILL(64, 2);
+  else if (head_dim == 64 && G == 4) OGM_ATTN_PREFILL(64, 4);
+  else if (head_dim == 64 && G == 8) OGM_ATTN_PREFILL(64, 8);
+  else return hipErrorInvalidValue;
+#undef OGM_ATTN_PREFILL
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(ogm_attn_combine_rows_kernel, dim3((n + 255u) / 256u, n_tokens), dim3(64), 0, stream, part_o,
+                     part_ml, pos0, max_splits, n, head_dim, attn_out);
+  return hipGetLastError();
+}
+
+// h = silu(gate) * up over n values (all rows of a batch at once)
+__global__ __launch_bounds__(256) void ogm_swiglu_rows_kernel(const float *__restrict__ gate,
+                                                              const float *__restrict__ up, size_t n,
+                                                              float *__restrict__ h) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x * 4u;
+  for (size_t e0 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4u; e0 < n; e0 += stride) {
+    const float4 g = *(const float4 *)(gate + e0), u = *(const float4 *)(up + e0);
+    *(float4 *)(h + e0) = make_float4(g.x / (1.0f + expf(-g.x)) * u.x, g.y / (1.0f + expf(-g.y)) * u.y,
+                                      g.z / (1.0f + expf(-g.z)) * u.z, g.w / (1.0f + expf(-g.w)) * u.w);
+  }
+}
+
+hipError_t ogm_launch_swiglu_rows(const float *gate, const float *up, size_t n, float *h, hipStream_t stream) {
+  if (n == 0 || n % 4u != 0) return hipErrorInvalidValue;
+  size_t blocks = (n / 4u + 255u) / 256u;
+  if (blocks > 4096u) blocks = 4096u;
+  hipLaunchKernelGGL(ogm_swiglu_rows_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, gate, up, n, h);
   return hipGetLastError();
 }

@@ -65,7 +65,7 @@ PRE_SIZES = {"q_bias": lambda nh, nkv, hd: nh * hd, "k_bias": lambda nh, nkv, hd
 
 
 def build(be, *, n_embd, n_head, n_kv, hd, n_ff, n_vocab, n_layer, types, max_ctx, seed, rope_dim=None,
-          base=10000.0, pre=(), neox=False, freq_factors=None):
+          base=10000.0, pre=(), neox=False, freq_factors=None, attn_norm_scale=1.0):
     from orangu_amd import LlamaDecoder, QuantMatrix
     rng = np.random.default_rng(seed)
     tq, tv, tdown, tout = types
@@ -77,7 +77,7 @@ def build(be, *, n_embd, n_head, n_kv, hd, n_ff, n_vocab, n_layer, types, max_ct
                               mk(tv, n_embd, n_kv * hd, s + 3), mk(tq, n_head * hd, n_embd, s + 4),
                               mk(tq, n_embd, n_ff, s + 5), mk(tq, n_embd, n_ff, s + 6),
                               mk(tdown, n_ff, n_embd, s + 7),
-                              (1 + 0.1 * rng.standard_normal(n_embd)).astype(f32),
+                              (attn_norm_scale * (1 + 0.1 * rng.standard_normal(n_embd))).astype(f32),
                               (1 + 0.1 * rng.standard_normal(n_embd)).astype(f32)))
         for name in pre:   # biases of the projections' own size, norm weights around one
             n = PRE_SIZES[name](n_head, n_kv, hd)
@@ -217,7 +217,7 @@ def test_attention_head_shapes_across_a_chunk_boundary(be, hd, group, n_kv, wtyp
         dev.close()
 
 
-def prefill_both(ref, dev, rng, n_layer, n_pre, kv_dim):
+def fill_cache_both(ref, dev, rng, n_layer, n_pre, kv_dim):
     for l in range(n_layer):
         k = rng.standard_normal((n_pre, kv_dim)).astype(f32)
         v = rng.standard_normal((n_pre, kv_dim)).astype(f32)
@@ -236,7 +236,7 @@ def test_attention_with_odd_query_groups(be, hd, group, n_kv, wtype):
     ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=2,
                           types=(wtype, wtype, wtype, wtype), max_ctx=160, seed=3 * hd + group)
     try:
-        prefill_both(ref, dev, rng, 2, 127, n_kv * hd)
+        fill_cache_both(ref, dev, rng, 2, 127, n_kv * hd)
         for pos in range(127, 130):
             step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"hd {hd} group {group} pos {pos}")
     finally:
@@ -273,7 +273,7 @@ def test_bias_head_norm_pairing_and_frequency_factors(be, pre, neox, ff, rope_di
         dev.close()
     ref, dev, rng = build(be, **kw)
     try:
-        prefill_both(ref, dev, rng, 2, 127, n_kv * hd)
+        fill_cache_both(ref, dev, rng, 2, 127, n_kv * hd)
         for pos in (127, 128):
             step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"{pre} neox {neox} ff {ff} pos {pos}")
     finally:
@@ -329,6 +329,119 @@ def test_matrices_uploaded_from_a_gguf_file_multiply_like_direct_uploads(be, tmp
         xd.free()
         yd.free()
     g.close()
+
+
+# The synthetic K-quant weights give projections of magnitude 30 to 200 and with them attention
+# scores in the thousands: a softmax that picks one position, discontinuously.  Small attention
+# norm weights bring the scores of the batch tests to order one.
+TAME = {Q4_K: 0.02, Q5_K: 0.02, Q4_0: 0.1}
+
+
+def prefill_both(ref, dev, X, pos0, what, via_tokens=None):
+    """A batch of tokens on both sides, cache rows in lock-step as in `step_both`.  A flipped
+    activation rounding touches one token's rows from the next layer on.  Measured on 600 tokens of
+    the two-layer test model: about 50 such events (3e-5 per rounded element), each confined to one
+    token, moving its next rows by 1e-4 .. 2e-2 of their largest value (one quantizer step of one
+    activation times a column of the synthetic weights).  So up to 1 + T/8 tokens may be off the
+    tight bound by up to 5e-2, and the last token's outputs are compared loosely when it is among
+    them; an error of the code would show on every token, or be of order one."""
+    T = X.shape[0]
+    got_logits, got_tok = dev.prefill(X, pos0) if via_tokens is None else dev.prefill_tokens(via_tokens[0], via_tokens[1], pos0)
+    got_hidden = dev.hidden()
+    rows = [dev.kv_read(l, pos0, T) for l in range(dev.n_layer)]
+    flagged = set()
+
+    def hook(li, p, k_row, v_row):
+        out = []
+        for name, mine, theirs in (("k", k_row, rows[li][0][p - pos0]), ("v", v_row, rows[li][1][p - pos0])):
+            a, b = mine.astype(np.float64), theirs.astype(np.float64)
+            ulp = np.spacing(np.maximum(np.abs(mine), np.abs(theirs)).astype(np.float16)).astype(np.float64)
+            rowmax = np.abs(b).max()
+            if not (np.abs(a - b) <= ulp + 1e-5 * rowmax).all():
+                assert (np.abs(a - b) <= ulp + 5 * LOOSE * rowmax).all(), \
+                    f"{what}: position {p} layer {li} {name} cache row differs by more than one f16 step and the f32 budget"
+                flagged.add(p)
+            out.append(theirs.copy())
+        return out
+
+    ref.kv_hook = hook
+    want_logits, want_hidden = R.forward(ref, X, pos0)
+    ref.kv_hook = None
+    assert len(flagged) <= 1 + T // 8, f"{what}: {len(flagged)} of {T} tokens off the tight bound: {sorted(flagged)}"
+    tol = 5 * LOOSE if pos0 + T - 1 in flagged else TOL
+    for name, got, want in (("hidden state", got_hidden, want_hidden), ("logits", got_logits, want_logits)):
+        err = np.abs(np.asarray(got, np.float64) - want).max() / (np.abs(want).max() + 1e-30)
+        assert np.isfinite(got).all() and err <= tol, f"{what}: {name}: max error {err:.3e}"
+    top = np.sort(want_logits)[-2:]
+    if top[1] - top[0] > tol * np.abs(want_logits).max():
+        assert got_tok == R.argmax(want_logits), f"{what}: greedy token"
+    say(what, f"{T} tokens from {pos0}: flagged {sorted(flagged)}, token {got_tok}")
+
+
+@pytest.mark.parametrize("types", [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q5_K, Q3_K, Q6_K, Q5_K),
+                                   (Q4_0, Q5_0, IQ4_NL, Q8_0)])
+@pytest.mark.parametrize("n_tokens", [2, 7, 40])
+def test_prefill_from_an_empty_cache_then_decode(be, types, n_tokens):
+    """run_layers at n_tokens > 1 (llama.rs:594-932): 2 and 7 tokens take the multi-token GEMV in
+    the GEMM's float order, 40 the MFMA GEMMs; the decode steps after it continue on the cache the
+    prefill wrote."""
+    n_layer = 1 if Q3_K in types else 2    # two layers of the large synthetic Q3_K weights cancel badly
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=n_layer,
+                          types=types, max_ctx=64, seed=51, attn_norm_scale=TAME.get(types[0], 1.0))
+    try:
+        prefill_both(ref, dev, rng.standard_normal((n_tokens, 256)).astype(f32), 0, f"types {types}")
+        for pos in (n_tokens, n_tokens + 1):
+            step_both(ref, dev, rng.standard_normal(256).astype(f32), pos, f"types {types} then pos {pos}")
+    finally:
+        dev.close()
+
+
+@pytest.mark.parametrize("hd,group,n_kv,pre,neox,ff", [
+    (128, 4, 2, (), False, True),
+    (128, 3, 2, ("q_bias", "k_bias", "v_bias"), True, False),
+    (64, 7, 4, ("q_norm", "k_norm"), True, False),
+    (64, 8, 1, ("q_bias", "k_norm"), False, True),
+])
+def test_prefill_across_attention_chunks_and_in_two_parts(be, hd, group, n_kv, pre, neox, ff):
+    """A prompt in two calls (100 tokens, then 60 that cross position 128), each token attending to
+    the chunks its position has, with every option of the projections' post-processing."""
+    n_head = group * n_kv
+    n_embd = n_head * hd
+    factors = np.linspace(1.0, 8.0, hd // 4).astype(f32) if ff else None
+    wtype = Q4_K if n_embd % 256 == 0 else Q8_0
+    ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=2,
+                          types=(wtype, wtype, wtype, wtype), max_ctx=192, seed=61 + group, rope_dim=hd // 2,
+                          pre=pre, neox=neox, freq_factors=factors, attn_norm_scale=TAME.get(wtype, 1.0))
+    try:
+        prefill_both(ref, dev, rng.standard_normal((100, n_embd)).astype(f32), 0, f"hd {hd} group {group} part 1")
+        prefill_both(ref, dev, rng.standard_normal((60, n_embd)).astype(f32), 100, f"hd {hd} group {group} part 2")
+        step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), 160, f"hd {hd} group {group} then pos 160")
+    finally:
+        dev.close()
+
+
+def test_prefill_longer_than_one_pass_and_from_token_ids(be):
+    """600 tokens run as two passes over the layers (512 + 88); from token ids the embedding rows
+    are dequantized on the device (llama.rs:609-614) and give the same bits as rows passed in."""
+    import oracle
+    from orangu_amd import QuantMatrix
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=640, seed=71, attn_norm_scale=TAME[Q4_K])
+    embd_raw = synth_weights(Q6_K, 256, 320, seed=72)
+    table = oracle.dequantize(Q6_K, embd_raw, 320 * 256).reshape(320, 256)
+    tokens = rng.integers(0, 320, 600).astype(np.uint32)
+    try:
+        prefill_both(ref, dev, table[tokens], 0, "600 tokens by id", via_tokens=(QuantMatrix(embd_raw, Q6_K, 256, 320), tokens))
+        lg_ids = dev.prefill_tokens(QuantMatrix(embd_raw, Q6_K, 256, 320), tokens[:40], 0)[0]
+        lg_rows = dev.prefill(table[tokens[:40]], 0)[0]
+        assert np.array_equal(lg_ids.view(np.uint32), lg_rows.view(np.uint32))
+        from orangu_amd import OgmError
+        with pytest.raises(OgmError):
+            dev.prefill(table[tokens[:100]], 600)            # beyond the cache
+        with pytest.raises(OgmError):
+            dev.prefill_tokens(QuantMatrix(embd_raw, Q6_K, 256, 320), np.array([5, 320], np.uint32), 0)   # no such token
+    finally:
+        dev.close()
 
 
 def model_gguf(ref, arch, *, n_ctx=4096, tok_embd=None, vec_type=0, omit=(), extra_kvs=(), explicit=True):

@@ -332,12 +332,50 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     x = synth_x(T, in_dim, seed=T)
     w = qm(raw, Q4_K, in_dim, out_dim)
     say("gemm", in_dim, out_dim, T)
-    got = be.matmul(x, T, w)
-    # beyond 256 tokens the 128 x 256 tile kernel runs
-    assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 else "ogm_gemm_q4k_kernel")
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
+    got = be.matmul(x, T, w)
+    # beyond 256 tokens the 128 x 256 tile kernel runs once the 128 x 128 tiling would take more
+    # than one round of workgroups (256)
+    tiles = ((T + 127) // 128) * ((out_dim + 127) // 128)
+    assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 and tiles > 256 else "ogm_gemm_q4k_kernel")
     assert_close(got, want, "mfma gemm")
     assert_bits(got, want, "mfma gemm")
+    if T > 256:   # the wide kernel on this (small, ragged) shape as well
+        be.set_tuning("gemm_wide_min_wgs", 1)
+        try:
+            got = be.matmul(x, T, w)
+            assert be.last_kernel() == "ogm_gemm_q4k_wide_kernel"
+        finally:
+            be.set_tuning("gemm_wide_min_wgs", 0)
+        assert_bits(got, want, "wide mfma gemm")
+
+
+@pytest.mark.parametrize("n_tokens,outs,kernel", [
+    (40, (300, 130, 64), "ogm_gemm_q4k_kernel"),          # one round of 128 x 128 tiles
+    (300, (520, 70), "ogm_gemm_q4k_kernel"),              # more than 256 tokens, still one round
+    (300, (6000, 3000, 2100), "ogm_gemm_q4k_wide_kernel"),  # 264 tiles of 128 x 128: the wide tiling
+])
+def test_q4k_matrices_over_one_input_share_a_gemm_launch(be, n_tokens, outs, kernel):
+    """q / k / v (llama.rs:730-746) at prefill widths: Q4_K matrices over the same activations go
+    out as one launch whose row tiles run through the matrices in turn; every output bit equals
+    the CPU GEMM's, ragged last tiles included."""
+    from orangu_amd.hiprt import DeviceBuffer, device_synchronize
+    in_dim = 512
+    raws = [synth_weights(Q4_K, in_dim, od, seed=90 + i) for i, od in enumerate(outs)]
+    hs = [be.upload_raw(r, Q4_K, in_dim, od) for r, od in zip(raws, outs)]
+    x = synth_x(n_tokens, in_dim, seed=17)
+    xd = DeviceBuffer.from_numpy(x)
+    yds = [DeviceBuffer(4 * n_tokens * od) for od in outs]
+    be.matmul_multi_dev(hs, xd.ptr, n_tokens, [y.ptr for y in yds])
+    device_synchronize()
+    assert be.last_kernel() == kernel
+    for r, od, yd in zip(raws, outs, yds):
+        want = oracle.matmul(Q4_K, r, in_dim, od, x, n_tokens)
+        assert_bits(yd.to_numpy(np.float32, n_tokens * od), want, f"{od} rows of {outs}")
+    for h in hs:
+        be.free_weight(h)
+    for b in [xd] + yds:
+        b.free()
 
 
 def test_mfma_gemm_equals_small_batch_kernel_and_is_batch_independent(be):
@@ -385,7 +423,11 @@ def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T):
         x[:, 128:256] *= -1
         x[3] = -127.0
     raw = blocks.reshape(-1)
-    got = be.matmul(x, T, qm(raw, Q4_K, in_dim, out_dim))
+    be.set_tuning("gemm_wide_min_wgs", 1)   # beyond 256 tokens the wide kernel, however few tiles
+    try:
+        got = be.matmul(x, T, qm(raw, Q4_K, in_dim, out_dim))
+    finally:
+        be.set_tuning("gemm_wide_min_wgs", 0)
     assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 else "ogm_gemm_q4k_kernel")
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     assert_bits(got, want, "extreme ranges")

@@ -213,3 +213,43 @@ def test_first_position_sees_only_v_and_its_bias():
     assert not np.array_equal(other1, plain1)
     vb0, _ = run(dataclasses.replace(base, v_bias=np.full(n_kv * hd, 0.5, f32)))
     assert not np.array_equal(vb0, plain0)
+
+
+def test_prefill_of_several_tokens_matches_decoding_them_one_by_one():
+    """forward over T rows at once (GEMM float order, llama.rs:594-932 at n_tokens > 1) against T
+    single-token steps (GEMV order): the same cache rows and last logits up to f32 rounding, also
+    when the batch continues a cache that already holds positions; causality: the rows of the
+    earlier tokens do not move when later tokens join the batch."""
+    from helpers import Q4_K, Q6_K, synth_weights
+    rng = np.random.default_rng(11)
+    n_embd, n_head, n_kv, hd, n_ff, n_vocab = 256, 4, 2, 64, 256, 64
+    mk = lambda t, i, o, s: (t, synth_weights(t, i, o, seed=s), i, o)
+    layers = [R.Layer(mk(Q4_K, n_embd, n_head * hd, 1 + 10 * l), mk(Q4_K, n_embd, n_kv * hd, 2 + 10 * l),
+                      mk(Q6_K, n_embd, n_kv * hd, 3 + 10 * l), mk(Q4_K, n_head * hd, n_embd, 4 + 10 * l),
+                      mk(Q4_K, n_embd, n_ff, 5 + 10 * l), mk(Q4_K, n_embd, n_ff, 6 + 10 * l),
+                      mk(Q6_K, n_ff, n_embd, 7 + 10 * l), np.ones(n_embd, f32), np.ones(n_embd, f32),
+                      q_bias=rng.standard_normal(n_head * hd).astype(f32)) for l in range(2)]
+    new = lambda: R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 10000.0, layers, np.ones(n_embd, f32),
+                          mk(Q6_K, n_embd, n_vocab, 99), rope_neox=True, kv_dtype=np.float32)
+    X = rng.standard_normal((7, n_embd)).astype(f32)
+    one = new()
+    for t in range(7):
+        lg_one, h_one = R.decode_step(one, X[t], t)
+    batch = new()
+    lg_b, h_b = R.forward(batch, X, 0)
+    split = new()
+    R.forward(split, X[:3], 0)
+    lg_s, h_s = R.forward(split, X[3:], 3)
+    for other, lg, h in ((batch, lg_b, h_b), (split, lg_s, h_s)):
+        np.testing.assert_allclose(h, h_one, rtol=0, atol=2e-5 * np.abs(h_one).max())
+        np.testing.assert_allclose(lg, lg_one, rtol=0, atol=2e-5 * np.abs(lg_one).max())
+        for l in range(2):
+            a, b = np.stack(other.k_cache[l]), np.stack(one.k_cache[l])
+            np.testing.assert_allclose(a, b, rtol=0, atol=2e-5 * np.abs(b).max())
+            a, b = np.stack(other.v_cache[l]), np.stack(one.v_cache[l])
+            np.testing.assert_allclose(a, b, rtol=0, atol=2e-5 * np.abs(b).max())
+    short = new()
+    R.forward(short, X[:4], 0)
+    for l in range(2):   # bit for bit: rows of a GEMM do not depend on the other rows of the batch
+        np.testing.assert_array_equal(np.stack(short.k_cache[l]), np.stack(batch.k_cache[l])[:4])
+        np.testing.assert_array_equal(np.stack(short.v_cache[l]), np.stack(batch.v_cache[l])[:4])
