@@ -162,6 +162,11 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     for _ in range(3):
         dec.prefill_tokens(up("output"), prompt, 0)
     dt_pre = (time.perf_counter() - t0) / 3
+    long_prompt = rng.integers(0, n_vocab, 2048).astype(np.uint32)
+    dec.prefill_tokens(up("output"), long_prompt, 0)
+    t0 = time.perf_counter()
+    dec.prefill_tokens(up("output"), long_prompt, 0)
+    dt_pre_long = time.perf_counter() - t0
     weights = n_layer * sum(o * (i // 256) * (144 if t == Q4_K else 210) for t, i, o in shapes.values()) \
         + n_vocab * (n_embd // 256) * 210
     kv_bytes = 2 * n_layer * ctx * n_kv * hd * 2
@@ -169,6 +174,7 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
            "tok_per_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4),
            "generate_tok_per_s": round(1.0 / dt_gen, 1), "generated": [int(t) for t in toks[:4]],
            "prefill_512_ms": round(dt_pre * 1e3, 2), "prefill_tok_per_s": round(512 / dt_pre, 1),
+           "prefill_2048_ms": round(dt_pre_long * 1e3, 2), "prefill_2048_tok_per_s": round(2048 / dt_pre_long, 1),
            "bytes_per_token": weights + kv_bytes,
            "GBps": round((weights + kv_bytes) / dt / 1e9, 1),
            "frac_of_hbm_peak": round((weights + kv_bytes) / dt / 1e9 / HBM_PEAK_GBS, 4)}

@@ -246,7 +246,7 @@ int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_
  * through run_layers at n_tokens > 1 (llama.rs:594-932): the matmuls in the GEMM kernels' float order
  * (Backend::matmul, cpu.rs:445-458), K/V rows appended to the cache, causal attention; then the last
  * row alone through the output norm and projection (forward, llama.rs:1007-1032).  last_logits
- * ([n_vocab]) and argmax may each be null.  Runs in chunks of 512 tokens; synchronizes. */
+ * ([n_vocab]) and argmax may each be null.  Runs in chunks of 1024 tokens; synchronizes. */
 int ogm_llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos0, uint32_t n_tokens,
                       float *last_logits, uint32_t *argmax);
 /* The same from token ids (host), their embedding rows read on the device from an uploaded

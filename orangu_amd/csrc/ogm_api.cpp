@@ -1086,9 +1086,11 @@ extern "C" int ogm_dequant_rows(ogm_ctx *ctx, const ogm_weight *w, uint32_t row0
   const size_t bytes = (size_t)n_rows * w->in_dim * 4;
   int rc = ensure_dev(ctx, ctx->y, bytes);
   if (rc != OGM_OK) return rc;
-  for (uint32_t r = 0; r < n_rows; r++)
-    HIPCHK(ctx, ogm_launch_dequant_row(w->dev, w->ggml_type, w->in_dim, w->out_dim, row0 + r, nullptr,
+  for (uint32_t r = 0; r < n_rows; r += 32768u) {
+    const uint32_t nr = n_rows - r < 32768u ? n_rows - r : 32768u;
+    HIPCHK(ctx, ogm_launch_dequant_row(w->dev, w->ggml_type, w->in_dim, w->out_dim, row0 + r, nullptr, nr,
                                        (float *)ctx->y.p + (size_t)r * w->in_dim, ctx->stream));
+  }
   HIPCHK(ctx, hipMemcpyAsync(out, ctx->y.p, bytes, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   return OGM_OK;
@@ -1113,7 +1115,7 @@ extern "C" int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
   for (uint32_t i = 0; i < n_tokens; i++) {
     // the embedding row goes straight into the residual stream
     HIPCHK(ctx, ogm_launch_dequant_row(tok_embd->dev, tok_embd->ggml_type, tok_embd->in_dim, tok_embd->out_dim, 0,
-                                       toks + i, m->x, ctx->stream));
+                                       toks + i, 1, m->x, ctx->stream));
     rc = llama_decode_enqueue(ctx, m, m->x, pos0 + i, nullptr, toks + i + 1, ctx->stream);
     if (rc != OGM_OK) return rc;
   }
@@ -1126,7 +1128,7 @@ extern "C" int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
 
 // ---- prefill: run_layers at n_tokens > 1 (llama.rs:594-932) ------------------------------------
 
-static const uint32_t OGM_PREFILL_CHUNK = 512;             // tokens per pass over the layers
+static const uint32_t OGM_PREFILL_CHUNK = 1024;            // tokens per pass over the layers
 static const size_t OGM_PREFILL_PART_BYTES = 256u << 20;   // attention partials per launch
 
 static int llama_prefill_buffers(ogm_ctx *ctx, ogm_llama *m) {
@@ -1258,9 +1260,8 @@ static int llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x_host, const 
     if (tok_embd) {
       // the embedding rows (llama.rs:609-614), dequantized on the device
       HIPCHK(ctx, hipMemcpyAsync(m->pf.tokens, tokens + t0, (size_t)T * 4, hipMemcpyHostToDevice, s));
-      for (uint32_t i = 0; i < T; i++)
-        HIPCHK(ctx, ogm_launch_dequant_row(tok_embd->dev, tok_embd->ggml_type, tok_embd->in_dim, tok_embd->out_dim, 0,
-                                           m->pf.tokens + i, m->pf.x + (size_t)i * c.n_embd, s));
+      HIPCHK(ctx, ogm_launch_dequant_row(tok_embd->dev, tok_embd->ggml_type, tok_embd->in_dim, tok_embd->out_dim, 0,
+                                         m->pf.tokens, T, m->pf.x, s));
     } else {
       HIPCHK(ctx, hipMemcpyAsync(m->pf.x, x_host + (size_t)t0 * c.n_embd, (size_t)T * c.n_embd * 4,
                                  hipMemcpyHostToDevice, s));

@@ -65,10 +65,12 @@ hipError_t ogm_launch_argmax(const float *logits, uint32_t n, uint32_t *scratch,
 // f32 -> f16 (round to nearest even) for cache rows handed over by the host.
 hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStream_t stream);
 
-// Row `row` (or *row_dev when not null) of a tile-planar quantized matrix as f32 [in_dim]: the
-// embedding lookup (llama.rs:609-614 over quant.rs:639-649, 666-697, 746-787), bit-identical.
+// Rows row .. row + n_rows (or row_dev[0 .. n_rows) when not null) of a tile-planar quantized matrix
+// as f32 [n_rows][in_dim]: the embedding lookup (llama.rs:609-614 over quant.rs:639-649, 666-697,
+// 746-787), bit-identical.
 hipError_t ogm_launch_dequant_row(const uint8_t *wt, uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim,
-                                  uint32_t row, const uint32_t *row_dev, float *out, hipStream_t stream);
+                                  uint32_t row, const uint32_t *row_dev, uint32_t n_rows, float *out,
+                                  hipStream_t stream);
 
 // ---- the same layer over a batch of tokens (prefill, llama.rs:594-932 at n_tokens > 1) ----------
 // The matmuls between these are GEMMs that quantize their own input: plain f32 rows throughout.

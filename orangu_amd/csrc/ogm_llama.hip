@@ -735,7 +735,9 @@ __global__ __launch_bounds__(256) void ogm_dequant_row_kernel(const uint8_t *__r
                                                               float *__restrict__ out) {
   const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= in_dim) return;
-  if (row_dev) row = *row_dev;
+  // blockIdx.y: the n-th row asked for (row + n, or row_dev[n]) into the n-th output row
+  row = row_dev ? row_dev[blockIdx.y] : row + blockIdx.y;
+  out += (size_t)blockIdx.y * in_dim;
   if (row >= out_dim) row = out_dim - 1u;   // a token id beyond the table reads its last row
   OgmLayout l;
   ogm_layout_for(ggml_type, &l);
@@ -829,12 +831,14 @@ __global__ __launch_bounds__(256) void ogm_dequant_row_kernel(const uint8_t *__r
 }
 
 hipError_t ogm_launch_dequant_row(const uint8_t *wt, uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim,
-                                  uint32_t row, const uint32_t *row_dev, float *out, hipStream_t stream) {
+                                  uint32_t row, const uint32_t *row_dev, uint32_t n_rows, float *out,
+                                  hipStream_t stream) {
   OgmLayout l;
   if (!ogm_layout_for(ggml_type, &l) || in_dim == 0 || in_dim % l.block_elems != 0 || out_dim == 0)
     return hipErrorInvalidValue;
-  hipLaunchKernelGGL(ogm_dequant_row_kernel, dim3((in_dim + 255u) / 256u), dim3(256), 0, stream, wt, ggml_type,
-                     in_dim, out_dim, row, row_dev, out);
+  if (n_rows == 0 || n_rows > 65535u) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ogm_dequant_row_kernel, dim3((in_dim + 255u) / 256u, n_rows), dim3(256), 0, stream, wt,
+                     ggml_type, in_dim, out_dim, row, row_dev, out);
   return hipGetLastError();
 }
 

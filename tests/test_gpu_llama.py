@@ -342,9 +342,10 @@ def prefill_both(ref, dev, X, pos0, what, via_tokens=None):
     activation rounding touches one token's rows from the next layer on.  Measured on 600 tokens of
     the two-layer test model: about 50 such events (3e-5 per rounded element), each confined to one
     token, moving its next rows by 1e-4 .. 2e-2 of their largest value (one quantizer step of one
-    activation times a column of the synthetic weights).  So up to 1 + T/8 tokens may be off the
-    tight bound by up to 5e-2, and the last token's outputs are compared loosely when it is among
-    them; an error of the code would show on every token, or be of order one."""
+    activation times a column of the synthetic weights; over 1100 tokens the largest seen is 6e-2).
+    So up to 1 + T/8 tokens may be off the tight bound, by up to 0.2, and the last token's outputs
+    are compared loosely when it is among them; an error of the code would show on every token, or
+    be of order one.  All other tokens' rows match to 1e-5 plus one f16 step."""
     T = X.shape[0]
     got_logits, got_tok = dev.prefill(X, pos0) if via_tokens is None else dev.prefill_tokens(via_tokens[0], via_tokens[1], pos0)
     got_hidden = dev.hidden()
@@ -358,7 +359,7 @@ def prefill_both(ref, dev, X, pos0, what, via_tokens=None):
             ulp = np.spacing(np.maximum(np.abs(mine), np.abs(theirs)).astype(np.float16)).astype(np.float64)
             rowmax = np.abs(b).max()
             if not (np.abs(a - b) <= ulp + 1e-5 * rowmax).all():
-                assert (np.abs(a - b) <= ulp + 5 * LOOSE * rowmax).all(), \
+                assert (np.abs(a - b) <= ulp + 0.2 * rowmax).all(), \
                     f"{what}: position {p} layer {li} {name} cache row differs by more than one f16 step and the f32 budget"
                 flagged.add(p)
             out.append(theirs.copy())
@@ -368,7 +369,7 @@ def prefill_both(ref, dev, X, pos0, what, via_tokens=None):
     want_logits, want_hidden = R.forward(ref, X, pos0)
     ref.kv_hook = None
     assert len(flagged) <= 1 + T // 8, f"{what}: {len(flagged)} of {T} tokens off the tight bound: {sorted(flagged)}"
-    tol = 5 * LOOSE if pos0 + T - 1 in flagged else TOL
+    tol = 0.2 if pos0 + T - 1 in flagged else TOL
     for name, got, want in (("hidden state", got_hidden, want_hidden), ("logits", got_logits, want_logits)):
         err = np.abs(np.asarray(got, np.float64) - want).max() / (np.abs(want).max() + 1e-30)
         assert np.isfinite(got).all() and err <= tol, f"{what}: {name}: max error {err:.3e}"
@@ -421,23 +422,23 @@ def test_prefill_across_attention_chunks_and_in_two_parts(be, hd, group, n_kv, p
 
 
 def test_prefill_longer_than_one_pass_and_from_token_ids(be):
-    """600 tokens run as two passes over the layers (512 + 88); from token ids the embedding rows
+    """1100 tokens run as two passes over the layers (1024 + 76); from token ids the embedding rows
     are dequantized on the device (llama.rs:609-614) and give the same bits as rows passed in."""
     import oracle
     from orangu_amd import QuantMatrix
     ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
-                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=640, seed=71, attn_norm_scale=TAME[Q4_K])
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=1152, seed=71, attn_norm_scale=TAME[Q4_K])
     embd_raw = synth_weights(Q6_K, 256, 320, seed=72)
     table = oracle.dequantize(Q6_K, embd_raw, 320 * 256).reshape(320, 256)
-    tokens = rng.integers(0, 320, 600).astype(np.uint32)
+    tokens = rng.integers(0, 320, 1100).astype(np.uint32)
     try:
-        prefill_both(ref, dev, table[tokens], 0, "600 tokens by id", via_tokens=(QuantMatrix(embd_raw, Q6_K, 256, 320), tokens))
+        prefill_both(ref, dev, table[tokens], 0, "1100 tokens by id", via_tokens=(QuantMatrix(embd_raw, Q6_K, 256, 320), tokens))
         lg_ids = dev.prefill_tokens(QuantMatrix(embd_raw, Q6_K, 256, 320), tokens[:40], 0)[0]
         lg_rows = dev.prefill(table[tokens[:40]], 0)[0]
         assert np.array_equal(lg_ids.view(np.uint32), lg_rows.view(np.uint32))
         from orangu_amd import OgmError
         with pytest.raises(OgmError):
-            dev.prefill(table[tokens[:100]], 600)            # beyond the cache
+            dev.prefill(table[tokens[:100]], 1100)           # beyond the cache
         with pytest.raises(OgmError):
             dev.prefill_tokens(QuantMatrix(embd_raw, Q6_K, 256, 320), np.array([5, 320], np.uint32), 0)   # no such token
     finally:
