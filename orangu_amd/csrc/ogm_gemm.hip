@@ -1030,18 +1030,35 @@ __global__ __launch_bounds__(768) void ogm_gemm_flat_kernel(GemmFlatParams p) {
 // bits in ql[64h + 32(r&1) + 16k + j] (low nibble for r < 2, high for r >= 2), bits 4..5 in
 // qh[32h + 16k + j] >> 2r, and scale sc[8h + 2r + k].
 
+//
+// The same two chains carry the other K-quants whose scaled weights leave f16's exact range:
+//   Q3_K (a KKind::Q6K row, vecdot.rs:2100-2117): 16 groups with scales sc - 32 in [-32, 31] and
+//     weights in [-4, 3]; element 32p + l has its low two bits in qs[32(p/4) + l] >> 2(p%4) and its
+//     third bit, stored inverted, in bit p of hmask[l] (quant.rs:841-871).
+//   Q5_K (a KKind::Q4K row, vecdot.rs:2064-2088): 8 sub-blocks of 32 with scales in [0, 63] and
+//     unsigned weights in [0, 31] (nibble of qs[32(j/2) + l], fifth bit = bit j of qh[l]); chains
+//     3*31*127*256 = 3.0e6 and 15*31*127*256 = 1.5e7.  Its -dmin*m correction runs first, over
+//     every super-block, as in gemm_k_q4_k (vecdot.rs:2213-2255).
+
+#define GK_Q6K 0
+#define GK_Q3K 1
+#define GK_Q5K 2
+
 struct Gemm6Params {
-  const uint8_t *wt;      // tile-planar Q6_K
+  const uint8_t *wt;      // tile-planar weights
   const _Float16 *xh;     // [T][in_dim] int8 activations as f16
   const float *ad;        // [T][nsb] activation scales (per 256)
+  const int16_t *bsum;    // [T][in_dim / 32] sums of 32 activations (Q5_K's mins)
   float *y;               // [T][out_dim]
   uint32_t in_dim, out_dim, n_tokens, nsb;
   uint32_t c_shift, r_shift, nct;
 };
 
-#define G6_TILE_BYTES 13440u   // 64 units of 210 bytes: 13 pieces of 1 KiB, then 64 two-byte tails
-
-__global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) {
+template <int KIND>
+__device__ __forceinline__ void gemm_k2_body(const Gemm6Params &p) {
+  // bytes of a tile of 64 units: Q6_K 13 pieces of 1 KiB and 64 two-byte tails; Q3_K 7 pieces;
+  // Q5_K 11 pieces
+  constexpr uint32_t G6_TILE_BYTES = KIND == GK_Q6K ? 13440u : KIND == GK_Q3K ? 7168u : 11264u;
   extern __shared__ __align__(16) uint8_t lds[];
   _Float16 *Ah_l = (_Float16 *)lds;                 // [2][128][64]  a * (q - 32)
   _Float16 *Al_l = Ah_l + 2 * GM_STAGE_HALFS;       // [2][128][64]  b * (q - 32)
@@ -1074,8 +1091,84 @@ __global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) {
 #pragma unroll
   for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
 
+  if constexpr (KIND == GK_Q5K) {
+    // pass 1 (vecdot.rs:2226-2240): acc -= (ad * dmin) * imin for every super-block, imin the
+    // exact sum of the eight 6-bit mins times the sums of 32 activations.  A lane owns one token
+    // and 32 rows; the rows' mins and dmin of the super-block go through LDS.
+    // Four super-blocks per round (one trip to memory each): thread tid stages row tid % 128 of
+    // super-block s0 + tid / 128.
+    uint2 *mins_l = (uint2 *)lds;               // [4][128 rows] eight mins, one byte each
+    float *dmin_l = (float *)(lds + 4096);      // [4][128]
+    const uint32_t prow = min(r0 + (tid & 127u), p.out_dim - 1u);
+    const uint32_t punit = (prow >> p.r_shift) * p.nct * G6_TILE_BYTES + (prow & ((1u << p.r_shift) - 1u)) * 16u;
+    const int16_t *bs = p.bsum + (size_t)min(t0 + 32u * wt_ + l32, p.n_tokens - 1u) * p.nsb * 8u;
+    for (uint32_t s0 = 0; s0 < p.nsb; s0 += 4u) {
+      {
+        const uint32_t sx = min(s0 + (tid >> 7), p.nsb - 1u);
+        const uint4 z = *(const uint4 *)(p.wt + (punit + sb_tile(sx) + sb_lane(sx) * 16u));   // d, dmin, scales[12]
+        // get_scale_min_k4 (quant.rs:653-662): m_j = q[j+4] & 63 for j < 4, else (q[j+4] >> 4) | ((q[j] >> 6) << 4)
+        const uint32_t q1 = z.z, q2 = z.w;   // scales bytes 4..7, 8..11
+        uint2 mm;
+        mm.x = q1 & 0x3F3F3F3Fu;
+        mm.y = ((q2 >> 4) & 0x0F0F0F0Fu) | ((q1 >> 2) & 0x30303030u);
+        mins_l[tid] = mm;
+        dmin_l[tid] = gm_f16_bits_to_f32(z.x >> 16);
+      }
+      uint4 bqv[4];
+      float advv[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const uint32_t sx = min(s0 + (uint32_t)k, p.nsb - 1u);
+        bqv[k] = *(const uint4 *)(bs + (size_t)sx * 8u);
+        advv[k] = p.ad[tko + sx];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        if (s0 + (uint32_t)k >= p.nsb) break;
+        const uint4 bq = bqv[k];
+        const float adv1 = advv[k];
+        // each sum of 32 activations (|.| <= 4064) as 64 * hi + lo with lo in [0, 63], hi in
+        // [-64, 63]: four byte-wise dot products per row give the exact imin
+        uint32_t bl[2], bh[2];
+        {
+          const uint32_t w4[4] = {bq.x, bq.y, bq.z, bq.w};
+#pragma unroll
+          for (int h = 0; h < 2; h++) {
+            const int v0 = (int)(short)(w4[2 * h] & 0xFFFFu), v1 = (int)w4[2 * h] >> 16;
+            const int v2 = (int)(short)(w4[2 * h + 1] & 0xFFFFu), v3 = (int)w4[2 * h + 1] >> 16;
+            bl[h] = (uint32_t)(v0 & 63) | ((uint32_t)(v1 & 63) << 8) | ((uint32_t)(v2 & 63) << 16) |
+                    ((uint32_t)(v3 & 63) << 24);
+            bh[h] = ((uint32_t)(v0 >> 6) & 0xFFu) | (((uint32_t)(v1 >> 6) & 0xFFu) << 8) |
+                    (((uint32_t)(v2 >> 6) & 0xFFu) << 16) | (((uint32_t)(v3 >> 6) & 0xFFu) << 24);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const uint32_t rl = 128u * k + 64u * wr + 32u * i + 8u * q4 + 4u * lh + e;
+              const uint2 mm = mins_l[rl];
+              const int hi = __builtin_amdgcn_sdot4((int)mm.y, (int)bh[1], __builtin_amdgcn_sdot4((int)mm.x, (int)bh[0], 0, false), false);
+              const int lo = __builtin_amdgcn_sdot4((int)mm.y, (int)bl[1], __builtin_amdgcn_sdot4((int)mm.x, (int)bl[0], 0, false), false);
+              const int imin = hi * 64 + lo;
+              const float term = (adv1 * dmin_l[rl]) * (float)imin;
+              if (i == 0) y0[4 * q4 + e] -= term;
+              else y1[4 * q4 + e] -= term;
+            }
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+
   // loads run two stages ahead through three rotating register sets
   uint4 ql_0, ql_1, ql_2, qh_0, qh_1, qh_2, bx0_0, bx0_1, bx0_2, bx1_0, bx1_1, bx1_2;
+  uint4 hmx = make_uint4(0, 0, 0, 0);   // Q3_K / Q5_K: the thread's piece of the high-bit plane
+  uint32_t hmw[4] = {0, 0, 0, 0};
   uint4 scx = make_uint4(0, 0, 0, 0);   // the super-block's 16 scales
   uint32_t d16 = 0;
   uint32_t scw[4] = {0, 0, 0, 0};
@@ -1085,25 +1178,44 @@ __global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) {
   do {                                                                                            \
     const uint32_t uo_ = unit_off + sb_tile(S) + sb_lane(S) * 16u;                                \
     const uint32_t h_ = (G) >> 1;                                                                 \
-    if ((G) == 0) {                                                                               \
-      scx = *(const uint4 *)(p.wt + (uo_ + 12u * 1024u));                                         \
-      d16 = *(const uint16_t *)(p.wt + (tail_off + sb_tile(S) + sb_lane(S) * 2u));                \
+    if constexpr (KIND == GK_Q6K) {                                                               \
+      if ((G) == 0) {                                                                             \
+        scx = *(const uint4 *)(p.wt + (uo_ + 12u * 1024u));                                       \
+        d16 = *(const uint16_t *)(p.wt + (tail_off + sb_tile(S) + sb_lane(S) * 2u));              \
+      }                                                                                           \
+      ql_##K = *(const uint4 *)(p.wt + (uo_ + (4u * h_ + t16) * 1024u));                          \
+      qh_##K = *(const uint4 *)(p.wt + (uo_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));              \
+    } else if constexpr (KIND == GK_Q3K) {                                                        \
+      /* pieces: hmask 0..1, qs 2..5, then scales[12] | d | two bytes of padding */               \
+      if ((G) == 0) {                                                                             \
+        scx = *(const uint4 *)(p.wt + (uo_ + 6u * 1024u));                                        \
+        hmx = *(const uint4 *)(p.wt + (uo_ + (t16 & 1u) * 1024u));                                \
+      }                                                                                           \
+      ql_##K = *(const uint4 *)(p.wt + (uo_ + (2u + 2u * h_ + (t16 & 1u)) * 1024u));              \
+      qh_##K = ql_##K;                                                                            \
+    } else {                                                                                      \
+      /* pieces: d | dmin | scales[12], qh 1..2, qs 3..10 */                                      \
+      if ((G) == 0) {                                                                             \
+        scx = *(const uint4 *)(p.wt + uo_);                                                       \
+        hmx = *(const uint4 *)(p.wt + (uo_ + (1u + (t16 & 1u)) * 1024u));                         \
+      }                                                                                           \
+      ql_##K = *(const uint4 *)(p.wt + (uo_ + (3u + 2u * (G) + (t16 & 1u)) * 1024u));             \
+      qh_##K = ql_##K;                                                                            \
     }                                                                                             \
-    ql_##K = *(const uint4 *)(p.wt + (uo_ + (4u * h_ + t16) * 1024u));                            \
-    qh_##K = *(const uint4 *)(p.wt + (uo_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));                \
     const uint32_t ko_ = (S) * 256u + (G) * 64u;                                                  \
     bx0_##K = *(const uint4 *)(p.xh + (bo0 + ko_));                                               \
     bx1_##K = *(const uint4 *)(p.xh + (bo1 + ko_));                                               \
   } while (0)
 
-  // Four bytes of 6-bit values (still carrying the +32) -> (v - 32) * a and (v - 32) * b as f16
+  // Four bytes of small unsigned values v -> (v - zero point) * a and (v - zero point) * b as f16
+  // (zero point 32 for Q6_K, 4 for Q3_K, 0 for Q5_K)
 #define G6_DEQ(V, HI01, HI23, LO01, LO23)                                                         \
   do {                                                                                            \
     union { uint32_t u; half2v h; } e_, f_;                                                       \
     e_.u = __builtin_amdgcn_perm(0u, (V), 0x0c010c00u) | 0x64006400u; /* 1024 + v */              \
     f_.u = __builtin_amdgcn_perm(0u, (V), 0x0c030c02u) | 0x64006400u;                             \
-    e_.h = e_.h + k1056_;                                                                         \
-    f_.h = f_.h + k1056_;                                                                         \
+    e_.h = e_.h + koff_;                                                                          \
+    f_.h = f_.h + koff_;                                                                          \
     union { uint32_t u; half2v h; } o_;                                                           \
     o_.h = e_.h * a2_; HI01 = o_.u;                                                               \
     o_.h = f_.h * a2_; HI23 = o_.u;                                                               \
@@ -1115,22 +1227,57 @@ __global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) {
   do {                                                                                            \
     if ((G) == 0) {                                                                               \
       scw[0] = scx.x; scw[1] = scx.y; scw[2] = scx.z; scw[3] = scx.w;                             \
-      dnext = gm_f16_bits_to_f32(d16);                                                            \
+      hmw[0] = hmx.x; hmw[1] = hmx.y; hmw[2] = hmx.z; hmw[3] = hmx.w;                             \
+      if constexpr (KIND == GK_Q6K) dnext = gm_f16_bits_to_f32(d16);                              \
+      else if constexpr (KIND == GK_Q3K) dnext = gm_f16_bits_to_f32(scx.w & 0xFFFFu);             \
+      else dnext = gm_f16_bits_to_f32(scx.x & 0xFFFFu);                                           \
     }                                                                                             \
     /* scale of group 4G + t16, split as 16 a + b */                                              \
-    const uint32_t sw_ = (G) == 0 ? scw[0] : (G) == 1 ? scw[1] : (G) == 2 ? scw[2] : scw[3];      \
-    const int sc_ = (int)(int8_t)((sw_ >> (8u * t16)) & 0xFFu);                                   \
+    int sc_;                                                                                      \
+    uint32_t zp_;      /* zero point of the stored values, as f16 bits of -(1024 + zero point) */ \
+    if constexpr (KIND == GK_Q6K) {                                                               \
+      const uint32_t sw_ = (G) == 0 ? scw[0] : (G) == 1 ? scw[1] : (G) == 2 ? scw[2] : scw[3];    \
+      sc_ = (int)(int8_t)((sw_ >> (8u * t16)) & 0xFFu);                                           \
+      zp_ = 1056u;                                                                                \
+    } else if constexpr (KIND == GK_Q3K) {                                                        \
+      /* quant.rs:883-897: scale i = 4G + t16 has its low four bits in a nibble of byte i % 8 and \
+         its two high bits at bit 2 (i / 4) of byte 8 + i % 4; all biased by 32 */                \
+      const uint32_t lw_ = ((G) & 1u) ? scw[1] : scw[0];      /* bytes 4(G&1) .. 4(G&1) + 3 */     \
+      const uint32_t low_ = ((lw_ >> (8u * t16)) >> ((G) >= 2 ? 4u : 0u)) & 0xFu;                 \
+      const uint32_t high_ = ((scw[2] >> (8u * t16)) >> (2u * (G))) & 3u;                         \
+      sc_ = (int)(low_ | (high_ << 4)) - 32;                                                      \
+      zp_ = 1028u;                                                                                \
+    } else {                                                                                      \
+      /* get_scale_min_k4 (quant.rs:653-662) of sub-block j = 2G + t16/2 over scales bytes        \
+         q[0..12) = scw[1..3]: sc = q[j] & 63 for j < 4, else (q[j+4] & 15) | ((q[j-4] >> 6) << 4) */ \
+      const uint32_t j_ = 2u * (G) + (t16 >> 1);                                                  \
+      const uint32_t qa_ = (scw[1] >> (8u * (j_ & 3u))) & 0xFFu;  /* q[j] or q[j-4] */            \
+      const uint32_t qb_ = (scw[3] >> (8u * (j_ & 3u))) & 0xFFu;  /* q[j+4] for j >= 4 */         \
+      sc_ = (G) < 2 ? (int)(qa_ & 63u) : (int)((qb_ & 15u) | ((qa_ >> 6) << 4));                  \
+      zp_ = 1024u;                                                                                \
+    }                                                                                             \
     const _Float16 af_ = (_Float16)(float)(sc_ >> 4), bf_ = (_Float16)(float)(sc_ & 15);          \
     const half2v a2_ = {af_, af_}, b2_ = {bf_, bf_};                                              \
-    const half2v k1056_ = {(_Float16)-1056.0f, (_Float16)-1056.0f};                               \
+    const _Float16 kz_ = (_Float16)(-(float)zp_);                                                 \
+    const half2v koff_ = {kz_, kz_};                                                              \
     const uint32_t m4_ = 0x0F0F0F0Fu, m2_ = 0x30303030u;                                          \
     const uint32_t rr_ = 2u * ((G) & 1u) + (t16 >> 1);        /* run of 32 inside the half block */ \
     const uint32_t qlw_[4] = {ql_##K.x, ql_##K.y, ql_##K.z, ql_##K.w};                            \
     const uint32_t qhw_[4] = {qh_##K.x, qh_##K.y, qh_##K.z, qh_##K.w};                            \
     uint32_t hi_[8], lo_[8];                                                                      \
     _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
-      const uint32_t nib_ = (((G) & 1u) ? (qlw_[w_] >> 4) : qlw_[w_]) & m4_;                      \
-      const uint32_t v_ = nib_ | ((((qhw_[w_] >> (2u * rr_)) << 4)) & m2_);                       \
+      uint32_t v_;                                                                                \
+      if constexpr (KIND == GK_Q6K) {                                                             \
+        const uint32_t nib_ = (((G) & 1u) ? (qlw_[w_] >> 4) : qlw_[w_]) & m4_;                    \
+        v_ = nib_ | ((((qhw_[w_] >> (2u * rr_)) << 4)) & m2_);                                    \
+      } else if constexpr (KIND == GK_Q3K) {                                                      \
+        /* run p = 2G + t16/2 of 32: two bits at 2 (p % 4) = 2 rr, third bit = bit p of hmask */  \
+        v_ = ((qlw_[w_] >> (2u * rr_)) & 0x03030303u) |                                           \
+             (((hmw[w_] >> (2u * (G) + (t16 >> 1))) & 0x01010101u) << 2);                         \
+      } else {                                                                                    \
+        const uint32_t nib_ = ((t16 >> 1) ? (qlw_[w_] >> 4) : qlw_[w_]) & m4_;                    \
+        v_ = nib_ | (((hmw[w_] >> (2u * (G) + (t16 >> 1))) & 0x01010101u) << 4);                  \
+      }                                                                                           \
       G6_DEQ(v_, hi_[2 * w_], hi_[2 * w_ + 1], lo_[2 * w_], lo_[2 * w_ + 1]);                     \
     }                                                                                             \
     _Float16 *ah_ = Ah_l + (BUF) * GM_STAGE_HALFS, *al_ = Al_l + (BUF) * GM_STAGE_HALFS;          \
@@ -1238,6 +1385,10 @@ __global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) {
   }
 }
 
+__global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) { gemm_k2_body<GK_Q6K>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q3k_kernel(Gemm6Params p) { gemm_k2_body<GK_Q3K>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q5k_kernel(Gemm6Params p) { gemm_k2_body<GK_Q5K>(p); }
+
 static const uint32_t G6_LDS_BYTES = 6 * GM_STAGE_HALFS * 2 + 2 * 128 * 4;
 
 static const uint32_t GM_LDS_BYTES = 4 * GM_STAGE_HALFS * 2 + 2 * 128 * 16 * 2 + 128 * 4;
@@ -1261,10 +1412,12 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
     return (uint64_t)ogm_tiling_for(in_dim / 32u, out_dim).nrb * 64u * (in_dim / 32u) * l.block_bytes <= lim &&
            (uint64_t)in_dim * n_tokens <= lim;
   }
-  if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K) || in_dim == 0 || in_dim % 256u != 0) return false;
+  if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K && ggml_type != OGM_Q3_K && ggml_type != OGM_Q5_K) ||
+      in_dim == 0 || in_dim % 256u != 0)
+    return false;
   // Q4_K's pass 1 keeps one f32 per (row, super-block) of the workgroup in LDS
   if (ggml_type == OGM_Q4_K && GM_LDS_BYTES + (size_t)(in_dim / 256u) * 512u > GM_LDS_MAX) return false;
-  const uint64_t block = ggml_type == OGM_Q4_K ? 144u : 210u;
+  const uint64_t block = ggml_type == OGM_Q4_K ? 144u : ggml_type == OGM_Q6_K ? 210u : ggml_type == OGM_Q3_K ? 112u : 176u;
   return (uint64_t)ogm_tiling_for(in_dim / 256u, out_dim).nrb * 64u * (in_dim / 256u) * block <= lim &&
          (uint64_t)in_dim * n_tokens * 2u <= lim;
 }
@@ -1321,11 +1474,12 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   // power-of-two number of token tiles each XCD's L2 sees few distinct activation tiles
   const dim3 grid((a.n_tokens + GM_BT - 1) / GM_BT, row_tiles);
   hipError_t e;
-  if (a.ggml_type == OGM_Q6_K) {
+  if (a.ggml_type != OGM_Q4_K) {
     Gemm6Params p;
     p.wt = a.wt;
     p.xh = xh;
     p.ad = a.act.d;
+    p.bsum = a.act.bsum;
     p.y = a.y;
     p.in_dim = a.in_dim;
     p.out_dim = a.out_dim;
@@ -1335,11 +1489,21 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.r_shift = 6 - c_shift;
     p.nct = tl.nct;
     // more dynamic LDS than the 64 KB a kernel gets without asking
-    e = hipFuncSetAttribute((const void *)ogm_gemm_q6k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)G6_LDS_BYTES);
+    const void *fn = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_q6k_kernel
+                     : a.ggml_type == OGM_Q3_K ? (const void *)ogm_gemm_q3k_kernel
+                                               : (const void *)ogm_gemm_q5k_kernel;
+    e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)G6_LDS_BYTES);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(ogm_gemm_q6k_kernel, grid, dim3(512), G6_LDS_BYTES, stream, p);
-    if (kernel_name) *kernel_name = "ogm_gemm_q6k_kernel";
+    if (a.ggml_type == OGM_Q6_K) {
+      hipLaunchKernelGGL(ogm_gemm_q6k_kernel, grid, dim3(512), G6_LDS_BYTES, stream, p);
+      if (kernel_name) *kernel_name = "ogm_gemm_q6k_kernel";
+    } else if (a.ggml_type == OGM_Q3_K) {
+      hipLaunchKernelGGL(ogm_gemm_q3k_kernel, grid, dim3(512), G6_LDS_BYTES, stream, p);
+      if (kernel_name) *kernel_name = "ogm_gemm_q3k_kernel";
+    } else {
+      hipLaunchKernelGGL(ogm_gemm_q5k_kernel, grid, dim3(512), G6_LDS_BYTES, stream, p);
+      if (kernel_name) *kernel_name = "ogm_gemm_q5k_kernel";
+    }
     return hipGetLastError();
   }
   GemmParams p;

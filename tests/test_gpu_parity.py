@@ -490,6 +490,89 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign):
     say("extreme q6k isum", int(np.abs(isum).max()))
 
 
+@pytest.mark.parametrize("t,kernel", [(Q3_K, "ogm_gemm_q3k_kernel"), (Q5_K, "ogm_gemm_q5k_kernel")])
+@pytest.mark.parametrize("in_dim,out_dim,T", [
+    (256, 5, 9), (512, 130, 17), (768, 64, 129), (1024, 100, 64), (1280, 257, 40), (2048, 37, 128),
+    (4096, 200, 130), (14336, 96, 257), (4096, 1000, 512), (1792, 33, 10),
+])
+def test_mfma_gemm_q3k_q5k_match_cpu_gemm(be, t, kernel, in_dim, out_dim, T):
+    """Q3_K (a KKind::Q6K row, vecdot.rs:2100-2117) and Q5_K (a KKind::Q4K row, :2064-2088) on the
+    two-chain MFMA kernel: every bit of gemm_k_q6_k / gemm_k_q4_k (vecdot.rs:2213-2255, 2352-2398),
+    and of the multi-token GEMV that served these types before."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T + 1)
+    w = qm(raw, t, in_dim, out_dim)
+    say("gemm", kernel, in_dim, out_dim, T)
+    got = be.matmul(x, T, w)
+    assert be.last_kernel() == kernel
+    want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
+    assert_close(got, want, kernel)
+    assert_bits(got, want, kernel)
+    be.set_tuning("gemm_min_tokens", 100000)
+    try:
+        small = be.matmul(x, T, w)
+        assert be.last_kernel().startswith("ogm_gemv_kernel")
+    finally:
+        be.set_tuning("gemm_min_tokens", 0)
+    assert_bits(got, small, "mfma vs multi-token gemv")
+
+
+@pytest.mark.parametrize("qs,qh,sc,sign", [(0xFF, 0xFF, 0xFF, "alt"), (0x00, 0x00, 0xFF, "pos"), (0xFF, 0xFF, 0xFF, "neg"),
+                                           (0xFF, 0xFF, 0x3F, "block"), (0xF0, 0x55, 0xC7, "alt"), (0x0F, 0xAA, 0x00, "pos")])
+def test_mfma_gemm_q5k_adversarial_integer_ranges(be, qs, qh, sc, sign):
+    """Weights 0 and 31, scales and mins 63, activations +-127: a super-block's sum reaches
+    63 * 31 * 127 * 256 = 6.3e7 and the mins' 63 * 8 * 4064 = 2.0e6; the two scale digits' chains
+    stay exact and 16 * c_hi + c_lo rounds like `isum as f32`."""
+    in_dim, out_dim, T = 1024, 32, 16
+    blocks = np.zeros((out_dim * 4, 176), np.uint8)
+    blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    blocks[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
+    blocks[:, 4:16] = sc
+    blocks[:, 16:48] = qh
+    blocks[:, 48:176] = qs
+    x = np.full((T, in_dim), 127.0, np.float32)
+    if sign == "alt":
+        x[1::2] *= -1
+        x[:, ::7] = 126.0
+    elif sign == "neg":
+        x *= -1
+    elif sign == "block":
+        x[:, 128:256] *= -1
+        x[3] = -127.0
+    raw = blocks.reshape(-1)
+    got = be.matmul(x, T, qm(raw, Q5_K, in_dim, out_dim))
+    assert be.last_kernel() == "ogm_gemm_q5k_kernel"
+    assert_bits(got, oracle.matmul(Q5_K, raw, in_dim, out_dim, x, T), "extreme ranges")
+    isum, imin = be.dump_block_sums(x[0], 1, qm(raw, Q5_K, in_dim, out_dim))
+    say("extreme q5k isum", int(np.abs(isum).max()), "imin", int(np.abs(imin).max()))
+
+
+@pytest.mark.parametrize("qs,hm,sc,sign", [(0xFF, 0xFF, 0xFF, "alt"), (0x00, 0x00, 0x00, "pos"), (0x00, 0x00, 0xFF, "neg"),
+                                           (0xFF, 0x00, 0x00, "block"), (0x1B, 0x5A, 0x9C, "alt"), (0xE4, 0xA5, 0x63, "pos")])
+def test_mfma_gemm_q3k_adversarial_integer_ranges(be, qs, hm, sc, sign):
+    """Weights -4 and 3, scales -32 and 31 (every six-bit pattern's bytes at their extremes) and
+    activations +-127."""
+    in_dim, out_dim, T = 1024, 32, 16
+    blocks = np.zeros((out_dim * 4, 110), np.uint8)
+    blocks[:, 0:32] = hm
+    blocks[:, 32:96] = qs
+    blocks[:, 96:108] = sc
+    blocks[:, 108:110] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    x = np.full((T, in_dim), 127.0, np.float32)
+    if sign == "alt":
+        x[1::2] *= -1
+        x[:, ::7] = 126.0
+    elif sign == "neg":
+        x *= -1
+    elif sign == "block":
+        x[:, 128:256] *= -1
+        x[3] = -127.0
+    raw = blocks.reshape(-1)
+    got = be.matmul(x, T, qm(raw, Q3_K, in_dim, out_dim))
+    assert be.last_kernel() == "ogm_gemm_q3k_kernel"
+    assert_bits(got, oracle.matmul(Q3_K, raw, in_dim, out_dim, x, T), "extreme ranges")
+
+
 # ---------------------------------------------------------------- quantize inside the GEMV, grouped launches
 
 @pytest.mark.parametrize("t,in_dim,out_dim", [
