@@ -239,7 +239,7 @@ def main() -> int:
 
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only; --gpus N with N > 1 is not supported "
-              "(the path has no collectives; see DESIGN.md for how it would shard).", file=sys.stderr)
+              "(the path has no collectives).", file=sys.stderr)
         return 2
 
     import helpers

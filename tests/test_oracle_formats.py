@@ -1,22 +1,18 @@
 """Pins the oracle's block formats against what the reference's own tests hold
 (engine/quant.rs tests, cited per case).  CPU only."""
+import json
+import os
+
 import numpy as np
 import pytest
 
 import oracle
 from helpers import IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0
 
-# quant.rs:1389-1417 GOLDEN (the types on the path)
-GOLDEN = [
-    (Q4_0, "q4_0", 256, 0x162325C968C10725),
-    (Q5_0, "q5_0", 256, 0x813F8949E12B3725),
-    (Q8_0, "q8_0", 256, 0xC5D58782F54E52E5),
-    (IQ4_NL, "iq4_nl", 256, 0x7956C82FEBA12125),
-    (Q3_K, "q3_k", 512, 0x2183E0B0538C6BE5),
-    (Q4_K, "q4_k", 512, 0x9A7268A432A5C5FA),
-    (Q5_K, "q5_k", 512, 0x41C70B9BE1696E6D),
-    (Q6_K, "q6_k", 512, 0x61001D333CB0CFD1),
-]
+# quant.rs:1389-1417 GOLDEN (the types on the path), kept as data in tests/golden/
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "dequantize_checksums.json")) as _f:
+    GOLDEN = [(v["ggml_type"], v["name"], v["count"], int(v["checksum"], 16)) for v in json.load(_f)["vectors"]]
+assert {g[0] for g in GOLDEN} == {Q4_0, Q5_0, Q8_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K}
 
 
 @pytest.mark.parametrize("ggml_type,name,count,expected", GOLDEN)
