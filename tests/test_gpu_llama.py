@@ -397,6 +397,31 @@ def test_prefill_from_an_empty_cache_then_decode(be, types, n_tokens):
         dev.close()
 
 
+def test_prefill_of_one_token_is_a_decode_step(be):
+    """n_tokens == 1 through the batch entry point: the single-token kernels' float order
+    (Backend::matmul at one token, cpu.rs:445-458), the same cache row and logits as the step."""
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=8, seed=81)
+    ref2, dev2, _ = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=8, seed=81)
+    try:
+        for pos in range(3):
+            x = rng.standard_normal(256).astype(f32)
+            step_both(ref, dev, x, pos, f"step pos {pos}")
+            lg_step, tok_step = dev.decode(x, pos)      # the same step again: same cache row, same logits
+            lg_batch, tok_batch = dev2.prefill(x[None, :], pos)
+            close(lg_batch, lg_step, f"one-token prefill pos {pos}")
+            for l in range(2):
+                ks, vs = dev.kv_read(l, pos, 1)
+                kb, vb = dev2.kv_read(l, pos, 1)
+                assert np.abs(ks.astype(f32) - kb.astype(f32)).max() <= 2e-3 * np.abs(ks.astype(f32)).max()
+                assert np.abs(vs.astype(f32) - vb.astype(f32)).max() <= 2e-3 * np.abs(vs.astype(f32)).max()
+        prefill_both(ref, dev, rng.standard_normal((1, 256)).astype(f32), 3, "one token as a batch")
+    finally:
+        dev.close()
+        dev2.close()
+
+
 @pytest.mark.parametrize("hd,group,n_kv,pre,neox,ff", [
     (128, 4, 2, (), False, True),
     (128, 3, 2, ("q_bias", "k_bias", "v_bias"), True, False),
