@@ -1048,11 +1048,13 @@ struct Gemm6Params {
   const uint8_t *wt;      // tile-planar weights
   const _Float16 *xh;     // [T][in_dim] int8 activations as f16
   const float *ad;        // [T][nsb] activation scales (per 256)
-  const int16_t *bsum;    // [T][in_dim / 32] sums of 32 activations (Q5_K's mins)
+  const _Float16 *bs16;   // [T][nsb][16]: floor(bsum_j / 64) for j = 0..7, then bsum_j mod 64 (Q5_K's mins)
   float *y;               // [T][out_dim]
   uint32_t in_dim, out_dim, n_tokens, nsb;
   uint32_t c_shift, r_shift, nct;
 };
+
+#define G6_LDS_BYTES_STATIC (6u * GM_STAGE_HALFS * 2u + 2u * 128u * 4u)   // three tiles, two buffers each, and d
 
 template <int KIND>
 __device__ __forceinline__ void gemm_k2_body(const Gemm6Params &p) {
@@ -1092,77 +1094,65 @@ __device__ __forceinline__ void gemm_k2_body(const Gemm6Params &p) {
   for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
 
   if constexpr (KIND == GK_Q5K) {
-    // pass 1 (vecdot.rs:2226-2240): acc -= (ad * dmin) * imin for every super-block, imin the
-    // exact sum of the eight 6-bit mins times the sums of 32 activations.  A lane owns one token
-    // and 32 rows; the rows' mins and dmin of the super-block go through LDS.
-    // Four super-blocks per round (one trip to memory each): thread tid stages row tid % 128 of
-    // super-block s0 + tid / 128.
-    uint2 *mins_l = (uint2 *)lds;               // [4][128 rows] eight mins, one byte each
-    float *dmin_l = (float *)(lds + 4096);      // [4][128]
-    const uint32_t prow = min(r0 + (tid & 127u), p.out_dim - 1u);
-    const uint32_t punit = (prow >> p.r_shift) * p.nct * G6_TILE_BYTES + (prow & ((1u << p.r_shift) - 1u)) * 16u;
-    const int16_t *bs = p.bsum + (size_t)min(t0 + 32u * wt_ + l32, p.n_tokens - 1u) * p.nsb * 8u;
-    for (uint32_t s0 = 0; s0 < p.nsb; s0 += 4u) {
-      {
-        const uint32_t sx = min(s0 + (tid >> 7), p.nsb - 1u);
-        const uint4 z = *(const uint4 *)(p.wt + (punit + sb_tile(sx) + sb_lane(sx) * 16u));   // d, dmin, scales[12]
-        // get_scale_min_k4 (quant.rs:653-662): m_j = q[j+4] & 63 for j < 4, else (q[j+4] >> 4) | ((q[j] >> 6) << 4)
-        const uint32_t q1 = z.z, q2 = z.w;   // scales bytes 4..7, 8..11
-        uint2 mm;
-        mm.x = q1 & 0x3F3F3F3Fu;
-        mm.y = ((q2 >> 4) & 0x0F0F0F0Fu) | ((q1 >> 2) & 0x30303030u);
-        mins_l[tid] = mm;
-        dmin_l[tid] = gm_f16_bits_to_f32(z.x >> 16);
+    // pass 1 (vecdot.rs:2226-2240): acc -= (ad * dmin) * imin for every super-block first, imin =
+    // sum_j m_j * bsum_j on the matrix cores exactly as the Q4_K kernel forms it (the two formats
+    // share their 16-byte header): operand k 0..7 = 64 m_j against floor(bsum_j / 64), k 8..15 =
+    // m_j against bsum_j mod 64, all exact in f16, the sum below 2^24.
+    float *dmin_t = (float *)(lds + G6_LDS_BYTES_STATIC);   // [nsb][128]
+    auto unit_of = [&](uint32_t row) -> uint32_t {
+      row = min(row, p.out_dim - 1u);
+      return (row >> p.r_shift) * p.nct * G6_TILE_BYTES + (row & ((1u << p.r_shift) - 1u)) * 16u;
+    };
+    for (uint32_t i = tid; i < p.nsb * 128u; i += 512u) {
+      const uint32_t s = i >> 7, lr = i & 127u;
+      const uint32_t h = *(const uint32_t *)(p.wt + (unit_of(r0 + lr) + sb_tile(s) + sb_lane(s) * 16u));
+      dmin_t[i] = gm_f16_bits_to_f32(h >> 16);
+    }
+    __syncthreads();
+    const uint32_t ro0 = unit_of(r0 + 64u * wr + l32), ro1 = unit_of(r0 + 64u * wr + 32u + l32);
+    const float side_scale = lh ? 1.0f : 64.0f;
+    // four super-blocks at a time, so that four sets of loads share one trip to memory
+#pragma unroll 1
+    for (uint32_t sg = 0; sg < p.nsb; sg += 4u) {
+      uint4 hd0[4], hd1[4];
+      half8 b2[4];
+      float adv1[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const uint32_t su = min(sg + u, p.nsb - 1u);
+        const uint32_t so = sb_tile(su) + sb_lane(su) * 16u;
+        hd0[u] = *(const uint4 *)(p.wt + (ro0 + so));
+        hd1[u] = *(const uint4 *)(p.wt + (ro1 + so));
+        b2[u] = *(const half8 *)(p.bs16 + ((tko + su) * 16u + 8u * lh));
+        adv1[u] = p.ad[tko + su];
       }
-      uint4 bqv[4];
-      float advv[4];
 #pragma unroll
-      for (int k = 0; k < 4; k++) {
-        const uint32_t sx = min(s0 + (uint32_t)k, p.nsb - 1u);
-        bqv[k] = *(const uint4 *)(bs + (size_t)sx * 8u);
-        advv[k] = p.ad[tko + sx];
-      }
-      __syncthreads();
-#pragma unroll
-      for (int k = 0; k < 4; k++) {
-        if (s0 + (uint32_t)k >= p.nsb) break;
-        const uint4 bq = bqv[k];
-        const float adv1 = advv[k];
-        // each sum of 32 activations (|.| <= 4064) as 64 * hi + lo with lo in [0, 63], hi in
-        // [-64, 63]: four byte-wise dot products per row give the exact imin
-        uint32_t bl[2], bh[2];
-        {
-          const uint32_t w4[4] = {bq.x, bq.y, bq.z, bq.w};
-#pragma unroll
-          for (int h = 0; h < 2; h++) {
-            const int v0 = (int)(short)(w4[2 * h] & 0xFFFFu), v1 = (int)w4[2 * h] >> 16;
-            const int v2 = (int)(short)(w4[2 * h + 1] & 0xFFFFu), v3 = (int)w4[2 * h + 1] >> 16;
-            bl[h] = (uint32_t)(v0 & 63) | ((uint32_t)(v1 & 63) << 8) | ((uint32_t)(v2 & 63) << 16) |
-                    ((uint32_t)(v3 & 63) << 24);
-            bh[h] = ((uint32_t)(v0 >> 6) & 0xFFu) | (((uint32_t)(v1 >> 6) & 0xFFu) << 8) |
-                    (((uint32_t)(v2 >> 6) & 0xFFu) << 16) | (((uint32_t)(v3 >> 6) & 0xFFu) << 24);
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
+      for (int u = 0; u < 4; u++) {
+        if (sg + u < p.nsb) {
+          uint32_t mna, mnb;
+          q4k_mins(hd0[u], mna, mnb);
+          const half8 a10 = side_operand(mna, mnb, side_scale);
+          q4k_mins(hd1[u], mna, mnb);
+          const half8 a11 = side_operand(mna, mnb, side_scale);
+          const float16v im0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a10, b2[u], zero, 0, 0, 0);
+          const float16v im1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a11, b2[u], zero, 0, 0, 0);
+          const float *dm = dmin_t + (sg + u) * 128u + 64u * wr + 4u * lh;
 #pragma unroll
           for (int q4 = 0; q4 < 4; q4++) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const uint32_t rl = 128u * k + 64u * wr + 32u * i + 8u * q4 + 4u * lh + e;
-              const uint2 mm = mins_l[rl];
-              const int hi = __builtin_amdgcn_sdot4((int)mm.y, (int)bh[1], __builtin_amdgcn_sdot4((int)mm.x, (int)bh[0], 0, false), false);
-              const int lo = __builtin_amdgcn_sdot4((int)mm.y, (int)bl[1], __builtin_amdgcn_sdot4((int)mm.x, (int)bl[0], 0, false), false);
-              const int imin = hi * 64 + lo;
-              const float term = (adv1 * dmin_l[rl]) * (float)imin;
-              if (i == 0) y0[4 * q4 + e] -= term;
-              else y1[4 * q4 + e] -= term;
-            }
+            const float4 m0 = *(const float4 *)(dm + 8 * q4), m1 = *(const float4 *)(dm + 32 + 8 * q4);
+            y0[4 * q4 + 0] -= adv1[u] * m0.x * im0[4 * q4 + 0];
+            y0[4 * q4 + 1] -= adv1[u] * m0.y * im0[4 * q4 + 1];
+            y0[4 * q4 + 2] -= adv1[u] * m0.z * im0[4 * q4 + 2];
+            y0[4 * q4 + 3] -= adv1[u] * m0.w * im0[4 * q4 + 3];
+            y1[4 * q4 + 0] -= adv1[u] * m1.x * im1[4 * q4 + 0];
+            y1[4 * q4 + 1] -= adv1[u] * m1.y * im1[4 * q4 + 1];
+            y1[4 * q4 + 2] -= adv1[u] * m1.z * im1[4 * q4 + 2];
+            y1[4 * q4 + 3] -= adv1[u] * m1.w * im1[4 * q4 + 3];
           }
         }
       }
-      __syncthreads();
     }
+    __syncthreads();   // dmin_t is not reused, but the stage buffers below are written next
   }
 
   // loads run two stages ahead through three rotating register sets
@@ -1389,7 +1379,7 @@ __global__ __launch_bounds__(512) void ogm_gemm_q6k_kernel(Gemm6Params p) { gemm
 __global__ __launch_bounds__(512) void ogm_gemm_q3k_kernel(Gemm6Params p) { gemm_k2_body<GK_Q3K>(p); }
 __global__ __launch_bounds__(512) void ogm_gemm_q5k_kernel(Gemm6Params p) { gemm_k2_body<GK_Q5K>(p); }
 
-static const uint32_t G6_LDS_BYTES = 6 * GM_STAGE_HALFS * 2 + 2 * 128 * 4;
+static const uint32_t G6_LDS_BYTES = G6_LDS_BYTES_STATIC;
 
 static const uint32_t GM_LDS_BYTES = 4 * GM_STAGE_HALFS * 2 + 2 * 128 * 16 * 2 + 128 * 4;
 static const uint32_t GM_LDS_MAX = 160 * 1024;   // LDS of a CU
@@ -1417,6 +1407,7 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
     return false;
   // Q4_K's pass 1 keeps one f32 per (row, super-block) of the workgroup in LDS
   if (ggml_type == OGM_Q4_K && GM_LDS_BYTES + (size_t)(in_dim / 256u) * 512u > GM_LDS_MAX) return false;
+  if (ggml_type == OGM_Q5_K && G6_LDS_BYTES + (size_t)(in_dim / 256u) * 512u > GM_LDS_MAX) return false;
   const uint64_t block = ggml_type == OGM_Q4_K ? 144u : ggml_type == OGM_Q6_K ? 210u : ggml_type == OGM_Q3_K ? 112u : 176u;
   return (uint64_t)ogm_tiling_for(in_dim / 256u, out_dim).nrb * 64u * (in_dim / 256u) * block <= lim &&
          (uint64_t)in_dim * n_tokens * 2u <= lim;
@@ -1479,7 +1470,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.wt = a.wt;
     p.xh = xh;
     p.ad = a.act.d;
-    p.bsum = a.act.bsum;
+    p.bs16 = bs16;
     p.y = a.y;
     p.in_dim = a.in_dim;
     p.out_dim = a.out_dim;
@@ -1492,7 +1483,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     const void *fn = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_q6k_kernel
                      : a.ggml_type == OGM_Q3_K ? (const void *)ogm_gemm_q3k_kernel
                                                : (const void *)ogm_gemm_q5k_kernel;
-    e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)G6_LDS_BYTES);
+    const uint32_t lds5 = G6_LDS_BYTES + nsb * 512u;   // Q5_K: + the table of dmin of its first pass
+    e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)(a.ggml_type == OGM_Q5_K ? GM_LDS_MAX : G6_LDS_BYTES));
     if (e != hipSuccess) return e;
     if (a.ggml_type == OGM_Q6_K) {
       hipLaunchKernelGGL(ogm_gemm_q6k_kernel, grid, dim3(512), G6_LDS_BYTES, stream, p);
@@ -1501,7 +1494,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       hipLaunchKernelGGL(ogm_gemm_q3k_kernel, grid, dim3(512), G6_LDS_BYTES, stream, p);
       if (kernel_name) *kernel_name = "ogm_gemm_q3k_kernel";
     } else {
-      hipLaunchKernelGGL(ogm_gemm_q5k_kernel, grid, dim3(512), G6_LDS_BYTES, stream, p);
+      hipLaunchKernelGGL(ogm_gemm_q5k_kernel, grid, dim3(512), lds5, stream, p);
       if (kernel_name) *kernel_name = "ogm_gemm_q5k_kernel";
     }
     return hipGetLastError();
