@@ -401,8 +401,8 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
     int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w0->in_dim, n_tokens));
     if (rc != OGM_OK) return rc;
-    // Q4_K matrices over the same input (q, k, v; gate, up) share a launch, up to OGM_GEMM_MAX_MATS
-    const size_t per_launch = w0->ggml_type == OGM_TYPE_Q4_K ? OGM_GEMM_MAX_MATS : 1;
+    // K-quant matrices over the same input (q, k, v; gate, up) share a launch, up to OGM_GEMM_MAX_MATS
+    const size_t per_launch = block_elems_of(w0->ggml_type) == 256 ? OGM_GEMM_MAX_MATS : 1;
     for (size_t i = 0; i < n_tg; i += per_launch) {
       const size_t ng = n_tg - i < per_launch ? n_tg - i : per_launch;
       OgmGemmArgs g;

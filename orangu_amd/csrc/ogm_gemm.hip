@@ -1052,12 +1052,17 @@ struct Gemm6Params {
   float *y;               // [T][out_dim]
   uint32_t in_dim, out_dim, n_tokens, nsb;
   uint32_t c_shift, r_shift, nct;
+  // further matrices over the same activations, their row tiles following in grid.y
+  uint32_t n_extra;
+  const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1];
+  float *extra_y[OGM_GEMM_MAX_MATS - 1];
+  uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
 };
 
 #define G6_LDS_BYTES_STATIC (6u * GM_STAGE_HALFS * 2u + 2u * 128u * 4u)   // three tiles, two buffers each, and d
 
 template <int KIND>
-__device__ __forceinline__ void gemm_k2_body(const Gemm6Params &p) {
+__device__ __forceinline__ void gemm_k2_body(Gemm6Params p) {
   // bytes of a tile of 64 units: Q6_K 13 pieces of 1 KiB and 64 two-byte tails; Q3_K 7 pieces;
   // Q5_K 11 pieces
   constexpr uint32_t G6_TILE_BYTES = KIND == GK_Q6K ? 13440u : KIND == GK_Q3K ? 7168u : 11264u;
@@ -1069,7 +1074,20 @@ __device__ __forceinline__ void gemm_k2_body(const Gemm6Params &p) {
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t wr = wave & 1u, wt_ = wave >> 1;   // wave's row half (64 rows) and token quarter (32)
-  const uint32_t t0 = blockIdx.x * GM_BT, r0 = blockIdx.y * GM_BN;
+  uint32_t row_tile = blockIdx.y;
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + 127u) / 128u;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = blockIdx.x * GM_BT, r0 = row_tile * GM_BN;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
   // staging role: row lr_a, group t16 (16 weights) of the stage
@@ -1416,6 +1434,7 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name) {
   if (a.n_tokens == 0 || a.out_dim == 0) return hipSuccess;
   if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return hipErrorInvalidValue;
+  if (a.n_extra > OGM_GEMM_MAX_MATS - 1 || (is_flat32(a.ggml_type) && a.n_extra != 0)) return hipErrorInvalidValue;
   if (is_flat32(a.ggml_type)) {
     GemmFlatParams p;
     p.wt = a.wt;
@@ -1452,8 +1471,6 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   // shorter chain per workgroup wins (4096 -> 4096 at 512 tokens: 76 us against 103 us), beyond it
   // the wide tile's halved weight traffic does (4096 -> 14336: 119 us against 166 us)
   uint32_t row_tiles = (a.out_dim + GM_BN - 1) / GM_BN;
-  if (a.ggml_type != OGM_Q4_K && a.n_extra != 0) return hipErrorInvalidValue;
-  if (a.n_extra > OGM_GEMM_MAX_MATS - 1) return hipErrorInvalidValue;
   for (uint32_t m = 0; m < a.n_extra; m++) row_tiles += (a.extra_out_dim[m] + GM_BN - 1) / GM_BN;
   const uint32_t wgs128 = ((a.n_tokens + GM_BT - 1) / GM_BT) * row_tiles;
   const bool wide = a.ggml_type == OGM_Q4_K && a.n_tokens > 256u && wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
@@ -1471,6 +1488,12 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.xh = xh;
     p.ad = a.act.d;
     p.bs16 = bs16;
+    p.n_extra = a.n_extra;
+    for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
+      p.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
+      p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
+      p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
+    }
     p.y = a.y;
     p.in_dim = a.in_dim;
     p.out_dim = a.out_dim;

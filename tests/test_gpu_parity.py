@@ -350,19 +350,22 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
         assert_bits(got, want, "wide mfma gemm")
 
 
-@pytest.mark.parametrize("n_tokens,outs,kernel", [
-    (40, (300, 130, 64), "ogm_gemm_q4k_kernel"),          # one round of 128 x 128 tiles
-    (300, (520, 70), "ogm_gemm_q4k_kernel"),              # more than 256 tokens, still one round
-    (300, (6000, 3000, 2100), "ogm_gemm_q4k_wide_kernel"),  # 264 tiles of 128 x 128: the wide tiling
+@pytest.mark.parametrize("t,n_tokens,outs,kernel", [
+    (Q4_K, 40, (300, 130, 64), "ogm_gemm_q4k_kernel"),          # one round of 128 x 128 tiles
+    (Q4_K, 300, (520, 70), "ogm_gemm_q4k_kernel"),              # more than 256 tokens, still one round
+    (Q4_K, 300, (6000, 3000, 2100), "ogm_gemm_q4k_wide_kernel"),  # 264 tiles of 128 x 128: the wide tiling
+    (Q6_K, 40, (300, 130, 64), "ogm_gemm_q6k_kernel"),
+    (Q5_K, 130, (520, 70, 129), "ogm_gemm_q5k_kernel"),
+    (Q3_K, 40, (128, 300), "ogm_gemm_q3k_kernel"),
 ])
-def test_q4k_matrices_over_one_input_share_a_gemm_launch(be, n_tokens, outs, kernel):
-    """q / k / v (llama.rs:730-746) at prefill widths: Q4_K matrices over the same activations go
-    out as one launch whose row tiles run through the matrices in turn; every output bit equals
-    the CPU GEMM's, ragged last tiles included."""
+def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, outs, kernel):
+    """q / k / v (llama.rs:730-746) at prefill widths: K-quant matrices of one type over the same
+    activations go out as one launch whose row tiles run through the matrices in turn; every
+    output bit equals the CPU GEMM's, ragged last tiles included."""
     from orangu_amd.hiprt import DeviceBuffer, device_synchronize
     in_dim = 512
-    raws = [synth_weights(Q4_K, in_dim, od, seed=90 + i) for i, od in enumerate(outs)]
-    hs = [be.upload_raw(r, Q4_K, in_dim, od) for r, od in zip(raws, outs)]
+    raws = [synth_weights(t, in_dim, od, seed=90 + i) for i, od in enumerate(outs)]
+    hs = [be.upload_raw(r, t, in_dim, od) for r, od in zip(raws, outs)]
     x = synth_x(n_tokens, in_dim, seed=17)
     xd = DeviceBuffer.from_numpy(x)
     yds = [DeviceBuffer(4 * n_tokens * od) for od in outs]
@@ -370,7 +373,7 @@ def test_q4k_matrices_over_one_input_share_a_gemm_launch(be, n_tokens, outs, ker
     device_synchronize()
     assert be.last_kernel() == kernel
     for r, od, yd in zip(raws, outs, yds):
-        want = oracle.matmul(Q4_K, r, in_dim, od, x, n_tokens)
+        want = oracle.matmul(t, r, in_dim, od, x, n_tokens)
         assert_bits(yd.to_numpy(np.float32, n_tokens * od), want, f"{od} rows of {outs}")
     for h in hs:
         be.free_weight(h)
