@@ -374,8 +374,10 @@ def main() -> int:
         gemm = {"workload": f"Q4_K 4096->14336, {T} tokens (config a14 shape)", "kernel": gemm_kernel}
         if us_gemm is not None:
             flops = 2.0 * T * HIDDEN * FFN
-            gemm.update({"us_per_matmul": round(us_gemm, 1), "tflops": round(flops / us_gemm / 1e6, 1),
-                         "frac_of_f16_mfma_peak": round(flops / us_gemm / 1e6 / 2500.0, 4)})
+            # the kernel multiplies int8 operands (v_mfma_i32_32x32x32_i8): priced against the dense
+            # int8 peak of 5.0 POP/s (against the 2.5 PFLOP/s f16 peak it would read twice as high)
+            gemm.update({"us_per_matmul": round(us_gemm, 1), "tops": round(flops / us_gemm / 1e6, 1),
+                         "mfma_type": "i8", "frac_of_int8_mfma_peak": round(flops / us_gemm / 1e6 / 5000.0, 4)})
         if not args.only_gemm and args.cpu_seconds > 0:
             import oracle
             rows = np.r_[0:32, 7000:7032, FFN - 32:FFN]

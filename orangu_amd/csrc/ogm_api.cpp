@@ -46,6 +46,7 @@ struct ogm_ctx {
   int tune_wg_waves = 0;
   int tune_gemm_min_tokens = 9;  // matmul at n_tokens >= this takes the MFMA GEMM
   int tune_gemm_wide_min_wgs = 0;
+  int tune_gemm_q4k_variant = 0;
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
   const char *last_kernel = "";
@@ -211,6 +212,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemm_wide_min_wgs") == 0) {
     if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_wide_min_wgs must be >= 0");
     ctx->tune_gemm_wide_min_wgs = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_q4k_variant") == 0) {
+    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_q4k_variant must be 0, 1 or 2");
+    ctx->tune_gemm_q4k_variant = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemv_rb_per_wg") == 0) {
@@ -415,6 +421,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.y = tg[i].y;
       g.xh = ctx->xh.p;
       g.wide_min_wgs = (uint32_t)ctx->tune_gemm_wide_min_wgs;
+      g.q4k_variant = (uint32_t)ctx->tune_gemm_q4k_variant;
       g.n_extra = (uint32_t)ng - 1;
       for (size_t j = 1; j < ng; j++) {
         g.extra_wt[j - 1] = tg[i + j].w->dev;

@@ -451,6 +451,261 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q4k_kernel(GemmParams p) {
 }
 
 // ------------------------------------------------------------------------------------------
+// Q4_K on the int8 matrix cores: 128 rows x 128 tokens per workgroup, four multiplying and four
+// feeding waves.
+//
+// The f16 kernels above fold the sub-block scale into the weight operand (sc_j * (q - 8) as f16)
+// so that the matrix cores produce isum directly; the price is two-byte operands and, for the
+// other K-quants, two chains.  Here the operands stay int8 - the nibbles as they are, and the
+// activations as the quantizer left them - and one v_mfma_i32_32x32x32_i8 produces the 32 x 32
+// exact dot products of ONE sub-block (dot32 of vecdot.rs:471-502); the scale is applied to that
+// partial sum with integer multiply-adds, isum += sc_j * dot32_j exactly as accumulate_sym32
+// (vecdot.rs:2271-2303) does, in 32-bit integers with no 2^24 bound to respect.  The tokens are
+// the matrix instruction's row operand and the weight rows its column operand: a lane then
+// owns one weight row (its column) and 16 tokens (its registers), so the scale of a
+// multiply-add is one register for all sixteen.  Half the LDS bytes per product, twice the
+// matrix rate, sixteen integer multiply-adds per matrix instruction.
+//
+// LDS rows hold the 64 bytes of a stage (two sub-blocks) in 80 bytes; a lane's operand is the 16
+// bytes at 32 * sub-block + 16 * (lane / 32) of its row - both operands use the same bytes of k,
+// which is all the dot product asks.
+
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int16v __attribute__((ext_vector_type(16)));
+
+#define GI_ROW 80u                   // bytes of an LDS row (64 int8 + padding)
+#define GI_WTILE (128u * GI_ROW)     // the weight tile of a stage
+
+// Twelve waves: eight multiply (wave w: rows 64 (w / 4) .. + 63, tokens 32 (w % 4) .. + 31 of the
+// workgroup's 128 x 128) and four feed them.  Two multiplying waves per SIMD, so that one's matrix
+// instructions run under the other's multiply-adds; the two kinds of waves run loops of their
+// own (same number of barriers), so that what one keeps in registers is not kept alive in the other.
+__global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) {
+  __shared__ __align__(16) uint8_t w_l[2][GI_WTILE];   // weights 0..15, [row][64 of 80]
+  __shared__ __align__(16) uint8_t x_l[2][GI_WTILE];   // activations, [token][64 of 80]
+  __shared__ __align__(8) uint2 sc_l[2][128];          // per super-block: the rows' eight scales, one byte each
+  __shared__ __align__(16) float d_l[2][128];          // the rows' d
+  __shared__ __align__(16) float ad_l[2][128];         // the tokens' activation scale
+  __shared__ __align__(16) float p1_dmin[8][128];      // pass 1, eight super-blocks at a time
+  __shared__ __align__(16) float p1_ad[8][128];
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const bool producer = wave >= 8u;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  const uint32_t tq = wave & 3u, rh = (wave >> 2) & 1u;
+  const uint32_t t0 = blockIdx.x * 128u, r0 = gm_pick_matrix(p, blockIdx.y) * 128u;
+  const uint32_t tw = 32u * tq;   // the wave's first token within the workgroup
+
+  auto row_off = [&](uint32_t row) -> uint32_t {
+    row = min(row, p.out_dim - 1u);
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    return rb * p.nct * 9216u + r * 16u;
+  };
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    const uint32_t ct = s >> p.c_shift, cl = s & ((1u << p.c_shift) - 1u);
+    return ct * 9216u + (cl << p.r_shift) * 16u;
+  };
+
+  // y0 / y1: tokens t0 + tw + (8 (r / 4) + 4 lh + r % 4), rows r0 + 64 rh + l32 and + 32
+  float16v y0, y1;
+#pragma unroll
+  for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
+
+  // ---------------- pass 1: acc -= (ad * dmin) * sum_j m_j * bsum_j, all super-blocks first
+  // (vecdot.rs:2226-2240), on the f16 matrix cores as in the kernels above, tokens as rows
+  {
+    float16v zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.0f;
+    const uint32_t ro0 = row_off(r0 + 64u * rh + l32), ro1 = row_off(r0 + 64u * rh + 32u + l32);
+    const uint32_t tk = min(t0 + tw + l32, p.n_tokens - 1u) * p.nsb;
+    const float side_scale = lh ? 1.0f : 64.0f;
+    for (uint32_t sg = 0; sg < p.nsb; sg += 8u) {
+      // the tables of this round: dmin of (super-block, row) and ad of (super-block, token)
+      for (uint32_t i = tid; i < 8u * 128u; i += 768u) {
+        const uint32_t u = i >> 7, k = i & 127u, su = min(sg + u, p.nsb - 1u);
+        const uint32_t h = *(const uint32_t *)(p.wt + (row_off(r0 + k) + sb_off(su)));
+        p1_dmin[u][k] = gm_f16_bits_to_f32(h >> 16);
+        p1_ad[u][k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + su];
+      }
+      __syncthreads();
+      if (!producer) {
+#pragma unroll 2
+        for (uint32_t u = 0; u < 8u; u++) {
+          if (sg + u >= p.nsb) break;
+          const uint32_t su = sg + u;
+          const uint4 hd0 = *(const uint4 *)(p.wt + (ro0 + sb_off(su)));
+          const uint4 hd1 = *(const uint4 *)(p.wt + (ro1 + sb_off(su)));
+          const half8 b2 = *(const half8 *)(p.bs16 + ((tk + su) * 16u + 8u * lh));
+          uint32_t mna, mnb;
+          q4k_mins(hd0, mna, mnb);
+          const half8 a10 = side_operand(mna, mnb, side_scale);
+          q4k_mins(hd1, mna, mnb);
+          const half8 a11 = side_operand(mna, mnb, side_scale);
+          const float dm0 = p1_dmin[u][64u * rh + l32], dm1 = p1_dmin[u][64u * rh + 32u + l32];
+          const float16v im0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2, a10, zero, 0, 0, 0);
+          const float16v im1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2, a11, zero, 0, 0, 0);
+          const float *adp = &p1_ad[u][tw + 4u * lh];
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++) {
+            const float4 a4 = *(const float4 *)(adp + 8 * q4);
+            y0[4 * q4 + 0] -= a4.x * dm0 * im0[4 * q4 + 0];
+            y0[4 * q4 + 1] -= a4.y * dm0 * im0[4 * q4 + 1];
+            y0[4 * q4 + 2] -= a4.z * dm0 * im0[4 * q4 + 2];
+            y0[4 * q4 + 3] -= a4.w * dm0 * im0[4 * q4 + 3];
+            y1[4 * q4 + 0] -= a4.x * dm1 * im1[4 * q4 + 0];
+            y1[4 * q4 + 1] -= a4.y * dm1 * im1[4 * q4 + 1];
+            y1[4 * q4 + 2] -= a4.z * dm1 * im1[4 * q4 + 2];
+            y1[4 * q4 + 3] -= a4.w * dm1 * im1[4 * q4 + 3];
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+
+  // ---------------- pass 2: acc += ad * (d * sum_j sc_j * dot32_j)
+  if (producer) {
+    // Feeding thread pt stages half a stage row of weights (one 16-byte piece of qs: 16 low
+    // nibbles for sub-block 2g, 16 high nibbles for 2g + 1) and half a stage row of activations
+    // (32 bytes); once per super-block 128 of them the rows' scales and d, the other 128 the
+    // tokens' ad.
+    const uint32_t pt = tid - 512u;
+    const uint32_t prow = pt >> 1, phalf = pt & 1u;
+    const uint32_t wro = row_off(r0 + prow) + (1u + phalf) * 1024u;                 // + sb_off + 2048 g
+    const uint32_t xro = min(t0 + prow, p.n_tokens - 1u) * p.in_dim + 32u * phalf;  // + 256 s + 64 g
+    const uint32_t hro = row_off(r0 + (pt & 127u));
+    const uint32_t aro = min(t0 + (pt & 127u), p.n_tokens - 1u) * p.nsb;
+    // the ring of stages in flight, slot = stage % 4 = g (named registers: an array handed to a
+    // function by reference ends up in scratch memory)
+    uint4 wq0, wq1, wq2, wq3, xa0_, xa1_, xa2_, xa3_, xb0_, xb1_, xb2_, xb3_;
+    uint4 hdr = make_uint4(0, 0, 0, 0);
+    float adn = 0.0f;
+#define GI_LOAD(S, G, K)                                                                          \
+  do {                                                                                            \
+    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded again, never used */ \
+    wq##K = *(const uint4 *)(p.wt + (wro + sb_off(s_) + 2048u * (G)));                            \
+    const uint4 *xp_ = (const uint4 *)(p.xq + (xro + 256u * s_ + 64u * (G)));                     \
+    xa##K##_ = xp_[0];                                                                            \
+    xb##K##_ = xp_[1];                                                                            \
+    if ((G) == 0u) {                                                                              \
+      if (pt < 128u) hdr = *(const uint4 *)(p.wt + (hro + sb_off(s_)));                           \
+      else adn = p.ad[aro + s_];                                                                  \
+    }                                                                                             \
+  } while (0)
+  // Q4_K's nibbles are unsigned weights 0..15 (the minimum is a term of its own): int8 as they are
+#define GI_STORE(S, G, BUF, K)                                                                    \
+  do {                                                                                            \
+    uint8_t *wr_ = &w_l[BUF][prow * GI_ROW + 16u * phalf];                                        \
+    *(uint4 *)wr_ = make_uint4(wq##K.x & 0x0F0F0F0Fu, wq##K.y & 0x0F0F0F0Fu, wq##K.z & 0x0F0F0F0Fu, \
+                               wq##K.w & 0x0F0F0F0Fu);                                            \
+    *(uint4 *)(wr_ + 32u) = make_uint4((wq##K.x >> 4) & 0x0F0F0F0Fu, (wq##K.y >> 4) & 0x0F0F0F0Fu, \
+                                       (wq##K.z >> 4) & 0x0F0F0F0Fu, (wq##K.w >> 4) & 0x0F0F0F0Fu); \
+    uint8_t *xr_ = &x_l[BUF][prow * GI_ROW + 32u * phalf];                                        \
+    *(uint4 *)xr_ = xa##K##_;                                                                     \
+    *(uint4 *)(xr_ + 16u) = xb##K##_;                                                             \
+    if ((G) == 0u) {                                                                              \
+      if (pt < 128u) {                                                                            \
+        uint32_t sca_, scb_;                                                                      \
+        q4k_scales(hdr, sca_, scb_);                                                              \
+        sc_l[(S) & 1u][pt] = make_uint2(sca_, scb_);                                              \
+        d_l[(S) & 1u][pt] = gm_f16_bits_to_f32(hdr.x & 0xFFFFu);                                  \
+      } else {                                                                                    \
+        ad_l[(S) & 1u][pt - 128u] = adn;                                                          \
+      }                                                                                           \
+    }                                                                                             \
+  } while (0)
+    GI_LOAD(0u, 0u, 0);
+    GI_LOAD(0u, 1u, 1);
+    GI_LOAD(0u, 2u, 2);
+    GI_STORE(0u, 0u, 0u, 0);
+    GI_LOAD(0u, 3u, 3);
+    __syncthreads();
+    // During stage n = 4 s + g (in LDS buffer g % 2): stage n + 1 goes to the other buffer (it
+    // arrived long ago), stage n + 4 is requested into the slot stage n left
+    for (uint32_t s = 0; s < p.nsb; s++) {
+      GI_STORE(s, 1u, 1u, 1);
+      GI_LOAD(s + 1u, 0u, 0);
+      __syncthreads();
+      GI_STORE(s, 2u, 0u, 2);
+      GI_LOAD(s + 1u, 1u, 1);
+      __syncthreads();
+      GI_STORE(s, 3u, 1u, 3);
+      GI_LOAD(s + 1u, 2u, 2);
+      __syncthreads();
+      if (s + 1u < p.nsb) GI_STORE(s + 1u, 0u, 0u, 0);
+      GI_LOAD(s + 1u, 3u, 3);
+      __syncthreads();
+    }
+#undef GI_LOAD
+#undef GI_STORE
+  } else {
+    __syncthreads();
+    int16v i0, i1;   // isum of the running super-block
+    const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const uint32_t xrow = (tw + l32) * GI_ROW + 16u * lh;
+    const uint32_t wrow0 = (64u * rh + l32) * GI_ROW + 16u * lh, wrow1 = wrow0 + 32u * GI_ROW;
+    for (uint32_t s = 0; s < p.nsb; s++) {
+      const uint2 scw0 = sc_l[s & 1u][64u * rh + l32], scw1 = sc_l[s & 1u][64u * rh + 32u + l32];
+#pragma unroll
+      for (uint32_t g = 0; g < 4u; g++) {
+        const uint32_t buf = g & 1u;
+#pragma unroll
+        for (uint32_t sub = 0; sub < 2u; sub++) {
+          const uint32_t j = 2u * g + sub;
+          const int sc0 = (int)(((j < 4u ? scw0.x : scw0.y) >> (8u * (j & 3u))) & 0xFFu);
+          const int sc1 = (int)(((j < 4u ? scw1.x : scw1.y) >> (8u * (j & 3u))) & 0xFFu);
+          const int4v xa = *(const int4v *)&x_l[buf][xrow + 32u * sub];
+          const int4v wb0 = *(const int4v *)&w_l[buf][wrow0 + 32u * sub];
+          const int4v wb1 = *(const int4v *)&w_l[buf][wrow1 + 32u * sub];
+          const int16v p0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wb0, zi, 0, 0, 0);
+          const int16v p1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wb1, zi, 0, 0, 0);
+          if (j == 0u) {   // the super-block starts fresh sums
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              i0[r] = __mul24(p0[r], sc0);
+              i1[r] = __mul24(p1[r], sc1);
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              i0[r] = __mul24(p0[r], sc0) + i0[r];
+              i1[r] = __mul24(p1[r], sc1) + i1[r];
+            }
+          }
+        }
+        if (g == 3u) {
+          const float d0 = d_l[s & 1u][64u * rh + l32], d1 = d_l[s & 1u][64u * rh + 32u + l32];
+          const float *adp = &ad_l[s & 1u][tw + 4u * lh];
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++) {
+            const float4 a4 = *(const float4 *)(adp + 8 * q4);
+            y0[4 * q4 + 0] += a4.x * (d0 * (float)i0[4 * q4 + 0]);
+            y0[4 * q4 + 1] += a4.y * (d0 * (float)i0[4 * q4 + 1]);
+            y0[4 * q4 + 2] += a4.z * (d0 * (float)i0[4 * q4 + 2]);
+            y0[4 * q4 + 3] += a4.w * (d0 * (float)i0[4 * q4 + 3]);
+            y1[4 * q4 + 0] += a4.x * (d1 * (float)i1[4 * q4 + 0]);
+            y1[4 * q4 + 1] += a4.y * (d1 * (float)i1[4 * q4 + 1]);
+            y1[4 * q4 + 2] += a4.z * (d1 * (float)i1[4 * q4 + 2]);
+            y1[4 * q4 + 3] += a4.w * (d1 * (float)i1[4 * q4 + 3]);
+          }
+        }
+        __syncthreads();
+      }
+    }
+    const uint32_t row0 = r0 + 64u * rh + l32;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const uint32_t t = t0 + tw + 8u * (r >> 2) + 4u * lh + (r & 3);
+      if (t < p.n_tokens) {
+        if (row0 < p.out_dim) p.y[(size_t)t * p.out_dim + row0] = y0[r];
+        if (row0 + 32u < p.out_dim) p.y[(size_t)t * p.out_dim + row0 + 32u] = y1[r];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
 //
 // The 128 x 128 kernel above is bound by LDS bandwidth: a multiplying wave reads (64 + 32) k-rows
@@ -1473,9 +1728,14 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   uint32_t row_tiles = (a.out_dim + GM_BN - 1) / GM_BN;
   for (uint32_t m = 0; m < a.n_extra; m++) row_tiles += (a.extra_out_dim[m] + GM_BN - 1) / GM_BN;
   const uint32_t wgs128 = ((a.n_tokens + GM_BT - 1) / GM_BT) * row_tiles;
-  const bool wide = a.ggml_type == OGM_Q4_K && a.n_tokens > 256u && wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
-  hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((wide ? n_sb : n8) + 255) / 256)), dim3(256), 0,
-                     stream, a.act.q, a.act.bsum, wide ? (_Float16 *)nullptr : xh, bs16, n8, n_sb);
+  // Q4_K runs on the int8 kernel unless the f16 kernels are asked for (q4k_variant 2); of those the
+  // wide one takes over as described above
+  const bool i8 = a.ggml_type == OGM_Q4_K && a.q4k_variant != 2u;
+  const bool wide = a.ggml_type == OGM_Q4_K && !i8 && a.n_tokens > 256u &&
+                    wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
+  const bool raw_x = wide || i8;   // these read the int8 activations as they are: only (bh, bl) to prepare
+  hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((raw_x ? n_sb : n8) + 255) / 256)), dim3(256), 0,
+                     stream, a.act.q, a.act.bsum, raw_x ? (_Float16 *)nullptr : xh, bs16, n8, n_sb);
   const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
   const uint32_t c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
   // token tiles vary fastest: workgroups that run together share weight rows, and with a
@@ -1541,6 +1801,11 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
     p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
     p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
+  }
+  if (i8) {
+    hipLaunchKernelGGL(ogm_gemm_q4k_i8_kernel, grid, dim3(768), 0, stream, p);
+    if (kernel_name) *kernel_name = "ogm_gemm_q4k_i8_kernel";
+    return hipGetLastError();
   }
   if (wide) {
     const dim3 wgrid((a.n_tokens + GW_BT - 1) / GW_BT, row_tiles);

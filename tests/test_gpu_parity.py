@@ -326,32 +326,40 @@ def test_q6k_vocab_projection_batches_1_4_8(be):
     (256, 5, 257), (2304, 130, 600), (4096, 257, 1030), (1024, 129, 256), (512, 64, 513),
 ])
 def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
-    """ogm_matmul at n_tokens >= 9 takes the MFMA kernel; values must equal CpuBackend's K-quant
-    GEMM (vecdot.rs:2213-2303): integer sums exact on the matrix cores, f32 order the reference's."""
+    """ogm_matmul at n_tokens >= 9 takes the matrix-core kernels; values must equal CpuBackend's
+    K-quant GEMM (vecdot.rs:2213-2303): integer sums exact, f32 order the reference's.  The int8
+    kernel (the default) and the two f16 kernels it replaced each produce the same bits."""
     raw = synth_weights(Q4_K, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T)
     w = qm(raw, Q4_K, in_dim, out_dim)
     say("gemm", in_dim, out_dim, T)
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     got = be.matmul(x, T, w)
-    # beyond 256 tokens the 128 x 256 tile kernel runs once the 128 x 128 tiling would take more
-    # than one round of workgroups (256)
-    tiles = ((T + 127) // 128) * ((out_dim + 127) // 128)
-    assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 and tiles > 256 else "ogm_gemm_q4k_kernel")
-    assert_close(got, want, "mfma gemm")
-    assert_bits(got, want, "mfma gemm")
-    if T > 256:   # the wide kernel on this (small, ragged) shape as well
-        be.set_tuning("gemm_wide_min_wgs", 1)
-        try:
+    assert be.last_kernel() == "ogm_gemm_q4k_i8_kernel"
+    assert_close(got, want, "int8 mfma gemm")
+    assert_bits(got, want, "int8 mfma gemm")
+    be.set_tuning("gemm_q4k_variant", 2)
+    try:
+        got = be.matmul(x, T, w)
+        # beyond 256 tokens the 128 x 256 tile kernel runs once the 128 x 128 tiling would take more
+        # than one round of workgroups (256)
+        tiles = ((T + 127) // 128) * ((out_dim + 127) // 128)
+        assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 and tiles > 256 else "ogm_gemm_q4k_kernel")
+        assert_bits(got, want, "f16 mfma gemm")
+        if T > 256:   # the wide kernel on this (small, ragged) shape as well
+            be.set_tuning("gemm_wide_min_wgs", 1)
             got = be.matmul(x, T, w)
             assert be.last_kernel() == "ogm_gemm_q4k_wide_kernel"
-        finally:
-            be.set_tuning("gemm_wide_min_wgs", 0)
-        assert_bits(got, want, "wide mfma gemm")
+            assert_bits(got, want, "wide f16 mfma gemm")
+    finally:
+        be.set_tuning("gemm_wide_min_wgs", 0)
+        be.set_tuning("gemm_q4k_variant", 0)
 
 
 @pytest.mark.parametrize("t,n_tokens,outs,kernel", [
-    (Q4_K, 40, (300, 130, 64), "ogm_gemm_q4k_kernel"),          # one round of 128 x 128 tiles
+    (Q4_K, 40, (300, 130, 64), "ogm_gemm_q4k_i8_kernel"),
+    (Q4_K, 300, (520, 70), "ogm_gemm_q4k_i8_kernel"),
+    (Q4_K, 40, (300, 130, 64), "ogm_gemm_q4k_kernel"),          # the f16 kernels: one round of 128 x 128 tiles
     (Q4_K, 300, (520, 70), "ogm_gemm_q4k_kernel"),              # more than 256 tokens, still one round
     (Q4_K, 300, (6000, 3000, 2100), "ogm_gemm_q4k_wide_kernel"),  # 264 tiles of 128 x 128: the wide tiling
     (Q6_K, 40, (300, 130, 64), "ogm_gemm_q6k_kernel"),
@@ -369,7 +377,11 @@ def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, ou
     x = synth_x(n_tokens, in_dim, seed=17)
     xd = DeviceBuffer.from_numpy(x)
     yds = [DeviceBuffer(4 * n_tokens * od) for od in outs]
-    be.matmul_multi_dev(hs, xd.ptr, n_tokens, [y.ptr for y in yds])
+    be.set_tuning("gemm_q4k_variant", 0 if kernel.endswith("_i8_kernel") else 2)
+    try:
+        be.matmul_multi_dev(hs, xd.ptr, n_tokens, [y.ptr for y in yds])
+    finally:
+        be.set_tuning("gemm_q4k_variant", 0)
     device_synchronize()
     assert be.last_kernel() == kernel
     for r, od, yd in zip(raws, outs, yds):
@@ -401,14 +413,16 @@ def test_mfma_gemm_equals_small_batch_kernel_and_is_batch_independent(be):
         assert_bits(part, full[:n], f"{n} of 40")
 
 
+@pytest.mark.parametrize("variant", [0, 2])
 @pytest.mark.parametrize("T", [16, 272])
 @pytest.mark.parametrize("qs_lo,qs_hi,sign", [(0xFF, 0xFF, "alt"), (0x00, 0x00, "alt"), (0x0F, 0xF0, "pos"),
                                                (0xF0, 0x0F, "neg"), (0xFF, 0x00, "block")])
-def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T):
+def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T, variant):
     """Largest magnitudes the integer stage can see: nibbles 0 or 15, scales and mins 63, activations
     +-127.  The per-super-block sum reaches 3.1e7 > 2^24 and the centred partial sums and their
     correction reach +-1.64e7 each (and cancel when every nibble is 0), so the f32 add of the exact
-    parts must round exactly like `isum as f32`."""
+    parts must round exactly like `isum as f32` (f16 kernels, variant 2); the int8 kernel keeps the
+    whole sum in 32-bit integers and converts once."""
     in_dim, out_dim = 1024, 32
     blocks = np.zeros((out_dim * 4, 144), np.uint8)
     blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
@@ -426,12 +440,15 @@ def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T):
         x[:, 128:256] *= -1
         x[3] = -127.0
     raw = blocks.reshape(-1)
-    be.set_tuning("gemm_wide_min_wgs", 1)   # beyond 256 tokens the wide kernel, however few tiles
+    be.set_tuning("gemm_wide_min_wgs", 1)   # f16 kernels: beyond 256 tokens the wide one, however few tiles
+    be.set_tuning("gemm_q4k_variant", variant)
     try:
         got = be.matmul(x, T, qm(raw, Q4_K, in_dim, out_dim))
     finally:
         be.set_tuning("gemm_wide_min_wgs", 0)
-    assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 else "ogm_gemm_q4k_kernel")
+        be.set_tuning("gemm_q4k_variant", 0)
+    assert be.last_kernel() == ("ogm_gemm_q4k_i8_kernel" if variant == 0 else
+                                "ogm_gemm_q4k_wide_kernel" if T > 256 else "ogm_gemm_q4k_kernel")
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     assert_bits(got, want, "extreme ranges")
     isum, imin = be.dump_block_sums(x[0], 1, qm(raw, Q4_K, in_dim, out_dim))
