@@ -90,7 +90,7 @@ def sweep(be, helpers, hiprt) -> dict:
     return out
 
 
-def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool) -> dict:
+def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool, only_prefill: int = 0) -> dict:
     """Batch-1 decode of an 8B-shaped Llama (32 layers: wq, wo 4096x4096, wk, wv 4096->1024, gate, up
     4096->14336 in Q4_K; down 14336->4096 and the 128256-row output in Q6_K; f16 KV cache holding `ctx`
     random positions): tokens per second of ogm_llama_decode_dev with the embedding row, the logits and
@@ -131,6 +131,18 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
         dec.kv_write(l, 0, k, v)
         if check and l < 2:
             kvs.append((k, v))
+    if only_prefill:   # for profiles: nothing but prompts of this length (one warm-up, three timed)
+        prompt = rng.integers(0, n_vocab, only_prefill).astype(np.uint32)
+        dec.prefill_tokens(up("output"), prompt, 0)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            dec.prefill_tokens(up("output"), prompt, 0)
+        dt_pre = (time.perf_counter() - t0) / 3
+        dec.close()
+        for h in mats.values():
+            be.free_weight(h)
+        return {"workload": f"configs[4] model, prefill of {only_prefill} tokens from an empty cache",
+                "prefill_ms": round(dt_pre * 1e3, 2), "prefill_tok_per_s": round(only_prefill / dt_pre, 1)}
     x_h = rng.standard_normal(n_embd).astype(np.float32)
     x_d = hiprt.DeviceBuffer.from_numpy(x_h)
     tok_d = hiprt.DeviceBuffer(4)
@@ -230,6 +242,8 @@ def main() -> int:
                     help="tokens of the 8B-shaped decode leg (config 5); 0 skips it")
     ap.add_argument("--decode-ctx", type=int, default=2048, help="cached positions of the decode leg")
     ap.add_argument("--only-decode", action="store_true", help="run only the decode leg (for rocprofv3)")
+    ap.add_argument("--only-prefill", type=int, default=0, metavar="N",
+                    help="run only prefills of N tokens on the decode leg's model (for rocprofv3)")
     ap.add_argument("--sweep", action="store_true",
                     help="time every benchmark configuration's kernels instead (one JSON object, not the "
                          "headline line)")
@@ -249,6 +263,11 @@ def main() -> int:
     be = Mi355xBackend()  # raises without the HIP library or a gfx950 device
     if args.sweep:
         print(json.dumps(sweep(be, helpers, hiprt)))
+        be.close()
+        return 0
+    if args.only_prefill:
+        print(json.dumps(decode_leg(be, helpers, hiprt, 1, 0, max(args.decode_ctx, args.only_prefill), False,
+                                    only_prefill=args.only_prefill)))
         be.close()
         return 0
     if args.only_decode:

@@ -480,8 +480,13 @@ typedef int int16v __attribute__((ext_vector_type(16)));
 // workgroup's 128 x 128) and four feed them.  Two multiplying waves per SIMD, so that one's matrix
 // instructions run under the other's multiply-adds; the two kinds of waves run loops of their
 // own (same number of barriers), so that what one keeps in registers is not kept alive in the other.
-__global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) {
-  __shared__ __align__(16) uint8_t w_l[2][GI_WTILE];   // weights 0..15, [row][64 of 80]
+// Q5_K (KKind::Q4K rows as well, vecdot.rs:2064-2088) differs in the staging alone: the weight is
+// the nibble with bit j of qh[l] on top, 0..31, and its unit has 11 pieces (header, qh, qs).
+template <bool Q5>
+__device__ __forceinline__ void gemm_i8_body(GemmParams p) {
+  constexpr uint32_t TILE_BYTES = Q5 ? 11264u : 9216u;   // 64 units of 176 / 144 bytes
+  constexpr uint32_t QS_PIECE0 = Q5 ? 3u : 1u;           // first piece of qs
+  __shared__ __align__(16) uint8_t w_l[2][GI_WTILE];   // weights 0..15 (Q5_K: 0..31), [row][64 of 80]
   __shared__ __align__(16) uint8_t x_l[2][GI_WTILE];   // activations, [token][64 of 80]
   __shared__ __align__(8) uint2 sc_l[2][128];          // per super-block: the rows' eight scales, one byte each
   __shared__ __align__(16) float d_l[2][128];          // the rows' d
@@ -499,11 +504,11 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) {
   auto row_off = [&](uint32_t row) -> uint32_t {
     row = min(row, p.out_dim - 1u);
     const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
-    return rb * p.nct * 9216u + r * 16u;
+    return rb * p.nct * TILE_BYTES + r * 16u;
   };
   auto sb_off = [&](uint32_t s) -> uint32_t {
     const uint32_t ct = s >> p.c_shift, cl = s & ((1u << p.c_shift) - 1u);
-    return ct * 9216u + (cl << p.r_shift) * 16u;
+    return ct * TILE_BYTES + (cl << p.r_shift) * 16u;
   };
 
   // y0 / y1: tokens t0 + tw + (8 (r / 4) + 4 lh + r % 4), rows r0 + 64 rh + l32 and + 32
@@ -572,7 +577,8 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) {
     // tokens' ad.
     const uint32_t pt = tid - 512u;
     const uint32_t prow = pt >> 1, phalf = pt & 1u;
-    const uint32_t wro = row_off(r0 + prow) + (1u + phalf) * 1024u;                 // + sb_off + 2048 g
+    const uint32_t wro = row_off(r0 + prow) + (QS_PIECE0 + phalf) * 1024u;          // + sb_off + 2048 g
+    const uint32_t qho = row_off(r0 + prow) + (1u + phalf) * 1024u;                 // Q5_K: the thread's 16 bytes of qh
     const uint32_t xro = min(t0 + prow, p.n_tokens - 1u) * p.in_dim + 32u * phalf;  // + 256 s + 64 g
     const uint32_t hro = row_off(r0 + (pt & 127u));
     const uint32_t aro = min(t0 + (pt & 127u), p.n_tokens - 1u) * p.nsb;
@@ -580,6 +586,7 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) {
     // function by reference ends up in scratch memory)
     uint4 wq0, wq1, wq2, wq3, xa0_, xa1_, xa2_, xa3_, xb0_, xb1_, xb2_, xb3_;
     uint4 hdr = make_uint4(0, 0, 0, 0);
+    uint4 qhn = make_uint4(0, 0, 0, 0), qhc = make_uint4(0, 0, 0, 0);   // Q5_K: qh of the next / the stored super-block
     float adn = 0.0f;
 #define GI_LOAD(S, G, K)                                                                          \
   do {                                                                                            \
@@ -591,16 +598,31 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) {
     if ((G) == 0u) {                                                                              \
       if (pt < 128u) hdr = *(const uint4 *)(p.wt + (hro + sb_off(s_)));                           \
       else adn = p.ad[aro + s_];                                                                  \
+      if constexpr (Q5) qhn = *(const uint4 *)(p.wt + (qho + sb_off(s_)));                        \
     }                                                                                             \
   } while (0)
-  // Q4_K's nibbles are unsigned weights 0..15 (the minimum is a term of its own): int8 as they are
+  // The nibbles are unsigned weights 0..15 (the minimum is a term of its own): int8 as they are;
+  // Q5_K puts bit 2g (2g + 1) of the qh byte on top of the low (high) nibble
 #define GI_STORE(S, G, BUF, K)                                                                    \
   do {                                                                                            \
+    if constexpr (Q5) { if ((G) == 0u) qhc = qhn; }                                               \
     uint8_t *wr_ = &w_l[BUF][prow * GI_ROW + 16u * phalf];                                        \
-    *(uint4 *)wr_ = make_uint4(wq##K.x & 0x0F0F0F0Fu, wq##K.y & 0x0F0F0F0Fu, wq##K.z & 0x0F0F0F0Fu, \
-                               wq##K.w & 0x0F0F0F0Fu);                                            \
-    *(uint4 *)(wr_ + 32u) = make_uint4((wq##K.x >> 4) & 0x0F0F0F0Fu, (wq##K.y >> 4) & 0x0F0F0F0Fu, \
-                                       (wq##K.z >> 4) & 0x0F0F0F0Fu, (wq##K.w >> 4) & 0x0F0F0F0Fu); \
+    uint4 lo_ = make_uint4(wq##K.x & 0x0F0F0F0Fu, wq##K.y & 0x0F0F0F0Fu, wq##K.z & 0x0F0F0F0Fu,   \
+                           wq##K.w & 0x0F0F0F0Fu);                                                \
+    uint4 hi_ = make_uint4((wq##K.x >> 4) & 0x0F0F0F0Fu, (wq##K.y >> 4) & 0x0F0F0F0Fu,            \
+                           (wq##K.z >> 4) & 0x0F0F0F0Fu, (wq##K.w >> 4) & 0x0F0F0F0Fu);           \
+    if constexpr (Q5) {                                                                           \
+      lo_.x |= ((qhc.x >> (2u * (G))) & 0x01010101u) << 4;                                        \
+      lo_.y |= ((qhc.y >> (2u * (G))) & 0x01010101u) << 4;                                        \
+      lo_.z |= ((qhc.z >> (2u * (G))) & 0x01010101u) << 4;                                        \
+      lo_.w |= ((qhc.w >> (2u * (G))) & 0x01010101u) << 4;                                        \
+      hi_.x |= ((qhc.x >> (2u * (G) + 1u)) & 0x01010101u) << 4;                                   \
+      hi_.y |= ((qhc.y >> (2u * (G) + 1u)) & 0x01010101u) << 4;                                   \
+      hi_.z |= ((qhc.z >> (2u * (G) + 1u)) & 0x01010101u) << 4;                                   \
+      hi_.w |= ((qhc.w >> (2u * (G) + 1u)) & 0x01010101u) << 4;                                   \
+    }                                                                                             \
+    *(uint4 *)wr_ = lo_;                                                                          \
+    *(uint4 *)(wr_ + 32u) = hi_;                                                                  \
     uint8_t *xr_ = &x_l[BUF][prow * GI_ROW + 32u * phalf];                                        \
     *(uint4 *)xr_ = xa##K##_;                                                                     \
     *(uint4 *)(xr_ + 16u) = xb##K##_;                                                             \
@@ -650,30 +672,38 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) {
 #pragma unroll
       for (uint32_t g = 0; g < 4u; g++) {
         const uint32_t buf = g & 1u;
+        // both sub-blocks' matrix instructions first, then their multiply-adds: four results in
+        // flight keep the matrix pipe busy under the vector work
+        const uint32_t ja = 2u * g, jb = 2u * g + 1u;
+        const int sc0a = (int)(((ja < 4u ? scw0.x : scw0.y) >> (8u * (ja & 3u))) & 0xFFu);
+        const int sc1a = (int)(((ja < 4u ? scw1.x : scw1.y) >> (8u * (ja & 3u))) & 0xFFu);
+        const int sc0b = (int)(((jb < 4u ? scw0.x : scw0.y) >> (8u * (jb & 3u))) & 0xFFu);
+        const int sc1b = (int)(((jb < 4u ? scw1.x : scw1.y) >> (8u * (jb & 3u))) & 0xFFu);
+        const int4v xa_a = *(const int4v *)&x_l[buf][xrow];
+        const int4v wb0a = *(const int4v *)&w_l[buf][wrow0];
+        const int4v wb1a = *(const int4v *)&w_l[buf][wrow1];
+        const int4v xa_b = *(const int4v *)&x_l[buf][xrow + 32u];
+        const int4v wb0b = *(const int4v *)&w_l[buf][wrow0 + 32u];
+        const int4v wb1b = *(const int4v *)&w_l[buf][wrow1 + 32u];
+        const int16v p0a = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_a, wb0a, zi, 0, 0, 0);
+        const int16v p1a = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_a, wb1a, zi, 0, 0, 0);
+        const int16v p0b = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_b, wb0b, zi, 0, 0, 0);
+        const int16v p1b = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_b, wb1b, zi, 0, 0, 0);
+        if (g == 0u) {   // the super-block starts fresh sums
 #pragma unroll
-        for (uint32_t sub = 0; sub < 2u; sub++) {
-          const uint32_t j = 2u * g + sub;
-          const int sc0 = (int)(((j < 4u ? scw0.x : scw0.y) >> (8u * (j & 3u))) & 0xFFu);
-          const int sc1 = (int)(((j < 4u ? scw1.x : scw1.y) >> (8u * (j & 3u))) & 0xFFu);
-          const int4v xa = *(const int4v *)&x_l[buf][xrow + 32u * sub];
-          const int4v wb0 = *(const int4v *)&w_l[buf][wrow0 + 32u * sub];
-          const int4v wb1 = *(const int4v *)&w_l[buf][wrow1 + 32u * sub];
-          const int16v p0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wb0, zi, 0, 0, 0);
-          const int16v p1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wb1, zi, 0, 0, 0);
-          if (j == 0u) {   // the super-block starts fresh sums
+          for (int r = 0; r < 16; r++) i0[r] = __mul24(p0a[r], sc0a);
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-              i0[r] = __mul24(p0[r], sc0);
-              i1[r] = __mul24(p1[r], sc1);
-            }
-          } else {
+          for (int r = 0; r < 16; r++) i1[r] = __mul24(p1a[r], sc1a);
+        } else {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-              i0[r] = __mul24(p0[r], sc0) + i0[r];
-              i1[r] = __mul24(p1[r], sc1) + i1[r];
-            }
-          }
+          for (int r = 0; r < 16; r++) i0[r] = __mul24(p0a[r], sc0a) + i0[r];
+#pragma unroll
+          for (int r = 0; r < 16; r++) i1[r] = __mul24(p1a[r], sc1a) + i1[r];
         }
+#pragma unroll
+        for (int r = 0; r < 16; r++) i0[r] = __mul24(p0b[r], sc0b) + i0[r];
+#pragma unroll
+        for (int r = 0; r < 16; r++) i1[r] = __mul24(p1b[r], sc1b) + i1[r];
         if (g == 3u) {
           const float d0 = d_l[s & 1u][64u * rh + l32], d1 = d_l[s & 1u][64u * rh + 32u + l32];
           const float *adp = &ad_l[s & 1u][tw + 4u * lh];
@@ -704,6 +734,9 @@ __global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) {
     }
   }
 }
+
+__global__ __launch_bounds__(768) void ogm_gemm_q4k_i8_kernel(GemmParams p) { gemm_i8_body<false>(p); }
+__global__ __launch_bounds__(768) void ogm_gemm_q5k_i8_kernel(GemmParams p) { gemm_i8_body<true>(p); }
 
 // ------------------------------------------------------------------------------------------
 // Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
@@ -1728,9 +1761,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   uint32_t row_tiles = (a.out_dim + GM_BN - 1) / GM_BN;
   for (uint32_t m = 0; m < a.n_extra; m++) row_tiles += (a.extra_out_dim[m] + GM_BN - 1) / GM_BN;
   const uint32_t wgs128 = ((a.n_tokens + GM_BT - 1) / GM_BT) * row_tiles;
-  // Q4_K runs on the int8 kernel unless the f16 kernels are asked for (q4k_variant 2); of those the
-  // wide one takes over as described above
-  const bool i8 = a.ggml_type == OGM_Q4_K && a.q4k_variant != 2u;
+  // Q4_K and Q5_K run on the int8 kernel unless the f16 kernels are asked for (q4k_variant 2); of
+  // Q4_K's the wide one takes over as described above
+  const bool i8 = (a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K) && a.q4k_variant != 2u;
   const bool wide = a.ggml_type == OGM_Q4_K && !i8 && a.n_tokens > 256u &&
                     wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
   const bool raw_x = wide || i8;   // these read the int8 activations as they are: only (bh, bl) to prepare
@@ -1742,6 +1775,36 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   // power-of-two number of token tiles each XCD's L2 sees few distinct activation tiles
   const dim3 grid((a.n_tokens + GM_BT - 1) / GM_BT, row_tiles);
   hipError_t e;
+  if (i8) {
+    GemmParams p;
+    p.wt = a.wt;
+    p.xh = nullptr;
+    p.bs16 = bs16;
+    p.ad = a.act.d;
+    p.y = a.y;
+    p.in_dim = a.in_dim;
+    p.out_dim = a.out_dim;
+    p.n_tokens = a.n_tokens;
+    p.nsb = nsb;
+    p.c_shift = c_shift;
+    p.r_shift = 6 - c_shift;
+    p.nct = tl.nct;
+    p.xq = a.act.q;
+    p.n_extra = a.n_extra;
+    for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
+      p.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
+      p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
+      p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
+    }
+    if (a.ggml_type == OGM_Q4_K) {
+      hipLaunchKernelGGL(ogm_gemm_q4k_i8_kernel, grid, dim3(768), 0, stream, p);
+      if (kernel_name) *kernel_name = "ogm_gemm_q4k_i8_kernel";
+    } else {
+      hipLaunchKernelGGL(ogm_gemm_q5k_i8_kernel, grid, dim3(768), 0, stream, p);
+      if (kernel_name) *kernel_name = "ogm_gemm_q5k_i8_kernel";
+    }
+    return hipGetLastError();
+  }
   if (a.ggml_type != OGM_Q4_K) {
     Gemm6Params p;
     p.wt = a.wt;
@@ -1801,11 +1864,6 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
     p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
     p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
-  }
-  if (i8) {
-    hipLaunchKernelGGL(ogm_gemm_q4k_i8_kernel, grid, dim3(768), 0, stream, p);
-    if (kernel_name) *kernel_name = "ogm_gemm_q4k_i8_kernel";
-    return hipGetLastError();
   }
   if (wide) {
     const dim3 wgrid((a.n_tokens + GW_BT - 1) / GW_BT, row_tiles);

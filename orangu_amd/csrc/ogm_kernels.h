@@ -60,7 +60,7 @@ struct OgmGemmArgs {
   float *y;            // [n_tokens][out_dim]
   void *xh;            // scratch
   uint32_t wide_min_wgs = 0;   // Q4_K: least 128x128 workgroups from which the wide tiling runs (0 = default)
-  uint32_t q4k_variant = 0;    // Q4_K: 0 or 1 = the int8 kernel, 2 = the f16 kernels (128 x 128 or wide, by shape)
+  uint32_t q4k_variant = 0;    // Q4_K, Q5_K: 0 or 1 = the int8 kernel, 2 = the f16 kernels
   // K-quants: further matrices of the same type and in_dim over the same activations, in the same launch
   uint32_t n_extra = 0;
   const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1] = {};

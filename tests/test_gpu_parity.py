@@ -364,6 +364,7 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     (Q4_K, 300, (6000, 3000, 2100), "ogm_gemm_q4k_wide_kernel"),  # 264 tiles of 128 x 128: the wide tiling
     (Q6_K, 40, (300, 130, 64), "ogm_gemm_q6k_kernel"),
     (Q5_K, 130, (520, 70, 129), "ogm_gemm_q5k_kernel"),
+    (Q5_K, 130, (520, 70, 129), "ogm_gemm_q5k_i8_kernel"),
     (Q3_K, 40, (128, 300), "ogm_gemm_q3k_kernel"),
 ])
 def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, outs, kernel):
@@ -510,7 +511,8 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign):
     say("extreme q6k isum", int(np.abs(isum).max()))
 
 
-@pytest.mark.parametrize("t,kernel", [(Q3_K, "ogm_gemm_q3k_kernel"), (Q5_K, "ogm_gemm_q5k_kernel")])
+@pytest.mark.parametrize("t,kernel", [(Q3_K, "ogm_gemm_q3k_kernel"), (Q5_K, "ogm_gemm_q5k_kernel"),
+                                      (Q5_K, "ogm_gemm_q5k_i8_kernel")])
 @pytest.mark.parametrize("in_dim,out_dim,T", [
     (256, 5, 9), (512, 130, 17), (768, 64, 129), (1024, 100, 64), (1280, 257, 40), (2048, 37, 128),
     (4096, 200, 130), (14336, 96, 257), (4096, 1000, 512), (1792, 33, 10),
@@ -523,7 +525,11 @@ def test_mfma_gemm_q3k_q5k_match_cpu_gemm(be, t, kernel, in_dim, out_dim, T):
     x = synth_x(T, in_dim, seed=T + 1)
     w = qm(raw, t, in_dim, out_dim)
     say("gemm", kernel, in_dim, out_dim, T)
-    got = be.matmul(x, T, w)
+    be.set_tuning("gemm_q4k_variant", 0 if kernel.endswith("_i8_kernel") or t == Q3_K else 2)   # Q5_K: int8 by default
+    try:
+        got = be.matmul(x, T, w)
+    finally:
+        be.set_tuning("gemm_q4k_variant", 0)
     assert be.last_kernel() == kernel
     want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
     assert_close(got, want, kernel)
@@ -537,9 +543,10 @@ def test_mfma_gemm_q3k_q5k_match_cpu_gemm(be, t, kernel, in_dim, out_dim, T):
     assert_bits(got, small, "mfma vs multi-token gemv")
 
 
+@pytest.mark.parametrize("variant", [0, 2])
 @pytest.mark.parametrize("qs,qh,sc,sign", [(0xFF, 0xFF, 0xFF, "alt"), (0x00, 0x00, 0xFF, "pos"), (0xFF, 0xFF, 0xFF, "neg"),
                                            (0xFF, 0xFF, 0x3F, "block"), (0xF0, 0x55, 0xC7, "alt"), (0x0F, 0xAA, 0x00, "pos")])
-def test_mfma_gemm_q5k_adversarial_integer_ranges(be, qs, qh, sc, sign):
+def test_mfma_gemm_q5k_adversarial_integer_ranges(be, qs, qh, sc, sign, variant):
     """Weights 0 and 31, scales and mins 63, activations +-127: a super-block's sum reaches
     63 * 31 * 127 * 256 = 6.3e7 and the mins' 63 * 8 * 4064 = 2.0e6; the two scale digits' chains
     stay exact and 16 * c_hi + c_lo rounds like `isum as f32`."""
@@ -560,8 +567,12 @@ def test_mfma_gemm_q5k_adversarial_integer_ranges(be, qs, qh, sc, sign):
         x[:, 128:256] *= -1
         x[3] = -127.0
     raw = blocks.reshape(-1)
-    got = be.matmul(x, T, qm(raw, Q5_K, in_dim, out_dim))
-    assert be.last_kernel() == "ogm_gemm_q5k_kernel"
+    be.set_tuning("gemm_q4k_variant", variant)
+    try:
+        got = be.matmul(x, T, qm(raw, Q5_K, in_dim, out_dim))
+    finally:
+        be.set_tuning("gemm_q4k_variant", 0)
+    assert be.last_kernel() == ("ogm_gemm_q5k_i8_kernel" if variant == 0 else "ogm_gemm_q5k_kernel")
     assert_bits(got, oracle.matmul(Q5_K, raw, in_dim, out_dim, x, T), "extreme ranges")
     isum, imin = be.dump_block_sums(x[0], 1, qm(raw, Q5_K, in_dim, out_dim))
     say("extreme q5k isum", int(np.abs(isum).max()), "imin", int(np.abs(imin).max()))
