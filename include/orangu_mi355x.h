@@ -327,11 +327,14 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * keys: "gemv_wg_waves" (waves per workgroup of the GEMV kernel, 1..16; 0 = heuristic);
  * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default 9,
  * below it the multi-token GEMV kernel runs in the GEMM's float order);
- * "gemm_q4k_variant" (Q4_K GEMM: 0 = default, the int8 matrix-core kernel; 2 = the f16 kernels);
+ * "gemm_q4k_variant" (K-quant GEMM: 0 = default, the int8 matrix-core kernels of Q4_K, Q5_K and Q6_K;
+ * 1 = the same with Q6_K always on its 64-row tile; 2 = the f16 kernels);
  * "gemm_wide_min_wgs" (f16 Q4_K kernels: 128 x 128 workgroups from which the 128 x 256 tile runs; 0 = 256);
+ * "attn_prefill_variant" (attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the
+ * decode step's kernel per token and chunk of the cache; they agree to f32 rounding, not bit for bit);
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
- * the quantizer kernel first; 0 or -1 = default, off).  No setting changes a result bit. */
+ * the quantizer kernel first; 0 or -1 = default, off).  No other setting changes a result bit. */
 int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value);
 /* Name of the kernel the last matmul on this context launched (for profiles). */
 const char *ogm_last_kernel(ogm_ctx *ctx);

@@ -47,6 +47,7 @@ struct ogm_ctx {
   int tune_gemm_min_tokens = 9;  // matmul at n_tokens >= this takes the MFMA GEMM
   int tune_gemm_wide_min_wgs = 0;
   int tune_gemm_q4k_variant = 0;
+  int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
   const char *last_kernel = "";
@@ -212,6 +213,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemm_wide_min_wgs") == 0) {
     if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_wide_min_wgs must be >= 0");
     ctx->tune_gemm_wide_min_wgs = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "attn_prefill_variant") == 0) {
+    if (value < 0 || value > 1) return fail(ctx, OGM_ERR_INVALID, "attn_prefill_variant must be 0 or 1");
+    ctx->tune_attn_prefill_variant = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_q4k_variant") == 0) {
@@ -1209,7 +1215,10 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_qkv_pre(P.q, P.k, P.v, P.cs, c.rope_dim, pre, c.n_head, c.n_head_kv, c.head_dim, kc, vc,
                                    pos0, T, s));
-    for (uint32_t t0 = 0; t0 < T; t0 += P.attn_tokens) {
+    if (ctx->tune_attn_prefill_variant == 0) {
+      HIPCHK(ctx, ogm_launch_attn_prefill_mfma(P.q, kc, vc, pos0, T, c.n_head, c.n_head_kv, c.head_dim, scale, P.attn, s));
+    }
+    for (uint32_t t0 = 0; ctx->tune_attn_prefill_variant != 0 && t0 < T; t0 += P.attn_tokens) {
       const uint32_t nt = T - t0 < P.attn_tokens ? T - t0 : P.attn_tokens;
       HIPCHK(ctx, ogm_launch_attn_prefill(P.q + (size_t)t0 * qd, kc, vc, pos0 + t0, nt, m->max_splits, c.n_head,
                                           c.n_head_kv, c.head_dim, scale, P.part_o, P.part_ml,

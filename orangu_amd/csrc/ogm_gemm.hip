@@ -741,11 +741,10 @@ __global__ __launch_bounds__(768) void ogm_gemm_q5k_i8_kernel(GemmParams p) { ge
 // ------------------------------------------------------------------------------------------
 // Q6_K on the int8 matrix cores (gemm_k_q6_k, vecdot.rs:2352-2398): scales per 16 weights would
 // mean one multiply-add per output for every 16 products, so here the feeding waves fold the
-// scale into the weight, w' = sc_g * (q - 32) in [-4096, 4064], and split it into two int8
-// planes, w' = 64 h + l with l = w' & 63 in [0, 63] and h = w' >> 6 in [-64, 63].  The multiplying
-// waves then run two plain chains of v_mfma_i32_32x32x32_i8 over the whole super-block,
-// accumulating in the instruction itself, and isum = 64 H + L in 32-bit integers: exact, one
-// `as f32` per super-block.  Same tile, waves and orientation as gemm_i8_body.
+// scale into the weight, w' = sc_g * (q - 32) in [-4064, 4096], and split it into two int8
+// planes, w' = 256 h + l with l in [-128, 127] and h in [-16, 16].  The multiplying waves then run
+// two plain chains of v_mfma_i32_32x32x32_i8 over the whole super-block, accumulating in the
+// instruction itself, and isum = 256 H + L in 32-bit integers: exact, one `as f32` per super-block.  Same tile, waves and orientation as gemm_i8_body.
 
 typedef short short2v __attribute__((ext_vector_type(2)));
 
@@ -762,25 +761,31 @@ struct GemmI8pParams {
   uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
 };
 
-__global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) {
+// ROWS = 128: eight multiplying waves (64 rows x 32 tokens each) and four feeding ones; ROWS = 64:
+// four and two, half the LDS, and two workgroups to a CU, which fills the chip when a launch has
+// few row tiles and lets one workgroup's LDS traffic run under the other's matrix instructions.
+template <uint32_t ROWS>
+__device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
+  constexpr uint32_t NC = ROWS / 16u;                // multiplying waves
+  constexpr uint32_t WT = ROWS * GI_ROW;             // bytes of a plane's stage
   constexpr uint32_t TILE_BYTES = 13440u;   // 64 units of 210 bytes: 13 pieces of 1 KiB, then 64 two-byte tails
   // three stages of 64 weights in LDS: one being multiplied, the next being read into registers
   // behind it, the third being written by the feeding waves
   extern __shared__ __align__(16) uint8_t lds[];
-  uint8_t *wh_l = lds;                          // [3][128 rows][64 of 80]: plane h
-  uint8_t *wl_l = lds + 3u * GI_WTILE;          // plane l
-  uint8_t *x_l = lds + 6u * GI_WTILE;           // [3][128 tokens][64 of 80]: activations
-  float *d_l = (float *)(lds + 9u * GI_WTILE);  // [2][128] the rows' d
-  float *ad_l = d_l + 256;                      // [2][128] the tokens' activation scale
+  uint8_t *wh_l = lds;                                      // [3][ROWS][64 of 80]: plane h
+  uint8_t *wl_l = lds + 3u * WT;                            // plane l
+  uint8_t *x_l = lds + 6u * WT;                             // [3][128 tokens][64 of 80]: activations
+  float *d_l = (float *)(lds + 6u * WT + 3u * GI_WTILE);    // [2][ROWS] the rows' d
+  float *ad_l = d_l + 2u * ROWS;                            // [2][128] the tokens' activation scale
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const bool producer = wave >= 8u;
+  const bool producer = wave >= NC;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
-  const uint32_t tq = wave & 3u, rh = (wave >> 2) & 1u;
+  const uint32_t tq = wave & 3u, rh = ROWS == 128u ? (wave >> 2) & 1u : 0u;
   uint32_t row_tile = blockIdx.y;
 #pragma unroll
   for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
-    const uint32_t tiles = (p.out_dim + 127u) / 128u;
+    const uint32_t tiles = (p.out_dim + ROWS - 1u) / ROWS;
     if (m < p.n_extra && row_tile >= tiles) {
       row_tile -= tiles;
       p.wt = p.extra_wt[m];
@@ -790,39 +795,45 @@ __global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) {
       break;
     }
   }
-  const uint32_t t0 = blockIdx.x * 128u, r0 = row_tile * 128u;
+  const uint32_t t0 = blockIdx.x * 128u, r0 = row_tile * ROWS;
   const uint32_t tw = 32u * tq;
 
   auto sb_tile = [&](uint32_t s) -> uint32_t { return (s >> p.c_shift) * TILE_BYTES; };
   auto sb_lane = [&](uint32_t s) -> uint32_t { return (s & ((1u << p.c_shift) - 1u)) << p.r_shift; };
 
   if (producer) {
-    // Feeding thread pt stages two groups of 16 weights per stage (rows pt % 64 and pt % 64 + 64,
-    // group pt / 64, the same for a whole wave: one ql piece, one qh piece, one scale each; a
-    // wave's loads are 1 KiB runs and its LDS rows are 80 bytes apart, which spreads over all banks)
-    // and 32 bytes of activations; once per super-block the rows' d (128 threads) and the tokens' ad
-    // (the other 128).
-    const uint32_t pt = tid - 512u;
-    const uint32_t t16 = __builtin_amdgcn_readfirstlane(pt >> 6), prw = pt & 63u;
-    uint32_t uo[2], to[2];
+    // Feeding thread pt stages two groups of 16 weights per stage, a and b: one ql piece, one qh
+    // piece, one scale each.  A wave has one group index and 64 consecutive rows: its loads are
+    // 1 KiB runs and its LDS rows are 80 bytes apart, which spreads over all banks.  ROWS = 128:
+    // rows pt % 64 and pt % 64 + 64, group pt / 64; ROWS = 64: row pt % 64, groups pt / 64 and
+    // pt / 64 + 2, which share the qh piece and the scales.  And the activations: 32 bytes of a
+    // token (64 with half as many feeding threads).  Once per super-block the rows' d and the
+    // tokens' ad.
+    const uint32_t pt = tid - 64u * NC;
+    const uint32_t t16a = __builtin_amdgcn_readfirstlane(pt >> 6), prw = pt & 63u;
+    const uint32_t t16b = ROWS == 128u ? t16a : t16a + 2u, prwb = ROWS == 128u ? prw + 64u : prw;
+    uint32_t uo[2];
 #pragma unroll
     for (int k = 0; k < 2; k++) {
-      const uint32_t row = min(r0 + prw + 64u * k, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+      const uint32_t row = min(r0 + (k ? prwb : prw), p.out_dim - 1u);   // rows past the matrix: clamped, never stored
       const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
       uo[k] = rb * p.nct * TILE_BYTES + r * 16u;
-      to[k] = rb * p.nct * TILE_BYTES + 13u * 1024u + r * 2u;
     }
-    const uint32_t xrow_ = pt >> 1, xhalf = pt & 1u;
-    const uint32_t xro = min(t0 + xrow_, p.n_tokens - 1u) * p.in_dim + 32u * xhalf;   // + 256 s + 64 g
-    uint32_t dto;   // this thread's row for d (pt < 128), or token for ad
+    constexpr uint32_t XB = ROWS == 128u ? 32u : 64u;   // bytes of a token's stage per feeding thread
+    const uint32_t xrow_ = ROWS == 128u ? pt >> 1 : pt, xhalf = ROWS == 128u ? pt & 1u : 0u;
+    const uint32_t xro = min(t0 + xrow_, p.n_tokens - 1u) * p.in_dim + XB * xhalf;   // + 256 s + 64 g
+    const bool has_d = pt < ROWS, has_ad = ROWS == 128u ? pt >= 128u : true;
+    const uint32_t ad_tok = ROWS == 128u ? pt - 128u : pt;
+    uint32_t dto;   // the row whose d this thread fetches
     {
-      const uint32_t row = min(r0 + (pt & 127u), p.out_dim - 1u);
+      const uint32_t row = min(r0 + (pt & (ROWS - 1u)), p.out_dim - 1u);
       dto = (row >> p.r_shift) * p.nct * TILE_BYTES + 13u * 1024u + (row & ((1u << p.r_shift) - 1u)) * 2u;
     }
-    const uint32_t aro = min(t0 + (pt & 127u), p.n_tokens - 1u) * p.nsb;
+    const uint32_t aro = min(t0 + (ad_tok & 127u), p.n_tokens - 1u) * p.nsb;
     // the ring of stages in flight, slot = stage % 4 = g, in named registers
     uint4 qla0, qla1, qla2, qla3, qha0, qha1, qha2, qha3, qlb0, qlb1, qlb2, qlb3, qhb0, qhb1, qhb2, qhb3;
     uint4 xa0_, xa1_, xa2_, xa3_, xb0_, xb1_, xb2_, xb3_;
+    uint4 xc0_, xc1_, xc2_, xc3_, xd0_, xd1_, xd2_, xd3_;   // ROWS = 64: the token's other 32 bytes
     uint4 scxa = make_uint4(0, 0, 0, 0), scxb = make_uint4(0, 0, 0, 0);   // the 16 scales of the two rows, next super-block
     uint32_t sca[4] = {0, 0, 0, 0}, scb[4] = {0, 0, 0, 0};                // ... of the super-block being stored
     uint32_t d16 = 0;
@@ -831,28 +842,34 @@ __global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) {
   do {                                                                                            \
     const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded again, never used */ \
     const uint32_t so_ = sb_tile(s_) + sb_lane(s_) * 16u, h_ = (G) >> 1;                          \
-    qla##K = *(const uint4 *)(p.wt + (uo[0] + so_ + (4u * h_ + t16) * 1024u));                    \
-    qha##K = *(const uint4 *)(p.wt + (uo[0] + so_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));        \
-    qlb##K = *(const uint4 *)(p.wt + (uo[1] + so_ + (4u * h_ + t16) * 1024u));                    \
-    qhb##K = *(const uint4 *)(p.wt + (uo[1] + so_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));        \
+    qla##K = *(const uint4 *)(p.wt + (uo[0] + so_ + (4u * h_ + t16a) * 1024u));                   \
+    qha##K = *(const uint4 *)(p.wt + (uo[0] + so_ + (8u + 2u * h_ + (t16a & 1u)) * 1024u));       \
+    qlb##K = *(const uint4 *)(p.wt + (uo[1] + so_ + (4u * h_ + t16b) * 1024u));                   \
+    if constexpr (ROWS == 128u)                                                                   \
+      qhb##K = *(const uint4 *)(p.wt + (uo[1] + so_ + (8u + 2u * h_ + (t16b & 1u)) * 1024u));     \
     const uint4 *xp_ = (const uint4 *)(p.xq + (xro + 256u * s_ + 64u * (G)));                     \
     xa##K##_ = xp_[0];                                                                            \
     xb##K##_ = xp_[1];                                                                            \
+    if constexpr (ROWS == 64u) {                                                                  \
+      xc##K##_ = xp_[2];                                                                          \
+      xd##K##_ = xp_[3];                                                                          \
+    }                                                                                             \
     if ((G) == 0u) {                                                                              \
       scxa = *(const uint4 *)(p.wt + (uo[0] + so_ + 12u * 1024u));                                \
-      scxb = *(const uint4 *)(p.wt + (uo[1] + so_ + 12u * 1024u));                                \
-      if (pt < 128u) d16 = *(const uint16_t *)(p.wt + (dto + sb_tile(s_) + sb_lane(s_) * 2u));    \
-      else adn = p.ad[aro + s_];                                                                  \
+      if constexpr (ROWS == 128u) scxb = *(const uint4 *)(p.wt + (uo[1] + so_ + 12u * 1024u));    \
+      if (has_d) d16 = *(const uint16_t *)(p.wt + (dto + sb_tile(s_) + sb_lane(s_) * 2u));        \
+      if (has_ad) adn = p.ad[aro + s_];                                                           \
     }                                                                                             \
   } while (0)
-  // sixteen 6-bit weights of one group -> sc * (q - 32) as two int8 planes, into the group's 16
-  // bytes of the row in each plane's tile
-#define GP_GROUP(QL, QH, SCW, G, BUF, ROWOFF)                                                     \
+  // sixteen 6-bit weights of one group -> the two int8 planes of sc * (q - 32), into the group's
+  // 16 bytes of the row in each plane's tile.  u = sc * q + (128 - 32 sc) is a 16-bit lane whose
+  // high byte is h and whose low byte, top bit flipped and read as int8, is l = (u & 255) - 128.
+#define GP_GROUP(QL, QH, SCW, G, BUF, ROWOFF, T16)                                                  \
   do {                                                                                            \
-    const int sc_ = (int)(int8_t)(((SCW)[(G)] >> (8u * t16)) & 0xFFu);                            \
+    const int sc_ = (int)(int8_t)(((SCW)[(G)] >> (8u * (T16))) & 0xFFu);                          \
     const short2v sc2_ = {(short)sc_, (short)sc_};                                                \
-    const short2v k32_ = {32, 32};                                                                \
-    const uint32_t rr_ = 2u * ((G) & 1u) + (t16 >> 1);        /* run of 32 inside the half block */ \
+    const short2v c2_ = {(short)(128 - 32 * sc_), (short)(128 - 32 * sc_)};                       \
+    const uint32_t rr_ = 2u * ((G) & 1u) + ((T16) >> 1);      /* run of 32 inside the half block */ \
     const uint32_t qlw_[4] = {QL.x, QL.y, QL.z, QL.w}, qhw_[4] = {QH.x, QH.y, QH.z, QH.w};        \
     uint32_t ph_[4], pl_[4];                                                                      \
     _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
@@ -861,34 +878,39 @@ __global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) {
       union { uint32_t u; short2v s; } e_, f_;                                                    \
       e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
       f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
-      e_.s = (e_.s - k32_) * sc2_;                                                                \
-      f_.s = (f_.s - k32_) * sc2_;                                                                \
-      union { uint32_t u; short2v s; } eh_, fh_;                                                  \
-      eh_.s = e_.s >> 6;                                                                          \
-      fh_.s = f_.s >> 6;                                                                          \
-      /* bytes 0 and 2 of each pair: the low bytes of its two 16-bit lanes */                     \
-      pl_[w_] = __builtin_amdgcn_perm(f_.u & 0x003F003Fu, e_.u & 0x003F003Fu, 0x06040200u);       \
-      ph_[w_] = __builtin_amdgcn_perm(fh_.u, eh_.u, 0x06040200u);                                 \
+      e_.s = e_.s * sc2_ + c2_;                                                                   \
+      f_.s = f_.s * sc2_ + c2_;                                                                   \
+      ph_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x07050301u);                /* high bytes */   \
+      pl_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u) ^ 0x80808080u;  /* low bytes */    \
     }                                                                                             \
-    *(uint4 *)&wh_l[(BUF) + (ROWOFF) * GI_ROW + 16u * t16] = make_uint4(ph_[0], ph_[1], ph_[2], ph_[3]); \
-    *(uint4 *)&wl_l[(BUF) + (ROWOFF) * GI_ROW + 16u * t16] = make_uint4(pl_[0], pl_[1], pl_[2], pl_[3]); \
+    *(uint4 *)&wh_l[(BUF) + (ROWOFF) * GI_ROW + 16u * (T16)] = make_uint4(ph_[0], ph_[1], ph_[2], ph_[3]); \
+    *(uint4 *)&wl_l[(BUF) + (ROWOFF) * GI_ROW + 16u * (T16)] = make_uint4(pl_[0], pl_[1], pl_[2], pl_[3]); \
   } while (0)
 #define GP_STORE(S, G, K)                                                                         \
   do {                                                                                            \
     if ((G) == 0u) {                                                                              \
       sca[0] = scxa.x; sca[1] = scxa.y; sca[2] = scxa.z; sca[3] = scxa.w;                         \
-      scb[0] = scxb.x; scb[1] = scxb.y; scb[2] = scxb.z; scb[3] = scxb.w;                         \
-      if (pt < 128u) d_l[128u * ((S) & 1u) + pt] = gm_f16_bits_to_f32(d16);                       \
-      else ad_l[128u * ((S) & 1u) + pt - 128u] = adn;                                             \
+      if constexpr (ROWS == 128u) {                                                               \
+        scb[0] = scxb.x; scb[1] = scxb.y; scb[2] = scxb.z; scb[3] = scxb.w;                       \
+      }                                                                                           \
+      if (has_d) d_l[ROWS * ((S) & 1u) + pt] = gm_f16_bits_to_f32(d16);                           \
+      if (has_ad) ad_l[128u * ((S) & 1u) + ad_tok] = adn;                                         \
     }                                                                                             \
-    GP_GROUP(qla##K, qha##K, sca, G, pb, prw);                                                    \
-    GP_GROUP(qlb##K, qhb##K, scb, G, pb, prw + 64u);                                              \
-    uint8_t *xr_ = &x_l[pb + xrow_ * GI_ROW + 32u * xhalf];                                       \
+    GP_GROUP(qla##K, qha##K, sca, G, pw, prw, t16a);                                              \
+    if constexpr (ROWS == 128u) GP_GROUP(qlb##K, qhb##K, scb, G, pw, prwb, t16b);                 \
+    else GP_GROUP(qlb##K, qha##K, sca, G, pw, prwb, t16b);                                        \
+    uint8_t *xr_ = &x_l[px + xrow_ * GI_ROW + XB * xhalf];                                        \
     *(uint4 *)xr_ = xa##K##_;                                                                     \
     *(uint4 *)(xr_ + 16u) = xb##K##_;                                                             \
-    pb = pb == 2u * GI_WTILE ? 0u : pb + GI_WTILE;   /* stages go round the three buffers */      \
+    if constexpr (ROWS == 64u) {                                                                  \
+      *(uint4 *)(xr_ + 32u) = xc##K##_;                                                           \
+      *(uint4 *)(xr_ + 48u) = xd##K##_;                                                           \
+    }                                                                                             \
+    /* stages go round the three buffers */                                                       \
+    pw = pw == 2u * WT ? 0u : pw + WT;                                                            \
+    px = px == 2u * GI_WTILE ? 0u : px + GI_WTILE;                                                \
   } while (0)
-    uint32_t pb = 0;
+    uint32_t pw = 0, px = 0;   // byte offsets of the stage being stored: weight planes, activations
     GP_LOAD(0u, 0u, 0);
     GP_LOAD(0u, 1u, 1);
     GP_LOAD(0u, 2u, 2);
@@ -928,21 +950,21 @@ __global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) {
     // operands of the stage's first 32 weights (a) and last 32 (b); a of the next stage is read
     // while b multiplies, b while a does
     int4v xa, wh0a, wh1a, wl0a, wl1a, xb, wh0b, wh1b, wl0b, wl1b;
-    uint32_t cb = 0;   // byte offset of the stage's buffer
-#define GP_READ(SUF, OFF)                                     \
+    uint32_t cw = 0, cx = 0;   // byte offsets of the stage's buffers: weight planes, activations
+#define GP_READ(SUF, OFFW, OFFX)                              \
   do {                                                        \
-    x##SUF = *(const int4v *)&x_l[(OFF) + xrow];              \
-    wh0##SUF = *(const int4v *)&wh_l[(OFF) + wrow0];          \
-    wh1##SUF = *(const int4v *)&wh_l[(OFF) + wrow1];          \
-    wl0##SUF = *(const int4v *)&wl_l[(OFF) + wrow0];          \
-    wl1##SUF = *(const int4v *)&wl_l[(OFF) + wrow1];          \
+    x##SUF = *(const int4v *)&x_l[(OFFX) + xrow];             \
+    wh0##SUF = *(const int4v *)&wh_l[(OFFW) + wrow0];         \
+    wh1##SUF = *(const int4v *)&wh_l[(OFFW) + wrow1];         \
+    wl0##SUF = *(const int4v *)&wl_l[(OFFW) + wrow0];         \
+    wl1##SUF = *(const int4v *)&wl_l[(OFFW) + wrow1];         \
   } while (0)
-    GP_READ(a, 0u);
+    GP_READ(a, 0u, 0u);
     for (uint32_t s = 0; s < p.nsb; s++) {
 #pragma unroll
       for (uint32_t g = 0; g < 4u; g++) {
-        const uint32_t nb = cb == 2u * GI_WTILE ? 0u : cb + GI_WTILE;
-        GP_READ(b, cb + 32u);
+        const uint32_t nw = cw == 2u * WT ? 0u : cw + WT, nx = cx == 2u * GI_WTILE ? 0u : cx + GI_WTILE;
+        GP_READ(b, cw + 32u, cx + 32u);
         if (g == 0u) {   // the super-block starts fresh sums
           h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh0a, zi, 0, 0, 0);
           h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh1a, zi, 0, 0, 0);
@@ -954,14 +976,15 @@ __global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) {
           l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl0a, l0, 0, 0, 0);
           l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl1a, l1, 0, 0, 0);
         }
-        GP_READ(a, nb);   // complete since the last barrier; past the last stage: read, never used
+        GP_READ(a, nw, nx);   // complete since the last barrier; past the last stage: read, never used
         h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wh0b, h0, 0, 0, 0);
         h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wh1b, h1, 0, 0, 0);
         l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wl0b, l0, 0, 0, 0);
         l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wl1b, l1, 0, 0, 0);
-        cb = nb;
+        cw = nw;
+        cx = nx;
         if (g == 3u) {
-          const float d0 = d_l[128u * (s & 1u) + 64u * rh + l32], d1 = d_l[128u * (s & 1u) + 64u * rh + 32u + l32];
+          const float d0 = d_l[ROWS * (s & 1u) + 64u * rh + l32], d1 = d_l[ROWS * (s & 1u) + 64u * rh + 32u + l32];
           const float *adp = &ad_l[128u * (s & 1u) + tw + 4u * lh];
 #pragma unroll
           for (int q4 = 0; q4 < 4; q4++) {
@@ -969,8 +992,8 @@ __global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) {
             const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-              const int is0 = h0[4 * q4 + e] * 64 + l0[4 * q4 + e];
-              const int is1 = h1[4 * q4 + e] * 64 + l1[4 * q4 + e];
+              const int is0 = h0[4 * q4 + e] * 256 + l0[4 * q4 + e];
+              const int is1 = h1[4 * q4 + e] * 256 + l1[4 * q4 + e];
               y0[4 * q4 + e] += a4v[e] * (d0 * (float)is0);
               y1[4 * q4 + e] += a4v[e] * (d1 * (float)is1);
             }
@@ -991,6 +1014,9 @@ __global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) {
     }
   }
 }
+
+__global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u>(p); }
+__global__ __launch_bounds__(384) void ogm_gemm_q6k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u>(p); }
 
 // ------------------------------------------------------------------------------------------
 // Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
@@ -2079,11 +2105,26 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
       p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
     }
-    const uint32_t lds_bytes = 9u * GI_WTILE + 4u * 128u * 4u;
-    hipError_t e = hipFuncSetAttribute((const void *)ogm_gemm_q6k_i8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    // 64-row tiles when asked for (q4k_variant 1), or when they still come one to a CU: then twice
+    // as many CUs work (14336 -> 4096 x 512 tokens: 150 us against 180 us).  Two of them sharing a CU
+    // are slower than one 128-row tile (4096 -> 14336 x 512: 165 us against 118 us).
+    uint32_t tiles64 = (a.out_dim + 63u) / 64u;
+    for (uint32_t m = 0; m < a.n_extra; m++) tiles64 += (a.extra_out_dim[m] + 63u) / 64u;
+    const bool r64 = a.q4k_variant == 1u || ((a.n_tokens + 127u) / 128u) * tiles64 <= 256u;
+    const uint32_t rows = r64 ? 64u : 128u;
+    const uint32_t tiles = r64 ? tiles64 : row_tiles;
+    const dim3 pgrid((a.n_tokens + 127u) / 128u, tiles);
+    const uint32_t lds_bytes = 6u * rows * GI_ROW + 3u * GI_WTILE + (2u * rows + 256u) * 4u;
+    const void *fn = r64 ? (const void *)ogm_gemm_q6k_i8_r64_kernel : (const void *)ogm_gemm_q6k_i8_kernel;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(ogm_gemm_q6k_i8_kernel, grid, dim3(768), lds_bytes, stream, p);
-    if (kernel_name) *kernel_name = "ogm_gemm_q6k_i8_kernel";
+    if (r64) {
+      hipLaunchKernelGGL(ogm_gemm_q6k_i8_r64_kernel, pgrid, dim3(384), lds_bytes, stream, p);
+      if (kernel_name) *kernel_name = "ogm_gemm_q6k_i8_r64_kernel";
+    } else {
+      hipLaunchKernelGGL(ogm_gemm_q6k_i8_kernel, pgrid, dim3(768), lds_bytes, stream, p);
+      if (kernel_name) *kernel_name = "ogm_gemm_q6k_i8_kernel";
+    }
     return hipGetLastError();
   }
   if (a.ggml_type != OGM_Q4_K) {

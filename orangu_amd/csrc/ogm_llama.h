@@ -95,5 +95,11 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
                                    uint32_t head_dim, float scale, float *part_o, float *part_ml, float *attn_out,
                                    hipStream_t stream);
 
+// The same on the matrix cores, one launch and no partial results: query tiles of 32 tokens, cache
+// tiles of 64 positions, running softmax.  head_dim 64 or 128, at most 8 query heads per K/V head.
+hipError_t ogm_launch_attn_prefill_mfma(const float *q, void *k_cache_layer, void *v_cache_layer, uint32_t pos0,
+                                        uint32_t n_tokens, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
+                                        float scale, float *attn_out, hipStream_t stream);
+
 // h = silu(gate) * up over n values.  n % 4 == 0.
 hipError_t ogm_launch_swiglu_rows(const float *gate, const float *up, size_t n, float *h, hipStream_t stream);

@@ -1025,6 +1025,236 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
   return hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------
+// Prefill attention on the matrix cores.  Workgroup (query tile of 32 tokens, K/V head, group of
+// four query heads), four waves: wave w takes query head 4 z + w of the K/V head and walks the
+// cache in tiles of 64 positions up to the tile's last query (causal), with a running maximum and
+// sum per query (the softmax of llama.rs's attention, tensor.rs softmax_rows, regrouped).
+//
+//   scores^T = K . Q^T    A = K rows from LDS (16 bytes of a row are 8 consecutive dimensions),
+//                         B = Q^T from registers; the result has one query per lane and 16
+//                         positions per 32 x 32 block in its registers, so maximum and sum of a
+//                         query are in-lane reductions plus one exchange between the lane halves
+//   out^T += V^T . P^T    A = V^T from LDS, B = P^T: exactly the registers the scores came in
+//
+// V is transposed on its way into LDS (8 x 8 blocks in registers, byte permutes); its columns are
+// stored in the order in which a lane half holds the positions (within each 16: 0-3, 8-11, 4-7,
+// 12-15), so that an operand is 16 contiguous bytes.  K, V are f16 in the cache and exact in the
+// products; q and the probabilities are f32 and go in as two f16 terms each (value = hi + lo),
+// which keeps 22 bits of them: the results differ from f32 arithmetic by f32 rounding only.
+
+typedef _Float16 ah8 __attribute__((ext_vector_type(8)));
+typedef float af16 __attribute__((ext_vector_type(16)));
+
+#define AM_KT 64u                      // positions per tile
+#define AM_VROW (AM_KT * 2u + 16u)     // bytes of a row of V^T in LDS
+
+__device__ __forceinline__ void am_split(float v, _Float16 &hi, _Float16 &lo) {
+  hi = (_Float16)v;
+  lo = (_Float16)(v - (float)hi);
+}
+
+template <int HD>
+__global__ __launch_bounds__(256) void ogm_attn_prefill_mfma_kernel(const float *__restrict__ q,
+                                                                    const __half *__restrict__ kc,
+                                                                    const __half *__restrict__ vc, uint32_t pos0,
+                                                                    uint32_t n_tokens, uint32_t n_head_kv, uint32_t gq,
+                                                                    float scale, float *__restrict__ attn_out) {
+  constexpr uint32_t KROW = HD * 2u + 16u;   // bytes of a K row in LDS
+  constexpr int NS = HD / 16;                // k steps of a score block
+  constexpr int NDB = HD / 32;               // 32-dimension blocks of the output
+  constexpr uint32_t PPR = HD / 8;           // 16-byte pieces per cache row
+  constexpr int NK = (int)(AM_KT * PPR / 128u);   // pieces a K-copying thread moves per tile (8 or 4)
+  __shared__ __align__(16) uint8_t k_l[AM_KT * KROW];
+  __shared__ __align__(16) uint8_t vt_l[HD * AM_VROW];
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  const uint32_t qt = gridDim.x - 1u - blockIdx.x;   // long tiles first
+  const uint32_t kvh = blockIdx.y, g = 4u * blockIdx.z + wave;
+  const bool live = g < gq;
+  const uint32_t n_head = n_head_kv * gq, kv_dim = n_head_kv * HD;
+  const uint32_t tok = min(32u * qt + l32, n_tokens - 1u);   // this lane's query (clamped: computed, not stored)
+  const uint32_t q_abs = pos0 + tok;
+  const uint32_t last_pos = pos0 + min(32u * qt + 31u, n_tokens - 1u);
+  const uint32_t n_tiles = last_pos / AM_KT + 1u;
+  const uint32_t max_row = pos0 + n_tokens - 1u;   // last cache row that holds data
+
+  // q of this lane's query, head g: for k step s the dimensions 16 s + 8 lh + 0..7, as hi + lo
+  ah8 qh[NS], ql[NS];
+  {
+    const float *qp = q + ((size_t)tok * n_head + (size_t)kvh * gq + (live ? g : 0u)) * HD + 8u * lh;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+      const float4 a = *(const float4 *)(qp + 16 * s), b = *(const float4 *)(qp + 16 * s + 4);
+      const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        _Float16 hi, lo;
+        am_split(v[e], hi, lo);
+        qh[s][e] = hi;
+        ql[s][e] = lo;
+      }
+    }
+  }
+
+  // staging roles: threads 0..127 transpose V (one 8 x 8 block each: position group pg, dimension
+  // block db), threads 128..255 copy K (NK pieces each)
+  const bool v_thread = tid < 128u;
+  const uint32_t vdb = tid % PPR, vpg = tid / PPR;           // pg = 4 pb + 2 j + lh', 8 of them
+  const bool v_active = v_thread && vpg < 8u;
+  const uint32_t vp0 = 32u * (vpg >> 2) + 16u * ((vpg >> 1) & 1u) + 4u * (vpg & 1u);   // positions vp0 + 0..3, vp0 + 8 + 0..3
+  const uint32_t kt_ = tid - 128u;
+  uint4 pf[8];
+#define AM_LOAD(TILE)                                                                             \
+  do {                                                                                            \
+    const uint32_t base_ = (TILE) * AM_KT;                                                        \
+    if (v_thread) {                                                                               \
+      if (v_active) {                                                                             \
+        _Pragma("unroll") for (int e = 0; e < 8; e++) {                                           \
+          const uint32_t row_ = min(base_ + vp0 + 8u * (e >> 2) + (e & 3), max_row);              \
+          pf[e] = *(const uint4 *)(vc + (size_t)row_ * kv_dim + kvh * HD + 8u * vdb);             \
+        }                                                                                         \
+      }                                                                                           \
+    } else {                                                                                      \
+      _Pragma("unroll") for (int u = 0; u < NK; u++) {                                            \
+        const uint32_t i_ = kt_ + 128u * u;                                                       \
+        const uint32_t row_ = min(base_ + i_ / PPR, max_row);                                     \
+        pf[u] = *(const uint4 *)(kc + (size_t)row_ * kv_dim + kvh * HD + 8u * (i_ % PPR));        \
+      }                                                                                           \
+    }                                                                                             \
+  } while (0)
+#define AM_STORE()                                                                                \
+  do {                                                                                            \
+    if (v_thread) {                                                                               \
+      if (v_active) {                                                                             \
+        const uint32_t r_[8][4] = {{pf[0].x, pf[0].y, pf[0].z, pf[0].w}, {pf[1].x, pf[1].y, pf[1].z, pf[1].w}, \
+                                   {pf[2].x, pf[2].y, pf[2].z, pf[2].w}, {pf[3].x, pf[3].y, pf[3].z, pf[3].w}, \
+                                   {pf[4].x, pf[4].y, pf[4].z, pf[4].w}, {pf[5].x, pf[5].y, pf[5].z, pf[5].w}, \
+                                   {pf[6].x, pf[6].y, pf[6].z, pf[6].w}, {pf[7].x, pf[7].y, pf[7].z, pf[7].w}}; \
+        _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                        \
+          /* dimensions 2 w_ (low halves) and 2 w_ + 1 (high halves) of the eight positions */    \
+          uint4 lo_, hi_;                                                                         \
+          lo_.x = __builtin_amdgcn_perm(r_[1][w_], r_[0][w_], 0x05040100u);                       \
+          lo_.y = __builtin_amdgcn_perm(r_[3][w_], r_[2][w_], 0x05040100u);                       \
+          lo_.z = __builtin_amdgcn_perm(r_[5][w_], r_[4][w_], 0x05040100u);                       \
+          lo_.w = __builtin_amdgcn_perm(r_[7][w_], r_[6][w_], 0x05040100u);                       \
+          hi_.x = __builtin_amdgcn_perm(r_[1][w_], r_[0][w_], 0x07060302u);                       \
+          hi_.y = __builtin_amdgcn_perm(r_[3][w_], r_[2][w_], 0x07060302u);                       \
+          hi_.z = __builtin_amdgcn_perm(r_[5][w_], r_[4][w_], 0x07060302u);                       \
+          hi_.w = __builtin_amdgcn_perm(r_[7][w_], r_[6][w_], 0x07060302u);                       \
+          *(uint4 *)&vt_l[(8u * vdb + 2u * w_) * AM_VROW + 16u * vpg] = lo_;                      \
+          *(uint4 *)&vt_l[(8u * vdb + 2u * w_ + 1u) * AM_VROW + 16u * vpg] = hi_;                 \
+        }                                                                                         \
+      }                                                                                           \
+    } else {                                                                                      \
+      _Pragma("unroll") for (int u = 0; u < NK; u++) {                                            \
+        const uint32_t i_ = kt_ + 128u * u;                                                       \
+        *(uint4 *)&k_l[(i_ / PPR) * KROW + 16u * (i_ % PPR)] = pf[u];                             \
+      }                                                                                           \
+    }                                                                                             \
+  } while (0)
+
+  af16 o[NDB];
+#pragma unroll
+  for (int d = 0; d < NDB; d++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[d][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;   // l_run: this lane half's share of the sum
+
+  AM_LOAD(0u);
+  for (uint32_t it = 0; it < n_tiles; it++) {
+    AM_STORE();
+    __syncthreads();
+    if (it + 1u < n_tiles) AM_LOAD(it + 1u);
+    if (live) {
+      af16 s0, s1;
+#pragma unroll
+      for (int r = 0; r < 16; r++) s0[r] = s1[r] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < NS; s++) {
+        const ah8 a0 = *(const ah8 *)&k_l[l32 * KROW + 32u * s + 16u * lh];
+        const ah8 a1 = *(const ah8 *)&k_l[(l32 + 32u) * KROW + 32u * s + 16u * lh];
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, qh[s], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, qh[s], s1, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, ql[s], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, ql[s], s1, 0, 0, 0);
+      }
+      // register r of block pb: position it * 64 + 32 pb + 8 (r / 4) + 4 lh + r % 4
+      const uint32_t pbase = it * AM_KT + 4u * lh;
+      float mt = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const uint32_t p_ = pbase + 8u * (r >> 2) + (r & 3);
+        s0[r] = p_ <= q_abs ? s0[r] * scale : -INFINITY;
+        s1[r] = p_ + 32u <= q_abs ? s1[r] * scale : -INFINITY;
+        mt = fmaxf(mt, fmaxf(s0[r], s1[r]));
+      }
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float m_new = fmaxf(m_run, mt);   // finite: position 0 is never masked
+      const float alpha = __expf(m_run - m_new);
+      m_run = m_new;
+      float lsum = 0.0f;
+      ah8 ph[4], pl[4];   // k step 2 pb + j: registers 8 j .. 8 j + 7 of block pb
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float p0_ = __expf(s0[r] - m_new), p1_ = __expf(s1[r] - m_new);
+        lsum += p0_ + p1_;
+        _Float16 hi, lo;
+        am_split(p0_, hi, lo);
+        ph[r >> 3][r & 7] = hi;
+        pl[r >> 3][r & 7] = lo;
+        am_split(p1_, hi, lo);
+        ph[2 + (r >> 3)][r & 7] = hi;
+        pl[2 + (r >> 3)][r & 7] = lo;
+      }
+      l_run = l_run * alpha + lsum;
+#pragma unroll
+      for (int d = 0; d < NDB; d++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+#pragma unroll
+        for (int js = 0; js < 4; js++) {
+          const ah8 a = *(const ah8 *)&vt_l[(32u * d + l32) * AM_VROW + 32u * js + 16u * lh];
+          o[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ph[js], o[d], 0, 0, 0);
+          o[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pl[js], o[d], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+#undef AM_LOAD
+#undef AM_STORE
+  if (live && 32u * qt + l32 < n_tokens) {
+    const float l = l_run + __shfl_xor(l_run, 32, 64);
+    float *op = attn_out + ((size_t)tok * n_head + (size_t)kvh * gq + g) * HD + 4u * lh;
+#pragma unroll
+    for (int d = 0; d < NDB; d++)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; r4++)   // registers 4 r4 .. + 3: dimensions 32 d + 8 r4 + 4 lh + 0..3
+        *(float4 *)(op + 32 * d + 8 * r4) = make_float4(o[d][4 * r4] / l, o[d][4 * r4 + 1] / l, o[d][4 * r4 + 2] / l,
+                                                        o[d][4 * r4 + 3] / l);
+  }
+}
+
+hipError_t ogm_launch_attn_prefill_mfma(const float *q, void *k_cache_layer, void *v_cache_layer, uint32_t pos0,
+                                        uint32_t n_tokens, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
+                                        float scale, float *attn_out, hipStream_t stream) {
+  if (n_head_kv == 0 || n_head % n_head_kv != 0 || n_tokens == 0) return hipErrorInvalidValue;
+  const uint32_t gq = n_head / n_head_kv;
+  if (n_head_kv > 65535u || gq > 8u) return hipErrorInvalidValue;
+  const dim3 grid((n_tokens + 31u) / 32u, n_head_kv, (gq + 3u) / 4u);
+  if (head_dim == 128)
+    hipLaunchKernelGGL(ogm_attn_prefill_mfma_kernel<128>, grid, dim3(256), 0, stream, q, (const __half *)k_cache_layer,
+                       (const __half *)v_cache_layer, pos0, n_tokens, n_head_kv, gq, scale, attn_out);
+  else if (head_dim == 64)
+    hipLaunchKernelGGL(ogm_attn_prefill_mfma_kernel<64>, grid, dim3(256), 0, stream, q, (const __half *)k_cache_layer,
+                       (const __half *)v_cache_layer, pos0, n_tokens, n_head_kv, gq, scale, attn_out);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
 // h = silu(gate) * up over n values (all rows of a batch at once)
 __global__ __launch_bounds__(256) void ogm_swiglu_rows_kernel(const float *__restrict__ gate,
                                                               const float *__restrict__ up, size_t n,

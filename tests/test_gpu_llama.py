@@ -470,6 +470,37 @@ def test_prefill_longer_than_one_pass_and_from_token_ids(be):
         dev.close()
 
 
+@pytest.mark.parametrize("hd,group,n_kv,n_tokens,pos0", [(128, 4, 2, 200, 0), (64, 4, 2, 77, 0), (128, 1, 2, 130, 31),
+                                                        (64, 5, 1, 33, 64), (128, 8, 1, 65, 7), (64, 2, 4, 300, 100)])
+def test_prefill_attention_kernels_agree(be, hd, group, n_kv, n_tokens, pos0):
+    """The matrix-core attention of a prefill batch (q and the probabilities as two f16 terms each,
+    running softmax over tiles of 64 positions) against the decode step's kernel run per token
+    (f32 multiply-adds, chunks of 128 merged afterwards): one layer, so that the cache rows do not
+    depend on attention, and outputs that agree to f32 rounding.  Dropping either low-order term
+    would show as 1e-4."""
+    n_head = group * n_kv
+    n_embd = n_head * hd
+    wtype = Q4_K if n_embd % 256 == 0 else Q8_0
+    outs = []
+    for variant in (0, 1):
+        ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=1,
+                              types=(wtype, wtype, wtype, wtype), max_ctx=pos0 + n_tokens, seed=5,
+                              attn_norm_scale=TAME.get(wtype, 1.0))
+        be.set_tuning("attn_prefill_variant", variant)
+        try:
+            if pos0:
+                dev.prefill(rng.standard_normal((pos0, n_embd)).astype(f32), 0)
+            logits, _ = dev.prefill(rng.standard_normal((n_tokens, n_embd)).astype(f32), pos0)
+            outs.append((np.asarray(logits, np.float64), np.asarray(dev.hidden(), np.float64)))
+        finally:
+            be.set_tuning("attn_prefill_variant", 0)
+            dev.close()
+    for name, a, b in (("logits", outs[0][0], outs[1][0]), ("hidden state", outs[0][1], outs[1][1])):
+        err = np.abs(a - b).max() / np.abs(b).max()
+        say(f"attention kernels hd {hd} group {group} {n_tokens} tokens from {pos0}: {name} differ by {err:.2e}")
+        assert err <= 2e-5, f"{name}: the two attention kernels differ by {err:.3e}"
+
+
 def model_gguf(ref, arch, *, n_ctx=4096, tok_embd=None, vec_type=0, omit=(), extra_kvs=(), explicit=True):
     """A reference model as the bytes of a GGUF file with the tensor names and metadata keys
     LlamaModel::load_with_backend and read_model_config read (llama.rs:123-220, loader.rs:1652-1714).

@@ -363,7 +363,8 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     (Q4_K, 300, (520, 70), "ogm_gemm_q4k_kernel"),              # more than 256 tokens, still one round
     (Q4_K, 300, (6000, 3000, 2100), "ogm_gemm_q4k_wide_kernel"),  # 264 tiles of 128 x 128: the wide tiling
     (Q6_K, 40, (300, 130, 64), "ogm_gemm_q6k_kernel"),
-    (Q6_K, 140, (300, 130, 64), "ogm_gemm_q6k_i8_kernel"),
+    (Q6_K, 140, (300, 130, 64), "ogm_gemm_q6k_i8_r64_kernel"),
+    (Q6_K, 300, (6000, 3000, 2100), "ogm_gemm_q6k_i8_kernel"),
     (Q5_K, 130, (520, 70, 129), "ogm_gemm_q5k_kernel"),
     (Q5_K, 130, (520, 70, 129), "ogm_gemm_q5k_i8_kernel"),
     (Q3_K, 40, (128, 300), "ogm_gemm_q3k_kernel"),
@@ -379,7 +380,7 @@ def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, ou
     x = synth_x(n_tokens, in_dim, seed=17)
     xd = DeviceBuffer.from_numpy(x)
     yds = [DeviceBuffer(4 * n_tokens * od) for od in outs]
-    be.set_tuning("gemm_q4k_variant", 0 if kernel.endswith("_i8_kernel") else 2)
+    be.set_tuning("gemm_q4k_variant", 0 if "_i8_" in kernel else 2)
     try:
         be.matmul_multi_dev(hs, xd.ptr, n_tokens, [y.ptr for y in yds])
     finally:
@@ -459,14 +460,14 @@ def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T, variant
 
 @pytest.mark.parametrize("in_dim,out_dim,T", [
     (256, 5, 9), (512, 130, 17), (768, 64, 129), (1024, 100, 64), (1280, 257, 40), (2048, 37, 128),
-    (4096, 200, 130), (14336, 96, 257), (4096, 1000, 512), (1792, 33, 10),
+    (4096, 200, 130), (14336, 96, 257), (4096, 1000, 512), (1792, 33, 10), (512, 4200, 513),
 ])
-@pytest.mark.parametrize("variant", [0, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2])
 def test_mfma_gemm_q6k_matches_cpu_gemm(be, in_dim, out_dim, T, variant):
     """Q6_K at n_tokens >= 9 takes an MFMA kernel; values must equal gemm_k_q6_k (vecdot.rs:2352-2398).
     The int8 kernel (default) folds each scale into its weights and splits the 13-bit products into
-    two int8 planes; the f16 kernel (variant 2) splits the scale as 16a + b; both keep every
-    integer exact."""
+    two int8 planes, on 128-row tiles or, when those are few, 64-row tiles (variant 1: always); the
+    f16 kernel (variant 2) splits the scale as 16a + b; all keep every integer exact."""
     raw = synth_weights(Q6_K, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T + 1)
     w = qm(raw, Q6_K, in_dim, out_dim)
@@ -476,7 +477,9 @@ def test_mfma_gemm_q6k_matches_cpu_gemm(be, in_dim, out_dim, T, variant):
         got = be.matmul(x, T, w)
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
-    assert be.last_kernel() == ("ogm_gemm_q6k_i8_kernel" if variant == 0 else "ogm_gemm_q6k_kernel")
+    small_grid = ((T + 127) // 128) * ((out_dim + 63) // 64) <= 256
+    assert be.last_kernel() == ("ogm_gemm_q6k_kernel" if variant == 2 else "ogm_gemm_q6k_i8_r64_kernel"
+                                if variant == 1 or small_grid else "ogm_gemm_q6k_i8_kernel")
     want = oracle.matmul(Q6_K, raw, in_dim, out_dim, x, T)
     assert_close(got, want, "mfma gemm q6k")
     assert_bits(got, want, "mfma gemm q6k")
@@ -491,13 +494,15 @@ def test_mfma_gemm_q6k_matches_cpu_gemm(be, in_dim, out_dim, T, variant):
 
 @pytest.mark.parametrize("ql,qh,sc,sign", [(0xFF, 0xFF, 0x7F, "alt"), (0x00, 0x00, 0x80, "pos"), (0xFF, 0xFF, 0x80, "neg"),
                                            (0x00, 0x00, 0x7F, "alt"), (0xF0, 0x0F, 0x8F, "block"), (0x0F, 0xF0, 0x70, "pos")])
-@pytest.mark.parametrize("variant", [0, 2])
+@pytest.mark.parametrize("variant", [0, 3, 2])
 def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign, variant):
     """Extreme 6-bit values (0 -> -32, 63 -> +31), scales -128 / +127 / -113 / +112 and activations
     +-127: |isum| reaches 1.3e8, far past 2^24.  In the f16 kernel the high and low scale digits'
     chains reach their bounds, and 16 * c_hi + c_lo must round exactly like `isum as f32`; in the int8
-    kernel -128 * -32 = 4096 is the one product whose high plane is +64, and 64 H + L stays in 32 bits."""
-    in_dim, out_dim, T = 1024, 32, 16
+    kernels (64-row tiles on this small grid; variant 3 here: 128-row tiles, by way of 300 tokens x 6000
+    rows) -128 * -32 = 4096 is the product with the largest high plane, +16, and 256 H + L stays in
+    32 bits."""
+    in_dim, out_dim, T = (1024, 6000, 300) if variant == 3 else (1024, 32, 16)
     blocks = np.zeros((out_dim * 4, 210), np.uint8)
     blocks[:, 0:128] = ql
     blocks[:, 128:192] = qh
@@ -513,12 +518,12 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign, variant)
         x[:, 128:256] *= -1
         x[3] = -127.0
     raw = blocks.reshape(-1)
-    be.set_tuning("gemm_q4k_variant", variant)
+    be.set_tuning("gemm_q4k_variant", variant % 3)
     try:
         got = be.matmul(x, T, qm(raw, Q6_K, in_dim, out_dim))
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
-    assert be.last_kernel() == ("ogm_gemm_q6k_i8_kernel" if variant == 0 else "ogm_gemm_q6k_kernel")
+    assert be.last_kernel() == {0: "ogm_gemm_q6k_i8_r64_kernel", 3: "ogm_gemm_q6k_i8_kernel", 2: "ogm_gemm_q6k_kernel"}[variant]
     want = oracle.matmul(Q6_K, raw, in_dim, out_dim, x, T)
     assert_bits(got, want, "extreme ranges")
     isum, _ = be.dump_block_sums(x[0], 1, qm(raw, Q6_K, in_dim, out_dim))
