@@ -761,9 +761,12 @@ struct GemmI8pParams {
   uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
 };
 
-// ROWS = 128: eight multiplying waves (64 rows x 32 tokens each) and four feeding ones; ROWS = 64:
-// four and two, half the LDS, and two workgroups to a CU, which fills the chip when a launch has
-// few row tiles and lets one workgroup's LDS traffic run under the other's matrix instructions.
+// ROWS = 128: eight multiplying waves (64 rows x 32 tokens each) and eight feeding ones; ROWS = 64:
+// four and four, and half the LDS: twice as many workgroups, which fills the chip when a launch has
+// few row tiles.  As many feeding as multiplying waves, because a stage's unpacking, behind the
+// latency of its loads, takes a feeding wave about as long as eight matrix instructions and their
+// operand reads take a multiplying one (with half as many feeding waves the multiplying ones sat
+// idle for more than half of every stage).
 template <uint32_t ROWS>
 __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   constexpr uint32_t NC = ROWS / 16u;                // multiplying waves
@@ -802,61 +805,45 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   auto sb_lane = [&](uint32_t s) -> uint32_t { return (s & ((1u << p.c_shift) - 1u)) << p.r_shift; };
 
   if (producer) {
-    // Feeding thread pt stages two groups of 16 weights per stage, a and b: one ql piece, one qh
-    // piece, one scale each.  A wave has one group index and 64 consecutive rows: its loads are
-    // 1 KiB runs and its LDS rows are 80 bytes apart, which spreads over all banks.  ROWS = 128:
-    // rows pt % 64 and pt % 64 + 64, group pt / 64; ROWS = 64: row pt % 64, groups pt / 64 and
-    // pt / 64 + 2, which share the qh piece and the scales.  And the activations: 32 bytes of a
-    // token (64 with half as many feeding threads).  Once per super-block the rows' d and the
+    // Feeding thread pt stages one group of 16 weights per stage: one ql piece, one qh piece, one
+    // scale.  A wave has one group index and 64 consecutive rows: its loads are 1 KiB runs and its
+    // LDS rows are 80 bytes apart, which spreads over all banks.  And 16 bytes of a token's
+    // activations (32 with half as many feeding threads).  Once per super-block the rows' d and the
     // tokens' ad.
     const uint32_t pt = tid - 64u * NC;
-    const uint32_t t16a = __builtin_amdgcn_readfirstlane(pt >> 6), prw = pt & 63u;
-    const uint32_t t16b = ROWS == 128u ? t16a : t16a + 2u, prwb = ROWS == 128u ? prw + 64u : prw;
-    uint32_t uo[2];
-#pragma unroll
-    for (int k = 0; k < 2; k++) {
-      const uint32_t row = min(r0 + (k ? prwb : prw), p.out_dim - 1u);   // rows past the matrix: clamped, never stored
-      const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
-      uo[k] = rb * p.nct * TILE_BYTES + r * 16u;
-    }
-    constexpr uint32_t XB = ROWS == 128u ? 32u : 64u;   // bytes of a token's stage per feeding thread
-    const uint32_t xrow_ = ROWS == 128u ? pt >> 1 : pt, xhalf = ROWS == 128u ? pt & 1u : 0u;
-    const uint32_t xro = min(t0 + xrow_, p.n_tokens - 1u) * p.in_dim + XB * xhalf;   // + 256 s + 64 g
-    const bool has_d = pt < ROWS, has_ad = ROWS == 128u ? pt >= 128u : true;
-    const uint32_t ad_tok = ROWS == 128u ? pt - 128u : pt;
-    uint32_t dto;   // the row whose d this thread fetches
+    const uint32_t t16 = __builtin_amdgcn_readfirstlane(pt / ROWS), prw = pt % ROWS;
+    uint32_t uo, dto;   // the row's 16-byte pieces and its two-byte tail (d)
     {
-      const uint32_t row = min(r0 + (pt & (ROWS - 1u)), p.out_dim - 1u);
-      dto = (row >> p.r_shift) * p.nct * TILE_BYTES + 13u * 1024u + (row & ((1u << p.r_shift) - 1u)) * 2u;
+      const uint32_t row = min(r0 + prw, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+      const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+      uo = rb * p.nct * TILE_BYTES + r * 16u;
+      dto = rb * p.nct * TILE_BYTES + 13u * 1024u + r * 2u;
     }
+    constexpr uint32_t XB = ROWS == 128u ? 16u : 32u;   // bytes of a token's stage per feeding thread
+    const uint32_t xrow_ = pt / (64u / XB), xpart = pt % (64u / XB);
+    const uint32_t xro = min(t0 + xrow_, p.n_tokens - 1u) * p.in_dim + XB * xpart;   // + 256 s + 64 g
+    const bool has_d = pt < ROWS, has_ad = pt >= ROWS && pt < ROWS + 128u;
+    const uint32_t ad_tok = pt - ROWS;
     const uint32_t aro = min(t0 + (ad_tok & 127u), p.n_tokens - 1u) * p.nsb;
     // the ring of stages in flight, slot = stage % 4 = g, in named registers
-    uint4 qla0, qla1, qla2, qla3, qha0, qha1, qha2, qha3, qlb0, qlb1, qlb2, qlb3, qhb0, qhb1, qhb2, qhb3;
-    uint4 xa0_, xa1_, xa2_, xa3_, xb0_, xb1_, xb2_, xb3_;
-    uint4 xc0_, xc1_, xc2_, xc3_, xd0_, xd1_, xd2_, xd3_;   // ROWS = 64: the token's other 32 bytes
-    uint4 scxa = make_uint4(0, 0, 0, 0), scxb = make_uint4(0, 0, 0, 0);   // the 16 scales of the two rows, next super-block
-    uint32_t sca[4] = {0, 0, 0, 0}, scb[4] = {0, 0, 0, 0};                // ... of the super-block being stored
+    uint4 qla0, qla1, qla2, qla3, qha0, qha1, qha2, qha3;
+    uint4 xa0_, xa1_, xa2_, xa3_;
+    uint4 xb0_, xb1_, xb2_, xb3_;   // ROWS = 64: the thread's other 16 bytes
+    uint4 scxa = make_uint4(0, 0, 0, 0);      // the 16 scales of the row, next super-block
+    uint32_t sca[4] = {0, 0, 0, 0};           // ... of the super-block being stored
     uint32_t d16 = 0;
     float adn = 0.0f;
 #define GP_LOAD(S, G, K)                                                                          \
   do {                                                                                            \
     const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded again, never used */ \
     const uint32_t so_ = sb_tile(s_) + sb_lane(s_) * 16u, h_ = (G) >> 1;                          \
-    qla##K = *(const uint4 *)(p.wt + (uo[0] + so_ + (4u * h_ + t16a) * 1024u));                   \
-    qha##K = *(const uint4 *)(p.wt + (uo[0] + so_ + (8u + 2u * h_ + (t16a & 1u)) * 1024u));       \
-    qlb##K = *(const uint4 *)(p.wt + (uo[1] + so_ + (4u * h_ + t16b) * 1024u));                   \
-    if constexpr (ROWS == 128u)                                                                   \
-      qhb##K = *(const uint4 *)(p.wt + (uo[1] + so_ + (8u + 2u * h_ + (t16b & 1u)) * 1024u));     \
+    qla##K = *(const uint4 *)(p.wt + (uo + so_ + (4u * h_ + t16) * 1024u));                       \
+    qha##K = *(const uint4 *)(p.wt + (uo + so_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));           \
     const uint4 *xp_ = (const uint4 *)(p.xq + (xro + 256u * s_ + 64u * (G)));                     \
     xa##K##_ = xp_[0];                                                                            \
-    xb##K##_ = xp_[1];                                                                            \
-    if constexpr (ROWS == 64u) {                                                                  \
-      xc##K##_ = xp_[2];                                                                          \
-      xd##K##_ = xp_[3];                                                                          \
-    }                                                                                             \
+    if constexpr (ROWS == 64u) xb##K##_ = xp_[1];                                                 \
     if ((G) == 0u) {                                                                              \
-      scxa = *(const uint4 *)(p.wt + (uo[0] + so_ + 12u * 1024u));                                \
-      if constexpr (ROWS == 128u) scxb = *(const uint4 *)(p.wt + (uo[1] + so_ + 12u * 1024u));    \
+      scxa = *(const uint4 *)(p.wt + (uo + so_ + 12u * 1024u));                                   \
       if (has_d) d16 = *(const uint16_t *)(p.wt + (dto + sb_tile(s_) + sb_lane(s_) * 2u));        \
       if (has_ad) adn = p.ad[aro + s_];                                                           \
     }                                                                                             \
@@ -890,22 +877,13 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   do {                                                                                            \
     if ((G) == 0u) {                                                                              \
       sca[0] = scxa.x; sca[1] = scxa.y; sca[2] = scxa.z; sca[3] = scxa.w;                         \
-      if constexpr (ROWS == 128u) {                                                               \
-        scb[0] = scxb.x; scb[1] = scxb.y; scb[2] = scxb.z; scb[3] = scxb.w;                       \
-      }                                                                                           \
       if (has_d) d_l[ROWS * ((S) & 1u) + pt] = gm_f16_bits_to_f32(d16);                           \
       if (has_ad) ad_l[128u * ((S) & 1u) + ad_tok] = adn;                                         \
     }                                                                                             \
-    GP_GROUP(qla##K, qha##K, sca, G, pw, prw, t16a);                                              \
-    if constexpr (ROWS == 128u) GP_GROUP(qlb##K, qhb##K, scb, G, pw, prwb, t16b);                 \
-    else GP_GROUP(qlb##K, qha##K, sca, G, pw, prwb, t16b);                                        \
-    uint8_t *xr_ = &x_l[px + xrow_ * GI_ROW + XB * xhalf];                                        \
+    GP_GROUP(qla##K, qha##K, sca, G, pw, prw, t16);                                               \
+    uint8_t *xr_ = &x_l[px + xrow_ * GI_ROW + XB * xpart];                                        \
     *(uint4 *)xr_ = xa##K##_;                                                                     \
-    *(uint4 *)(xr_ + 16u) = xb##K##_;                                                             \
-    if constexpr (ROWS == 64u) {                                                                  \
-      *(uint4 *)(xr_ + 32u) = xc##K##_;                                                           \
-      *(uint4 *)(xr_ + 48u) = xd##K##_;                                                           \
-    }                                                                                             \
+    if constexpr (ROWS == 64u) *(uint4 *)(xr_ + 16u) = xb##K##_;                                  \
     /* stages go round the three buffers */                                                       \
     pw = pw == 2u * WT ? 0u : pw + WT;                                                            \
     px = px == 2u * GI_WTILE ? 0u : px + GI_WTILE;                                                \
@@ -1015,8 +993,8 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   }
 }
 
-__global__ __launch_bounds__(768) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u>(p); }
-__global__ __launch_bounds__(384) void ogm_gemm_q6k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q6k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u>(p); }
 
 // ------------------------------------------------------------------------------------------
 // Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
@@ -2119,10 +2097,10 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
     if (r64) {
-      hipLaunchKernelGGL(ogm_gemm_q6k_i8_r64_kernel, pgrid, dim3(384), lds_bytes, stream, p);
+      hipLaunchKernelGGL(ogm_gemm_q6k_i8_r64_kernel, pgrid, dim3(512), lds_bytes, stream, p);
       if (kernel_name) *kernel_name = "ogm_gemm_q6k_i8_r64_kernel";
     } else {
-      hipLaunchKernelGGL(ogm_gemm_q6k_i8_kernel, pgrid, dim3(768), lds_bytes, stream, p);
+      hipLaunchKernelGGL(ogm_gemm_q6k_i8_kernel, pgrid, dim3(1024), lds_bytes, stream, p);
       if (kernel_name) *kernel_name = "ogm_gemm_q6k_i8_kernel";
     }
     return hipGetLastError();
