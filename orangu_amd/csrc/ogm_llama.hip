@@ -1080,18 +1080,36 @@ __global__ __launch_bounds__(256) void ogm_attn_prefill_mfma_kernel(const float 
   const uint32_t n_tiles = last_pos / AM_KT + 1u;
   const uint32_t max_row = pos0 + n_tokens - 1u;   // last cache row that holds data
 
-  // q of this lane's query, head g: for k step s the dimensions 16 s + 8 lh + 0..7, as hi + lo
+  // q of this lane's query, head g: for k step s the dimensions 16 s + 8 lh + 0..7, as hi + lo.  A
+  // row whose largest |q| is 2^14 or more is first scaled down by a power of two (the f16 terms
+  // would overflow at 65504) and its scores scaled back up with `scale`: exact both ways.
   ah8 qh[NS], ql[NS];
+  float scale_q = scale;
   {
     const float *qp = q + ((size_t)tok * n_head + (size_t)kvh * gq + (live ? g : 0u)) * HD + 8u * lh;
+    float4 qa[NS], qb[NS];
+    float amax = 0.0f;
 #pragma unroll
     for (int s = 0; s < NS; s++) {
-      const float4 a = *(const float4 *)(qp + 16 * s), b = *(const float4 *)(qp + 16 * s + 4);
-      const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      qa[s] = *(const float4 *)(qp + 16 * s);
+      qb[s] = *(const float4 *)(qp + 16 * s + 4);
+      amax = fmaxf(amax, fmaxf(fmaxf(fabsf(qa[s].x), fabsf(qa[s].y)), fmaxf(fabsf(qa[s].z), fabsf(qa[s].w))));
+      amax = fmaxf(amax, fmaxf(fmaxf(fabsf(qb[s].x), fabsf(qb[s].y)), fmaxf(fabsf(qb[s].z), fabsf(qb[s].w))));
+    }
+    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));   // the row's other dimensions are in the other lane half
+    float down = 1.0f;
+    if (amax >= 16384.0f && amax < INFINITY) {
+      const int k = (int)((__float_as_uint(amax) >> 23) & 0xFFu) - 127 - 13;   // amax * 2^-k in [2^13, 2^14)
+      down = __uint_as_float((uint32_t)(127 - k) << 23);
+      scale_q = scale * __uint_as_float((uint32_t)(127 + k) << 23);
+    }
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+      const float v[8] = {qa[s].x, qa[s].y, qa[s].z, qa[s].w, qb[s].x, qb[s].y, qb[s].z, qb[s].w};
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         _Float16 hi, lo;
-        am_split(v[e], hi, lo);
+        am_split(v[e] * down, hi, lo);
         qh[s][e] = hi;
         ql[s][e] = lo;
       }
@@ -1186,8 +1204,8 @@ __global__ __launch_bounds__(256) void ogm_attn_prefill_mfma_kernel(const float 
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const uint32_t p_ = pbase + 8u * (r >> 2) + (r & 3);
-        s0[r] = p_ <= q_abs ? s0[r] * scale : -INFINITY;
-        s1[r] = p_ + 32u <= q_abs ? s1[r] * scale : -INFINITY;
+        s0[r] = p_ <= q_abs ? s0[r] * scale_q : -INFINITY;
+        s1[r] = p_ + 32u <= q_abs ? s1[r] * scale_q : -INFINITY;
         mt = fmaxf(mt, fmaxf(s0[r], s1[r]));
       }
       mt = fmaxf(mt, __shfl_xor(mt, 32, 64));

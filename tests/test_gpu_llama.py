@@ -65,7 +65,7 @@ PRE_SIZES = {"q_bias": lambda nh, nkv, hd: nh * hd, "k_bias": lambda nh, nkv, hd
 
 
 def build(be, *, n_embd, n_head, n_kv, hd, n_ff, n_vocab, n_layer, types, max_ctx, seed, rope_dim=None,
-          base=10000.0, pre=(), neox=False, freq_factors=None, attn_norm_scale=1.0):
+          base=10000.0, pre=(), neox=False, freq_factors=None, attn_norm_scale=1.0, pre_scale=None):
     from orangu_amd import LlamaDecoder, QuantMatrix
     rng = np.random.default_rng(seed)
     tq, tv, tdown, tout = types
@@ -84,7 +84,7 @@ def build(be, *, n_embd, n_head, n_kv, hd, n_ff, n_vocab, n_layer, types, max_ct
             # a bias of the size the synthetic weights of that type give the projection itself
             mag = {Q8_0: 0.2, Q4_K: 30.0, Q6_K: 200.0}.get(tv if name == "v_bias" else tq, 1.0)
             vec = (1 + 0.2 * rng.standard_normal(n)) if name.endswith("norm") else mag * rng.standard_normal(n)
-            setattr(layers[-1], name, vec.astype(f32))
+            setattr(layers[-1], name, (vec * (pre_scale or {}).get(name, 1.0)).astype(f32))
     out_norm = (1 + 0.1 * rng.standard_normal(n_embd)).astype(f32)
     output = mk(tout, n_embd, n_vocab, seed * 1000 + 999)
     ref = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd if rope_dim is None else rope_dim, 1e-5, base,
@@ -499,6 +499,33 @@ def test_prefill_attention_kernels_agree(be, hd, group, n_kv, n_tokens, pos0):
         err = np.abs(a - b).max() / np.abs(b).max()
         say(f"attention kernels hd {hd} group {group} {n_tokens} tokens from {pos0}: {name} differ by {err:.2e}")
         assert err <= 2e-5, f"{name}: the two attention kernels differ by {err:.3e}"
+
+
+@pytest.mark.parametrize("hd", [128, 64])
+def test_prefill_attention_with_queries_beyond_f16(be, hd):
+    """Per-head norms that leave q at magnitudes up to 1.5e5 (an f16 holds 65504) and k around 1e-3:
+    the matrix-core kernel scales such a query row by a power of two before it splits it into f16
+    terms and scales the scores back, exactly; the per-token f32 kernel needs nothing of the kind.
+    They must still agree (and be finite)."""
+    n_head, n_kv = 4, 2
+    n_embd = n_head * hd
+    wtype = Q4_K if n_embd % 256 == 0 else Q8_0
+    outs = []
+    for variant in (0, 1):
+        ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=1,
+                              types=(wtype, wtype, wtype, wtype), max_ctx=150, seed=9, pre=("q_norm", "k_norm"),
+                              pre_scale={"q_norm": 4e4, "k_norm": 1e-3}, attn_norm_scale=TAME.get(wtype, 1.0))
+        be.set_tuning("attn_prefill_variant", variant)
+        try:
+            logits, _ = dev.prefill(rng.standard_normal((150, n_embd)).astype(f32), 0)
+            outs.append(np.asarray(dev.hidden(), np.float64))
+        finally:
+            be.set_tuning("attn_prefill_variant", 0)
+            dev.close()
+    assert np.isfinite(outs[0]).all() and np.isfinite(outs[1]).all()
+    err = np.abs(outs[0] - outs[1]).max() / np.abs(outs[1]).max()
+    say(f"large q, hd {hd}: hidden states of the two attention kernels differ by {err:.2e}")
+    assert err <= 2e-5
 
 
 def model_gguf(ref, arch, *, n_ctx=4096, tok_embd=None, vec_type=0, omit=(), extra_kvs=(), explicit=True):
