@@ -780,8 +780,8 @@ struct ogm_llama {
   // prefill rows, allocated at the first prefill for OGM_PREFILL_CHUNK tokens
   struct Prefill {
     float *x = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
-    float *proj = nullptr, *gate = nullptr, *up = nullptr, *h = nullptr, *cs = nullptr;
-    float *part_o = nullptr, *part_ml = nullptr;
+    float *proj = nullptr, *gate = nullptr, *up = nullptr, *cs = nullptr;
+    float *part_o = nullptr, *part_ml = nullptr;   // attn_prefill_variant 1 only, allocated when it first runs
     uint32_t *tokens = nullptr;
     uint32_t attn_tokens = 0;   // query rows one attention launch takes (bounded by part_o)
     bool ready = false;
@@ -1148,11 +1148,6 @@ static int llama_prefill_buffers(ogm_ctx *ctx, ogm_llama *m) {
   if (m->pf.ready) return OGM_OK;
   const ogm_llama_config &c = m->cfg;
   const size_t T = OGM_PREFILL_CHUNK, qd = (size_t)c.n_head * c.head_dim, kvd = (size_t)c.n_head_kv * c.head_dim;
-  // query rows per attention launch: as many as keep the partial results within their budget
-  const size_t per_token = (size_t)c.n_head * m->max_splits * c.head_dim * 4;
-  size_t at = OGM_PREFILL_PART_BYTES / per_token;
-  if (at < 1) at = 1;
-  if (at > T) at = T;
   int rc = OGM_OK;
   auto A = [&](float **p, size_t n) { if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)p, n * 4); };
   A(&m->pf.x, T * c.n_embd);
@@ -1164,14 +1159,26 @@ static int llama_prefill_buffers(ogm_ctx *ctx, ogm_llama *m) {
   A(&m->pf.proj, T * c.n_embd);
   A(&m->pf.gate, T * c.n_ff);
   A(&m->pf.up, T * c.n_ff);
-  A(&m->pf.h, T * c.n_ff);
   A(&m->pf.cs, T * (c.rope_dim / 2 + 1) * 2);
-  A(&m->pf.part_o, at * per_token / 4);
-  A(&m->pf.part_ml, at * (size_t)c.n_head * m->max_splits * 2);
   A((float **)&m->pf.tokens, T);
   if (rc != OGM_OK) return rc;
-  m->pf.attn_tokens = (uint32_t)at;
   m->pf.ready = true;
+  return OGM_OK;
+}
+
+// The per-token attention kernel's partial results (attn_prefill_variant 1): query rows per launch
+// as many as keep them within OGM_PREFILL_PART_BYTES.
+static int llama_prefill_partials(ogm_ctx *ctx, ogm_llama *m) {
+  if (m->pf.part_o) return OGM_OK;
+  const ogm_llama_config &c = m->cfg;
+  const size_t per_token = (size_t)c.n_head * m->max_splits * c.head_dim * 4;
+  size_t at = OGM_PREFILL_PART_BYTES / per_token;
+  if (at < 1) at = 1;
+  if (at > OGM_PREFILL_CHUNK) at = OGM_PREFILL_CHUNK;
+  int rc = llama_alloc(ctx, m, (void **)&m->pf.part_o, at * per_token);
+  if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)&m->pf.part_ml, at * (size_t)c.n_head * m->max_splits * 2 * 4);
+  if (rc != OGM_OK) return rc;
+  m->pf.attn_tokens = (uint32_t)at;
   return OGM_OK;
 }
 
@@ -1193,6 +1200,48 @@ static int llama_matmul_rows(ogm_ctx *ctx, const ogm_weight *const *ws, float *c
   return OGM_OK;
 }
 
+// Matmuls of a batch over activations a producer kernel has already quantized into the context's
+// scratch (mode `mode`, `in_dim` wide, T rows): the weights are grouped by type as in
+// llama_matmul_rows; all of them must take that mode.
+static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n,
+                                       int mode, uint32_t in_dim, uint32_t T, hipStream_t s) {
+  ctx->act_mode = mode;
+  ctx->act_in_dim = in_dim;
+  ctx->act_tokens = T;
+  size_t i = 0;
+  while (i < n) {
+    Target tg[OGM_GEMV_MAX_MATS];
+    size_t e = i;
+    while (e < n && e - i < OGM_GEMV_MAX_MATS && ws[e]->ggml_type == ws[i]->ggml_type) {
+      tg[e - i] = Target{ws[e], ys[e]};
+      e++;
+    }
+    int rc = enqueue_gemv(ctx, tg, e - i, T, 0, s, nullptr, nullptr, nullptr);
+    if (rc != OGM_OK) return rc;
+    i = e;
+  }
+  return OGM_OK;
+}
+
+// x += delta, RMSNorm, and the matmuls over the normed rows.  When every weight takes the same
+// activation format the norm kernel quantizes its own output (the decode step's kernel, one
+// workgroup per row) and the f32 rows are never stored; otherwise they are, and each group of
+// weights quantizes them for itself.
+static int llama_norm_matmul_rows(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *const *ws, float *const *ys, size_t n,
+                                  const float *delta, const float *norm_w, uint32_t T, hipStream_t s) {
+  const ogm_llama_config &c = m->cfg;
+  ogm_llama::Prefill &P = m->pf;
+  const int mode = act_mode_for(ws[0]->ggml_type);
+  bool same = true;
+  for (size_t i = 1; i < n; i++) same = same && act_mode_for(ws[i]->ggml_type) == mode;
+  int rc = ensure_act(ctx, c.n_embd, T);
+  if (rc != OGM_OK) return rc;
+  HIPCHK(ctx, ogm_launch_norm_quant(mode, P.x, delta, norm_w, c.n_embd, c.rms_eps, same ? nullptr : P.normed,
+                                    act_view(ctx, c.n_embd, mode, 0), s, T));
+  if (same) return llama_matmul_quantized_rows(ctx, ws, ys, n, mode, c.n_embd, T, s);
+  return llama_matmul_rows(ctx, ws, ys, n, P.normed, T, s);
+}
+
 // One chunk of T <= OGM_PREFILL_CHUNK tokens whose embedding rows sit in m->pf.x.  With `last`,
 // the final row's hidden state ends in m->x and its logits in m->logits.
 static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32_t T, bool last, hipStream_t s) {
@@ -1207,10 +1256,9 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     const float *attn_norm = m->norms + (size_t)l * 2 * c.n_embd, *ffn_norm = attn_norm + c.n_embd;
     void *kc = (uint8_t *)m->k_cache + (size_t)l * c.max_ctx * kvd * 2;
     void *vc = (uint8_t *)m->v_cache + (size_t)l * c.max_ctx * kvd * 2;
-    HIPCHK(ctx, ogm_launch_norm_rows(P.x, delta, attn_norm, c.n_embd, T, c.rms_eps, P.normed, s));
     const ogm_weight *w3[3] = {L.wq, L.wk, L.wv};
     float *y3[3] = {P.q, P.k, P.v};
-    int rc = llama_matmul_rows(ctx, w3, y3, 3, P.normed, T, s);
+    int rc = llama_norm_matmul_rows(ctx, m, w3, y3, 3, delta, attn_norm, T, s);
     if (rc != OGM_OK) return rc;
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_qkv_pre(P.q, P.k, P.v, P.cs, c.rope_dim, pre, c.n_head, c.n_head_kv, c.head_dim, kc, vc,
@@ -1218,6 +1266,7 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     if (ctx->tune_attn_prefill_variant == 0) {
       HIPCHK(ctx, ogm_launch_attn_prefill_mfma(P.q, kc, vc, pos0, T, c.n_head, c.n_head_kv, c.head_dim, scale, P.attn, s));
     }
+    if (ctx->tune_attn_prefill_variant != 0 && (rc = llama_prefill_partials(ctx, m)) != OGM_OK) return rc;
     for (uint32_t t0 = 0; ctx->tune_attn_prefill_variant != 0 && t0 < T; t0 += P.attn_tokens) {
       const uint32_t nt = T - t0 < P.attn_tokens ? T - t0 : P.attn_tokens;
       HIPCHK(ctx, ogm_launch_attn_prefill(P.q + (size_t)t0 * qd, kc, vc, pos0 + t0, nt, m->max_splits, c.n_head,
@@ -1227,13 +1276,15 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     const ogm_weight *w1[1] = {L.wo};
     float *y1[1] = {P.proj};
     if ((rc = llama_matmul_rows(ctx, w1, y1, 1, P.attn, T, s)) != OGM_OK) return rc;
-    HIPCHK(ctx, ogm_launch_norm_rows(P.x, P.proj, ffn_norm, c.n_embd, T, c.rms_eps, P.normed, s));
     const ogm_weight *w2[2] = {L.w_gate, L.w_up};
     float *y2[2] = {P.gate, P.up};
-    if ((rc = llama_matmul_rows(ctx, w2, y2, 2, P.normed, T, s)) != OGM_OK) return rc;
-    HIPCHK(ctx, ogm_launch_swiglu_rows(P.gate, P.up, (size_t)T * c.n_ff, P.h, s));
+    if ((rc = llama_norm_matmul_rows(ctx, m, w2, y2, 2, P.proj, ffn_norm, T, s)) != OGM_OK) return rc;
+    // SwiGLU quantizes its own output for the down projection: h is never stored as f32
     const ogm_weight *wd[1] = {L.w_down};
-    if ((rc = llama_matmul_rows(ctx, wd, y1, 1, P.h, T, s)) != OGM_OK) return rc;
+    const int mode_d = act_mode_for(L.w_down->ggml_type);
+    if ((rc = ensure_act(ctx, c.n_ff, T)) != OGM_OK) return rc;
+    HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, P.gate, P.up, c.n_ff, nullptr, act_view(ctx, c.n_ff, mode_d, 0), s, T));
+    if ((rc = llama_matmul_quantized_rows(ctx, wd, y1, 1, mode_d, c.n_ff, T, s)) != OGM_OK) return rc;
     delta = P.proj;
   }
   ctx->act_mode = -1;   // the activation scratch was the matmuls'

@@ -2026,8 +2026,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
                     wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
   const bool i8p = a.ggml_type == OGM_Q6_K && a.q4k_variant != 2u;   // needs nothing prepared
   const bool raw_x = wide || i8 || i8p;   // these read the int8 activations as they are: only (bh, bl) to prepare
-  hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((raw_x ? n_sb : n8) + 255) / 256)), dim3(256), 0,
-                     stream, a.act.q, a.act.bsum, raw_x ? (_Float16 *)nullptr : xh, bs16, n8, n_sb);
+  if (!i8p)
+    hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((raw_x ? n_sb : n8) + 255) / 256)), dim3(256), 0,
+                       stream, a.act.q, a.act.bsum, raw_x ? (_Float16 *)nullptr : xh, bs16, n8, n_sb);
   const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
   const uint32_t c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
   // token tiles vary fastest: workgroups that run together share weight rows, and with a

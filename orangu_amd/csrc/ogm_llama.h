@@ -12,9 +12,10 @@
 // x += delta (when delta is given; x is updated in place), then
 // normed = x * (1 / sqrt(mean(x^2) + eps)) * weight        (tensor.rs:732-757)
 // quantized for the next matmul in `mode` (0: per 32, 1: per 256) into `act`; `normed` (f32) is
-// also stored when not null.  n <= 16384, n % 32 == 0.
+// also stored when not null.  n <= 16384, n % 32 == 0.  With n_rows > 1: that many rows of x, delta,
+// normed and act, one workgroup each.
 hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const float *weight, uint32_t n,
-                                 float eps, float *normed, OgmActDev act, hipStream_t stream);
+                                 float eps, float *normed, OgmActDev act, hipStream_t stream, uint32_t n_rows = 1);
 
 // cos / sin of pos * freq[p] for the rope_dim / 2 rotated pairs, as float2 (cos, sin): once per
 // token, every layer rotates by the same angles (tensor.rs:1147-1160, freq_scale 1, no YaRN;
@@ -53,9 +54,10 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
                                   hipStream_t stream);
 
 // h = silu(gate) * up with silu(g) = g / (1 + exp(-g))     (tensor.rs:825-827, arch/mod.rs:1071-1106)
-// quantized for the down projection in `mode`; h (f32) is also stored when not null.
+// quantized for the down projection in `mode`; h (f32) is also stored when not null.  With
+// n_rows > 1: that many rows of n values each.
 hipError_t ogm_launch_swiglu_quant(int mode, const float *gate, const float *up, uint32_t n, float *h,
-                                   OgmActDev act, hipStream_t stream);
+                                   OgmActDev act, hipStream_t stream, uint32_t n_rows = 1);
 
 // Index of the largest logit; of several equal ones the last (sampling.rs:336-343).  `scratch`
 // holds 2 * 256 words.
@@ -73,11 +75,8 @@ hipError_t ogm_launch_dequant_row(const uint8_t *wt, uint32_t ggml_type, uint32_
                                   hipStream_t stream);
 
 // ---- the same layer over a batch of tokens (prefill, llama.rs:594-932 at n_tokens > 1) ----------
-// The matmuls between these are GEMMs that quantize their own input: plain f32 rows throughout.
-
-// Rows of n values: x += delta (when given, in place), normed = RMSNorm(x) * weight.  n % 4 == 0.
-hipError_t ogm_launch_norm_rows(float *x, const float *delta, const float *weight, uint32_t n, uint32_t n_rows,
-                                float eps, float *normed, hipStream_t stream);
+// The norm and the SwiGLU are the decode step's kernels over n_rows rows (they quantize their own
+// output for the GEMMs that follow); the rest works on plain f32 rows.
 
 // q [n_tokens][n_head*head_dim] in place, k and v [n_tokens][n_head_kv*head_dim] into the cache
 // rows pos0 .. pos0 + n_tokens as f16: bias, per-head norm, RoPE (row t of `cs`) as in
@@ -101,5 +100,3 @@ hipError_t ogm_launch_attn_prefill_mfma(const float *q, void *k_cache_layer, voi
                                         uint32_t n_tokens, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
                                         float scale, float *attn_out, hipStream_t stream);
 
-// h = silu(gate) * up over n values.  n % 4 == 0.
-hipError_t ogm_launch_swiglu_rows(const float *gate, const float *up, size_t n, float *h, hipStream_t stream);

@@ -27,6 +27,16 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
                                                               OgmActDev act) {
   __shared__ float red[16];
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, n_wave = blockDim.x >> 6;
+  {   // one workgroup per row of a batch
+    const size_t row = (size_t)blockIdx.x * n;
+    x += row;
+    if (delta) delta += row;
+    if (normed) normed += row;
+    act.q += row;
+    act.d += (size_t)blockIdx.x * (n / GROUP);
+    act.sums += (size_t)blockIdx.x * (n / 16u);
+    act.bsum += (size_t)blockIdx.x * (n / 32u);
+  }
   float4 v[4], wv[4];
   float ss = 0.0f;
   // every load first (x, the residual delta and the norm weights share one trip to memory)
@@ -71,15 +81,15 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
 }
 
 hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const float *weight, uint32_t n,
-                                 float eps, float *normed, OgmActDev act, hipStream_t stream) {
-  if (n == 0 || n % 32u != 0 || n > 16384u) return hipErrorInvalidValue;
+                                 float eps, float *normed, OgmActDev act, hipStream_t stream, uint32_t n_rows) {
+  if (n == 0 || n % 32u != 0 || n > 16384u || n_rows == 0) return hipErrorInvalidValue;
   const uint32_t runs = (n + 255u) / 256u;
   const uint32_t waves = runs < 16u ? runs : 16u;
   if (mode == 0)
-    hipLaunchKernelGGL(ogm_norm_quant_kernel<32>, dim3(1), dim3(waves * 64), 0, stream, x, delta, weight,
+    hipLaunchKernelGGL(ogm_norm_quant_kernel<32>, dim3(n_rows), dim3(waves * 64), 0, stream, x, delta, weight,
                        n, eps, normed, act);
   else
-    hipLaunchKernelGGL(ogm_norm_quant_kernel<256>, dim3(1), dim3(waves * 64), 0, stream, x, delta, weight,
+    hipLaunchKernelGGL(ogm_norm_quant_kernel<256>, dim3(n_rows), dim3(waves * 64), 0, stream, x, delta, weight,
                        n, eps, normed, act);
   return hipGetLastError();
 }
@@ -627,6 +637,16 @@ __global__ __launch_bounds__(64) void ogm_swiglu_quant_kernel(const float *__res
   const uint32_t lane = threadIdx.x;
   const uint32_t e0 = blockIdx.x * 256u + 4u * lane;
   const bool active = e0 < n;
+  {   // blockIdx.y: the row of a batch
+    const size_t row = (size_t)blockIdx.y * n;
+    gate += row;
+    up += row;
+    if (h) h += row;
+    act.q += row;
+    act.d += (size_t)blockIdx.y * (n / GROUP);
+    act.sums += (size_t)blockIdx.y * (n / 16u);
+    act.bsum += (size_t)blockIdx.y * (n / 32u);
+  }
   float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
   if (active) {
     const float4 g = *(const float4 *)(gate + e0), u = *(const float4 *)(up + e0);
@@ -640,9 +660,9 @@ __global__ __launch_bounds__(64) void ogm_swiglu_quant_kernel(const float *__res
 }
 
 hipError_t ogm_launch_swiglu_quant(int mode, const float *gate, const float *up, uint32_t n, float *h,
-                                   OgmActDev act, hipStream_t stream) {
-  if (n == 0 || n % 32u != 0) return hipErrorInvalidValue;
-  const dim3 grid((n + 255u) / 256u);
+                                   OgmActDev act, hipStream_t stream, uint32_t n_rows) {
+  if (n == 0 || n % 32u != 0 || n_rows == 0 || n_rows > 65535u) return hipErrorInvalidValue;
+  const dim3 grid((n + 255u) / 256u, n_rows);
   if (mode == 0)
     hipLaunchKernelGGL(ogm_swiglu_quant_kernel<32>, grid, dim3(64), 0, stream, gate, up, n, h, act);
   else
@@ -845,44 +865,6 @@ hipError_t ogm_launch_dequant_row(const uint8_t *wt, uint32_t ggml_type, uint32_
 // ------------------------------------------------------------------------------------------
 // prefill: the same layer over a batch of tokens.  The matmuls are GEMMs that quantize their
 // own input, so these kernels leave plain f32 rows.
-
-// One workgroup per token row: x += delta (when given), normed = x * (1 / sqrt(mean(x^2) + eps)) * w.
-__global__ __launch_bounds__(256) void ogm_norm_rows_kernel(float *__restrict__ x, const float *__restrict__ delta,
-                                                            const float *__restrict__ weight, uint32_t n, float eps,
-                                                            float *__restrict__ normed) {
-  __shared__ float red[4];
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const size_t row = (size_t)blockIdx.x * n;
-  float ss = 0.0f;
-  for (uint32_t e0 = 4u * tid; e0 < n; e0 += 1024u) {
-    float4 v = *(const float4 *)(x + row + e0);
-    if (delta) {
-      const float4 d = *(const float4 *)(delta + row + e0);
-      v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
-      *(float4 *)(x + row + e0) = v;
-    }
-    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-  }
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) ss += __shfl_xor(ss, m, 64);
-  if (lane == 0) red[wave] = ss;
-  __syncthreads();
-  const float total = red[0] + red[1] + red[2] + red[3];
-  const float scale = 1.0f / sqrtf(total / (float)n + eps);
-  for (uint32_t e0 = 4u * tid; e0 < n; e0 += 1024u) {
-    const float4 v = *(const float4 *)(x + row + e0);   // this thread's own stores above
-    const float4 w = *(const float4 *)(weight + e0);
-    *(float4 *)(normed + row + e0) = make_float4(v.x * scale * w.x, v.y * scale * w.y, v.z * scale * w.z,
-                                                 v.w * scale * w.w);
-  }
-}
-
-hipError_t ogm_launch_norm_rows(float *x, const float *delta, const float *weight, uint32_t n, uint32_t n_rows,
-                                float eps, float *normed, hipStream_t stream) {
-  if (n == 0 || n % 4u != 0 || n_rows == 0) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(ogm_norm_rows_kernel, dim3(n_rows), dim3(256), 0, stream, x, delta, weight, n, eps, normed);
-  return hipGetLastError();
-}
 
 // One wave per (token, head of q | k | v): bias, per-head norm and RoPE as the decode kernel's
 // first phase; q is rewritten in place, k and v go to their cache rows as f16.
@@ -1273,22 +1255,3 @@ hipError_t ogm_launch_attn_prefill_mfma(const float *q, void *k_cache_layer, voi
   return hipGetLastError();
 }
 
-// h = silu(gate) * up over n values (all rows of a batch at once)
-__global__ __launch_bounds__(256) void ogm_swiglu_rows_kernel(const float *__restrict__ gate,
-                                                              const float *__restrict__ up, size_t n,
-                                                              float *__restrict__ h) {
-  const size_t stride = (size_t)gridDim.x * blockDim.x * 4u;
-  for (size_t e0 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4u; e0 < n; e0 += stride) {
-    const float4 g = *(const float4 *)(gate + e0), u = *(const float4 *)(up + e0);
-    *(float4 *)(h + e0) = make_float4(g.x / (1.0f + expf(-g.x)) * u.x, g.y / (1.0f + expf(-g.y)) * u.y,
-                                      g.z / (1.0f + expf(-g.z)) * u.z, g.w / (1.0f + expf(-g.w)) * u.w);
-  }
-}
-
-hipError_t ogm_launch_swiglu_rows(const float *gate, const float *up, size_t n, float *h, hipStream_t stream) {
-  if (n == 0 || n % 4u != 0) return hipErrorInvalidValue;
-  size_t blocks = (n / 4u + 255u) / 256u;
-  if (blocks > 4096u) blocks = 4096u;
-  hipLaunchKernelGGL(ogm_swiglu_rows_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, gate, up, n, h);
-  return hipGetLastError();
-}
