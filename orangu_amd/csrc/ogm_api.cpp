@@ -779,7 +779,7 @@ struct ogm_llama {
   size_t stage_cap = 0;
   // prefill rows, allocated at the first prefill for OGM_PREFILL_CHUNK tokens
   struct Prefill {
-    float *x = nullptr, *normed = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
+    float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
     float *proj = nullptr, *gate = nullptr, *up = nullptr, *cs = nullptr;
     float *part_o = nullptr, *part_ml = nullptr;   // attn_prefill_variant 1 only, allocated when it first runs
     uint32_t *tokens = nullptr;
@@ -1151,7 +1151,6 @@ static int llama_prefill_buffers(ogm_ctx *ctx, ogm_llama *m) {
   int rc = OGM_OK;
   auto A = [&](float **p, size_t n) { if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)p, n * 4); };
   A(&m->pf.x, T * c.n_embd);
-  A(&m->pf.normed, T * c.n_embd);
   A(&m->pf.q, T * qd);
   A(&m->pf.k, T * kvd);
   A(&m->pf.v, T * kvd);
@@ -1223,23 +1222,21 @@ static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws
   return OGM_OK;
 }
 
-// x += delta, RMSNorm, and the matmuls over the normed rows.  When every weight takes the same
-// activation format the norm kernel quantizes its own output (the decode step's kernel, one
-// workgroup per row) and the f32 rows are never stored; otherwise they are, and each group of
-// weights quantizes them for itself.
+// x += delta, RMSNorm, and the matmuls over the normed rows: the norm kernel quantizes its own
+// output (the decode step's kernel, one workgroup per row) and the f32 rows are never stored.  As in
+// the decode step, the matrices behind one norm must take the same activation format.
 static int llama_norm_matmul_rows(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *const *ws, float *const *ys, size_t n,
                                   const float *delta, const float *norm_w, uint32_t T, hipStream_t s) {
   const ogm_llama_config &c = m->cfg;
-  ogm_llama::Prefill &P = m->pf;
   const int mode = act_mode_for(ws[0]->ggml_type);
-  bool same = true;
-  for (size_t i = 1; i < n; i++) same = same && act_mode_for(ws[i]->ggml_type) == mode;
+  for (size_t i = 1; i < n; i++)
+    if (act_mode_for(ws[i]->ggml_type) != mode)
+      return fail(ctx, OGM_ERR_UNSUPPORTED, "matrices over one input must share an activation mode");
   int rc = ensure_act(ctx, c.n_embd, T);
   if (rc != OGM_OK) return rc;
-  HIPCHK(ctx, ogm_launch_norm_quant(mode, P.x, delta, norm_w, c.n_embd, c.rms_eps, same ? nullptr : P.normed,
+  HIPCHK(ctx, ogm_launch_norm_quant(mode, m->pf.x, delta, norm_w, c.n_embd, c.rms_eps, nullptr,
                                     act_view(ctx, c.n_embd, mode, 0), s, T));
-  if (same) return llama_matmul_quantized_rows(ctx, ws, ys, n, mode, c.n_embd, T, s);
-  return llama_matmul_rows(ctx, ws, ys, n, P.normed, T, s);
+  return llama_matmul_quantized_rows(ctx, ws, ys, n, mode, c.n_embd, T, s);
 }
 
 // One chunk of T <= OGM_PREFILL_CHUNK tokens whose embedding rows sit in m->pf.x.  With `last`,

@@ -767,18 +767,20 @@ struct GemmI8pParams {
 // latency of its loads, takes a feeding wave about as long as eight matrix instructions and their
 // operand reads take a multiplying one (with half as many feeding waves the multiplying ones sat
 // idle for more than half of every stage).
-template <uint32_t ROWS>
+template <uint32_t ROWS, bool Q3>
 __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   constexpr uint32_t NC = ROWS / 16u;                // multiplying waves
   constexpr uint32_t WT = ROWS * GI_ROW;             // bytes of a plane's stage
-  constexpr uint32_t TILE_BYTES = 13440u;   // 64 units of 210 bytes: 13 pieces of 1 KiB, then 64 two-byte tails
+  // Q6_K: 64 units of 210 bytes are 13 pieces of 1 KiB, then 64 two-byte tails; Q3_K: 7 pieces
+  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : 13440u;
+  constexpr uint32_t NPL = Q3 ? 1u : 2u;             // operand planes
   // three stages of 64 weights in LDS: one being multiplied, the next being read into registers
   // behind it, the third being written by the feeding waves
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *wh_l = lds;                                      // [3][ROWS][64 of 80]: plane h
-  uint8_t *wl_l = lds + 3u * WT;                            // plane l
-  uint8_t *x_l = lds + 6u * WT;                             // [3][128 tokens][64 of 80]: activations
-  float *d_l = (float *)(lds + 6u * WT + 3u * GI_WTILE);    // [2][ROWS] the rows' d
+  uint8_t *wl_l = lds + 3u * WT;                            // plane l (Q6_K)
+  uint8_t *x_l = lds + 3u * NPL * WT;                       // [3][128 tokens][64 of 80]: activations
+  float *d_l = (float *)(lds + 3u * NPL * WT + 3u * GI_WTILE);   // [2][ROWS] the rows' d
   float *ad_l = d_l + 2u * ROWS;                            // [2][128] the tokens' activation scale
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -831,20 +833,32 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     uint4 xb0_, xb1_, xb2_, xb3_;   // ROWS = 64: the thread's other 16 bytes
     uint4 scxa = make_uint4(0, 0, 0, 0);      // the 16 scales of the row, next super-block
     uint32_t sca[4] = {0, 0, 0, 0};           // ... of the super-block being stored
+    uint4 hmxn = make_uint4(0, 0, 0, 0);      // Q3_K: the group's 16 bytes of hmask, next super-block
+    uint32_t hmw[4] = {0, 0, 0, 0};           // ... of the super-block being stored
     uint32_t d16 = 0;
     float adn = 0.0f;
 #define GP_LOAD(S, G, K)                                                                          \
   do {                                                                                            \
     const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded again, never used */ \
     const uint32_t so_ = sb_tile(s_) + sb_lane(s_) * 16u, h_ = (G) >> 1;                          \
-    qla##K = *(const uint4 *)(p.wt + (uo + so_ + (4u * h_ + t16) * 1024u));                       \
-    qha##K = *(const uint4 *)(p.wt + (uo + so_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));           \
+    if constexpr (Q3) {                                                                           \
+      /* pieces: hmask 0..1, qs 2..5, then scales[12] | d | two bytes of padding */               \
+      qla##K = *(const uint4 *)(p.wt + (uo + so_ + (2u + 2u * h_ + (t16 & 1u)) * 1024u));         \
+    } else {                                                                                      \
+      qla##K = *(const uint4 *)(p.wt + (uo + so_ + (4u * h_ + t16) * 1024u));                     \
+      qha##K = *(const uint4 *)(p.wt + (uo + so_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));         \
+    }                                                                                             \
     const uint4 *xp_ = (const uint4 *)(p.xq + (xro + 256u * s_ + 64u * (G)));                     \
     xa##K##_ = xp_[0];                                                                            \
     if constexpr (ROWS == 64u) xb##K##_ = xp_[1];                                                 \
     if ((G) == 0u) {                                                                              \
-      scxa = *(const uint4 *)(p.wt + (uo + so_ + 12u * 1024u));                                   \
-      if (has_d) d16 = *(const uint16_t *)(p.wt + (dto + sb_tile(s_) + sb_lane(s_) * 2u));        \
+      if constexpr (Q3) {                                                                         \
+        scxa = *(const uint4 *)(p.wt + (uo + so_ + 6u * 1024u));                                  \
+        hmxn = *(const uint4 *)(p.wt + (uo + so_ + (t16 & 1u) * 1024u));                          \
+      } else {                                                                                    \
+        scxa = *(const uint4 *)(p.wt + (uo + so_ + 12u * 1024u));                                 \
+        if (has_d) d16 = *(const uint16_t *)(p.wt + (dto + sb_tile(s_) + sb_lane(s_) * 2u));      \
+      }                                                                                           \
       if (has_ad) adn = p.ad[aro + s_];                                                           \
     }                                                                                             \
   } while (0)
@@ -873,14 +887,48 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     *(uint4 *)&wh_l[(BUF) + (ROWOFF) * GI_ROW + 16u * (T16)] = make_uint4(ph_[0], ph_[1], ph_[2], ph_[3]); \
     *(uint4 *)&wl_l[(BUF) + (ROWOFF) * GI_ROW + 16u * (T16)] = make_uint4(pl_[0], pl_[1], pl_[2], pl_[3]); \
   } while (0)
+  // Q3_K (gemm_k_q6_k over unpacked rows, vecdot.rs:2100-2117): sixteen 3-bit weights, q - 4 in
+  // [-4, 3], times the group's scale sc - 32 in [-32, 31] (quant.rs:883-897: low four bits in a
+  // nibble of byte i % 8, two high bits at bit 2 (i / 4) of byte 8 + i % 4, i = 4 G + t16).  The
+  // product reaches +128, its negative fits int8: one plane of sc * (4 - q), and isum = -H.
+#define GP_GROUP3(QL, G, BUF, ROWOFF, T16)                                                        \
+  do {                                                                                            \
+    const uint32_t lw_ = ((G) & 1u) ? sca[1] : sca[0];                                            \
+    const uint32_t low_ = ((lw_ >> (8u * (T16))) >> ((G) >= 2u ? 4u : 0u)) & 0xFu;                \
+    const uint32_t high_ = ((sca[2] >> (8u * (T16))) >> (2u * (G))) & 3u;                         \
+    const int sc_ = (int)(low_ | (high_ << 4)) - 32;                                              \
+    const short2v msc2_ = {(short)(-sc_), (short)(-sc_)};                                         \
+    const short2v c2_ = {(short)(4 * sc_), (short)(4 * sc_)};                                     \
+    const uint32_t rr_ = 2u * ((G) & 1u) + ((T16) >> 1);      /* run of 32 inside the half block */ \
+    const uint32_t qlw_[4] = {QL.x, QL.y, QL.z, QL.w};                                            \
+    uint32_t ph_[4];                                                                              \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      /* run p = 2 G + t16 / 2 of 32: two bits at 2 (p % 4), third bit = bit p of hmask */        \
+      const uint32_t v_ = ((qlw_[w_] >> (2u * rr_)) & 0x03030303u) |                              \
+                          (((hmw[w_] >> (2u * (G) + ((T16) >> 1))) & 0x01010101u) << 2);          \
+      union { uint32_t u; short2v s; } e_, f_;                                                    \
+      e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
+      f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
+      e_.s = e_.s * msc2_ + c2_;                                                                  \
+      f_.s = f_.s * msc2_ + c2_;                                                                  \
+      ph_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u);   /* the lanes' low bytes */      \
+    }                                                                                             \
+    *(uint4 *)&wh_l[(BUF) + (ROWOFF) * GI_ROW + 16u * (T16)] = make_uint4(ph_[0], ph_[1], ph_[2], ph_[3]); \
+  } while (0)
 #define GP_STORE(S, G, K)                                                                         \
   do {                                                                                            \
     if ((G) == 0u) {                                                                              \
       sca[0] = scxa.x; sca[1] = scxa.y; sca[2] = scxa.z; sca[3] = scxa.w;                         \
-      if (has_d) d_l[ROWS * ((S) & 1u) + pt] = gm_f16_bits_to_f32(d16);                           \
+      if constexpr (Q3) {                                                                         \
+        hmw[0] = hmxn.x; hmw[1] = hmxn.y; hmw[2] = hmxn.z; hmw[3] = hmxn.w;                       \
+        if (has_d) d_l[ROWS * ((S) & 1u) + pt] = gm_f16_bits_to_f32(scxa.w & 0xFFFFu);            \
+      } else {                                                                                    \
+        if (has_d) d_l[ROWS * ((S) & 1u) + pt] = gm_f16_bits_to_f32(d16);                         \
+      }                                                                                           \
       if (has_ad) ad_l[128u * ((S) & 1u) + ad_tok] = adn;                                         \
     }                                                                                             \
-    GP_GROUP(qla##K, qha##K, sca, G, pw, prw, t16);                                               \
+    if constexpr (Q3) GP_GROUP3(qla##K, G, pw, prw, t16);                                         \
+    else GP_GROUP(qla##K, qha##K, sca, G, pw, prw, t16);                                          \
     uint8_t *xr_ = &x_l[px + xrow_ * GI_ROW + XB * xpart];                                        \
     *(uint4 *)xr_ = xa##K##_;                                                                     \
     if constexpr (ROWS == 64u) *(uint4 *)(xr_ + 16u) = xb##K##_;                                  \
@@ -914,6 +962,7 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     }
 #undef GP_LOAD
 #undef GP_GROUP
+#undef GP_GROUP3
 #undef GP_STORE
   } else {
     // y0 / y1: tokens t0 + tw + (8 (r / 4) + 4 lh + r % 4), rows r0 + 64 rh + l32 and + 32
@@ -934,8 +983,10 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     x##SUF = *(const int4v *)&x_l[(OFFX) + xrow];             \
     wh0##SUF = *(const int4v *)&wh_l[(OFFW) + wrow0];         \
     wh1##SUF = *(const int4v *)&wh_l[(OFFW) + wrow1];         \
-    wl0##SUF = *(const int4v *)&wl_l[(OFFW) + wrow0];         \
-    wl1##SUF = *(const int4v *)&wl_l[(OFFW) + wrow1];         \
+    if constexpr (!Q3) {                                      \
+      wl0##SUF = *(const int4v *)&wl_l[(OFFW) + wrow0];       \
+      wl1##SUF = *(const int4v *)&wl_l[(OFFW) + wrow1];       \
+    }                                                         \
   } while (0)
     GP_READ(a, 0u, 0u);
     for (uint32_t s = 0; s < p.nsb; s++) {
@@ -946,19 +997,25 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
         if (g == 0u) {   // the super-block starts fresh sums
           h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh0a, zi, 0, 0, 0);
           h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh1a, zi, 0, 0, 0);
-          l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl0a, zi, 0, 0, 0);
-          l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl1a, zi, 0, 0, 0);
+          if constexpr (!Q3) {
+            l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl0a, zi, 0, 0, 0);
+            l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl1a, zi, 0, 0, 0);
+          }
         } else {
           h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh0a, h0, 0, 0, 0);
           h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh1a, h1, 0, 0, 0);
-          l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl0a, l0, 0, 0, 0);
-          l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl1a, l1, 0, 0, 0);
+          if constexpr (!Q3) {
+            l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl0a, l0, 0, 0, 0);
+            l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl1a, l1, 0, 0, 0);
+          }
         }
         GP_READ(a, nw, nx);   // complete since the last barrier; past the last stage: read, never used
         h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wh0b, h0, 0, 0, 0);
         h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wh1b, h1, 0, 0, 0);
-        l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wl0b, l0, 0, 0, 0);
-        l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wl1b, l1, 0, 0, 0);
+        if constexpr (!Q3) {
+          l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wl0b, l0, 0, 0, 0);
+          l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wl1b, l1, 0, 0, 0);
+        }
         cw = nw;
         cx = nx;
         if (g == 3u) {
@@ -970,8 +1027,8 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
             const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-              const int is0 = h0[4 * q4 + e] * 256 + l0[4 * q4 + e];
-              const int is1 = h1[4 * q4 + e] * 256 + l1[4 * q4 + e];
+              const int is0 = Q3 ? -h0[4 * q4 + e] : h0[4 * q4 + e] * 256 + l0[4 * q4 + e];
+              const int is1 = Q3 ? -h1[4 * q4 + e] : h1[4 * q4 + e] * 256 + l1[4 * q4 + e];
               y0[4 * q4 + e] += a4v[e] * (d0 * (float)is0);
               y1[4 * q4 + e] += a4v[e] * (d1 * (float)is1);
             }
@@ -993,8 +1050,10 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   }
 }
 
-__global__ __launch_bounds__(1024) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u>(p); }
-__global__ __launch_bounds__(512) void ogm_gemm_q6k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, false>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q6k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, false>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q3k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, true>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q3k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, true>(p); }
 
 // ------------------------------------------------------------------------------------------
 // Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
@@ -2024,7 +2083,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   const bool i8 = (a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K) && a.q4k_variant != 2u;
   const bool wide = a.ggml_type == OGM_Q4_K && !i8 && a.n_tokens > 256u &&
                     wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
-  const bool i8p = a.ggml_type == OGM_Q6_K && a.q4k_variant != 2u;   // needs nothing prepared
+  const bool i8p = (a.ggml_type == OGM_Q6_K || a.ggml_type == OGM_Q3_K) && a.q4k_variant != 2u;   // needs nothing prepared
   const bool raw_x = wide || i8 || i8p;   // these read the int8 activations as they are: only (bh, bl) to prepare
   if (!i8p)
     hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((raw_x ? n_sb : n8) + 255) / 256)), dim3(256), 0,
@@ -2065,7 +2124,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     }
     return hipGetLastError();
   }
-  if (a.ggml_type == OGM_Q6_K && a.q4k_variant != 2u) {
+  if (i8p) {
     GemmI8pParams p;
     p.wt = a.wt;
     p.xq = a.act.q;
@@ -2093,17 +2152,27 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     const uint32_t rows = r64 ? 64u : 128u;
     const uint32_t tiles = r64 ? tiles64 : row_tiles;
     const dim3 pgrid((a.n_tokens + 127u) / 128u, tiles);
-    const uint32_t lds_bytes = 6u * rows * GI_ROW + 3u * GI_WTILE + (2u * rows + 256u) * 4u;
-    const void *fn = r64 ? (const void *)ogm_gemm_q6k_i8_r64_kernel : (const void *)ogm_gemm_q6k_i8_kernel;
+    const bool q3 = a.ggml_type == OGM_Q3_K;
+    const uint32_t lds_bytes = (q3 ? 3u : 6u) * rows * GI_ROW + 3u * GI_WTILE + (2u * rows + 256u) * 4u;
+    const void *fn = q3 ? (r64 ? (const void *)ogm_gemm_q3k_i8_r64_kernel : (const void *)ogm_gemm_q3k_i8_kernel)
+                        : (r64 ? (const void *)ogm_gemm_q6k_i8_r64_kernel : (const void *)ogm_gemm_q6k_i8_kernel);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
-    if (r64) {
+    const char *name;
+    if (q3 && r64) {
+      hipLaunchKernelGGL(ogm_gemm_q3k_i8_r64_kernel, pgrid, dim3(512), lds_bytes, stream, p);
+      name = "ogm_gemm_q3k_i8_r64_kernel";
+    } else if (q3) {
+      hipLaunchKernelGGL(ogm_gemm_q3k_i8_kernel, pgrid, dim3(1024), lds_bytes, stream, p);
+      name = "ogm_gemm_q3k_i8_kernel";
+    } else if (r64) {
       hipLaunchKernelGGL(ogm_gemm_q6k_i8_r64_kernel, pgrid, dim3(512), lds_bytes, stream, p);
-      if (kernel_name) *kernel_name = "ogm_gemm_q6k_i8_r64_kernel";
+      name = "ogm_gemm_q6k_i8_r64_kernel";
     } else {
       hipLaunchKernelGGL(ogm_gemm_q6k_i8_kernel, pgrid, dim3(1024), lds_bytes, stream, p);
-      if (kernel_name) *kernel_name = "ogm_gemm_q6k_i8_kernel";
+      name = "ogm_gemm_q6k_i8_kernel";
     }
+    if (kernel_name) *kernel_name = name;
     return hipGetLastError();
   }
   if (a.ggml_type != OGM_Q4_K) {

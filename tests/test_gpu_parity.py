@@ -368,6 +368,8 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     (Q5_K, 130, (520, 70, 129), "ogm_gemm_q5k_kernel"),
     (Q5_K, 130, (520, 70, 129), "ogm_gemm_q5k_i8_kernel"),
     (Q3_K, 40, (128, 300), "ogm_gemm_q3k_kernel"),
+    (Q3_K, 140, (128, 300, 70), "ogm_gemm_q3k_i8_r64_kernel"),
+    (Q3_K, 300, (6000, 3000, 2100), "ogm_gemm_q3k_i8_kernel"),
 ])
 def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, outs, kernel):
     """q / k / v (llama.rs:730-746) at prefill widths: K-quant matrices of one type over the same
@@ -530,25 +532,28 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign, variant)
     say("extreme q6k isum", int(np.abs(isum).max()))
 
 
-@pytest.mark.parametrize("t,kernel", [(Q3_K, "ogm_gemm_q3k_kernel"), (Q5_K, "ogm_gemm_q5k_kernel"),
-                                      (Q5_K, "ogm_gemm_q5k_i8_kernel")])
+@pytest.mark.parametrize("t,kernel", [(Q3_K, "ogm_gemm_q3k_kernel"), (Q3_K, "ogm_gemm_q3k_i8_kernel"),
+                                      (Q5_K, "ogm_gemm_q5k_kernel"), (Q5_K, "ogm_gemm_q5k_i8_kernel")])
 @pytest.mark.parametrize("in_dim,out_dim,T", [
     (256, 5, 9), (512, 130, 17), (768, 64, 129), (1024, 100, 64), (1280, 257, 40), (2048, 37, 128),
-    (4096, 200, 130), (14336, 96, 257), (4096, 1000, 512), (1792, 33, 10),
+    (4096, 200, 130), (14336, 96, 257), (4096, 1000, 512), (1792, 33, 10), (512, 4200, 513),
 ])
 def test_mfma_gemm_q3k_q5k_match_cpu_gemm(be, t, kernel, in_dim, out_dim, T):
     """Q3_K (a KKind::Q6K row, vecdot.rs:2100-2117) and Q5_K (a KKind::Q4K row, :2064-2088) on the
-    two-chain MFMA kernel: every bit of gemm_k_q6_k / gemm_k_q4_k (vecdot.rs:2213-2255, 2352-2398),
-    and of the multi-token GEMV that served these types before."""
+    two-chain f16 MFMA kernel and on their int8 kernels (Q3_K: one plane of scale-folded weights, on
+    64-row tiles when those are few): every bit of gemm_k_q6_k / gemm_k_q4_k (vecdot.rs:2213-2255,
+    2352-2398), and of the multi-token GEMV that served these types before."""
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T + 1)
     w = qm(raw, t, in_dim, out_dim)
     say("gemm", kernel, in_dim, out_dim, T)
-    be.set_tuning("gemm_q4k_variant", 0 if kernel.endswith("_i8_kernel") or t == Q3_K else 2)   # Q5_K: int8 by default
+    be.set_tuning("gemm_q4k_variant", 0 if kernel.endswith("_i8_kernel") else 2)   # int8 by default
     try:
         got = be.matmul(x, T, w)
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
+    if kernel == "ogm_gemm_q3k_i8_kernel" and ((T + 127) // 128) * ((out_dim + 63) // 64) <= 256:
+        kernel = "ogm_gemm_q3k_i8_r64_kernel"
     assert be.last_kernel() == kernel
     want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
     assert_close(got, want, kernel)
@@ -599,10 +604,13 @@ def test_mfma_gemm_q5k_adversarial_integer_ranges(be, qs, qh, sc, sign, variant)
 
 @pytest.mark.parametrize("qs,hm,sc,sign", [(0xFF, 0xFF, 0xFF, "alt"), (0x00, 0x00, 0x00, "pos"), (0x00, 0x00, 0xFF, "neg"),
                                            (0xFF, 0x00, 0x00, "block"), (0x1B, 0x5A, 0x9C, "alt"), (0xE4, 0xA5, 0x63, "pos")])
-def test_mfma_gemm_q3k_adversarial_integer_ranges(be, qs, hm, sc, sign):
+@pytest.mark.parametrize("variant", [0, 3, 2])
+def test_mfma_gemm_q3k_adversarial_integer_ranges(be, qs, hm, sc, sign, variant):
     """Weights -4 and 3, scales -32 and 31 (every six-bit pattern's bytes at their extremes) and
-    activations +-127."""
-    in_dim, out_dim, T = 1024, 32, 16
+    activations +-127.  -32 * -4 = 128 is the product that does not fit an int8: the int8 kernels
+    (variant 0: 64-row tiles on this small grid; 3: 128-row tiles, by way of 300 tokens x 6000 rows)
+    carry the negated product, -128; variant 2 is the f16 kernel."""
+    in_dim, out_dim, T = (1024, 6000, 300) if variant == 3 else (1024, 32, 16)
     blocks = np.zeros((out_dim * 4, 110), np.uint8)
     blocks[:, 0:32] = hm
     blocks[:, 32:96] = qs
@@ -618,8 +626,12 @@ def test_mfma_gemm_q3k_adversarial_integer_ranges(be, qs, hm, sc, sign):
         x[:, 128:256] *= -1
         x[3] = -127.0
     raw = blocks.reshape(-1)
-    got = be.matmul(x, T, qm(raw, Q3_K, in_dim, out_dim))
-    assert be.last_kernel() == "ogm_gemm_q3k_kernel"
+    be.set_tuning("gemm_q4k_variant", variant % 3)
+    try:
+        got = be.matmul(x, T, qm(raw, Q3_K, in_dim, out_dim))
+    finally:
+        be.set_tuning("gemm_q4k_variant", 0)
+    assert be.last_kernel() == {0: "ogm_gemm_q3k_i8_r64_kernel", 3: "ogm_gemm_q3k_i8_kernel", 2: "ogm_gemm_q3k_kernel"}[variant]
     assert_bits(got, oracle.matmul(Q3_K, raw, in_dim, out_dim, x, T), "extreme ranges")
 
 
