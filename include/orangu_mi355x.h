@@ -327,8 +327,9 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * keys: "gemv_wg_waves" (waves per workgroup of the GEMV kernel, 1..16; 0 = heuristic);
  * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default 9,
  * below it the multi-token GEMV kernel runs in the GEMM's float order);
- * "gemm_q4k_variant" (K-quant GEMM: 0 = default, the int8 matrix-core kernels;
- * 1 = the same with Q6_K and Q3_K always on their 64-row tiles; 2 = the f16 kernels);
+ * "gemm_q4k_variant" (K-quant GEMM: 0 = default, the int8 matrix-core kernels over scale-folded
+ * weight planes; 1 = the same, always on 64-row tiles; 2 = the f16 kernels; 3 = for Q4_K and Q5_K the
+ * int8 kernel that scales partial sums by multiply-adds);
  * "gemm_wide_min_wgs" (f16 Q4_K kernels: 128 x 128 workgroups from which the 128 x 256 tile runs; 0 = 256);
  * "attn_prefill_variant" (attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the
  * decode step's kernel per token and chunk of the cache; they agree to f32 rounding, not bit for bit);

@@ -221,7 +221,7 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     return OGM_OK;
   }
   if (strcmp(key, "gemm_q4k_variant") == 0) {
-    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_q4k_variant must be 0, 1 or 2");
+    if (value < 0 || value > 3) return fail(ctx, OGM_ERR_INVALID, "gemm_q4k_variant must be 0..3");
     ctx->tune_gemm_q4k_variant = value;
     return OGM_OK;
   }

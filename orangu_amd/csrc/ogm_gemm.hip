@@ -749,9 +749,10 @@ __global__ __launch_bounds__(768) void ogm_gemm_q5k_i8_kernel(GemmParams p) { ge
 typedef short short2v __attribute__((ext_vector_type(2)));
 
 struct GemmI8pParams {
-  const uint8_t *wt;      // tile-planar Q6_K
+  const uint8_t *wt;      // tile-planar weights
   const int8_t *xq;       // [T][in_dim] int8 activations
   const float *ad;        // [T][nsb]
+  const _Float16 *bs16;   // Q4_K / Q5_K: the quantizer's sums per 32 as (bsum / 64, bsum % 64) in f16
   float *y;               // [T][out_dim]
   uint32_t in_dim, out_dim, n_tokens, nsb;
   uint32_t c_shift, r_shift, nct;
@@ -767,12 +768,19 @@ struct GemmI8pParams {
 // latency of its loads, takes a feeding wave about as long as eight matrix instructions and their
 // operand reads take a multiplying one (with half as many feeding waves the multiplying ones sat
 // idle for more than half of every stage).
-template <uint32_t ROWS, bool Q3>
+#define GP_Q6K 0
+#define GP_Q3K 1
+#define GP_Q4K 2
+#define GP_Q5K 3
+template <uint32_t ROWS, int KIND>
 __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
+  constexpr bool Q3 = KIND == GP_Q3K, Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K;
   constexpr uint32_t NC = ROWS / 16u;                // multiplying waves
   constexpr uint32_t WT = ROWS * GI_ROW;             // bytes of a plane's stage
-  // Q6_K: 64 units of 210 bytes are 13 pieces of 1 KiB, then 64 two-byte tails; Q3_K: 7 pieces
-  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : 13440u;
+  // Q6_K: 64 units of 210 bytes are 13 pieces of 1 KiB, then 64 two-byte tails; Q3_K: 7 pieces;
+  // Q4_K: 9 (header, qs); Q5_K: 11 (header, qh, qs)
+  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : KIND == GP_Q4K ? 9216u : Q5 ? 11264u : 13440u;
+  constexpr uint32_t QS_PIECE0 = Q5 ? 3u : 1u;       // Q4_K / Q5_K: first piece of qs
   constexpr uint32_t NPL = Q3 ? 1u : 2u;             // operand planes
   // three stages of 64 weights in LDS: one being multiplied, the next being read into registers
   // behind it, the third being written by the feeding waves
@@ -806,6 +814,73 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   auto sb_tile = [&](uint32_t s) -> uint32_t { return (s >> p.c_shift) * TILE_BYTES; };
   auto sb_lane = [&](uint32_t s) -> uint32_t { return (s & ((1u << p.c_shift) - 1u)) << p.r_shift; };
 
+  // y0 / y1 of a multiplying wave: tokens t0 + tw + (8 (r / 4) + 4 lh + r % 4), rows r0 + 64 rh + l32 and + 32
+  float16v y0, y1;
+#pragma unroll
+  for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
+
+  if constexpr (Q45) {
+    // ---------------- pass 1 of gemm_k_q4_k: acc -= (ad * dmin) * sum_j m_j * bsum_j, all super-blocks
+    // first (vecdot.rs:2226-2240), on the f16 matrix cores with tokens as rows: 64 m_j against
+    // bsum_j / 64 and m_j against bsum_j % 64 in one K = 16 instruction per 32 x 32 outputs
+    __shared__ __align__(16) float p1_dmin[8][ROWS];   // eight super-blocks at a time
+    __shared__ __align__(16) float p1_ad[8][128];
+    auto row_off = [&](uint32_t row) -> uint32_t {
+      row = min(row, p.out_dim - 1u);
+      const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+      return rb * p.nct * TILE_BYTES + r * 16u;
+    };
+    float16v zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.0f;
+    const uint32_t ro0 = row_off(r0 + 64u * rh + l32), ro1 = row_off(r0 + 64u * rh + 32u + l32);
+    const uint32_t tk = min(t0 + tw + l32, p.n_tokens - 1u) * p.nsb;
+    const float side_scale = lh ? 1.0f : 64.0f;
+    for (uint32_t sg = 0; sg < p.nsb; sg += 8u) {
+      for (uint32_t i = tid; i < 8u * ROWS; i += blockDim.x) {
+        const uint32_t u = i / ROWS, k = i % ROWS, su = min(sg + u, p.nsb - 1u);
+        const uint32_t h = *(const uint32_t *)(p.wt + (row_off(r0 + k) + sb_tile(su) + sb_lane(su) * 16u));
+        p1_dmin[u][k] = gm_f16_bits_to_f32(h >> 16);
+      }
+      for (uint32_t i = tid; i < 8u * 128u; i += blockDim.x) {
+        const uint32_t u = i >> 7, k = i & 127u, su = min(sg + u, p.nsb - 1u);
+        p1_ad[u][k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + su];
+      }
+      __syncthreads();
+      if (!producer) {
+#pragma unroll 2
+        for (uint32_t u = 0; u < 8u; u++) {
+          if (sg + u >= p.nsb) break;
+          const uint32_t su = sg + u, so = sb_tile(su) + sb_lane(su) * 16u;
+          const uint4 hd0 = *(const uint4 *)(p.wt + (ro0 + so));
+          const uint4 hd1 = *(const uint4 *)(p.wt + (ro1 + so));
+          const half8 b2 = *(const half8 *)(p.bs16 + ((tk + su) * 16u + 8u * lh));
+          uint32_t mna, mnb;
+          q4k_mins(hd0, mna, mnb);
+          const half8 a10 = side_operand(mna, mnb, side_scale);
+          q4k_mins(hd1, mna, mnb);
+          const half8 a11 = side_operand(mna, mnb, side_scale);
+          const float dm0 = p1_dmin[u][64u * rh + l32], dm1 = p1_dmin[u][64u * rh + 32u + l32];
+          const float16v im0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2, a10, zero, 0, 0, 0);
+          const float16v im1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2, a11, zero, 0, 0, 0);
+          const float *adp = &p1_ad[u][tw + 4u * lh];
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++) {
+            const float4 a4 = *(const float4 *)(adp + 8 * q4);
+            const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              y0[4 * q4 + e] -= a4v[e] * dm0 * im0[4 * q4 + e];
+              y1[4 * q4 + e] -= a4v[e] * dm1 * im1[4 * q4 + e];
+            }
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+
+  // ---------------- the products: acc += ad * (d * isum) per super-block
   if (producer) {
     // Feeding thread pt stages one group of 16 weights per stage: one ql piece, one qh piece, one
     // scale.  A wave has one group index and 64 consecutive rows: its loads are 1 KiB runs and its
@@ -844,6 +919,9 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     if constexpr (Q3) {                                                                           \
       /* pieces: hmask 0..1, qs 2..5, then scales[12] | d | two bytes of padding */               \
       qla##K = *(const uint4 *)(p.wt + (uo + so_ + (2u + 2u * h_ + (t16 & 1u)) * 1024u));         \
+    } else if constexpr (Q45) {                                                                   \
+      /* 32 bytes of qs per pair of sub-blocks: low nibbles 2 G, high nibbles 2 G + 1 */          \
+      qla##K = *(const uint4 *)(p.wt + (uo + so_ + (QS_PIECE0 + 2u * (G) + (t16 & 1u)) * 1024u)); \
     } else {                                                                                      \
       qla##K = *(const uint4 *)(p.wt + (uo + so_ + (4u * h_ + t16) * 1024u));                     \
       qha##K = *(const uint4 *)(p.wt + (uo + so_ + (8u + 2u * h_ + (t16 & 1u)) * 1024u));         \
@@ -855,6 +933,9 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
       if constexpr (Q3) {                                                                         \
         scxa = *(const uint4 *)(p.wt + (uo + so_ + 6u * 1024u));                                  \
         hmxn = *(const uint4 *)(p.wt + (uo + so_ + (t16 & 1u) * 1024u));                          \
+      } else if constexpr (Q45) {                                                                 \
+        scxa = *(const uint4 *)(p.wt + (uo + so_));   /* d | dmin, then the 12 scale bytes */     \
+        if constexpr (Q5) hmxn = *(const uint4 *)(p.wt + (uo + so_ + (1u + (t16 & 1u)) * 1024u)); \
       } else {                                                                                    \
         scxa = *(const uint4 *)(p.wt + (uo + so_ + 12u * 1024u));                                 \
         if (has_d) d16 = *(const uint16_t *)(p.wt + (dto + sb_tile(s_) + sb_lane(s_) * 2u));      \
@@ -915,6 +996,37 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     }                                                                                             \
     *(uint4 *)&wh_l[(BUF) + (ROWOFF) * GI_ROW + 16u * (T16)] = make_uint4(ph_[0], ph_[1], ph_[2], ph_[3]); \
   } while (0)
+  // Q4_K / Q5_K (KKind::Q4K rows, vecdot.rs:2064-2088): sixteen weights 0..15 (Q5_K: 0..31 with
+  // bit j of qh on top) of sub-block j = 2 G + T16 / 2, times its scale 0..63 (get_scale_min_k4,
+  // quant.rs:653-662): u = sc * q + 128 <= 2081, planes as for Q6_K.
+#define GP_GROUP45(QL, G, BUF, ROWOFF, T16)                                                       \
+  do {                                                                                            \
+    uint32_t sc4a_, sc4b_;   /* the scales of sub-blocks 0..3 and 4..7, a byte each */            \
+    {                                                                                             \
+      const uint4 hd_ = make_uint4(sca[0], sca[1], sca[2], sca[3]);                               \
+      q4k_scales(hd_, sc4a_, sc4b_);                                                              \
+    }                                                                                             \
+    const uint32_t hi_ = (T16) >> 1, j_ = 2u * (G) + hi_;                                         \
+    const uint32_t scw_ = (G) < 2u ? sc4a_ : sc4b_;                                               \
+    const int sc_ = (int)((scw_ >> (8u * (j_ & 3u))) & 0xFFu);                                    \
+    const short2v sc2_ = {(short)sc_, (short)sc_};                                                \
+    const short2v c2_ = {128, 128};                                                               \
+    const uint32_t qlw_[4] = {QL.x, QL.y, QL.z, QL.w};                                            \
+    uint32_t ph_[4], pl_[4];                                                                      \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      uint32_t v_ = (hi_ ? (qlw_[w_] >> 4) : qlw_[w_]) & 0x0F0F0F0Fu;                             \
+      if constexpr (Q5) v_ |= ((hmw[w_] >> j_) & 0x01010101u) << 4;                               \
+      union { uint32_t u; short2v s; } e_, f_;                                                    \
+      e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
+      f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
+      e_.s = e_.s * sc2_ + c2_;                                                                   \
+      f_.s = f_.s * sc2_ + c2_;                                                                   \
+      ph_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x07050301u);                /* high bytes */   \
+      pl_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u) ^ 0x80808080u;  /* low bytes */    \
+    }                                                                                             \
+    *(uint4 *)&wh_l[(BUF) + (ROWOFF) * GI_ROW + 16u * (T16)] = make_uint4(ph_[0], ph_[1], ph_[2], ph_[3]); \
+    *(uint4 *)&wl_l[(BUF) + (ROWOFF) * GI_ROW + 16u * (T16)] = make_uint4(pl_[0], pl_[1], pl_[2], pl_[3]); \
+  } while (0)
 #define GP_STORE(S, G, K)                                                                         \
   do {                                                                                            \
     if ((G) == 0u) {                                                                              \
@@ -922,12 +1034,16 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
       if constexpr (Q3) {                                                                         \
         hmw[0] = hmxn.x; hmw[1] = hmxn.y; hmw[2] = hmxn.z; hmw[3] = hmxn.w;                       \
         if (has_d) d_l[ROWS * ((S) & 1u) + pt] = gm_f16_bits_to_f32(scxa.w & 0xFFFFu);            \
+      } else if constexpr (Q45) {                                                                 \
+        if constexpr (Q5) { hmw[0] = hmxn.x; hmw[1] = hmxn.y; hmw[2] = hmxn.z; hmw[3] = hmxn.w; } \
+        if (has_d) d_l[ROWS * ((S) & 1u) + pt] = gm_f16_bits_to_f32(scxa.x & 0xFFFFu);            \
       } else {                                                                                    \
         if (has_d) d_l[ROWS * ((S) & 1u) + pt] = gm_f16_bits_to_f32(d16);                         \
       }                                                                                           \
       if (has_ad) ad_l[128u * ((S) & 1u) + ad_tok] = adn;                                         \
     }                                                                                             \
     if constexpr (Q3) GP_GROUP3(qla##K, G, pw, prw, t16);                                         \
+    else if constexpr (Q45) GP_GROUP45(qla##K, G, pw, prw, t16);                                  \
     else GP_GROUP(qla##K, qha##K, sca, G, pw, prw, t16);                                          \
     uint8_t *xr_ = &x_l[px + xrow_ * GI_ROW + XB * xpart];                                        \
     *(uint4 *)xr_ = xa##K##_;                                                                     \
@@ -963,12 +1079,9 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
 #undef GP_LOAD
 #undef GP_GROUP
 #undef GP_GROUP3
+#undef GP_GROUP45
 #undef GP_STORE
   } else {
-    // y0 / y1: tokens t0 + tw + (8 (r / 4) + 4 lh + r % 4), rows r0 + 64 rh + l32 and + 32
-    float16v y0, y1;
-#pragma unroll
-    for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
     __syncthreads();
     int16v h0, h1, l0, l1;   // the two planes' sums of the running super-block
     const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -1050,10 +1163,14 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   }
 }
 
-__global__ __launch_bounds__(1024) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, false>(p); }
-__global__ __launch_bounds__(512) void ogm_gemm_q6k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, false>(p); }
-__global__ __launch_bounds__(1024) void ogm_gemm_q3k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, true>(p); }
-__global__ __launch_bounds__(512) void ogm_gemm_q3k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, true>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q6k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q6K>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q6k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q6K>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q3k_i8_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q3K>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q3k_i8_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q3K>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q4k_i8p_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q4K>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q4k_i8p_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q4K>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q5k_i8p_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q5K>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q5k_i8p_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q5K>(p); }
 
 // ------------------------------------------------------------------------------------------
 // Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
@@ -2078,14 +2195,17 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   uint32_t row_tiles = (a.out_dim + GM_BN - 1) / GM_BN;
   for (uint32_t m = 0; m < a.n_extra; m++) row_tiles += (a.extra_out_dim[m] + GM_BN - 1) / GM_BN;
   const uint32_t wgs128 = ((a.n_tokens + GM_BT - 1) / GM_BT) * row_tiles;
-  // Q4_K and Q5_K run on the int8 kernel unless the f16 kernels are asked for (q4k_variant 2); of
-  // Q4_K's the wide one takes over as described above
-  const bool i8 = (a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K) && a.q4k_variant != 2u;
-  const bool wide = a.ggml_type == OGM_Q4_K && !i8 && a.n_tokens > 256u &&
+  // K-quants run on the int8 kernels unless the f16 kernels are asked for (q4k_variant 2): the ones
+  // with scale-folded weight planes, or for Q4_K and Q5_K the one that scales partial sums by
+  // integer multiply-adds (q4k_variant 3).  Of the f16 Q4_K kernels the wide one takes over as
+  // described above.
+  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  const bool i8 = q45 && a.q4k_variant == 3u;
+  const bool i8p = a.q4k_variant != 2u && !i8;
+  const bool wide = a.ggml_type == OGM_Q4_K && a.q4k_variant == 2u && a.n_tokens > 256u &&
                     wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
-  const bool i8p = (a.ggml_type == OGM_Q6_K || a.ggml_type == OGM_Q3_K) && a.q4k_variant != 2u;   // needs nothing prepared
   const bool raw_x = wide || i8 || i8p;   // these read the int8 activations as they are: only (bh, bl) to prepare
-  if (!i8p)
+  if (!i8p || q45)   // the plane kernels of Q6_K and Q3_K need nothing prepared
     hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((raw_x ? n_sb : n8) + 255) / 256)), dim3(256), 0,
                        stream, a.act.q, a.act.bsum, raw_x ? (_Float16 *)nullptr : xh, bs16, n8, n_sb);
   const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
@@ -2129,6 +2249,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.wt = a.wt;
     p.xq = a.act.q;
     p.ad = a.act.d;
+    p.bs16 = bs16;
     p.y = a.y;
     p.in_dim = a.in_dim;
     p.out_dim = a.out_dim;
@@ -2154,24 +2275,27 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     const dim3 pgrid((a.n_tokens + 127u) / 128u, tiles);
     const bool q3 = a.ggml_type == OGM_Q3_K;
     const uint32_t lds_bytes = (q3 ? 3u : 6u) * rows * GI_ROW + 3u * GI_WTILE + (2u * rows + 256u) * 4u;
-    const void *fn = q3 ? (r64 ? (const void *)ogm_gemm_q3k_i8_r64_kernel : (const void *)ogm_gemm_q3k_i8_kernel)
-                        : (r64 ? (const void *)ogm_gemm_q6k_i8_r64_kernel : (const void *)ogm_gemm_q6k_i8_kernel);
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    struct Pick { uint32_t type; bool r64; const void *fn; const char *name; };
+    const Pick picks[] = {
+        {OGM_Q6_K, false, (const void *)ogm_gemm_q6k_i8_kernel, "ogm_gemm_q6k_i8_kernel"},
+        {OGM_Q6_K, true, (const void *)ogm_gemm_q6k_i8_r64_kernel, "ogm_gemm_q6k_i8_r64_kernel"},
+        {OGM_Q3_K, false, (const void *)ogm_gemm_q3k_i8_kernel, "ogm_gemm_q3k_i8_kernel"},
+        {OGM_Q3_K, true, (const void *)ogm_gemm_q3k_i8_r64_kernel, "ogm_gemm_q3k_i8_r64_kernel"},
+        {OGM_Q4_K, false, (const void *)ogm_gemm_q4k_i8p_kernel, "ogm_gemm_q4k_i8p_kernel"},
+        {OGM_Q4_K, true, (const void *)ogm_gemm_q4k_i8p_r64_kernel, "ogm_gemm_q4k_i8p_r64_kernel"},
+        {OGM_Q5_K, false, (const void *)ogm_gemm_q5k_i8p_kernel, "ogm_gemm_q5k_i8p_kernel"},
+        {OGM_Q5_K, true, (const void *)ogm_gemm_q5k_i8p_r64_kernel, "ogm_gemm_q5k_i8p_r64_kernel"},
+    };
+    const Pick *pick = nullptr;
+    for (const Pick &c : picks)
+      if (c.type == a.ggml_type && c.r64 == r64) pick = &c;
+    if (!pick) return hipErrorInvalidValue;
+    hipError_t e = hipFuncSetAttribute(pick->fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
-    const char *name;
-    if (q3 && r64) {
-      hipLaunchKernelGGL(ogm_gemm_q3k_i8_r64_kernel, pgrid, dim3(512), lds_bytes, stream, p);
-      name = "ogm_gemm_q3k_i8_r64_kernel";
-    } else if (q3) {
-      hipLaunchKernelGGL(ogm_gemm_q3k_i8_kernel, pgrid, dim3(1024), lds_bytes, stream, p);
-      name = "ogm_gemm_q3k_i8_kernel";
-    } else if (r64) {
-      hipLaunchKernelGGL(ogm_gemm_q6k_i8_r64_kernel, pgrid, dim3(512), lds_bytes, stream, p);
-      name = "ogm_gemm_q6k_i8_r64_kernel";
-    } else {
-      hipLaunchKernelGGL(ogm_gemm_q6k_i8_kernel, pgrid, dim3(1024), lds_bytes, stream, p);
-      name = "ogm_gemm_q6k_i8_kernel";
-    }
+    void *kargs[] = {(void *)&p};
+    e = hipLaunchKernel(pick->fn, pgrid, dim3(r64 ? 512 : 1024), kargs, lds_bytes, stream);
+    if (e != hipSuccess) return e;
+    const char *name = pick->name;
     if (kernel_name) *kernel_name = name;
     return hipGetLastError();
   }

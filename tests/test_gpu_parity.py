@@ -320,6 +320,22 @@ def test_q6k_vocab_projection_batches_1_4_8(be):
 
 # ---------------------------------------------------------------- prefill GEMM on MFMA
 
+def plane_kernel(base, T, outs):
+    """Name of the int8 plane kernel a K-quant GEMM launch takes: `base` (e.g. "ogm_gemm_q4k_i8p") on
+    128-row tiles, or its 64-row variant when those tiles still come one to a compute unit."""
+    outs = outs if isinstance(outs, (tuple, list)) else (outs,)
+    small = ((T + 127) // 128) * sum((o + 63) // 64 for o in outs) <= 256
+    return base + ("_r64_kernel" if small else "_kernel")
+
+
+def variant_of(kernel):
+    """gemm_q4k_variant that makes the launcher pick `kernel`: 0 the plane kernels (default), 3 the
+    multiply-add int8 kernels of Q4_K / Q5_K, 2 the f16 kernels."""
+    if "_i8p_" in kernel or kernel.startswith(("ogm_gemm_q6k_i8", "ogm_gemm_q3k_i8")):
+        return 0
+    return 3 if kernel.endswith("_i8_kernel") else 2
+
+
 @pytest.mark.parametrize("in_dim,out_dim,T", [
     (1024, 64, 9), (1024, 100, 64), (2048, 37, 128), (4096, 200, 130), (1024, 16, 300), (8192, 70, 33),
     (256, 5, 9), (512, 130, 17), (768, 64, 129), (1280, 257, 40), (14336, 96, 257), (4096, 1000, 512),
@@ -328,18 +344,27 @@ def test_q6k_vocab_projection_batches_1_4_8(be):
 def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     """ogm_matmul at n_tokens >= 9 takes the matrix-core kernels; values must equal CpuBackend's
     K-quant GEMM (vecdot.rs:2213-2303): integer sums exact, f32 order the reference's.  The int8
-    kernel (the default) and the two f16 kernels it replaced each produce the same bits."""
+    plane kernel (the default; both tile heights), the int8 multiply-add kernel and the two f16
+    kernels each produce the same bits."""
     raw = synth_weights(Q4_K, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T)
     w = qm(raw, Q4_K, in_dim, out_dim)
     say("gemm", in_dim, out_dim, T)
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     got = be.matmul(x, T, w)
-    assert be.last_kernel() == "ogm_gemm_q4k_i8_kernel"
-    assert_close(got, want, "int8 mfma gemm")
-    assert_bits(got, want, "int8 mfma gemm")
-    be.set_tuning("gemm_q4k_variant", 2)
+    assert be.last_kernel() == plane_kernel("ogm_gemm_q4k_i8p", T, out_dim)
+    assert_close(got, want, "int8 plane gemm")
+    assert_bits(got, want, "int8 plane gemm")
+    be.set_tuning("gemm_q4k_variant", 1)   # the 64-row tiles whatever the grid
     try:
+        got = be.matmul(x, T, w)
+        assert be.last_kernel() == "ogm_gemm_q4k_i8p_r64_kernel"
+        assert_bits(got, want, "int8 plane gemm, 64-row tiles")
+        be.set_tuning("gemm_q4k_variant", 3)
+        got = be.matmul(x, T, w)
+        assert be.last_kernel() == "ogm_gemm_q4k_i8_kernel"
+        assert_bits(got, want, "int8 multiply-add gemm")
+        be.set_tuning("gemm_q4k_variant", 2)
         got = be.matmul(x, T, w)
         # beyond 256 tokens the 128 x 256 tile kernel runs once the 128 x 128 tiling would take more
         # than one round of workgroups (256)
@@ -359,6 +384,10 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
 @pytest.mark.parametrize("t,n_tokens,outs,kernel", [
     (Q4_K, 40, (300, 130, 64), "ogm_gemm_q4k_i8_kernel"),
     (Q4_K, 300, (520, 70), "ogm_gemm_q4k_i8_kernel"),
+    (Q4_K, 40, (300, 130, 64), "ogm_gemm_q4k_i8p_r64_kernel"),
+    (Q4_K, 300, (6000, 3000, 2100), "ogm_gemm_q4k_i8p_kernel"),
+    (Q5_K, 130, (520, 70, 129), "ogm_gemm_q5k_i8p_r64_kernel"),
+    (Q5_K, 300, (6000, 3000, 2100), "ogm_gemm_q5k_i8p_kernel"),
     (Q4_K, 40, (300, 130, 64), "ogm_gemm_q4k_kernel"),          # the f16 kernels: one round of 128 x 128 tiles
     (Q4_K, 300, (520, 70), "ogm_gemm_q4k_kernel"),              # more than 256 tokens, still one round
     (Q4_K, 300, (6000, 3000, 2100), "ogm_gemm_q4k_wide_kernel"),  # 264 tiles of 128 x 128: the wide tiling
@@ -382,7 +411,7 @@ def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, ou
     x = synth_x(n_tokens, in_dim, seed=17)
     xd = DeviceBuffer.from_numpy(x)
     yds = [DeviceBuffer(4 * n_tokens * od) for od in outs]
-    be.set_tuning("gemm_q4k_variant", 0 if "_i8_" in kernel else 2)
+    be.set_tuning("gemm_q4k_variant", variant_of(kernel))
     try:
         be.matmul_multi_dev(hs, xd.ptr, n_tokens, [y.ptr for y in yds])
     finally:
@@ -418,7 +447,7 @@ def test_mfma_gemm_equals_small_batch_kernel_and_is_batch_independent(be):
         assert_bits(part, full[:n], f"{n} of 40")
 
 
-@pytest.mark.parametrize("variant", [0, 2])
+@pytest.mark.parametrize("variant", [0, 3, 2])
 @pytest.mark.parametrize("T", [16, 272])
 @pytest.mark.parametrize("qs_lo,qs_hi,sign", [(0xFF, 0xFF, "alt"), (0x00, 0x00, "alt"), (0x0F, 0xF0, "pos"),
                                                (0xF0, 0x0F, "neg"), (0xFF, 0x00, "block")])
@@ -426,8 +455,9 @@ def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T, variant
     """Largest magnitudes the integer stage can see: nibbles 0 or 15, scales and mins 63, activations
     +-127.  The per-super-block sum reaches 3.1e7 > 2^24 and the centred partial sums and their
     correction reach +-1.64e7 each (and cancel when every nibble is 0), so the f32 add of the exact
-    parts must round exactly like `isum as f32` (f16 kernels, variant 2); the int8 kernel keeps the
-    whole sum in 32-bit integers and converts once."""
+    parts must round exactly like `isum as f32` (f16 kernels, variant 2); the int8 kernels keep the
+    whole sum in 32-bit integers and convert once (variant 0: 63 * 15 + 128 = 1073 split into the
+    planes 4 and -79; variant 3: multiply-adds on the sub-blocks' sums)."""
     in_dim, out_dim = 1024, 32
     blocks = np.zeros((out_dim * 4, 144), np.uint8)
     blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
@@ -452,7 +482,8 @@ def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T, variant
     finally:
         be.set_tuning("gemm_wide_min_wgs", 0)
         be.set_tuning("gemm_q4k_variant", 0)
-    assert be.last_kernel() == ("ogm_gemm_q4k_i8_kernel" if variant == 0 else
+    assert be.last_kernel() == ("ogm_gemm_q4k_i8p_r64_kernel" if variant == 0 else
+                                "ogm_gemm_q4k_i8_kernel" if variant == 3 else
                                 "ogm_gemm_q4k_wide_kernel" if T > 256 else "ogm_gemm_q4k_kernel")
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     assert_bits(got, want, "extreme ranges")
@@ -533,27 +564,28 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign, variant)
 
 
 @pytest.mark.parametrize("t,kernel", [(Q3_K, "ogm_gemm_q3k_kernel"), (Q3_K, "ogm_gemm_q3k_i8_kernel"),
-                                      (Q5_K, "ogm_gemm_q5k_kernel"), (Q5_K, "ogm_gemm_q5k_i8_kernel")])
+                                      (Q5_K, "ogm_gemm_q5k_kernel"), (Q5_K, "ogm_gemm_q5k_i8_kernel"),
+                                      (Q5_K, "ogm_gemm_q5k_i8p_kernel")])
 @pytest.mark.parametrize("in_dim,out_dim,T", [
     (256, 5, 9), (512, 130, 17), (768, 64, 129), (1024, 100, 64), (1280, 257, 40), (2048, 37, 128),
     (4096, 200, 130), (14336, 96, 257), (4096, 1000, 512), (1792, 33, 10), (512, 4200, 513),
 ])
 def test_mfma_gemm_q3k_q5k_match_cpu_gemm(be, t, kernel, in_dim, out_dim, T):
     """Q3_K (a KKind::Q6K row, vecdot.rs:2100-2117) and Q5_K (a KKind::Q4K row, :2064-2088) on the
-    two-chain f16 MFMA kernel and on their int8 kernels (Q3_K: one plane of scale-folded weights, on
-    64-row tiles when those are few): every bit of gemm_k_q6_k / gemm_k_q4_k (vecdot.rs:2213-2255,
+    two-chain f16 MFMA kernel and on their int8 kernels (planes of scale-folded weights, on 64-row
+    tiles when those are few; Q5_K also with multiply-adds on the sub-blocks' sums): every bit of gemm_k_q6_k / gemm_k_q4_k (vecdot.rs:2213-2255,
     2352-2398), and of the multi-token GEMV that served these types before."""
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T + 1)
     w = qm(raw, t, in_dim, out_dim)
     say("gemm", kernel, in_dim, out_dim, T)
-    be.set_tuning("gemm_q4k_variant", 0 if kernel.endswith("_i8_kernel") else 2)   # int8 by default
+    be.set_tuning("gemm_q4k_variant", variant_of(kernel))
     try:
         got = be.matmul(x, T, w)
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
-    if kernel == "ogm_gemm_q3k_i8_kernel" and ((T + 127) // 128) * ((out_dim + 63) // 64) <= 256:
-        kernel = "ogm_gemm_q3k_i8_r64_kernel"
+    if variant_of(kernel) == 0:
+        kernel = plane_kernel(kernel[:-len("_kernel")], T, out_dim)
     assert be.last_kernel() == kernel
     want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
     assert_close(got, want, kernel)
@@ -567,7 +599,7 @@ def test_mfma_gemm_q3k_q5k_match_cpu_gemm(be, t, kernel, in_dim, out_dim, T):
     assert_bits(got, small, "mfma vs multi-token gemv")
 
 
-@pytest.mark.parametrize("variant", [0, 2])
+@pytest.mark.parametrize("variant", [0, 3, 2])
 @pytest.mark.parametrize("qs,qh,sc,sign", [(0xFF, 0xFF, 0xFF, "alt"), (0x00, 0x00, 0xFF, "pos"), (0xFF, 0xFF, 0xFF, "neg"),
                                            (0xFF, 0xFF, 0x3F, "block"), (0xF0, 0x55, 0xC7, "alt"), (0x0F, 0xAA, 0x00, "pos")])
 def test_mfma_gemm_q5k_adversarial_integer_ranges(be, qs, qh, sc, sign, variant):
@@ -596,7 +628,7 @@ def test_mfma_gemm_q5k_adversarial_integer_ranges(be, qs, qh, sc, sign, variant)
         got = be.matmul(x, T, qm(raw, Q5_K, in_dim, out_dim))
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
-    assert be.last_kernel() == ("ogm_gemm_q5k_i8_kernel" if variant == 0 else "ogm_gemm_q5k_kernel")
+    assert be.last_kernel() == {0: "ogm_gemm_q5k_i8p_r64_kernel", 3: "ogm_gemm_q5k_i8_kernel", 2: "ogm_gemm_q5k_kernel"}[variant]
     assert_bits(got, oracle.matmul(Q5_K, raw, in_dim, out_dim, x, T), "extreme ranges")
     isum, imin = be.dump_block_sums(x[0], 1, qm(raw, Q5_K, in_dim, out_dim))
     say("extreme q5k isum", int(np.abs(isum).max()), "imin", int(np.abs(imin).max()))
