@@ -762,7 +762,7 @@ struct GemmI8pParams {
   uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
 };
 
-// ROWS = 128: eight multiplying waves (64 rows x 32 tokens each) and eight feeding ones; ROWS = 64:
+// ROWS = 128: eight multiplying waves (32 rows x 64 tokens each) and eight feeding ones; ROWS = 64:
 // four and four, and half the LDS: twice as many workgroups, which fills the chip when a launch has
 // few row tiles.  As many feeding as multiplying waves, because a stage's unpacking, behind the
 // latency of its loads, takes a feeding wave about as long as eight matrix instructions and their
@@ -794,7 +794,9 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const bool producer = wave >= NC;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
-  const uint32_t tq = wave & 3u, rh = ROWS == 128u ? (wave >> 2) & 1u : 0u;
+  // a multiplying wave: 32 rows (block rq) x 64 tokens (half th): one weight operand per plane feeds
+  // two matrix instructions, which keeps the LDS reads at four per 32 k
+  const uint32_t rq = wave % (ROWS / 32u), th = (wave / (ROWS / 32u)) & 1u;
   uint32_t row_tile = blockIdx.y;
 #pragma unroll
   for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
@@ -809,12 +811,12 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     }
   }
   const uint32_t t0 = blockIdx.x * 128u, r0 = row_tile * ROWS;
-  const uint32_t tw = 32u * tq;
+  const uint32_t tw = 64u * th;   // the wave's first token within the workgroup
 
   auto sb_tile = [&](uint32_t s) -> uint32_t { return (s >> p.c_shift) * TILE_BYTES; };
   auto sb_lane = [&](uint32_t s) -> uint32_t { return (s & ((1u << p.c_shift) - 1u)) << p.r_shift; };
 
-  // y0 / y1 of a multiplying wave: tokens t0 + tw + (8 (r / 4) + 4 lh + r % 4), rows r0 + 64 rh + l32 and + 32
+  // y0 / y1 of a multiplying wave: row r0 + 32 rq + l32, tokens t0 + tw + (8 (r / 4) + 4 lh + r % 4) and + 32
   float16v y0, y1;
 #pragma unroll
   for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
@@ -822,61 +824,49 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   if constexpr (Q45) {
     // ---------------- pass 1 of gemm_k_q4_k: acc -= (ad * dmin) * sum_j m_j * bsum_j, all super-blocks
     // first (vecdot.rs:2226-2240), on the f16 matrix cores with tokens as rows: 64 m_j against
-    // bsum_j / 64 and m_j against bsum_j % 64 in one K = 16 instruction per 32 x 32 outputs
-    __shared__ __align__(16) float p1_dmin[8][ROWS];   // eight super-blocks at a time
-    __shared__ __align__(16) float p1_ad[8][128];
-    auto row_off = [&](uint32_t row) -> uint32_t {
-      row = min(row, p.out_dim - 1u);
-      const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
-      return rb * p.nct * TILE_BYTES + r * 16u;
-    };
-    float16v zero;
+    // bsum_j / 64 and m_j against bsum_j % 64 in one K = 16 instruction per 32 x 32 outputs.  The
+    // tokens' ad of every super-block go to LDS once; a row's dmin and mins come with its header.
+    float *ad_all = ad_l + 256;   // [nsb][128]
+    for (uint32_t i = tid; i < 128u * p.nsb; i += blockDim.x) {
+      const uint32_t k = i / p.nsb, su = i - k * p.nsb;   // consecutive threads: consecutive super-blocks of a token
+      ad_all[su * 128u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + su];
+    }
+    __syncthreads();
+    if (!producer) {
+      float16v zero;
 #pragma unroll
-    for (int r = 0; r < 16; r++) zero[r] = 0.0f;
-    const uint32_t ro0 = row_off(r0 + 64u * rh + l32), ro1 = row_off(r0 + 64u * rh + 32u + l32);
-    const uint32_t tk = min(t0 + tw + l32, p.n_tokens - 1u) * p.nsb;
-    const float side_scale = lh ? 1.0f : 64.0f;
-    for (uint32_t sg = 0; sg < p.nsb; sg += 8u) {
-      for (uint32_t i = tid; i < 8u * ROWS; i += blockDim.x) {
-        const uint32_t u = i / ROWS, k = i % ROWS, su = min(sg + u, p.nsb - 1u);
-        const uint32_t h = *(const uint32_t *)(p.wt + (row_off(r0 + k) + sb_tile(su) + sb_lane(su) * 16u));
-        p1_dmin[u][k] = gm_f16_bits_to_f32(h >> 16);
+      for (int r = 0; r < 16; r++) zero[r] = 0.0f;
+      uint32_t ro0;
+      {
+        const uint32_t row = min(r0 + 32u * rq + l32, p.out_dim - 1u);
+        ro0 = (row >> p.r_shift) * p.nct * TILE_BYTES + (row & ((1u << p.r_shift) - 1u)) * 16u;
       }
-      for (uint32_t i = tid; i < 8u * 128u; i += blockDim.x) {
-        const uint32_t u = i >> 7, k = i & 127u, su = min(sg + u, p.nsb - 1u);
-        p1_ad[u][k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + su];
-      }
-      __syncthreads();
-      if (!producer) {
-#pragma unroll 2
-        for (uint32_t u = 0; u < 8u; u++) {
-          if (sg + u >= p.nsb) break;
-          const uint32_t su = sg + u, so = sb_tile(su) + sb_lane(su) * 16u;
-          const uint4 hd0 = *(const uint4 *)(p.wt + (ro0 + so));
-          const uint4 hd1 = *(const uint4 *)(p.wt + (ro1 + so));
-          const half8 b2 = *(const half8 *)(p.bs16 + ((tk + su) * 16u + 8u * lh));
-          uint32_t mna, mnb;
-          q4k_mins(hd0, mna, mnb);
-          const half8 a10 = side_operand(mna, mnb, side_scale);
-          q4k_mins(hd1, mna, mnb);
-          const half8 a11 = side_operand(mna, mnb, side_scale);
-          const float dm0 = p1_dmin[u][64u * rh + l32], dm1 = p1_dmin[u][64u * rh + 32u + l32];
-          const float16v im0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2, a10, zero, 0, 0, 0);
-          const float16v im1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2, a11, zero, 0, 0, 0);
-          const float *adp = &p1_ad[u][tw + 4u * lh];
+      const uint32_t tk0 = min(t0 + tw + l32, p.n_tokens - 1u) * p.nsb;
+      const uint32_t tk1 = min(t0 + tw + 32u + l32, p.n_tokens - 1u) * p.nsb;
+      const float side_scale = lh ? 1.0f : 64.0f;
+#pragma unroll 4
+      for (uint32_t su = 0; su < p.nsb; su++) {
+        const uint4 hd0 = *(const uint4 *)(p.wt + (ro0 + sb_tile(su) + sb_lane(su) * 16u));
+        const half8 b20 = *(const half8 *)(p.bs16 + ((tk0 + su) * 16u + 8u * lh));
+        const half8 b21 = *(const half8 *)(p.bs16 + ((tk1 + su) * 16u + 8u * lh));
+        uint32_t mna, mnb;
+        q4k_mins(hd0, mna, mnb);
+        const half8 a1 = side_operand(mna, mnb, side_scale);
+        const float dm = gm_f16_bits_to_f32(hd0.x >> 16);
+        const float16v im0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b20, a1, zero, 0, 0, 0);
+        const float16v im1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b21, a1, zero, 0, 0, 0);
+        const float *adp = &ad_all[su * 128u + tw + 4u * lh];
 #pragma unroll
-          for (int q4 = 0; q4 < 4; q4++) {
-            const float4 a4 = *(const float4 *)(adp + 8 * q4);
-            const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+        for (int q4 = 0; q4 < 4; q4++) {
+          const float4 a4 = *(const float4 *)(adp + 8 * q4), b4 = *(const float4 *)(adp + 32 + 8 * q4);
+          const float a4v[4] = {a4.x, a4.y, a4.z, a4.w}, b4v[4] = {b4.x, b4.y, b4.z, b4.w};
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-              y0[4 * q4 + e] -= a4v[e] * dm0 * im0[4 * q4 + e];
-              y1[4 * q4 + e] -= a4v[e] * dm1 * im1[4 * q4 + e];
-            }
+          for (int e = 0; e < 4; e++) {
+            y0[4 * q4 + e] -= a4v[e] * dm * im0[4 * q4 + e];
+            y1[4 * q4 + e] -= b4v[e] * dm * im1[4 * q4 + e];
           }
         }
       }
-      __syncthreads();
     }
   }
 
@@ -1085,21 +1075,18 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     __syncthreads();
     int16v h0, h1, l0, l1;   // the two planes' sums of the running super-block
     const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    const uint32_t xrow = (tw + l32) * GI_ROW + 16u * lh;
-    const uint32_t wrow0 = (64u * rh + l32) * GI_ROW + 16u * lh, wrow1 = wrow0 + 32u * GI_ROW;
+    const uint32_t xrow0 = (tw + l32) * GI_ROW + 16u * lh, xrow1 = xrow0 + 32u * GI_ROW;
+    const uint32_t wrow = (32u * rq + l32) * GI_ROW + 16u * lh;
     // operands of the stage's first 32 weights (a) and last 32 (b); a of the next stage is read
     // while b multiplies, b while a does
-    int4v xa, wh0a, wh1a, wl0a, wl1a, xb, wh0b, wh1b, wl0b, wl1b;
+    int4v x0a, x1a, wha, wla, x0b, x1b, whb, wlb;
     uint32_t cw = 0, cx = 0;   // byte offsets of the stage's buffers: weight planes, activations
 #define GP_READ(SUF, OFFW, OFFX)                              \
   do {                                                        \
-    x##SUF = *(const int4v *)&x_l[(OFFX) + xrow];             \
-    wh0##SUF = *(const int4v *)&wh_l[(OFFW) + wrow0];         \
-    wh1##SUF = *(const int4v *)&wh_l[(OFFW) + wrow1];         \
-    if constexpr (!Q3) {                                      \
-      wl0##SUF = *(const int4v *)&wl_l[(OFFW) + wrow0];       \
-      wl1##SUF = *(const int4v *)&wl_l[(OFFW) + wrow1];       \
-    }                                                         \
+    x0##SUF = *(const int4v *)&x_l[(OFFX) + xrow0];           \
+    x1##SUF = *(const int4v *)&x_l[(OFFX) + xrow1];           \
+    wh##SUF = *(const int4v *)&wh_l[(OFFW) + wrow];           \
+    if constexpr (!Q3) wl##SUF = *(const int4v *)&wl_l[(OFFW) + wrow]; \
   } while (0)
     GP_READ(a, 0u, 0u);
     for (uint32_t s = 0; s < p.nsb; s++) {
@@ -1108,42 +1095,42 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
         const uint32_t nw = cw == 2u * WT ? 0u : cw + WT, nx = cx == 2u * GI_WTILE ? 0u : cx + GI_WTILE;
         GP_READ(b, cw + 32u, cx + 32u);
         if (g == 0u) {   // the super-block starts fresh sums
-          h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh0a, zi, 0, 0, 0);
-          h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh1a, zi, 0, 0, 0);
+          h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0a, wha, zi, 0, 0, 0);
+          h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1a, wha, zi, 0, 0, 0);
           if constexpr (!Q3) {
-            l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl0a, zi, 0, 0, 0);
-            l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl1a, zi, 0, 0, 0);
+            l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0a, wla, zi, 0, 0, 0);
+            l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1a, wla, zi, 0, 0, 0);
           }
         } else {
-          h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh0a, h0, 0, 0, 0);
-          h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wh1a, h1, 0, 0, 0);
+          h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0a, wha, h0, 0, 0, 0);
+          h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1a, wha, h1, 0, 0, 0);
           if constexpr (!Q3) {
-            l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl0a, l0, 0, 0, 0);
-            l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, wl1a, l1, 0, 0, 0);
+            l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0a, wla, l0, 0, 0, 0);
+            l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1a, wla, l1, 0, 0, 0);
           }
         }
         GP_READ(a, nw, nx);   // complete since the last barrier; past the last stage: read, never used
-        h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wh0b, h0, 0, 0, 0);
-        h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wh1b, h1, 0, 0, 0);
+        h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0b, whb, h0, 0, 0, 0);
+        h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1b, whb, h1, 0, 0, 0);
         if constexpr (!Q3) {
-          l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wl0b, l0, 0, 0, 0);
-          l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xb, wl1b, l1, 0, 0, 0);
+          l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0b, wlb, l0, 0, 0, 0);
+          l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1b, wlb, l1, 0, 0, 0);
         }
         cw = nw;
         cx = nx;
         if (g == 3u) {
-          const float d0 = d_l[ROWS * (s & 1u) + 64u * rh + l32], d1 = d_l[ROWS * (s & 1u) + 64u * rh + 32u + l32];
+          const float d0 = d_l[ROWS * (s & 1u) + 32u * rq + l32];
           const float *adp = &ad_l[128u * (s & 1u) + tw + 4u * lh];
 #pragma unroll
           for (int q4 = 0; q4 < 4; q4++) {
-            const float4 a4 = *(const float4 *)(adp + 8 * q4);
-            const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+            const float4 a4 = *(const float4 *)(adp + 8 * q4), b4 = *(const float4 *)(adp + 32 + 8 * q4);
+            const float a4v[4] = {a4.x, a4.y, a4.z, a4.w}, b4v[4] = {b4.x, b4.y, b4.z, b4.w};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
               const int is0 = Q3 ? -h0[4 * q4 + e] : h0[4 * q4 + e] * 256 + l0[4 * q4 + e];
               const int is1 = Q3 ? -h1[4 * q4 + e] : h1[4 * q4 + e] * 256 + l1[4 * q4 + e];
               y0[4 * q4 + e] += a4v[e] * (d0 * (float)is0);
-              y1[4 * q4 + e] += a4v[e] * (d1 * (float)is1);
+              y1[4 * q4 + e] += b4v[e] * (d0 * (float)is1);
             }
           }
         }
@@ -1151,13 +1138,13 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
       }
     }
 #undef GP_READ
-    const uint32_t row0 = r0 + 64u * rh + l32;
+    const uint32_t row0 = r0 + 32u * rq + l32;
+    if (row0 < p.out_dim) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const uint32_t t = t0 + tw + 8u * (r >> 2) + 4u * lh + (r & 3);
-      if (t < p.n_tokens) {
-        if (row0 < p.out_dim) p.y[(size_t)t * p.out_dim + row0] = y0[r];
-        if (row0 + 32u < p.out_dim) p.y[(size_t)t * p.out_dim + row0 + 32u] = y1[r];
+      for (int r = 0; r < 16; r++) {
+        const uint32_t t = t0 + tw + 8u * (r >> 2) + 4u * lh + (r & 3);
+        if (t < p.n_tokens) p.y[(size_t)t * p.out_dim + row0] = y0[r];
+        if (t + 32u < p.n_tokens) p.y[(size_t)(t + 32u) * p.out_dim + row0] = y1[r];
       }
     }
   }
@@ -2200,7 +2187,8 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   // integer multiply-adds (q4k_variant 3).  Of the f16 Q4_K kernels the wide one takes over as
   // described above.
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
-  const bool i8 = q45 && a.q4k_variant == 3u;
+  // (the plane kernel keeps a table of nsb * 512 bytes in LDS next to its 94 KB of stages)
+  const bool i8 = q45 && (a.q4k_variant == 3u || nsb * 512u + 98304u > GM_LDS_MAX);
   const bool i8p = a.q4k_variant != 2u && !i8;
   const bool wide = a.ggml_type == OGM_Q4_K && a.q4k_variant == 2u && a.n_tokens > 256u &&
                     wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
@@ -2274,7 +2262,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     const uint32_t tiles = r64 ? tiles64 : row_tiles;
     const dim3 pgrid((a.n_tokens + 127u) / 128u, tiles);
     const bool q3 = a.ggml_type == OGM_Q3_K;
-    const uint32_t lds_bytes = (q3 ? 3u : 6u) * rows * GI_ROW + 3u * GI_WTILE + (2u * rows + 256u) * 4u;
+    // Q4_K / Q5_K: + the tokens' ad of every super-block for the first pass
+    const uint32_t lds_bytes = (q3 ? 3u : 6u) * rows * GI_ROW + 3u * GI_WTILE + (2u * rows + 256u) * 4u +
+                               (q45 ? nsb * 512u : 0u);
     struct Pick { uint32_t type; bool r64; const void *fn; const char *name; };
     const Pick picks[] = {
         {OGM_Q6_K, false, (const void *)ogm_gemm_q6k_i8_kernel, "ogm_gemm_q6k_i8_kernel"},
