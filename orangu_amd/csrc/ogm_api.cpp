@@ -41,7 +41,7 @@ struct ogm_ctx {
   std::vector<ogm_weight *> weights;
   // scratch, grown on demand and reused (the vendor backends allocate per call,
   // engine/backend/rocm.rs:352-376; a pool is what the Vulkan op_cache does instead)
-  DevBuf x, y, q, d, sums, bsum, isum, imin, xh;
+  DevBuf x, y, q, d, sums, bsum, bs16, isum, imin, xh;
   DevBuf hx, hy;  // pinned host staging
   int tune_wg_waves = 0;
   int tune_gemm_min_tokens = 9;  // matmul at n_tokens >= this takes the MFMA GEMM
@@ -116,6 +116,7 @@ static int ensure_act(ogm_ctx *ctx, uint32_t in_dim, uint32_t n_tokens) {
   if ((rc = ensure_dev(ctx, ctx->d, n / 32 * 4)) != OGM_OK) return rc;
   if ((rc = ensure_dev(ctx, ctx->sums, n / 16 * 4)) != OGM_OK) return rc;
   if ((rc = ensure_dev(ctx, ctx->bsum, n / 32 * 2)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->bs16, n / 16 * 2)) != OGM_OK) return rc;
   return OGM_OK;
 }
 
@@ -125,6 +126,7 @@ static OgmActDev act_view(ogm_ctx *ctx, uint32_t in_dim, int mode, uint32_t toke
   a.d = (float *)ctx->d.p + (size_t)token0 * (in_dim / (mode == OGM_ACT_PER_32 ? 32 : 256));
   a.sums = (int32_t *)ctx->sums.p + (size_t)token0 * (in_dim / 16);
   a.bsum = (int16_t *)ctx->bsum.p + (size_t)token0 * (in_dim / 32);
+  a.bs16 = mode == OGM_ACT_PER_32 ? nullptr : (uint16_t *)ctx->bs16.p + (size_t)token0 * (in_dim / 16);
   return a;
 }
 
@@ -171,7 +173,8 @@ extern "C" void ogm_destroy(ogm_ctx *ctx) {
     if (w->dev) (void)hipFree(w->dev);
     delete w;
   }
-  DevBuf *dev[] = {&ctx->x, &ctx->y, &ctx->q, &ctx->d, &ctx->sums, &ctx->bsum, &ctx->isum, &ctx->imin, &ctx->xh};
+  DevBuf *dev[] = {&ctx->x,    &ctx->y,    &ctx->q,    &ctx->d,  &ctx->sums,
+                   &ctx->bsum, &ctx->bs16, &ctx->isum, &ctx->imin, &ctx->xh};
   for (DevBuf *b : dev)
     if (b->p) (void)hipFree(b->p);
   if (ctx->hx.p) (void)hipHostFree(ctx->hx.p);

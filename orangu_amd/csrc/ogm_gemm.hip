@@ -2193,7 +2193,12 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   const bool wide = a.ggml_type == OGM_Q4_K && a.q4k_variant == 2u && a.n_tokens > 256u &&
                     wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
   const bool raw_x = wide || i8 || i8p;   // these read the int8 activations as they are: only (bh, bl) to prepare
-  if (!i8p || q45)   // the plane kernels of Q6_K and Q3_K need nothing prepared
+  // The first-pass operand (the quantizer's sums per 32 as f16 pairs) comes from the quantizer itself
+  // when it wrote one; the f16 kernels also want the activations as f16.  The plane kernels of Q6_K
+  // and Q3_K need neither.
+  const bool have_bs16 = raw_x && a.act.bs16 != nullptr;
+  if (have_bs16) bs16 = (_Float16 *)a.act.bs16;
+  if ((!i8p || q45) && !have_bs16)
     hipLaunchKernelGGL(ogm_gemm_prep_kernel, dim3((unsigned)(((raw_x ? n_sb : n8) + 255) / 256)), dim3(256), 0,
                        stream, a.act.q, a.act.bsum, raw_x ? (_Float16 *)nullptr : xh, bs16, n8, n_sb);
   const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);

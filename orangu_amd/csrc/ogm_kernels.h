@@ -13,6 +13,9 @@ struct OgmActDev {
   float *d;
   int32_t *sums;
   int16_t *bsum;
+  // per-256 mode only: the sums per 32 once more as f16 pairs (bsum >> 6, bsum & 63), sixteen halves
+  // per super-block (eight high parts, then eight low parts): the K-quant GEMMs' first-pass operand
+  uint16_t *bs16;
 };
 
 // mode 0: one scale per 32 (vecdot.rs:95-126); mode 1: one per 256 (vecdot.rs:3030-3053).

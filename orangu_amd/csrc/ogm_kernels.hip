@@ -61,7 +61,8 @@ __global__ __launch_bounds__(64) void ogm_quantize_kernel(const float *__restric
   if (active) v = *(const float4 *)(x + (size_t)t * in_dim + e0);
   ogm_quantize_store<GROUP>(v, e0, active, lane, act.q + (size_t)t * in_dim,
                             act.d + (size_t)t * (in_dim / GROUP), act.sums + (size_t)t * (in_dim / 16),
-                            act.bsum + (size_t)t * (in_dim / 32));
+                            act.bsum + (size_t)t * (in_dim / 32),
+                            act.bs16 ? act.bs16 + (size_t)t * (in_dim / 16) : nullptr);
 }
 
 hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,

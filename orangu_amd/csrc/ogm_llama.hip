@@ -36,6 +36,7 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
     act.d += (size_t)blockIdx.x * (n / GROUP);
     act.sums += (size_t)blockIdx.x * (n / 16u);
     act.bsum += (size_t)blockIdx.x * (n / 32u);
+    if (act.bs16) act.bs16 += (size_t)blockIdx.x * (n / 16u);
   }
   float4 v[4], wv[4];
   float ss = 0.0f;
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
       if (normed) *(float4 *)(normed + e0) = o;
     }
     if ((wave + k * n_wave) * 256u < n)  // wave-uniform: the run exists
-      ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum);
+      ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
   }
 }
 
@@ -546,7 +547,7 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
         ov.x /= den; ov.y /= den; ov.z /= den; ov.w /= den;
         if (attn_out) *(float4 *)(attn_out + e0) = ov;
       }
-      ogm_quantize_store<GROUP>(ov, e0, active, lane, act.q, act.d, act.sums, act.bsum);
+      ogm_quantize_store<GROUP>(ov, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
     }
   }
 }
@@ -570,7 +571,7 @@ __global__ __launch_bounds__(64) void ogm_attn_combine_quant_kernel(const float 
     o = make_float4(pt.o.x / pt.den, pt.o.y / pt.den, pt.o.z / pt.den, pt.o.w / pt.den);
     if (attn_out) *(float4 *)(attn_out + e0) = o;
   }
-  ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum);
+  ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
 }
 
 hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
@@ -646,6 +647,7 @@ __global__ __launch_bounds__(64) void ogm_swiglu_quant_kernel(const float *__res
     act.d += (size_t)blockIdx.y * (n / GROUP);
     act.sums += (size_t)blockIdx.y * (n / 16u);
     act.bsum += (size_t)blockIdx.y * (n / 32u);
+    if (act.bs16) act.bs16 += (size_t)blockIdx.y * (n / 16u);
   }
   float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
   if (active) {
@@ -656,7 +658,7 @@ __global__ __launch_bounds__(64) void ogm_swiglu_quant_kernel(const float *__res
     o.w = g.w / (1.0f + expf(-g.w)) * u.w;
     if (h) *(float4 *)(h + e0) = o;
   }
-  ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum);
+  ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
 }
 
 hipError_t ogm_launch_swiglu_quant(int mode, const float *gate, const float *up, uint32_t n, float *h,

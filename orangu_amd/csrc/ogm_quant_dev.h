@@ -6,6 +6,7 @@
 //   scale = amax / 127 ; inv = scale > 0 ? 1/scale : 0   (vecdot.rs:106-107)
 //   q     = clamp(round_half_away(v * inv), -127, 127), NaN -> 0   (vecdot.rs:117)
 #pragma once
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -48,14 +49,23 @@ __device__ __forceinline__ uint32_t ogm_quantize4(const float4 &v, float &scale,
 // 4*lane) of token-major activations with row length in_dim; t_off* are the token's offsets.
 template <int GROUP>
 __device__ __forceinline__ void ogm_quantize_store(const float4 &v, uint32_t e0, bool active, uint32_t lane,
-                                                   int8_t *q, float *d, int32_t *sums, int16_t *bsum) {
+                                                   int8_t *q, float *d, int32_t *sums, int16_t *bsum,
+                                                   uint16_t *bs16) {
   float scale;
   int s16, s32;
   const uint32_t packed = ogm_quantize4<GROUP>(v, scale, s16, s32);
   if (active) {
     *(uint32_t *)(q + e0) = packed;
     if ((lane & 3u) == 0) sums[e0 / 16] = s16;
-    if ((lane & 7u) == 0) bsum[e0 / 32] = (int16_t)s32;
+    if ((lane & 7u) == 0) {
+      bsum[e0 / 32] = (int16_t)s32;
+      if (GROUP == 256 && bs16 != nullptr) {
+        // |s32| <= 32 * 127: floor(s32 / 64) and s32 mod 64 are exact in f16
+        uint16_t *b = bs16 + (e0 / 256u) * 16u + ((e0 / 32u) & 7u);
+        b[0] = __half_as_ushort(__float2half_rn((float)(s32 >> 6)));
+        b[8] = __half_as_ushort(__float2half_rn((float)(s32 & 63)));
+      }
+    }
     if ((lane & (GROUP / 4 - 1)) == 0) d[e0 / GROUP] = scale;
   }
 }
