@@ -844,7 +844,6 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
       const uint32_t tk0 = min(t0 + tw + l32, p.n_tokens - 1u) * p.nsb;
       const uint32_t tk1 = min(t0 + tw + 32u + l32, p.n_tokens - 1u) * p.nsb;
       const float side_scale = lh ? 1.0f : 64.0f;
-#pragma unroll 4
       for (uint32_t su = 0; su < p.nsb; su++) {
         const uint4 hd0 = *(const uint4 *)(p.wt + (ro0 + sb_tile(su) + sb_lane(su) * 16u));
         const half8 b20 = *(const half8 *)(p.bs16 + ((tk0 + su) * 16u + 8u * lh));
