@@ -381,6 +381,22 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
         be.set_tuning("gemm_q4k_variant", 0)
 
 
+def test_mfma_gemm_rows_too_long_for_the_plane_kernel(be):
+    """The Q4_K plane kernel keeps the tokens' scale of every super-block in LDS for the first pass;
+    rows beyond 128 super-blocks (32768 values) take the multiply-add int8 kernel instead, with the
+    same bits.  (Q5_K rows that long are outside what the GEMM path accepts at all: they go through
+    the multi-token GEMV.)"""
+    t, in_dim, out_dim, T = Q4_K, 33792, 40, 20
+    raw = synth_weights(t, in_dim, out_dim, seed=4)
+    x = synth_x(T, in_dim, seed=5)
+    got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
+    assert be.last_kernel() == "ogm_gemm_q4k_i8_kernel"
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "long rows")
+    got = be.matmul(x, T, qm(synth_weights(Q5_K, in_dim, out_dim, seed=6), Q5_K, in_dim, out_dim))
+    assert be.last_kernel().startswith("ogm_gemv_kernel")
+    assert_bits(got, oracle.matmul(Q5_K, synth_weights(Q5_K, in_dim, out_dim, seed=6), in_dim, out_dim, x, T), "long rows, Q5_K")
+
+
 @pytest.mark.parametrize("t,n_tokens,outs,kernel", [
     (Q4_K, 40, (300, 130, 64), "ogm_gemm_q4k_i8_kernel"),
     (Q4_K, 300, (520, 70), "ogm_gemm_q4k_i8_kernel"),
