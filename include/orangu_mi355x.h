@@ -325,7 +325,7 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
 
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.
  * keys: "gemv_wg_waves" (waves per workgroup of the GEMV kernel, 1..16; 0 = heuristic);
- * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default 9,
+ * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default 17,
  * below it the multi-token GEMV kernel runs in the GEMM's float order);
  * "gemm_q4k_variant" (K-quant GEMM: 0 = default, the int8 matrix-core kernels over scale-folded
  * weight planes; 1 = the same, always on 64-row tiles; 2 = the f16 kernels; 3 = for Q4_K and Q5_K the

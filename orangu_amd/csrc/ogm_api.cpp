@@ -44,7 +44,11 @@ struct ogm_ctx {
   DevBuf x, y, q, d, sums, bsum, bs16, isum, imin, xh;
   DevBuf hx, hy;  // pinned host staging
   int tune_wg_waves = 0;
-  int tune_gemm_min_tokens = 9;  // matmul at n_tokens >= this takes the MFMA GEMM
+  // matmul at n_tokens >= this takes the MFMA GEMM.  A GEMM launch costs about the same from 9 to 128
+  // tokens (its workgroups unpack every weight once whatever the tile holds), the GEMV kernel in
+  // chunks of 8 tokens grows with the count: they cross between 12 and 32 tokens depending on the
+  // shape (Q4_K 4096 -> 4096: 21 against 38 us at 16 tokens, 39 against 39 at 32).
+  int tune_gemm_min_tokens = 17;
   int tune_gemm_wide_min_wgs = 0;
   int tune_gemm_q4k_variant = 0;
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
@@ -210,7 +214,7 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   }
   if (strcmp(key, "gemm_min_tokens") == 0) {
     if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_min_tokens must be >= 0");
-    ctx->tune_gemm_min_tokens = value ? value : 9;
+    ctx->tune_gemm_min_tokens = value ? value : 17;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_wide_min_wgs") == 0) {

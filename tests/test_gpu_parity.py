@@ -22,11 +22,18 @@ def say(*a):
     sys.stdout.flush()
 
 
+# The library takes its matrix-core GEMMs from 17 tokens on (below that the GEMV kernel in chunks of 8
+# tokens is faster); these tests run them from 9 tokens on, so that tiles with 9, 10, 12 or 16 tokens
+# are covered too.  test_gemm_threshold_default checks the library's own choice.
+GEMM_FROM = 9
+
+
 @pytest.fixture(scope="module")
 def be():
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()  # raises if the HIP library or the device is missing: no fallback
     say("device:", b.device_name())
+    b.set_tuning("gemm_min_tokens", GEMM_FROM)
     yield b
     b.close()
 
@@ -381,6 +388,26 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
         be.set_tuning("gemm_q4k_variant", 0)
 
 
+def test_gemm_threshold_default():
+    """A context of its own with no tuning: 16 tokens go through the GEMV kernel in the GEMM's float
+    order, 17 through the matrix-core GEMM, with the same bits either way."""
+    from orangu_amd import Mi355xBackend
+    b = Mi355xBackend()
+    try:
+        raw = synth_weights(Q4_K, 1024, 70, seed=3)
+        x = synth_x(17, 1024, seed=4)
+        w = qm(raw, Q4_K, 1024, 70)
+        y16 = b.matmul(x[:16], 16, w)
+        assert b.last_kernel().startswith("ogm_gemv_kernel")
+        y17 = b.matmul(x, 17, w)
+        assert b.last_kernel().startswith("ogm_gemm_q4k_i8p")
+        want = oracle.matmul(Q4_K, raw, 1024, 70, x, 17)
+        assert_bits(y17, want, "17 tokens")
+        assert_bits(y16, want.reshape(17, 70)[:16], "16 tokens")
+    finally:
+        b.close()
+
+
 def test_mfma_gemm_rows_too_long_for_the_plane_kernel(be):
     """The Q4_K plane kernel keeps the tokens' scale of every super-block in LDS for the first pass;
     rows beyond 128 super-blocks (32768 values) take the multiply-add int8 kernel instead, with the
@@ -456,7 +483,7 @@ def test_mfma_gemm_equals_small_batch_kernel_and_is_batch_independent(be):
         small = be.matmul(x, 40, w).reshape(40, out_dim)
         assert be.last_kernel().startswith("ogm_gemv_kernel")
     finally:
-        be.set_tuning("gemm_min_tokens", 0)
+        be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(full, small, "mfma vs multi-token gemv")
     for n in (9, 17, 33):
         part = be.matmul(x[:n], n, w).reshape(n, out_dim)
@@ -537,7 +564,7 @@ def test_mfma_gemm_q6k_matches_cpu_gemm(be, in_dim, out_dim, T, variant):
         small = be.matmul(x, T, w)
         assert be.last_kernel().startswith("ogm_gemv_kernel")
     finally:
-        be.set_tuning("gemm_min_tokens", 0)
+        be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(got, small, "mfma vs multi-token gemv")
 
 
@@ -611,7 +638,7 @@ def test_mfma_gemm_q3k_q5k_match_cpu_gemm(be, t, kernel, in_dim, out_dim, T):
         small = be.matmul(x, T, w)
         assert be.last_kernel().startswith("ogm_gemv_kernel")
     finally:
-        be.set_tuning("gemm_min_tokens", 0)
+        be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(got, small, "mfma vs multi-token gemv")
 
 
@@ -954,7 +981,7 @@ def test_mfma_gemm_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T):
         small = be.matmul(x, T, w)
         assert be.last_kernel().startswith("ogm_gemv_kernel")
     finally:
-        be.set_tuning("gemm_min_tokens", 0)
+        be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(small, want, "multi-token gemv")
 
 
