@@ -325,12 +325,16 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
 
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.
  * keys: "gemv_wg_waves" (waves per workgroup of the GEMV kernel, 1..16; 0 = heuristic);
- * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default 17,
+ * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default: 9 for
+ * Q4_K, Q5_K and Q6_K, 17 for the other types;
  * below it the multi-token GEMV kernel runs in the GEMM's float order);
  * "gemm_q4k_variant" (K-quant GEMM: 0 = default, the int8 matrix-core kernels over scale-folded
  * weight planes; 1 = the same, always on 64-row tiles; 2 = the f16 kernels; 3 = for Q4_K and Q5_K the
  * int8 kernel that scales partial sums by multiply-adds);
  * "gemm_wide_min_wgs" (f16 Q4_K kernels: 128 x 128 workgroups from which the 128 x 256 tile runs; 0 = 256);
+ * "gemm_small_max_tokens" (K-quant GEMMs of at most this many tokens take the small-batch kernel, whose
+ * waves work on different super-blocks of the same rows; 0 = default 64, or 128 for matrices of up to
+ * 8192 rows; 1 = never);
  * "attn_prefill_variant" (attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the
  * decode step's kernel per token and chunk of the cache; they agree to f32 rounding, not bit for bit);
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);

@@ -44,13 +44,14 @@ struct ogm_ctx {
   DevBuf x, y, q, d, sums, bsum, bs16, isum, imin, xh;
   DevBuf hx, hy;  // pinned host staging
   int tune_wg_waves = 0;
-  // matmul at n_tokens >= this takes the MFMA GEMM.  A GEMM launch costs about the same from 9 to 128
-  // tokens (its workgroups unpack every weight once whatever the tile holds), the GEMV kernel in
-  // chunks of 8 tokens grows with the count: they cross between 12 and 32 tokens depending on the
-  // shape (Q4_K 4096 -> 4096: 21 against 38 us at 16 tokens, 39 against 39 at 32).
-  int tune_gemm_min_tokens = 17;
+  // matmul at n_tokens >= this takes the MFMA GEMM; 0 = by type: 9 for Q4_K, Q5_K and Q6_K, whose
+  // small-batch kernel beats the GEMV kernel's chunks of 8 tokens from there on (Q4_K 4096 -> 4096 at 9
+  // tokens: 12 against 16 us), 17 for the others, whose tiled kernels cost about the same from 9 to 128
+  // tokens while the chunked GEMV grows with the count (they cross between 12 and 32 tokens).
+  int tune_gemm_min_tokens = 0;
   int tune_gemm_wide_min_wgs = 0;
   int tune_gemm_q4k_variant = 0;
+  int tune_gemm_small_max = 0;   // most tokens for the small-batch GEMM kernel: 0 = default, 1 = never
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
@@ -214,12 +215,17 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   }
   if (strcmp(key, "gemm_min_tokens") == 0) {
     if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_min_tokens must be >= 0");
-    ctx->tune_gemm_min_tokens = value ? value : 17;
+    ctx->tune_gemm_min_tokens = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_wide_min_wgs") == 0) {
     if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_wide_min_wgs must be >= 0");
     ctx->tune_gemm_wide_min_wgs = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_small_max_tokens") == 0) {
+    if (value < 0 || value > 1024) return fail(ctx, OGM_ERR_INVALID, "gemm_small_max_tokens must be 0..1024");
+    ctx->tune_gemm_small_max = value;
     return OGM_OK;
   }
   if (strcmp(key, "attn_prefill_variant") == 0) {
@@ -415,7 +421,10 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
   // n_tokens == 1 and every matmul_decode take the GEMV's.
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
-  if (gemm_order && !dump_isum && !dump_imin && n_tokens >= (uint32_t)ctx->tune_gemm_min_tokens &&
+  const uint32_t t0 = w0->ggml_type;
+  const uint32_t gemm_from = ctx->tune_gemm_min_tokens ? (uint32_t)ctx->tune_gemm_min_tokens
+                             : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 9u : 17u;
+  if (gemm_order && !dump_isum && !dump_imin && n_tokens >= gemm_from &&
       all_gemm_supported(tg, n_tg, n_tokens)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
     int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w0->in_dim, n_tokens));
@@ -435,6 +444,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.xh = ctx->xh.p;
       g.wide_min_wgs = (uint32_t)ctx->tune_gemm_wide_min_wgs;
       g.q4k_variant = (uint32_t)ctx->tune_gemm_q4k_variant;
+      g.small_max_tokens = (uint32_t)ctx->tune_gemm_small_max;
       g.n_extra = (uint32_t)ng - 1;
       for (size_t j = 1; j < ng; j++) {
         g.extra_wt[j - 1] = tg[i + j].w->dev;

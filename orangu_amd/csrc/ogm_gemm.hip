@@ -1159,6 +1159,356 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q5k_i8p_kernel(GemmI8pParams p)
 __global__ __launch_bounds__(512) void ogm_gemm_q5k_i8p_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q5K>(p); }
 
 // ------------------------------------------------------------------------------------------
+// Small batches (up to a few dozen tokens): the tiled kernels above cost the same for 9 tokens as
+// for 128, because a workgroup walks its rows' super-blocks one after the other.  Here a workgroup
+// owns 32 rows x 32 tokens and its eight waves take different super-blocks of those rows at the same
+// time, each unpacking the weights straight into the matrix instruction's operand registers (a
+// lane's operand is 16 consecutive weights of one row) and reading the int8 activations from
+// memory as they are.  A super-block's contribution ad * (d * isum) does not depend on the others;
+// only the additions are ordered, so the waves leave their terms in LDS and after every round of
+// eight super-blocks the terms are added in ascending order, as gemm_k_q6_k does
+// (vecdot.rs:2352-2398).  The chain of a workgroup is nsb / 8 rounds long instead of 4 nsb stages.
+
+struct GemmSbParams {
+  const uint8_t *wt;      // tile-planar weights
+  const int8_t *xq;       // [T][in_dim] int8 activations
+  const float *ad;        // [T][nsb]
+  const _Float16 *bs16;   // Q4_K / Q5_K: the quantizer's sums per 32 as (bsum / 64, bsum % 64) in f16
+  float *y;               // [T][out_dim]
+  uint32_t in_dim, out_dim, n_tokens, nsb;
+  uint32_t c_shift, r_shift, nct;
+  uint32_t n_extra;
+  const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1];
+  float *extra_y[OGM_GEMM_MAX_MATS - 1];
+  uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
+};
+
+__global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) {
+  constexpr uint32_t TILE_BYTES = 13440u;
+  extern __shared__ __align__(16) uint8_t sb_lds[];
+  float *terms = (float *)sb_lds;            // [8 waves][32 tokens][32 rows]
+  float *ad_l = terms + 8u * 32u * 32u;      // [nsb][32 tokens]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  uint32_t row_tile = blockIdx.y;
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + 31u) / 32u;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = blockIdx.x * 32u, r0 = row_tile * 32u;
+  uint32_t uo, to;   // this lane's row: its 16-byte pieces (the upper lane half: the next piece) and its tail
+  {
+    const uint32_t row = min(r0 + l32, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    uo = rb * p.nct * TILE_BYTES + r * 16u + lh * 1024u;
+    to = rb * p.nct * TILE_BYTES + 13u * 1024u + r * 2u;
+  }
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
+  };
+  auto sb_tail = [&](uint32_t s) -> uint32_t {
+    return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 2u;
+  };
+  const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + 256 s + 32 sub
+  const uint32_t sc_shift = 8u * lh;
+
+  // the tokens' ad of every super-block: ad_l[s][token]
+  for (uint32_t i = tid; i < 32u * p.nsb; i += 512u) {
+    const uint32_t k = i / p.nsb, s = i - k * p.nsb;
+    ad_l[s * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + s];
+  }
+
+  uint4 wA0, wB0, wQ0, wA1, wB1, wQ1, scw;
+  uint32_t d16;
+#define SB_LOADW(S)                                                                               \
+  do {                                                                                            \
+    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded, never used */    \
+    const uint32_t so_ = uo + sb_off(s_);                                                         \
+    wA0 = *(const uint4 *)(p.wt + so_);                                                           \
+    wB0 = *(const uint4 *)(p.wt + (so_ + 2u * 1024u));                                            \
+    wA1 = *(const uint4 *)(p.wt + (so_ + 4u * 1024u));                                            \
+    wB1 = *(const uint4 *)(p.wt + (so_ + 6u * 1024u));                                            \
+    wQ0 = *(const uint4 *)(p.wt + (so_ + 8u * 1024u));                                            \
+    wQ1 = *(const uint4 *)(p.wt + (so_ + 10u * 1024u));                                           \
+    scw = *(const uint4 *)(p.wt + (so_ - lh * 1024u + 12u * 1024u));                              \
+    d16 = *(const uint16_t *)(p.wt + (to + sb_tail(s_)));                                         \
+  } while (0)
+  // 16 weights of run 2 (G % 2) + SUB of a half block -> the two operand planes: u = sc * q +
+  // (128 - 32 sc) as a 16-bit lane, high byte h, low byte with its top bit flipped l
+#define SB_UNPACK(DH, DL, QL, QH, SCW, G, SUB)                                                    \
+  do {                                                                                            \
+    const int sc_ = __builtin_amdgcn_sbfe((int)(SCW), sc_shift + 16u * (SUB), 8u);                \
+    const short2v sc2_ = {(short)sc_, (short)sc_};                                                \
+    const short2v c2_ = {(short)(128 - 32 * sc_), (short)(128 - 32 * sc_)};                       \
+    constexpr uint32_t rr_ = 2u * ((G) & 1u) + (SUB);                                             \
+    const uint32_t qlw_[4] = {QL.x, QL.y, QL.z, QL.w}, qhw_[4] = {QH.x, QH.y, QH.z, QH.w};        \
+    uint32_t ph_[4], pl_[4];                                                                      \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      const uint32_t nib_ = (((G) & 1u) ? (qlw_[w_] >> 4) : qlw_[w_]) & 0x0F0F0F0Fu;              \
+      const uint32_t hi_ = rr_ < 2u ? (qhw_[w_] << (4u - 2u * rr_)) : (qhw_[w_] >> (2u * rr_ - 4u)); \
+      const uint32_t v_ = (hi_ & 0x30303030u) | nib_;                                             \
+      union { uint32_t u; short2v s; } e_, f_;                                                    \
+      e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
+      f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
+      e_.s = e_.s * sc2_ + c2_;                                                                   \
+      f_.s = f_.s * sc2_ + c2_;                                                                   \
+      ph_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x07050301u);                                   \
+      pl_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u) ^ 0x80808080u;                     \
+    }                                                                                             \
+    DH = (int4v){(int)ph_[0], (int)ph_[1], (int)ph_[2], (int)ph_[3]};                             \
+    DL = (int4v){(int)pl_[0], (int)pl_[1], (int)pl_[2], (int)pl_[3]};                             \
+  } while (0)
+#define SB_STEP(QL, QH, SCW, G, SUB, FIRST)                                                       \
+  do {                                                                                            \
+    int4v bh_, bl_;                                                                               \
+    SB_UNPACK(bh_, bl_, QL, QH, SCW, G, SUB);                                                     \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 64u * (G) + 32u * (SUB)));                   \
+    H = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bh_, (FIRST) ? zi : H, 0, 0, 0);               \
+    L = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bl_, (FIRST) ? zi : L, 0, 0, 0);               \
+  } while (0)
+
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  float acc0 = 0.0f, acc1 = 0.0f;   // outputs (token, row) = (tid / 32, tid % 32) and (tid / 32 + 16, tid % 32)
+  SB_LOADW(wave);
+  __syncthreads();   // ad_l
+  for (uint32_t s0 = 0; s0 < p.nsb; s0 += 8u) {
+    const uint32_t s = s0 + wave;
+    if (s < p.nsb) {   // wave-uniform
+      const uint32_t xs_ = xro + 256u * s;
+      int16v H, L;
+      SB_STEP(wA0, wQ0, scw.x, 0, 0, true);
+      SB_STEP(wB0, wQ0, scw.x, 0, 1, false);
+      SB_STEP(wA0, wQ0, scw.y, 1, 0, false);
+      SB_STEP(wB0, wQ0, scw.y, 1, 1, false);
+      SB_STEP(wA1, wQ1, scw.z, 2, 0, false);
+      SB_STEP(wB1, wQ1, scw.z, 2, 1, false);
+      SB_STEP(wA1, wQ1, scw.w, 3, 0, false);
+      SB_STEP(wB1, wQ1, scw.w, 3, 1, false);
+      const float d = gm_f16_bits_to_f32(d16);
+      const float *adp = &ad_l[s * 32u + 4u * lh];
+      float *tp = terms + (wave * 32u + 4u * lh) * 32u + l32;   // [wave][token][row]
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const float4 a4 = *(const float4 *)(adp + 8 * q4);
+        const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int is_ = H[4 * q4 + e] * 256 + L[4 * q4 + e];
+          tp[(8 * q4 + e) * 32] = a4v[e] * (d * (float)is_);
+        }
+      }
+    }
+    SB_LOADW(s + 8u);   // the next round's weights, in flight over the barrier and the additions
+    __syncthreads();
+    {
+      const uint32_t n_here = min(8u, p.nsb - s0);
+      for (uint32_t w = 0; w < n_here; w++) {   // ascending super-blocks, one accumulator per output
+        acc0 += terms[w * 1024u + tid];
+        acc1 += terms[w * 1024u + 512u + tid];
+      }
+    }
+    __syncthreads();
+  }
+#undef SB_LOADW
+#undef SB_UNPACK
+#undef SB_STEP
+  {
+    const uint32_t tok = t0 + (tid >> 5), row = r0 + (tid & 31u);
+    if (row < p.out_dim) {
+      if (tok < p.n_tokens) p.y[(size_t)tok * p.out_dim + row] = acc0;
+      if (tok + 16u < p.n_tokens) p.y[(size_t)(tok + 16u) * p.out_dim + row] = acc1;
+    }
+  }
+}
+
+// The same for Q4_K and Q5_K (gemm_k_q4_k, vecdot.rs:2213-2303): first a sweep over the super-blocks
+// for the terms (ad * dmin) * imin, which the reference subtracts before anything else (rounds of
+// sixteen super-blocks, two per wave: header and the quantizer's sums per 32 only, one f16 matrix
+// instruction each), then the sweep of the products as above.  A lane's 16 weights of sub-block j
+// are the low (j even) or high nibbles of one 16-byte piece of qs, Q5_K's fifth bit is bit j of
+// its piece of qh; u = sc_j * q + 128 splits into the two int8 planes.
+template <bool Q5>
+__global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
+  constexpr uint32_t TILE_BYTES = Q5 ? 11264u : 9216u;
+  constexpr uint32_t QS_PIECE0 = Q5 ? 3u : 1u;
+  extern __shared__ __align__(16) uint8_t sb_lds[];
+  float *terms = (float *)sb_lds;             // [16 super-blocks][32 tokens][32 rows] (second sweep: 8)
+  float *ad_l = terms + 16u * 32u * 32u;      // [nsb][32 tokens]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  uint32_t row_tile = blockIdx.y;
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + 31u) / 32u;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = blockIdx.x * 32u, r0 = row_tile * 32u;
+  uint32_t uo;   // this lane's row: its header piece
+  {
+    const uint32_t row = min(r0 + l32, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    uo = rb * p.nct * TILE_BYTES + r * 16u;
+  }
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
+  };
+  const uint32_t tok = min(t0 + l32, p.n_tokens - 1u);
+  const uint32_t xro = tok * p.in_dim + 16u * lh;   // + 256 s + 32 j
+  const uint32_t tk = tok * p.nsb;
+
+  for (uint32_t i = tid; i < 32u * p.nsb; i += 512u) {
+    const uint32_t k = i / p.nsb, s = i - k * p.nsb;
+    ad_l[s * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + s];
+  }
+  __syncthreads();
+
+  float acc0 = 0.0f, acc1 = 0.0f;   // outputs (token, row) = (tid / 32, tid % 32) and (tid / 32 + 16, tid % 32)
+  // ---- first sweep: acc -= (ad * dmin) * sum_j m_j * bsum_j
+  {
+    float16v zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.0f;
+    const float side_scale = lh ? 1.0f : 64.0f;
+    for (uint32_t s0 = 0; s0 < p.nsb; s0 += 16u) {
+#pragma unroll
+      for (uint32_t u = 0; u < 2u; u++) {
+        const uint32_t sl = wave + 8u * u, s = s0 + sl;
+        if (s < p.nsb) {   // wave-uniform
+          const uint4 hd = *(const uint4 *)(p.wt + (uo + sb_off(s)));
+          const half8 b2 = *(const half8 *)(p.bs16 + ((tk + s) * 16u + 8u * lh));
+          uint32_t mna, mnb;
+          q4k_mins(hd, mna, mnb);
+          const half8 a1 = side_operand(mna, mnb, side_scale);
+          const float dm = gm_f16_bits_to_f32(hd.x >> 16);
+          const float16v im = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2, a1, zero, 0, 0, 0);
+          const float *adp = &ad_l[s * 32u + 4u * lh];
+          float *tp = terms + (sl * 32u + 4u * lh) * 32u + l32;   // [super-block][token][row]
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++) {
+            const float4 a4 = *(const float4 *)(adp + 8 * q4);
+            const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) tp[(8 * q4 + e) * 32] = a4v[e] * dm * im[4 * q4 + e];
+          }
+        }
+      }
+      __syncthreads();
+      const uint32_t n_here = min(16u, p.nsb - s0);
+      for (uint32_t w = 0; w < n_here; w++) {
+        acc0 -= terms[w * 1024u + tid];
+        acc1 -= terms[w * 1024u + 512u + tid];
+      }
+      __syncthreads();
+    }
+  }
+  // ---- second sweep: acc += ad * (d * sum_j sc_j * dot32_j)
+  uint4 hdr, w0, w1, w2, w3, qh5 = make_uint4(0, 0, 0, 0);
+#define SB_LOADW(S)                                                                               \
+  do {                                                                                            \
+    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded, never used */    \
+    const uint32_t so_ = uo + sb_off(s_);                                                         \
+    hdr = *(const uint4 *)(p.wt + so_);                                                           \
+    w0 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 0u + lh) * 1024u));                          \
+    w1 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 2u + lh) * 1024u));                          \
+    w2 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 4u + lh) * 1024u));                          \
+    w3 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 6u + lh) * 1024u));                          \
+    if constexpr (Q5) qh5 = *(const uint4 *)(p.wt + (so_ + (1u + lh) * 1024u));                   \
+  } while (0)
+#define SB_STEP(QS, J, FIRST)                                                                     \
+  do {                                                                                            \
+    const int sc_ = (int)((((J) < 4 ? sca_ : scb_) >> (8u * ((J) & 3u))) & 0xFFu);                \
+    const short2v sc2_ = {(short)sc_, (short)sc_};                                                \
+    const short2v c2_ = {128, 128};                                                               \
+    const uint32_t qsw_[4] = {QS.x, QS.y, QS.z, QS.w}, q5w_[4] = {qh5.x, qh5.y, qh5.z, qh5.w};    \
+    uint32_t ph_[4], pl_[4];                                                                      \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      uint32_t v_ = (((J) & 1) ? (qsw_[w_] >> 4) : qsw_[w_]) & 0x0F0F0F0Fu;                       \
+      if constexpr (Q5) v_ |= ((q5w_[w_] >> (J)) & 0x01010101u) << 4;                             \
+      union { uint32_t u; short2v s; } e_, f_;                                                    \
+      e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
+      f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
+      e_.s = e_.s * sc2_ + c2_;                                                                   \
+      f_.s = f_.s * sc2_ + c2_;                                                                   \
+      ph_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x07050301u);                                   \
+      pl_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u) ^ 0x80808080u;                     \
+    }                                                                                             \
+    const int4v bh_ = {(int)ph_[0], (int)ph_[1], (int)ph_[2], (int)ph_[3]};                       \
+    const int4v bl_ = {(int)pl_[0], (int)pl_[1], (int)pl_[2], (int)pl_[3]};                       \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 32u * (J)));                                 \
+    H = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bh_, (FIRST) ? zi : H, 0, 0, 0);               \
+    L = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bl_, (FIRST) ? zi : L, 0, 0, 0);               \
+  } while (0)
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  SB_LOADW(wave);
+  for (uint32_t s0 = 0; s0 < p.nsb; s0 += 8u) {
+    const uint32_t s = s0 + wave;
+    if (s < p.nsb) {   // wave-uniform
+      const uint32_t xs_ = xro + 256u * s;
+      uint32_t sca_, scb_;
+      q4k_scales(hdr, sca_, scb_);
+      int16v H, L;
+      SB_STEP(w0, 0, true);
+      SB_STEP(w0, 1, false);
+      SB_STEP(w1, 2, false);
+      SB_STEP(w1, 3, false);
+      SB_STEP(w2, 4, false);
+      SB_STEP(w2, 5, false);
+      SB_STEP(w3, 6, false);
+      SB_STEP(w3, 7, false);
+      const float d = gm_f16_bits_to_f32(hdr.x & 0xFFFFu);
+      const float *adp = &ad_l[s * 32u + 4u * lh];
+      float *tp = terms + (wave * 32u + 4u * lh) * 32u + l32;   // [wave][token][row]
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const float4 a4 = *(const float4 *)(adp + 8 * q4);
+        const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int is_ = H[4 * q4 + e] * 256 + L[4 * q4 + e];
+          tp[(8 * q4 + e) * 32] = a4v[e] * (d * (float)is_);
+        }
+      }
+    }
+    SB_LOADW(s + 8u);   // the next round's weights, in flight over the barrier and the additions
+    __syncthreads();
+    {
+      const uint32_t n_here = min(8u, p.nsb - s0);
+      for (uint32_t w = 0; w < n_here; w++) {   // ascending super-blocks, one accumulator per output
+        acc0 += terms[w * 1024u + tid];
+        acc1 += terms[w * 1024u + 512u + tid];
+      }
+    }
+    __syncthreads();
+  }
+#undef SB_LOADW
+#undef SB_STEP
+  {
+    const uint32_t tok_o = t0 + (tid >> 5), row = r0 + (tid & 31u);
+    if (row < p.out_dim) {
+      if (tok_o < p.n_tokens) p.y[(size_t)tok_o * p.out_dim + row] = acc0;
+      if (tok_o + 16u < p.n_tokens) p.y[(size_t)(tok_o + 16u) * p.out_dim + row] = acc1;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
 //
 // The 128 x 128 kernel above is bound by LDS bandwidth: a multiplying wave reads (64 + 32) k-rows
@@ -2234,6 +2584,51 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       hipLaunchKernelGGL(ogm_gemm_q5k_i8_kernel, grid, dim3(768), 0, stream, p);
       if (kernel_name) *kernel_name = "ogm_gemm_q5k_i8_kernel";
     }
+    return hipGetLastError();
+  }
+  // Small batches: the kernel whose waves take different super-blocks.  By default up to 64 tokens
+  // (Q4_K 4096 -> 14336: 18 / 35 / 50 us at 32 / 64 / 96 tokens against 42-45 us tiled), and up to 128
+  // when the tiled kernel's grid would leave half the CUs idle (4096 -> 4096: 12 / 15 / 21 us at 32 /
+  // 64 / 128 tokens against 38-41; 14336 -> 4096: 36 / 39 / 57 against 123-130).
+  uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
+  for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
+  const uint32_t small_max = a.small_max_tokens ? a.small_max_tokens : (tiles64_all <= 128u ? 128u : 64u);
+  if (i8p && a.ggml_type != OGM_Q3_K && a.small_max_tokens != 1u && a.n_tokens <= small_max &&
+      (q45 ? 16u : 8u) * 4096u + 128u * nsb <= GM_LDS_MAX) {
+    GemmSbParams p;
+    p.wt = a.wt;
+    p.xq = a.act.q;
+    p.ad = a.act.d;
+    p.bs16 = bs16;
+    p.y = a.y;
+    p.in_dim = a.in_dim;
+    p.out_dim = a.out_dim;
+    p.n_tokens = a.n_tokens;
+    p.nsb = nsb;
+    p.c_shift = c_shift;
+    p.r_shift = 6 - c_shift;
+    p.nct = tl.nct;
+    p.n_extra = a.n_extra;
+    uint32_t tiles = (a.out_dim + 31u) / 32u;
+    for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
+      p.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
+      p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
+      p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
+      if (m < a.n_extra) tiles += (a.extra_out_dim[m] + 31u) / 32u;
+    }
+    const uint32_t lds_bytes = (q45 ? 16u : 8u) * 4096u + 128u * nsb;
+    const void *fn = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_sb_q6k_kernel
+                     : a.ggml_type == OGM_Q4_K ? (const void *)ogm_gemm_sb_q45k_kernel<false>
+                                               : (const void *)ogm_gemm_sb_q45k_kernel<true>;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    void *kargs[] = {(void *)&p};
+    e = hipLaunchKernel(fn, dim3((a.n_tokens + 31u) / 32u, tiles), dim3(512), kargs, lds_bytes, stream);
+    if (e != hipSuccess) return e;
+    if (kernel_name)
+      *kernel_name = a.ggml_type == OGM_Q6_K   ? "ogm_gemm_sb_q6k_kernel"
+                     : a.ggml_type == OGM_Q4_K ? "ogm_gemm_sb_q4k_kernel"
+                                               : "ogm_gemm_sb_q5k_kernel";
     return hipGetLastError();
   }
   if (i8p) {

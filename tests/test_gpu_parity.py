@@ -22,9 +22,11 @@ def say(*a):
     sys.stdout.flush()
 
 
-# The library takes its matrix-core GEMMs from 17 tokens on (below that the GEMV kernel in chunks of 8
-# tokens is faster); these tests run them from 9 tokens on, so that tiles with 9, 10, 12 or 16 tokens
-# are covered too.  test_gemm_threshold_default checks the library's own choice.
+# The library takes its tiled matrix-core GEMMs from 17 tokens on (below that the GEMV kernel in chunks
+# of 8 tokens is faster) and gives batches of up to 64 or 128 tokens of Q4_K, Q5_K and Q6_K to a
+# small-batch kernel; these tests run the tiled kernels from 9 tokens on and keep the small-batch
+# kernel out, so that tiles with 9, 10, 12 or 16 tokens are covered too.  The small-batch kernel has
+# tests of its own, and test_gemm_threshold_default checks the library's own choices.
 GEMM_FROM = 9
 
 
@@ -34,6 +36,7 @@ def be():
     b = Mi355xBackend()  # raises if the HIP library or the device is missing: no fallback
     say("device:", b.device_name())
     b.set_tuning("gemm_min_tokens", GEMM_FROM)
+    b.set_tuning("gemm_small_max_tokens", 1)
     yield b
     b.close()
 
@@ -338,7 +341,7 @@ def plane_kernel(base, T, outs):
 def variant_of(kernel):
     """gemm_q4k_variant that makes the launcher pick `kernel`: 0 the plane kernels (default), 3 the
     multiply-add int8 kernels of Q4_K / Q5_K, 2 the f16 kernels."""
-    if "_i8p_" in kernel or kernel.startswith(("ogm_gemm_q6k_i8", "ogm_gemm_q3k_i8")):
+    if "_i8p_" in kernel or "_sb_" in kernel or kernel.startswith(("ogm_gemm_q6k_i8", "ogm_gemm_q3k_i8")):
         return 0
     return 3 if kernel.endswith("_i8_kernel") else 2
 
@@ -389,23 +392,84 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
 
 
 def test_gemm_threshold_default():
-    """A context of its own with no tuning: 16 tokens go through the GEMV kernel in the GEMM's float
-    order, 17 through the matrix-core GEMM, with the same bits either way."""
+    """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
+    float order, 17 through the matrix-core GEMM.  Q4_K: 8 tokens through the GEMV kernel, 9 and 128
+    through the small-batch kernel (a matrix of few rows), 129 through the tiled one; a matrix of
+    many rows leaves the small-batch kernel after 64 tokens.  Same bits everywhere."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
     try:
-        raw = synth_weights(Q4_K, 1024, 70, seed=3)
-        x = synth_x(17, 1024, seed=4)
-        w = qm(raw, Q4_K, 1024, 70)
+        raw = synth_weights(Q8_0, 1024, 70, seed=3)
+        x = synth_x(129, 1024, seed=4)
+        w = qm(raw, Q8_0, 1024, 70)
+        want = oracle.matmul(Q8_0, raw, 1024, 70, x[:17], 17).reshape(17, 70)
         y16 = b.matmul(x[:16], 16, w)
         assert b.last_kernel().startswith("ogm_gemv_kernel")
-        y17 = b.matmul(x, 17, w)
-        assert b.last_kernel().startswith("ogm_gemm_q4k_i8p")
-        want = oracle.matmul(Q4_K, raw, 1024, 70, x, 17)
-        assert_bits(y17, want, "17 tokens")
-        assert_bits(y16, want.reshape(17, 70)[:16], "16 tokens")
+        y17 = b.matmul(x[:17], 17, w)
+        assert b.last_kernel() == "ogm_gemm_flat_kernel"
+        assert_bits(y17, want, "Q8_0, 17 tokens")
+        assert_bits(y16, want[:16], "Q8_0, 16 tokens")
+        raw = synth_weights(Q4_K, 1024, 70, seed=5)
+        w = qm(raw, Q4_K, 1024, 70)
+        want = oracle.matmul(Q4_K, raw, 1024, 70, x, 129).reshape(129, 70)
+        for n, kernel in ((8, "ogm_gemv_kernel"), (9, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
+                          (129, "ogm_gemm_q4k_i8p_r64_kernel")):
+            y = b.matmul(x[:n], n, w)
+            assert b.last_kernel().startswith(kernel), (n, b.last_kernel())
+            assert_bits(y, want[:n], f"Q4_K, {n} tokens")
+        raw = synth_weights(Q6_K, 256, 8300, seed=6)   # 130 tiles of 64 rows
+        w = qm(raw, Q6_K, 256, 8300)
+        want = oracle.matmul(Q6_K, raw, 256, 8300, np.ascontiguousarray(x[:65, :256]), 65).reshape(65, 8300)
+        for n, kernel in ((64, "ogm_gemm_sb_q6k_kernel"), (65, "ogm_gemm_q6k_i8_r64_kernel")):
+            y = b.matmul(np.ascontiguousarray(x[:n, :256]), n, w)
+            assert b.last_kernel() == kernel, (n, b.last_kernel())
+            assert_bits(y, want[:n], f"Q6_K, {n} tokens")
     finally:
         b.close()
+
+
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("in_dim,out_dim,T", [
+    (256, 5, 9), (1024, 100, 17), (768, 64, 32), (1280, 257, 40), (2048, 37, 64), (14336, 96, 33), (1792, 33, 10),
+    (4096, 300, 20), (512, 31, 63), (2304, 130, 100), (1024, 70, 128), (256, 1, 1000),
+])
+def test_small_batch_gemm_matches_cpu_gemm(be, t, in_dim, out_dim, T):
+    """The small-batch kernel of the K-quants (a workgroup's eight waves on different super-blocks of
+    32 rows x 32 tokens, terms added in ascending order afterwards): every bit of gemm_k_q4_k /
+    gemm_k_q6_k (vecdot.rs:2213-2303, 2352-2398), at any token count it is asked for."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T + 2)
+    be.set_tuning("gemm_small_max_tokens", 1024)
+    try:
+        got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
+    finally:
+        be.set_tuning("gemm_small_max_tokens", 1)
+    assert be.last_kernel() == {Q4_K: "ogm_gemm_sb_q4k_kernel", Q5_K: "ogm_gemm_sb_q5k_kernel", Q6_K: "ogm_gemm_sb_q6k_kernel"}[t]
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "small-batch gemm")
+
+
+@pytest.mark.parametrize("t,block,hi", [(Q4_K, 144, 0xFF), (Q5_K, 176, 0xFF), (Q6_K, 210, 0x7F), (Q6_K, 210, 0x80)])
+def test_small_batch_gemm_extreme_integer_ranges(be, t, block, hi):
+    """Every weight bit and scale byte at its extreme (Q6_K: scales +127 and -128), activations +-127."""
+    in_dim, out_dim, T = 1024, 40, 24
+    blocks = np.full((out_dim * 4, block), 0xFF, np.uint8)
+    if t == Q6_K:
+        blocks[:, 192:208] = hi
+        blocks[:, 208:210] = np.frombuffer(np.float16(0.003).tobytes(), np.uint8)
+    else:
+        blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+        blocks[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
+    x = np.full((T, in_dim), 127.0, np.float32)
+    x[1::2] *= -1
+    x[:, ::7] = 126.0
+    raw = blocks.reshape(-1)
+    be.set_tuning("gemm_small_max_tokens", 1024)
+    try:
+        got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
+    finally:
+        be.set_tuning("gemm_small_max_tokens", 1)
+    assert be.last_kernel().startswith("ogm_gemm_sb_")
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "extreme ranges")
 
 
 def test_mfma_gemm_rows_too_long_for_the_plane_kernel(be):
@@ -442,6 +506,9 @@ def test_mfma_gemm_rows_too_long_for_the_plane_kernel(be):
     (Q3_K, 40, (128, 300), "ogm_gemm_q3k_kernel"),
     (Q3_K, 140, (128, 300, 70), "ogm_gemm_q3k_i8_r64_kernel"),
     (Q3_K, 300, (6000, 3000, 2100), "ogm_gemm_q3k_i8_kernel"),
+    (Q4_K, 40, (300, 130, 64), "ogm_gemm_sb_q4k_kernel"),
+    (Q5_K, 20, (520, 70, 129), "ogm_gemm_sb_q5k_kernel"),
+    (Q6_K, 33, (300, 31), "ogm_gemm_sb_q6k_kernel"),
 ])
 def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, outs, kernel):
     """q / k / v (llama.rs:730-746) at prefill widths: K-quant matrices of one type over the same
@@ -455,10 +522,12 @@ def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, ou
     xd = DeviceBuffer.from_numpy(x)
     yds = [DeviceBuffer(4 * n_tokens * od) for od in outs]
     be.set_tuning("gemm_q4k_variant", variant_of(kernel))
+    be.set_tuning("gemm_small_max_tokens", 1024 if "_sb_" in kernel else 1)
     try:
         be.matmul_multi_dev(hs, xd.ptr, n_tokens, [y.ptr for y in yds])
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
+        be.set_tuning("gemm_small_max_tokens", 1)
     device_synchronize()
     assert be.last_kernel() == kernel
     for r, od, yd in zip(raws, outs, yds):
