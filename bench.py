@@ -244,6 +244,8 @@ def main() -> int:
     ap.add_argument("--only-decode", action="store_true", help="run only the decode leg (for rocprofv3)")
     ap.add_argument("--only-prefill", type=int, default=0, metavar="N",
                     help="run only prefills of N tokens on the decode leg's model (for rocprofv3)")
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="a kernel choice of ogm_set_tuning for this run (repeatable), e.g. gemm_small_max_tokens=1")
     ap.add_argument("--sweep", action="store_true",
                     help="time every benchmark configuration's kernels instead (one JSON object, not the "
                          "headline line)")
@@ -261,6 +263,9 @@ def main() -> int:
     from orangu_amd import hiprt
 
     be = Mi355xBackend()  # raises without the HIP library or a gfx950 device
+    for kv in args.tune:
+        key, _, value = kv.partition("=")
+        be.set_tuning(key, int(value))
     if args.sweep:
         print(json.dumps(sweep(be, helpers, hiprt)))
         be.close()
