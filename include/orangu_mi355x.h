@@ -339,7 +339,10 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * decode step's kernel per token and chunk of the cache; they agree to f32 rounding, not bit for bit);
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
- * the quantizer kernel first; 0 or -1 = default, off).  No other setting changes a result bit. */
+ * the quantizer kernel first; 0 or -1 = default, off);
+ * "decode_fuse_tails" (1: the decode step's FFN norm, SwiGLU and next attention norm run inside the
+ * GEMV launch before them, in its last workgroup to finish; 0 = default, kernels of their own, which
+ * is faster; same bits).  No other setting changes a result bit. */
 int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value);
 /* Name of the kernel the last matmul on this context launched (for profiles). */
 const char *ogm_last_kernel(ogm_ctx *ctx);

@@ -52,6 +52,7 @@ struct ogm_ctx {
   int tune_gemm_wide_min_wgs = 0;
   int tune_gemm_q4k_variant = 0;
   int tune_gemm_small_max = 0;   // most tokens for the small-batch GEMM kernel: 0 = default, 1 = never
+  int tune_decode_fuse_tails = 0;      // 1: the decode step's norms and SwiGLU inside the GEMV before them (slower)
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
@@ -228,6 +229,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_gemm_small_max = value;
     return OGM_OK;
   }
+  if (strcmp(key, "decode_fuse_tails") == 0) {
+    if (value < 0 || value > 1) return fail(ctx, OGM_ERR_INVALID, "decode_fuse_tails must be 0 or 1");
+    ctx->tune_decode_fuse_tails = value;
+    return OGM_OK;
+  }
   if (strcmp(key, "attn_prefill_variant") == 0) {
     if (value < 0 || value > 1) return fail(ctx, OGM_ERR_INVALID, "attn_prefill_variant must be 0 or 1");
     ctx->tune_attn_prefill_variant = value;
@@ -376,7 +382,7 @@ struct Target {
 
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
                         hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
-                        const float *x_f32);
+                        const float *x_f32, const OgmGemvTail *tail = nullptr);
 
 // Whether a single-token launch quantizes inside the GEMV (every workgroup repeats the
 // quantizer on its way in) instead of running the quantizer kernel first.  Off unless asked
@@ -415,8 +421,9 @@ static bool all_gemm_supported(const Target *tg, size_t n_tg, uint32_t n_tokens)
 // one token of f32 activations that the kernel quantizes itself).  Caller holds the lock.
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
                         hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
-                        const float *x_f32) {
+                        const float *x_f32, const OgmGemvTail *tail) {
   const ogm_weight *w0 = tg[0].w;
+  if (tail && (n_tokens != 1 || n_tg > OGM_GEMV_MAX_MATS)) return fail(ctx, OGM_ERR_INVALID, "a GEMV tail needs one launch of one token");
   const int mode = act_mode_for(w0->ggml_type);
   // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
   // n_tokens == 1 and every matmul_decode take the GEMV's.
@@ -482,6 +489,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
         a.extra_y[i - 1] = tg[g0 + i].y + (size_t)t0 * tg[g0 + i].w->out_dim;
       }
       a.x_f32 = x_f32;
+      if (tail) a.tail = *tail;
       HIPCHK(ctx, ogm_launch_gemv(a, stream, &ctx->last_kernel));
     }
   }
@@ -782,7 +790,7 @@ struct ogm_llama {
   float *pre = nullptr;       // [n_layer][q_bias qd | k_bias kvd | v_bias kvd | q_norm hd | k_norm hd]
   float *freq = nullptr;      // [rope_dim / 2], frequency factors applied
   float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
-  uint32_t *attn_tickets = nullptr;   // [n_head_kv], zero between launches
+  uint32_t *attn_tickets = nullptr;   // [n_head_kv + OGM_TAIL_TICKETS], zero between launches; the last ones are the GEMV tails'
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
   void *v_cache = nullptr;
   float *x = nullptr;         // hidden state [n_embd]
@@ -869,7 +877,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   A((void **)&m->pre, (size_t)c.n_layer * pre_stride * 4);
   A((void **)&m->freq, (size_t)(c.rope_dim / 2 + 1) * 4);
   A((void **)&m->rope_cs, (size_t)(c.rope_dim / 2 + 1) * 8);
-  A((void **)&m->attn_tickets, (size_t)c.n_head_kv * 4);
+  A((void **)&m->attn_tickets, ((size_t)c.n_head_kv + OGM_TAIL_TICKETS) * 4);   // + the GEMV tails' tickets
   A(&m->k_cache, cache_bytes);
   A(&m->v_cache, cache_bytes);
   A((void **)&m->x, (size_t)c.n_embd * 4);
@@ -922,7 +930,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   hipError_t e = hipMemcpy(m->norms, host.data(), host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->pre, pre_host.data(), pre_host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, (size_t)c.n_head_kv * 4);
+  if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, ((size_t)c.n_head_kv + OGM_TAIL_TICKETS) * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
   if (e != hipSuccess) {
@@ -990,8 +998,14 @@ extern "C" int ogm_llama_kv_read(ogm_ctx *ctx, ogm_llama *m, uint32_t layer, uin
 }
 
 // One matmul group of the step over the activations the previous kernel quantized.
-static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, hipStream_t s) {
+static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, hipStream_t s,
+                        const OgmGemvTail *tail = nullptr) {
   // weights of one type go out as one launch; a mixed group (Q4_K q/k with a Q6_K v) as several
+  if (tail) {   // the caller has checked that the group is one launch
+    Target tg[OGM_GEMV_MAX_MATS];
+    for (size_t i = 0; i < n; i++) tg[i] = Target{ws[i], ys[i]};
+    return enqueue_gemv(ctx, tg, n, 1, 0, s, nullptr, nullptr, nullptr, tail);
+  }
   size_t i = 0;
   while (i < n) {
     Target tg[OGM_GEMV_MAX_MATS];
@@ -1016,6 +1030,19 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   if (x_dev != m->x) HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
   HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos, 1, c.rope_dim, m->rope_cs, s));
   const float *delta = nullptr;  // what the next norm adds to x first: the last block's output
+  // On request, with per-256 activations on the consumer's side, a norm or the SwiGLU runs as the
+  // tail of the GEMV launch before it (its last workgroup to finish) instead of as a kernel of its
+  // own.  Same bits, but slower on MI355X (8B-shaped model: 2.59 against 1.94 ms per token): every
+  // workgroup then waits for its coherent stores and a ticket before it leaves, which costs more
+  // than the three 4 us kernels a layer saves.
+  const bool fuse = ctx->tune_decode_fuse_tails != 0 && ctx->tune_fuse_quant <= 0;
+  auto tail_ok = [&](const ogm_weight *producer, uint32_t n, int consumer_mode) {
+    return fuse && consumer_mode == OGM_ACT_PER_256 && n % 32u == 0 && producer->out_dim == n &&
+           n <= ogm_gemv_norm_tail_max(producer->ggml_type, producer->in_dim, n, (uint32_t)ctx->tune_wg_waves);
+  };
+  const int mode_out = act_mode_for(m->output->ggml_type);
+  const float *out_norm = m->norms + (size_t)c.n_layer * 2 * c.n_embd;
+  bool normed = false;   // the next norm already ran as a tail
   for (uint32_t l = 0; l < c.n_layer; l++) {
     const ogm_llama_layer &L = m->layers[l];
     const float *attn_norm = m->norms + (size_t)l * 2 * c.n_embd, *ffn_norm = attn_norm + c.n_embd;
@@ -1026,8 +1053,9 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     const int mode_qkv = act_mode_for(L.wq->ggml_type);
     if (act_mode_for(L.wk->ggml_type) != mode_qkv || act_mode_for(L.wv->ggml_type) != mode_qkv)
       return fail(ctx, OGM_ERR_UNSUPPORTED, "wq, wk and wv must share an activation mode");
-    HIPCHK(ctx, ogm_launch_norm_quant(mode_qkv, m->x, delta, attn_norm, c.n_embd, c.rms_eps, nullptr,
-                                      act_view(ctx, c.n_embd, mode_qkv, 0), s));
+    if (!normed)
+      HIPCHK(ctx, ogm_launch_norm_quant(mode_qkv, m->x, delta, attn_norm, c.n_embd, c.rms_eps, nullptr,
+                                        act_view(ctx, c.n_embd, mode_qkv, 0), s));
     const ogm_weight *w3[3] = {L.wq, L.wk, L.wv};
     float *y3[3] = {m->q, m->k, m->v};
     int rc = llama_matmul(ctx, w3, y3, 3, s);
@@ -1037,27 +1065,63 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, m->rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
                                        c.n_head, c.n_head_kv, c.head_dim, scale, m->part_o, m->part_ml,
                                        m->attn_tickets, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s));
-    const ogm_weight *w1[1] = {L.wo};
-    float *y1[1] = {m->proj};
-    if ((rc = llama_matmul(ctx, w1, y1, 1, s)) != OGM_OK) return rc;
     const int mode_ff = act_mode_for(L.w_gate->ggml_type);
     if (act_mode_for(L.w_up->ggml_type) != mode_ff)
       return fail(ctx, OGM_ERR_UNSUPPORTED, "w_gate and w_up must share an activation mode");
-    HIPCHK(ctx, ogm_launch_norm_quant(mode_ff, m->x, m->proj, ffn_norm, c.n_embd, c.rms_eps, nullptr,
-                                      act_view(ctx, c.n_embd, mode_ff, 0), s));
+    const ogm_weight *w1[1] = {L.wo};
+    float *y1[1] = {m->proj};
+    OgmGemvTail tail;
+    tail.ticket = m->attn_tickets + c.n_head_kv;
+    if (tail_ok(L.wo, c.n_embd, mode_ff)) {
+      tail.kind = OGM_TAIL_NORM;
+      tail.n = c.n_embd;
+      tail.x = m->x;
+      tail.weight = ffn_norm;
+      tail.eps = c.rms_eps;
+      tail.act = act_view(ctx, c.n_embd, mode_ff, 0);
+      if ((rc = llama_matmul(ctx, w1, y1, 1, s, &tail)) != OGM_OK) return rc;
+    } else {
+      if ((rc = llama_matmul(ctx, w1, y1, 1, s)) != OGM_OK) return rc;
+      HIPCHK(ctx, ogm_launch_norm_quant(mode_ff, m->x, m->proj, ffn_norm, c.n_embd, c.rms_eps, nullptr,
+                                        act_view(ctx, c.n_embd, mode_ff, 0), s));
+    }
     const ogm_weight *w2[2] = {L.w_gate, L.w_up};
     float *y2[2] = {m->gate, m->up};
-    if ((rc = llama_matmul(ctx, w2, y2, 2, s)) != OGM_OK) return rc;
     const int mode_d = act_mode_for(L.w_down->ggml_type);
-    HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr,
-                                        act_view(ctx, c.n_ff, mode_d, 0), s));
+    if (fuse && mode_d == OGM_ACT_PER_256 && L.w_gate->ggml_type == L.w_up->ggml_type &&
+        block_elems_of(L.w_gate->ggml_type) == 256) {
+      tail.kind = OGM_TAIL_SWIGLU;
+      tail.n = c.n_ff;
+      tail.x = nullptr;
+      tail.weight = nullptr;
+      tail.act = act_view(ctx, c.n_ff, mode_d, 0);
+      if ((rc = llama_matmul(ctx, w2, y2, 2, s, &tail)) != OGM_OK) return rc;
+    } else {
+      if ((rc = llama_matmul(ctx, w2, y2, 2, s)) != OGM_OK) return rc;
+      HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr,
+                                          act_view(ctx, c.n_ff, mode_d, 0), s));
+    }
     const ogm_weight *wd[1] = {L.w_down};
-    if ((rc = llama_matmul(ctx, wd, y1, 1, s)) != OGM_OK) return rc;
+    // the next norm: the next layer's attention norm, or the output norm after the last layer
+    const bool last_layer = l + 1 == c.n_layer;
+    const int mode_next = last_layer ? mode_out : act_mode_for(m->layers[l + 1].wq->ggml_type);
+    normed = tail_ok(L.w_down, c.n_embd, mode_next);
+    if (normed) {
+      tail.kind = OGM_TAIL_NORM;
+      tail.n = c.n_embd;
+      tail.x = m->x;
+      tail.weight = last_layer ? out_norm : attn_norm + 2 * (size_t)c.n_embd;
+      tail.eps = c.rms_eps;
+      tail.act = act_view(ctx, c.n_embd, mode_next, 0);
+      if ((rc = llama_matmul(ctx, wd, y1, 1, s, &tail)) != OGM_OK) return rc;
+    } else {
+      if ((rc = llama_matmul(ctx, wd, y1, 1, s)) != OGM_OK) return rc;
+    }
     delta = m->proj;
   }
-  const int mode_out = act_mode_for(m->output->ggml_type);
-  HIPCHK(ctx, ogm_launch_norm_quant(mode_out, m->x, delta, m->norms + (size_t)c.n_layer * 2 * c.n_embd,
-                                    c.n_embd, c.rms_eps, nullptr, act_view(ctx, c.n_embd, mode_out, 0), s));
+  if (!normed)
+    HIPCHK(ctx, ogm_launch_norm_quant(mode_out, m->x, delta, out_norm, c.n_embd, c.rms_eps, nullptr,
+                                      act_view(ctx, c.n_embd, mode_out, 0), s));
   float *lg = logits_dev ? logits_dev : m->logits;
   const ogm_weight *wo_[1] = {m->output};
   float *yo[1] = {lg};

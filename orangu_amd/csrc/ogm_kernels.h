@@ -24,6 +24,26 @@ hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32
 
 #define OGM_GEMV_MAX_MATS 4
 
+// What the last workgroup of a single-token GEMV launch to finish does with the launch's outputs,
+// in place of a kernel of its own (per-256 activations only):
+//   OGM_TAIL_NORM   x += y; act = quantize(rmsnorm(x) * weight)       one matrix, out_dim = n
+//   OGM_TAIL_SWIGLU act = quantize(silu(y0) * y1)                     two matrices, out_dims = n
+// `ticket` is OGM_TAIL_TICKETS zeroed uint32 on the device that the launch leaves zero again.  `act` may be
+// the buffer the launch read its own activations from: every workgroup has finished by then.
+#define OGM_TAIL_TICKETS 65u
+#define OGM_TAIL_NONE 0u
+#define OGM_TAIL_NORM 1u
+#define OGM_TAIL_SWIGLU 2u
+struct OgmGemvTail {
+  uint32_t kind = OGM_TAIL_NONE;
+  uint32_t n = 0;
+  uint32_t *ticket = nullptr;
+  float *x = nullptr;             // NORM: the residual stream, updated in place
+  const float *weight = nullptr;  // NORM: the norm's weights
+  float eps = 0.0f;
+  OgmActDev act = {};
+};
+
 struct OgmGemvArgs {
   uint32_t ggml_type;
   const uint8_t *wt;  // tile-planar weights
@@ -45,11 +65,14 @@ struct OgmGemvArgs {
   // When set (one token, GEMV order, no dumps): f32 activations [in_dim]; every workgroup
   // quantizes them itself on its way in and `act` is not read.
   const float *x_f32;
+  OgmGemvTail tail;   // one token, GEMV order, no dumps, no x_f32
 };
 
 // Largest token count one launch can take for this shape (LDS budget), at least 1.
 uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order);
 hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name);
+// Longest row an OGM_TAIL_NORM tail of a single-token launch over this matrix can take (0: none).
+uint32_t ogm_gemv_norm_tail_max(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves);
 
 // Prefill GEMM on MFMA (ogm_gemm.hip).  Same operands as the GEMV plus a scratch buffer `xh` of
 // ogm_gemm_xh_bytes() for the activations as f16.  Follows the CPU path's GEMM float order.

@@ -622,6 +622,7 @@ struct GemvParams {
   uint32_t in_dim, upr;            // upr = blocks per row
   uint32_t n_tokens;
   uint32_t C, nct;                // tile shape: C blocks x R rows, nct = upr / C column tiles
+  OgmGemvTail tail;
 };
 
 template <class F, bool GEMM_ORDER>
@@ -694,7 +695,9 @@ struct UnpackedOf<F, true, true> { typedef typename F::Unpacked type; };
 // QUANT: the workgroup quantizes the f32 activations p.x itself (one token) instead of reading
 // the quantizer kernel's output.
 // UNPACK: several tokens and a format whose block is expensive to unpack: unpack once per tile.
-template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP, bool QUANT, bool UNPACK = false>
+// TAIL: the outputs are stored device-coherently and the last workgroup to finish runs p.tail.
+template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP, bool QUANT, bool UNPACK = false,
+          bool TAIL = false>
 __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t tid = threadIdx.x, nthr = blockDim.x;
@@ -888,7 +891,42 @@ __global__ __launch_bounds__(F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) 
       float acc = 0.0f;
       if (NT == 2) acc = ordered_sum<true>(acc, terms + (size_t)T * K * term_stride, upr, R);
       acc = ordered_sum<false>(acc, terms, upr, R);
-      y[(size_t)t * out_dim + orow] = acc;
+      if constexpr (TAIL) __hip_atomic_store(&y[(size_t)t * out_dim + orow], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else y[(size_t)t * out_dim + orow] = acc;
+    }
+  }
+  if constexpr (TAIL) {
+    // The outputs went out device-coherently; once every wave's stores are acknowledged (vmcnt 0)
+    // and the workgroup has met, one ticket tells whether all workgroups of the launch are done.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    uint32_t *l_last = (uint32_t *)lds;
+    if (tid == 0) {
+      // Tickets in two levels (atomics on one address are served one after the other, and a launch
+      // has up to a few thousand workgroups): workgroup i draws from counter 1 + i % 64, the last
+      // of each of those from counter 0.  Whoever draws a last ticket leaves its counter at zero.
+      const uint32_t n_grp = gridDim.x < OGM_TAIL_TICKETS - 1u ? gridDim.x : OGM_TAIL_TICKETS - 1u;
+      const uint32_t grp = blockIdx.x % (OGM_TAIL_TICKETS - 1u);
+      const uint32_t in_grp = (gridDim.x - grp + OGM_TAIL_TICKETS - 2u) / (OGM_TAIL_TICKETS - 1u);
+      bool last = false;
+      uint32_t *c1 = p.tail.ticket + 1u + grp;
+      if (__hip_atomic_fetch_add(c1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_grp - 1u) {
+        __hip_atomic_store(c1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__hip_atomic_fetch_add(p.tail.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_grp - 1u) {
+          __hip_atomic_store(p.tail.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          last = true;
+        }
+      }
+      l_last[0] = last ? 1u : 0u;
+    }
+    __syncthreads();
+    if (l_last[0] == 0u) return;
+    if (p.tail.kind == OGM_TAIL_NORM) {
+      ogm_norm_quant_row<256, true>(p.tail.x, p.y[0], p.tail.weight, p.tail.n, p.tail.eps, nullptr, p.tail.act,
+                                    (float *)lds + 16, tid, n_wave);
+    } else {
+      for (uint32_t run = wave; run * 256u < p.tail.n; run += n_wave)
+        ogm_swiglu_quant_run<256, true>(p.y[0], p.y[1], p.tail.n, nullptr, p.tail.act, run, lane);
     }
   }
 }
@@ -928,8 +966,48 @@ uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order
   }
 }
 
+// Waves per workgroup: the largest divisor of the row block's tile count up to 8 (measured on
+// MI355X: 4 waves x 1 tile at 4096 -> 14336, 7 waves x 2 tiles at 14336 -> 4096 beat 14 x 1).
+static uint32_t pick_waves(uint32_t nct, uint32_t wg_waves, int max_threads) {
+  uint32_t waves = wg_waves;
+  if (waves == 0) {
+    waves = 1;
+    for (uint32_t w = 2; w <= 8 && w <= nct; w++)
+      if (nct % w == 0) waves = w;
+  }
+  if (waves > nct) waves = nct;
+  if (waves > (uint32_t)max_threads / 64) waves = max_threads / 64;
+  if (waves == 0) waves = 1;
+  return waves;
+}
+
+uint32_t ogm_gemv_norm_tail_max(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves) {
+  int max_threads;
+  switch (ggml_type) {
+    case OGM_Q4_K: max_threads = FmtQ4K::MAX_THREADS; break;
+    case OGM_Q5_K: max_threads = FmtQ5K::MAX_THREADS; break;
+    case OGM_Q3_K: max_threads = FmtQ3K::MAX_THREADS; break;
+    case OGM_Q6_K: max_threads = FmtQ6K::MAX_THREADS; break;
+    default: return 0;
+  }
+  if (in_dim == 0 || in_dim % 256u != 0) return 0;
+  const OgmTiling tl = ogm_tiling_for(in_dim / 256u, out_dim);
+  return 1024u * pick_waves(tl.nct, wg_waves, max_threads);
+}
+
 template <class F, bool QUANT>
 static void launch_single(const GemvParams &p, dim3 g, dim3 b, size_t lds, hipStream_t stream) {
+  if constexpr (!QUANT && F::ELEMS == 256) {
+    if (p.tail.kind != OGM_TAIL_NONE) {
+      if (p.upr == 16)
+        hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false, false, false, true>), g, b, lds, stream, p);
+      else if (p.upr == 56)
+        hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false, false, false, true>), g, b, lds, stream, p);
+      else
+        hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false, false, false, true>), g, b, lds, stream, p);
+      return;
+    }
+  }
   // single-token decode: the hot shapes get their row length as a compile-time constant
   if (F::ELEMS == 256 && p.upr == 16)
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false, QUANT>), g, b, lds, stream, p);
@@ -949,6 +1027,16 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   GemvParams p;
   p.act = a.act;
   p.x = a.x_f32;
+  p.tail = a.tail;
+  if (a.tail.kind != OGM_TAIL_NONE) {
+    const bool shape_ok = a.tail.kind == OGM_TAIL_NORM ? (a.n_extra == 0 && a.out_dim == a.tail.n && a.tail.x && a.tail.weight)
+                          : a.tail.kind == OGM_TAIL_SWIGLU
+                              ? (a.n_extra == 1 && a.out_dim == a.tail.n && a.extra_out_dim[0] == a.tail.n)
+                              : false;
+    if (!shape_ok || F::ELEMS != 256 || a.n_tokens != 1 || GEMM_ORDER || dump || a.x_f32 || !a.tail.ticket ||
+        a.tail.n == 0 || a.tail.n % 32u != 0)
+      return hipErrorInvalidValue;
+  }
   p.dump_isum = a.dump_isum;
   p.dump_imin = a.dump_imin;
   p.in_dim = a.in_dim;
@@ -984,17 +1072,8 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   }
   const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, K);
   if (lds > OGM_LDS_BUDGET) return hipErrorInvalidValue;
-  // Waves per workgroup: the largest divisor of the row block's tile count up to 8 (measured on
-  // MI355X: 4 waves x 1 tile at 4096 -> 14336, 7 waves x 2 tiles at 14336 -> 4096 beat 14 x 1).
-  uint32_t waves = a.wg_waves;
-  if (waves == 0) {
-    waves = 1;
-    for (uint32_t w = 2; w <= 8 && w <= tl.nct; w++)
-      if (tl.nct % w == 0) waves = w;
-  }
-  if (waves > tl.nct) waves = tl.nct;
-  if (waves > (uint32_t)F::MAX_THREADS / 64) waves = F::MAX_THREADS / 64;
-  if (waves == 0) waves = 1;
+  const uint32_t waves = pick_waves(tl.nct, a.wg_waves, F::MAX_THREADS);
+  if (a.tail.kind == OGM_TAIL_NORM && a.tail.n > 1024u * waves) return hipErrorInvalidValue;
   const dim3 g(n_wg), b(waves * 64);
   if (dump) {
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true, false>), g, b, lds, stream, p);

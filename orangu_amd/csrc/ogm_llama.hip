@@ -17,16 +17,15 @@
 // ------------------------------------------------------------------------------------------
 // residual add + RMSNorm + quantize
 
-// One workgroup; wave w owns the 256-runs w, w + n_wave, ... (at most four), lane l their
-// elements 4l..4l+3, kept in registers between the two passes.
+// One workgroup per row (ogm_norm_quant_row).
 template <int GROUP>
 __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict__ x,
                                                               const float *__restrict__ delta,
                                                               const float *__restrict__ weight, uint32_t n,
                                                               float eps, float *__restrict__ normed,
                                                               OgmActDev act) {
-  __shared__ float red[16];
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, n_wave = blockDim.x >> 6;
+  __shared__ float red[64];
+  const uint32_t tid = threadIdx.x, n_wave = blockDim.x >> 6;
   {   // one workgroup per row of a batch
     const size_t row = (size_t)blockIdx.x * n;
     x += row;
@@ -38,47 +37,7 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
     act.bsum += (size_t)blockIdx.x * (n / 32u);
     if (act.bs16) act.bs16 += (size_t)blockIdx.x * (n / 16u);
   }
-  float4 v[4], wv[4];
-  float ss = 0.0f;
-  // every load first (x, the residual delta and the norm weights share one trip to memory)
-#pragma unroll
-  for (int k = 0; k < 4; k++) {
-    const uint32_t e0 = (wave + k * n_wave) * 256u + 4u * lane;
-    v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-    wv[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-    float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (e0 < n) {
-      v[k] = *(const float4 *)(x + e0);
-      wv[k] = *(const float4 *)(weight + e0);
-      if (delta) d = *(const float4 *)(delta + e0);
-    }
-    if (e0 < n && delta) {
-      v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
-      *(float4 *)(x + e0) = v[k];
-    }
-    ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
-  }
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) ss += __shfl_xor(ss, m, 64);
-  if (lane == 0) red[wave] = ss;
-  __syncthreads();
-  float total = 0.0f;
-  for (uint32_t w = 0; w < n_wave; w++) total += red[w];
-  const float mean_sq = total / (float)n;
-  const float scale = 1.0f / sqrtf(mean_sq + eps);
-#pragma unroll
-  for (int k = 0; k < 4; k++) {
-    const uint32_t e0 = (wave + k * n_wave) * 256u + 4u * lane;
-    const bool active = e0 < n;
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (active) {
-      o.x = v[k].x * scale * wv[k].x; o.y = v[k].y * scale * wv[k].y;
-      o.z = v[k].z * scale * wv[k].z; o.w = v[k].w * scale * wv[k].w;
-      if (normed) *(float4 *)(normed + e0) = o;
-    }
-    if ((wave + k * n_wave) * 256u < n)  // wave-uniform: the run exists
-      ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
-  }
+  ogm_norm_quant_row<GROUP, false>(x, delta, weight, n, eps, normed, act, red, tid, n_wave);
 }
 
 hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const float *weight, uint32_t n,
@@ -636,8 +595,6 @@ __global__ __launch_bounds__(64) void ogm_swiglu_quant_kernel(const float *__res
                                                               const float *__restrict__ up, uint32_t n,
                                                               float *__restrict__ h, OgmActDev act) {
   const uint32_t lane = threadIdx.x;
-  const uint32_t e0 = blockIdx.x * 256u + 4u * lane;
-  const bool active = e0 < n;
   {   // blockIdx.y: the row of a batch
     const size_t row = (size_t)blockIdx.y * n;
     gate += row;
@@ -649,16 +606,7 @@ __global__ __launch_bounds__(64) void ogm_swiglu_quant_kernel(const float *__res
     act.bsum += (size_t)blockIdx.y * (n / 32u);
     if (act.bs16) act.bs16 += (size_t)blockIdx.y * (n / 16u);
   }
-  float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (active) {
-    const float4 g = *(const float4 *)(gate + e0), u = *(const float4 *)(up + e0);
-    o.x = g.x / (1.0f + expf(-g.x)) * u.x;
-    o.y = g.y / (1.0f + expf(-g.y)) * u.y;
-    o.z = g.z / (1.0f + expf(-g.z)) * u.z;
-    o.w = g.w / (1.0f + expf(-g.w)) * u.w;
-    if (h) *(float4 *)(h + e0) = o;
-  }
-  ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
+  ogm_swiglu_quant_run<GROUP, false>(gate, up, n, h, act, blockIdx.x, lane);
 }
 
 hipError_t ogm_launch_swiglu_quant(int mode, const float *gate, const float *up, uint32_t n, float *h,

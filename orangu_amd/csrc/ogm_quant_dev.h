@@ -10,6 +10,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "ogm_kernels.h"
+
 __device__ __forceinline__ float ogm_nan_blind_max(float m, float a) { return a > m ? a : m; }
 
 __device__ __forceinline__ int ogm_quantize_one(float v, float inv) {
@@ -68,4 +70,98 @@ __device__ __forceinline__ void ogm_quantize_store(const float4 &v, uint32_t e0,
     }
     if ((lane & (GROUP / 4 - 1)) == 0) d[e0 / GROUP] = scale;
   }
+}
+
+// Four floats that another workgroup of the same kernel may have stored device-coherently.
+template <bool COHERENT>
+__device__ __forceinline__ float4 ogm_ld4(const float *p) {
+  if constexpr (COHERENT) {
+    const uint64_t a = __hip_atomic_load((const uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t b = __hip_atomic_load((const uint64_t *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return make_float4(__uint_as_float((uint32_t)a), __uint_as_float((uint32_t)(a >> 32)),
+                       __uint_as_float((uint32_t)b), __uint_as_float((uint32_t)(b >> 32)));
+  } else {
+    return *(const float4 *)p;
+  }
+}
+
+// Residual add, RMSNorm and quantization of one row by one workgroup of n_wave waves (n <= 1024 *
+// n_wave): wave w owns the 256-runs w, w + n_wave, ... (at most four), lane l their elements
+// 4l..4l+3, kept in registers between the two passes.  red: 64 floats of LDS.  COHERENT_DELTA:
+// delta was written by other workgroups of the calling kernel.
+template <int GROUP, bool COHERENT_DELTA>
+__device__ __forceinline__ void ogm_norm_quant_row(float *__restrict__ x, const float *__restrict__ delta,
+                                                   const float *__restrict__ weight, uint32_t n, float eps,
+                                                   float *__restrict__ normed, const OgmActDev &act,
+                                                   float *red, uint32_t tid, uint32_t n_wave) {
+  const uint32_t lane = tid & 63u, wave = tid >> 6;
+  float4 v[4], wv[4];
+  float ss[4];
+  // every load first (x, the residual delta and the norm weights share one trip to memory)
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    const uint32_t e0 = (wave + k * n_wave) * 256u + 4u * lane;
+    v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    wv[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (e0 < n) {
+      v[k] = *(const float4 *)(x + e0);
+      wv[k] = *(const float4 *)(weight + e0);
+      if (delta) d = ogm_ld4<COHERENT_DELTA>(delta + e0);
+    }
+    if (e0 < n && delta) {
+      v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
+      *(float4 *)(x + e0) = v[k];
+    }
+    ss[k] = v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+  }
+  // one sum per 256-run, then the runs in ascending order: the same value whatever the
+  // number of waves
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) ss[k] += __shfl_xor(ss[k], m, 64);
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+      if ((wave + k * n_wave) * 256u < n) red[wave + k * n_wave] = ss[k];
+  }
+  __syncthreads();
+  float total = 0.0f;
+  for (uint32_t r = 0; r * 256u < n; r++) total += red[r];
+  const float mean_sq = total / (float)n;
+  const float scale = 1.0f / sqrtf(mean_sq + eps);
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    const uint32_t e0 = (wave + k * n_wave) * 256u + 4u * lane;
+    const bool active = e0 < n;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (active) {
+      o.x = v[k].x * scale * wv[k].x; o.y = v[k].y * scale * wv[k].y;
+      o.z = v[k].z * scale * wv[k].z; o.w = v[k].w * scale * wv[k].w;
+      if (normed) *(float4 *)(normed + e0) = o;
+    }
+    if ((wave + k * n_wave) * 256u < n)  // wave-uniform: the run exists
+      ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
+  }
+}
+
+// SwiGLU and quantization of one 256-run by one wave: h = silu(gate) * up.
+template <int GROUP, bool COHERENT>
+__device__ __forceinline__ void ogm_swiglu_quant_run(const float *__restrict__ gate, const float *__restrict__ up,
+                                                     uint32_t n, float *__restrict__ h, const OgmActDev &act,
+                                                     uint32_t run, uint32_t lane) {
+  const uint32_t e0 = run * 256u + 4u * lane;
+  const bool active = e0 < n;
+  float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (active) {
+    const float4 g = ogm_ld4<COHERENT>(gate + e0), u = ogm_ld4<COHERENT>(up + e0);
+    o.x = g.x / (1.0f + expf(-g.x)) * u.x;
+    o.y = g.y / (1.0f + expf(-g.y)) * u.y;
+    o.z = g.z / (1.0f + expf(-g.z)) * u.z;
+    o.w = g.w / (1.0f + expf(-g.w)) * u.w;
+    if (h) *(float4 *)(h + e0) = o;
+  }
+  ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
 }

@@ -160,6 +160,32 @@ def test_decode_steps_from_an_empty_cache(be, types):
         dev.close()
 
 
+@pytest.mark.parametrize("types,n_embd,n_ff", [((Q4_K, Q6_K, Q6_K, Q6_K), 256, 512), ((Q4_K, Q4_K, Q6_K, Q6_K), 1024, 2816),
+                                               ((Q5_K, Q3_K, Q3_K, Q5_K), 512, 1280), ((Q4_K, Q4_K, Q8_0, Q8_0), 256, 512),
+                                               ((Q8_0, Q8_0, Q4_K, Q6_K), 256, 512)])
+def test_norms_and_swiglu_as_gemv_tails_change_no_bit(be, types, n_embd, n_ff):
+    """On request (decode_fuse_tails) the decode step runs the FFN norm, the SwiGLU and the next
+    attention (or output) norm as the tail of the GEMV launch before them (its last workgroup to
+    finish) wherever the consumer takes per-256 activations, instead of as kernels of their own: the
+    same arithmetic either way, so logits and greedy tokens agree to the bit over several steps."""
+    outs = []
+    xs = np.random.default_rng(11).standard_normal((4, n_embd)).astype(f32)
+    for fuse in (1, 0, 1):
+        ref, dev, rng = build(be, n_embd=n_embd, n_head=4, n_kv=2, hd=64, n_ff=n_ff, n_vocab=320, n_layer=3,
+                              types=types, max_ctx=16, seed=9)
+        be.set_tuning("decode_fuse_tails", fuse)
+        try:
+            got = [dev.decode(xs[pos], pos) for pos in range(4)]
+        finally:
+            be.set_tuning("decode_fuse_tails", 0)
+            dev.close()
+        outs.append(got)
+    for other in outs[1:]:
+        for pos, ((la, ta), (lb, tb)) in enumerate(zip(outs[0], other)):
+            assert ta == tb, pos
+            assert np.array_equal(la.view(np.uint32), lb.view(np.uint32)), (types, pos)
+
+
 def test_decode_with_q3_k_value_and_down_projections(be):
     """Q3_K in the v and down projections (what a Q3_K_M file does), one layer: the synthetic Q3_K
     weights are large, and with two layers of them the final hidden state is a small difference of
