@@ -335,6 +335,8 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * "gemm_small_max_tokens" (K-quant GEMMs of at most this many tokens take the small-batch kernel, whose
  * waves work on different super-blocks of the same rows; 0 = default 64, or 128 for matrices of up to
  * 8192 rows; 1 = never);
+ * "gemm_sb_waves" (waves of a small-batch workgroup: 8 or 16; 0 = default, 16 for launches of at most
+ * 256 workgroups over rows of at least 16 super-blocks);
  * "attn_prefill_variant" (attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the
  * decode step's kernel per token and chunk of the cache; they agree to f32 rounding, not bit for bit);
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);

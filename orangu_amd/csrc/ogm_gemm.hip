@@ -1183,11 +1183,14 @@ struct GemmSbParams {
   uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
 };
 
-__global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) {
+// NW waves (8 or 16): sixteen halve the chain once more and suit launches of few workgroups.
+template <uint32_t NW>
+__device__ __forceinline__ void gemm_sb_q6k_body(GemmSbParams p) {
+  constexpr uint32_t NT = 64u * NW, NACC = 1024u / NT;
   constexpr uint32_t TILE_BYTES = 13440u;
   extern __shared__ __align__(16) uint8_t sb_lds[];
-  float *terms = (float *)sb_lds;            // [8 waves][32 tokens][32 rows]
-  float *ad_l = terms + 8u * 32u * 32u;      // [nsb][32 tokens]
+  float *terms = (float *)sb_lds;            // [NW waves][32 tokens][32 rows]
+  float *ad_l = terms + NW * 32u * 32u;      // [nsb][32 tokens]
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
@@ -1222,7 +1225,7 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) {
   const uint32_t sc_shift = 8u * lh;
 
   // the tokens' ad of every super-block: ad_l[s][token]
-  for (uint32_t i = tid; i < 32u * p.nsb; i += 512u) {
+  for (uint32_t i = tid; i < 32u * p.nsb; i += NT) {
     const uint32_t k = i / p.nsb, s = i - k * p.nsb;
     ad_l[s * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + s];
   }
@@ -1277,10 +1280,12 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) {
   } while (0)
 
   const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  float acc0 = 0.0f, acc1 = 0.0f;   // outputs (token, row) = (tid / 32, tid % 32) and (tid / 32 + 16, tid % 32)
+  float acc[NACC];   // outputs (token, row) = (tid / 32 + a NT / 32, tid % 32)
+#pragma unroll
+  for (uint32_t a = 0; a < NACC; a++) acc[a] = 0.0f;
   SB_LOADW(wave);
   __syncthreads();   // ad_l
-  for (uint32_t s0 = 0; s0 < p.nsb; s0 += 8u) {
+  for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
     const uint32_t s = s0 + wave;
     if (s < p.nsb) {   // wave-uniform
       const uint32_t xs_ = xro + 256u * s;
@@ -1307,13 +1312,13 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) {
         }
       }
     }
-    SB_LOADW(s + 8u);   // the next round's weights, in flight over the barrier and the additions
+    SB_LOADW(s + NW);   // the next round's weights, in flight over the barrier and the additions
     __syncthreads();
     {
-      const uint32_t n_here = min(8u, p.nsb - s0);
+      const uint32_t n_here = min(NW, p.nsb - s0);
       for (uint32_t w = 0; w < n_here; w++) {   // ascending super-blocks, one accumulator per output
-        acc0 += terms[w * 1024u + tid];
-        acc1 += terms[w * 1024u + 512u + tid];
+#pragma unroll
+        for (uint32_t a = 0; a < NACC; a++) acc[a] += terms[w * 1024u + a * NT + tid];
       }
     }
     __syncthreads();
@@ -1322,13 +1327,17 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) {
 #undef SB_UNPACK
 #undef SB_STEP
   {
-    const uint32_t tok = t0 + (tid >> 5), row = r0 + (tid & 31u);
-    if (row < p.out_dim) {
-      if (tok < p.n_tokens) p.y[(size_t)tok * p.out_dim + row] = acc0;
-      if (tok + 16u < p.n_tokens) p.y[(size_t)(tok + 16u) * p.out_dim + row] = acc1;
+    const uint32_t row = r0 + (tid & 31u);
+#pragma unroll
+    for (uint32_t a = 0; a < NACC; a++) {
+      const uint32_t tok = t0 + (tid >> 5) + a * (NT / 32u);
+      if (row < p.out_dim && tok < p.n_tokens) p.y[(size_t)tok * p.out_dim + row] = acc[a];
     }
   }
 }
+
+__global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) { gemm_sb_q6k_body<8u>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_sb_q6k_w16_kernel(GemmSbParams p) { gemm_sb_q6k_body<16u>(p); }
 
 // The same for Q4_K and Q5_K (gemm_k_q4_k, vecdot.rs:2213-2303): first a sweep over the super-blocks
 // for the terms (ad * dmin) * imin, which the reference subtracts before anything else (rounds of
@@ -1336,12 +1345,13 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) {
 // instruction each), then the sweep of the products as above.  A lane's 16 weights of sub-block j
 // are the low (j even) or high nibbles of one 16-byte piece of qs, Q5_K's fifth bit is bit j of
 // its piece of qh; u = sc_j * q + 128 splits into the two int8 planes.
-template <bool Q5>
-__global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
+template <bool Q5, uint32_t NW>
+__device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
+  constexpr uint32_t NT = 64u * NW, NACC = 1024u / NT;
   constexpr uint32_t TILE_BYTES = Q5 ? 11264u : 9216u;
   constexpr uint32_t QS_PIECE0 = Q5 ? 3u : 1u;
   extern __shared__ __align__(16) uint8_t sb_lds[];
-  float *terms = (float *)sb_lds;             // [16 super-blocks][32 tokens][32 rows] (second sweep: 8)
+  float *terms = (float *)sb_lds;             // [16 super-blocks][32 tokens][32 rows] (second sweep: NW)
   float *ad_l = terms + 16u * 32u * 32u;      // [nsb][32 tokens]
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -1373,13 +1383,15 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
   const uint32_t xro = tok * p.in_dim + 16u * lh;   // + 256 s + 32 j
   const uint32_t tk = tok * p.nsb;
 
-  for (uint32_t i = tid; i < 32u * p.nsb; i += 512u) {
+  for (uint32_t i = tid; i < 32u * p.nsb; i += NT) {
     const uint32_t k = i / p.nsb, s = i - k * p.nsb;
     ad_l[s * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + s];
   }
   __syncthreads();
 
-  float acc0 = 0.0f, acc1 = 0.0f;   // outputs (token, row) = (tid / 32, tid % 32) and (tid / 32 + 16, tid % 32)
+  float acc[NACC];   // outputs (token, row) = (tid / 32 + a NT / 32, tid % 32)
+#pragma unroll
+  for (uint32_t a = 0; a < NACC; a++) acc[a] = 0.0f;
   // ---- first sweep: acc -= (ad * dmin) * sum_j m_j * bsum_j
   {
     float16v zero;
@@ -1388,8 +1400,8 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
     const float side_scale = lh ? 1.0f : 64.0f;
     for (uint32_t s0 = 0; s0 < p.nsb; s0 += 16u) {
 #pragma unroll
-      for (uint32_t u = 0; u < 2u; u++) {
-        const uint32_t sl = wave + 8u * u, s = s0 + sl;
+      for (uint32_t u = 0; u < 16u / NW; u++) {
+        const uint32_t sl = wave + NW * u, s = s0 + sl;
         if (s < p.nsb) {   // wave-uniform
           const uint4 hd = *(const uint4 *)(p.wt + (uo + sb_off(s)));
           const half8 b2 = *(const half8 *)(p.bs16 + ((tk + s) * 16u + 8u * lh));
@@ -1412,8 +1424,8 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
       __syncthreads();
       const uint32_t n_here = min(16u, p.nsb - s0);
       for (uint32_t w = 0; w < n_here; w++) {
-        acc0 -= terms[w * 1024u + tid];
-        acc1 -= terms[w * 1024u + 512u + tid];
+#pragma unroll
+        for (uint32_t a = 0; a < NACC; a++) acc[a] -= terms[w * 1024u + a * NT + tid];
       }
       __syncthreads();
     }
@@ -1457,7 +1469,7 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
   } while (0)
   const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   SB_LOADW(wave);
-  for (uint32_t s0 = 0; s0 < p.nsb; s0 += 8u) {
+  for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
     const uint32_t s = s0 + wave;
     if (s < p.nsb) {   // wave-uniform
       const uint32_t xs_ = xro + 256u * s;
@@ -1486,13 +1498,13 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
         }
       }
     }
-    SB_LOADW(s + 8u);   // the next round's weights, in flight over the barrier and the additions
+    SB_LOADW(s + NW);   // the next round's weights, in flight over the barrier and the additions
     __syncthreads();
     {
-      const uint32_t n_here = min(8u, p.nsb - s0);
+      const uint32_t n_here = min(NW, p.nsb - s0);
       for (uint32_t w = 0; w < n_here; w++) {   // ascending super-blocks, one accumulator per output
-        acc0 += terms[w * 1024u + tid];
-        acc1 += terms[w * 1024u + 512u + tid];
+#pragma unroll
+        for (uint32_t a = 0; a < NACC; a++) acc[a] += terms[w * 1024u + a * NT + tid];
       }
     }
     __syncthreads();
@@ -1500,13 +1512,19 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
 #undef SB_LOADW
 #undef SB_STEP
   {
-    const uint32_t tok_o = t0 + (tid >> 5), row = r0 + (tid & 31u);
-    if (row < p.out_dim) {
-      if (tok_o < p.n_tokens) p.y[(size_t)tok_o * p.out_dim + row] = acc0;
-      if (tok_o + 16u < p.n_tokens) p.y[(size_t)(tok_o + 16u) * p.out_dim + row] = acc1;
+    const uint32_t row = r0 + (tid & 31u);
+#pragma unroll
+    for (uint32_t a = 0; a < NACC; a++) {
+      const uint32_t tok_o = t0 + (tid >> 5) + a * (NT / 32u);
+      if (row < p.out_dim && tok_o < p.n_tokens) p.y[(size_t)tok_o * p.out_dim + row] = acc[a];
     }
   }
 }
+
+template <bool Q5>
+__global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) { gemm_sb_q45k_body<Q5, 8u>(p); }
+template <bool Q5>
+__global__ __launch_bounds__(1024) void ogm_gemm_sb_q45k_w16_kernel(GemmSbParams p) { gemm_sb_q45k_body<Q5, 16u>(p); }
 
 // ------------------------------------------------------------------------------------------
 // Q4_K, wide tile: 128 rows x 256 tokens per workgroup, twelve waves.
@@ -2616,19 +2634,23 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
       if (m < a.n_extra) tiles += (a.extra_out_dim[m] + 31u) / 32u;
     }
-    const uint32_t lds_bytes = (q45 ? 16u : 8u) * 4096u + 128u * nsb;
-    const void *fn = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_sb_q6k_kernel
-                     : a.ggml_type == OGM_Q4_K ? (const void *)ogm_gemm_sb_q45k_kernel<false>
-                                               : (const void *)ogm_gemm_sb_q45k_kernel<true>;
+    // sixteen waves when the launch leaves compute units idle and the rows are long enough
+    const uint32_t n_wg = ((a.n_tokens + 31u) / 32u) * tiles;
+    const bool w16 = (a.sb_waves ? a.sb_waves == 16u : (n_wg <= 256u && nsb >= 16u)) &&
+                     16u * 4096u + 128u * nsb <= GM_LDS_MAX;
+    const uint32_t lds_bytes = ((q45 || w16) ? 16u : 8u) * 4096u + 128u * nsb;
+    const void *fn = a.ggml_type == OGM_Q6_K   ? (w16 ? (const void *)ogm_gemm_sb_q6k_w16_kernel : (const void *)ogm_gemm_sb_q6k_kernel)
+                     : a.ggml_type == OGM_Q4_K ? (w16 ? (const void *)ogm_gemm_sb_q45k_w16_kernel<false> : (const void *)ogm_gemm_sb_q45k_kernel<false>)
+                                               : (w16 ? (const void *)ogm_gemm_sb_q45k_w16_kernel<true> : (const void *)ogm_gemm_sb_q45k_kernel<true>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
     void *kargs[] = {(void *)&p};
-    e = hipLaunchKernel(fn, dim3((a.n_tokens + 31u) / 32u, tiles), dim3(512), kargs, lds_bytes, stream);
+    e = hipLaunchKernel(fn, dim3((a.n_tokens + 31u) / 32u, tiles), dim3(w16 ? 1024 : 512), kargs, lds_bytes, stream);
     if (e != hipSuccess) return e;
     if (kernel_name)
-      *kernel_name = a.ggml_type == OGM_Q6_K   ? "ogm_gemm_sb_q6k_kernel"
-                     : a.ggml_type == OGM_Q4_K ? "ogm_gemm_sb_q4k_kernel"
-                                               : "ogm_gemm_sb_q5k_kernel";
+      *kernel_name = a.ggml_type == OGM_Q6_K   ? (w16 ? "ogm_gemm_sb_q6k_w16_kernel" : "ogm_gemm_sb_q6k_kernel")
+                     : a.ggml_type == OGM_Q4_K ? (w16 ? "ogm_gemm_sb_q4k_w16_kernel" : "ogm_gemm_sb_q4k_kernel")
+                                               : (w16 ? "ogm_gemm_sb_q5k_w16_kernel" : "ogm_gemm_sb_q5k_kernel");
     return hipGetLastError();
   }
   if (i8p) {

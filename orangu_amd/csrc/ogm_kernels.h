@@ -88,6 +88,7 @@ struct OgmGemmArgs {
   uint32_t wide_min_wgs = 0;   // Q4_K: least 128x128 workgroups from which the wide tiling runs (0 = default)
   uint32_t q4k_variant = 0;    // K-quants: 0 / 1 the int8 plane kernels, 2 the f16 kernels, 3 int8 multiply-adds
   uint32_t small_max_tokens = 0;   // most tokens for the small-batch kernel (0 = default 64, 1 = never)
+  uint32_t sb_waves = 0;           // waves of a small-batch workgroup: 8 or 16 (0 = by the size of the launch)
   // K-quants: further matrices of the same type and in_dim over the same activations, in the same launch
   uint32_t n_extra = 0;
   const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1] = {};

@@ -37,6 +37,7 @@ def be():
     say("device:", b.device_name())
     b.set_tuning("gemm_min_tokens", GEMM_FROM)
     b.set_tuning("gemm_small_max_tokens", 1)
+    b.set_tuning("gemm_sb_waves", 8)
     yield b
     b.close()
 
@@ -417,6 +418,11 @@ def test_gemm_threshold_default():
             y = b.matmul(x[:n], n, w)
             assert b.last_kernel().startswith(kernel), (n, b.last_kernel())
             assert_bits(y, want[:n], f"Q4_K, {n} tokens")
+        raw = synth_weights(Q5_K, 4096, 70, seed=7)    # few workgroups, sixteen super-blocks: sixteen waves
+        x4 = synth_x(12, 4096, seed=8)
+        y = b.matmul(x4, 12, qm(raw, Q5_K, 4096, 70))
+        assert b.last_kernel() == "ogm_gemm_sb_q5k_w16_kernel"
+        assert_bits(y, oracle.matmul(Q5_K, raw, 4096, 70, x4, 12), "Q5_K, 12 tokens")
         raw = synth_weights(Q6_K, 256, 8300, seed=6)   # 130 tiles of 64 rows
         w = qm(raw, Q6_K, 256, 8300)
         want = oracle.matmul(Q6_K, raw, 256, 8300, np.ascontiguousarray(x[:65, :256]), 65).reshape(65, 8300)
@@ -433,23 +439,28 @@ def test_gemm_threshold_default():
     (256, 5, 9), (1024, 100, 17), (768, 64, 32), (1280, 257, 40), (2048, 37, 64), (14336, 96, 33), (1792, 33, 10),
     (4096, 300, 20), (512, 31, 63), (2304, 130, 100), (1024, 70, 128), (256, 1, 1000),
 ])
-def test_small_batch_gemm_matches_cpu_gemm(be, t, in_dim, out_dim, T):
-    """The small-batch kernel of the K-quants (a workgroup's eight waves on different super-blocks of
+@pytest.mark.parametrize("waves", [8, 16])
+def test_small_batch_gemm_matches_cpu_gemm(be, t, in_dim, out_dim, T, waves):
+    """The small-batch kernel of the K-quants (a workgroup's eight or sixteen waves on different super-blocks of
     32 rows x 32 tokens, terms added in ascending order afterwards): every bit of gemm_k_q4_k /
     gemm_k_q6_k (vecdot.rs:2213-2303, 2352-2398), at any token count it is asked for."""
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T + 2)
     be.set_tuning("gemm_small_max_tokens", 1024)
+    be.set_tuning("gemm_sb_waves", waves)
     try:
         got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
     finally:
         be.set_tuning("gemm_small_max_tokens", 1)
-    assert be.last_kernel() == {Q4_K: "ogm_gemm_sb_q4k_kernel", Q5_K: "ogm_gemm_sb_q5k_kernel", Q6_K: "ogm_gemm_sb_q6k_kernel"}[t]
+        be.set_tuning("gemm_sb_waves", 8)
+    assert be.last_kernel() == {Q4_K: "ogm_gemm_sb_q4k", Q5_K: "ogm_gemm_sb_q5k", Q6_K: "ogm_gemm_sb_q6k"}[t] + \
+        ("_w16_kernel" if waves == 16 else "_kernel")
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "small-batch gemm")
 
 
 @pytest.mark.parametrize("t,block,hi", [(Q4_K, 144, 0xFF), (Q5_K, 176, 0xFF), (Q6_K, 210, 0x7F), (Q6_K, 210, 0x80)])
-def test_small_batch_gemm_extreme_integer_ranges(be, t, block, hi):
+@pytest.mark.parametrize("waves", [8, 16])
+def test_small_batch_gemm_extreme_integer_ranges(be, t, block, hi, waves):
     """Every weight bit and scale byte at its extreme (Q6_K: scales +127 and -128), activations +-127."""
     in_dim, out_dim, T = 1024, 40, 24
     blocks = np.full((out_dim * 4, block), 0xFF, np.uint8)
@@ -464,11 +475,13 @@ def test_small_batch_gemm_extreme_integer_ranges(be, t, block, hi):
     x[:, ::7] = 126.0
     raw = blocks.reshape(-1)
     be.set_tuning("gemm_small_max_tokens", 1024)
+    be.set_tuning("gemm_sb_waves", waves)
     try:
         got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
     finally:
         be.set_tuning("gemm_small_max_tokens", 1)
-    assert be.last_kernel().startswith("ogm_gemm_sb_")
+        be.set_tuning("gemm_sb_waves", 8)
+    assert be.last_kernel().startswith("ogm_gemm_sb_") and ("_w16_" in be.last_kernel()) == (waves == 16)
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "extreme ranges")
 
 
