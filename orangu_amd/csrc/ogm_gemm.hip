@@ -1344,7 +1344,7 @@ __global__ __launch_bounds__(1024) void ogm_gemm_sb_q6k_w16_kernel(GemmSbParams 
 // sixteen super-blocks, two per wave: header and the quantizer's sums per 32 only, one f16 matrix
 // instruction each), then the sweep of the products as above.  A lane's 16 weights of sub-block j
 // are the low (j even) or high nibbles of one 16-byte piece of qs, Q5_K's fifth bit is bit j of
-// its piece of qh; u = sc_j * q + 128 splits into the two int8 planes.
+// its piece of qh.
 template <bool Q5, uint32_t NW>
 __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
   constexpr uint32_t NT = 64u * NW, NACC = 1024u / NT;
@@ -1443,29 +1443,26 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
     w3 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 6u + lh) * 1024u));                          \
     if constexpr (Q5) qh5 = *(const uint4 *)(p.wt + (so_ + (1u + lh) * 1024u));                   \
   } while (0)
-#define SB_STEP(QS, J, FIRST)                                                                     \
+  // One matrix instruction per sub-block on the bare quants (K = 32 is exactly a sub-block; a lane's
+  // operand is its row's 16 nibbles, with Q5_K's fifth bit on top), then isum += sc_j * dot_j as
+  // 24-bit integer multiply-adds (|dot_j| <= 31 * 127 * 32 < 2^17, sc_j < 64): the same integer.
+#define SB_MMA(D, QS, J)                                                                          \
+  do {                                                                                            \
+    const uint32_t qsw_[4] = {QS.x, QS.y, QS.z, QS.w}, q5w_[4] = {qh5.x, qh5.y, qh5.z, qh5.w};    \
+    uint32_t v_[4];                                                                               \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      v_[w_] = (((J) & 1) ? (qsw_[w_] >> 4) : qsw_[w_]) & 0x0F0F0F0Fu;                            \
+      if constexpr (Q5) v_[w_] |= ((q5w_[w_] >> (J)) & 0x01010101u) << 4;                         \
+    }                                                                                             \
+    const int4v b_ = {(int)v_[0], (int)v_[1], (int)v_[2], (int)v_[3]};                            \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 32u * (J)));                                 \
+    D = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, b_, zi, 0, 0, 0);                              \
+  } while (0)
+#define SB_ACC(D, J, FIRST)                                                                       \
   do {                                                                                            \
     const int sc_ = (int)((((J) < 4 ? sca_ : scb_) >> (8u * ((J) & 3u))) & 0xFFu);                \
-    const short2v sc2_ = {(short)sc_, (short)sc_};                                                \
-    const short2v c2_ = {128, 128};                                                               \
-    const uint32_t qsw_[4] = {QS.x, QS.y, QS.z, QS.w}, q5w_[4] = {qh5.x, qh5.y, qh5.z, qh5.w};    \
-    uint32_t ph_[4], pl_[4];                                                                      \
-    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
-      uint32_t v_ = (((J) & 1) ? (qsw_[w_] >> 4) : qsw_[w_]) & 0x0F0F0F0Fu;                       \
-      if constexpr (Q5) v_ |= ((q5w_[w_] >> (J)) & 0x01010101u) << 4;                             \
-      union { uint32_t u; short2v s; } e_, f_;                                                    \
-      e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
-      f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
-      e_.s = e_.s * sc2_ + c2_;                                                                   \
-      f_.s = f_.s * sc2_ + c2_;                                                                   \
-      ph_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x07050301u);                                   \
-      pl_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u) ^ 0x80808080u;                     \
-    }                                                                                             \
-    const int4v bh_ = {(int)ph_[0], (int)ph_[1], (int)ph_[2], (int)ph_[3]};                       \
-    const int4v bl_ = {(int)pl_[0], (int)pl_[1], (int)pl_[2], (int)pl_[3]};                       \
-    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 32u * (J)));                                 \
-    H = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bh_, (FIRST) ? zi : H, 0, 0, 0);               \
-    L = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bl_, (FIRST) ? zi : L, 0, 0, 0);               \
+    _Pragma("unroll") for (int r_ = 0; r_ < 16; r_++)                                             \
+      I[r_] = (FIRST) ? __mul24(sc_, D[r_]) : __mul24(sc_, D[r_]) + I[r_];                        \
   } while (0)
   const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   SB_LOADW(wave);
@@ -1475,15 +1472,23 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
       const uint32_t xs_ = xro + 256u * s;
       uint32_t sca_, scb_;
       q4k_scales(hdr, sca_, scb_);
-      int16v H, L;
-      SB_STEP(w0, 0, true);
-      SB_STEP(w0, 1, false);
-      SB_STEP(w1, 2, false);
-      SB_STEP(w1, 3, false);
-      SB_STEP(w2, 4, false);
-      SB_STEP(w2, 5, false);
-      SB_STEP(w3, 6, false);
-      SB_STEP(w3, 7, false);
+      int16v I, Da, Db;   // the products of a sub-block are under way while the one before is added
+      SB_MMA(Da, w0, 0);
+      SB_MMA(Db, w0, 1);
+      SB_ACC(Da, 0, true);
+      SB_MMA(Da, w1, 2);
+      SB_ACC(Db, 1, false);
+      SB_MMA(Db, w1, 3);
+      SB_ACC(Da, 2, false);
+      SB_MMA(Da, w2, 4);
+      SB_ACC(Db, 3, false);
+      SB_MMA(Db, w2, 5);
+      SB_ACC(Da, 4, false);
+      SB_MMA(Da, w3, 6);
+      SB_ACC(Db, 5, false);
+      SB_MMA(Db, w3, 7);
+      SB_ACC(Da, 6, false);
+      SB_ACC(Db, 7, false);
       const float d = gm_f16_bits_to_f32(hdr.x & 0xFFFFu);
       const float *adp = &ad_l[s * 32u + 4u * lh];
       float *tp = terms + (wave * 32u + 4u * lh) * 32u + l32;   // [wave][token][row]
@@ -1493,7 +1498,7 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
         const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          const int is_ = H[4 * q4 + e] * 256 + L[4 * q4 + e];
+          const int is_ = I[4 * q4 + e];
           tp[(8 * q4 + e) * 32] = a4v[e] * (d * (float)is_);
         }
       }
@@ -1510,7 +1515,8 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
     __syncthreads();
   }
 #undef SB_LOADW
-#undef SB_STEP
+#undef SB_MMA
+#undef SB_ACC
   {
     const uint32_t row = r0 + (tid & 31u);
 #pragma unroll
