@@ -118,14 +118,12 @@ __device__ __forceinline__ void ogm_norm_quant_row(float *__restrict__ x, const 
   // one sum per 256-run, then the runs in ascending order: the same value whatever the
   // number of waves
 #pragma unroll
-  for (int m = 1; m < 64; m <<= 1) {
+  for (int k = 0; k < 4; k++) {
+    if ((wave + k * n_wave) * 256u < n) {   // wave-uniform: the run exists
 #pragma unroll
-    for (int k = 0; k < 4; k++) ss[k] += __shfl_xor(ss[k], m, 64);
-  }
-  if (lane == 0) {
-#pragma unroll
-    for (int k = 0; k < 4; k++)
-      if ((wave + k * n_wave) * 256u < n) red[wave + k * n_wave] = ss[k];
+      for (int m = 1; m < 64; m <<= 1) ss[k] += __shfl_xor(ss[k], m, 64);
+      if (lane == 0) red[wave + k * n_wave] = ss[k];
+    }
   }
   __syncthreads();
   float total = 0.0f;
