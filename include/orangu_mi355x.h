@@ -317,7 +317,10 @@ int ogm_gguf_upload_matrix(ogm_ctx *ctx, ogm_gguf *g, const char *name, ogm_weig
  * pairing rope_layout_for gives the architecture.  Every matrix goes through ogm_gguf_upload_matrix
  * (the context keeps them); *tok_embd (nullable) receives the embedding matrix for
  * ogm_llama_generate / ogm_dequant_rows, *cfg_out (nullable) the configuration used.  Errors are
- * reported through ogm_gguf_last_error. */
+ * reported through ogm_gguf_last_error.  Hyperparameters that do not fit 32 bits (or whose
+ * head_count * key_length does not) are rejected before any upload.  Matrices uploaded before a later
+ * failure stay in the context's weight cache, keyed by their mapped bytes, until ogm_destroy: a retry
+ * over the same mapping finds them there. */
 int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama **model,
                         const ogm_weight **tok_embd, ogm_llama_config *cfg_out);
 

@@ -35,6 +35,7 @@ struct ogm_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
   std::mutex mu;
+  std::mutex err_mu;   // guards err alone: argument checks fail before mu is taken
   std::string err;
   std::string name;
   std::map<std::pair<uint64_t, uint64_t>, ogm_weight *> cache;
@@ -65,11 +66,14 @@ struct ogm_ctx {
 
 static thread_local std::string g_init_err;
 
+// Callable with or without ctx->mu held: the message has a lock of its own.
 static int fail(ogm_ctx *ctx, int status, const std::string &msg) {
-  if (ctx)
+  if (ctx) {
+    std::lock_guard<std::mutex> lock(ctx->err_mu);
     ctx->err = msg;
-  else
+  } else {
     g_init_err = msg;
+  }
   return status;
 }
 
@@ -160,7 +164,9 @@ extern "C" int ogm_init(int device, ogm_ctx **out) {
   ogm_ctx *ctx = new (std::nothrow) ogm_ctx();
   if (!ctx) return fail(nullptr, OGM_ERR_OOM, "out of host memory");
   ctx->device = device;
-  ctx->name = std::string(prop.name) + " (" + prop.gcnArchName + ")";
+  // Some driver stacks leave the marketing name empty: fall back to the architecture's name.
+  const std::string board = prop.name[0] ? prop.name : "AMD Instinct (gfx950)";
+  ctx->name = board + " (" + prop.gcnArchName + ")";
   e = hipSetDevice(device);
   if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
   if (e != hipSuccess) {
@@ -193,7 +199,7 @@ extern "C" void ogm_destroy(ogm_ctx *ctx) {
 extern "C" const char *ogm_last_error(ogm_ctx *ctx) {
   static thread_local std::string copy;
   if (ctx) {
-    std::lock_guard<std::mutex> lock(ctx->mu);
+    std::lock_guard<std::mutex> lock(ctx->err_mu);
     copy = ctx->err;
   } else {
     copy = g_init_err;
@@ -263,7 +269,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   return fail(ctx, OGM_ERR_INVALID, std::string("unknown tuning key ") + key);
 }
 
-extern "C" const char *ogm_last_kernel(ogm_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
+extern "C" const char *ogm_last_kernel(ogm_ctx *ctx) {
+  if (!ctx) return "";
+  std::lock_guard<std::mutex> lock(ctx->mu);   // launches write it under the same lock
+  return ctx->last_kernel;
+}
 
 // ------------------------------------------------------------------------------------------
 // weights
@@ -647,13 +657,19 @@ extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, i
   // Every op gets its own slice of the transfer buffers; the activation scratch is shared,
   // which is safe because one stream runs each quantize after the kernels that read the last.
   // Ops that read the very same host slice (q/k/v, gate/up) share one device copy of it.
-  std::vector<size_t> xoff(n_ops), yoff(n_ops);
+  // src[i] is the first op whose device copy of x op i shares (itself when it brings its own).  An
+  // op without tokens brings and shares nothing, so it never stands in for a later op's input.
+  std::vector<size_t> xoff(n_ops), yoff(n_ops), src(n_ops);
   size_t xb = 0, yb = 0;
   for (size_t i = 0; i < n_ops; i++) {
-    size_t j = 0;
-    while (j < i && !(ops[j].x == ops[i].x && ops[j].n_tokens == ops[i].n_tokens &&
-                      ops[j].w->in_dim == ops[i].w->in_dim))
-      j++;
+    size_t j = i;
+    if (ops[i].n_tokens != 0) {
+      j = 0;
+      while (j < i && !(ops[j].n_tokens != 0 && ops[j].x == ops[i].x && ops[j].n_tokens == ops[i].n_tokens &&
+                        ops[j].w->in_dim == ops[i].w->in_dim))
+        j++;
+    }
+    src[i] = j;
     if (j < i) {
       xoff[i] = xoff[j];
     } else {
@@ -678,16 +694,14 @@ extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, i
   for (size_t i = 0; i < n_ops; i++) {
     const ogm_op &op = ops[i];
     const size_t bytes = (size_t)op.n_tokens * op.w->in_dim * 4;
-    bool first = true;
-    for (size_t j = 0; j < i; j++) first = first && xoff[j] != xoff[i];
-    if (bytes && first) memcpy((uint8_t *)ctx->hx.p + xoff[i], op.x, bytes);
+    if (bytes && src[i] == i) memcpy((uint8_t *)ctx->hx.p + xoff[i], op.x, bytes);
   }
   HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, ctx->hx.p, xb, hipMemcpyHostToDevice, ctx->stream));
   std::vector<Target> tg;
   for (size_t i = 0; i < n_ops;) {
     // a run of neighbouring ops over one input and one weight type: one group
     size_t e = i + 1;
-    while (e < n_ops && xoff[e] == xoff[i] && ops[e].n_tokens == ops[i].n_tokens &&
+    while (e < n_ops && ops[i].n_tokens != 0 && src[e] == src[i] && ops[e].n_tokens == ops[i].n_tokens &&
            ops[e].w->ggml_type == ops[i].w->ggml_type && ops[e].w->in_dim == ops[i].w->in_dim)
       e++;
     const ogm_op &op = ops[i];

@@ -575,7 +575,11 @@ extern "C" int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, 
   float freq_base = 10000.0f, rms_eps = 1e-5f;
   (void)meta_f32_of(g, arch + ".rope.freq_base", &freq_base);
   (void)meta_f32_of(g, arch + ".attention.layer_norm_rms_epsilon", &rms_eps);
-  if (n_layer == 0 || n_layer > 4096 || n_embd > UINT32_MAX || n_vocab > UINT32_MAX) {
+  // Every one of these is an untrusted u64 that ends up in a u32 field (and n_head * head_dim in a
+  // u32 product inside ogm_llama_create): reject what does not fit before anything is uploaded.
+  if (n_layer == 0 || n_layer > 4096 || n_embd > UINT32_MAX || n_vocab > UINT32_MAX || n_head > UINT32_MAX ||
+      n_head_kv > UINT32_MAX || head_dim > UINT32_MAX || rope_dim > UINT32_MAX ||
+      n_head * head_dim > UINT32_MAX || n_head_kv * head_dim > UINT32_MAX) {
     g->err = "model dimensions out of range";
     return OGM_ERR_INVALID;
   }

@@ -59,7 +59,7 @@ struct OgmTiling {
   uint32_t nrb;   // row blocks (ceil(out_dim / R))
 };
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define OGM_HD __host__ __device__
 #else
 #define OGM_HD

@@ -82,6 +82,13 @@ hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t n_tok
 // chunk of positions, and (in the workgroup that finishes last) the merge of the chunks with the
 // quantizer of the next matmul
 
+// K/V rows are cached as f16 (the reference's host cache is f32, kv_cache.rs:75-78): a component
+// beyond the f16 range saturates at +-65504 instead of becoming an infinity, which would turn a
+// zero weight into NaN in the weighted V sum and swamp every score it touches in K.  NaN stays NaN.
+__device__ __forceinline__ __half ogm_f16_sat(float v) {
+  return __float2half_rn(v != v ? v : fminf(fmaxf(v, -65504.0f), 65504.0f));
+}
+
 __device__ __forceinline__ float2 rope_pair(float2 ab, float2 cs) {
   return make_float2(ab.x * cs.x - ab.y * cs.y, ab.x * cs.y + ab.y * cs.x);
 }
@@ -292,7 +299,7 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
           qs[u][ia[j]] = ab.x;
           qs[u][ib[j]] = ab.y;
         } else {
-          const __half ha = __float2half_rn(ab.x), hb = __float2half_rn(ab.y);
+          const __half ha = ogm_f16_sat(ab.x), hb = ogm_f16_sat(ab.y);
           __half *lds = is_v ? vcur : kcur;
           __half *cache = (is_v ? vc : kc) + (size_t)pos * kv_dim + kvh * HD;
           lds[ia[j]] = ha;
@@ -621,28 +628,36 @@ hipError_t ogm_launch_swiglu_quant(int mode, const float *gate, const float *up,
 }
 
 // ------------------------------------------------------------------------------------------
-// argmax (last of equal maxima, as Iterator::max_by returns it)
+// argmax as sampling.rs:336-343 takes it: Iterator::max_by over f32::total_cmp, which returns the
+// last of several equal maxima.  total_cmp orders -NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN; the
+// key below is the usual monotone map of that order onto signed integers.
 
-__device__ __forceinline__ bool argmax_better(float v, uint32_t i, float bv, uint32_t bi) {
-  return v > bv || (v == bv && i > bi);
+__device__ __forceinline__ int32_t argmax_key(float v) {
+  const int32_t k = __float_as_int(v);
+  return k ^ ((k >> 31) & 0x7FFFFFFF);
+}
+__device__ __forceinline__ bool argmax_better(int32_t k, uint32_t i, int32_t bk, uint32_t bi) {
+  return k > bk || (k == bk && i > bi);
 }
 
 __global__ __launch_bounds__(256) void ogm_argmax_kernel(const float *__restrict__ x, uint32_t n,
                                                          uint32_t *__restrict__ scratch, uint32_t *__restrict__ out,
                                                          int final_stage) {
-  __shared__ float sv[256];
+  __shared__ int32_t sv[256];
   __shared__ uint32_t si[256];
   const uint32_t tid = threadIdx.x;
-  float bv = -INFINITY;
+  int32_t bk = INT32_MIN;   // the key of the smallest value there is
   uint32_t bi = 0;
   if (!final_stage) {
-    for (uint32_t i = blockIdx.x * 256u + tid; i < n; i += gridDim.x * 256u)
-      if (argmax_better(x[i], i, bv, bi)) { bv = x[i]; bi = i; }
+    for (uint32_t i = blockIdx.x * 256u + tid; i < n; i += gridDim.x * 256u) {
+      const int32_t k = argmax_key(x[i]);
+      if (argmax_better(k, i, bk, bi)) { bk = k; bi = i; }
+    }
   } else {
-    // scratch: 256 values then 256 indices, one per first-stage workgroup
-    if (tid < n) { bv = __uint_as_float(scratch[tid]); bi = scratch[256 + tid]; }
+    // scratch: 256 keys then 256 indices, one per first-stage workgroup
+    if (tid < n) { bk = (int32_t)scratch[tid]; bi = scratch[256 + tid]; }
   }
-  sv[tid] = bv;
+  sv[tid] = bk;
   si[tid] = bi;
   __syncthreads();
   for (uint32_t s = 128; s > 0; s >>= 1) {
@@ -654,7 +669,7 @@ __global__ __launch_bounds__(256) void ogm_argmax_kernel(const float *__restrict
   }
   if (tid == 0) {
     if (!final_stage) {
-      scratch[blockIdx.x] = __float_as_uint(sv[0]);
+      scratch[blockIdx.x] = (uint32_t)sv[0];
       scratch[256 + blockIdx.x] = si[0];
     } else {
       *out = si[0];
@@ -676,7 +691,7 @@ hipError_t ogm_launch_argmax(const float *logits, uint32_t n, uint32_t *scratch,
 
 __global__ void ogm_f32_to_f16_kernel(const float *__restrict__ src, __half *__restrict__ dst, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) dst[i] = __float2half_rn(src[i]);
+  if (i < n) dst[i] = ogm_f16_sat(src[i]);
 }
 
 hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStream_t stream) {
@@ -880,8 +895,8 @@ __global__ __launch_bounds__(256) void ogm_qkv_pre_kernel(float *__restrict__ q,
       qrow[ib[j]] = ab.y;
     } else {
       __half *cache = (is_v ? vc : kc) + (size_t)(pos0 + tok) * kv_dim + row;
-      cache[ia[j]] = __float2half_rn(ab.x);
-      cache[ib[j]] = __float2half_rn(ab.y);
+      cache[ia[j]] = ogm_f16_sat(ab.x);
+      cache[ib[j]] = ogm_f16_sat(ab.y);
     }
   }
 }
