@@ -172,6 +172,15 @@ int ogm_matmul_multi_act_dev(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n
  * (per-16 sums of q, i32).  Host pointers; n % 32 (resp. 256) must be 0. */
 int ogm_quantize_act(ogm_ctx *ctx, int mode, const float *x, size_t n, int8_t *q, float *d,
                      int32_t *sums);
+/* The same quantizer over a batch, as the multi-token matmuls launch it: x is [n_tokens][in_dim]
+ * (host), the results token-major -- q [T][in_dim], d [T][in_dim/group], sums i32 [T][in_dim/16], bsum
+ * i16 [T][in_dim/32] (ActQ8K's per-32 sums, vecdot.rs:1849-1852) and, per 256 only, bs16 [T][in_dim/16]:
+ * per super-block eight f16 values floor(bsum_j / 64) followed by eight f16 values bsum_j mod 64, the
+ * K-quant GEMMs' first-pass operand.  The values are those of ActQ8K::quantize / ActQ8Flat::quantize
+ * (vecdot.rs:1858-1910, 2483-2525); only their 4-token interleave is not materialised.  sums, bsum
+ * and bs16 may be null. */
+int ogm_quantize_act_tokens(ogm_ctx *ctx, int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,
+                            int8_t *q, float *d, int32_t *sums, int16_t *bsum, uint16_t *bs16);
 /* Per (token, row, block) integer sums the matmul kernels form before any float is touched:
  * Q4_K and Q5_K: isum = sum_j sc_j * dot32_j and imin = sum_j m_j * bsum_j per super-block
  * (vecdot.rs:3152-3213); Q6_K and Q3_K: isum per super-block (vecdot.rs:3215-3241, 3273-3292),
@@ -267,9 +276,26 @@ int ogm_dequant_rows(ogm_ctx *ctx, const ogm_weight *w, uint32_t row0, uint32_t 
 int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *tok_embd, uint32_t first_token,
                        uint32_t pos0, uint32_t n_tokens, uint32_t *tokens_out, float *last_logits);
 
+/* The decode step's greedy pick on its own, for parity checks: index of the maximum of n logits (host
+ * pointers) as sampling::argmax takes it (engine/sampling.rs:336-343) -- Iterator::max_by over
+ * f32::total_cmp, so -0 < +0, a positive NaN beats every number, and of equal maxima the last wins. */
+int ogm_argmax(ogm_ctx *ctx, const float *logits, uint32_t n, uint32_t *out);
+
 /* The last decode's final hidden state, before the output norm ([n_embd] host f32; what
  * run_layers returns), for parity checks. */
 int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out);
+
+/* Debug capture for parity checks.  With capture on, every decode step also keeps the quantized
+ * activations each group of matmuls read (the int8 values and their scales, as the producing kernel
+ * left them): site 4*layer + 0 the q/k/v input, + 1 the wo input, + 2 the gate/up input, + 3 the down
+ * input, site 4*n_layer the vocabulary projection's input.  A test compares them with
+ * vecdot::quantize_act / quantize_act_k_row (vecdot.rs:79-126, 3030-3053) of the CPU forward pass and
+ * lets the CPU continue from the device's values where an f32 last-bit difference tipped a rounding.
+ * ogm_llama_debug_act copies one site of the last step: q has room for max(n_embd, n_ff,
+ * n_head*head_dim) values, d for a 32nd of that; *n receives the element count, *group 32 or 256. */
+int ogm_llama_debug_capture(ogm_ctx *ctx, ogm_llama *m, int enable);
+int ogm_llama_debug_act(ogm_ctx *ctx, ogm_llama *m, uint32_t site, int8_t *q, float *d, uint32_t *n,
+                        uint32_t *group);
 
 /* ---- GGUF reader -> uploader -------------------------------------------------------------------- */
 

@@ -84,6 +84,7 @@ def lib() -> C.CDLL:
         L.ogo_matmul.argtypes = mm
         L.ogo_matmul_decode.argtypes = mm
         L.ogo_matmul_dequant.argtypes = mm
+        L.ogo_gemv_act.argtypes = [C.c_uint32, u8p, sz, sz, sz, i8p, f32p, i32p, f32p, C.c_int]
         L.ogo_k_gemm_t.argtypes = [C.c_uint32, u8p, sz, sz, sz, f32p, sz, f32p]
         L.ogo_block_sums.argtypes = [C.c_uint32, u8p, sz, sz, sz, f32p, sz, i32p, i32p]
         _lib = L
@@ -299,6 +300,25 @@ def _mm(fn, ggml_type, raw, in_dim, out_dim, x, n_tokens, threads):
 def matmul(ggml_type, raw, in_dim, out_dim, x, n_tokens=1, threads=0) -> np.ndarray:
     """CpuBackend::matmul (backend/cpu.rs:445-458): y[n_tokens][out_dim]."""
     return _mm(lib().ogo_matmul, ggml_type, raw, in_dim, out_dim, x, n_tokens, threads)
+
+
+def gemv_act(ggml_type, raw, in_dim, out_dim, q, d, threads=0) -> np.ndarray:
+    """The single-token GEMV of CpuBackend::matmul over an activation that is already quantized:
+    q int8 [in_dim], d f32 [in_dim / 32] (per-32 types) or [in_dim / 256] (K-quants); the per-16 sums
+    are those of q (vecdot.rs:119-124).  Same dot_row / dot_k_row calls as `matmul` at one token."""
+    raw = _u8(raw)
+    bb, be = BLOCK_LAYOUT[ggml_type]
+    row_bytes = in_dim // be * bb
+    assert raw.size == row_bytes * out_dim, (raw.size, row_bytes, out_dim)
+    q = np.ascontiguousarray(q, np.int8).reshape(-1)
+    d = np.ascontiguousarray(d, np.float32).reshape(-1)
+    assert q.size == in_dim and d.size == in_dim // (32 if be == 32 else 256), (q.size, d.size)
+    sums = np.ascontiguousarray(q.astype(np.int32).reshape(-1, 16).sum(axis=1), np.int32)
+    y = np.empty(out_dim, np.float32)
+    rc = lib().ogo_gemv_act(ggml_type, _p(raw), row_bytes, in_dim, out_dim, _p(q), _p(d), _p(sums), _p(y), threads)
+    if rc != 0:
+        raise ValueError(f"oracle gemv_act rc={rc}")
+    return y
 
 
 def matmul_decode(ggml_type, raw, in_dim, out_dim, x, n_tokens=1, threads=0) -> np.ndarray:

@@ -123,11 +123,21 @@ def silu(x: np.ndarray) -> np.ndarray:
         return (x / (f32(1.0) + np.exp(-x, dtype=f32))).astype(f32)
 
 
+def to_cache(row: np.ndarray, dtype) -> np.ndarray:
+    """A K or V row as the cache keeps it.  The reference's host cache is f32 (kv_cache.rs:75-78); the
+    device build keeps f16 and saturates at +-65504 rather than storing an infinity."""
+    if dtype == np.float16:
+        row = np.clip(row, -65504.0, 65504.0)   # NaN passes through
+    return row.astype(dtype)
+
+
 def argmax(logits: np.ndarray) -> int:
-    """sampling.rs:336-343: max_by keeps the last of several equal maxima."""
-    logits = np.asarray(logits, f32)
-    m = logits.max()
-    return int(np.nonzero(logits == m)[0][-1])
+    """sampling.rs:336-343: max_by over f32::total_cmp keeps the last of several equal maxima.
+    total_cmp orders -NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN: compare the bit patterns as
+    sign-magnitude integers."""
+    bits = np.ascontiguousarray(logits, f32).view(np.int32).astype(np.int64)
+    keys = np.where(bits < 0, -(bits & 0x7FFFFFFF) - 1, bits)
+    return int(np.nonzero(keys == keys.max())[0][-1])
 
 
 @dataclass
@@ -168,6 +178,12 @@ class Model:
     # kv_hook(layer, pos, k_row, v_row) -> (k_row, v_row): lets a test look at the rows about to be
     # cached and replace them (by a device's rows that differ in the last f16 bit, say)
     kv_hook: object = None
+    # act_hook(site, x, group) -> (q, d) or None, at one token only: lets a test look at the f32 input
+    # of matmul site `site` (4*layer + 0 q/k/v, + 1 wo, + 2 gate/up, + 3 down; 4*n_layer the output
+    # projection) and hand back the quantized activation the matmuls of that site are to use (a
+    # device's, which may differ by one unit where an f32 last bit tipped a rounding).  `group` is the
+    # quantizer's group of the site's first matrix: 32 or 256.
+    act_hook: object = None
     k_cache: list = field(default_factory=list)   # per layer: list of rows
     v_cache: list = field(default_factory=list)
 
@@ -194,10 +210,24 @@ def forward(m: Model, X: np.ndarray, pos0: int):
     X = np.array(X, f32).reshape(-1, m.n_embd)
     T = X.shape[0]
     rows = lambda fn, A: np.stack([fn(A[t]) for t in range(T)])
-    mm = lambda w, A: _mm(w, A if T > 1 else A[0], T).reshape(T, -1)
+
+    def mms(site, ws, A):
+        """The matmuls of one site over the same input; with an act_hook (one token) they all read the
+        quantized activation the hook returns."""
+        n_tok = A.shape[0]
+        mm = lambda w, A: _mm(w, A if n_tok > 1 else A[0], n_tok).reshape(n_tok, -1)
+        if m.act_hook is None or n_tok != 1:
+            return [mm(w, A) for w in ws]
+        import oracle
+        group = 32 if oracle.BLOCK_LAYOUT[ws[0][0]][1] == 32 else 256
+        got = m.act_hook(site, A[0], group)
+        if got is None:
+            return [mm(w, A) for w in ws]
+        return [oracle.gemv_act(w[0], w[1], w[2], w[3], got[0], got[1]).reshape(1, -1) for w in ws]
+
     for li, L in enumerate(m.layers):
         normed = rows(lambda r: rmsnorm(r, L.attn_norm, m.rms_eps), X)
-        q, k, v = mm(L.wq, normed), mm(L.wk, normed), mm(L.wv, normed)
+        q, k, v = mms(4 * li, (L.wq, L.wk, L.wv), normed)
         if L.q_bias is not None:                       # llama.rs:757-765
             q = (q + np.asarray(L.q_bias, f32)).astype(f32)
         if L.k_bias is not None:
@@ -215,19 +245,19 @@ def forward(m: Model, X: np.ndarray, pos0: int):
             pos = pos0 + t
             qt = rope(q[t], m.n_head, m.head_dim, pos, m.rope_dim, m.rope_freq_base, m.rope_freq_factors, m.rope_neox)
             kt = rope(k[t], m.n_head_kv, m.head_dim, pos, m.rope_dim, m.rope_freq_base, m.rope_freq_factors, m.rope_neox)
-            k_row, v_row = kt.astype(m.kv_dtype), v[t].astype(m.kv_dtype)
+            k_row, v_row = to_cache(kt, m.kv_dtype), to_cache(v[t], m.kv_dtype)
             if m.kv_hook is not None:
                 k_row, v_row = m.kv_hook(li, pos, k_row, v_row)
             kc.append(k_row)
             vc.append(v_row)
             attn[t] = attention(qt, np.stack(kc).astype(f32), np.stack(vc).astype(f32), m.n_head, m.n_head_kv, m.head_dim)
-        X = (X + mm(L.wo, attn)).astype(f32)
+        X = (X + mms(4 * li + 1, (L.wo,), attn)[0]).astype(f32)
         normed2 = rows(lambda r: rmsnorm(r, L.ffn_norm, m.rms_eps), X)
-        gate, up = mm(L.w_gate, normed2), mm(L.w_up, normed2)
+        gate, up = mms(4 * li + 2, (L.w_gate, L.w_up), normed2)
         h = (silu(gate) * up).astype(f32)
-        X = (X + mm(L.w_down, h)).astype(f32)
+        X = (X + mms(4 * li + 3, (L.w_down,), h)[0]).astype(f32)
     last = rmsnorm(X[-1], m.output_norm, m.rms_eps)
-    return _mm(m.output, last), X[-1]
+    return mms(4 * len(m.layers), (m.output,), last.reshape(1, -1))[0].reshape(-1), X[-1]
 
 
 def decode_step(m: Model, x: np.ndarray, pos: int):

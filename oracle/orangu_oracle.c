@@ -900,6 +900,35 @@ static int gemv_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size
   return 0;
 }
 
+/* The single-token GEMV of gemv_t over an activation that is already quantized (q, d and the per-16
+ * sums as quantize_act / quantize_act_k_row leave them): the same dot_row / dot_k_row calls, so a
+ * test can continue from a device's int8 activations.  y is [out_dim]. */
+int ogo_gemv_act(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t in_dim, size_t out_dim,
+                 const int8_t *q, const float *d, const int32_t *sums, float *y, int n_threads) {
+  if (!ogo_supports(ggml_type, in_dim)) return -1;
+  int threads = pick_threads(n_threads);
+  long long n_out = (long long)out_dim;
+#pragma omp parallel for schedule(dynamic, 16) num_threads(threads)
+  for (long long oo = 0; oo < n_out; oo++) {
+    const uint8_t *row = raw + (size_t)oo * row_bytes;
+    float v;
+    if (ggml_type == OGO_TYPE_Q4_K)
+      v = DISPATCH(dot_k_row_q4_k, row, in_dim, q, d, sums, NULL, NULL);
+    else if (ggml_type == OGO_TYPE_Q5_K)
+      v = DISPATCH(dot_k_row_q5_k, row, in_dim, q, d, sums, NULL, NULL);
+    else if (ggml_type == OGO_TYPE_Q6_K)
+      v = DISPATCH(dot_k_row_q6_k, row, in_dim, q, d, NULL);
+    else if (ggml_type == OGO_TYPE_Q3_K)
+      v = DISPATCH(dot_k_row_q3_k, row, in_dim, q, d, NULL);
+    else if (ggml_type == OGO_TYPE_Q8_0)
+      v = DISPATCH(dot_q8_0, row, in_dim, q, d, NULL);
+    else
+      v = DISPATCH(dot_flat32, ggml_type, row, in_dim, q, d, NULL);
+    y[oo] = v;
+  }
+  return 0;
+}
+
 /* backend/cpu.rs:55-167 matmul_fused_into + :445-458 */
 int ogo_matmul(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t in_dim,
                size_t out_dim, const float *x, size_t n_tokens, float *y, int n_threads) {

@@ -132,6 +132,8 @@ int ogo_supports_flat(uint32_t ggml_type, size_t in_dim);   /* vecdot.rs:2456-24
 int ogo_matmul(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t in_dim,
                size_t out_dim, const float *x, size_t n_tokens, float *y, int n_threads);
                                                                     /* cpu.rs:55-245, 445-458 */
+int ogo_gemv_act(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t in_dim, size_t out_dim,
+                 const int8_t *q, const float *d, const int32_t *sums, float *y, int n_threads);
 int ogo_matmul_decode(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t in_dim,
                       size_t out_dim, const float *x, size_t n_tokens, float *y, int n_threads);
                                                                     /* cpu.rs:265-317 */

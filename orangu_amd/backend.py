@@ -208,6 +208,22 @@ class Mi355xBackend:
                     "ogm_quantize_act")
         return q, d, s
 
+    def quantize_act_tokens(self, x, in_dim: int, n_tokens: int, per_256: bool):
+        """The quantizer over a batch as the multi-token matmuls launch it: token-major
+        (q [T][in], d [T][in/group], sums [T][in/16], bsum [T][in/32], bs16 [T][in/16] or None)."""
+        x = np.ascontiguousarray(x, np.float32).reshape(n_tokens, in_dim)
+        g = 256 if per_256 else 32
+        q = np.empty((n_tokens, in_dim), np.int8)
+        d = np.empty((n_tokens, in_dim // g), np.float32)
+        s = np.empty((n_tokens, in_dim // 16), np.int32)
+        b = np.empty((n_tokens, in_dim // 32), np.int16)
+        h = np.empty((n_tokens, in_dim // 16), np.uint16) if per_256 else None
+        self._check(self._lib.ogm_quantize_act_tokens(self._ctx, int(per_256), x.ctypes.data, in_dim, n_tokens,
+                                                      q.ctypes.data, d.ctypes.data, s.ctypes.data, b.ctypes.data,
+                                                      h.ctypes.data if h is not None else None),
+                    "ogm_quantize_act_tokens")
+        return q, d, s, b, h
+
     def dump_block_sums(self, x, n_tokens: int, w: QuantMatrix):
         x = self._x(x, n_tokens, w)
         _, be = BLOCK_LAYOUT[w.ggml_type()]
@@ -274,6 +290,12 @@ class Mi355xBackend:
         """Releases a device copy made by upload_raw (cached uploads live as long as the backend)."""
         self._check(self._lib.ogm_weight_free(self._ctx, w_handle), "ogm_weight_free")
 
+    def evict(self, w: QuantMatrix):
+        """Frees the device copy of ``w`` and forgets its cache key.  The reference's backends never
+        evict (engine/backend/rocm.rs:329-350); tests that build multi-gigabyte models do."""
+        self.free_weight(self.upload(w))
+        self._keepalive.pop(w.cache_key(), None)
+
     def dequant_rows(self, w, row0: int, n_rows: int, in_dim: int | None = None) -> np.ndarray:
         """Rows of an uploaded matrix (a QuantMatrix, or a handle together with its in_dim) as f32,
         from the device copy (quant.rs dequantize_*)."""
@@ -288,6 +310,13 @@ class Mi355xBackend:
 
     def last_kernel(self) -> str:
         return self._lib.ogm_last_kernel(self._ctx).decode()
+
+    def argmax(self, logits: np.ndarray) -> int:
+        """sampling::argmax (engine/sampling.rs:336-343) on the device: the decode step's greedy pick."""
+        logits = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1)
+        out = C.c_uint32(0)
+        self._check(self._lib.ogm_argmax(self._ctx, logits.ctypes.data, logits.size, C.byref(out)), "ogm_argmax")
+        return int(out.value)
 
 
 class LlamaDecoder:
@@ -341,6 +370,7 @@ class LlamaDecoder:
                   "ogm_llama_create")
         self._h = h.value
         self.n_embd, self.n_vocab, self.kv_dim, self.n_layer = n_embd, n_vocab, n_head_kv * head_dim, len(layers)
+        self._act_width = max(n_embd, n_ff, n_head * head_dim)
 
     @classmethod
     def from_gguf(cls, be: "Mi355xBackend", gguf, max_ctx: int) -> "LlamaDecoder":
@@ -356,6 +386,7 @@ class LlamaDecoder:
         self._h, self.tok_embd, self.config = h.value, embd.value, cfg
         self.n_embd, self.n_vocab, self.n_layer = cfg.n_embd, cfg.n_vocab, cfg.n_layer
         self.kv_dim = cfg.n_head_kv * cfg.head_dim
+        self._act_width = max(cfg.n_embd, cfg.n_ff, cfg.n_head * cfg.head_dim)
         return self
 
     def kv_write(self, layer: int, pos0: int, k, v):
@@ -423,6 +454,22 @@ class LlamaDecoder:
         self._be._check(self._be._lib.ogm_llama_debug_hidden(self._be._ctx, self._h, out.ctypes.data),
                         "ogm_llama_debug_hidden")
         return out
+
+    def capture_acts(self, on: bool = True):
+        """Debug: keep the quantized activations every matmul group of a decode step reads."""
+        self._be._check(self._be._lib.ogm_llama_debug_capture(self._be._ctx, self._h, 1 if on else 0),
+                        "ogm_llama_debug_capture")
+
+    def act(self, site: int):
+        """(q int8 [n], d f32 [n / group], group) of matmul site ``site`` of the last decode step:
+        4*layer + 0 q/k/v input, + 1 wo input, + 2 gate/up input, + 3 down input; 4*n_layer the output
+        projection's input."""
+        q = np.empty(self._act_width, np.int8)
+        d = np.empty(self._act_width // 32 + 1, np.float32)
+        n, group = C.c_uint32(0), C.c_uint32(0)
+        self._be._check(self._be._lib.ogm_llama_debug_act(self._be._ctx, self._h, site, q.ctypes.data, d.ctypes.data,
+                                                          C.byref(n), C.byref(group)), "ogm_llama_debug_act")
+        return q[:n.value].copy(), d[:n.value // group.value].copy(), int(group.value)
 
     def close(self):
         if self._h:

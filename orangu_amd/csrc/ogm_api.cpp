@@ -131,14 +131,21 @@ static int ensure_act(ogm_ctx *ctx, uint32_t in_dim, uint32_t n_tokens) {
   return OGM_OK;
 }
 
-static OgmActDev act_view(ogm_ctx *ctx, uint32_t in_dim, int mode, uint32_t token0) {
+// The activations of token `token0` on in a token-major buffer set whose first token is `base`.
+static OgmActDev act_offset(const OgmActDev &base, uint32_t in_dim, int mode, uint32_t token0) {
   OgmActDev a;
-  a.q = (int8_t *)ctx->q.p + (size_t)token0 * in_dim;
-  a.d = (float *)ctx->d.p + (size_t)token0 * (in_dim / (mode == OGM_ACT_PER_32 ? 32 : 256));
-  a.sums = (int32_t *)ctx->sums.p + (size_t)token0 * (in_dim / 16);
-  a.bsum = (int16_t *)ctx->bsum.p + (size_t)token0 * (in_dim / 32);
-  a.bs16 = mode == OGM_ACT_PER_32 ? nullptr : (uint16_t *)ctx->bs16.p + (size_t)token0 * (in_dim / 16);
+  a.q = base.q + (size_t)token0 * in_dim;
+  a.d = base.d + (size_t)token0 * (in_dim / (mode == OGM_ACT_PER_32 ? 32 : 256));
+  a.sums = base.sums + (size_t)token0 * (in_dim / 16);
+  a.bsum = base.bsum + (size_t)token0 * (in_dim / 32);
+  a.bs16 = (mode == OGM_ACT_PER_32 || !base.bs16) ? nullptr : base.bs16 + (size_t)token0 * (in_dim / 16);
   return a;
+}
+
+static OgmActDev act_view(ogm_ctx *ctx, uint32_t in_dim, int mode, uint32_t token0) {
+  const OgmActDev base{(int8_t *)ctx->q.p, (float *)ctx->d.p, (int32_t *)ctx->sums.p, (int16_t *)ctx->bsum.p,
+                       (uint16_t *)ctx->bs16.p};
+  return act_offset(base, in_dim, mode, token0);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -398,7 +405,7 @@ struct Target {
 
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
                         hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
-                        const float *x_f32, const OgmGemvTail *tail = nullptr);
+                        const float *x_f32, const OgmGemvTail *tail = nullptr, const OgmActDev *act_base = nullptr);
 
 // Whether a single-token launch quantizes inside the GEMV (every workgroup repeats the
 // quantizer on its way in) instead of running the quantizer kernel first.  Off unless asked
@@ -435,9 +442,11 @@ static bool all_gemm_supported(const Target *tg, size_t n_tg, uint32_t n_tokens)
 
 // Enqueues the matmul kernels over the context's quantized activations (or, with x_f32, over
 // one token of f32 activations that the kernel quantizes itself).  Caller holds the lock.
+// act_base: the quantized activations to read instead of the context's scratch; such a call stays
+// on the GEMV kernels whatever the token count (the tiled GEMMs stage through context buffers).
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
                         hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
-                        const float *x_f32, const OgmGemvTail *tail) {
+                        const float *x_f32, const OgmGemvTail *tail, const OgmActDev *act_base) {
   const ogm_weight *w0 = tg[0].w;
   if (tail && (n_tokens != 1 || n_tg > OGM_GEMV_MAX_MATS)) return fail(ctx, OGM_ERR_INVALID, "a GEMV tail needs one launch of one token");
   const int mode = act_mode_for(w0->ggml_type);
@@ -447,7 +456,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   const uint32_t t0 = w0->ggml_type;
   const uint32_t gemm_from = ctx->tune_gemm_min_tokens ? (uint32_t)ctx->tune_gemm_min_tokens
                              : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 9u : 17u;
-  if (gemm_order && !dump_isum && !dump_imin && n_tokens >= gemm_from &&
+  if (gemm_order && !dump_isum && !dump_imin && !act_base && n_tokens >= gemm_from &&
       all_gemm_supported(tg, n_tg, n_tokens)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
     int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w0->in_dim, n_tokens));
@@ -491,7 +500,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       a.wt = tg[g0].w->dev;
       a.in_dim = w0->in_dim;
       a.out_dim = tg[g0].w->out_dim;
-      a.act = act_view(ctx, w0->in_dim, mode, t0);
+      a.act = act_base ? act_offset(*act_base, w0->in_dim, mode, t0) : act_view(ctx, w0->in_dim, mode, t0);
       a.n_tokens = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
       a.y = tg[g0].y + (size_t)t0 * a.out_dim;
       a.gemm_order = gemm_order;
@@ -754,6 +763,37 @@ extern "C" int ogm_quantize_act(ogm_ctx *ctx, int mode, const float *x, size_t n
   return OGM_OK;
 }
 
+// The quantizer as the multi-token matmuls launch it (one grid row per token), with everything it
+// writes copied back.
+extern "C" int ogm_quantize_act_tokens(ogm_ctx *ctx, int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,
+                                       int8_t *q, float *d, int32_t *sums, int16_t *bsum, uint16_t *bs16) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (mode != OGM_ACT_PER_32 && mode != OGM_ACT_PER_256) return fail(ctx, OGM_ERR_INVALID, "bad mode");
+  const uint32_t group = mode == OGM_ACT_PER_32 ? 32u : 256u;
+  if (n_tokens == 0) return OGM_OK;
+  if (!x || !q || !d) return fail(ctx, OGM_ERR_INVALID, "null pointer");
+  if (in_dim == 0 || in_dim % group != 0 || (uint64_t)in_dim * n_tokens > 0x7FFFFFFFu || n_tokens > 65535u)
+    return fail(ctx, OGM_ERR_INVALID, "in_dim is not a whole number of groups, or the batch is too large");
+  if (bs16 && mode != OGM_ACT_PER_256) return fail(ctx, OGM_ERR_INVALID, "the f16 sub-block sums exist per 256 only");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  const size_t n = (size_t)in_dim * n_tokens;
+  int rc;
+  if ((rc = ensure_dev(ctx, ctx->x, n * 4)) != OGM_OK) return rc;
+  if ((rc = ensure_act(ctx, in_dim, n_tokens)) != OGM_OK) return rc;
+  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, x, n * 4, hipMemcpyHostToDevice, ctx->stream));
+  HIPCHK(ctx, ogm_launch_quantize(mode, (const float *)ctx->x.p, in_dim, n_tokens, act_view(ctx, in_dim, mode, 0),
+                                  ctx->stream));
+  ctx->act_mode = -1;   // the scratch no longer holds what ogm_act_quantize_dev left
+  HIPCHK(ctx, hipMemcpyAsync(q, ctx->q.p, n, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipMemcpyAsync(d, ctx->d.p, n / group * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (sums) HIPCHK(ctx, hipMemcpyAsync(sums, ctx->sums.p, n / 16 * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (bsum) HIPCHK(ctx, hipMemcpyAsync(bsum, ctx->bsum.p, n / 32 * 2, hipMemcpyDeviceToHost, ctx->stream));
+  if (bs16) HIPCHK(ctx, hipMemcpyAsync(bs16, ctx->bs16.p, n / 16 * 2, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return OGM_OK;
+}
+
 extern "C" int ogm_dump_block_sums(ogm_ctx *ctx, const ogm_weight *w, const float *x,
                                    uint32_t n_tokens, int32_t *isum, int32_t *imin) {
   int rc = check_matmul_args(ctx, w, x, isum, n_tokens);
@@ -833,6 +873,13 @@ struct ogm_llama {
     bool ready = false;
   } pf;
   uint32_t max_splits = 0;
+  // debug capture (ogm_llama_debug_capture): the quantized activations every matmul group of the
+  // last decode step read, site after site, cap_width bytes of q and cap_width / 32 scales each
+  bool cap_on = false;
+  int8_t *cap_q = nullptr;   // allocated when capture is first switched on, freed with the model
+  float *cap_d = nullptr;
+  uint32_t cap_width = 0;
+  std::vector<uint32_t> cap_n, cap_group;   // per site: elements and quantizer group of the last step
   std::vector<void *> allocs;
 };
 
@@ -1018,6 +1065,20 @@ extern "C" int ogm_llama_kv_read(ogm_ctx *ctx, ogm_llama *m, uint32_t layer, uin
   return OGM_OK;
 }
 
+// Debug capture: keeps what the activation scratch holds right now (n elements quantized per
+// `mode`) as the input of matmul site `site`.  A no-op unless capture is on.
+static int llama_capture(ogm_ctx *ctx, ogm_llama *m, uint32_t site, uint32_t n, int mode, hipStream_t s) {
+  if (!m->cap_on) return OGM_OK;
+  const uint32_t group = mode == OGM_ACT_PER_32 ? 32u : 256u;
+  const OgmActDev a = act_view(ctx, n, mode, 0);
+  HIPCHK(ctx, hipMemcpyAsync(m->cap_q + (size_t)site * m->cap_width, a.q, n, hipMemcpyDeviceToDevice, s));
+  HIPCHK(ctx, hipMemcpyAsync(m->cap_d + (size_t)site * (m->cap_width / 32u), a.d, (size_t)(n / group) * 4,
+                             hipMemcpyDeviceToDevice, s));
+  m->cap_n[site] = n;
+  m->cap_group[site] = group;
+  return OGM_OK;
+}
+
 // One matmul group of the step over the activations the previous kernel quantized.
 static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, hipStream_t s,
                         const OgmGemvTail *tail = nullptr) {
@@ -1079,8 +1140,9 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
                                         act_view(ctx, c.n_embd, mode_qkv, 0), s));
     const ogm_weight *w3[3] = {L.wq, L.wk, L.wv};
     float *y3[3] = {m->q, m->k, m->v};
-    int rc = llama_matmul(ctx, w3, y3, 3, s);
+    int rc = llama_capture(ctx, m, 4 * l, c.n_embd, mode_qkv, s);
     if (rc != OGM_OK) return rc;
+    if ((rc = llama_matmul(ctx, w3, y3, 3, s)) != OGM_OK) return rc;
     const int mode_o = act_mode_for(L.wo->ggml_type);
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, m->rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
@@ -1091,6 +1153,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
       return fail(ctx, OGM_ERR_UNSUPPORTED, "w_gate and w_up must share an activation mode");
     const ogm_weight *w1[1] = {L.wo};
     float *y1[1] = {m->proj};
+    if ((rc = llama_capture(ctx, m, 4 * l + 1, qd, mode_o, s)) != OGM_OK) return rc;
     OgmGemvTail tail;
     tail.ticket = m->attn_tickets + c.n_head_kv;
     if (tail_ok(L.wo, c.n_embd, mode_ff)) {
@@ -1109,6 +1172,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     const ogm_weight *w2[2] = {L.w_gate, L.w_up};
     float *y2[2] = {m->gate, m->up};
     const int mode_d = act_mode_for(L.w_down->ggml_type);
+    if ((rc = llama_capture(ctx, m, 4 * l + 2, c.n_embd, mode_ff, s)) != OGM_OK) return rc;
     if (fuse && mode_d == OGM_ACT_PER_256 && L.w_gate->ggml_type == L.w_up->ggml_type &&
         block_elems_of(L.w_gate->ggml_type) == 256) {
       tail.kind = OGM_TAIL_SWIGLU;
@@ -1123,6 +1187,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
                                           act_view(ctx, c.n_ff, mode_d, 0), s));
     }
     const ogm_weight *wd[1] = {L.w_down};
+    if ((rc = llama_capture(ctx, m, 4 * l + 3, c.n_ff, mode_d, s)) != OGM_OK) return rc;
     // the next norm: the next layer's attention norm, or the output norm after the last layer
     const bool last_layer = l + 1 == c.n_layer;
     const int mode_next = last_layer ? mode_out : act_mode_for(m->layers[l + 1].wq->ggml_type);
@@ -1146,8 +1211,9 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   float *lg = logits_dev ? logits_dev : m->logits;
   const ogm_weight *wo_[1] = {m->output};
   float *yo[1] = {lg};
-  int rc = llama_matmul(ctx, wo_, yo, 1, s);
+  int rc = llama_capture(ctx, m, 4 * c.n_layer, c.n_embd, mode_out, s);
   if (rc != OGM_OK) return rc;
+  if ((rc = llama_matmul(ctx, wo_, yo, 1, s)) != OGM_OK) return rc;
   if (argmax_dev) HIPCHK(ctx, ogm_launch_argmax(lg, c.n_vocab, m->amax_scratch, argmax_dev, s));
   // the activation scratch no longer holds what ogm_act_quantize_dev left there
   ctx->act_mode = -1;
@@ -1188,6 +1254,67 @@ extern "C" int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out) 
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   // the output norm added the last block's output to x in place before normalising
   HIPCHK(ctx, hipMemcpy(x_out, m->x, (size_t)m->cfg.n_embd * 4, hipMemcpyDeviceToHost));
+  return OGM_OK;
+}
+
+extern "C" int ogm_llama_debug_capture(ogm_ctx *ctx, ogm_llama *m, int enable) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  if (!enable || m->cap_q) {   // the buffers stay with the model until it is destroyed
+    m->cap_on = enable != 0;
+    return OGM_OK;
+  }
+  const ogm_llama_config &c = m->cfg;
+  const uint32_t qd = c.n_head * c.head_dim;
+  uint32_t widest = c.n_embd > c.n_ff ? c.n_embd : c.n_ff;
+  if (qd > widest) widest = qd;
+  const size_t sites = (size_t)4 * c.n_layer + 1;
+  m->cap_width = (widest + 31u) & ~31u;
+  int rc = llama_alloc(ctx, m, (void **)&m->cap_q, sites * m->cap_width);
+  if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)&m->cap_d, sites * (m->cap_width / 32u) * 4);
+  if (rc != OGM_OK) {
+    m->cap_q = nullptr;
+    m->cap_d = nullptr;
+    return rc;
+  }
+  m->cap_n.assign(sites, 0u);
+  m->cap_group.assign(sites, 0u);
+  m->cap_on = true;
+  return OGM_OK;
+}
+
+extern "C" int ogm_llama_debug_act(ogm_ctx *ctx, ogm_llama *m, uint32_t site, int8_t *q, float *d, uint32_t *n,
+                                   uint32_t *group) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !q || !d || !n || !group) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (!m->cap_q) return fail(ctx, OGM_ERR_INVALID, "capture was never on (ogm_llama_debug_capture)");
+  if (site >= m->cap_n.size() || m->cap_n[site] == 0) return fail(ctx, OGM_ERR_INVALID, "no such site in the last decode step");
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  *n = m->cap_n[site];
+  *group = m->cap_group[site];
+  HIPCHK(ctx, hipMemcpy(q, m->cap_q + (size_t)site * m->cap_width, *n, hipMemcpyDeviceToHost));
+  HIPCHK(ctx, hipMemcpy(d, m->cap_d + (size_t)site * (m->cap_width / 32u), (size_t)(*n / *group) * 4, hipMemcpyDeviceToHost));
+  return OGM_OK;
+}
+
+extern "C" int ogm_argmax(ogm_ctx *ctx, const float *logits, uint32_t n, uint32_t *out) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!logits || !out || n == 0) return fail(ctx, OGM_ERR_INVALID, "null pointer or no logits");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  int rc;
+  if ((rc = ensure_dev(ctx, ctx->x, (size_t)n * 4)) != OGM_OK) return rc;
+  if ((rc = ensure_dev(ctx, ctx->isum, 513 * 4)) != OGM_OK) return rc;   // 512 scratch words + the result
+  uint32_t *scratch = (uint32_t *)ctx->isum.p;
+  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, logits, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
+  HIPCHK(ctx, ogm_launch_argmax((const float *)ctx->x.p, n, scratch, scratch + 512, ctx->stream));
+  HIPCHK(ctx, hipMemcpyAsync(out, scratch + 512, 4, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   return OGM_OK;
 }
 

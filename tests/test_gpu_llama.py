@@ -3,14 +3,16 @@ oracle/llama_ref.py on the same seeded model.  The matmuls inside are bit-exact 
 test_gpu_parity.py); the element-wise kernels use tree reductions and the device's exp / sin /
 cos, so the bar here is a tolerance: hidden state and logits within 2e-4 of the largest magnitude
 (stated in `close`), greedy token equal unless the CPU's top two logits are within that tolerance.
+Every decode step holds that bound; there is no looser allowance.
 
 Two roundings inside the step are discontinuous, and an f32 difference in the last bit upstream can
-tip either: the f16 rounding of a cache row (handled in `step_both`: the CPU side checks its row
-against the device's and continues with the device's) and the int8 rounding of one activation
-element in a quantizer (about 1e-5 per element and quantizer call).  The second moves every output
-of that matmul by one quantizer step of one input times its weights (with the synthetic Q8_0
-weights here: up to 4e-3 of the largest output); `close` and the cache-row check therefore let ONE
-step per test go up to 1e-2, and fail on the second: an error of the code shows at every step."""
+tip either: the f16 rounding of a cache row and the int8 rounding of an activation element in a
+quantizer.  `step_both` therefore runs the two sides in lock-step at exactly those points: the
+device goes first with its debug capture on; the CPU restatement then checks each cache row it is
+about to append against the device's (equal up to one f16 step on a few elements) and each
+activation it is about to quantize against the device's int8 values and scales (equal up to one
+unit on a few elements, scales to 1e-5), and continues from the device's.  What is compared at the
+end is then the arithmetic between those points, free of the two amplifiers."""
 import sys
 
 import numpy as np
@@ -22,14 +24,6 @@ from oracle import llama_ref as R
 pytestmark = pytest.mark.gpu
 f32 = np.float32
 TOL = 2e-4
-LOOSE = 1e-2
-SOFT = {"steps": set()}   # steps of the running test that used the looser bound
-
-
-@pytest.fixture(autouse=True)
-def fresh_soft_budget():
-    SOFT["steps"] = set()
-    yield
 
 
 def say(*a):
@@ -50,11 +44,6 @@ def close(got, want, what):
     scale = np.abs(want).max() + 1e-30
     err = np.abs(got - want).max() / scale
     assert np.isfinite(got).all(), what
-    if TOL < err <= LOOSE:
-        SOFT["steps"].add(what.split(":")[0])
-        say(f"{what}: error {err:.3e} above {TOL:g}: taken as one flipped activation rounding")
-        assert len(SOFT["steps"]) <= 1, f"{what}: a second step above {TOL:g} ({sorted(SOFT['steps'])})"
-        return err
     assert err <= TOL, f"{what}: max error {err:.3e} of the largest magnitude {scale:.3e}"
     return err
 
@@ -103,15 +92,22 @@ def build(be, *, n_embd, n_head, n_kv, hd, n_ff, n_vocab, n_layer, types, max_ct
 
 
 def step_both(ref, dev, x, pos, what):
-    """One step on both sides.  The device goes first; the CPU restatement then checks each cache
-    row it is about to append against the device's (equal, or for a few elements the neighbouring
-    f16 value: an f32 difference in the last bits can fall either side of an f16 rounding
-    boundary; on top of that 1e-5 of the row's largest magnitude, a hundredth of the tolerance
-    the f32 outputs are held to) and continues with the device's row, so that such a bit does not blur the
-    comparison of everything downstream."""
+    """One step on both sides, in lock-step at the two discontinuous roundings (module docstring).
+    The device goes first.  The CPU restatement then
+      * checks each cache row it is about to append against the device's: equal, or for a few
+        elements the neighbouring f16 value (an f32 difference in the last bits can fall either
+        side of an f16 rounding boundary), plus 1e-5 of the row's largest magnitude; and
+      * checks each activation it is about to quantize (vecdot::quantize_act / quantize_act_k_row)
+        against the int8 values and scales the device's producing kernel left: scales within 1e-5,
+        values equal except for a few elements one unit apart;
+    and continues from the device's row and the device's int8 activation."""
+    import oracle
+    dev.capture_acts(True)
     got_logits, got_tok = dev.decode(x, pos)
     got_hidden = dev.hidden()
     rows = [dev.kv_read(l, pos, 1) for l in range(dev.n_layer)]
+    acts = [dev.act(site) for site in range(4 * dev.n_layer + 1)]
+    dev.capture_acts(False)
 
     def hook(li, p, k_row, v_row):
         out = []
@@ -119,24 +115,37 @@ def step_both(ref, dev, x, pos, what):
             a, b = mine.astype(np.float64), theirs.astype(np.float64)
             ulp = np.spacing(np.maximum(np.abs(mine), np.abs(theirs)).astype(np.float16)).astype(np.float64)
             off = a != b
-            # the f32 value's own error follows the row's size; beyond that, a flipped activation
-            # rounding in an earlier layer of this step shows here first (see the module docstring)
             rowmax = np.abs(b).max()
-            if not (np.abs(a - b) <= ulp + 1e-5 * rowmax).all():
-                assert (np.abs(a - b) <= ulp + LOOSE * rowmax).all(), \
-                    f"{what}: layer {li} {name} cache row differs by more than one f16 step and the f32 budget"
-                SOFT["steps"].add(what)
-                say(f"{what}: layer {li} {name} cache row off by {np.abs(a - b).max() / rowmax:.2e} of its largest "
-                    "value: taken as one flipped activation rounding")
-                assert len(SOFT["steps"]) <= 1, f"{what}: a second step above the tight bound ({sorted(SOFT['steps'])})"
-            elif what not in SOFT["steps"]:
-                assert off.mean() <= 0.05, f"{what}: layer {li} {name} cache row: {off.sum()} of {off.size} elements differ"
+            # f32 budget: 1e-5 of the row's largest value, plus what one ulp of a pair's frequency
+            # (powf is not correctly rounded everywhere) does to the angle p * freq: p * 2^-23 radians
+            budget = (1e-5 + (p * 2.0 ** -23 if name == "k" else 0.0)) * rowmax
+            assert (np.abs(a - b) <= ulp + budget).all(), \
+                f"{what}: layer {li} {name} cache row differs by more than one f16 step and the f32 budget " \
+                f"(worst {np.abs(a - b).max():.3g}, allowed {(ulp + budget)[np.abs(a - b).argmax()]:.3g})"
+            assert off.mean() <= 0.05 + (0.5 if name == "k" and p >= 1024 else 0.0), f"{what}: layer {li} {name} cache row: {off.sum()} of {off.size} elements differ"
             out.append(theirs.copy())
         return out
 
+    def act_hook(site, xin, group):
+        q_dev, d_dev, g_dev = acts[site]
+        assert g_dev == group and q_dev.size == xin.size, f"{what}: site {site}: quantizer group or width"
+        q_cpu, d_cpu, _ = (oracle.quantize_act if group == 32 else oracle.quantize_act_k_row)(xin)
+        assert np.allclose(d_dev, d_cpu, rtol=1e-5, atol=1e-30), f"{what}: site {site}: activation scales"
+        diff = np.abs(q_dev.astype(np.int32) - q_cpu.astype(np.int32))
+        n_off = int((diff != 0).sum())
+        assert diff.max() <= 1 and n_off <= max(3, q_dev.size // 500), \
+            f"{what}: site {site}: {n_off} of {q_dev.size} int8 activations differ, by up to {diff.max()}"
+        if n_off:
+            say(f"{what}: site {site}: {n_off} int8 activation(s) one unit apart; the CPU continues from the device's")
+        return q_dev, d_dev
+
+    ref.act_hook = act_hook
     ref.kv_hook = hook
-    want_logits, want_hidden = R.decode_step(ref, x, pos)
-    ref.kv_hook = None
+    try:
+        want_logits, want_hidden = R.decode_step(ref, x, pos)
+    finally:
+        ref.kv_hook = None
+        ref.act_hook = None
     e1 = close(got_hidden, want_hidden, f"{what}: hidden state")
     e2 = close(got_logits, want_logits, f"{what}: logits")
     top = np.sort(want_logits)[-2:]
@@ -215,6 +224,77 @@ def test_decode_over_a_prefilled_cache_with_several_attention_chunks(be):
             ref.v_cache[l] = [r.astype(np.float16) for r in v]
         for pos in (300, 301, 302):
             step_both(ref, dev, rng.standard_normal(1024).astype(f32), pos, f"prefilled pos {pos}")
+    finally:
+        dev.close()
+
+
+def test_llama_8b_shaped_layers_at_context_2048(be):
+    """Config 5 at its real shapes: a two-layer prefix of the 8B-shaped Q4_K_M-like model (hidden 4096,
+    32 query heads over 8 K/V heads of 128, FFN 14336 with a Q6_K down projection, the Q6_K 128256-row
+    output, RoPE base 500000) over an f16 cache holding 2048 random positions, two decode steps
+    against the CPU restatement."""
+    n_embd, n_head, n_kv, hd, n_ff, n_vocab, ctx = 4096, 32, 8, 128, 14336, 128256, 2048
+    from orangu_amd import LlamaDecoder, QuantMatrix
+    rng = np.random.default_rng(515)
+    shapes = {"wq": (Q4_K, n_embd, n_embd), "wk": (Q4_K, n_embd, n_kv * hd), "wv": (Q4_K, n_embd, n_kv * hd),
+              "wo": (Q4_K, n_embd, n_embd), "w_gate": (Q4_K, n_embd, n_ff), "w_up": (Q4_K, n_embd, n_ff),
+              "w_down": (Q6_K, n_ff, n_embd)}
+    order = ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")
+    ref_layers, dev_layers = [], []
+    for l in range(2):
+        w = {k: (t, synth_weights(t, i, o, seed=600 + 10 * l + n), i, o) for n, (k, (t, i, o)) in enumerate(shapes.items())}
+        norms = [(1 + 0.05 * rng.standard_normal(n_embd)).astype(f32) for _ in range(2)]
+        ref_layers.append(R.Layer(*[w[k] for k in order], *norms))
+        dev_layers.append({**{k: QuantMatrix(w[k][1], w[k][0], w[k][2], w[k][3]) for k in order},
+                           "attn_norm": norms[0], "ffn_norm": norms[1]})
+    out_norm = (1 + 0.05 * rng.standard_normal(n_embd)).astype(f32)
+    out = (Q6_K, synth_weights(Q6_K, n_embd, n_vocab, seed=699), n_embd, n_vocab)
+    ref = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 500000.0, ref_layers, out_norm, out)
+    ref.reset()
+    out_qm = QuantMatrix(out[1], out[0], out[2], out[3])
+    dev = LlamaDecoder(be, n_embd=n_embd, n_head=n_head, n_head_kv=n_kv, head_dim=hd, n_ff=n_ff, n_vocab=n_vocab,
+                       max_ctx=ctx + 2, rms_eps=1e-5, rope_freq_base=500000.0, layers=dev_layers,
+                       output_norm=out_norm, output=out_qm)
+    try:
+        for l in range(2):
+            k = rng.standard_normal((ctx, n_kv * hd)).astype(f32)
+            v = rng.standard_normal((ctx, n_kv * hd)).astype(f32)
+            dev.kv_write(l, 0, k, v)
+            ref.k_cache[l] = [r.astype(np.float16) for r in k]
+            ref.v_cache[l] = [r.astype(np.float16) for r in v]
+        for pos in (ctx, ctx + 1):
+            step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"8B shapes pos {pos}")
+    finally:
+        dev.close()
+        for L in dev_layers:   # 0.9 GB of weights: give them back before the next test
+            for k in order:
+                be.evict(L[k])
+        be.evict(out_qm)
+
+
+def test_cache_rows_beyond_the_f16_range_saturate(be):
+    """K/V components beyond +-65504 are cached as +-65504, not as infinities: rows handed over from
+    the host and rows the decode step writes itself (a v bias of 1e5), and the step after them stays
+    finite and agrees with the CPU restatement, whose f16 cache saturates the same way."""
+    n_kv, hd = 2, 64
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=300, n_layer=2,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=16, seed=77, pre=("v_bias",),
+                          pre_scale={"v_bias": 500.0})
+    try:
+        k = rng.standard_normal((3, n_kv * hd)).astype(f32)
+        v = rng.standard_normal((3, n_kv * hd)).astype(f32)
+        v[1, 7], v[2, 9], k[0, 3] = 1.0e6, -7.0e4, 65519.0
+        for l in range(2):
+            dev.kv_write(l, 0, k, v)
+            ref.k_cache[l] = [R.to_cache(r, np.float16) for r in k]
+            ref.v_cache[l] = [R.to_cache(r, np.float16) for r in v]
+        kb, vb = dev.kv_read(0, 0, 3)
+        assert vb.view(np.uint16)[1, 7] == 0x7BFF and vb.view(np.uint16)[2, 9] == 0xFBFF and kb.view(np.uint16)[0, 3] == 0x7BFF
+        for pos in (3, 4):
+            step_both(ref, dev, rng.standard_normal(256).astype(f32), pos, f"saturated cache pos {pos}")
+        _, vb = dev.kv_read(1, 3, 2)
+        assert np.isfinite(vb.astype(f32)).all()
+        assert (np.abs(vb.astype(f32)) == 65504.0).any(), "the bias was meant to push some v components out of range"
     finally:
         dev.close()
 
@@ -554,7 +634,8 @@ def test_prefill_attention_with_queries_beyond_f16(be, hd):
     assert err <= 2e-5
 
 
-def model_gguf(ref, arch, *, n_ctx=4096, tok_embd=None, vec_type=0, omit=(), extra_kvs=(), explicit=True):
+def model_gguf(ref, arch, *, n_ctx=4096, tok_embd=None, vec_type=0, omit=(), extra_kvs=(), explicit=True,
+               override_kvs=None):
     """A reference model as the bytes of a GGUF file with the tensor names and metadata keys
     LlamaModel::load_with_backend and read_model_config read (llama.rs:123-220, loader.rs:1652-1714).
     vec_type 0 stores the vectors as F32, 1 as F16."""
@@ -571,6 +652,9 @@ def model_gguf(ref, arch, *, n_ctx=4096, tok_embd=None, vec_type=0, omit=(), ext
     else:
         kvs.append(kv("tokenizer.ggml.tokens", 9, u32(8) + u64(ref.n_vocab) + b"".join(gstr("t%d" % i) for i in range(ref.n_vocab))))
     kvs += list(extra_kvs)
+    if override_kvs:   # {key suffix: encoded key/value}: replaces that key's entry
+        kvs = [k for k in kvs if not any(k.startswith(gstr(f"{arch}.{suffix}")) for suffix in override_kvs)]
+        kvs += list(override_kvs.values())
     tensors = []
 
     def mat(name, w):
@@ -691,6 +775,13 @@ def test_gguf_model_loading_errors(be, tmp_path):
     ref.n_head = 0                               # head_count must be nonzero
     with pytest.raises(OgmError, match="nonzero"):
         load(model_gguf(ref, "llama"))
+    ref.n_head = 4
+    # hyperparameters that do not fit 32 bits (or whose product does not) are refused before any upload
+    from test_gguf_cpu import u64
+    for key, value in (("attention.head_count", 1 << 32), ("attention.head_count_kv", (1 << 32) + 2),
+                       ("attention.key_length", 1 << 31), ("rope.dimension_count", 1 << 40)):
+        with pytest.raises(OgmError, match="out of range"):
+            load(model_gguf(ref, "llama", override_kvs={key: kv(f"llama.{key}", 10, u64(value))}))
 
 
 @pytest.mark.parametrize("t,in_dim,out_dim", [

@@ -254,6 +254,63 @@ def test_matmul_batch_equals_single_calls_and_stripes(be):
         assert_bits(y, be.matmul_decode(op.x, op.n_tokens, op.w), "decode batch")
 
 
+def test_matmul_batch_with_an_op_without_tokens_in_front(be):
+    """An op with n_tokens == 0 brings no input and must not stand in for the input of the op
+    behind it (both would otherwise sit at the same staging offset)."""
+    from orangu_amd import MatmulOp
+    in_dim = 512
+    w = qm(np.concatenate([fixture_row(Q4_K, in_dim, 3 + o) for o in range(7)]), Q4_K, in_dim, 7)
+    w6 = qm(np.concatenate([fixture_row(Q6_K, in_dim, 5 + o) for o in range(4)]), Q6_K, in_dim, 4)
+    xa, xb = activations_t(in_dim, 1), np.concatenate([activations_t(in_dim, 2 + j) for j in range(3)])
+    empty = np.zeros(0, np.float32)
+    for ops in ([MatmulOp(empty, 0, w), MatmulOp(xa, 1, w), MatmulOp(xb, 3, w6)],
+                [MatmulOp(xa, 1, w), MatmulOp(empty, 0, w6), MatmulOp(xb, 3, w6), MatmulOp(empty, 0, w)],
+                [MatmulOp(empty, 0, w), MatmulOp(empty, 0, w6)]):
+        for decode in (False, True):
+            outs = (be.matmul_batch_decode if decode else be.matmul_batch)(ops)
+            for op, y in zip(ops, outs):
+                assert np.asarray(y).size == op.n_tokens * op.w.out_dim
+                if op.n_tokens:
+                    want = (oracle.matmul_decode if decode else oracle.matmul)(
+                        op.w.ggml_type(), op.w.raw_bytes(), in_dim, op.w.out_dim, op.x, op.n_tokens)
+                    assert_bits(y, want, "batch with an empty op")
+
+
+@pytest.mark.parametrize("T", [2, 5, 9])
+@pytest.mark.parametrize("in_dim", [256, 1024, 4096])
+def test_multi_token_quantizer_matches_act_q8k_and_act_q8flat(be, T, in_dim):
+    """The quantizer as the multi-token matmuls launch it, against ActQ8K::quantize and
+    ActQ8Flat::quantize (vecdot.rs:1858-1910, 2483-2525): int8 values, scales and the per-32 sums bit
+    for bit (the reference's 4-token interleave undone on the host), and the f16 pairs
+    (floor(bsum / 64), bsum mod 64) the K-quant GEMMs' first pass reads."""
+    x = synth_x(T, in_dim, seed=40 + T).reshape(T, in_dim)
+    x[0, :32] = 0.0                       # an all-zero block: scale 0
+    x[T - 1, 5] = np.float32("nan")       # NaN quantizes to 0 and does not enter the maximum
+    x[T - 1, 40] = 3.0e38
+    # per 256
+    q, d, sums, bsum, bs16 = be.quantize_act_tokens(x, in_dim, T, True)
+    wq, wd, wb = oracle.act_q8k_quantize(x, in_dim, T)     # [tile][in/32][4][32], [tile][in/256][4], [tile][in/256][4][8]
+    for t in range(T):
+        tl, k = divmod(t, 4)
+        assert np.array_equal(q[t], wq[tl, :, k, :].reshape(-1)), f"token {t}: q"
+        assert np.array_equal(d[t].view(np.uint32), wd[tl, :, k].view(np.uint32)), f"token {t}: d"
+        assert np.array_equal(bsum[t], wb[tl, :, k, :].reshape(-1)), f"token {t}: bsum"
+        rq, rd, rs = oracle.quantize_act_k_row(x[t])      # the decode quantizer gives the same values
+        assert np.array_equal(q[t], rq) and np.array_equal(sums[t], rs)
+        b = bsum[t].astype(np.int32).reshape(-1, 8)
+        h = bs16[t].view(np.float16).astype(np.float64).reshape(-1, 16)
+        assert np.array_equal(h[:, :8], b >> 6) and np.array_equal(h[:, 8:], b & 63), f"token {t}: bs16"
+    # per 32
+    q, d, sums, bsum, _ = be.quantize_act_tokens(x, in_dim, T, False)
+    wq, wd = oracle.act_q8flat_quantize(x, in_dim, T)      # [tile][in/32][4][32], [tile][in/32][4]
+    for t in range(T):
+        tl, k = divmod(t, 4)
+        assert np.array_equal(q[t], wq[tl, :, k, :].reshape(-1)), f"token {t}: q (per 32)"
+        assert np.array_equal(d[t].view(np.uint32), wd[tl, :, k].view(np.uint32)), f"token {t}: d (per 32)"
+        assert np.array_equal(bsum[t], q[t].astype(np.int32).reshape(-1, 32).sum(axis=1))
+        assert np.array_equal(sums[t], q[t].astype(np.int32).reshape(-1, 16).sum(axis=1))
+
+
 def test_row_views_share_bytes_but_not_handles(be):
     """QuantMatrix::rows (loader.rs:627-646): a view's cache key differs from its parent's."""
     in_dim, out_dim = 512, 12
@@ -303,6 +360,78 @@ def test_benchmark_shapes_match_cpu(be, t, in_dim, out_dim):
         be.set_tuning("gemv_wg_waves", waves)
         assert_bits(be.matmul(x, 1, w), want, f"wg_waves={waves}")
     be.set_tuning("gemv_wg_waves", 0)
+
+
+@pytest.mark.parametrize("out_dim", [4096, 1024])
+@pytest.mark.parametrize("T", [4, 8])
+def test_q4k_attention_projections_at_verify_batches(be, out_dim, T):
+    """Config 3: the Q4_K attention projections 4096 -> 4096 (q / o) and 4096 -> 1024 (k / v) at the
+    speculative-verify batches 4 and 8, full size, through Backend::matmul (GEMM float order) and
+    Backend::matmul_decode (each row the single-token kernel): bit for bit."""
+    in_dim = 4096
+    raw = synth_weights(Q4_K, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T)
+    w = qm(raw, Q4_K, in_dim, out_dim)
+    say("verify batch", out_dim, T)
+    got = be.matmul(x, T, w)
+    want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
+    assert_close(got, want, "matmul")
+    assert_bits(got, want, "matmul")
+    got = be.matmul_decode(x, T, w)
+    want = oracle.matmul_decode(Q4_K, raw, in_dim, out_dim, x, T)
+    assert_close(got, want, "matmul_decode")
+    assert_bits(got, want, "matmul_decode")
+    one = be.matmul(x.reshape(T, in_dim)[T - 1], 1, w)
+    assert_bits(np.asarray(got).reshape(T, out_dim)[T - 1], one, "matmul_decode row == the token alone")
+
+
+@pytest.mark.parametrize("M", [128, 512, 2048])
+def test_prefill_gemm_at_the_benchmark_sizes(be, M):
+    """Config 4: Q4_K 4096 -> 14336 over M = 128 / 512 / 2048 tokens at full size with the library's
+    own kernel choice, against the CPU GEMM on sampled rows (the first, a middle and the last row
+    tile) bit for bit, and -- the size-independent property over every row -- batch independence:
+    the first 16 token rows of the result equal the matmul of those 16 tokens alone
+    (vecdot.rs:4522-4549)."""
+    in_dim, out_dim = 4096, 14336
+    raw = synth_weights(Q4_K, in_dim, out_dim, seed=77)
+    x = synth_x(M, in_dim, seed=M)
+    w = qm(raw, Q4_K, in_dim, out_dim)
+    be.set_tuning("gemm_min_tokens", 0)
+    be.set_tuning("gemm_small_max_tokens", 0)
+    be.set_tuning("gemm_sb_waves", 0)
+    try:
+        got = np.asarray(be.matmul(x, M, w)).reshape(M, out_dim)
+        say("prefill GEMM", M, be.last_kernel())
+        head = np.asarray(be.matmul(x.reshape(M, in_dim)[:16], 16, w)).reshape(16, out_dim)
+    finally:
+        be.set_tuning("gemm_min_tokens", GEMM_FROM)
+        be.set_tuning("gemm_small_max_tokens", 1)
+        be.set_tuning("gemm_sb_waves", 8)
+    rows = np.r_[0:32, 7000:7032, out_dim - 32:out_dim]
+    rb = row_bytes(Q4_K, in_dim)
+    sub = np.concatenate([raw[r * rb:(r + 1) * rb] for r in rows])
+    want = oracle.matmul(Q4_K, sub, in_dim, rows.size, x, M).reshape(M, rows.size)
+    assert_close(got[:, rows], want, "sampled rows")
+    assert_bits(got[:, rows], want, "sampled rows")
+    assert_bits(got[:16], head, "batch independence over all rows")
+
+
+def test_argmax_follows_total_cmp(be):
+    """sampling::argmax (sampling.rs:336-343): max_by over total_cmp -- the last of equal maxima,
+    -0 below +0, a positive NaN above every number, a negative NaN below."""
+    from oracle import llama_ref as R
+    nan, inf = np.float32("nan"), np.float32("inf")
+    neg_nan = np.array([0xFFC00000], np.uint32).view(np.float32)[0]
+    cases = [[1.0, 5.0, 2.0, 5.0, 0.0], [-3.0], [-0.0, 0.0, -0.0], [0.0, -0.0], [1.0, nan, 7.0], [neg_nan, -inf, neg_nan],
+             [-inf, -inf], [inf, 3.0, inf, nan, nan], [neg_nan], [neg_nan, neg_nan]]
+    rng = np.random.default_rng(12)
+    big = rng.standard_normal(128256).astype(np.float32)
+    big[[5, 70000, 128255]] = big.max() + 1.0
+    cases += [big, np.where(rng.random(70001) < 0.01, nan, rng.standard_normal(70001)).astype(np.float32),
+              np.zeros(513, np.float32), -np.zeros(1000, np.float32)]
+    for c in cases:
+        c = np.asarray(c, np.float32)
+        assert be.argmax(c) == R.argmax(c), c[:8]
 
 
 def test_q6k_vocab_projection_batches_1_4_8(be):

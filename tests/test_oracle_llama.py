@@ -116,6 +116,24 @@ def test_softmax_silu_argmax():
     assert abs(float(R.silu(f32(-1.0))) + 0.26894143) < 1e-6
     assert R.argmax(np.array([1.0, 5.0, 2.0, 5.0, 0.0], f32)) == 3   # last of equal maxima
     assert R.argmax(np.array([-3.0], f32)) == 0
+    # max_by over total_cmp (sampling.rs:336-343): -NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN
+    nan, inf = f32("nan"), f32("inf")
+    neg_nan = np.array([0xFFC00000], np.uint32).view(f32)[0]
+    assert R.argmax(np.array([1.0, nan, 7.0], f32)) == 1
+    assert R.argmax(np.array([-0.0, 0.0, -0.0], f32)) == 1
+    assert R.argmax(np.array([0.0, -0.0], f32)) == 0
+    assert R.argmax(np.array([neg_nan, -inf, neg_nan], f32)) == 1
+    assert R.argmax(np.array([neg_nan, neg_nan], f32)) == 1
+    assert R.argmax(np.array([inf, 3.0, inf], f32)) == 2
+
+
+def test_cache_rows_saturate_at_the_f16_range():
+    row = np.array([1.0, 65504.0, 65519.0, 65520.0, 1e9, -1e9, np.inf, -np.inf, np.nan], f32)
+    got = R.to_cache(row, np.float16)
+    assert got.dtype == np.float16
+    np.testing.assert_array_equal(got[:8].astype(f32), [1.0, 65504.0, 65504.0, 65504.0, 65504.0, -65504.0, 65504.0, -65504.0])
+    assert np.isnan(got[8])
+    np.testing.assert_array_equal(R.to_cache(row, f32)[:6], row[:6])   # the reference's f32 cache keeps everything
 
 
 def test_attention_closed_forms_and_head_mapping():
