@@ -143,6 +143,19 @@ int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, int decode,
 int ogm_matmul_dev(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
                    float *y_dev, int decode, void *stream);
 
+/* ogm_matmul_dev for callers that cannot allocate.  It has no counterpart in the reference; it is for
+ * code that must not call hipMalloc -- a HIP graph under capture, a tight serving loop, a harness that
+ * forbids allocation.  Same arguments and values as ogm_matmul_dev (bit for bit), but the quantized
+ * activations go to a static device array the library holds on every GPU it runs on (400 KiB, kept
+ * until the process ends) instead of the context's grown-on-demand scratch, and no hipMalloc, hipFree
+ * or other allocating routine is called.  Limits: n_tokens <= 8 and n_tokens * in_dim <= 262144;
+ * beyond them the call returns OGM_ERR_INVALID and enqueues nothing.  Every call on one GPU -- from
+ * any context or thread -- shares that GPU's array: calls that overlap on one GPU (two streams, two
+ * contexts) race on it; calls on one stream do not.  The array keeps the last call's contents; each
+ * call overwrites all it reads. */
+int ogm_matmul_dev_static(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
+                          float *y_dev, int decode, void *stream);
+
 /* The same path in two steps, so that ops reading one input (a layer's q/k/v, or gate/up:
  * engine/arch/mod.rs:1082-1096) quantize it once.  ogm_act_quantize_dev quantizes x_dev
  * ([n_tokens][in_dim]) into the context's activation buffer with the mode `ggml_type` needs

@@ -249,6 +249,13 @@ class Mi355xBackend:
         self._check(self._lib.ogm_matmul_dev(self._ctx, w_handle, x_ptr, n_tokens, y_ptr,
                                              int(decode), stream or None), "ogm_matmul_dev")
 
+    def matmul_dev_static(self, w_handle: int, x_ptr: int, n_tokens: int, y_ptr: int, decode: bool = False,
+                          stream: int = 0):
+        """ogm_matmul_dev without any allocation: the library's static device scratch takes the
+        quantized activations (at most 8 tokens and 262144 activations per call)."""
+        self._check(self._lib.ogm_matmul_dev_static(self._ctx, w_handle, x_ptr, n_tokens, y_ptr,
+                                                    int(decode), stream or None), "ogm_matmul_dev_static")
+
     def act_quantize_dev(self, ggml_type: int, x_ptr: int, in_dim: int, n_tokens: int, stream: int = 0):
         self._check(self._lib.ogm_act_quantize_dev(self._ctx, ggml_type, x_ptr, in_dim, n_tokens,
                                                    stream or None), "ogm_act_quantize_dev")

@@ -28,7 +28,7 @@ SYMBOLS = [
     "ogm_gguf_open", "ogm_gguf_parse", "ogm_gguf_close", "ogm_gguf_last_error", "ogm_gguf_info",
     "ogm_gguf_meta_u64", "ogm_gguf_meta_f64", "ogm_gguf_meta_string", "ogm_gguf_meta_array",
     "ogm_gguf_find_tensor", "ogm_gguf_tensor", "ogm_gguf_tensor_data", "ogm_gguf_matrix",
-    "ogm_gguf_upload_matrix", "ogm_argmax", "ogm_quantize_act_tokens", "ogm_llama_debug_capture", "ogm_llama_debug_act",
+    "ogm_gguf_upload_matrix", "ogm_argmax", "ogm_matmul_dev_static", "ogm_quantize_act_tokens", "ogm_llama_debug_capture", "ogm_llama_debug_act",
 ]
 
 
@@ -88,6 +88,7 @@ def load_library() -> C.CDLL:
     L.ogm_matmul_decode.argtypes = [vp, vp, vp, u32, vp]
     L.ogm_matmul_batch.argtypes = [vp, C.POINTER(OgmOp), sz, C.c_int, u32]
     L.ogm_matmul_dev.argtypes = [vp, vp, vp, u32, vp, C.c_int, vp]
+    L.ogm_matmul_dev_static.argtypes = [vp, vp, vp, u32, vp, C.c_int, vp]
     L.ogm_act_quantize_dev.argtypes = [vp, u32, vp, u32, u32, vp]
     L.ogm_matmul_act_dev.argtypes = [vp, vp, u32, vp, C.c_int, vp]
     L.ogm_matmul_multi_dev.argtypes = [vp, C.POINTER(vp), sz, vp, u32, C.POINTER(vp), C.c_int, vp]

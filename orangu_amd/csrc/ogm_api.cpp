@@ -59,6 +59,7 @@ struct ogm_ctx {
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
   const char *last_kernel = "";
+  uint8_t *static_scratch = nullptr;   // this device's copy of the library's static scratch array (ogm_static.hip)
   // what the activation buffer currently holds (ogm_act_quantize_dev)
   int act_mode = -1;
   uint32_t act_in_dim = 0, act_tokens = 0;
@@ -178,6 +179,14 @@ extern "C" int ogm_init(int device, ogm_ctx **out) {
   if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
   if (e != hipSuccess) {
     std::string msg = std::string("stream creation: ") + hipGetErrorString(e);
+    delete ctx;
+    return fail(nullptr, OGM_ERR_HIP, msg);
+  }
+  // the device is current: resolve this device's address of the static scratch once, here
+  e = ogm_static_scratch_address(&ctx->static_scratch);
+  if (e != hipSuccess) {
+    std::string msg = std::string("static scratch address: ") + hipGetErrorString(e);
+    (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return fail(nullptr, OGM_ERR_HIP, msg);
   }
@@ -571,6 +580,31 @@ extern "C" int ogm_matmul_dev(ogm_ctx *ctx, const ogm_weight *w, const float *x_
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
   return enqueue_matmul(ctx, w, x_dev, n_tokens, y_dev, decode, s, nullptr, nullptr);
+}
+
+// ogm_matmul_dev for callers that cannot allocate: the quantized activations go to the library's
+// static device array instead of the context's grown-on-demand scratch, and only the GEMV kernels
+// run.  No hipMalloc, hipFree or allocating routine is reached from here.
+extern "C" int ogm_matmul_dev_static(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
+                                     float *y_dev, int decode, void *stream) {
+  int rc = check_matmul_args(ctx, w, x_dev, y_dev, n_tokens);
+  if (rc != OGM_OK) return rc;
+  if (n_tokens == 0) return OGM_OK;
+  if (n_tokens > OGM_STATIC_MAX_TOKENS || (uint64_t)n_tokens * w->in_dim > OGM_STATIC_MAX_ELEMS)
+    return fail(ctx, OGM_ERR_INVALID,
+                "ogm_matmul_dev_static: at most " + std::to_string(OGM_STATIC_MAX_TOKENS) + " tokens and " +
+                    std::to_string(OGM_STATIC_MAX_ELEMS) + " activations (n_tokens * in_dim) fit the static scratch; got " +
+                    std::to_string(n_tokens) + " x " + std::to_string(w->in_dim));
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
+  const int mode = act_mode_for(w->ggml_type);
+  const OgmActDev act = ogm_static_act_view(ctx->static_scratch);
+  // The quantizer writes every value the kernels below read for these tokens: nothing in the
+  // array has to start at zero, and what an earlier call left beyond them is never read.
+  HIPCHK(ctx, ogm_launch_quantize(mode, x_dev, w->in_dim, n_tokens, act, s));
+  const Target t{w, y_dev};
+  return enqueue_gemv(ctx, &t, 1, n_tokens, decode, s, nullptr, nullptr, nullptr, nullptr, &act);
 }
 
 extern "C" int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev,

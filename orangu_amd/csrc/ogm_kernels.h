@@ -100,3 +100,13 @@ size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens);
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name);
 
 hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hipStream_t stream);
+
+// The library's static scratch (ogm_static.hip): a file-scope device array every GPU holds its own
+// copy of, for the entry point that must not allocate.  It takes the quantized activations of up to
+// OGM_STATIC_MAX_TOKENS tokens totalling OGM_STATIC_MAX_ELEMS elements (400 KiB in all).
+#define OGM_STATIC_MAX_TOKENS 8u
+#define OGM_STATIC_MAX_ELEMS 262144u
+// Address of the array on the device that is current, from hipGetSymbolAddress; call once per device.
+hipError_t ogm_static_scratch_address(uint8_t **ptr);
+// The array cut into the five activation buffers, for OGM_STATIC_MAX_ELEMS elements.
+OgmActDev ogm_static_act_view(uint8_t *scratch);
