@@ -381,6 +381,10 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * 256 workgroups over rows of at least 16 super-blocks);
  * "attn_prefill_variant" (attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the
  * decode step's kernel per token and chunk of the cache; they agree to f32 rounding, not bit for bit);
+ * "gemm_plane_cache_mb" (device memory, in MiB, that the K-quant matrices' prefill planes may take in all:
+ * on a matrix's first tiled GEMM its scale-folded int8 planes -- 2 bytes per weight, 1 for Q3_K -- are
+ * built once and kept, so that later calls multiply them instead of unpacking the weights again;
+ * 0 = the default: build none and unpack on every call; ogm_weight_download is unaffected either way);
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
  * the quantizer kernel first; 0 or -1 = default, off);

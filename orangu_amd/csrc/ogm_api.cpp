@@ -24,6 +24,12 @@ struct ogm_weight {
   size_t row_bytes, device_bytes;
   uint8_t *dev;  // tile-planar
   uint64_t key_addr, key_len;
+  // K-quants: the scale-folded int8 planes the tiled prefill GEMMs multiply (ogm_gemm_build_planes),
+  // built on the matrix's first such GEMM and kept while the context's budget allows; null before
+  // that.  A second, prefill-only layout: the tile-planar bytes stay what ogm_weight_download returns.
+  uint8_t *planes = nullptr;
+  size_t plane_bytes = 0;
+  bool planes_refused = false;   // over budget or out of memory once: not tried again
 };
 
 struct DevBuf {
@@ -58,6 +64,10 @@ struct ogm_ctx {
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
+  // Device memory the prefill planes of all weights may take, in MiB; 0 (the default) = build none.
+  // A model's planes are 3.3 times its Q4_K bytes.
+  int tune_plane_cache_mb = 0;
+  size_t plane_bytes_used = 0;
   const char *last_kernel = "";
   uint8_t *static_scratch = nullptr;   // this device's copy of the library's static scratch array (ogm_static.hip)
   // what the activation buffer currently holds (ogm_act_quantize_dev)
@@ -200,6 +210,7 @@ extern "C" void ogm_destroy(ogm_ctx *ctx) {
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
   for (ogm_weight *w : ctx->weights) {
     if (w->dev) (void)hipFree(w->dev);
+    if (w->planes) (void)hipFree(w->planes);
     delete w;
   }
   DevBuf *dev[] = {&ctx->x,    &ctx->y,    &ctx->q,    &ctx->d,  &ctx->sums,
@@ -275,6 +286,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemv_rb_per_wg") == 0) {
     if (value < 0 || value > 64) return fail(ctx, OGM_ERR_INVALID, "gemv_rb_per_wg must be 0..64");
     ctx->tune_rb_per_wg = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_plane_cache_mb") == 0) {
+    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_cache_mb must be >= 0");
+    ctx->tune_plane_cache_mb = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemv_fuse_quant") == 0) {
@@ -374,6 +390,10 @@ extern "C" int ogm_weight_free(ogm_ctx *ctx, ogm_weight *w) {
       ctx->weights.erase(ctx->weights.begin() + (long)i);
       if (w->key_len != 0) ctx->cache.erase({w->key_addr, w->key_len});
       if (w->dev) HIPCHK(ctx, hipFree(w->dev));
+      if (w->planes) {
+        HIPCHK(ctx, hipFree(w->planes));
+        ctx->plane_bytes_used -= w->plane_bytes;
+      }
       delete w;
       return OGM_OK;
     }
@@ -443,6 +463,37 @@ static int enqueue_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev,
   return enqueue_matmul(ctx, &t, 1, x_dev, n_tokens, decode, stream, dump_isum, dump_imin);
 }
 
+// Builds the prefill planes of a K-quant matrix on first use, within the context's budget.  Returns
+// whether the matrix has planes afterwards; a refusal (budget, memory) is remembered and is no
+// error: the kernels then unpack the tile-planar bytes as before.  Caller holds the lock.
+static bool ensure_planes(ogm_ctx *ctx, const ogm_weight *cw, hipStream_t stream) {
+  ogm_weight *w = const_cast<ogm_weight *>(cw);   // the planes are a cache beside the weight's bytes
+  if (w->planes) return true;
+  if (w->planes_refused) return false;
+  const size_t bytes = ogm_gemm_plane_bytes(w->ggml_type, w->in_dim, w->out_dim);
+  const size_t budget = (size_t)ctx->tune_plane_cache_mb << 20;
+  if (bytes == 0 || ctx->plane_bytes_used + bytes > budget) {
+    w->planes_refused = bytes == 0;   // a budget may be raised later
+    return false;
+  }
+  uint8_t *p = nullptr;
+  if (hipMalloc((void **)&p, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    w->planes_refused = true;
+    return false;
+  }
+  if (ogm_gemm_build_planes(w->ggml_type, w->dev, w->in_dim, w->out_dim, p, stream) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipFree(p);
+    w->planes_refused = true;
+    return false;
+  }
+  w->planes = p;
+  w->plane_bytes = bytes;
+  ctx->plane_bytes_used += bytes;
+  return true;
+}
+
 static bool all_gemm_supported(const Target *tg, size_t n_tg, uint32_t n_tokens) {
   for (size_t i = 0; i < n_tg; i++)
     if (!ogm_gemm_supported(tg[i].w->ggml_type, tg[i].w->in_dim, tg[i].w->out_dim, n_tokens)) return false;
@@ -492,6 +543,15 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
         g.extra_wt[j - 1] = tg[i + j].w->dev;
         g.extra_out_dim[j - 1] = tg[i + j].w->out_dim;
         g.extra_y[j - 1] = tg[i + j].y;
+      }
+      if (ogm_gemm_uses_planes(g)) {
+        // a tiled int8 kernel: over the matrices' planes when all of them have (or now get) theirs
+        bool all = true;
+        for (size_t j = 0; j < ng; j++) all = ensure_planes(ctx, tg[i + j].w, stream) && all;
+        if (all) {
+          g.planes = tg[i].w->planes;
+          for (size_t j = 1; j < ng; j++) g.extra_planes[j - 1] = tg[i + j].w->planes;
+        }
       }
       HIPCHK(ctx, ogm_launch_gemm(g, stream, &ctx->last_kernel));
     }
@@ -970,7 +1030,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   m->cfg.rope_freq_factors = nullptr;   // folded into the frequency table below; the caller's array is not kept
   m->layers.assign(layers, layers + c.n_layer);
   m->output = output;
-  m->max_splits = (c.max_ctx + OGM_ATTN_CHUNK - 1) / OGM_ATTN_CHUNK;
+  m->max_splits = (c.max_ctx + OGM_ATTN_CHUNK_MIN - 1) / OGM_ATTN_CHUNK_MIN;
   const size_t cache_bytes = (size_t)c.n_layer * c.max_ctx * kvd * 2;
   int rc = OGM_OK;
   auto A = [&](void **p, size_t b) { if (rc == OGM_OK) rc = llama_alloc(ctx, m, p, b); };

@@ -760,7 +760,20 @@ struct GemmI8pParams {
   const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1];
   float *extra_y[OGM_GEMM_MAX_MATS - 1];
   uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
+  // PRE kernels: the planes built once per matrix by ogm_gemm_build_planes_kernel
+  const uint8_t *planes;
+  const uint8_t *extra_planes[OGM_GEMM_MAX_MATS - 1];
 };
+
+// The planes of a matrix, built once and kept beside its tile-planar bytes (2 bytes per weight; 1
+// for Q3_K): what the feeding waves of the kernels below otherwise recompute on every call.  Row
+// blocks of 64 rows; for row block rb, super-block s, stage g (64 weights), group t (16 weights):
+// 64 rows x 16 bytes of plane h, then (two-plane types) 64 rows x 16 bytes of plane l -- one
+// feeding wave's share of a stage is one contiguous run of 1 or 2 KiB.
+__host__ __device__ inline size_t gp_plane_offset(uint32_t rb, uint32_t nsb, uint32_t s, uint32_t g, uint32_t t16,
+                                                  uint32_t npl) {
+  return ((((size_t)rb * nsb + s) * 4u + g) * 4u + t16) * (npl * 1024u);
+}
 
 // ROWS = 128: eight multiplying waves (32 rows x 64 tokens each) and eight feeding ones; ROWS = 64:
 // four and four, and half the LDS: twice as many workgroups, which fills the chip when a launch has
@@ -772,7 +785,30 @@ struct GemmI8pParams {
 #define GP_Q3K 1
 #define GP_Q4K 2
 #define GP_Q5K 3
-template <uint32_t ROWS, int KIND>
+// Ablation switches for timing experiments (scratch builds define them; the library never does):
+// each removes one ingredient of the kernel below, results become wrong, and the time that goes
+// away is what that ingredient costs.
+#ifndef GP_ABL_NOMFMA
+#define GP_ABL_NOMFMA 0
+#endif
+#ifndef GP_ABL_NOLDSREAD
+#define GP_ABL_NOLDSREAD 0
+#endif
+#ifndef GP_ABL_NOFEED
+#define GP_ABL_NOFEED 0
+#endif
+#ifndef GP_ABL_NOBARRIER
+#define GP_ABL_NOBARRIER 0
+#endif
+#ifndef GP_ABL_NOPASS1
+#define GP_ABL_NOPASS1 0
+#endif
+#ifndef GP_ABL_NOEPI
+#define GP_ABL_NOEPI 0
+#endif
+#define GP_SYNC() do { if (!GP_ABL_NOBARRIER) __syncthreads(); } while (0)
+
+template <uint32_t ROWS, int KIND, bool PRE = false>
 __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   constexpr bool Q3 = KIND == GP_Q3K, Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K;
   constexpr uint32_t NC = ROWS / 16u;                // multiplying waves
@@ -806,6 +842,7 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
       p.wt = p.extra_wt[m];
       p.y = p.extra_y[m];
       p.out_dim = p.extra_out_dim[m];
+      p.planes = p.extra_planes[m];
     } else {
       break;
     }
@@ -821,7 +858,7 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
 #pragma unroll
   for (int r = 0; r < 16; r++) y0[r] = y1[r] = 0.0f;
 
-  if constexpr (Q45) {
+  if constexpr (Q45 && !GP_ABL_NOPASS1) {
     // ---------------- pass 1 of gemm_k_q4_k: acc -= (ad * dmin) * sum_j m_j * bsum_j, all super-blocks
     // first (vecdot.rs:2226-2240), on the f16 matrix cores with tokens as rows: 64 m_j against
     // bsum_j / 64 and m_j against bsum_j % 64 in one K = 16 instruction per 32 x 32 outputs.  The
@@ -885,6 +922,10 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
       uo = rb * p.nct * TILE_BYTES + r * 16u;
       dto = rb * p.nct * TILE_BYTES + 13u * 1024u + r * 2u;
     }
+    // PRE: this thread's 16 bytes of each plane, per (super-block, stage): row block of 64 rows
+    // (clamped to the matrix's last one; such rows are never stored), its row within it
+    [[maybe_unused]] const uint32_t prb = min((r0 + prw) >> 6, (p.out_dim - 1u) >> 6);
+    [[maybe_unused]] const uint8_t *pl_base = PRE ? p.planes + (prw & 63u) * 16u : nullptr;
     constexpr uint32_t XB = ROWS == 128u ? 16u : 32u;   // bytes of a token's stage per feeding thread
     const uint32_t xrow_ = pt / (64u / XB), xpart = pt % (64u / XB);
     const uint32_t xro = min(t0 + xrow_, p.n_tokens - 1u) * p.in_dim + XB * xpart;   // + 256 s + 64 g
@@ -903,9 +944,14 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     float adn = 0.0f;
 #define GP_LOAD(S, G, K)                                                                          \
   do {                                                                                            \
+    if (GP_ABL_NOFEED) break;                                                                     \
     const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded again, never used */ \
     const uint32_t so_ = sb_tile(s_) + sb_lane(s_) * 16u, h_ = (G) >> 1;                          \
-    if constexpr (Q3) {                                                                           \
+    if constexpr (PRE) {                                                                          \
+      const uint8_t *pp_ = pl_base + gp_plane_offset(prb, p.nsb, s_, (G), t16, NPL);              \
+      qla##K = *(const uint4 *)pp_;                                                               \
+      if constexpr (!Q3) qha##K = *(const uint4 *)(pp_ + 1024u);                                  \
+    } else if constexpr (Q3) {                                                                    \
       /* pieces: hmask 0..1, qs 2..5, then scales[12] | d | two bytes of padding */               \
       qla##K = *(const uint4 *)(p.wt + (uo + so_ + (2u + 2u * h_ + (t16 & 1u)) * 1024u));         \
     } else if constexpr (Q45) {                                                                   \
@@ -920,13 +966,13 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     if constexpr (ROWS == 64u) xb##K##_ = xp_[1];                                                 \
     if ((G) == 0u) {                                                                              \
       if constexpr (Q3) {                                                                         \
-        scxa = *(const uint4 *)(p.wt + (uo + so_ + 6u * 1024u));                                  \
-        hmxn = *(const uint4 *)(p.wt + (uo + so_ + (t16 & 1u) * 1024u));                          \
+        if (!PRE || has_d) scxa = *(const uint4 *)(p.wt + (uo + so_ + 6u * 1024u));               \
+        if constexpr (!PRE) hmxn = *(const uint4 *)(p.wt + (uo + so_ + (t16 & 1u) * 1024u));      \
       } else if constexpr (Q45) {                                                                 \
-        scxa = *(const uint4 *)(p.wt + (uo + so_));   /* d | dmin, then the 12 scale bytes */     \
-        if constexpr (Q5) hmxn = *(const uint4 *)(p.wt + (uo + so_ + (1u + (t16 & 1u)) * 1024u)); \
+        if (!PRE || has_d) scxa = *(const uint4 *)(p.wt + (uo + so_));   /* d | dmin, then the 12 scale bytes */ \
+        if constexpr (Q5 && !PRE) hmxn = *(const uint4 *)(p.wt + (uo + so_ + (1u + (t16 & 1u)) * 1024u)); \
       } else {                                                                                    \
-        scxa = *(const uint4 *)(p.wt + (uo + so_ + 12u * 1024u));                                 \
+        if constexpr (!PRE) scxa = *(const uint4 *)(p.wt + (uo + so_ + 12u * 1024u));             \
         if (has_d) d16 = *(const uint16_t *)(p.wt + (dto + sb_tile(s_) + sb_lane(s_) * 2u));      \
       }                                                                                           \
       if (has_ad) adn = p.ad[aro + s_];                                                           \
@@ -1018,6 +1064,7 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
   } while (0)
 #define GP_STORE(S, G, K)                                                                         \
   do {                                                                                            \
+    if (GP_ABL_NOFEED) break;                                                                     \
     if ((G) == 0u) {                                                                              \
       sca[0] = scxa.x; sca[1] = scxa.y; sca[2] = scxa.z; sca[3] = scxa.w;                         \
       if constexpr (Q3) {                                                                         \
@@ -1031,7 +1078,10 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
       }                                                                                           \
       if (has_ad) ad_l[128u * ((S) & 1u) + ad_tok] = adn;                                         \
     }                                                                                             \
-    if constexpr (Q3) GP_GROUP3(qla##K, G, pw, prw, t16);                                         \
+    if constexpr (PRE) {                                                                          \
+      *(uint4 *)&wh_l[pw + prw * GI_ROW + 16u * t16] = qla##K;                                    \
+      if constexpr (!Q3) *(uint4 *)&wl_l[pw + prw * GI_ROW + 16u * t16] = qha##K;                 \
+    } else if constexpr (Q3) GP_GROUP3(qla##K, G, pw, prw, t16);                                  \
     else if constexpr (Q45) GP_GROUP45(qla##K, G, pw, prw, t16);                                  \
     else GP_GROUP(qla##K, qha##K, sca, G, pw, prw, t16);                                          \
     uint8_t *xr_ = &x_l[px + xrow_ * GI_ROW + XB * xpart];                                        \
@@ -1049,21 +1099,21 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
     GP_LOAD(0u, 3u, 3);
     GP_STORE(0u, 1u, 1);
     GP_LOAD(1u, 0u, 0);
-    __syncthreads();
+    GP_SYNC();
     // each period stores the stage two ahead of the one being multiplied and loads the one five ahead
     for (uint32_t s = 0; s < p.nsb; s++) {
       GP_STORE(s, 2u, 2);
       GP_LOAD(s + 1u, 1u, 1);
-      __syncthreads();
+      GP_SYNC();
       GP_STORE(s, 3u, 3);
       GP_LOAD(s + 1u, 2u, 2);
-      __syncthreads();
+      GP_SYNC();
       if (s + 1u < p.nsb) GP_STORE(s + 1u, 0u, 0);
       GP_LOAD(s + 1u, 3u, 3);
-      __syncthreads();
+      GP_SYNC();
       if (s + 1u < p.nsb) GP_STORE(s + 1u, 1u, 1);
       GP_LOAD(s + 2u, 0u, 0);
-      __syncthreads();
+      GP_SYNC();
     }
 #undef GP_LOAD
 #undef GP_GROUP
@@ -1071,17 +1121,23 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
 #undef GP_GROUP45
 #undef GP_STORE
   } else {
-    __syncthreads();
+    GP_SYNC();
+#if GP_ABL_NOMFMA
+#define GP_MFMA(A, B, C, X, Y, Z) ((C) + (A).x + (B).x)   /* keeps the operands alive */
+#else
+#define GP_MFMA(A, B, C, X, Y, Z) __builtin_amdgcn_mfma_i32_32x32x32_i8(A, B, C, X, Y, Z)
+#endif
     int16v h0, h1, l0, l1;   // the two planes' sums of the running super-block
     const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const uint32_t xrow0 = (tw + l32) * GI_ROW + 16u * lh, xrow1 = xrow0 + 32u * GI_ROW;
     const uint32_t wrow = (32u * rq + l32) * GI_ROW + 16u * lh;
     // operands of the stage's first 32 weights (a) and last 32 (b); a of the next stage is read
     // while b multiplies, b while a does
-    int4v x0a, x1a, wha, wla, x0b, x1b, whb, wlb;
+    int4v x0a = {0, 0, 0, 0}, x1a = x0a, wha = x0a, wla = x0a, x0b = x0a, x1b = x0a, whb = x0a, wlb = x0a;
     uint32_t cw = 0, cx = 0;   // byte offsets of the stage's buffers: weight planes, activations
 #define GP_READ(SUF, OFFW, OFFX)                              \
   do {                                                        \
+    if (GP_ABL_NOLDSREAD) break;                              \
     x0##SUF = *(const int4v *)&x_l[(OFFX) + xrow0];           \
     x1##SUF = *(const int4v *)&x_l[(OFFX) + xrow1];           \
     wh##SUF = *(const int4v *)&wh_l[(OFFW) + wrow];           \
@@ -1094,30 +1150,30 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
         const uint32_t nw = cw == 2u * WT ? 0u : cw + WT, nx = cx == 2u * GI_WTILE ? 0u : cx + GI_WTILE;
         GP_READ(b, cw + 32u, cx + 32u);
         if (g == 0u) {   // the super-block starts fresh sums
-          h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0a, wha, zi, 0, 0, 0);
-          h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1a, wha, zi, 0, 0, 0);
+          h0 = GP_MFMA(x0a, wha, zi, 0, 0, 0);
+          h1 = GP_MFMA(x1a, wha, zi, 0, 0, 0);
           if constexpr (!Q3) {
-            l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0a, wla, zi, 0, 0, 0);
-            l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1a, wla, zi, 0, 0, 0);
+            l0 = GP_MFMA(x0a, wla, zi, 0, 0, 0);
+            l1 = GP_MFMA(x1a, wla, zi, 0, 0, 0);
           }
         } else {
-          h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0a, wha, h0, 0, 0, 0);
-          h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1a, wha, h1, 0, 0, 0);
+          h0 = GP_MFMA(x0a, wha, h0, 0, 0, 0);
+          h1 = GP_MFMA(x1a, wha, h1, 0, 0, 0);
           if constexpr (!Q3) {
-            l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0a, wla, l0, 0, 0, 0);
-            l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1a, wla, l1, 0, 0, 0);
+            l0 = GP_MFMA(x0a, wla, l0, 0, 0, 0);
+            l1 = GP_MFMA(x1a, wla, l1, 0, 0, 0);
           }
         }
         GP_READ(a, nw, nx);   // complete since the last barrier; past the last stage: read, never used
-        h0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0b, whb, h0, 0, 0, 0);
-        h1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1b, whb, h1, 0, 0, 0);
+        h0 = GP_MFMA(x0b, whb, h0, 0, 0, 0);
+        h1 = GP_MFMA(x1b, whb, h1, 0, 0, 0);
         if constexpr (!Q3) {
-          l0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0b, wlb, l0, 0, 0, 0);
-          l1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1b, wlb, l1, 0, 0, 0);
+          l0 = GP_MFMA(x0b, wlb, l0, 0, 0, 0);
+          l1 = GP_MFMA(x1b, wlb, l1, 0, 0, 0);
         }
         cw = nw;
         cx = nx;
-        if (g == 3u) {
+        if (g == 3u && !GP_ABL_NOEPI) {
           const float d0 = d_l[ROWS * (s & 1u) + 32u * rq + l32];
           const float *adp = &ad_l[128u * (s & 1u) + tw + 4u * lh];
 #pragma unroll
@@ -1133,10 +1189,11 @@ __device__ __forceinline__ void gemm_q6k_i8_body(GemmI8pParams p) {
             }
           }
         }
-        __syncthreads();
+        GP_SYNC();
       }
     }
 #undef GP_READ
+#undef GP_MFMA
     const uint32_t row0 = r0 + 32u * rq + l32;
     if (row0 < p.out_dim) {
 #pragma unroll
@@ -1157,6 +1214,111 @@ __global__ __launch_bounds__(1024) void ogm_gemm_q4k_i8p_kernel(GemmI8pParams p)
 __global__ __launch_bounds__(512) void ogm_gemm_q4k_i8p_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q4K>(p); }
 __global__ __launch_bounds__(1024) void ogm_gemm_q5k_i8p_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q5K>(p); }
 __global__ __launch_bounds__(512) void ogm_gemm_q5k_i8p_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q5K>(p); }
+// the same kernels over planes built beforehand: the feeding waves only copy
+__global__ __launch_bounds__(1024) void ogm_gemm_q6k_i8_pre_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q6K, true>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q6k_i8_pre_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q6K, true>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q3k_i8_pre_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q3K, true>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q3k_i8_pre_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q3K, true>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q4k_i8p_pre_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q4K, true>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q4k_i8p_pre_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q4K, true>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_q5k_i8p_pre_kernel(GemmI8pParams p) { gemm_q6k_i8_body<128u, GP_Q5K, true>(p); }
+__global__ __launch_bounds__(512) void ogm_gemm_q5k_i8p_pre_r64_kernel(GemmI8pParams p) { gemm_q6k_i8_body<64u, GP_Q5K, true>(p); }
+
+// Builds a matrix's planes from its tile-planar bytes: thread (t = tid / 64, r = tid % 64) of
+// workgroup (4 s + g, rb) turns the sixteen weights 256 s + 64 g + 16 t .. of row 64 rb + r into their
+// 16 bytes of each plane -- the arithmetic of the feeding waves above, done once.
+//   Q6_K: u = sc_g (q - 32) + 128, sc the int8 scale of the group of 16       (vecdot.rs:2119-2143)
+//   Q3_K: one plane, (sc - 32)(4 - q) with the six-bit scale of the group      (vecdot.rs:2100-2117)
+//   Q4_K / Q5_K: u = sc_j q + 128, sc the six-bit scale of the sub-block of 32 (vecdot.rs:2036-2088)
+// h = u >> 8, l = (u & 255) - 128 as int8: sc * q' = 256 h + l.
+struct GemmPlaneBuildParams {
+  const uint8_t *wt;
+  uint8_t *planes;
+  uint32_t out_dim, nsb, c_shift, r_shift, nct;
+};
+
+template <int KIND>
+__global__ __launch_bounds__(256) void ogm_gemm_build_planes_kernel(GemmPlaneBuildParams p) {
+  constexpr bool Q3 = KIND == GP_Q3K, Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K;
+  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : KIND == GP_Q4K ? 9216u : Q5 ? 11264u : 13440u;
+  constexpr uint32_t QS_PIECE0 = Q5 ? 3u : 1u;
+  constexpr uint32_t NPL = Q3 ? 1u : 2u;
+  const uint32_t t16 = threadIdx.x >> 6, r = threadIdx.x & 63u;
+  const uint32_t s = blockIdx.x >> 2, g = blockIdx.x & 3u, rb = blockIdx.y;
+  const uint32_t row = min(64u * rb + r, p.out_dim - 1u);   // rows past the matrix repeat its last one
+  const uint32_t uo = (row >> p.r_shift) * p.nct * TILE_BYTES + (row & ((1u << p.r_shift) - 1u)) * 16u;
+  const uint32_t so = (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
+  const uint8_t *u0 = p.wt + uo + so;
+  const uint32_t h_ = g >> 1;
+  uint4 ql, qh = make_uint4(0, 0, 0, 0);
+  int sc;
+  short addc;   // the constant added to sc * q
+  uint32_t shift_q = 0, mask_q, hi_shift = 0, hi_mask = 0, hi_lsh = 0;   // q = (ql >> shift_q) & mask_q | ((qh >> hi_shift) & hi_mask) << hi_lsh
+  if constexpr (Q3) {
+    // run of 32: rr = 2 (g & 1) + t16 / 2 inside the half block; two bits at 2 rr, third bit = bit 2 g + t16 / 2 of hmask
+    ql = *(const uint4 *)(u0 + (2u + 2u * h_ + (t16 & 1u)) * 1024u);
+    qh = *(const uint4 *)(u0 + (t16 & 1u) * 1024u);
+    const uint4 scx = *(const uint4 *)(u0 + 6u * 1024u);
+    const uint32_t lw = (g & 1u) ? scx.y : scx.x;
+    const uint32_t low = ((lw >> (8u * t16)) >> (g >= 2u ? 4u : 0u)) & 0xFu;
+    const uint32_t high = ((scx.z >> (8u * t16)) >> (2u * g)) & 3u;
+    const int scv = (int)(low | (high << 4)) - 32;
+    sc = -scv;
+    addc = (short)(4 * scv);
+    shift_q = 2u * (2u * (g & 1u) + (t16 >> 1));
+    mask_q = 0x03030303u;
+    hi_shift = 2u * g + (t16 >> 1);
+    hi_mask = 0x01010101u;
+    hi_lsh = 2;
+  } else if constexpr (Q45) {
+    ql = *(const uint4 *)(u0 + (QS_PIECE0 + 2u * g + (t16 & 1u)) * 1024u);
+    if constexpr (Q5) qh = *(const uint4 *)(u0 + (1u + (t16 & 1u)) * 1024u);
+    const uint4 hd = *(const uint4 *)u0;
+    uint32_t sc4a, sc4b;
+    q4k_scales(hd, sc4a, sc4b);
+    const uint32_t hi = t16 >> 1, j = 2u * g + hi;
+    sc = (int)(((g < 2u ? sc4a : sc4b) >> (8u * (j & 3u))) & 0xFFu);
+    addc = 128;
+    shift_q = hi ? 4u : 0u;
+    mask_q = 0x0F0F0F0Fu;
+    hi_shift = j;
+    hi_mask = Q5 ? 0x01010101u : 0u;
+    hi_lsh = 4;
+  } else {
+    ql = *(const uint4 *)(u0 + (4u * h_ + t16) * 1024u);
+    qh = *(const uint4 *)(u0 + (8u + 2u * h_ + (t16 & 1u)) * 1024u);
+    const uint4 scx = *(const uint4 *)(u0 + 12u * 1024u);
+    const uint32_t scw[4] = {scx.x, scx.y, scx.z, scx.w};
+    sc = (int)(int8_t)((scw[g] >> (8u * t16)) & 0xFFu);
+    addc = (short)(128 - 32 * sc);
+    shift_q = (g & 1u) ? 4u : 0u;
+    mask_q = 0x0F0F0F0Fu;
+    hi_shift = 2u * (2u * (g & 1u) + (t16 >> 1));
+    hi_mask = 0x03030303u;
+    hi_lsh = 4;
+  }
+  const short2v sc2 = {(short)sc, (short)sc}, c2 = {addc, addc};
+  const uint32_t qlw[4] = {ql.x, ql.y, ql.z, ql.w}, qhw[4] = {qh.x, qh.y, qh.z, qh.w};
+  uint32_t ph[4], pl[4];
+#pragma unroll
+  for (int w = 0; w < 4; w++) {
+    const uint32_t v = ((qlw[w] >> shift_q) & mask_q) | (((qhw[w] >> hi_shift) & hi_mask) << hi_lsh);
+    union { uint32_t u; short2v s; } e, f;
+    e.u = __builtin_amdgcn_perm(0u, v, 0x0c010c00u);   // (b0, b1) as 16-bit lanes
+    f.u = __builtin_amdgcn_perm(0u, v, 0x0c030c02u);   // (b2, b3)
+    e.s = e.s * sc2 + c2;
+    f.s = f.s * sc2 + c2;
+    if constexpr (Q3) {
+      ph[w] = __builtin_amdgcn_perm(f.u, e.u, 0x06040200u);   // the lanes' low bytes
+    } else {
+      ph[w] = __builtin_amdgcn_perm(f.u, e.u, 0x07050301u);                 // high bytes
+      pl[w] = __builtin_amdgcn_perm(f.u, e.u, 0x06040200u) ^ 0x80808080u;   // low bytes, top bit flipped
+    }
+  }
+  uint8_t *dst = p.planes + gp_plane_offset(rb, p.nsb, s, g, t16, NPL) + r * 16u;
+  *(uint4 *)dst = make_uint4(ph[0], ph[1], ph[2], ph[3]);
+  if constexpr (!Q3) *(uint4 *)(dst + 1024u) = make_uint4(pl[0], pl[1], pl[2], pl[3]);
+}
 
 // ------------------------------------------------------------------------------------------
 // Small batches (up to a few dozen tokens): the tiled kernels above cost the same for 9 tokens as
@@ -2513,6 +2675,61 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
          (uint64_t)in_dim * n_tokens * 2u <= lim;
 }
 
+size_t ogm_gemm_plane_bytes(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim) {
+  if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K && ggml_type != OGM_Q3_K && ggml_type != OGM_Q5_K) ||
+      in_dim == 0 || in_dim % 256u != 0 || out_dim == 0)
+    return 0;
+  const uint32_t npl = ggml_type == OGM_Q3_K ? 1u : 2u;
+  return gp_plane_offset((out_dim + 63u) / 64u, in_dim / 256u, 0, 0, 0, npl);
+}
+
+hipError_t ogm_gemm_build_planes(uint32_t ggml_type, const uint8_t *wt, uint32_t in_dim, uint32_t out_dim,
+                                 uint8_t *planes, hipStream_t stream) {
+  if (ogm_gemm_plane_bytes(ggml_type, in_dim, out_dim) == 0 || !wt || !planes) return hipErrorInvalidValue;
+  GemmPlaneBuildParams p;
+  p.wt = wt;
+  p.planes = planes;
+  p.out_dim = out_dim;
+  p.nsb = in_dim / 256u;
+  const OgmTiling tl = ogm_tiling_for(p.nsb, out_dim);
+  p.c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
+  p.r_shift = 6 - p.c_shift;
+  p.nct = tl.nct;
+  const dim3 grid(4u * p.nsb, (out_dim + 63u) / 64u);
+  if (grid.y > 65535u) return hipErrorInvalidValue;
+  switch (ggml_type) {
+    case OGM_Q6_K: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_Q6K>, grid, dim3(256), 0, stream, p); break;
+    case OGM_Q3_K: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_Q3K>, grid, dim3(256), 0, stream, p); break;
+    case OGM_Q4_K: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_Q4K>, grid, dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_Q5K>, grid, dim3(256), 0, stream, p); break;
+  }
+  return hipGetLastError();
+}
+
+// Which family of kernels a K-quant launch takes: 0 the f16 kernels, 1 the int8 multiply-add kernel,
+// 2 the small-batch kernel, 3 a tiled int8 plane kernel.
+static int gemm_k_path(const OgmGemmArgs &a) {
+  const uint32_t nsb = a.in_dim / 256;
+  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  // (the plane kernel keeps a table of nsb * 512 bytes in LDS next to its 94 KB of stages)
+  const bool i8 = q45 && (a.q4k_variant == 3u || nsb * 512u + 98304u > GM_LDS_MAX);
+  if (i8) return 1;
+  if (a.q4k_variant == 2u) return 0;
+  uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
+  for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
+  const uint32_t small_max = a.small_max_tokens ? a.small_max_tokens : (tiles64_all <= 128u ? 128u : 64u);
+  if (a.ggml_type != OGM_Q3_K && a.small_max_tokens != 1u && a.n_tokens <= small_max &&
+      (q45 ? 16u : 8u) * 4096u + 128u * nsb <= GM_LDS_MAX)
+    return 2;
+  return 3;
+}
+
+bool ogm_gemm_uses_planes(const OgmGemmArgs &a) {
+  if (a.n_tokens == 0 || a.out_dim == 0 || is_flat32(a.ggml_type)) return false;
+  if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return false;
+  return gemm_k_path(a) == 3;
+}
+
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name) {
   if (a.n_tokens == 0 || a.out_dim == 0) return hipSuccess;
   if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return hipErrorInvalidValue;
@@ -2560,9 +2777,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   // integer multiply-adds (q4k_variant 3).  Of the f16 Q4_K kernels the wide one takes over as
   // described above.
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
-  // (the plane kernel keeps a table of nsb * 512 bytes in LDS next to its 94 KB of stages)
-  const bool i8 = q45 && (a.q4k_variant == 3u || nsb * 512u + 98304u > GM_LDS_MAX);
-  const bool i8p = a.q4k_variant != 2u && !i8;
+  const int path = gemm_k_path(a);
+  const bool i8 = path == 1;
+  const bool i8p = path >= 2;
   const bool wide = a.ggml_type == OGM_Q4_K && a.q4k_variant == 2u && a.n_tokens > 256u &&
                     wgs128 > (a.wide_min_wgs ? a.wide_min_wgs : 256u);
   const bool raw_x = wide || i8 || i8p;   // these read the int8 activations as they are: only (bh, bl) to prepare
@@ -2614,11 +2831,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   // (Q4_K 4096 -> 14336: 18 / 35 / 50 us at 32 / 64 / 96 tokens against 42-45 us tiled), and up to 128
   // when the tiled kernel's grid would leave half the CUs idle (4096 -> 4096: 12 / 15 / 21 us at 32 /
   // 64 / 128 tokens against 38-41; 14336 -> 4096: 36 / 39 / 57 against 123-130).
-  uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
-  for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
-  const uint32_t small_max = a.small_max_tokens ? a.small_max_tokens : (tiles64_all <= 128u ? 128u : 64u);
-  if (i8p && a.ggml_type != OGM_Q3_K && a.small_max_tokens != 1u && a.n_tokens <= small_max &&
-      (q45 ? 16u : 8u) * 4096u + 128u * nsb <= GM_LDS_MAX) {
+  if (path == 2) {
     GemmSbParams p;
     p.wt = a.wt;
     p.xq = a.act.q;
@@ -2674,10 +2887,14 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.r_shift = 6 - c_shift;
     p.nct = tl.nct;
     p.n_extra = a.n_extra;
+    bool pre = a.planes != nullptr;
+    p.planes = a.planes;
     for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
       p.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
       p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
       p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
+      p.extra_planes[m] = m < a.n_extra ? a.extra_planes[m] : nullptr;
+      if (m < a.n_extra && !a.extra_planes[m]) pre = false;   // every matrix of the launch, or none
     }
     // 64-row tiles when asked for (q4k_variant 1), or when they still come one to a CU: then twice
     // as many CUs work (14336 -> 4096 x 512 tokens: 150 us against 180 us).  Two of them sharing a CU
@@ -2692,20 +2909,28 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     // Q4_K / Q5_K: + the tokens' ad of every super-block for the first pass
     const uint32_t lds_bytes = (q3 ? 3u : 6u) * rows * GI_ROW + 3u * GI_WTILE + (2u * rows + 256u) * 4u +
                                (q45 ? nsb * 512u : 0u);
-    struct Pick { uint32_t type; bool r64; const void *fn; const char *name; };
+    struct Pick { uint32_t type; bool r64, pre; const void *fn; const char *name; };
     const Pick picks[] = {
-        {OGM_Q6_K, false, (const void *)ogm_gemm_q6k_i8_kernel, "ogm_gemm_q6k_i8_kernel"},
-        {OGM_Q6_K, true, (const void *)ogm_gemm_q6k_i8_r64_kernel, "ogm_gemm_q6k_i8_r64_kernel"},
-        {OGM_Q3_K, false, (const void *)ogm_gemm_q3k_i8_kernel, "ogm_gemm_q3k_i8_kernel"},
-        {OGM_Q3_K, true, (const void *)ogm_gemm_q3k_i8_r64_kernel, "ogm_gemm_q3k_i8_r64_kernel"},
-        {OGM_Q4_K, false, (const void *)ogm_gemm_q4k_i8p_kernel, "ogm_gemm_q4k_i8p_kernel"},
-        {OGM_Q4_K, true, (const void *)ogm_gemm_q4k_i8p_r64_kernel, "ogm_gemm_q4k_i8p_r64_kernel"},
-        {OGM_Q5_K, false, (const void *)ogm_gemm_q5k_i8p_kernel, "ogm_gemm_q5k_i8p_kernel"},
-        {OGM_Q5_K, true, (const void *)ogm_gemm_q5k_i8p_r64_kernel, "ogm_gemm_q5k_i8p_r64_kernel"},
+        {OGM_Q6_K, false, false, (const void *)ogm_gemm_q6k_i8_kernel, "ogm_gemm_q6k_i8_kernel"},
+        {OGM_Q6_K, true, false, (const void *)ogm_gemm_q6k_i8_r64_kernel, "ogm_gemm_q6k_i8_r64_kernel"},
+        {OGM_Q3_K, false, false, (const void *)ogm_gemm_q3k_i8_kernel, "ogm_gemm_q3k_i8_kernel"},
+        {OGM_Q3_K, true, false, (const void *)ogm_gemm_q3k_i8_r64_kernel, "ogm_gemm_q3k_i8_r64_kernel"},
+        {OGM_Q4_K, false, false, (const void *)ogm_gemm_q4k_i8p_kernel, "ogm_gemm_q4k_i8p_kernel"},
+        {OGM_Q4_K, true, false, (const void *)ogm_gemm_q4k_i8p_r64_kernel, "ogm_gemm_q4k_i8p_r64_kernel"},
+        {OGM_Q5_K, false, false, (const void *)ogm_gemm_q5k_i8p_kernel, "ogm_gemm_q5k_i8p_kernel"},
+        {OGM_Q5_K, true, false, (const void *)ogm_gemm_q5k_i8p_r64_kernel, "ogm_gemm_q5k_i8p_r64_kernel"},
+        {OGM_Q6_K, false, true, (const void *)ogm_gemm_q6k_i8_pre_kernel, "ogm_gemm_q6k_i8_pre_kernel"},
+        {OGM_Q6_K, true, true, (const void *)ogm_gemm_q6k_i8_pre_r64_kernel, "ogm_gemm_q6k_i8_pre_r64_kernel"},
+        {OGM_Q3_K, false, true, (const void *)ogm_gemm_q3k_i8_pre_kernel, "ogm_gemm_q3k_i8_pre_kernel"},
+        {OGM_Q3_K, true, true, (const void *)ogm_gemm_q3k_i8_pre_r64_kernel, "ogm_gemm_q3k_i8_pre_r64_kernel"},
+        {OGM_Q4_K, false, true, (const void *)ogm_gemm_q4k_i8p_pre_kernel, "ogm_gemm_q4k_i8p_pre_kernel"},
+        {OGM_Q4_K, true, true, (const void *)ogm_gemm_q4k_i8p_pre_r64_kernel, "ogm_gemm_q4k_i8p_pre_r64_kernel"},
+        {OGM_Q5_K, false, true, (const void *)ogm_gemm_q5k_i8p_pre_kernel, "ogm_gemm_q5k_i8p_pre_kernel"},
+        {OGM_Q5_K, true, true, (const void *)ogm_gemm_q5k_i8p_pre_r64_kernel, "ogm_gemm_q5k_i8p_pre_r64_kernel"},
     };
     const Pick *pick = nullptr;
     for (const Pick &c : picks)
-      if (c.type == a.ggml_type && c.r64 == r64) pick = &c;
+      if (c.type == a.ggml_type && c.r64 == r64 && c.pre == pre) pick = &c;
     if (!pick) return hipErrorInvalidValue;
     hipError_t e = hipFuncSetAttribute(pick->fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;

@@ -94,7 +94,19 @@ struct OgmGemmArgs {
   const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1] = {};
   uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1] = {};
   float *extra_y[OGM_GEMM_MAX_MATS - 1] = {};
+  // K-quants: the matrices' scale-folded int8 planes (ogm_gemm_build_planes), or null.  When every
+  // matrix of the launch has them, the tiled int8 kernels read them instead of unpacking the
+  // weights again on every call.
+  const uint8_t *planes = nullptr;
+  const uint8_t *extra_planes[OGM_GEMM_MAX_MATS - 1] = {};
 };
+// Whether this launch would run a tiled int8 plane kernel, i.e. whether planes would be read.
+bool ogm_gemm_uses_planes(const OgmGemmArgs &a);
+// Bytes of a K-quant matrix's planes (0: the type has none), and the kernel that builds them from
+// the tile-planar bytes (2 bytes per weight, 1 for Q3_K; rows padded to a multiple of 64).
+size_t ogm_gemm_plane_bytes(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim);
+hipError_t ogm_gemm_build_planes(uint32_t ggml_type, const uint8_t *wt, uint32_t in_dim, uint32_t out_dim,
+                                 uint8_t *planes, hipStream_t stream);
 bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens);
 size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens);
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name);

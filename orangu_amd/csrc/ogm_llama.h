@@ -7,7 +7,9 @@
 
 #include "ogm_kernels.h"
 
-#define OGM_ATTN_CHUNK 128u   // cache positions per workgroup of the attention kernel
+#define OGM_ATTN_CHUNK 128u       // cache positions per workgroup of the attention kernel ...
+#define OGM_ATTN_CHUNK_MIN 64u    // ... or half as many while the launch stays within one round of workgroups;
+                                  // the partial-result buffers are sized for this one
 
 // x += delta (when delta is given; x is updated in place), then
 // normed = x * (1 / sqrt(mean(x^2) + eps)) * weight        (tensor.rs:732-757)
@@ -40,18 +42,19 @@ struct OgmAttnPre {
 //     table `cs`, k and v rounded to f16 into the cache rows of position `pos`;
 //   * causal attention over cache positions 0..pos (engine/attention.rs:426-549): scores =
 //     (q . k) * scale, softmax over positions, out = sum w * v; grouped-query heads share their
-//     K/V head (1 to 8 query heads per K/V head).  Split over chunks of OGM_ATTN_CHUNK positions
-//     and merged;
+//     K/V head (1 to 8 query heads per K/V head).  Split over chunks of `chunk` positions (64 or
+//     128; 0 = by the size of the launch) and merged;
 //   * the merged output quantized for the next matmul in `mode`, and stored as f32 when attn_out
 //     is not null.
-// part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch;
-// counters: n_head_kv words, zero before the first launch (the kernel leaves them zero).
+// part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch, with
+// max_splits >= pos / chunk + 1; counters: n_head_kv words, zero before the first launch (the
+// kernel leaves them zero).
 hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
                                   uint32_t rope_dim, const OgmAttnPre &pre, void *k_cache_layer,
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
                                   uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
                                   float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
-                                  hipStream_t stream);
+                                  hipStream_t stream, uint32_t chunk = 0);
 
 // h = silu(gate) * up with silu(g) = g / (1 + exp(-g))     (tensor.rs:825-827, arch/mod.rs:1071-1106)
 // quantized for the down projection in `mode`; h (f32) is also stored when not null.  With

@@ -110,6 +110,19 @@ __device__ __forceinline__ void st_one(float *p, float v) {
   else *p = v;
 }
 
+// Wall-clock stamps for timeline builds of the attention kernel (a scratch build defines
+// OGM_ATTN_STAMPS and the buffer; the library never does).
+#ifdef OGM_ATTN_STAMPS
+__device__ unsigned long long ogm_attn_stamps[4096 * 8];
+#define OGM_STAMP(i)                                                                              \
+  do {                                                                                            \
+    if (threadIdx.x == 0)                                                                         \
+      ogm_attn_stamps[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = wall_clock64(); \
+  } while (0)
+#else
+#define OGM_STAMP(i) do { } while (0)
+#endif
+
 // A partial softmax over some chunks of four neighbouring output elements: running maximum,
 // denominator and weighted sums relative to that maximum.
 struct AttnPart {
@@ -178,8 +191,8 @@ __device__ __forceinline__ AttnPart attn_merge_chunks(const float *part_o, const
 // attends to positions 0 .. pos + t).  q arrives with bias, norm and RoPE applied and every K/V
 // row is in the cache already (ogm_qkv_pre_kernel), workgroups past a token's last chunk leave at
 // once, and nothing is quantized: the next matmul is a GEMM that quantizes its own input.
-template <int HD, int G, int GROUP, bool PREFILL = false>
-__global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
+template <int HD, int G, int GROUP, bool PREFILL = false, int CHUNK = (int)OGM_ATTN_CHUNK>
+__global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
                                                        const float *__restrict__ v_new,
                                                        const float2 *__restrict__ cs, uint32_t rope_half,
                                                        OgmAttnPre pre, uint32_t gq,
@@ -188,39 +201,39 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
                                                        float scale, float *part_o, float *part_ml,
                                                        uint32_t *counters, float *__restrict__ attn_out,
                                                        OgmActDev act) {
-  constexpr int NT = 512, NW = NT / 64;
+  constexpr int NT = 4 * CHUNK, NW = NT / 64;   // four threads per cache position
   constexpr int KU = HD / 32;             // 16-byte pieces of a K row per thread
   constexpr int TPR = HD / 8;             // threads per V row
   constexpr int ROWS = NT / TPR;          // V rows in flight per step
-  constexpr int STEPS = OGM_ATTN_CHUNK / ROWS;
+  constexpr int STEPS = CHUNK / ROWS;
   constexpr int NV = G * 8;               // phase-2 partial sums per lane
   constexpr int NF = G >= 4 ? G / 4 : 1;  // scores a lane ends phase 1 with
-  static_assert(OGM_ATTN_CHUNK * 4 == NT, "four threads per cache position");
   __shared__ __align__(16) float qs[G][HD];
   __shared__ __align__(16) __half kcur[HD];
   __shared__ __align__(16) __half vcur[HD];
-  __shared__ float sc[G][OGM_ATTN_CHUNK];
+  __shared__ float sc[G][CHUNK];
   __shared__ float red[2][G][NW];
   __shared__ __align__(16) float osum[NW][G][HD];
   __shared__ uint32_t s_last;
   __shared__ float mrg[GROUP != 0 ? 6 : 1][GROUP != 0 ? NT : 1];   // the final merge's slices
   static_assert(!PREFILL || GROUP == 0, "a prefill batch merges in its own launch");
+  OGM_STAMP(0);
   const uint32_t kvh = blockIdx.x, split = blockIdx.y;
   if constexpr (PREFILL) {
     const uint32_t tok = blockIdx.z;
     pos += tok;
-    if (split > pos / OGM_ATTN_CHUNK) return;   // the whole workgroup: this token has no such chunk
+    if (split > pos / (uint32_t)CHUNK) return;   // the whole workgroup: this token has no such chunk
     const size_t n_head = (size_t)n_head_kv * gq;
     q += tok * n_head * HD;
     part_o += tok * n_head * max_splits * HD;
     part_ml += tok * n_head * max_splits * 2;
   }
-  const uint32_t n_splits = PREFILL ? pos / OGM_ATTN_CHUNK + 1u : gridDim.y;
+  const uint32_t n_splits = PREFILL ? pos / (uint32_t)CHUNK + 1u : gridDim.y;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t kv_dim = n_head_kv * HD;
   const uint32_t n_pos = pos + 1u;
-  const uint32_t p0 = split * OGM_ATTN_CHUNK;
-  const uint32_t n_here = min(OGM_ATTN_CHUNK, n_pos - p0);
+  const uint32_t p0 = split * (uint32_t)CHUNK;
+  const uint32_t n_here = min((uint32_t)CHUNK, n_pos - p0);
   const bool is_last = !PREFILL && split == n_splits - 1u;   // holds the current position, not yet cached
   const uint32_t cur = pos - p0;                 // meaningful in the last chunk only
 
@@ -318,6 +331,7 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
   for (int st = 0; st < STEPS; st++) asm volatile("" : "+v"(vr[st].x), "+v"(vr[st].y), "+v"(vr[st].z), "+v"(vr[st].w));
   __syncthreads();
 
+  OGM_STAMP(1);
   // ---- phase 1: scores
   if (is_last && r == cur) {
 #pragma unroll
@@ -407,6 +421,7 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
     st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2 + 1], l);
   }
 
+  OGM_STAMP(2);
   // ---- phase 2: weighted sum of V rows
   {
     float o[NV];
@@ -463,12 +478,14 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
     }
   }
 
+  OGM_STAMP(3);
   // ---- the last workgroup of this K/V head merges the chunks and quantizes
   if constexpr (GROUP != 0) {
     // The partial results were stored device-coherently; once this wave's stores are acknowledged
     // (vmcnt 0) and the workgroup has met, one ticket tells whether every chunk of the head is in.
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
+    OGM_STAMP(4);
     if (tid == 0) {
       const uint32_t ticket =
           __hip_atomic_fetch_add(&counters[kvh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -477,6 +494,7 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
         __hip_atomic_store(&counters[kvh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
     }
     __syncthreads();
+    OGM_STAMP(5);
     if (!s_last) return;
     // every thread merges a slice of the chunks of one group of four outputs (one trip to memory
     // up to 8 * NSL chunks), then the slices meet in LDS
@@ -492,6 +510,7 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
       mrg[2][tid] = pt.o.x; mrg[3][tid] = pt.o.y; mrg[4][tid] = pt.o.z; mrg[5][tid] = pt.o.w;
     }
     __syncthreads();
+    OGM_STAMP(6);
     constexpr int RUNS = (NG + 63) / 64;
     for (int run = wave; run < RUNS; run += NW) {
       const uint32_t eg = run * 64u + lane;
@@ -515,6 +534,7 @@ __global__ __launch_bounds__(512) void ogm_attn_kernel(const float *__restrict__
       }
       ogm_quantize_store<GROUP>(ov, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
     }
+    OGM_STAMP(7);
   }
 }
 
@@ -545,10 +565,18 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
                                   uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
                                   float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
-                                  hipStream_t stream) {
+                                  hipStream_t stream, uint32_t chunk) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0) return hipErrorInvalidValue;
   if (rope_dim > head_dim || rope_dim % 2u != 0) return hipErrorInvalidValue;
-  const uint32_t n_splits = pos / OGM_ATTN_CHUNK + 1u;
+  // Cache positions per workgroup: 128; 64 only for short contexts.  The kernel is a chain of
+  // latencies (cache loads 2.1 us, scores 1.5, V sum 1.5, hand-over of the partial results 0.9,
+  // merge 2.8, quantizer 1.0 at 2048 positions) of which only the two middle ones shrink with the
+  // chunk, while the merge grows with the number of chunks: measured on MI355X with eight K/V heads,
+  // 64 against 128 positions per workgroup take 8.4 against 8.9 us at 512 cached positions but 13.6
+  // against 10.7 at 2048 and 20.5 against 14.1 at 4096.
+  if (chunk == 0) chunk = (pos / 64u + 1u) * n_head_kv <= 96u ? 64u : 128u;
+  if (chunk != 64u && chunk != 128u) return hipErrorInvalidValue;
+  const uint32_t n_splits = pos / chunk + 1u;
   if (n_splits > max_splits) return hipErrorInvalidValue;
   const uint32_t n = n_head * head_dim;
   if (n % 32u != 0) return hipErrorInvalidValue;
@@ -560,11 +588,16 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
   // the merge rides in the attention kernel when every head slot is a head and a K/V head's
   // outputs are whole quantizer groups
   const uint32_t fused = (G == gq && (G * head_dim) % group == 0) ? group : 0u;
-#define OGM_ATTN_LAUNCH(HD_, G_, GR_)                                                                  \
-  hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, GR_>), grid, dim3(512), 0, stream, q, k_new, v_new,      \
-                     (const float2 *)cs, rope_dim / 2u, pre, gq, (__half *)k_cache_layer,               \
+#define OGM_ATTN_LAUNCH_C(HD_, G_, GR_, CH_)                                                           \
+  hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, GR_, false, CH_>), grid, dim3(4 * CH_), 0, stream, q, k_new, \
+                     v_new, (const float2 *)cs, rope_dim / 2u, pre, gq, (__half *)k_cache_layer,        \
                      (__half *)v_cache_layer, pos, max_splits, n_head_kv, scale, part_o, part_ml,       \
                      counters, attn_out, act)
+#define OGM_ATTN_LAUNCH(HD_, G_, GR_)                    \
+  do {                                                   \
+    if (chunk == 64u) OGM_ATTN_LAUNCH_C(HD_, G_, GR_, 64); \
+    else OGM_ATTN_LAUNCH_C(HD_, G_, GR_, 128);           \
+  } while (0)
 #define OGM_ATTN_GROUPS(HD_, G_)                                \
   do {                                                          \
     if (fused == 32u) OGM_ATTN_LAUNCH(HD_, G_, 32);             \
@@ -582,6 +615,7 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
   else return hipErrorInvalidValue;
 #undef OGM_ATTN_GROUPS
 #undef OGM_ATTN_LAUNCH
+#undef OGM_ATTN_LAUNCH_C
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || fused != 0u) return e;
   const dim3 cgrid((n + 255u) / 256u);

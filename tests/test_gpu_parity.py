@@ -2,6 +2,7 @@
 seeded inputs.  Bar: activation quantization and per-block integer sums bit-exact; f32 outputs
 within 1e-3 relative / 1e-5 absolute (they are in fact expected bit-identical, and the tests
 report that separately so a regression in the stronger property is visible)."""
+import re
 import sys
 
 import numpy as np
@@ -30,16 +31,30 @@ def say(*a):
 GEMM_FROM = 9
 
 
-@pytest.fixture(scope="module")
-def be():
+# Every test of this module runs twice: with the K-quant matrices' prefill planes built on first use
+# and kept (gemm_plane_cache_mb > 0; the tiled int8 kernels then carry "_pre" in their name) and with
+# none (the default: the same kernels unpack the weights on every call).  Same bits both ways.
+@pytest.fixture(scope="module", params=["planes", "unpack"])
+def be(request):
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()  # raises if the HIP library or the device is missing: no fallback
-    say("device:", b.device_name())
+    say("device:", b.device_name(), "mode:", request.param)
     b.set_tuning("gemm_min_tokens", GEMM_FROM)
     b.set_tuning("gemm_small_max_tokens", 1)
     b.set_tuning("gemm_sb_waves", 8)
+    b.set_tuning("gemm_plane_cache_mb", 65536 if request.param == "planes" else 0)
+    b.plane_mode = request.param
     yield b
     b.close()
+
+
+def kname(b):
+    """The last kernel's name without the "_pre" that marks a tiled int8 kernel reading prebuilt
+    planes; checks that the mark is there exactly when the backend keeps planes."""
+    name = b.last_kernel()
+    if re.match(r"ogm_gemm_q(6k_i8|3k_i8|4k_i8p|5k_i8p)(_pre)?(_r64)?_kernel$", name):
+        assert ("_pre" in name) == (getattr(b, "plane_mode", "unpack") == "planes"), name
+    return name.replace("_pre", "")
 
 
 def qm(raw, t, in_dim, out_dim):
@@ -492,29 +507,29 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
     say("gemm", in_dim, out_dim, T)
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
     got = be.matmul(x, T, w)
-    assert be.last_kernel() == plane_kernel("ogm_gemm_q4k_i8p", T, out_dim)
+    assert kname(be) == plane_kernel("ogm_gemm_q4k_i8p", T, out_dim)
     assert_close(got, want, "int8 plane gemm")
     assert_bits(got, want, "int8 plane gemm")
     be.set_tuning("gemm_q4k_variant", 1)   # the 64-row tiles whatever the grid
     try:
         got = be.matmul(x, T, w)
-        assert be.last_kernel() == "ogm_gemm_q4k_i8p_r64_kernel"
+        assert kname(be) == "ogm_gemm_q4k_i8p_r64_kernel"
         assert_bits(got, want, "int8 plane gemm, 64-row tiles")
         be.set_tuning("gemm_q4k_variant", 3)
         got = be.matmul(x, T, w)
-        assert be.last_kernel() == "ogm_gemm_q4k_i8_kernel"
+        assert kname(be) == "ogm_gemm_q4k_i8_kernel"
         assert_bits(got, want, "int8 multiply-add gemm")
         be.set_tuning("gemm_q4k_variant", 2)
         got = be.matmul(x, T, w)
         # beyond 256 tokens the 128 x 256 tile kernel runs once the 128 x 128 tiling would take more
         # than one round of workgroups (256)
         tiles = ((T + 127) // 128) * ((out_dim + 127) // 128)
-        assert be.last_kernel() == ("ogm_gemm_q4k_wide_kernel" if T > 256 and tiles > 256 else "ogm_gemm_q4k_kernel")
+        assert kname(be) == ("ogm_gemm_q4k_wide_kernel" if T > 256 and tiles > 256 else "ogm_gemm_q4k_kernel")
         assert_bits(got, want, "f16 mfma gemm")
         if T > 256:   # the wide kernel on this (small, ragged) shape as well
             be.set_tuning("gemm_wide_min_wgs", 1)
             got = be.matmul(x, T, w)
-            assert be.last_kernel() == "ogm_gemm_q4k_wide_kernel"
+            assert kname(be) == "ogm_gemm_q4k_wide_kernel"
             assert_bits(got, want, "wide f16 mfma gemm")
     finally:
         be.set_tuning("gemm_wide_min_wgs", 0)
@@ -534,9 +549,9 @@ def test_gemm_threshold_default():
         w = qm(raw, Q8_0, 1024, 70)
         want = oracle.matmul(Q8_0, raw, 1024, 70, x[:17], 17).reshape(17, 70)
         y16 = b.matmul(x[:16], 16, w)
-        assert b.last_kernel().startswith("ogm_gemv_kernel")
+        assert kname(b).startswith("ogm_gemv_kernel")
         y17 = b.matmul(x[:17], 17, w)
-        assert b.last_kernel() == "ogm_gemm_flat_kernel"
+        assert kname(b) == "ogm_gemm_flat_kernel"
         assert_bits(y17, want, "Q8_0, 17 tokens")
         assert_bits(y16, want[:16], "Q8_0, 16 tokens")
         raw = synth_weights(Q4_K, 1024, 70, seed=5)
@@ -545,19 +560,19 @@ def test_gemm_threshold_default():
         for n, kernel in ((8, "ogm_gemv_kernel"), (9, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
                           (129, "ogm_gemm_q4k_i8p_r64_kernel")):
             y = b.matmul(x[:n], n, w)
-            assert b.last_kernel().startswith(kernel), (n, b.last_kernel())
+            assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, want[:n], f"Q4_K, {n} tokens")
         raw = synth_weights(Q5_K, 4096, 70, seed=7)    # few workgroups, sixteen super-blocks: sixteen waves
         x4 = synth_x(12, 4096, seed=8)
         y = b.matmul(x4, 12, qm(raw, Q5_K, 4096, 70))
-        assert b.last_kernel() == "ogm_gemm_sb_q5k_w16_kernel"
+        assert kname(b) == "ogm_gemm_sb_q5k_w16_kernel"
         assert_bits(y, oracle.matmul(Q5_K, raw, 4096, 70, x4, 12), "Q5_K, 12 tokens")
         raw = synth_weights(Q6_K, 256, 8300, seed=6)   # 130 tiles of 64 rows
         w = qm(raw, Q6_K, 256, 8300)
         want = oracle.matmul(Q6_K, raw, 256, 8300, np.ascontiguousarray(x[:65, :256]), 65).reshape(65, 8300)
         for n, kernel in ((64, "ogm_gemm_sb_q6k_kernel"), (65, "ogm_gemm_q6k_i8_r64_kernel")):
             y = b.matmul(np.ascontiguousarray(x[:n, :256]), n, w)
-            assert b.last_kernel() == kernel, (n, b.last_kernel())
+            assert kname(b) == kernel, (n, kname(b))
             assert_bits(y, want[:n], f"Q6_K, {n} tokens")
     finally:
         b.close()
@@ -582,7 +597,7 @@ def test_small_batch_gemm_matches_cpu_gemm(be, t, in_dim, out_dim, T, waves):
     finally:
         be.set_tuning("gemm_small_max_tokens", 1)
         be.set_tuning("gemm_sb_waves", 8)
-    assert be.last_kernel() == {Q4_K: "ogm_gemm_sb_q4k", Q5_K: "ogm_gemm_sb_q5k", Q6_K: "ogm_gemm_sb_q6k"}[t] + \
+    assert kname(be) == {Q4_K: "ogm_gemm_sb_q4k", Q5_K: "ogm_gemm_sb_q5k", Q6_K: "ogm_gemm_sb_q6k"}[t] + \
         ("_w16_kernel" if waves == 16 else "_kernel")
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "small-batch gemm")
 
@@ -610,7 +625,7 @@ def test_small_batch_gemm_extreme_integer_ranges(be, t, block, hi, waves):
     finally:
         be.set_tuning("gemm_small_max_tokens", 1)
         be.set_tuning("gemm_sb_waves", 8)
-    assert be.last_kernel().startswith("ogm_gemm_sb_") and ("_w16_" in be.last_kernel()) == (waves == 16)
+    assert kname(be).startswith("ogm_gemm_sb_") and ("_w16_" in kname(be)) == (waves == 16)
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "extreme ranges")
 
 
@@ -623,10 +638,10 @@ def test_mfma_gemm_rows_too_long_for_the_plane_kernel(be):
     raw = synth_weights(t, in_dim, out_dim, seed=4)
     x = synth_x(T, in_dim, seed=5)
     got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
-    assert be.last_kernel() == "ogm_gemm_q4k_i8_kernel"
+    assert kname(be) == "ogm_gemm_q4k_i8_kernel"
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "long rows")
     got = be.matmul(x, T, qm(synth_weights(Q5_K, in_dim, out_dim, seed=6), Q5_K, in_dim, out_dim))
-    assert be.last_kernel().startswith("ogm_gemv_kernel")
+    assert kname(be).startswith("ogm_gemv_kernel")
     assert_bits(got, oracle.matmul(Q5_K, synth_weights(Q5_K, in_dim, out_dim, seed=6), in_dim, out_dim, x, T), "long rows, Q5_K")
 
 
@@ -671,7 +686,7 @@ def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, ou
         be.set_tuning("gemm_q4k_variant", 0)
         be.set_tuning("gemm_small_max_tokens", 1)
     device_synchronize()
-    assert be.last_kernel() == kernel
+    assert kname(be) == kernel
     for r, od, yd in zip(raws, outs, yds):
         want = oracle.matmul(t, r, in_dim, od, x, n_tokens)
         assert_bits(yd.to_numpy(np.float32, n_tokens * od), want, f"{od} rows of {outs}")
@@ -692,7 +707,7 @@ def test_mfma_gemm_equals_small_batch_kernel_and_is_batch_independent(be):
     be.set_tuning("gemm_min_tokens", 1000)
     try:
         small = be.matmul(x, 40, w).reshape(40, out_dim)
-        assert be.last_kernel().startswith("ogm_gemv_kernel")
+        assert kname(be).startswith("ogm_gemv_kernel")
     finally:
         be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(full, small, "mfma vs multi-token gemv")
@@ -736,7 +751,7 @@ def test_mfma_gemm_adversarial_integer_ranges(be, qs_lo, qs_hi, sign, T, variant
     finally:
         be.set_tuning("gemm_wide_min_wgs", 0)
         be.set_tuning("gemm_q4k_variant", 0)
-    assert be.last_kernel() == ("ogm_gemm_q4k_i8p_r64_kernel" if variant == 0 else
+    assert kname(be) == ("ogm_gemm_q4k_i8p_r64_kernel" if variant == 0 else
                                 "ogm_gemm_q4k_i8_kernel" if variant == 3 else
                                 "ogm_gemm_q4k_wide_kernel" if T > 256 else "ogm_gemm_q4k_kernel")
     want = oracle.matmul(Q4_K, raw, in_dim, out_dim, x, T)
@@ -765,7 +780,7 @@ def test_mfma_gemm_q6k_matches_cpu_gemm(be, in_dim, out_dim, T, variant):
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
     small_grid = ((T + 127) // 128) * ((out_dim + 63) // 64) <= 256
-    assert be.last_kernel() == ("ogm_gemm_q6k_kernel" if variant == 2 else "ogm_gemm_q6k_i8_r64_kernel"
+    assert kname(be) == ("ogm_gemm_q6k_kernel" if variant == 2 else "ogm_gemm_q6k_i8_r64_kernel"
                                 if variant == 1 or small_grid else "ogm_gemm_q6k_i8_kernel")
     want = oracle.matmul(Q6_K, raw, in_dim, out_dim, x, T)
     assert_close(got, want, "mfma gemm q6k")
@@ -773,7 +788,7 @@ def test_mfma_gemm_q6k_matches_cpu_gemm(be, in_dim, out_dim, T, variant):
     be.set_tuning("gemm_min_tokens", 100000)
     try:
         small = be.matmul(x, T, w)
-        assert be.last_kernel().startswith("ogm_gemv_kernel")
+        assert kname(be).startswith("ogm_gemv_kernel")
     finally:
         be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(got, small, "mfma vs multi-token gemv")
@@ -810,7 +825,7 @@ def test_mfma_gemm_q6k_adversarial_integer_ranges(be, ql, qh, sc, sign, variant)
         got = be.matmul(x, T, qm(raw, Q6_K, in_dim, out_dim))
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
-    assert be.last_kernel() == {0: "ogm_gemm_q6k_i8_r64_kernel", 3: "ogm_gemm_q6k_i8_kernel", 2: "ogm_gemm_q6k_kernel"}[variant]
+    assert kname(be) == {0: "ogm_gemm_q6k_i8_r64_kernel", 3: "ogm_gemm_q6k_i8_kernel", 2: "ogm_gemm_q6k_kernel"}[variant]
     want = oracle.matmul(Q6_K, raw, in_dim, out_dim, x, T)
     assert_bits(got, want, "extreme ranges")
     isum, _ = be.dump_block_sums(x[0], 1, qm(raw, Q6_K, in_dim, out_dim))
@@ -840,14 +855,14 @@ def test_mfma_gemm_q3k_q5k_match_cpu_gemm(be, t, kernel, in_dim, out_dim, T):
         be.set_tuning("gemm_q4k_variant", 0)
     if variant_of(kernel) == 0:
         kernel = plane_kernel(kernel[:-len("_kernel")], T, out_dim)
-    assert be.last_kernel() == kernel
+    assert kname(be) == kernel
     want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
     assert_close(got, want, kernel)
     assert_bits(got, want, kernel)
     be.set_tuning("gemm_min_tokens", 100000)
     try:
         small = be.matmul(x, T, w)
-        assert be.last_kernel().startswith("ogm_gemv_kernel")
+        assert kname(be).startswith("ogm_gemv_kernel")
     finally:
         be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(got, small, "mfma vs multi-token gemv")
@@ -882,7 +897,7 @@ def test_mfma_gemm_q5k_adversarial_integer_ranges(be, qs, qh, sc, sign, variant)
         got = be.matmul(x, T, qm(raw, Q5_K, in_dim, out_dim))
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
-    assert be.last_kernel() == {0: "ogm_gemm_q5k_i8p_r64_kernel", 3: "ogm_gemm_q5k_i8_kernel", 2: "ogm_gemm_q5k_kernel"}[variant]
+    assert kname(be) == {0: "ogm_gemm_q5k_i8p_r64_kernel", 3: "ogm_gemm_q5k_i8_kernel", 2: "ogm_gemm_q5k_kernel"}[variant]
     assert_bits(got, oracle.matmul(Q5_K, raw, in_dim, out_dim, x, T), "extreme ranges")
     isum, imin = be.dump_block_sums(x[0], 1, qm(raw, Q5_K, in_dim, out_dim))
     say("extreme q5k isum", int(np.abs(isum).max()), "imin", int(np.abs(imin).max()))
@@ -917,7 +932,7 @@ def test_mfma_gemm_q3k_adversarial_integer_ranges(be, qs, hm, sc, sign, variant)
         got = be.matmul(x, T, qm(raw, Q3_K, in_dim, out_dim))
     finally:
         be.set_tuning("gemm_q4k_variant", 0)
-    assert be.last_kernel() == {0: "ogm_gemm_q3k_i8_r64_kernel", 3: "ogm_gemm_q3k_i8_kernel", 2: "ogm_gemm_q3k_kernel"}[variant]
+    assert kname(be) == {0: "ogm_gemm_q3k_i8_r64_kernel", 3: "ogm_gemm_q3k_i8_kernel", 2: "ogm_gemm_q3k_kernel"}[variant]
     assert_bits(got, oracle.matmul(Q3_K, raw, in_dim, out_dim, x, T), "extreme ranges")
 
 
@@ -1183,14 +1198,14 @@ def test_mfma_gemm_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T):
     w = qm(raw, t, in_dim, out_dim)
     say("flat gemm", t, in_dim, out_dim, T)
     got = be.matmul(x, T, w)
-    assert be.last_kernel() == "ogm_gemm_flat_kernel"
+    assert kname(be) == "ogm_gemm_flat_kernel"
     want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
     assert_close(got, want, "flat mfma gemm")
     assert_bits(got, want, "flat mfma gemm")
     be.set_tuning("gemm_min_tokens", 100000)
     try:
         small = be.matmul(x, T, w)
-        assert be.last_kernel().startswith("ogm_gemv_kernel")
+        assert kname(be).startswith("ogm_gemv_kernel")
     finally:
         be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(small, want, "multi-token gemv")
@@ -1213,7 +1228,7 @@ def test_mfma_gemm_flat_extreme_block_sums(be, t):
     x[:, 5::11] = -127.0
     w = qm(raw, t, in_dim, out_dim)
     got = be.matmul(x, T, w)
-    assert be.last_kernel() == "ogm_gemm_flat_kernel"
+    assert kname(be) == "ogm_gemm_flat_kernel"
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "extreme sums")
     isum, _ = be.dump_block_sums(x[0], 1, w)
     say("flat extreme isum", t, int(np.abs(isum).max()))
