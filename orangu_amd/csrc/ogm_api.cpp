@@ -60,6 +60,7 @@ struct ogm_ctx {
   int tune_gemm_q4k_variant = 0;
   int tune_gemm_small_max = 0;   // most tokens for the small-batch GEMM kernel: 0 = default, 1 = never
   int tune_gemm_sb_waves = 0;          // small-batch GEMM: 8 or 16 waves per workgroup, 0 = by the launch
+  int tune_gemm_plane_kernel = 0;      // with planes: 0 the all-waves-multiply kernel, 1 the feeding-wave kernels
   int tune_decode_fuse_tails = 0;      // 1: the decode step's norms and SwiGLU inside the GEMV before them (slower)
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
@@ -261,6 +262,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemm_small_max_tokens") == 0) {
     if (value < 0 || value > 1024) return fail(ctx, OGM_ERR_INVALID, "gemm_small_max_tokens must be 0..1024");
     ctx->tune_gemm_small_max = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_plane_kernel") == 0) {
+    if (value != 0 && value != 1) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_kernel must be 0 or 1");
+    ctx->tune_gemm_plane_kernel = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_sb_waves") == 0) {
@@ -538,6 +544,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.q4k_variant = (uint32_t)ctx->tune_gemm_q4k_variant;
       g.small_max_tokens = (uint32_t)ctx->tune_gemm_small_max;
       g.sb_waves = (uint32_t)ctx->tune_gemm_sb_waves;
+      g.plane_kernel = (uint32_t)ctx->tune_gemm_plane_kernel;
       g.n_extra = (uint32_t)ng - 1;
       for (size_t j = 1; j < ng; j++) {
         g.extra_wt[j - 1] = tg[i + j].w->dev;

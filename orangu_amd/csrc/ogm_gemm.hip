@@ -1321,6 +1321,400 @@ __global__ __launch_bounds__(256) void ogm_gemm_build_planes_kernel(GemmPlaneBui
 }
 
 // ------------------------------------------------------------------------------------------
+// The K-quant GEMM over prebuilt planes with every wave multiplying (no feeding waves): operands
+// go from global memory straight into LDS (global_load_lds_dwordx4: no registers, no vector
+// work), in the order the matrix instruction wants them, so a wave's operand read is 64 lanes x 16
+// consecutive bytes.  Same arithmetic and f32 order as gemm_q6k_i8_body; bit-identical results.
+//
+//   workgroup  256 threads = 4 waves; 128 rows x 128 tokens; wave w: rows 32 w .. + 31, all tokens.
+//              Two workgroups share a compute unit (two waves per SIMD, 74 KiB of LDS each): while
+//              one adds a super-block's sums up in f32 the other multiplies.
+//   step       32 weights of k: per wave the planes of its 32 rows (1 KiB each, fetched by the wave
+//              itself), per workgroup four token blocks of activations (1 KiB each, one per wave)
+//   ring       six steps in LDS: one multiplied, the next being read into registers behind it,
+//              four in flight.  At the top of step k a wave waits until its loads of step k + 1
+//              have landed (all but the newest three steps' loads), meets the others at a barrier,
+//              and fetches step k + 5 into the slot step k - 1 left.
+//   per super-block: the tokens' activation scales and the rows' d, fetched the same way one
+//              super-block ahead (4 bytes a lane), then acc += ad * (d * isum) as the CPU path adds it
+//
+// The compiler cannot tell which LDS reads a load-to-LDS in flight may alias and would wait for all
+// of them before every LDS read; the operand and table reads of the main loop are therefore written
+// as ds_read instructions with their own waits (LDS reads return in order: "at most N outstanding"
+// means all but the newest N have landed).  No scalar loads may be issued inside the loop (they
+// share the counter and return out of order), which the launch parameters being read up front ensures.
+//
+// Registers: 8 accumulators of the planes (4 token blocks x h, l), 4 of y, 6 operands: 216 of a wave's 256.
+struct GemmDmaParams {
+  const uint8_t *wt;       // tile-planar weights (headers: d, dmin, mins)
+  const uint8_t *planes;   // ogm_gemm_build_planes_kernel's output
+  const int8_t *xt;        // ogm_gemm_xtile_kernel's output: [T / 32][in_dim / 32] operand chunks of 1 KiB
+  const float *ad;         // [T][nsb]
+  const _Float16 *bs16;    // Q4_K / Q5_K first pass
+  float *y;
+  uint32_t in_dim, out_dim, n_tokens, nsb;
+  uint32_t c_shift, r_shift, nct;
+  uint32_t n_extra;
+  const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1];
+  const uint8_t *extra_planes[OGM_GEMM_MAX_MATS - 1];
+  float *extra_y[OGM_GEMM_MAX_MATS - 1];
+  uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
+};
+
+#define GD_NW 4u                       // waves of a workgroup
+#define GD_ROWS (32u * GD_NW)
+#define GD_TOK 128u
+// timing experiments only (results are wrong with any of these set)
+#ifndef GD_ABL_SAMEROW
+#define GD_ABL_SAMEROW 0   // every workgroup reads row block 0's planes
+#endif
+#ifndef GD_ABL_NOSWZ
+#define GD_ABL_NOSWZ 0     // workgroups keep the grid's order
+#endif
+#ifndef GD_ABL_NOPASS1
+#define GD_ABL_NOPASS1 0
+#endif
+#ifndef GD_ABL_NOEPI
+#define GD_ABL_NOEPI 0
+#endif
+#ifndef GD_ABL_NOMFMA
+#define GD_ABL_NOMFMA 0
+#endif
+#ifndef GD_ABL_NODMA
+#define GD_ABL_NODMA 0
+#endif
+#ifndef GD_ABL_NOBAR
+#define GD_ABL_NOBAR 0
+#endif
+#ifndef GD_ABL_NOLDS
+#define GD_ABL_NOLDS 0
+#endif
+#define GD_RING 6u
+#define GD_AHEAD (GD_RING - 1u)        // steps fetched ahead of the one multiplied
+#define GD_XOFF (GD_NW * 2048u)        // activations of a step, after the weights' 2 KiB per wave
+#define GD_SLOT (GD_XOFF + 4096u)      // bytes of a step in LDS (one-plane types leave half the weights' part unused)
+#define GD_TAB (GD_RING * GD_SLOT)     // two slots of per-super-block tables: 128 ad, then the rows' header words
+#define GD_TAB_SLOT (512u + 4u * GD_ROWS)
+#define GD_LDS_BYTES (GD_TAB + 2u * GD_TAB_SLOT)
+
+__device__ __forceinline__ void gd_dma16(const uint8_t *src, uint8_t *lds_chunk) {
+  // 16 bytes per lane from src (per lane) to lds_chunk + 16 * lane (lds_chunk is wave-uniform)
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                   (__attribute__((address_space(3))) void *)lds_chunk, 16, 0, 0);
+}
+__device__ __forceinline__ void gd_dma4(const uint8_t *src, uint8_t *lds_chunk) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                   (__attribute__((address_space(3))) void *)lds_chunk, 4, 0, 0);
+}
+// LDS reads the compiler does not see, and the waits that go with them.  A wait names the
+// registers it makes valid, so that their uses stay behind it.
+#define GD_READ16(DST, ADDR, OFF) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(DST) : "v"(ADDR), "n"(OFF))
+#define GD_READ4(DST, ADDR, OFF) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(DST) : "v"(ADDR), "n"(OFF))
+#define GD_WAIT1(N, A) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(A) : "n"(N))
+#define GD_WAIT2(N, A, B) asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(A), "+v"(B) : "n"(N))
+// all loads of this wave but the newest N have landed; then the workgroup's barrier (no fence: the
+// data other waves wait for came by load-to-LDS, which the wait covers)
+#if GD_ABL_NOBAR
+#define GD_SYNC(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
+#else
+#define GD_SYNC(N) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory")
+#endif
+
+// The activations in the matrix instruction's operand order: chunk (token block of 32, step of 32 k)
+// is 1 KiB, lane (l32, lh)'s 16 bytes -- the activations 32 step + 16 lh .. of token 32 block + l32 --
+// at 16 (32 lh + l32).  A chunk is then one contiguous load; fetched row by row it would be 32 pieces
+// of 32 distinct cache lines.  Tokens past the last repeat it (never stored).
+__global__ __launch_bounds__(256) void ogm_gemm_xtile_kernel(const int8_t *__restrict__ xq, int8_t *__restrict__ xt,
+                                                             uint32_t in_dim, uint32_t n_tokens, uint32_t n_pieces) {
+  // thread = one 16-byte piece, pieces of a token consecutive: whole rows are read in order
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= n_pieces) return;
+  const uint32_t ppr = in_dim / 16u, tok = i / ppr, c = i - tok * ppr;
+  const uint4 v = *(const uint4 *)(xq + (size_t)min(tok, n_tokens - 1u) * in_dim + 16u * c);
+  const uint32_t chunk = (tok >> 5) * (in_dim / 32u) + (c >> 1);
+  *(uint4 *)(xt + (size_t)chunk * 1024u + (32u * (c & 1u) + (tok & 31u)) * 16u) = v;
+}
+
+#if GD_ABL_NOMFMA
+#define GD_MFMA(A, B, C, X, Y, Z) ((C) + (A).x + (B).x)
+#else
+#define GD_MFMA(A, B, C, X, Y, Z) __builtin_amdgcn_mfma_i32_32x32x32_i8(A, B, C, X, Y, Z)
+#endif
+#if GD_ABL_NOLDS
+#define GD_RD if (0)
+#else
+#define GD_RD
+#endif
+template <int KIND>
+__global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaParams p) {
+  constexpr bool Q3 = KIND == GP_Q3K, Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K, Q6 = KIND == GP_Q6K;
+  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : KIND == GP_Q4K ? 9216u : Q5 ? 11264u : 13440u;
+  constexpr uint32_t NPL = Q3 ? 1u : 2u;
+  constexpr int PER = (int)NPL + 1;   // loads a wave issues per step
+  extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  // Workgroups are dealt to the eight XCDs in turn, each with an L2 of its own: the token tiles of
+  // one row tile go to one XCD back to back, so the row tile's planes leave memory once.
+  uint32_t tok_tile = blockIdx.x, row_tile = blockIdx.y;
+  {
+    const uint32_t nt = gridDim.x, lin = blockIdx.y * nt + blockIdx.x;
+    if (!GD_ABL_NOSWZ && lin < (gridDim.y & ~7u) * nt) {
+      const uint32_t j = lin >> 3;
+      tok_tile = j % nt;
+      row_tile = (j / nt) * 8u + (lin & 7u);
+    }
+  }
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + GD_ROWS - 1u) / GD_ROWS;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.planes = p.extra_planes[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = tok_tile * GD_TOK, r0 = row_tile * GD_ROWS;
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
+  };
+
+  float16v y[4];
+#pragma unroll
+  for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) y[tb][r] = 0.0f;
+
+  if constexpr (Q45 && !GD_ABL_NOPASS1) {
+    // ---------------- pass 1 of gemm_k_q4_k: acc -= (ad * dmin) * sum_j m_j * bsum_j over all
+    // super-blocks first (vecdot.rs:2226-2240), as gemm_q6k_i8_body does it: 64 m_j against bsum_j / 64
+    // and m_j against bsum_j % 64 in one K = 16 f16 instruction per 32 x 32 outputs.  The tokens' ad of
+    // every super-block sit in LDS (where the ring will be) for this pass.
+    // this lane's weight row (clamped: rows past the matrix are computed and never stored)
+    const uint32_t row = min(r0 + 32u * wave + l32, p.out_dim - 1u);
+    const uint32_t uo = (row >> p.r_shift) * p.nct * TILE_BYTES + (row & ((1u << p.r_shift) - 1u)) * 16u;
+    float *ad_all = (float *)lds;   // [nsb][128]
+    for (uint32_t i = tid; i < GD_TOK * p.nsb; i += 64u * GD_NW) {
+      const uint32_t k = i / p.nsb, su = i - k * p.nsb;
+      ad_all[su * GD_TOK + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + su];
+    }
+    __syncthreads();
+    float16v zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.0f;
+    uint32_t tk[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) tk[tb] = min(t0 + 32u * tb + l32, p.n_tokens - 1u) * p.nsb;
+    const float side_scale = lh ? 1.0f : 64.0f;
+    // the header and the four tokens' sums of the next super-block are loaded while this one is added up
+    uint4 hd_n = *(const uint4 *)(p.wt + uo);
+    half8 b2_n[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) b2_n[tb] = *(const half8 *)(p.bs16 + (tk[tb] * 16u + 8u * lh));
+    for (uint32_t su = 0; su < p.nsb; su++) {
+      const uint4 hd0 = hd_n;
+      half8 b2[4];
+#pragma unroll
+      for (int tb = 0; tb < 4; tb++) b2[tb] = b2_n[tb];
+      {
+        const uint32_t sn = min(su + 1u, p.nsb - 1u);   // past the end: loaded again, never used
+        hd_n = *(const uint4 *)(p.wt + (uo + sb_off(sn)));
+#pragma unroll
+        for (int tb = 0; tb < 4; tb++) b2_n[tb] = *(const half8 *)(p.bs16 + ((tk[tb] + sn) * 16u + 8u * lh));
+      }
+      uint32_t mna, mnb;
+      q4k_mins(hd0, mna, mnb);
+      const half8 a1 = side_operand(mna, mnb, side_scale);
+      const float dm = gm_f16_bits_to_f32(hd0.x >> 16);
+#pragma unroll
+      for (int tb = 0; tb < 4; tb++) {
+        const float16v im = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2[tb], a1, zero, 0, 0, 0);
+        const float *adp = &ad_all[su * GD_TOK + 32u * tb + 4u * lh];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          const float4 a4 = *(const float4 *)(adp + 8 * q4);
+          const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+          for (int e = 0; e < 4; e++) y[tb][4 * q4 + e] -= a4v[e] * dm * im[4 * q4 + e];
+        }
+      }
+    }
+    __syncthreads();   // the table's LDS becomes the ring
+  }
+
+  // ---------------- the products
+  // What this wave fetches per step: the plane chunks of its 32 rows (lane (l32, lh): the 16 weights
+  // 16 lh .. of row l32, the matrix instruction's operand), and token block `wave` of the activations
+  // (one chunk of ogm_gemm_xtile_kernel's layout).
+  const uint32_t prb = GD_ABL_SAMEROW ? 0u : min((r0 + 32u * wave) >> 6, (p.out_dim - 1u) >> 6);
+  uint32_t w_src = (prb * p.nsb * 16u + lh) * (NPL * 1024u) + (32u * (wave & 1u) + l32) * 16u;   // + step * NPL * 2048
+  // (token blocks past the last one read it again; their outputs are never stored)
+  uint32_t x_src = min((t0 >> 5) + wave, (p.n_tokens - 1u) >> 5) * (p.in_dim / 32u) * 1024u + lane * 16u;   // + step * 1024
+  const uint32_t w_dst = wave * 2048u, x_dst = GD_XOFF + wave * 1024u;
+  // tables: waves 0, 1 fetch 64 tokens' ad each, waves 2, 3 the header word of 64 rows each
+  uint32_t tab_src;   // byte offset from p.ad (waves 0, 1) or p.wt (waves 2..5) for super-block 0
+  if (wave < 2u) {
+    tab_src = min(t0 + 64u * wave + lane, p.n_tokens - 1u) * p.nsb * 4u;
+  } else {
+    const uint32_t tab_row = min(r0 + 64u * ((wave - 2u) & 3u) + lane, p.out_dim - 1u);
+    const uint32_t tab_rb = tab_row >> p.r_shift, tab_r = tab_row & ((1u << p.r_shift) - 1u);
+    if constexpr (Q6)        // d is the block's two-byte tail behind the 13 pieces: the aligned word that holds it
+      tab_src = tab_rb * p.nct * TILE_BYTES + 13u * 1024u + ((tab_r * 2u) & ~3u);
+    else if constexpr (Q3)   // scales[12] | d | padding
+      tab_src = tab_rb * p.nct * TILE_BYTES + tab_r * 16u + 6u * 1024u + 12u;
+    else                     // d | dmin
+      tab_src = tab_rb * p.nct * TILE_BYTES + tab_r * 16u;
+  }
+  auto fetch_tables = [&](uint32_t s) {   // for super-block s, into table slot s & 1
+    uint8_t *slot = lds + GD_TAB + (s & 1u) * GD_TAB_SLOT;
+    if (wave < 2u) {
+      gd_dma4((const uint8_t *)p.ad + (tab_src + 4u * s), slot + 256u * wave);
+    } else {
+      const uint32_t so = Q6 ? (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 2u : sb_off(s);
+      gd_dma4(p.wt + (tab_src + so), slot + 512u + 256u * (wave - 2u));
+    }
+  };
+  uint32_t slot_fetch = 0;   // byte offset of the ring slot of the next step to fetch
+  auto fetch_step = [&]() {   // the next step (they are fetched in ascending order) into its ring slot
+    uint8_t *slot = lds + slot_fetch;
+    slot_fetch = slot_fetch == (GD_RING - 1u) * GD_SLOT ? 0u : slot_fetch + GD_SLOT;
+#if !GD_ABL_NOWDMA
+    gd_dma16(p.planes + w_src, slot + w_dst);
+    if constexpr (!Q3) gd_dma16(p.planes + (w_src + 1024u), slot + w_dst + 1024u);
+#endif
+#if !GD_ABL_NOXDMA
+    gd_dma16((const uint8_t *)p.xt + x_src, slot + x_dst);
+#endif
+    w_src += NPL * 2048u;
+    x_src += 1024u;
+  };
+
+  fetch_tables(0u);
+#pragma unroll
+  for (uint32_t k = 0; k < GD_AHEAD; k++) fetch_step();
+  GD_SYNC((GD_AHEAD - 1) * PER);   // step 0 and the first tables have landed
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+  const uint32_t w_rd = lds0 + w_dst + lane * 16u, x_rd = lds0 + GD_XOFF + lane * 16u;
+  const uint32_t tab_rd = lds0 + GD_TAB + 16u * lh;                    // + 128 tb + 32 q4: four tokens' ad
+  const uint32_t hw_rd = lds0 + GD_TAB + 512u + 4u * (32u * wave + l32);   // the row's header word
+  int16v h[4], l[4];
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  int4v wh, wl = {0, 0, 0, 0}, x0, x1, x2, x3;
+  // LDS reads outstanding at the top of a step, oldest first: wh, x0, x1, x2, x3, wl (one-plane types: no wl)
+  GD_READ16(wh, w_rd, 0);
+  GD_READ16(x0, x_rd, 0);
+  GD_READ16(x1, x_rd, 1024);
+  GD_READ16(x2, x_rd, 2048);
+  GD_READ16(x3, x_rd, 3072);
+  if constexpr (!Q3) GD_READ16(wl, w_rd, 1024);
+  uint32_t slot_next = GD_SLOT;   // byte offset of step k + 1's ring slot
+  for (uint32_t s = 0; s < p.nsb; s++) {
+#pragma unroll
+    for (uint32_t kk = 0; kk < 8u; kk++) {
+      // step k = 8 s + kk: step k + 1 landed (all but the loads of the steps after it, at most four), for every wave
+      const bool more = s + 1u < p.nsb;   // in the last super-block the steps in flight run out
+      // (steps after k + 1 in flight: GD_AHEAD - 2, fewer at the end)
+      if (kk + GD_AHEAD <= 8u || more) GD_SYNC((GD_AHEAD - 2) * PER);
+      else GD_SYNC(kk >= 6u ? 0 : (int)(6u - kk) * PER);
+      if (kk == 0u && more) fetch_tables(s + 1u);
+      if ((kk + GD_AHEAD < 8u || more) && !GD_ABL_NODMA) fetch_step();   // step k + GD_AHEAD
+      const uint32_t w_nx = w_rd + slot_next, x_nx = x_rd + slot_next;
+      slot_next = slot_next == (GD_RING - 1u) * GD_SLOT ? 0u : slot_next + GD_SLOT;
+      if constexpr (!Q3) {
+        constexpr int A0 = 4;   // outstanding after wh and x0: x1, x2, x3, wl
+        GD_WAIT2(A0, wh, x0);
+        h[0] = GD_MFMA(x0, wh, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : h[0], 0, 0, 0);
+        GD_WAIT1(3, x1);
+        h[1] = GD_MFMA(x1, wh, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : h[1], 0, 0, 0);
+        GD_WAIT1(2, x2);
+        h[2] = GD_MFMA(x2, wh, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : h[2], 0, 0, 0);
+        GD_WAIT1(1, x3);
+        h[3] = GD_MFMA(x3, wh, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : h[3], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:0" : "=v"(wh) : "0"(wh), "v"(w_nx));
+        GD_WAIT1(1, wl);
+        l[0] = GD_MFMA(x0, wl, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : l[0], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:0" : "=v"(x0) : "0"(x0), "v"(x_nx));
+        l[1] = GD_MFMA(x1, wl, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : l[1], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:1024" : "=v"(x1) : "0"(x1), "v"(x_nx));
+        l[2] = GD_MFMA(x2, wl, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : l[2], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:2048" : "=v"(x2) : "0"(x2), "v"(x_nx));
+        l[3] = GD_MFMA(x3, wl, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : l[3], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:3072" : "=v"(x3) : "0"(x3), "v"(x_nx));
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:1024" : "=v"(wl) : "0"(wl), "v"(w_nx));
+      } else {
+        // one plane: the next step's weights go to a second register set (this one is in use to the
+        // end); outstanding at the top, oldest first: wh, x0, x1, x2, x3
+        int4v wn;
+        GD_READ16(wn, w_nx, 0);
+        GD_WAIT2(4, wh, x0);
+        h[0] = GD_MFMA(x0, wh, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : h[0], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:0" : "=v"(x0) : "0"(x0), "v"(x_nx));
+        GD_WAIT1(4, x1);
+        h[1] = GD_MFMA(x1, wh, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : h[1], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:1024" : "=v"(x1) : "0"(x1), "v"(x_nx));
+        GD_WAIT1(4, x2);
+        h[2] = GD_MFMA(x2, wh, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : h[2], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:2048" : "=v"(x2) : "0"(x2), "v"(x_nx));
+        GD_WAIT1(4, x3);
+        h[3] = GD_MFMA(x3, wh, (kk == 0u && (!GD_ABL_NOEPI || s == 0u)) ? zi : h[3], 0, 0, 0);
+        GD_RD asm volatile("ds_read_b128 %0, %2 offset:3072" : "=v"(x3) : "0"(x3), "v"(x_nx));
+        // the next step wants wn first in line: it was issued before these four
+        GD_WAIT1(4, wn);
+        wh = wn;
+      }
+      if (kk == 7u && (!GD_ABL_NOEPI || s + 1u == p.nsb)) {
+        // acc += ad * (d * isum) for the super-block (vecdot.rs:2242-2300 in the order of its sums)
+        const uint32_t tsl = (s & 1u) * GD_TAB_SLOT;
+        uint32_t hw;
+        GD_READ4(hw, hw_rd + tsl, 0);
+        GD_WAIT1(0, hw);
+        // Q6_K's word holds the d of a pair of rows
+        const float d0 = gm_f16_bits_to_f32(Q6 && (l32 & 1u) ? (hw >> 16) : (hw & 0xFFFFu));
+        const uint32_t ta = tab_rd + tsl;
+#pragma unroll
+        for (int tb = 0; tb < 4; tb++) {
+          typedef float float4v __attribute__((ext_vector_type(4)));
+          float4v a40, a41, a42, a43;
+          GD_READ16(a40, ta, 128 * tb);
+          GD_READ16(a41, ta, 128 * tb + 32);
+          GD_READ16(a42, ta, 128 * tb + 64);
+          GD_READ16(a43, ta, 128 * tb + 96);
+          GD_WAIT2(0, a40, a41);
+          GD_WAIT2(0, a42, a43);
+          const float4v a4[4] = {a40, a41, a42, a43};
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++) {
+            const float a4v[4] = {a4[q4].x, a4[q4].y, a4[q4].z, a4[q4].w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const int is = Q3 ? -h[tb][4 * q4 + e] : h[tb][4 * q4 + e] * 256 + l[tb][4 * q4 + e];
+              y[tb][4 * q4 + e] += a4v[e] * (d0 * (float)is);
+            }
+          }
+        }
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wh), "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3), "+v"(wl));   // the reads past the last step
+  const uint32_t row0 = r0 + 32u * wave + l32;
+  if (row0 < p.out_dim) {
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const uint32_t t = t0 + 32u * tb + 8u * (r >> 2) + 4u * lh + (r & 3);
+        if (t < p.n_tokens) p.y[(size_t)t * p.out_dim + row0] = y[tb][r];
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Small batches (up to a few dozen tokens): the tiled kernels above cost the same for 9 tokens as
 // for 128, because a workgroup walks its rows' super-blocks one after the other.  Here a workgroup
 // owns 32 rows x 32 tokens and its eight waves take different super-blocks of those rows at the same
@@ -2895,6 +3289,58 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
       p.extra_planes[m] = m < a.n_extra ? a.extra_planes[m] : nullptr;
       if (m < a.n_extra && !a.extra_planes[m]) pre = false;   // every matrix of the launch, or none
+    }
+    // (the kernel addresses planes, weights and activations by 32-bit offsets)
+    // and wants the activations in operand chunks, for which the f16 scratch has room from 32 tokens
+    const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
+    bool dma = pre && a.plane_kernel == 0u && (!q45 || nsb * 512u <= GD_TAB) && a.n_tokens >= 32u && a.xh &&
+               (uint64_t)t_pad * a.in_dim < (1ull << 32);
+    for (uint32_t m = 0; m <= a.n_extra && dma; m++) {
+      const uint32_t od = m ? a.extra_out_dim[m - 1] : a.out_dim;
+      dma = (uint64_t)((od + 63u) / 64u) * 64u * a.in_dim * 2u < (1ull << 32);
+    }
+    if (dma) {
+      const uint32_t n_pieces = t_pad * (a.in_dim / 16u);
+      hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3((n_pieces + 255u) / 256u), dim3(256), 0, stream, a.act.q,
+                         (int8_t *)a.xh, a.in_dim, a.n_tokens, n_pieces);
+      GemmDmaParams d;
+      d.wt = a.wt;
+      d.planes = a.planes;
+      d.xt = (const int8_t *)a.xh;
+      d.ad = a.act.d;
+      d.bs16 = bs16;
+      d.y = a.y;
+      d.in_dim = a.in_dim;
+      d.out_dim = a.out_dim;
+      d.n_tokens = a.n_tokens;
+      d.nsb = nsb;
+      d.c_shift = c_shift;
+      d.r_shift = 6 - c_shift;
+      d.nct = tl.nct;
+      d.n_extra = a.n_extra;
+      uint32_t tiles256 = (a.out_dim + GD_ROWS - 1u) / GD_ROWS;
+      for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
+        d.extra_wt[m] = p.extra_wt[m];
+        d.extra_planes[m] = p.extra_planes[m];
+        d.extra_y[m] = p.extra_y[m];
+        d.extra_out_dim[m] = p.extra_out_dim[m];
+        if (m < a.n_extra) tiles256 += (a.extra_out_dim[m] + GD_ROWS - 1u) / GD_ROWS;
+      }
+      const void *fn = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_dma_kernel<GP_Q6K>
+                       : a.ggml_type == OGM_Q3_K ? (const void *)ogm_gemm_dma_kernel<GP_Q3K>
+                       : a.ggml_type == OGM_Q4_K ? (const void *)ogm_gemm_dma_kernel<GP_Q4K>
+                                                 : (const void *)ogm_gemm_dma_kernel<GP_Q5K>;
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)GD_LDS_BYTES);
+      if (e != hipSuccess) return e;
+      void *kargs[] = {(void *)&d};
+      e = hipLaunchKernel(fn, dim3((a.n_tokens + GD_TOK - 1u) / GD_TOK, tiles256), dim3(64u * GD_NW), kargs, GD_LDS_BYTES, stream);
+      if (e != hipSuccess) return e;
+      if (kernel_name)
+        *kernel_name = a.ggml_type == OGM_Q6_K   ? "ogm_gemm_q6k_dma_kernel"
+                       : a.ggml_type == OGM_Q3_K ? "ogm_gemm_q3k_dma_kernel"
+                       : a.ggml_type == OGM_Q4_K ? "ogm_gemm_q4k_dma_kernel"
+                                                 : "ogm_gemm_q5k_dma_kernel";
+      return hipGetLastError();
     }
     // 64-row tiles when asked for (q4k_variant 1), or when they still come one to a CU: then twice
     // as many CUs work (14336 -> 4096 x 512 tokens: 150 us against 180 us).  Two of them sharing a CU

@@ -31,10 +31,11 @@ def say(*a):
 GEMM_FROM = 9
 
 
-# Every test of this module runs twice: with the K-quant matrices' prefill planes built on first use
-# and kept (gemm_plane_cache_mb > 0; the tiled int8 kernels then carry "_pre" in their name) and with
-# none (the default: the same kernels unpack the weights on every call).  Same bits both ways.
-@pytest.fixture(scope="module", params=["planes", "unpack"])
+# Every test of this module runs three times: with the K-quant matrices' prefill planes built on first
+# use and kept (gemm_plane_cache_mb > 0) and read by the kernel whose waves all multiply ("planes":
+# ogm_gemm_q*_dma_kernel) or by the feeding-wave kernels ("planes_fed": "_pre" in their name), and with
+# none (the default: the feeding waves unpack the weights on every call).  Same bits all three ways.
+@pytest.fixture(scope="module", params=["planes", "planes_fed", "unpack"])
 def be(request):
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()  # raises if the HIP library or the device is missing: no fallback
@@ -42,18 +43,39 @@ def be(request):
     b.set_tuning("gemm_min_tokens", GEMM_FROM)
     b.set_tuning("gemm_small_max_tokens", 1)
     b.set_tuning("gemm_sb_waves", 8)
-    b.set_tuning("gemm_plane_cache_mb", 65536 if request.param == "planes" else 0)
+    b.set_tuning("gemm_plane_cache_mb", 0 if request.param == "unpack" else 65536)
+    b.set_tuning("gemm_plane_kernel", 1 if request.param == "planes_fed" else 0)
     b.plane_mode = request.param
     yield b
     b.close()
 
 
+class _TiledPlaneKernel(str):
+    """Name of the plane kernel that has no 64-row variant: equal to both names of its family."""
+
+    def __eq__(self, other):
+        return other in (str(self) + "_kernel", str(self) + "_r64_kernel")
+
+    def __ne__(self, other):
+        return not self.__eq__(other)
+
+    __hash__ = str.__hash__
+
+
 def kname(b):
-    """The last kernel's name without the "_pre" that marks a tiled int8 kernel reading prebuilt
-    planes; checks that the mark is there exactly when the backend keeps planes."""
+    """The last kernel's name as the tests of the unpacking kernels expect it: without the "_pre" of
+    a feeding-wave kernel that read prebuilt planes, and ogm_gemm_q*_dma_kernel as its family's tiled
+    kernel (of either row tiling).  Checks that the name fits the mode the backend runs in."""
     name = b.last_kernel()
+    mode = getattr(b, "plane_mode", "unpack")
+    m = re.match(r"ogm_gemm_q(6k|3k|4k|5k)_dma_kernel$", name)
+    if m:
+        assert mode == "planes", name
+        return _TiledPlaneKernel({"6k": "ogm_gemm_q6k_i8", "3k": "ogm_gemm_q3k_i8", "4k": "ogm_gemm_q4k_i8p",
+                                  "5k": "ogm_gemm_q5k_i8p"}[m.group(1)])
     if re.match(r"ogm_gemm_q(6k_i8|3k_i8|4k_i8p|5k_i8p)(_pre)?(_r64)?_kernel$", name):
-        assert ("_pre" in name) == (getattr(b, "plane_mode", "unpack") == "planes"), name
+        # (below 32 tokens the planes are read by a feeding-wave kernel in either mode)
+        assert ("_pre" in name) == (mode != "unpack"), name
     return name.replace("_pre", "")
 
 
