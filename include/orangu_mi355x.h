@@ -381,10 +381,15 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * 256 workgroups over rows of at least 16 super-blocks);
  * "attn_prefill_variant" (attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the
  * decode step's kernel per token and chunk of the cache; they agree to f32 rounding, not bit for bit);
- * "gemm_plane_cache_mb" (device memory, in MiB, that the K-quant matrices' prefill planes may take in all:
- * on a matrix's first tiled GEMM its scale-folded int8 planes -- 2 bytes per weight, 1 for Q3_K -- are
- * built once and kept, so that later calls multiply them instead of unpacking the weights again;
- * 0 = the default: build none and unpack on every call; ogm_weight_download is unaffected either way);
+ * "gemm_plane_cache_mb" (device memory, in MiB, that the K-quant matrices' prefill planes may take in all,
+ * default 32768: on a matrix's first GEMM that would read them its scale-folded int8 planes -- 2 bytes
+ * per weight, 1 for Q3_K -- are built once and kept, and later calls multiply them instead of unpacking the
+ * weights again; a matrix that no longer fits the budget, and every matrix at 0, is unpacked on every call;
+ * same bits either way, and ogm_weight_download is unaffected);
+ * "gemm_plane_kernel" (which kernel reads the planes: 0 = default, the one whose waves all multiply, fed by
+ * loads straight into LDS, when the launch has more than 256 tiles of 128 rows x 128 tokens, and otherwise
+ * none: the feeding-wave kernels unpack; 1 = the feeding-wave kernels read them; 2 = the former whatever the
+ * grid, from 32 tokens; same bits);
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
  * the quantizer kernel first; 0 or -1 = default, off);

@@ -60,14 +60,14 @@ struct ogm_ctx {
   int tune_gemm_q4k_variant = 0;
   int tune_gemm_small_max = 0;   // most tokens for the small-batch GEMM kernel: 0 = default, 1 = never
   int tune_gemm_sb_waves = 0;          // small-batch GEMM: 8 or 16 waves per workgroup, 0 = by the launch
-  int tune_gemm_plane_kernel = 0;      // with planes: 0 the all-waves-multiply kernel, 1 the feeding-wave kernels
+  int tune_gemm_plane_kernel = 0;      // who reads planes: 0 the all-waves-multiply kernel on large grids, 1 the feeding-wave kernels, 2 the former always
   int tune_decode_fuse_tails = 0;      // 1: the decode step's norms and SwiGLU inside the GEMV before them (slower)
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
   // Device memory the prefill planes of all weights may take, in MiB; 0 (the default) = build none.
   // A model's planes are 3.3 times its Q4_K bytes.
-  int tune_plane_cache_mb = 0;
+  int tune_plane_cache_mb = 32768;   // MiB the K-quant matrices' prefill planes may take in all
   size_t plane_bytes_used = 0;
   const char *last_kernel = "";
   uint8_t *static_scratch = nullptr;   // this device's copy of the library's static scratch array (ogm_static.hip)
@@ -265,7 +265,7 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     return OGM_OK;
   }
   if (strcmp(key, "gemm_plane_kernel") == 0) {
-    if (value != 0 && value != 1) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_kernel must be 0 or 1");
+    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_kernel must be 0, 1 or 2");
     ctx->tune_gemm_plane_kernel = value;
     return OGM_OK;
   }

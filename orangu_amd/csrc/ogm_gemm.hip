@@ -3118,10 +3118,32 @@ static int gemm_k_path(const OgmGemmArgs &a) {
   return 3;
 }
 
+// Whether a tiled plane launch (gemm_k_path 3) goes to the kernel whose waves all multiply, given
+// planes.  It wants more 128 x 128 workgroups than there are compute units (two share one, and one
+// alone is slower than the feeding-wave kernels: Q4_K 4096 -> 14336 at 256 tokens 69 us against 57, at
+// 384 tokens 87 against 104), the activations in operand chunks, for which the f16 scratch has room
+// from 32 tokens, and everything within 32-bit byte offsets.  (plane_kernel 2: whatever the grid.)
+static bool gemm_dma_eligible(const OgmGemmArgs &a) {
+  const uint32_t nsb = a.in_dim / 256;
+  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
+  if (a.plane_kernel == 1u || (q45 && nsb * 512u > GD_TAB) || a.n_tokens < 32u || !a.xh ||
+      (uint64_t)t_pad * a.in_dim >= (1ull << 32))
+    return false;
+  uint32_t tiles = 0;
+  for (uint32_t m = 0; m <= a.n_extra; m++) {
+    const uint32_t od = m ? a.extra_out_dim[m - 1] : a.out_dim;
+    if ((uint64_t)((od + 63u) / 64u) * 64u * a.in_dim * 2u >= (1ull << 32)) return false;
+    tiles += (od + GD_ROWS - 1u) / GD_ROWS;
+  }
+  return a.plane_kernel == 2u || ((a.n_tokens + GD_TOK - 1u) / GD_TOK) * tiles > 256u;
+}
+
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a) {
   if (a.n_tokens == 0 || a.out_dim == 0 || is_flat32(a.ggml_type)) return false;
   if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return false;
-  return gemm_k_path(a) == 3;
+  // the feeding-wave kernels read planes only when asked to (they are no faster for it)
+  return gemm_k_path(a) == 3 && (a.plane_kernel == 1u || gemm_dma_eligible(a));
 }
 
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name) {
@@ -3290,15 +3312,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       p.extra_planes[m] = m < a.n_extra ? a.extra_planes[m] : nullptr;
       if (m < a.n_extra && !a.extra_planes[m]) pre = false;   // every matrix of the launch, or none
     }
-    // (the kernel addresses planes, weights and activations by 32-bit offsets)
-    // and wants the activations in operand chunks, for which the f16 scratch has room from 32 tokens
     const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
-    bool dma = pre && a.plane_kernel == 0u && (!q45 || nsb * 512u <= GD_TAB) && a.n_tokens >= 32u && a.xh &&
-               (uint64_t)t_pad * a.in_dim < (1ull << 32);
-    for (uint32_t m = 0; m <= a.n_extra && dma; m++) {
-      const uint32_t od = m ? a.extra_out_dim[m - 1] : a.out_dim;
-      dma = (uint64_t)((od + 63u) / 64u) * 64u * a.in_dim * 2u < (1ull << 32);
-    }
+    const bool dma = pre && gemm_dma_eligible(a);
+    if (a.plane_kernel != 1u) pre = false;   // planes given, but not for the feeding-wave kernels
     if (dma) {
       const uint32_t n_pieces = t_pad * (a.in_dim / 16u);
       hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3((n_pieces + 255u) / 256u), dim3(256), 0, stream, a.act.q,

@@ -99,7 +99,10 @@ struct OgmGemmArgs {
   // weights again on every call.
   const uint8_t *planes = nullptr;
   const uint8_t *extra_planes[OGM_GEMM_MAX_MATS - 1] = {};
-  uint32_t plane_kernel = 0;   // with planes: 0 the kernel whose waves all multiply (operands by load-to-LDS), 1 the feeding-wave kernels
+  // which kernel reads planes: 0 the one whose waves all multiply (operands by load-to-LDS) when the
+  // grid fills the device twice, else none (the feeding waves unpack); 1 the feeding-wave kernels; 2
+  // the former whatever the grid
+  uint32_t plane_kernel = 0;
 };
 // Whether this launch would run a tiled int8 plane kernel, i.e. whether planes would be read.
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a);

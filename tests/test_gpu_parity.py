@@ -33,8 +33,9 @@ GEMM_FROM = 9
 
 # Every test of this module runs three times: with the K-quant matrices' prefill planes built on first
 # use and kept (gemm_plane_cache_mb > 0) and read by the kernel whose waves all multiply ("planes":
-# ogm_gemm_q*_dma_kernel) or by the feeding-wave kernels ("planes_fed": "_pre" in their name), and with
-# none (the default: the feeding waves unpack the weights on every call).  Same bits all three ways.
+# ogm_gemm_q*_dma_kernel, here whatever the grid, from 32 tokens) or by the feeding-wave kernels
+# ("planes_fed": "_pre" in their name), and with none (the feeding waves unpack the weights on every
+# call).  Same bits all three ways.
 @pytest.fixture(scope="module", params=["planes", "planes_fed", "unpack"])
 def be(request):
     from orangu_amd import Mi355xBackend
@@ -44,7 +45,7 @@ def be(request):
     b.set_tuning("gemm_small_max_tokens", 1)
     b.set_tuning("gemm_sb_waves", 8)
     b.set_tuning("gemm_plane_cache_mb", 0 if request.param == "unpack" else 65536)
-    b.set_tuning("gemm_plane_kernel", 1 if request.param == "planes_fed" else 0)
+    b.set_tuning("gemm_plane_kernel", 1 if request.param == "planes_fed" else 2)
     b.plane_mode = request.param
     yield b
     b.close()
@@ -59,6 +60,9 @@ class _TiledPlaneKernel(str):
     def __ne__(self, other):
         return not self.__eq__(other)
 
+    def startswith(self, prefix, *a):
+        return (str(self) + "_kernel").startswith(prefix, *a) or (str(self) + "_r64_kernel").startswith(prefix, *a)
+
     __hash__ = str.__hash__
 
 
@@ -67,15 +71,14 @@ def kname(b):
     a feeding-wave kernel that read prebuilt planes, and ogm_gemm_q*_dma_kernel as its family's tiled
     kernel (of either row tiling).  Checks that the name fits the mode the backend runs in."""
     name = b.last_kernel()
-    mode = getattr(b, "plane_mode", "unpack")
+    mode = getattr(b, "plane_mode", "planes")   # a context with no tuning reads planes on large grids
     m = re.match(r"ogm_gemm_q(6k|3k|4k|5k)_dma_kernel$", name)
     if m:
         assert mode == "planes", name
         return _TiledPlaneKernel({"6k": "ogm_gemm_q6k_i8", "3k": "ogm_gemm_q3k_i8", "4k": "ogm_gemm_q4k_i8p",
                                   "5k": "ogm_gemm_q5k_i8p"}[m.group(1)])
     if re.match(r"ogm_gemm_q(6k_i8|3k_i8|4k_i8p|5k_i8p)(_pre)?(_r64)?_kernel$", name):
-        # (below 32 tokens the planes are read by a feeding-wave kernel in either mode)
-        assert ("_pre" in name) == (mode != "unpack"), name
+        assert ("_pre" in name) == (mode == "planes_fed"), name
     return name.replace("_pre", "")
 
 
@@ -562,7 +565,9 @@ def test_gemm_threshold_default():
     """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
     float order, 17 through the matrix-core GEMM.  Q4_K: 8 tokens through the GEMV kernel, 9 and 128
     through the small-batch kernel (a matrix of few rows), 129 through the tiled one; a matrix of
-    many rows leaves the small-batch kernel after 64 tokens.  Same bits everywhere."""
+    many rows leaves the small-batch kernel after 64 tokens, and one of so many that 128 x 128 tiles
+    outnumber the compute units has its planes built and read by the kernel whose waves all multiply.
+    Same bits everywhere."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
     try:
@@ -596,6 +601,14 @@ def test_gemm_threshold_default():
             y = b.matmul(np.ascontiguousarray(x[:n, :256]), n, w)
             assert kname(b) == kernel, (n, kname(b))
             assert_bits(y, want[:n], f"Q6_K, {n} tokens")
+        raw = synth_weights(Q4_K, 256, 16600, seed=9)   # 130 tiles of 128 rows x 2 of 128 tokens
+        w = qm(raw, Q4_K, 256, 16600)
+        x5 = np.ascontiguousarray(x[:129, :256])
+        y = b.matmul(x5, 129, w)
+        assert b.last_kernel() == "ogm_gemm_q4k_dma_kernel"
+        assert_bits(y, oracle.matmul(Q4_K, raw, 256, 16600, x5, 129), "Q4_K, 129 tokens x 16600 rows")
+        y = b.matmul(x5[:128], 128, w)                   # one token tile: 130 workgroups
+        assert b.last_kernel() == "ogm_gemm_q4k_i8p_kernel"
     finally:
         b.close()
 
