@@ -39,7 +39,27 @@ def gemv_bytes(in_dim: int, out_dim: int, t: int = 1) -> int:
     return out_dim * (in_dim // 256 * 144) + 4 * in_dim * t + 4 * out_dim * t
 
 
-def sweep(be, helpers, hiprt) -> dict:
+def batched_us(hiprt, stream, launch, batches: int, per_batch: int, warm: int = 10) -> dict:
+    """Times `batches` runs of `per_batch` back-to-back launches with HIP events on the launch stream;
+    the figures are microseconds per launch: the fastest batch, the median batch and the mean."""
+    for i in range(warm):
+        launch(i)
+    stream.synchronize()
+    ev = [(hiprt.Event(), hiprt.Event()) for _ in range(batches)]
+    k = warm
+    for e0, e1 in ev:
+        e0.record(stream)
+        for _ in range(per_batch):
+            launch(k)
+            k += 1
+        e1.record(stream)
+    ev[-1][1].synchronize()
+    us = sorted(e0.elapsed_ms(e1) * 1e3 / per_batch for e0, e1 in ev)
+    return {"min": round(us[0], 3), "median": round(us[len(us) // 2], 3), "mean": round(sum(us) / len(us), 3),
+            "launches": batches * per_batch}
+
+
+def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
     """Kernel timings at the full size of every benchmark configuration: device-resident inputs,
     back-to-back calls over weight copies totalling more than the 256 MB last-level cache, HIP events
     on the launch stream.  Each figure covers the whole call (activation quantizer + matmul kernels)."""
@@ -47,29 +67,30 @@ def sweep(be, helpers, hiprt) -> dict:
     blk = {Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256)}
     names = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
     stream = hiprt.Stream()
-    out = {"device": be.device_name(), "unit": "us per call; GB/s and TFLOP/s are algorithmic", "rows": []}
+    out = {"device": be.device_name(),
+           "unit": "us per call (activation quantizer + matmul kernels), median and fastest of 8 batches of "
+                   "back-to-back calls, HIP events on the launch stream; GB/s and TFLOP/s are algorithmic, "
+                   "from the median", "rows": []}
 
-    def run(t, in_dim, out_dim, T, decode, label, n=60):
+    def run(t, in_dim, out_dim, T, decode, label, n=256):
+        if only and only not in label:
+            return
         w_bytes = out_dim * (in_dim // blk[t][1]) * blk[t][0]
         copies = max(2, min(24, (300 << 20) // w_bytes + 1))
         raw = helpers.synth_weights(t, in_dim, out_dim, 11)
         hs = [be.upload_raw(raw, t, in_dim, out_dim) for _ in range(copies)]
         x = hiprt.DeviceBuffer.from_numpy(helpers.synth_x(T, in_dim, 5))
         y = hiprt.DeviceBuffer(4 * T * out_dim)
-        for i in range(5):
-            be.matmul_dev(hs[i % copies], x.ptr, T, y.ptr, decode, stream.ptr)
-        stream.synchronize()
-        e0, e1 = hiprt.Event(), hiprt.Event()
-        e0.record(stream)
-        for i in range(n):
-            be.matmul_dev(hs[i % copies], x.ptr, T, y.ptr, decode, stream.ptr)
-        e1.record(stream)
-        e1.synchronize()
-        us = e0.elapsed_ms(e1) * 1e3 / n
+        if light:
+            n = max(32, n // 2)
+        st = batched_us(hiprt, stream, lambda i: be.matmul_dev(hs[i % copies], x.ptr, T, y.ptr, decode, stream.ptr),
+                        8, max(4, n // 8), warm=5)
+        us = st["median"]
         nbytes = w_bytes + 4 * T * (in_dim + out_dim)
         flops = 2.0 * T * in_dim * out_dim
         out["rows"].append({"config": label, "type": names[t], "in": in_dim, "out": out_dim, "tokens": T,
-                            "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                            "us": round(us, 2), "us_min": round(st["min"], 2), "launches": st["launches"],
+                            "GBps": round(nbytes / us / 1e3, 1),
                             "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                             "TFLOPs": round(flops / us / 1e6, 2), "kernel": be.last_kernel()})
         for h in hs:
@@ -81,11 +102,11 @@ def sweep(be, helpers, hiprt) -> dict:
     run(Q4_K, HIDDEN, FFN, 1, False, "C2 gate/up GEMV")
     run(Q4_K, FFN, HIDDEN, 1, False, "C2 down GEMV")
     for T in (1, 4, 8):
-        run(Q6_K, 4096, 128256, T, False, f"C3 vocab batch {T}", n=20)
+        run(Q6_K, 4096, 128256, T, False, f"C3 vocab batch {T}", n=64)
         run(Q4_K, 4096, 4096, T, False, f"C3 q/o batch {T}")
         run(Q4_K, 4096, 1024, T, False, f"C3 k/v batch {T}")
     for T in (128, 512, 2048):
-        run(Q4_K, HIDDEN, FFN, T, False, f"C4 prefill GEMM M={T}", n=20)
+        run(Q4_K, HIDDEN, FFN, T, False, f"C4 prefill GEMM M={T}", n=64)
     run(Q6_K, FFN, HIDDEN, 1, False, "C5 ffn_down GEMV")
     return out
 
@@ -220,6 +241,50 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     return res
 
 
+def trait_path(be, helpers, raw, shapes, x_h, h_h, copies: int, reps: int) -> dict:
+    """What Backend::matmul really costs (backend/mod.rs:313, 362): host slices in, host slices out,
+    through ogm_matmul / ogm_matmul_batch -- pinned staging, quantizer, GEMV, wait -- on weight copies
+    that rotate like the headline's.  Wall clock per call, issued from compiled code
+    (ogm_time_host_calls) as the reference's FFI would; and, for the record, from this interpreter,
+    where a call costs about 5 us more."""
+    from orangu_amd import MatmulOp, QuantMatrix
+    mats = {k: [QuantMatrix(raw[k].copy(), Q4_K, *shapes[k]) for _ in range(copies)] for k in shapes}
+    for k in mats:
+        for m in mats[k]:
+            be.upload(m)
+
+    def stat(variants, groups):
+        be.time_host_calls(variants, groups, 30)
+        ts = np.sort(be.time_host_calls(variants, groups, reps))
+        return {"min": round(float(ts[0]), 2), "median": round(float(ts[len(ts) // 2]), 2),
+                "p90": round(float(ts[len(ts) * 9 // 10]), 2), "calls": reps}
+
+    gate = [[MatmulOp(x_h, 1, mats["gate"][c])] for c in range(copies)]
+    down = [[MatmulOp(h_h, 1, mats["down"][c])] for c in range(copies)]
+    pair = [[MatmulOp(x_h, 1, mats["gate"][c]), MatmulOp(x_h, 1, mats["up"][c])] for c in range(copies)]
+    ffn = [[MatmulOp(x_h, 1, mats["gate"][c]), MatmulOp(x_h, 1, mats["up"][c]), MatmulOp(h_h, 1, mats["down"][c])]
+           for c in range(copies)]
+    rows = {
+        "matmul 4096->14336": stat(gate, [1]),
+        "matmul 14336->4096": stat(down, [1]),
+        "matmul_batch {gate, up}": stat(pair, [2]),
+        "FFN block: matmul_batch {gate, up} + matmul down": stat(ffn, [2, 1]),
+    }
+    ts = []
+    for i in range(reps + 20):
+        a = time.perf_counter()
+        be.matmul(x_h, 1, mats["gate"][i % copies])
+        ts.append((time.perf_counter() - a) * 1e6)
+    ts = sorted(ts[20:])
+    rows["matmul 4096->14336 called from Python"] = {"min": round(ts[0], 2), "median": round(ts[len(ts) // 2], 2),
+                                                     "calls": reps}
+    for k in mats:
+        for m in mats[k]:
+            be.evict(m)
+    return {"unit": "us per call, wall clock, host pointers in and out; calls issued by ogm_time_host_calls "
+                    "(compiled code) unless the row says otherwise", "rows": rows}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -249,8 +314,16 @@ def main() -> int:
     ap.add_argument("--sweep", action="store_true",
                     help="time every benchmark configuration's kernels instead (one JSON object, not the "
                          "headline line)")
+    ap.add_argument("--only-row", default="", metavar="TEXT",
+                    help="with --sweep: only the rows whose label contains TEXT (for rocprofv3), e.g. 'C3 vocab batch 1'")
+    ap.add_argument("--no-sweep", action="store_true", help="leave the sweep rows out of the headline line")
+    ap.add_argument("--no-trait", action="store_true", help="leave the host-pointer rows out of the headline line")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the dominant-kernel leg (for rocprofv3 --kernel-trace --stats)")
+    ap.add_argument("--only-stream", action="store_true",
+                    help="run only the read-only launch over gate+up's bytes (the measured peak; for rocprofv3)")
+    ap.add_argument("--only-single", default="", choices=["", "gate", "down"],
+                    help="run only the single-matrix GEMV launches of this shape (for rocprofv3)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -267,7 +340,7 @@ def main() -> int:
         key, _, value = kv.partition("=")
         be.set_tuning(key, int(value))
     if args.sweep:
-        print(json.dumps(sweep(be, helpers, hiprt)))
+        print(json.dumps(sweep(be, helpers, hiprt, only=args.only_row)))
         be.close()
         return 0
     if args.only_prefill:
@@ -286,6 +359,7 @@ def main() -> int:
     if args.fuse_quant != -1:
         be.set_tuning("gemv_fuse_quant", args.fuse_quant)
     stream = hiprt.Stream()
+    only_leg = args.only_roofline or args.only_gemm or args.only_stream or bool(args.only_single)
 
     # ---- synthetic inputs -------------------------------------------------------------------
     seed = 20240607
@@ -314,93 +388,132 @@ def main() -> int:
 
     step_bytes = 2 * gemv_bytes(HIDDEN, FFN) + gemv_bytes(FFN, HIDDEN)
     result = {}
+    step_stats = None
 
-    if not args.only_roofline and not args.only_gemm:
+    if not only_leg:
+        def timed_steps(k0: int, n: int) -> float:
+            stream.synchronize()
+            hiprt.device_synchronize()
+            t0 = time.perf_counter()
+            for i in range(n):
+                step(k0 + i)
+            stream.synchronize()
+            hiprt.device_synchronize()
+            return (time.perf_counter() - t0) * 1e3 / n
+
         for i in range(args.warmup):
             step(i)
-        stream.synchronize()
-        hiprt.device_synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            step(args.warmup + i)
-        stream.synchronize()
-        hiprt.device_synchronize()
-        t1 = time.perf_counter()
-        ms_per_step = (t1 - t0) * 1e3 / args.steps
+        # the headline: exactly --steps steps between two synchronizations
+        ms_per_step = timed_steps(args.warmup, args.steps)
         result["ms_per_step"] = ms_per_step
         result["value"] = step_bytes / (ms_per_step * 1e-3) / 1e9
+        # the same region again, until at least 200 (and at least four times --steps) further steps have
+        # run: how much one such region varies
+        reps = [ms_per_step]
+        extra = max(4, -(-200 // max(1, args.steps)))
+        for r in range(extra):
+            reps.append(timed_steps(args.warmup + (r + 1) * args.steps, args.steps))
+        reps_sorted = sorted(reps)
+        step_stats = {"regions": len(reps), "steps_each": args.steps,
+                      "ms_per_step_min": round(reps_sorted[0], 5),
+                      "ms_per_step_median": round(reps_sorted[len(reps) // 2], 5),
+                      "ms_per_step_max": round(reps_sorted[-1], 5),
+                      "GBps_median": round(step_bytes / (reps_sorted[len(reps) // 2] * 1e-3) / 1e9, 1)}
 
     # ---- dominant kernel: the Q4_K GEMV over gate+up (4096 -> 2 x 14336 in one launch), ---------
-    # back-to-back over pre-quantized activations, HIP events on its stream
-    def timed(launch, n):
-        for i in range(50):
-            launch(i)
-        stream.synchronize()
-        e0, e1 = hiprt.Event(), hiprt.Event()
-        e0.record(stream)
-        for i in range(n):
-            launch(i)
-        e1.record(stream)
-        e1.synchronize()
-        return e0.elapsed_ms(e1) * 1e3 / n
-
-    n_launch = args.roofline_launches if not args.only_gemm else 1
-    be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr)
-    us_per_launch = timed(lambda i: be.matmul_multi_act_dev(
-        [handles["gate"][i % copies], handles["up"][i % copies]], 1, [y_gate.ptr, y_up.ptr], False,
-        stream.ptr), n_launch)
-    kernel_name = be.last_kernel()
+    # back-to-back over pre-quantized activations, HIP events on its stream, in batches
+    n_launch = max(40, args.roofline_launches)
+    per_batch = 20
+    batches = max(2, n_launch // per_batch)
     kbytes = 2 * gemv_bytes(HIDDEN, FFN) - 4 * HIDDEN  # both matrices read the same x
-    achieved = kbytes / (us_per_launch * 1e-6) / 1e9
-    others = None
-    if not args.only_roofline and not args.only_gemm:
-        # the other launch shapes of the step, for the record (left out of the profiled run so
-        # that the trace's average for the GEMV kernel covers the gate+up launches only)
-        mats = handles["gate"] + handles["up"]
-        us_one = timed(lambda i: be.matmul_act_dev(mats[i % len(mats)], 1, y_gate.ptr, False, stream.ptr),
-                       n_launch)
-        be.act_quantize_dev(Q4_K, h_d.ptr, FFN, 1, stream.ptr)
-        us_down = timed(lambda i: be.matmul_act_dev(handles["down"][i % copies], 1, y_down.ptr, False,
-                                                    stream.ptr), n_launch)
-        us_quant = timed(lambda i: be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr), n_launch)
-        others = {"gemv 4096->14336 alone": round(us_one, 3), "gemv 14336->4096": round(us_down, 3),
-                  "activation quantize 4096": round(us_quant, 3)}
-    if args.only_roofline:
-        # One plain device-to-device copy of known size: under `rocprofv3 --pmc FETCH_SIZE` /
-        # `WRITE_SIZE` its counter reading calibrates the GEMV's (bytes per counter unit).
-        cal = 64 << 20
-        src, dst = hiprt.DeviceBuffer(cal), hiprt.DeviceBuffer(cal)
-        src.fill(1)
-        hiprt.check(hiprt.hip().hipMemcpy(dst.ptr, src.ptr, cal, 3), "hipMemcpy D2D")
-        hiprt.device_synchronize()
-    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_Q4K_GATE_UP_TRAFFIC,
-                "kernel": kernel_name + " over gate+up", "us_per_launch": round(us_per_launch, 3),
-                "bytes_per_launch": kbytes, "launches": n_launch,
-                "other_launches_us": others}
+    weight_bytes2 = 2 * FFN * (HIDDEN // 256 * 144)
+    roofline = None
+    kernel_name = ""
+    us_per_launch = 0.0
+    achieved = 0.0
+    if not args.only_gemm:
+        be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr)
+        legs = {}
+        if not args.only_stream and not args.only_single:
+            legs["gate+up"] = batched_us(hiprt, stream, lambda i: be.matmul_multi_act_dev(
+                [handles["gate"][i % copies], handles["up"][i % copies]], 1, [y_gate.ptr, y_up.ptr], False,
+                stream.ptr), batches, per_batch, warm=50)
+            kernel_name = be.last_kernel()
+        if not args.only_roofline and not args.only_single:
+            # the yardstick: the same bytes through a launch that only reads them
+            legs["read probe"] = batched_us(hiprt, stream, lambda i: be.weights_read_probe(
+                [handles["gate"][i % copies], handles["up"][i % copies]], stream.ptr), batches, per_batch, warm=50)
+        if not args.only_roofline and not args.only_stream:
+            mats = handles["gate"] + handles["up"]
+            if args.only_single in ("", "gate"):
+                legs["gate alone"] = batched_us(hiprt, stream, lambda i: be.matmul_act_dev(
+                    mats[i % len(mats)], 1, y_gate.ptr, False, stream.ptr), batches, per_batch, warm=50)
+            if args.only_single in ("", "down"):
+                be.act_quantize_dev(Q4_K, h_d.ptr, FFN, 1, stream.ptr)
+                legs["down"] = batched_us(hiprt, stream, lambda i: be.matmul_act_dev(
+                    handles["down"][i % copies], 1, y_down.ptr, False, stream.ptr), batches, per_batch, warm=50)
+            if not args.only_single:
+                legs["quantize 4096"] = batched_us(hiprt, stream, lambda i: be.act_quantize_dev(
+                    Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr), batches, per_batch, warm=50)
+        if args.only_roofline or args.only_stream:
+            # One plain device-to-device copy of known size: under `rocprofv3 --pmc FETCH_SIZE` /
+            # `WRITE_SIZE` its counter reading calibrates the kernel's (bytes per counter unit).
+            cal = 64 << 20
+            src, dst = hiprt.DeviceBuffer(cal), hiprt.DeviceBuffer(cal)
+            src.fill(1)
+            hiprt.check(hiprt.hip().hipMemcpy(dst.ptr, src.ptr, cal, 3), "hipMemcpy D2D")
+            hiprt.device_synchronize()
+        main_leg = legs.get("gate+up") or legs.get("read probe") or next(iter(legs.values()))
+        us_per_launch = main_leg["median"]
+        achieved = kbytes / (us_per_launch * 1e-6) / 1e9
+        one = gemv_bytes(HIDDEN, FFN)
+        per_leg_bytes = {"gate+up": kbytes, "read probe": weight_bytes2, "gate alone": one,
+                         "down": gemv_bytes(FFN, HIDDEN), "quantize 4096": 4 * HIDDEN + HIDDEN + 64}
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_Q4K_GATE_UP_TRAFFIC,
+                    "traffic_source": "rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on `bench.py --only-roofline`, "
+                                      "each scaled by the same counter's reading for that run's 64 MiB copy "
+                                      "(profiles/gemv_q4k_gate_up_4096x14336_hbm_counters.md)",
+                    "kernel": (kernel_name or "(not run)") + " over gate+up", "us_per_launch": us_per_launch,
+                    "us_per_launch_min": main_leg["min"], "bytes_per_launch": kbytes,
+                    "launches": main_leg["launches"],
+                    "timing": f"HIP events on the launch stream round {batches} batches of {per_batch} back-to-back "
+                              "launches; median batch (achieved, frac) and fastest batch",
+                    "legs_us": {k: {**v, "GBps_median": round(per_leg_bytes[k] / v["median"] / 1e3, 1)}
+                                for k, v in legs.items()}}
+        if "read probe" in legs and "gate+up" in legs:
+            peak_meas = weight_bytes2 / legs["read probe"]["median"] / 1e3
+            roofline["measured_peak"] = {
+                "GBps": round(peak_meas, 1), "us": legs["read probe"]["median"], "bytes": weight_bytes2,
+                "what": "one launch that only reads gate+up's device bytes with the GEMV's non-temporal loads "
+                        "(ogm_weights_read_probe), same rotation over weight copies",
+                "frac_of_measured": round(achieved / peak_meas, 4)}
 
-    # ---- prefill GEMM on MFMA: Q4_K 4096 -> 14336 at --gemm-tokens tokens (quantize + f16 staging
+    # ---- prefill GEMM on MFMA: Q4_K 4096 -> 14336 at --gemm-tokens tokens (quantize + operand staging
     # + GEMM kernel per call), checked against the CPU path on a sample of rows
     gemm = None
-    if args.gemm_tokens > 0 and not args.only_roofline:
+    if args.gemm_tokens > 0 and (not only_leg or args.only_gemm):
         T = args.gemm_tokens
         xg_h = helpers.synth_x(T, HIDDEN, seed + 7)
         xg = hiprt.DeviceBuffer.from_numpy(xg_h)
         yg = hiprt.DeviceBuffer(4 * T * FFN)
-        n_g = 20 if not args.only_gemm else 5
-        us_gemm = timed(lambda i: be.matmul_dev(handles["gate"][i % copies], xg.ptr, T, yg.ptr, False,
-                                                stream.ptr), n_g) if not args.only_gemm else None
+        st_g = None
         if args.only_gemm:
-            for i in range(n_g):
+            for i in range(5):
                 be.matmul_dev(handles["gate"][i % copies], xg.ptr, T, yg.ptr, False, stream.ptr)
             stream.synchronize()
+        else:
+            st_g = batched_us(hiprt, stream, lambda i: be.matmul_dev(handles["gate"][i % copies], xg.ptr, T, yg.ptr,
+                                                                     False, stream.ptr), 10, 4, warm=12)
         gemm_kernel = be.last_kernel()
         gemm = {"workload": f"Q4_K 4096->14336, {T} tokens (config a14 shape)", "kernel": gemm_kernel}
-        if us_gemm is not None:
+        if st_g is not None:
             flops = 2.0 * T * HIDDEN * FFN
+            us_gemm = st_g["median"]
             # the kernel multiplies int8 operands (v_mfma_i32_32x32x32_i8): priced against the dense
             # int8 peak of 5.0 POP/s (against the 2.5 PFLOP/s f16 peak it would read twice as high)
-            gemm.update({"us_per_matmul": round(us_gemm, 1), "tops": round(flops / us_gemm / 1e6, 1),
+            gemm.update({"us_per_matmul": round(us_gemm, 1), "us_per_matmul_min": round(st_g["min"], 1),
+                         "calls": st_g["launches"], "tops": round(flops / us_gemm / 1e6, 1),
                          "mfma_type": "i8", "frac_of_int8_mfma_peak": round(flops / us_gemm / 1e6 / 5000.0, 4)})
         if not args.only_gemm and args.cpu_seconds > 0:
             import oracle
@@ -411,11 +524,13 @@ def main() -> int:
             got = yg.to_numpy(np.float32, T * FFN).reshape(T, FFN)[:, rows]
             gemm["parity_vs_cpu"] = "bit-exact" if np.array_equal(got.view(np.uint32), want.view(np.uint32)) \
                 else ("within 1e-3/1e-5" if np.all(np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-5) else "FAILED")
+        xg.free()
+        yg.free()
 
     # ---- parity of what was just timed + CPU baseline (the oracle, all host cores) -------------
     cpu = None
     parity = None
-    if not args.only_roofline and not args.only_gemm and args.cpu_seconds > 0:
+    if not only_leg and args.cpu_seconds > 0:
         import oracle
         step(0)
         stream.synchronize()
@@ -454,11 +569,19 @@ def main() -> int:
         if parity == "FAILED":
             print("bench.py: GPU output differs from the CPU oracle beyond 1e-3/1e-5", file=sys.stderr)
 
+    trait = None
+    if not only_leg and not args.no_trait:
+        trait = trait_path(be, helpers, raw, shapes, x_h, h_h, min(copies, 6), 200)
+
+    for k in handles:          # make room: the legs below bring their own weights
+        for h in handles[k]:
+            be.free_weight(h)
+    sweep_rows = None
+    if not only_leg and not args.no_sweep:
+        sweep_rows = sweep(be, helpers, hiprt, light=True)
+
     decode = None
-    if args.decode_steps > 0 and not args.only_roofline and not args.only_gemm:
-        for k in handles:          # make room: the decode leg brings its own 4.8 GB of weights
-            for h in handles[k]:
-                be.free_weight(h)
+    if args.decode_steps > 0 and not only_leg:
         decode = decode_leg(be, helpers, hiprt, args.decode_steps, 8, args.decode_ctx, args.cpu_seconds > 0)
 
     out = {
@@ -466,7 +589,7 @@ def main() -> int:
         "value": round(result.get("value", achieved), 1),
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps if not args.only_roofline else n_launch,
+        "steps": args.steps if not only_leg else n_launch,
         "warmup": args.warmup,
         "ms_per_step": round(result.get("ms_per_step", us_per_launch * 1e-3), 5),
         "higher_is_better": True,
@@ -479,10 +602,13 @@ def main() -> int:
                                "quantize(h) + GEMV down",
                    "algorithmic_bytes_per_step": step_bytes, "weight_copies": copies,
                    "frac_of_hbm_peak": round(result.get("value", achieved) / HBM_PEAK_GBS, 4),
+                   "step_regions": step_stats,
                    "parity_vs_cpu": parity, "device": be.device_name()},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "prefill_gemm": gemm,
+        "trait_path": trait,
+        "sweep": sweep_rows,
         "decode": decode,
     }
     print(json.dumps(out))

@@ -367,8 +367,9 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
 
 /* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.
  * keys: "gemv_wg_waves" (waves per workgroup of the GEMV kernel, 1..16; 0 = heuristic);
- * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default: 9 for
- * Q4_K, Q5_K and Q6_K, 17 for the other types;
+ * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default: 6 for
+ * Q4_K, Q5_K and Q6_K -- Q6_K 4096 -> 128256 at 8 tokens: 122 us on the small-batch kernel against 178 us --
+ * and 17 for the other types;
  * below it the multi-token GEMV kernel runs in the GEMM's float order);
  * "gemm_q4k_variant" (K-quant GEMM: 0 = default, the int8 matrix-core kernels over scale-folded
  * weight planes; 1 = the same, always on 64-row tiles; 2 = the f16 kernels; 3 = for Q4_K and Q5_K the
@@ -390,6 +391,10 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * loads straight into LDS, when the launch has more than 256 tiles of 128 rows x 128 tokens, and otherwise
  * none: the feeding-wave kernels unpack; 1 = the feeding-wave kernels read them; 2 = the former whatever the
  * grid, from 32 tokens; same bits);
+ * "host_zero_copy" (1 = default: a host-pointer call -- ogm_matmul, ogm_matmul_decode, ogm_matmul_batch --
+ * whose x and y together are at most 512 KiB runs its kernels directly on the pinned staging buffers, with
+ * no copy-engine transfer: 23 us against 33 us per 4096 -> 14336 call; 0: always stage through device
+ * memory, as larger calls do);
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
  * the quantizer kernel first; 0 or -1 = default, off);
@@ -397,6 +402,16 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * GEMV launch before them, in its last workgroup to finish; 0 = default, kernels of their own, which
  * is faster; same bits).  No other setting changes a result bit. */
 int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value);
+/* For benchmarks driven from an interpreter: runs host-pointer calls from compiled code and writes each
+ * repetition's wall time in microseconds to us_out[reps].  `ops` holds n_variants sets of n_ops ops;
+ * repetition r walks set r % n_variants, in groups of group_sizes[] ops: a group of one is an ogm_matmul,
+ * a longer one an ogm_matmul_batch.  No counterpart in the reference. */
+int ogm_time_host_calls(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, size_t n_variants,
+                        const uint32_t *group_sizes, size_t n_groups, uint32_t reps, double *us_out);
+/* For benchmarks: one launch that only reads the device bytes of 1..4 uploaded weights (each of 9 KiB or
+ * more) with the GEMV's non-temporal 16-byte loads and stores nothing -- the rate the memory system gives
+ * that footprint with no arithmetic behind the loads.  No counterpart in the reference. */
+int ogm_weights_read_probe(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n_ws, void *stream);
 /* Name of the kernel the last matmul on this context launched (for profiles). */
 const char *ogm_last_kernel(ogm_ctx *ctx);
 

@@ -283,6 +283,33 @@ class Mi355xBackend:
         self._check(self._lib.ogm_matmul_multi_act_dev(self._ctx, ws, n, n_tokens, ys, int(decode),
                                                        stream or None), "ogm_matmul_multi_act_dev")
 
+    def time_host_calls(self, variants, group_sizes, reps: int) -> np.ndarray:
+        """Wall time in microseconds of `reps` repetitions of host-pointer calls issued from compiled
+        code: `variants` is a list of equally long lists of MatmulOp (repetition r takes variants[r %
+        len]), walked in groups of `group_sizes` ops -- one op: ogm_matmul, several: ogm_matmul_batch."""
+        n_ops = len(variants[0])
+        arr = (OgmOp * (n_ops * len(variants)))()
+        keep = []
+        for v, ops in enumerate(variants):
+            assert len(ops) == n_ops
+            for i, op in enumerate(ops):
+                x = self._x(op.x, op.n_tokens, op.w)
+                y = np.empty(op.n_tokens * op.w.out_dim, np.float32)
+                keep += [x, y]
+                a = arr[v * n_ops + i]
+                a.w, a.x, a.n_tokens, a.y = self.upload(op.w), x.ctypes.data, op.n_tokens, y.ctypes.data
+        gs = (C.c_uint32 * len(group_sizes))(*group_sizes)
+        out = (C.c_double * reps)()
+        self._check(self._lib.ogm_time_host_calls(self._ctx, arr, n_ops, len(variants), gs, len(group_sizes), reps, out),
+                    "ogm_time_host_calls")
+        return np.array(out[:], np.float64)
+
+    def weights_read_probe(self, w_handles, stream: int = 0):
+        """One launch that only reads the device bytes of 1..4 uploaded weights (for benchmarks)."""
+        n = len(w_handles)
+        ws = (C.c_void_p * n)(*w_handles)
+        self._check(self._lib.ogm_weights_read_probe(self._ctx, ws, n, stream or None), "ogm_weights_read_probe")
+
     def upload_raw(self, raw: np.ndarray, ggml_type: int, in_dim: int, out_dim: int) -> int:
         """Uploads without a cache key: every call makes a new device copy."""
         raw = np.ascontiguousarray(raw, np.uint8)

@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include <map>
+#include <chrono>
 #include <mutex>
 #include <new>
 #include <string>
@@ -48,7 +49,7 @@ struct ogm_ctx {
   std::vector<ogm_weight *> weights;
   // scratch, grown on demand and reused (the vendor backends allocate per call,
   // engine/backend/rocm.rs:352-376; a pool is what the Vulkan op_cache does instead)
-  DevBuf x, y, q, d, sums, bsum, bs16, isum, imin, xh;
+  DevBuf x, y, q, d, sums, bsum, bs16, isum, imin, xh, probe_sink;
   DevBuf hx, hy;  // pinned host staging
   int tune_wg_waves = 0;
   // matmul at n_tokens >= this takes the MFMA GEMM; 0 = by type: 9 for Q4_K, Q5_K and Q6_K, whose
@@ -60,6 +61,7 @@ struct ogm_ctx {
   int tune_gemm_q4k_variant = 0;
   int tune_gemm_small_max = 0;   // most tokens for the small-batch GEMM kernel: 0 = default, 1 = never
   int tune_gemm_sb_waves = 0;          // small-batch GEMM: 8 or 16 waves per workgroup, 0 = by the launch
+  int tune_host_zero_copy = 1;         // host-pointer calls of up to OGM_ZERO_COPY_MAX bytes: kernels read x / write y in pinned host memory
   int tune_gemm_plane_kernel = 0;      // who reads planes: 0 the all-waves-multiply kernel on large grids, 1 the feeding-wave kernels, 2 the former always
   int tune_decode_fuse_tails = 0;      // 1: the decode step's norms and SwiGLU inside the GEMV before them (slower)
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
@@ -215,7 +217,7 @@ extern "C" void ogm_destroy(ogm_ctx *ctx) {
     delete w;
   }
   DevBuf *dev[] = {&ctx->x,    &ctx->y,    &ctx->q,    &ctx->d,  &ctx->sums,
-                   &ctx->bsum, &ctx->bs16, &ctx->isum, &ctx->imin, &ctx->xh};
+                   &ctx->bsum, &ctx->bs16, &ctx->isum, &ctx->imin, &ctx->xh, &ctx->probe_sink};
   for (DevBuf *b : dev)
     if (b->p) (void)hipFree(b->p);
   if (ctx->hx.p) (void)hipHostFree(ctx->hx.p);
@@ -262,6 +264,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemm_small_max_tokens") == 0) {
     if (value < 0 || value > 1024) return fail(ctx, OGM_ERR_INVALID, "gemm_small_max_tokens must be 0..1024");
     ctx->tune_gemm_small_max = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "host_zero_copy") == 0) {
+    if (value != 0 && value != 1) return fail(ctx, OGM_ERR_INVALID, "host_zero_copy must be 0 or 1");
+    ctx->tune_host_zero_copy = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_plane_kernel") == 0) {
@@ -521,7 +528,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
   const uint32_t t0 = w0->ggml_type;
   const uint32_t gemm_from = ctx->tune_gemm_min_tokens ? (uint32_t)ctx->tune_gemm_min_tokens
-                             : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 9u : 17u;
+                             : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 6u : 17u;
   if (gemm_order && !dump_isum && !dump_imin && !act_base && n_tokens >= gemm_from &&
       all_gemm_supported(tg, n_tg, n_tokens)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
@@ -606,6 +613,13 @@ static int check_matmul_args(ogm_ctx *ctx, const ogm_weight *w, const void *x, c
   return OGM_OK;
 }
 
+// Host-pointer calls whose x and y together stay under this size skip the copy engine: the pinned
+// staging buffers are device-visible, and the quantizer and the matmul kernels use them in place.
+#define OGM_ZERO_COPY_MAX (512u << 10)
+static bool zero_copy(const ogm_ctx *ctx, size_t bytes) {
+  return ctx->tune_host_zero_copy != 0 && bytes <= OGM_ZERO_COPY_MAX;
+}
+
 static int host_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint32_t n_tokens,
                        float *y, int decode) {
   int rc = check_matmul_args(ctx, w, x, y, n_tokens);
@@ -614,17 +628,25 @@ static int host_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x, uint32
   std::lock_guard<std::mutex> lock(ctx->mu);
   HIPCHK(ctx, hipSetDevice(ctx->device));
   const size_t xb = (size_t)n_tokens * w->in_dim * 4, yb = (size_t)n_tokens * w->out_dim * 4;
-  if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
-  if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
   if ((rc = ensure_host(ctx, ctx->hx, xb)) != OGM_OK) return rc;
   if ((rc = ensure_host(ctx, ctx->hy, yb)) != OGM_OK) return rc;
   memcpy(ctx->hx.p, x, xb);
-  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, ctx->hx.p, xb, hipMemcpyHostToDevice, ctx->stream));
-  rc = enqueue_matmul(ctx, w, (const float *)ctx->x.p, n_tokens, (float *)ctx->y.p, decode,
-                      ctx->stream, nullptr, nullptr);
-  if (rc != OGM_OK) return rc;
-  HIPCHK(ctx, hipMemcpyAsync(ctx->hy.p, ctx->y.p, yb, hipMemcpyDeviceToHost, ctx->stream));
-  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  if (zero_copy(ctx, xb + yb)) {
+    // a decode-sized call: the kernels read x from, and write y to, the pinned staging buffers over
+    // the bus themselves; two copy-engine transfers and their latencies fall away
+    rc = enqueue_matmul(ctx, w, (const float *)ctx->hx.p, n_tokens, (float *)ctx->hy.p, decode, ctx->stream,
+                        nullptr, nullptr);
+    if (rc != OGM_OK) return rc;
+  } else {
+    if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
+    if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
+    HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, ctx->hx.p, xb, hipMemcpyHostToDevice, ctx->stream));
+    rc = enqueue_matmul(ctx, w, (const float *)ctx->x.p, n_tokens, (float *)ctx->y.p, decode,
+                        ctx->stream, nullptr, nullptr);
+    if (rc != OGM_OK) return rc;
+    HIPCHK(ctx, hipMemcpyAsync(ctx->hy.p, ctx->y.p, yb, hipMemcpyDeviceToHost, ctx->stream));
+  }
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));   // (polling hipStreamQuery instead measured slower)
   memcpy(y, ctx->hy.p, yb);
   return OGM_OK;
 }
@@ -672,6 +694,56 @@ extern "C" int ogm_matmul_dev_static(ogm_ctx *ctx, const ogm_weight *w, const fl
   HIPCHK(ctx, ogm_launch_quantize(mode, x_dev, w->in_dim, n_tokens, act, s));
   const Target t{w, y_dev};
   return enqueue_gemv(ctx, &t, 1, n_tokens, decode, s, nullptr, nullptr, nullptr, nullptr, &act);
+}
+
+// For benchmarks driven from an interpreter: runs host-pointer calls `reps` times from compiled code and
+// records each repetition's wall time.  A repetition walks one variant's ops (variant = rep % n_variants,
+// so that weights rotate), split into groups: a group of one op is an ogm_matmul, a longer one an
+// ogm_matmul_batch.
+extern "C" int ogm_time_host_calls(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, size_t n_variants,
+                                   const uint32_t *group_sizes, size_t n_groups, uint32_t reps, double *us_out) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!ops || !group_sizes || !us_out || n_ops == 0 || n_variants == 0 || n_groups == 0)
+    return fail(ctx, OGM_ERR_INVALID, "ogm_time_host_calls: null or empty argument");
+  size_t sum = 0;
+  for (size_t g = 0; g < n_groups; g++) sum += group_sizes[g];
+  if (sum != n_ops) return fail(ctx, OGM_ERR_INVALID, "ogm_time_host_calls: group sizes do not add up to n_ops");
+  for (uint32_t r = 0; r < reps; r++) {
+    const ogm_op *v = ops + (r % n_variants) * n_ops;
+    const auto t0 = std::chrono::steady_clock::now();
+    size_t at = 0;
+    for (size_t g = 0; g < n_groups; g++) {
+      const int rc = group_sizes[g] == 1 ? ogm_matmul(ctx, v[at].w, v[at].x, v[at].n_tokens, v[at].y)
+                                         : ogm_matmul_batch(ctx, v + at, group_sizes[g], 0, 0);
+      if (rc != OGM_OK) return rc;
+      at += group_sizes[g];
+    }
+    us_out[r] = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+  }
+  return OGM_OK;
+}
+
+// The device bytes of up to four weights streamed through one read-only launch (for benchmarks: the
+// rate the memory system gives this footprint with nothing behind the loads).
+extern "C" int ogm_weights_read_probe(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n_ws, void *stream) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (n_ws == 0) return OGM_OK;
+  if (!ws || n_ws > OGM_PROBE_MAX_BUFS) return fail(ctx, OGM_ERR_INVALID, "ogm_weights_read_probe takes 1..4 weights");
+  const uint8_t *bufs[OGM_PROBE_MAX_BUFS];
+  size_t bytes[OGM_PROBE_MAX_BUFS];
+  for (size_t i = 0; i < n_ws; i++) {
+    if (!ws[i] || ws[i]->device_bytes < 9216) return fail(ctx, OGM_ERR_INVALID, "a weight is null or under 9 KiB");
+    bufs[i] = ws[i]->dev;
+    bytes[i] = ws[i]->device_bytes;
+  }
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
+  int rc = ensure_dev(ctx, ctx->probe_sink, 256);
+  if (rc != OGM_OK) return rc;
+  HIPCHK(ctx, ogm_launch_read_probe(bufs, bytes, (uint32_t)n_ws, (uint32_t *)ctx->probe_sink.p, s));
+  ctx->last_kernel = "ogm_read_probe_kernel";
+  return OGM_OK;
 }
 
 extern "C" int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev,
@@ -791,10 +863,14 @@ extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, i
   }
   if (xb == 0) return OGM_OK;
   int rc;
-  if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
-  if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
+  const bool zc = zero_copy(ctx, xb + yb);   // see host_matmul
+  if (!zc) {
+    if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
+    if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
+  }
   if ((rc = ensure_host(ctx, ctx->hx, xb)) != OGM_OK) return rc;
   if ((rc = ensure_host(ctx, ctx->hy, yb)) != OGM_OK) return rc;
+  uint8_t *const x_base = (uint8_t *)(zc ? ctx->hx.p : ctx->x.p), *const y_base = (uint8_t *)(zc ? ctx->hy.p : ctx->y.p);
   // Size the activation scratch for the largest stripe before anything is enqueued, so it is
   // never reallocated under kernels in flight.
   for (size_t i = 0; i < n_ops; i++) {
@@ -806,7 +882,7 @@ extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, i
     const size_t bytes = (size_t)op.n_tokens * op.w->in_dim * 4;
     if (bytes && src[i] == i) memcpy((uint8_t *)ctx->hx.p + xoff[i], op.x, bytes);
   }
-  HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, ctx->hx.p, xb, hipMemcpyHostToDevice, ctx->stream));
+  if (!zc) HIPCHK(ctx, hipMemcpyAsync(ctx->x.p, ctx->hx.p, xb, hipMemcpyHostToDevice, ctx->stream));
   std::vector<Target> tg;
   for (size_t i = 0; i < n_ops;) {
     // a run of neighbouring ops over one input and one weight type: one group
@@ -815,19 +891,19 @@ extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, i
            ops[e].w->ggml_type == ops[i].w->ggml_type && ops[e].w->in_dim == ops[i].w->in_dim)
       e++;
     const ogm_op &op = ops[i];
-    const float *xd = (const float *)((uint8_t *)ctx->x.p + xoff[i]);
+    const float *xd = (const float *)(x_base + xoff[i]);
     for (uint32_t t0 = 0; t0 < op.n_tokens; t0 += cap) {
       const uint32_t nt = op.n_tokens - t0 < cap ? op.n_tokens - t0 : cap;
       tg.clear();
       for (size_t k = i; k < e; k++)
-        tg.push_back(Target{ops[k].w, (float *)((uint8_t *)ctx->y.p + yoff[k]) + (size_t)t0 * ops[k].w->out_dim});
+        tg.push_back(Target{ops[k].w, (float *)(y_base + yoff[k]) + (size_t)t0 * ops[k].w->out_dim});
       rc = enqueue_matmul(ctx, tg.data(), tg.size(), xd + (size_t)t0 * op.w->in_dim, nt, decode,
                           ctx->stream, nullptr, nullptr);
       if (rc != OGM_OK) return rc;
     }
     i = e;
   }
-  HIPCHK(ctx, hipMemcpyAsync(ctx->hy.p, ctx->y.p, yb, hipMemcpyDeviceToHost, ctx->stream));
+  if (!zc) HIPCHK(ctx, hipMemcpyAsync(ctx->hy.p, ctx->y.p, yb, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   size_t yo = 0;
   for (size_t i = 0; i < n_ops; i++) {

@@ -117,6 +117,12 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
 
 hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hipStream_t stream);
 
+// One launch that only reads the given buffers (each at least 9 KiB, 16-byte aligned) with the GEMV's
+// non-temporal loads; `sink` is one device word that is never written.
+#define OGM_PROBE_MAX_BUFS 4u
+hipError_t ogm_launch_read_probe(const uint8_t *const *bufs, const size_t *bytes, uint32_t n, uint32_t *sink,
+                                 hipStream_t stream);
+
 // The library's static scratch (ogm_static.hip): a file-scope device array every GPU holds its own
 // copy of, for the entry point that must not allocate.  It takes the quantized activations of up to
 // OGM_STATIC_MAX_TOKENS tokens totalling OGM_STATIC_MAX_ELEMS elements (400 KiB in all).

@@ -1181,6 +1181,55 @@ __global__ void ogm_f16_kernel(const uint16_t *bits, size_t n, float *out) {
   if (i < n) out[i] = f16_bits_to_f32(bits[i]);
 }
 
+// A launch that only reads: every wave pulls 9 KiB (nine non-temporal 16-byte loads a lane, the
+// shape of a Q4_K tile) and folds them into a word nobody stores.  What the memory system delivers
+// for a given footprint with no arithmetic, LDS or ordered sum behind the loads: the yardstick the
+// benchmark prices the GEMV against.
+struct ReadProbeParams {
+  const uint8_t *buf[OGM_PROBE_MAX_BUFS];
+  uint64_t chunks[OGM_PROBE_MAX_BUFS];   // 9 KiB chunks of each buffer (the last may overlap the one before)
+  uint64_t bytes[OGM_PROBE_MAX_BUFS];
+  uint32_t n;
+  uint32_t *sink;
+};
+__global__ __launch_bounds__(512) void ogm_read_probe_kernel(ReadProbeParams p) {
+  const uint32_t lane = threadIdx.x & 63u;
+  uint64_t c = (uint64_t)blockIdx.x * 8u + (threadIdx.x >> 6);
+  uint32_t b = 0;
+  while (b < p.n && c >= p.chunks[b]) c -= p.chunks[b++];
+  if (b == p.n) return;
+  // the last chunk of a buffer that is not a multiple of 9 KiB long starts early enough to end with it
+  const uint64_t off = min(c * 9216u, p.bytes[b] - 9216u);
+  const uint8_t *src = p.buf[b] + off + lane * 16u;
+  uint4 r[9];
+#pragma unroll
+  for (int i = 0; i < 9; i++) r[i] = ldw16(src + i * 1024);
+  uint32_t acc = 0;
+#pragma unroll
+  for (int i = 0; i < 9; i++) acc ^= r[i].x ^ r[i].y ^ r[i].z ^ r[i].w;
+  if (acc == 0x9E3779B9u) p.sink[blockIdx.x & 63u] = acc;   // practically never: keeps the loads alive
+}
+
+hipError_t ogm_launch_read_probe(const uint8_t *const *bufs, const size_t *bytes, uint32_t n, uint32_t *sink,
+                                 hipStream_t stream) {
+  if (n == 0 || n > OGM_PROBE_MAX_BUFS) return hipErrorInvalidValue;
+  ReadProbeParams p = {};
+  uint64_t total = 0;
+  for (uint32_t i = 0; i < n; i++) {
+    if (bytes[i] < 9216u || ((uintptr_t)bufs[i] & 15u)) return hipErrorInvalidValue;
+    p.buf[i] = bufs[i];
+    p.bytes[i] = bytes[i];
+    p.chunks[i] = (bytes[i] + 9215u) / 9216u;
+    total += p.chunks[i];
+  }
+  p.n = n;
+  p.sink = sink;
+  const uint64_t wgs = (total + 7u) / 8u;
+  if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ogm_read_probe_kernel, dim3((unsigned)wgs), dim3(512), 0, stream, p);
+  return hipGetLastError();
+}
+
 hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hipStream_t stream) {
   if (n == 0) return hipSuccess;
   hipLaunchKernelGGL(ogm_f16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, bits,

@@ -563,7 +563,7 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
 
 def test_gemm_threshold_default():
     """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
-    float order, 17 through the matrix-core GEMM.  Q4_K: 8 tokens through the GEMV kernel, 9 and 128
+    float order, 17 through the matrix-core GEMM.  Q4_K: 5 tokens through the GEMV kernel, 6 and 128
     through the small-batch kernel (a matrix of few rows), 129 through the tiled one; a matrix of
     many rows leaves the small-batch kernel after 64 tokens, and one of so many that 128 x 128 tiles
     outnumber the compute units has its planes built and read by the kernel whose waves all multiply.
@@ -584,7 +584,7 @@ def test_gemm_threshold_default():
         raw = synth_weights(Q4_K, 1024, 70, seed=5)
         w = qm(raw, Q4_K, 1024, 70)
         want = oracle.matmul(Q4_K, raw, 1024, 70, x, 129).reshape(129, 70)
-        for n, kernel in ((8, "ogm_gemv_kernel"), (9, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
+        for n, kernel in ((5, "ogm_gemv_kernel"), (6, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
                           (129, "ogm_gemm_q4k_i8p_r64_kernel")):
             y = b.matmul(x[:n], n, w)
             assert kname(b).startswith(kernel), (n, kname(b))
@@ -1140,6 +1140,33 @@ def test_concurrent_callers_share_one_backend(be):
     for th in threads:
         th.join()
     assert not errors, errors
+
+
+def test_host_calls_on_pinned_buffers_and_through_device_copies_agree(be):
+    """A host-pointer call of up to 512 KiB runs its kernels on the pinned staging buffers in place
+    (host_zero_copy 1, the default); larger calls, and all of them with host_zero_copy 0, go through
+    device copies.  Same bits either way, for one GEMV, a small GEMM, a batch over a shared input and a
+    call just past the limit."""
+    from orangu_amd import MatmulOp
+    in_dim = 1024
+    wa, wb = synth_weights(Q4_K, in_dim, 300, seed=41), synth_weights(Q6_K, in_dim, 130, seed=42)
+    ma, mb = qm(wa, Q4_K, in_dim, 300), qm(wb, Q6_K, in_dim, 130)
+    x1, x7, x100 = synth_x(1, in_dim, 43), synth_x(7, in_dim, 44), synth_x(100, in_dim, 45)   # 100 tokens: 529 KiB
+    res = {}
+    for zc in (1, 0):
+        be.set_tuning("host_zero_copy", zc)
+        try:
+            ops = [MatmulOp(x7.reshape(-1), 7, ma), MatmulOp(x7.reshape(-1), 7, mb), MatmulOp(x1.reshape(-1), 1, mb)]
+            res[zc] = [be.matmul(x1.reshape(-1), 1, ma), be.matmul_decode(x7.reshape(-1), 7, mb),
+                       be.matmul(x7.reshape(-1), 7, ma), be.matmul(x100.reshape(-1), 100, ma),
+                       *be.matmul_batch(ops), *be.matmul_batch_decode(ops)]
+        finally:
+            be.set_tuning("host_zero_copy", 1)
+    for a, b in zip(res[1], res[0]):
+        assert_bits(a, b, "pinned in place vs device copies")
+    assert_bits(res[1][0], oracle.matmul(Q4_K, wa, in_dim, 300, x1, 1), "GEMV on pinned buffers")
+    assert_bits(res[1][2], oracle.matmul(Q4_K, wa, in_dim, 300, x7, 7), "small GEMM on pinned buffers")
+    assert_bits(res[1][5], oracle.matmul(Q6_K, wb, in_dim, 130, x7, 7), "batch on pinned buffers")
 
 
 @pytest.mark.parametrize("sign", ["pos", "alt"])
