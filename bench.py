@@ -31,7 +31,7 @@ HIDDEN, FFN = 4096, 14336
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of `bench.py --only-roofline`, calibrated on that run's 64 MiB copy (profiles/).
-GEMV_Q4K_GATE_UP_TRAFFIC = 66243599
+GEMV_Q4K_GATE_UP_TRAFFIC = 66248100
 
 
 def gemv_bytes(in_dim: int, out_dim: int, t: int = 1) -> int:
@@ -111,7 +111,8 @@ def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
     return out
 
 
-def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool, only_prefill: int = 0) -> dict:
+def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool, only_prefill: int = 0,
+               with_prefill: bool = True) -> dict:
     """Batch-1 decode of an 8B-shaped Llama (32 layers: wq, wo 4096x4096, wk, wv 4096->1024, gate, up
     4096->14336 in Q4_K; down 14336->4096 and the 128256-row output in Q6_K; f16 KV cache holding `ctx`
     random positions): tokens per second of ogm_llama_decode_dev with the embedding row, the logits and
@@ -189,25 +190,29 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     pos += steps
     # prefill of a 512-token prompt from position 0 (GEMM matmuls, batch attention); the first
     # call allocates the batch buffers
-    prompt = rng.integers(0, n_vocab, 512).astype(np.uint32)
-    dec.prefill_tokens(up("output"), prompt, 0)
-    t0 = time.perf_counter()
-    for _ in range(3):
+    dt_pre = dt_pre_long = None
+    if with_prefill:
+        prompt = rng.integers(0, n_vocab, 512).astype(np.uint32)
         dec.prefill_tokens(up("output"), prompt, 0)
-    dt_pre = (time.perf_counter() - t0) / 3
-    long_prompt = rng.integers(0, n_vocab, 2048).astype(np.uint32)
-    dec.prefill_tokens(up("output"), long_prompt, 0)
-    t0 = time.perf_counter()
-    dec.prefill_tokens(up("output"), long_prompt, 0)
-    dt_pre_long = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        for _ in range(3):
+            dec.prefill_tokens(up("output"), prompt, 0)
+        dt_pre = (time.perf_counter() - t0) / 3
+        long_prompt = rng.integers(0, n_vocab, 2048).astype(np.uint32)
+        dec.prefill_tokens(up("output"), long_prompt, 0)
+        t0 = time.perf_counter()
+        dec.prefill_tokens(up("output"), long_prompt, 0)
+        dt_pre_long = time.perf_counter() - t0
     weights = n_layer * sum(o * (i // 256) * (144 if t == Q4_K else 210) for t, i, o in shapes.values()) \
         + n_vocab * (n_embd // 256) * 210
     kv_bytes = 2 * n_layer * ctx * n_kv * hd * 2
     res = {"workload": f"configs[4]: 8B-shaped Llama Q4_K_M-like, batch-1 greedy decode at context {ctx}",
            "tok_per_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4),
            "generate_tok_per_s": round(1.0 / dt_gen, 1), "generated": [int(t) for t in toks[:4]],
-           "prefill_512_ms": round(dt_pre * 1e3, 2), "prefill_tok_per_s": round(512 / dt_pre, 1),
-           "prefill_2048_ms": round(dt_pre_long * 1e3, 2), "prefill_2048_tok_per_s": round(2048 / dt_pre_long, 1),
+           "prefill_512_ms": round(dt_pre * 1e3, 2) if dt_pre else None,
+           "prefill_tok_per_s": round(512 / dt_pre, 1) if dt_pre else None,
+           "prefill_2048_ms": round(dt_pre_long * 1e3, 2) if dt_pre_long else None,
+           "prefill_2048_tok_per_s": round(2048 / dt_pre_long, 1) if dt_pre_long else None,
            "bytes_per_token": weights + kv_bytes,
            "GBps": round((weights + kv_bytes) / dt / 1e9, 1),
            "frac_of_hbm_peak": round((weights + kv_bytes) / dt / 1e9 / HBM_PEAK_GBS, 4)}
@@ -349,7 +354,8 @@ def main() -> int:
         be.close()
         return 0
     if args.only_decode:
-        print(json.dumps(decode_leg(be, helpers, hiprt, max(1, args.decode_steps), 8, args.decode_ctx, False)))
+        print(json.dumps(decode_leg(be, helpers, hiprt, max(1, args.decode_steps), 8, args.decode_ctx, False,
+                                    with_prefill=False)))
         be.close()
         return 0
     if args.wg_waves:
