@@ -16,9 +16,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liborangu_oracle.so")
 
-Q4_0, Q5_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL = 2, 6, 8, 11, 12, 13, 14, 20
-BLOCK_LAYOUT = {Q4_0: (18, 32), Q5_0: (22, 32), Q8_0: (34, 32), Q3_K: (110, 256), Q4_K: (144, 256), Q5_K: (176, 256),
-                Q6_K: (210, 256), IQ4_NL: (18, 32)}
+Q4_0, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 2, 6, 7, 8, 10, 11, 12, 13, 14, 20, 23
+BLOCK_LAYOUT = {Q4_0: (18, 32), Q5_0: (22, 32), Q5_1: (24, 32), Q8_0: (34, 32), Q2_K: (84, 256), Q3_K: (110, 256),
+                Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256)}
 
 
 def build() -> str:
@@ -72,6 +72,14 @@ def lib() -> C.CDLL:
         L.ogo_dot_k_row_q6_k.argtypes = [u8p, sz, i8p, f32p, i32p]
         L.ogo_dot_k_row_q3_k.restype = C.c_float
         L.ogo_dot_k_row_q3_k.argtypes = [u8p, sz, i8p, f32p, i32p]
+        L.ogo_dot_q5_1.restype = C.c_float
+        L.ogo_dot_q5_1.argtypes = [u8p, sz, i8p, f32p, i32p, i32p]
+        L.ogo_dot_k_row_iq4_xs.restype = C.c_float
+        L.ogo_dot_k_row_iq4_xs.argtypes = [u8p, sz, i8p, f32p, i32p]
+        L.ogo_dot_k_row_q2_k.restype = C.c_float
+        L.ogo_dot_k_row_q2_k.argtypes = [u8p, sz, i8p, f32p, i32p, i32p, i32p]
+        L.ogo_dot_unpacked_q2_k.restype = C.c_float
+        L.ogo_dot_unpacked_q2_k.argtypes = [u8p, sz, i8p, f32p, i32p]
         L.ogo_unpack_q3_k_scales.argtypes = [u8p, i32p]
         L.ogo_dot_flat32.restype = C.c_float
         L.ogo_dot_flat32.argtypes = [C.c_uint32, u8p, sz, i8p, f32p, i32p]
@@ -225,7 +233,17 @@ def dot_row(ggml_type: int, row, act) -> np.float32:
         return np.float32(L.ogo_dot_q4_k(_p(r), n, _p(q), _p(d), _p(s)))
     if ggml_type == Q6_K:
         return np.float32(L.ogo_dot_q6_k(_p(r), n, _p(q), _p(d)))
+    if ggml_type == Q5_1:
+        return np.float32(L.ogo_dot_q5_1(_p(r), n, _p(q), _p(d), _p(s), None))
     raise ValueError(ggml_type)
+
+
+def dot_unpacked_q2_k(row, act) -> np.float32:
+    """unpack_q2_k + dot_unpacked (vecdot.rs:1144-1164, 407-428) over a per-32 ActQ8 ``(q, d, sums)``: what
+    matmul computes per token for Q2_K at n_tokens > 1."""
+    r = _u8(row)
+    q, d, s = act
+    return np.float32(lib().ogo_dot_unpacked_q2_k(_p(r), q.size, _p(q), _p(d), _p(s)))
 
 
 def unpack_flat_block(ggml_type: int, block):
@@ -260,6 +278,10 @@ def dot_k_row(ggml_type: int, row, act, want_sums: bool = False):
         v = L.ogo_dot_k_row_q6_k(_p(r), n, _p(q), _p(d), _p(isum))
     elif ggml_type == Q3_K:
         v = L.ogo_dot_k_row_q3_k(_p(r), n, _p(q), _p(d), _p(isum))
+    elif ggml_type == IQ4_XS:
+        v = L.ogo_dot_k_row_iq4_xs(_p(r), n, _p(q), _p(d), _p(isum))
+    elif ggml_type == Q2_K:
+        v = L.ogo_dot_k_row_q2_k(_p(r), n, _p(q), _p(d), _p(s), _p(isum), _p(imin))
     else:
         raise ValueError(ggml_type)
     return (np.float32(v), isum, imin) if want_sums else np.float32(v)

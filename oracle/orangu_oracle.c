@@ -67,7 +67,10 @@ int ogo_block_layout(uint32_t ggml_type, size_t *block_bytes, size_t *block_elem
     case OGO_TYPE_F16: bb = 2; be = 1; break;
     case OGO_TYPE_Q4_0: bb = 2 + 16; be = 32; break;
     case OGO_TYPE_Q5_0: bb = 2 + 4 + 16; be = 32; break;
+    case OGO_TYPE_Q5_1: bb = 2 + 2 + 4 + 16; be = 32; break;
     case OGO_TYPE_Q8_0: bb = 2 + 32; be = 32; break;
+    case OGO_TYPE_Q2_K: bb = 16 + 64 + 2 + 2; be = 256; break;
+    case OGO_TYPE_IQ4_XS: bb = 2 + 2 + 4 + 128; be = 256; break;
     case OGO_TYPE_IQ4_NL: bb = 2 + 16; be = 32; break;
     case OGO_TYPE_Q3_K: bb = 32 + 64 + 12 + 2; be = 256; break;
     case OGO_TYPE_Q4_K: bb = 2 + 2 + 12 + 128; be = 256; break;
@@ -197,6 +200,82 @@ static void dequantize_flat32(uint32_t ggml_type, const uint8_t *bytes, size_t n
   }
 }
 
+/* unpack_block_q5_1 (vecdot.rs:1032-1034, :1001-1017 with bias 0): block = d | m | qh | qs[16] */
+static inline void unpack_block_q5_1(const uint8_t *block, int8_t *w) {
+  uint32_t qh = (uint32_t)block[4] | ((uint32_t)block[5] << 8) | ((uint32_t)block[6] << 16) | ((uint32_t)block[7] << 24);
+  const uint8_t *qs = block + 8;
+  for (int j = 0; j < 16; j++) {
+    uint32_t hi_lo = ((qh >> j) << 4) & 0x10;
+    uint32_t hi_hi = (qh >> (j + 12)) & 0x10;
+    w[j] = (int8_t)((uint32_t)(qs[j] & 0x0F) | hi_lo);
+    w[16 + j] = (int8_t)((uint32_t)(qs[j] >> 4) | hi_hi);
+  }
+}
+
+/* quant.rs:615-636 */
+static void dequantize_q5_1(const uint8_t *bytes, size_t n, float *out) {
+  int8_t w[32];
+  for (size_t b = 0; b < n / 32; b++) {
+    const uint8_t *block = bytes + b * 24;
+    float d = read_f16(block, 0), m = read_f16(block, 2);
+    unpack_block_q5_1(block, w);
+    for (int j = 0; j < 32; j++) out[b * 32 + (size_t)j] = (float)w[j] * d + m;
+  }
+}
+
+/* unpack_block_iq4_nl (vecdot.rs:937-942) */
+static inline void unpack_block_iq4_nl(const uint8_t *qs, int8_t *w) {
+  for (int j = 0; j < 16; j++) {
+    w[j] = KVALUES_IQ4NL[qs[j] & 0x0F];
+    w[j + 16] = KVALUES_IQ4NL[qs[j] >> 4];
+  }
+}
+
+/* The six-bit scale of sub-block ib, biased by 32 (vecdot.rs:3257-3259): block = d | scales_h:u16 | scales_l[4] | qs[128] */
+static inline int32_t iq4_xs_scale(const uint8_t *block, int ib) {
+  uint32_t scales_h = (uint32_t)block[2] | ((uint32_t)block[3] << 8);
+  uint32_t low = (block[4 + ib / 2] >> (4 * (ib % 2))) & 0x0F;
+  uint32_t high = (scales_h >> (2 * ib)) & 3;
+  return (int32_t)(low | (high << 4)) - 32;
+}
+
+/* quant.rs:1350-1375 */
+static void dequantize_iq4_xs(const uint8_t *bytes, size_t n, float *out) {
+  for (size_t s = 0; s < n / 256; s++) {
+    const uint8_t *block = bytes + s * 136;
+    float d = read_f16(block, 0);
+    for (int ib = 0; ib < 8; ib++) {
+      float dl = d * (float)iq4_xs_scale(block, ib);
+      const uint8_t *qs = block + 8 + 16 * ib;
+      for (int j = 0; j < 16; j++) {
+        out[s * 256 + 32 * (size_t)ib + (size_t)j] = dl * (float)KVALUES_IQ4NL[qs[j] & 0xF];
+        out[s * 256 + 32 * (size_t)ib + (size_t)j + 16] = dl * (float)KVALUES_IQ4NL[qs[j] >> 4];
+      }
+    }
+  }
+}
+
+/* quant.rs:798-827 */
+static void dequantize_q2_k(const uint8_t *bytes, size_t n, float *out) {
+  for (size_t s = 0; s < n / 256; s++) {
+    const uint8_t *block = bytes + s * 84;
+    const uint8_t *scales = block, *qs = block + 16;
+    float d = read_f16(block, 80), dmin = read_f16(block, 82);
+    int is = 0;
+    size_t o = s * 256;
+    for (int q_off = 0; q_off < 64; q_off += 32) {
+      const uint8_t *q = qs + q_off;
+      for (int shift = 0; shift < 8; shift += 2) {
+        for (int half = 0; half < 2; half++) {
+          uint8_t sc = scales[is++];
+          float dl = d * (float)(sc & 0xF), ml = dmin * (float)(sc >> 4);
+          for (int l = 0; l < 16; l++) out[o++] = dl * (float)((q[half * 16 + l] >> shift) & 3) - ml;
+        }
+      }
+    }
+  }
+}
+
 /* quant.rs:883-897 */
 void ogo_unpack_q3_k_scales(const uint8_t *packed, int32_t *scales) {
   for (int i = 0; i < 16; i++) {
@@ -274,6 +353,9 @@ int ogo_dequantize(uint32_t ggml_type, const uint8_t *bytes, size_t element_coun
     case OGO_TYPE_Q4_0:
     case OGO_TYPE_Q5_0:
     case OGO_TYPE_IQ4_NL: dequantize_flat32(ggml_type, bytes, element_count, out); return 0;
+    case OGO_TYPE_Q5_1: dequantize_q5_1(bytes, element_count, out); return 0;
+    case OGO_TYPE_Q2_K: dequantize_q2_k(bytes, element_count, out); return 0;
+    case OGO_TYPE_IQ4_XS: dequantize_iq4_xs(bytes, element_count, out); return 0;
     case OGO_TYPE_Q3_K: dequantize_q3_k(bytes, element_count, out); return 0;
     case OGO_TYPE_Q4_K: dequantize_q4_k(bytes, element_count, out); return 0;
     case OGO_TYPE_Q5_K: dequantize_q5_k(bytes, element_count, out); return 0;
@@ -535,6 +617,23 @@ static void unpack_k_q5_k(const uint8_t *row, size_t in_dim, ogo_krow *out) {
 static const struct { size_t off; int shift; } Q2K_RUNS[8] = {
     {0, 0}, {0, 2}, {0, 4}, {0, 6}, {32, 0}, {32, 2}, {32, 4}, {32, 6}};
 
+/* vecdot.rs:1117-1121 unpack_q2k_run */
+static inline void unpack_q2k_run(const uint8_t *qs, int shift, int8_t *w) {
+  for (int j = 0; j < 32; j++) w[j] = (int8_t)((qs[j] >> shift) & 3);
+}
+
+/* vecdot.rs:2333-2350 unpack_k_iq4_xs */
+static void unpack_k_iq4_xs(const uint8_t *row, size_t in_dim, ogo_krow *out) {
+  for (size_t s = 0; s < in_dim / 256; s++) {
+    const uint8_t *block = row + s * 136;
+    out->d[s] = read_f16(block, 0);
+    for (int ib = 0; ib < 8; ib++) {
+      out->sc[s * 8 + (size_t)ib] = (int16_t)iq4_xs_scale(block, ib);
+      unpack_block_iq4_nl(block + 8 + ib * 16, out->q + (s * 8 + (size_t)ib) * 32);
+    }
+  }
+}
+
 /* vecdot.rs:1131-1136 unpack_q3k_run */
 static inline void unpack_q3k_run(const uint8_t *qs, const uint8_t *hmask, int shift, uint8_t bit,
                                   int8_t *w) {
@@ -675,6 +774,20 @@ float ogo_dot_k_row_q6_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
                          int32_t *isum_out) {
   return DISPATCH(dot_k_row_q6_k, row, in_dim, q, d, isum_out);
 }
+float ogo_dot_q5_1(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d, const int32_t *sums,
+                   int32_t *isum_out) {
+  return DISPATCH(dot_q5_1, row, in_dim, q, d, sums, isum_out);
+}
+float ogo_dot_k_row_iq4_xs(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d, int32_t *isum_out) {
+  return DISPATCH(dot_k_row_iq4_xs, row, in_dim, q, d, isum_out);
+}
+float ogo_dot_k_row_q2_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d, const int32_t *sums,
+                         int32_t *isum_out, int32_t *imin_out) {
+  return DISPATCH(dot_k_row_q2_k, row, in_dim, q, d, sums, isum_out, imin_out);
+}
+float ogo_dot_unpacked_q2_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d, const int32_t *sums) {
+  return DISPATCH(dot_unpacked_q2_k, row, in_dim, q, d, sums);
+}
 float ogo_dot_k_row_q3_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
                          int32_t *isum_out) {
   return DISPATCH(dot_k_row_q3_k, row, in_dim, q, d, isum_out);
@@ -682,19 +795,25 @@ float ogo_dot_k_row_q3_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
 
 /* ------------------------------------------------------------------ predicates */
 
-/* vecdot.rs:274-283, restricted to the types on the path */
+/* vecdot.rs:274-283 */
 int ogo_supports(uint32_t t, size_t in_dim) {
-  if (t == OGO_TYPE_Q8_0 || t == OGO_TYPE_Q5_0 || t == OGO_TYPE_Q4_0 || t == OGO_TYPE_IQ4_NL) return in_dim % 32 == 0;
-  if (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) return in_dim % 256 == 0;
+  if (t == OGO_TYPE_Q8_0 || t == OGO_TYPE_Q5_0 || t == OGO_TYPE_Q4_0 || t == OGO_TYPE_Q5_1 || t == OGO_TYPE_IQ4_NL)
+    return in_dim % 32 == 0;
+  if (t == OGO_TYPE_Q2_K || t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K ||
+      t == OGO_TYPE_IQ4_XS)
+    return in_dim % 256 == 0;
   return 0;
 }
 /* vecdot.rs:1821-1826 */
 int ogo_supports_k(uint32_t t, size_t in_dim) {
-  return (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
+  return (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K || t == OGO_TYPE_IQ4_XS) &&
+         in_dim % 256 == 0;
 }
 /* vecdot.rs:3083-3093 */
 int ogo_supports_k_row(uint32_t t, size_t in_dim) {
-  return (t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K) && in_dim % 256 == 0;
+  return (t == OGO_TYPE_Q2_K || t == OGO_TYPE_Q3_K || t == OGO_TYPE_Q4_K || t == OGO_TYPE_Q5_K || t == OGO_TYPE_Q6_K ||
+          t == OGO_TYPE_IQ4_XS) &&
+         in_dim % 256 == 0;
 }
 /* vecdot.rs:2456-2461 */
 int ogo_supports_flat(uint32_t t, size_t in_dim) {
@@ -732,6 +851,8 @@ static void dot_k_pair(uint32_t ggml_type, const ogo_krow *w0, const ogo_krow *w
                        const ogo_actq8k *a, float *out0, float *out1) {
   if (ggml_type == OGO_TYPE_Q4_K || ggml_type == OGO_TYPE_Q5_K) {   /* both fill a KKind::Q4K row */
     DISPATCH(gemm_k_q4_k, w0, w1, a, out0, out1);
+  } else if (ggml_type == OGO_TYPE_IQ4_XS) {
+    DISPATCH(gemm_k_iq4_xs, w0, w1, a, out0, out1);
   } else {
     DISPATCH(gemm_k_q6_k, w0, w1, a, out0, out1);
   }
@@ -744,6 +865,8 @@ static void unpack_k_row(uint32_t ggml_type, const uint8_t *row, size_t in_dim, 
     unpack_k_q5_k(row, in_dim, out);
   } else if (ggml_type == OGO_TYPE_Q3_K) {
     unpack_k_q3_k(row, in_dim, out);
+  } else if (ggml_type == OGO_TYPE_IQ4_XS) {
+    unpack_k_iq4_xs(row, in_dim, out);
   } else {
     unpack_k_q6_k(row, in_dim, out);
   }
@@ -850,10 +973,14 @@ static int flat_gemm_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes,
 /* One GEMV per (row, token) with the kernel cpu.rs picks at n_tokens == 1; yt is
  * [out_dim][n_tokens].  Shared by matmul at T == 1 (cpu.rs:100-137) and matmul_decode at any T
  * (cpu.rs:265-317). */
+/* generic: the rows-unpacked-once path of matmul at n_tokens > 1 for a type with neither a K GEMM nor a
+ * flat one (cpu.rs:113-163): per-32 activations for every type.  Per token it is dot_unpacked_impl's
+ * arithmetic, which for Q5_1 equals dot_q5_1's bit for bit (scale * isum - (-m) * bsum) and for Q2_K
+ * does not equal dot_k_row_q2_k's. */
 static int gemv_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t in_dim,
                   size_t out_dim, const float *x, size_t n_tokens, float *yt, int threads,
-                  int32_t *isum_out, int32_t *imin_out) {
-  int k_row = ogo_supports_k_row(ggml_type, in_dim);
+                  int32_t *isum_out, int32_t *imin_out, int generic) {
+  int k_row = !generic && ogo_supports_k_row(ggml_type, in_dim);
   size_t n_d = k_row ? in_dim / 256 : in_dim / 32;
   int8_t *q = (int8_t *)malloc(n_tokens * in_dim);
   float *d = (float *)malloc(sizeof(float) * n_tokens * n_d);
@@ -887,6 +1014,13 @@ static int gemv_t(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size
         v = DISPATCH(dot_k_row_q6_k, row, in_dim, qt, dt, io);
       else if (ggml_type == OGO_TYPE_Q3_K)
         v = DISPATCH(dot_k_row_q3_k, row, in_dim, qt, dt, io);
+      else if (ggml_type == OGO_TYPE_IQ4_XS)
+        v = DISPATCH(dot_k_row_iq4_xs, row, in_dim, qt, dt, io);
+      else if (ggml_type == OGO_TYPE_Q2_K)
+        v = generic ? DISPATCH(dot_unpacked_q2_k, row, in_dim, qt, dt, st)
+                    : DISPATCH(dot_k_row_q2_k, row, in_dim, qt, dt, st, io, mo);
+      else if (ggml_type == OGO_TYPE_Q5_1)
+        v = DISPATCH(dot_q5_1, row, in_dim, qt, dt, st, io);
       else if (ggml_type == OGO_TYPE_Q8_0)
         v = DISPATCH(dot_q8_0, row, in_dim, qt, dt, io);
       else
@@ -920,6 +1054,12 @@ int ogo_gemv_act(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_
       v = DISPATCH(dot_k_row_q6_k, row, in_dim, q, d, NULL);
     else if (ggml_type == OGO_TYPE_Q3_K)
       v = DISPATCH(dot_k_row_q3_k, row, in_dim, q, d, NULL);
+    else if (ggml_type == OGO_TYPE_IQ4_XS)
+      v = DISPATCH(dot_k_row_iq4_xs, row, in_dim, q, d, NULL);
+    else if (ggml_type == OGO_TYPE_Q2_K)
+      v = DISPATCH(dot_k_row_q2_k, row, in_dim, q, d, sums, NULL, NULL);
+    else if (ggml_type == OGO_TYPE_Q5_1)
+      v = DISPATCH(dot_q5_1, row, in_dim, q, d, sums, NULL);
     else if (ggml_type == OGO_TYPE_Q8_0)
       v = DISPATCH(dot_q8_0, row, in_dim, q, d, NULL);
     else
@@ -943,7 +1083,7 @@ int ogo_matmul(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, size_t 
   else if (n_tokens > 1 && ogo_supports_flat(ggml_type, in_dim))
     rc = flat_gemm_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads);
   else
-    rc = gemv_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads, NULL, NULL);
+    rc = gemv_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads, NULL, NULL, n_tokens > 1);
   if (rc == 0) finish_into(y, yt, n_tokens, out_dim);
   free(yt);
   return rc;
@@ -957,7 +1097,7 @@ int ogo_matmul_decode(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, 
   int threads = pick_threads(n_threads);
   float *yt = (float *)malloc(sizeof(float) * out_dim * n_tokens);
   if (!yt) return -3;
-  int rc = gemv_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads, NULL, NULL);
+  int rc = gemv_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, threads, NULL, NULL, 0);
   if (rc == 0) finish_into(y, yt, n_tokens, out_dim);
   free(yt);
   return rc;
@@ -970,8 +1110,8 @@ int ogo_block_sums(uint32_t ggml_type, const uint8_t *raw, size_t row_bytes, siz
   if (!ogo_supports(ggml_type, in_dim)) return -1;
   float *yt = (float *)malloc(sizeof(float) * out_dim * n_tokens);
   if (!yt) return -3;
-  int rc = gemv_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, pick_threads(0),
-                  isum, (ggml_type == OGO_TYPE_Q4_K || ggml_type == OGO_TYPE_Q5_K) ? imin : NULL);
+  int rc = gemv_t(ggml_type, raw, row_bytes, in_dim, out_dim, x, n_tokens, yt, pick_threads(0), isum,
+                  (ggml_type == OGO_TYPE_Q4_K || ggml_type == OGO_TYPE_Q5_K || ggml_type == OGO_TYPE_Q2_K) ? imin : NULL, 0);
   free(yt);
   return rc;
 }

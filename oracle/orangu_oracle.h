@@ -50,12 +50,15 @@ extern "C" {
 #define OGO_TYPE_F16 1u
 #define OGO_TYPE_Q4_0 2u
 #define OGO_TYPE_Q5_0 6u
+#define OGO_TYPE_Q5_1 7u
 #define OGO_TYPE_Q8_0 8u
+#define OGO_TYPE_Q2_K 10u
 #define OGO_TYPE_Q3_K 11u
 #define OGO_TYPE_Q4_K 12u
 #define OGO_TYPE_Q5_K 13u
 #define OGO_TYPE_Q6_K 14u
 #define OGO_TYPE_IQ4_NL 20u
+#define OGO_TYPE_IQ4_XS 23u
 
 #define OGO_ACT_BLOCK 32   /* vecdot.rs ACT_BLOCK */
 #define OGO_GROUP 16       /* vecdot.rs:63 */
@@ -106,6 +109,16 @@ float ogo_dot_k_row_q5_k(const uint8_t *row, size_t in_dim, const int8_t *q, con
                          const int32_t *sums, int32_t *isum_out, int32_t *imin_out); /* :3181-3213 */
 float ogo_dot_k_row_q6_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
                          int32_t *isum_out);                                          /* :3215-3241 */
+/* vecdot.rs:2886-2899 dot_q5_1 (per-32 activations; sums are the per-16 sums of quantize_act) */
+float ogo_dot_q5_1(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d, const int32_t *sums,
+                   int32_t *isum_out);
+/* vecdot.rs:3245-3266 dot_k_row_iq4_xs, :3296-3318 dot_k_row_q2_k (per-256 activations) */
+float ogo_dot_k_row_iq4_xs(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d, int32_t *isum_out);
+float ogo_dot_k_row_q2_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d, const int32_t *sums,
+                         int32_t *isum_out, int32_t *imin_out);
+/* vecdot.rs:1144-1164 unpack_q2_k + :407-428 dot_unpacked_impl: Q2_K against per-32 activations, a term per
+ * group of 16 (the prefill path of a type that supports_k leaves out) */
+float ogo_dot_unpacked_q2_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d, const int32_t *sums);
 float ogo_dot_k_row_q3_k(const uint8_t *row, size_t in_dim, const int8_t *q, const float *d,
                          int32_t *isum_out);                                          /* :3273-3292 */
 /* quant.rs:883-897: the 16 six-bit scales of a Q3_K block, still biased by 32 */

@@ -16,8 +16,8 @@ import numpy as np
 from . import capi
 from .capi import OgmError, OgmOp
 
-BLOCK_LAYOUT = {2: (18, 32), 6: (22, 32), 8: (34, 32), 11: (110, 256), 12: (144, 256), 13: (176, 256), 14: (210, 256),
-                20: (18, 32)}
+BLOCK_LAYOUT = {2: (18, 32), 6: (22, 32), 7: (24, 32), 8: (34, 32), 10: (84, 256), 11: (110, 256), 12: (144, 256),
+                13: (176, 256), 14: (210, 256), 20: (18, 32), 23: (136, 256)}
 
 # backend/mod.rs:304-306
 MATMUL_ONLY_SURFACE = "matmul only - no fused layer chain, GPU attention or GPU sampling"

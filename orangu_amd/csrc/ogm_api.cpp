@@ -129,8 +129,11 @@ static uint32_t block_elems_of(uint32_t ggml_type) {
   return ogm_layout_for(ggml_type, &l) ? l.block_elems : 256u;
 }
 
-static int act_mode_for(uint32_t ggml_type) {
-  // backend/cpu.rs:100-116: the K-quants take quantize_act_k_row (per 256), the per-32 types quantize_act
+static int act_mode_for(uint32_t ggml_type, uint32_t n_tokens = 1, int decode = 1) {
+  // backend/cpu.rs:100-116: the K-quants take quantize_act_k_row (per 256), the per-32 types quantize_act.
+  // Q2_K has a per-256 dot for one token (supports_k_row) but no K GEMM (supports_k): matmul of several
+  // tokens unpacks its rows once and runs them against quantize_act's per-32 activations (cpu.rs:113-163).
+  if (ggml_type == OGM_Q2_K && !decode && n_tokens > 1) return OGM_ACT_PER_32;
   return block_elems_of(ggml_type) == 32 ? OGM_ACT_PER_32 : OGM_ACT_PER_256;
 }
 
@@ -464,7 +467,7 @@ static int enqueue_matmul(ogm_ctx *ctx, const Target *tg, size_t n_tg, const flo
   const ogm_weight *w = tg[0].w;
   if (n_tokens == 1 && !dump_isum && !dump_imin && fuse_quantize(ctx, tg, n_tg))
     return enqueue_gemv(ctx, tg, n_tg, 1, decode, stream, nullptr, nullptr, x_dev);
-  int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type), x_dev, w->in_dim, n_tokens, stream);
+  int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type, n_tokens, decode), x_dev, w->in_dim, n_tokens, stream);
   if (rc != OGM_OK) return rc;
   return enqueue_gemv(ctx, tg, n_tg, n_tokens, decode, stream, dump_isum, dump_imin, nullptr);
 }
@@ -522,7 +525,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
                         const float *x_f32, const OgmGemvTail *tail, const OgmActDev *act_base) {
   const ogm_weight *w0 = tg[0].w;
   if (tail && (n_tokens != 1 || n_tg > OGM_GEMV_MAX_MATS)) return fail(ctx, OGM_ERR_INVALID, "a GEMV tail needs one launch of one token");
-  const int mode = act_mode_for(w0->ggml_type);
+  const int mode = act_mode_for(w0->ggml_type, n_tokens, decode);
   // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
   // n_tokens == 1 and every matmul_decode take the GEMV's.
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
@@ -687,7 +690,7 @@ extern "C" int ogm_matmul_dev_static(ogm_ctx *ctx, const ogm_weight *w, const fl
   std::lock_guard<std::mutex> lock(ctx->mu);
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
-  const int mode = act_mode_for(w->ggml_type);
+  const int mode = act_mode_for(w->ggml_type, n_tokens, decode);
   const OgmActDev act = ogm_static_act_view(ctx->static_scratch);
   // The quantizer writes every value the kernels below read for these tokens: nothing in the
   // array has to start at zero, and what an earlier call left beyond them is never read.
@@ -755,7 +758,8 @@ extern "C" int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const floa
   std::lock_guard<std::mutex> lock(ctx->mu);
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
-  return enqueue_quantize(ctx, act_mode_for(ggml_type), x_dev, in_dim, n_tokens, s);
+  // (for matmul's arithmetic: Q2_K at several tokens is quantized per 32, and a decode batch over it is refused below)
+  return enqueue_quantize(ctx, act_mode_for(ggml_type, n_tokens, 0), x_dev, in_dim, n_tokens, s);
 }
 
 extern "C" int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens,
@@ -765,7 +769,7 @@ extern "C" int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_
   if (n_tokens == 0) return OGM_OK;
   if (!y_dev) return fail(ctx, OGM_ERR_INVALID, "y is null");
   std::lock_guard<std::mutex> lock(ctx->mu);
-  if (ctx->act_mode != act_mode_for(w->ggml_type) || ctx->act_in_dim != w->in_dim ||
+  if (ctx->act_mode != act_mode_for(w->ggml_type, n_tokens, decode) || ctx->act_in_dim != w->in_dim ||
       ctx->act_tokens < n_tokens)
     return fail(ctx, OGM_ERR_INVALID, "the quantized activations do not fit this weight "
                 "(call ogm_act_quantize_dev with its type, in_dim and token count first)");
@@ -813,7 +817,7 @@ extern "C" int ogm_matmul_multi_act_dev(ogm_ctx *ctx, const ogm_weight *const *w
   int rc = group_targets(ctx, ws, n_ws, ys_dev /* stands in for x: only null-checked */, n_tokens, ys_dev, tg);
   if (rc != OGM_OK) return rc;
   std::lock_guard<std::mutex> lock(ctx->mu);
-  if (ctx->act_mode != act_mode_for(ws[0]->ggml_type) || ctx->act_in_dim != ws[0]->in_dim ||
+  if (ctx->act_mode != act_mode_for(ws[0]->ggml_type, n_tokens, decode) || ctx->act_in_dim != ws[0]->in_dim ||
       ctx->act_tokens < n_tokens)
     return fail(ctx, OGM_ERR_INVALID, "the quantized activations do not fit these weights "
                 "(call ogm_act_quantize_dev with their type, in_dim and token count first)");
@@ -981,7 +985,7 @@ extern "C" int ogm_dump_block_sums(ogm_ctx *ctx, const ogm_weight *w, const floa
   const size_t blocks = (size_t)w->in_dim / block_elems_of(w->ggml_type);
   const size_t nb = (size_t)n_tokens * w->out_dim * blocks * 4;
   const size_t xb = (size_t)n_tokens * w->in_dim * 4, yb = (size_t)n_tokens * w->out_dim * 4;
-  const bool want_min = imin && (w->ggml_type == OGM_Q4_K || w->ggml_type == OGM_Q5_K);
+  const bool want_min = imin && (w->ggml_type == OGM_Q4_K || w->ggml_type == OGM_Q5_K || w->ggml_type == OGM_Q2_K);
   if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
   if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
   if ((rc = ensure_dev(ctx, ctx->isum, nb)) != OGM_OK) return rc;
@@ -1634,9 +1638,9 @@ static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws
 static int llama_norm_matmul_rows(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *const *ws, float *const *ys, size_t n,
                                   const float *delta, const float *norm_w, uint32_t T, hipStream_t s) {
   const ogm_llama_config &c = m->cfg;
-  const int mode = act_mode_for(ws[0]->ggml_type);
+  const int mode = act_mode_for(ws[0]->ggml_type, T, 0);
   for (size_t i = 1; i < n; i++)
-    if (act_mode_for(ws[i]->ggml_type) != mode)
+    if (act_mode_for(ws[i]->ggml_type, T, 0) != mode)
       return fail(ctx, OGM_ERR_UNSUPPORTED, "matrices over one input must share an activation mode");
   int rc = ensure_act(ctx, c.n_embd, T);
   if (rc != OGM_OK) return rc;
@@ -1684,7 +1688,7 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     if ((rc = llama_norm_matmul_rows(ctx, m, w2, y2, 2, P.proj, ffn_norm, T, s)) != OGM_OK) return rc;
     // SwiGLU quantizes its own output for the down projection: h is never stored as f32
     const ogm_weight *wd[1] = {L.w_down};
-    const int mode_d = act_mode_for(L.w_down->ggml_type);
+    const int mode_d = act_mode_for(L.w_down->ggml_type, T, 0);
     if ((rc = ensure_act(ctx, c.n_ff, T)) != OGM_OK) return rc;
     HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, P.gate, P.up, c.n_ff, nullptr, act_view(ctx, c.n_ff, mode_d, 0), s, T));
     if ((rc = llama_matmul_quantized_rows(ctx, wd, y1, 1, mode_d, c.n_ff, T, s)) != OGM_OK) return rc;

@@ -59,6 +59,16 @@ __device__ __forceinline__ uint32_t ldw2(const uint8_t *p) {
 #endif
 }
 
+__device__ __forceinline__ uint32_t ldw4(const uint8_t *p) {
+#if OGM_WEIGHT_NT
+  return __builtin_nontemporal_load((const uint32_t *)p);
+#else
+  return *(const uint32_t *)p;
+#endif
+}
+// component c (a constant after unrolling) of a four-word piece
+__device__ __forceinline__ uint32_t u4c(const uint4 &v, int c) { return c == 0 ? v.x : c == 1 ? v.y : c == 2 ? v.z : v.w; }
+
 __device__ __forceinline__ int byte_of(uint32_t w, int i) { return (int)((w >> (8 * i)) & 0xFFu); }
 __device__ __forceinline__ int sbyte_of(uint32_t w, int i) { return (int)(int8_t)((w >> (8 * i)) & 0xFFu); }
 __device__ __forceinline__ int lo16(uint32_t w) { return (int)(int16_t)(w & 0xFFFFu); }
@@ -112,6 +122,7 @@ struct ActLds {
 
 // Q4_K: d:f16 | dmin:f16 | scales:u8[12] | qs:u8[128]            (quant.rs:664-697)
 struct FmtQ4K {
+  static constexpr int TERMS = 1;   // f32 terms a block leaves for the ordered sum
   static constexpr uint32_t TYPE = OGM_Q4_K;
   static constexpr int PIECES = 9, TILE_BYTES = 64 * 144, ELEMS = 256;
   static constexpr int XPIECES = 16;   // 16-byte activation chunks per block
@@ -209,6 +220,7 @@ struct FmtQ4K {
 // stored inverted: clear means subtract 4.  Sixteen six-bit scales, biased by 32, one per 16.
 // Repacked as seven pieces, the last one holding scales and d (and two bytes of padding).
 struct FmtQ3K {
+  static constexpr int TERMS = 1;   // f32 terms a block leaves for the ordered sum
   static constexpr uint32_t TYPE = OGM_Q3_K;
   static constexpr int PIECES = 7, TILE_BYTES = 64 * 112, ELEMS = 256;
   static constexpr int XPIECES = 16;
@@ -282,6 +294,7 @@ struct FmtQ3K {
 // Q5_K: d:f16 | dmin:f16 | scales:u8[12] | qh:u8[32] | qs:u8[128]          (quant.rs:699-742)
 // Q4_K with a fifth bit: bit j of qh[l] belongs to element l of sub-block j.
 struct FmtQ5K {
+  static constexpr int TERMS = 1;   // f32 terms a block leaves for the ordered sum
   static constexpr uint32_t TYPE = OGM_Q5_K;
   static constexpr int PIECES = 11, TILE_BYTES = 64 * 176, ELEMS = 256;
   static constexpr int XPIECES = 16;
@@ -380,6 +393,7 @@ struct FmtQ5K {
 
 // Q6_K: ql:u8[128] | qh:u8[64] | scales:i8[16] | d:f16                      (quant.rs:744-787)
 struct FmtQ6K {
+  static constexpr int TERMS = 1;   // f32 terms a block leaves for the ordered sum
   static constexpr uint32_t TYPE = OGM_Q6_K;
   static constexpr int PIECES = 13, TILE_BYTES = 64 * 210, ELEMS = 256;
   static constexpr int XPIECES = 16;
@@ -513,6 +527,7 @@ struct FmtQ6K {
 
 // Q8_0: d:f16 | qs:i8[32]                                                     (quant.rs:638-649)
 struct FmtQ80 {
+  static constexpr int TERMS = 1;   // f32 terms a block leaves for the ordered sum
   static constexpr uint32_t TYPE = OGM_Q8_0;
   static constexpr int PIECES = 2, TILE_BYTES = 64 * 34, ELEMS = 32;
   static constexpr int XPIECES = 2;
@@ -567,8 +582,9 @@ struct FmtQ80 {
 // (nibble indexes the sixteen levels of iq_grids.rs:5941-5943).
 template <int KIND>
 struct FmtNib32 {
-  static constexpr uint32_t TYPE = KIND == 0 ? OGM_Q4_0 : (KIND == 1 ? OGM_Q5_0 : OGM_IQ4_NL);
-  static constexpr int TAIL = KIND == 1 ? 6 : 2;
+  static constexpr int TERMS = 1;
+  static constexpr uint32_t TYPE = KIND == 0 ? OGM_Q4_0 : (KIND == 1 ? OGM_Q5_0 : (KIND == 2 ? OGM_IQ4_NL : OGM_Q5_1));
+  static constexpr int TAIL = KIND == 1 ? 6 : (KIND == 3 ? 8 : 2);
   static constexpr int PIECES = 1, TILE_BYTES = 64 * (16 + TAIL), ELEMS = 32;
   static constexpr int XPIECES = 2;
   static constexpr int AUX16 = 0;
@@ -579,14 +595,19 @@ struct FmtNib32 {
   static constexpr bool HAS_UNPACK = false;
   struct Regs {
     uint4 p[PIECES];
-    uint32_t d16, qh;
+    uint32_t d16, qh;   // Q5_1: d16 = d | m << 16
   };
   __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
     const uint8_t *tb = wt + tile * TILE_BYTES;
     r.p[0] = ldw16(tb + lane * 16u);
-    const uint8_t *t = tb + 1024 + lane * TAIL;   // d, then qh (two-byte aligned)
-    r.d16 = ldw2(t);
-    r.qh = KIND == 1 ? (ldw2(t + 2) | (ldw2(t + 4) << 16)) : 0u;
+    const uint8_t *t = tb + 1024 + lane * TAIL;   // d, then qh (two-byte aligned); Q5_1: d, m, qh (eight-byte aligned)
+    if constexpr (KIND == 3) {
+      r.d16 = ldw4(t);
+      r.qh = ldw4(t + 4);
+    } else {
+      r.d16 = ldw2(t);
+      r.qh = KIND == 1 ? (ldw2(t + 2) | (ldw2(t + 4) << 16)) : 0u;
+    }
   }
   __device__ static __forceinline__ uint32_t weights(uint32_t n, uint32_t h4) {
     return ogm_nib32_weights<KIND>(n, h4);
@@ -607,20 +628,181 @@ struct FmtNib32 {
     }
     isum = acc;
     imin = 0;
+    if constexpr (KIND == 3) {   // Q5_1: the block's activation sum (block_sum, vecdot.rs:2701-2703), from the int8 themselves
+      int bs = 0;
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        bs = dot4(0x01010101u, xl[k], bs);
+        bs = dot4(0x01010101u, xh[k], bs);
+      }
+      imin = bs;
+    }
   }
-  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int) {
-    return f16_bits_to_f32(r.d16) * ad * (float)isum;
+  // Q5_1 (vecdot.rs:2886-2899): total += act.d[b] * (dw * isum + m * block_sum); the rows-unpacked-once
+  // form of several tokens (scale * isum - (-m) * block_sum, vecdot.rs:1302-1314, 1698) has the same bits
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int bs) {
+    if constexpr (KIND == 3)
+      return ad * (f16_bits_to_f32(r.d16 & 0xFFFFu) * (float)isum + f16_bits_to_f32(r.d16 >> 16) * (float)bs);
+    else
+      return f16_bits_to_f32(r.d16) * ad * (float)isum;
   }
   // flat GEMM: acc += d * s * dot32 (vecdot.rs:2622-2623)
-  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int,
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int bs,
                                                    float &tmin, float &tdot) {
     tmin = 0.0f;
-    tdot = ad * f16_bits_to_f32(r.d16) * (float)isum;
+    if constexpr (KIND == 3) tdot = term_gemv(r, ad, isum, bs);
+    else tdot = ad * f16_bits_to_f32(r.d16) * (float)isum;
   }
 };
 typedef FmtNib32<0> FmtQ40;
 typedef FmtNib32<1> FmtQ50;
 typedef FmtNib32<2> FmtIQ4NL;
+typedef FmtNib32<3> FmtQ51;
+
+// IQ4_XS: d:f16 | scales_h:u16 | scales_l:u8[4] | qs:u8[128]                 (quant.rs:1350-1375)
+// Eight sub-blocks of 32: sixteen bytes of nibbles each (elements 0..16 low, 16..32 high, through
+// IQ4_NL's sixteen levels), a six-bit scale biased by 32.  The block's 136 bytes are cut at
+// multiples of 16 from its start, so sub-block ib's bytes are the upper half of piece ib and the
+// lower half of piece ib + 1.
+struct FmtIQ4XS {
+  static constexpr int TERMS = 1;
+  static constexpr uint32_t TYPE = OGM_IQ4_XS;
+  static constexpr int PIECES = 9, TILE_BYTES = 64 * 144, ELEMS = 256;
+  static constexpr int XPIECES = 16;
+  static constexpr int AUX16 = 0;
+  static constexpr int ACT_GROUP = 256;
+  static constexpr bool HAS_MIN = false;
+  static constexpr int MAX_THREADS = 512;
+  static constexpr int MAX_THREADS_SINGLE = 1024;
+  static constexpr bool HAS_UNPACK = false;
+  struct Regs {
+    uint4 p[PIECES];
+  };
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
+    const uint8_t *base = wt + tile * TILE_BYTES + lane * 16u;
+#pragma unroll
+    for (int i = 0; i < PIECES; i++) r.p[i] = ldw16(base + i * 1024);
+  }
+  // isum = sum_ib ls_ib * dot32(levels_ib, x_ib)                             (vecdot.rs:3245-3266)
+  template <int UPR>
+  __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col, int &isum, int &imin) {
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;
+    const uint4 *xp = a.xq + col;
+    const uint32_t sh = r.p[0].x >> 16, sl = r.p[0].y, m4 = 0x0F0F0F0Fu;
+    isum = 0;
+    imin = 0;
+#pragma unroll
+    for (int ib = 0; ib < 8; ib++) {
+      const uint4 xl = xp[(2 * ib) * st], xh = xp[(2 * ib + 1) * st];
+      int dot = 0;
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const int w = 2 + 4 * ib + k;   // word of the block: bytes 8 + 16 ib + 4 k ..
+        const uint32_t qw = u4c(r.p[w >> 2], w & 3);
+        dot = dot4(ogm_nib32_weights<2>(qw & m4, 0u), u4c(xl, k), dot);
+        dot = dot4(ogm_nib32_weights<2>((qw >> 4) & m4, 0u), u4c(xh, k), dot);
+      }
+      const int ls = (int)(((sl >> (4 * ib)) & 0xFu) | (((sh >> (2 * ib)) & 3u) << 4)) - 32;
+      isum += ls * dot;
+    }
+  }
+  // GEMV: total += act.d[s] * d * isum                                        (vecdot.rs:3263)
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int) {
+    return ad * f16_bits_to_f32(r.p[0].x & 0xFFFFu) * (float)isum;
+  }
+  // GEMM: acc += ad * (d * isum)                                             (vecdot.rs:2296-2300)
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int, float &tmin, float &tdot) {
+    tmin = 0.0f;
+    tdot = ad * (f16_bits_to_f32(r.p[0].x & 0xFFFFu) * (float)isum);
+  }
+};
+
+// Q2_K: scales:u8[16] | qs:u8[64] | d:f16 | dmin:f16                         (quant.rs:798-827)
+// Eight runs of 32 two-bit values: run p takes qs[32 (p / 4) + j] >> 2 (p % 4); group g of 16 has a
+// four-bit scale (low nibble of scales[g]) and a four-bit min (high nibble).
+// GENERIC false: one token against per-256 activations (dot_k_row_q2_k, vecdot.rs:3296-3318).
+// GENERIC true: several tokens through matmul, the rows-unpacked-once path over per-32 activations
+// (unpack_q2_k + dot_unpacked, vecdot.rs:1144-1164, 420-425, 1722-1728): sixteen f32 terms a block,
+// act.d[g / 2] * ((d * sc_g) * isum_g - (dmin * mn_g) * sums[g]), added in group order.
+template <bool GENERIC>
+struct FmtQ2KT {
+  static constexpr int TERMS = GENERIC ? 16 : 1;
+  static constexpr uint32_t TYPE = OGM_Q2_K;
+  static constexpr int PIECES = 5, TILE_BYTES = 64 * 84, ELEMS = 256;
+  static constexpr int XPIECES = 16;
+  static constexpr int AUX16 = 2;   // per-16 sums of q: 16 x i16 per block
+  static constexpr int ACT_GROUP = GENERIC ? 32 : 256;
+  static constexpr bool HAS_MIN = !GENERIC;
+  static constexpr int MAX_THREADS = 512;
+  static constexpr int MAX_THREADS_SINGLE = 1024;
+  static constexpr bool HAS_UNPACK = false;
+  struct Regs {
+    uint4 p[PIECES];
+    uint32_t dd;   // d | dmin << 16
+  };
+  __device__ static __forceinline__ void load(Regs &r, const uint8_t *wt, size_t tile, uint32_t lane) {
+    const uint8_t *tb = wt + tile * TILE_BYTES;
+    const uint8_t *base = tb + lane * 16u;
+#pragma unroll
+    for (int i = 0; i < PIECES; i++) r.p[i] = ldw16(base + i * 1024);
+    r.dd = ldw4(tb + PIECES * 1024 + lane * 4u);
+  }
+  // the integer dot of group g (sixteen weights) and its activation sum
+  template <int UPR>
+  __device__ static __forceinline__ void group(const Regs &r, const ActLds &a, uint32_t col, const uint32_t *sw, int g,
+                                               int &dot, int &s16, int &sc) {
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;
+    const int p = g >> 1, shift = 2 * (p & 3);
+    const uint4 q = r.p[1 + 2 * (p >> 2) + (g & 1)];   // bytes 16 (g & 1) .. of the run's 32
+    const uint4 x = a.xq[g * st + col];
+    dot = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) dot = dot4((u4c(q, k) >> shift) & 0x03030303u, u4c(x, k), dot);
+    s16 = (g & 1) ? hi16(sw[g >> 1]) : lo16(sw[g >> 1]);
+    sc = byte_of(u4c(r.p[0], g >> 2), g & 3);
+  }
+  template <int UPR>
+  __device__ static __forceinline__ void sums(const Regs &r, const ActLds &a, uint32_t col, int &isum, int &imin) {
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;
+    const uint4 s_lo = a.aux[col], s_hi = a.aux[st + col];  // sum16 of groups 0..7, 8..15
+    const uint32_t sw[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+    isum = 0;
+    imin = 0;
+#pragma unroll
+    for (int g = 0; g < 16; g++) {
+      int dot, s16, sc;
+      group<UPR>(r, a, col, sw, g, dot, s16, sc);
+      isum += (sc & 0xF) * dot;
+      imin += (sc >> 4) * s16;
+    }
+  }
+  template <int UPR>
+  __device__ static __forceinline__ void terms(const Regs &r, const ActLds &a, uint32_t col, float *out) {
+    const uint32_t st = UPR ? (uint32_t)UPR : a.upr;
+    const uint4 s_lo = a.aux[col], s_hi = a.aux[st + col];
+    const uint32_t sw[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+    const float d = f16_bits_to_f32(r.dd & 0xFFFFu), dmin = f16_bits_to_f32(r.dd >> 16);
+#pragma unroll
+    for (int g = 0; g < 16; g++) {
+      int dot, s16, sc;
+      group<UPR>(r, a, col, sw, g, dot, s16, sc);
+      const float scale = d * (float)(sc & 0xF), mn = dmin * (float)(sc >> 4);
+      out[g] = a.d[col * 8u + (g >> 1)] * (scale * (float)dot - mn * (float)s16);
+    }
+  }
+  // GEMV: total += act.d[s] * (d * isum - dmin * imin)                        (vecdot.rs:3315)
+  __device__ static __forceinline__ float term_gemv(const Regs &r, float ad, int isum, int imin) {
+    const float d = f16_bits_to_f32(r.dd & 0xFFFFu), dmin = f16_bits_to_f32(r.dd >> 16);
+    return ad * (d * (float)isum - dmin * (float)imin);
+  }
+  // (the per-256 form has no several-token order of its own: matmul takes the GENERIC form)
+  __device__ static __forceinline__ void term_gemm(const Regs &r, float ad, int isum, int imin, float &tmin, float &tdot) {
+    tmin = 0.0f;
+    tdot = term_gemv(r, ad, isum, imin);
+  }
+};
+typedef FmtQ2KT<false> FmtQ2K;
+typedef FmtQ2KT<true> FmtQ2KGen;
 
 // ------------------------------------------------------------------------------------------
 // GEMV kernel
@@ -656,7 +838,7 @@ struct GemvParams {
 
 template <class F, bool GEMM_ORDER>
 __host__ __device__ constexpr int n_term_arrays() {
-  return (GEMM_ORDER && F::HAS_MIN) ? 2 : 1;
+  return (GEMM_ORDER && F::HAS_MIN && F::TYPE != OGM_Q2_K) ? 2 : 1;   // Q4_K, Q5_K: the min pass first
 }
 
 // Dynamic LDS bytes of one workgroup.
@@ -669,7 +851,7 @@ static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rb_per
   b += (size_t)n_tokens * upr * F::AUX16 * 16;              // aux
   b += (size_t)n_tokens * n_scale * 4;                      // act.d
   b = (b + 15) & ~(size_t)15;
-  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * rb_per_wg * upr * tl.R * 4;  // terms
+  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * rb_per_wg * upr * tl.R * 4 * F::TERMS;  // terms
   return b;
 }
 
@@ -755,7 +937,7 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP) ? F::MAX_THREA
   const uint32_t R = 64u / C, nct = upr / C;
   const uint32_t xch = upr * F::XPIECES;           // 16-byte chunks of q per token
   const uint32_t n_scale = upr * (F::ELEMS / F::ACT_GROUP);
-  const uint32_t term_stride = upr * R;            // floats per token in the term table
+  const uint32_t term_stride = upr * R * F::TERMS;  // floats per token in the term table
   constexpr int NT = n_term_arrays<F, GEMM_ORDER>();
 
   uint4 *l_xq = (uint4 *)lds;                                   // [T][xch]
@@ -904,6 +1086,15 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP) ? F::MAX_THREA
       int isum, imin;
       if constexpr (UNPACK) F::template sums_unpacked<UPR>(unp, cur, a, col, isum, imin);
       else F::template sums<UPR>(cur, a, col, isum, imin);
+      if constexpr (F::TERMS > 1) {
+        // a block leaves several terms, in the order the row adds them
+        float tt[F::TERMS];
+        F::template terms<UPR>(cur, a, col, tt);
+        float *dst = l_term + (size_t)(t * K + rbk) * term_stride + (size_t)col * F::TERMS * R + r_local;
+#pragma unroll
+        for (int g = 0; g < F::TERMS; g++) dst[g * R] = tt[g];
+        continue;
+      }
       const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
       const size_t slot = (size_t)(t * K + rbk) * term_stride + col * R + r_local;
       if (GEMM_ORDER) {
@@ -937,7 +1128,7 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP) ? F::MAX_THREA
       const float *terms = l_term + (size_t)(t * K + rbk) * term_stride + r;
       float acc = 0.0f;
       if (NT == 2) acc = ordered_sum<true>(acc, terms + (size_t)T * K * term_stride, upr, R);
-      acc = ordered_sum<false>(acc, terms, upr, R);
+      acc = ordered_sum<false>(acc, terms, upr * F::TERMS, R);
       if constexpr (TAIL) __hip_atomic_store(&y[(size_t)t * out_dim + orow], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       else y[(size_t)t * out_dim + orow] = acc;
     }
@@ -1008,6 +1199,12 @@ uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order
       return gemm_order ? max_tokens_t<FmtQ50, true>(in_dim) : max_tokens_t<FmtQ50, false>(in_dim);
     case OGM_IQ4_NL:
       return gemm_order ? max_tokens_t<FmtIQ4NL, true>(in_dim) : max_tokens_t<FmtIQ4NL, false>(in_dim);
+    case OGM_Q5_1:
+      return gemm_order ? max_tokens_t<FmtQ51, true>(in_dim) : max_tokens_t<FmtQ51, false>(in_dim);
+    case OGM_IQ4_XS:
+      return gemm_order ? max_tokens_t<FmtIQ4XS, true>(in_dim) : max_tokens_t<FmtIQ4XS, false>(in_dim);
+    case OGM_Q2_K:
+      return gemm_order ? max_tokens_t<FmtQ2KGen, true>(in_dim) : max_tokens_t<FmtQ2K, false>(in_dim);
     default:
       return 0;
   }
@@ -1168,6 +1365,18 @@ hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char 
     case OGM_IQ4_NL:
       if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtIQ4NL,gemm>" : "ogm_gemv_kernel<FmtIQ4NL,gemv>";
       return a.gemm_order ? launch_t<FmtIQ4NL, true>(a, stream) : launch_t<FmtIQ4NL, false>(a, stream);
+    case OGM_Q5_1:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ51,gemm>" : "ogm_gemv_kernel<FmtQ51,gemv>";
+      return a.gemm_order ? launch_t<FmtQ51, true>(a, stream) : launch_t<FmtQ51, false>(a, stream);
+    case OGM_IQ4_XS:
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtIQ4XS,gemm>" : "ogm_gemv_kernel<FmtIQ4XS,gemv>";
+      return a.gemm_order ? launch_t<FmtIQ4XS, true>(a, stream) : launch_t<FmtIQ4XS, false>(a, stream);
+    case OGM_Q2_K:
+      // matmul of several tokens: the rows-unpacked-once arithmetic over per-32 activations; everything
+      // else (one token, matmul_decode): per-256 activations
+      if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ2KGen,gemm>" : "ogm_gemv_kernel<FmtQ2K,gemv>";
+      if (a.gemm_order) return (a.dump_isum || a.dump_imin || a.x_f32) ? hipErrorInvalidValue : launch_t<FmtQ2KGen, true>(a, stream);
+      return launch_t<FmtQ2K, false>(a, stream);
     default:
       return hipErrorInvalidValue;
   }

@@ -1,8 +1,8 @@
 // Tile-planar weight layout shared by the host repacker and the device kernels.
 //
 // A matrix is out_dim rows of `upr` blocks ("units"; one unit is one GGUF block: Q8_0 34 B / 32
-// weights, Q4_0 and IQ4_NL 18 B / 32, Q5_0 22 B / 32, Q3_K 110 B / 256, Q4_K 144 B / 256, Q5_K 176 B / 256, Q6_K 210 B / 256;
-// engine/quant.rs:638-871).  A *tile* holds 64
+// weights, Q4_0 and IQ4_NL 18 B / 32, Q5_0 22 B / 32, Q5_1 24 B / 32, Q2_K 84 B / 256, Q3_K 110 B / 256, Q4_K 144 B / 256,
+// Q5_K 176 B / 256, Q6_K 210 B / 256, IQ4_XS 136 B / 256; engine/quant.rs:537-871, 1350-1375).  A *tile* holds 64
 // units: R consecutive rows x C consecutive blocks, with C = 4 when a row has a multiple of four
 // blocks (else 2, else 1) and R = 64 / C.  Tiles are ordered [row block][column tile]; inside a
 // tile the unit of (row r, block c) is lane c*R + r.
@@ -21,6 +21,9 @@
 //   Q8_0   2  (qs[0..32))                           d      (2 B)
 //   Q4_0   1  (qs[0..16))                           d      (2 B)      (IQ4_NL the same)
 //   Q5_0   1  (qs[0..16))                           d, qh  (6 B)
+//   Q5_1   1  (qs[0..16))                           d, m, qh (8 B)
+//   Q2_K   5  (scales[0..16) | qs[0..64))           d, dmin (4 B)
+//   IQ4_XS 9  (d,scales_h,scales_l,qs[0..8) | qs[8..24) | ... | qs[120..128) + 8 bytes of padding)   -
 //   Q3_K   7  (hmask[0..32) | qs[0..64) | scales,d + 2 bytes of padding)   -
 //   Q4_K   9  (d,dmin,scales | qs[0..128))          -
 //   Q5_K   11 (d,dmin,scales | qh[0..32) | qs)      -
@@ -31,12 +34,15 @@
 
 #define OGM_Q4_0 2u
 #define OGM_Q5_0 6u
+#define OGM_Q5_1 7u
 #define OGM_Q8_0 8u
+#define OGM_Q2_K 10u
 #define OGM_Q3_K 11u
 #define OGM_Q4_K 12u
 #define OGM_Q5_K 13u
 #define OGM_Q6_K 14u
 #define OGM_IQ4_NL 20u
+#define OGM_IQ4_XS 23u
 
 #define OGM_TILE_UNITS 64u
 
@@ -44,7 +50,7 @@ struct OgmLayout {
   uint32_t block_bytes;   // raw bytes per unit
   uint32_t block_elems;   // weights per unit
   uint32_t pieces;        // 16-byte pieces per unit
-  uint32_t tail_bytes;    // bytes kept after all pieces (0, 2 or 6), lane after lane
+  uint32_t tail_bytes;    // bytes kept after all pieces (0, 2, 4, 6 or 8), lane after lane
   uint32_t piece_off;     // raw offset of piece 0 inside the block
   uint32_t tail_off;      // raw offset of the tail inside the block
   uint32_t tile_bytes;    // 64 * block_bytes
@@ -73,6 +79,15 @@ OGM_HD inline bool ogm_layout_for(uint32_t ggml_type, OgmLayout *l) {
       return true;
     case OGM_Q5_0:  // d:f16 | qh:u32 | qs:u8[16]
       *l = OgmLayout{22, 32, 1, 6, 6, 0, 64 * 22};
+      return true;
+    case OGM_Q5_1:  // d:f16 | m:f16 | qh:u32 | qs:u8[16]
+      *l = OgmLayout{24, 32, 1, 8, 8, 0, 64 * 24};
+      return true;
+    case OGM_Q2_K:  // scales:u8[16] | qs:u8[64] | d:f16 | dmin:f16
+      *l = OgmLayout{84, 256, 5, 4, 0, 80, 64 * 84};
+      return true;
+    case OGM_IQ4_XS:  // d:f16 | scales_h:u16 | scales_l:u8[4] | qs:u8[128]; the last piece holds 8 bytes
+      *l = OgmLayout{136, 256, 9, 0, 0, 0, 64 * 144};
       return true;
     case OGM_Q8_0:  // d:f16 | qs:i8[32]
       *l = OgmLayout{34, 32, 2, 2, 2, 0, 64 * 34};

@@ -737,8 +737,8 @@ hipError_t ogm_launch_f32_to_f16(const float *src, void *dst, size_t n, hipStrea
 
 // ------------------------------------------------------------------------------------------
 // one row of a quantized matrix as f32: the embedding lookup (LlamaModel::run_layers,
-// llama.rs:609-614, over dequantize_q8_0 / _q4_0 / _q5_0 / _iq4_nl / _q3_k / _q4_k / _q5_k / _q6_k,
-// quant.rs:537-580, 639-649, 666-787, 841-871, 1320-1337),
+// llama.rs:609-614, over dequantize_q8_0 / _q4_0 / _q5_0 / _q5_1 / _iq4_nl / _iq4_xs / _q2_k / _q3_k / _q4_k /
+// _q5_k / _q6_k, quant.rs:537-636, 639-649, 666-827, 841-871, 1320-1375),
 // reading the tile-planar device copy.  One thread per element; the f32 expressions are the
 // reference's, so the values are bit-identical (built without FMA contraction).
 
@@ -837,6 +837,34 @@ __global__ __launch_bounds__(256) void ogm_dequant_row_kernel(const uint8_t *__r
     const float d = __half2float(__ushort_as_half((unsigned short)(piece_byte(108u) | (piece_byte(109u) << 8))));
     const float dl = d * (float)sc;
     v = dl * (float)qv;
+  } else if (ggml_type == OGM_Q5_1) {
+    // one piece of nibbles; the tail holds d, m and qh (quant.rs:615-636): value = q * d + m
+    const uint8_t *tail = tb + 1024u + lane * 8u;
+    const float d = dq_f16(tail), mm = dq_f16(tail + 2);
+    const uint32_t qh = tail[4] | (tail[5] << 8) | (tail[6] << 16) | ((uint32_t)tail[7] << 24);
+    const uint32_t byte = piece_byte(j & 15u);
+    const uint32_t nib = j < 16 ? (byte & 0xFu) : (byte >> 4);
+    v = (float)(nib | (((qh >> j) & 1u) << 4)) * d + mm;
+  } else if (ggml_type == OGM_IQ4_XS) {
+    // d | scales_h | scales_l[4] | qs[128], all inside the pieces (quant.rs:1350-1375)
+    const int8_t levels[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+    const uint32_t ib = j >> 5, jj = j & 31u;
+    const float d = __half2float(__ushort_as_half((unsigned short)(piece_byte(0u) | (piece_byte(1u) << 8))));
+    const uint32_t sh = piece_byte(2u) | (piece_byte(3u) << 8);
+    const uint32_t low = (piece_byte(4u + (ib >> 1)) >> (4u * (ib & 1u))) & 0xFu;
+    const int ls = (int)(low | (((sh >> (2u * ib)) & 3u) << 4)) - 32;
+    const uint32_t byte = piece_byte(8u + 16u * ib + (jj & 15u));
+    const float dl = d * (float)ls;
+    v = dl * (float)levels[jj < 16 ? (byte & 0xFu) : (byte >> 4)];
+  } else if (ggml_type == OGM_Q2_K) {
+    // scales[16] | qs[64] in the pieces, d and dmin in the tail (quant.rs:798-827)
+    const uint8_t *tail = tb + l.pieces * 1024u + lane * 4u;
+    const float d = dq_f16(tail), dmin = dq_f16(tail + 2);
+    const uint32_t p = j >> 5, jj = j & 31u, g = j >> 4;
+    const uint32_t sc = piece_byte(g);
+    const uint32_t qv = (piece_byte(16u + 32u * (p >> 2) + jj) >> (2u * (p & 3u))) & 3u;
+    const float dl = d * (float)(sc & 0xFu), ml = dmin * (float)(sc >> 4);
+    v = dl * (float)qv - ml;
   } else {  // Q6_K
     const float d = dq_f16(tb + l.pieces * 1024u + lane * 2u);
     const uint32_t h = j >> 7, jj = j & 127u, qd = jj >> 5, li = jj & 31u;

@@ -7,7 +7,7 @@
 // Four nibbles `n` (one per byte, 0..15) as four signed int8 weights.  KIND 0: Q4_0, n - 8;
 // KIND 1: Q5_0, (n | fifth bit) - 16 with the four fifth bits in the low bits of h4; KIND 2: IQ4_NL,
 // n indexes the sixteen levels -127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89,
-// 113 (iq_grids.rs:5941-5943).
+// 113 (iq_grids.rs:5941-5943); KIND 3: Q5_1, n | fifth bit, unsigned 0..31 (unpack_block_q5_1, vecdot.rs:1032).
 template <int KIND>
 __device__ __forceinline__ uint32_t ogm_nib32_weights(uint32_t n, uint32_t h4) {
   if (KIND == 2) {
@@ -18,6 +18,7 @@ __device__ __forceinline__ uint32_t ogm_nib32_weights(uint32_t n, uint32_t h4) {
     const uint32_t pick = ((n >> 3) & 0x01010101u) * 0xFFu;
     return (lo & ~pick) | (hi & pick);
   }
+  if (KIND == 3) return n | (((h4 * 0x00204081u) & 0x01010101u) << 4);
   // v - bias per byte without borrows between bytes: set bit 7, subtract, flip bit 7 back
   const uint32_t v = KIND == 1 ? (n | (((h4 * 0x00204081u) & 0x01010101u) << 4)) : n;
   const uint32_t bias = KIND == 1 ? 0x10101010u : 0x08080808u;

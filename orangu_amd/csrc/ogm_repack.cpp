@@ -8,8 +8,8 @@
 
 extern "C" int ogm_supports_type(uint32_t ggml_type) {
   return ggml_type == OGM_Q8_0 || ggml_type == OGM_Q5_0 || ggml_type == OGM_Q4_0 || ggml_type == OGM_IQ4_NL ||
-         ggml_type == OGM_Q3_K || ggml_type == OGM_Q4_K || ggml_type == OGM_Q5_K ||
-         ggml_type == OGM_Q6_K;
+         ggml_type == OGM_Q3_K || ggml_type == OGM_Q4_K || ggml_type == OGM_Q5_K || ggml_type == OGM_Q6_K ||
+         ggml_type == OGM_Q5_1 || ggml_type == OGM_Q2_K || ggml_type == OGM_IQ4_XS;
 }
 
 extern "C" int ogm_supports(uint32_t ggml_type, uint32_t in_dim) {

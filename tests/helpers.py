@@ -8,12 +8,15 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_0, Q5_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL = 2, 6, 8, 11, 12, 13, 14, 20
+Q4_0, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 2, 6, 7, 8, 10, 11, 12, 13, 14, 20, 23
 FLAT32 = (Q8_0, Q5_0, Q4_0, IQ4_NL)   # symmetric, one f16 scale per 32 (vecdot.rs:2456-2461)
-BLOCK = {Q4_0: (18, 32), Q5_0: (22, 32), Q8_0: (34, 32), Q3_K: (110, 256), Q4_K: (144, 256), Q5_K: (176, 256),
-         Q6_K: (210, 256), IQ4_NL: (18, 32)}
-TYPE_NAME = {Q4_0: "q4_0", Q5_0: "q5_0", Q8_0: "q8_0", Q3_K: "q3_k", Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k",
-             IQ4_NL: "iq4_nl"}
+BLOCK = {Q4_0: (18, 32), Q5_0: (22, 32), Q5_1: (24, 32), Q8_0: (34, 32), Q2_K: (84, 256), Q3_K: (110, 256),
+         Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256), IQ4_NL: (18, 32), IQ4_XS: (136, 256)}
+TYPE_NAME = {Q4_0: "q4_0", Q5_0: "q5_0", Q5_1: "q5_1", Q8_0: "q8_0", Q2_K: "q2_k", Q3_K: "q3_k", Q4_K: "q4_k",
+             Q5_K: "q5_k", Q6_K: "q6_k", IQ4_NL: "iq4_nl", IQ4_XS: "iq4_xs"}
+# where a block's f16 fields sit: (offset of d, offset of the second field -- dmin or m -- or None)
+F16_FIELDS = {Q4_0: (0, None), Q5_0: (0, None), Q5_1: (0, 2), Q8_0: (0, None), IQ4_NL: (0, None), Q2_K: (80, 82),
+              Q3_K: (108, None), Q4_K: (0, 2), Q5_K: (0, 2), Q6_K: (208, None), IQ4_XS: (0, None)}
 
 
 def row_bytes(ggml_type: int, in_dim: int) -> int:
@@ -67,6 +70,14 @@ def pin_scales(raw: np.ndarray, ggml_type: int) -> np.ndarray:
         blocks[:, 208:210] = (0x00, 0x30)
     elif ggml_type == Q3_K:   # vecdot.rs:3478
         blocks[:, 108:110] = (0x00, 0x30)
+    elif ggml_type == Q5_1:   # vecdot.rs:3462-3465: d then m
+        blocks[:, 0:2] = (0x00, 0x30)
+        blocks[:, 2:4] = (0x00, 0x2C)
+    elif ggml_type == Q2_K:   # vecdot.rs:3472-3475: d then dmin at the end of the block
+        blocks[:, 80:82] = (0x00, 0x30)
+        blocks[:, 82:84] = (0x00, 0x2C)
+    elif ggml_type == IQ4_XS:   # vecdot.rs:3480
+        blocks[:, 0:2] = (0x00, 0x30)
     return raw
 
 
@@ -114,7 +125,7 @@ def cpu_rs_weights(ggml_type: int, in_dim: int, out_dim: int, nb: NextByte) -> n
         scale = np.float32(0.05) + (np.float32(nb()) / np.float32(255.0)) * np.float32(1.95)
         block[0:2] = np.frombuffer(np.float16(scale).tobytes(), np.uint8)
         qf = 2
-        if ggml_type in (Q4_K, Q5_K):
+        if ggml_type in (Q4_K, Q5_K, Q5_1):
             dmin = np.float32(0.05) + (np.float32(nb()) / np.float32(255.0)) * np.float32(0.95)
             block[2:4] = np.frombuffer(np.float16(dmin).tobytes(), np.uint8)
             qf = 4
@@ -142,6 +153,19 @@ def synth_weights(ggml_type: int, in_dim: int, out_dim: int, seed: int) -> np.nd
     elif ggml_type in (Q4_0, Q5_0, IQ4_NL):
         d = (np.abs(rng.normal(0, 0.02, nblk)) / (127 if ggml_type == IQ4_NL else 16)).astype(np.float16)
         raw[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+    elif ggml_type == Q5_1:
+        d = (np.abs(rng.normal(0, 0.02, nblk)) / 16).astype(np.float16)
+        m = rng.normal(0, 0.01, nblk).astype(np.float16)
+        raw[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+        raw[:, 2:4] = m.view(np.uint8).reshape(-1, 2)
+    elif ggml_type == IQ4_XS:
+        d = (np.abs(rng.normal(0, 0.01, nblk)) / 64).astype(np.float16)
+        raw[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+    elif ggml_type == Q2_K:
+        d = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)
+        dm = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)
+        raw[:, 80:82] = d.view(np.uint8).reshape(-1, 2)
+        raw[:, 82:84] = dm.view(np.uint8).reshape(-1, 2)
     elif ggml_type in (Q4_K, Q5_K):
         d = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)
         dm = np.abs(rng.normal(0, 0.01, nblk)).astype(np.float16)

@@ -7,7 +7,7 @@ import re
 import numpy as np
 import pytest
 
-from helpers import BLOCK, IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0, row_bytes
+from helpers import BLOCK, IQ4_NL, IQ4_XS, Q2_K, Q3_K, Q4_0, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, row_bytes
 from orangu_amd import capi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -35,7 +35,10 @@ def test_supports_predicates_follow_vecdot(lib):
     assert lib.ogm_supports_type(11) and lib.ogm_supports(11, 512) and not lib.ogm_supports(11, 896)   # Q3_K
     for t in (2, 6, 20):   # Q4_0, Q5_0, IQ4_NL
         assert lib.ogm_supports_type(t) and lib.ogm_supports(t, 896) and not lib.ogm_supports(t, 24)
-    assert not lib.ogm_supports_type(0) and not lib.ogm_supports_type(10) and not lib.ogm_supports_type(3)
+    assert lib.ogm_supports_type(Q5_1) and lib.ogm_supports(Q5_1, 896) and not lib.ogm_supports(Q5_1, 24)
+    for t in (Q2_K, IQ4_XS):
+        assert lib.ogm_supports_type(t) and lib.ogm_supports(t, 2048) and not lib.ogm_supports(t, 896)
+    assert not lib.ogm_supports_type(0) and not lib.ogm_supports_type(3) and not lib.ogm_supports_type(16)
     assert lib.ogm_supports(Q8_0, 96) and not lib.ogm_supports(Q8_0, 100)
     assert lib.ogm_supports(Q4_K, 512) and not lib.ogm_supports(Q4_K, 896)
     assert lib.ogm_supports(Q6_K, 256) and not lib.ogm_supports(Q6_K, 0)
@@ -53,11 +56,12 @@ def tiling(upr, out_dim):
     return C_, R, upr // C_, (out_dim + R - 1) // R
 
 
-# bytes a unit takes in the tile-planar form: the raw block, except Q3_K whose last piece is padded
-TILE_UNIT = {Q4_0: 18, Q5_0: 22, Q8_0: 34, IQ4_NL: 18, Q3_K: 112, Q4_K: 144, Q5_K: 176, Q6_K: 210}
+# bytes a unit takes in the tile-planar form: the raw block, except Q3_K and IQ4_XS whose last piece is padded
+TILE_UNIT = {Q4_0: 18, Q5_0: 22, Q5_1: 24, Q8_0: 34, IQ4_NL: 18, Q2_K: 84, Q3_K: 112, Q4_K: 144, Q5_K: 176, Q6_K: 210,
+             IQ4_XS: 144}
 
 
-@pytest.mark.parametrize("ggml_type", [Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ggml_type", [Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K, Q5_1, Q2_K, IQ4_XS])
 @pytest.mark.parametrize("in_blocks,out_dim", [(1, 1), (3, 11), (16, 64), (7, 130), (6, 33), (8, 70)])
 def test_repack_is_a_bijection_on_the_raw_bytes(lib, ggml_type, in_blocks, out_dim):
     bb, be = BLOCK[ggml_type]
@@ -81,7 +85,8 @@ def test_repack_is_a_bijection_on_the_raw_bytes(lib, ggml_type, in_blocks, out_d
 @pytest.mark.parametrize("t,npieces,piece_off,tail_off,tail", [(Q4_K, 9, 0, 0, 0), (Q6_K, 13, 0, 208, 2),
                                                               (Q8_0, 2, 2, 0, 2), (Q5_K, 11, 0, 0, 0),
                                                               (Q3_K, 7, 0, 0, 0), (Q4_0, 1, 2, 0, 2),
-                                                              (Q5_0, 1, 6, 0, 6), (IQ4_NL, 1, 2, 0, 2)])
+                                                              (Q5_0, 1, 6, 0, 6), (IQ4_NL, 1, 2, 0, 2),
+                                                              (Q5_1, 1, 8, 0, 8), (Q2_K, 5, 0, 80, 4), (IQ4_XS, 9, 0, 0, 0)])
 @pytest.mark.parametrize("in_blocks,out_dim", [(8, 70), (6, 40), (3, 65)])
 def test_repack_places_pieces_in_planes(lib, t, npieces, piece_off, tail_off, tail, in_blocks, out_dim):
     """Unit (row o, block b): tile (o / R) * nct + b / C, lane (b % C) * R + o % R; piece p at

@@ -1,0 +1,154 @@
+"""Q5_1, Q2_K and IQ4_XS on the device against the CPU restatement: bit-exact through every entry point
+(one token, decode batches, matmul of several tokens in the reference's several-token arithmetic), the
+integer stage, the extremes of the integer ranges, full-size shapes, and the rows an embedding lookup reads."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import (BLOCK, IQ4_XS, Q2_K, Q5_1, activations_t, pin_scales, pseudo_bytes_fast, row_bytes, synth_weights,
+                     synth_x)
+
+pytestmark = pytest.mark.gpu
+NEW = [Q5_1, Q2_K, IQ4_XS]
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def be():
+    from orangu_amd import Mi355xBackend
+    b = Mi355xBackend()  # raises if the HIP library or the device is missing: no fallback
+    yield b
+    b.close()
+
+
+def qm(raw, t, in_dim, out_dim):
+    from orangu_amd import QuantMatrix
+    return QuantMatrix(np.ascontiguousarray(raw), t, in_dim, out_dim)
+
+
+def assert_bits(got, want, what):
+    got = np.asarray(got, np.float32).reshape(-1)
+    want = np.asarray(want, np.float32).reshape(-1)
+    same = got.view(np.uint32) == want.view(np.uint32)
+    assert same.all(), f"{what}: {(~same).sum()} of {got.size} differ in bits; first at " \
+                       f"{np.nonzero(~same)[0][:5]} got {got[~same][:5]} want {want[~same][:5]}"
+
+
+@pytest.mark.parametrize("t", NEW)
+def test_types_are_supported_and_round_trip(be, t):
+    """supports (vecdot.rs:274-283) and unrepack(repack(W)) == W through the device."""
+    bb, bel = BLOCK[t]
+    assert be.supports_type(t)
+    in_dim, out_dim = bel * 5, 77
+    raw = np.random.default_rng(t).integers(0, 256, row_bytes(t, in_dim) * out_dim, dtype=np.uint8)
+    assert np.array_equal(be.download(qm(raw, t, in_dim, out_dim)), raw)
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim", [
+    (Q5_1, 32, 5), (Q5_1, 896, 19), (Q5_1, 4096, 130), (Q5_1, 4864, 7),
+    (Q2_K, 256, 6), (Q2_K, 512, 5), (Q2_K, 4096, 130), (Q2_K, 5632, 33),
+    (IQ4_XS, 256, 4), (IQ4_XS, 512, 5), (IQ4_XS, 4096, 130), (IQ4_XS, 5632, 33)])
+def test_one_token_and_decode_batches_are_bit_exact(be, t, in_dim, out_dim):
+    """dot_q5_1 / dot_k_row_q2_k / dot_k_row_iq4_xs (vecdot.rs:2886-2899, 3296-3318, 3245-3266) through matmul at
+    one token and matmul_decode at 1..9 tokens (cpu.rs:265-317: each row of the batch is the one-token result)."""
+    raw = pin_scales(pseudo_bytes_fast(row_bytes(t, in_dim) * out_dim, in_dim + out_dim), t)
+    w = qm(raw, t, in_dim, out_dim)
+    x = np.concatenate([activations_t(in_dim, k) for k in range(9)])
+    say("new type", t, in_dim, out_dim)
+    assert_bits(be.matmul(x[:in_dim], 1, w), oracle.matmul(t, raw, in_dim, out_dim, x[:in_dim], 1), "one token")
+    for T in (1, 2, 5, 9):
+        got = be.matmul_decode(x[:T * in_dim], T, w)
+        assert_bits(got, oracle.matmul_decode(t, raw, in_dim, out_dim, x[:T * in_dim], T), f"decode batch of {T}")
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim", [
+    (Q5_1, 64, 17), (Q5_1, 896, 33), (Q5_1, 4096, 70),
+    (Q2_K, 512, 5), (Q2_K, 1024, 70), (Q2_K, 4096, 33),
+    (IQ4_XS, 512, 5), (IQ4_XS, 1024, 70), (IQ4_XS, 4096, 33)])
+@pytest.mark.parametrize("T", [2, 3, 7, 17, 130])
+def test_matmul_of_several_tokens_is_bit_exact(be, t, in_dim, out_dim, T):
+    """matmul at n_tokens > 1 (cpu.rs:55-167): IQ4_XS the K GEMM (gemm_k_iq4_xs, vecdot.rs:2305-2322: ad * (d * isum)),
+    Q5_1 and Q2_K the rows-unpacked-once path over per-32 activations (vecdot.rs:1302-1314, 1144-1164, 1684-1745) --
+    for Q2_K a different quantization and a term per group of 16.  Token counts cover the tile of four and its tail
+    (the reference's cross_check_n_tokens shapes, vulkan/tests.rs:2612-2683)."""
+    raw = synth_weights(t, in_dim, out_dim, seed=t * 1000 + in_dim + T)
+    x = synth_x(T, in_dim, seed=T + 3)
+    got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
+    say("new type matmul", t, in_dim, out_dim, T, be.last_kernel())
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "several tokens")
+
+
+@pytest.mark.parametrize("t", NEW)
+def test_integer_stage_is_exact(be, t):
+    """The per-block integer sums of the one-token path against the CPU's."""
+    in_dim, out_dim, T = 1024, 9, 3
+    raw = pin_scales(pseudo_bytes_fast(row_bytes(t, in_dim) * out_dim, 77), t)
+    x = synth_x(T, in_dim, seed=5)
+    isum, imin = be.dump_block_sums(x, T, qm(raw, t, in_dim, out_dim))
+    wi, wm = oracle.block_sums(t, raw, in_dim, out_dim, x, T)
+    assert np.array_equal(isum, wi)
+    if t == Q2_K:
+        assert np.array_equal(imin, wm)
+
+
+@pytest.mark.parametrize("t", NEW)
+@pytest.mark.parametrize("sign", ["pos", "neg", "alt"])
+def test_extreme_integer_ranges(be, t, sign):
+    """Every quant at its largest magnitude with the largest scales against activations of +-127: Q5_1 31 * 127 per
+    element (and the largest block sum for its m term), Q2_K scale and min 15 with quants 3, IQ4_XS level -127 with
+    scale -32 (|isum| 32 * 127 * 127 * 256 = 1.3e8, inside i32)."""
+    in_dim, out_dim, T = 1024, 7, 4
+    bb, be_ = BLOCK[t]
+    blocks = np.zeros((out_dim * in_dim // be_, bb), np.uint8)
+    half = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    if t == Q5_1:
+        blocks[:, 0:2], blocks[:, 2:4] = half, np.frombuffer(np.float16(-0.37).tobytes(), np.uint8)
+        blocks[:, 4:] = 0xFF
+    elif t == Q2_K:
+        blocks[:, 0:80] = 0xFF
+        blocks[:, 80:82], blocks[:, 82:84] = half, half
+    else:
+        blocks[:, 0:2] = half
+        blocks[:, 2:8] = 0      # ls = 0 - 32 = -32 for every sub-block
+        blocks[:, 8:] = 0       # index 0: level -127
+    x = np.full((T, in_dim), 127.0, np.float32)
+    if sign == "neg":
+        x *= -1
+    elif sign == "alt":
+        x[:, 1::2] *= -1
+        x[1] = -127.0
+    raw = blocks.reshape(-1)
+    w = qm(raw, t, in_dim, out_dim)
+    assert_bits(be.matmul(x[0], 1, w), oracle.matmul(t, raw, in_dim, out_dim, x[0], 1), "extremes, one token")
+    assert_bits(be.matmul(x, T, w), oracle.matmul(t, raw, in_dim, out_dim, x, T), "extremes, several tokens")
+    assert_bits(be.matmul_decode(x, T, w), oracle.matmul_decode(t, raw, in_dim, out_dim, x, T), "extremes, decode batch")
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim", [(Q5_1, 4096, 4096), (Q2_K, 4096, 14336), (IQ4_XS, 14336, 4096),
+                                              (IQ4_XS, 4096, 14336)])
+def test_full_size_shapes(be, t, in_dim, out_dim):
+    """The benchmark's FFN shapes at one token, bit for bit, and at 8 tokens on sampled rows."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + t)
+    x = synth_x(8, in_dim, seed=2)
+    w = qm(raw, t, in_dim, out_dim)
+    assert_bits(be.matmul(x[0], 1, w), oracle.matmul(t, raw, in_dim, out_dim, x[0], 1), "full size, one token")
+    got = np.asarray(be.matmul(x, 8, w)).reshape(8, out_dim)
+    rows = np.r_[0:16, out_dim // 2:out_dim // 2 + 16, out_dim - 16:out_dim]
+    rb = row_bytes(t, in_dim)
+    sub = np.concatenate([raw[r * rb:(r + 1) * rb] for r in rows])
+    assert_bits(got[:, rows], oracle.matmul(t, sub, in_dim, rows.size, x, 8), "full size, 8 tokens, sampled rows")
+    be.evict(w)
+
+
+@pytest.mark.parametrize("t", NEW)
+def test_dequantized_rows_match_the_cpu_dequantizer(be, t):
+    """The rows an embedding lookup reads (llama.rs:609-614 over quant.rs:615-636, 798-827, 1350-1375)."""
+    in_dim, out_dim = 1024, 37
+    raw = pin_scales(pseudo_bytes_fast(row_bytes(t, in_dim) * out_dim, 11), t)
+    got = be.dequant_rows(qm(raw, t, in_dim, out_dim), 3, 20)
+    rb = row_bytes(t, in_dim)
+    want = np.stack([oracle.dequantize(t, raw[r * rb:(r + 1) * rb], in_dim) for r in range(3, 23)])
+    assert_bits(got, want, "dequantized rows")

@@ -12,7 +12,7 @@ from helpers import IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0
 # quant.rs:1389-1417 GOLDEN (the types on the path), kept as data in tests/golden/
 with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "dequantize_checksums.json")) as _f:
     GOLDEN = [(v["ggml_type"], v["name"], v["count"], int(v["checksum"], 16)) for v in json.load(_f)["vectors"]]
-assert {g[0] for g in GOLDEN} == {Q4_0, Q5_0, Q8_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K}
+assert {g[0] for g in GOLDEN} == {Q4_0, Q5_0, Q8_0, IQ4_NL, Q3_K, Q4_K, Q5_K, Q6_K, 7, 10, 23}   # + Q5_1, Q2_K, IQ4_XS
 
 
 @pytest.mark.parametrize("ggml_type,name,count,expected", GOLDEN)
