@@ -1633,20 +1633,31 @@ static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws
 }
 
 // x += delta, RMSNorm, and the matmuls over the normed rows: the norm kernel quantizes its own
-// output (the decode step's kernel, one workgroup per row) and the f32 rows are never stored.  As in
-// the decode step, the matrices behind one norm must take the same activation format.
+// output (the decode step's kernel, one workgroup per row) and the f32 rows are never stored.
 static int llama_norm_matmul_rows(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *const *ws, float *const *ys, size_t n,
                                   const float *delta, const float *norm_w, uint32_t T, hipStream_t s) {
   const ogm_llama_config &c = m->cfg;
-  const int mode = act_mode_for(ws[0]->ggml_type, T, 0);
-  for (size_t i = 1; i < n; i++)
-    if (act_mode_for(ws[i]->ggml_type, T, 0) != mode)
-      return fail(ctx, OGM_ERR_UNSUPPORTED, "matrices over one input must share an activation mode");
   int rc = ensure_act(ctx, c.n_embd, T);
   if (rc != OGM_OK) return rc;
-  HIPCHK(ctx, ogm_launch_norm_quant(mode, m->pf.x, delta, norm_w, c.n_embd, c.rms_eps, nullptr,
-                                    act_view(ctx, c.n_embd, mode, 0), s, T));
-  return llama_matmul_quantized_rows(ctx, ws, ys, n, mode, c.n_embd, T, s);
+  // Matrices that take different activation formats (Q2_K at several tokens wants per-32 ones beside
+  // K-quants' per-256) are served one format after the other; the residual is added once.
+  bool first = true;
+  for (int mode : {OGM_ACT_PER_256, OGM_ACT_PER_32}) {
+    const ogm_weight *wm[OGM_GEMV_MAX_MATS];
+    float *ym[OGM_GEMV_MAX_MATS];
+    size_t k = 0;
+    for (size_t i = 0; i < n && k < OGM_GEMV_MAX_MATS; i++)
+      if (act_mode_for(ws[i]->ggml_type, T, 0) == mode) {
+        wm[k] = ws[i];
+        ym[k++] = ys[i];
+      }
+    if (k == 0) continue;
+    HIPCHK(ctx, ogm_launch_norm_quant(mode, m->pf.x, first ? delta : nullptr, norm_w, c.n_embd, c.rms_eps, nullptr,
+                                      act_view(ctx, c.n_embd, mode, 0), s, T));
+    first = false;
+    if ((rc = llama_matmul_quantized_rows(ctx, wm, ym, k, mode, c.n_embd, T, s)) != OGM_OK) return rc;
+  }
+  return OGM_OK;
 }
 
 // One chunk of T <= OGM_PREFILL_CHUNK tokens whose embedding rows sit in m->pf.x.  With `last`,

@@ -56,6 +56,7 @@ bool block_layout(uint32_t t, uint32_t *bytes, uint32_t *elems) {
     case 13: *bytes = 176; *elems = 256; return true; // Q5_K
     case 14: *bytes = 210; *elems = 256; return true; // Q6_K
     case 20: *bytes = 18; *elems = 32; return true;   // IQ4_NL
+    case 23: *bytes = 136; *elems = 256; return true; // IQ4_XS
     case 26: *bytes = 4; *elems = 1; return true;     // I32
     case 30: *bytes = 2; *elems = 1; return true;     // BF16
     default: return false;

@@ -18,7 +18,7 @@ import sys
 import numpy as np
 import pytest
 
-from helpers import IQ4_NL, Q3_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0, synth_weights
+from helpers import IQ4_NL, IQ4_XS, Q2_K, Q3_K, Q4_0, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, synth_weights
 from oracle import llama_ref as R
 
 pytestmark = pytest.mark.gpu
@@ -156,12 +156,13 @@ def step_both(ref, dev, x, pos, what):
 
 
 @pytest.mark.parametrize("types", [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q4_K, Q4_K, Q4_K, Q4_K),
-                                   (Q5_K, Q5_K, Q6_K, Q5_K), (Q4_0, Q5_0, IQ4_NL, Q8_0)])
+                                   (Q5_K, Q5_K, Q6_K, Q5_K), (Q4_0, Q5_0, IQ4_NL, Q8_0), (IQ4_XS, Q2_K, IQ4_XS, Q2_K),
+                                   (Q5_1, Q5_1, Q5_1, Q5_1)])
 def test_decode_steps_from_an_empty_cache(be, types):
     """Positions 0..5 one after the other: RMSNorm, q/k/v, RoPE, cache append, attention over the
     growing cache, wo, residual, SwiGLU FFN, output norm and vocabulary projection."""
-    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
-                          types=types, max_ctx=16, seed=5)
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320,
+                          n_layer=1 if Q2_K in types else 2, types=types, max_ctx=16, seed=5)
     try:
         for pos in range(6):
             step_both(ref, dev, rng.standard_normal(256).astype(f32), pos, f"types {types} pos {pos}")
@@ -486,13 +487,13 @@ def prefill_both(ref, dev, X, pos0, what, via_tokens=None):
 
 
 @pytest.mark.parametrize("types", [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q5_K, Q3_K, Q6_K, Q5_K),
-                                   (Q4_0, Q5_0, IQ4_NL, Q8_0)])
+                                   (Q4_0, Q5_0, IQ4_NL, Q8_0), (IQ4_XS, Q2_K, IQ4_XS, Q2_K), (Q5_1, Q5_1, Q5_1, Q5_1)])
 @pytest.mark.parametrize("n_tokens", [2, 7, 40])
 def test_prefill_from_an_empty_cache_then_decode(be, types, n_tokens):
     """run_layers at n_tokens > 1 (llama.rs:594-932): 2 and 7 tokens take the multi-token GEMV in
     the GEMM's float order, 40 the MFMA GEMMs; the decode steps after it continue on the cache the
     prefill wrote."""
-    n_layer = 1 if Q3_K in types else 2    # two layers of the large synthetic Q3_K weights cancel badly
+    n_layer = 1 if Q3_K in types or Q2_K in types else 2    # two layers of the large synthetic Q3_K / Q2_K weights cancel badly
     ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=n_layer,
                           types=types, max_ctx=64, seed=51, attn_norm_scale=TAME.get(types[0], 1.0))
     try:
