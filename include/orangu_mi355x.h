@@ -378,6 +378,10 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * "gemm_small_max_tokens" (K-quant GEMMs of at most this many tokens take the small-batch kernel, whose
  * waves work on different super-blocks of the same rows; 0 = default 64, or 128 for matrices of up to
  * 8192 rows; 1 = never);
+ * "gemm_few_tokens_min_rows" (2 to 16 tokens over a Q6_K matrix -- matmul and matmul_decode alike -- take
+ * the kernel that streams the weights once and multiplies every token on the matrix cores when the matrix
+ * has at least this many rows: 0 = default 65536, i.e. a vocabulary projection; 1 = whenever the shape
+ * allows: in_dim a multiple of 1024 whose int8 rows fit LDS; -1 = never);
  * "gemm_sb_waves" (waves of a small-batch workgroup: 8 or 16; 0 = default, 16 for launches of at most
  * 256 workgroups over rows of at least 16 super-blocks);
  * "attn_prefill_variant" (attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the

@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "liborangu_mi355x.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 
-SOURCES = ["ogm_kernels.hip", "ogm_gemm.hip", "ogm_llama.hip", "ogm_static.hip", "ogm_api.cpp", "ogm_repack.cpp", "ogm_gguf.cpp"]
+SOURCES = ["ogm_kernels.hip", "ogm_gemm.hip", "ogm_gemm_ft.hip", "ogm_llama.hip", "ogm_static.hip", "ogm_api.cpp", "ogm_repack.cpp", "ogm_gguf.cpp"]
 
 # -ffp-contract=off: the kernels reproduce the CPU path's f32 results bit for bit, which an FMA
 #   contraction would break.

@@ -60,6 +60,7 @@ struct ogm_ctx {
   int tune_gemm_wide_min_wgs = 0;
   int tune_gemm_q4k_variant = 0;
   int tune_gemm_small_max = 0;   // most tokens for the small-batch GEMM kernel: 0 = default, 1 = never
+  int tune_gemm_ft_min_rows = 0;  // few-token Q6_K kernel: fewest rows it takes (0 = default, 1 = any shape it can, -1 = never)
   int tune_gemm_sb_waves = 0;          // small-batch GEMM: 8 or 16 waves per workgroup, 0 = by the launch
   int tune_host_zero_copy = 1;         // host-pointer calls of up to OGM_ZERO_COPY_MAX bytes: kernels read x / write y in pinned host memory
   int tune_gemm_plane_kernel = 0;      // who reads planes: 0 the all-waves-multiply kernel on large grids, 1 the feeding-wave kernels, 2 the former always
@@ -277,6 +278,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemm_plane_kernel") == 0) {
     if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_kernel must be 0, 1 or 2");
     ctx->tune_gemm_plane_kernel = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_few_tokens_min_rows") == 0) {
+    if (value < -1) return fail(ctx, OGM_ERR_INVALID, "gemm_few_tokens_min_rows must be >= -1");
+    ctx->tune_gemm_ft_min_rows = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_sb_waves") == 0) {
@@ -532,6 +538,29 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   const uint32_t t0 = w0->ggml_type;
   const uint32_t gemm_from = ctx->tune_gemm_min_tokens ? (uint32_t)ctx->tune_gemm_min_tokens
                              : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 6u : 17u;
+  // A few tokens over a Q6_K matrix of many rows (the vocabulary projection of a decode batch): one
+  // streaming pass on the matrix cores, in either float order.
+  if (n_tokens > 1 && !dump_isum && !dump_imin && !act_base && !x_f32 && !tail && ctx->tune_gemm_ft_min_rows >= 0) {
+    bool all = true;
+    for (size_t i = 0; i < n_tg; i++)
+      all = all && ogm_gemm_ft_eligible(tg[i].w->ggml_type, tg[i].w->in_dim, tg[i].w->out_dim, n_tokens,
+                                        (uint32_t)ctx->tune_gemm_ft_min_rows);
+    if (all) {
+      for (size_t i = 0; i < n_tg; i++) {
+        OgmGemmArgs g;
+        g.ggml_type = tg[i].w->ggml_type;
+        g.wt = tg[i].w->dev;
+        g.in_dim = tg[i].w->in_dim;
+        g.out_dim = tg[i].w->out_dim;
+        g.act = act_view(ctx, w0->in_dim, mode, 0);
+        g.n_tokens = n_tokens;
+        g.y = tg[i].y;
+        g.xh = nullptr;
+        HIPCHK(ctx, ogm_launch_gemm_ft(g, gemm_order, stream, &ctx->last_kernel));
+      }
+      return OGM_OK;
+    }
+  }
   if (gemm_order && !dump_isum && !dump_imin && !act_base && n_tokens >= gemm_from &&
       all_gemm_supported(tg, n_tg, n_tokens)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
