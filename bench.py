@@ -9,8 +9,12 @@ quantizer and the GEMV for down, through the library's C ABI with inputs and out
 every pass streams from HBM rather than from the last-level cache.
 
 Prints ONE JSON line: whole-step throughput in algorithmic GB/s, a roofline object for the
-dominant kernel (the Q4_K GEMV over gate+up, timed with HIP events over back-to-back
-launches) and the CPU path (the C oracle, all host cores) timed on a bounded sample.
+dominant kernel (the Q4_K GEMV over gate+up, timed with HIP events over batches of back-to-back
+launches: median and fastest batch; beside it a launch that only reads the same bytes, as the measured
+streaming peak for this footprint) and the CPU path (the C oracle, all host cores) timed on a bounded
+sample.  The same line carries the other legs: the 512-token prefill GEMM, the host-pointer (trait)
+path, the sweep over the other benchmark configurations and the 8B-shaped decode step; `--only-*`,
+`--sweep` and `--only-row` run single legs, which is what the profiles under profiles/ were taken over.
 """
 from __future__ import annotations
 
