@@ -402,6 +402,12 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
  * the quantizer kernel first; 0 or -1 = default, off);
+ * "decode_fuse_heads" (1: the decode step's attention norm, FFN norm and SwiGLU run at the head of the GEMV
+ * launch after them -- extra workgroups at the front of the launch, a flag, the others waiting behind their first
+ * weight loads -- instead of as kernels of their own; same bits, measured slower, off by default; with it
+ * "decode_head_delay" (what the waiting workgroups sleep before their weight loads, in units of 64 clocks,
+ * default 64) and "decode_head_spin_limit" (polls before a waiting workgroup gives up, 0 = default 200000: the
+ * step then fails with OGM_ERR_HIP at its next synchronisation instead of returning its results as good));
  * "decode_fuse_tails" (1: the decode step's FFN norm, SwiGLU and next attention norm run inside the
  * GEMV launch before them, in its last workgroup to finish; 0 = default, kernels of their own, which
  * is faster; same bits).  No other setting changes a result bit. */

@@ -64,6 +64,9 @@ struct ogm_ctx {
   int tune_gemm_sb_waves = 0;          // small-batch GEMM: 8 or 16 waves per workgroup, 0 = by the launch
   int tune_host_zero_copy = 1;         // host-pointer calls of up to OGM_ZERO_COPY_MAX bytes: kernels read x / write y in pinned host memory
   int tune_gemm_plane_kernel = 0;      // who reads planes: 0 the all-waves-multiply kernel on large grids, 1 the feeding-wave kernels, 2 the former always
+  int tune_decode_fuse_heads = 0;      // 1: the decode step's norms and SwiGLU at the head of the GEMV after them
+  int tune_decode_head_delay = 64;     // fused heads: what the waiting workgroups sleep before their weight loads, x 64 clocks
+  int tune_decode_head_spin = 0;       // fused heads: polls before a waiting workgroup gives up (0 = default)
   int tune_decode_fuse_tails = 0;      // 1: the decode step's norms and SwiGLU inside the GEMV before them (slower)
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
@@ -290,6 +293,21 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_gemm_sb_waves = value;
     return OGM_OK;
   }
+  if (strcmp(key, "decode_fuse_heads") == 0) {
+    if (value < 0 || value > 1) return fail(ctx, OGM_ERR_INVALID, "decode_fuse_heads must be 0 or 1");
+    ctx->tune_decode_fuse_heads = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "decode_head_spin_limit") == 0) {
+    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "decode_head_spin_limit must be >= 0");
+    ctx->tune_decode_head_spin = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "decode_head_delay") == 0) {
+    if (value < 0 || value > 1000) return fail(ctx, OGM_ERR_INVALID, "decode_head_delay must be 0..1000");
+    ctx->tune_decode_head_delay = value;
+    return OGM_OK;
+  }
   if (strcmp(key, "decode_fuse_tails") == 0) {
     if (value < 0 || value > 1) return fail(ctx, OGM_ERR_INVALID, "decode_fuse_tails must be 0 or 1");
     ctx->tune_decode_fuse_tails = value;
@@ -456,7 +474,8 @@ struct Target {
 
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
                         hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
-                        const float *x_f32, const OgmGemvTail *tail = nullptr, const OgmActDev *act_base = nullptr);
+                        const float *x_f32, const OgmGemvTail *tail = nullptr, const OgmActDev *act_base = nullptr,
+                        const OgmGemvHead *head = nullptr);
 
 // Whether a single-token launch quantizes inside the GEMV (every workgroup repeats the
 // quantizer on its way in) instead of running the quantizer kernel first.  Off unless asked
@@ -528,8 +547,10 @@ static bool all_gemm_supported(const Target *tg, size_t n_tg, uint32_t n_tokens)
 // on the GEMV kernels whatever the token count (the tiled GEMMs stage through context buffers).
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
                         hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
-                        const float *x_f32, const OgmGemvTail *tail, const OgmActDev *act_base) {
+                        const float *x_f32, const OgmGemvTail *tail, const OgmActDev *act_base,
+                        const OgmGemvHead *head) {
   const ogm_weight *w0 = tg[0].w;
+  if (head && (n_tokens != 1 || tail || x_f32 || dump_isum || dump_imin)) return fail(ctx, OGM_ERR_INVALID, "a GEMV head needs a plain launch of one token");
   if (tail && (n_tokens != 1 || n_tg > OGM_GEMV_MAX_MATS)) return fail(ctx, OGM_ERR_INVALID, "a GEMV tail needs one launch of one token");
   const int mode = act_mode_for(w0->ggml_type, n_tokens, decode);
   // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
@@ -631,6 +652,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       }
       a.x_f32 = x_f32;
       if (tail) a.tail = *tail;
+      if (head && g0 == 0 && t0 == 0) a.head = *head;   // the first launch of the group brings the producers
       HIPCHK(ctx, ogm_launch_gemv(a, stream, &ctx->last_kernel));
     }
   }
@@ -1061,6 +1083,7 @@ struct ogm_llama {
   float *pre = nullptr;       // [n_layer][q_bias qd | k_bias kvd | v_bias kvd | q_norm hd | k_norm hd]
   float *freq = nullptr;      // [rope_dim / 2], frequency factors applied
   float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
+  uint32_t head_epoch = 0;            // value of the GEMV heads' flag (the three words after the tickets) after the last launch
   uint32_t *attn_tickets = nullptr;   // [n_head_kv + OGM_TAIL_TICKETS], zero between launches; the last ones are the GEMV tails'
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
   void *v_cache = nullptr;
@@ -1155,7 +1178,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   A((void **)&m->pre, (size_t)c.n_layer * pre_stride * 4);
   A((void **)&m->freq, (size_t)(c.rope_dim / 2 + 1) * 4);
   A((void **)&m->rope_cs, (size_t)(c.rope_dim / 2 + 1) * 8);
-  A((void **)&m->attn_tickets, ((size_t)c.n_head_kv + OGM_TAIL_TICKETS) * 4);   // + the GEMV tails' tickets
+  A((void **)&m->attn_tickets, ((size_t)c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);   // + the GEMV tails' tickets
   A(&m->k_cache, cache_bytes);
   A(&m->v_cache, cache_bytes);
   A((void **)&m->x, (size_t)c.n_embd * 4);
@@ -1208,7 +1231,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   hipError_t e = hipMemcpy(m->norms, host.data(), host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->pre, pre_host.data(), pre_host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, ((size_t)c.n_head_kv + OGM_TAIL_TICKETS) * 4);
+  if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, ((size_t)c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
   if (e != hipSuccess) {
@@ -1291,7 +1314,7 @@ static int llama_capture(ogm_ctx *ctx, ogm_llama *m, uint32_t site, uint32_t n, 
 
 // One matmul group of the step over the activations the previous kernel quantized.
 static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, hipStream_t s,
-                        const OgmGemvTail *tail = nullptr) {
+                        const OgmGemvTail *tail = nullptr, const OgmGemvHead *head = nullptr) {
   // weights of one type go out as one launch; a mixed group (Q4_K q/k with a Q6_K v) as several
   if (tail) {   // the caller has checked that the group is one launch
     Target tg[OGM_GEMV_MAX_MATS];
@@ -1306,7 +1329,8 @@ static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const 
       tg[e - i] = Target{ws[e], ys[e]};
       e++;
     }
-    int rc = enqueue_gemv(ctx, tg, e - i, 1, 0, s, nullptr, nullptr, nullptr);
+    // (a head's producers ride on the first launch; the launches after it are ordered behind it)
+    int rc = enqueue_gemv(ctx, tg, e - i, 1, 0, s, nullptr, nullptr, nullptr, nullptr, nullptr, i == 0 ? head : nullptr);
     if (rc != OGM_OK) return rc;
     i = e;
   }
@@ -1332,6 +1356,33 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     return fuse && consumer_mode == OGM_ACT_PER_256 && n % 32u == 0 && producer->out_dim == n &&
            n <= ogm_gemv_norm_tail_max(producer->ggml_type, producer->in_dim, n, (uint32_t)ctx->tune_wg_waves);
   };
+  // On request the norms and the SwiGLU run at the *head* of the GEMV launch after them: extra
+  // workgroups at the front of the launch compute and quantize the row while the others already have
+  // their first weights in flight, and hand it over through device-coherent stores and a flag.  Same
+  // bits, and slower on MI355X (8B-shaped model: 2.06 against 1.86 ms per token): the hand-over is a
+  // chain of trips to the memory all compute dies share (stores acknowledged, flag stored, flag
+  // polled, activations loaded) that costs what the kernel boundary it replaces costs, and the
+  // producers' own loads queue behind the launch's weight stream.
+  const bool heads = ctx->tune_decode_fuse_heads != 0 && !fuse && ctx->tune_fuse_quant <= 0;
+  uint32_t *head_flag = m->attn_tickets + ((c.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u);   // 128-byte aligned
+  auto head_ok = [&](const ogm_weight *first, int mode, bool norm) {   // first: the matrix of the group's first launch
+    if (!heads || mode != OGM_ACT_PER_256) return false;
+    const uint32_t waves = ogm_gemv_head_waves(first->ggml_type, first->in_dim, first->out_dim, (uint32_t)ctx->tune_wg_waves);
+    return waves != 0 && (!norm || first->in_dim <= 1024u * waves);   // one producer workgroup norms the whole row
+  };
+  auto norm_head = [&](const float *delta_, const float *weight_) {
+    OgmGemvHead h;
+    h.kind = OGM_HEAD_NORM;
+    h.flag = head_flag;
+    h.epoch = ++m->head_epoch;
+    h.x = m->x;
+    h.delta = delta_;
+    h.weight = weight_;
+    h.eps = c.rms_eps;
+    h.delay = (uint32_t)ctx->tune_decode_head_delay;
+    h.spin_limit = (uint32_t)ctx->tune_decode_head_spin;
+    return h;
+  };
   const int mode_out = act_mode_for(m->output->ggml_type);
   const float *out_norm = m->norms + (size_t)c.n_layer * 2 * c.n_embd;
   bool normed = false;   // the next norm already ran as a tail
@@ -1345,14 +1396,21 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     const int mode_qkv = act_mode_for(L.wq->ggml_type);
     if (act_mode_for(L.wk->ggml_type) != mode_qkv || act_mode_for(L.wv->ggml_type) != mode_qkv)
       return fail(ctx, OGM_ERR_UNSUPPORTED, "wq, wk and wv must share an activation mode");
-    if (!normed)
-      HIPCHK(ctx, ogm_launch_norm_quant(mode_qkv, m->x, delta, attn_norm, c.n_embd, c.rms_eps, nullptr,
-                                        act_view(ctx, c.n_embd, mode_qkv, 0), s));
     const ogm_weight *w3[3] = {L.wq, L.wk, L.wv};
     float *y3[3] = {m->q, m->k, m->v};
-    int rc = llama_capture(ctx, m, 4 * l, c.n_embd, mode_qkv, s);
-    if (rc != OGM_OK) return rc;
-    if ((rc = llama_matmul(ctx, w3, y3, 3, s)) != OGM_OK) return rc;
+    int rc;
+    if (!normed && head_ok(L.wq, mode_qkv, true)) {
+      // the norm rides at the head of the q/k/v launch
+      OgmGemvHead head = norm_head(delta, attn_norm);
+      if ((rc = llama_matmul(ctx, w3, y3, 3, s, nullptr, &head)) != OGM_OK) return rc;
+      if ((rc = llama_capture(ctx, m, 4 * l, c.n_embd, mode_qkv, s)) != OGM_OK) return rc;
+    } else {
+      if (!normed)
+        HIPCHK(ctx, ogm_launch_norm_quant(mode_qkv, m->x, delta, attn_norm, c.n_embd, c.rms_eps, nullptr,
+                                          act_view(ctx, c.n_embd, mode_qkv, 0), s));
+      if ((rc = llama_capture(ctx, m, 4 * l, c.n_embd, mode_qkv, s)) != OGM_OK) return rc;
+      if ((rc = llama_matmul(ctx, w3, y3, 3, s)) != OGM_OK) return rc;
+    }
     const int mode_o = act_mode_for(L.wo->ggml_type);
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, m->rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
@@ -1366,6 +1424,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     if ((rc = llama_capture(ctx, m, 4 * l + 1, qd, mode_o, s)) != OGM_OK) return rc;
     OgmGemvTail tail;
     tail.ticket = m->attn_tickets + c.n_head_kv;
+    bool ffn_head = false;
     if (tail_ok(L.wo, c.n_embd, mode_ff)) {
       tail.kind = OGM_TAIL_NORM;
       tail.n = c.n_embd;
@@ -1376,12 +1435,23 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
       if ((rc = llama_matmul(ctx, w1, y1, 1, s, &tail)) != OGM_OK) return rc;
     } else {
       if ((rc = llama_matmul(ctx, w1, y1, 1, s)) != OGM_OK) return rc;
-      HIPCHK(ctx, ogm_launch_norm_quant(mode_ff, m->x, m->proj, ffn_norm, c.n_embd, c.rms_eps, nullptr,
-                                        act_view(ctx, c.n_embd, mode_ff, 0), s));
+      ffn_head = head_ok(L.w_gate, mode_ff, true);
+      if (!ffn_head)
+        HIPCHK(ctx, ogm_launch_norm_quant(mode_ff, m->x, m->proj, ffn_norm, c.n_embd, c.rms_eps, nullptr,
+                                          act_view(ctx, c.n_embd, mode_ff, 0), s));
     }
     const ogm_weight *w2[2] = {L.w_gate, L.w_up};
     float *y2[2] = {m->gate, m->up};
     const int mode_d = act_mode_for(L.w_down->ggml_type);
+    const bool down_head = head_ok(L.w_down, mode_d, false);
+    if (ffn_head) {
+      OgmGemvHead head = norm_head(m->proj, ffn_norm);
+      if ((rc = llama_matmul(ctx, w2, y2, 2, s, nullptr, &head)) != OGM_OK) return rc;
+      if ((rc = llama_capture(ctx, m, 4 * l + 2, c.n_embd, mode_ff, s)) != OGM_OK) return rc;
+      if (!down_head)
+        HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr,
+                                            act_view(ctx, c.n_ff, mode_d, 0), s));
+    } else {
     if ((rc = llama_capture(ctx, m, 4 * l + 2, c.n_embd, mode_ff, s)) != OGM_OK) return rc;
     if (fuse && mode_d == OGM_ACT_PER_256 && L.w_gate->ggml_type == L.w_up->ggml_type &&
         block_elems_of(L.w_gate->ggml_type) == 256) {
@@ -1393,14 +1463,30 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
       if ((rc = llama_matmul(ctx, w2, y2, 2, s, &tail)) != OGM_OK) return rc;
     } else {
       if ((rc = llama_matmul(ctx, w2, y2, 2, s)) != OGM_OK) return rc;
-      HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr,
-                                          act_view(ctx, c.n_ff, mode_d, 0), s));
+      if (!down_head)
+        HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr,
+                                            act_view(ctx, c.n_ff, mode_d, 0), s));
+    }
     }
     const ogm_weight *wd[1] = {L.w_down};
-    if ((rc = llama_capture(ctx, m, 4 * l + 3, c.n_ff, mode_d, s)) != OGM_OK) return rc;
     // the next norm: the next layer's attention norm, or the output norm after the last layer
     const bool last_layer = l + 1 == c.n_layer;
     const int mode_next = last_layer ? mode_out : act_mode_for(m->layers[l + 1].wq->ggml_type);
+    if (down_head) {
+      // the SwiGLU rides at the head of the down projection
+      OgmGemvHead head;
+      head.kind = OGM_HEAD_SWIGLU;
+      head.flag = head_flag;
+      head.epoch = ++m->head_epoch;
+      head.gate = m->gate;
+      head.up = m->up;
+      head.delay = (uint32_t)ctx->tune_decode_head_delay;
+      head.spin_limit = (uint32_t)ctx->tune_decode_head_spin;
+      if ((rc = llama_matmul(ctx, wd, y1, 1, s, nullptr, &head)) != OGM_OK) return rc;
+      if ((rc = llama_capture(ctx, m, 4 * l + 3, c.n_ff, mode_d, s)) != OGM_OK) return rc;
+      normed = false;
+    } else {
+    if ((rc = llama_capture(ctx, m, 4 * l + 3, c.n_ff, mode_d, s)) != OGM_OK) return rc;
     normed = tail_ok(L.w_down, c.n_embd, mode_next);
     if (normed) {
       tail.kind = OGM_TAIL_NORM;
@@ -1412,6 +1498,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
       if ((rc = llama_matmul(ctx, wd, y1, 1, s, &tail)) != OGM_OK) return rc;
     } else {
       if ((rc = llama_matmul(ctx, wd, y1, 1, s)) != OGM_OK) return rc;
+    }
     }
     delta = m->proj;
   }
@@ -1439,6 +1526,18 @@ extern "C" int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_d
   return llama_decode_enqueue(ctx, m, x_dev, pos, logits_dev, argmax_dev, stream ? (hipStream_t)stream : ctx->stream);
 }
 
+// After a synchronisation: whether a workgroup of a launch with a head gave up waiting for its producers
+// (the step's results are then not to be trusted).  Clears the word.
+static int llama_check_heads(ogm_ctx *ctx, ogm_llama *m) {
+  if (m->head_epoch == 0) return OGM_OK;   // no such launch yet
+  uint32_t *word = m->attn_tickets + ((m->cfg.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u) + OGM_HEAD_FLAG_COPIES * 32u + 1u;
+  uint32_t gave_up = 0;
+  HIPCHK(ctx, hipMemcpy(&gave_up, word, 4, hipMemcpyDeviceToHost));
+  if (!gave_up) return OGM_OK;
+  HIPCHK(ctx, hipMemset(word, 0, 4));
+  return fail(ctx, OGM_ERR_HIP, "a workgroup gave up waiting for the producers at the head of its launch");
+}
+
 extern "C" int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos, float *logits,
                                 uint32_t *argmax) {
   if (!ctx) return OGM_ERR_INVALID;
@@ -1453,7 +1552,7 @@ extern "C" int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint
   if (logits) HIPCHK(ctx, hipMemcpyAsync(logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   if (argmax) HIPCHK(ctx, hipMemcpyAsync(argmax, m->amax_out, 4, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-  return OGM_OK;
+  return llama_check_heads(ctx, m);
 }
 
 extern "C" int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out) {
@@ -1575,7 +1674,7 @@ extern "C" int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
   if (last_logits)
     HIPCHK(ctx, hipMemcpyAsync(last_logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-  return OGM_OK;
+  return llama_check_heads(ctx, m);
 }
 
 // ---- prefill: run_layers at n_tokens > 1 (llama.rs:594-932) ------------------------------------

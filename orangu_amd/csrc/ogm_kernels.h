@@ -44,6 +44,40 @@ struct OgmGemvTail {
   OgmActDev act = {};
 };
 
+// What extra workgroups at the front of a single-token GEMV launch (per-256 activations) compute before
+// its other workgroups read their activations, in place of a kernel of its own ahead of the launch:
+//   OGM_HEAD_NORM   x += delta; act = quantize(rmsnorm(x) * weight)    one producer workgroup, n = in_dim
+//   OGM_HEAD_SWIGLU act = quantize(silu(gate) * up)                    ceil(in_dim / 256 / waves) of them
+// The launch's `act` is what the producers write and the others read.  The producers are the launch's
+// first workgroups, which the hardware starts first; they store device-coherently, and the last of
+// them to finish raises flag[0] to `epoch`.  Every other workgroup requests its first tile of
+// weights, then polls the flag (at most spin_limit times; it then sets the gave-up word and goes on
+// with whatever the activations hold, so every wave ends) and reads the activations.
+// flag: OGM_HEAD_FLAG_WORDS uint32 on the device, zero before the first launch: OGM_HEAD_FLAG_COPIES
+// copies of the flag, 128 bytes apart (a waiting workgroup polls copy `its index % copies`: polls of
+// one address are served one after the other), which only ever grow; then the producers' own counter,
+// zero between launches, and the word a workgroup that gave up sets.  epoch: the flag's value before
+// the launch plus one (launches over one flag must be stream-ordered).
+#define OGM_HEAD_FLAG_COPIES 64u
+#define OGM_HEAD_FLAG_WORDS (OGM_HEAD_FLAG_COPIES * 32u + 2u)
+#define OGM_HEAD_NONE 0u
+#define OGM_HEAD_NORM 1u
+#define OGM_HEAD_SWIGLU 2u
+struct OgmGemvHead {
+  uint32_t kind = OGM_HEAD_NONE;
+  uint32_t *flag = nullptr;
+  uint32_t epoch = 0;
+  uint32_t spin_limit = 0;        // 0: the default (about a tenth of a second)
+  float *x = nullptr;             // NORM: the residual stream, updated in place
+  const float *delta = nullptr;   // NORM: what is added to x first (may be null)
+  const float *weight = nullptr;  // NORM: the norm's weights
+  float eps = 0.0f;
+  const float *gate = nullptr;    // SWIGLU
+  const float *up = nullptr;
+  uint32_t delay = 0;             // what the other workgroups sleep before their first weight loads, in units of 64 clocks
+  uint32_t n_prod = 0;            // filled in by the launcher
+};
+
 struct OgmGemvArgs {
   uint32_t ggml_type;
   const uint8_t *wt;  // tile-planar weights
@@ -66,6 +100,7 @@ struct OgmGemvArgs {
   // quantizes them itself on its way in and `act` is not read.
   const float *x_f32;
   OgmGemvTail tail;   // one token, GEMV order, no dumps, no x_f32
+  OgmGemvHead head;   // one token, GEMV order, no dumps, no x_f32, no tail; per-256 activations
 };
 
 // Largest token count one launch can take for this shape (LDS budget), at least 1.
@@ -73,6 +108,9 @@ uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order
 hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name);
 // Longest row an OGM_TAIL_NORM tail of a single-token launch over this matrix can take (0: none).
 uint32_t ogm_gemv_norm_tail_max(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves);
+// Waves per workgroup of a single-token launch with a head over this matrix (0: the type takes none).
+// An OGM_HEAD_NORM head needs in_dim <= 1024 * that.
+uint32_t ogm_gemv_head_waves(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves);
 
 // Prefill GEMM on MFMA (ogm_gemm.hip).  Same operands as the GEMV plus a scratch buffer `xh` of
 // ogm_gemm_xh_bytes() for the activations as f16.  Follows the CPU path's GEMM float order.

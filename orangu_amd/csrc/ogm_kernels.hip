@@ -834,7 +834,25 @@ struct GemvParams {
   uint32_t n_tokens;
   uint32_t C, nct;                // tile shape: C blocks x R rows, nct = upr / C column tiles
   OgmGemvTail tail;
+  OgmGemvHead head;
 };
+
+// Sixteen bytes / four bytes that another workgroup of the same kernel stored device-coherently.
+__device__ __forceinline__ uint4 ldc16(const void *p) {
+  const uint64_t a = __hip_atomic_load((const uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint64_t b = __hip_atomic_load((const uint64_t *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
+}
+__device__ __forceinline__ float ldc4f(const float *p) {
+  return __uint_as_float(__hip_atomic_load((const uint32_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+#define OGM_HEAD_SPIN_DEFAULT 200000u
+// The activations behind a head's flag: 1 reads them device-coherently (past L2), 0 with plain loads.
+// No workgroup of the launch touches them before it has seen the flag and every L2 starts a kernel
+// invalidated, so plain loads cannot meet a stale line.
+#ifndef OGM_HEAD_COHERENT_READS
+#define OGM_HEAD_COHERENT_READS 0
+#endif
 
 template <class F, bool GEMM_ORDER>
 __host__ __device__ constexpr int n_term_arrays() {
@@ -925,9 +943,11 @@ struct UnpackedOf<F, true, true> { typedef typename F::Unpacked type; };
 // the quantizer kernel's output.
 // UNPACK: several tokens and a format whose block is expensive to unpack: unpack once per tile.
 // TAIL: the outputs are stored device-coherently and the last workgroup to finish runs p.tail.
+// HEAD: the first p.head.n_prod workgroups compute the activations (p.head), the others wait for them
+// behind their first weight loads and read the activations device-coherently.
 template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP, bool QUANT, bool UNPACK = false,
-          bool TAIL = false>
-__global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP) ? F::MAX_THREADS_SINGLE : F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) {
+          bool TAIL = false, bool HEAD = false>
+__global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::MAX_THREADS_SINGLE : F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t tid = threadIdx.x, nthr = blockDim.x;
   const uint32_t lane = tid & 63u, wave = tid >> 6, n_wave = nthr >> 6;
@@ -946,12 +966,42 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP) ? F::MAX_THREA
   const size_t head = ((size_t)T * (xch * 16 + upr * F::AUX16 * 16 + n_scale * 4) + 15) & ~(size_t)15;
   float *l_term = (float *)(lds + head);                        // [NT][T][K][upr][R]
 
+  uint32_t bid = blockIdx.x;
+  if constexpr (HEAD) {
+    if (bid < p.head.n_prod) {
+      // ---- a producer: the activations of the launch, stored for the other workgroups
+      if (p.head.kind == OGM_HEAD_NORM) {
+        ogm_norm_quant_row<256, false, true>(p.head.x, p.head.delta, p.head.weight, p.in_dim, p.head.eps, nullptr,
+                                             p.act, (float *)lds, tid, n_wave);
+      } else {
+        const uint32_t run = bid * n_wave + wave;
+        if (run * 256u < p.in_dim)
+          ogm_swiglu_quant_run<256, false, true>(p.head.gate, p.head.up, p.in_dim, nullptr, p.act, run, lane);
+      }
+      // every wave's stores acknowledged, the workgroup met: the last producer raises the flag
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      uint32_t *l_last = (uint32_t *)lds;
+      if (tid == 0) {
+        uint32_t *count = p.head.flag + OGM_HEAD_FLAG_COPIES * 32u;
+        const bool last = __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.head.n_prod - 1u;
+        if (last) __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        l_last[0] = last ? 1u : 0u;
+      }
+      __syncthreads();
+      // every copy of the flag sits in a cache line of its own: the waiting workgroups spread over them
+      if (l_last[0] != 0u && tid < OGM_HEAD_FLAG_COPIES)
+        __hip_atomic_store(p.head.flag + tid * 32u, p.head.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    bid -= p.head.n_prod;
+  }
   // ---- which matrix of the launch this workgroup belongs to, and which of its row blocks
   uint32_t m = 0;
-  if (blockIdx.x >= p.wg_end[0]) m = 1;
-  if (blockIdx.x >= p.wg_end[1]) m = 2;
-  if (blockIdx.x >= p.wg_end[2]) m = 3;
-  const uint32_t wg = blockIdx.x - (m == 0 ? 0u : m == 1 ? p.wg_end[0] : m == 2 ? p.wg_end[1] : p.wg_end[2]);
+  if (bid >= p.wg_end[0]) m = 1;
+  if (bid >= p.wg_end[1]) m = 2;
+  if (bid >= p.wg_end[2]) m = 3;
+  const uint32_t wg = bid - (m == 0 ? 0u : m == 1 ? p.wg_end[0] : m == 2 ? p.wg_end[1] : p.wg_end[2]);
   const uint32_t K = p.rb_per_wg;
   const uint32_t rb0 = wg * K;
   const uint8_t *wt = m == 0 ? p.wt[0] : m == 1 ? p.wt[1] : m == 2 ? p.wt[2] : p.wt[3];
@@ -974,33 +1024,55 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP) ? F::MAX_THREA
     return *(const float4 *)(p.x + min(e0, p.in_dim - 4u));
   };
   constexpr int QPEEL = (UPR == 16) ? 4 : 8;  // 4096-wide rows: four groups for each of four waves
+  // (with producers in the launch the activations are read device-coherently, and only later)
+  auto ld_q = [&](uint32_t i) -> uint4 {
+    if constexpr (HEAD && OGM_HEAD_COHERENT_READS) return ldc16(gq + i);
+    else return gq[i];
+  };
+  auto ld_bsum = [&](uint32_t i) -> uint4 {   // Q4_K: bsum, 8 x i16 per block
+    if constexpr (HEAD && OGM_HEAD_COHERENT_READS) return ldc16((const uint4 *)p.act.bsum + i);
+    else return ((const uint4 *)p.act.bsum)[i];
+  };
+  auto ld_sums16 = [&](uint32_t i) -> uint4 {   // Q6_K: per-16 sums narrowed to i16, groups 0..7 / 8..15 of a block
+    const int4 *src = (const int4 *)(p.act.sums + (size_t)(i >> 1) * 16 + (i & 1u) * 8);
+    uint4 a, b;
+    if constexpr (HEAD && OGM_HEAD_COHERENT_READS) { a = ldc16(src); b = ldc16(src + 1); }
+    else { const int4 a_ = src[0], b_ = src[1]; a = make_uint4(a_.x, a_.y, a_.z, a_.w); b = make_uint4(b_.x, b_.y, b_.z, b_.w); }
+    uint4 o;
+    o.x = (a.x & 0xFFFFu) | (a.y << 16);
+    o.y = (a.z & 0xFFFFu) | (a.w << 16);
+    o.z = (b.x & 0xFFFFu) | (b.y << 16);
+    o.w = (b.z & 0xFFFFu) | (b.w << 16);
+    return o;
+  };
+  auto ld_d = [&](uint32_t i) -> float {
+    if constexpr (HEAD && OGM_HEAD_COHERENT_READS) return ldc4f(p.act.d + i);
+    else return p.act.d[i];
+  };
+  auto stage_loads = [&]() {
+    st0 = ld_q(min(tid, n_xq - 1));
+    st1 = ld_q(min(tid + nthr, n_xq - 1));
+    st2 = ld_q(min(tid + 2 * nthr, n_xq - 1));
+    st3 = ld_q(min(tid + 3 * nthr, n_xq - 1));
+    if (F::AUX16 == 1) st_aux = ld_bsum(min(tid, n_aux - 1));
+    else if (F::AUX16 == 2) st_aux = ld_sums16(min(tid, n_aux - 1));
+    st_d = ld_d(min(tid, n_d - 1));
+  };
   if constexpr (QUANT) {
     xs0 = xload(0); xs1 = xload(1); xs2 = xload(2); xs3 = xload(3);
     if constexpr (QPEEL == 8) { xs4 = xload(4); xs5 = xload(5); xs6 = xload(6); xs7 = xload(7); }
-  } else {
-    st0 = gq[min(tid, n_xq - 1)];
-    st1 = gq[min(tid + nthr, n_xq - 1)];
-    st2 = gq[min(tid + 2 * nthr, n_xq - 1)];
-    st3 = gq[min(tid + 3 * nthr, n_xq - 1)];
-    if (F::AUX16 == 1) {
-      st_aux = ((const uint4 *)p.act.bsum)[min(tid, n_aux - 1)];  // Q4_K: bsum, 8 x i16 per block
-    } else if (F::AUX16 == 2) {
-      // Q6_K: per-16 sums narrowed to i16, groups 0..7 / 8..15 of a block
-      const uint32_t i = min(tid, n_aux - 1);
-      const int4 *src = (const int4 *)(p.act.sums + (size_t)(i >> 1) * 16 + (i & 1u) * 8);
-      const int4 a = src[0], b = src[1];
-      st_aux.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
-      st_aux.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
-      st_aux.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
-      st_aux.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
-    }
-    st_d = p.act.d[min(tid, n_d - 1)];
+  } else if constexpr (!HEAD) {
+    stage_loads();
   }
 
   // Keeps every staging load of the workgroup ahead of every weight load in the CU's
   // memory pipeline (no data is waited for here).
   __syncthreads();
 
+  if constexpr (HEAD) {
+    // the producers' few loads go out ahead of the launch's weight stream, not behind it
+    for (uint32_t i = 0; i < p.head.delay; i++) __builtin_amdgcn_s_sleep(1);
+  }
   // ---- ... then this wave's first tile of weights (the long pole) ...
   const uint32_t r_local = lane & (R - 1), c_local = lane / R;
   uint32_t it = wave;  // every wave has at least one item: n_wave <= nct <= n_items
@@ -1009,6 +1081,24 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP) ? F::MAX_THREA
   // Nothing below may be scheduled above the weight loads: work on the activations would
   // otherwise wait for them first and hold the weight loads back by a memory round trip.
   __builtin_amdgcn_sched_barrier(0);
+
+  if constexpr (HEAD) {
+    // ---- the producers' flag, polled by one lane behind the weight loads; then the activations
+    if (tid == 0) {
+      const uint32_t limit = p.head.spin_limit ? p.head.spin_limit : OGM_HEAD_SPIN_DEFAULT;
+      const uint32_t *mine = p.head.flag + (bid % OGM_HEAD_FLAG_COPIES) * 32u;
+      uint32_t polls = 0;
+      while ((int32_t)(__hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - p.head.epoch) < 0) {
+        if (++polls >= limit) {   // gives up, says so, and lets every wave end
+          __hip_atomic_store(p.head.flag + OGM_HEAD_FLAG_COPIES * 32u + 1u, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+    }
+    __syncthreads();
+    stage_loads();
+  }
 
   // ---- ... and park the activations in LDS while the weights are in flight.
   // q is permuted so that chunk c of block `col` lands at [c*upr + col].
@@ -1047,25 +1137,18 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP) ? F::MAX_THREA
     for (uint32_t i = tid + OGM_STAGE_PEEL * nthr; i < n_xq; i += nthr) {
       const uint32_t t = i / xch, ch = i - t * xch;
       const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
-      l_xq[(size_t)t * xch + c * upr + col] = gq[i];
+      l_xq[(size_t)t * xch + c * upr + col] = ld_q(i);
     }
     if (F::AUX16 == 1) {
-      for (uint32_t i = tid + nthr; i < n_aux; i += nthr) l_aux[i] = ((const uint4 *)p.act.bsum)[i];
+      for (uint32_t i = tid + nthr; i < n_aux; i += nthr) l_aux[i] = ld_bsum(i);
     } else if (F::AUX16 == 2) {
       for (uint32_t i = tid + nthr; i < n_aux; i += nthr) {
         const uint32_t blk = i >> 1, k = i & 1u;
         const uint32_t t = blk / upr, col = blk - t * upr;
-        const int4 *src = (const int4 *)(p.act.sums + (size_t)blk * 16 + k * 8);
-        const int4 a = src[0], b = src[1];
-        uint4 o;
-        o.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
-        o.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
-        o.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
-        o.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
-        l_aux[(size_t)t * upr * 2 + k * upr + col] = o;
+        l_aux[(size_t)t * upr * 2 + k * upr + col] = ld_sums16(i);
       }
     }
-    for (uint32_t i = tid + nthr; i < n_d; i += nthr) l_d[i] = p.act.d[i];
+    for (uint32_t i = tid + nthr; i < n_d; i += nthr) l_d[i] = ld_d(i);
   }
   __syncthreads();
 
@@ -1239,8 +1322,35 @@ uint32_t ogm_gemv_norm_tail_max(uint32_t ggml_type, uint32_t in_dim, uint32_t ou
   return 1024u * pick_waves(tl.nct, wg_waves, max_threads);
 }
 
+uint32_t ogm_gemv_head_waves(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves) {
+  int max_threads;
+  switch (ggml_type) {
+    case OGM_Q4_K: max_threads = FmtQ4K::MAX_THREADS; break;
+    case OGM_Q5_K: max_threads = FmtQ5K::MAX_THREADS; break;
+    case OGM_Q3_K: max_threads = FmtQ3K::MAX_THREADS; break;
+    case OGM_Q6_K: max_threads = FmtQ6K::MAX_THREADS; break;
+    case OGM_IQ4_XS: max_threads = FmtIQ4XS::MAX_THREADS; break;
+    case OGM_Q2_K: max_threads = FmtQ2K::MAX_THREADS; break;
+    default: return 0;
+  }
+  if (in_dim == 0 || in_dim % 256u != 0) return 0;
+  const OgmTiling tl = ogm_tiling_for(in_dim / 256u, out_dim);
+  return pick_waves(tl.nct, wg_waves, max_threads);
+}
+
 template <class F, bool QUANT>
 static void launch_single(const GemvParams &p, dim3 g, dim3 b, size_t lds, hipStream_t stream) {
+  if constexpr (!QUANT && F::ELEMS == 256 && F::ACT_GROUP == 256) {
+    if (p.head.kind != OGM_HEAD_NONE) {
+      if (p.upr == 16)
+        hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false, false, false, false, true>), g, b, lds, stream, p);
+      else if (p.upr == 56)
+        hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false, false, false, false, true>), g, b, lds, stream, p);
+      else
+        hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false, false, false, false, true>), g, b, lds, stream, p);
+      return;
+    }
+  }
   if constexpr (!QUANT && F::ELEMS == 256) {
     if (p.tail.kind != OGM_TAIL_NONE) {
       if (p.upr == 16)
@@ -1281,6 +1391,14 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
         a.tail.n == 0 || a.tail.n % 32u != 0)
       return hipErrorInvalidValue;
   }
+  p.head = a.head;
+  if (a.head.kind != OGM_HEAD_NONE) {
+    const bool ptrs_ok = a.head.kind == OGM_HEAD_NORM ? (a.head.x && a.head.weight)
+                         : a.head.kind == OGM_HEAD_SWIGLU ? (a.head.gate && a.head.up) : false;
+    if (!ptrs_ok || F::ELEMS != 256 || F::ACT_GROUP != 256 || a.n_tokens != 1 || GEMM_ORDER || dump || a.x_f32 ||
+        a.tail.kind != OGM_TAIL_NONE || !a.head.flag || a.in_dim % 256u != 0)
+      return hipErrorInvalidValue;
+  }
   p.dump_isum = a.dump_isum;
   p.dump_imin = a.dump_imin;
   p.in_dim = a.in_dim;
@@ -1318,13 +1436,20 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   if (lds > OGM_LDS_BUDGET) return hipErrorInvalidValue;
   // the plain single-token kernels of most formats need well under 128 registers and are built for up
   // to sixteen waves
-  const bool plain_single = a.n_tokens == 1 && !GEMM_ORDER && !dump && !a.x_f32 && a.tail.kind == OGM_TAIL_NONE;
+  const bool plain_single = a.n_tokens == 1 && !GEMM_ORDER && !dump && !a.x_f32 && a.tail.kind == OGM_TAIL_NONE &&
+                            a.head.kind == OGM_HEAD_NONE;
   // the per-32 formats' tiles are small (2 KB of Q8_0): sixteen of them per workgroup measure 7 %
   // faster than eight at 4096 x 4096
   const uint32_t waves = pick_waves(tl.nct, a.wg_waves, plain_single ? F::MAX_THREADS_SINGLE : F::MAX_THREADS,
                                     (plain_single && F::ELEMS == 32) ? 16u : 8u);
   if (a.tail.kind == OGM_TAIL_NORM && a.tail.n > 1024u * waves) return hipErrorInvalidValue;
-  const dim3 g(n_wg), b(waves * 64);
+  if (a.head.kind == OGM_HEAD_NORM) {
+    if (a.in_dim > 1024u * waves) return hipErrorInvalidValue;
+    p.head.n_prod = 1;
+  } else if (a.head.kind == OGM_HEAD_SWIGLU) {
+    p.head.n_prod = (a.in_dim / 256u + waves - 1u) / waves;
+  }
+  const dim3 g(n_wg + p.head.n_prod), b(waves * 64);
   if (dump) {
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true, false>), g, b, lds, stream, p);
   } else if (a.n_tokens == 1 && !GEMM_ORDER) {

@@ -47,9 +47,18 @@ __device__ __forceinline__ uint32_t ogm_quantize4(const float4 &v, float &scale,
          ((uint32_t)(q3 & 0xFF) << 24);
 }
 
+// A store that workgroups of the same kernel on other compute dies may read (with a device-coherent
+// load) once this wave's stores are acknowledged: it goes through to the level all dies share.
+template <bool COHERENT, class T>
+__device__ __forceinline__ void ogm_st(T *p, T v) {
+  if constexpr (COHERENT) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *p = v;
+}
+
 // Quantizes and stores one lane's share of a 256-run whose first element is e0 (= 256*run +
 // 4*lane) of token-major activations with row length in_dim; t_off* are the token's offsets.
-template <int GROUP>
+// COHERENT_OUT: the stores are for other workgroups of the same kernel (ogm_st).
+template <int GROUP, bool COHERENT_OUT = false>
 __device__ __forceinline__ void ogm_quantize_store(const float4 &v, uint32_t e0, bool active, uint32_t lane,
                                                    int8_t *q, float *d, int32_t *sums, int16_t *bsum,
                                                    uint16_t *bs16) {
@@ -57,18 +66,18 @@ __device__ __forceinline__ void ogm_quantize_store(const float4 &v, uint32_t e0,
   int s16, s32;
   const uint32_t packed = ogm_quantize4<GROUP>(v, scale, s16, s32);
   if (active) {
-    *(uint32_t *)(q + e0) = packed;
-    if ((lane & 3u) == 0) sums[e0 / 16] = s16;
+    ogm_st<COHERENT_OUT>((uint32_t *)(q + e0), packed);
+    if ((lane & 3u) == 0) ogm_st<COHERENT_OUT>(sums + e0 / 16, (int32_t)s16);
     if ((lane & 7u) == 0) {
-      bsum[e0 / 32] = (int16_t)s32;
+      ogm_st<COHERENT_OUT>(bsum + e0 / 32, (int16_t)s32);
       if (GROUP == 256 && bs16 != nullptr) {
         // |s32| <= 32 * 127: floor(s32 / 64) and s32 mod 64 are exact in f16
         uint16_t *b = bs16 + (e0 / 256u) * 16u + ((e0 / 32u) & 7u);
-        b[0] = __half_as_ushort(__float2half_rn((float)(s32 >> 6)));
-        b[8] = __half_as_ushort(__float2half_rn((float)(s32 & 63)));
+        ogm_st<COHERENT_OUT>(b, __half_as_ushort(__float2half_rn((float)(s32 >> 6))));
+        ogm_st<COHERENT_OUT>(b + 8, __half_as_ushort(__float2half_rn((float)(s32 & 63))));
       }
     }
-    if ((lane & (GROUP / 4 - 1)) == 0) d[e0 / GROUP] = scale;
+    if ((lane & (GROUP / 4 - 1)) == 0) ogm_st<COHERENT_OUT>(d + e0 / GROUP, scale);
   }
 }
 
@@ -88,8 +97,9 @@ __device__ __forceinline__ float4 ogm_ld4(const float *p) {
 // Residual add, RMSNorm and quantization of one row by one workgroup of n_wave waves (n <= 1024 *
 // n_wave): wave w owns the 256-runs w, w + n_wave, ... (at most four), lane l their elements
 // 4l..4l+3, kept in registers between the two passes.  red: 64 floats of LDS.  COHERENT_DELTA:
-// delta was written by other workgroups of the calling kernel.
-template <int GROUP, bool COHERENT_DELTA>
+// delta was written by other workgroups of the calling kernel.  COHERENT_OUT: the quantized row is
+// for other workgroups of the calling kernel.
+template <int GROUP, bool COHERENT_DELTA, bool COHERENT_OUT = false>
 __device__ __forceinline__ void ogm_norm_quant_row(float *__restrict__ x, const float *__restrict__ delta,
                                                    const float *__restrict__ weight, uint32_t n, float eps,
                                                    float *__restrict__ normed, const OgmActDev &act,
@@ -141,12 +151,13 @@ __device__ __forceinline__ void ogm_norm_quant_row(float *__restrict__ x, const 
       if (normed) *(float4 *)(normed + e0) = o;
     }
     if ((wave + k * n_wave) * 256u < n)  // wave-uniform: the run exists
-      ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
+      ogm_quantize_store<GROUP, COHERENT_OUT>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
   }
 }
 
-// SwiGLU and quantization of one 256-run by one wave: h = silu(gate) * up.
-template <int GROUP, bool COHERENT>
+// SwiGLU and quantization of one 256-run by one wave: h = silu(gate) * up.  COHERENT: gate and up were
+// written by other workgroups of the calling kernel; COHERENT_OUT: the quantized run is for them.
+template <int GROUP, bool COHERENT, bool COHERENT_OUT = false>
 __device__ __forceinline__ void ogm_swiglu_quant_run(const float *__restrict__ gate, const float *__restrict__ up,
                                                      uint32_t n, float *__restrict__ h, const OgmActDev &act,
                                                      uint32_t run, uint32_t lane) {
@@ -161,5 +172,5 @@ __device__ __forceinline__ void ogm_swiglu_quant_run(const float *__restrict__ g
     o.w = g.w / (1.0f + expf(-g.w)) * u.w;
     if (h) *(float4 *)(h + e0) = o;
   }
-  ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
+  ogm_quantize_store<GROUP, COHERENT_OUT>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
 }
