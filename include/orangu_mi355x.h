@@ -268,7 +268,7 @@ int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_
  * through run_layers at n_tokens > 1 (llama.rs:594-932): the matmuls in the GEMM kernels' float order
  * (Backend::matmul, cpu.rs:445-458), K/V rows appended to the cache, causal attention; then the last
  * row alone through the output norm and projection (forward, llama.rs:1007-1032).  last_logits
- * ([n_vocab]) and argmax may each be null.  Runs in chunks of 1024 tokens; synchronizes. */
+ * ([n_vocab]) and argmax may each be null.  Runs in passes of up to 2048 tokens (tuning key prefill_chunk_tokens); synchronizes. */
 int ogm_llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos0, uint32_t n_tokens,
                       float *last_logits, uint32_t *argmax);
 /* The same from token ids (host), their embedding rows read on the device from an uploaded
@@ -402,6 +402,9 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
  * the quantizer kernel first; 0 or -1 = default, off);
+ * "prefill_chunk_tokens" (tokens per pass of ogm_llama_prefill over the layers, default 2048; a model keeps
+ * the value of its first prefill, whose row buffers are allocated for it; 8B shapes: 2048 tokens 45.3 against
+ * 49.0 ms with 1024, a pass of 4096 is slower again);
  * "decode_fuse_heads" (1: the decode step's attention norm, FFN norm and SwiGLU run at the head of the GEMV
  * launch after them -- extra workgroups at the front of the launch, a flag, the others waiting behind their first
  * weight loads -- instead of as kernels of their own; same bits, measured slower, off by default; with it

@@ -67,6 +67,7 @@ struct ogm_ctx {
   int tune_decode_fuse_heads = 0;      // 1: the decode step's norms and SwiGLU at the head of the GEMV after them
   int tune_decode_head_delay = 64;     // fused heads: what the waiting workgroups sleep before their weight loads, x 64 clocks
   int tune_decode_head_spin = 0;       // fused heads: polls before a waiting workgroup gives up (0 = default)
+  int tune_prefill_chunk = 2048;       // tokens per prefill pass over the layers (fixed per model at its first prefill)
   int tune_decode_fuse_tails = 0;      // 1: the decode step's norms and SwiGLU inside the GEMV before them (slower)
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
@@ -306,6 +307,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "decode_head_delay") == 0) {
     if (value < 0 || value > 1000) return fail(ctx, OGM_ERR_INVALID, "decode_head_delay must be 0..1000");
     ctx->tune_decode_head_delay = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "prefill_chunk_tokens") == 0) {
+    if (value < 1 || value > 16384) return fail(ctx, OGM_ERR_INVALID, "prefill_chunk_tokens must be 1..16384");
+    ctx->tune_prefill_chunk = value;
     return OGM_OK;
   }
   if (strcmp(key, "decode_fuse_tails") == 0) {
@@ -1096,13 +1102,14 @@ struct ogm_llama {
   uint32_t *amax_scratch = nullptr, *amax_out = nullptr;
   float *stage = nullptr;     // host->device staging for ogm_llama_kv_write
   size_t stage_cap = 0;
-  // prefill rows, allocated at the first prefill for OGM_PREFILL_CHUNK tokens
+  // prefill rows, allocated at the first prefill for the pass size of that moment (prefill_chunk_tokens)
   struct Prefill {
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
     float *proj = nullptr, *gate = nullptr, *up = nullptr, *cs = nullptr;
     float *part_o = nullptr, *part_ml = nullptr;   // attn_prefill_variant 1 only, allocated when it first runs
     uint32_t *tokens = nullptr;
     uint32_t attn_tokens = 0;   // query rows one attention launch takes (bounded by part_o)
+    uint32_t chunk = 0;         // tokens per pass over the layers: what the rows above were allocated for
     bool ready = false;
   } pf;
   uint32_t max_splits = 0;
@@ -1679,13 +1686,13 @@ extern "C" int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
 
 // ---- prefill: run_layers at n_tokens > 1 (llama.rs:594-932) ------------------------------------
 
-static const uint32_t OGM_PREFILL_CHUNK = 1024;            // tokens per pass over the layers
 static const size_t OGM_PREFILL_PART_BYTES = 256u << 20;   // attention partials per launch
 
 static int llama_prefill_buffers(ogm_ctx *ctx, ogm_llama *m) {
   if (m->pf.ready) return OGM_OK;
   const ogm_llama_config &c = m->cfg;
-  const size_t T = OGM_PREFILL_CHUNK, qd = (size_t)c.n_head * c.head_dim, kvd = (size_t)c.n_head_kv * c.head_dim;
+  m->pf.chunk = (uint32_t)ctx->tune_prefill_chunk;
+  const size_t T = m->pf.chunk, qd = (size_t)c.n_head * c.head_dim, kvd = (size_t)c.n_head_kv * c.head_dim;
   int rc = OGM_OK;
   auto A = [&](float **p, size_t n) { if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)p, n * 4); };
   A(&m->pf.x, T * c.n_embd);
@@ -1711,7 +1718,7 @@ static int llama_prefill_partials(ogm_ctx *ctx, ogm_llama *m) {
   const size_t per_token = (size_t)c.n_head * m->max_splits * c.head_dim * 4;
   size_t at = OGM_PREFILL_PART_BYTES / per_token;
   if (at < 1) at = 1;
-  if (at > OGM_PREFILL_CHUNK) at = OGM_PREFILL_CHUNK;
+  if (at > m->pf.chunk) at = m->pf.chunk;
   int rc = llama_alloc(ctx, m, (void **)&m->pf.part_o, at * per_token);
   if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)&m->pf.part_ml, at * (size_t)c.n_head * m->max_splits * 2 * 4);
   if (rc != OGM_OK) return rc;
@@ -1788,7 +1795,7 @@ static int llama_norm_matmul_rows(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
   return OGM_OK;
 }
 
-// One chunk of T <= OGM_PREFILL_CHUNK tokens whose embedding rows sit in m->pf.x.  With `last`,
+// One chunk of T <= m->pf.chunk tokens whose embedding rows sit in m->pf.x.  With `last`,
 // the final row's hidden state ends in m->x and its logits in m->logits.
 static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32_t T, bool last, hipStream_t s) {
   const ogm_llama_config &c = m->cfg;
@@ -1868,8 +1875,8 @@ static int llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x_host, const 
   int rc = llama_prefill_buffers(ctx, m);
   if (rc != OGM_OK) return rc;
   hipStream_t s = ctx->stream;
-  for (uint32_t t0 = 0; t0 < n_tokens; t0 += OGM_PREFILL_CHUNK) {
-    const uint32_t T = n_tokens - t0 < OGM_PREFILL_CHUNK ? n_tokens - t0 : OGM_PREFILL_CHUNK;
+  for (uint32_t t0 = 0; t0 < n_tokens; t0 += m->pf.chunk) {
+    const uint32_t T = n_tokens - t0 < m->pf.chunk ? n_tokens - t0 : m->pf.chunk;
     if (tok_embd) {
       // the embedding rows (llama.rs:609-614), dequantized on the device
       HIPCHK(ctx, hipMemcpyAsync(m->pf.tokens, tokens + t0, (size_t)T * 4, hipMemcpyHostToDevice, s));

@@ -609,10 +609,12 @@ def test_prefill_across_attention_chunks_and_in_two_parts(be, hd, group, n_kv, p
 
 
 def test_prefill_longer_than_one_pass_and_from_token_ids(be):
-    """1100 tokens run as two passes over the layers (1024 + 76); from token ids the embedding rows
-    are dequantized on the device (llama.rs:609-614) and give the same bits as rows passed in."""
+    """1100 tokens run as two passes over the layers (1024 + 76, with the pass size set to 1024; it is fixed
+    at a model's first prefill); from token ids the embedding rows are dequantized on the device
+    (llama.rs:609-614) and give the same bits as rows passed in."""
     import oracle
     from orangu_amd import QuantMatrix
+    be.set_tuning("prefill_chunk_tokens", 1024)
     ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
                           types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=1152, seed=71, attn_norm_scale=TAME[Q4_K])
     embd_raw = synth_weights(Q6_K, 256, 320, seed=72)
@@ -629,6 +631,7 @@ def test_prefill_longer_than_one_pass_and_from_token_ids(be):
         with pytest.raises(OgmError):
             dev.prefill_tokens(QuantMatrix(embd_raw, Q6_K, 256, 320), np.array([5, 320], np.uint32), 0)   # no such token
     finally:
+        be.set_tuning("prefill_chunk_tokens", 2048)
         dev.close()
 
 
