@@ -380,7 +380,7 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * 8192 rows; 1 = never);
  * "gemm_few_tokens_min_rows" (2 to 16 tokens over a Q6_K matrix -- matmul and matmul_decode alike -- take
  * the kernel that streams the weights once and multiplies every token on the matrix cores when the matrix
- * has at least this many rows: 0 = default 65536, i.e. a vocabulary projection; 1 = whenever the shape
+ * has at least this many rows: 0 = default, 30000 rows (a vocabulary projection) and at least three tokens; 1 = whenever the shape
  * allows: in_dim a multiple of 1024 whose int8 rows fit LDS; -1 = never);
  * "gemm_sb_waves" (waves of a small-batch workgroup: 8 or 16; 0 = default, 16 for launches of at most
  * 256 workgroups over rows of at least 16 super-blocks);

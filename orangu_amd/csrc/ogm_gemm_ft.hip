@@ -213,17 +213,19 @@ __global__ __launch_bounds__(64 * FT_WAVES) void ogm_gemm_ft_q6k_kernel(GemmFtPa
   }
 }
 
-// Shapes the kernel takes: Q6_K rows of a multiple of four super-blocks (tiles of 16 rows), an even
-// count of at least two; 2 to 16 tokens whose int8 rows fit LDS; and enough rows that every compute
-// unit gets `min_waves_per_cu` waves of 32 (0: the default, 8), since a wave streams its rows alone,
-// two super-blocks in flight.
+// Shapes the kernel takes: Q6_K rows of a multiple of four super-blocks (tiles of 16 rows); 2 to 16
+// tokens whose int8 rows fit LDS; and at least min_rows rows, since a wave streams its 32 rows alone,
+// two super-blocks in flight, and the launch needs a few waves per SIMD.  min_rows 0, the default
+// rule: from 30000 rows (a 32000-row vocabulary: 25 us at 4 tokens against 29 us token by token, 26
+// against 34 at 8; at 14336 rows the other kernels win, 18 against 22) and from three tokens (at two
+// the GEMV kernel is level or ahead).
 bool ogm_gemm_ft_eligible(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens,
                           uint32_t min_rows) {
   if (ggml_type != OGM_Q6_K || in_dim == 0 || in_dim % 1024u != 0 || n_tokens < 2u || n_tokens > 16u) return false;
   const uint32_t tp = n_tokens <= 8u ? 8u : 16u;
   if ((size_t)in_dim * tp + (size_t)(in_dim / 256u) * tp * 4u > 160u * 1024u) return false;
   if ((uint64_t)n_tokens * in_dim >= (1ull << 31)) return false;
-  return out_dim >= (min_rows ? min_rows : 65536u);
+  return min_rows ? out_dim >= min_rows : (out_dim >= 30000u && n_tokens >= 3u);
 }
 
 hipError_t ogm_launch_gemm_ft(const OgmGemmArgs &a, int gemm_order, hipStream_t stream, const char **kernel_name) {

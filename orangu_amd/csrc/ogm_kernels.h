@@ -155,7 +155,8 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
 
 // 2 to 16 tokens over a Q6_K matrix of many rows (ogm_gemm_ft.hip): every wave streams 32 rows once and
 // multiplies them with all tokens on the matrix cores.  Reads a.wt, a.act.q, a.act.d; writes a.y.
-// gemm_order as OgmGemvArgs.  min_rows: fewest rows from which it is taken (0: the default).
+// gemm_order as OgmGemvArgs.  min_rows: fewest rows from which it is taken (0: the default rule, 30000
+// rows and three tokens).
 bool ogm_gemm_ft_eligible(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens,
                           uint32_t min_rows);
 hipError_t ogm_launch_gemm_ft(const OgmGemmArgs &a, int gemm_order, hipStream_t stream, const char **kernel_name);

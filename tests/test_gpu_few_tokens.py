@@ -114,8 +114,8 @@ def test_grouped_calls_and_other_types_keep_their_kernels(be):
 
 
 def test_default_routing_takes_it_for_the_vocabulary_projection_only():
-    """Without the tuning key: 4096 -> 128256 at 2 to 16 tokens runs the kernel, 4096 -> 14336 does not; and the
-    full-size results are bit-exact in both orders (checked on a sample of rows against the oracle over the same
+    """Without the tuning key: 4096 -> 128256 and 4096 -> 32000 at 3 to 16 tokens run the kernel, two tokens and
+    4096 -> 14336 do not; and the full-size results are bit-exact in both orders (checked on a sample of rows against the oracle over the same
     rows as a smaller matrix -- a row's result does not depend on the others)."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
@@ -126,15 +126,20 @@ def test_default_routing_takes_it_for_the_vocabulary_projection_only():
         rb = row_bytes(Q6_K, in_dim)
         rows = np.r_[0:40, 64000:64040, out_dim - 40:out_dim]
         sub = np.ascontiguousarray(raw.reshape(out_dim, rb)[rows]).reshape(-1)
-        for T in (2, 4, 8, 16):
+        for T in (2, 3, 4, 8, 16):
             x = synth_x(T, in_dim, seed=T)
             say("vocabulary projection", T)
             got = b.matmul(x, T, w).reshape(T, out_dim)
-            assert b.last_kernel() == kernel_for(T), b.last_kernel()
+            assert (b.last_kernel() == kernel_for(T)) == (T >= 3), b.last_kernel()
             assert_bits(got[:, rows], oracle.matmul(Q6_K, sub, in_dim, len(rows), x, T), f"matmul {T}")
             got = b.matmul_decode(x, T, w).reshape(T, out_dim)
-            assert b.last_kernel() == kernel_for(T), b.last_kernel()
+            assert (b.last_kernel() == kernel_for(T)) == (T >= 3), b.last_kernel()
             assert_bits(got[:, rows], oracle.matmul_decode(Q6_K, sub, in_dim, len(rows), x, T), f"decode {T}")
+        w32 = qm(raw[:rb * 32000], Q6_K, in_dim, 32000)
+        x = synth_x(4, in_dim, seed=2)
+        got = b.matmul(x, 4, w32)
+        assert b.last_kernel() == kernel_for(4), b.last_kernel()
+        assert_bits(np.asarray(got).reshape(4, 32000)[:, :40], oracle.matmul(Q6_K, sub[:rb * 40], in_dim, 40, x, 4), "32000 rows")
         small = qm(synth_weights(Q6_K, 4096, 14336, seed=4), Q6_K, 4096, 14336)
         b.matmul(synth_x(4, 4096, seed=1), 4, small)
         assert not b.last_kernel().startswith("ogm_gemm_ft"), b.last_kernel()
