@@ -1425,14 +1425,20 @@ __device__ __forceinline__ void gd_dma4(const uint8_t *src, uint8_t *lds_chunk) 
 // at 16 (32 lh + l32).  A chunk is then one contiguous load; fetched row by row it would be 32 pieces
 // of 32 distinct cache lines.  Tokens past the last repeat it (never stored).
 __global__ __launch_bounds__(256) void ogm_gemm_xtile_kernel(const int8_t *__restrict__ xq, int8_t *__restrict__ xt,
-                                                             uint32_t in_dim, uint32_t n_tokens, uint32_t n_pieces) {
-  // thread = one 16-byte piece, pieces of a token consecutive: whole rows are read in order
-  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-  if (i >= n_pieces) return;
-  const uint32_t ppr = in_dim / 16u, tok = i / ppr, c = i - tok * ppr;
-  const uint4 v = *(const uint4 *)(xq + (size_t)min(tok, n_tokens - 1u) * in_dim + 16u * c);
-  const uint32_t chunk = (tok >> 5) * (in_dim / 32u) + (c >> 1);
-  *(uint4 *)(xt + (size_t)chunk * 1024u + (32u * (c & 1u) + (tok & 31u)) * 16u) = v;
+                                                             uint32_t in_dim, uint32_t n_tokens) {
+  // workgroup = 32 tokens x 128 activations = four chunks: read as eight 16-byte pieces a token (whole
+  // 128-byte lines), turned through LDS (rows padded by a piece against bank conflicts), written as 4 KiB
+  // in a row
+  __shared__ uint4 tile[32][9];
+  const uint32_t tid = threadIdx.x, tb = blockIdx.y, k0 = blockIdx.x * 128u;
+  {
+    const uint32_t tok = min(tb * 32u + (tid >> 3), n_tokens - 1u), piece = tid & 7u;
+    tile[tid >> 3][piece] = *(const uint4 *)(xq + (size_t)tok * in_dim + k0 + 16u * piece);
+  }
+  __syncthreads();
+  const uint32_t step = tid >> 6, slot = tid & 63u;   // the chunk of the four, the lane of its operand
+  const uint4 v = tile[slot & 31u][2u * step + (slot >> 5)];
+  *(uint4 *)(xt + ((size_t)tb * (in_dim / 32u) + k0 / 32u + step) * 1024u + slot * 16u) = v;
 }
 
 #if GD_ABL_NOMFMA
@@ -3316,9 +3322,8 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     const bool dma = pre && gemm_dma_eligible(a);
     if (a.plane_kernel != 1u) pre = false;   // planes given, but not for the feeding-wave kernels
     if (dma) {
-      const uint32_t n_pieces = t_pad * (a.in_dim / 16u);
-      hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3((n_pieces + 255u) / 256u), dim3(256), 0, stream, a.act.q,
-                         (int8_t *)a.xh, a.in_dim, a.n_tokens, n_pieces);
+      hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3(a.in_dim / 128u, t_pad / 32u), dim3(256), 0, stream, a.act.q,
+                         (int8_t *)a.xh, a.in_dim, a.n_tokens);
       GemmDmaParams d;
       d.wt = a.wt;
       d.planes = a.planes;
