@@ -44,7 +44,9 @@ hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const f
                                  float eps, float *normed, OgmActDev act, hipStream_t stream, uint32_t n_rows) {
   if (n == 0 || n % 32u != 0 || n > 16384u || n_rows == 0) return hipErrorInvalidValue;
   const uint32_t runs = (n + 255u) / 256u;
-  const uint32_t waves = runs < 16u ? runs : 16u;
+  // few rows: a wave per run, the shortest chain; from 1024 rows (2048 rows: 2 % of a prefill): four runs per wave
+  // (the row's bits do not depend on it)
+  const uint32_t waves = n_rows >= 1024u ? (runs + 3u) / 4u : (runs < 16u ? runs : 16u);
   if (mode == 0)
     hipLaunchKernelGGL(ogm_norm_quant_kernel<32>, dim3(n_rows), dim3(waves * 64), 0, stream, x, delta, weight,
                        n, eps, normed, act);
