@@ -152,3 +152,20 @@ def test_dequantized_rows_match_the_cpu_dequantizer(be, t):
     rb = row_bytes(t, in_dim)
     want = np.stack([oracle.dequantize(t, raw[r * rb:(r + 1) * rb], in_dim) for r in range(3, 23)])
     assert_bits(got, want, "dequantized rows")
+
+
+def test_q5_1_min_term_is_added_not_subtracted_on_the_device(be):
+    """vecdot.rs:4195-4218 through the device: d = 0, m = 2.5 makes every weight 2.5; one token, a decode batch and
+    matmul of several tokens give 2.5 * sum(x_q) * scale_x, bit for bit what the CPU restatement gives."""
+    block = np.concatenate([np.frombuffer(np.float16(0.0).tobytes(), np.uint8), np.frombuffer(np.float16(2.5).tobytes(), np.uint8),
+                            np.zeros(4, np.uint8), np.zeros(16, np.uint8)])
+    raw = np.tile(block, 4 * 3)   # three rows of four blocks
+    w = qm(raw, Q5_1, 128, 3)
+    x = np.concatenate([activations_t(128, k) for k in range(3)])
+    one = be.matmul(x[:128], 1, w)
+    q, d, _ = oracle.quantize_act(x[:128])
+    known = float(sum(np.float64(2.5) * d[b] * q[32 * b:32 * b + 32].astype(np.int64).sum() for b in range(4)))
+    assert np.allclose(np.asarray(one, np.float64), known, rtol=1e-5, atol=1e-6), (one, known)
+    assert_bits(one, oracle.matmul(Q5_1, raw, 128, 3, x[:128], 1), "one token")
+    assert_bits(be.matmul_decode(x, 3, w), oracle.matmul_decode(Q5_1, raw, 128, 3, x, 3), "decode batch")
+    assert_bits(be.matmul(x, 3, w), oracle.matmul(Q5_1, raw, 128, 3, x, 3), "several tokens")

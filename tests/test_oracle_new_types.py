@@ -226,3 +226,19 @@ def test_scalar_and_vector_builds_agree_on_the_new_types():
             oracle.force_scalar(False)
         for u, v in zip(a, b):
             assert np.array_equal(u.view(np.uint32), v.view(np.uint32))
+
+
+def test_q5_1_min_term_is_added_not_subtracted():
+    """vecdot.rs:4195-4218: with d = 0 the quantized term vanishes and every weight is exactly m = 2.5 -- a sign
+    slip would bias every weight by 2m.  The fused dot of that block against x is then 2.5 * sum(q_x) * scale_x, and
+    through matmul at several tokens (the rows-unpacked-once path, where the min enters as -2.5) the same value."""
+    block = np.concatenate([np.frombuffer(np.float16(0.0).tobytes(), np.uint8), np.frombuffer(np.float16(2.5).tobytes(), np.uint8),
+                            np.zeros(4, np.uint8), np.zeros(16, np.uint8)])
+    assert np.all(np.abs(oracle.dequantize(Q5_1, block, 32) - 2.5) < 1e-6)
+    x = activations(32)
+    q, d, _ = oracle.quantize_act(x)
+    want = f(2.5) * d[0] * f(q.astype(np.int64).sum())
+    got1 = oracle.matmul(Q5_1, block, 32, 1, x, 1)[0]
+    assert abs(got1 - want) <= 1e-6 * max(1.0, abs(want)), (got1, want)
+    got3 = oracle.matmul(Q5_1, block, 32, 1, np.concatenate([x, x, x]), 3).reshape(-1)
+    assert np.all(np.abs(got3 - want) <= 1e-5 * max(1.0, abs(want))), (got3, want)
