@@ -1389,7 +1389,9 @@ struct GemmDmaParams {
 #ifndef GD_ABL_NOLDS
 #define GD_ABL_NOLDS 0
 #endif
+#ifndef GD_RING
 #define GD_RING 6u
+#endif
 #define GD_AHEAD (GD_RING - 1u)        // steps fetched ahead of the one multiplied
 #define GD_XOFF (GD_NW * 2048u)        // activations of a step, after the weights' 2 KiB per wave
 #define GD_SLOT (GD_XOFF + 4096u)      // bytes of a step in LDS (one-plane types leave half the weights' part unused)
