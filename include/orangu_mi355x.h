@@ -402,6 +402,9 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
  * the quantizer kernel first; 0 or -1 = default, off);
+ * "attn_decode_share" (decode attention: 1 = default, one workgroup per K/V head and chunk of the cache; 2 = the
+ * query heads of a K/V head split over two workgroups where four or eight of them allow it: twice the
+ * workgroups, measured 2 us a layer slower at 2048 cached positions; results agree to f32 rounding);
  * "prefill_chunk_tokens" (tokens per pass of ogm_llama_prefill over the layers, default 2048; a model keeps
  * the value of its first prefill, whose row buffers are allocated for it; 8B shapes: 2048 tokens 45.3 against
  * 49.0 ms with 1024, a pass of 4096 is slower again);

@@ -67,6 +67,7 @@ struct ogm_ctx {
   int tune_decode_fuse_heads = 0;      // 1: the decode step's norms and SwiGLU at the head of the GEMV after them
   int tune_decode_head_delay = 64;     // fused heads: what the waiting workgroups sleep before their weight loads, x 64 clocks
   int tune_decode_head_spin = 0;       // fused heads: polls before a waiting workgroup gives up (0 = default)
+  int tune_attn_decode_share = 1;      // decode attention: 2 splits a K/V head's query heads over two workgroups where possible (slower), 1 never
   int tune_prefill_chunk = 2048;       // tokens per prefill pass over the layers (fixed per model at its first prefill)
   int tune_decode_fuse_tails = 0;      // 1: the decode step's norms and SwiGLU inside the GEMV before them (slower)
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
@@ -307,6 +308,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "decode_head_delay") == 0) {
     if (value < 0 || value > 1000) return fail(ctx, OGM_ERR_INVALID, "decode_head_delay must be 0..1000");
     ctx->tune_decode_head_delay = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "attn_decode_share") == 0) {
+    if (value < 1 || value > 2) return fail(ctx, OGM_ERR_INVALID, "attn_decode_share must be 1 or 2");
+    ctx->tune_attn_decode_share = value;
     return OGM_OK;
   }
   if (strcmp(key, "prefill_chunk_tokens") == 0) {
@@ -1090,7 +1096,7 @@ struct ogm_llama {
   float *freq = nullptr;      // [rope_dim / 2], frequency factors applied
   float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
   uint32_t head_epoch = 0;            // value of the GEMV heads' flag (the three words after the tickets) after the last launch
-  uint32_t *attn_tickets = nullptr;   // [n_head_kv + OGM_TAIL_TICKETS], zero between launches; the last ones are the GEMV tails'
+  uint32_t *attn_tickets = nullptr;   // [2 n_head_kv] the attention kernel's, then the GEMV tails' tickets and the heads' flags; zero between launches
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
   void *v_cache = nullptr;
   float *x = nullptr;         // hidden state [n_embd]
@@ -1185,7 +1191,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   A((void **)&m->pre, (size_t)c.n_layer * pre_stride * 4);
   A((void **)&m->freq, (size_t)(c.rope_dim / 2 + 1) * 4);
   A((void **)&m->rope_cs, (size_t)(c.rope_dim / 2 + 1) * 8);
-  A((void **)&m->attn_tickets, ((size_t)c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);   // + the GEMV tails' tickets
+  A((void **)&m->attn_tickets, ((size_t)2 * c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);   // + the GEMV tails' tickets
   A(&m->k_cache, cache_bytes);
   A(&m->v_cache, cache_bytes);
   A((void **)&m->x, (size_t)c.n_embd * 4);
@@ -1238,7 +1244,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   hipError_t e = hipMemcpy(m->norms, host.data(), host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->pre, pre_host.data(), pre_host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, ((size_t)c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);
+  if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, ((size_t)2 * c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
   if (e != hipSuccess) {
@@ -1371,7 +1377,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   // polled, activations loaded) that costs what the kernel boundary it replaces costs, and the
   // producers' own loads queue behind the launch's weight stream.
   const bool heads = ctx->tune_decode_fuse_heads != 0 && !fuse && ctx->tune_fuse_quant <= 0;
-  uint32_t *head_flag = m->attn_tickets + ((c.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u);   // 128-byte aligned
+  uint32_t *head_flag = m->attn_tickets + ((2u * c.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u);   // 128-byte aligned
   auto head_ok = [&](const ogm_weight *first, int mode, bool norm) {   // first: the matrix of the group's first launch
     if (!heads || mode != OGM_ACT_PER_256) return false;
     const uint32_t waves = ogm_gemv_head_waves(first->ggml_type, first->in_dim, first->out_dim, (uint32_t)ctx->tune_wg_waves);
@@ -1422,7 +1428,8 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, m->rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
                                        c.n_head, c.n_head_kv, c.head_dim, scale, m->part_o, m->part_ml,
-                                       m->attn_tickets, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s));
+                                       m->attn_tickets, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s, 0u,
+                                       ctx->tune_attn_decode_share == 2 ? 0u : 1u));   // 0: wherever the shape allows
     const int mode_ff = act_mode_for(L.w_gate->ggml_type);
     if (act_mode_for(L.w_up->ggml_type) != mode_ff)
       return fail(ctx, OGM_ERR_UNSUPPORTED, "w_gate and w_up must share an activation mode");
@@ -1430,7 +1437,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     float *y1[1] = {m->proj};
     if ((rc = llama_capture(ctx, m, 4 * l + 1, qd, mode_o, s)) != OGM_OK) return rc;
     OgmGemvTail tail;
-    tail.ticket = m->attn_tickets + c.n_head_kv;
+    tail.ticket = m->attn_tickets + 2u * c.n_head_kv;
     bool ffn_head = false;
     if (tail_ok(L.wo, c.n_embd, mode_ff)) {
       tail.kind = OGM_TAIL_NORM;
@@ -1537,7 +1544,7 @@ extern "C" int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_d
 // (the step's results are then not to be trusted).  Clears the word.
 static int llama_check_heads(ogm_ctx *ctx, ogm_llama *m) {
   if (m->head_epoch == 0) return OGM_OK;   // no such launch yet
-  uint32_t *word = m->attn_tickets + ((m->cfg.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u) + OGM_HEAD_FLAG_COPIES * 32u + 1u;
+  uint32_t *word = m->attn_tickets + ((2u * m->cfg.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u) + OGM_HEAD_FLAG_COPIES * 32u + 1u;
   uint32_t gave_up = 0;
   HIPCHK(ctx, hipMemcpy(&gave_up, word, 4, hipMemcpyDeviceToHost));
   if (!gave_up) return OGM_OK;

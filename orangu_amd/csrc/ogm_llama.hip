@@ -200,7 +200,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
                                                        OgmAttnPre pre, uint32_t gq,
                                                        __half *__restrict__ kc, __half *__restrict__ vc,
                                                        uint32_t pos, uint32_t max_splits, uint32_t n_head_kv,
-                                                       float scale, float *part_o, float *part_ml,
+                                                       uint32_t kv_share, float scale, float *part_o, float *part_ml,
                                                        uint32_t *counters, float *__restrict__ attn_out,
                                                        OgmActDev act) {
   constexpr int NT = 4 * CHUNK, NW = NT / 64;   // four threads per cache position
@@ -220,7 +220,9 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
   __shared__ float mrg[GROUP != 0 ? 6 : 1][GROUP != 0 ? NT : 1];   // the final merge's slices
   static_assert(!PREFILL || GROUP == 0, "a prefill batch merges in its own launch");
   OGM_STAMP(0);
-  const uint32_t kvh = blockIdx.x, split = blockIdx.y;
+  // blockIdx.x: a group of gq query heads (G head slots) that share a K/V head; kv_share such groups
+  // per K/V head (1: all its query heads in one workgroup)
+  const uint32_t hg = blockIdx.x, split = blockIdx.y, kvh = hg / kv_share;
   if constexpr (PREFILL) {
     const uint32_t tok = blockIdx.z;
     pos += tok;
@@ -260,7 +262,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
     for (uint32_t i = tid; i < (uint32_t)(G * HD / 4); i += NT) {
       const uint32_t g = i / (HD / 4), d4 = i - g * (HD / 4);
       float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (g < gq) v4 = *(const float4 *)(q + ((size_t)kvh * gq + g) * HD + 4u * d4);
+      if (g < gq) v4 = *(const float4 *)(q + ((size_t)hg * gq + g) * HD + 4u * d4);
       *(float4 *)&qs[g][4u * d4] = v4;
     }
   } else {
@@ -269,7 +271,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
     for (uint32_t u = wave; u < n_units; u += NW) {
       const bool is_q = u < (uint32_t)G, is_v = u == (uint32_t)G + 1u;
       const bool live = !is_q || u < gq;
-      const size_t row = (is_q ? (size_t)kvh * gq + u : (size_t)kvh) * HD;
+      const size_t row = (is_q ? (size_t)hg * gq + u : (size_t)kvh) * HD;
       const float *src = (is_q ? q : is_v ? v_new : k_new) + row;
       const float *bias = is_q ? pre.q_bias : is_v ? pre.v_bias : pre.k_bias;
       const float *nw = is_q ? pre.q_norm : is_v ? nullptr : pre.k_norm;
@@ -418,7 +420,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
       m = fmaxf(m, red[0][tid][w]);
       l += red[1][tid][w];
     }
-    const uint32_t h = kvh * gq + tid;
+    const uint32_t h = hg * gq + tid;
     st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2], m);
     st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2 + 1], l);
   }
@@ -476,7 +478,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
       float t = 0.0f;
 #pragma unroll
       for (int w = 0; w < NW; w++) t += osum[w][g][d];
-      if (g < gq) st_one<GROUP != 0>(&part_o[((size_t)(kvh * gq + g) * max_splits + split) * HD + d], t);
+      if (g < gq) st_one<GROUP != 0>(&part_o[((size_t)(hg * gq + g) * max_splits + split) * HD + d], t);
     }
   }
 
@@ -490,10 +492,10 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
     OGM_STAMP(4);
     if (tid == 0) {
       const uint32_t ticket =
-          __hip_atomic_fetch_add(&counters[kvh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_fetch_add(&counters[hg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       s_last = ticket == n_splits - 1u;
       if (ticket == n_splits - 1u)
-        __hip_atomic_store(&counters[kvh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        __hip_atomic_store(&counters[hg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
     }
     __syncthreads();
     OGM_STAMP(5);
@@ -506,7 +508,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
     {
       const uint32_t eg = tid % NG, slice = tid / NG;
       const uint32_t el = 4u * eg;
-      const AttnPart pt = attn_merge_chunks<true>(part_o, part_ml, kvh * G + el / HD, el % HD, slice, NSL, n_splits,
+      const AttnPart pt = attn_merge_chunks<true>(part_o, part_ml, hg * G + el / HD, el % HD, slice, NSL, n_splits,
                                                   max_splits, HD);
       mrg[0][tid] = pt.m; mrg[1][tid] = pt.den;
       mrg[2][tid] = pt.o.x; mrg[3][tid] = pt.o.y; mrg[4][tid] = pt.o.z; mrg[5][tid] = pt.o.w;
@@ -517,7 +519,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
     for (int run = wave; run < RUNS; run += NW) {
       const uint32_t eg = run * 64u + lane;
       const bool active = eg < (uint32_t)NG;
-      const uint32_t e0 = kvh * (uint32_t)(G * HD) + 4u * eg;
+      const uint32_t e0 = hg * (uint32_t)(G * HD) + 4u * eg;
       float4 ov = make_float4(0.f, 0.f, 0.f, 0.f);
       if (active) {
         float M = mrg[0][eg];   // slice 0 always holds chunk 0
@@ -567,7 +569,7 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
                                   uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
                                   float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
-                                  hipStream_t stream, uint32_t chunk) {
+                                  hipStream_t stream, uint32_t chunk, uint32_t share) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0) return hipErrorInvalidValue;
   if (rope_dim > head_dim || rope_dim % 2u != 0) return hipErrorInvalidValue;
   // Cache positions per workgroup: 128; 64 only for short contexts.  The kernel is a chain of
@@ -582,9 +584,20 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
   if (n_splits > max_splits) return hipErrorInvalidValue;
   const uint32_t n = n_head * head_dim;
   if (n % 32u != 0) return hipErrorInvalidValue;
-  const dim3 grid(n_head_kv, n_splits);
-  const uint32_t gq = n_head / n_head_kv;
+  uint32_t gq = n_head / n_head_kv;
   if (gq > 8u) return hipErrorInvalidValue;
+  // Four or eight query heads per K/V head are split over two workgroups of half as many when those
+  // still fill whole quantizer groups (the merge stays in the kernel): twice the workgroups, each with
+  // half the scores, sums and merge, for reading the chunk's K and V rows twice out of L2 (both write
+  // the new cache row, with the same bits).  share: 0 this rule, 1 never, 2 asked for.  Measured on
+  // MI355X (32 query heads on 8 K/V heads, 2048 cached positions): 2 us a layer slower than one workgroup
+  // per K/V head -- the kernel is a chain of latencies, not of work -- so the decode step asks for 1.
+  const uint32_t group_ = mode == 0 ? 32u : 256u;
+  const bool can_share = (gq == 4u || gq == 8u) && ((gq / 2u) * head_dim) % group_ == 0;
+  if (share > 2u || (share == 2u && !can_share)) return hipErrorInvalidValue;
+  const uint32_t kv_share = (share == 0u ? can_share : share == 2u) ? 2u : 1u;
+  gq /= kv_share;
+  const dim3 grid(n_head_kv * kv_share, n_splits);
   const uint32_t G = gq <= 2u ? gq : (gq <= 4u ? 4u : 8u);   // head slots of the kernel
   const uint32_t group = mode == 0 ? 32u : 256u;
   // the merge rides in the attention kernel when every head slot is a head and a K/V head's
@@ -593,7 +606,7 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
 #define OGM_ATTN_LAUNCH_C(HD_, G_, GR_, CH_)                                                           \
   hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, GR_, false, CH_>), grid, dim3(4 * CH_), 0, stream, q, k_new, \
                      v_new, (const float2 *)cs, rope_dim / 2u, pre, gq, (__half *)k_cache_layer,        \
-                     (__half *)v_cache_layer, pos, max_splits, n_head_kv, scale, part_o, part_ml,       \
+                     (__half *)v_cache_layer, pos, max_splits, n_head_kv, kv_share, scale, part_o, part_ml, \
                      counters, attn_out, act)
 #define OGM_ATTN_LAUNCH(HD_, G_, GR_)                    \
   do {                                                   \
@@ -1017,7 +1030,7 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
 #define OGM_ATTN_PREFILL(HD_, G_)                                                                           \
   hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, 0, true>), grid, dim3(512), 0, stream, q, (const float *)nullptr, \
                      (const float *)nullptr, (const float2 *)nullptr, 0u, none, gq, (__half *)k_cache_layer,  \
-                     (__half *)v_cache_layer, pos0, max_splits, n_head_kv, scale, part_o, part_ml,            \
+                     (__half *)v_cache_layer, pos0, max_splits, n_head_kv, 1u, scale, part_o, part_ml,        \
                      (uint32_t *)nullptr, (float *)nullptr, no_act)
   if (head_dim == 128 && G == 1) OGM_ATTN_PREFILL(128, 1);
   else if (head_dim == 128 && G == 2) OGM_ATTN_PREFILL(128, 2);

@@ -251,6 +251,24 @@ def test_a_head_whose_flag_never_comes_is_given_up_and_reported(be):
         dev.close()
 
 
+def test_decode_with_a_kv_heads_query_heads_split_over_two_workgroups(be):
+    """attn_decode_share 2: four query heads per K/V head of head_dim 128 run as two workgroups of two (each
+    merges and quantizes one group of 256 outputs); against the CPU restatement like every other step, over a
+    prefilled cache of several chunks."""
+    n_kv, hd = 2, 128
+    ref, dev, rng = build(be, n_embd=512, n_head=8, n_kv=n_kv, hd=hd, n_ff=1024, n_vocab=320, n_layer=2,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=400, seed=21, attn_norm_scale=TAME[Q4_K])
+    be.set_tuning("attn_decode_share", 2)
+    try:
+        X = rng.standard_normal((300, 512)).astype(f32)
+        prefill_both(ref, dev, X, 0, "300 tokens")
+        for pos in range(300, 304):
+            step_both(ref, dev, rng.standard_normal(512).astype(f32), pos, f"shared K/V heads pos {pos}")
+    finally:
+        be.set_tuning("attn_decode_share", 1)
+        dev.close()
+
+
 def test_decode_with_q3_k_value_and_down_projections(be):
     """Q3_K in the v and down projections (what a Q3_K_M file does), one layer: the synthetic Q3_K
     weights are large, and with two layers of them the final hidden state is a small difference of
