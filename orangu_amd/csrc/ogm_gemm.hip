@@ -3119,7 +3119,11 @@ static int gemm_k_path(const OgmGemmArgs &a) {
   if (a.q4k_variant == 2u) return 0;
   uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
   for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
-  const uint32_t small_max = a.small_max_tokens ? a.small_max_tokens : (tiles64_all <= 128u ? 128u : 64u);
+  // (measured, Q4_K from 4096 inputs, small-batch against tiled, us: 4096 rows at 192 / 256 / 384 tokens 36 against 45,
+  // 39 against 46, 57 against 49; 6144 rows at 128 / 192: 37 against 47, 47 against 47; 14336 rows at 64 / 96: 38 against 44,
+  // 51 against 46)
+  const uint32_t small_max =
+      a.small_max_tokens ? a.small_max_tokens : (tiles64_all <= 64u ? 256u : tiles64_all <= 128u ? 128u : 64u);
   if (a.ggml_type != OGM_Q3_K && a.small_max_tokens != 1u && a.n_tokens <= small_max &&
       (q45 ? 16u : 8u) * 4096u + 128u * nsb <= GM_LDS_MAX)
     return 2;
@@ -3150,7 +3154,8 @@ static bool gemm_dma_eligible(const OgmGemmArgs &a) {
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a) {
   if (a.n_tokens == 0 || a.out_dim == 0 || is_flat32(a.ggml_type)) return false;
   if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return false;
-  // the feeding-wave kernels read planes only when asked to (they are no faster for it)
+  // the feeding-wave kernels read planes only when asked to (they are no faster for it: Q4_K 4096 -> 14336 at 256
+  // tokens 66 against 66 us; Q6_K 14336 -> 4096 at 512 tokens 96 against 98)
   return gemm_k_path(a) == 3 && (a.plane_kernel == 1u || gemm_dma_eligible(a));
 }
 

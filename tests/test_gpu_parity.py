@@ -71,10 +71,10 @@ def kname(b):
     a feeding-wave kernel that read prebuilt planes, and ogm_gemm_q*_dma_kernel as its family's tiled
     kernel (of either row tiling).  Checks that the name fits the mode the backend runs in."""
     name = b.last_kernel()
-    mode = getattr(b, "plane_mode", "planes")   # a context with no tuning reads planes on large grids
+    mode = getattr(b, "plane_mode", None)   # None: a context with no tuning reads planes on large grids
     m = re.match(r"ogm_gemm_q(6k|3k|4k|5k)_dma_kernel$", name)
     if m:
-        assert mode == "planes", name
+        assert mode in (None, "planes"), name
         return _TiledPlaneKernel({"6k": "ogm_gemm_q6k_i8", "3k": "ogm_gemm_q3k_i8", "4k": "ogm_gemm_q4k_i8p",
                                   "5k": "ogm_gemm_q5k_i8p"}[m.group(1)])
     if re.match(r"ogm_gemm_q(6k_i8|3k_i8|4k_i8p|5k_i8p)(_pre)?(_r64)?_kernel$", name):
@@ -563,8 +563,8 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
 
 def test_gemm_threshold_default():
     """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
-    float order, 17 through the matrix-core GEMM.  Q4_K: 5 tokens through the GEMV kernel, 6 and 128
-    through the small-batch kernel (a matrix of few rows), 129 through the tiled one; a matrix of
+    float order, 17 through the matrix-core GEMM.  Q4_K: 5 tokens through the GEMV kernel, 6 to 256
+    through the small-batch kernel (a matrix of few rows), 257 through the tiled one; a matrix of
     many rows leaves the small-batch kernel after 64 tokens, and one of so many that 128 x 128 tiles
     outnumber the compute units has its planes built and read by the kernel whose waves all multiply.
     Same bits everywhere."""
@@ -572,7 +572,7 @@ def test_gemm_threshold_default():
     b = Mi355xBackend()
     try:
         raw = synth_weights(Q8_0, 1024, 70, seed=3)
-        x = synth_x(129, 1024, seed=4)
+        x = synth_x(257, 1024, seed=4)
         w = qm(raw, Q8_0, 1024, 70)
         want = oracle.matmul(Q8_0, raw, 1024, 70, x[:17], 17).reshape(17, 70)
         y16 = b.matmul(x[:16], 16, w)
@@ -583,9 +583,10 @@ def test_gemm_threshold_default():
         assert_bits(y16, want[:16], "Q8_0, 16 tokens")
         raw = synth_weights(Q4_K, 1024, 70, seed=5)
         w = qm(raw, Q4_K, 1024, 70)
-        want = oracle.matmul(Q4_K, raw, 1024, 70, x, 129).reshape(129, 70)
+        want = oracle.matmul(Q4_K, raw, 1024, 70, x, 257).reshape(257, 70)
+        # (up to 64 tiles of 64 rows the small-batch kernel keeps batches of up to 256 tokens)
         for n, kernel in ((5, "ogm_gemv_kernel"), (6, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
-                          (129, "ogm_gemm_q4k_i8p_r64_kernel")):
+                          (256, "ogm_gemm_sb_q4k_kernel"), (257, "ogm_gemm_q4k_i8p_r64_kernel")):
             y = b.matmul(x[:n], n, w)
             assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, want[:n], f"Q4_K, {n} tokens")
