@@ -309,7 +309,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--copies", type=int, default=12,
                     help="distinct copies of the three matrices (12 x 99 MB = 1.2 GB > 256 MB cache)")
-    ap.add_argument("--roofline-launches", type=int, default=600)
+    ap.add_argument("--roofline-launches", type=int, default=1200)
+    ap.add_argument("--roofline-batch", type=int, default=100,
+                    help="back-to-back launches between two HIP events (the event records leave a gap of their own)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--wg-waves", type=int, default=0, help="waves per workgroup override (0 = heuristic)")
     ap.add_argument("--fuse-quant", type=int, default=-1,
@@ -441,8 +443,8 @@ def main() -> int:
     # ---- dominant kernel: the Q4_K GEMV over gate+up (4096 -> 2 x 14336 in one launch), ---------
     # back-to-back over pre-quantized activations, HIP events on its stream, in batches
     n_launch = max(40, args.roofline_launches)
-    per_batch = 20
-    batches = max(2, n_launch // per_batch)
+    per_batch = max(1, args.roofline_batch)
+    batches = max(3, n_launch // per_batch)
     kbytes = 2 * gemv_bytes(HIDDEN, FFN) - 4 * HIDDEN  # both matrices read the same x
     weight_bytes2 = 2 * FFN * (HIDDEN // 256 * 144)
     roofline = None
