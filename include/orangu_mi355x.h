@@ -276,6 +276,15 @@ int ogm_llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos0,
 int ogm_llama_prefill_tokens(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *tok_embd, const uint32_t *tokens,
                              uint32_t pos0, uint32_t n_tokens, float *last_logits, uint32_t *argmax);
 
+/* forward_hidden_states (llama.rs:1034-1045): the n_tokens tokens at positions 0 .. through run_layers
+ * from an empty cache, then every row through the output norm: out is [n_tokens][n_embd] (host f32),
+ * what an embeddings request pools over.  The tokens come as embedding rows x ([n_tokens][n_embd], host)
+ * or, with x null, as ids into tok_embd (an uploaded [n_embd -> n_vocab] matrix).  The reference makes a
+ * cache of its own for the call; here the model's cache rows 0 .. n_tokens-1 are overwritten, so a decode in
+ * progress on this model does not survive the call.  Synchronizes. */
+int ogm_llama_hidden_states(ogm_ctx *ctx, ogm_llama *m, const float *x, const ogm_weight *tok_embd,
+                            const uint32_t *tokens, uint32_t n_tokens, float *out);
+
 /* Rows row0 .. row0+n_rows of an uploaded matrix as f32 ([n_rows][in_dim], host memory), from the
  * device copy: dequantize_q8_0 / _q4_k / _q6_k (engine/quant.rs:639-649, 666-697, 746-787), bit for
  * bit.  This is the embedding lookup of run_layers (llama.rs:609-614). */

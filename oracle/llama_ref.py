@@ -200,11 +200,12 @@ def _mm(w: tuple, x: np.ndarray, n_tokens: int = 1) -> np.ndarray:
     return y.reshape(-1) if n_tokens == 1 else y.reshape(n_tokens, out_dim)
 
 
-def forward(m: Model, X: np.ndarray, pos0: int):
+def forward(m: Model, X: np.ndarray, pos0: int, all_rows: bool = False):
     """llama.rs:594-932 + 1007-1032 for the tokens whose embedding rows are X [n_tokens][n_embd], at
     positions pos0 ..: every matmul over all rows at once, K/V rows appended in order, token t
     attending to cache rows 0 .. pos0 + t; the LAST row alone goes through the output norm and
-    projection.  Returns (logits of the last token, its final hidden state)."""
+    projection.  Returns (logits of the last token, its final hidden state); with all_rows instead every
+    row after the output norm and no projection (llama.rs:1034-1045)."""
     if not m.k_cache:
         m.reset()
     X = np.array(X, f32).reshape(-1, m.n_embd)
@@ -256,8 +257,17 @@ def forward(m: Model, X: np.ndarray, pos0: int):
         gate, up = mms(4 * li + 2, (L.w_gate, L.w_up), normed2)
         h = (silu(gate) * up).astype(f32)
         X = (X + mms(4 * li + 3, (L.w_down,), h)[0]).astype(f32)
+    if all_rows:
+        return rows(lambda r: rmsnorm(r, m.output_norm, m.rms_eps), X)
     last = rmsnorm(X[-1], m.output_norm, m.rms_eps)
     return mms(4 * len(m.layers), (m.output,), last.reshape(1, -1))[0].reshape(-1), X[-1]
+
+
+def hidden_states(m: Model, X: np.ndarray) -> np.ndarray:
+    """forward_hidden_states (llama.rs:1034-1045): run_layers over the tokens from position 0 on a cache
+    of its own, then rmsnorm_inplace of every row with the output norm.  [n_tokens][n_embd]."""
+    m.reset()
+    return forward(m, X, 0, all_rows=True)
 
 
 def decode_step(m: Model, x: np.ndarray, pos: int):

@@ -469,6 +469,24 @@ class LlamaDecoder:
                         "ogm_llama_prefill_tokens")
         return logits, am.value
 
+    def hidden_states(self, x=None, tok_embd=None, tokens=None) -> np.ndarray:
+        """forward_hidden_states (llama.rs:1034-1045): [n_tokens][n_embd], every token's final hidden state
+        after the output norm, from embedding rows x or from token ids into tok_embd (a QuantMatrix or a
+        handle).  Starts from position 0 and overwrites the model's cache rows."""
+        if (x is None) == (tok_embd is None):
+            raise ValueError("give embedding rows or a matrix with token ids")
+        if x is not None:
+            x = np.ascontiguousarray(x, np.float32).reshape(-1, self.n_embd)
+            n, xp, hp, tp = x.shape[0], x.ctypes.data, None, None
+        else:
+            hp = tok_embd if isinstance(tok_embd, int) else self._be.upload(tok_embd)
+            tokens = np.ascontiguousarray(tokens, np.uint32).reshape(-1)
+            n, xp, tp = tokens.size, None, tokens.ctypes.data
+        out = np.empty((n, self.n_embd), np.float32)
+        self._be._check(self._be._lib.ogm_llama_hidden_states(self._be._ctx, self._h, xp, hp, tp, n, out.ctypes.data),
+                        "ogm_llama_hidden_states")
+        return out
+
     def decode_dev(self, x_ptr: int, pos: int, logits_ptr: int = 0, argmax_ptr: int = 0, stream: int = 0):
         self._be._check(self._be._lib.ogm_llama_decode_dev(self._be._ctx, self._h, x_ptr, pos, logits_ptr or None,
                                                            argmax_ptr or None, stream or None), "ogm_llama_decode_dev")

@@ -24,7 +24,7 @@ SYMBOLS = [
     "ogm_quantize_act", "ogm_dump_block_sums", "ogm_f16_to_f32", "ogm_set_tuning",
     "ogm_last_kernel", "ogm_act_quantize_dev", "ogm_matmul_act_dev", "ogm_matmul_multi_dev", "ogm_matmul_multi_act_dev",
     "ogm_llama_create", "ogm_llama_destroy", "ogm_llama_kv_write", "ogm_llama_kv_read", "ogm_llama_decode", "ogm_llama_decode_dev",
-    "ogm_llama_debug_hidden", "ogm_dequant_rows", "ogm_llama_generate", "ogm_llama_load_gguf", "ogm_llama_prefill", "ogm_llama_prefill_tokens",
+    "ogm_llama_debug_hidden", "ogm_dequant_rows", "ogm_llama_generate", "ogm_llama_load_gguf", "ogm_llama_prefill", "ogm_llama_prefill_tokens", "ogm_llama_hidden_states",
     "ogm_gguf_open", "ogm_gguf_parse", "ogm_gguf_close", "ogm_gguf_last_error", "ogm_gguf_info",
     "ogm_gguf_meta_u64", "ogm_gguf_meta_f64", "ogm_gguf_meta_string", "ogm_gguf_meta_array",
     "ogm_gguf_find_tensor", "ogm_gguf_tensor", "ogm_gguf_tensor_data", "ogm_gguf_matrix",
@@ -103,6 +103,7 @@ def load_library() -> C.CDLL:
     L.ogm_llama_kv_read.argtypes = [vp, vp, u32, u32, u32, vp, vp]
     L.ogm_llama_prefill.argtypes = [vp, vp, vp, u32, u32, vp, vp]
     L.ogm_llama_prefill_tokens.argtypes = [vp, vp, vp, vp, u32, u32, vp, vp]
+    L.ogm_llama_hidden_states.argtypes = [vp, vp, vp, vp, vp, u32, vp]
     L.ogm_llama_load_gguf.argtypes = [vp, vp, u32, C.POINTER(vp), C.POINTER(vp), C.POINTER(OgmLlamaConfig)]
     L.ogm_llama_decode.argtypes = [vp, vp, vp, u32, vp, vp]
     L.ogm_llama_decode_dev.argtypes = [vp, vp, vp, u32, vp, vp, vp]

@@ -1804,7 +1804,8 @@ static int llama_norm_matmul_rows(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
 
 // One chunk of T <= m->pf.chunk tokens whose embedding rows sit in m->pf.x.  With `last`,
 // the final row's hidden state ends in m->x and its logits in m->logits.
-static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32_t T, bool last, hipStream_t s) {
+static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32_t T, bool last, hipStream_t s,
+                               float *normed_rows = nullptr) {
   const ogm_llama_config &c = m->cfg;
   ogm_llama::Prefill &P = m->pf;
   const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
@@ -1848,6 +1849,15 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     delta = P.proj;
   }
   ctx->act_mode = -1;   // the activation scratch was the matmuls'
+  if (normed_rows) {
+    // forward_hidden_states (llama.rs:1034-1045): every row through the output norm, no projection
+    int rc = ensure_act(ctx, c.n_embd, T);
+    if (rc != OGM_OK) return rc;
+    const int mode_out = act_mode_for(m->output->ggml_type, T, 0);
+    HIPCHK(ctx, ogm_launch_norm_quant(mode_out, P.x, delta, m->norms + (size_t)c.n_layer * 2 * c.n_embd, c.n_embd,
+                                      c.rms_eps, normed_rows, act_view(ctx, c.n_embd, mode_out, 0), s, T));
+    return OGM_OK;
+  }
   if (!last) return OGM_OK;
   // forward (llama.rs:1007-1032): the last row alone goes through the output norm and projection
   float *x_last = P.x + (size_t)(T - 1) * c.n_embd;
@@ -1868,7 +1878,7 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
 
 static int llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x_host, const ogm_weight *tok_embd,
                          const uint32_t *tokens, uint32_t pos0, uint32_t n_tokens, float *last_logits,
-                         uint32_t *argmax) {
+                         uint32_t *argmax, float *hidden_rows = nullptr) {
   const ogm_llama_config &c = m->cfg;
   if (n_tokens == 0) return fail(ctx, OGM_ERR_INVALID, "no tokens");
   if ((uint64_t)pos0 + n_tokens > c.max_ctx) return fail(ctx, OGM_ERR_INVALID, "positions beyond the KV cache");
@@ -1893,11 +1903,16 @@ static int llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x_host, const 
       HIPCHK(ctx, hipMemcpyAsync(m->pf.x, x_host + (size_t)t0 * c.n_embd, (size_t)T * c.n_embd * 4,
                                  hipMemcpyHostToDevice, s));
     }
-    rc = llama_prefill_chunk(ctx, m, pos0 + t0, T, t0 + T == n_tokens, s);
+    // (the normed rows of a chunk land in the gate buffer, which the layers are done with: n_ff >= n_embd)
+    rc = llama_prefill_chunk(ctx, m, pos0 + t0, T, t0 + T == n_tokens, s, hidden_rows ? m->pf.gate : nullptr);
     if (rc != OGM_OK) return rc;
+    if (hidden_rows)
+      HIPCHK(ctx, hipMemcpyAsync(hidden_rows + (size_t)t0 * c.n_embd, m->pf.gate, (size_t)T * c.n_embd * 4,
+                                 hipMemcpyDeviceToHost, s));
     // the staging copies above read caller memory and m->pf.tokens is reused: finish the chunk first
     HIPCHK(ctx, hipStreamSynchronize(s));
   }
+  if (hidden_rows) return OGM_OK;
   if (last_logits) HIPCHK(ctx, hipMemcpy(last_logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost));
   if (argmax) HIPCHK(ctx, hipMemcpy(argmax, m->amax_out, 4, hipMemcpyDeviceToHost));
   return OGM_OK;
@@ -1908,6 +1923,15 @@ extern "C" int ogm_llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x, uin
   if (!ctx) return OGM_ERR_INVALID;
   if (!m || !x) return fail(ctx, OGM_ERR_INVALID, "null argument");
   return llama_prefill(ctx, m, x, nullptr, nullptr, pos0, n_tokens, last_logits, argmax);
+}
+
+extern "C" int ogm_llama_hidden_states(ogm_ctx *ctx, ogm_llama *m, const float *x, const ogm_weight *tok_embd,
+                                       const uint32_t *tokens, uint32_t n_tokens, float *out) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || !out || (x == nullptr) == (tok_embd == nullptr) || (tok_embd && !tokens))
+    return fail(ctx, OGM_ERR_INVALID, "ogm_llama_hidden_states takes embedding rows or a matrix with token ids");
+  if (m->cfg.n_ff < m->cfg.n_embd) return fail(ctx, OGM_ERR_UNSUPPORTED, "n_ff below n_embd");
+  return llama_prefill(ctx, m, x, tok_embd, tokens, 0, n_tokens, nullptr, nullptr, out);
 }
 
 extern "C" int ogm_llama_prefill_tokens(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *tok_embd,

@@ -653,6 +653,60 @@ def test_prefill_longer_than_one_pass_and_from_token_ids(be):
         dev.close()
 
 
+@pytest.mark.parametrize("n_tokens", [1, 7, 40, 300])
+def test_hidden_states_of_every_token(be, n_tokens):
+    """forward_hidden_states (llama.rs:1034-1045): every token's final hidden state after the output norm,
+    from position 0 whatever the cache held, against the CPU restatement in lock-step on the cache rows
+    (see prefill_both: an activation rounding that flips moves one token's later rows; here it can also
+    flip in the last layer, where no cache row shows it); from token ids the same bits as from rows."""
+    import oracle
+    from orangu_amd import OgmError, QuantMatrix
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=320, seed=81, attn_norm_scale=TAME[Q4_K])
+    embd_raw = synth_weights(Q6_K, 256, 320, seed=82)
+    table = oracle.dequantize(Q6_K, embd_raw, 320 * 256).reshape(320, 256)
+    tokens = rng.integers(0, 320, n_tokens).astype(np.uint32)
+    X = np.ascontiguousarray(table[tokens])
+    T = n_tokens
+    try:
+        dev.prefill(rng.standard_normal((5, 256)).astype(f32), 0)    # a cache the call must not continue
+        got = dev.hidden_states(X)
+        assert got.shape == (T, 256) and np.isfinite(got).all()
+        rows = [dev.kv_read(l, 0, T) for l in range(dev.n_layer)]
+        flagged = set()
+
+        def hook(li, p, k_row, v_row):
+            out = []
+            for mine, theirs in ((k_row, rows[li][0][p]), (v_row, rows[li][1][p])):
+                a, b = mine.astype(np.float64), theirs.astype(np.float64)
+                ulp = np.spacing(np.maximum(np.abs(mine), np.abs(theirs)).astype(np.float16)).astype(np.float64)
+                rowmax = np.abs(b).max()
+                if not (np.abs(a - b) <= ulp + 1e-5 * rowmax).all():
+                    assert (np.abs(a - b) <= ulp + 0.2 * rowmax).all(), f"position {p} layer {li}: cache row"
+                    flagged.add(p)
+                out.append(theirs.copy())
+            return out
+
+        ref.kv_hook = hook
+        want = R.hidden_states(ref, X)
+        ref.kv_hook = None
+        err = np.abs(got.astype(np.float64) - want).max(axis=1) / (np.abs(want).max(axis=1) + 1e-30)
+        loose = set(np.nonzero(err > TOL)[0].tolist())
+        assert err.max() <= 0.2, f"row {int(err.argmax())}: {err.max():.3e}"
+        assert len(loose | flagged) <= 1 + T // 8, f"{len(loose | flagged)} of {T} rows off the tight bound"
+        say(f"hidden states of {T} tokens: flagged {sorted(flagged)}, loose {sorted(loose)}, max {err.max():.2e}")
+        by_id = dev.hidden_states(tok_embd=QuantMatrix(embd_raw, Q6_K, 256, 320), tokens=tokens)
+        assert np.array_equal(by_id.view(np.uint32), got.view(np.uint32))
+        with pytest.raises(ValueError):
+            dev.hidden_states()
+        with pytest.raises(OgmError):
+            dev.hidden_states(rng.standard_normal((321, 256)).astype(f32))   # beyond the cache
+        with pytest.raises(OgmError):
+            dev.hidden_states(tok_embd=QuantMatrix(embd_raw, Q6_K, 256, 320), tokens=np.array([320], np.uint32))
+    finally:
+        dev.close()
+
+
 @pytest.mark.parametrize("hd,group,n_kv,n_tokens,pos0", [(128, 4, 2, 200, 0), (64, 4, 2, 77, 0), (128, 1, 2, 130, 31),
                                                         (64, 5, 1, 33, 64), (128, 8, 1, 65, 7), (64, 2, 4, 300, 100)])
 def test_prefill_attention_kernels_agree(be, hd, group, n_kv, n_tokens, pos0):

@@ -271,3 +271,42 @@ def test_prefill_of_several_tokens_matches_decoding_them_one_by_one():
     for l in range(2):   # bit for bit: rows of a GEMM do not depend on the other rows of the batch
         np.testing.assert_array_equal(np.stack(short.k_cache[l]), np.stack(batch.k_cache[l])[:4])
         np.testing.assert_array_equal(np.stack(short.v_cache[l]), np.stack(batch.v_cache[l])[:4])
+
+
+def test_hidden_states_are_the_normed_final_rows_of_every_prefix():
+    """forward_hidden_states (llama.rs:1034-1045): row t is the output norm of the hidden state the last
+    token of the prefix 0 .. t ends with -- causality makes it independent of the tokens after it (bit for
+    bit: a GEMM row does not depend on the other rows) -- and of single-token steps up to f32 rounding;
+    the call starts from an empty cache of its own whatever the model held before."""
+    from helpers import Q4_K, Q6_K, synth_weights
+    rng = np.random.default_rng(13)
+    n_embd, n_head, n_kv, hd, n_ff, n_vocab = 256, 4, 2, 64, 256, 64
+    mk = lambda t, i, o, s: (t, synth_weights(t, i, o, seed=s), i, o)
+    layers = [R.Layer(mk(Q4_K, n_embd, n_head * hd, 1 + 10 * l), mk(Q4_K, n_embd, n_kv * hd, 2 + 10 * l),
+                      mk(Q6_K, n_embd, n_kv * hd, 3 + 10 * l), mk(Q4_K, n_head * hd, n_embd, 4 + 10 * l),
+                      mk(Q4_K, n_embd, n_ff, 5 + 10 * l), mk(Q4_K, n_embd, n_ff, 6 + 10 * l),
+                      mk(Q6_K, n_ff, n_embd, 7 + 10 * l), np.ones(n_embd, f32), np.ones(n_embd, f32)) for l in range(2)]
+    out_norm = rng.uniform(0.5, 2.0, n_embd).astype(f32)
+    new = lambda: R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 10000.0, layers, out_norm,
+                          mk(Q6_K, n_embd, n_vocab, 99), kv_dtype=np.float32)
+    X = rng.standard_normal((6, n_embd)).astype(f32)
+    m = new()
+    R.forward(m, X[:2], 0)                      # a cache the call must not continue
+    H = R.hidden_states(m, X)
+    assert H.shape == (6, n_embd) and H.dtype == f32 and [len(c) for c in m.k_cache] == [6, 6]
+    for t in (1, 3, 5):                         # prefixes of several tokens: the same GEMM kernels, the same bits
+        _, h_last = R.forward(new(), X[:t + 1], 0)
+        np.testing.assert_array_equal(H[t], R.rmsnorm(h_last, out_norm, 1e-5))
+    one = new()
+    for t in range(6):
+        _, h = R.decode_step(one, X[t], t)
+        want = R.rmsnorm(h, out_norm, 1e-5)
+        np.testing.assert_allclose(H[t], want, rtol=0, atol=2e-5 * np.abs(want).max())
+    # the norm weight enters once per element: halving one weight halves that column and no other
+    out_norm2 = out_norm.copy()
+    out_norm2[7] *= 0.5
+    m2 = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 10000.0, layers, out_norm2,
+                 mk(Q6_K, n_embd, n_vocab, 99), kv_dtype=np.float32)
+    H2 = R.hidden_states(m2, X)
+    np.testing.assert_array_equal(H2[:, 7], H[:, 7] * f32(0.5))
+    np.testing.assert_array_equal(np.delete(H2, 7, axis=1), np.delete(H, 7, axis=1))
