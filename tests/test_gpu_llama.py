@@ -91,7 +91,7 @@ def build(be, *, n_embd, n_head, n_kv, hd, n_ff, n_vocab, n_layer, types, max_ct
     return ref, dev, rng
 
 
-def step_both(ref, dev, x, pos, what):
+def step_both(ref, dev, x, pos, what, attn_rtol=1e-5):
     """One step on both sides, in lock-step at the two discontinuous roundings (module docstring).
     The device goes first.  The CPU restatement then
       * checks each cache row it is about to append against the device's: equal, or for a few
@@ -100,7 +100,10 @@ def step_both(ref, dev, x, pos, what):
       * checks each activation it is about to quantize (vecdot::quantize_act / quantize_act_k_row)
         against the int8 values and scales the device's producing kernel left: scales within 1e-5,
         values equal except for a few elements one unit apart;
-    and continues from the device's row and the device's int8 activation."""
+    and continues from the device's row and the device's int8 activation.  attn_rtol: the bound on the
+    scales of the attention output (site 4 l + 1) alone -- the restatement adds a softmax's terms one
+    after the other in f32 as attention.rs does, the device in trees per chunk, and over thousands of
+    cached positions with values of both signs the two sums drift apart by more than 1e-5 of the result."""
     import oracle
     dev.capture_acts(True)
     got_logits, got_tok = dev.decode(x, pos)
@@ -130,10 +133,11 @@ def step_both(ref, dev, x, pos, what):
         q_dev, d_dev, g_dev = acts[site]
         assert g_dev == group and q_dev.size == xin.size, f"{what}: site {site}: quantizer group or width"
         q_cpu, d_cpu, _ = (oracle.quantize_act if group == 32 else oracle.quantize_act_k_row)(xin)
-        assert np.allclose(d_dev, d_cpu, rtol=1e-5, atol=1e-30), f"{what}: site {site}: activation scales"
+        rtol = attn_rtol if site % 4 == 1 else 1e-5
+        assert np.allclose(d_dev, d_cpu, rtol=rtol, atol=1e-30), f"{what}: site {site}: activation scales"
         diff = np.abs(q_dev.astype(np.int32) - q_cpu.astype(np.int32))
         n_off = int((diff != 0).sum())
-        assert diff.max() <= 1 and n_off <= max(3, q_dev.size // 500), \
+        assert diff.max() <= 1 and n_off <= max(3, q_dev.size // 500, int(q_dev.size * rtol * 100)), \
             f"{what}: site {site}: {n_off} of {q_dev.size} int8 activations differ, by up to {diff.max()}"
         if n_off:
             say(f"{what}: site {site}: {n_off} int8 activation(s) one unit apart; the CPU continues from the device's")
@@ -298,6 +302,27 @@ def test_decode_over_a_prefilled_cache_with_several_attention_chunks(be):
             ref.v_cache[l] = [r.astype(np.float16) for r in v]
         for pos in (300, 301, 302):
             step_both(ref, dev, rng.standard_normal(1024).astype(f32), pos, f"prefilled pos {pos}")
+    finally:
+        dev.close()
+
+
+@pytest.mark.parametrize("hd,group,n_kv,n_pre", [(128, 4, 1, 4500), (128, 8, 1, 2200), (64, 4, 2, 8300), (128, 1, 2, 16500)])
+def test_decode_at_contexts_whose_chunks_merge_in_several_rounds(be, hd, group, n_kv, n_pre):
+    """The workgroup that merges a K/V head's chunks takes up to eight chunks per slice in one trip to
+    memory (32 chunks at head_dim 128 with four query heads, 16 with eight, 64 at head_dim 64 with four, 128
+    with one query head) and goes round again for longer contexts, carrying its running maximum; here 36, 18, 65
+    and 129 chunks, the last one partial.  (The attention output's scales differ from the restatement's by up to 1.5e-4
+    of their value at these lengths -- its softmax sums run term by term in f32 -- against 1e-2 and more for a chunk left
+    out; the bound grows with the context.)"""
+    n_head = group * n_kv
+    n_embd = 256
+    ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=320, n_layer=1,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=n_pre + 4, seed=9, base=500000.0,
+                          attn_norm_scale=TAME[Q4_K])   # scores of order one: every chunk carries weight
+    try:
+        fill_cache_both(ref, dev, rng, 1, n_pre, n_kv * hd)
+        for pos in (n_pre, n_pre + 1):
+            step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"context {pos}", attn_rtol=1e-5 * n_pre / 250)
     finally:
         dev.close()
 
