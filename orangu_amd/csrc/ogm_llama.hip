@@ -1051,9 +1051,13 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
 
 // ------------------------------------------------------------------------------------------
 // Prefill attention on the matrix cores.  Workgroup (query tile of 32 tokens, K/V head, group of
-// four query heads), four waves: wave w takes query head 4 z + w of the K/V head and walks the
-// cache in tiles of 64 positions up to the tile's last query (causal), with a running maximum and
-// sum per query (the softmax of llama.rs's attention, tensor.rs softmax_rows, regrouped).
+// four query heads), eight waves: wave w takes query head 4 z + w % 4 of the K/V head and walks
+// every second cache tile of 64 positions (the even ones for waves 0-3, the odd ones for waves 4-7)
+// up to the tile's last query (causal), with a running maximum and sum per query (the softmax of
+// llama.rs's attention, tensor.rs softmax_rows, regrouped); at the end the two halves' partial
+// softmaxes meet in LDS.  A launch takes as long as its longest workgroup -- the last query tile,
+// whose walk is the whole context (one workgroup alone on a compute unit: 3.0 us per cache tile) --
+// so the walk is what the second set of waves halves.
 //
 //   scores^T = K . Q^T    A = K rows from LDS (16 bytes of a row are 8 consecutive dimensions),
 //                         B = Q^T from registers; the result has one query per lane and 16
@@ -1079,7 +1083,7 @@ __device__ __forceinline__ void am_split(float v, _Float16 &hi, _Float16 &lo) {
 }
 
 template <int HD>
-__global__ __launch_bounds__(256) void ogm_attn_prefill_mfma_kernel(const float *__restrict__ q,
+__global__ __launch_bounds__(512, 2) void ogm_attn_prefill_mfma_kernel(const float *__restrict__ q,
                                                                     const __half *__restrict__ kc,
                                                                     const __half *__restrict__ vc, uint32_t pos0,
                                                                     uint32_t n_tokens, uint32_t n_head_kv, uint32_t gq,
@@ -1089,13 +1093,18 @@ __global__ __launch_bounds__(256) void ogm_attn_prefill_mfma_kernel(const float 
   constexpr int NDB = HD / 32;               // 32-dimension blocks of the output
   constexpr uint32_t PPR = HD / 8;           // 16-byte pieces per cache row
   constexpr int NK = (int)(AM_KT * PPR / 128u);   // pieces a K-copying thread moves per tile (8 or 4)
-  __shared__ __align__(16) uint8_t k_l[AM_KT * KROW];
-  __shared__ __align__(16) uint8_t vt_l[HD * AM_VROW];
+  constexpr uint32_t K_BYTES = AM_KT * KROW, V_BYTES = HD * AM_VROW;
+  extern __shared__ __align__(16) uint8_t am_lds[];   // per half: a K tile, then a V^T tile
+  const uint32_t half = threadIdx.x >> 8;             // which of the two tiles of an iteration
+  uint8_t *const k_l = am_lds + half * (K_BYTES + V_BYTES);
+  uint8_t *const vt_l = k_l + K_BYTES;
 
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t tid = threadIdx.x & 255u, lane = tid & 63u, wave = tid >> 6;   // within the half
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
-  const uint32_t qt = gridDim.x - 1u - blockIdx.x;   // long tiles first
-  const uint32_t kvh = blockIdx.y, g = 4u * blockIdx.z + wave;
+  // Long tiles first, across the whole launch: workgroups start in the grid's order (x fastest), and a long tile
+  // that starts late is what the launch then waits for (2048 tokens, 8 K/V heads, with the tiles on x: 165 us)
+  const uint32_t qt = gridDim.y - 1u - blockIdx.y;
+  const uint32_t kvh = blockIdx.x % n_head_kv, g = 4u * (blockIdx.x / n_head_kv) + wave;
   const bool live = g < gq;
   const uint32_t n_head = n_head_kv * gq, kv_dim = n_head_kv * HD;
   const uint32_t tok = min(32u * qt + l32, n_tokens - 1u);   // this lane's query (clamped: computed, not stored)
@@ -1204,12 +1213,16 @@ __global__ __launch_bounds__(256) void ogm_attn_prefill_mfma_kernel(const float 
     for (int r = 0; r < 16; r++) o[d][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;   // l_run: this lane half's share of the sum
 
-  AM_LOAD(0u);
-  for (uint32_t it = 0; it < n_tiles; it++) {
+  // iteration i: tile 2 i + half (a tile past the walk is loaded from clamped rows and not used)
+  const uint32_t n_iter = (n_tiles + 1u) / 2u;
+  const uint32_t q_min = pos0 + min(32u * qt, n_tokens - 1u);   // the tile's first query
+  AM_LOAD(half);
+  for (uint32_t i2 = 0; i2 < n_iter; i2++) {
+    const uint32_t it = 2u * i2 + half;
     AM_STORE();
     __syncthreads();
-    if (it + 1u < n_tiles) AM_LOAD(it + 1u);
-    if (live) {
+    if (i2 + 1u < n_iter) AM_LOAD(it + 2u);
+    if (live && it < n_tiles) {
       af16 s0, s1;
 #pragma unroll
       for (int r = 0; r < 16; r++) s0[r] = s1[r] = 0.0f;
@@ -1225,17 +1238,28 @@ __global__ __launch_bounds__(256) void ogm_attn_prefill_mfma_kernel(const float 
       // register r of block pb: position it * 64 + 32 pb + 8 (r / 4) + 4 lh + r % 4
       const uint32_t pbase = it * AM_KT + 4u * lh;
       float mt = -INFINITY;
+      if (it * AM_KT + (AM_KT - 1u) <= q_min) {   // every query of the tile sees the whole cache tile
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const uint32_t p_ = pbase + 8u * (r >> 2) + (r & 3);
-        s0[r] = p_ <= q_abs ? s0[r] * scale_q : -INFINITY;
-        s1[r] = p_ + 32u <= q_abs ? s1[r] * scale_q : -INFINITY;
-        mt = fmaxf(mt, fmaxf(s0[r], s1[r]));
+        for (int r = 0; r < 16; r++) {
+          s0[r] *= scale_q;
+          s1[r] *= scale_q;
+          mt = fmaxf(mt, fmaxf(s0[r], s1[r]));
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const uint32_t p_ = pbase + 8u * (r >> 2) + (r & 3);
+          s0[r] = p_ <= q_abs ? s0[r] * scale_q : -INFINITY;
+          s1[r] = p_ + 32u <= q_abs ? s1[r] * scale_q : -INFINITY;
+          mt = fmaxf(mt, fmaxf(s0[r], s1[r]));
+        }
       }
       mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-      const float m_new = fmaxf(m_run, mt);   // finite: position 0 is never masked
+      // (a query may see nothing of the odd half's first tile: then everything stays at zero)
+      const float m_max = fmaxf(m_run, mt);
+      const float m_new = m_max == -INFINITY ? 0.0f : m_max;
       const float alpha = __expf(m_run - m_new);
-      m_run = m_new;
+      m_run = m_max;
       float lsum = 0.0f;
       ah8 ph[4], pl[4];   // k step 2 pb + j: registers 8 j .. 8 j + 7 of block pb
 #pragma unroll
@@ -1267,6 +1291,31 @@ __global__ __launch_bounds__(256) void ogm_attn_prefill_mfma_kernel(const float 
   }
 #undef AM_LOAD
 #undef AM_STORE
+  // the odd half's partial softmax goes through LDS (the tiles' space: the loop ended on a barrier) to the
+  // even half's wave of the same head, lane to lane: [register][wave][lane]
+  {
+    float *mrg = (float *)am_lds;
+    constexpr uint32_t NR = NDB * 16u + 2u;
+    const uint32_t slot = wave * 64u + lane;
+    if (half == 1u) {
+#pragma unroll
+      for (int d = 0; d < NDB; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mrg[(16u * d + r) * 256u + slot] = o[d][r];
+      mrg[(NR - 2u) * 256u + slot] = m_run;
+      mrg[(NR - 1u) * 256u + slot] = l_run;
+    }
+    __syncthreads();
+    if (half == 1u) return;
+    const float m1 = mrg[(NR - 2u) * 256u + slot], l1 = mrg[(NR - 1u) * 256u + slot];
+    const float m = fmaxf(m_run, m1);   // finite: the even half saw position 0
+    const float a0 = __expf(m_run - m), a1 = __expf(m1 - m);
+    l_run = l_run * a0 + l1 * a1;
+#pragma unroll
+    for (int d = 0; d < NDB; d++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[d][r] = o[d][r] * a0 + mrg[(16u * d + r) * 256u + slot] * a1;
+  }
   if (live && 32u * qt + l32 < n_tokens) {
     const float l = l_run + __shfl_xor(l_run, 32, 64);
     float *op = attn_out + ((size_t)tok * n_head + (size_t)kvh * gq + g) * HD + 4u * lh;
@@ -1285,15 +1334,20 @@ hipError_t ogm_launch_attn_prefill_mfma(const float *q, void *k_cache_layer, voi
   if (n_head_kv == 0 || n_head % n_head_kv != 0 || n_tokens == 0) return hipErrorInvalidValue;
   const uint32_t gq = n_head / n_head_kv;
   if (n_head_kv > 65535u || gq > 8u) return hipErrorInvalidValue;
-  const dim3 grid((n_tokens + 31u) / 32u, n_head_kv, (gq + 3u) / 4u);
+  if ((n_tokens + 31u) / 32u > 65535u) return hipErrorInvalidValue;
+  const dim3 grid(n_head_kv * ((gq + 3u) / 4u), (n_tokens + 31u) / 32u);
+  if (head_dim != 128 && head_dim != 64) return hipErrorInvalidValue;
+  // two (K, V^T) tiles, rows padded by 16 bytes; at head_dim 128 more than a kernel gets without asking
+  const uint32_t lds_bytes = 2u * (AM_KT * (head_dim * 2u + 16u) + head_dim * AM_VROW);
+  const void *fn = head_dim == 128 ? (const void *)ogm_attn_prefill_mfma_kernel<128> : (const void *)ogm_attn_prefill_mfma_kernel<64>;
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  if (e != hipSuccess) return e;
   if (head_dim == 128)
-    hipLaunchKernelGGL(ogm_attn_prefill_mfma_kernel<128>, grid, dim3(256), 0, stream, q, (const __half *)k_cache_layer,
-                       (const __half *)v_cache_layer, pos0, n_tokens, n_head_kv, gq, scale, attn_out);
-  else if (head_dim == 64)
-    hipLaunchKernelGGL(ogm_attn_prefill_mfma_kernel<64>, grid, dim3(256), 0, stream, q, (const __half *)k_cache_layer,
+    hipLaunchKernelGGL(ogm_attn_prefill_mfma_kernel<128>, grid, dim3(512), lds_bytes, stream, q, (const __half *)k_cache_layer,
                        (const __half *)v_cache_layer, pos0, n_tokens, n_head_kv, gq, scale, attn_out);
   else
-    return hipErrorInvalidValue;
+    hipLaunchKernelGGL(ogm_attn_prefill_mfma_kernel<64>, grid, dim3(512), lds_bytes, stream, q, (const __half *)k_cache_layer,
+                       (const __half *)v_cache_layer, pos0, n_tokens, n_head_kv, gq, scale, attn_out);
   return hipGetLastError();
 }
 
