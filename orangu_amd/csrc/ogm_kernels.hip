@@ -833,6 +833,7 @@ struct GemvParams {
   uint32_t in_dim, upr;            // upr = blocks per row
   uint32_t n_tokens;
   uint32_t C, nct;                // tile shape: C blocks x R rows, nct = upr / C column tiles
+  uint32_t lane_acc;              // formats of several terms a block, tiles one block wide, one wave: see gemv_lane_acc
   OgmGemvTail tail;
   OgmGemvHead head;
 };
@@ -859,6 +860,9 @@ __host__ __device__ constexpr int n_term_arrays() {
   return (GEMM_ORDER && F::HAS_MIN && F::TYPE != OGM_Q2_K) ? 2 : 1;   // Q4_K, Q5_K: the min pass first
 }
 
+static const size_t OGM_LDS_BUDGET = 64 * 1024;   // what a launch aims for: batches and row blocks are cut to fit
+static const size_t OGM_LDS_MAX = 160 * 1024;     // what a workgroup can have when even one token of one row block needs more
+
 // Dynamic LDS bytes of one workgroup.
 template <class F, bool GEMM_ORDER>
 static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rb_per_wg = 1) {
@@ -871,6 +875,25 @@ static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rb_per
   b = (b + 15) & ~(size_t)15;
   b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * rb_per_wg * upr * tl.R * 4 * F::TERMS;  // terms
   return b;
+}
+
+// A format that leaves several terms a block (Q2_K over per-32 activations: sixteen) keeps upr * R * TERMS floats
+// per token for the ordered sum; where a row has an odd number of blocks the tiles are one block wide and 64 rows
+// high, and a long row (Llama-2-7B's 11008 inputs: 43 blocks, 176 KB) no longer fits a workgroup's LDS.  In such
+// tiles a lane owns its row's block of every column tile, so a workgroup of ONE wave that walks the column tiles in
+// order can add the terms up as they come, in the row's order, and needs one float per token and lane.
+template <class F, bool GEMM_ORDER>
+static bool gemv_lane_acc(uint32_t in_dim) {
+  if (F::TERMS <= 1 || n_term_arrays<F, GEMM_ORDER>() != 1) return false;
+  const OgmTiling tl = ogm_tiling_for(in_dim / F::ELEMS, 1);
+  return tl.C == 1 && gemv_lds_bytes<F, GEMM_ORDER>(in_dim, 1) > OGM_LDS_BUDGET;
+}
+template <class F>
+static size_t gemv_lds_bytes_lane_acc(uint32_t in_dim, uint32_t n_tokens) {
+  const size_t upr = in_dim / F::ELEMS, n_scale = in_dim / F::ACT_GROUP;
+  size_t b = (size_t)n_tokens * in_dim + (size_t)n_tokens * upr * F::AUX16 * 16 + (size_t)n_tokens * n_scale * 4;
+  b = (b + 15) & ~(size_t)15;
+  return b + (size_t)n_tokens * 64 * 4;
 }
 
 #define OGM_STAGE_PEEL 4
@@ -1152,6 +1175,10 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
   }
   __syncthreads();
 
+  if constexpr (F::TERMS > 1) {
+    if (p.lane_acc)   // one wave: its lanes' running sums, one per token
+      for (uint32_t t = 0; t < T; t++) l_term[t * 64u + lane] = 0.0f;
+  }
   // ---- tiles of this wave
   for (; it < n_items; it += n_wave) {
     const uint32_t rbk = it / nct, ct = it - rbk * nct;
@@ -1173,6 +1200,13 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
         // a block leaves several terms, in the order the row adds them
         float tt[F::TERMS];
         F::template terms<UPR>(cur, a, col, tt);
+        if (p.lane_acc) {   // this lane's row, the column tiles in order: the row's own sequence of additions
+          float acc = l_term[t * 64u + lane];
+#pragma unroll
+          for (int g = 0; g < F::TERMS; g++) acc += tt[g];
+          l_term[t * 64u + lane] = acc;
+          continue;
+        }
         float *dst = l_term + (size_t)(t * K + rbk) * term_stride + (size_t)col * F::TERMS * R + r_local;
 #pragma unroll
         for (int g = 0; g < F::TERMS; g++) dst[g * R] = tt[g];
@@ -1201,6 +1235,14 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
   }
   __syncthreads();
 
+  if constexpr (F::TERMS > 1) {
+    if (p.lane_acc) {
+      const uint32_t orow = rb0 * R + lane;
+      if (orow < out_dim)
+        for (uint32_t t = 0; t < T; t++) y[(size_t)t * out_dim + orow] = l_term[t * 64u + lane];
+      return;
+    }
+  }
   // One lane per (token, row): the row's block terms in ascending order, one accumulator.
   const uint32_t KR = K * R;
   for (uint32_t i = tid; i < KR * T; i += nthr) {
@@ -1255,11 +1297,14 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
 // ------------------------------------------------------------------------------------------
 // host side of the launch
 
-static const size_t OGM_LDS_BUDGET = 64 * 1024;
 
 template <class F, bool GEMM_ORDER>
 static uint32_t max_tokens_t(uint32_t in_dim) {
   uint32_t t = 8;
+  if (gemv_lane_acc<F, GEMM_ORDER>(in_dim)) {
+    while (t > 1 && gemv_lds_bytes_lane_acc<F>(in_dim, t) > OGM_LDS_BUDGET) t--;
+    return t;
+  }
   while (t > 1 && gemv_lds_bytes<F, GEMM_ORDER>(in_dim, t) > OGM_LDS_BUDGET) t--;
   return t;
 }
@@ -1369,8 +1414,14 @@ static void launch_single(const GemvParams &p, dim3 g, dim3 b, size_t lds, hipSt
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false, QUANT>), g, b, lds, stream, p);
   else if (F::ELEMS == 32 && p.upr == 128)
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 128, true, false, false, QUANT>), g, b, lds, stream, p);
-  else
+  else {
+    // (a long row of an odd number of blocks -- 64-row tiles one block wide -- stages more than a launch gets unasked)
+    if (lds > OGM_LDS_BUDGET &&
+        hipFuncSetAttribute((const void *)ogm_gemv_kernel<F, 0, true, false, false, QUANT>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return;   // the launch below then fails and reports it
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false, QUANT>), g, b, lds, stream, p);
+  }
 }
 
 template <class F, bool GEMM_ORDER>
@@ -1432,16 +1483,30 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
     }
     p.wg_end[m] = n_wg;
   }
-  const size_t lds = gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, K);
-  if (lds > OGM_LDS_BUDGET) return hipErrorInvalidValue;
+  // (rows of many blocks in a format that leaves sixteen terms a block -- Q2_K over per-32 activations at
+  // 14336 inputs: 74 KB for one token -- go beyond the budget; they get what they need, up to the hardware's limit)
+  const bool lane_acc = gemv_lane_acc<F, GEMM_ORDER>(a.in_dim) && !dump && a.tail.kind == OGM_TAIL_NONE &&
+                        a.head.kind == OGM_HEAD_NONE;
+  p.lane_acc = lane_acc ? 1u : 0u;
+  const size_t lds = lane_acc ? gemv_lds_bytes_lane_acc<F>(a.in_dim, a.n_tokens) : gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, K);
+  if (lds > OGM_LDS_MAX) return hipErrorInvalidValue;
+  auto launch = [&](void (*kernel)(GemvParams), dim3 g_, dim3 b_) -> hipError_t {
+    if (lds > OGM_LDS_BUDGET) {
+      const hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kernel, g_, b_, lds, stream, p);
+    return hipGetLastError();
+  };
   // the plain single-token kernels of most formats need well under 128 registers and are built for up
   // to sixteen waves
   const bool plain_single = a.n_tokens == 1 && !GEMM_ORDER && !dump && !a.x_f32 && a.tail.kind == OGM_TAIL_NONE &&
                             a.head.kind == OGM_HEAD_NONE;
   // the per-32 formats' tiles are small (2 KB of Q8_0): sixteen of them per workgroup measure 7 %
   // faster than eight at 4096 x 4096
-  const uint32_t waves = pick_waves(tl.nct, a.wg_waves, plain_single ? F::MAX_THREADS_SINGLE : F::MAX_THREADS,
-                                    (plain_single && F::ELEMS == 32) ? 16u : 8u);
+  const uint32_t waves = lane_acc ? 1u
+                                  : pick_waves(tl.nct, a.wg_waves, plain_single ? F::MAX_THREADS_SINGLE : F::MAX_THREADS,
+                                               (plain_single && F::ELEMS == 32) ? 16u : 8u);
   if (a.tail.kind == OGM_TAIL_NORM && a.tail.n > 1024u * waves) return hipErrorInvalidValue;
   if (a.head.kind == OGM_HEAD_NORM) {
     if (a.in_dim > 1024u * waves) return hipErrorInvalidValue;
@@ -1450,17 +1515,16 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
     p.head.n_prod = (a.in_dim / 256u + waves - 1u) / waves;
   }
   const dim3 g(n_wg + p.head.n_prod), b(waves * 64);
-  if (dump) {
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true, false>), g, b, lds, stream, p);
-  } else if (a.n_tokens == 1 && !GEMM_ORDER) {
+  if (dump) return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true, false>, g, b);
+  if (a.n_tokens == 1 && !GEMM_ORDER) {
+    // (the kernels with a compile-time row length, tails and heads are for rows that fit the budget many times over)
+    if (lds > OGM_LDS_BUDGET && (a.tail.kind != OGM_TAIL_NONE || a.head.kind != OGM_HEAD_NONE)) return hipErrorInvalidValue;
     if (a.x_f32) launch_single<F, true>(p, g, b, lds, stream);
     else launch_single<F, false>(p, g, b, lds, stream);
-  } else if (F::HAS_UNPACK && a.n_tokens >= 6) {
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false, F::HAS_UNPACK>), g, b, lds, stream, p);
-  } else {
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false>), g, b, lds, stream, p);
+    return hipGetLastError();
   }
-  return hipGetLastError();
+  if (F::HAS_UNPACK && a.n_tokens >= 6) return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false, F::HAS_UNPACK>, g, b);
+  return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false>, g, b);
 }
 
 hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name) {

@@ -1,0 +1,101 @@
+"""A seeded walk over (type, in_dim, out_dim, tokens) through a context with no tuning: whatever kernel the
+library's own routing picks -- GEMV, chunked GEMV in GEMM order, few-token, small-batch, feeding-wave, flat
+or plane kernel -- `matmul` must give every bit of the CPU restatement's matmul (gemm_k_* / dot_flat_pair from
+two tokens on, the GEMV forms at one; cpu.rs:445-458) and `matmul_decode` every bit of the GEMV forms per token
+(cpu.rs:265-317).  Shapes are drawn around the routing thresholds (token counts 5/6, 16/17, 64/65, 128/129,
+256/257; row counts around 64-row tile multiples) and ragged on purpose."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import BLOCK, TYPE_NAME, pin_scales, pseudo_bytes_fast, row_bytes, synth_weights, synth_x
+
+pytestmark = pytest.mark.gpu
+
+TYPES = sorted(BLOCK)
+TOKENS = (1, 2, 3, 5, 6, 8, 9, 16, 17, 31, 32, 33, 63, 64, 65, 100, 128, 129, 200, 256, 257, 300)
+ROWS = (1, 2, 31, 33, 63, 64, 65, 127, 129, 200, 257, 500, 700, 1100, 2100, 4100, 8300)
+
+
+def cases(n, seed, long_rows=False):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        t = TYPES[int(rng.integers(len(TYPES)))]
+        elems = BLOCK[t][1]
+        if long_rows:   # rows of many blocks: the staging of activations and terms in LDS grows with them
+            in_dim = int(rng.choice((8192, 11008, 14336, 16384, 28672))) if elems == 256 else \
+                int(rng.choice((8192, 11008, 14336, 16384, 28672, 9248)))
+        else:
+            in_dim = int(rng.choice((256, 512, 768, 1024, 2048, 2304, 4096, 14336))) if elems == 256 else \
+                int(rng.choice((32, 64, 96, 256, 544, 1024, 2048, 4096, 14336)))
+        T = int(rng.choice(TOKENS))
+        out_dim = int(rng.choice(ROWS))
+        if T * out_dim * in_dim > 150e6:     # keeps the CPU side of the whole module within seconds
+            out_dim = max(1, int(150e6 // (T * in_dim)))
+        out.append(pytest.param(t, in_dim, out_dim, T, i, id=f"{TYPE_NAME[t]}-{in_dim}x{out_dim}-T{T}"))
+    return out
+
+
+@pytest.fixture(scope="module")
+def be():
+    from orangu_amd import Mi355xBackend
+    b = Mi355xBackend()  # raises if the HIP library or the device is missing: no fallback
+    yield b
+    b.close()
+
+
+def bits(a):
+    return np.asarray(a, np.float32).reshape(-1).view(np.uint32)
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim,T,i", cases(400, 20240611) + cases(150, 977, long_rows=True))
+def test_default_routing_is_bit_exact(be, t, in_dim, out_dim, T, i):
+    from orangu_amd import QuantMatrix
+    if i % 3 == 0:   # arbitrary bytes with finite scales, as the reference's own fixtures are made (vecdot.rs:3436-3526)
+        raw = pin_scales(pseudo_bytes_fast(row_bytes(t, in_dim) * out_dim, 1000 + i), t)
+    else:
+        raw = synth_weights(t, in_dim, out_dim, seed=2000 + i)
+    x = synth_x(T, in_dim, seed=3000 + i)
+    print("case", TYPE_NAME[t], in_dim, out_dim, T, flush=True)
+    w = QuantMatrix(np.ascontiguousarray(raw), t, in_dim, out_dim)
+    try:
+        got = be.matmul(x, T, w)
+        k1 = be.last_kernel()
+        want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
+        bad = np.nonzero(bits(got) != bits(want))[0]
+        assert bad.size == 0, f"matmul via {k1}: {bad.size} of {want.size} differ, first {bad[:4]}"
+        got = be.matmul_decode(x, T, w)
+        k2 = be.last_kernel()
+        want = oracle.matmul_decode(t, raw, in_dim, out_dim, x, T)
+        bad = np.nonzero(bits(got) != bits(want))[0]
+        assert bad.size == 0, f"matmul_decode via {k2}: {bad.size} of {want.size} differ, first {bad[:4]}"
+    finally:
+        be.evict(w)
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim,T,decode", [
+    (10, 14336, 33, 32, False),    # Q2_K over per-32 activations: sixteen terms a block, 74 KB of them for one token
+    (10, 11008, 70, 5, False),     # ... and 43 blocks a row (tiles one block wide): 176 KB, more than a workgroup can have
+    (10, 11008, 130, 40, False),
+    (20, 9248, 200, 3, True),      # IQ4_NL, 289 blocks a row: 74 KB of terms for one token in GEMV order
+    (8, 9248, 65, 1, False),
+])
+def test_long_rows_that_outgrow_the_default_lds(be, t, in_dim, out_dim, T, decode):
+    """Rows whose staging does not fit the 64 KB a launch aims for: the launch asks for what it needs, and where a
+    format of several terms a block meets tiles one block wide, one wave adds a row's terms up in its lanes as the
+    column tiles come (the row's own order) instead of keeping them all.  Same bits as ever."""
+    from orangu_amd import QuantMatrix
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim)
+    x = synth_x(T, in_dim, seed=T)
+    w = QuantMatrix(np.ascontiguousarray(raw), t, in_dim, out_dim)
+    try:
+        if decode:
+            got, want = be.matmul_decode(x, T, w), oracle.matmul_decode(t, raw, in_dim, out_dim, x, T)
+        else:
+            got, want = be.matmul(x, T, w), oracle.matmul(t, raw, in_dim, out_dim, x, T)
+        assert be.last_kernel().startswith("ogm_gemv_kernel"), be.last_kernel()
+        bad = np.nonzero(bits(got) != bits(want))[0]
+        assert bad.size == 0, f"{be.last_kernel()}: {bad.size} of {want.size} differ, first {bad[:4]}"
+    finally:
+        be.evict(w)
