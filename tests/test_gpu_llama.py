@@ -1009,3 +1009,38 @@ def test_generate_matches_stepwise(be, embd_t):
     finally:
         dev.close()
         dev2.close()
+
+
+def _random_models(n, seed):
+    rng = np.random.default_rng(seed)
+    combos = [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q5_K, Q5_K, Q6_K, Q5_K), (Q4_0, Q5_0, IQ4_NL, Q8_0)]
+    out = []
+    for i in range(n):
+        types = combos[int(rng.integers(len(combos)))]
+        hd = int(rng.choice((64, 128)))
+        n_kv = int(rng.choice((1, 2, 3)))
+        group = int(rng.choice((1, 2, 3, 4, 5, 8)))
+        n_embd = int(rng.choice((256, 512, 768, 1280)))
+        n_ff = int(rng.choice((256, 768, 1792, 2816, 11008)))
+        T = int(rng.choice((1, 2, 5, 6, 9, 17, 33, 70)))
+        if n_kv * group * hd % 256 != 0 and types[0] not in (Q8_0, Q4_0):   # wo's input must be whole K-quant blocks
+            group = 4 if hd == 64 else 2
+        out.append(pytest.param(types, hd, n_kv, group, n_embd, n_ff, T, i,
+                                id=f"{i}-hd{hd}-kv{n_kv}-g{group}-e{n_embd}-ff{n_ff}-T{T}"))
+    return out
+
+
+@pytest.mark.parametrize("types,hd,n_kv,group,n_embd,n_ff,T,i", _random_models(28, 4242))
+def test_a_seeded_walk_over_model_shapes(be, types, hd, n_kv, group, n_embd, n_ff, T, i):
+    """Widths of the residual stream, of the heads together (not n_embd: Qwen3) and of the FFN drawn independently,
+    FFN widths of an odd number of blocks (11008) among them; a prompt of T tokens, then two decode steps."""
+    n_head = group * n_kv
+    ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=n_ff, n_vocab=320, n_layer=1,
+                          types=types, max_ctx=T + 4, seed=900 + i, attn_norm_scale=TAME.get(types[0], 1.0),
+                          neox=bool(i & 1), pre=("q_norm", "k_norm") if i % 3 == 0 else ())
+    try:
+        prefill_both(ref, dev, rng.standard_normal((T, n_embd)).astype(f32), 0, f"model {i}")
+        for pos in (T, T + 1):
+            step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"model {i} pos {pos}")
+    finally:
+        dev.close()
