@@ -99,3 +99,56 @@ def test_long_rows_that_outgrow_the_default_lds(be, t, in_dim, out_dim, T, decod
         assert bad.size == 0, f"{be.last_kernel()}: {bad.size} of {want.size} differ, first {bad[:4]}"
     finally:
         be.evict(w)
+
+
+def _batches(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        n_ops = int(rng.integers(1, 7))
+        in_dims = [int(rng.choice((256, 512, 1024, 2048, 4096))) for _ in range(2)]
+        ops = []
+        for _ in range(n_ops):
+            t = TYPES[int(rng.integers(len(TYPES)))]
+            ops.append((t, in_dims[int(rng.integers(2))], int(rng.choice((1, 31, 64, 65, 129, 300, 1100))),
+                        int(rng.integers(3))))          # which of three inputs of that width it reads
+        T = int(rng.choice((0, 1, 2, 5, 6, 8, 9, 17, 40, 70, 130)))
+        out.append(pytest.param(ops, T, bool(rng.integers(2)), int(rng.choice((0, 0, 16, 64))), i, id=f"batch{i}-{n_ops}ops-T{T}"))
+    return out
+
+
+@pytest.mark.parametrize("ops,T,decode,stripe,i", _batches(60, 31337))
+def test_batches_of_mixed_ops_are_bit_exact(be, ops, T, decode, stripe, i):
+    """matmul_batch / matmul_batch_decode (mod.rs:362-366, 405) over ops of mixed types and widths, several of
+    which share an input (they are quantized once and grouped into one launch where their type allows), with
+    token stripes (mod.rs:154-172) and empty ops in between: every op's result is that of its own matmul."""
+    from orangu_amd import MatmulOp, QuantMatrix
+    xs = {}
+    ms, want = [], []
+    for k, (t, in_dim, out_dim, which) in enumerate(ops):
+        n_tok = 0 if (k == 1 and i % 5 == 0) else T      # now and then an op of no tokens in front of others
+        key = (in_dim, which, n_tok)
+        if key not in xs:
+            xs[key] = synth_x(max(n_tok, 1), in_dim, seed=5000 + 10 * i + which)[:n_tok]
+        raw = synth_weights(t, in_dim, out_dim, seed=6000 + 10 * i + k)
+        w = QuantMatrix(np.ascontiguousarray(raw), t, in_dim, out_dim)
+        ms.append(MatmulOp(xs[key], n_tok, w))
+        if n_tok == 0:
+            want.append(np.zeros(0, np.float32))
+        else:
+            # a striped op is the backend's matmul of every stripe (guarded_matmul_op, mod.rs:154-172): a last
+            # stripe of one token takes the single-token forms
+            step = stripe if (stripe and not decode) else n_tok
+            fn = oracle.matmul_decode if decode else oracle.matmul
+            want.append(np.concatenate([
+                np.asarray(fn(t, raw, in_dim, out_dim, np.ascontiguousarray(xs[key][s0:s0 + step]), min(step, n_tok - s0))).reshape(-1)
+                for s0 in range(0, n_tok, step)]))
+    print("batch", i, [(TYPE_NAME[o[0]], o[1], o[2], o[3]) for o in ops], "T", T, "decode", decode, "stripe", stripe, flush=True)
+    try:
+        got = be.matmul_batch_decode(ms) if decode else be.matmul_batch(ms, stripe)
+        for k, (g, w_) in enumerate(zip(got, want)):
+            bad = np.nonzero(bits(g) != bits(w_))[0] if w_.size else np.zeros(0)
+            assert np.asarray(g).size == w_.size and bad.size == 0, f"op {k} {ops[k]}: {bad.size} of {w_.size} differ (last kernel {be.last_kernel()})"
+    finally:
+        for m in ms:
+            be.evict(m.w)
