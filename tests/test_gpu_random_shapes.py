@@ -152,3 +152,43 @@ def test_batches_of_mixed_ops_are_bit_exact(be, ops, T, decode, stripe, i):
     finally:
         for m in ms:
             be.evict(m.w)
+
+
+def _large_grids(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        t = int(rng.choice((10, 11, 12, 13, 14, 23, 8)))
+        in_dim = int(rng.choice((256, 512, 1024)))
+        out_dim = int(rng.choice((16600, 20000, 33000, 41000)))
+        T = int(rng.choice((3, 4, 9, 16, 130, 260, 390)))
+        if T * out_dim * in_dim > 3e9:
+            T = max(3, int(3e9 // (out_dim * in_dim)))
+        out.append(pytest.param(t, in_dim, out_dim, T, i, id=f"{TYPE_NAME[t]}-{in_dim}x{out_dim}-T{T}"))
+    return out
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim,T,i", _large_grids(16, 555))
+def test_default_routing_on_matrices_of_many_rows(be, t, in_dim, out_dim, T, i):
+    """Row counts at which the launches outnumber the compute units: the few-token kernel's default range (Q6_K from
+    30 000 rows, 3 to 16 tokens) and the grids of more than 256 tiles of 128 x 128 that go to the plane kernel whose
+    waves all multiply, next to the kernels the other types take there."""
+    from orangu_amd import QuantMatrix
+    raw = synth_weights(t, in_dim, out_dim, seed=7000 + i)
+    x = synth_x(T, in_dim, seed=8000 + i)
+    w = QuantMatrix(np.ascontiguousarray(raw), t, in_dim, out_dim)
+    print("case", TYPE_NAME[t], in_dim, out_dim, T, flush=True)
+    try:
+        got = be.matmul(x, T, w)
+        k1 = be.last_kernel()
+        want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
+        bad = np.nonzero(bits(got) != bits(want))[0]
+        assert bad.size == 0, f"matmul via {k1}: {bad.size} of {want.size} differ, first {bad[:4]}"
+        print("  via", k1, flush=True)
+        if T <= 16:
+            got = be.matmul_decode(x, T, w)
+            want = oracle.matmul_decode(t, raw, in_dim, out_dim, x, T)
+            bad = np.nonzero(bits(got) != bits(want))[0]
+            assert bad.size == 0, f"matmul_decode via {be.last_kernel()}: {bad.size} of {want.size} differ"
+    finally:
+        be.evict(w)
