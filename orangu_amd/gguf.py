@@ -55,7 +55,7 @@ class GgufFile:
         rc = self._lib.ogm_gguf_tensor(self._h, index, C.byref(name), C.byref(nd), dims, C.byref(t), C.byref(off))
         if rc != 0:
             self._fail(rc, "ogm_gguf_tensor")
-        return name.value.decode(), list(dims[:nd.value]), t.value, off.value
+        return name.value.decode(errors="replace"), list(dims[:nd.value]), t.value, off.value   # (from_utf8_lossy, gguf.rs:384)
 
     def find_tensor(self, name: str) -> int:
         return self._lib.ogm_gguf_find_tensor(self._h, name.encode())

@@ -158,3 +158,116 @@ def test_open_from_a_file_at_an_offset(tmp_path):
         GgufFile(str(p))                       # no GGUF at offset 0
     with pytest.raises(OgmError):
         GgufFile(str(tmp_path / "absent.gguf"))
+
+
+def test_mutated_files_are_refused_or_read_without_leaving_the_buffer():
+    """The file is untrusted input: a seeded series of byte flips, truncations and overwritten lengths over a
+    file with every value type, nested arrays and three tensors with data.  Whatever the parser makes of one,
+    an error or a parse, every accessor afterwards answers from inside the buffer (a read outside it would
+    crash the test run); what parses must keep its own invariants."""
+    from orangu_amd import OgmError
+    rng = np.random.default_rng(20240612)
+    kvs = [kv("general.architecture", 8, gstr("llama")), kv("u8", 0, struct.pack("<B", 200)),
+           kv("i32", 5, struct.pack("<i", -7)), kv("f32", 6, struct.pack("<f", 1.5)), kv("bool", 7, b"\x01"),
+           kv("arr", 9, u32(4) + u64(3) + u32(1) + u32(2) + u32(3)),
+           kv("strs", 9, u32(8) + u64(3) + gstr("a") + gstr("bb") + gstr("ccc")),
+           kv("nested", 9, u32(9) + u64(2) + (u32(0) + u64(2) + b"\x01\x02") + (u32(8) + u64(1) + gstr("x"))),
+           kv("u64", 10, u64(1 << 40)), kv("f64", 12, struct.pack("<d", 1e-5)), kv("general.alignment", 4, u32(32))]
+    w8 = synth_weights(Q8_0, 64, 3, seed=1)
+    w4 = synth_weights(Q4_K, 256, 2, seed=2)
+    data = bytes(w8) + b"\0" * ((-len(w8)) % 32) + bytes(w4) + b"\0" * ((-len(w4)) % 32) + struct.pack("<8f", *range(8))
+    off4 = len(w8) + (-len(w8)) % 32
+    tensors = [tensor_info("a.weight", [64, 3], Q8_0, 0), tensor_info("b.weight", [256, 2], Q4_K, off4),
+               tensor_info("c", [8], 0, off4 + len(w4) + (-len(w4)) % 32)]
+    good, head_len = gguf(kvs, tensors, data=data)
+    g = open_bytes(good)
+    assert g.n_tensors == 3 and g.matrix("b.weight")[:3] == (Q4_K, 256, 2)
+    g.close()
+    keys = ["general.architecture", "u8", "i32", "f32", "bool", "arr", "strs", "nested", "u64", "f64", "general.alignment"]
+    parsed = refused = 0
+    for trial in range(12000):
+        b = bytearray(good)
+        kind = trial % 4
+        if kind == 0:      # a few flipped bytes in the header part
+            for _ in range(int(rng.integers(1, 6))):
+                b[int(rng.integers(0, head_len))] ^= int(rng.integers(1, 256))
+        elif kind == 1:    # cut anywhere
+            b = b[:int(rng.integers(0, len(b)))]
+        elif kind == 2:    # an aligned 8-byte field overwritten with a length that cannot be
+            pos = int(rng.integers(1, head_len // 8)) * 8
+            vals = [0xFFFFFFFFFFFFFFFF, 1 << 63, 1 << 32, (1 << 31) + 5, len(good), len(good) - 1]
+            b[pos:pos + 8] = struct.pack("<Q", vals[int(rng.integers(len(vals)))])
+        else:              # the same at an arbitrary position, and a flip in the data part's offsets
+            pos = int(rng.integers(4, head_len - 8))
+            vals = [0xFFFFFFFFFFFFFFFF, 1 << 62, 1 << 33, 0]
+            b[pos:pos + 8] = struct.pack("<Q", vals[int(rng.integers(len(vals)))])
+        try:
+            g = open_bytes(bytes(b))
+        except OgmError:
+            refused += 1
+            continue
+        parsed += 1
+        try:
+            assert g.n_tensors <= 1 << 20 and g.data_offset % max(g.alignment, 1) == 0
+            for k in keys:
+                g.meta_u64(k), g.meta_f64(k), g.meta_string(k), g.meta_array(k)
+            for i in range(min(g.n_tensors, 8)):
+                try:
+                    name, dims, t, off = g.tensor(i)
+                    d = g.tensor_data(i)
+                    assert g.data_offset + off + d.size <= len(b)
+                except OgmError:
+                    pass
+            for name in ("a.weight", "b.weight", "c", "nope"):
+                try:
+                    t, i_, o_, rb, raw = g.matrix(name)
+                    assert raw.size == rb * o_
+                except OgmError:
+                    pass
+        finally:
+            g.close()
+    assert parsed > 100 and refused > 100, (parsed, refused)
+
+
+def test_the_model_loader_under_sanitizers_on_mutated_model_files(tmp_path):
+    """ogm_gguf_parse + ogm_llama_load_gguf (read_model_config, loader.rs:1652-1714; load_with_backend,
+    llama.rs:123-220) over 20 000 seeded mutations of a small model file's header, compiled with AddressSanitizer and
+    UBSan beside a driver that stubs the uploads out and reads every byte range the loader hands them: no report,
+    and both outcomes -- refused, and parsed as far as the model's creation -- occur."""
+    import os
+    import shutil
+    import subprocess
+    import sys
+    if not shutil.which("g++"):
+        pytest.skip("no host compiler")
+    from oracle import llama_ref as R
+    from test_gpu_llama import model_gguf
+    from orangu_amd.gguf import GgufFile
+    f32 = np.float32
+    n_embd, n_head, n_kv, hd, n_ff, n_vocab = 256, 4, 2, 64, 256, 64
+    mk = lambda i, o, s: (Q8_0, synth_weights(Q8_0, i, o, seed=s), i, o)
+    L = R.Layer(mk(n_embd, n_head * hd, 1), mk(n_embd, n_kv * hd, 2), mk(n_embd, n_kv * hd, 3), mk(n_head * hd, n_embd, 4),
+                mk(n_embd, n_ff, 5), mk(n_embd, n_ff, 6), mk(n_ff, n_embd, 7), np.ones(n_embd, f32), np.ones(n_embd, f32))
+    L.q_bias = np.linspace(-1, 1, n_head * hd).astype(f32)
+    L.q_norm = np.ones(hd, f32)
+    m = R.Model(n_embd, n_head, n_kv, hd, n_ff, n_vocab, hd, 1e-5, 10000.0, [L], np.ones(n_embd, f32), mk(n_embd, n_vocab, 9),
+                rope_freq_factors=np.linspace(1, 2, hd // 2).astype(f32))
+    blob = model_gguf(m, "llama", tok_embd=mk(n_embd, n_vocab, 10))
+    g = GgufFile(data=blob)
+    head = g.data_offset
+    g.close()
+    path = tmp_path / "model.gguf"
+    path.write_bytes(blob)
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = str(tmp_path / "gguf_fuzz")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+                    "-o", exe, os.path.join(here, "gguf_fuzz_driver.cpp"),
+                    os.path.join(here, "..", "orangu_amd", "csrc", "ogm_gguf.cpp")], check=True)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")   # (a failed load leaves its uploads to ogm_destroy; the stubs' are never freed)
+    r = subprocess.run([exe, str(head), "20000", str(path)], capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-4000:])
+    import re
+    mo = re.search(r"parsed (\d+) refused (\d+), loader errors (\d+), uploads (\d+), creates reached (\d+)", r.stdout)
+    assert mo, r.stdout
+    parsed, refused, _, uploads, creates = map(int, mo.groups())
+    assert parsed > 1000 and refused > 1000 and uploads > parsed and creates > 100, r.stdout
