@@ -202,7 +202,7 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     pos += steps
     # prefill of a 512-token prompt from position 0 (GEMM matmuls, batch attention); the first
     # call allocates the batch buffers
-    dt_pre = dt_pre_long = None
+    dt_pre = dt_pre_long = dt_pre_long_one = None
     if with_prefill:
         prompt = rng.integers(0, n_vocab, 512).astype(np.uint32)
         dec.prefill_tokens(up("output"), prompt, 0)
@@ -215,6 +215,16 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
         t0 = time.perf_counter()
         dec.prefill_tokens(up("output"), long_prompt, 0)
         dt_pre_long = time.perf_counter() - t0
+        # the same 2048-token prompt with the Q4_K GEMMs' min pass folded into the super-block step (an option,
+        # off by default: f32 results not the reference's bits)
+        be.set_tuning("gemm_one_pass", 1)
+        try:
+            dec.prefill_tokens(up("output"), long_prompt, 0)
+            t0 = time.perf_counter()
+            dec.prefill_tokens(up("output"), long_prompt, 0)
+            dt_pre_long_one = time.perf_counter() - t0
+        finally:
+            be.set_tuning("gemm_one_pass", 0)
     weights = n_layer * sum(o * (i // 256) * (144 if t == Q4_K else 210) for t, i, o in shapes.values()) \
         + n_vocab * (n_embd // 256) * 210
     kv_bytes = 2 * n_layer * ctx * n_kv * hd * 2
@@ -225,6 +235,7 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
            "prefill_tok_per_s": round(512 / dt_pre, 1) if dt_pre else None,
            "prefill_2048_ms": round(dt_pre_long * 1e3, 2) if dt_pre_long else None,
            "prefill_2048_tok_per_s": round(2048 / dt_pre_long, 1) if dt_pre_long else None,
+           "prefill_2048_ms_one_pass_option": round(dt_pre_long_one * 1e3, 2) if dt_pre_long_one else None,
            "bytes_per_token": weights + kv_bytes,
            "GBps": round((weights + kv_bytes) / dt / 1e9, 1),
            "frac_of_hbm_peak": round((weights + kv_bytes) / dt / 1e9 / HBM_PEAK_GBS, 4)}
@@ -535,6 +546,20 @@ def main() -> int:
             gemm.update({"us_per_matmul": round(us_gemm, 1), "us_per_matmul_min": round(st_g["min"], 1),
                          "calls": st_g["launches"], "tops": round(flops / us_gemm / 1e6, 1),
                          "mfma_type": "i8", "frac_of_int8_mfma_peak": round(flops / us_gemm / 1e6 / 5000.0, 4)})
+            # the same call with the reference's separate min pass folded into the super-block step: an option,
+            # off by default, whose f32 results are not the reference's bits (same integer sums)
+            be.set_tuning("gemm_one_pass", 1)
+            try:
+                st_o = batched_us(hiprt, stream, lambda i: be.matmul_dev(handles["gate"][i % copies], xg.ptr, T,
+                                                                         yg.ptr, False, stream.ptr), 10, 4, warm=12)
+                gemm["one_pass_option"] = {"kernel": be.last_kernel(), "us_per_matmul": round(st_o["median"], 1),
+                                           "tops": round(flops / st_o["median"] / 1e6, 1),
+                                           "parity": "integer sums exact; f32 within 1e-3 * sum|w x| of the "
+                                                     "reference order, not its bits"}
+            finally:
+                be.set_tuning("gemm_one_pass", 0)
+            be.matmul_dev(handles["gate"][0], xg.ptr, T, yg.ptr, False, stream.ptr)   # what the parity check reads
+            stream.synchronize()
         if not args.only_gemm and args.cpu_seconds > 0:
             import oracle
             rows = np.r_[0:32, 7000:7032, FFN - 32:FFN]

@@ -404,6 +404,13 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * loads straight into LDS, when the launch has more than 256 tiles of 128 rows x 128 tokens, and otherwise
  * none: the feeding-wave kernels unpack; 1 = the feeding-wave kernels read them; 2 = the former whatever the
  * grid, from 32 tokens; same bits);
+ * "gemm_one_pass" (0 = default; 1: Q4_K and Q5_K on that kernel skip the reference GEMM's separate first pass over
+ * the mins (vecdot.rs:2229-2240) and add ad * (d * isum - dmin * imin) per super-block, the single-token
+ * expression of vecdot.rs:3152-3178: the integer sums are the same, the f32 result is no longer the reference
+ * GEMM's bits -- both orders sit about 1e-7 of sum|w x| from exact arithmetic, well inside the 1e-3 * sum|w x| the
+ * reference's tests allow between its two orders (vecdot.rs:3518-3525), but an output whose terms cancel to near
+ * zero can differ from the reference's by more than 1e-3 of itself; 4096 -> 14336 at 512 tokens: 94 against 112 us
+ * per call, a 2048-token prefill of the 8B shapes 38.2 against 42.8 ms);
  * "host_zero_copy" (1 = default: a host-pointer call -- ogm_matmul, ogm_matmul_decode, ogm_matmul_batch --
  * whose x and y together are at most 512 KiB runs its kernels directly on the pinned staging buffers, with
  * no copy-engine transfer: 23 us against 33 us per 4096 -> 14336 call; 0: always stage through device

@@ -64,6 +64,7 @@ struct ogm_ctx {
   int tune_gemm_sb_waves = 0;          // small-batch GEMM: 8 or 16 waves per workgroup, 0 = by the launch
   int tune_host_zero_copy = 1;         // host-pointer calls of up to OGM_ZERO_COPY_MAX bytes: kernels read x / write y in pinned host memory
   int tune_gemm_plane_kernel = 0;      // who reads planes: 0 the all-waves-multiply kernel on large grids, 1 the feeding-wave kernels, 2 the former always
+  int tune_gemm_one_pass = 0;          // 1: Q4_K / Q5_K on that kernel fold the min pass into the super-block step (f32 to rounding, not to the bit)
   int tune_decode_fuse_heads = 0;      // 1: the decode step's norms and SwiGLU at the head of the GEMV after them
   int tune_decode_head_delay = 64;     // fused heads: what the waiting workgroups sleep before their weight loads, x 64 clocks
   int tune_decode_head_spin = 0;       // fused heads: polls before a waiting workgroup gives up (0 = default)
@@ -283,6 +284,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemm_plane_kernel") == 0) {
     if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_kernel must be 0, 1 or 2");
     ctx->tune_gemm_plane_kernel = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_one_pass") == 0) {
+    if (value != 0 && value != 1) return fail(ctx, OGM_ERR_INVALID, "gemm_one_pass must be 0 or 1");
+    ctx->tune_gemm_one_pass = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_few_tokens_min_rows") == 0) {
@@ -617,6 +623,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.small_max_tokens = (uint32_t)ctx->tune_gemm_small_max;
       g.sb_waves = (uint32_t)ctx->tune_gemm_sb_waves;
       g.plane_kernel = (uint32_t)ctx->tune_gemm_plane_kernel;
+      g.one_pass = (uint32_t)ctx->tune_gemm_one_pass;
       g.n_extra = (uint32_t)ng - 1;
       for (size_t j = 1; j < ng; j++) {
         g.extra_wt[j - 1] = tg[i + j].w->dev;

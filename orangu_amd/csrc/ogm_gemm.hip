@@ -1398,6 +1398,10 @@ struct GemmDmaParams {
 #define GD_TAB (GD_RING * GD_SLOT)     // two slots of per-super-block tables: 128 ad, then the rows' header words
 #define GD_TAB_SLOT (512u + 4u * GD_ROWS)
 #define GD_LDS_BYTES (GD_TAB + 2u * GD_TAB_SLOT)
+// one-pass variant: 128 ad, the rows' 16-byte headers, the tokens' sums per 32 as f16 pairs (32 bytes a token)
+#define GD_RING_ONEPASS 5u
+#define GD_TAB_SLOT_ONEPASS (512u + 16u * GD_ROWS + 32u * GD_TOK)
+#define GD_LDS_BYTES_ONEPASS (GD_RING_ONEPASS * GD_SLOT + 2u * GD_TAB_SLOT_ONEPASS)
 
 __device__ __forceinline__ void gd_dma16(const uint8_t *src, uint8_t *lds_chunk) {
   // 16 bytes per lane from src (per lane) to lds_chunk + 16 * lane (lds_chunk is wave-uniform)
@@ -1453,9 +1457,16 @@ __global__ __launch_bounds__(256) void ogm_gemm_xtile_kernel(const int8_t *__res
 #else
 #define GD_RD
 #endif
-template <int KIND>
+// ONEPASS (Q4_K, Q5_K): no first pass; a super-block's step is acc += ad * (d * isum - dmin * imin), the
+// single-token expression (vecdot.rs:3152-3178), with imin from the same K = 16 f16 instruction.  The integer
+// sums are the same; the f32 result differs from the two-pass order by rounding only.  The rows' whole headers
+// and the tokens' sums per 32 then travel with the tables, and the ring is one step shorter to make room.
+template <int KIND, bool ONEPASS = false>
 __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaParams p) {
   constexpr bool Q3 = KIND == GP_Q3K, Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K, Q6 = KIND == GP_Q6K;
+  static_assert(!ONEPASS || Q45, "only the types with mins have a first pass to fold");
+  constexpr uint32_t RING = ONEPASS ? GD_RING_ONEPASS : GD_RING, AHEAD = RING - 1u;
+  constexpr uint32_t TAB = RING * GD_SLOT, TAB_SLOT = ONEPASS ? GD_TAB_SLOT_ONEPASS : GD_TAB_SLOT;
   constexpr uint32_t TILE_BYTES = Q3 ? 7168u : KIND == GP_Q4K ? 9216u : Q5 ? 11264u : 13440u;
   constexpr uint32_t NPL = Q3 ? 1u : 2u;
   constexpr int PER = (int)NPL + 1;   // loads a wave issues per step
@@ -1498,7 +1509,7 @@ __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaPara
 #pragma unroll
     for (int r = 0; r < 16; r++) y[tb][r] = 0.0f;
 
-  if constexpr (Q45 && !GD_ABL_NOPASS1) {
+  if constexpr (Q45 && !ONEPASS && !GD_ABL_NOPASS1) {
     // ---------------- pass 1 of gemm_k_q4_k: acc -= (ad * dmin) * sum_j m_j * bsum_j over all
     // super-blocks first (vecdot.rs:2226-2240), as gemm_q6k_i8_body does it: 64 m_j against bsum_j / 64
     // and m_j against bsum_j % 64 in one K = 16 f16 instruction per 32 x 32 outputs.  The tokens' ad of
@@ -1578,19 +1589,24 @@ __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaPara
     else                     // d | dmin
       tab_src = tab_rb * p.nct * TILE_BYTES + tab_r * 16u;
   }
+  // one-pass: token block `wave`'s sums per 32 (lane (l32, lh): the eight f16 of half lh of token l32)
+  const uint32_t bs_src = (min(t0 + 32u * wave + l32, p.n_tokens - 1u) * p.nsb * 16u + 8u * lh) * 2u;   // + 32 s
   auto fetch_tables = [&](uint32_t s) {   // for super-block s, into table slot s & 1
-    uint8_t *slot = lds + GD_TAB + (s & 1u) * GD_TAB_SLOT;
+    uint8_t *slot = lds + TAB + (s & 1u) * TAB_SLOT;
     if (wave < 2u) {
       gd_dma4((const uint8_t *)p.ad + (tab_src + 4u * s), slot + 256u * wave);
     } else {
       const uint32_t so = Q6 ? (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 2u : sb_off(s);
-      gd_dma4(p.wt + (tab_src + so), slot + 512u + 256u * (wave - 2u));
+      if constexpr (ONEPASS) gd_dma16(p.wt + (tab_src + so), slot + 512u + 1024u * (wave - 2u));
+      else gd_dma4(p.wt + (tab_src + so), slot + 512u + 256u * (wave - 2u));
     }
+    if constexpr (ONEPASS)
+      gd_dma16((const uint8_t *)p.bs16 + (bs_src + 32u * s), slot + 512u + 16u * GD_ROWS + 1024u * wave);
   };
   uint32_t slot_fetch = 0;   // byte offset of the ring slot of the next step to fetch
   auto fetch_step = [&]() {   // the next step (they are fetched in ascending order) into its ring slot
     uint8_t *slot = lds + slot_fetch;
-    slot_fetch = slot_fetch == (GD_RING - 1u) * GD_SLOT ? 0u : slot_fetch + GD_SLOT;
+    slot_fetch = slot_fetch == (RING - 1u) * GD_SLOT ? 0u : slot_fetch + GD_SLOT;
 #if !GD_ABL_NOWDMA
     gd_dma16(p.planes + w_src, slot + w_dst);
     if constexpr (!Q3) gd_dma16(p.planes + (w_src + 1024u), slot + w_dst + 1024u);
@@ -1604,13 +1620,15 @@ __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaPara
 
   fetch_tables(0u);
 #pragma unroll
-  for (uint32_t k = 0; k < GD_AHEAD; k++) fetch_step();
-  GD_SYNC((GD_AHEAD - 1) * PER);   // step 0 and the first tables have landed
+  for (uint32_t k = 0; k < AHEAD; k++) fetch_step();
+  GD_SYNC((AHEAD - 1) * PER);   // step 0 and the first tables have landed
 
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
   const uint32_t w_rd = lds0 + w_dst + lane * 16u, x_rd = lds0 + GD_XOFF + lane * 16u;
-  const uint32_t tab_rd = lds0 + GD_TAB + 16u * lh;                    // + 128 tb + 32 q4: four tokens' ad
-  const uint32_t hw_rd = lds0 + GD_TAB + 512u + 4u * (32u * wave + l32);   // the row's header word
+  const uint32_t tab_rd = lds0 + TAB + 16u * lh;                    // + 128 tb + 32 q4: four tokens' ad
+  // the row's header word (one-pass: its 16-byte header)
+  const uint32_t hw_rd = lds0 + TAB + 512u + (ONEPASS ? 16u : 4u) * (32u * wave + l32);
+  const uint32_t bs_rd = lds0 + TAB + 512u + 16u * GD_ROWS + 16u * lane;   // one-pass: + 1024 tb
   int16v h[4], l[4];
   const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   int4v wh, wl = {0, 0, 0, 0}, x0, x1, x2, x3;
@@ -1628,12 +1646,12 @@ __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaPara
       // step k = 8 s + kk: step k + 1 landed (all but the loads of the steps after it, at most four), for every wave
       const bool more = s + 1u < p.nsb;   // in the last super-block the steps in flight run out
       // (steps after k + 1 in flight: GD_AHEAD - 2, fewer at the end)
-      if (kk + GD_AHEAD <= 8u || more) GD_SYNC((GD_AHEAD - 2) * PER);
+      if (kk + AHEAD <= 8u || more) GD_SYNC((AHEAD - 2) * PER);
       else GD_SYNC(kk >= 6u ? 0 : (int)(6u - kk) * PER);
       if (kk == 0u && more) fetch_tables(s + 1u);
-      if ((kk + GD_AHEAD < 8u || more) && !GD_ABL_NODMA) fetch_step();   // step k + GD_AHEAD
+      if ((kk + AHEAD < 8u || more) && !GD_ABL_NODMA) fetch_step();   // step k + AHEAD
       const uint32_t w_nx = w_rd + slot_next, x_nx = x_rd + slot_next;
-      slot_next = slot_next == (GD_RING - 1u) * GD_SLOT ? 0u : slot_next + GD_SLOT;
+      slot_next = slot_next == (RING - 1u) * GD_SLOT ? 0u : slot_next + GD_SLOT;
       if constexpr (!Q3) {
         constexpr int A0 = 4;   // outstanding after wh and x0: x1, x2, x3, wl
         GD_WAIT2(A0, wh, x0);
@@ -1678,17 +1696,56 @@ __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaPara
       }
       if (kk == 7u && (!GD_ABL_NOEPI || s + 1u == p.nsb)) {
         // acc += ad * (d * isum) for the super-block (vecdot.rs:2242-2300 in the order of its sums)
-        const uint32_t tsl = (s & 1u) * GD_TAB_SLOT;
+        const uint32_t tsl = (s & 1u) * TAB_SLOT;
         uint32_t hw;
-        GD_READ4(hw, hw_rd + tsl, 0);
-        GD_WAIT1(0, hw);
+        half8 a1 = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (ONEPASS) {
+          int4v hd;
+          GD_READ16(hd, hw_rd + tsl, 0);
+          GD_WAIT1(0, hd);
+          hw = (uint32_t)hd.x;
+          uint32_t mna, mnb;
+          q4k_mins(make_uint4((uint32_t)hd.x, (uint32_t)hd.y, (uint32_t)hd.z, (uint32_t)hd.w), mna, mnb);
+          a1 = side_operand(mna, mnb, lh ? 1.0f : 64.0f);
+        } else {
+          GD_READ4(hw, hw_rd + tsl, 0);
+          GD_WAIT1(0, hw);
+        }
         // Q6_K's word holds the d of a pair of rows
         const float d0 = gm_f16_bits_to_f32(Q6 && (l32 & 1u) ? (hw >> 16) : (hw & 0xFFFFu));
+        const float ndm = -gm_f16_bits_to_f32(hw >> 16);   // one-pass: -dmin
         const uint32_t ta = tab_rd + tsl;
 #pragma unroll
         for (int tb = 0; tb < 4; tb++) {
           typedef float float4v __attribute__((ext_vector_type(4)));
           float4v a40, a41, a42, a43;
+          if constexpr (ONEPASS) {
+            // d * isum of the block's 16 outputs first (the integer sums die here), then imin into the registers
+            // they leave, then one multiply-add each for the mins and for the token's scale
+            half8 b2;
+            GD_READ16(b2, bs_rd + tsl, 1024 * tb);
+            float t[16];
+#pragma unroll
+            for (int r = 0; r < 16; r++) t[r] = d0 * (float)(h[tb][r] * 256 + l[tb][r]);
+            GD_WAIT1(0, b2);
+            const float16v zf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const float16v im = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2, a1, zf, 0, 0, 0);
+            GD_READ16(a40, ta, 128 * tb);
+            GD_READ16(a41, ta, 128 * tb + 32);
+            GD_READ16(a42, ta, 128 * tb + 64);
+            GD_READ16(a43, ta, 128 * tb + 96);
+            GD_WAIT2(0, a40, a41);
+            GD_WAIT2(0, a42, a43);
+            const float4v a4[4] = {a40, a41, a42, a43};
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+              const float a4v[4] = {a4[q4].x, a4[q4].y, a4[q4].z, a4[q4].w};
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                y[tb][4 * q4 + e] = __builtin_fmaf(a4v[e], __builtin_fmaf(ndm, im[4 * q4 + e], t[4 * q4 + e]), y[tb][4 * q4 + e]);
+            }
+            continue;
+          }
           GD_READ16(a40, ta, 128 * tb);
           GD_READ16(a41, ta, 128 * tb + 32);
           GD_READ16(a42, ta, 128 * tb + 64);
@@ -3354,20 +3411,24 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
         d.extra_out_dim[m] = p.extra_out_dim[m];
         if (m < a.n_extra) tiles256 += (a.extra_out_dim[m] + GD_ROWS - 1u) / GD_ROWS;
       }
+      const bool one_pass = q45 && a.one_pass != 0u;
       const void *fn = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_dma_kernel<GP_Q6K>
                        : a.ggml_type == OGM_Q3_K ? (const void *)ogm_gemm_dma_kernel<GP_Q3K>
-                       : a.ggml_type == OGM_Q4_K ? (const void *)ogm_gemm_dma_kernel<GP_Q4K>
-                                                 : (const void *)ogm_gemm_dma_kernel<GP_Q5K>;
-      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)GD_LDS_BYTES);
+                       : a.ggml_type == OGM_Q4_K ? (one_pass ? (const void *)ogm_gemm_dma_kernel<GP_Q4K, true>
+                                                             : (const void *)ogm_gemm_dma_kernel<GP_Q4K>)
+                                                 : (one_pass ? (const void *)ogm_gemm_dma_kernel<GP_Q5K, true>
+                                                             : (const void *)ogm_gemm_dma_kernel<GP_Q5K>);
+      const uint32_t dma_lds = one_pass ? GD_LDS_BYTES_ONEPASS : GD_LDS_BYTES;
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dma_lds);
       if (e != hipSuccess) return e;
       void *kargs[] = {(void *)&d};
-      e = hipLaunchKernel(fn, dim3((a.n_tokens + GD_TOK - 1u) / GD_TOK, tiles256), dim3(64u * GD_NW), kargs, GD_LDS_BYTES, stream);
+      e = hipLaunchKernel(fn, dim3((a.n_tokens + GD_TOK - 1u) / GD_TOK, tiles256), dim3(64u * GD_NW), kargs, dma_lds, stream);
       if (e != hipSuccess) return e;
       if (kernel_name)
         *kernel_name = a.ggml_type == OGM_Q6_K   ? "ogm_gemm_q6k_dma_kernel"
                        : a.ggml_type == OGM_Q3_K ? "ogm_gemm_q3k_dma_kernel"
-                       : a.ggml_type == OGM_Q4_K ? "ogm_gemm_q4k_dma_kernel"
-                                                 : "ogm_gemm_q5k_dma_kernel";
+                       : a.ggml_type == OGM_Q4_K ? (one_pass ? "ogm_gemm_q4k_dma_onepass_kernel" : "ogm_gemm_q4k_dma_kernel")
+                                                 : (one_pass ? "ogm_gemm_q5k_dma_onepass_kernel" : "ogm_gemm_q5k_dma_kernel");
       return hipGetLastError();
     }
     // 64-row tiles when asked for (q4k_variant 1), or when they still come one to a CU: then twice

@@ -141,6 +141,7 @@ struct OgmGemmArgs {
   // grid fills the device twice, else none (the feeding waves unpack); 1 the feeding-wave kernels; 2
   // the former whatever the grid
   uint32_t plane_kernel = 0;
+  uint32_t one_pass = 0;   // Q4_K / Q5_K on the all-waves-multiply kernel: fold the min pass into the super-block step (f32 to rounding, not to the bit)
 };
 // Whether this launch would run a tiled int8 plane kernel, i.e. whether planes would be read.
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a);
