@@ -140,3 +140,16 @@ def test_init_without_a_device_is_a_status_not_a_crash(lib):
     # null-context calls return a status
     assert lib.ogm_matmul(None, None, None, 1, None) == -1
     assert lib.ogm_set_tuning(None, b"gemv_wg_waves", 1) == -1
+
+
+def test_every_tuning_key_the_library_accepts_is_documented_in_the_header():
+    """ogm_set_tuning's keys are compared by name in ogm_api.cpp; the header is where a host maintainer
+    reads what each one does."""
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = open(os.path.join(root, "orangu_amd", "csrc", "ogm_api.cpp")).read()
+    header = open(os.path.join(root, "include", "orangu_mi355x.h")).read()
+    keys = re.findall(r'strcmp\(key, "([a-z0-9_]+)"\)', src)
+    assert len(keys) >= 20 and len(set(keys)) == len(keys)
+    missing = [k for k in keys if f'"{k}"' not in header]
+    assert not missing, missing
