@@ -333,6 +333,8 @@ def main() -> int:
     ap.add_argument("--gemm-tokens", type=int, default=512,
                     help="tokens of the prefill GEMM leg (Q4_K 4096 -> 14336 on MFMA); 0 skips it")
     ap.add_argument("--only-gemm", action="store_true", help="run only the prefill GEMM leg (for rocprofv3)")
+    ap.add_argument("--gemm-one-pass", action="store_true",
+                    help="with --only-gemm: the one-pass option of the large-grid kernel (tuning key gemm_one_pass)")
     ap.add_argument("--decode-steps", type=int, default=64,
                     help="tokens of the 8B-shaped decode leg (config 5); 0 skips it")
     ap.add_argument("--decode-ctx", type=int, default=2048, help="cached positions of the decode leg")
@@ -530,6 +532,7 @@ def main() -> int:
         yg = hiprt.DeviceBuffer(4 * T * FFN)
         st_g = None
         if args.only_gemm:
+            be.set_tuning("gemm_one_pass", 1 if args.gemm_one_pass else 0)
             for i in range(5):
                 be.matmul_dev(handles["gate"][i % copies], xg.ptr, T, yg.ptr, False, stream.ptr)
             stream.synchronize()
