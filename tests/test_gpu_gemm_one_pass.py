@@ -125,3 +125,49 @@ def test_one_pass_is_refused_nothing_and_changes_nothing_elsewhere(be):
     finally:
         be.set_tuning("gemm_one_pass", 0)
         be.set_tuning("gemm_plane_kernel", 2)
+
+
+def test_one_pass_over_several_matrices_in_one_launch(be):
+    """gate and up read the same rows and share one launch (arch/mod.rs:1082-1096): with the option on, each
+    matrix's result is what the matrix alone gives, bit for bit (the same kernel arithmetic per row tile)."""
+    from orangu_amd import MatmulOp, QuantMatrix
+    in_dim, T = 1024, 200
+    x = synth_x(T, in_dim, seed=3)
+    ws = [QuantMatrix(np.ascontiguousarray(synth_weights(Q4_K, in_dim, o, seed=40 + o)), Q4_K, in_dim, o)
+          for o in (300, 257, 128)]
+    be.set_tuning("gemm_one_pass", 1)
+    try:
+        alone = []
+        for w in ws:
+            alone.append(np.asarray(be.matmul(x, T, w)))
+            assert be.last_kernel() == "ogm_gemm_q4k_dma_onepass_kernel"
+        together = be.matmul_batch([MatmulOp(x, T, w) for w in ws])
+        assert be.last_kernel() == "ogm_gemm_q4k_dma_onepass_kernel"
+    finally:
+        be.set_tuning("gemm_one_pass", 0)
+    for a, b in zip(alone, together):
+        assert np.array_equal(a.reshape(-1).view(np.uint32), np.asarray(b).reshape(-1).view(np.uint32))
+
+
+def test_a_prefill_with_one_pass_gemms_holds_the_models_tolerance(be):
+    """run_layers over a batch (llama.rs:594-932) with the Q4_K projections' GEMMs in the one-pass order: hidden
+    state and logits within the model tests' 2e-4 of the largest magnitude of the CPU restatement, same greedy
+    token, and the decode steps after it continue on the cache it wrote."""
+    from test_gpu_llama import TAME, build, prefill_both, step_both
+    f32 = np.float32
+    ref, dev, rng = build(be, n_embd=512, n_head=4, n_kv=2, hd=128, n_ff=1024, n_vocab=320, n_layer=2,
+                          types=(Q4_K, Q4_K, Q4_K, Q4_K), max_ctx=256, seed=77, attn_norm_scale=TAME[Q4_K])
+    be.set_tuning("gemm_one_pass", 1)
+    try:
+        X = rng.standard_normal((150, 512)).astype(f32)
+        prefill_both(ref, dev, X, 0, "one-pass prefill")
+        step_both(ref, dev, rng.standard_normal(512).astype(f32), 150, "then a decode step")
+        # the option did reach the batch's GEMMs: the same prompt without it ends in other bits
+        one = np.asarray(dev.prefill(X, 0)[0]).copy()
+        be.set_tuning("gemm_one_pass", 0)
+        two = np.asarray(dev.prefill(X, 0)[0])
+        assert not np.array_equal(one.view(np.uint32), two.view(np.uint32))
+        assert np.abs(one - two).max() <= 2e-4 * np.abs(two).max()
+    finally:
+        be.set_tuning("gemm_one_pass", 0)
+        dev.close()
