@@ -1634,3 +1634,20 @@ hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hip
                      n, out);
   return hipGetLastError();
 }
+
+// ------------------------------------------------------------------------------------------
+// A word in pinned host memory that tells a polling host thread that everything enqueued on the stream
+// before this launch has finished: a kernel starts only after its predecessors on the stream have completed
+// and their stores have been acknowledged, and the store below goes out at system scope behind a fence.
+__global__ __launch_bounds__(64) void ogm_host_flag_kernel(uint32_t *flag, uint32_t value) {
+  if (threadIdx.x == 0) {
+    __threadfence_system();
+    __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+hipError_t ogm_launch_host_flag(uint32_t *flag, uint32_t value, hipStream_t stream) {
+  if (!flag) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ogm_host_flag_kernel, dim3(1), dim3(64), 0, stream, flag, value);
+  return hipGetLastError();
+}
