@@ -418,7 +418,8 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * "host_flag_wait" (1 = default: such a call waits for its results by polling a word in pinned memory that a
  * one-thread kernel behind the call's kernels stores, instead of waiting on the stream: 19 us against 23 us per
  * 4096 -> 14336 call; after 5 ms without the word, and on every 256th call, the stream is synchronized after all;
- * 0: always hipStreamSynchronize);
+ * 0: always hipStreamSynchronize; 2: for tests of the bounded wait, the word never matches and every call runs
+ * into the 5 ms);
  * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
  * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
  * the quantizer kernel first; 0 or -1 = default, off);

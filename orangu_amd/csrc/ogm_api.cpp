@@ -281,7 +281,7 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     return OGM_OK;
   }
   if (strcmp(key, "host_flag_wait") == 0) {
-    if (value != 0 && value != 1) return fail(ctx, OGM_ERR_INVALID, "host_flag_wait must be 0 or 1");
+    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "host_flag_wait must be 0, 1 or 2");
     ctx->tune_host_flag_wait = value;
     return OGM_OK;
   }
@@ -722,7 +722,8 @@ static int host_wait(ogm_ctx *ctx, bool zero_copied) {
   }
   const uint32_t epoch = ++ctx->flag_epoch;
   uint32_t *flag = (uint32_t *)ctx->hflag.p;
-  HIPCHK(ctx, ogm_launch_host_flag(flag, epoch, ctx->stream));
+  // (2: the kernel stores another number, so the wait below runs into its bound -- for tests of that path)
+  HIPCHK(ctx, ogm_launch_host_flag(flag, ctx->tune_host_flag_wait == 2 ? epoch ^ 0x80000000u : epoch, ctx->stream));
   const auto t0 = std::chrono::steady_clock::now();
   for (uint32_t spins = 0; __atomic_load_n(flag, __ATOMIC_ACQUIRE) != epoch; spins++) {
     __builtin_ia32_pause();

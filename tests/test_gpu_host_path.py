@@ -68,3 +68,24 @@ def test_batches_and_single_calls_interleave(be):
             assert np.array_equal(np.asarray(got).reshape(-1).view(np.uint32), want.view(np.uint32)), rep
         got = np.asarray(be.matmul(c[1], c[2], c[0])).reshape(-1)
         assert np.array_equal(got.view(np.uint32), c[3].view(np.uint32)), rep
+
+
+def test_a_word_that_never_comes_ends_in_a_stream_synchronization(be):
+    """The poll is bounded: with the trailing kernel made to store another number (host_flag_wait 2) every call
+    runs into the bound, synchronizes the stream after all and still returns the finished result."""
+    import time
+    pairs = _pairs()
+    be.set_tuning("host_flag_wait", 2)
+    try:
+        for k in (0, 3, 5):
+            w, x, T, want = pairs[k]
+            t0 = time.perf_counter()
+            got = np.asarray(be.matmul(x, T, w), np.float32).reshape(-1)
+            dt = time.perf_counter() - t0
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+            assert 0.004 < dt < 1.0, dt
+    finally:
+        be.set_tuning("host_flag_wait", 1)
+    w, x, T, want = pairs[1]
+    got = np.asarray(be.matmul(x, T, w), np.float32).reshape(-1)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
