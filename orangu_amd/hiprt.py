@@ -54,6 +54,13 @@ def device_synchronize():
     check(hip().hipDeviceSynchronize(), "hipDeviceSynchronize")
 
 
+def mem_get_info():
+    """(free, total) bytes of the current device."""
+    free, total = C.c_size_t(), C.c_size_t()
+    check(hip().hipMemGetInfo(C.byref(free), C.byref(total)), "hipMemGetInfo")
+    return free.value, total.value
+
+
 class DeviceBuffer:
     def __init__(self, nbytes: int):
         self.nbytes = nbytes
