@@ -89,3 +89,35 @@ def test_a_word_that_never_comes_ends_in_a_stream_synchronization(be):
     w, x, T, want = pairs[1]
     got = np.asarray(be.matmul(x, T, w), np.float32).reshape(-1)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_several_backends_in_one_process_run_side_by_side():
+    """Each context has its own stream, staging buffers and completion word: four of them, each driven by a thread
+    of its own over its own weights, return their own results (the reference's backends are per-model objects,
+    backend/mod.rs:309-312)."""
+    import threading
+    from orangu_amd import Mi355xBackend
+    pairs = _pairs()
+    backends = [Mi355xBackend() for _ in range(4)]
+    errors = []
+
+    def worker(k):
+        try:
+            b = backends[k]
+            for n in range(400):
+                w, x, T, want = pairs[(n + 2 * k) % len(pairs)]
+                got = np.asarray(b.matmul(x, T, w), np.float32).reshape(-1)
+                if not np.array_equal(got.view(np.uint32), want.view(np.uint32)):
+                    errors.append((k, n))
+                    return
+        except Exception as e:   # noqa: BLE001 - reported below
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for b in backends:
+        b.close()
+    assert not errors, errors
