@@ -14,6 +14,49 @@
 
 __device__ __forceinline__ float ogm_nan_blind_max(float m, float a) { return a > m ? a : m; }
 
+// One step of a butterfly all-reduce over the wave: joins groups of M lanes pairwise with a commutative
+// `op`.  For a value that is already equal within each group of M lanes (the state of a butterfly after its
+// steps 1 .. M / 2) any lane of the partner group serves, which lets the steps stay in the vector pipe --
+// quad permutes, the row mirrors, and gfx950's swaps of 16- and 32-lane halves -- instead of going through
+// LDS addressing (ds_bpermute) sixty-odd clocks at a time.  Same pairs as `v op shfl_xor(v, M)`: same bits.
+template <int M, class Op>
+__device__ __forceinline__ float ogm_butterfly_step(float v, Op op) {
+  typedef unsigned ogm_u2 __attribute__((ext_vector_type(2)));
+  if constexpr (M == 1) {
+    return op(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true)));   // quad_perm 1,0,3,2
+  } else if constexpr (M == 2) {
+    return op(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true)));   // quad_perm 2,3,0,1
+  } else if constexpr (M == 4) {
+    return op(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true)));  // row_half_mirror
+  } else if constexpr (M == 8) {
+    return op(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true)));  // row_mirror
+  } else if constexpr (M == 16) {
+    const ogm_u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return op(__uint_as_float(r.x), __uint_as_float(r.y));   // every lane: its pair of rows' two values
+  } else {
+    static_assert(M == 32, "a wave has 64 lanes");
+    const ogm_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return op(__uint_as_float(r.x), __uint_as_float(r.y));
+  }
+}
+template <int M>
+__device__ __forceinline__ int ogm_butterfly_add_i32(int v) {
+  static_assert(M == 1 || M == 2 || M == 4, "the quantizer's sums stop at eight lanes");
+  constexpr int CTRL = M == 1 ? 0xB1 : M == 2 ? 0x4E : 0x141;
+  return v + __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+struct OgmOpAdd { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+struct OgmOpNanBlindMax { __device__ __forceinline__ float operator()(float a, float b) const { return ogm_nan_blind_max(a, b); } };
+// v summed over the wave, in the butterfly's order: ((lane + lane^1) + ...) level by level
+__device__ __forceinline__ float ogm_wave_sum(float v) {
+  v = ogm_butterfly_step<1>(v, OgmOpAdd());
+  v = ogm_butterfly_step<2>(v, OgmOpAdd());
+  v = ogm_butterfly_step<4>(v, OgmOpAdd());
+  v = ogm_butterfly_step<8>(v, OgmOpAdd());
+  v = ogm_butterfly_step<16>(v, OgmOpAdd());
+  return ogm_butterfly_step<32>(v, OgmOpAdd());
+}
+
 __device__ __forceinline__ int ogm_quantize_one(float v, float inv) {
   float r = roundf(v * inv);
   if (r != r) r = 0.0f;
@@ -32,17 +75,26 @@ __device__ __forceinline__ uint32_t ogm_quantize4(const float4 &v, float &scale,
   amax = ogm_nan_blind_max(amax, fabsf(v.y));
   amax = ogm_nan_blind_max(amax, fabsf(v.z));
   amax = ogm_nan_blind_max(amax, fabsf(v.w));
-#pragma unroll
-  for (int m = 1; m < GROUP / 4; m <<= 1) amax = ogm_nan_blind_max(amax, __shfl_xor(amax, m, 64));
+  // (no lane's amax is NaN -- the fold starts at 0 and skips them -- so the max commutes)
+  amax = ogm_butterfly_step<1>(amax, OgmOpNanBlindMax());
+  amax = ogm_butterfly_step<2>(amax, OgmOpNanBlindMax());
+  amax = ogm_butterfly_step<4>(amax, OgmOpNanBlindMax());
+  if constexpr (GROUP == 256) {
+    amax = ogm_butterfly_step<8>(amax, OgmOpNanBlindMax());
+    amax = ogm_butterfly_step<16>(amax, OgmOpNanBlindMax());
+    amax = ogm_butterfly_step<32>(amax, OgmOpNanBlindMax());
+  } else {
+    static_assert(GROUP == 32, "groups of 32 or 256");
+  }
   scale = amax / 127.0f;
   const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
   const int q0 = ogm_quantize_one(v.x, inv), q1 = ogm_quantize_one(v.y, inv);
   const int q2 = ogm_quantize_one(v.z, inv), q3 = ogm_quantize_one(v.w, inv);
   int s = q0 + q1 + q2 + q3;
-  s += __shfl_xor(s, 1, 64);
-  s += __shfl_xor(s, 2, 64);
+  s = ogm_butterfly_add_i32<1>(s);
+  s = ogm_butterfly_add_i32<2>(s);
   s16 = s;
-  s32 = s + __shfl_xor(s, 4, 64);
+  s32 = ogm_butterfly_add_i32<4>(s);
   return (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
          ((uint32_t)(q3 & 0xFF) << 24);
 }
@@ -130,8 +182,7 @@ __device__ __forceinline__ void ogm_norm_quant_row(float *__restrict__ x, const 
 #pragma unroll
   for (int k = 0; k < 4; k++) {
     if ((wave + k * n_wave) * 256u < n) {   // wave-uniform: the run exists
-#pragma unroll
-      for (int m = 1; m < 64; m <<= 1) ss[k] += __shfl_xor(ss[k], m, 64);
+      ss[k] = ogm_wave_sum(ss[k]);
       if (lane == 0) red[wave + k * n_wave] = ss[k];
     }
   }
