@@ -294,8 +294,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
         ss += a[j] * a[j] + b[j] * b[j];
       }
       if (nw != nullptr) {
-#pragma unroll
-        for (int k = 1; k < 64; k <<= 1) ss += __shfl_xor(ss, k, 64);
+        ss = ogm_wave_sum(ss);
         const float sc_n = 1.0f / sqrtf(ss / (float)HD + pre.eps);
 #pragma unroll
         for (int j = 0; j < PPL; j++) {
@@ -379,11 +378,11 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
         for (int i = 0; i < n; i++) {
           float lo = acc[i], hi = acc[n + i];
           asm volatile("" : "+v"(lo), "+v"(hi));   // keeps the selects on values, not on array slots
-          acc[i] = (up ? hi : lo) + __shfl_xor(up ? lo : hi, b, 64);
+          acc[i] = (up ? hi : lo) + (b == 1 ? ogm_quad_xor<1>(up ? lo : hi) : ogm_quad_xor<2>(up ? lo : hi));
         }
         g0 += up ? n : 0;
       } else {
-        acc[0] += __shfl_xor(acc[0], b, 64);
+        acc[0] += b == 1 ? ogm_quad_xor<1>(acc[0]) : ogm_quad_xor<2>(acc[0]);
         owner = owner && !up;
       }
     }
@@ -393,9 +392,10 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
 #pragma unroll
   for (int i = 0; i < NF; i++) {
     sv[i] = valid ? acc[i] * scale : -INFINITY;
-    float m = sv[i];
-#pragma unroll
-    for (int k = 4; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
+    // over the wave's sixteen rows of four lanes, lane by lane of the row
+    float m = ogm_row_quads_allreduce(sv[i], OgmOpMax());
+    m = ogm_butterfly_step<16>(m, OgmOpMax());
+    m = ogm_butterfly_step<32>(m, OgmOpMax());
     if (lane < 4u && owner) red[0][g0 + i][wave] = m;
   }
   __syncthreads();
@@ -407,9 +407,9 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
     mv[i] = m;
     const float e = valid ? expf(sv[i] - m) : 0.0f;
     if (owner) sc[g0 + i][r] = e;
-    float l = e;
-#pragma unroll
-    for (int k = 4; k < 64; k <<= 1) l += __shfl_xor(l, k, 64);
+    float l = ogm_row_quads_allreduce(e, OgmOpAdd());
+    l = ogm_butterfly_step<16>(l, OgmOpAdd());
+    l = ogm_butterfly_step<32>(l, OgmOpAdd());
     if (lane < 4u && owner) red[1][g0 + i][wave] = l;
   }
   __syncthreads();
@@ -462,7 +462,9 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
       for (int i = 0; i < n; i++) {
         float lo = o[i], hi = o[n + i];
         asm volatile("" : "+v"(lo), "+v"(hi));   // keeps the selects on values, not on array slots
-        o[i] = (up ? hi : lo) + __shfl_xor(up ? lo : hi, b, 64);
+        const float send = up ? lo : hi;
+        o[i] = (up ? hi : lo) + (b == 16 ? ogm_half_xor<16>(send, up) : b == 32 ? ogm_half_xor<32>(send, up)
+                                                                                 : __shfl_xor(send, b, 64));
       }
       sel += up ? n : 0;
     }
@@ -949,8 +951,7 @@ __global__ __launch_bounds__(256) void ogm_qkv_pre_kernel(float *__restrict__ q,
     ss += a[j] * a[j] + b[j] * b[j];
   }
   if (nw != nullptr) {
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) ss += __shfl_xor(ss, m, 64);
+    ss = ogm_wave_sum(ss);
     const float sc_n = 1.0f / sqrtf(ss / (float)HD + pre.eps);
 #pragma unroll
     for (int j = 0; j < PPL; j++) {
@@ -1129,7 +1130,7 @@ __global__ __launch_bounds__(512, 2) void ogm_attn_prefill_mfma_kernel(const flo
       amax = fmaxf(amax, fmaxf(fmaxf(fabsf(qa[s].x), fabsf(qa[s].y)), fmaxf(fabsf(qa[s].z), fabsf(qa[s].w))));
       amax = fmaxf(amax, fmaxf(fmaxf(fabsf(qb[s].x), fabsf(qb[s].y)), fmaxf(fabsf(qb[s].z), fabsf(qb[s].w))));
     }
-    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));   // the row's other dimensions are in the other lane half
+    amax = ogm_butterfly_step<32>(amax, OgmOpMax());   // the row's other dimensions are in the other lane half
     float down = 1.0f;
     if (amax >= 16384.0f && amax < INFINITY) {
       const int k = (int)((__float_as_uint(amax) >> 23) & 0xFFu) - 127 - 13;   // amax * 2^-k in [2^13, 2^14)
@@ -1254,7 +1255,7 @@ __global__ __launch_bounds__(512, 2) void ogm_attn_prefill_mfma_kernel(const flo
           mt = fmaxf(mt, fmaxf(s0[r], s1[r]));
         }
       }
-      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      mt = ogm_butterfly_step<32>(mt, OgmOpMax());
       // (a query may see nothing of the odd half's first tile: then everything stays at zero)
       const float m_max = fmaxf(m_run, mt);
       const float m_new = m_max == -INFINITY ? 0.0f : m_max;
@@ -1317,7 +1318,7 @@ __global__ __launch_bounds__(512, 2) void ogm_attn_prefill_mfma_kernel(const flo
       for (int r = 0; r < 16; r++) o[d][r] = o[d][r] * a0 + mrg[(16u * d + r) * 256u + slot] * a1;
   }
   if (live && 32u * qt + l32 < n_tokens) {
-    const float l = l_run + __shfl_xor(l_run, 32, 64);
+    const float l = ogm_butterfly_step<32>(l_run, OgmOpAdd());
     float *op = attn_out + ((size_t)tok * n_head + (size_t)kvh * gq + g) * HD + 4u * lh;
 #pragma unroll
     for (int d = 0; d < NDB; d++)

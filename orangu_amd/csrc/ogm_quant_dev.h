@@ -45,6 +45,31 @@ __device__ __forceinline__ int ogm_butterfly_add_i32(int v) {
   constexpr int CTRL = M == 1 ? 0xB1 : M == 2 ? 0x4E : 0x141;
   return v + __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
 }
+// The value lane ^ M holds, for M = 1 or 2 (any values: a quad permute is a true exchange).
+template <int M>
+__device__ __forceinline__ float ogm_quad_xor(float v) {
+  static_assert(M == 1 || M == 2, "within a quad");
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), M == 1 ? 0xB1 : 0x4E, 0xF, 0xF, true));
+}
+// The value lane ^ M holds, for M = 16 or 32 (any values: the half swaps exchange lanes at equal positions);
+// upper = whether this lane has bit M set.
+template <int M>
+__device__ __forceinline__ float ogm_half_xor(float v, bool upper) {
+  typedef unsigned ogm_u2 __attribute__((ext_vector_type(2)));
+  static_assert(M == 16 || M == 32, "rows of 16 or halves of 32");
+  ogm_u2 r;
+  if constexpr (M == 16) r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  else r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(upper ? r.x : r.y);
+}
+// op over the four quads of a row of 16 lanes, lane by lane of the quads (values may differ within a quad):
+// two rotations of the row.  Quad 0 ends with (q0 op q1) op (q2 op q3), the butterfly's order.
+template <class Op>
+__device__ __forceinline__ float ogm_row_quads_allreduce(float v, Op op) {
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x12C, 0xF, 0xF, true)));   // row_ror:12 = from lane + 4
+  return op(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true)));   // row_ror:8
+}
+struct OgmOpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 struct OgmOpAdd { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 struct OgmOpNanBlindMax { __device__ __forceinline__ float operator()(float a, float b) const { return ogm_nan_blind_max(a, b); } };
 // v summed over the wave, in the butterfly's order: ((lane + lane^1) + ...) level by level
