@@ -1146,6 +1146,7 @@ struct ogm_llama {
   float *pre = nullptr;       // [n_layer][q_bias qd | k_bias kvd | v_bias kvd | q_norm hd | k_norm hd]
   float *freq = nullptr;      // [rope_dim / 2], frequency factors applied
   float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
+  float *rope_all = nullptr;  // the same for every position of the cache, filled at creation (null: too large, computed per token)
   uint32_t head_epoch = 0;            // value of the GEMV heads' flag (the three words after the tickets) after the last launch
   uint32_t *attn_tickets = nullptr;   // [2 n_head_kv] the attention kernel's, then the GEMV tails' tickets and the heads' flags; zero between launches
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
@@ -1242,6 +1243,10 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   A((void **)&m->pre, (size_t)c.n_layer * pre_stride * 4);
   A((void **)&m->freq, (size_t)(c.rope_dim / 2 + 1) * 4);
   A((void **)&m->rope_cs, (size_t)(c.rope_dim / 2 + 1) * 8);
+  // every position's rotation table once, where it stays small (64 pairs x 8 bytes x the context: 4 MiB at 8192
+  // positions); a decode step then launches no table kernel
+  const size_t rope_all_bytes = (size_t)c.max_ctx * (c.rope_dim / 2) * 8;
+  if (c.rope_dim != 0 && rope_all_bytes <= ((size_t)64 << 20)) A((void **)&m->rope_all, rope_all_bytes);
   A((void **)&m->attn_tickets, ((size_t)2 * c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);   // + the GEMV tails' tickets
   A(&m->k_cache, cache_bytes);
   A(&m->v_cache, cache_bytes);
@@ -1298,6 +1303,11 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, ((size_t)2 * c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
+  for (uint32_t p0 = 0; m->rope_all && e == hipSuccess && p0 < c.max_ctx; p0 += 32768u) {
+    const uint32_t np = c.max_ctx - p0 < 32768u ? c.max_ctx - p0 : 32768u;
+    e = ogm_launch_rope_table(m->freq, p0, np, c.rope_dim, m->rope_all + (size_t)p0 * (c.rope_dim / 2) * 2, ctx->stream);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   if (e != hipSuccess) {
     llama_free(m);
     return fail(ctx, OGM_ERR_HIP, std::string("ogm_llama_create: ") + hipGetErrorString(e));
@@ -1407,8 +1417,9 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   if (pos >= c.max_ctx) return fail(ctx, OGM_ERR_INVALID, "position beyond the KV cache");
   const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
   const float scale = 1.0f / sqrtf((float)c.head_dim);
-  if (x_dev != m->x) HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
-  HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos, 1, c.rope_dim, m->rope_cs, s));
+  // (the table of this position: from the one made at creation, or computed now)
+  const float *rope_cs = m->rope_all ? m->rope_all + (size_t)pos * (c.rope_dim / 2) * 2 : m->rope_cs;
+  if (!m->rope_all) HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos, 1, c.rope_dim, m->rope_cs, s));
   const float *delta = nullptr;  // what the next norm adds to x first: the last block's output
   // On request, with per-256 activations on the consumer's side, a norm or the SwiGLU runs as the
   // tail of the GEMV launch before it (its last workgroup to finish) instead of as a kernel of its
@@ -1428,6 +1439,13 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   // polled, activations loaded) that costs what the kernel boundary it replaces costs, and the
   // producers' own loads queue behind the launch's weight stream.
   const bool heads = ctx->tune_decode_fuse_heads != 0 && !fuse && ctx->tune_fuse_quant <= 0;
+  // The caller's row becomes the residual stream: the first norm reads it where it lies and stores it to
+  // m->x, unless that norm runs inside a GEMV launch, which works on m->x alone.
+  const float *x_first = nullptr;
+  if (x_dev != m->x) {
+    if (fuse || heads) HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
+    else x_first = x_dev;
+  }
   uint32_t *head_flag = m->attn_tickets + ((2u * c.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u);   // 128-byte aligned
   auto head_ok = [&](const ogm_weight *first, int mode, bool norm) {   // first: the matrix of the group's first launch
     if (!heads || mode != OGM_ACT_PER_256) return false;
@@ -1471,13 +1489,13 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     } else {
       if (!normed)
         HIPCHK(ctx, ogm_launch_norm_quant(mode_qkv, m->x, delta, attn_norm, c.n_embd, c.rms_eps, nullptr,
-                                          act_view(ctx, c.n_embd, mode_qkv, 0), s));
+                                          act_view(ctx, c.n_embd, mode_qkv, 0), s, 1, l == 0 ? x_first : nullptr));
       if ((rc = llama_capture(ctx, m, 4 * l, c.n_embd, mode_qkv, s)) != OGM_OK) return rc;
       if ((rc = llama_matmul(ctx, w3, y3, 3, s)) != OGM_OK) return rc;
     }
     const int mode_o = act_mode_for(L.wo->ggml_type);
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
-    HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, m->rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
+    HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
                                        c.n_head, c.n_head_kv, c.head_dim, scale, m->part_o, m->part_ml,
                                        m->attn_tickets, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s, 0u,
                                        ctx->tune_attn_decode_share == 2 ? 0u : 1u));   // 0: wherever the shape allows

@@ -17,7 +17,8 @@
 // also stored when not null.  n <= 16384, n % 32 == 0.  With n_rows > 1: that many rows of x, delta,
 // normed and act, one workgroup each.
 hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const float *weight, uint32_t n,
-                                 float eps, float *normed, OgmActDev act, hipStream_t stream, uint32_t n_rows = 1);
+                                 float eps, float *normed, OgmActDev act, hipStream_t stream, uint32_t n_rows = 1,
+                                 const float *x_src = nullptr);   // x_src: the rows are read from there and stored to x
 
 // cos / sin of pos * freq[p] for the rope_dim / 2 rotated pairs, as float2 (cos, sin): once per
 // token, every layer rotates by the same angles (tensor.rs:1147-1160, freq_scale 1, no YaRN;

@@ -23,12 +23,13 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
                                                               const float *__restrict__ delta,
                                                               const float *__restrict__ weight, uint32_t n,
                                                               float eps, float *__restrict__ normed,
-                                                              OgmActDev act) {
+                                                              OgmActDev act, const float *__restrict__ x_src) {
   __shared__ float red[64];
   const uint32_t tid = threadIdx.x, n_wave = blockDim.x >> 6;
   {   // one workgroup per row of a batch
     const size_t row = (size_t)blockIdx.x * n;
     x += row;
+    if (x_src) x_src += row;
     if (delta) delta += row;
     if (normed) normed += row;
     act.q += row;
@@ -37,11 +38,12 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
     act.bsum += (size_t)blockIdx.x * (n / 32u);
     if (act.bs16) act.bs16 += (size_t)blockIdx.x * (n / 16u);
   }
-  ogm_norm_quant_row<GROUP, false>(x, delta, weight, n, eps, normed, act, red, tid, n_wave);
+  ogm_norm_quant_row<GROUP, false>(x, delta, weight, n, eps, normed, act, red, tid, n_wave, x_src);
 }
 
 hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const float *weight, uint32_t n,
-                                 float eps, float *normed, OgmActDev act, hipStream_t stream, uint32_t n_rows) {
+                                 float eps, float *normed, OgmActDev act, hipStream_t stream, uint32_t n_rows,
+                                 const float *x_src) {
   if (n == 0 || n % 32u != 0 || n > 16384u || n_rows == 0) return hipErrorInvalidValue;
   const uint32_t runs = (n + 255u) / 256u;
   // few rows: a wave per run, the shortest chain; from 1024 rows (2048 rows: 2 % of a prefill): four runs per wave
@@ -49,10 +51,10 @@ hipError_t ogm_launch_norm_quant(int mode, float *x, const float *delta, const f
   const uint32_t waves = n_rows >= 1024u ? (runs + 3u) / 4u : (runs < 16u ? runs : 16u);
   if (mode == 0)
     hipLaunchKernelGGL(ogm_norm_quant_kernel<32>, dim3(n_rows), dim3(waves * 64), 0, stream, x, delta, weight,
-                       n, eps, normed, act);
+                       n, eps, normed, act, x_src);
   else
     hipLaunchKernelGGL(ogm_norm_quant_kernel<256>, dim3(n_rows), dim3(waves * 64), 0, stream, x, delta, weight,
-                       n, eps, normed, act);
+                       n, eps, normed, act, x_src);
   return hipGetLastError();
 }
 

@@ -175,12 +175,14 @@ __device__ __forceinline__ float4 ogm_ld4(const float *p) {
 // n_wave): wave w owns the 256-runs w, w + n_wave, ... (at most four), lane l their elements
 // 4l..4l+3, kept in registers between the two passes.  red: 64 floats of LDS.  COHERENT_DELTA:
 // delta was written by other workgroups of the calling kernel.  COHERENT_OUT: the quantized row is
-// for other workgroups of the calling kernel.
+// for other workgroups of the calling kernel.  x_src (optional): the row is read from there instead of
+// from x, and stored to x.
 template <int GROUP, bool COHERENT_DELTA, bool COHERENT_OUT = false>
 __device__ __forceinline__ void ogm_norm_quant_row(float *__restrict__ x, const float *__restrict__ delta,
                                                    const float *__restrict__ weight, uint32_t n, float eps,
                                                    float *__restrict__ normed, const OgmActDev &act,
-                                                   float *red, uint32_t tid, uint32_t n_wave) {
+                                                   float *red, uint32_t tid, uint32_t n_wave,
+                                                   const float *__restrict__ x_src = nullptr) {
   const uint32_t lane = tid & 63u, wave = tid >> 6;
   float4 v[4], wv[4];
   float ss[4];
@@ -192,14 +194,12 @@ __device__ __forceinline__ void ogm_norm_quant_row(float *__restrict__ x, const 
     wv[k] = make_float4(0.f, 0.f, 0.f, 0.f);
     float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
     if (e0 < n) {
-      v[k] = *(const float4 *)(x + e0);
+      v[k] = *(const float4 *)((x_src ? x_src : x) + e0);
       wv[k] = *(const float4 *)(weight + e0);
       if (delta) d = ogm_ld4<COHERENT_DELTA>(delta + e0);
     }
-    if (e0 < n && delta) {
-      v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
-      *(float4 *)(x + e0) = v[k];
-    }
+    if (e0 < n && delta) { v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w; }
+    if (e0 < n && (delta || x_src)) *(float4 *)(x + e0) = v[k];
     ss[k] = v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
   }
   // one sum per 256-run, then the runs in ascending order: the same value whatever the

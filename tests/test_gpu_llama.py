@@ -174,6 +174,18 @@ def test_decode_steps_from_an_empty_cache(be, types):
         dev.close()
 
 
+def test_decode_with_a_cache_too_long_for_a_table_of_every_position(be):
+    """The rotation table of every position is made once at creation while it stays under 64 MiB; a longer
+    cache (here 300 000 positions of 32 pairs) computes each token's row when it is decoded.  Same steps."""
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=1, hd=64, n_ff=512, n_vocab=320, n_layer=1,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=300000, seed=8)
+    try:
+        for pos in range(4):
+            step_both(ref, dev, rng.standard_normal(256).astype(f32), pos, f"long cache pos {pos}")
+    finally:
+        dev.close()
+
+
 @pytest.mark.parametrize("types,n_embd,n_ff", [((Q4_K, Q6_K, Q6_K, Q6_K), 256, 512), ((Q4_K, Q4_K, Q6_K, Q6_K), 1024, 2816),
                                                ((Q5_K, Q3_K, Q3_K, Q5_K), 512, 1280), ((Q4_K, Q4_K, Q8_0, Q8_0), 256, 512),
                                                ((Q8_0, Q8_0, Q4_K, Q6_K), 256, 512)])
