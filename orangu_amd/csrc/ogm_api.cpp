@@ -1148,7 +1148,8 @@ struct ogm_llama {
   float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
   float *rope_all = nullptr;  // the same for every position of the cache, filled at creation (null: too large, computed per token)
   uint32_t head_epoch = 0;            // value of the GEMV heads' flag (the three words after the tickets) after the last launch
-  uint32_t *attn_tickets = nullptr;   // [2 n_head_kv] the attention kernel's, then the GEMV tails' tickets and the heads' flags; zero between launches
+  uint32_t *attn_counters = nullptr;  // [2 n_head_kv][OGM_ATTN_TICKET_STRIDE] the attention kernel's tickets, a line each; zero between launches
+  uint32_t *attn_tickets = nullptr;   // [2 n_head_kv] (unused),  then the GEMV tails' tickets and the heads' flags; zero between launches
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
   void *v_cache = nullptr;
   float *x = nullptr;         // hidden state [n_embd]
@@ -1248,6 +1249,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   const size_t rope_all_bytes = (size_t)c.max_ctx * (c.rope_dim / 2) * 8;
   if (c.rope_dim != 0 && rope_all_bytes <= ((size_t)64 << 20)) A((void **)&m->rope_all, rope_all_bytes);
   A((void **)&m->attn_tickets, ((size_t)2 * c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);   // + the GEMV tails' tickets
+  A((void **)&m->attn_counters, (size_t)2 * c.n_head_kv * OGM_ATTN_TICKET_STRIDE * 4);
   A(&m->k_cache, cache_bytes);
   A(&m->v_cache, cache_bytes);
   A((void **)&m->x, (size_t)c.n_embd * 4);
@@ -1301,6 +1303,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   if (e == hipSuccess) e = hipMemcpy(m->pre, pre_host.data(), pre_host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, ((size_t)2 * c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);
+  if (e == hipSuccess) e = hipMemset(m->attn_counters, 0, (size_t)2 * c.n_head_kv * OGM_ATTN_TICKET_STRIDE * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
   for (uint32_t p0 = 0; m->rope_all && e == hipSuccess && p0 < c.max_ctx; p0 += 32768u) {
@@ -1497,7 +1500,7 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
                                        c.n_head, c.n_head_kv, c.head_dim, scale, m->part_o, m->part_ml,
-                                       m->attn_tickets, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s, 0u,
+                                       m->attn_counters, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s, 0u,
                                        ctx->tune_attn_decode_share == 2 ? 0u : 1u));   // 0: wherever the shape allows
     const int mode_ff = act_mode_for(L.w_gate->ggml_type);
     if (act_mode_for(L.w_up->ggml_type) != mode_ff)

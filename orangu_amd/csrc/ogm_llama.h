@@ -8,6 +8,10 @@
 #include "ogm_kernels.h"
 
 #define OGM_ATTN_CHUNK 128u       // cache positions per workgroup of the attention kernel ...
+// The tickets of the K/V heads are 128 bytes apart: the workgroups of a launch draw theirs within a microsecond
+// of each other, and tickets that share a line queue up behind one another at the memory's atomic unit (136 of
+// them in one line: the last came back 2.9 us after its store; a line each: see the decode step's timeline).
+#define OGM_ATTN_TICKET_STRIDE 32u
 #define OGM_ATTN_CHUNK_MIN 64u    // ... or half as many while the launch stays within one round of workgroups;
                                   // the partial-result buffers are sized for this one
 

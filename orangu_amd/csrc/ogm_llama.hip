@@ -496,10 +496,10 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
     OGM_STAMP(4);
     if (tid == 0) {
       const uint32_t ticket =
-          __hip_atomic_fetch_add(&counters[hg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_fetch_add(&counters[OGM_ATTN_TICKET_STRIDE * hg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       s_last = ticket == n_splits - 1u;
       if (ticket == n_splits - 1u)
-        __hip_atomic_store(&counters[hg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        __hip_atomic_store(&counters[OGM_ATTN_TICKET_STRIDE * hg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
     }
     __syncthreads();
     OGM_STAMP(5);
