@@ -22,6 +22,9 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
+    # scalar and pointer arguments at the front of a kernel's argument list arrive in SGPRs with the wave instead of
+    # behind a scalar load at its start (gfx940 and later): 0.6 % of a decode step of 257 dependent launches
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 
 
