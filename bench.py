@@ -36,6 +36,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of `bench.py --only-roofline`, calibrated on that run's 64 MiB copy (profiles/).
 GEMV_Q4K_GATE_UP_TRAFFIC = 66248100
+# The same kernel's duration by `rocprofv3 --kernel-trace --stats` on `bench.py --only-roofline`, condensed by
+# `bench.py --trace-summary` (profiles/gemv_q4k_gate_up_4096x14336_kernel_trace.md): mean over all dispatches,
+# median, and mean of the dispatches that started within 500 ns of their predecessor's end.  Under the profiler
+# one dispatch in five starts on an idle device and runs longer; the events of an unprofiled run see none such.
+GEMV_Q4K_GATE_UP_ROCPROF = {"avg_us": 11.878, "median_us": 11.759, "back_to_back_avg_us": 11.809, "dispatches": 1250}
 
 
 def gemv_bytes(in_dim: int, out_dim: int, t: int = 1) -> int:
@@ -43,19 +48,28 @@ def gemv_bytes(in_dim: int, out_dim: int, t: int = 1) -> int:
     return out_dim * (in_dim // 256 * 144) + 4 * in_dim * t + 4 * out_dim * t
 
 
-def batched_us(hiprt, stream, launch, batches: int, per_batch: int, warm: int = 10) -> dict:
+def batched_us(hiprt, stream, launch, batches: int, per_batch: int, warm: int = 10, many=None) -> dict:
     """Times `batches` runs of `per_batch` back-to-back launches with HIP events on the launch stream;
-    the figures are microseconds per launch: the fastest batch, the median batch and the mean."""
-    for i in range(warm):
-        launch(i)
+    the figures are microseconds per launch: the fastest batch, the median batch and the mean.
+    `launch(i)` enqueues launch number i; `many(i, n)`, where given, enqueues launches i .. i + n - 1 from
+    compiled code instead (no interpreter between two launches)."""
+    if many is not None:
+        many(0, warm)
+    else:
+        for i in range(warm):
+            launch(i)
     stream.synchronize()
     ev = [(hiprt.Event(), hiprt.Event()) for _ in range(batches)]
     k = warm
     for e0, e1 in ev:
         e0.record(stream)
-        for _ in range(per_batch):
-            launch(k)
-            k += 1
+        if many is not None:
+            many(k, per_batch)
+            k += per_batch
+        else:
+            for _ in range(per_batch):
+                launch(k)
+                k += 1
         e1.record(stream)
     ev[-1][1].synchronize()
     us = [e0.elapsed_ms(e1) * 1e3 / per_batch for e0, e1 in ev]
@@ -64,6 +78,63 @@ def batched_us(hiprt, stream, launch, batches: int, per_batch: int, warm: int = 
     us = sorted(us)
     return {"min": round(us[0], 3), "median": round(us[len(us) // 2], 3), "mean": round(sum(us) / len(us), 3),
             "launches": batches * per_batch}
+
+
+def trace_summary(path: str, period: int = 0) -> dict:
+    """Condenses a `rocprofv3 --kernel-trace --output-format csv` trace (the *_kernel_trace.csv file, or a
+    folder searched for one) per kernel name: dispatch count, mean / median / min / max duration from the
+    dispatches' own start and end stamps, and -- over runs of consecutive dispatches of the same kernel with
+    no gap above 20 us between them -- (last end - first start) / dispatches and the mean gap from one
+    dispatch's end to the next one's start, how many of those gaps exceed 500 ns (the device sat idle: the
+    host, slowed by the profiler's hooks, did not keep up) and the mean duration of the dispatches that started
+    within 500 ns of their predecessor's end (back to back, as in an unprofiled run)."""
+    import csv
+    import glob
+    if os.path.isdir(path):
+        found = sorted(glob.glob(os.path.join(path, "**", "*kernel_trace.csv"), recursive=True))
+        if not found:
+            raise SystemExit(f"no *kernel_trace.csv under {path}")
+        path = found[0]
+    rows = []
+    with open(path, newline="") as f:
+        for r in csv.DictReader(f):
+            rows.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), r["Kernel_Name"]))
+    rows.sort()
+    per = {}
+    i = 0
+    while i < len(rows):
+        j = i
+        while j + 1 < len(rows) and rows[j + 1][2] == rows[i][2] and rows[j + 1][0] - rows[j][1] <= 20000:
+            j += 1
+        k = per.setdefault(rows[i][2], {"dur": [], "span_ns": 0, "span_n": 0, "gaps": [], "b2b": [], "seq": []})
+        k["dur"] += [e - b for b, e, _ in rows[i:j + 1]]
+        k["seq"] += [e - b for b, e, _ in rows[i:j + 1]]   # in dispatch order (dur is sorted below)
+        if j > i:   # a run of at least two
+            k["span_ns"] += rows[j][1] - rows[i][0]
+            k["span_n"] += j - i + 1
+            k["gaps"] += [rows[n + 1][0] - rows[n][1] for n in range(i, j)]
+            # dispatches that started within 500 ns of their predecessor's end: the device was not left idle
+            k["b2b"] += [rows[n + 1][1] - rows[n + 1][0] for n in range(i, j) if rows[n + 1][0] - rows[n][1] <= 500]
+        i = j + 1
+    out = {"file": path, "kernels": []}
+    for name, k in sorted(per.items(), key=lambda kv: -sum(kv[1]["dur"])):
+        d = sorted(k["dur"])
+        row = {"kernel": name[:120], "dispatches": len(d), "mean_ns": round(sum(d) / len(d), 1),
+               "median_ns": d[len(d) // 2], "min_ns": d[0], "max_ns": d[-1]}
+        if k["span_n"]:
+            row.update({"dispatches_in_runs": k["span_n"],
+                        "span_ns_per_dispatch": round(k["span_ns"] / k["span_n"], 1),
+                        "mean_gap_ns": round(sum(k["gaps"]) / len(k["gaps"]), 1),
+                        "gaps_over_500ns": sum(1 for g in k["gaps"] if g > 500)})
+            if k["b2b"]:
+                row.update({"back_to_back_dispatches": len(k["b2b"]),
+                            "back_to_back_mean_ns": round(sum(k["b2b"]) / len(k["b2b"]), 1)})
+        if period > 1 and len(k["seq"]) >= 2 * period:
+            # mean duration by dispatch number modulo the rotation's length: one entry per weight copy
+            row["mean_ns_by_dispatch_mod_%d" % period] = [
+                round(sum(k["seq"][i::period]) / len(k["seq"][i::period]), 1) for i in range(period)]
+        out["kernels"].append(row)
+    return out
 
 
 def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
@@ -356,7 +427,19 @@ def main() -> int:
                     help="run only the read-only launch over gate+up's bytes (the measured peak; for rocprofv3)")
     ap.add_argument("--only-single", default="", choices=["", "gate", "down"],
                     help="run only the single-matrix GEMV launches of this shape (for rocprofv3)")
+    ap.add_argument("--legs", default="", metavar="NAME[,NAME]",
+                    help="run only these legs of the dominant-kernel section (for rocprofv3): gate+up, read probe, "
+                         "gate alone, down, read probe one matrix, empty launch 1, empty launch 1792, quantize 4096")
+    ap.add_argument("--trace-summary", default="", metavar="PATH",
+                    help="no GPU work: condense a rocprofv3 kernel trace (csv file or the folder it is under) "
+                         "into per-kernel durations and span per dispatch, as JSON")
+    ap.add_argument("--trace-period", type=int, default=0, metavar="N",
+                    help="with --trace-summary: also the mean duration by dispatch number modulo N (N = --copies "
+                         "shows each weight copy of the rotation on its own)")
     args = ap.parse_args()
+    if args.trace_summary:
+        print(json.dumps(trace_summary(args.trace_summary, args.trace_period), indent=1))
+        return 0
 
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only; --gpus N with N > 1 is not supported "
@@ -392,7 +475,7 @@ def main() -> int:
     if args.fuse_quant != -1:
         be.set_tuning("gemv_fuse_quant", args.fuse_quant)
     stream = hiprt.Stream()
-    only_leg = args.only_roofline or args.only_gemm or args.only_stream or bool(args.only_single)
+    only_leg = args.only_roofline or args.only_gemm or args.only_stream or bool(args.only_single) or bool(args.legs)
 
     # ---- synthetic inputs -------------------------------------------------------------------
     seed = 20240607
@@ -467,28 +550,54 @@ def main() -> int:
     if not args.only_gemm:
         be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr)
         legs = {}
-        if not args.only_stream and not args.only_single:
-            legs["gate+up"] = batched_us(hiprt, stream, lambda i: be.matmul_multi_act_dev(
-                [handles["gate"][i % copies], handles["up"][i % copies]], 1, [y_gate.ptr, y_up.ptr], False,
-                stream.ptr), batches, per_batch, warm=50)
+        # which legs run: all of them in the headline run, a named subset under a profiler
+        all_legs = ["gate+up", "read probe", "gate alone", "down", "read probe one matrix", "empty launch 1",
+                    "empty launch 1792", "quantize 4096"]
+        if args.legs:
+            want = [l.strip() for l in args.legs.split(",") if l.strip()]
+            bad = [l for l in want if l not in all_legs]
+            if bad:
+                raise SystemExit(f"--legs: unknown {bad}; known: {all_legs}")
+        elif args.only_roofline:
+            want = ["gate+up"]
+        elif args.only_stream:
+            want = ["read probe"]
+        elif args.only_single:
+            want = ["gate alone" if args.only_single == "gate" else "down"]
+        else:
+            want = all_legs
+        mats = handles["gate"] + handles["up"]
+
+        def timed(name, launch=None, many=None):
+            if name in want:
+                legs[name] = batched_us(hiprt, stream, launch, batches, per_batch, warm=50, many=many)
+
+        # The launches of these legs are enqueued from compiled code (ogm_enqueue_repeated): the interpreter's
+        # own time per call would otherwise show as idle gaps between kernels this short -- under rocprofv3,
+        # whose hooks add to every call, gaps of 2 us between 12 us kernels.
+        pair_sets = [[handles["gate"][c], handles["up"][c]] for c in range(copies)]
+        single_sets = [[h] for h in mats]
+        timed("gate+up", many=lambda i, n: be.enqueue_repeated(0, pair_sets, 1, [y_gate.ptr, y_up.ptr], i % copies, n,
+                                                               False, stream.ptr))
+        if "gate+up" in legs:
             kernel_name = be.last_kernel()
-        if not args.only_roofline and not args.only_single:
-            # the yardstick: the same bytes through a launch that only reads them
-            legs["read probe"] = batched_us(hiprt, stream, lambda i: be.weights_read_probe(
-                [handles["gate"][i % copies], handles["up"][i % copies]], stream.ptr), batches, per_batch, warm=50)
-        if not args.only_roofline and not args.only_stream:
-            mats = handles["gate"] + handles["up"]
-            if args.only_single in ("", "gate"):
-                legs["gate alone"] = batched_us(hiprt, stream, lambda i: be.matmul_act_dev(
-                    mats[i % len(mats)], 1, y_gate.ptr, False, stream.ptr), batches, per_batch, warm=50)
-            if args.only_single in ("", "down"):
-                be.act_quantize_dev(Q4_K, h_d.ptr, FFN, 1, stream.ptr)
-                legs["down"] = batched_us(hiprt, stream, lambda i: be.matmul_act_dev(
-                    handles["down"][i % copies], 1, y_down.ptr, False, stream.ptr), batches, per_batch, warm=50)
-            if not args.only_single:
-                legs["quantize 4096"] = batched_us(hiprt, stream, lambda i: be.act_quantize_dev(
-                    Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr), batches, per_batch, warm=50)
-        if args.only_roofline or args.only_stream:
+        # the yardstick: the same bytes through a launch that only reads them
+        timed("read probe", many=lambda i, n: be.enqueue_repeated(1, pair_sets, 1, [], i % copies, n, False, stream.ptr))
+        timed("gate alone", many=lambda i, n: be.enqueue_repeated(0, single_sets, 1, [y_gate.ptr], i % len(mats), n,
+                                                                  False, stream.ptr))
+        if "down" in want:
+            be.act_quantize_dev(Q4_K, h_d.ptr, FFN, 1, stream.ptr)
+            timed("down", many=lambda i, n: be.enqueue_repeated(0, [[h] for h in handles["down"]], 1, [y_down.ptr],
+                                                                i % copies, n, False, stream.ptr))
+        # one matrix's bytes through the read-only launch: what a launch of 33 MB can reach at all
+        timed("read probe one matrix", many=lambda i, n: be.enqueue_repeated(1, single_sets, 1, [], i % len(mats), n,
+                                                                             False, stream.ptr))
+        # launches that do nothing, one workgroup wide and as wide as the gate+up GEMV (1792 workgroups of 256
+        # threads): the kernel boundary, host and device side together, back to back on one stream
+        timed("empty launch 1", many=lambda i, n: be.enqueue_repeated(2, [], 1, [], 0, n, False, stream.ptr))
+        timed("empty launch 1792", many=lambda i, n: be.enqueue_repeated(2, [], 1792, [], 0, n, False, stream.ptr))
+        timed("quantize 4096", lambda i: be.act_quantize_dev(Q4_K, x_d.ptr, HIDDEN, 1, stream.ptr))
+        if args.only_roofline or args.only_stream or args.legs:
             # One plain device-to-device copy of known size: under `rocprofv3 --pmc FETCH_SIZE` /
             # `WRITE_SIZE` its counter reading calibrates the kernel's (bytes per counter unit).
             cal = 64 << 20
@@ -501,17 +610,26 @@ def main() -> int:
         achieved = kbytes / (us_per_launch * 1e-6) / 1e9
         one = gemv_bytes(HIDDEN, FFN)
         per_leg_bytes = {"gate+up": kbytes, "read probe": weight_bytes2, "gate alone": one,
-                         "down": gemv_bytes(FFN, HIDDEN), "quantize 4096": 4 * HIDDEN + HIDDEN + 64}
+                         "down": gemv_bytes(FFN, HIDDEN), "read probe one matrix": weight_bytes2 // 2,
+                         "empty launch 1": 0, "empty launch 1792": 0, "quantize 4096": 4 * HIDDEN + HIDDEN + 64}
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_Q4K_GATE_UP_TRAFFIC,
                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on `bench.py --only-roofline`, "
                                       "each scaled by the same counter's reading for that run's 64 MiB copy "
                                       "(profiles/gemv_q4k_gate_up_4096x14336_hbm_counters.md)",
+                    "rocprof_avg_us": GEMV_Q4K_GATE_UP_ROCPROF["avg_us"],
+                    "rocprof_median_us": GEMV_Q4K_GATE_UP_ROCPROF["median_us"],
+                    "rocprof_back_to_back_avg_us": GEMV_Q4K_GATE_UP_ROCPROF["back_to_back_avg_us"],
+                    "rocprof_frac": round(kbytes / GEMV_Q4K_GATE_UP_ROCPROF["avg_us"] / 1e3 / HBM_PEAK_GBS, 4),
+                    "rocprof_source": "rocprofv3 --kernel-trace --stats on `bench.py --only-roofline`, "
+                                      f"{GEMV_Q4K_GATE_UP_ROCPROF['dispatches']} dispatches, condensed by `bench.py "
+                                      "--trace-summary` (profiles/gemv_q4k_gate_up_4096x14336_kernel_trace.md); "
+                                      "us_per_launch beside it is measured live in this run",
                     "kernel": (kernel_name or "(not run)") + " over gate+up", "us_per_launch": us_per_launch,
                     "us_per_launch_min": main_leg["min"], "bytes_per_launch": kbytes,
                     "launches": main_leg["launches"],
                     "timing": f"HIP events on the launch stream round {batches} batches of {per_batch} back-to-back "
-                              "launches; median batch (achieved, frac) and fastest batch",
+                              "launches enqueued from compiled code; median batch (achieved, frac) and fastest batch",
                     "legs_us": {k: {**v, "GBps_median": round(per_leg_bytes[k] / v["median"] / 1e3, 1)}
                                 for k, v in legs.items()}}
         if "read probe" in legs and "gate+up" in legs:

@@ -160,9 +160,16 @@ int ogm_matmul_dev_static(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev,
  * engine/arch/mod.rs:1082-1096) quantize it once.  ogm_act_quantize_dev quantizes x_dev
  * ([n_tokens][in_dim]) into the context's activation buffer with the mode `ggml_type` needs
  * (backend/cpu.rs:100-116); ogm_matmul_act_dev then multiplies any weight of the same in_dim and
- * activation mode by it.  Values equal ogm_matmul_dev's: the quantizer is a pure function of x. */
+ * activation mode by it.  Values equal ogm_matmul_dev's: the quantizer is a pure function of x.
+ * ogm_act_quantize_dev quantizes for a following call with decode = 0 (Backend::matmul),
+ * ogm_act_quantize_decode_dev for one with decode = 1 (Backend::matmul_decode).  The two differ for one case
+ * only: Q2_K at n_tokens > 1, which matmul runs over per-32 activations (backend/cpu.rs:113-163) and
+ * matmul_decode over per-256 ones (cpu.rs:265-317); a matmul step over the other mode's activations returns
+ * OGM_ERR_INVALID and says which quantizer it needs. */
 int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev, uint32_t in_dim,
                          uint32_t n_tokens, void *stream);
+int ogm_act_quantize_decode_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev, uint32_t in_dim,
+                                uint32_t n_tokens, void *stream);
 int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, float *y_dev,
                        int decode, void *stream);
 
@@ -449,6 +456,17 @@ int ogm_time_host_calls(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, size_t n_
  * more) with the GEMV's non-temporal 16-byte loads and stores nothing -- the rate the memory system gives
  * that footprint with no arithmetic behind the loads.  No counterpart in the reference. */
 int ogm_weights_read_probe(ogm_ctx *ctx, const ogm_weight *const *ws, size_t n_ws, void *stream);
+/* For benchmarks: one launch of `workgroups` (1..1048576) workgroups of 256 threads that does nothing -- what
+ * a kernel boundary costs behind a launch of that width.  No counterpart in the reference. */
+int ogm_empty_launch(ogm_ctx *ctx, uint32_t workgroups, void *stream);
+/* For benchmarks driven from an interpreter: enqueues `reps` launches back to back from compiled code, so that
+ * the caller's own overhead per call leaves no gap between short kernels.  `ws` holds n_variants sets of n_ws
+ * weights; launch r takes set (first + r) % n_variants.  kind 0: ogm_matmul_multi_act_dev over the set into
+ * ys_dev[n_ws]; kind 1: ogm_weights_read_probe over the set; kind 2: ogm_empty_launch of n_tokens workgroups (ws
+ * unused).  No counterpart in the reference. */
+int ogm_enqueue_repeated(ogm_ctx *ctx, int kind, const ogm_weight *const *ws, size_t n_ws, size_t n_variants,
+                         uint32_t n_tokens, float *const *ys_dev, int decode, uint32_t first, uint32_t reps,
+                         void *stream);
 /* Name of the kernel the last matmul on this context launched (for profiles). */
 const char *ogm_last_kernel(ogm_ctx *ctx);
 

@@ -256,9 +256,13 @@ class Mi355xBackend:
         self._check(self._lib.ogm_matmul_dev_static(self._ctx, w_handle, x_ptr, n_tokens, y_ptr,
                                                     int(decode), stream or None), "ogm_matmul_dev_static")
 
-    def act_quantize_dev(self, ggml_type: int, x_ptr: int, in_dim: int, n_tokens: int, stream: int = 0):
-        self._check(self._lib.ogm_act_quantize_dev(self._ctx, ggml_type, x_ptr, in_dim, n_tokens,
-                                                   stream or None), "ogm_act_quantize_dev")
+    def act_quantize_dev(self, ggml_type: int, x_ptr: int, in_dim: int, n_tokens: int, stream: int = 0,
+                         decode: bool = False):
+        """Quantizes device-resident x for following matmul_act_dev calls: with decode=False in matmul's activation
+        mode, with decode=True in matmul_decode's (they differ for Q2_K at several tokens only)."""
+        fn = self._lib.ogm_act_quantize_decode_dev if decode else self._lib.ogm_act_quantize_dev
+        self._check(fn(self._ctx, ggml_type, x_ptr, in_dim, n_tokens, stream or None),
+                    "ogm_act_quantize_decode_dev" if decode else "ogm_act_quantize_dev")
 
     def matmul_act_dev(self, w_handle: int, n_tokens: int, y_ptr: int, decode: bool = False,
                        stream: int = 0):
@@ -309,6 +313,23 @@ class Mi355xBackend:
         n = len(w_handles)
         ws = (C.c_void_p * n)(*w_handles)
         self._check(self._lib.ogm_weights_read_probe(self._ctx, ws, n, stream or None), "ogm_weights_read_probe")
+
+    def empty_launch(self, workgroups: int, stream: int = 0):
+        """One launch of `workgroups` workgroups that does nothing (for benchmarks: a kernel boundary)."""
+        self._check(self._lib.ogm_empty_launch(self._ctx, workgroups, stream or None), "ogm_empty_launch")
+
+    def enqueue_repeated(self, kind: int, w_sets, n_tokens: int, y_ptrs, first: int, reps: int, decode: bool = False,
+                         stream: int = 0):
+        """`reps` launches back to back from compiled code, rotating over `w_sets` (equally long lists of weight
+        handles) from set `first`: kind 0 the grouped GEMV over quantized activations, 1 the read-only probe,
+        2 empty launches of n_tokens workgroups (w_sets and y_ptrs unused)."""
+        n_var = max(1, len(w_sets))
+        n_ws = len(w_sets[0]) if w_sets else 0
+        flat = [h for s in w_sets for h in s]
+        ws = (C.c_void_p * max(1, len(flat)))(*flat)
+        ys = (C.c_void_p * max(1, len(y_ptrs)))(*y_ptrs)
+        self._check(self._lib.ogm_enqueue_repeated(self._ctx, kind, ws, n_ws, n_var, n_tokens, ys, int(decode),
+                                                   first, reps, stream or None), "ogm_enqueue_repeated")
 
     def upload_raw(self, raw: np.ndarray, ggml_type: int, in_dim: int, out_dim: int) -> int:
         """Uploads without a cache key: every call makes a new device copy."""

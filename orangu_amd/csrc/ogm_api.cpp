@@ -66,6 +66,7 @@ struct ogm_ctx {
   int tune_gemm_sb_waves = 0;          // small-batch GEMM: 8 or 16 waves per workgroup, 0 = by the launch
   int tune_host_flag_wait = 1;         // zero-copy host calls wait on a word a trailing kernel stores to pinned memory instead of on the stream
   int tune_host_zero_copy = 1;         // host-pointer calls of up to OGM_ZERO_COPY_MAX bytes: kernels read x / write y in pinned host memory
+  bool host_coherent = true;           // the pinned staging buffers are fine-grained (asked for by name); false once the runtime has refused
   int tune_gemm_plane_kernel = 0;      // who reads planes: 0 the all-waves-multiply kernel on large grids, 1 the feeding-wave kernels, 2 the former always
   int tune_gemm_one_pass = 0;          // 1: Q4_K / Q5_K on that kernel fold the min pass into the super-block step (f32 to rounding, not to the bit)
   int tune_decode_fuse_heads = 0;      // 1: the decode step's norms and SwiGLU at the head of the GEMV after them
@@ -77,6 +78,7 @@ struct ogm_ctx {
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
+  int tune_weight_alloc_mb = 0;  // device allocations of weights of 1 MiB and more are rounded up to a multiple of this many MiB (0 = exact size)
   // Device memory the prefill planes of all weights may take, in MiB; 0 (the default) = build none.
   // A model's planes are 3.3 times its Q4_K bytes.
   int tune_plane_cache_mb = 32768;   // MiB the K-quant matrices' prefill planes may take in all
@@ -122,6 +124,21 @@ static int ensure_dev(ogm_ctx *ctx, DevBuf &b, size_t bytes) {
   return OGM_OK;
 }
 
+// Pinned host memory the kernels of a zero-copy call read x from and store y and the completion word to.  The
+// host reads y after seeing the word, with no runtime call between: that is only sound for fine-grained
+// (coherent) host memory, where a kernel's stores are visible to the host as they are acknowledged.  So
+// coherence is asked for by name; where the runtime refuses it, the memory is plain pinned memory and the
+// context stops running kernels on it in place (host_coherent false: device copies and a stream
+// synchronization per call instead).
+static hipError_t host_alloc_coherent(ogm_ctx *ctx, void **p, size_t bytes) {
+  if (ctx->host_coherent) {
+    if (hipHostMalloc(p, bytes, hipHostMallocCoherent) == hipSuccess) return hipSuccess;
+    (void)hipGetLastError();
+    ctx->host_coherent = false;
+  }
+  return hipHostMalloc(p, bytes, hipHostMallocDefault);
+}
+
 static int ensure_host(ogm_ctx *ctx, DevBuf &b, size_t bytes) {
   if (bytes <= b.cap) return OGM_OK;
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
@@ -129,7 +146,7 @@ static int ensure_host(ogm_ctx *ctx, DevBuf &b, size_t bytes) {
   b.p = nullptr;
   b.cap = 0;
   size_t cap = (bytes + 4095) & ~(size_t)4095;
-  HIPCHK(ctx, hipHostMalloc(&b.p, cap, hipHostMallocDefault));
+  HIPCHK(ctx, host_alloc_coherent(ctx, &b.p, cap));
   b.cap = cap;
   return OGM_OK;
 }
@@ -360,6 +377,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_plane_cache_mb = value;
     return OGM_OK;
   }
+  if (strcmp(key, "weight_alloc_mb") == 0) {
+    if (value < 0 || value > 1024) return fail(ctx, OGM_ERR_INVALID, "weight_alloc_mb must be 0..1024");
+    ctx->tune_weight_alloc_mb = value;
+    return OGM_OK;
+  }
   if (strcmp(key, "gemv_fuse_quant") == 0) {
     if (value < -1 || value > 1) return fail(ctx, OGM_ERR_INVALID, "gemv_fuse_quant must be -1, 0 or 1");
     ctx->tune_fuse_quant = value < 0 ? 0 : value;  // -1 = the default
@@ -420,7 +442,12 @@ extern "C" int ogm_weight_upload(ogm_ctx *ctx, uint32_t ggml_type, const void *r
   w->key_addr = key_addr;
   w->key_len = key_len;
   w->dev = nullptr;
-  hipError_t e = hipMalloc((void **)&w->dev, bytes);
+  size_t alloc_bytes = bytes;
+  if (ctx->tune_weight_alloc_mb > 0 && bytes >= (1u << 20)) {
+    const size_t g = (size_t)ctx->tune_weight_alloc_mb << 20;
+    alloc_bytes = (bytes + g - 1) / g * g;
+  }
+  hipError_t e = hipMalloc((void **)&w->dev, alloc_bytes);
   if (e == hipSuccess) e = hipMemcpyAsync(w->dev, staging, bytes, hipMemcpyHostToDevice, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   (void)hipHostFree(staging);
@@ -699,7 +726,7 @@ static int check_matmul_args(ogm_ctx *ctx, const ogm_weight *w, const void *x, c
 // staging buffers are device-visible, and the quantizer and the matmul kernels use them in place.
 #define OGM_ZERO_COPY_MAX (512u << 10)
 static bool zero_copy(const ogm_ctx *ctx, size_t bytes) {
-  return ctx->tune_host_zero_copy != 0 && bytes <= OGM_ZERO_COPY_MAX;
+  return ctx->tune_host_zero_copy != 0 && ctx->host_coherent && bytes <= OGM_ZERO_COPY_MAX;
 }
 
 // Waits for what a host-pointer call has enqueued on the context's stream.  A zero-copy call's results land
@@ -710,15 +737,20 @@ static bool zero_copy(const ogm_ctx *ctx, size_t bytes) {
 // or a kernel has faulted -- the stream is synchronized after all and reports.  Every 256th call synchronizes
 // anyway, so the runtime can retire its records of the launches.
 static int host_wait(ogm_ctx *ctx, bool zero_copied) {
-  if (!zero_copied || ctx->tune_host_flag_wait == 0 || ++ctx->flag_unsynced >= 256u) {
+  if (!zero_copied || !ctx->host_coherent || ctx->tune_host_flag_wait == 0 || ++ctx->flag_unsynced >= 256u) {
     ctx->flag_unsynced = 0;
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     return OGM_OK;
   }
   if (!ctx->hflag.p) {
-    HIPCHK(ctx, hipHostMalloc(&ctx->hflag.p, 4096, hipHostMallocDefault));
+    HIPCHK(ctx, host_alloc_coherent(ctx, &ctx->hflag.p, 4096));
     ctx->hflag.cap = 4096;
     *(volatile uint32_t *)ctx->hflag.p = 0;
+    if (!ctx->host_coherent) {   // refused just now: this call's y sits in plain pinned memory, so wait on the stream
+      ctx->flag_unsynced = 0;
+      HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+      return OGM_OK;
+    }
   }
   const uint32_t epoch = ++ctx->flag_epoch;
   uint32_t *flag = (uint32_t *)ctx->hflag.p;
@@ -863,8 +895,22 @@ extern "C" int ogm_weights_read_probe(ogm_ctx *ctx, const ogm_weight *const *ws,
   return OGM_OK;
 }
 
-extern "C" int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev,
-                                    uint32_t in_dim, uint32_t n_tokens, void *stream) {
+// A launch that does nothing, `workgroups` workgroups wide (for benchmarks: the cost of a kernel boundary).
+extern "C" int ogm_empty_launch(ogm_ctx *ctx, uint32_t workgroups, void *stream) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (workgroups == 0 || workgroups > (1u << 20)) return fail(ctx, OGM_ERR_INVALID, "ogm_empty_launch takes 1..1048576 workgroups");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
+  int rc = ensure_dev(ctx, ctx->probe_sink, 256);
+  if (rc != OGM_OK) return rc;
+  HIPCHK(ctx, ogm_launch_empty(workgroups, (uint32_t *)ctx->probe_sink.p, s));
+  ctx->last_kernel = "ogm_empty_kernel";
+  return OGM_OK;
+}
+
+static int act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev, uint32_t in_dim, uint32_t n_tokens,
+                            int decode, void *stream) {
   if (!ctx) return OGM_ERR_INVALID;
   if (!ogm_supports(ggml_type, in_dim)) return fail(ctx, OGM_ERR_UNSUPPORTED, "type / in_dim without a kernel");
   if (n_tokens == 0) return OGM_OK;
@@ -872,8 +918,33 @@ extern "C" int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const floa
   std::lock_guard<std::mutex> lock(ctx->mu);
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
-  // (for matmul's arithmetic: Q2_K at several tokens is quantized per 32, and a decode batch over it is refused below)
-  return enqueue_quantize(ctx, act_mode_for(ggml_type, n_tokens, 0), x_dev, in_dim, n_tokens, s);
+  return enqueue_quantize(ctx, act_mode_for(ggml_type, n_tokens, decode), x_dev, in_dim, n_tokens, s);
+}
+
+// The activation mode of Backend::matmul (for Q2_K at several tokens: per 32, cpu.rs:113-163) ...
+extern "C" int ogm_act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev,
+                                    uint32_t in_dim, uint32_t n_tokens, void *stream) {
+  return act_quantize_dev(ctx, ggml_type, x_dev, in_dim, n_tokens, 0, stream);
+}
+
+// ... and of Backend::matmul_decode (per 256 for Q2_K too: its k_row dot, cpu.rs:265-317).  The two differ for
+// Q2_K at several tokens only.
+extern "C" int ogm_act_quantize_decode_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev,
+                                           uint32_t in_dim, uint32_t n_tokens, void *stream) {
+  return act_quantize_dev(ctx, ggml_type, x_dev, in_dim, n_tokens, 1, stream);
+}
+
+// Why the activation buffer does not fit a two-step call, in the caller's terms.
+static std::string act_mismatch(const ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens, int decode) {
+  const int want = act_mode_for(w->ggml_type, n_tokens, decode);
+  if (ctx->act_mode >= 0 && ctx->act_mode != want && ctx->act_in_dim == w->in_dim && ctx->act_tokens >= n_tokens)
+    return std::string("the activations were quantized per ") + (ctx->act_mode == OGM_ACT_PER_32 ? "32" : "256") +
+           " and this call needs per " + (want == OGM_ACT_PER_32 ? "32" : "256") +
+           (w->ggml_type == OGM_Q2_K ? " (Q2_K at several tokens: ogm_act_quantize_dev serves decode = 0, "
+                                       "ogm_act_quantize_decode_dev serves decode = 1)"
+                                     : " (quantize with this weight's type)");
+  return "the quantized activations do not fit this weight (call ogm_act_quantize_dev, or for decode = 1 "
+         "ogm_act_quantize_decode_dev, with its type, in_dim and token count first)";
 }
 
 extern "C" int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_tokens,
@@ -885,8 +956,7 @@ extern "C" int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (ctx->act_mode != act_mode_for(w->ggml_type, n_tokens, decode) || ctx->act_in_dim != w->in_dim ||
       ctx->act_tokens < n_tokens)
-    return fail(ctx, OGM_ERR_INVALID, "the quantized activations do not fit this weight "
-                "(call ogm_act_quantize_dev with its type, in_dim and token count first)");
+    return fail(ctx, OGM_ERR_INVALID, act_mismatch(ctx, w, n_tokens, decode));
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
   const Target t{w, y_dev};
@@ -933,11 +1003,28 @@ extern "C" int ogm_matmul_multi_act_dev(ogm_ctx *ctx, const ogm_weight *const *w
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (ctx->act_mode != act_mode_for(ws[0]->ggml_type, n_tokens, decode) || ctx->act_in_dim != ws[0]->in_dim ||
       ctx->act_tokens < n_tokens)
-    return fail(ctx, OGM_ERR_INVALID, "the quantized activations do not fit these weights "
-                "(call ogm_act_quantize_dev with their type, in_dim and token count first)");
+    return fail(ctx, OGM_ERR_INVALID, act_mismatch(ctx, ws[0], n_tokens, decode));
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
   return enqueue_gemv(ctx, tg.data(), n_ws, n_tokens, decode, s, nullptr, nullptr, nullptr);
+}
+
+// `reps` launches enqueued back to back from compiled code (for benchmarks driven from an interpreter, whose
+// own call overhead would otherwise leave the device idle between short kernels, under a profiler above all).
+extern "C" int ogm_enqueue_repeated(ogm_ctx *ctx, int kind, const ogm_weight *const *ws, size_t n_ws, size_t n_variants,
+                                    uint32_t n_tokens, float *const *ys_dev, int decode, uint32_t first,
+                                    uint32_t reps, void *stream) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (kind < 0 || kind > 2) return fail(ctx, OGM_ERR_INVALID, "ogm_enqueue_repeated: kind is 0, 1 or 2");
+  if (kind != 2 && (!ws || n_ws == 0 || n_variants == 0)) return fail(ctx, OGM_ERR_INVALID, "ogm_enqueue_repeated: no weights");
+  for (uint32_t r = 0; r < reps; r++) {
+    const ogm_weight *const *set = kind == 2 ? nullptr : ws + ((size_t)first + r) % n_variants * n_ws;
+    int rc = kind == 0   ? ogm_matmul_multi_act_dev(ctx, set, n_ws, n_tokens, ys_dev, decode, stream)
+             : kind == 1 ? ogm_weights_read_probe(ctx, set, n_ws, stream)
+                         : ogm_empty_launch(ctx, n_tokens, stream);
+    if (rc != OGM_OK) return rc;
+  }
+  return OGM_OK;
 }
 
 // Backend::matmul_batch (backend/mod.rs:362-366) with guarded_matmul_op's token stripes
@@ -981,13 +1068,13 @@ extern "C" int ogm_matmul_batch(ogm_ctx *ctx, const ogm_op *ops, size_t n_ops, i
   }
   if (xb == 0) return OGM_OK;
   int rc;
-  const bool zc = zero_copy(ctx, xb + yb);   // see host_matmul
+  if ((rc = ensure_host(ctx, ctx->hx, xb)) != OGM_OK) return rc;
+  if ((rc = ensure_host(ctx, ctx->hy, yb)) != OGM_OK) return rc;
+  const bool zc = zero_copy(ctx, xb + yb);   // see host_matmul (after the staging buffers exist: it asks whether they are coherent)
   if (!zc) {
     if ((rc = ensure_dev(ctx, ctx->x, xb)) != OGM_OK) return rc;
     if ((rc = ensure_dev(ctx, ctx->y, yb)) != OGM_OK) return rc;
   }
-  if ((rc = ensure_host(ctx, ctx->hx, xb)) != OGM_OK) return rc;
-  if ((rc = ensure_host(ctx, ctx->hy, yb)) != OGM_OK) return rc;
   uint8_t *const x_base = (uint8_t *)(zc ? ctx->hx.p : ctx->x.p), *const y_base = (uint8_t *)(zc ? ctx->hy.p : ctx->y.p);
   // Size the activation scratch for the largest stripe before anything is enqueued, so it is
   // never reallocated under kernels in flight.

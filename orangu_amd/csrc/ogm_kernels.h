@@ -170,6 +170,7 @@ hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hip
 hipError_t ogm_launch_read_probe(const uint8_t *const *bufs, const size_t *bytes, uint32_t n, uint32_t *sink,
                                  hipStream_t stream);
 // Stores `value` to the pinned host word `flag` once everything before it on the stream has finished.
+hipError_t ogm_launch_empty(uint32_t workgroups, uint32_t *sink, hipStream_t stream);
 hipError_t ogm_launch_host_flag(uint32_t *flag, uint32_t value, hipStream_t stream);
 
 // The library's static scratch (ogm_static.hip): a file-scope device array every GPU holds its own

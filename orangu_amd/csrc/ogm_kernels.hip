@@ -1628,6 +1628,18 @@ hipError_t ogm_launch_read_probe(const uint8_t *const *bufs, const size_t *bytes
   return hipGetLastError();
 }
 
+// A launch of `workgroups` workgroups of 256 threads that does nothing (one pointer and one word of
+// arguments, like a real kernel): what a kernel boundary costs behind a launch of a given width.
+__global__ __launch_bounds__(256) void ogm_empty_kernel(uint32_t *sink, uint32_t never) {
+  if (never == 0x9E3779B9u && threadIdx.x == 0) sink[blockIdx.x & 63u] = never;
+}
+
+hipError_t ogm_launch_empty(uint32_t workgroups, uint32_t *sink, hipStream_t stream) {
+  if (workgroups == 0 || workgroups > 0x7FFFFFFFu || !sink) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(ogm_empty_kernel, dim3(workgroups), dim3(256), 0, stream, sink, 0u);
+  return hipGetLastError();
+}
+
 hipError_t ogm_launch_f16_to_f32(const uint16_t *bits, size_t n, float *out, hipStream_t stream) {
   if (n == 0) return hipSuccess;
   hipLaunchKernelGGL(ogm_f16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, bits,
