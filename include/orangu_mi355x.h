@@ -467,6 +467,10 @@ int ogm_empty_launch(ogm_ctx *ctx, uint32_t workgroups, void *stream);
 int ogm_enqueue_repeated(ogm_ctx *ctx, int kind, const ogm_weight *const *ws, size_t n_ws, size_t n_variants,
                          uint32_t n_tokens, float *const *ys_dev, int decode, uint32_t first, uint32_t reps,
                          void *stream);
+/* Bytes of device and pinned host scratch this context has allocated so far (activation buffers, staging;
+ * weights and prefill planes not counted).  It grows on demand and never shrinks before ogm_destroy; a call
+ * that leaves it unchanged has allocated no scratch.  No counterpart in the reference. */
+size_t ogm_scratch_bytes(ogm_ctx *ctx);
 /* Name of the kernel the last matmul on this context launched (for profiles). */
 const char *ogm_last_kernel(ogm_ctx *ctx);
 

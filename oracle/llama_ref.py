@@ -51,10 +51,40 @@ def rmsnorm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
     return (x * scale).astype(f32) * np.asarray(weight, f32)
 
 
+_libm = None
+
+
+def _libm_f32():
+    """The C library's single-precision powf, sinf and cosf: what f32::powf and f32::sin_cos
+    (tensor.rs:1147, 1160) bind to on Linux.  numpy's float32 power and sin / cos are its own SIMD
+    routines and differ from them in the last bit here and there, which at position p turns into
+    p ulps of angle; the restatement therefore calls the reference's own functions."""
+    global _libm
+    if _libm is None:
+        import ctypes
+        import ctypes.util
+        L = ctypes.CDLL(ctypes.util.find_library("m") or "libm.so.6")
+        L.powf.restype = ctypes.c_float
+        L.powf.argtypes = [ctypes.c_float, ctypes.c_float]
+        for fn in (L.sinf, L.cosf):
+            fn.restype = ctypes.c_float
+            fn.argtypes = [ctypes.c_float]
+        _libm = L
+    return _libm
+
+
 def rope_freqs(rope_dim: int, freq_base: float) -> np.ndarray:
-    """tensor.rs:1147: freq_i = base^(-2i / rope_dim), in f32."""
-    i = np.arange(rope_dim // 2, dtype=f32)
-    return np.power(f32(freq_base), (f32(-2.0) * i / f32(rope_dim)).astype(f32), dtype=f32)
+    """tensor.rs:1147: freq_i = base.powf(-2 i / rope_dim), in f32."""
+    L = _libm_f32()
+    expo = (f32(-2.0) * np.arange(rope_dim // 2, dtype=f32) / f32(rope_dim)).astype(f32)
+    return np.array([L.powf(float(f32(freq_base)), float(e)) for e in expo], f32)
+
+
+def rope_sin_cos(theta: np.ndarray):
+    """tensor.rs:1160: theta.sin_cos() per pair, in f32."""
+    L = _libm_f32()
+    t = np.asarray(theta, f32).reshape(-1)
+    return (np.array([L.sinf(float(v)) for v in t], f32), np.array([L.cosf(float(v)) for v in t], f32))
 
 
 def rope(x: np.ndarray, n_head: int, head_dim: int, pos: int, rope_dim: int, freq_base: float,
@@ -67,7 +97,7 @@ def rope(x: np.ndarray, n_head: int, head_dim: int, pos: int, rope_dim: int, fre
     if freq_factors is not None:
         freq = (freq / np.asarray(freq_factors, f32)[:rope_dim // 2]).astype(f32)
     theta = (f32(pos) * freq).astype(f32)
-    sin, cos = np.sin(theta, dtype=f32), np.cos(theta, dtype=f32)
+    sin, cos = rope_sin_cos(theta)
     half = rope_dim // 2
     lo = slice(0, half) if neox else slice(0, 2 * half, 2)
     hi = slice(half, 2 * half) if neox else slice(1, 2 * half, 2)

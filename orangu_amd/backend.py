@@ -331,6 +331,10 @@ class Mi355xBackend:
         self._check(self._lib.ogm_enqueue_repeated(self._ctx, kind, ws, n_ws, n_var, n_tokens, ys, int(decode),
                                                    first, reps, stream or None), "ogm_enqueue_repeated")
 
+    def scratch_bytes(self) -> int:
+        """Bytes of device and pinned scratch the context has grown so far (weights not counted)."""
+        return int(self._lib.ogm_scratch_bytes(self._ctx))
+
     def upload_raw(self, raw: np.ndarray, ggml_type: int, in_dim: int, out_dim: int) -> int:
         """Uploads without a cache key: every call makes a new device copy."""
         raw = np.ascontiguousarray(raw, np.uint8)

@@ -29,7 +29,7 @@ SYMBOLS = [
     "ogm_gguf_meta_u64", "ogm_gguf_meta_f64", "ogm_gguf_meta_string", "ogm_gguf_meta_array",
     "ogm_gguf_find_tensor", "ogm_gguf_tensor", "ogm_gguf_tensor_data", "ogm_gguf_matrix",
     "ogm_gguf_upload_matrix", "ogm_argmax", "ogm_matmul_dev_static", "ogm_quantize_act_tokens", "ogm_llama_debug_capture", "ogm_llama_debug_act",
-    "ogm_weights_read_probe", "ogm_time_host_calls", "ogm_empty_launch", "ogm_act_quantize_decode_dev", "ogm_enqueue_repeated",
+    "ogm_weights_read_probe", "ogm_time_host_calls", "ogm_empty_launch", "ogm_scratch_bytes", "ogm_act_quantize_decode_dev", "ogm_enqueue_repeated",
 ]
 
 
@@ -97,6 +97,8 @@ def load_library() -> C.CDLL:
     L.ogm_matmul_multi_act_dev.argtypes = [vp, C.POINTER(vp), sz, u32, C.POINTER(vp), C.c_int, vp]
     L.ogm_weights_read_probe.argtypes = [vp, C.POINTER(vp), sz, vp]
     L.ogm_empty_launch.argtypes = [vp, u32, vp]
+    L.ogm_scratch_bytes.argtypes = [vp]
+    L.ogm_scratch_bytes.restype = sz
     L.ogm_enqueue_repeated.argtypes = [vp, C.c_int, C.POINTER(vp), sz, sz, u32, C.POINTER(vp), C.c_int, u32, u32, vp]
     L.ogm_time_host_calls.argtypes = [vp, C.POINTER(OgmOp), sz, sz, C.POINTER(u32), sz, u32, C.POINTER(C.c_double)]
     L.ogm_llama_create.argtypes = [vp, C.POINTER(OgmLlamaConfig), C.POINTER(OgmLlamaLayer), vp, vp, C.POINTER(vp)]

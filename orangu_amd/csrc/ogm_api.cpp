@@ -78,7 +78,6 @@ struct ogm_ctx {
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
   int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
   int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
-  int tune_weight_alloc_mb = 0;  // device allocations of weights of 1 MiB and more are rounded up to a multiple of this many MiB (0 = exact size)
   // Device memory the prefill planes of all weights may take, in MiB; 0 (the default) = build none.
   // A model's planes are 3.3 times its Q4_K bytes.
   int tune_plane_cache_mb = 32768;   // MiB the K-quant matrices' prefill planes may take in all
@@ -377,17 +376,23 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_plane_cache_mb = value;
     return OGM_OK;
   }
-  if (strcmp(key, "weight_alloc_mb") == 0) {
-    if (value < 0 || value > 1024) return fail(ctx, OGM_ERR_INVALID, "weight_alloc_mb must be 0..1024");
-    ctx->tune_weight_alloc_mb = value;
-    return OGM_OK;
-  }
   if (strcmp(key, "gemv_fuse_quant") == 0) {
     if (value < -1 || value > 1) return fail(ctx, OGM_ERR_INVALID, "gemv_fuse_quant must be -1, 0 or 1");
     ctx->tune_fuse_quant = value < 0 ? 0 : value;  // -1 = the default
     return OGM_OK;
   }
   return fail(ctx, OGM_ERR_INVALID, std::string("unknown tuning key ") + key);
+}
+
+// Bytes of device and pinned host scratch the context has grown so far (weights and planes not counted).
+extern "C" size_t ogm_scratch_bytes(ogm_ctx *ctx) {
+  if (!ctx) return 0;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  const DevBuf *all[] = {&ctx->x,    &ctx->y,    &ctx->q,  &ctx->d,          &ctx->sums, &ctx->bsum, &ctx->bs16,
+                         &ctx->isum, &ctx->imin, &ctx->xh, &ctx->probe_sink, &ctx->hx,   &ctx->hy,   &ctx->hflag};
+  size_t n = 0;
+  for (const DevBuf *b : all) n += b->cap;
+  return n;
 }
 
 extern "C" const char *ogm_last_kernel(ogm_ctx *ctx) {
@@ -442,12 +447,7 @@ extern "C" int ogm_weight_upload(ogm_ctx *ctx, uint32_t ggml_type, const void *r
   w->key_addr = key_addr;
   w->key_len = key_len;
   w->dev = nullptr;
-  size_t alloc_bytes = bytes;
-  if (ctx->tune_weight_alloc_mb > 0 && bytes >= (1u << 20)) {
-    const size_t g = (size_t)ctx->tune_weight_alloc_mb << 20;
-    alloc_bytes = (bytes + g - 1) / g * g;
-  }
-  hipError_t e = hipMalloc((void **)&w->dev, alloc_bytes);
+  hipError_t e = hipMalloc((void **)&w->dev, bytes);
   if (e == hipSuccess) e = hipMemcpyAsync(w->dev, staging, bytes, hipMemcpyHostToDevice, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   (void)hipHostFree(staging);
@@ -1393,9 +1393,19 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   if (e == hipSuccess) e = hipMemset(m->attn_counters, 0, (size_t)2 * c.n_head_kv * OGM_ATTN_TICKET_STRIDE * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
-  for (uint32_t p0 = 0; m->rope_all && e == hipSuccess && p0 < c.max_ctx; p0 += 32768u) {
-    const uint32_t np = c.max_ctx - p0 < 32768u ? c.max_ctx - p0 : 32768u;
-    e = ogm_launch_rope_table(m->freq, p0, np, c.rope_dim, m->rope_all + (size_t)p0 * (c.rope_dim / 2) * 2, ctx->stream);
+  if (m->rope_all && e == hipSuccess) {
+    // (cos, sin) of pos * freq_i for every cache position, by the host's sinf / cosf -- the functions the
+    // reference's f32::sin_cos is (tensor.rs:1160) -- so a rotated row is the reference's to the bit given the
+    // same q or k.  (A cache too long for the table has each token's row computed on the device instead.)
+    const size_t half = c.rope_dim / 2;
+    std::vector<float> table((size_t)c.max_ctx * half * 2);
+    for (uint32_t p = 0; p < c.max_ctx; p++)
+      for (size_t i = 0; i < half; i++) {
+        const float theta = (float)p * freq[i];
+        table[((size_t)p * half + i) * 2] = cosf(theta);
+        table[((size_t)p * half + i) * 2 + 1] = sinf(theta);
+      }
+    e = hipMemcpy(m->rope_all, table.data(), table.size() * 4, hipMemcpyHostToDevice);
   }
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   if (e != hipSuccess) {

@@ -52,8 +52,8 @@ struct OgmAttnPre {
 //   * the merged output quantized for the next matmul in `mode`, and stored as f32 when attn_out
 //     is not null.
 // part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch, with
-// max_splits >= pos / chunk + 1; counters: 2 * n_head_kv words, zero before the first launch (the
-// kernel leaves them zero).  share: whether a K/V head's query heads are split over two workgroups
+// max_splits >= pos / chunk + 1; counters: 2 * n_head_kv * OGM_ATTN_TICKET_STRIDE words (one ticket per
+// cache line), zero before the first launch (the kernel leaves them zero).  share: whether a K/V head's query heads are split over two workgroups
 // (0: when there are four or eight of them and a half still fills whole quantizer groups; 1: never;
 // 2: asked for, an error where it cannot be).
 hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,

@@ -67,9 +67,13 @@ __global__ __launch_bounds__(64) void ogm_rope_table_kernel(const float *__restr
   const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= rope_half) return;
   const float theta = (float)(pos + blockIdx.y) * freq[p];   // row blockIdx.y: the token at pos + blockIdx.y
-  float sn, c;
-  sincosf(theta, &sn, &c);
-  cs[(size_t)blockIdx.y * rope_half + p] = make_float2(c, sn);
+  // The f32 angle's sine and cosine in double precision, rounded once: the correctly rounded f32 values but for
+  // rare double roundings, which is what the C library's sinf / cosf (the reference's f32::sin_cos) return as
+  // well.  The single-precision device routine differs from them in the last bit often enough to move a rotated
+  // K component across an f16 rounding boundary in a visible share of a cache row.
+  double sn, c;
+  sincos((double)theta, &sn, &c);
+  cs[(size_t)blockIdx.y * rope_half + p] = make_float2((float)c, (float)sn);
 }
 
 hipError_t ogm_launch_rope_table(const float *freq, uint32_t pos, uint32_t n_tokens, uint32_t rope_dim, void *cs,

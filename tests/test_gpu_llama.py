@@ -119,13 +119,13 @@ def step_both(ref, dev, x, pos, what, attn_rtol=1e-5):
             ulp = np.spacing(np.maximum(np.abs(mine), np.abs(theirs)).astype(np.float16)).astype(np.float64)
             off = a != b
             rowmax = np.abs(b).max()
-            # f32 budget: 1e-5 of the row's largest value, plus what one ulp of a pair's frequency
-            # (powf is not correctly rounded everywhere) does to the angle p * freq: p * 2^-23 radians
-            budget = (1e-5 + (p * 2.0 ** -23 if name == "k" else 0.0)) * rowmax
+            # f32 budget: 1e-5 of the row's largest value (the rotation's cosines and sines are the C library's
+            # on both sides, so position adds nothing)
+            budget = 1e-5 * rowmax
             assert (np.abs(a - b) <= ulp + budget).all(), \
                 f"{what}: layer {li} {name} cache row differs by more than one f16 step and the f32 budget " \
                 f"(worst {np.abs(a - b).max():.3g}, allowed {(ulp + budget)[np.abs(a - b).argmax()]:.3g})"
-            assert off.mean() <= 0.05 + (0.5 if name == "k" and p >= 1024 else 0.0), f"{what}: layer {li} {name} cache row: {off.sum()} of {off.size} elements differ"
+            assert off.mean() <= 0.05, f"{what}: layer {li} {name} cache row: {off.sum()} of {off.size} elements differ"
             out.append(theirs.copy())
         return out
 

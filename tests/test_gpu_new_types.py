@@ -169,3 +169,29 @@ def test_q5_1_min_term_is_added_not_subtracted_on_the_device(be):
     assert_bits(one, oracle.matmul(Q5_1, raw, 128, 3, x[:128], 1), "one token")
     assert_bits(be.matmul_decode(x, 3, w), oracle.matmul_decode(Q5_1, raw, 128, 3, x, 3), "decode batch")
     assert_bits(be.matmul(x, 3, w), oracle.matmul(Q5_1, raw, 128, 3, x, 3), "several tokens")
+
+
+def test_q2_k_two_step_calls_in_both_activation_modes(be):
+    """The two-step path (quantize once, multiply several weights) for Q2_K at several tokens: matmul runs over per-32
+    activations (cpu.rs:113-163), matmul_decode over per-256 ones (cpu.rs:265-317), so each has a quantize step of its
+    own; a matmul step over the other mode's activations is refused and says which step it needs."""
+    from orangu_amd import OgmError, hiprt
+    in_dim, out_dim, T = 1024, 37, 3
+    raw = synth_weights(Q2_K, in_dim, out_dim, seed=71)
+    x = synth_x(T, in_dim, seed=72)
+    h = be.upload_raw(raw, Q2_K, in_dim, out_dim)
+    xd, yd = hiprt.DeviceBuffer.from_numpy(x), hiprt.DeviceBuffer(4 * T * out_dim)
+    try:
+        for decode, ref in ((True, oracle.matmul_decode), (False, oracle.matmul)):
+            yd.fill(0xFF)
+            be.act_quantize_dev(Q2_K, xd.ptr, in_dim, T, decode=decode)
+            be.matmul_act_dev(h, T, yd.ptr, decode)
+            hiprt.device_synchronize()
+            assert_bits(yd.to_numpy(np.float32, T * out_dim), ref(Q2_K, raw, in_dim, out_dim, x, T),
+                        f"two-step Q2_K, decode={decode}")
+            with pytest.raises(OgmError, match="ogm_act_quantize_decode_dev"):
+                be.matmul_act_dev(h, T, yd.ptr, not decode)
+    finally:
+        be.free_weight(h)
+        xd.free()
+        yd.free()

@@ -1,6 +1,7 @@
 """The entry point that allocates nothing (ogm_matmul_dev_static) against ogm_matmul_dev, through
 the C ABI: same bits, on calls in a row that share the GPU's static scratch array, the later ones
-smaller than the first; sizes beyond the array are refused."""
+smaller than the first; sizes beyond the array are refused; and nothing is allocated (free device memory and
+the context's scratch unchanged across the calls, from a fresh context on)."""
 import numpy as np
 import pytest
 
@@ -52,6 +53,48 @@ def test_static_scratch_entry_equals_matmul_dev_on_calls_in_a_row(be):
         cpu = (oracle.matmul_decode if decode else oracle.matmul)(t, raw, in_dim, out_dim, x, T).reshape(-1)
         assert np.all(np.abs(got.astype(np.float64) - cpu) <= 1e-3 * np.abs(cpu) + 1e-5), (n, "against the CPU path")
     stream.destroy()
+
+
+def test_static_scratch_entry_allocates_nothing(be):
+    """The defining property: on a fresh context, whose grown-on-demand scratch is still empty, calls in a row --
+    the largest the array admits first -- leave the device's free memory and the context's scratch where they were."""
+    from orangu_amd import Mi355xBackend, hiprt
+    fresh = Mi355xBackend()
+    stream = hiprt.Stream()
+    shapes = [(Q4_K, 32768, 40, 8, False), (Q6_K, 14336, 70, 8, True), (Q8_0, 4096, 65, 3, False),
+              (Q4_K, 4096, 130, 1, False)]
+    held = []
+    try:
+        for n, (t, in_dim, out_dim, T, decode) in enumerate(shapes):
+            h = fresh.upload_raw(synth_weights(t, in_dim, out_dim, seed=300 + n), t, in_dim, out_dim)
+            xd = hiprt.DeviceBuffer.from_numpy(synth_x(T, in_dim, seed=400 + n))
+            yd = hiprt.DeviceBuffer(4 * T * out_dim)
+            held.append((h, xd, yd, T, decode))
+        # warm-up on another context: the runtime loads a kernel's code on its first launch in a process
+        for h, xd, yd, T, decode in held:
+            be.matmul_dev_static(h, xd.ptr, T, yd.ptr, decode, stream.ptr)
+        stream.synchronize()
+        hiprt.device_synchronize()
+        assert fresh.scratch_bytes() == 0          # nothing has run on this context yet
+        free0 = hiprt.mem_get_info()[0]
+        for _ in range(2):
+            for h, xd, yd, T, decode in held:
+                fresh.matmul_dev_static(h, xd.ptr, T, yd.ptr, decode, stream.ptr)
+        stream.synchronize()
+        assert fresh.scratch_bytes() == 0
+        assert hiprt.mem_get_info()[0] == free0
+        # the allocating entry point on the same inputs does grow the scratch: the check above can see a regression
+        h, xd, yd, T, decode = held[0]
+        fresh.matmul_dev(h, xd.ptr, T, yd.ptr, decode, stream.ptr)
+        stream.synchronize()
+        assert fresh.scratch_bytes() > 0
+    finally:
+        for h, xd, yd, _, _ in held:
+            fresh.free_weight(h)
+            xd.free()
+            yd.free()
+        stream.destroy()
+        fresh.close()
 
 
 def test_static_scratch_entry_refuses_what_does_not_fit(be):
