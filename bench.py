@@ -396,9 +396,6 @@ def main() -> int:
                     help="back-to-back launches between two HIP events (the event records leave a gap of their own)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--wg-waves", type=int, default=0, help="waves per workgroup override (0 = heuristic)")
-    ap.add_argument("--fuse-quant", type=int, default=-1,
-                    help="quantize inside the GEMV: -1 library's choice, 0 never, 1 always")
-    ap.add_argument("--rb-per-wg", type=int, default=0, help="row blocks per GEMV workgroup (0 = heuristic)")
     ap.add_argument("--separate", action="store_true",
                     help="issue gate and up as two calls instead of one grouped call")
     ap.add_argument("--gemm-tokens", type=int, default=512,
@@ -470,10 +467,6 @@ def main() -> int:
         return 0
     if args.wg_waves:
         be.set_tuning("gemv_wg_waves", args.wg_waves)
-    if args.rb_per_wg:
-        be.set_tuning("gemv_rb_per_wg", args.rb_per_wg)
-    if args.fuse_quant != -1:
-        be.set_tuning("gemv_fuse_quant", args.fuse_quant)
     stream = hiprt.Stream()
     only_leg = args.only_roofline or args.only_gemm or args.only_stream or bool(args.only_single) or bool(args.legs)
 

@@ -1,8 +1,9 @@
 /*
  * orangu_mi355x.h -- C ABI of the MI355X (gfx950) quantized matmul backend for orangu-server.
  *
- * This is the boundary a Rust `impl Backend` binds through FFI.  It replaces, for the GGUF types
- * Q8_0, Q5_0, Q4_0, IQ4_NL, Q3_K, Q4_K, Q5_K and Q6_K, what `engine::backend::Backend` asks of a device
+ * This is the boundary a Rust `impl Backend` binds through FFI.  It replaces, for the eleven GGUF types of the
+ * reference's fused path (vecdot.rs:274-283: Q8_0, Q5_0, Q5_1, Q4_0, IQ4_NL, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K and
+ * IQ4_XS), what `engine::backend::Backend` asks of a device
  * (src/bin/orangu-server/engine/backend/mod.rs:309-496) and reproduces the arithmetic of
  * `CpuBackend` (engine/backend/cpu.rs:55-317) over `engine::vecdot`:
  *   - activation int8 quantization, per-block integer sums: bit-exact with the CPU path;
@@ -47,12 +48,15 @@ typedef enum ogm_status {
 /* ggml type ids (engine/quant.rs:50-61) */
 #define OGM_TYPE_Q4_0 2u
 #define OGM_TYPE_Q5_0 6u
+#define OGM_TYPE_Q5_1 7u
 #define OGM_TYPE_Q8_0 8u
+#define OGM_TYPE_Q2_K 10u
 #define OGM_TYPE_Q3_K 11u
 #define OGM_TYPE_Q4_K 12u
 #define OGM_TYPE_Q5_K 13u
 #define OGM_TYPE_Q6_K 14u
 #define OGM_TYPE_IQ4_NL 20u
+#define OGM_TYPE_IQ4_XS 23u
 
 /* Activation quantization modes */
 #define OGM_ACT_PER_32 0  /* vecdot::quantize_act,       vecdot.rs:79-126   (Q8_0 weights)   */
@@ -381,70 +385,54 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
 
 /* ---- tuning / introspection ------------------------------------------------------------------ */
 
-/* Kernel launch parameters the host picks per shape; exposed so a benchmark can sweep them.
- * keys: "gemv_wg_waves" (waves per workgroup of the GEMV kernel, 1..16; 0 = heuristic);
- * "gemm_min_tokens" (ogm_matmul takes the MFMA GEMM from this many tokens on; 0 = default: 6 for
- * Q4_K, Q5_K and Q6_K -- Q6_K 4096 -> 128256 at 8 tokens: 122 us on the small-batch kernel against 178 us --
- * and 17 for the other types;
- * below it the multi-token GEMV kernel runs in the GEMM's float order);
- * "gemm_q4k_variant" (K-quant GEMM: 0 = default, the int8 matrix-core kernels over scale-folded
- * weight planes; 1 = the same, always on 64-row tiles; 2 = the f16 kernels; 3 = for Q4_K and Q5_K the
- * int8 kernel that scales partial sums by multiply-adds);
- * "gemm_wide_min_wgs" (f16 Q4_K kernels: 128 x 128 workgroups from which the 128 x 256 tile runs; 0 = 256);
- * "gemm_small_max_tokens" (K-quant GEMMs of at most this many tokens take the small-batch kernel, whose
- * waves work on different super-blocks of the same rows; 0 = default 64, or 128 for matrices of up to
- * 8192 rows; 1 = never);
- * "gemm_few_tokens_min_rows" (2 to 16 tokens over a Q6_K matrix -- matmul and matmul_decode alike -- take
- * the kernel that streams the weights once and multiplies every token on the matrix cores when the matrix
- * has at least this many rows: 0 = default, 30000 rows (a vocabulary projection) and at least three tokens; 1 = whenever the shape
- * allows: in_dim a multiple of 1024 whose int8 rows fit LDS; -1 = never);
- * "gemm_sb_waves" (waves of a small-batch workgroup: 8 or 16; 0 = default, 16 for launches of at most
- * 256 workgroups over rows of at least 16 super-blocks);
- * "attn_prefill_variant" (attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the
- * decode step's kernel per token and chunk of the cache; they agree to f32 rounding, not bit for bit);
- * "gemm_plane_cache_mb" (device memory, in MiB, that the K-quant matrices' prefill planes may take in all,
- * default 32768: on a matrix's first GEMM that would read them its scale-folded int8 planes -- 2 bytes
- * per weight, 1 for Q3_K -- are built once and kept, and later calls multiply them instead of unpacking the
- * weights again; a matrix that no longer fits the budget, and every matrix at 0, is unpacked on every call;
- * same bits either way, and ogm_weight_download is unaffected);
- * "gemm_plane_kernel" (which kernel reads the planes: 0 = default, the one whose waves all multiply, fed by
- * loads straight into LDS, when the launch has more than 256 tiles of 128 rows x 128 tokens, and otherwise
- * none: the feeding-wave kernels unpack; 1 = the feeding-wave kernels read them; 2 = the former whatever the
- * grid, from 32 tokens; same bits);
- * "gemm_one_pass" (0 = default; 1: Q4_K and Q5_K on that kernel skip the reference GEMM's separate first pass over
- * the mins (vecdot.rs:2229-2240) and add ad * (d * isum - dmin * imin) per super-block, the single-token
- * expression of vecdot.rs:3152-3178: the integer sums are the same, the f32 result is no longer the reference
- * GEMM's bits -- both orders sit about 1e-7 of sum|w x| from exact arithmetic, well inside the 1e-3 * sum|w x| the
- * reference's tests allow between its two orders (vecdot.rs:3518-3525), but an output whose terms cancel to near
- * zero can differ from the reference's by more than 1e-3 of itself; 4096 -> 14336 at 512 tokens: 94 against 112 us
- * per call, a 2048-token prefill of the 8B shapes 38.2 against 42.8 ms);
- * "host_zero_copy" (1 = default: a host-pointer call -- ogm_matmul, ogm_matmul_decode, ogm_matmul_batch --
- * whose x and y together are at most 512 KiB runs its kernels directly on the pinned staging buffers, with
- * no copy-engine transfer: 23 us against 33 us per 4096 -> 14336 call; 0: always stage through device
- * memory, as larger calls do);
- * "host_flag_wait" (1 = default: such a call waits for its results by polling a word in pinned memory that a
- * one-thread kernel behind the call's kernels stores, instead of waiting on the stream: 19 us against 23 us per
- * 4096 -> 14336 call; after 5 ms without the word, and on every 256th call, the stream is synchronized after all;
- * 0: always hipStreamSynchronize; 2: for tests of the bounded wait, the word never matches and every call runs
- * into the 5 ms);
- * "gemv_rb_per_wg" (row blocks one GEMV workgroup owns, 1..64; 0 = default 1);
- * "gemv_fuse_quant" (1: a single-token GEMV quantizes its activations itself instead of running
- * the quantizer kernel first; 0 or -1 = default, off);
- * "attn_decode_share" (decode attention: 1 = default, one workgroup per K/V head and chunk of the cache; 2 = the
- * query heads of a K/V head split over two workgroups where four or eight of them allow it: twice the
- * workgroups, measured 2 us a layer slower at 2048 cached positions; results agree to f32 rounding);
- * "prefill_chunk_tokens" (tokens per pass of ogm_llama_prefill over the layers, default 2048; a model keeps
- * the value of its first prefill, whose row buffers are allocated for it; 8B shapes: 2048 tokens 45.3 against
- * 49.0 ms with 1024, a pass of 4096 is slower again);
- * "decode_fuse_heads" (1: the decode step's attention norm, FFN norm and SwiGLU run at the head of the GEMV
- * launch after them -- extra workgroups at the front of the launch, a flag, the others waiting behind their first
- * weight loads -- instead of as kernels of their own; same bits, measured slower, off by default; with it
- * "decode_head_delay" (what the waiting workgroups sleep before their weight loads, in units of 64 clocks,
- * default 64) and "decode_head_spin_limit" (polls before a waiting workgroup gives up, 0 = default 200000: the
- * step then fails with OGM_ERR_HIP at its next synchronisation instead of returning its results as good));
- * "decode_fuse_tails" (1: the decode step's FFN norm, SwiGLU and next attention norm run inside the
- * GEMV launch before them, in its last workgroup to finish; 0 = default, kernels of their own, which
- * is faster; same bits).  No other setting changes a result bit. */
+/* Kernel choices the host makes per shape, exposed so that a benchmark can sweep them and a test can reach
+ * every kernel on small shapes.  Unknown keys and values out of range return OGM_ERR_INVALID.  Only
+ * "gemm_one_pass" and "attn_prefill_variant" can change a result bit; every other setting selects among
+ * kernels that produce the same bits.
+ *   "gemv_wg_waves"            waves per workgroup of the GEMV kernel, 1..16; 0 = by the row's tile count
+ *   "gemm_min_tokens"          ogm_matmul takes a matrix-core GEMM from this many tokens on; 0 = default (6 for
+ *                              Q4_K, Q5_K and Q6_K, 17 for the other types); below it the multi-token GEMV
+ *                              kernel runs in the GEMM's float order
+ *   "gemm_small_max_tokens"    K-quant GEMMs of at most this many tokens take the small-batch kernel, whose
+ *                              waves work on different super-blocks of the same rows; 0 = default (64, more
+ *                              for matrices of few rows), 1 = never
+ *   "gemm_sb_waves"            waves of a small-batch workgroup: 8 or 16; 0 = by the size of the launch
+ *   "gemm_tile_rows"           feeding-wave GEMMs: 64 = always their 64-row tiles; 0 = by the size of the launch
+ *   "gemm_few_tokens_min_rows" 2 to 16 tokens over a Q6_K matrix (matmul and matmul_decode alike) take the
+ *                              kernel that streams the weights once when the matrix has at least this many
+ *                              rows; 0 = default (30000 rows and three tokens), 1 = whenever the shape allows,
+ *                              -1 = never
+ *   "gemm_plane_cache_mb"      device memory, in MiB, that the K-quant matrices' prefill planes may take in all
+ *                              (default 32768): on a matrix's first GEMM that would read them its scale-folded
+ *                              int8 planes (2 bytes per weight, 1 for Q3_K) are built once and kept; a matrix
+ *                              that does not fit, and every matrix at 0, is unpacked on every call;
+ *                              ogm_weight_download is unaffected
+ *   "gemm_plane_kernel"        when the kernel that multiplies the planes (all waves multiply, operands loaded
+ *                              straight into LDS) runs: 0 = default, when the launch has more than 256 tiles of
+ *                              128 rows x 128 tokens (the feeding-wave kernels unpack otherwise); 2 = whatever
+ *                              the grid, from 32 tokens
+ *   "gemm_one_pass"            0 = default.  1: Q4_K and Q5_K on that kernel skip the reference GEMM's separate
+ *                              first pass over the mins (vecdot.rs:2229-2240) and add
+ *                              ad * (d * isum - dmin * imin) per super-block, the single-token expression of
+ *                              vecdot.rs:3152-3178.  The integer sums are the same; the f32 result is within
+ *                              rounding of the reference GEMM's, not its bits: an output whose terms cancel to
+ *                              near zero can differ from the reference's by more than 1e-3 of itself
+ *   "attn_prefill_variant"     attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the decode
+ *                              step's kernel per token and chunk of the cache; they agree to f32 rounding
+ *   "prefill_chunk_tokens"     tokens per pass of ogm_llama_prefill over the layers, default 2048; a model keeps
+ *                              the value of its first prefill, whose row buffers are allocated for it
+ *   "host_zero_copy"           1 = default: a host-pointer call (ogm_matmul, ogm_matmul_decode,
+ *                              ogm_matmul_batch) whose x and y together are at most 512 KiB runs its kernels
+ *                              directly on the pinned staging buffers, with no copy-engine transfer; 0 = always
+ *                              stage through device memory, as larger calls do.  The staging buffers are
+ *                              allocated as coherent (fine-grained) host memory by name; where the runtime
+ *                              refuses that, the context behaves as with 0 and "host_flag_wait" 0
+ *   "host_flag_wait"           1 = default: such a call waits for its results by polling a word in that pinned
+ *                              memory which a one-thread kernel behind the call's kernels stores, instead of
+ *                              waiting on the stream; after 5 ms without the word, and on every 256th call,
+ *                              the stream is synchronized after all; 0 = always hipStreamSynchronize; 2 = for
+ *                              tests of the bounded wait: the word never matches and every call runs into the
+ *                              5 ms */
 int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value);
 /* For benchmarks driven from an interpreter: runs host-pointer calls from compiled code and writes each
  * repetition's wall time in microseconds to us_out[reps].  `ops` holds n_variants sets of n_ops ops;

@@ -59,25 +59,17 @@ struct ogm_ctx {
   // tokens: 12 against 16 us), 17 for the others, whose tiled kernels cost about the same from 9 to 128
   // tokens while the chunked GEMV grows with the count (they cross between 12 and 32 tokens).
   int tune_gemm_min_tokens = 0;
-  int tune_gemm_wide_min_wgs = 0;
-  int tune_gemm_q4k_variant = 0;
+  int tune_gemm_tile_rows = 0;   // feeding-wave GEMMs: 64 forces their 64-row tiles, 0 = by the size of the launch
   int tune_gemm_small_max = 0;   // most tokens for the small-batch GEMM kernel: 0 = default, 1 = never
   int tune_gemm_ft_min_rows = 0;  // few-token Q6_K kernel: fewest rows it takes (0 = default, 1 = any shape it can, -1 = never)
   int tune_gemm_sb_waves = 0;          // small-batch GEMM: 8 or 16 waves per workgroup, 0 = by the launch
   int tune_host_flag_wait = 1;         // zero-copy host calls wait on a word a trailing kernel stores to pinned memory instead of on the stream
   int tune_host_zero_copy = 1;         // host-pointer calls of up to OGM_ZERO_COPY_MAX bytes: kernels read x / write y in pinned host memory
   bool host_coherent = true;           // the pinned staging buffers are fine-grained (asked for by name); false once the runtime has refused
-  int tune_gemm_plane_kernel = 0;      // who reads planes: 0 the all-waves-multiply kernel on large grids, 1 the feeding-wave kernels, 2 the former always
+  int tune_gemm_plane_kernel = 0;      // the all-waves-multiply kernel over planes: 0 on large grids, 2 whatever the grid
   int tune_gemm_one_pass = 0;          // 1: Q4_K / Q5_K on that kernel fold the min pass into the super-block step (f32 to rounding, not to the bit)
-  int tune_decode_fuse_heads = 0;      // 1: the decode step's norms and SwiGLU at the head of the GEMV after them
-  int tune_decode_head_delay = 64;     // fused heads: what the waiting workgroups sleep before their weight loads, x 64 clocks
-  int tune_decode_head_spin = 0;       // fused heads: polls before a waiting workgroup gives up (0 = default)
-  int tune_attn_decode_share = 1;      // decode attention: 2 splits a K/V head's query heads over two workgroups where possible (slower), 1 never
   int tune_prefill_chunk = 2048;       // tokens per prefill pass over the layers (fixed per model at its first prefill)
-  int tune_decode_fuse_tails = 0;      // 1: the decode step's norms and SwiGLU inside the GEMV before them (slower)
   int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
-  int tune_rb_per_wg = 0;        // row blocks per GEMV workgroup, 0 = by shape
-  int tune_fuse_quant = 0;       // quantize inside the single-token GEMV: 0 no, 1 yes
   // Device memory the prefill planes of all weights may take, in MiB; 0 (the default) = build none.
   // A model's planes are 3.3 times its Q4_K bytes.
   int tune_plane_cache_mb = 32768;   // MiB the K-quant matrices' prefill planes may take in all
@@ -286,11 +278,6 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_gemm_min_tokens = value;
     return OGM_OK;
   }
-  if (strcmp(key, "gemm_wide_min_wgs") == 0) {
-    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_wide_min_wgs must be >= 0");
-    ctx->tune_gemm_wide_min_wgs = value;
-    return OGM_OK;
-  }
   if (strcmp(key, "gemm_small_max_tokens") == 0) {
     if (value < 0 || value > 1024) return fail(ctx, OGM_ERR_INVALID, "gemm_small_max_tokens must be 0..1024");
     ctx->tune_gemm_small_max = value;
@@ -306,8 +293,13 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_host_zero_copy = value;
     return OGM_OK;
   }
+  if (strcmp(key, "gemm_tile_rows") == 0) {
+    if (value != 0 && value != 64) return fail(ctx, OGM_ERR_INVALID, "gemm_tile_rows must be 0 or 64");
+    ctx->tune_gemm_tile_rows = value;
+    return OGM_OK;
+  }
   if (strcmp(key, "gemm_plane_kernel") == 0) {
-    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_kernel must be 0, 1 or 2");
+    if (value != 0 && value != 2) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_kernel must be 0 or 2");
     ctx->tune_gemm_plane_kernel = value;
     return OGM_OK;
   }
@@ -326,34 +318,9 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_gemm_sb_waves = value;
     return OGM_OK;
   }
-  if (strcmp(key, "decode_fuse_heads") == 0) {
-    if (value < 0 || value > 1) return fail(ctx, OGM_ERR_INVALID, "decode_fuse_heads must be 0 or 1");
-    ctx->tune_decode_fuse_heads = value;
-    return OGM_OK;
-  }
-  if (strcmp(key, "decode_head_spin_limit") == 0) {
-    if (value < 0) return fail(ctx, OGM_ERR_INVALID, "decode_head_spin_limit must be >= 0");
-    ctx->tune_decode_head_spin = value;
-    return OGM_OK;
-  }
-  if (strcmp(key, "decode_head_delay") == 0) {
-    if (value < 0 || value > 1000) return fail(ctx, OGM_ERR_INVALID, "decode_head_delay must be 0..1000");
-    ctx->tune_decode_head_delay = value;
-    return OGM_OK;
-  }
-  if (strcmp(key, "attn_decode_share") == 0) {
-    if (value < 1 || value > 2) return fail(ctx, OGM_ERR_INVALID, "attn_decode_share must be 1 or 2");
-    ctx->tune_attn_decode_share = value;
-    return OGM_OK;
-  }
   if (strcmp(key, "prefill_chunk_tokens") == 0) {
     if (value < 1 || value > 16384) return fail(ctx, OGM_ERR_INVALID, "prefill_chunk_tokens must be 1..16384");
     ctx->tune_prefill_chunk = value;
-    return OGM_OK;
-  }
-  if (strcmp(key, "decode_fuse_tails") == 0) {
-    if (value < 0 || value > 1) return fail(ctx, OGM_ERR_INVALID, "decode_fuse_tails must be 0 or 1");
-    ctx->tune_decode_fuse_tails = value;
     return OGM_OK;
   }
   if (strcmp(key, "attn_prefill_variant") == 0) {
@@ -361,24 +328,9 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_attn_prefill_variant = value;
     return OGM_OK;
   }
-  if (strcmp(key, "gemm_q4k_variant") == 0) {
-    if (value < 0 || value > 3) return fail(ctx, OGM_ERR_INVALID, "gemm_q4k_variant must be 0..3");
-    ctx->tune_gemm_q4k_variant = value;
-    return OGM_OK;
-  }
-  if (strcmp(key, "gemv_rb_per_wg") == 0) {
-    if (value < 0 || value > 64) return fail(ctx, OGM_ERR_INVALID, "gemv_rb_per_wg must be 0..64");
-    ctx->tune_rb_per_wg = value;
-    return OGM_OK;
-  }
   if (strcmp(key, "gemm_plane_cache_mb") == 0) {
     if (value < 0) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_cache_mb must be >= 0");
     ctx->tune_plane_cache_mb = value;
-    return OGM_OK;
-  }
-  if (strcmp(key, "gemv_fuse_quant") == 0) {
-    if (value < -1 || value > 1) return fail(ctx, OGM_ERR_INVALID, "gemv_fuse_quant must be -1, 0 or 1");
-    ctx->tune_fuse_quant = value < 0 ? 0 : value;  // -1 = the default
     return OGM_OK;
   }
   return fail(ctx, OGM_ERR_INVALID, std::string("unknown tuning key ") + key);
@@ -528,14 +480,7 @@ struct Target {
 
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
                         hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
-                        const float *x_f32, const OgmGemvTail *tail = nullptr, const OgmActDev *act_base = nullptr,
-                        const OgmGemvHead *head = nullptr);
-
-// Whether a single-token launch quantizes inside the GEMV (every workgroup repeats the
-// quantizer on its way in) instead of running the quantizer kernel first.  Off unless asked
-// for: on MI355X the repeated work costs more than the launch it saves (Llama-8B FFN block:
-// 28.3 us per pass against 25.9 us).
-static bool fuse_quantize(ogm_ctx *ctx, const Target *, size_t) { return ctx->tune_fuse_quant > 0; }
+                        const OgmActDev *act_base = nullptr);
 
 // Enqueues quantize + kernels for tokens of x_dev into the targets' outputs.  Caller holds the
 // lock and has checked that the targets share type and in_dim.
@@ -544,11 +489,9 @@ static int enqueue_matmul(ogm_ctx *ctx, const Target *tg, size_t n_tg, const flo
                           int32_t *dump_imin) {
   if (n_tokens == 0 || n_tg == 0) return OGM_OK;
   const ogm_weight *w = tg[0].w;
-  if (n_tokens == 1 && !dump_isum && !dump_imin && fuse_quantize(ctx, tg, n_tg))
-    return enqueue_gemv(ctx, tg, n_tg, 1, decode, stream, nullptr, nullptr, x_dev);
   int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type, n_tokens, decode), x_dev, w->in_dim, n_tokens, stream);
   if (rc != OGM_OK) return rc;
-  return enqueue_gemv(ctx, tg, n_tg, n_tokens, decode, stream, dump_isum, dump_imin, nullptr);
+  return enqueue_gemv(ctx, tg, n_tg, n_tokens, decode, stream, dump_isum, dump_imin);
 }
 
 static int enqueue_matmul(ogm_ctx *ctx, const ogm_weight *w, const float *x_dev, uint32_t n_tokens,
@@ -595,17 +538,12 @@ static bool all_gemm_supported(const Target *tg, size_t n_tg, uint32_t n_tokens)
   return true;
 }
 
-// Enqueues the matmul kernels over the context's quantized activations (or, with x_f32, over
-// one token of f32 activations that the kernel quantizes itself).  Caller holds the lock.
+// Enqueues the matmul kernels over the context's quantized activations.  Caller holds the lock.
 // act_base: the quantized activations to read instead of the context's scratch; such a call stays
 // on the GEMV kernels whatever the token count (the tiled GEMMs stage through context buffers).
 static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_tokens, int decode,
-                        hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin,
-                        const float *x_f32, const OgmGemvTail *tail, const OgmActDev *act_base,
-                        const OgmGemvHead *head) {
+                        hipStream_t stream, int32_t *dump_isum, int32_t *dump_imin, const OgmActDev *act_base) {
   const ogm_weight *w0 = tg[0].w;
-  if (head && (n_tokens != 1 || tail || x_f32 || dump_isum || dump_imin)) return fail(ctx, OGM_ERR_INVALID, "a GEMV head needs a plain launch of one token");
-  if (tail && (n_tokens != 1 || n_tg > OGM_GEMV_MAX_MATS)) return fail(ctx, OGM_ERR_INVALID, "a GEMV tail needs one launch of one token");
   const int mode = act_mode_for(w0->ggml_type, n_tokens, decode);
   // backend/cpu.rs:55-167: matmul at n_tokens > 1 takes the GEMM kernels (their float order);
   // n_tokens == 1 and every matmul_decode take the GEMV's.
@@ -615,7 +553,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
                              : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 6u : 17u;
   // A few tokens over a Q6_K matrix of many rows (the vocabulary projection of a decode batch): one
   // streaming pass on the matrix cores, in either float order.
-  if (n_tokens > 1 && !dump_isum && !dump_imin && !act_base && !x_f32 && !tail && ctx->tune_gemm_ft_min_rows >= 0) {
+  if (n_tokens > 1 && !dump_isum && !dump_imin && !act_base && ctx->tune_gemm_ft_min_rows >= 0) {
     bool all = true;
     for (size_t i = 0; i < n_tg; i++)
       all = all && ogm_gemm_ft_eligible(tg[i].w->ggml_type, tg[i].w->in_dim, tg[i].w->out_dim, n_tokens,
@@ -654,8 +592,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.n_tokens = n_tokens;
       g.y = tg[i].y;
       g.xh = ctx->xh.p;
-      g.wide_min_wgs = (uint32_t)ctx->tune_gemm_wide_min_wgs;
-      g.q4k_variant = (uint32_t)ctx->tune_gemm_q4k_variant;
+      g.tile_rows = (uint32_t)ctx->tune_gemm_tile_rows;
       g.small_max_tokens = (uint32_t)ctx->tune_gemm_small_max;
       g.sb_waves = (uint32_t)ctx->tune_gemm_sb_waves;
       g.plane_kernel = (uint32_t)ctx->tune_gemm_plane_kernel;
@@ -696,7 +633,6 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       a.y = tg[g0].y + (size_t)t0 * a.out_dim;
       a.gemm_order = gemm_order;
       a.wg_waves = wg_waves;
-      a.rb_per_wg = (uint32_t)ctx->tune_rb_per_wg;
       a.dump_isum = dump_isum ? dump_isum + (size_t)t0 * a.out_dim * blocks_per_row : nullptr;
       a.dump_imin = dump_imin ? dump_imin + (size_t)t0 * a.out_dim * blocks_per_row : nullptr;
       a.n_extra = (uint32_t)ng - 1;
@@ -705,9 +641,6 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
         a.extra_out_dim[i - 1] = tg[g0 + i].w->out_dim;
         a.extra_y[i - 1] = tg[g0 + i].y + (size_t)t0 * tg[g0 + i].w->out_dim;
       }
-      a.x_f32 = x_f32;
-      if (tail) a.tail = *tail;
-      if (head && g0 == 0 && t0 == 0) a.head = *head;   // the first launch of the group brings the producers
       HIPCHK(ctx, ogm_launch_gemv(a, stream, &ctx->last_kernel));
     }
   }
@@ -842,7 +775,7 @@ extern "C" int ogm_matmul_dev_static(ogm_ctx *ctx, const ogm_weight *w, const fl
   // array has to start at zero, and what an earlier call left beyond them is never read.
   HIPCHK(ctx, ogm_launch_quantize(mode, x_dev, w->in_dim, n_tokens, act, s));
   const Target t{w, y_dev};
-  return enqueue_gemv(ctx, &t, 1, n_tokens, decode, s, nullptr, nullptr, nullptr, nullptr, &act);
+  return enqueue_gemv(ctx, &t, 1, n_tokens, decode, s, nullptr, nullptr, &act);
 }
 
 // For benchmarks driven from an interpreter: runs host-pointer calls `reps` times from compiled code and
@@ -960,7 +893,7 @@ extern "C" int ogm_matmul_act_dev(ogm_ctx *ctx, const ogm_weight *w, uint32_t n_
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
   const Target t{w, y_dev};
-  return enqueue_gemv(ctx, &t, 1, n_tokens, decode, s, nullptr, nullptr, nullptr);
+  return enqueue_gemv(ctx, &t, 1, n_tokens, decode, s, nullptr, nullptr);
 }
 
 // Checks a group of weights and collects its targets.
@@ -1006,7 +939,7 @@ extern "C" int ogm_matmul_multi_act_dev(ogm_ctx *ctx, const ogm_weight *const *w
     return fail(ctx, OGM_ERR_INVALID, act_mismatch(ctx, ws[0], n_tokens, decode));
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
-  return enqueue_gemv(ctx, tg.data(), n_ws, n_tokens, decode, s, nullptr, nullptr, nullptr);
+  return enqueue_gemv(ctx, tg.data(), n_ws, n_tokens, decode, s, nullptr, nullptr);
 }
 
 // `reps` launches enqueued back to back from compiled code (for benchmarks driven from an interpreter, whose
@@ -1234,9 +1167,7 @@ struct ogm_llama {
   float *freq = nullptr;      // [rope_dim / 2], frequency factors applied
   float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
   float *rope_all = nullptr;  // the same for every position of the cache, filled at creation (null: too large, computed per token)
-  uint32_t head_epoch = 0;            // value of the GEMV heads' flag (the three words after the tickets) after the last launch
   uint32_t *attn_counters = nullptr;  // [2 n_head_kv][OGM_ATTN_TICKET_STRIDE] the attention kernel's tickets, a line each; zero between launches
-  uint32_t *attn_tickets = nullptr;   // [2 n_head_kv] (unused),  then the GEMV tails' tickets and the heads' flags; zero between launches
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
   void *v_cache = nullptr;
   float *x = nullptr;         // hidden state [n_embd]
@@ -1335,7 +1266,6 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   // positions); a decode step then launches no table kernel
   const size_t rope_all_bytes = (size_t)c.max_ctx * (c.rope_dim / 2) * 8;
   if (c.rope_dim != 0 && rope_all_bytes <= ((size_t)64 << 20)) A((void **)&m->rope_all, rope_all_bytes);
-  A((void **)&m->attn_tickets, ((size_t)2 * c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);   // + the GEMV tails' tickets
   A((void **)&m->attn_counters, (size_t)2 * c.n_head_kv * OGM_ATTN_TICKET_STRIDE * 4);
   A(&m->k_cache, cache_bytes);
   A(&m->v_cache, cache_bytes);
@@ -1389,7 +1319,6 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   hipError_t e = hipMemcpy(m->norms, host.data(), host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->pre, pre_host.data(), pre_host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMemset(m->attn_tickets, 0, ((size_t)2 * c.n_head_kv + OGM_TAIL_TICKETS + 32 + OGM_HEAD_FLAG_WORDS) * 4);
   if (e == hipSuccess) e = hipMemset(m->attn_counters, 0, (size_t)2 * c.n_head_kv * OGM_ATTN_TICKET_STRIDE * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
@@ -1487,14 +1416,8 @@ static int llama_capture(ogm_ctx *ctx, ogm_llama *m, uint32_t site, uint32_t n, 
 }
 
 // One matmul group of the step over the activations the previous kernel quantized.
-static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, hipStream_t s,
-                        const OgmGemvTail *tail = nullptr, const OgmGemvHead *head = nullptr) {
+static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n, hipStream_t s) {
   // weights of one type go out as one launch; a mixed group (Q4_K q/k with a Q6_K v) as several
-  if (tail) {   // the caller has checked that the group is one launch
-    Target tg[OGM_GEMV_MAX_MATS];
-    for (size_t i = 0; i < n; i++) tg[i] = Target{ws[i], ys[i]};
-    return enqueue_gemv(ctx, tg, n, 1, 0, s, nullptr, nullptr, nullptr, tail);
-  }
   size_t i = 0;
   while (i < n) {
     Target tg[OGM_GEMV_MAX_MATS];
@@ -1503,14 +1426,15 @@ static int llama_matmul(ogm_ctx *ctx, const ogm_weight *const *ws, float *const 
       tg[e - i] = Target{ws[e], ys[e]};
       e++;
     }
-    // (a head's producers ride on the first launch; the launches after it are ordered behind it)
-    int rc = enqueue_gemv(ctx, tg, e - i, 1, 0, s, nullptr, nullptr, nullptr, nullptr, nullptr, i == 0 ? head : nullptr);
+    int rc = enqueue_gemv(ctx, tg, e - i, 1, 0, s, nullptr, nullptr);
     if (rc != OGM_OK) return rc;
     i = e;
   }
   return OGM_OK;
 }
 
+// LlamaModel::run_layers + forward at one token (arch/llama.rs:594-932, 1007-1032), eight launches a layer:
+// norm (+ quantize), q/k/v, attention (+ quantize), wo, norm (+ quantize), gate/up, SwiGLU (+ quantize), down.
 static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, uint32_t pos, float *logits_dev,
                                 uint32_t *argmax_dev, hipStream_t s) {
   const ogm_llama_config &c = m->cfg;
@@ -1521,53 +1445,11 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
   const float *rope_cs = m->rope_all ? m->rope_all + (size_t)pos * (c.rope_dim / 2) * 2 : m->rope_cs;
   if (!m->rope_all) HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos, 1, c.rope_dim, m->rope_cs, s));
   const float *delta = nullptr;  // what the next norm adds to x first: the last block's output
-  // On request, with per-256 activations on the consumer's side, a norm or the SwiGLU runs as the
-  // tail of the GEMV launch before it (its last workgroup to finish) instead of as a kernel of its
-  // own.  Same bits, but slower on MI355X (8B-shaped model: 2.59 against 1.94 ms per token): every
-  // workgroup then waits for its coherent stores and a ticket before it leaves, which costs more
-  // than the three 4 us kernels a layer saves.
-  const bool fuse = ctx->tune_decode_fuse_tails != 0 && ctx->tune_fuse_quant <= 0;
-  auto tail_ok = [&](const ogm_weight *producer, uint32_t n, int consumer_mode) {
-    return fuse && consumer_mode == OGM_ACT_PER_256 && n % 32u == 0 && producer->out_dim == n &&
-           n <= ogm_gemv_norm_tail_max(producer->ggml_type, producer->in_dim, n, (uint32_t)ctx->tune_wg_waves);
-  };
-  // On request the norms and the SwiGLU run at the *head* of the GEMV launch after them: extra
-  // workgroups at the front of the launch compute and quantize the row while the others already have
-  // their first weights in flight, and hand it over through device-coherent stores and a flag.  Same
-  // bits, and slower on MI355X (8B-shaped model: 2.06 against 1.86 ms per token): the hand-over is a
-  // chain of trips to the memory all compute dies share (stores acknowledged, flag stored, flag
-  // polled, activations loaded) that costs what the kernel boundary it replaces costs, and the
-  // producers' own loads queue behind the launch's weight stream.
-  const bool heads = ctx->tune_decode_fuse_heads != 0 && !fuse && ctx->tune_fuse_quant <= 0;
-  // The caller's row becomes the residual stream: the first norm reads it where it lies and stores it to
-  // m->x, unless that norm runs inside a GEMV launch, which works on m->x alone.
-  const float *x_first = nullptr;
-  if (x_dev != m->x) {
-    if (fuse || heads) HIPCHK(ctx, hipMemcpyAsync(m->x, x_dev, (size_t)c.n_embd * 4, hipMemcpyDeviceToDevice, s));
-    else x_first = x_dev;
-  }
-  uint32_t *head_flag = m->attn_tickets + ((2u * c.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u);   // 128-byte aligned
-  auto head_ok = [&](const ogm_weight *first, int mode, bool norm) {   // first: the matrix of the group's first launch
-    if (!heads || mode != OGM_ACT_PER_256) return false;
-    const uint32_t waves = ogm_gemv_head_waves(first->ggml_type, first->in_dim, first->out_dim, (uint32_t)ctx->tune_wg_waves);
-    return waves != 0 && (!norm || first->in_dim <= 1024u * waves);   // one producer workgroup norms the whole row
-  };
-  auto norm_head = [&](const float *delta_, const float *weight_) {
-    OgmGemvHead h;
-    h.kind = OGM_HEAD_NORM;
-    h.flag = head_flag;
-    h.epoch = ++m->head_epoch;
-    h.x = m->x;
-    h.delta = delta_;
-    h.weight = weight_;
-    h.eps = c.rms_eps;
-    h.delay = (uint32_t)ctx->tune_decode_head_delay;
-    h.spin_limit = (uint32_t)ctx->tune_decode_head_spin;
-    return h;
-  };
+  // The caller's row becomes the residual stream: the first norm reads it where it lies and stores it to m->x.
+  const float *x_first = x_dev != m->x ? x_dev : nullptr;
   const int mode_out = act_mode_for(m->output->ggml_type);
   const float *out_norm = m->norms + (size_t)c.n_layer * 2 * c.n_embd;
-  bool normed = false;   // the next norm already ran as a tail
+  int rc;
   for (uint32_t l = 0; l < c.n_layer; l++) {
     const ogm_llama_layer &L = m->layers[l];
     const float *attn_norm = m->norms + (size_t)l * 2 * c.n_embd, *ffn_norm = attn_norm + c.n_embd;
@@ -1580,119 +1462,41 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
       return fail(ctx, OGM_ERR_UNSUPPORTED, "wq, wk and wv must share an activation mode");
     const ogm_weight *w3[3] = {L.wq, L.wk, L.wv};
     float *y3[3] = {m->q, m->k, m->v};
-    int rc;
-    if (!normed && head_ok(L.wq, mode_qkv, true)) {
-      // the norm rides at the head of the q/k/v launch
-      OgmGemvHead head = norm_head(delta, attn_norm);
-      if ((rc = llama_matmul(ctx, w3, y3, 3, s, nullptr, &head)) != OGM_OK) return rc;
-      if ((rc = llama_capture(ctx, m, 4 * l, c.n_embd, mode_qkv, s)) != OGM_OK) return rc;
-    } else {
-      if (!normed)
-        HIPCHK(ctx, ogm_launch_norm_quant(mode_qkv, m->x, delta, attn_norm, c.n_embd, c.rms_eps, nullptr,
-                                          act_view(ctx, c.n_embd, mode_qkv, 0), s, 1, l == 0 ? x_first : nullptr));
-      if ((rc = llama_capture(ctx, m, 4 * l, c.n_embd, mode_qkv, s)) != OGM_OK) return rc;
-      if ((rc = llama_matmul(ctx, w3, y3, 3, s)) != OGM_OK) return rc;
-    }
+    HIPCHK(ctx, ogm_launch_norm_quant(mode_qkv, m->x, delta, attn_norm, c.n_embd, c.rms_eps, nullptr,
+                                      act_view(ctx, c.n_embd, mode_qkv, 0), s, 1, l == 0 ? x_first : nullptr));
+    if ((rc = llama_capture(ctx, m, 4 * l, c.n_embd, mode_qkv, s)) != OGM_OK) return rc;
+    if ((rc = llama_matmul(ctx, w3, y3, 3, s)) != OGM_OK) return rc;
     const int mode_o = act_mode_for(L.wo->ggml_type);
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
                                        c.n_head, c.n_head_kv, c.head_dim, scale, m->part_o, m->part_ml,
-                                       m->attn_counters, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s, 0u,
-                                       ctx->tune_attn_decode_share == 2 ? 0u : 1u));   // 0: wherever the shape allows
+                                       m->attn_counters, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s, 0u));
     const int mode_ff = act_mode_for(L.w_gate->ggml_type);
     if (act_mode_for(L.w_up->ggml_type) != mode_ff)
       return fail(ctx, OGM_ERR_UNSUPPORTED, "w_gate and w_up must share an activation mode");
     const ogm_weight *w1[1] = {L.wo};
     float *y1[1] = {m->proj};
     if ((rc = llama_capture(ctx, m, 4 * l + 1, qd, mode_o, s)) != OGM_OK) return rc;
-    OgmGemvTail tail;
-    tail.ticket = m->attn_tickets + 2u * c.n_head_kv;
-    bool ffn_head = false;
-    if (tail_ok(L.wo, c.n_embd, mode_ff)) {
-      tail.kind = OGM_TAIL_NORM;
-      tail.n = c.n_embd;
-      tail.x = m->x;
-      tail.weight = ffn_norm;
-      tail.eps = c.rms_eps;
-      tail.act = act_view(ctx, c.n_embd, mode_ff, 0);
-      if ((rc = llama_matmul(ctx, w1, y1, 1, s, &tail)) != OGM_OK) return rc;
-    } else {
-      if ((rc = llama_matmul(ctx, w1, y1, 1, s)) != OGM_OK) return rc;
-      ffn_head = head_ok(L.w_gate, mode_ff, true);
-      if (!ffn_head)
-        HIPCHK(ctx, ogm_launch_norm_quant(mode_ff, m->x, m->proj, ffn_norm, c.n_embd, c.rms_eps, nullptr,
-                                          act_view(ctx, c.n_embd, mode_ff, 0), s));
-    }
+    if ((rc = llama_matmul(ctx, w1, y1, 1, s)) != OGM_OK) return rc;
+    HIPCHK(ctx, ogm_launch_norm_quant(mode_ff, m->x, m->proj, ffn_norm, c.n_embd, c.rms_eps, nullptr,
+                                      act_view(ctx, c.n_embd, mode_ff, 0), s));
     const ogm_weight *w2[2] = {L.w_gate, L.w_up};
     float *y2[2] = {m->gate, m->up};
     const int mode_d = act_mode_for(L.w_down->ggml_type);
-    const bool down_head = head_ok(L.w_down, mode_d, false);
-    if (ffn_head) {
-      OgmGemvHead head = norm_head(m->proj, ffn_norm);
-      if ((rc = llama_matmul(ctx, w2, y2, 2, s, nullptr, &head)) != OGM_OK) return rc;
-      if ((rc = llama_capture(ctx, m, 4 * l + 2, c.n_embd, mode_ff, s)) != OGM_OK) return rc;
-      if (!down_head)
-        HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr,
-                                            act_view(ctx, c.n_ff, mode_d, 0), s));
-    } else {
     if ((rc = llama_capture(ctx, m, 4 * l + 2, c.n_embd, mode_ff, s)) != OGM_OK) return rc;
-    if (fuse && mode_d == OGM_ACT_PER_256 && L.w_gate->ggml_type == L.w_up->ggml_type &&
-        block_elems_of(L.w_gate->ggml_type) == 256) {
-      tail.kind = OGM_TAIL_SWIGLU;
-      tail.n = c.n_ff;
-      tail.x = nullptr;
-      tail.weight = nullptr;
-      tail.act = act_view(ctx, c.n_ff, mode_d, 0);
-      if ((rc = llama_matmul(ctx, w2, y2, 2, s, &tail)) != OGM_OK) return rc;
-    } else {
-      if ((rc = llama_matmul(ctx, w2, y2, 2, s)) != OGM_OK) return rc;
-      if (!down_head)
-        HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr,
-                                            act_view(ctx, c.n_ff, mode_d, 0), s));
-    }
-    }
+    if ((rc = llama_matmul(ctx, w2, y2, 2, s)) != OGM_OK) return rc;
+    HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, m->gate, m->up, c.n_ff, nullptr, act_view(ctx, c.n_ff, mode_d, 0), s));
     const ogm_weight *wd[1] = {L.w_down};
-    // the next norm: the next layer's attention norm, or the output norm after the last layer
-    const bool last_layer = l + 1 == c.n_layer;
-    const int mode_next = last_layer ? mode_out : act_mode_for(m->layers[l + 1].wq->ggml_type);
-    if (down_head) {
-      // the SwiGLU rides at the head of the down projection
-      OgmGemvHead head;
-      head.kind = OGM_HEAD_SWIGLU;
-      head.flag = head_flag;
-      head.epoch = ++m->head_epoch;
-      head.gate = m->gate;
-      head.up = m->up;
-      head.delay = (uint32_t)ctx->tune_decode_head_delay;
-      head.spin_limit = (uint32_t)ctx->tune_decode_head_spin;
-      if ((rc = llama_matmul(ctx, wd, y1, 1, s, nullptr, &head)) != OGM_OK) return rc;
-      if ((rc = llama_capture(ctx, m, 4 * l + 3, c.n_ff, mode_d, s)) != OGM_OK) return rc;
-      normed = false;
-    } else {
     if ((rc = llama_capture(ctx, m, 4 * l + 3, c.n_ff, mode_d, s)) != OGM_OK) return rc;
-    normed = tail_ok(L.w_down, c.n_embd, mode_next);
-    if (normed) {
-      tail.kind = OGM_TAIL_NORM;
-      tail.n = c.n_embd;
-      tail.x = m->x;
-      tail.weight = last_layer ? out_norm : attn_norm + 2 * (size_t)c.n_embd;
-      tail.eps = c.rms_eps;
-      tail.act = act_view(ctx, c.n_embd, mode_next, 0);
-      if ((rc = llama_matmul(ctx, wd, y1, 1, s, &tail)) != OGM_OK) return rc;
-    } else {
-      if ((rc = llama_matmul(ctx, wd, y1, 1, s)) != OGM_OK) return rc;
-    }
-    }
+    if ((rc = llama_matmul(ctx, wd, y1, 1, s)) != OGM_OK) return rc;
     delta = m->proj;
   }
-  if (!normed)
-    HIPCHK(ctx, ogm_launch_norm_quant(mode_out, m->x, delta, out_norm, c.n_embd, c.rms_eps, nullptr,
-                                      act_view(ctx, c.n_embd, mode_out, 0), s));
+  HIPCHK(ctx, ogm_launch_norm_quant(mode_out, m->x, delta, out_norm, c.n_embd, c.rms_eps, nullptr,
+                                    act_view(ctx, c.n_embd, mode_out, 0), s));
   float *lg = logits_dev ? logits_dev : m->logits;
   const ogm_weight *wo_[1] = {m->output};
   float *yo[1] = {lg};
-  int rc = llama_capture(ctx, m, 4 * c.n_layer, c.n_embd, mode_out, s);
-  if (rc != OGM_OK) return rc;
+  if ((rc = llama_capture(ctx, m, 4 * c.n_layer, c.n_embd, mode_out, s)) != OGM_OK) return rc;
   if ((rc = llama_matmul(ctx, wo_, yo, 1, s)) != OGM_OK) return rc;
   if (argmax_dev) HIPCHK(ctx, ogm_launch_argmax(lg, c.n_vocab, m->amax_scratch, argmax_dev, s));
   // the activation scratch no longer holds what ogm_act_quantize_dev left there
@@ -1709,18 +1513,6 @@ extern "C" int ogm_llama_decode_dev(ogm_ctx *ctx, ogm_llama *m, const float *x_d
   return llama_decode_enqueue(ctx, m, x_dev, pos, logits_dev, argmax_dev, stream ? (hipStream_t)stream : ctx->stream);
 }
 
-// After a synchronisation: whether a workgroup of a launch with a head gave up waiting for its producers
-// (the step's results are then not to be trusted).  Clears the word.
-static int llama_check_heads(ogm_ctx *ctx, ogm_llama *m) {
-  if (m->head_epoch == 0) return OGM_OK;   // no such launch yet
-  uint32_t *word = m->attn_tickets + ((2u * m->cfg.n_head_kv + OGM_TAIL_TICKETS + 31u) & ~31u) + OGM_HEAD_FLAG_COPIES * 32u + 1u;
-  uint32_t gave_up = 0;
-  HIPCHK(ctx, hipMemcpy(&gave_up, word, 4, hipMemcpyDeviceToHost));
-  if (!gave_up) return OGM_OK;
-  HIPCHK(ctx, hipMemset(word, 0, 4));
-  return fail(ctx, OGM_ERR_HIP, "a workgroup gave up waiting for the producers at the head of its launch");
-}
-
 extern "C" int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos, float *logits,
                                 uint32_t *argmax) {
   if (!ctx) return OGM_ERR_INVALID;
@@ -1735,7 +1527,7 @@ extern "C" int ogm_llama_decode(ogm_ctx *ctx, ogm_llama *m, const float *x, uint
   if (logits) HIPCHK(ctx, hipMemcpyAsync(logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   if (argmax) HIPCHK(ctx, hipMemcpyAsync(argmax, m->amax_out, 4, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-  return llama_check_heads(ctx, m);
+  return OGM_OK;
 }
 
 extern "C" int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out) {
@@ -1857,7 +1649,7 @@ extern "C" int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
   if (last_logits)
     HIPCHK(ctx, hipMemcpyAsync(last_logits, m->logits, (size_t)c.n_vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-  return llama_check_heads(ctx, m);
+  return OGM_OK;
 }
 
 // ---- prefill: run_layers at n_tokens > 1 (llama.rs:594-932) ------------------------------------
@@ -1936,7 +1728,7 @@ static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws
       tg[e - i] = Target{ws[e], ys[e]};
       e++;
     }
-    int rc = enqueue_gemv(ctx, tg, e - i, T, 0, s, nullptr, nullptr, nullptr);
+    int rc = enqueue_gemv(ctx, tg, e - i, T, 0, s, nullptr, nullptr);
     if (rc != OGM_OK) return rc;
     i = e;
   }

@@ -24,60 +24,6 @@ hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32
 
 #define OGM_GEMV_MAX_MATS 4
 
-// What the last workgroup of a single-token GEMV launch to finish does with the launch's outputs,
-// in place of a kernel of its own (per-256 activations only):
-//   OGM_TAIL_NORM   x += y; act = quantize(rmsnorm(x) * weight)       one matrix, out_dim = n
-//   OGM_TAIL_SWIGLU act = quantize(silu(y0) * y1)                     two matrices, out_dims = n
-// `ticket` is OGM_TAIL_TICKETS zeroed uint32 on the device that the launch leaves zero again.  `act` may be
-// the buffer the launch read its own activations from: every workgroup has finished by then.
-#define OGM_TAIL_TICKETS 65u
-#define OGM_TAIL_NONE 0u
-#define OGM_TAIL_NORM 1u
-#define OGM_TAIL_SWIGLU 2u
-struct OgmGemvTail {
-  uint32_t kind = OGM_TAIL_NONE;
-  uint32_t n = 0;
-  uint32_t *ticket = nullptr;
-  float *x = nullptr;             // NORM: the residual stream, updated in place
-  const float *weight = nullptr;  // NORM: the norm's weights
-  float eps = 0.0f;
-  OgmActDev act = {};
-};
-
-// What extra workgroups at the front of a single-token GEMV launch (per-256 activations) compute before
-// its other workgroups read their activations, in place of a kernel of its own ahead of the launch:
-//   OGM_HEAD_NORM   x += delta; act = quantize(rmsnorm(x) * weight)    one producer workgroup, n = in_dim
-//   OGM_HEAD_SWIGLU act = quantize(silu(gate) * up)                    ceil(in_dim / 256 / waves) of them
-// The launch's `act` is what the producers write and the others read.  The producers are the launch's
-// first workgroups, which the hardware starts first; they store device-coherently, and the last of
-// them to finish raises flag[0] to `epoch`.  Every other workgroup requests its first tile of
-// weights, then polls the flag (at most spin_limit times; it then sets the gave-up word and goes on
-// with whatever the activations hold, so every wave ends) and reads the activations.
-// flag: OGM_HEAD_FLAG_WORDS uint32 on the device, zero before the first launch: OGM_HEAD_FLAG_COPIES
-// copies of the flag, 128 bytes apart (a waiting workgroup polls copy `its index % copies`: polls of
-// one address are served one after the other), which only ever grow; then the producers' own counter,
-// zero between launches, and the word a workgroup that gave up sets.  epoch: the flag's value before
-// the launch plus one (launches over one flag must be stream-ordered).
-#define OGM_HEAD_FLAG_COPIES 64u
-#define OGM_HEAD_FLAG_WORDS (OGM_HEAD_FLAG_COPIES * 32u + 2u)
-#define OGM_HEAD_NONE 0u
-#define OGM_HEAD_NORM 1u
-#define OGM_HEAD_SWIGLU 2u
-struct OgmGemvHead {
-  uint32_t kind = OGM_HEAD_NONE;
-  uint32_t *flag = nullptr;
-  uint32_t epoch = 0;
-  uint32_t spin_limit = 0;        // 0: the default (about a tenth of a second)
-  float *x = nullptr;             // NORM: the residual stream, updated in place
-  const float *delta = nullptr;   // NORM: what is added to x first (may be null)
-  const float *weight = nullptr;  // NORM: the norm's weights
-  float eps = 0.0f;
-  const float *gate = nullptr;    // SWIGLU
-  const float *up = nullptr;
-  uint32_t delay = 0;             // what the other workgroups sleep before their first weight loads, in units of 64 clocks
-  uint32_t n_prod = 0;            // filled in by the launcher
-};
-
 struct OgmGemvArgs {
   uint32_t ggml_type;
   const uint8_t *wt;  // tile-planar weights
@@ -87,7 +33,6 @@ struct OgmGemvArgs {
   float *y;           // [n_tokens][out_dim], row stride out_dim
   int gemm_order;     // 0: GEMV float order (cpu.rs T==1 / matmul_decode), 1: GEMM order (T>1)
   uint32_t wg_waves;     // waves per workgroup, 0 = by shape
-  uint32_t rb_per_wg;    // row blocks per workgroup, 0 = by shape
   int32_t *dump_isum;    // optional [n_tokens][out_dim][blocks/row]
   int32_t *dump_imin;    // optional, Q4_K only
   // Further matrices of the same type and in_dim that read the same activations (q/k/v,
@@ -96,24 +41,13 @@ struct OgmGemvArgs {
   const uint8_t *extra_wt[OGM_GEMV_MAX_MATS - 1];
   uint32_t extra_out_dim[OGM_GEMV_MAX_MATS - 1];
   float *extra_y[OGM_GEMV_MAX_MATS - 1];
-  // When set (one token, GEMV order, no dumps): f32 activations [in_dim]; every workgroup
-  // quantizes them itself on its way in and `act` is not read.
-  const float *x_f32;
-  OgmGemvTail tail;   // one token, GEMV order, no dumps, no x_f32
-  OgmGemvHead head;   // one token, GEMV order, no dumps, no x_f32, no tail; per-256 activations
 };
 
 // Largest token count one launch can take for this shape (LDS budget), at least 1.
 uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order);
 hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name);
-// Longest row an OGM_TAIL_NORM tail of a single-token launch over this matrix can take (0: none).
-uint32_t ogm_gemv_norm_tail_max(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves);
-// Waves per workgroup of a single-token launch with a head over this matrix (0: the type takes none).
-// An OGM_HEAD_NORM head needs in_dim <= 1024 * that.
-uint32_t ogm_gemv_head_waves(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves);
-
 // Prefill GEMM on MFMA (ogm_gemm.hip).  Same operands as the GEMV plus a scratch buffer `xh` of
-// ogm_gemm_xh_bytes() for the activations as f16.  Follows the CPU path's GEMM float order.
+// ogm_gemm_xh_bytes() for the int8 activations in operand chunks.  Follows the CPU path's GEMM float order.
 #define OGM_GEMM_MAX_MATS 3   // matrices one GEMM launch can take (q, k, v)
 struct OgmGemmArgs {
   uint32_t ggml_type;
@@ -123,8 +57,7 @@ struct OgmGemmArgs {
   uint32_t n_tokens;
   float *y;            // [n_tokens][out_dim]
   void *xh;            // scratch
-  uint32_t wide_min_wgs = 0;   // Q4_K: least 128x128 workgroups from which the wide tiling runs (0 = default)
-  uint32_t q4k_variant = 0;    // K-quants: 0 / 1 the int8 plane kernels, 2 the f16 kernels, 3 int8 multiply-adds
+  uint32_t tile_rows = 0;          // feeding-wave kernels: 64 forces their 64-row tiles (0 = by the size of the launch)
   uint32_t small_max_tokens = 0;   // most tokens for the small-batch kernel (0 = default 64, 1 = never)
   uint32_t sb_waves = 0;           // waves of a small-batch workgroup: 8 or 16 (0 = by the size of the launch)
   // K-quants: further matrices of the same type and in_dim over the same activations, in the same launch
@@ -133,13 +66,11 @@ struct OgmGemmArgs {
   uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1] = {};
   float *extra_y[OGM_GEMM_MAX_MATS - 1] = {};
   // K-quants: the matrices' scale-folded int8 planes (ogm_gemm_build_planes), or null.  When every
-  // matrix of the launch has them, the tiled int8 kernels read them instead of unpacking the
-  // weights again on every call.
+  // matrix of the launch has them, the kernel whose waves all multiply reads them (operands by load-to-LDS).
   const uint8_t *planes = nullptr;
   const uint8_t *extra_planes[OGM_GEMM_MAX_MATS - 1] = {};
-  // which kernel reads planes: 0 the one whose waves all multiply (operands by load-to-LDS) when the
-  // grid fills the device twice, else none (the feeding waves unpack); 1 the feeding-wave kernels; 2
-  // the former whatever the grid
+  // when that kernel runs: 0 when the grid fills the device twice (else the feeding waves unpack), 2 whatever
+  // the grid
   uint32_t plane_kernel = 0;
   uint32_t one_pass = 0;   // Q4_K / Q5_K on the all-waves-multiply kernel: fold the min pass into the super-block step (f32 to rounding, not to the bit)
 };

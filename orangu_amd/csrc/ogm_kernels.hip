@@ -826,34 +826,13 @@ struct GemvParams {
   float *y[OGM_GEMV_MAX_MATS];
   uint32_t out_dim[OGM_GEMV_MAX_MATS];
   uint32_t wg_end[OGM_GEMV_MAX_MATS];  // workgroups of matrices 0..m, running total
-  uint32_t rb_per_wg;                  // consecutive row blocks one workgroup owns
   OgmActDev act;
-  const float *x;                  // f32 activations of the kernels that quantize on the way in
   int32_t *dump_isum, *dump_imin;
   uint32_t in_dim, upr;            // upr = blocks per row
   uint32_t n_tokens;
   uint32_t C, nct;                // tile shape: C blocks x R rows, nct = upr / C column tiles
   uint32_t lane_acc;              // formats of several terms a block, tiles one block wide, one wave: see gemv_lane_acc
-  OgmGemvTail tail;
-  OgmGemvHead head;
 };
-
-// Sixteen bytes / four bytes that another workgroup of the same kernel stored device-coherently.
-__device__ __forceinline__ uint4 ldc16(const void *p) {
-  const uint64_t a = __hip_atomic_load((const uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const uint64_t b = __hip_atomic_load((const uint64_t *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
-}
-__device__ __forceinline__ float ldc4f(const float *p) {
-  return __uint_as_float(__hip_atomic_load((const uint32_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-}
-#define OGM_HEAD_SPIN_DEFAULT 200000u
-// The activations behind a head's flag: 1 reads them device-coherently (past L2), 0 with plain loads.
-// No workgroup of the launch touches them before it has seen the flag and every L2 starts a kernel
-// invalidated, so plain loads cannot meet a stale line.
-#ifndef OGM_HEAD_COHERENT_READS
-#define OGM_HEAD_COHERENT_READS 0
-#endif
 
 template <class F, bool GEMM_ORDER>
 __host__ __device__ constexpr int n_term_arrays() {
@@ -865,7 +844,7 @@ static const size_t OGM_LDS_MAX = 160 * 1024;     // what a workgroup can have w
 
 // Dynamic LDS bytes of one workgroup.
 template <class F, bool GEMM_ORDER>
-static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rb_per_wg = 1) {
+static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens) {
   const size_t upr = in_dim / F::ELEMS;
   const size_t n_scale = in_dim / F::ACT_GROUP;
   const OgmTiling tl = ogm_tiling_for((uint32_t)upr, 1);
@@ -873,7 +852,7 @@ static size_t gemv_lds_bytes(uint32_t in_dim, uint32_t n_tokens, uint32_t rb_per
   b += (size_t)n_tokens * upr * F::AUX16 * 16;              // aux
   b += (size_t)n_tokens * n_scale * 4;                      // act.d
   b = (b + 15) & ~(size_t)15;
-  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * rb_per_wg * upr * tl.R * 4 * F::TERMS;  // terms
+  b += (size_t)n_term_arrays<F, GEMM_ORDER>() * n_tokens * upr * tl.R * 4 * F::TERMS;  // terms
   return b;
 }
 
@@ -897,28 +876,6 @@ static size_t gemv_lds_bytes_lane_acc(uint32_t in_dim, uint32_t n_tokens) {
 }
 
 #define OGM_STAGE_PEEL 4
-
-// The activation quantizer inside the GEMV: quantizes the 256 activations of group g held four
-// per lane (lane l: elements 256g + 4l ..) exactly as ogm_quantize_kernel does and leaves q, the
-// scale and the side sums in LDS where the formats read them.  Every lane of the wave calls it.
-template <class F>
-__device__ __forceinline__ void quantize_park(const float4 &v, uint32_t g, bool active, uint32_t lane,
-                                              uint32_t upr, uint4 *l_xq, uint4 *l_aux, float *l_d) {
-  float scale;
-  int s, s32;
-  const uint32_t packed = ogm_quantize4<F::ACT_GROUP>(v, scale, s, s32);
-  if (!active) return;
-  const uint32_t ch = g * 16u + (lane >> 2);    // 16-byte chunk of the token
-  const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
-  ((uint32_t *)(l_xq + c * upr + col))[lane & 3u] = packed;
-  if (F::AUX16 == 1) {          // Q4_K: bsum, eight i16 per block
-    if ((lane & 7u) == 0) ((int16_t *)(l_aux + col))[lane >> 3] = (int16_t)s32;
-  } else if (F::AUX16 == 2) {   // Q6_K: per-16 sums as i16, groups 0..7 | 8..15 of a block
-    const uint32_t gi = lane >> 2;
-    if ((lane & 3u) == 0) ((int16_t *)(l_aux + (gi >> 3) * upr + col))[gi & 7u] = (int16_t)s;
-  }
-  if ((lane & (F::ACT_GROUP / 4 - 1)) == 0) l_d[(g * 256u + lane * 4u) / F::ACT_GROUP] = scale;
-}
 
 // acc (+|-)= p[0], p[stride], ... in ascending order, one accumulator.  Eight LDS reads are in
 // flight and the next eight are requested before these are added: the adds are a serial chain
@@ -962,15 +919,9 @@ template <class F>
 struct UnpackedOf<F, true, true> { typedef typename F::Unpacked type; };
 
 // UPR: blocks per row when known at compile time (the hot shapes), 0 = read it from the params.
-// QUANT: the workgroup quantizes the f32 activations p.x itself (one token) instead of reading
-// the quantizer kernel's output.
 // UNPACK: several tokens and a format whose block is expensive to unpack: unpack once per tile.
-// TAIL: the outputs are stored device-coherently and the last workgroup to finish runs p.tail.
-// HEAD: the first p.head.n_prod workgroups compute the activations (p.head), the others wait for them
-// behind their first weight loads and read the activations device-coherently.
-template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP, bool QUANT, bool UNPACK = false,
-          bool TAIL = false, bool HEAD = false>
-__global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::MAX_THREADS_SINGLE : F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) {
+template <class F, int UPR, bool SINGLE, bool GEMM_ORDER, bool DUMP, bool UNPACK = false>
+__global__ __launch_bounds__((SINGLE && !DUMP) ? F::MAX_THREADS_SINGLE : F::MAX_THREADS) void ogm_gemv_kernel(GemvParams p) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t tid = threadIdx.x, nthr = blockDim.x;
   const uint32_t lane = tid & 63u, wave = tid >> 6, n_wave = nthr >> 6;
@@ -987,52 +938,20 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
   uint4 *l_aux = l_xq + (size_t)T * xch;                        // [T][AUX16][upr]
   float *l_d = (float *)(l_aux + (size_t)T * upr * F::AUX16);   // [T][n_scale]
   const size_t head = ((size_t)T * (xch * 16 + upr * F::AUX16 * 16 + n_scale * 4) + 15) & ~(size_t)15;
-  float *l_term = (float *)(lds + head);                        // [NT][T][K][upr][R]
+  float *l_term = (float *)(lds + head);                        // [NT][T][upr][R]
 
-  uint32_t bid = blockIdx.x;
-  if constexpr (HEAD) {
-    if (bid < p.head.n_prod) {
-      // ---- a producer: the activations of the launch, stored for the other workgroups
-      if (p.head.kind == OGM_HEAD_NORM) {
-        ogm_norm_quant_row<256, false, true>(p.head.x, p.head.delta, p.head.weight, p.in_dim, p.head.eps, nullptr,
-                                             p.act, (float *)lds, tid, n_wave);
-      } else {
-        const uint32_t run = bid * n_wave + wave;
-        if (run * 256u < p.in_dim)
-          ogm_swiglu_quant_run<256, false, true>(p.head.gate, p.head.up, p.in_dim, nullptr, p.act, run, lane);
-      }
-      // every wave's stores acknowledged, the workgroup met: the last producer raises the flag
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
-      uint32_t *l_last = (uint32_t *)lds;
-      if (tid == 0) {
-        uint32_t *count = p.head.flag + OGM_HEAD_FLAG_COPIES * 32u;
-        const bool last = __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.head.n_prod - 1u;
-        if (last) __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        l_last[0] = last ? 1u : 0u;
-      }
-      __syncthreads();
-      // every copy of the flag sits in a cache line of its own: the waiting workgroups spread over them
-      if (l_last[0] != 0u && tid < OGM_HEAD_FLAG_COPIES)
-        __hip_atomic_store(p.head.flag + tid * 32u, p.head.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      return;
-    }
-    bid -= p.head.n_prod;
-  }
   // ---- which matrix of the launch this workgroup belongs to, and which of its row blocks
+  const uint32_t bid = blockIdx.x;
   uint32_t m = 0;
   if (bid >= p.wg_end[0]) m = 1;
   if (bid >= p.wg_end[1]) m = 2;
   if (bid >= p.wg_end[2]) m = 3;
-  const uint32_t wg = bid - (m == 0 ? 0u : m == 1 ? p.wg_end[0] : m == 2 ? p.wg_end[1] : p.wg_end[2]);
-  const uint32_t K = p.rb_per_wg;
-  const uint32_t rb0 = wg * K;
+  const uint32_t rb0 = bid - (m == 0 ? 0u : m == 1 ? p.wg_end[0] : m == 2 ? p.wg_end[1] : p.wg_end[2]);
   const uint8_t *wt = m == 0 ? p.wt[0] : m == 1 ? p.wt[1] : m == 2 ? p.wt[2] : p.wt[3];
   float *y = m == 0 ? p.y[0] : m == 1 ? p.y[1] : m == 2 ? p.y[2] : p.y[3];
   const uint32_t out_dim = m == 0 ? p.out_dim[0] : m == 1 ? p.out_dim[1] : m == 2 ? p.out_dim[2] : p.out_dim[3];
-  // The workgroup's tiles are consecutive in memory: item i is tile rb0 * nct + i, i.e. column
-  // tile i % nct of row block rb0 + i / nct.
-  const uint32_t n_items = min(K, (out_dim + R - 1) / R - rb0) * nct;
+  // The row block's tiles are consecutive in memory: item i is tile rb0 * nct + i, column tile i.
+  const uint32_t n_items = nct;
   const size_t tile0 = (size_t)rb0 * nct;
 
   // ---- issue the activation loads (few, L2-resident) ...
@@ -1040,101 +959,43 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
   const uint4 *gq = (const uint4 *)p.act.q;
   uint4 st0, st1, st2, st3, st_aux = make_uint4(0, 0, 0, 0);
   float st_d = 0.0f;
-  // f32 activations of the quantizing kernels: group k of this wave is 256 * (wave + k * n_wave)
-  float4 xs0, xs1, xs2, xs3, xs4, xs5, xs6, xs7;
-  auto xload = [&](uint32_t k) -> float4 {
-    const uint32_t e0 = (wave + k * n_wave) * 256u + lane * 4u;
-    return *(const float4 *)(p.x + min(e0, p.in_dim - 4u));
-  };
-  constexpr int QPEEL = (UPR == 16) ? 4 : 8;  // 4096-wide rows: four groups for each of four waves
-  // (with producers in the launch the activations are read device-coherently, and only later)
-  auto ld_q = [&](uint32_t i) -> uint4 {
-    if constexpr (HEAD && OGM_HEAD_COHERENT_READS) return ldc16(gq + i);
-    else return gq[i];
-  };
   auto ld_bsum = [&](uint32_t i) -> uint4 {   // Q4_K: bsum, 8 x i16 per block
-    if constexpr (HEAD && OGM_HEAD_COHERENT_READS) return ldc16((const uint4 *)p.act.bsum + i);
-    else return ((const uint4 *)p.act.bsum)[i];
+    return ((const uint4 *)p.act.bsum)[i];
   };
   auto ld_sums16 = [&](uint32_t i) -> uint4 {   // Q6_K: per-16 sums narrowed to i16, groups 0..7 / 8..15 of a block
     const int4 *src = (const int4 *)(p.act.sums + (size_t)(i >> 1) * 16 + (i & 1u) * 8);
-    uint4 a, b;
-    if constexpr (HEAD && OGM_HEAD_COHERENT_READS) { a = ldc16(src); b = ldc16(src + 1); }
-    else { const int4 a_ = src[0], b_ = src[1]; a = make_uint4(a_.x, a_.y, a_.z, a_.w); b = make_uint4(b_.x, b_.y, b_.z, b_.w); }
+    const int4 a = src[0], b = src[1];
     uint4 o;
-    o.x = (a.x & 0xFFFFu) | (a.y << 16);
-    o.y = (a.z & 0xFFFFu) | (a.w << 16);
-    o.z = (b.x & 0xFFFFu) | (b.y << 16);
-    o.w = (b.z & 0xFFFFu) | (b.w << 16);
+    o.x = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)a.y << 16);
+    o.y = ((uint32_t)a.z & 0xFFFFu) | ((uint32_t)a.w << 16);
+    o.z = ((uint32_t)b.x & 0xFFFFu) | ((uint32_t)b.y << 16);
+    o.w = ((uint32_t)b.z & 0xFFFFu) | ((uint32_t)b.w << 16);
     return o;
   };
-  auto ld_d = [&](uint32_t i) -> float {
-    if constexpr (HEAD && OGM_HEAD_COHERENT_READS) return ldc4f(p.act.d + i);
-    else return p.act.d[i];
-  };
-  auto stage_loads = [&]() {
-    st0 = ld_q(min(tid, n_xq - 1));
-    st1 = ld_q(min(tid + nthr, n_xq - 1));
-    st2 = ld_q(min(tid + 2 * nthr, n_xq - 1));
-    st3 = ld_q(min(tid + 3 * nthr, n_xq - 1));
-    if (F::AUX16 == 1) st_aux = ld_bsum(min(tid, n_aux - 1));
-    else if (F::AUX16 == 2) st_aux = ld_sums16(min(tid, n_aux - 1));
-    st_d = ld_d(min(tid, n_d - 1));
-  };
-  if constexpr (QUANT) {
-    xs0 = xload(0); xs1 = xload(1); xs2 = xload(2); xs3 = xload(3);
-    if constexpr (QPEEL == 8) { xs4 = xload(4); xs5 = xload(5); xs6 = xload(6); xs7 = xload(7); }
-  } else if constexpr (!HEAD) {
-    stage_loads();
-  }
+  st0 = gq[min(tid, n_xq - 1)];
+  st1 = gq[min(tid + nthr, n_xq - 1)];
+  st2 = gq[min(tid + 2 * nthr, n_xq - 1)];
+  st3 = gq[min(tid + 3 * nthr, n_xq - 1)];
+  if (F::AUX16 == 1) st_aux = ld_bsum(min(tid, n_aux - 1));
+  else if (F::AUX16 == 2) st_aux = ld_sums16(min(tid, n_aux - 1));
+  st_d = p.act.d[min(tid, n_d - 1)];
 
   // Keeps every staging load of the workgroup ahead of every weight load in the CU's
   // memory pipeline (no data is waited for here).
   __syncthreads();
 
-  if constexpr (HEAD) {
-    // the producers' few loads go out ahead of the launch's weight stream, not behind it
-    for (uint32_t i = 0; i < p.head.delay; i++) __builtin_amdgcn_s_sleep(1);
-  }
   // ---- ... then this wave's first tile of weights (the long pole) ...
   const uint32_t r_local = lane & (R - 1), c_local = lane / R;
-  uint32_t it = wave;  // every wave has at least one item: n_wave <= nct <= n_items
+  uint32_t it = wave;  // every wave has at least one item: n_wave <= nct
   typename F::Regs cur;
   F::load(cur, wt, tile0 + it, lane);
   // Nothing below may be scheduled above the weight loads: work on the activations would
   // otherwise wait for them first and hold the weight loads back by a memory round trip.
   __builtin_amdgcn_sched_barrier(0);
 
-  if constexpr (HEAD) {
-    // ---- the producers' flag, polled by one lane behind the weight loads; then the activations
-    if (tid == 0) {
-      const uint32_t limit = p.head.spin_limit ? p.head.spin_limit : OGM_HEAD_SPIN_DEFAULT;
-      const uint32_t *mine = p.head.flag + (bid % OGM_HEAD_FLAG_COPIES) * 32u;
-      uint32_t polls = 0;
-      while ((int32_t)(__hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - p.head.epoch) < 0) {
-        if (++polls >= limit) {   // gives up, says so, and lets every wave end
-          __hip_atomic_store(p.head.flag + OGM_HEAD_FLAG_COPIES * 32u + 1u, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          break;
-        }
-        __builtin_amdgcn_s_sleep(2);
-      }
-    }
-    __syncthreads();
-    stage_loads();
-  }
-
   // ---- ... and park the activations in LDS while the weights are in flight.
   // q is permuted so that chunk c of block `col` lands at [c*upr + col].
-  if constexpr (QUANT) {
-    const uint32_t n_g = (p.in_dim + 255u) / 256u;
-    auto qpark = [&](uint32_t k, const float4 &v) {
-      const uint32_t g = wave + k * n_wave;
-      quantize_park<F>(v, g, g * 256u + lane * 4u < p.in_dim, lane, upr, l_xq, l_aux, l_d);
-    };
-    qpark(0, xs0); qpark(1, xs1); qpark(2, xs2); qpark(3, xs3);
-    if constexpr (QPEEL == 8) { qpark(4, xs4); qpark(5, xs5); qpark(6, xs6); qpark(7, xs7); }
-    for (uint32_t k = QPEEL; wave + k * n_wave < n_g; k++) qpark(k, xload(k));  // longer rows
-  } else {
+  {
     auto park = [&](uint32_t i, const uint4 &v) {
       if (i < n_xq) {
         const uint32_t t = i / xch, ch = i - t * xch;
@@ -1160,7 +1021,7 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
     for (uint32_t i = tid + OGM_STAGE_PEEL * nthr; i < n_xq; i += nthr) {
       const uint32_t t = i / xch, ch = i - t * xch;
       const uint32_t col = ch / F::XPIECES, c = ch - col * F::XPIECES;
-      l_xq[(size_t)t * xch + c * upr + col] = ld_q(i);
+      l_xq[(size_t)t * xch + c * upr + col] = gq[i];
     }
     if (F::AUX16 == 1) {
       for (uint32_t i = tid + nthr; i < n_aux; i += nthr) l_aux[i] = ld_bsum(i);
@@ -1171,7 +1032,7 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
         l_aux[(size_t)t * upr * 2 + k * upr + col] = ld_sums16(i);
       }
     }
-    for (uint32_t i = tid + nthr; i < n_d; i += nthr) l_d[i] = ld_d(i);
+    for (uint32_t i = tid + nthr; i < n_d; i += nthr) l_d[i] = p.act.d[i];
   }
   __syncthreads();
 
@@ -1181,8 +1042,7 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
   }
   // ---- tiles of this wave
   for (; it < n_items; it += n_wave) {
-    const uint32_t rbk = it / nct, ct = it - rbk * nct;
-    const uint32_t col = ct * C + c_local;  // block index within the row
+    const uint32_t col = it * C + c_local;  // block index within the row
     // many tokens: unpack the block once where that is the expensive part (Q6_K; measured at
     // 4096 -> 128256: 159 us against 182 us at 8 tokens, but 112 us against 97 us at 4)
     [[maybe_unused]] typename UnpackedOf<F, UNPACK>::type unp;
@@ -1207,23 +1067,23 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
           l_term[t * 64u + lane] = acc;
           continue;
         }
-        float *dst = l_term + (size_t)(t * K + rbk) * term_stride + (size_t)col * F::TERMS * R + r_local;
+        float *dst = l_term + (size_t)t * term_stride + (size_t)col * F::TERMS * R + r_local;
 #pragma unroll
         for (int g = 0; g < F::TERMS; g++) dst[g * R] = tt[g];
         continue;
       }
       const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
-      const size_t slot = (size_t)(t * K + rbk) * term_stride + col * R + r_local;
+      const size_t slot = (size_t)t * term_stride + col * R + r_local;
       if (GEMM_ORDER) {
         float tmin, tdot;
         F::term_gemm(cur, ad, isum, imin, tmin, tdot);
         l_term[slot] = tdot;
-        if (NT == 2) l_term[(size_t)T * K * term_stride + slot] = tmin;
+        if (NT == 2) l_term[(size_t)T * term_stride + slot] = tmin;
       } else {
         l_term[slot] = F::term_gemv(cur, ad, isum, imin);
       }
       if (DUMP) {
-        const uint32_t row = (rb0 + rbk) * R + r_local;
+        const uint32_t row = rb0 * R + r_local;
         if (row < out_dim) {
           const size_t o = ((size_t)t * out_dim + row) * upr + col;
           if (p.dump_isum) p.dump_isum[o] = isum;
@@ -1244,52 +1104,15 @@ __global__ __launch_bounds__((SINGLE && !QUANT && !TAIL && !DUMP && !HEAD) ? F::
     }
   }
   // One lane per (token, row): the row's block terms in ascending order, one accumulator.
-  const uint32_t KR = K * R;
-  for (uint32_t i = tid; i < KR * T; i += nthr) {
-    const uint32_t t = i / KR, rr = i - t * KR;
-    const uint32_t rbk = rr / R, r = rr - rbk * R;
-    const uint32_t orow = (rb0 + rbk) * R + r;
+  for (uint32_t i = tid; i < R * T; i += nthr) {
+    const uint32_t t = i / R, r = i - t * R;
+    const uint32_t orow = rb0 * R + r;
     if (orow < out_dim) {
-      const float *terms = l_term + (size_t)(t * K + rbk) * term_stride + r;
+      const float *terms = l_term + (size_t)t * term_stride + r;
       float acc = 0.0f;
-      if (NT == 2) acc = ordered_sum<true>(acc, terms + (size_t)T * K * term_stride, upr, R);
+      if (NT == 2) acc = ordered_sum<true>(acc, terms + (size_t)T * term_stride, upr, R);
       acc = ordered_sum<false>(acc, terms, upr * F::TERMS, R);
-      if constexpr (TAIL) __hip_atomic_store(&y[(size_t)t * out_dim + orow], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      else y[(size_t)t * out_dim + orow] = acc;
-    }
-  }
-  if constexpr (TAIL) {
-    // The outputs went out device-coherently; once every wave's stores are acknowledged (vmcnt 0)
-    // and the workgroup has met, one ticket tells whether all workgroups of the launch are done.
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    uint32_t *l_last = (uint32_t *)lds;
-    if (tid == 0) {
-      // Tickets in two levels (atomics on one address are served one after the other, and a launch
-      // has up to a few thousand workgroups): workgroup i draws from counter 1 + i % 64, the last
-      // of each of those from counter 0.  Whoever draws a last ticket leaves its counter at zero.
-      const uint32_t n_grp = gridDim.x < OGM_TAIL_TICKETS - 1u ? gridDim.x : OGM_TAIL_TICKETS - 1u;
-      const uint32_t grp = blockIdx.x % (OGM_TAIL_TICKETS - 1u);
-      const uint32_t in_grp = (gridDim.x - grp + OGM_TAIL_TICKETS - 2u) / (OGM_TAIL_TICKETS - 1u);
-      bool last = false;
-      uint32_t *c1 = p.tail.ticket + 1u + grp;
-      if (__hip_atomic_fetch_add(c1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_grp - 1u) {
-        __hip_atomic_store(c1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (__hip_atomic_fetch_add(p.tail.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_grp - 1u) {
-          __hip_atomic_store(p.tail.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          last = true;
-        }
-      }
-      l_last[0] = last ? 1u : 0u;
-    }
-    __syncthreads();
-    if (l_last[0] == 0u) return;
-    if (p.tail.kind == OGM_TAIL_NORM) {
-      ogm_norm_quant_row<256, true>(p.tail.x, p.y[0], p.tail.weight, p.tail.n, p.tail.eps, nullptr, p.tail.act,
-                                    (float *)lds + 16, tid, n_wave);
-    } else {
-      for (uint32_t run = wave; run * 256u < p.tail.n; run += n_wave)
-        ogm_swiglu_quant_run<256, true>(p.y[0], p.y[1], p.tail.n, nullptr, p.tail.act, run, lane);
+      y[(size_t)t * out_dim + orow] = acc;
     }
   }
 }
@@ -1353,74 +1176,22 @@ static uint32_t pick_waves(uint32_t nct, uint32_t wg_waves, int max_threads, uin
   return waves;
 }
 
-uint32_t ogm_gemv_norm_tail_max(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves) {
-  int max_threads;
-  switch (ggml_type) {
-    case OGM_Q4_K: max_threads = FmtQ4K::MAX_THREADS; break;
-    case OGM_Q5_K: max_threads = FmtQ5K::MAX_THREADS; break;
-    case OGM_Q3_K: max_threads = FmtQ3K::MAX_THREADS; break;
-    case OGM_Q6_K: max_threads = FmtQ6K::MAX_THREADS; break;
-    default: return 0;
-  }
-  if (in_dim == 0 || in_dim % 256u != 0) return 0;
-  const OgmTiling tl = ogm_tiling_for(in_dim / 256u, out_dim);
-  return 1024u * pick_waves(tl.nct, wg_waves, max_threads);
-}
-
-uint32_t ogm_gemv_head_waves(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t wg_waves) {
-  int max_threads;
-  switch (ggml_type) {
-    case OGM_Q4_K: max_threads = FmtQ4K::MAX_THREADS; break;
-    case OGM_Q5_K: max_threads = FmtQ5K::MAX_THREADS; break;
-    case OGM_Q3_K: max_threads = FmtQ3K::MAX_THREADS; break;
-    case OGM_Q6_K: max_threads = FmtQ6K::MAX_THREADS; break;
-    case OGM_IQ4_XS: max_threads = FmtIQ4XS::MAX_THREADS; break;
-    case OGM_Q2_K: max_threads = FmtQ2K::MAX_THREADS; break;
-    default: return 0;
-  }
-  if (in_dim == 0 || in_dim % 256u != 0) return 0;
-  const OgmTiling tl = ogm_tiling_for(in_dim / 256u, out_dim);
-  return pick_waves(tl.nct, wg_waves, max_threads);
-}
-
-template <class F, bool QUANT>
+template <class F>
 static void launch_single(const GemvParams &p, dim3 g, dim3 b, size_t lds, hipStream_t stream) {
-  if constexpr (!QUANT && F::ELEMS == 256 && F::ACT_GROUP == 256) {
-    if (p.head.kind != OGM_HEAD_NONE) {
-      if (p.upr == 16)
-        hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false, false, false, false, true>), g, b, lds, stream, p);
-      else if (p.upr == 56)
-        hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false, false, false, false, true>), g, b, lds, stream, p);
-      else
-        hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false, false, false, false, true>), g, b, lds, stream, p);
-      return;
-    }
-  }
-  if constexpr (!QUANT && F::ELEMS == 256) {
-    if (p.tail.kind != OGM_TAIL_NONE) {
-      if (p.upr == 16)
-        hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false, false, false, true>), g, b, lds, stream, p);
-      else if (p.upr == 56)
-        hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false, false, false, true>), g, b, lds, stream, p);
-      else
-        hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false, false, false, true>), g, b, lds, stream, p);
-      return;
-    }
-  }
   // single-token decode: the hot shapes get their row length as a compile-time constant
   if (F::ELEMS == 256 && p.upr == 16)
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false, QUANT>), g, b, lds, stream, p);
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 16, true, false, false>), g, b, lds, stream, p);
   else if (F::ELEMS == 256 && p.upr == 56)
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false, QUANT>), g, b, lds, stream, p);
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 56, true, false, false>), g, b, lds, stream, p);
   else if (F::ELEMS == 32 && p.upr == 128)
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 128, true, false, false, QUANT>), g, b, lds, stream, p);
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 128, true, false, false>), g, b, lds, stream, p);
   else {
     // (a long row of an odd number of blocks -- 64-row tiles one block wide -- stages more than a launch gets unasked)
     if (lds > OGM_LDS_BUDGET &&
-        hipFuncSetAttribute((const void *)ogm_gemv_kernel<F, 0, true, false, false, QUANT>,
+        hipFuncSetAttribute((const void *)ogm_gemv_kernel<F, 0, true, false, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return;   // the launch below then fails and reports it
-    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false, QUANT>), g, b, lds, stream, p);
+    hipLaunchKernelGGL((ogm_gemv_kernel<F, 0, true, false, false>), g, b, lds, stream, p);
   }
 }
 
@@ -1428,28 +1199,8 @@ template <class F, bool GEMM_ORDER>
 static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   const bool dump = a.dump_isum || a.dump_imin;
   if (a.n_extra > OGM_GEMV_MAX_MATS - 1 || (dump && a.n_extra)) return hipErrorInvalidValue;
-  if (a.x_f32 && (a.n_tokens != 1 || GEMM_ORDER || dump)) return hipErrorInvalidValue;
   GemvParams p;
   p.act = a.act;
-  p.x = a.x_f32;
-  p.tail = a.tail;
-  if (a.tail.kind != OGM_TAIL_NONE) {
-    const bool shape_ok = a.tail.kind == OGM_TAIL_NORM ? (a.n_extra == 0 && a.out_dim == a.tail.n && a.tail.x && a.tail.weight)
-                          : a.tail.kind == OGM_TAIL_SWIGLU
-                              ? (a.n_extra == 1 && a.out_dim == a.tail.n && a.extra_out_dim[0] == a.tail.n)
-                              : false;
-    if (!shape_ok || F::ELEMS != 256 || a.n_tokens != 1 || GEMM_ORDER || dump || a.x_f32 || !a.tail.ticket ||
-        a.tail.n == 0 || a.tail.n % 32u != 0)
-      return hipErrorInvalidValue;
-  }
-  p.head = a.head;
-  if (a.head.kind != OGM_HEAD_NONE) {
-    const bool ptrs_ok = a.head.kind == OGM_HEAD_NORM ? (a.head.x && a.head.weight)
-                         : a.head.kind == OGM_HEAD_SWIGLU ? (a.head.gate && a.head.up) : false;
-    if (!ptrs_ok || F::ELEMS != 256 || F::ACT_GROUP != 256 || a.n_tokens != 1 || GEMM_ORDER || dump || a.x_f32 ||
-        a.tail.kind != OGM_TAIL_NONE || !a.head.flag || a.in_dim % 256u != 0)
-      return hipErrorInvalidValue;
-  }
   p.dump_isum = a.dump_isum;
   p.dump_imin = a.dump_imin;
   p.in_dim = a.in_dim;
@@ -1458,24 +1209,16 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   const OgmTiling tl = ogm_tiling_for(p.upr, a.out_dim);
   p.C = tl.C;
   p.nct = tl.nct;
-  uint32_t n_rb = 0;
-  for (uint32_t m = 0; m <= a.n_extra; m++)
-    n_rb += ((m ? a.extra_out_dim[m - 1] : a.out_dim) + tl.R - 1) / tl.R;
-  if (n_rb == 0) return hipSuccess;
-  // Row blocks per workgroup.  One is the measured optimum on MI355X at every shape tried
-  // (4096 -> 14336 x2: 2, 4 and 8 row blocks cost 7%, 25% and 60% more time): many small
-  // workgroups keep more loads in flight than the shared activation staging saves.
-  uint32_t K = a.rb_per_wg ? a.rb_per_wg : 1;
-  while (K > 1 && gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, K) > OGM_LDS_BUDGET) K--;
-  if (dump) K = 1;
-  p.rb_per_wg = K;
+  // One row block per workgroup: the measured optimum on MI355X at every shape tried (4096 -> 14336 x2: 2, 4 and 8
+  // row blocks a workgroup cost 7 %, 25 % and 60 % more time): many small workgroups keep more loads in flight
+  // than the shared activation staging saves.
   uint32_t n_wg = 0;
   for (uint32_t m = 0; m < OGM_GEMV_MAX_MATS; m++) {
     if (m <= a.n_extra) {
       p.wt[m] = m ? a.extra_wt[m - 1] : a.wt;
       p.y[m] = m ? a.extra_y[m - 1] : a.y;
       p.out_dim[m] = m ? a.extra_out_dim[m - 1] : a.out_dim;
-      n_wg += ((p.out_dim[m] + tl.R - 1) / tl.R + K - 1) / K;
+      n_wg += (p.out_dim[m] + tl.R - 1) / tl.R;
     } else {
       p.wt[m] = nullptr;
       p.y[m] = nullptr;
@@ -1483,12 +1226,12 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
     }
     p.wg_end[m] = n_wg;
   }
+  if (n_wg == 0) return hipSuccess;
   // (rows of many blocks in a format that leaves sixteen terms a block -- Q2_K over per-32 activations at
   // 14336 inputs: 74 KB for one token -- go beyond the budget; they get what they need, up to the hardware's limit)
-  const bool lane_acc = gemv_lane_acc<F, GEMM_ORDER>(a.in_dim) && !dump && a.tail.kind == OGM_TAIL_NONE &&
-                        a.head.kind == OGM_HEAD_NONE;
+  const bool lane_acc = gemv_lane_acc<F, GEMM_ORDER>(a.in_dim) && !dump;
   p.lane_acc = lane_acc ? 1u : 0u;
-  const size_t lds = lane_acc ? gemv_lds_bytes_lane_acc<F>(a.in_dim, a.n_tokens) : gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens, K);
+  const size_t lds = lane_acc ? gemv_lds_bytes_lane_acc<F>(a.in_dim, a.n_tokens) : gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens);
   if (lds > OGM_LDS_MAX) return hipErrorInvalidValue;
   auto launch = [&](void (*kernel)(GemvParams), dim3 g_, dim3 b_) -> hipError_t {
     if (lds > OGM_LDS_BUDGET) {
@@ -1500,31 +1243,20 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   };
   // the plain single-token kernels of most formats need well under 128 registers and are built for up
   // to sixteen waves
-  const bool plain_single = a.n_tokens == 1 && !GEMM_ORDER && !dump && !a.x_f32 && a.tail.kind == OGM_TAIL_NONE &&
-                            a.head.kind == OGM_HEAD_NONE;
+  const bool plain_single = a.n_tokens == 1 && !GEMM_ORDER && !dump;
   // the per-32 formats' tiles are small (2 KB of Q8_0): sixteen of them per workgroup measure 7 %
   // faster than eight at 4096 x 4096
   const uint32_t waves = lane_acc ? 1u
                                   : pick_waves(tl.nct, a.wg_waves, plain_single ? F::MAX_THREADS_SINGLE : F::MAX_THREADS,
                                                (plain_single && F::ELEMS == 32) ? 16u : 8u);
-  if (a.tail.kind == OGM_TAIL_NORM && a.tail.n > 1024u * waves) return hipErrorInvalidValue;
-  if (a.head.kind == OGM_HEAD_NORM) {
-    if (a.in_dim > 1024u * waves) return hipErrorInvalidValue;
-    p.head.n_prod = 1;
-  } else if (a.head.kind == OGM_HEAD_SWIGLU) {
-    p.head.n_prod = (a.in_dim / 256u + waves - 1u) / waves;
-  }
-  const dim3 g(n_wg + p.head.n_prod), b(waves * 64);
-  if (dump) return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true, false>, g, b);
+  const dim3 g(n_wg), b(waves * 64);
+  if (dump) return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, true>, g, b);
   if (a.n_tokens == 1 && !GEMM_ORDER) {
-    // (the kernels with a compile-time row length, tails and heads are for rows that fit the budget many times over)
-    if (lds > OGM_LDS_BUDGET && (a.tail.kind != OGM_TAIL_NONE || a.head.kind != OGM_HEAD_NONE)) return hipErrorInvalidValue;
-    if (a.x_f32) launch_single<F, true>(p, g, b, lds, stream);
-    else launch_single<F, false>(p, g, b, lds, stream);
+    launch_single<F>(p, g, b, lds, stream);
     return hipGetLastError();
   }
-  if (F::HAS_UNPACK && a.n_tokens >= 6) return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false, F::HAS_UNPACK>, g, b);
-  return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, false>, g, b);
+  if (F::HAS_UNPACK && a.n_tokens >= 6) return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false, F::HAS_UNPACK>, g, b);
+  return launch(ogm_gemv_kernel<F, 0, false, GEMM_ORDER, false>, g, b);
 }
 
 hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name) {
@@ -1564,7 +1296,7 @@ hipError_t ogm_launch_gemv(const OgmGemvArgs &a, hipStream_t stream, const char 
       // matmul of several tokens: the rows-unpacked-once arithmetic over per-32 activations; everything
       // else (one token, matmul_decode): per-256 activations
       if (kernel_name) *kernel_name = a.gemm_order ? "ogm_gemv_kernel<FmtQ2KGen,gemm>" : "ogm_gemv_kernel<FmtQ2K,gemv>";
-      if (a.gemm_order) return (a.dump_isum || a.dump_imin || a.x_f32) ? hipErrorInvalidValue : launch_t<FmtQ2KGen, true>(a, stream);
+      if (a.gemm_order) return (a.dump_isum || a.dump_imin) ? hipErrorInvalidValue : launch_t<FmtQ2KGen, true>(a, stream);
       return launch_t<FmtQ2K, false>(a, stream);
     default:
       return hipErrorInvalidValue;

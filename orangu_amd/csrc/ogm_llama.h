@@ -53,15 +53,13 @@ struct OgmAttnPre {
 //     is not null.
 // part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch, with
 // max_splits >= pos / chunk + 1; counters: 2 * n_head_kv * OGM_ATTN_TICKET_STRIDE words (one ticket per
-// cache line), zero before the first launch (the kernel leaves them zero).  share: whether a K/V head's query heads are split over two workgroups
-// (0: when there are four or eight of them and a half still fills whole quantizer groups; 1: never;
-// 2: asked for, an error where it cannot be).
+// cache line), zero before the first launch (the kernel leaves them zero).
 hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
                                   uint32_t rope_dim, const OgmAttnPre &pre, void *k_cache_layer,
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
                                   uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
                                   float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
-                                  hipStream_t stream, uint32_t chunk = 0, uint32_t share = 0);
+                                  hipStream_t stream, uint32_t chunk = 0);
 
 // h = silu(gate) * up with silu(g) = g / (1 + exp(-g))     (tensor.rs:825-827, arch/mod.rs:1071-1106)
 // quantized for the down projection in `mode`; h (f32) is also stored when not null.  With

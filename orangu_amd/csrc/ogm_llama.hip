@@ -206,7 +206,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
                                                        OgmAttnPre pre, uint32_t gq,
                                                        __half *__restrict__ kc, __half *__restrict__ vc,
                                                        uint32_t pos, uint32_t max_splits, uint32_t n_head_kv,
-                                                       uint32_t kv_share, float scale, float *part_o, float *part_ml,
+                                                       float scale, float *part_o, float *part_ml,
                                                        uint32_t *counters, float *__restrict__ attn_out,
                                                        OgmActDev act) {
   constexpr int NT = 4 * CHUNK, NW = NT / 64;   // four threads per cache position
@@ -226,9 +226,8 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
   __shared__ float mrg[GROUP != 0 ? 6 : 1][GROUP != 0 ? NT : 1];   // the final merge's slices
   static_assert(!PREFILL || GROUP == 0, "a prefill batch merges in its own launch");
   OGM_STAMP(0);
-  // blockIdx.x: a group of gq query heads (G head slots) that share a K/V head; kv_share such groups
-  // per K/V head (1: all its query heads in one workgroup)
-  const uint32_t hg = blockIdx.x, split = blockIdx.y, kvh = hg / kv_share;
+  // blockIdx.x: a K/V head and the gq query heads (G head slots) that share it
+  const uint32_t hg = blockIdx.x, split = blockIdx.y, kvh = hg;
   if constexpr (PREFILL) {
     const uint32_t tok = blockIdx.z;
     pos += tok;
@@ -577,7 +576,7 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
                                   uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
                                   float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
-                                  hipStream_t stream, uint32_t chunk, uint32_t share) {
+                                  hipStream_t stream, uint32_t chunk) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0) return hipErrorInvalidValue;
   if (rope_dim > head_dim || rope_dim % 2u != 0) return hipErrorInvalidValue;
   // Cache positions per workgroup: 128; 64 only for short contexts.  The kernel is a chain of
@@ -594,18 +593,7 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
   if (n % 32u != 0) return hipErrorInvalidValue;
   uint32_t gq = n_head / n_head_kv;
   if (gq > 8u) return hipErrorInvalidValue;
-  // Four or eight query heads per K/V head are split over two workgroups of half as many when those
-  // still fill whole quantizer groups (the merge stays in the kernel): twice the workgroups, each with
-  // half the scores, sums and merge, for reading the chunk's K and V rows twice out of L2 (both write
-  // the new cache row, with the same bits).  share: 0 this rule, 1 never, 2 asked for.  Measured on
-  // MI355X (32 query heads on 8 K/V heads, 2048 cached positions): 2 us a layer slower than one workgroup
-  // per K/V head -- the kernel is a chain of latencies, not of work -- so the decode step asks for 1.
-  const uint32_t group_ = mode == 0 ? 32u : 256u;
-  const bool can_share = (gq == 4u || gq == 8u) && ((gq / 2u) * head_dim) % group_ == 0;
-  if (share > 2u || (share == 2u && !can_share)) return hipErrorInvalidValue;
-  const uint32_t kv_share = (share == 0u ? can_share : share == 2u) ? 2u : 1u;
-  gq /= kv_share;
-  const dim3 grid(n_head_kv * kv_share, n_splits);
+  const dim3 grid(n_head_kv, n_splits);
   const uint32_t G = gq <= 2u ? gq : (gq <= 4u ? 4u : 8u);   // head slots of the kernel
   const uint32_t group = mode == 0 ? 32u : 256u;
   // the merge rides in the attention kernel when every head slot is a head and a K/V head's
@@ -614,7 +602,7 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
 #define OGM_ATTN_LAUNCH_C(HD_, G_, GR_, CH_)                                                           \
   hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, GR_, false, CH_>), grid, dim3(4 * CH_), 0, stream, q, k_new, \
                      v_new, (const float2 *)cs, rope_dim / 2u, pre, gq, (__half *)k_cache_layer,        \
-                     (__half *)v_cache_layer, pos, max_splits, n_head_kv, kv_share, scale, part_o, part_ml, \
+                     (__half *)v_cache_layer, pos, max_splits, n_head_kv, scale, part_o, part_ml, \
                      counters, attn_out, act)
 #define OGM_ATTN_LAUNCH(HD_, G_, GR_)                    \
   do {                                                   \
@@ -1037,7 +1025,7 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
 #define OGM_ATTN_PREFILL(HD_, G_)                                                                           \
   hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, 0, true>), grid, dim3(512), 0, stream, q, (const float *)nullptr, \
                      (const float *)nullptr, (const float2 *)nullptr, 0u, none, gq, (__half *)k_cache_layer,  \
-                     (__half *)v_cache_layer, pos0, max_splits, n_head_kv, 1u, scale, part_o, part_ml,        \
+                     (__half *)v_cache_layer, pos0, max_splits, n_head_kv, scale, part_o, part_ml,            \
                      (uint32_t *)nullptr, (float *)nullptr, no_act)
   if (head_dim == 128 && G == 1) OGM_ATTN_PREFILL(128, 1);
   else if (head_dim == 128 && G == 2) OGM_ATTN_PREFILL(128, 2);

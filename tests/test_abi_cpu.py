@@ -150,6 +150,6 @@ def test_every_tuning_key_the_library_accepts_is_documented_in_the_header():
     src = open(os.path.join(root, "orangu_amd", "csrc", "ogm_api.cpp")).read()
     header = open(os.path.join(root, "include", "orangu_mi355x.h")).read()
     keys = re.findall(r'strcmp\(key, "([a-z0-9_]+)"\)', src)
-    assert len(keys) >= 20 and len(set(keys)) == len(keys)
+    assert len(keys) >= 10 and len(set(keys)) == len(keys)
     missing = [k for k in keys if f'"{k}"' not in header]
     assert not missing, missing

@@ -107,24 +107,24 @@ def test_one_pass_gemm_against_exact_arithmetic_and_the_reference_order(be, ggml
 
 def test_one_pass_is_refused_nothing_and_changes_nothing_elsewhere(be):
     """The key only reaches Q4_K / Q5_K on the all-waves-multiply kernel: Q6_K on it, and Q4_K on the
-    feeding-wave kernels, keep the reference's bits with the key set."""
+    feeding-wave kernels (a matrix without planes), keep the reference's bits with the key set."""
     from orangu_amd import QuantMatrix
     from helpers import Q6_K
     be.set_tuning("gemm_one_pass", 1)
     try:
-        for ggml_type, plane_kernel in ((Q6_K, 2), (Q4_K, 1)):
+        for ggml_type, planes in ((Q6_K, True), (Q4_K, False)):
             in_dim, out_dim, T = 1024, 200, 140
             raw = synth_weights(ggml_type, in_dim, out_dim, seed=5)
             x = synth_x(T, in_dim, seed=6)
-            be.set_tuning("gemm_plane_kernel", plane_kernel)
+            be.set_tuning("gemm_plane_cache_mb", 65536 if planes else 0)
             got = np.asarray(be.matmul(x, T, QuantMatrix(np.ascontiguousarray(raw), ggml_type, in_dim, out_dim)))
             say("   ", be.last_kernel())
-            assert "onepass" not in be.last_kernel()
+            assert "onepass" not in be.last_kernel() and ("_dma_" in be.last_kernel()) == planes
             want = oracle.matmul(ggml_type, raw, in_dim, out_dim, x, T)
             assert np.array_equal(got.reshape(-1).view(np.uint32), want.reshape(-1).view(np.uint32))
     finally:
         be.set_tuning("gemm_one_pass", 0)
-        be.set_tuning("gemm_plane_kernel", 2)
+        be.set_tuning("gemm_plane_cache_mb", 65536)
 
 
 def test_one_pass_over_several_matrices_in_one_launch(be):

@@ -186,105 +186,6 @@ def test_decode_with_a_cache_too_long_for_a_table_of_every_position(be):
         dev.close()
 
 
-@pytest.mark.parametrize("types,n_embd,n_ff", [((Q4_K, Q6_K, Q6_K, Q6_K), 256, 512), ((Q4_K, Q4_K, Q6_K, Q6_K), 1024, 2816),
-                                               ((Q5_K, Q3_K, Q3_K, Q5_K), 512, 1280), ((Q4_K, Q4_K, Q8_0, Q8_0), 256, 512),
-                                               ((Q8_0, Q8_0, Q4_K, Q6_K), 256, 512)])
-def test_norms_and_swiglu_as_gemv_tails_change_no_bit(be, types, n_embd, n_ff):
-    """On request (decode_fuse_tails) the decode step runs the FFN norm, the SwiGLU and the next
-    attention (or output) norm as the tail of the GEMV launch before them (its last workgroup to
-    finish) wherever the consumer takes per-256 activations, instead of as kernels of their own: the
-    same arithmetic either way, so logits and greedy tokens agree to the bit over several steps."""
-    outs = []
-    xs = np.random.default_rng(11).standard_normal((4, n_embd)).astype(f32)
-    for fuse in (1, 0, 1):
-        ref, dev, rng = build(be, n_embd=n_embd, n_head=4, n_kv=2, hd=64, n_ff=n_ff, n_vocab=320, n_layer=3,
-                              types=types, max_ctx=16, seed=9)
-        be.set_tuning("decode_fuse_tails", fuse)
-        try:
-            got = [dev.decode(xs[pos], pos) for pos in range(4)]
-        finally:
-            be.set_tuning("decode_fuse_tails", 0)
-            dev.close()
-        outs.append(got)
-    for other in outs[1:]:
-        for pos, ((la, ta), (lb, tb)) in enumerate(zip(outs[0], other)):
-            assert ta == tb, pos
-            assert np.array_equal(la.view(np.uint32), lb.view(np.uint32)), (types, pos)
-
-
-@pytest.mark.parametrize("types,n_embd,n_ff", [((Q4_K, Q6_K, Q6_K, Q6_K), 256, 512), ((Q4_K, Q4_K, Q6_K, Q6_K), 1024, 2816),
-                                               ((Q5_K, Q3_K, Q3_K, Q5_K), 512, 1280), ((Q4_K, Q4_K, Q8_0, Q8_0), 256, 512),
-                                               ((IQ4_XS, Q2_K, IQ4_XS, Q2_K), 512, 1024), ((Q4_K, Q4_K, Q4_K, Q6_K), 4096, 1024)])
-def test_norms_and_swiglu_as_gemv_heads_change_no_bit(be, types, n_embd, n_ff):
-    """On request (decode_fuse_heads) the decode step runs the attention norm, the FFN norm and the SwiGLU at
-    the head of the GEMV launch after them (extra workgroups at its front, a flag, the others waiting behind
-    their first weight loads) wherever that launch takes per-256 activations, instead of as kernels of their
-    own: the same arithmetic either way, so logits and greedy tokens agree to the bit over several steps, with
-    and without the waiting workgroups' delay.  (Matrices of a group in different types -- the second entry's v
-    -- go out as several launches of which the first brings the producers.)"""
-    outs = []
-    n_head, n_kv = (4, 2) if n_embd < 4096 else (32, 8)
-    xs = np.random.default_rng(11).standard_normal((5, n_embd)).astype(f32)
-    for fuse, delay in ((1, 64), (0, 64), (1, 0)):
-        ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=64, n_ff=n_ff, n_vocab=320,
-                              n_layer=1 if Q2_K in types else 3, types=types, max_ctx=16, seed=9)
-        be.set_tuning("decode_fuse_heads", fuse)
-        be.set_tuning("decode_head_delay", delay)
-        try:
-            got = [dev.decode(xs[pos], pos) for pos in range(5)]
-        finally:
-            be.set_tuning("decode_fuse_heads", 0)
-            be.set_tuning("decode_head_delay", 64)
-            dev.close()
-        outs.append(got)
-    for other in outs[1:]:
-        for pos, ((la, ta), (lb, tb)) in enumerate(zip(outs[0], other)):
-            assert ta == tb, pos
-            assert np.array_equal(la.view(np.uint32), lb.view(np.uint32)), (types, pos)
-
-
-def test_a_head_whose_flag_never_comes_is_given_up_and_reported(be):
-    """The waiting workgroups' poll is bounded: with a limit of one poll they give up before the producers can
-    have finished, every wave still ends, and the step reports it instead of returning its logits as good; the
-    next step, with the default limit, is right again."""
-    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
-                          types=(Q4_K, Q4_K, Q6_K, Q6_K), max_ctx=16, seed=3)
-    x = np.random.default_rng(2).standard_normal(256).astype(f32)
-    try:
-        want = dev.decode(x, 0)
-        be.set_tuning("decode_fuse_heads", 1)
-        be.set_tuning("decode_head_spin_limit", 1)
-        be.set_tuning("decode_head_delay", 0)
-        with pytest.raises(RuntimeError, match="gave up"):
-            dev.decode(x, 0)
-        be.set_tuning("decode_head_spin_limit", 0)
-        got = dev.decode(x, 0)
-        assert got[1] == want[1] and np.array_equal(got[0].view(np.uint32), want[0].view(np.uint32))
-    finally:
-        be.set_tuning("decode_fuse_heads", 0)
-        be.set_tuning("decode_head_spin_limit", 0)
-        be.set_tuning("decode_head_delay", 64)
-        dev.close()
-
-
-def test_decode_with_a_kv_heads_query_heads_split_over_two_workgroups(be):
-    """attn_decode_share 2: four query heads per K/V head of head_dim 128 run as two workgroups of two (each
-    merges and quantizes one group of 256 outputs); against the CPU restatement like every other step, over a
-    prefilled cache of several chunks."""
-    n_kv, hd = 2, 128
-    ref, dev, rng = build(be, n_embd=512, n_head=8, n_kv=n_kv, hd=hd, n_ff=1024, n_vocab=320, n_layer=2,
-                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=400, seed=21, attn_norm_scale=TAME[Q4_K])
-    be.set_tuning("attn_decode_share", 2)
-    try:
-        X = rng.standard_normal((300, 512)).astype(f32)
-        prefill_both(ref, dev, X, 0, "300 tokens")
-        for pos in range(300, 304):
-            step_both(ref, dev, rng.standard_normal(512).astype(f32), pos, f"shared K/V heads pos {pos}")
-    finally:
-        be.set_tuning("attn_decode_share", 1)
-        dev.close()
-
-
 def test_decode_with_q3_k_value_and_down_projections(be):
     """Q3_K in the v and down projections (what a Q3_K_M file does), one layer: the synthetic Q3_K
     weights are large, and with two layers of them the final hidden state is a small difference of
