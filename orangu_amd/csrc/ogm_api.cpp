@@ -79,6 +79,7 @@ struct ogm_ctx {
   // what the activation buffer currently holds (ogm_act_quantize_dev)
   int act_mode = -1;
   uint32_t act_in_dim = 0, act_tokens = 0;
+  bool act_xt = false;   // ... and xh holds the same activations in the tiled GEMM's operand chunks
 };
 
 static thread_local std::string g_init_err;
@@ -461,14 +462,18 @@ extern "C" int ogm_weight_info(const ogm_weight *w, uint32_t *ggml_type, uint32_
 // matmul
 
 // Enqueues the activation quantizer.  Caller holds the lock.
+// with_xt: the int8 activations also go to ctx->xh in the operand chunks of the GEMM whose waves all multiply.
 static int enqueue_quantize(ogm_ctx *ctx, int mode, const float *x_dev, uint32_t in_dim,
-                            uint32_t n_tokens, hipStream_t stream) {
+                            uint32_t n_tokens, hipStream_t stream, bool with_xt = false) {
   int rc = ensure_act(ctx, in_dim, n_tokens);
   if (rc != OGM_OK) return rc;
-  HIPCHK(ctx, ogm_launch_quantize(mode, x_dev, in_dim, n_tokens, act_view(ctx, in_dim, mode, 0), stream));
+  if (with_xt && (rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(in_dim, n_tokens))) != OGM_OK) return rc;
+  HIPCHK(ctx, ogm_launch_quantize(mode, x_dev, in_dim, n_tokens, act_view(ctx, in_dim, mode, 0), stream,
+                                  with_xt ? (int8_t *)ctx->xh.p : nullptr));
   ctx->act_mode = mode;
   ctx->act_in_dim = in_dim;
   ctx->act_tokens = n_tokens;
+  ctx->act_xt = with_xt;
   return OGM_OK;
 }
 
@@ -489,7 +494,12 @@ static int enqueue_matmul(ogm_ctx *ctx, const Target *tg, size_t n_tg, const flo
                           int32_t *dump_imin) {
   if (n_tokens == 0 || n_tg == 0) return OGM_OK;
   const ogm_weight *w = tg[0].w;
-  int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type, n_tokens, decode), x_dev, w->in_dim, n_tokens, stream);
+  // A batch that may go to the GEMM over prebuilt planes has its activations laid out for it by the quantizer
+  // itself (32 tokens on, K-quants with planes enabled); whether that kernel runs is decided per launch.
+  const bool with_xt = !decode && n_tokens >= 32 && !dump_isum && !dump_imin && ctx->tune_plane_cache_mb > 0 &&
+                       ogm_gemm_plane_bytes(w->ggml_type, w->in_dim, w->out_dim) != 0 &&
+                       (uint64_t)((n_tokens + 31u) & ~31u) * w->in_dim < (1ull << 32);
+  int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type, n_tokens, decode), x_dev, w->in_dim, n_tokens, stream, with_xt);
   if (rc != OGM_OK) return rc;
   return enqueue_gemv(ctx, tg, n_tg, n_tokens, decode, stream, dump_isum, dump_imin);
 }
@@ -592,6 +602,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.n_tokens = n_tokens;
       g.y = tg[i].y;
       g.xh = ctx->xh.p;
+      g.xt_ready = ctx->act_xt && ctx->act_in_dim == w0->in_dim && ctx->act_tokens == n_tokens;
       g.tile_rows = (uint32_t)ctx->tune_gemm_tile_rows;
       g.small_max_tokens = (uint32_t)ctx->tune_gemm_small_max;
       g.sb_waves = (uint32_t)ctx->tune_gemm_sb_waves;
@@ -1720,6 +1731,7 @@ static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws
   ctx->act_mode = mode;
   ctx->act_in_dim = in_dim;
   ctx->act_tokens = T;
+  ctx->act_xt = false;   // the producers wrote the token-major buffers only
   size_t i = 0;
   while (i < n) {
     Target tg[OGM_GEMV_MAX_MATS];

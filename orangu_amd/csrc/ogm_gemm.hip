@@ -1869,8 +1869,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   for (uint32_t m = 0; m < a.n_extra; m++) have_planes = have_planes && a.extra_planes[m] != nullptr;   // every matrix of the launch, or none
   if (have_planes && gemm_dma_eligible(a)) {
     const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
-    hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3(a.in_dim / 128u, t_pad / 32u), dim3(256), 0, stream, a.act.q,
-                       (int8_t *)a.xh, a.in_dim, a.n_tokens);
+    if (!a.xt_ready)
+      hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3(a.in_dim / 128u, t_pad / 32u), dim3(256), 0, stream, a.act.q,
+                         (int8_t *)a.xh, a.in_dim, a.n_tokens);
     GemmDmaParams d;
     d.wt = a.wt;
     d.planes = a.planes;

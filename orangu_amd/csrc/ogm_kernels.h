@@ -19,8 +19,10 @@ struct OgmActDev {
 };
 
 // mode 0: one scale per 32 (vecdot.rs:95-126); mode 1: one per 256 (vecdot.rs:3030-3053).
+// xt (per-256 mode only): when not null, the int8 activations are also written there in the operand chunks of
+// the GEMM whose waves all multiply (ogm_gemm_xh_bytes() bytes), which then needs no relayout pass of its own.
 hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,
-                               OgmActDev act, hipStream_t stream);
+                               OgmActDev act, hipStream_t stream, int8_t *xt = nullptr);
 
 #define OGM_GEMV_MAX_MATS 4
 
@@ -57,6 +59,7 @@ struct OgmGemmArgs {
   uint32_t n_tokens;
   float *y;            // [n_tokens][out_dim]
   void *xh;            // scratch
+  bool xt_ready = false;   // the quantizer has already written the operand chunks to xh
   uint32_t tile_rows = 0;          // feeding-wave kernels: 64 forces their 64-row tiles (0 = by the size of the launch)
   uint32_t small_max_tokens = 0;   // most tokens for the small-batch kernel (0 = default 64, 1 = never)
   uint32_t sb_waves = 0;           // waves of a small-batch workgroup: 8 or 16 (0 = by the size of the launch)

@@ -98,9 +98,50 @@ __global__ __launch_bounds__(64) void ogm_quantize_kernel(const float *__restric
                             act.bs16 ? act.bs16 + (size_t)t * (in_dim / 16) : nullptr);
 }
 
+// The per-256 quantizer of a prefill batch that also lays the int8 activations out in the operand order of the
+// GEMM whose waves all multiply (ogm_gemm.hip): chunk (token block of 32, step of 32 k) is 1 KiB, lane (l32, lh)'s
+// 16 bytes -- the activations 32 step + 16 lh .. of token 32 block + l32 -- at 16 (32 lh + l32).  A workgroup takes
+// 32 tokens x 256 activations, each of its eight waves four of the tokens; the eight chunks it fills are 8 KiB in
+// a row, written as whole lines out of LDS.  Tokens past the last repeat it in the chunks (never multiplied into
+// a stored output); their token-major outputs are not written.
+__global__ __launch_bounds__(512) void ogm_quantize_xt_kernel(const float *__restrict__ x, uint32_t in_dim,
+                                                              uint32_t n_tokens, OgmActDev act, int8_t *__restrict__ xt) {
+  __shared__ uint4 tile[32][17];   // [token][16-byte piece], rows padded by a piece against bank conflicts
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t run = blockIdx.x, tb = blockIdx.y;
+  const uint32_t e0 = run * 256u + lane * 4u;
+  float4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t t = min(tb * 32u + wave + 8u * i, n_tokens - 1u);
+    v[i] = *(const float4 *)(x + (size_t)t * in_dim + e0);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t tl = wave + 8u * i, t = tb * 32u + tl;
+    const bool active = t < n_tokens;
+    const uint32_t tc = min(t, n_tokens - 1u);
+    const uint32_t packed = ogm_quantize_store<256>(v[i], e0, active, lane, act.q + (size_t)tc * in_dim,
+                                                    act.d + (size_t)tc * (in_dim / 256), act.sums + (size_t)tc * (in_dim / 16),
+                                                    act.bsum + (size_t)tc * (in_dim / 32),
+                                                    act.bs16 ? act.bs16 + (size_t)tc * (in_dim / 16) : nullptr);
+    ((uint32_t *)&tile[tl][lane >> 2])[lane & 3u] = packed;
+  }
+  __syncthreads();
+  const uint32_t step = tid >> 6, slot = tid & 63u;   // the chunk of the eight, the lane of its operand
+  const uint4 o = tile[slot & 31u][2u * step + (slot >> 5)];
+  *(uint4 *)(xt + ((size_t)tb * (in_dim / 32u) + run * 8u + step) * 1024u + slot * 16u) = o;
+}
+
 hipError_t ogm_launch_quantize(int mode, const float *x, uint32_t in_dim, uint32_t n_tokens,
-                               OgmActDev act, hipStream_t stream) {
+                               OgmActDev act, hipStream_t stream, int8_t *xt) {
   if (n_tokens == 0) return hipSuccess;
+  if (xt != nullptr) {
+    if (mode != 1 || in_dim % 256u != 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(ogm_quantize_xt_kernel, dim3(in_dim / 256u, (n_tokens + 31u) / 32u), dim3(512), 0, stream, x,
+                       in_dim, n_tokens, act, xt);
+    return hipGetLastError();
+  }
   dim3 grid((in_dim + 255) / 256, n_tokens);
   if (mode == 0)
     hipLaunchKernelGGL(ogm_quantize_kernel<32>, grid, dim3(64), 0, stream, x, in_dim, act);

@@ -133,12 +133,13 @@ __device__ __forceinline__ void ogm_st(T *p, T v) {
 }
 
 // Quantizes and stores one lane's share of a 256-run whose first element is e0 (= 256*run +
-// 4*lane) of token-major activations with row length in_dim; t_off* are the token's offsets.
+// 4*lane) of token-major activations with row length in_dim; t_off* are the token's offsets.  Returns the
+// lane's four quantized values, packed.
 // COHERENT_OUT: the stores are for other workgroups of the same kernel (ogm_st).
 template <int GROUP, bool COHERENT_OUT = false>
-__device__ __forceinline__ void ogm_quantize_store(const float4 &v, uint32_t e0, bool active, uint32_t lane,
-                                                   int8_t *q, float *d, int32_t *sums, int16_t *bsum,
-                                                   uint16_t *bs16) {
+__device__ __forceinline__ uint32_t ogm_quantize_store(const float4 &v, uint32_t e0, bool active, uint32_t lane,
+                                                       int8_t *q, float *d, int32_t *sums, int16_t *bsum,
+                                                       uint16_t *bs16) {
   float scale;
   int s16, s32;
   const uint32_t packed = ogm_quantize4<GROUP>(v, scale, s16, s32);
@@ -156,6 +157,7 @@ __device__ __forceinline__ void ogm_quantize_store(const float4 &v, uint32_t e0,
     }
     if ((lane & (GROUP / 4 - 1)) == 0) ogm_st<COHERENT_OUT>(d + e0 / GROUP, scale);
   }
+  return packed;   // the lane's four int8 values, also for callers that lay them out a second way
 }
 
 // Four floats that another workgroup of the same kernel may have stored device-coherently.
