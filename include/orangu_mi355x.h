@@ -397,6 +397,9 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              waves work on different super-blocks of the same rows; 0 = default (64, more
  *                              for matrices of few rows), 1 = never
  *   "gemm_sb_waves"            waves of a small-batch workgroup: 8 or 16; 0 = by the size of the launch
+ *   "gemm_medium"              the Q4_K / Q5_K kernel for one or two nearly full tiles of 128 tokens (32 rows x
+ *                              128 tokens a workgroup, its waves on different super-blocks): 0 = by the size of
+ *                              the launch, 1 = never, 2 = whenever the shape allows
  *   "gemm_tile_rows"           feeding-wave GEMMs: 64 = always their 64-row tiles; 0 = by the size of the launch
  *   "gemm_few_tokens_min_rows" 2 to 16 tokens over a Q6_K matrix (matmul and matmul_decode alike) take the
  *                              kernel that streams the weights once when the matrix has at least this many

@@ -59,6 +59,7 @@ struct ogm_ctx {
   // tokens: 12 against 16 us), 17 for the others, whose tiled kernels cost about the same from 9 to 128
   // tokens while the chunked GEMV grows with the count (they cross between 12 and 32 tokens).
   int tune_gemm_min_tokens = 0;
+  int tune_gemm_medium = 0;      // Q4_K / Q5_K medium-batch kernel: 0 by the size of the launch, 1 never, 2 whenever the shape allows
   int tune_gemm_tile_rows = 0;   // feeding-wave GEMMs: 64 forces their 64-row tiles, 0 = by the size of the launch
   int tune_gemm_small_max = 0;   // most tokens for the small-batch GEMM kernel: 0 = default, 1 = never
   int tune_gemm_ft_min_rows = 0;  // few-token Q6_K kernel: fewest rows it takes (0 = default, 1 = any shape it can, -1 = never)
@@ -292,6 +293,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "host_zero_copy") == 0) {
     if (value != 0 && value != 1) return fail(ctx, OGM_ERR_INVALID, "host_zero_copy must be 0 or 1");
     ctx->tune_host_zero_copy = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_medium") == 0) {
+    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_medium must be 0, 1 or 2");
+    ctx->tune_gemm_medium = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_tile_rows") == 0) {
@@ -604,6 +610,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.xh = ctx->xh.p;
       g.xt_ready = ctx->act_xt && ctx->act_in_dim == w0->in_dim && ctx->act_tokens == n_tokens;
       g.tile_rows = (uint32_t)ctx->tune_gemm_tile_rows;
+      g.medium = (uint32_t)ctx->tune_gemm_medium;
       g.small_max_tokens = (uint32_t)ctx->tune_gemm_small_max;
       g.sb_waves = (uint32_t)ctx->tune_gemm_sb_waves;
       g.plane_kernel = (uint32_t)ctx->tune_gemm_plane_kernel;

@@ -1452,6 +1452,256 @@ __global__ __launch_bounds__(512) void ogm_gemm_sb_q45k_kernel(GemmSbParams p) {
 template <bool Q5>
 __global__ __launch_bounds__(1024) void ogm_gemm_sb_q45k_w16_kernel(GemmSbParams p) { gemm_sb_q45k_body<Q5, 16u>(p); }
 
+// ------------------------------------------------------------------------------------------
+// Medium batches of Q4_K / Q5_K (some 65 to 256 tokens over a matrix whose 128 x 128 tiles would leave compute
+// units idle): the small-batch scheme on 32 rows x 128 tokens.  A workgroup has four waves, wave w takes the
+// super-blocks s = w (mod 4); it unpacks a sub-block's 16 weights per lane once into the two scale-folded int8
+// planes (u = sc_j q + 128 = 256 h + (l + 128)) and multiplies them with the four token blocks' activations,
+// which it reads as whole operand chunks (the quantizer's second layout) straight from memory: two plain chains of
+// v_mfma_i32_32x32x32_i8 per token block over the super-block, isum = 256 H + L.  The terms ad * (d * isum) -- and,
+// in a sweep of their own before, (ad * dmin) * imin -- go to LDS and are added in ascending super-block order after
+// every round of four, one accumulator per output: gemm_k_q4_k's sequence (vecdot.rs:2213-2303).
+
+struct GemmSbwParams {
+  const uint8_t *wt;      // tile-planar weights
+  const int8_t *xt;       // the int8 activations in operand chunks: [T / 32][in_dim / 32] x 1 KiB
+  const float *ad;        // [T][nsb]
+  const _Float16 *bs16;   // the quantizer's sums per 32 as (bsum / 64, bsum % 64) in f16
+  float *y;               // [T][out_dim]
+  uint32_t in_dim, out_dim, n_tokens, nsb;
+  uint32_t c_shift, r_shift, nct;
+  uint32_t n_extra;
+  const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1];
+  float *extra_y[OGM_GEMM_MAX_MATS - 1];
+  uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
+};
+
+#ifndef SBW_ABL
+#define SBW_ABL 0   // timing experiments only: 1 no activation loads after a super-block's first, 2 no first sweep, 4 no ordered adds
+#endif
+#define SBW_NW 4u
+#define SBW_TOK 128u
+#define SBW_TERMS_BYTES (SBW_NW * SBW_TOK * 32u * 4u)   // 64 KB
+
+template <bool Q5>
+__global__ __launch_bounds__(64 * SBW_NW, 2) void ogm_gemm_sbw_q45k_kernel(GemmSbwParams p) {
+  constexpr uint32_t TILE_BYTES = Q5 ? 11264u : 9216u;
+  constexpr uint32_t QS_PIECE0 = Q5 ? 3u : 1u;
+  constexpr uint32_t NT = 64u * SBW_NW, NACC = SBW_TOK * 32u / NT;   // 16 outputs a thread
+  extern __shared__ __align__(16) uint8_t sbw_lds[];
+  float *terms = (float *)sbw_lds;                 // [4 waves][128 tokens][32 rows]
+  float *ad_l = terms + SBW_NW * SBW_TOK * 32u;    // [nsb][128 tokens]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  uint32_t row_tile = blockIdx.y;
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + 31u) / 32u;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = blockIdx.x * SBW_TOK, r0 = row_tile * 32u;
+  uint32_t uo;   // this lane's row: its header piece
+  {
+    const uint32_t row = min(r0 + l32, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    uo = rb * p.nct * TILE_BYTES + r * 16u;
+  }
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
+  };
+
+  for (uint32_t i = tid; i < SBW_TOK * p.nsb; i += NT) {
+    const uint32_t k = i / p.nsb, s = i - k * p.nsb;
+    ad_l[s * SBW_TOK + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + s];
+  }
+  __syncthreads();
+
+  float acc[NACC];   // outputs (token, row) = (tid / 32 + 8 a, tid % 32)
+#pragma unroll
+  for (uint32_t a = 0; a < NACC; a++) acc[a] = 0.0f;
+  // the first round's weights of the second sweep are in flight over the first
+  uint4 hdr, w0, w1, w2, w3, qh5 = make_uint4(0, 0, 0, 0);
+#define SBW_LOADW(S)                                                                              \
+  do {                                                                                            \
+    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded, never used */    \
+    const uint32_t so_ = uo + sb_off(s_);                                                         \
+    hdr = *(const uint4 *)(p.wt + so_);                                                           \
+    w0 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 0u + lh) * 1024u));                          \
+    w1 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 2u + lh) * 1024u));                          \
+    w2 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 4u + lh) * 1024u));                          \
+    w3 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 6u + lh) * 1024u));                          \
+    if constexpr (Q5) qh5 = *(const uint4 *)(p.wt + (so_ + (1u + lh) * 1024u));                   \
+  } while (0)
+  SBW_LOADW(wave);
+
+  // ---- first sweep: acc -= (ad * dmin) * sum_j m_j * bsum_j, every super-block, in order
+  if (!(SBW_ABL & 2)) {
+    float16v zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.0f;
+    const float side_scale = lh ? 1.0f : 64.0f;
+    uint32_t tk[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) tk[tb] = min(t0 + 32u * tb + l32, p.n_tokens - 1u) * p.nsb;
+    // (a round's header and sums are requested a round ahead: past the end they are loaded again, never used)
+    uint4 hd_n = *(const uint4 *)(p.wt + (uo + sb_off(min(wave, p.nsb - 1u))));
+    half8 b2_n[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) b2_n[tb] = *(const half8 *)(p.bs16 + ((tk[tb] + min(wave, p.nsb - 1u)) * 16u + 8u * lh));
+    for (uint32_t s0 = 0; s0 < p.nsb; s0 += SBW_NW) {
+      const uint32_t s = s0 + wave;
+      const uint4 hd = hd_n;
+      half8 b2[4];
+#pragma unroll
+      for (int tb = 0; tb < 4; tb++) b2[tb] = b2_n[tb];
+      {
+        const uint32_t sn = min(s + SBW_NW, p.nsb - 1u);
+        hd_n = *(const uint4 *)(p.wt + (uo + sb_off(sn)));
+#pragma unroll
+        for (int tb = 0; tb < 4; tb++) b2_n[tb] = *(const half8 *)(p.bs16 + ((tk[tb] + sn) * 16u + 8u * lh));
+      }
+      if (s < p.nsb) {   // wave-uniform
+        uint32_t mna, mnb;
+        q4k_mins(hd, mna, mnb);
+        const half8 a1 = side_operand(mna, mnb, side_scale);
+        const float dm = gm_f16_bits_to_f32(hd.x >> 16);
+#pragma unroll
+        for (int tb = 0; tb < 4; tb++) {
+          const float16v im = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2[tb], a1, zero, 0, 0, 0);
+          const float *adp = &ad_l[s * SBW_TOK + 32u * tb + 4u * lh];
+          float *tp = terms + (wave * SBW_TOK + 32u * tb + 4u * lh) * 32u + l32;   // [wave][token][row]
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++) {
+            const float4 a4 = *(const float4 *)(adp + 8 * q4);
+            const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) tp[(8 * q4 + e) * 32] = a4v[e] * dm * im[4 * q4 + e];
+          }
+        }
+      }
+      __syncthreads();
+      const uint32_t n_here = min(SBW_NW, p.nsb - s0);
+      for (uint32_t w = 0; w < n_here; w++) {
+#pragma unroll
+        for (uint32_t a = 0; a < NACC; a++) acc[a] -= terms[w * (SBW_TOK * 32u) + a * NT + tid];
+      }
+      __syncthreads();
+    }
+  }
+
+  // ---- second sweep: acc += ad * (d * sum_j sc_j * dot32_j)
+  // (token blocks past the last one read it again; their outputs are never stored)
+  uint32_t xo[4];
+#pragma unroll
+  for (int tb = 0; tb < 4; tb++)
+    xo[tb] = min((t0 >> 5) + (uint32_t)tb, (p.n_tokens - 1u) >> 5) * (p.in_dim / 32u) * 1024u + lane * 16u;   // + (8 s + j) * 1024
+#define SBW_LOADX(DST, XS, J)                                                                     \
+  do {                                                                                            \
+    if ((SBW_ABL & 1) && (J) > 1) break;                                                          \
+    _Pragma("unroll") for (int tb_ = 0; tb_ < 4; tb_++)                                           \
+      DST[tb_] = *(const int4v *)(p.xt + (xo[tb_] + (XS) + 1024u * (J)));                         \
+  } while (0)
+  // sub-block J: its 16 weights per lane -> the two planes, then the four token blocks
+#define SBW_STEP(QS, J, XA, FIRST)                                                                \
+  do {                                                                                            \
+    const int sc_ = (int)((((J) < 4 ? sca_ : scb_) >> (8u * ((J) & 3u))) & 0xFFu);                \
+    const short2v sc2_ = {(short)sc_, (short)sc_};                                                \
+    const short2v c2_ = {(short)128, (short)128};                                                 \
+    const uint32_t qsw_[4] = {QS.x, QS.y, QS.z, QS.w}, q5w_[4] = {qh5.x, qh5.y, qh5.z, qh5.w};    \
+    uint32_t ph_[4], pl_[4];                                                                      \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      uint32_t v_ = (((J) & 1) ? (qsw_[w_] >> 4) : qsw_[w_]) & 0x0F0F0F0Fu;                       \
+      if constexpr (Q5) v_ |= ((q5w_[w_] >> (J)) & 0x01010101u) << 4;                             \
+      union { uint32_t u; short2v s; } e_, f_;                                                    \
+      e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
+      f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
+      e_.s = e_.s * sc2_ + c2_;                                                                   \
+      f_.s = f_.s * sc2_ + c2_;                                                                   \
+      ph_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x07050301u);                                   \
+      pl_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u) ^ 0x80808080u;                     \
+    }                                                                                             \
+    const int4v bh_ = {(int)ph_[0], (int)ph_[1], (int)ph_[2], (int)ph_[3]};                       \
+    const int4v bl_ = {(int)pl_[0], (int)pl_[1], (int)pl_[2], (int)pl_[3]};                       \
+    _Pragma("unroll") for (int tb_ = 0; tb_ < 4; tb_++) {                                         \
+      H[tb_] = __builtin_amdgcn_mfma_i32_32x32x32_i8(XA[tb_], bh_, (FIRST) ? zi : H[tb_], 0, 0, 0); \
+      L[tb_] = __builtin_amdgcn_mfma_i32_32x32x32_i8(XA[tb_], bl_, (FIRST) ? zi : L[tb_], 0, 0, 0); \
+    }                                                                                             \
+  } while (0)
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  for (uint32_t s0 = 0; s0 < p.nsb; s0 += SBW_NW) {
+    const uint32_t s = s0 + wave;
+    if (s < p.nsb) {   // wave-uniform
+      const uint32_t xs_ = 8192u * s;   // eight chunks a super-block
+      uint32_t sca_, scb_;
+      q4k_scales(hdr, sca_, scb_);
+      int16v H[4], L[4];
+      int4v xa[4], xb[4];
+      SBW_LOADX(xa, xs_, 0);
+      SBW_LOADX(xb, xs_, 1);
+      SBW_STEP(w0, 0, xa, true);
+      SBW_LOADX(xa, xs_, 2);
+      SBW_STEP(w0, 1, xb, false);
+      SBW_LOADX(xb, xs_, 3);
+      SBW_STEP(w1, 2, xa, false);
+      SBW_LOADX(xa, xs_, 4);
+      SBW_STEP(w1, 3, xb, false);
+      SBW_LOADX(xb, xs_, 5);
+      SBW_STEP(w2, 4, xa, false);
+      SBW_LOADX(xa, xs_, 6);
+      SBW_STEP(w2, 5, xb, false);
+      SBW_LOADX(xb, xs_, 7);
+      SBW_STEP(w3, 6, xa, false);
+      SBW_STEP(w3, 7, xb, false);
+      const float d = gm_f16_bits_to_f32(hdr.x & 0xFFFFu);
+#pragma unroll
+      for (int tb = 0; tb < 4; tb++) {
+        const float *adp = &ad_l[s * SBW_TOK + 32u * tb + 4u * lh];
+        float *tp = terms + (wave * SBW_TOK + 32u * tb + 4u * lh) * 32u + l32;   // [wave][token][row]
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          const float4 a4 = *(const float4 *)(adp + 8 * q4);
+          const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int is_ = H[tb][4 * q4 + e] * 256 + L[tb][4 * q4 + e];
+            tp[(8 * q4 + e) * 32] = a4v[e] * (d * (float)is_);
+          }
+        }
+      }
+    }
+    SBW_LOADW(s + SBW_NW);   // the next round's weights, in flight over the barrier and the additions
+    __syncthreads();
+    if (!(SBW_ABL & 4) || s0 == 0) {
+      const uint32_t n_here = min(SBW_NW, p.nsb - s0);
+      for (uint32_t w = 0; w < n_here; w++) {   // ascending super-blocks, one accumulator per output
+#pragma unroll
+        for (uint32_t a = 0; a < NACC; a++) acc[a] += terms[w * (SBW_TOK * 32u) + a * NT + tid];
+      }
+    }
+    __syncthreads();
+  }
+#undef SBW_LOADW
+#undef SBW_LOADX
+#undef SBW_STEP
+  {
+    const uint32_t row = r0 + (tid & 31u);
+#pragma unroll
+    for (uint32_t a = 0; a < NACC; a++) {
+      const uint32_t tok_o = t0 + (tid >> 5) + a * (NT / 32u);
+      if (row < p.out_dim && tok_o < p.n_tokens) p.y[(size_t)tok_o * p.out_dim + row] = acc[a];
+    }
+  }
+}
+
 // Eight int8 activations (two dwords) -> eight f16, exact: with u = x + 128 (the sign bit flipped),
 // 0x6400 | u is the f16 1024 + u, and 1024 + u - 1152 = x.
 __device__ __forceinline__ half8 gw_i8_to_f16(uint32_t w0, uint32_t w1) {
@@ -1749,10 +1999,35 @@ static bool gemm_small_batch(const OgmGemmArgs &a) {
   // (measured, Q4_K from 4096 inputs, small-batch against tiled, us: 4096 rows at 192 / 256 / 384 tokens 36 against 45,
   // 39 against 46, 57 against 49; 6144 rows at 128 / 192: 37 against 47, 47 against 47; 14336 rows at 64 / 96: 38 against 44,
   // 51 against 46)
-  const uint32_t small_max =
-      a.small_max_tokens ? a.small_max_tokens : (tiles64_all <= 64u ? 256u : tiles64_all <= 128u ? 128u : 64u);
+  // (the last 32 tokens of the two larger limits belong to the medium-batch kernel where that runs: see gemm_medium_batch)
+  const bool med = q45 && a.medium != 1u;
+  const uint32_t small_max = a.small_max_tokens ? a.small_max_tokens
+                             : (tiles64_all <= 64u ? (med ? 224u : 256u) : tiles64_all <= 128u ? (med ? 96u : 128u) : 64u);
   return a.ggml_type != OGM_Q3_K && a.small_max_tokens != 1u && a.n_tokens <= small_max &&
          (q45 ? 16u : 8u) * 4096u + 128u * nsb <= GM_LDS_MAX;
+}
+
+// Whether a Q4_K / Q5_K launch beyond the small batches takes the medium-batch kernel (32 rows x 128 tokens per
+// workgroup, its waves on different super-blocks) instead of a tiled one.  medium: 0 by the size of the launch,
+// 1 never, 2 whenever the shape allows.
+static bool gemm_medium_batch(const OgmGemmArgs &a) {
+  const uint32_t nsb = a.in_dim / 256;
+  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
+  if (!q45 || a.medium == 1u || !a.xh || SBW_TERMS_BYTES + SBW_TOK * 4u * nsb > GM_LDS_MAX ||
+      (uint64_t)t_pad * a.in_dim >= (1ull << 32))
+    return false;
+  if (a.medium == 2u) return true;
+  // Measured on MI355X against the kernels it displaces, whole calls, us: 4096 -> 14336 at 128 tokens 42 against 50
+  // (feeding waves), at 192 / 256 tokens 78 / 77 against 65 / 65; 4096 -> 4096 at 256 tokens 35 against 39 (small
+  // batch), at 128 tokens 33 against 23; 4096 -> 6144 at 128 / 256 tokens 34 / 40 against 36 / 46; 14336 -> 4096 at
+  // 256 tokens 106 against 116.  It wants its token tiles of 128 nearly full, and at two of them matrices of at most
+  // 8192 rows (beyond, the 128-row tiles of the feeding-wave kernels outnumber the compute units' halves).
+  uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
+  for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
+  const uint32_t tok_tiles = (a.n_tokens + SBW_TOK - 1u) / SBW_TOK;
+  const bool full_enough = tok_tiles * SBW_TOK - a.n_tokens <= 32u;
+  return full_enough && (tok_tiles == 1u || (tok_tiles == 2u && tiles64_all <= 128u));
 }
 
 // Whether a tiled launch goes to the kernel whose waves all multiply, given planes.  It wants more
@@ -1867,7 +2142,45 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   }
   bool have_planes = a.planes != nullptr;
   for (uint32_t m = 0; m < a.n_extra; m++) have_planes = have_planes && a.extra_planes[m] != nullptr;   // every matrix of the launch, or none
-  if (have_planes && gemm_dma_eligible(a)) {
+  const bool dma = have_planes && gemm_dma_eligible(a);
+  if ((!dma || a.medium == 2u) && gemm_medium_batch(a)) {   // (asked for by name, it comes before the planes)
+    const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
+    if (!a.xt_ready)
+      hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3(a.in_dim / 128u, t_pad / 32u), dim3(256), 0, stream, a.act.q,
+                         (int8_t *)a.xh, a.in_dim, a.n_tokens);
+    GemmSbwParams p;
+    p.wt = a.wt;
+    p.xt = (const int8_t *)a.xh;
+    p.ad = a.act.d;
+    p.bs16 = bs16;
+    p.y = a.y;
+    p.in_dim = a.in_dim;
+    p.out_dim = a.out_dim;
+    p.n_tokens = a.n_tokens;
+    p.nsb = nsb;
+    p.c_shift = c_shift;
+    p.r_shift = 6 - c_shift;
+    p.nct = tl.nct;
+    p.n_extra = a.n_extra;
+    uint32_t tiles = (a.out_dim + 31u) / 32u;
+    for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
+      p.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
+      p.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
+      p.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
+      if (m < a.n_extra) tiles += (a.extra_out_dim[m] + 31u) / 32u;
+    }
+    const uint32_t lds_bytes = SBW_TERMS_BYTES + SBW_TOK * 4u * nsb;
+    const void *fn = a.ggml_type == OGM_Q4_K ? (const void *)ogm_gemm_sbw_q45k_kernel<false>
+                                             : (const void *)ogm_gemm_sbw_q45k_kernel<true>;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    void *kargs[] = {(void *)&p};
+    e = hipLaunchKernel(fn, dim3((a.n_tokens + SBW_TOK - 1u) / SBW_TOK, tiles), dim3(64u * SBW_NW), kargs, lds_bytes, stream);
+    if (e != hipSuccess) return e;
+    if (kernel_name) *kernel_name = a.ggml_type == OGM_Q4_K ? "ogm_gemm_sbw_q4k_kernel" : "ogm_gemm_sbw_q5k_kernel";
+    return hipGetLastError();
+  }
+  if (dma) {
     const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
     if (!a.xt_ready)
       hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3(a.in_dim / 128u, t_pad / 32u), dim3(256), 0, stream, a.act.q,

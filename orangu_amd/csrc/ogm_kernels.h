@@ -63,6 +63,7 @@ struct OgmGemmArgs {
   uint32_t tile_rows = 0;          // feeding-wave kernels: 64 forces their 64-row tiles (0 = by the size of the launch)
   uint32_t small_max_tokens = 0;   // most tokens for the small-batch kernel (0 = default 64, 1 = never)
   uint32_t sb_waves = 0;           // waves of a small-batch workgroup: 8 or 16 (0 = by the size of the launch)
+  uint32_t medium = 0;             // Q4_K / Q5_K medium-batch kernel: 0 by the size of the launch, 1 never, 2 whenever it can
   // K-quants: further matrices of the same type and in_dim over the same activations, in the same launch
   uint32_t n_extra = 0;
   const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1] = {};

@@ -42,6 +42,7 @@ def be(request):
     say("device:", b.device_name(), "mode:", request.param)
     b.set_tuning("gemm_min_tokens", GEMM_FROM)
     b.set_tuning("gemm_small_max_tokens", 1)
+    b.set_tuning("gemm_medium", 1)   # the medium-batch kernel has tests of its own below
     b.set_tuning("gemm_sb_waves", 8)
     b.set_tuning("gemm_plane_cache_mb", 0 if request.param == "unpack" else 65536)
     b.set_tuning("gemm_plane_kernel", 2)
@@ -536,12 +537,68 @@ def test_mfma_gemm_q4k_matches_cpu_gemm(be, in_dim, out_dim, T):
         tile_rows(be, 0)
 
 
+@pytest.mark.parametrize("t,in_dim,out_dim,T", [
+    (Q4_K, 256, 5, 9), (Q4_K, 1024, 200, 70), (Q4_K, 4096, 96, 128), (Q4_K, 512, 33, 129), (Q5_K, 1024, 130, 140),
+    (Q4_K, 2048, 64, 40), (Q5_K, 768, 257, 300), (Q4_K, 14336, 70, 257), (Q4_K, 8192, 100, 100), (Q5_K, 4096, 31, 128),
+])
+def test_medium_batch_kernel_matches_cpu_gemm(be, t, in_dim, out_dim, T):
+    """32 rows x 128 tokens per workgroup, its four waves on different super-blocks, the terms added in order
+    (gemm_k_q4_k, vecdot.rs:2213-2303): every bit of the CPU GEMM at ragged rows and tokens, with the operand
+    chunks written by the quantizer (from 32 tokens) or by the relayout kernel (below)."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T)
+    be.set_tuning("gemm_medium", 2)
+    try:
+        got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
+    finally:
+        be.set_tuning("gemm_medium", 1)
+    assert be.last_kernel() == ("ogm_gemm_sbw_q4k_kernel" if t == Q4_K else "ogm_gemm_sbw_q5k_kernel")
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "medium-batch gemm")
+
+
+def test_medium_batch_kernel_over_several_matrices_and_extreme_ranges(be):
+    """q / k / v in one launch (row tiles run through the matrices in turn), and the largest magnitudes the
+    integer stage can see: nibbles 15, scales and mins 63, activations +-127."""
+    from orangu_amd.hiprt import DeviceBuffer, device_synchronize
+    in_dim, T, outs = 1024, 150, (300, 130, 64)
+    raws = [synth_weights(Q4_K, in_dim, od, seed=90 + i) for i, od in enumerate(outs)]
+    hs = [be.upload_raw(r, Q4_K, in_dim, od) for r, od in zip(raws, outs)]
+    x = synth_x(T, in_dim, seed=17)
+    xd = DeviceBuffer.from_numpy(x)
+    yds = [DeviceBuffer(4 * T * od) for od in outs]
+    be.set_tuning("gemm_medium", 2)
+    try:
+        be.matmul_multi_dev(hs, xd.ptr, T, [y.ptr for y in yds])
+        device_synchronize()
+        assert be.last_kernel() == "ogm_gemm_sbw_q4k_kernel"
+        for r, od, yd in zip(raws, outs, yds):
+            assert_bits(yd.to_numpy(np.float32, T * od), oracle.matmul(Q4_K, r, in_dim, od, x, T), f"{od} rows of {outs}")
+        blocks = np.zeros((32 * 4, 144), np.uint8)
+        blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+        blocks[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
+        blocks[:, 4:16] = 0xFF
+        blocks[:, 16:] = 0xFF
+        xe = np.full((100, 1024), 127.0, np.float32)
+        xe[1::2] *= -1
+        xe[:, ::7] = 126.0
+        got = be.matmul(xe, 100, qm(blocks.reshape(-1), Q4_K, 1024, 32))
+        assert be.last_kernel() == "ogm_gemm_sbw_q4k_kernel"
+        assert_bits(got, oracle.matmul(Q4_K, blocks.reshape(-1), 1024, 32, xe, 100), "extreme ranges")
+    finally:
+        be.set_tuning("gemm_medium", 1)
+        for h in hs:
+            be.free_weight(h)
+        for b in [xd] + yds:
+            b.free()
+
+
 def test_gemm_threshold_default():
     """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
-    float order, 17 through the matrix-core GEMM.  Q4_K: 5 tokens through the GEMV kernel, 6 to 256
-    through the small-batch kernel (a matrix of few rows), 257 through the tiled one; a matrix of
-    many rows leaves the small-batch kernel after 64 tokens, and one of so many that 128 x 128 tiles
-    outnumber the compute units has its planes built and read by the kernel whose waves all multiply.
+    float order, 17 through the matrix-core GEMM.  Q4_K: 5 tokens through the GEMV kernel, 6 to 224
+    through the small-batch kernel (a matrix of few rows), 225 to 256 through the medium-batch kernel, 257
+    through the tiled one; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
+    many that 128 x 128 tiles outnumber the compute units has its planes built and read by the kernel whose
+    waves all multiply, while a single nearly full token tile goes to the medium-batch kernel.
     Same bits everywhere."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
@@ -559,9 +616,10 @@ def test_gemm_threshold_default():
         raw = synth_weights(Q4_K, 1024, 70, seed=5)
         w = qm(raw, Q4_K, 1024, 70)
         want = oracle.matmul(Q4_K, raw, 1024, 70, x, 257).reshape(257, 70)
-        # (up to 64 tiles of 64 rows the small-batch kernel keeps batches of up to 256 tokens)
+        # (up to 64 tiles of 64 rows the small-batch kernel keeps batches of up to 224 tokens)
         for n, kernel in ((5, "ogm_gemv_kernel"), (6, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
-                          (256, "ogm_gemm_sb_q4k_kernel"), (257, "ogm_gemm_q4k_i8p_r64_kernel")):
+                          (224, "ogm_gemm_sb_q4k_kernel"), (225, "ogm_gemm_sbw_q4k_kernel"),
+                          (256, "ogm_gemm_sbw_q4k_kernel"), (257, "ogm_gemm_q4k_i8p_r64_kernel")):
             y = b.matmul(x[:n], n, w)
             assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, want[:n], f"Q4_K, {n} tokens")
@@ -583,7 +641,10 @@ def test_gemm_threshold_default():
         y = b.matmul(x5, 129, w)
         assert b.last_kernel() == "ogm_gemm_q4k_dma_kernel"
         assert_bits(y, oracle.matmul(Q4_K, raw, 256, 16600, x5, 129), "Q4_K, 129 tokens x 16600 rows")
-        y = b.matmul(x5[:128], 128, w)                   # one token tile: 130 workgroups
+        y = b.matmul(x5[:128], 128, w)                   # one full token tile: the medium-batch kernel
+        assert b.last_kernel() == "ogm_gemm_sbw_q4k_kernel"
+        assert_bits(y, oracle.matmul(Q4_K, raw, 256, 16600, x5[:128], 128), "Q4_K, 128 tokens x 16600 rows")
+        y = b.matmul(x5[:90], 90, w)                     # a token tile a third empty: 130 workgroups of 128 rows
         assert b.last_kernel() == "ogm_gemm_q4k_i8p_kernel"
     finally:
         b.close()
