@@ -185,6 +185,9 @@ def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
         run(Q6_K, 4096, 128256, T, False, f"C3 vocab batch {T}", n=64)
         run(Q4_K, 4096, 4096, T, False, f"C3 q/o batch {T}")
         run(Q4_K, 4096, 1024, T, False, f"C3 k/v batch {T}")
+        if T > 1:   # the other two projections of a verify batch (their single-token rows are C2 and C5)
+            run(Q4_K, HIDDEN, FFN, T, False, f"C3 gate/up batch {T}")
+            run(Q6_K, FFN, HIDDEN, T, False, f"C3 ffn_down batch {T}")
     for T in (128, 512, 2048):
         run(Q4_K, HIDDEN, FFN, T, False, f"C4 prefill GEMM M={T}", n=64)
     run(Q6_K, FFN, HIDDEN, 1, False, "C5 ffn_down GEMV")
@@ -195,7 +198,7 @@ def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
 
 
 def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool, only_prefill: int = 0,
-               with_prefill: bool = True) -> dict:
+               with_prefill: bool = True, only_verify: int = 0) -> dict:
     """Batch-1 decode of an 8B-shaped Llama (32 layers: wq, wo 4096x4096, wk, wv 4096->1024, gate, up
     4096->14336 in Q4_K; down 14336->4096 and the 128256-row output in Q6_K; f16 KV cache holding `ctx`
     random positions): tokens per second of ogm_llama_decode_dev with the embedding row, the logits and
@@ -227,7 +230,7 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     layers = [{**{k: (k, l) for k in shapes}, "attn_norm": norms[2 * l], "ffn_norm": norms[2 * l + 1]}
               for l in range(n_layer)]
     dec = LlamaDecoder(be, n_embd=n_embd, n_head=n_head, n_head_kv=n_kv, head_dim=hd, n_ff=n_ff, n_vocab=n_vocab,
-                       max_ctx=ctx + warmup + 2 * steps + 2, rms_eps=1e-5, rope_freq_base=500000.0, layers=layers,
+                       max_ctx=ctx + max(16, warmup + 2 * steps + 2), rms_eps=1e-5, rope_freq_base=500000.0, layers=layers,
                        output_norm=norms[-1], output="output", upload=up)
     kvs = []
     for l in range(n_layer):
@@ -248,6 +251,18 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
             be.free_weight(h)
         return {"workload": f"configs[4] model, prefill of {only_prefill} tokens from an empty cache",
                 "prefill_ms": round(dt_pre * 1e3, 2), "prefill_tok_per_s": round(only_prefill / dt_pre, 1)}
+    if only_verify:    # for profiles: nothing but verify batches of this size appended at position `ctx`
+        xv = rng.standard_normal((only_verify, n_embd)).astype(np.float32)
+        dec.prefill(xv, ctx)
+        t0 = time.perf_counter()
+        for _ in range(10):
+            dec.prefill(xv, ctx)
+        dt_v = (time.perf_counter() - t0) / 10
+        dec.close()
+        for h in mats.values():
+            be.free_weight(h)
+        return {"workload": f"configs[4] model, verify batch of {only_verify} tokens at context {ctx}",
+                "ms": round(dt_v * 1e3, 3), "tokens_verified_per_s": round(only_verify / dt_v, 1)}
     x_h = rng.standard_normal(n_embd).astype(np.float32)
     x_d = hiprt.DeviceBuffer.from_numpy(x_h)
     tok_d = hiprt.DeviceBuffer(4)
@@ -271,6 +286,20 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     toks = dec.generate(up("output"), 1, pos, steps)
     dt_gen = (time.perf_counter() - t0) / steps
     pos += steps
+    # speculative-decode verify (generate.rs:1618-1674): the last accepted token plus a draft of 3 or 7 go
+    # through the whole model as one batch appended at position `ctx`, host embedding rows in, the last
+    # token's logits out (ogm_llama_prefill); wall clock per call, the first call of a size untimed
+    verify = {}
+    for n_v in (4, 8):
+        xv = rng.standard_normal((n_v, n_embd)).astype(np.float32)
+        dec.prefill(xv, ctx)
+        reps_v = max(3, min(20, steps // 10))
+        t0 = time.perf_counter()
+        for _ in range(reps_v):
+            dec.prefill(xv, ctx)
+        dt_v = (time.perf_counter() - t0) / reps_v
+        verify[f"verify_batch_{n_v}"] = {"ms": round(dt_v * 1e3, 3), "tokens_verified_per_s": round(n_v / dt_v, 1),
+                                         "calls": reps_v}
     # prefill of a 512-token prompt from position 0 (GEMM matmuls, batch attention); the first
     # call allocates the batch buffers
     dt_pre = dt_pre_long = dt_pre_long_one = None
@@ -307,6 +336,7 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
            "prefill_2048_ms": round(dt_pre_long * 1e3, 2) if dt_pre_long else None,
            "prefill_2048_tok_per_s": round(2048 / dt_pre_long, 1) if dt_pre_long else None,
            "prefill_2048_ms_one_pass_option": round(dt_pre_long_one * 1e3, 2) if dt_pre_long_one else None,
+           **verify,
            "bytes_per_token": weights + kv_bytes,
            "GBps": round((weights + kv_bytes) / dt / 1e9, 1),
            "frac_of_hbm_peak": round((weights + kv_bytes) / dt / 1e9 / HBM_PEAK_GBS, 4)}
@@ -407,6 +437,8 @@ def main() -> int:
                     help="tokens of the 8B-shaped decode leg (config 5); 0 skips it")
     ap.add_argument("--decode-ctx", type=int, default=2048, help="cached positions of the decode leg")
     ap.add_argument("--only-decode", action="store_true", help="run only the decode leg (for rocprofv3)")
+    ap.add_argument("--only-verify", type=int, default=0, metavar="N",
+                    help="run only verify batches of N tokens at the decode context (for rocprofv3)")
     ap.add_argument("--only-prefill", type=int, default=0, metavar="N",
                     help="run only prefills of N tokens on the decode leg's model (for rocprofv3)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
@@ -458,6 +490,10 @@ def main() -> int:
     if args.only_prefill:
         print(json.dumps(decode_leg(be, helpers, hiprt, 1, 0, max(args.decode_ctx, args.only_prefill), False,
                                     only_prefill=args.only_prefill)))
+        be.close()
+        return 0
+    if args.only_verify:
+        print(json.dumps(decode_leg(be, helpers, hiprt, 1, 0, args.decode_ctx, False, only_verify=args.only_verify)))
         be.close()
         return 0
     if args.only_decode:

@@ -420,8 +420,14 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              vecdot.rs:3152-3178.  The integer sums are the same; the f32 result is within
  *                              rounding of the reference GEMM's, not its bits: an output whose terms cancel to
  *                              near zero can differ from the reference's by more than 1e-3 of itself
- *   "attn_prefill_variant"     attention of a prefill batch: 0 = default, the matrix-core kernel; 1 = the decode
- *                              step's kernel per token and chunk of the cache; they agree to f32 rounding
+ *   "gemv_mma"                 2 to 16 tokens over Q4_K / Q5_K / Q6_K rows of a multiple of 1024 inputs on the kernel
+ *                              that gives a workgroup one row block and multiplies on the matrix cores: 1 =
+ *                              default, where it measured faster (Q6_K from two tokens, Q4_K / Q5_K from five);
+ *                              2 = wherever it can; 0 = never.  Same bits as the other kernels
+ *   "attn_prefill_variant"     attention of a prefill batch: 1 = the decode step's kernel per token and chunk of
+ *                              the cache; 2 = the matrix-core kernel; 0 = default: the first for batches of up to
+ *                              48 tokens (speculative-decode verify batches), the second above; they agree to
+ *                              f32 rounding
  *   "prefill_chunk_tokens"     tokens per pass of ogm_llama_prefill over the layers, default 2048; a model keeps
  *                              the value of its first prefill, whose row buffers are allocated for it
  *   "host_zero_copy"           1 = default: a host-pointer call (ogm_matmul, ogm_matmul_decode,

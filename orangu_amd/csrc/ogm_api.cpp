@@ -67,10 +67,11 @@ struct ogm_ctx {
   int tune_host_flag_wait = 1;         // zero-copy host calls wait on a word a trailing kernel stores to pinned memory instead of on the stream
   int tune_host_zero_copy = 1;         // host-pointer calls of up to OGM_ZERO_COPY_MAX bytes: kernels read x / write y in pinned host memory
   bool host_coherent = true;           // the pinned staging buffers are fine-grained (asked for by name); false once the runtime has refused
+  int tune_gemv_mma = 1;               // few tokens over Q4_K / Q5_K / Q6_K on the row-block matrix-core kernel: 0 never, 1 where it measured faster, 2 wherever it can
   int tune_gemm_plane_kernel = 0;      // the all-waves-multiply kernel over planes: 0 on large grids, 2 whatever the grid
   int tune_gemm_one_pass = 0;          // 1: Q4_K / Q5_K on that kernel fold the min pass into the super-block step (f32 to rounding, not to the bit)
   int tune_prefill_chunk = 2048;       // tokens per prefill pass over the layers (fixed per model at its first prefill)
-  int tune_attn_prefill_variant = 0;   // 0: matrix-core kernel; 1: the decode kernel per token and chunk
+  int tune_attn_prefill_variant = 0;   // 0: by batch size; 1: the decode kernel per token and chunk; 2: the matrix-core kernel
   // Device memory the prefill planes of all weights may take, in MiB; 0 (the default) = build none.
   // A model's planes are 3.3 times its Q4_K bytes.
   int tune_plane_cache_mb = 32768;   // MiB the K-quant matrices' prefill planes may take in all
@@ -330,8 +331,13 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_prefill_chunk = value;
     return OGM_OK;
   }
+  if (strcmp(key, "gemv_mma") == 0) {
+    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemv_mma must be 0, 1 or 2");
+    ctx->tune_gemv_mma = value;
+    return OGM_OK;
+  }
   if (strcmp(key, "attn_prefill_variant") == 0) {
-    if (value < 0 || value > 1) return fail(ctx, OGM_ERR_INVALID, "attn_prefill_variant must be 0 or 1");
+    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "attn_prefill_variant must be 0, 1 or 2");
     ctx->tune_attn_prefill_variant = value;
     return OGM_OK;
   }
@@ -589,6 +595,38 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       }
       return OGM_OK;
     }
+  }
+  // Two to sixteen tokens over a K-quant matrix (a speculative-decode verify batch, a decode batch): the GEMV's
+  // distribution with the products on the matrix cores, in either float order.
+  // Measured at the 8B shapes (4096 -> 1024 / 4096 / 14336 Q4_K, 14336 -> 4096 Q6_K): Q6_K from two tokens on
+  // (4 tokens: 18 us against 30), Q4_K / Q5_K from five (up to four the GEMV kernel's per-token dot instructions
+  // are level or ahead: 13 us against 15 at 14336 rows; at eight 16 against 17.5 for the small-batch GEMM).
+  const uint32_t mma_from = ctx->tune_gemv_mma == 2 ? 2u : t0 == OGM_Q6_K ? 2u : 5u;
+  if (ctx->tune_gemv_mma != 0 && n_tokens >= mma_from && !dump_isum && !dump_imin && !act_base &&
+      ogm_gemv_mma_eligible(w0->ggml_type, w0->in_dim, n_tokens, gemm_order)) {
+    for (size_t g0 = 0; g0 < n_tg; g0 += OGM_GEMV_MAX_MATS) {
+      const size_t ng = n_tg - g0 < OGM_GEMV_MAX_MATS ? n_tg - g0 : OGM_GEMV_MAX_MATS;
+      OgmGemvArgs a;
+      a.ggml_type = w0->ggml_type;
+      a.wt = tg[g0].w->dev;
+      a.in_dim = w0->in_dim;
+      a.out_dim = tg[g0].w->out_dim;
+      a.act = act_view(ctx, w0->in_dim, mode, 0);
+      a.n_tokens = n_tokens;
+      a.y = tg[g0].y;
+      a.gemm_order = gemm_order;
+      a.wg_waves = (uint32_t)ctx->tune_wg_waves;
+      a.dump_isum = nullptr;
+      a.dump_imin = nullptr;
+      a.n_extra = (uint32_t)ng - 1;
+      for (size_t i = 1; i < ng; i++) {
+        a.extra_wt[i - 1] = tg[g0 + i].w->dev;
+        a.extra_out_dim[i - 1] = tg[g0 + i].w->out_dim;
+        a.extra_y[i - 1] = tg[g0 + i].y;
+      }
+      HIPCHK(ctx, ogm_launch_gemv_mma(a, stream, &ctx->last_kernel));
+    }
+    return OGM_OK;
   }
   if (gemm_order && !dump_isum && !dump_imin && !act_base && n_tokens >= gemm_from &&
       all_gemm_supported(tg, n_tg, n_tokens)) {
@@ -1673,6 +1711,7 @@ extern "C" int ogm_llama_generate(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
 // ---- prefill: run_layers at n_tokens > 1 (llama.rs:594-932) ------------------------------------
 
 static const size_t OGM_PREFILL_PART_BYTES = 256u << 20;   // attention partials per launch
+static const uint32_t OGM_ATTN_PER_TOKEN_MAX = 48;         // batches up to this take the per-token attention kernel
 
 static int llama_prefill_buffers(ogm_ctx *ctx, ogm_llama *m) {
   if (m->pf.ready) return OGM_OK;
@@ -1705,6 +1744,7 @@ static int llama_prefill_partials(ogm_ctx *ctx, ogm_llama *m) {
   size_t at = OGM_PREFILL_PART_BYTES / per_token;
   if (at < 1) at = 1;
   if (at > m->pf.chunk) at = m->pf.chunk;
+  if (ctx->tune_attn_prefill_variant == 0 && at > 64) at = 64;   // only small batches come here
   int rc = llama_alloc(ctx, m, (void **)&m->pf.part_o, at * per_token);
   if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)&m->pf.part_ml, at * (size_t)c.n_head * m->max_splits * 2 * 4);
   if (rc != OGM_OK) return rc;
@@ -1791,6 +1831,15 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
   const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
   const float scale = 1.0f / sqrtf((float)c.head_dim);
   HIPCHK(ctx, ogm_launch_rope_table(m->freq, pos0, T, c.rope_dim, P.cs, s));
+  // The matrix-core attention kernel gives a workgroup 32 query tokens of four heads and the whole cache to walk: a
+  // verify batch of a few tokens on a long cache leaves it sixteen workgroups (8B shapes, 4 tokens at 2048
+  // positions: 79 us a layer).  The decode kernel over (K/V head, chunk of 128 positions, token) spreads the same
+  // work over the device and measures faster up to 64 tokens at 512, 2048 and 8192 cached positions.
+  const bool per_token = ctx->tune_attn_prefill_variant == 1 || (ctx->tune_attn_prefill_variant == 0 && T <= OGM_ATTN_PER_TOKEN_MAX);
+  if (per_token) {
+    const int rc = llama_prefill_partials(ctx, m);
+    if (rc != OGM_OK) return rc;
+  }
   const float *delta = nullptr;
   for (uint32_t l = 0; l < c.n_layer; l++) {
     const ogm_llama_layer &L = m->layers[l];
@@ -1804,11 +1853,10 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_qkv_pre(P.q, P.k, P.v, P.cs, c.rope_dim, pre, c.n_head, c.n_head_kv, c.head_dim, kc, vc,
                                    pos0, T, s));
-    if (ctx->tune_attn_prefill_variant == 0) {
+    if (!per_token) {
       HIPCHK(ctx, ogm_launch_attn_prefill_mfma(P.q, kc, vc, pos0, T, c.n_head, c.n_head_kv, c.head_dim, scale, P.attn, s));
     }
-    if (ctx->tune_attn_prefill_variant != 0 && (rc = llama_prefill_partials(ctx, m)) != OGM_OK) return rc;
-    for (uint32_t t0 = 0; ctx->tune_attn_prefill_variant != 0 && t0 < T; t0 += P.attn_tokens) {
+    for (uint32_t t0 = 0; per_token && t0 < T; t0 += P.attn_tokens) {
       const uint32_t nt = T - t0 < P.attn_tokens ? T - t0 : P.attn_tokens;
       HIPCHK(ctx, ogm_launch_attn_prefill(P.q + (size_t)t0 * qd, kc, vc, pos0 + t0, nt, m->max_splits, c.n_head,
                                           c.n_head_kv, c.head_dim, scale, P.part_o, P.part_ml,

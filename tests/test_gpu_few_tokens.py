@@ -1,26 +1,26 @@
-"""The kernel that takes 2 to 16 tokens over a Q6_K matrix of many rows in one streaming pass on the matrix
-cores (`ogm_gemm_ft_q6k_kernel`): bit for bit against the CPU restatement in both float orders -- matmul of
-several tokens (gemm_k_q6_k, vecdot.rs:2352-2398) and decode batches (dot_k_row_q6_k per token,
-vecdot.rs:3215-3241, cpu.rs:265-317) -- at ragged row counts, every token count, the extremes of the integer
-range, through grouped calls, and at the vocabulary projection's full size where it is the default."""
+"""GPU parity of the few-token kernel that gives a workgroup one row block of 16 rows (2 to 16 tokens over Q4_K,
+Q5_K and Q6_K: the projections of a speculative-decode verify batch, generate.rs:1618-1674, and of a decode
+batch, cpu.rs:265-317), through the C ABI against the CPU oracle: every bit of the f32 outputs, in the GEMM's
+float order (Backend::matmul at n_tokens > 1) and in the decode dot's (matmul_decode)."""
+import sys
+
 import numpy as np
 import pytest
 
 import oracle
-from helpers import Q4_K, Q6_K, activations_t, pin_scales, pseudo_bytes_fast, row_bytes, synth_weights, synth_x
+from helpers import Q4_K, Q5_K, Q6_K, synth_weights, synth_x
 
 pytestmark = pytest.mark.gpu
 
-
-def say(*a):
-    print(*a, flush=True)
+NAME = {Q4_K: "ogm_gemm_fk_kernel<Q4_K>", Q5_K: "ogm_gemm_fk_kernel<Q5_K>", Q6_K: "ogm_gemm_fk_kernel<Q6_K>"}
 
 
 @pytest.fixture(scope="module")
 def be():
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()  # raises if the HIP library or the device is missing: no fallback
-    b.set_tuning("gemm_few_tokens_min_rows", 1)   # whatever the row count
+    b.set_tuning("gemm_few_tokens_min_rows", -1)   # keep the many-rows few-token kernel out: this module is about the other one
+    b.set_tuning("gemv_mma", 2)                    # from two tokens on for every type (the default leaves Q4_K / Q5_K up to four tokens to the GEMV kernel)
     yield b
     b.close()
 
@@ -38,113 +38,116 @@ def assert_bits(got, want, what):
                        f"{np.nonzero(~same)[0][:5]} got {got[~same][:5]} want {want[~same][:5]}"
 
 
-def kernel_for(T):
-    return "ogm_gemm_ft_q6k_kernel" if T <= 8 else "ogm_gemm_ft_q6k_t16_kernel"
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("in_dim,out_dim", [(1024, 40), (2048, 16), (4096, 257), (3072, 100), (14336, 50)])
+@pytest.mark.parametrize("T", [2, 3, 4, 5, 8, 9, 13, 16])
+def test_row_block_kernel_matches_cpu_gemm(be, t, in_dim, out_dim, T):
+    """One, three, four and fourteen column tiles a row block (waves with one tile, and with several); row
+    blocks that end beyond the matrix; every token count of both slot widths."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T)
+    got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
+    if in_dim == 14336 and (T > 8 or t != Q6_K):
+        assert not be.last_kernel().startswith("ogm_gemm_fk"), "activations and terms beyond a workgroup's LDS"
+    else:
+        assert be.last_kernel() == NAME[t]
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), f"type {t} {in_dim}->{out_dim} at {T} tokens")
 
 
-@pytest.mark.parametrize("in_dim,out_dim", [(1024, 1), (1024, 31), (1024, 129), (2048, 300), (4096, 530), (14336, 70)])
-@pytest.mark.parametrize("T", [2, 3, 4, 5, 7, 8, 9, 12, 16])
-def test_both_float_orders_are_bit_exact(be, in_dim, out_dim, T):
-    raw = synth_weights(Q6_K, in_dim, out_dim, seed=in_dim + out_dim + T)
-    x = synth_x(T, in_dim, seed=T + 11)
-    w = qm(raw, Q6_K, in_dim, out_dim)
-    say("few tokens", in_dim, out_dim, T)
-    fits = in_dim * (8 if T <= 8 else 16) <= 150 * 1024
-    got = be.matmul(x, T, w)
-    assert (be.last_kernel() == kernel_for(T)) == fits, be.last_kernel()
-    assert_bits(got, oracle.matmul(Q6_K, raw, in_dim, out_dim, x, T), "matmul")
-    got = be.matmul_decode(x, T, w)
-    assert (be.last_kernel() == kernel_for(T)) == fits, be.last_kernel()
-    assert_bits(got, oracle.matmul_decode(Q6_K, raw, in_dim, out_dim, x, T), "decode batch")
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("T", [2, 4, 7, 8, 12])
+def test_row_block_kernel_in_the_decode_dots_order(be, t, T):
+    """matmul_decode over a batch (cpu.rs:265-317): every token's row equals the single-token GEMV's."""
+    in_dim, out_dim = 2048, 75
+    raw = synth_weights(t, in_dim, out_dim, seed=31 + T)
+    x = synth_x(T, in_dim, seed=T + 100)
+    w = qm(raw, t, in_dim, out_dim)
+    got = be.matmul_decode(x, T, w).reshape(T, out_dim)
+    assert be.last_kernel() == NAME[t]
+    want = oracle.matmul_decode(t, raw, in_dim, out_dim, x, T).reshape(T, out_dim)
+    assert_bits(got, want, f"type {t} decode order at {T} tokens")
+    for i in range(T):
+        assert_bits(be.matmul(x[i:i + 1], 1, w), want[i], f"token {i} alone")
 
 
-@pytest.mark.parametrize("T", [2, 8, 16])
-def test_extreme_integer_sums_are_exact(be, T):
-    """Every weight at one end of its range under the largest scales, every activation at +-127: the
-    per-group products reach 16 * 127 * 32 and a super-block's sum 1.3e8."""
-    in_dim, out_dim = 2048, 96
-    for fill, scale in ((0xFF, 0x7F), (0x00, 0x80), (0xFF, 0x80)):
-        blk = np.zeros(210, np.uint8)
-        blk[:192] = fill
-        blk[192:208] = scale
-        blk[208:210] = np.frombuffer(np.float16(0.001).tobytes(), np.uint8)
-        raw = np.tile(blk, (in_dim // 256) * out_dim)
-        w = qm(raw, Q6_K, in_dim, out_dim)
-        for sign in (1.0, -1.0):
-            x = np.full(T * in_dim, sign * 3.0, np.float32)
+def test_row_block_kernel_over_several_matrices(be):
+    """q / k / v over one input in one launch: the grid runs through the matrices' row blocks in turn."""
+    from orangu_amd.hiprt import DeviceBuffer, device_synchronize
+    in_dim, T, outs = 1024, 6, (300, 130, 64, 17)
+    raws = [synth_weights(Q4_K, in_dim, od, seed=190 + i) for i, od in enumerate(outs)]
+    hs = [be.upload_raw(r, Q4_K, in_dim, od) for r, od in zip(raws, outs)]
+    x = synth_x(T, in_dim, seed=18)
+    xd = DeviceBuffer.from_numpy(x)
+    yds = [DeviceBuffer(4 * T * od) for od in outs]
+    try:
+        be.matmul_multi_dev(hs, xd.ptr, T, [y.ptr for y in yds])
+        device_synchronize()
+        assert be.last_kernel() == NAME[Q4_K]
+        for r, od, yd in zip(raws, outs, yds):
+            assert_bits(yd.to_numpy(np.float32, T * od), oracle.matmul(Q4_K, r, in_dim, od, x, T), f"{od} rows of {outs}")
+    finally:
+        for h in hs:
+            be.free_weight(h)
+        xd.free()
+        for y in yds:
+            y.free()
+
+
+@pytest.mark.parametrize("sign", [1, -1])
+def test_row_block_kernel_extreme_integer_ranges(be, sign):
+    """The largest magnitudes the integer stage can see: Q4_K nibbles 15 with scales and mins 63, Q5_K with the
+    fifth bits set, Q6_K quants 63 (and 0: -32) under scales of +-127 and -128, activations +-127."""
+    T, in_dim, rows = 8, 1024, 32
+    xe = np.full((T, in_dim), 127.0 * sign, np.float32)
+    xe[1::2] *= -1
+    xe[:, ::7] = 126.0
+    b4 = np.zeros((rows * 4, 144), np.uint8)
+    b4[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    b4[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
+    b4[:, 4:] = 0xFF
+    b5 = np.zeros((rows * 4, 176), np.uint8)
+    b5[:, 0:4] = b4[:, 0:4]
+    b5[:, 4:] = 0xFF
+    for t, blocks in ((Q4_K, b4), (Q5_K, b5)):
+        got = be.matmul(xe, T, qm(blocks.reshape(-1), t, in_dim, rows))
+        assert be.last_kernel() == NAME[t]
+        assert_bits(got, oracle.matmul(t, blocks.reshape(-1), in_dim, rows, xe, T), f"type {t} extreme ranges")
+    for ql, qh, sc in ((0xFF, 0xFF, 127), (0x00, 0x00, 127), (0xFF, 0xFF, 0x80), (0x00, 0x00, 0x80), (0xF0, 0x33, 0x81)):
+        b6 = np.zeros((rows * 4, 210), np.uint8)
+        b6[:, 0:128] = ql
+        b6[:, 128:192] = qh
+        b6[:, 192:208] = sc
+        b6[:, 208:210] = np.frombuffer(np.float16(0.003).tobytes(), np.uint8)
+        got = be.matmul(xe, T, qm(b6.reshape(-1), Q6_K, in_dim, rows))
+        assert be.last_kernel() == NAME[Q6_K]
+        assert_bits(got, oracle.matmul(Q6_K, b6.reshape(-1), in_dim, rows, xe, T), f"Q6_K ql {ql:#x} qh {qh:#x} sc {sc:#x}")
+
+
+def test_row_block_kernel_at_the_8b_shapes(be):
+    """The four projections of an 8B-shaped layer at verify batches of 4 and 8."""
+    for t, in_dim, out_dim in ((Q4_K, 4096, 4096), (Q4_K, 4096, 1024), (Q4_K, 4096, 14336), (Q6_K, 14336, 4096)):
+        raw = synth_weights(t, in_dim, out_dim, seed=5)
+        w = qm(raw, t, in_dim, out_dim)
+        for T in (4, 8):
+            x = synth_x(T, in_dim, seed=T)
             got = be.matmul(x, T, w)
-            assert be.last_kernel() == kernel_for(T)
-            assert_bits(got, oracle.matmul(Q6_K, raw, in_dim, out_dim, x, T), f"extreme {fill:#x} {scale:#x} {sign}")
-            isum, _ = be.dump_block_sums(x[:in_dim], 1, w)
-            assert np.abs(isum).max() >= 16 * 16 * 127 * 31 * 127
+            assert be.last_kernel() == NAME[t]
+            assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), f"type {t} {in_dim}->{out_dim} at {T} tokens")
+        be.evict(w)
 
 
-def test_random_bytes_and_special_activations(be):
-    """Weights of arbitrary bytes (scales pinned finite) and activations with a row of zeros, a row of denormals and a NaN."""
-    in_dim, out_dim, T = 1024, 200, 6
-    raw = pin_scales(pseudo_bytes_fast(row_bytes(Q6_K, in_dim) * out_dim, 77), Q6_K)
-    x = np.concatenate([activations_t(in_dim, k) for k in range(T)])
-    x[in_dim:2 * in_dim] = 0.0
-    x[2 * in_dim:3 * in_dim] = np.float32(1e-42)
-    x[3 * in_dim + 5] = np.nan   # quantizes to 0 and leaves the row's scale alone (vecdot.rs:3030-3053)
-    w = qm(raw, Q6_K, in_dim, out_dim)
-    for fn, ref in ((be.matmul, oracle.matmul), (be.matmul_decode, oracle.matmul_decode)):
-        got = fn(x, T, w)
-        assert be.last_kernel() == kernel_for(T)
-        assert_bits(got, ref(Q6_K, raw, in_dim, out_dim, x, T), fn.__name__)
-
-
-def test_grouped_calls_and_other_types_keep_their_kernels(be):
-    """matmul_batch over Q6_K matrices that share their input launches the kernel once per matrix; a Q4_K matrix
-    and a single token stay where they were."""
-    from orangu_amd import MatmulOp
-    in_dim, T = 1024, 4
-    x = synth_x(T, in_dim, seed=5)
-    raws = [synth_weights(Q6_K, in_dim, o, seed=o) for o in (40, 129)]
-    ws = [qm(r, Q6_K, in_dim, o) for r, o in zip(raws, (40, 129))]
-    ys = be.matmul_batch([MatmulOp(x, T, w) for w in ws])
-    assert be.last_kernel() == kernel_for(T)
-    for y, r, o in zip(ys, raws, (40, 129)):
-        assert_bits(y, oracle.matmul(Q6_K, r, in_dim, o, x, T), f"grouped {o}")
-    raw4 = synth_weights(Q4_K, in_dim, 64, seed=9)
-    be.matmul(x, T, qm(raw4, Q4_K, in_dim, 64))
-    assert not be.last_kernel().startswith("ogm_gemm_ft")
-    be.matmul(np.asarray(x).reshape(-1)[:in_dim], 1, ws[0])
-    assert not be.last_kernel().startswith("ogm_gemm_ft")
-
-
-def test_default_routing_takes_it_for_the_vocabulary_projection_only():
-    """Without the tuning key: 4096 -> 128256 and 4096 -> 32000 at 3 to 16 tokens run the kernel, two tokens and
-    4096 -> 14336 do not; and the full-size results are bit-exact in both orders (checked on a sample of rows against the oracle over the same
-    rows as a smaller matrix -- a row's result does not depend on the others)."""
+def test_default_routing_of_few_token_batches():
+    """Without tuning: Q6_K goes to the row-block kernel from two tokens, Q4_K from five; one token never."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
     try:
-        in_dim, out_dim = 4096, 128256
-        raw = synth_weights(Q6_K, in_dim, out_dim, seed=3)
-        w = qm(raw, Q6_K, in_dim, out_dim)
-        rb = row_bytes(Q6_K, in_dim)
-        rows = np.r_[0:40, 64000:64040, out_dim - 40:out_dim]
-        sub = np.ascontiguousarray(raw.reshape(out_dim, rb)[rows]).reshape(-1)
-        for T in (2, 3, 4, 8, 16):
-            x = synth_x(T, in_dim, seed=T)
-            say("vocabulary projection", T)
-            got = b.matmul(x, T, w).reshape(T, out_dim)
-            assert (b.last_kernel() == kernel_for(T)) == (T >= 3), b.last_kernel()
-            assert_bits(got[:, rows], oracle.matmul(Q6_K, sub, in_dim, len(rows), x, T), f"matmul {T}")
-            got = b.matmul_decode(x, T, w).reshape(T, out_dim)
-            assert (b.last_kernel() == kernel_for(T)) == (T >= 3), b.last_kernel()
-            assert_bits(got[:, rows], oracle.matmul_decode(Q6_K, sub, in_dim, len(rows), x, T), f"decode {T}")
-        w32 = qm(raw[:rb * 32000], Q6_K, in_dim, 32000)
-        x = synth_x(4, in_dim, seed=2)
-        got = b.matmul(x, 4, w32)
-        assert b.last_kernel() == kernel_for(4), b.last_kernel()
-        assert_bits(np.asarray(got).reshape(4, 32000)[:, :40], oracle.matmul(Q6_K, sub[:rb * 40], in_dim, 40, x, 4), "32000 rows")
-        small = qm(synth_weights(Q6_K, 4096, 14336, seed=4), Q6_K, 4096, 14336)
-        b.matmul(synth_x(4, 4096, seed=1), 4, small)
-        assert not b.last_kernel().startswith("ogm_gemm_ft"), b.last_kernel()
-        b.set_tuning("gemm_few_tokens_min_rows", -1)
-        b.matmul(synth_x(4, in_dim, seed=1), 4, w)
-        assert not b.last_kernel().startswith("ogm_gemm_ft"), b.last_kernel()
+        for t, T, want in ((Q6_K, 1, "ogm_gemv_kernel<FmtQ6K,gemv>"), (Q6_K, 2, NAME[Q6_K]), (Q6_K, 8, NAME[Q6_K]), (Q6_K, 16, NAME[Q6_K]),
+                           (Q4_K, 4, "ogm_gemv_kernel<FmtQ4K,gemm>"), (Q4_K, 5, NAME[Q4_K]), (Q4_K, 16, NAME[Q4_K]),
+                           (Q5_K, 3, "ogm_gemv_kernel<FmtQ5K,gemm>"), (Q5_K, 9, NAME[Q5_K])):
+            raw = synth_weights(t, 1024, 48, seed=T)
+            x = synth_x(T, 1024, seed=T)
+            got = b.matmul(x, T, qm(raw, t, 1024, 48))
+            assert b.last_kernel() == want, (t, T, b.last_kernel())
+            assert_bits(got, oracle.matmul(t, raw, 1024, 48, x, T), f"type {t} at {T} tokens")
     finally:
         b.close()

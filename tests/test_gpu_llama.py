@@ -14,6 +14,7 @@ activation it is about to quantize against the device's int8 values and scales (
 unit on a few elements, scales to 1e-5), and continues from the device's.  What is compared at the
 end is then the arithmetic between those points, free of the two amplifiers."""
 import sys
+from contextlib import contextmanager
 
 import numpy as np
 import pytest
@@ -240,12 +241,12 @@ def test_decode_at_contexts_whose_chunks_merge_in_several_rounds(be, hd, group, 
         dev.close()
 
 
-def test_llama_8b_shaped_layers_at_context_2048(be):
-    """Config 5 at its real shapes: a two-layer prefix of the 8B-shaped Q4_K_M-like model (hidden 4096,
-    32 query heads over 8 K/V heads of 128, FFN 14336 with a Q6_K down projection, the Q6_K 128256-row
-    output, RoPE base 500000) over an f16 cache holding 2048 random positions, two decode steps
-    against the CPU restatement."""
-    n_embd, n_head, n_kv, hd, n_ff, n_vocab, ctx = 4096, 32, 8, 128, 14336, 128256, 2048
+@contextmanager
+def llama_8b_prefix(be, ctx):
+    """A two-layer prefix of the 8B-shaped Q4_K_M-like model (hidden 4096, 32 query heads over 8 K/V heads
+    of 128, FFN 14336 with a Q6_K down projection, the Q6_K 128256-row output, RoPE base 500000) on both
+    sides, over an f16 cache holding `ctx` random positions.  Yields (ref, dev, rng)."""
+    n_embd, n_head, n_kv, hd, n_ff, n_vocab = 4096, 32, 8, 128, 14336, 128256
     from orangu_amd import LlamaDecoder, QuantMatrix
     rng = np.random.default_rng(515)
     shapes = {"wq": (Q4_K, n_embd, n_embd), "wk": (Q4_K, n_embd, n_kv * hd), "wv": (Q4_K, n_embd, n_kv * hd),
@@ -265,7 +266,7 @@ def test_llama_8b_shaped_layers_at_context_2048(be):
     ref.reset()
     out_qm = QuantMatrix(out[1], out[0], out[2], out[3])
     dev = LlamaDecoder(be, n_embd=n_embd, n_head=n_head, n_head_kv=n_kv, head_dim=hd, n_ff=n_ff, n_vocab=n_vocab,
-                       max_ctx=ctx + 2, rms_eps=1e-5, rope_freq_base=500000.0, layers=dev_layers,
+                       max_ctx=ctx + 16, rms_eps=1e-5, rope_freq_base=500000.0, layers=dev_layers,
                        output_norm=out_norm, output=out_qm)
     try:
         for l in range(2):
@@ -274,14 +275,39 @@ def test_llama_8b_shaped_layers_at_context_2048(be):
             dev.kv_write(l, 0, k, v)
             ref.k_cache[l] = [r.astype(np.float16) for r in k]
             ref.v_cache[l] = [r.astype(np.float16) for r in v]
-        for pos in (ctx, ctx + 1):
-            step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"8B shapes pos {pos}")
+        yield ref, dev, rng
     finally:
         dev.close()
         for L in dev_layers:   # 0.9 GB of weights: give them back before the next test
             for k in order:
                 be.evict(L[k])
         be.evict(out_qm)
+
+
+def test_llama_8b_shaped_layers_at_context_2048(be):
+    """Config 5 at its real shapes: two decode steps of the two-layer 8B prefix at context 2048 against
+    the CPU restatement."""
+    ctx = 2048
+    with llama_8b_prefix(be, ctx) as (ref, dev, rng):
+        for pos in (ctx, ctx + 1):
+            step_both(ref, dev, rng.standard_normal(4096).astype(f32), pos, f"8B shapes pos {pos}")
+
+
+def test_llama_8b_shaped_verify_batches_at_context_2048(be):
+    """The speculative-decode verify shape (generate.rs:1618-1674: the last accepted token plus the draft
+    go through the model as one batch, matmuls at n_tokens = 1 + draft, cpu.rs:265-317) at the 8B shapes:
+    batches of 4 and then 8 tokens appended at position 2048 of the two-layer prefix, against the CPU
+    restatement.  The second batch starts where the first did, as after a draft that was rejected whole:
+    both sides drop the first batch's cache rows."""
+    ctx = 2048
+    with llama_8b_prefix(be, ctx) as (ref, dev, rng):
+        for n_tokens in (4, 8):
+            for l in range(2):
+                del ref.k_cache[l][ctx:], ref.v_cache[l][ctx:]
+            X = rng.standard_normal((n_tokens, 4096)).astype(f32)
+            prefill_both(ref, dev, X, ctx, f"8B shapes, verify batch of {n_tokens}")
+        # the step after an accepted batch continues on the rows the batch wrote
+        step_both(ref, dev, rng.standard_normal(4096).astype(f32), ctx + 8, "8B shapes, step after the verify batch")
 
 
 def test_cache_rows_beyond_the_f16_range_saturate(be):
@@ -657,7 +683,7 @@ def test_prefill_attention_kernels_agree(be, hd, group, n_kv, n_tokens, pos0):
     n_embd = n_head * hd
     wtype = Q4_K if n_embd % 256 == 0 else Q8_0
     outs = []
-    for variant in (0, 1):
+    for variant in (2, 1):   # the matrix-core kernel whatever the batch size, then the per-token one
         ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=1,
                               types=(wtype, wtype, wtype, wtype), max_ctx=pos0 + n_tokens, seed=5,
                               attn_norm_scale=TAME.get(wtype, 1.0))
@@ -686,7 +712,7 @@ def test_prefill_attention_with_queries_beyond_f16(be, hd):
     n_embd = n_head * hd
     wtype = Q4_K if n_embd % 256 == 0 else Q8_0
     outs = []
-    for variant in (0, 1):
+    for variant in (2, 1):   # the matrix-core kernel whatever the batch size, then the per-token one
         ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=1,
                               types=(wtype, wtype, wtype, wtype), max_ctx=150, seed=9, pre=("q_norm", "k_norm"),
                               pre_scale={"q_norm": 4e4, "k_norm": 1e-3}, attn_norm_scale=TAME.get(wtype, 1.0))
