@@ -1856,15 +1856,25 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     if (!per_token) {
       HIPCHK(ctx, ogm_launch_attn_prefill_mfma(P.q, kc, vc, pos0, T, c.n_head, c.n_head_kv, c.head_dim, scale, P.attn, s));
     }
+    // A small batch's merge quantizes its rows for wo itself (the tiled GEMMs of larger batches want the
+    // quantizer's second layout and keep their own quantizer launch).
+    const int mode_o = act_mode_for(L.wo->ggml_type, T, 0);
+    const bool fused_q = per_token && T < 32u && qd % (mode_o == OGM_ACT_PER_32 ? 32u : 256u) == 0;
+    if (fused_q && (rc = ensure_act(ctx, qd, T)) != OGM_OK) return rc;
     for (uint32_t t0 = 0; per_token && t0 < T; t0 += P.attn_tokens) {
       const uint32_t nt = T - t0 < P.attn_tokens ? T - t0 : P.attn_tokens;
       HIPCHK(ctx, ogm_launch_attn_prefill(P.q + (size_t)t0 * qd, kc, vc, pos0 + t0, nt, m->max_splits, c.n_head,
                                           c.n_head_kv, c.head_dim, scale, P.part_o, P.part_ml,
-                                          P.attn + (size_t)t0 * qd, s));
+                                          fused_q ? nullptr : P.attn + (size_t)t0 * qd, s, fused_q ? mode_o : -1,
+                                          fused_q ? act_view(ctx, qd, mode_o, t0) : OgmActDev{}));
     }
     const ogm_weight *w1[1] = {L.wo};
     float *y1[1] = {P.proj};
-    if ((rc = llama_matmul_rows(ctx, w1, y1, 1, P.attn, T, s)) != OGM_OK) return rc;
+    if (fused_q) {
+      if ((rc = llama_matmul_quantized_rows(ctx, w1, y1, 1, mode_o, qd, T, s)) != OGM_OK) return rc;
+    } else if ((rc = llama_matmul_rows(ctx, w1, y1, 1, P.attn, T, s)) != OGM_OK) {
+      return rc;
+    }
     const ogm_weight *w2[2] = {L.w_gate, L.w_up};
     float *y2[2] = {P.gate, P.up};
     if ((rc = llama_norm_matmul_rows(ctx, m, w2, y2, 2, P.proj, ffn_norm, T, s)) != OGM_OK) return rc;

@@ -990,28 +990,45 @@ hipError_t ogm_launch_qkv_pre(float *q, const float *k, const float *v, const vo
   return hipGetLastError();
 }
 
-// The chunks of every (token, head) merged: one wave per 256 outputs of a token.
+// The chunks of every (token, head) merged: one wave per 256 outputs of a token.  GROUP != 0: the wave also
+// quantizes its run for the next matmul (per 32 or per 256) into the token's row of `act`; n is then a multiple of
+// GROUP and every lane of the run takes part.
+template <int GROUP>
 __global__ __launch_bounds__(64) void ogm_attn_combine_rows_kernel(const float *__restrict__ part_o,
                                                                    const float *__restrict__ part_ml, uint32_t pos0,
                                                                    uint32_t max_splits, uint32_t n, uint32_t head_dim,
-                                                                   float *__restrict__ attn_out) {
+                                                                   float *__restrict__ attn_out, OgmActDev act) {
   const uint32_t lane = threadIdx.x, tok = blockIdx.y;
   const uint32_t e0 = blockIdx.x * 256u + 4u * lane;
-  if (e0 >= n) return;
+  const bool active = e0 < n;
+  if (GROUP == 0 && !active) return;
   const uint32_t n_head = n / head_dim;
   const uint32_t n_splits = (pos0 + tok) / OGM_ATTN_CHUNK + 1u;
-  const AttnPart pt = attn_merge_chunks<false>(part_o + (size_t)tok * n_head * max_splits * head_dim,
-                                               part_ml + (size_t)tok * n_head * max_splits * 2, e0 / head_dim,
-                                               e0 % head_dim, 0u, 1u, n_splits, max_splits, head_dim);
-  *(float4 *)(attn_out + (size_t)tok * n + e0) =
-      make_float4(pt.o.x / pt.den, pt.o.y / pt.den, pt.o.z / pt.den, pt.o.w / pt.den);
+  float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (active) {
+    const AttnPart pt = attn_merge_chunks<false>(part_o + (size_t)tok * n_head * max_splits * head_dim,
+                                                 part_ml + (size_t)tok * n_head * max_splits * 2, e0 / head_dim,
+                                                 e0 % head_dim, 0u, 1u, n_splits, max_splits, head_dim);
+    o = make_float4(pt.o.x / pt.den, pt.o.y / pt.den, pt.o.z / pt.den, pt.o.w / pt.den);
+    if (attn_out) *(float4 *)(attn_out + (size_t)tok * n + e0) = o;
+  }
+  if constexpr (GROUP != 0) {
+    act.q += (size_t)tok * n;
+    act.d += (size_t)tok * (n / GROUP);
+    act.sums += (size_t)tok * (n / 16u);
+    act.bsum += (size_t)tok * (n / 32u);
+    if (act.bs16) act.bs16 += (size_t)tok * (n / 16u);
+    ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
+  }
 }
 
 hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_cache_layer, uint32_t pos0,
                                    uint32_t n_tokens, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
                                    uint32_t head_dim, float scale, float *part_o, float *part_ml, float *attn_out,
-                                   hipStream_t stream) {
+                                   hipStream_t stream, int quant_mode, OgmActDev act) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0 || n_tokens == 0 || n_tokens > 65535u) return hipErrorInvalidValue;
+  if (quant_mode >= 0 && (n_head * head_dim) % (quant_mode == 0 ? 32u : 256u) != 0) return hipErrorInvalidValue;
+  if (quant_mode < 0 && attn_out == nullptr) return hipErrorInvalidValue;
   const uint32_t n_splits = (pos0 + n_tokens - 1u) / OGM_ATTN_CHUNK + 1u;   // of the last token
   if (n_splits > max_splits) return hipErrorInvalidValue;
   const uint32_t n = n_head * head_dim;
@@ -1039,8 +1056,16 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
 #undef OGM_ATTN_PREFILL
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(ogm_attn_combine_rows_kernel, dim3((n + 255u) / 256u, n_tokens), dim3(64), 0, stream, part_o,
-                     part_ml, pos0, max_splits, n, head_dim, attn_out);
+  const dim3 cgrid((n + 255u) / 256u, n_tokens);
+  if (quant_mode < 0)
+    hipLaunchKernelGGL(ogm_attn_combine_rows_kernel<0>, cgrid, dim3(64), 0, stream, part_o, part_ml, pos0, max_splits, n,
+                       head_dim, attn_out, no_act);
+  else if (quant_mode == 0)
+    hipLaunchKernelGGL(ogm_attn_combine_rows_kernel<32>, cgrid, dim3(64), 0, stream, part_o, part_ml, pos0, max_splits, n,
+                       head_dim, attn_out, act);
+  else
+    hipLaunchKernelGGL(ogm_attn_combine_rows_kernel<256>, cgrid, dim3(64), 0, stream, part_o, part_ml, pos0, max_splits,
+                       n, head_dim, attn_out, act);
   return hipGetLastError();
 }
 
