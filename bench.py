@@ -473,7 +473,13 @@ def main() -> int:
     ap.add_argument("--trace-period", type=int, default=0, metavar="N",
                     help="with --trace-summary: also the mean duration by dispatch number modulo N (N = --copies "
                          "shows each weight copy of the rotation on its own)")
+    ap.add_argument("--lib", default="", metavar="PATH",
+                    help="load this build of the library instead of the in-tree one (a variant built by "
+                         "`python3 orangu_amd/build.py --define ... --out PATH` with a kernel's timing switch set)")
     args = ap.parse_args()
+    if args.lib:
+        from orangu_amd import capi
+        capi.LIB_PATH = os.path.abspath(args.lib)
     if args.trace_summary:
         print(json.dumps(trace_summary(args.trace_summary, args.trace_period), indent=1))
         return 0

@@ -40,12 +40,18 @@ def hipcc() -> str:
 EXTRA_FLAGS = {"ogm_gemm_ft.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 
 
-def build(verbose: bool = False) -> str:
-    """Compiles every source to an object of its own (in parallel) and links the shared library."""
+def build(verbose: bool = False, defines=(), out: str | None = None) -> str:
+    """Compiles every source to an object of its own (in parallel) and links the shared library.
+    `defines` (NAME=VALUE strings, passed as -D) and `out` build a variant beside the library instead of it: the
+    kernels' timing switches (GD_ABL_*, SBW_ABL, FK_ABL: wrong results, for `bench.py --lib`)."""
     from concurrent.futures import ThreadPoolExecutor
     names = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    obj_dir = os.path.join(HERE, "build")
+    if defines and not out:
+        raise ValueError("a build with defines needs an output path of its own")
+    lib_path = os.path.abspath(out) if out else LIB_PATH
+    obj_dir = os.path.join(HERE, "build") if not out else lib_path + ".objs"
     os.makedirs(obj_dir, exist_ok=True)
+    dflags = ["-D" + d for d in defines]
     noise = "is not a recognized feature for this target"
 
     def run(cmd):
@@ -57,16 +63,24 @@ def build(verbose: bool = False) -> str:
 
     def compile_one(name):
         obj = os.path.join(obj_dir, name + ".o")
-        return obj, run([hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(name, []), "-c", os.path.join(CSRC, name), "-o", obj])
+        return obj, run([hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(name, []), *dflags, "-c", os.path.join(CSRC, name), "-o", obj])
 
     with ThreadPoolExecutor(max_workers=min(8, len(names))) as pool:
         done = list(pool.map(compile_one, names))
     log = "\n".join(l for _, l in done if l.strip())
-    log += run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *[o for o, _ in done]])
+    log += run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path, *[o for o, _ in done]])
+    if out:
+        shutil.rmtree(obj_dir, ignore_errors=True)
     if verbose and log.strip():
         print(log)
-    return LIB_PATH
+    return lib_path
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    import argparse
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--define", action="append", default=[], metavar="NAME=VALUE",
+                    help="a timing switch of the kernels (-DNAME=VALUE); needs --out")
+    ap.add_argument("--out", default=None, help="write the library here instead of in-tree")
+    a = ap.parse_args()
+    print(build(verbose=True, defines=a.define, out=a.out))

@@ -601,8 +601,12 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   // Measured at the 8B shapes (4096 -> 1024 / 4096 / 14336 Q4_K, 14336 -> 4096 Q6_K): Q6_K from two tokens on
   // (4 tokens: 18 us against 30), Q4_K / Q5_K from five (up to four the GEMV kernel's per-token dot instructions
   // are level or ahead: 13 us against 15 at 14336 rows; at eight 16 against 17.5 for the small-batch GEMM).
+  // Nine to sixteen tokens need sixteen token slots, whose activations and terms leave one workgroup of four
+  // waves to a compute unit (gate and up at 16 tokens: 56 us against 18 for the small-batch GEMM): by default the
+  // kernel stops at eight.
   const uint32_t mma_from = ctx->tune_gemv_mma == 2 ? 2u : t0 == OGM_Q6_K ? 2u : 5u;
-  if (ctx->tune_gemv_mma != 0 && n_tokens >= mma_from && !dump_isum && !dump_imin && !act_base &&
+  const uint32_t mma_to = ctx->tune_gemv_mma == 2 ? 16u : 8u;
+  if (ctx->tune_gemv_mma != 0 && n_tokens >= mma_from && n_tokens <= mma_to && !dump_isum && !dump_imin && !act_base &&
       ogm_gemv_mma_eligible(w0->ggml_type, w0->in_dim, n_tokens, gemm_order)) {
     for (size_t g0 = 0; g0 < n_tg; g0 += OGM_GEMV_MAX_MATS) {
       const size_t ng = n_tg - g0 < OGM_GEMV_MAX_MATS ? n_tg - g0 : OGM_GEMV_MAX_MATS;

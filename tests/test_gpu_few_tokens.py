@@ -137,13 +137,16 @@ def test_row_block_kernel_at_the_8b_shapes(be):
 
 
 def test_default_routing_of_few_token_batches():
-    """Without tuning: Q6_K goes to the row-block kernel from two tokens, Q4_K from five; one token never."""
+    """Without tuning: Q6_K goes to the row-block kernel from two tokens, Q4_K and Q5_K from five, all up to eight;
+    one token never, nine and more to the small-batch GEMM."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
     try:
-        for t, T, want in ((Q6_K, 1, "ogm_gemv_kernel<FmtQ6K,gemv>"), (Q6_K, 2, NAME[Q6_K]), (Q6_K, 8, NAME[Q6_K]), (Q6_K, 16, NAME[Q6_K]),
-                           (Q4_K, 4, "ogm_gemv_kernel<FmtQ4K,gemm>"), (Q4_K, 5, NAME[Q4_K]), (Q4_K, 16, NAME[Q4_K]),
-                           (Q5_K, 3, "ogm_gemv_kernel<FmtQ5K,gemm>"), (Q5_K, 9, NAME[Q5_K])):
+        for t, T, want in ((Q6_K, 1, "ogm_gemv_kernel<FmtQ6K,gemv>"), (Q6_K, 2, NAME[Q6_K]), (Q6_K, 8, NAME[Q6_K]),
+                           (Q6_K, 9, "ogm_gemm_sb_q6k_kernel"),
+                           (Q4_K, 4, "ogm_gemv_kernel<FmtQ4K,gemm>"), (Q4_K, 5, NAME[Q4_K]), (Q4_K, 8, NAME[Q4_K]),
+                           (Q4_K, 16, "ogm_gemm_sb_q4k_kernel"),
+                           (Q5_K, 3, "ogm_gemv_kernel<FmtQ5K,gemm>"), (Q5_K, 8, NAME[Q5_K]), (Q5_K, 9, "ogm_gemm_sb_q5k_kernel")):
             raw = synth_weights(t, 1024, 48, seed=T)
             x = synth_x(T, 1024, seed=T)
             got = b.matmul(x, T, qm(raw, t, 1024, 48))

@@ -595,9 +595,9 @@ def test_medium_batch_kernel_over_several_matrices_and_extreme_ranges(be):
 
 def test_gemm_threshold_default():
     """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
-    float order, 17 through the matrix-core GEMM.  Q4_K: 4 tokens through the GEMV kernel, 5 to 16 through the
+    float order, 17 through the matrix-core GEMM.  Q4_K: 4 tokens through the GEMV kernel, 5 to 8 through the
     row-block kernel (rows of a multiple of 1024 inputs; of other lengths the GEMV kernel up to 5 and the
-    small-batch kernel from 6), 17 to 224
+    small-batch kernel from 6), 9 to 224
     through the small-batch kernel (a matrix of few rows), 225 to 256 through the medium-batch kernel, 257
     through the tiled one; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
     many that 128 x 128 tiles outnumber the compute units has its planes built and read by the kernel whose
@@ -620,8 +620,8 @@ def test_gemm_threshold_default():
         w = qm(raw, Q4_K, 1024, 70)
         want = oracle.matmul(Q4_K, raw, 1024, 70, x, 257).reshape(257, 70)
         # (up to 64 tiles of 64 rows the small-batch kernel keeps batches of up to 224 tokens)
-        for n, kernel in ((4, "ogm_gemv_kernel"), (5, "ogm_gemm_fk_kernel<Q4_K>"), (16, "ogm_gemm_fk_kernel<Q4_K>"),
-                          (17, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
+        for n, kernel in ((4, "ogm_gemv_kernel"), (5, "ogm_gemm_fk_kernel<Q4_K>"), (8, "ogm_gemm_fk_kernel<Q4_K>"),
+                          (9, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
                           (224, "ogm_gemm_sb_q4k_kernel"), (225, "ogm_gemm_sbw_q4k_kernel"),
                           (256, "ogm_gemm_sbw_q4k_kernel"), (257, "ogm_gemm_q4k_i8p_r64_kernel")):
             y = b.matmul(x[:n], n, w)
@@ -635,10 +635,10 @@ def test_gemm_threshold_default():
             assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, oracle.matmul(Q4_K, raw, 768, 70, x3[:n], n), f"Q4_K of 768 inputs, {n} tokens")
         raw = synth_weights(Q5_K, 4096, 70, seed=7)    # few workgroups, sixteen super-blocks: sixteen waves
-        x4 = synth_x(20, 4096, seed=8)
-        y = b.matmul(x4, 20, qm(raw, Q5_K, 4096, 70))
+        x4 = synth_x(12, 4096, seed=8)
+        y = b.matmul(x4, 12, qm(raw, Q5_K, 4096, 70))
         assert kname(b) == "ogm_gemm_sb_q5k_w16_kernel"
-        assert_bits(y, oracle.matmul(Q5_K, raw, 4096, 70, x4, 20), "Q5_K, 20 tokens")
+        assert_bits(y, oracle.matmul(Q5_K, raw, 4096, 70, x4, 12), "Q5_K, 12 tokens")
         raw = synth_weights(Q6_K, 256, 8300, seed=6)   # 130 tiles of 64 rows
         w = qm(raw, Q6_K, 256, 8300)
         want = oracle.matmul(Q6_K, raw, 256, 8300, np.ascontiguousarray(x[:65, :256]), 65).reshape(65, 8300)
