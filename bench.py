@@ -206,7 +206,7 @@ def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
 
 
 def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool, only_prefill: int = 0,
-               with_prefill: bool = True, only_verify: int = 0) -> dict:
+               with_prefill: bool = True, only_verify: int = 0, attn_timeline: bool = False) -> dict:
     """Batch-1 decode of an 8B-shaped Llama (32 layers: wq, wo 4096x4096, wk, wv 4096->1024, gate, up
     4096->14336 in Q4_K; down 14336->4096 and the 128256-row output in Q6_K; f16 KV cache holding `ctx`
     random positions): tokens per second of ogm_llama_decode_dev with the embedding row, the logits and
@@ -276,6 +276,35 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     tok_d = hiprt.DeviceBuffer(4)
     stream = hiprt.Stream()
     pos = ctx
+    if attn_timeline:
+        # A variant of the library built with -DOGM_ATTN_STAMPS=1 (`--lib`): the wall-clock stamps of the last
+        # layer's attention launch of each of `steps` decode steps, phase by phase, medians over steps.
+        n_wg = n_kv * (ctx // 128 + 1)
+        phases = ["start -> q rotated, new K/V row written", "scores of the chunk", "weighted V sum",
+                  "partial results stored and acknowledged", "ticket drawn",
+                  "merging workgroup: chunks merged", "merging workgroup: row quantized"]
+        rows = {k: [] for k in phases}
+        spans = []
+        for i in range(warmup + steps):
+            dec.decode_dev(x_d.ptr, pos, 0, tok_d.ptr, stream.ptr)
+            stream.synchronize()
+            st = dec.attn_stamps(n_wg).astype(np.int64)
+            pos += 1
+            if i < warmup:
+                continue
+            d = np.diff(st, axis=1) * 10.0 / 1e3          # 100 MHz ticks -> us
+            merging = (st[:, 6] > st[:, 5]) & (st[:, 7] >= st[:, 6])   # (stamps of an earlier layer's merge are older)
+            for j, k in enumerate(phases):
+                sel = d[:, j] if j < 5 else d[merging, j]
+                rows[k].append(float(np.median(sel)))
+            spans.append((max(st[:, 5].max(), st[merging, 7].max()) - st[:, 0].min()) * 10.0 / 1e3)
+        dec.close()
+        for h in mats.values():
+            be.free_weight(h)
+        return {"workload": f"attention kernel of a decode step at context {ctx}: {n_wg} workgroups, 100 MHz stamps, "
+                            f"median over workgroups, then over {steps} steps",
+                "us": {k: round(float(np.median(v)), 2) for k, v in rows.items()},
+                "first start -> last end": round(float(np.median(spans)), 2)}
     for _ in range(warmup):
         dec.decode_dev(x_d.ptr, pos, 0, tok_d.ptr, stream.ptr)
         pos += 1
@@ -445,6 +474,8 @@ def main() -> int:
                     help="tokens of the 8B-shaped decode leg (config 5); 0 skips it")
     ap.add_argument("--decode-ctx", type=int, default=2048, help="cached positions of the decode leg")
     ap.add_argument("--only-decode", action="store_true", help="run only the decode leg (for rocprofv3)")
+    ap.add_argument("--attn-timeline", action="store_true",
+                    help="with --lib of a variant built with -DOGM_ATTN_STAMPS=1: the decode attention kernel's phases")
     ap.add_argument("--only-verify", type=int, default=0, metavar="N",
                     help="run only verify batches of N tokens at the decode context (for rocprofv3)")
     ap.add_argument("--only-prefill", type=int, default=0, metavar="N",
@@ -504,6 +535,10 @@ def main() -> int:
     if args.only_prefill:
         print(json.dumps(decode_leg(be, helpers, hiprt, 1, 0, max(args.decode_ctx, args.only_prefill), False,
                                     only_prefill=args.only_prefill)))
+        be.close()
+        return 0
+    if args.attn_timeline:
+        print(json.dumps(decode_leg(be, helpers, hiprt, 16, 4, args.decode_ctx, False, attn_timeline=True)))
         be.close()
         return 0
     if args.only_verify:

@@ -330,6 +330,13 @@ int ogm_llama_debug_capture(ogm_ctx *ctx, ogm_llama *m, int enable);
 int ogm_llama_debug_act(ogm_ctx *ctx, ogm_llama *m, uint32_t site, int8_t *q, float *d, uint32_t *n,
                         uint32_t *group);
 
+/* Measurement only, no counterpart in the reference: the wall-clock stamps (100 MHz) the decode step's attention
+ * kernel leaves in a variant of the library built with -DOGM_ATTN_STAMPS=1 -- eight per workgroup of the last
+ * launch, in the grid's order: start, q rotated, scores, V sum, partial results acknowledged, ticket drawn, and for
+ * the workgroup that merges: chunks merged, row quantized.  Reads n_words of them and clears them.
+ * OGM_ERR_UNSUPPORTED from the shipped library, which keeps none. */
+int ogm_debug_attn_stamps(ogm_ctx *ctx, uint64_t *out, size_t n_words);
+
 /* ---- GGUF reader -> uploader -------------------------------------------------------------------- */
 
 /* Reads a GGUF file's header, metadata and tensor table (GgufFile::open_at / read, src/gguf.rs:149-280,

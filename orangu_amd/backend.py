@@ -532,6 +532,13 @@ class LlamaDecoder:
                         "ogm_llama_debug_hidden")
         return out
 
+    def attn_stamps(self, n_workgroups: int) -> np.ndarray:
+        """Timeline builds only: [n_workgroups][8] wall-clock stamps (100 MHz) of the last attention launch."""
+        out = np.zeros((n_workgroups, 8), np.uint64)
+        self._be._check(self._be._lib.ogm_debug_attn_stamps(self._be._ctx, out.ctypes.data, out.size),
+                        "ogm_debug_attn_stamps")
+        return out
+
     def capture_acts(self, on: bool = True):
         """Debug: keep the quantized activations every matmul group of a decode step reads."""
         self._be._check(self._be._lib.ogm_llama_debug_capture(self._be._ctx, self._h, 1 if on else 0),

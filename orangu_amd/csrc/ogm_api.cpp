@@ -1601,6 +1601,19 @@ extern "C" int ogm_llama_debug_hidden(ogm_ctx *ctx, ogm_llama *m, float *x_out) 
   return OGM_OK;
 }
 
+extern "C" int ogm_debug_attn_stamps(ogm_ctx *ctx, uint64_t *out, size_t n_words) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!out) return fail(ctx, OGM_ERR_INVALID, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  const hipError_t e = ogm_attn_stamps_read((unsigned long long *)out, n_words);
+  if (e == hipErrorNotSupported)
+    return fail(ctx, OGM_ERR_UNSUPPORTED, "this build of the library keeps no attention stamps (build a variant with -DOGM_ATTN_STAMPS=1)");
+  HIPCHK(ctx, e);
+  return OGM_OK;
+}
+
 extern "C" int ogm_llama_debug_capture(ogm_ctx *ctx, ogm_llama *m, int enable) {
   if (!ctx) return OGM_ERR_INVALID;
   if (!m) return fail(ctx, OGM_ERR_INVALID, "null argument");

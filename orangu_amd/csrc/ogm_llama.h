@@ -110,3 +110,6 @@ hipError_t ogm_launch_attn_prefill_mfma(const float *q, void *k_cache_layer, voi
                                         uint32_t n_tokens, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim,
                                         float scale, float *attn_out, hipStream_t stream);
 
+// Timeline builds only (-DOGM_ATTN_STAMPS=1): the wall-clock stamps (100 MHz) of the last attention launch, eight per
+// workgroup; hipErrorNotSupported from the shipped library.
+hipError_t ogm_attn_stamps_read(unsigned long long *host_out, size_t n_words);

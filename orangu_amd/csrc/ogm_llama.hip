@@ -118,8 +118,9 @@ __device__ __forceinline__ void st_one(float *p, float v) {
   else *p = v;
 }
 
-// Wall-clock stamps for timeline builds of the attention kernel (a scratch build defines
-// OGM_ATTN_STAMPS and the buffer; the library never does).
+// Wall-clock stamps for timeline builds of the attention kernel: a variant of the library built with
+// -DOGM_ATTN_STAMPS=1 keeps eight stamps per workgroup of the last launch, and ogm_attn_stamps_read hands them out
+// (the shipped library has neither stamps nor buffer, and the reader reports that).
 #ifdef OGM_ATTN_STAMPS
 __device__ unsigned long long ogm_attn_stamps[4096 * 8];
 #define OGM_STAMP(i)                                                                              \
@@ -1371,3 +1372,19 @@ hipError_t ogm_launch_attn_prefill_mfma(const float *q, void *k_cache_layer, voi
   return hipGetLastError();
 }
 
+// The stamps of the last attention launch, eight per workgroup in the grid's order (x fastest), then cleared.
+hipError_t ogm_attn_stamps_read(unsigned long long *host_out, size_t n_words) {
+#ifdef OGM_ATTN_STAMPS
+  if (n_words > 4096u * 8u) return hipErrorInvalidValue;
+  hipError_t e = hipMemcpyFromSymbol(host_out, HIP_SYMBOL(ogm_attn_stamps), n_words * 8u);
+  if (e != hipSuccess) return e;
+  void *dev = nullptr;
+  e = hipGetSymbolAddress(&dev, HIP_SYMBOL(ogm_attn_stamps));
+  if (e != hipSuccess) return e;
+  return hipMemset(dev, 0, sizeof(unsigned long long) * 4096u * 8u);
+#else
+  (void)host_out;
+  (void)n_words;
+  return hipErrorNotSupported;
+#endif
+}
