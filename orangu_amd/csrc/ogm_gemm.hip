@@ -2022,12 +2022,15 @@ static bool gemm_medium_batch(const OgmGemmArgs &a) {
   // (feeding waves), at 192 / 256 tokens 78 / 77 against 65 / 65; 4096 -> 4096 at 256 tokens 35 against 39 (small
   // batch), at 128 tokens 33 against 23; 4096 -> 6144 at 128 / 256 tokens 34 / 40 against 36 / 46; 14336 -> 4096 at
   // 256 tokens 106 against 116.  It wants its token tiles of 128 nearly full, and at two of them matrices of at most
-  // 8192 rows (beyond, the 128-row tiles of the feeding-wave kernels outnumber the compute units' halves).
+  // 8192 rows (beyond, the 128-row tiles of the feeding-wave kernels outnumber the compute units' halves).  Its
+  // workgroups of 32 rows must fit the device in one round, two to a compute unit: gate and up together (28672 rows,
+  // 896 workgroups) take 63 us against 56 for the feeding-wave kernel (128-token prefill of the 8B shapes 7.0
+  // against 6.65 ms), so at one token tile the launch may have at most 16384 rows.
   uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
   for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
   const uint32_t tok_tiles = (a.n_tokens + SBW_TOK - 1u) / SBW_TOK;
   const bool full_enough = tok_tiles * SBW_TOK - a.n_tokens <= 32u;
-  return full_enough && (tok_tiles == 1u || (tok_tiles == 2u && tiles64_all <= 128u));
+  return full_enough && ((tok_tiles == 1u && tiles64_all <= 256u) || (tok_tiles == 2u && tiles64_all <= 128u));
 }
 
 // Whether a tiled launch goes to the kernel whose waves all multiply, given planes.  It wants more

@@ -601,7 +601,7 @@ def test_gemm_threshold_default():
     through the small-batch kernel (a matrix of few rows), 225 to 256 through the medium-batch kernel, 257
     through the tiled one; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
     many that 128 x 128 tiles outnumber the compute units has its planes built and read by the kernel whose
-    waves all multiply, while a single nearly full token tile goes to the medium-batch kernel.
+    waves all multiply, while a single nearly full token tile over at most 16384 rows goes to the medium-batch kernel.
     Same bits everywhere."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
@@ -652,11 +652,16 @@ def test_gemm_threshold_default():
         y = b.matmul(x5, 129, w)
         assert b.last_kernel() == "ogm_gemm_q4k_dma_kernel"
         assert_bits(y, oracle.matmul(Q4_K, raw, 256, 16600, x5, 129), "Q4_K, 129 tokens x 16600 rows")
-        y = b.matmul(x5[:128], 128, w)                   # one full token tile: the medium-batch kernel
-        assert b.last_kernel() == "ogm_gemm_sbw_q4k_kernel"
+        y = b.matmul(x5[:128], 128, w)                   # one full token tile, but more 32-row workgroups than one round
+        assert b.last_kernel() == "ogm_gemm_q4k_i8p_kernel"
         assert_bits(y, oracle.matmul(Q4_K, raw, 256, 16600, x5[:128], 128), "Q4_K, 128 tokens x 16600 rows")
         y = b.matmul(x5[:90], 90, w)                     # a token tile a third empty: 130 workgroups of 128 rows
         assert b.last_kernel() == "ogm_gemm_q4k_i8p_kernel"
+        raw = synth_weights(Q4_K, 256, 16000, seed=10)  # 500 workgroups of 32 rows: the medium-batch kernel's one round
+        w = qm(raw, Q4_K, 256, 16000)
+        y = b.matmul(x5[:128], 128, w)
+        assert b.last_kernel() == "ogm_gemm_sbw_q4k_kernel"
+        assert_bits(y, oracle.matmul(Q4_K, raw, 256, 16000, x5[:128], 128), "Q4_K, 128 tokens x 16000 rows")
     finally:
         b.close()
 
