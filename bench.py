@@ -261,10 +261,10 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
                 "prefill_ms": round(dt_pre * 1e3, 2), "prefill_tok_per_s": round(only_prefill / dt_pre, 1)}
     if only_verify:    # for profiles: nothing but verify batches of this size appended at position `ctx`
         xv = rng.standard_normal((only_verify, n_embd)).astype(np.float32)
-        dec.prefill(xv, ctx)
+        dec.forward_all_logits(xv, ctx, want_logits=False)
         t0 = time.perf_counter()
         for _ in range(10):
-            dec.prefill(xv, ctx)
+            dec.forward_all_logits(xv, ctx, want_logits=False)
         dt_v = (time.perf_counter() - t0) / 10
         dec.close()
         for h in mats.values():
@@ -324,19 +324,26 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     dt_gen = (time.perf_counter() - t0) / steps
     pos += steps
     # speculative-decode verify (generate.rs:1618-1674): the last accepted token plus a draft of 3 or 7 go
-    # through the whole model as one batch appended at position `ctx`, host embedding rows in, the last
-    # token's logits out (ogm_llama_prefill); wall clock per call, the first call of a size untimed
+    # through the whole model as one batch appended at position `ctx`; host embedding rows in, and out
+    # (a) the greedy token of EVERY position (ogm_llama_forward_all_logits: what the verify step compares the
+    # draft with; the logits of all positions stay on the device), (b) the last position's logits alone
+    # (ogm_llama_prefill).  Wall clock per call, the first call of a size untimed.
     verify = {}
     for n_v in (4, 8):
         xv = rng.standard_normal((n_v, n_embd)).astype(np.float32)
-        dec.prefill(xv, ctx)
         reps_v = max(3, min(20, steps // 10))
-        t0 = time.perf_counter()
-        for _ in range(reps_v):
-            dec.prefill(xv, ctx)
-        dt_v = (time.perf_counter() - t0) / reps_v
-        verify[f"verify_batch_{n_v}"] = {"ms": round(dt_v * 1e3, 3), "tokens_verified_per_s": round(n_v / dt_v, 1),
-                                         "calls": reps_v}
+        row = {"calls": reps_v}
+        for key, call in (("all_positions", lambda: dec.forward_all_logits(xv, ctx, want_logits=False)),
+                          ("last_position", lambda: dec.prefill(xv, ctx))):
+            call()
+            t0 = time.perf_counter()
+            for _ in range(reps_v):
+                call()
+            dt_v = (time.perf_counter() - t0) / reps_v
+            row[key] = {"ms": round(dt_v * 1e3, 3), "tokens_verified_per_s": round(n_v / dt_v, 1)}
+        row["ms"] = row["all_positions"]["ms"]
+        row["tokens_verified_per_s"] = row["all_positions"]["tokens_verified_per_s"]
+        verify[f"verify_batch_{n_v}"] = row
     # prefill of a 512-token prompt from position 0 (GEMM matmuls, batch attention); the first
     # call allocates the batch buffers
     dt_pre = dt_pre_long = dt_pre_long_one = None

@@ -287,6 +287,18 @@ int ogm_llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x, uint32_t pos0,
 int ogm_llama_prefill_tokens(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *tok_embd, const uint32_t *tokens,
                              uint32_t pos0, uint32_t n_tokens, float *last_logits, uint32_t *argmax);
 
+/* Model::forward_all_logits (the trait's contract, engine/arch/mod.rs:2110-2132; speculative_next's verify step
+ * calls it, engine/generate.rs:1641): like ogm_llama_prefill -- n_tokens positions appended at pos0, from embedding
+ * rows x [n_tokens][n_embd] or, with x null, from token ids into tok_embd -- but returns the next-token logits of
+ * EVERY position, logits [n_tokens][n_vocab] (may be null), and each position's greedy token, argmax [n_tokens]
+ * (may be null; sampling.rs:336-343's order): every row through the output norm and ONE matmul of all rows with
+ * the output matrix, the composition engine/arch/gemma.rs:2179-2186 uses (llama.rs itself leaves the trait's
+ * default, an error).  A rejected draft is rolled back by calling again at the position after the accepted
+ * prefix: cache rows from there on are overwritten (KvCache::truncate).  At most 64 positions a call. */
+int ogm_llama_forward_all_logits(ogm_ctx *ctx, ogm_llama *m, const float *x, const ogm_weight *tok_embd,
+                                 const uint32_t *tokens, uint32_t pos0, uint32_t n_tokens, float *logits,
+                                 uint32_t *argmax);
+
 /* forward_hidden_states (llama.rs:1034-1045): the n_tokens tokens at positions 0 .. through run_layers
  * from an empty cache, then every row through the output norm: out is [n_tokens][n_embd] (host f32),
  * what an embeddings request pools over.  The tokens come as embedding rows x ([n_tokens][n_embd], host)

@@ -230,12 +230,13 @@ def _mm(w: tuple, x: np.ndarray, n_tokens: int = 1) -> np.ndarray:
     return y.reshape(-1) if n_tokens == 1 else y.reshape(n_tokens, out_dim)
 
 
-def forward(m: Model, X: np.ndarray, pos0: int, all_rows: bool = False):
+def forward(m: Model, X: np.ndarray, pos0: int, all_rows: bool = False, all_logits: bool = False):
     """llama.rs:594-932 + 1007-1032 for the tokens whose embedding rows are X [n_tokens][n_embd], at
     positions pos0 ..: every matmul over all rows at once, K/V rows appended in order, token t
     attending to cache rows 0 .. pos0 + t; the LAST row alone goes through the output norm and
     projection.  Returns (logits of the last token, its final hidden state); with all_rows instead every
-    row after the output norm and no projection (llama.rs:1034-1045)."""
+    row after the output norm and no projection (llama.rs:1034-1045); with all_logits the logits of every row
+    [n_tokens][n_vocab] and the rows' final hidden states."""
     if not m.k_cache:
         m.reset()
     X = np.array(X, f32).reshape(-1, m.n_embd)
@@ -287,6 +288,11 @@ def forward(m: Model, X: np.ndarray, pos0: int, all_rows: bool = False):
         gate, up = mms(4 * li + 2, (L.w_gate, L.w_up), normed2)
         h = (silu(gate) * up).astype(f32)
         X = (X + mms(4 * li + 3, (L.w_down,), h)[0]).astype(f32)
+    if all_logits:
+        # forward_all_logits (arch/mod.rs:2110-2132, composed as gemma.rs:2179-2186): every row through the output
+        # norm, one matmul of all rows with the output matrix (the GEMM kernels at more than one row)
+        normed = rows(lambda r: rmsnorm(r, m.output_norm, m.rms_eps), X)
+        return mms(4 * len(m.layers), (m.output,), normed)[0], X
     if all_rows:
         return rows(lambda r: rmsnorm(r, m.output_norm, m.rms_eps), X)
     last = rmsnorm(X[-1], m.output_norm, m.rms_eps)

@@ -483,6 +483,25 @@ class LlamaDecoder:
                                                         logits.ctypes.data, C.byref(am)), "ogm_llama_prefill")
         return logits, am.value
 
+    def forward_all_logits(self, x=None, pos0: int = 0, tok_embd=None, tokens=None, want_logits: bool = True):
+        """Model::forward_all_logits (arch/mod.rs:2110-2132): the positions' embedding rows x [n][n_embd] (or token
+        ids into tok_embd) appended at pos0; returns (logits [n][n_vocab] or None, greedy token of every position)."""
+        if (x is None) == (tok_embd is None):
+            raise ValueError("give embedding rows or a matrix with token ids")
+        if x is not None:
+            x = np.ascontiguousarray(x, np.float32).reshape(-1, self.n_embd)
+            n, xp, hp, tp = x.shape[0], x.ctypes.data, None, None
+        else:
+            hp = tok_embd if isinstance(tok_embd, int) else self._be.upload(tok_embd)
+            tokens = np.ascontiguousarray(tokens, np.uint32).reshape(-1)
+            n, xp, tp = tokens.size, None, tokens.ctypes.data
+        logits = np.empty((n, self.n_vocab), np.float32) if want_logits else None
+        am = np.empty(n, np.uint32)
+        self._be._check(self._be._lib.ogm_llama_forward_all_logits(
+            self._be._ctx, self._h, xp, hp, tp, pos0, n, logits.ctypes.data if want_logits else None, am.ctypes.data),
+            "ogm_llama_forward_all_logits")
+        return logits, am
+
     def prefill_tokens(self, tok_embd, tokens, pos0: int = 0):
         """The same from token ids; tok_embd is a QuantMatrix [n_embd -> n_vocab] or a handle."""
         h = tok_embd if isinstance(tok_embd, int) else self._be.upload(tok_embd)

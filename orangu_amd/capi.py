@@ -28,7 +28,7 @@ SYMBOLS = [
     "ogm_gguf_open", "ogm_gguf_parse", "ogm_gguf_close", "ogm_gguf_last_error", "ogm_gguf_info",
     "ogm_gguf_meta_u64", "ogm_gguf_meta_f64", "ogm_gguf_meta_string", "ogm_gguf_meta_array",
     "ogm_gguf_find_tensor", "ogm_gguf_tensor", "ogm_gguf_tensor_data", "ogm_gguf_matrix",
-    "ogm_gguf_upload_matrix", "ogm_argmax", "ogm_matmul_dev_static", "ogm_quantize_act_tokens", "ogm_llama_debug_capture", "ogm_llama_debug_act", "ogm_debug_attn_stamps",
+    "ogm_gguf_upload_matrix", "ogm_argmax", "ogm_matmul_dev_static", "ogm_quantize_act_tokens", "ogm_llama_debug_capture", "ogm_llama_debug_act", "ogm_debug_attn_stamps", "ogm_llama_forward_all_logits",
     "ogm_weights_read_probe", "ogm_time_host_calls", "ogm_empty_launch", "ogm_scratch_bytes", "ogm_act_quantize_decode_dev", "ogm_enqueue_repeated",
 ]
 
@@ -142,6 +142,7 @@ def load_library() -> C.CDLL:
     L.ogm_llama_debug_capture.argtypes = [vp, vp, C.c_int]
     L.ogm_llama_debug_act.argtypes = [vp, vp, u32, vp, vp, C.POINTER(u32), C.POINTER(u32)]
     L.ogm_debug_attn_stamps.argtypes = [vp, vp, sz]
+    L.ogm_llama_forward_all_logits.argtypes = [vp, vp, vp, vp, vp, u32, u32, vp, vp]
     L.ogm_set_tuning.argtypes = [vp, C.c_char_p, C.c_int]
     L.ogm_last_kernel.argtypes = [vp]
     L.ogm_last_kernel.restype = C.c_char_p

@@ -1237,6 +1237,9 @@ struct ogm_llama {
   float *part_o = nullptr, *part_ml = nullptr;     // attention partials
   float *logits = nullptr;    // [n_vocab]
   uint32_t *amax_scratch = nullptr, *amax_out = nullptr;
+  // ogm_llama_forward_all_logits: every position's logits and greedy token, allocated at its first call
+  float *logits_all = nullptr;      // [OGM_ALL_LOGITS_MAX_TOKENS][n_vocab]
+  uint32_t *amax_all = nullptr;     // [OGM_ALL_LOGITS_MAX_TOKENS]
   float *stage = nullptr;     // host->device staging for ogm_llama_kv_write
   size_t stage_cap = 0;
   // prefill rows, allocated at the first prefill for the pass size of that moment (prefill_chunk_tokens)
@@ -1842,7 +1845,7 @@ static int llama_norm_matmul_rows(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
 // One chunk of T <= m->pf.chunk tokens whose embedding rows sit in m->pf.x.  With `last`,
 // the final row's hidden state ends in m->x and its logits in m->logits.
 static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32_t T, bool last, hipStream_t s,
-                               float *normed_rows = nullptr) {
+                               float *normed_rows = nullptr, bool all_logits = false) {
   const ogm_llama_config &c = m->cfg;
   ogm_llama::Prefill &P = m->pf;
   const uint32_t qd = c.n_head * c.head_dim, kvd = c.n_head_kv * c.head_dim;
@@ -1904,6 +1907,22 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     delta = P.proj;
   }
   ctx->act_mode = -1;   // the activation scratch was the matmuls'
+  if (all_logits) {
+    // forward_all_logits (the trait's contract, arch/mod.rs:2110-2132; composed as gemma.rs:2179-2186 does): every row
+    // through the output norm, one matmul of all rows with the output matrix, and each row's greedy token
+    int rc = ensure_act(ctx, c.n_embd, T);
+    if (rc != OGM_OK) return rc;
+    const int mode_out = act_mode_for(m->output->ggml_type, T, 0);
+    HIPCHK(ctx, ogm_launch_norm_quant(mode_out, P.x, delta, m->norms + (size_t)c.n_layer * 2 * c.n_embd, c.n_embd,
+                                      c.rms_eps, nullptr, act_view(ctx, c.n_embd, mode_out, 0), s, T));
+    const ogm_weight *wo_[1] = {m->output};
+    float *yo[1] = {m->logits_all};
+    if ((rc = llama_matmul_quantized_rows(ctx, wo_, yo, 1, mode_out, c.n_embd, T, s)) != OGM_OK) return rc;
+    for (uint32_t t = 0; t < T; t++)
+      HIPCHK(ctx, ogm_launch_argmax(m->logits_all + (size_t)t * c.n_vocab, c.n_vocab, m->amax_scratch, m->amax_all + t, s));
+    ctx->act_mode = -1;
+    return OGM_OK;
+  }
   if (normed_rows) {
     // forward_hidden_states (llama.rs:1034-1045): every row through the output norm, no projection
     int rc = ensure_act(ctx, c.n_embd, T);
@@ -1978,6 +1997,51 @@ extern "C" int ogm_llama_prefill(ogm_ctx *ctx, ogm_llama *m, const float *x, uin
   if (!ctx) return OGM_ERR_INVALID;
   if (!m || !x) return fail(ctx, OGM_ERR_INVALID, "null argument");
   return llama_prefill(ctx, m, x, nullptr, nullptr, pos0, n_tokens, last_logits, argmax);
+}
+
+static const uint32_t OGM_ALL_LOGITS_MAX_TOKENS = 64;
+
+extern "C" int ogm_llama_forward_all_logits(ogm_ctx *ctx, ogm_llama *m, const float *x, const ogm_weight *tok_embd,
+                                            const uint32_t *tokens, uint32_t pos0, uint32_t n_tokens, float *logits,
+                                            uint32_t *argmax) {
+  if (!ctx) return OGM_ERR_INVALID;
+  if (!m || (x == nullptr) == (tok_embd == nullptr) || (tok_embd && !tokens))
+    return fail(ctx, OGM_ERR_INVALID, "ogm_llama_forward_all_logits takes embedding rows or a matrix with token ids");
+  const ogm_llama_config &c = m->cfg;
+  if (n_tokens == 0) return fail(ctx, OGM_ERR_INVALID, "no tokens");
+  if (n_tokens > OGM_ALL_LOGITS_MAX_TOKENS)
+    return fail(ctx, OGM_ERR_UNSUPPORTED, "ogm_llama_forward_all_logits takes at most 64 positions a call");
+  if ((uint64_t)pos0 + n_tokens > c.max_ctx) return fail(ctx, OGM_ERR_INVALID, "positions beyond the KV cache");
+  if (tok_embd) {
+    if (tok_embd->in_dim != c.n_embd) return fail(ctx, OGM_ERR_INVALID, "embedding matrix shape");
+    for (uint32_t i = 0; i < n_tokens; i++)
+      if (tokens[i] >= tok_embd->out_dim) return fail(ctx, OGM_ERR_INVALID, "token id outside the vocabulary");
+  }
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIPCHK(ctx, hipSetDevice(ctx->device));
+  int rc = llama_prefill_buffers(ctx, m);
+  if (rc != OGM_OK) return rc;
+  if (n_tokens > m->pf.chunk) return fail(ctx, OGM_ERR_UNSUPPORTED, "more positions than one pass over the layers takes");
+  if (!m->logits_all) {
+    rc = llama_alloc(ctx, m, (void **)&m->logits_all, (size_t)OGM_ALL_LOGITS_MAX_TOKENS * c.n_vocab * 4);
+    if (rc == OGM_OK) rc = llama_alloc(ctx, m, (void **)&m->amax_all, (size_t)OGM_ALL_LOGITS_MAX_TOKENS * 4);
+    if (rc != OGM_OK) return rc;
+  }
+  hipStream_t s = ctx->stream;
+  if (tok_embd) {
+    HIPCHK(ctx, hipMemcpyAsync(m->pf.tokens, tokens, (size_t)n_tokens * 4, hipMemcpyHostToDevice, s));
+    HIPCHK(ctx, ogm_launch_dequant_row(tok_embd->dev, tok_embd->ggml_type, tok_embd->in_dim, tok_embd->out_dim, 0,
+                                       m->pf.tokens, n_tokens, m->pf.x, s));
+  } else {
+    HIPCHK(ctx, hipMemcpyAsync(m->pf.x, x, (size_t)n_tokens * c.n_embd * 4, hipMemcpyHostToDevice, s));
+  }
+  rc = llama_prefill_chunk(ctx, m, pos0, n_tokens, false, s, nullptr, true);
+  if (rc != OGM_OK) return rc;
+  if (argmax) HIPCHK(ctx, hipMemcpyAsync(argmax, m->amax_all, (size_t)n_tokens * 4, hipMemcpyDeviceToHost, s));
+  if (logits)
+    HIPCHK(ctx, hipMemcpyAsync(logits, m->logits_all, (size_t)n_tokens * c.n_vocab * 4, hipMemcpyDeviceToHost, s));
+  HIPCHK(ctx, hipStreamSynchronize(s));
+  return OGM_OK;
 }
 
 extern "C" int ogm_llama_hidden_states(ogm_ctx *ctx, ogm_llama *m, const float *x, const ogm_weight *tok_embd,

@@ -297,7 +297,8 @@ def test_llama_8b_shaped_verify_batches_at_context_2048(be):
     """The speculative-decode verify shape (generate.rs:1618-1674: the last accepted token plus the draft
     go through the model as one batch, matmuls at n_tokens = 1 + draft, cpu.rs:265-317) at the 8B shapes:
     batches of 4 and then 8 tokens appended at position 2048 of the two-layer prefix, against the CPU
-    restatement.  The second batch starts where the first did, as after a draft that was rejected whole:
+    restatement -- the first through forward_all_logits (every position's logits and greedy token: what the
+    verify step compares the draft with), the second through the prefill entry (the last position's).  The second batch starts where the first did, as after a draft that was rejected whole:
     both sides drop the first batch's cache rows."""
     ctx = 2048
     with llama_8b_prefix(be, ctx) as (ref, dev, rng):
@@ -305,7 +306,7 @@ def test_llama_8b_shaped_verify_batches_at_context_2048(be):
             for l in range(2):
                 del ref.k_cache[l][ctx:], ref.v_cache[l][ctx:]
             X = rng.standard_normal((n_tokens, 4096)).astype(f32)
-            prefill_both(ref, dev, X, ctx, f"8B shapes, verify batch of {n_tokens}")
+            prefill_both(ref, dev, X, ctx, f"8B shapes, verify batch of {n_tokens}", all_logits=n_tokens == 4)
         # the step after an accepted batch continues on the rows the batch wrote
         step_both(ref, dev, rng.standard_normal(4096).astype(f32), ctx + 8, "8B shapes, step after the verify batch")
 
@@ -481,7 +482,7 @@ def test_matrices_uploaded_from_a_gguf_file_multiply_like_direct_uploads(be, tmp
 TAME = {Q4_K: 0.02, Q5_K: 0.02, Q4_0: 0.1}
 
 
-def prefill_both(ref, dev, X, pos0, what, via_tokens=None):
+def prefill_both(ref, dev, X, pos0, what, via_tokens=None, all_logits=False):
     """A batch of tokens on both sides, cache rows in lock-step as in `step_both`.  A flipped
     activation rounding touches one token's rows from the next layer on.  Measured on 600 tokens of
     the two-layer test model: about 50 such events (3e-5 per rounded element), each confined to one
@@ -489,10 +490,15 @@ def prefill_both(ref, dev, X, pos0, what, via_tokens=None):
     activation times a column of the synthetic weights; over 1100 tokens the largest seen is 6e-2).
     So up to 1 + T/8 tokens may be off the tight bound, by up to 0.2, and the last token's outputs
     are compared loosely when it is among them; an error of the code would show on every token, or
-    be of order one.  All other tokens' rows match to 1e-5 plus one f16 step."""
+    be of order one.  All other tokens' rows match to 1e-5 plus one f16 step.
+    all_logits: through forward_all_logits instead -- every position's logits and greedy token."""
     T = X.shape[0]
-    got_logits, got_tok = dev.prefill(X, pos0) if via_tokens is None else dev.prefill_tokens(via_tokens[0], via_tokens[1], pos0)
-    got_hidden = dev.hidden()
+    if all_logits:
+        got_all, got_toks = dev.forward_all_logits(X, pos0) if via_tokens is None else \
+            dev.forward_all_logits(None, pos0, tok_embd=via_tokens[0], tokens=via_tokens[1])
+    else:
+        got_logits, got_tok = dev.prefill(X, pos0) if via_tokens is None else dev.prefill_tokens(via_tokens[0], via_tokens[1], pos0)
+        got_hidden = dev.hidden()
     rows = [dev.kv_read(l, pos0, T) for l in range(dev.n_layer)]
     flagged = set()
 
@@ -510,6 +516,21 @@ def prefill_both(ref, dev, X, pos0, what, via_tokens=None):
         return out
 
     ref.kv_hook = hook
+    if all_logits:
+        want_all, _ = R.forward(ref, X, pos0, all_logits=True)
+        ref.kv_hook = None
+        assert len(flagged) <= 1 + T // 8, f"{what}: {len(flagged)} of {T} tokens off the tight bound: {sorted(flagged)}"
+        want_all = np.asarray(want_all, np.float64).reshape(T, -1)
+        for t in range(T):
+            tol = 0.2 if pos0 + t in flagged else TOL
+            err = np.abs(got_all[t].astype(np.float64) - want_all[t]).max() / (np.abs(want_all[t]).max() + 1e-30)
+            assert np.isfinite(got_all[t]).all() and err <= tol, f"{what}: logits of position {pos0 + t}: max error {err:.3e}"
+            top = np.sort(want_all[t])[-2:]
+            if top[1] - top[0] > tol * np.abs(want_all[t]).max():
+                assert int(got_toks[t]) == R.argmax(want_all[t]), f"{what}: greedy token of position {pos0 + t}"
+            assert int(got_toks[t]) == R.argmax(got_all[t]), f"{what}: device argmax of its own logits, position {pos0 + t}"
+        say(what, f"{T} positions from {pos0}: flagged {sorted(flagged)}, tokens {[int(v) for v in got_toks]}")
+        return
     want_logits, want_hidden = R.forward(ref, X, pos0)
     ref.kv_hook = None
     assert len(flagged) <= 1 + T // 8, f"{what}: {len(flagged)} of {T} tokens off the tight bound: {sorted(flagged)}"
@@ -667,6 +688,49 @@ def test_hidden_states_of_every_token(be, n_tokens):
             dev.hidden_states(rng.standard_normal((321, 256)).astype(f32))   # beyond the cache
         with pytest.raises(OgmError):
             dev.hidden_states(tok_embd=QuantMatrix(embd_raw, Q6_K, 256, 320), tokens=np.array([320], np.uint32))
+    finally:
+        dev.close()
+
+
+@pytest.mark.parametrize("types", [(Q4_K, Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0, Q8_0, Q8_0), (Q5_K, Q5_K, Q6_K, Q5_K)])
+@pytest.mark.parametrize("n_draft", [1, 4, 8, 20])
+def test_forward_all_logits_of_a_verify_batch(be, types, n_draft):
+    """forward_all_logits (arch/mod.rs:2110-2132; speculative_next, generate.rs:1618-1674): a prompt, then the last
+    accepted token plus a draft as one batch; the logits and the greedy token of EVERY position against the CPU
+    restatement; then the draft is rejected from its second token on and the next batch overwrites those rows."""
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
+                          types=types, max_ctx=96, seed=61, attn_norm_scale=TAME.get(types[0], 1.0))
+    try:
+        prefill_both(ref, dev, rng.standard_normal((30, 256)).astype(f32), 0, f"types {types} prompt")
+        X = rng.standard_normal((1 + n_draft, 256)).astype(f32)
+        prefill_both(ref, dev, X, 30, f"types {types} verify {1 + n_draft}", all_logits=True)
+        for l in range(dev.n_layer):   # accept one drafted token: positions 30, 31 stay
+            del ref.k_cache[l][32:], ref.v_cache[l][32:]
+        prefill_both(ref, dev, rng.standard_normal((3, 256)).astype(f32), 32, f"types {types} next batch", all_logits=True)
+        step_both(ref, dev, rng.standard_normal(256).astype(f32), 35, f"types {types} then a decode step")
+    finally:
+        dev.close()
+
+
+def test_forward_all_logits_from_token_ids_and_limits(be):
+    """The same from token ids (the embedding rows dequantized on the device), and the call's limits."""
+    import oracle
+    from orangu_amd import OgmError, QuantMatrix
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=1,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=80, seed=62, attn_norm_scale=TAME[Q4_K])
+    try:
+        emb_raw = synth_weights(Q8_0, 256, 320, seed=63)
+        emb = QuantMatrix(emb_raw, Q8_0, 256, 320)
+        table = oracle.dequantize(Q8_0, emb_raw, 320 * 256).reshape(320, 256)
+        tokens = rng.integers(0, 320, 6).astype(np.uint32)
+        prefill_both(ref, dev, table[tokens], 0, "token ids", via_tokens=(emb, tokens), all_logits=True)
+        with pytest.raises(OgmError):
+            dev.forward_all_logits(rng.standard_normal((65, 256)).astype(f32), 0)        # more than 64 positions
+        with pytest.raises(OgmError):
+            dev.forward_all_logits(rng.standard_normal((10, 256)).astype(f32), 75)       # beyond the cache
+        with pytest.raises(OgmError):
+            dev.forward_all_logits(None, 0, tok_embd=emb, tokens=np.array([1, 400], np.uint32))   # id outside the vocabulary
+        be.evict(emb)
     finally:
         dev.close()
 
