@@ -293,7 +293,8 @@ struct GemmFkParams {
   const float *ad;                      // [n_tokens][nsb]
   const uint16_t *bs16;                 // [n_tokens][nsb][16] f16 bits (Q4_K / Q5_K)
   uint32_t in_dim, n_tokens, nsb, nct;
-  uint32_t rb_per_wg;                   // row blocks a workgroup takes (1 or 2)
+  uint32_t c_shift, r_shift;            // log2 of the tiling's blocks per tile row (4, 2 or 1) and rows per tile (16, 32, 64)
+  uint32_t rb_per_wg;                   // groups of 16 rows a workgroup takes (1 or 2)
 };
 
 #define FK_Q4K 0
@@ -320,13 +321,14 @@ __device__ __forceinline__ constexpr uint32_t fk_tile_bytes() {
   return KIND == FK_Q4K ? 64u * 144u : KIND == FK_Q5K ? 64u * 176u : 64u * 210u;
 }
 
-// rb_base: the row block's first tile; s: the super-block; r16: the lane's row in the block; hn: its half of
-// the super-block; lh: its half of every run.
+// rb_base: the row block's first tile; s: the super-block; rt: the lane's row in the tile; hn: its half of the
+// super-block; lh: its half of every run; cr: the tiling's shifts, c_shift | r_shift << 8.
 template <int KIND>
-__device__ __forceinline__ void fk_load(FkRegs<KIND> &r, const uint8_t *rb_base, uint32_t s, uint32_t r16, uint32_t hn,
-                                        uint32_t lh, const uint16_t *bs_tok) {
-  const uint8_t *tile = rb_base + (size_t)(s >> 2) * fk_tile_bytes<KIND>();
-  const uint32_t lt = (s & 3u) * 16u + r16;
+__device__ __forceinline__ void fk_load(FkRegs<KIND> &r, const uint8_t *rb_base, uint32_t s, uint32_t rt, uint32_t hn,
+                                        uint32_t lh, const uint16_t *bs_tok, uint32_t cr) {
+  const uint32_t c_shift = cr & 0xFFu, r_shift = cr >> 8;
+  const uint8_t *tile = rb_base + (size_t)(s >> c_shift) * fk_tile_bytes<KIND>();
+  const uint32_t lt = ((s & ((1u << c_shift) - 1u)) << r_shift) + rt;
   const uint8_t *b = tile + lt * 16u;
   if constexpr (KIND == FK_Q6K) {
 #pragma unroll
@@ -405,11 +407,15 @@ __global__ __launch_bounds__(TS == 8 ? 1024 : 512) void ogm_gemm_fk_kernel(GemmF
   if (bid >= p.wg_end[0]) m = 1;
   if (bid >= p.wg_end[1]) m = 2;
   if (bid >= p.wg_end[2]) m = 3;
-  const uint32_t rb = bid - (m == 0 ? 0u : m == 1 ? p.wg_end[0] : m == 2 ? p.wg_end[1] : p.wg_end[2]);
+  // g16: the group of 16 rows within its matrix; a row block of the tiling holds 1, 2 or 4 such groups
+  const uint32_t g16 = bid - (m == 0 ? 0u : m == 1 ? p.wg_end[0] : m == 2 ? p.wg_end[1] : p.wg_end[2]);
   const uint8_t *wt = m == 0 ? p.wt[0] : m == 1 ? p.wt[1] : m == 2 ? p.wt[2] : p.wt[3];
   float *y = m == 0 ? p.y[0] : m == 1 ? p.y[1] : m == 2 ? p.y[2] : p.y[3];
   const uint32_t out_dim = m == 0 ? p.out_dim[0] : m == 1 ? p.out_dim[1] : m == 2 ? p.out_dim[2] : p.out_dim[3];
-  const uint8_t *rb_base = wt + (size_t)rb * p.nct * fk_tile_bytes<KIND>();
+  const uint32_t sub_shift = p.r_shift - 4u;
+  const uint8_t *rb_base = wt + (size_t)(g16 >> sub_shift) * p.nct * fk_tile_bytes<KIND>();
+  const uint32_t rt = 16u * (g16 & ((1u << sub_shift) - 1u)) + r16;   // the lane's row in its tile
+  const uint32_t cr = p.c_shift | (p.r_shift << 8);
 
   // ---- the activations: 16-byte pieces of the token-major rows, requested first ...
   const uint32_t ppt = p.in_dim / 16u, n_piece = T * ppt;
@@ -426,7 +432,7 @@ __global__ __launch_bounds__(TS == 8 ? 1024 : 512) void ogm_gemm_fk_kernel(GemmF
   const uint32_t n_my = (nsb - wave + n_wave - 1u) / n_wave;
   const uint16_t *bs_tok = K4 ? p.bs16 + (size_t)min(ts, T - 1u) * nsb * 16u : nullptr;
   FkRegs<KIND> A, B;
-  fk_load<KIND>(A, rb_base, sb_of(0), r16, hn, lh, bs_tok);
+  fk_load<KIND>(A, rb_base, sb_of(0), rt, hn, lh, bs_tok, cr);
   __builtin_amdgcn_sched_barrier(0);
 
   auto park = [&](uint32_t idx, const fk_u32x4 &v) {
@@ -565,10 +571,10 @@ __global__ __launch_bounds__(TS == 8 ? 1024 : 512) void ogm_gemm_fk_kernel(GemmF
 
   for (uint32_t k = 0; k < n_my; k += 2) {   // wave-uniform branches
     const bool has_b = k + 1 < n_my;
-    if (has_b) fk_load<KIND>(B, rb_base, sb_of(k + 1), r16, hn, lh, bs_tok);
+    if (has_b) fk_load<KIND>(B, rb_base, sb_of(k + 1), rt, hn, lh, bs_tok, cr);
     process(A, sb_of(k));
     if (has_b) {
-      if (k + 2 < n_my) fk_load<KIND>(A, rb_base, sb_of(k + 2), r16, hn, lh, bs_tok);
+      if (k + 2 < n_my) fk_load<KIND>(A, rb_base, sb_of(k + 2), rt, hn, lh, bs_tok, cr);
       process(B, sb_of(k + 1));
     }
   }
@@ -577,7 +583,7 @@ __global__ __launch_bounds__(TS == 8 ? 1024 : 512) void ogm_gemm_fk_kernel(GemmF
   // ---- one lane per (token, row) of the team's row block: the row's terms in ascending order, one accumulator
   for (uint32_t i = tid - team * (n_wave * 64u); i < 16u * T; i += n_wave * 64u) {
     const uint32_t t = i >> 4, r = i & 15u;
-    const uint32_t row = rb * 16u + r;
+    const uint32_t row = g16 * 16u + r;
     if (row < out_dim && !idle) {
       float acc = 0.0f;
       if constexpr (TWO) acc = fk_ordered_sum<true>(acc, l_tmin + t * 16u + r, nsb, TS * 16u);
@@ -593,11 +599,11 @@ static size_t fk_lds_bytes(uint32_t ggml_type, uint32_t in_dim, uint32_t ts, int
   return (size_t)in_dim * ts + nsb * ts * 4u + rb_per_wg * arrays * nsb * ts * 16u * 4u;
 }
 
-// Shapes the kernel takes: Q4_K, Q5_K and Q6_K rows of a multiple of four super-blocks (tiles of 16 rows), 2 to
-// 16 tokens, activations and term tables within a workgroup's LDS.
+// Shapes the kernel takes: Q4_K, Q5_K and Q6_K, 2 to 16 tokens, activations and term tables within a workgroup's
+// LDS (any row length: a workgroup takes 16 rows of a tile of 16, 32 or 64).
 bool ogm_gemv_mma_eligible(uint32_t ggml_type, uint32_t in_dim, uint32_t n_tokens, int gemm_order) {
   if (ggml_type != OGM_Q4_K && ggml_type != OGM_Q5_K && ggml_type != OGM_Q6_K) return false;
-  if (in_dim == 0 || in_dim % 1024u != 0 || n_tokens < 2u || n_tokens > 16u) return false;
+  if (in_dim == 0 || in_dim % 256u != 0 || n_tokens < 2u || n_tokens > 16u) return false;
   if ((uint64_t)n_tokens * in_dim >= (1ull << 31)) return false;
   return fk_lds_bytes(ggml_type, in_dim, n_tokens <= 8u ? 8u : 16u, gemm_order) <= 160u * 1024u;
 }
@@ -613,7 +619,10 @@ hipError_t ogm_launch_gemv_mma(const OgmGemvArgs &a, hipStream_t stream, const c
   p.in_dim = a.in_dim;
   p.n_tokens = a.n_tokens;
   p.nsb = a.in_dim / 256u;
-  p.nct = p.nsb / 4u;
+  const OgmTiling tl = ogm_tiling_for(p.nsb, a.out_dim);
+  p.nct = tl.nct;
+  p.c_shift = tl.C == 4u ? 2u : tl.C == 2u ? 1u : 0u;
+  p.r_shift = tl.R == 16u ? 4u : tl.R == 32u ? 5u : 6u;
   uint32_t n_wg = 0;
   for (uint32_t m = 0; m < OGM_GEMV_MAX_MATS; m++) {
     if (m <= a.n_extra) {

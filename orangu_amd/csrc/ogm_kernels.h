@@ -96,8 +96,8 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
 bool ogm_gemm_ft_eligible(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens,
                           uint32_t min_rows);
 hipError_t ogm_launch_gemm_ft(const OgmGemmArgs &a, int gemm_order, hipStream_t stream, const char **kernel_name);
-// Two to sixteen tokens over Q4_K / Q5_K / Q6_K rows of a multiple of 1024 inputs (ogm_gemm_ft.hip): one workgroup
-// per row block of 16 rows, waves on different column tiles, products on the matrix cores, either float order.
+// Two to sixteen tokens over Q4_K / Q5_K / Q6_K (ogm_gemm_ft.hip): one workgroup per group of 16 rows, waves on
+// different super-blocks, products on the matrix cores, either float order.
 bool ogm_gemv_mma_eligible(uint32_t ggml_type, uint32_t in_dim, uint32_t n_tokens, int gemm_order);
 hipError_t ogm_launch_gemv_mma(const OgmGemvArgs &a, hipStream_t stream, const char **kernel_name);
 

@@ -871,7 +871,7 @@ struct GemvParams {
   int32_t *dump_isum, *dump_imin;
   uint32_t in_dim, upr;            // upr = blocks per row
   uint32_t n_tokens;
-  uint32_t C, nct;                // tile shape: C blocks x R rows, nct = upr / C column tiles
+  uint32_t C, nct;                // tile shape: C blocks x R rows, nct = ceil(upr / C) column tiles
   uint32_t lane_acc;              // formats of several terms a block, tiles one block wide, one wave: see gemv_lane_acc
 };
 
@@ -880,7 +880,8 @@ __host__ __device__ constexpr int n_term_arrays() {
   return (GEMM_ORDER && F::HAS_MIN && F::TYPE != OGM_Q2_K) ? 2 : 1;   // Q4_K, Q5_K: the min pass first
 }
 
-static const size_t OGM_LDS_BUDGET = 64 * 1024;   // what a launch aims for: batches and row blocks are cut to fit
+static const size_t OGM_LDS_BUDGET = 80 * 1024;   // what a launch aims for (two workgroups to a compute unit): batches are cut to fit
+static const size_t OGM_LDS_UNASKED = 64 * 1024;  // what a kernel gets without asking (hipFuncAttributeMaxDynamicSharedMemorySize)
 static const size_t OGM_LDS_MAX = 160 * 1024;     // what a workgroup can have when even one token of one row block needs more
 
 // Dynamic LDS bytes of one workgroup.
@@ -968,8 +969,8 @@ __global__ __launch_bounds__((SINGLE && !DUMP) ? F::MAX_THREADS_SINGLE : F::MAX_
   const uint32_t lane = tid & 63u, wave = tid >> 6, n_wave = nthr >> 6;
   const uint32_t T = SINGLE ? 1u : p.n_tokens;
   const uint32_t upr = UPR ? (uint32_t)UPR : p.upr;
-  const uint32_t C = UPR ? ((UPR % 4 == 0) ? 4u : ((UPR % 2 == 0) ? 2u : 1u)) : p.C;
-  const uint32_t R = 64u / C, nct = upr / C;
+  const uint32_t C = UPR ? ((UPR % 4 == 0) ? 4u : ((UPR % 2 == 0) ? 2u : 1u)) : p.C;   // (the UPR variants: 16, 56, 128)
+  const uint32_t R = 64u / C, nct = UPR ? upr / C : p.nct;
   const uint32_t xch = upr * F::XPIECES;           // 16-byte chunks of q per token
   const uint32_t n_scale = upr * (F::ELEMS / F::ACT_GROUP);
   const uint32_t term_stride = upr * R * F::TERMS;  // floats per token in the term table
@@ -1083,7 +1084,11 @@ __global__ __launch_bounds__((SINGLE && !DUMP) ? F::MAX_THREADS_SINGLE : F::MAX_
   }
   // ---- tiles of this wave
   for (; it < n_items; it += n_wave) {
-    const uint32_t col = it * C + c_local;  // block index within the row
+    // block index within the row; a lane of a padded column tile past the row's last block works on that block
+    // again (its own unit is zeros) and leaves nothing behind
+    const uint32_t col_own = it * C + c_local;
+    const bool live = col_own < upr;
+    const uint32_t col = live ? col_own : upr - 1u;
     // many tokens: unpack the block once where that is the expensive part (Q6_K; measured at
     // 4096 -> 128256: 159 us against 182 us at 8 tokens, but 112 us against 97 us at 4)
     [[maybe_unused]] typename UnpackedOf<F, UNPACK>::type unp;
@@ -1101,6 +1106,7 @@ __global__ __launch_bounds__((SINGLE && !DUMP) ? F::MAX_THREADS_SINGLE : F::MAX_
         // a block leaves several terms, in the order the row adds them
         float tt[F::TERMS];
         F::template terms<UPR>(cur, a, col, tt);
+        if (!live) continue;
         if (p.lane_acc) {   // this lane's row, the column tiles in order: the row's own sequence of additions
           float acc = l_term[t * 64u + lane];
 #pragma unroll
@@ -1113,6 +1119,7 @@ __global__ __launch_bounds__((SINGLE && !DUMP) ? F::MAX_THREADS_SINGLE : F::MAX_
         for (int g = 0; g < F::TERMS; g++) dst[g * R] = tt[g];
         continue;
       }
+      if (!live) continue;
       const float ad = a.d[col];  // one activation scale per block (per-32 and per-256 alike)
       const size_t slot = (size_t)t * term_stride + col * R + r_local;
       if (GEMM_ORDER) {
@@ -1202,14 +1209,25 @@ uint32_t ogm_gemv_max_tokens(uint32_t ggml_type, uint32_t in_dim, int gemm_order
   }
 }
 
-// Waves per workgroup: the largest divisor of the row block's tile count up to 8 (measured on
-// MI355X: 4 waves x 1 tile at 4096 -> 14336, 7 waves x 2 tiles at 14336 -> 4096 beat 14 x 1).
+// Waves per workgroup: a wave takes every waves-th tile of the row block.  Up to 8 (16 for the small tiles of the
+// per-32 formats): the count that divides the tile count where one exists in the upper half of that range
+// (measured on MI355X: 4 waves x 1 tile at 4096 -> 14336, 7 waves x 2 tiles at 14336 -> 4096 beat 14 x 1), else the
+// fewest waves that give the shortest chain of tiles per wave -- a row of 43 blocks (11008 inputs) has no divisor
+// but 1, and one wave walking 43 tiles took 52 us where eight take a fraction of that.
 static uint32_t pick_waves(uint32_t nct, uint32_t wg_waves, int max_threads, uint32_t auto_cap = 8) {
   uint32_t waves = wg_waves;
   if (waves == 0) {
-    waves = 1;
-    for (uint32_t w = 2; w <= auto_cap && w <= nct; w++)
-      if (nct % w == 0) waves = w;
+    const uint32_t cap = auto_cap < nct ? auto_cap : nct;
+    waves = 0;
+    for (uint32_t w = cap; w >= 1u && 2u * w > cap; w--)
+      if (nct % w == 0) {
+        waves = w;
+        break;
+      }
+    if (waves == 0) {
+      const uint32_t chain = (nct + cap - 1u) / cap;
+      waves = (nct + chain - 1u) / chain;
+    }
   }
   if (waves > nct) waves = nct;
   if (waves > (uint32_t)max_threads / 64) waves = max_threads / 64;
@@ -1228,7 +1246,7 @@ static void launch_single(const GemvParams &p, dim3 g, dim3 b, size_t lds, hipSt
     hipLaunchKernelGGL((ogm_gemv_kernel<F, 128, true, false, false>), g, b, lds, stream, p);
   else {
     // (a long row of an odd number of blocks -- 64-row tiles one block wide -- stages more than a launch gets unasked)
-    if (lds > OGM_LDS_BUDGET &&
+    if (lds > OGM_LDS_UNASKED &&
         hipFuncSetAttribute((const void *)ogm_gemv_kernel<F, 0, true, false, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return;   // the launch below then fails and reports it
@@ -1275,7 +1293,7 @@ static hipError_t launch_t(const OgmGemvArgs &a, hipStream_t stream) {
   const size_t lds = lane_acc ? gemv_lds_bytes_lane_acc<F>(a.in_dim, a.n_tokens) : gemv_lds_bytes<F, GEMM_ORDER>(a.in_dim, a.n_tokens);
   if (lds > OGM_LDS_MAX) return hipErrorInvalidValue;
   auto launch = [&](void (*kernel)(GemvParams), dim3 g_, dim3 b_) -> hipError_t {
-    if (lds > OGM_LDS_BUDGET) {
+    if (lds > OGM_LDS_UNASKED) {
       const hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess) return e;
     }

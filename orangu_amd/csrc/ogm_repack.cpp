@@ -62,8 +62,11 @@ extern "C" int ogm_repack_host(uint32_t ggml_type, const void *raw, size_t row_b
   const uint8_t *src = (const uint8_t *)raw;
   uint8_t *dst = (uint8_t *)repacked;
   const OgmTiling t = ogm_tiling_for(in_dim / l.block_elems, out_dim);
-  // Only the last row block can hold rows beyond out_dim: zero it first.
-  if (out_dim % t.R != 0)
+  // Zero units: rows beyond out_dim (the last row block only) and, where a row's blocks do not fill its last
+  // column tile, that tile of every row block.
+  if (t.upr % t.C != 0)
+    memset(dst, 0, (size_t)t.nrb * t.nct * l.tile_bytes);
+  else if (out_dim % t.R != 0)
     memset(dst + (size_t)(t.nrb - 1) * t.nct * l.tile_bytes, 0, (size_t)t.nct * l.tile_bytes);
   for (uint32_t o = 0; o < out_dim; o++) {
     for (uint32_t blk = 0; blk < t.upr; blk++) {

@@ -596,8 +596,7 @@ def test_medium_batch_kernel_over_several_matrices_and_extreme_ranges(be):
 def test_gemm_threshold_default():
     """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
     float order, 17 through the matrix-core GEMM.  Q4_K: 4 tokens through the GEMV kernel, 5 to 8 through the
-    row-block kernel (rows of a multiple of 1024 inputs; of other lengths the GEMV kernel up to 5 and the
-    small-batch kernel from 6), 9 to 224
+    row-block kernel, 9 to 224
     through the small-batch kernel (a matrix of few rows), 225 to 256 through the medium-batch kernel, 257
     through the tiled one; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
     many that 128 x 128 tiles outnumber the compute units has its planes built and read by the kernel whose
@@ -627,10 +626,10 @@ def test_gemm_threshold_default():
             y = b.matmul(x[:n], n, w)
             assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, want[:n], f"Q4_K, {n} tokens")
-        raw = synth_weights(Q4_K, 768, 70, seed=15)    # three super-blocks a row: no row-block kernel
+        raw = synth_weights(Q4_K, 768, 70, seed=15)    # three super-blocks a row: tiles of 64 rows, one block wide
         w3 = qm(raw, Q4_K, 768, 70)
-        x3 = np.ascontiguousarray(x[:6, :768])
-        for n, kernel in ((5, "ogm_gemv_kernel"), (6, "ogm_gemm_sb_q4k_kernel")):
+        x3 = np.ascontiguousarray(x[:9, :768])
+        for n, kernel in ((4, "ogm_gemv_kernel"), (6, "ogm_gemm_fk_kernel<Q4_K>"), (9, "ogm_gemm_sb_q4k_kernel")):
             y = b.matmul(x3[:n], n, w3)
             assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, oracle.matmul(Q4_K, raw, 768, 70, x3[:n], n), f"Q4_K of 768 inputs, {n} tokens")
