@@ -4,11 +4,11 @@
 // weights, Q4_0 and IQ4_NL 18 B / 32, Q5_0 22 B / 32, Q5_1 24 B / 32, Q2_K 84 B / 256, Q3_K 110 B / 256, Q4_K 144 B / 256,
 // Q5_K 176 B / 256, Q6_K 210 B / 256, IQ4_XS 136 B / 256; engine/quant.rs:537-871, 1350-1375).  A *tile* holds 64
 // units: R consecutive rows x C consecutive blocks, R = 64 / C.  C = 4 when a row has a multiple of four
-// blocks, and also when it has 24 or more of any count: the last column tile of a row block is then padded with
-// zero units (at most 3 in 24: a few per cent of bytes that no kernel's sums read), which keeps row blocks at 16
-// rows -- a row of 43 blocks (11008 inputs) in tiles one block wide would make row blocks of 64 rows and a
-// quarter as many workgroups in the decode GEMV.  Shorter rows of other counts take C = 2, else 1.  Tiles are
-// ordered [row block][column tile]; inside a tile the unit of (row r, block c) is lane c*R + r.
+// blocks, and also when filling its last column tile with zero units adds at most a tenth to the row (11, 19,
+// 22, 23 blocks and every count from 27 on): bytes that no kernel's sums read, which keep row blocks at 16 rows
+// -- a row of 43 blocks (11008 inputs) in tiles one block wide would make row blocks of 64 rows and a quarter as
+// many workgroups in the decode GEMV.  Other rows take C = 2, else 1.  Tiles are ordered [row block][column
+// tile]; inside a tile the unit of (row r, block c) is lane c*R + r.
 //
 // A unit is cut into 16-byte pieces plus a short tail; piece p of lane l sits at p*1024 + l*16
 // and the tails follow all pieces, lane after lane.  So
@@ -115,7 +115,8 @@ OGM_HD inline bool ogm_layout_for(uint32_t ggml_type, OgmLayout *l) {
 OGM_HD inline OgmTiling ogm_tiling_for(uint32_t upr, uint32_t out_dim) {
   OgmTiling t;
   t.upr = upr;
-  t.C = (upr % 4u == 0 || upr >= 24u) ? 4u : ((upr % 2u == 0) ? 2u : 1u);
+  const uint32_t pad = (4u - upr % 4u) % 4u;   // zero units a row would need to fill its last tile of four
+  t.C = (pad == 0 || pad * 10u <= upr) ? 4u : ((upr % 2u == 0) ? 2u : 1u);
   t.R = OGM_TILE_UNITS / t.C;
   t.nct = (upr + t.C - 1u) / t.C;
   t.nrb = (out_dim + t.R - 1) / t.R;
