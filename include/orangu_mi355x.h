@@ -433,6 +433,12 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              straight into LDS) runs: 0 = default, when the launch has more than 256 tiles of
  *                              128 rows x 128 tokens (the feeding-wave kernels unpack otherwise); 2 = whatever
  *                              the grid, from 32 tokens
+ *   "gemm_interleave"          the plane kernel with 64-row tiles that adds a super-block up between the next
+ *                              one's matrix instructions (Q4_K, Q5_K, Q6_K): 0 = default, on launches of three
+ *                              or more token tiles of 128 that leave the 128-row kernel's places under three
+ *                              quarters full and have at least 160 tiles of 64 rows (the 8B shapes' q/k/v, wo and
+ *                              down projections at 257 to 1024 tokens; their planes are built then); 1 = never;
+ *                              2 = wherever the plane kernel runs.  Same bits
  *   "gemm_one_pass"            0 = default.  1: Q4_K and Q5_K on that kernel skip the reference GEMM's separate
  *                              first pass over the mins (vecdot.rs:2229-2240) and add
  *                              ad * (d * isum - dmin * imin) per super-block, the single-token expression of

@@ -69,6 +69,7 @@ struct ogm_ctx {
   bool host_coherent = true;           // the pinned staging buffers are fine-grained (asked for by name); false once the runtime has refused
   int tune_gemv_mma = 1;               // few tokens over Q4_K / Q5_K / Q6_K on the row-block matrix-core kernel: 0 never, 1 where it measured faster, 2 wherever it can
   int tune_gemm_plane_kernel = 0;      // the all-waves-multiply kernel over planes: 0 on large grids, 2 whatever the grid
+  int tune_gemm_interleave = 0;        // the 64-row plane kernel with the f32 step between the matrix instructions: 0 by the launch's size, 1 never, 2 whenever it can
   int tune_gemm_one_pass = 0;          // 1: Q4_K / Q5_K on that kernel fold the min pass into the super-block step (f32 to rounding, not to the bit)
   int tune_prefill_chunk = 2048;       // tokens per prefill pass over the layers (fixed per model at its first prefill)
   int tune_attn_prefill_variant = 0;   // 0: by batch size; 1: the decode kernel per token and chunk; 2: the matrix-core kernel
@@ -309,6 +310,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemm_plane_kernel") == 0) {
     if (value != 0 && value != 2) return fail(ctx, OGM_ERR_INVALID, "gemm_plane_kernel must be 0 or 2");
     ctx->tune_gemm_plane_kernel = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "gemm_interleave") == 0) {
+    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_interleave must be 0, 1 or 2");
+    ctx->tune_gemm_interleave = value;
     return OGM_OK;
   }
   if (strcmp(key, "gemm_one_pass") == 0) {
@@ -657,6 +663,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       g.sb_waves = (uint32_t)ctx->tune_gemm_sb_waves;
       g.plane_kernel = (uint32_t)ctx->tune_gemm_plane_kernel;
       g.one_pass = (uint32_t)ctx->tune_gemm_one_pass;
+      g.interleave = (uint32_t)ctx->tune_gemm_interleave;
       g.n_extra = (uint32_t)ng - 1;
       for (size_t j = 1; j < ng; j++) {
         g.extra_wt[j - 1] = tg[i + j].w->dev;
@@ -1794,11 +1801,11 @@ static int llama_matmul_rows(ogm_ctx *ctx, const ogm_weight *const *ws, float *c
 // scratch (mode `mode`, `in_dim` wide, T rows): the weights are grouped by type as in
 // llama_matmul_rows; all of them must take that mode.
 static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws, float *const *ys, size_t n,
-                                       int mode, uint32_t in_dim, uint32_t T, hipStream_t s) {
+                                       int mode, uint32_t in_dim, uint32_t T, hipStream_t s, bool xt_written = false) {
   ctx->act_mode = mode;
   ctx->act_in_dim = in_dim;
   ctx->act_tokens = T;
-  ctx->act_xt = false;   // the producers wrote the token-major buffers only
+  ctx->act_xt = xt_written;   // whether the producer also filled the tiled GEMMs' operand chunks (llama_producer_xt)
   size_t i = 0;
   while (i < n) {
     Target tg[OGM_GEMV_MAX_MATS];
@@ -1812,6 +1819,20 @@ static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws
     i = e;
   }
   return OGM_OK;
+}
+
+// Where a producer kernel of a batch (norm, SwiGLU) should also lay its int8 rows out in the operand chunks of the
+// tiled GEMMs over planes, or null: the same condition as enqueue_matmul's for its quantizer.  Saves the GEMM's own
+// relayout launch (5 us a matmul at 512 tokens of the 8B shapes).
+static int llama_producer_xt(ogm_ctx *ctx, const ogm_weight *w, int mode, uint32_t in_dim, uint32_t T, int8_t **xt) {
+  *xt = nullptr;
+  if (mode != OGM_ACT_PER_256 || T < 32 || in_dim % 256u != 0 || ctx->tune_plane_cache_mb <= 0 ||
+      ogm_gemm_plane_bytes(w->ggml_type, w->in_dim, w->out_dim) == 0 ||
+      (uint64_t)((T + 31u) & ~31u) * in_dim >= (1ull << 32))
+    return OGM_OK;
+  const int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(in_dim, T));
+  if (rc == OGM_OK) *xt = (int8_t *)ctx->xh.p;
+  return rc;
 }
 
 // x += delta, RMSNorm, and the matmuls over the normed rows: the norm kernel quantizes its own
@@ -1834,10 +1855,11 @@ static int llama_norm_matmul_rows(ogm_ctx *ctx, ogm_llama *m, const ogm_weight *
         ym[k++] = ys[i];
       }
     if (k == 0) continue;
-    HIPCHK(ctx, ogm_launch_norm_quant(mode, m->pf.x, first ? delta : nullptr, norm_w, c.n_embd, c.rms_eps, nullptr,
-                                      act_view(ctx, c.n_embd, mode, 0), s, T));
+    OgmActDev act = act_view(ctx, c.n_embd, mode, 0);
+    if ((rc = llama_producer_xt(ctx, wm[0], mode, c.n_embd, T, &act.xt)) != OGM_OK) return rc;
+    HIPCHK(ctx, ogm_launch_norm_quant(mode, m->pf.x, first ? delta : nullptr, norm_w, c.n_embd, c.rms_eps, nullptr, act, s, T));
     first = false;
-    if ((rc = llama_matmul_quantized_rows(ctx, wm, ym, k, mode, c.n_embd, T, s)) != OGM_OK) return rc;
+    if ((rc = llama_matmul_quantized_rows(ctx, wm, ym, k, mode, c.n_embd, T, s, act.xt != nullptr)) != OGM_OK) return rc;
   }
   return OGM_OK;
 }
@@ -1902,8 +1924,10 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
     const ogm_weight *wd[1] = {L.w_down};
     const int mode_d = act_mode_for(L.w_down->ggml_type, T, 0);
     if ((rc = ensure_act(ctx, c.n_ff, T)) != OGM_OK) return rc;
-    HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, P.gate, P.up, c.n_ff, nullptr, act_view(ctx, c.n_ff, mode_d, 0), s, T));
-    if ((rc = llama_matmul_quantized_rows(ctx, wd, y1, 1, mode_d, c.n_ff, T, s)) != OGM_OK) return rc;
+    OgmActDev act_d = act_view(ctx, c.n_ff, mode_d, 0);
+    if ((rc = llama_producer_xt(ctx, L.w_down, mode_d, c.n_ff, T, &act_d.xt)) != OGM_OK) return rc;
+    HIPCHK(ctx, ogm_launch_swiglu_quant(mode_d, P.gate, P.up, c.n_ff, nullptr, act_d, s, T));
+    if ((rc = llama_matmul_quantized_rows(ctx, wd, y1, 1, mode_d, c.n_ff, T, s, act_d.xt != nullptr)) != OGM_OK) return rc;
     delta = P.proj;
   }
   ctx->act_mode = -1;   // the activation scratch was the matmuls'

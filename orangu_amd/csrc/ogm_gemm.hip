@@ -14,6 +14,7 @@
 //   * ogm_gemm_dma_kernel: the same tile over planes built once per matrix, all waves multiply;
 //   * ogm_gemm_flat_kernel: the per-32 types (f16 operands, one block per accumulator).
 #include <hip/hip_runtime.h>
+#include <type_traits>
 
 #include "ogm_kernels.h"
 #include "ogm_layout.h"
@@ -1079,6 +1080,396 @@ __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaPara
 }
 
 // ------------------------------------------------------------------------------------------
+// The same multiplication on 64-row tiles, for launches too small to fill the 128-row kernel's places (its grid
+// wants 384 tiles of 128 x 128; a 4096 x 4096 matrix at 512 tokens has 128), with the f32 step of a super-block
+// issued *between* the matrix instructions of the next one.  A SIMD runs a matrix instruction for 32 clocks; the
+// wave that issued it can issue about five vector instructions behind it for nothing (measured: eight matrix
+// instructions 128 ns, with five dependent v_fma behind each 131 ns, with eight 166 ns), while vector work that
+// waits for the end of a run of matrix instructions is paid in full: a workgroup that has a compute unit to itself
+// has no second wave on its SIMDs to hide it behind.  The step acc += ad * (d * isum) is five vector instructions
+// per output: one output per matrix instruction.  For that the planes' sums live in two register sets, one filled
+// while the other is added up, which a wave tile of 32 rows x 64 tokens leaves room for (2 sets x 64 + 32 of y).
+// On grids that fill the 128-row kernel this one is slower (4096 -> 14336 at 512 / 2048 tokens: 115 / 375 us
+// against 98 / 322): a step of four matrix instructions a wave carries the same waits, barrier and loads as one
+// of eight.
+//
+//   workgroup  256 threads = 4 waves; 64 rows x 128 tokens; wave w: rows 32 (w & 1) .. + 31, tokens
+//              64 (w >> 1) .. + 63.  Two workgroups share a compute unit (67 KiB of LDS each).
+//   step       32 weights of k: the row block's two planes (4 KiB, one piece of 1 KiB per wave) and
+//              four token blocks of activations (1 KiB each, one per wave), by load-to-LDS, issued behind
+//              the step's first matrix instruction
+//   ring       eight steps in LDS = the steps of a super-block (step kk of any super-block sits in slot kk:
+//              every LDS address of the loop is a constant), six in flight; one wait + barrier per step
+//   tables     per super-block the tokens' activation scales and the rows' header words, three slots:
+//              the one being added up, the one being multiplied, the one arriving
+//   LDS reads  of a step, in issue order: [header word], four tokens' ad, h plane, two token blocks,
+//              l plane -- issued one step ahead, between the matrix instructions, waited for by count
+//   first pass (Q4_K, Q5_K) two super-blocks in turn: the matrix instructions of the next are issued before the
+//              vector work of this one
+// Same arithmetic and f32 order as ogm_gemm_dma_kernel; bit-identical results.
+#define GX_NW 4u
+#define GX_ROWS 64u
+#define GX_TOK 128u
+#define GX_RING 8u
+#define GX_AHEAD (GX_RING - 1u)
+#define GX_SLOT 8192u                 // a step's planes (4 KiB) and activations (4 KiB)
+#define GX_TAB (GX_RING * GX_SLOT)
+#define GX_TAB_SLOT 1024u             // 128 ad | 64 header words | 256 bytes that absorb wave 3's load
+#define GX_LDS_BYTES (GX_TAB + 3u * GX_TAB_SLOT)
+// timing experiments only (results are wrong with any of these set)
+#ifndef GX_ABL_NOEPI
+#define GX_ABL_NOEPI 0   // the f32 step left out of the loop
+#endif
+#ifndef GX_ABL_NOPASS1
+#define GX_ABL_NOPASS1 0
+#endif
+#ifndef GX_ABL_NOMFMA
+#define GX_ABL_NOMFMA 0
+#endif
+#ifndef GX_ABL_NODMA
+#define GX_ABL_NODMA 0
+#endif
+#if GX_ABL_NOMFMA
+#define GX_MFMA(A, B, C) (C)
+#else
+#define GX_MFMA(A, B, C) __builtin_amdgcn_mfma_i32_32x32x32_i8(A, B, C, 0, 0, 0)
+#endif
+#define GX_SYNC(N) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory")
+#define GX_PIN() __builtin_amdgcn_sched_barrier(0)
+#define GX_WAITN(N) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory")
+
+template <int KIND>
+__global__ __launch_bounds__(64 * GX_NW, 2) void ogm_gemm_dmx_kernel(GemmDmaParams p) {
+  constexpr uint32_t NW = GX_NW, ROWS = GX_ROWS, SLOT = GX_SLOT, TAB = GX_TAB, TAB_SLOT = GX_TAB_SLOT;
+  constexpr bool Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K, Q6 = KIND == GP_Q6K;
+  static_assert(Q45 || Q6, "two-plane types only");
+  constexpr uint32_t TILE_BYTES = KIND == GP_Q4K ? 9216u : Q5 ? 11264u : 13440u;
+  constexpr uint32_t AHEAD = GX_AHEAD, PER = 2u;   // loads a wave issues per step
+  extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  const uint32_t rs = wave & 1u, th = wave >> 1;   // row slice of 32, token half
+  // token tiles of one row tile go to one XCD back to back (see ogm_gemm_dma_kernel)
+  uint32_t tok_tile = blockIdx.x, row_tile = blockIdx.y;
+  {
+    const uint32_t nt = gridDim.x, lin = blockIdx.y * nt + blockIdx.x;
+    if (lin < (gridDim.y & ~7u) * nt) {
+      const uint32_t j = lin >> 3;
+      tok_tile = j % nt;
+      row_tile = (j / nt) * 8u + (lin & 7u);
+    }
+  }
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + ROWS - 1u) / ROWS;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.planes = p.extra_planes[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = tok_tile * GX_TOK, r0 = row_tile * ROWS;
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
+  };
+
+  float16v y[2];
+#pragma unroll
+  for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) y[tb][r] = 0.0f;
+
+  if constexpr (Q45 && !GX_ABL_NOPASS1) {
+    // pass 1 of gemm_k_q4_k: acc -= (ad * dmin) * sum_j m_j * bsum_j over all super-blocks first
+    // (vecdot.rs:2226-2240), as in ogm_gemm_dma_kernel, for this wave's two token blocks
+    const uint32_t row = min(r0 + 32u * rs + l32, p.out_dim - 1u);
+    const uint32_t uo = (row >> p.r_shift) * p.nct * TILE_BYTES + (row & ((1u << p.r_shift) - 1u)) * 16u;
+    float *ad_all = (float *)lds;   // [nsb][128]
+    {
+      // element i of the tile's [128 tokens][nsb] block goes to [su][token]; eight loads in flight a thread, and the
+      // (token, su) of i + 256 from those of i without dividing again
+      const uint32_t total = GX_TOK * p.nsb, dq = (64u * NW) / p.nsb, dr = (64u * NW) % p.nsb;
+      uint32_t k = tid / p.nsb, su = tid - k * p.nsb;
+      for (uint32_t i0 = tid; i0 < total; i0 += 8u * 64u * NW) {
+        float v[8];
+        uint32_t dst[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; j++) {
+          const bool in = i0 + j * 64u * NW < total;
+          dst[j] = in ? su * GX_TOK + k : 0xFFFFFFFFu;
+          v[j] = in ? p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + su] : 0.0f;
+          k += dq;
+          su += dr;
+          if (su >= p.nsb) {
+            su -= p.nsb;
+            k++;
+          }
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; j++)
+          if (dst[j] != 0xFFFFFFFFu) ad_all[dst[j]] = v[j];
+      }
+    }
+    __syncthreads();
+    float16v zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.0f;
+    uint32_t tk[2];
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++) tk[tb] = min(t0 + 64u * th + 32u * tb + l32, p.n_tokens - 1u) * p.nsb;
+    const float side_scale = lh ? 1.0f : 64.0f;
+    // Two super-blocks in turn (sets X and Y): the matrix instructions of the next one are issued before the vector
+    // work of this one, and each set's header and token sums are loaded two super-blocks ahead.
+    uint4 hdX, hdY;
+    half8 b2X[2], b2Y[2];
+    float16v imX[2], imY[2];
+    float dmX = 0.0f, dmY = 0.0f;
+    auto load = [&](uint32_t su, uint4 &hd, half8(&b2)[2]) {
+      const uint32_t sn = min(su, p.nsb - 1u);   // past the end: loaded again, never used
+      hd = *(const uint4 *)(p.wt + (uo + sb_off(sn)));
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++) b2[tb] = *(const half8 *)(p.bs16 + ((tk[tb] + sn) * 16u + 8u * lh));
+    };
+    auto stage = [&](const uint4 &hd, const half8(&b2)[2], float16v(&im)[2], float &dm) {
+      uint32_t mna, mnb;
+      q4k_mins(hd, mna, mnb);
+      const half8 a1 = side_operand(mna, mnb, side_scale);
+      dm = gm_f16_bits_to_f32(hd.x >> 16);
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++) im[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b2[tb], a1, zero, 0, 0, 0);
+    };
+    auto consume = [&](uint32_t su, const float16v(&im)[2], float dm) {
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++) {
+        const float *adp = &ad_all[su * GX_TOK + 64u * th + 32u * tb + 4u * lh];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          const float4 a4 = *(const float4 *)(adp + 8 * q4);
+          const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+          for (int e = 0; e < 4; e++) y[tb][4 * q4 + e] -= a4v[e] * dm * im[tb][4 * q4 + e];
+        }
+      }
+    };
+    load(0u, hdX, b2X);
+    load(1u, hdY, b2Y);
+    stage(hdX, b2X, imX, dmX);
+    load(2u, hdX, b2X);
+    for (uint32_t su = 0; su < p.nsb; su += 2u) {
+      const bool two = su + 1u < p.nsb;
+      if (two) {
+        stage(hdY, b2Y, imY, dmY);
+        load(su + 3u, hdY, b2Y);
+      }
+      GX_PIN();
+      consume(su, imX, dmX);
+      GX_PIN();
+      if (two) {
+        if (su + 2u < p.nsb) {
+          stage(hdX, b2X, imX, dmX);
+          load(su + 4u, hdX, b2X);
+        }
+        GX_PIN();
+        consume(su + 1u, imY, dmY);
+        GX_PIN();
+      }
+    }
+    __syncthreads();   // the table's LDS becomes the ring
+  }
+
+  // ---------------- the products
+  // per step wave w fetches piece w of the row block's planes ((half of k, plane) = (w >> 1, w & 1): 64 rows x 16
+  // bytes) and token block w of the activations.  The ring has as many slots as a super-block has steps: step kk of
+  // any super-block sits in slot kk, so every LDS address of the loop is a constant.
+  static_assert(GX_RING == 8u, "the ring's slots are the steps of a super-block");
+  uint32_t w_src = row_tile * p.nsb * 8u * 4096u + wave * 1024u + lane * 16u;   // + 4096 per step
+  uint32_t x_src = min((t0 >> 5) + wave, (p.n_tokens - 1u) >> 5) * (p.in_dim / 32u) * 1024u + lane * 16u;   // + 1024 per step
+  const uint32_t w_dst = wave * 1024u, x_dst = 4096u + wave * 1024u;
+  // tables: waves 0, 1 fetch 64 tokens' ad each, wave 2 the header words of the 64 rows (wave 3 the same again,
+  // into spare bytes: every wave has the same number of loads in flight)
+  uint32_t tab_src;
+  if (wave < 2u) {
+    tab_src = min(t0 + 64u * wave + lane, p.n_tokens - 1u) * p.nsb * 4u;
+  } else {
+    const uint32_t tab_row = min(r0 + lane, p.out_dim - 1u);
+    const uint32_t tab_rb = tab_row >> p.r_shift, tab_r = tab_row & ((1u << p.r_shift) - 1u);
+    if constexpr (Q6) tab_src = tab_rb * p.nct * TILE_BYTES + 13u * 1024u + ((tab_r * 2u) & ~3u);
+    else tab_src = tab_rb * p.nct * TILE_BYTES + tab_r * 16u;
+  }
+  uint32_t tsl_prev = 0u, tsl_cur = 0u, tsl_next = TAB_SLOT;   // table slots of super-blocks s - 1, s, s + 1
+  auto fetch_tables = [&](uint32_t s, uint32_t tsl) {
+    uint8_t *slot = lds + TAB + tsl;
+    if (wave < 2u) {
+      gd_dma4((const uint8_t *)p.ad + (tab_src + 4u * s), slot + 256u * wave);
+    } else {
+      const uint32_t so = Q6 ? (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 2u : sb_off(s);
+      gd_dma4(p.wt + (tab_src + so), slot + 512u + 256u * (wave - 2u));
+    }
+  };
+  auto fetch_step = [&](uint32_t slot_off) {   // the next step (they are fetched in ascending order) into ring slot slot_off / SLOT
+    uint8_t *slot = lds + slot_off;
+    gd_dma16(p.planes + w_src, slot + w_dst);
+    gd_dma16((const uint8_t *)p.xt + x_src, slot + x_dst);
+    w_src += 4096u;
+    x_src += 1024u;
+  };
+
+  fetch_tables(0u, 0u);
+#pragma unroll
+  for (uint32_t k = 0; k < AHEAD; k++) fetch_step(k * SLOT);
+#define GX_SYNC_STEPS(N) GX_SYNC((N) * (int)PER)   // all but the newest N steps' loads of this wave have landed, then the barrier
+  GX_SYNC_STEPS(AHEAD - 1);   // step 0 and the first tables have landed
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+  const uint32_t w_rd = lds0 + lh * 2048u + (32u * rs + l32) * 16u;      // h plane; l plane + 1024
+  const uint32_t x_rd = lds0 + 4096u + 2048u * th + lane * 16u;          // token block 0 of the wave; block 1 + 1024
+  const uint32_t ad_rd = lds0 + TAB + 4u * (64u * th + 4u * lh);      // + 128 tb + 32 q4: four tokens' ad
+  const uint32_t hw_rd = lds0 + TAB + 512u + 4u * (32u * rs + l32);   // the row's header word
+  typedef float float4v __attribute__((ext_vector_type(4)));
+  int16v hA[2], lA[2], hB[2], lB[2];
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  int4v wh, wl, x0, x1;
+  float4v a4[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+  uint32_t hw = 0;
+  float d0 = 0.0f;
+  GD_READ16(wh, w_rd, 0);
+  GD_READ16(x0, x_rd, 0);
+  GD_READ16(x1, x_rd, 1024);
+  GD_READ16(wl, w_rd, 1024);
+
+  // One super-block: its 8 steps accumulate into (hc, lc) while, with EPI, the sums of the one before in
+  // (hp, lp) are added to y, one output behind every matrix instruction.
+  auto super_block = [&](auto set_c, auto epi_c, uint32_t s) {
+    constexpr bool SET = decltype(set_c)::value, EPI = decltype(epi_c)::value && !GX_ABL_NOEPI;
+    const bool more = s + 1u < p.nsb;   // in the last super-block the steps in flight run out
+    int16v(&hc)[2] = SET ? hB : hA;
+    int16v(&lc)[2] = SET ? lB : lA;
+    int16v(&hp)[2] = SET ? hA : hB;
+    int16v(&lp)[2] = SET ? lA : lB;
+    auto step = [&](auto kk_c) {
+      constexpr uint32_t kk = decltype(kk_c)::value;
+      // step k = 8 s + kk: step k + 1 has landed for every wave (all but the loads of the steps after it)
+      if (kk + AHEAD <= 8u || more) GX_SYNC_STEPS(AHEAD - 2);
+      else GX_SYNC_STEPS(kk >= 6u ? 0 : (int)(6u - kk));
+      constexpr uint32_t NX = ((kk + 1u) & 7u) * SLOT;   // step k + 1's ring slot
+      constexpr int tq = (int)(kk >> 2), q4 = (int)(kk & 3u);   // the four outputs added up in this step: y[tq][4 q4 ..]
+      constexpr int cur = (int)(kk & 1u), nxt = cur ^ 1;
+      // the next step's four ad: of the same super-block, or (from step 7) of this one, whose sums are complete then
+      const uint32_t ad_nx = ad_rd + (kk == 7u ? tsl_cur : tsl_prev) + 128u * (((kk + 1u) & 7u) >> 2) + 32u * ((kk + 1u) & 3u);
+      auto add_up = [&](auto e_c) {
+        constexpr int e = decltype(e_c)::value;
+        if constexpr (EPI) {
+          const int is = hp[tq][4 * q4 + e] * 256 + lp[tq][4 * q4 + e];
+          y[tq][4 * q4 + e] += a4[cur][e] * (d0 * (float)is);
+        }
+      };
+      GX_PIN();
+      // outstanding, oldest first: [hw at step 0], a4[cur], wh, x0, x1, wl  (without EPI and before step 7: no a4)
+      GX_WAITN(2);
+      asm volatile("" : "+v"(wh), "+v"(x0), "+v"(a4[cur]), "+v"(hw));
+      if (EPI && kk == 0u) d0 = gm_f16_bits_to_f32(Q6 && (l32 & 1u) ? (hw >> 16) : (hw & 0xFFFFu));
+      hc[0] = GX_MFMA(x0, wh, kk == 0u ? zi : hc[0]);
+      GX_PIN();
+      // the loads of step k + AHEAD (into the slot step k - 1 left) go out behind a matrix instruction
+      if (kk == 0u && more) fetch_tables(s + 1u, tsl_next);
+      if ((kk + AHEAD < 8u || more) && !GX_ABL_NODMA) fetch_step(((kk + AHEAD) & 7u) * SLOT);
+      GX_PIN();
+      add_up(std::integral_constant<int, 0>{});
+      GX_PIN();
+      GX_WAITN(1);
+      asm volatile("" : "+v"(x1));
+      hc[1] = GX_MFMA(x1, wh, kk == 0u ? zi : hc[1]);
+      GX_PIN();
+      if (kk == 7u) asm volatile("ds_read_b32 %0, %1" : "=v"(hw) : "v"(hw_rd + tsl_cur));
+      if (EPI || kk == 7u) asm volatile("ds_read_b128 %0, %1" : "=v"(a4[nxt]) : "v"(ad_nx));
+      asm volatile("ds_read_b128 %0, %2 offset:%3" : "=v"(wh) : "0"(wh), "v"(w_rd), "n"(NX));
+      GX_PIN();
+      add_up(std::integral_constant<int, 1>{});
+      GX_PIN();
+      // outstanding: wl, [hw], [a4 next], wh
+      if (kk == 7u) GX_WAITN(3);
+      else if (EPI) GX_WAITN(2);
+      else GX_WAITN(1);
+      asm volatile("" : "+v"(wl));
+      lc[0] = GX_MFMA(x0, wl, kk == 0u ? zi : lc[0]);
+      GX_PIN();
+      asm volatile("ds_read_b128 %0, %2 offset:%3" : "=v"(x0) : "0"(x0), "v"(x_rd), "n"(NX));
+      GX_PIN();
+      add_up(std::integral_constant<int, 2>{});
+      GX_PIN();
+      lc[1] = GX_MFMA(x1, wl, kk == 0u ? zi : lc[1]);
+      GX_PIN();
+      asm volatile("ds_read_b128 %0, %2 offset:%3" : "=v"(x1) : "0"(x1), "v"(x_rd), "n"(NX + 1024u));
+      asm volatile("ds_read_b128 %0, %2 offset:%3" : "=v"(wl) : "0"(wl), "v"(w_rd), "n"(NX + 1024u));
+      GX_PIN();
+      add_up(std::integral_constant<int, 3>{});
+      GX_PIN();
+    };
+    step(std::integral_constant<uint32_t, 0u>{});
+    step(std::integral_constant<uint32_t, 1u>{});
+    step(std::integral_constant<uint32_t, 2u>{});
+    step(std::integral_constant<uint32_t, 3u>{});
+    step(std::integral_constant<uint32_t, 4u>{});
+    step(std::integral_constant<uint32_t, 5u>{});
+    step(std::integral_constant<uint32_t, 6u>{});
+    step(std::integral_constant<uint32_t, 7u>{});
+    const uint32_t t = tsl_prev;   // the slots turn: s - 1's is free for s + 2
+    tsl_prev = tsl_cur;
+    tsl_cur = tsl_next;
+    tsl_next = (s == 0u) ? 2u * TAB_SLOT : t;
+  };
+  using std::false_type;
+  using std::true_type;
+  super_block(false_type{}, false_type{}, 0u);
+  for (uint32_t s = 1; s < p.nsb; s += 2u) {
+    super_block(true_type{}, true_type{}, s);
+    if (s + 1u < p.nsb) super_block(false_type{}, true_type{}, s + 1u);
+  }
+  // the last super-block's sums (its header word and first four ad were asked for in its last step)
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wh), "+v"(x0), "+v"(x1), "+v"(wl), "+v"(a4[0]), "+v"(hw));
+  {
+    d0 = gm_f16_bits_to_f32(Q6 && (l32 & 1u) ? (hw >> 16) : (hw & 0xFFFFu));
+    const uint32_t ta = ad_rd + tsl_prev;   // (the slots have turned once more)
+    const bool odd = (p.nsb & 1u) == 0u;    // the last super-block filled set B
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++) {
+      float4v b40, b41, b42, b43;
+      GD_READ16(b40, ta, 128 * tb);
+      GD_READ16(b41, ta, 128 * tb + 32);
+      GD_READ16(b42, ta, 128 * tb + 64);
+      GD_READ16(b43, ta, 128 * tb + 96);
+      GD_WAIT2(0, b40, b41);
+      GD_WAIT2(0, b42, b43);
+      const float4v b4[4] = {b40, b41, b42, b43};
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const float b4v[4] = {b4[q4].x, b4[q4].y, b4[q4].z, b4[q4].w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int is = odd ? hB[tb][4 * q4 + e] * 256 + lB[tb][4 * q4 + e] : hA[tb][4 * q4 + e] * 256 + lA[tb][4 * q4 + e];
+          y[tb][4 * q4 + e] += b4v[e] * (d0 * (float)is);
+        }
+      }
+    }
+  }
+  const uint32_t row0 = r0 + 32u * rs + l32;
+  if (row0 < p.out_dim) {
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const uint32_t t = t0 + 64u * th + 32u * tb + 8u * (r >> 2) + 4u * lh + (r & 3);
+        if (t < p.n_tokens) p.y[(size_t)t * p.out_dim + row0] = y[tb][r];
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Small batches (up to a few dozen tokens): the tiled kernels above cost the same for 9 tokens as
 // for 128, because a workgroup walks its rows' super-blocks one after the other.  Here a workgroup
 // owns 32 rows x 32 tokens and its eight waves take different super-blocks of those rows at the same
@@ -2038,6 +2429,30 @@ static bool gemm_medium_batch(const OgmGemmArgs &a) {
 // feeding-wave kernels: Q4_K 4096 -> 14336 at 256 tokens 69 us against 57, at 384 tokens 87 against 104), the
 // activations in operand chunks, and everything within 32-bit byte offsets.  (plane_kernel 2: whatever the
 // grid.)
+// Whether a launch over planes takes the kernel with 64-row tiles that adds a super-block up between the next one's
+// matrix instructions (ogm_gemm_dmx_kernel) instead of the one with 128-row tiles (ogm_gemm_dma_kernel).
+// interleave: 0 by the size of the launch, 1 never, 2 whenever the type allows.  Measured on MI355X, whole calls at
+// 512 tokens, us, 64-row interleaved / 128-row / feeding waves: Q6_K 14336 -> 4096 103 / 153 / 126, Q4_K 4096 ->
+// 4096 42 / 64 / 49, 4096 -> 6144 54 / 67 / 64, 14336 -> 4096 130 / 204 / 150; but 4096 -> 14336 115 / 98 / -, and
+// at 1024 tokens 4096 -> 6144 92 / 89, 4096 -> 4096 64 / 71: the 128-row kernel wants its 512 places (two workgroups
+// a compute unit) three quarters full, the 64-row one at least 160 tiles and three token tiles (at 256 tokens it
+// only draws with the kernels that need no planes: 4096 -> 14336 67 against 70, 4096 -> 6144 39 against 41).
+static bool gemm_interleaved(const OgmGemmArgs &a) {
+  const uint32_t nsb = a.in_dim / 256;
+  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  if (a.interleave == 1u || a.ggml_type == OGM_Q3_K || (q45 && a.one_pass != 0u) || nsb * 512u > GX_TAB || a.n_tokens < 32u)
+    return false;
+  if (a.interleave == 2u) return true;
+  uint32_t tiles128 = 0, tiles64 = 0;
+  for (uint32_t m = 0; m <= a.n_extra; m++) {
+    const uint32_t od = m ? a.extra_out_dim[m - 1] : a.out_dim;
+    tiles128 += (od + 127u) / 128u;
+    tiles64 += (od + 63u) / 64u;
+  }
+  const uint32_t tok_tiles = (a.n_tokens + 127u) / 128u;
+  return tok_tiles >= 3u && tok_tiles * tiles128 < 384u && tok_tiles * tiles64 >= 160u;
+}
+
 static bool gemm_dma_eligible(const OgmGemmArgs &a) {
   const uint32_t nsb = a.in_dim / 256;
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
@@ -2050,7 +2465,8 @@ static bool gemm_dma_eligible(const OgmGemmArgs &a) {
     if ((uint64_t)((od + 63u) / 64u) * 64u * a.in_dim * 2u >= (1ull << 32)) return false;
     tiles += (od + GD_ROWS - 1u) / GD_ROWS;
   }
-  return a.plane_kernel == 2u || ((a.n_tokens + GD_TOK - 1u) / GD_TOK) * tiles > 256u;
+  if (a.plane_kernel == 2u || ((a.n_tokens + GD_TOK - 1u) / GD_TOK) * tiles > 256u) return true;
+  return gemm_interleaved(a);
 }
 
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a) {
@@ -2188,6 +2604,8 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     if (!a.xt_ready)
       hipLaunchKernelGGL(ogm_gemm_xtile_kernel, dim3(a.in_dim / 128u, t_pad / 32u), dim3(256), 0, stream, a.act.q,
                          (int8_t *)a.xh, a.in_dim, a.n_tokens);
+    // the kernel that adds a super-block up between the next one's matrix instructions (64-row tiles)
+    const bool interleaved = gemm_interleaved(a);
     GemmDmaParams d;
     d.wt = a.wt;
     d.planes = a.planes;
@@ -2210,6 +2628,23 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       d.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
       d.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
       if (m < a.n_extra) tiles += (a.extra_out_dim[m] + GD_ROWS - 1u) / GD_ROWS;
+    }
+    if (interleaved) {
+      uint32_t tiles_x = (a.out_dim + GX_ROWS - 1u) / GX_ROWS;
+      for (uint32_t m = 0; m < a.n_extra; m++) tiles_x += (a.extra_out_dim[m] + GX_ROWS - 1u) / GX_ROWS;
+      const void *fx = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_dmx_kernel<GP_Q6K>
+                       : a.ggml_type == OGM_Q4_K ? (const void *)ogm_gemm_dmx_kernel<GP_Q4K>
+                                                 : (const void *)ogm_gemm_dmx_kernel<GP_Q5K>;
+      hipError_t ex = hipFuncSetAttribute(fx, hipFuncAttributeMaxDynamicSharedMemorySize, (int)GX_LDS_BYTES);
+      if (ex != hipSuccess) return ex;
+      void *xargs[] = {(void *)&d};
+      ex = hipLaunchKernel(fx, dim3((a.n_tokens + GX_TOK - 1u) / GX_TOK, tiles_x), dim3(64u * GX_NW), xargs, GX_LDS_BYTES, stream);
+      if (ex != hipSuccess) return ex;
+      if (kernel_name)
+        *kernel_name = a.ggml_type == OGM_Q6_K   ? "ogm_gemm_q6k_dmx_kernel"
+                       : a.ggml_type == OGM_Q4_K ? "ogm_gemm_q4k_dmx_kernel"
+                                                 : "ogm_gemm_q5k_dmx_kernel";
+      return hipGetLastError();
     }
     const bool one_pass = q45 && a.one_pass != 0u;
     const void *fn = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_dma_kernel<GP_Q6K>

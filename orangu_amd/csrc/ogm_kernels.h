@@ -16,6 +16,10 @@ struct OgmActDev {
   // per-256 mode only: the sums per 32 once more as f16 pairs (bsum >> 6, bsum & 63), sixteen halves
   // per super-block (eight high parts, then eight low parts): the K-quant GEMMs' first-pass operand
   uint16_t *bs16;
+  // per-256 mode, batches of rows only: when not null, the int8 activations are also written here in the operand
+  // chunks of the GEMMs whose waves all multiply (ogm_gemm_xh_bytes() bytes; the chunks' tokens past the last stay
+  // as they were: they are multiplied, never stored)
+  int8_t *xt = nullptr;
 };
 
 // mode 0: one scale per 32 (vecdot.rs:95-126); mode 1: one per 256 (vecdot.rs:3030-3053).
@@ -76,6 +80,7 @@ struct OgmGemmArgs {
   // when that kernel runs: 0 when the grid fills the device twice (else the feeding waves unpack), 2 whatever
   // the grid
   uint32_t plane_kernel = 0;
+  uint32_t interleave = 0;   // the plane kernel with 64-row tiles that adds a super-block up between the next one's matrix instructions: 0 by the size of the launch, 1 never, 2 whenever it can
   uint32_t one_pass = 0;   // Q4_K / Q5_K on the all-waves-multiply kernel: fold the min pass into the super-block step (f32 to rounding, not to the bit)
 };
 // Whether this launch would run a tiled int8 plane kernel, i.e. whether planes would be read.

@@ -37,6 +37,7 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
     act.sums += (size_t)blockIdx.x * (n / 16u);
     act.bsum += (size_t)blockIdx.x * (n / 32u);
     if (act.bs16) act.bs16 += (size_t)blockIdx.x * (n / 16u);
+    act.xt = ogm_xt_row(act.xt, blockIdx.x, n);
   }
   ogm_norm_quant_row<GROUP, false>(x, delta, weight, n, eps, normed, act, red, tid, n_wave, x_src);
 }
@@ -658,6 +659,7 @@ __global__ __launch_bounds__(64) void ogm_swiglu_quant_kernel(const float *__res
     act.sums += (size_t)blockIdx.y * (n / 16u);
     act.bsum += (size_t)blockIdx.y * (n / 32u);
     if (act.bs16) act.bs16 += (size_t)blockIdx.y * (n / 16u);
+    act.xt = ogm_xt_row(act.xt, blockIdx.y, n);
   }
   ogm_swiglu_quant_run<GROUP, false>(gate, up, n, h, act, blockIdx.x, lane);
 }

@@ -139,7 +139,7 @@ __device__ __forceinline__ void ogm_st(T *p, T v) {
 template <int GROUP, bool COHERENT_OUT = false>
 __device__ __forceinline__ uint32_t ogm_quantize_store(const float4 &v, uint32_t e0, bool active, uint32_t lane,
                                                        int8_t *q, float *d, int32_t *sums, int16_t *bsum,
-                                                       uint16_t *bs16) {
+                                                       uint16_t *bs16, int8_t *xt_row = nullptr) {
   float scale;
   int s16, s32;
   const uint32_t packed = ogm_quantize4<GROUP>(v, scale, s16, s32);
@@ -156,8 +156,16 @@ __device__ __forceinline__ uint32_t ogm_quantize_store(const float4 &v, uint32_t
       }
     }
     if ((lane & (GROUP / 4 - 1)) == 0) ogm_st<COHERENT_OUT>(d + e0 / GROUP, scale);
+    // the token's place in the operand chunks (ogm_xt_row): chunk e0 / 32, half (e0 / 16) & 1 of its k, byte e0 & 15
+    if (xt_row != nullptr) *(uint32_t *)(xt_row + (e0 >> 5) * 1024u + ((e0 >> 4) & 1u) * 512u + (e0 & 15u)) = packed;
   }
   return packed;   // the lane's four int8 values, also for callers that lay them out a second way
+}
+
+// Where token t's activations start in the operand chunks of a batch n wide: chunk (t / 32, k / 32) is 1 KiB, the
+// 16 activations 16 h .. of its token l at 16 (32 h + l).
+__device__ __forceinline__ int8_t *ogm_xt_row(int8_t *xt, uint32_t t, uint32_t n) {
+  return xt ? xt + (size_t)(t >> 5) * (n / 32u) * 1024u + (t & 31u) * 16u : nullptr;
 }
 
 // Four floats that another workgroup of the same kernel may have stored device-coherently.
@@ -229,7 +237,7 @@ __device__ __forceinline__ void ogm_norm_quant_row(float *__restrict__ x, const 
       if (normed) *(float4 *)(normed + e0) = o;
     }
     if ((wave + k * n_wave) * 256u < n)  // wave-uniform: the run exists
-      ogm_quantize_store<GROUP, COHERENT_OUT>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
+      ogm_quantize_store<GROUP, COHERENT_OUT>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16, act.xt);
   }
 }
 
@@ -250,5 +258,5 @@ __device__ __forceinline__ void ogm_swiglu_quant_run(const float *__restrict__ g
     o.w = g.w / (1.0f + expf(-g.w)) * u.w;
     if (h) *(float4 *)(h + e0) = o;
   }
-  ogm_quantize_store<GROUP, COHERENT_OUT>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
+  ogm_quantize_store<GROUP, COHERENT_OUT>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16, act.xt);
 }

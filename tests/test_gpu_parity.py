@@ -31,11 +31,12 @@ def say(*a):
 GEMM_FROM = 9
 
 
-# Every test of this module runs twice: with the K-quant matrices' prefill planes built on first
-# use and kept (gemm_plane_cache_mb > 0) and read by the kernel whose waves all multiply ("planes":
-# ogm_gemm_q*_dma_kernel, here whatever the grid, from 32 tokens), and with none ("unpack": the feeding
-# waves unpack the weights on every call).  Same bits both ways.
-@pytest.fixture(scope="module", params=["planes", "unpack"])
+# Every test of this module runs three times: with the K-quant matrices' prefill planes built on first
+# use and kept (gemm_plane_cache_mb > 0) and read by a kernel whose waves all multiply, here whatever the
+# grid, from 32 tokens ("planes": ogm_gemm_q*_dma_kernel, 128-row tiles; "planes64": ogm_gemm_q*_dmx_kernel,
+# 64-row tiles, the f32 step between the matrix instructions, wherever its types allow), and with none
+# ("unpack": the feeding waves unpack the weights on every call).  Same bits every way.
+@pytest.fixture(scope="module", params=["planes", "planes64", "unpack"])
 def be(request):
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()  # raises if the HIP library or the device is missing: no fallback
@@ -47,6 +48,7 @@ def be(request):
     b.set_tuning("gemm_sb_waves", 8)
     b.set_tuning("gemm_plane_cache_mb", 0 if request.param == "unpack" else 65536)
     b.set_tuning("gemm_plane_kernel", 2)
+    b.set_tuning("gemm_interleave", 2 if request.param == "planes64" else 1)
     b.plane_mode = request.param
     yield b
     b.close()
@@ -72,9 +74,10 @@ def kname(b):
     family's tiled kernel (of either row tiling).  Checks that the name fits the mode the backend runs in."""
     name = b.last_kernel()
     mode = getattr(b, "plane_mode", None)   # None: a context with no tuning reads planes on large grids
-    m = re.match(r"ogm_gemm_q(6k|3k|4k|5k)_dma_kernel$", name)
+    m = re.match(r"ogm_gemm_q(6k|3k|4k|5k)_dm([ax])_kernel$", name)
     if m:
-        assert mode in (None, "planes"), name
+        assert mode is None or mode == ("planes64" if m.group(2) == "x" else "planes") or \
+            (mode == "planes64" and m.group(1) == "3k"), name   # (Q3_K has no 64-row kernel)
         return _TiledPlaneKernel({"6k": "ogm_gemm_q6k_i8", "3k": "ogm_gemm_q3k_i8", "4k": "ogm_gemm_q4k_i8p",
                                   "5k": "ogm_gemm_q5k_i8p"}[m.group(1)])
     return name
@@ -651,6 +654,11 @@ def test_gemm_threshold_default():
         y = b.matmul(x5, 129, w)
         assert b.last_kernel() == "ogm_gemm_q4k_dma_kernel"
         assert_bits(y, oracle.matmul(Q4_K, raw, 256, 16600, x5, 129), "Q4_K, 129 tokens x 16600 rows")
+        raw7 = synth_weights(Q4_K, 256, 4000, seed=12)   # 63 tiles of 64 rows x 3 of 128 tokens: the 64-row plane kernel
+        x7 = synth_x(300, 256, seed=13)
+        y = b.matmul(x7, 300, qm(raw7, Q4_K, 256, 4000))
+        assert b.last_kernel() == "ogm_gemm_q4k_dmx_kernel"
+        assert_bits(y, oracle.matmul(Q4_K, raw7, 256, 4000, x7, 300), "Q4_K, 300 tokens x 4000 rows")
         y = b.matmul(x5[:128], 128, w)                   # one full token tile, but more 32-row workgroups than one round
         assert b.last_kernel() == "ogm_gemm_q4k_i8p_kernel"
         assert_bits(y, oracle.matmul(Q4_K, raw, 256, 16600, x5[:128], 128), "Q4_K, 128 tokens x 16600 rows")
