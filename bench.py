@@ -198,6 +198,10 @@ def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
             run(Q6_K, FFN, HIDDEN, T, False, f"C3 ffn_down batch {T}")
     for T in (128, 512, 2048):
         run(Q4_K, HIDDEN, FFN, T, False, f"C4 prefill GEMM M={T}", n=64)
+    # the 8B shapes' other projections at 512 tokens: grids that leave the 128-row plane kernel half empty
+    run(Q4_K, 4096, 4096, 512, False, "C4 wo-sized GEMM 4096->4096 M=512", n=64)
+    run(Q4_K, 4096, 6144, 512, False, "C4 q+k+v-sized GEMM 4096->6144 M=512", n=64)
+    run(Q6_K, FFN, HIDDEN, 512, False, "C4 ffn_down GEMM 14336->4096 M=512", n=64)
     run(Q6_K, FFN, HIDDEN, 1, False, "C5 ffn_down GEMV")
     for hs in uploaded.values():
         for h in hs:

@@ -27,17 +27,18 @@ __global__ __launch_bounds__(1024) void ogm_norm_quant_kernel(float *__restrict_
   __shared__ float red[64];
   const uint32_t tid = threadIdx.x, n_wave = blockDim.x >> 6;
   {   // one workgroup per row of a batch
-    const size_t row = (size_t)blockIdx.x * n;
+    const uint32_t r = act.xt ? ogm_xt_row_of_workgroup(blockIdx.x, gridDim.x) : blockIdx.x;
+    const size_t row = (size_t)r * n;
     x += row;
     if (x_src) x_src += row;
     if (delta) delta += row;
     if (normed) normed += row;
     act.q += row;
-    act.d += (size_t)blockIdx.x * (n / GROUP);
-    act.sums += (size_t)blockIdx.x * (n / 16u);
-    act.bsum += (size_t)blockIdx.x * (n / 32u);
-    if (act.bs16) act.bs16 += (size_t)blockIdx.x * (n / 16u);
-    act.xt = ogm_xt_row(act.xt, blockIdx.x, n);
+    act.d += (size_t)r * (n / GROUP);
+    act.sums += (size_t)r * (n / 16u);
+    act.bsum += (size_t)r * (n / 32u);
+    if (act.bs16) act.bs16 += (size_t)r * (n / 16u);
+    act.xt = ogm_xt_row(act.xt, r, n);
   }
   ogm_norm_quant_row<GROUP, false>(x, delta, weight, n, eps, normed, act, red, tid, n_wave, x_src);
 }
@@ -649,19 +650,22 @@ __global__ __launch_bounds__(64) void ogm_swiglu_quant_kernel(const float *__res
                                                               const float *__restrict__ up, uint32_t n,
                                                               float *__restrict__ h, OgmActDev act) {
   const uint32_t lane = threadIdx.x;
-  {   // blockIdx.y: the row of a batch
-    const size_t row = (size_t)blockIdx.y * n;
+  // blockIdx.y: the row of a batch.  (With a multiple of eight runs a row, the eight rows that share a line of the
+  // operand chunks are written from one XCD without further ado: workgroup (run, row) runs on XCD run % 8.)
+  const uint32_t r = blockIdx.y, run = blockIdx.x;
+  {
+    const size_t row = (size_t)r * n;
     gate += row;
     up += row;
     if (h) h += row;
     act.q += row;
-    act.d += (size_t)blockIdx.y * (n / GROUP);
-    act.sums += (size_t)blockIdx.y * (n / 16u);
-    act.bsum += (size_t)blockIdx.y * (n / 32u);
-    if (act.bs16) act.bs16 += (size_t)blockIdx.y * (n / 16u);
-    act.xt = ogm_xt_row(act.xt, blockIdx.y, n);
+    act.d += (size_t)r * (n / GROUP);
+    act.sums += (size_t)r * (n / 16u);
+    act.bsum += (size_t)r * (n / 32u);
+    if (act.bs16) act.bs16 += (size_t)r * (n / 16u);
+    act.xt = ogm_xt_row(act.xt, r, n);
   }
-  ogm_swiglu_quant_run<GROUP, false>(gate, up, n, h, act, blockIdx.x, lane);
+  ogm_swiglu_quant_run<GROUP, false>(gate, up, n, h, act, run, lane);
 }
 
 hipError_t ogm_launch_swiglu_quant(int mode, const float *gate, const float *up, uint32_t n, float *h,

@@ -168,6 +168,17 @@ __device__ __forceinline__ int8_t *ogm_xt_row(int8_t *xt, uint32_t t, uint32_t n
   return xt ? xt + (size_t)(t >> 5) * (n / 32u) * 1024u + (t & 31u) * 16u : nullptr;
 }
 
+// The row a workgroup of a row-per-workgroup producer takes when it also writes the operand chunks.  Eight
+// consecutive tokens share every 128-byte line of a chunk, and workgroups are dealt to the eight XCDs (each with an
+// L2 of its own) in turn: rows in the grid's order would put the eight writers of a line on eight L2s, none of which
+// ever holds the whole line.  Within a group of 64 workgroups, workgroup 8 i + x (on XCD x) takes row 8 x + i, so a
+// line's writers share an L2 and run within a few workgroups of each other.  (The last, partial group keeps the
+// grid's order.)
+__device__ __forceinline__ uint32_t ogm_xt_row_of_workgroup(uint32_t b, uint32_t n) {
+  if ((b | 63u) >= n) return b;
+  return (b & ~63u) | ((b & 7u) << 3) | ((b >> 3) & 7u);
+}
+
 // Four floats that another workgroup of the same kernel may have stored device-coherently.
 template <bool COHERENT>
 __device__ __forceinline__ float4 ogm_ld4(const float *p) {
