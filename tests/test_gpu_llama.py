@@ -562,6 +562,35 @@ def test_prefill_from_an_empty_cache_then_decode(be, types, n_tokens):
         dev.close()
 
 
+@pytest.mark.parametrize("interleave,n_tokens", [(1, 45), (2, 45), (1, 300), (2, 300), (2, 129)])
+def test_prefill_through_the_plane_kernels(be, interleave, n_tokens):
+    """The tiled GEMMs over prebuilt planes, forced on a small model (gemm_plane_kernel 2): the norm and SwiGLU
+    kernels then write the GEMMs' operand chunks themselves, here with a last token block of 13, 12 and 1 tokens
+    (the block's other places keep whatever the buffer held: multiplied, never stored), read by the 128-row kernel
+    (gemm_interleave 1) and by the 64-row one (2).  Checked like every prefill, and the matmuls' names."""
+    be.set_tuning("gemm_plane_kernel", 2)
+    be.set_tuning("gemm_interleave", interleave)
+    be.set_tuning("gemm_small_max_tokens", 1)
+    be.set_tuning("gemm_medium", 1)
+    ref, dev, rng = build(be, n_embd=256, n_head=4, n_kv=2, hd=64, n_ff=512, n_vocab=320, n_layer=2,
+                          types=(Q4_K, Q6_K, Q6_K, Q5_K), max_ctx=320, seed=57, attn_norm_scale=TAME[Q4_K])
+    try:
+        # a longer batch first, so that the chunks of the ragged batch hold another batch's tokens past its last
+        dev.prefill(rng.standard_normal((min(320, n_tokens + 19), 256)).astype(f32), 0)
+        prefill_both(ref, dev, rng.standard_normal((n_tokens, 256)).astype(f32), 0, f"plane kernels, interleave {interleave}")
+        # (under these settings a matmul of the model's shapes takes the kernel meant)
+        from orangu_amd import QuantMatrix
+        L0 = ref.layers[0].w_gate
+        be.matmul(rng.standard_normal(n_tokens * 256).astype(f32), n_tokens, QuantMatrix(np.ascontiguousarray(L0[1]), L0[0], L0[2], L0[3]))
+        assert be.last_kernel() == ("ogm_gemm_q4k_dmx_kernel" if interleave == 2 else "ogm_gemm_q4k_dma_kernel")
+    finally:
+        be.set_tuning("gemm_plane_kernel", 0)
+        be.set_tuning("gemm_interleave", 0)
+        be.set_tuning("gemm_small_max_tokens", 0)
+        be.set_tuning("gemm_medium", 0)
+        dev.close()
+
+
 def test_prefill_of_one_token_is_a_decode_step(be):
     """n_tokens == 1 through the batch entry point: the single-token kernels' float order
     (Backend::matmul at one token, cpu.rs:445-458), the same cache row and logits as the step."""
