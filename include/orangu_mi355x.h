@@ -251,7 +251,10 @@ typedef struct ogm_llama_layer {
 } ogm_llama_layer;
 
 /* Builds the device-side model over weights already uploaded with ogm_weight_upload (they must
- * outlive it).  `layers` has cfg->n_layer entries; output_norm is host f32 [n_embd]. */
+ * outlive it).  `layers` has cfg->n_layer entries; output_norm is host f32 [n_embd].
+ * OGM_ERR_UNSUPPORTED for shapes the forward-pass kernels are not built for: head_dim other than 64 or 128; a
+ * number of query heads per K/V head that is neither 1..8 nor, up to 64, divisible into equal parts of at most
+ * eight (16, 12, 10, 24 ... are taken; 9, 11, 13 ... are not); n_embd above 16384 or not a multiple of 32. */
 int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const ogm_llama_layer *layers,
                      const float *output_norm, const ogm_weight *output, ogm_llama **out);
 void ogm_llama_destroy(ogm_ctx *ctx, ogm_llama *m);

@@ -1234,7 +1234,7 @@ struct ogm_llama {
   float *freq = nullptr;      // [rope_dim / 2], frequency factors applied
   float *rope_cs = nullptr;   // [rope_dim / 2] (cos, sin) of the token being decoded
   float *rope_all = nullptr;  // the same for every position of the cache, filled at creation (null: too large, computed per token)
-  uint32_t *attn_counters = nullptr;  // [2 n_head_kv][OGM_ATTN_TICKET_STRIDE] the attention kernel's tickets, a line each; zero between launches
+  uint32_t *attn_counters = nullptr;  // [2 n_head_kv parts][OGM_ATTN_TICKET_STRIDE] the attention kernel's tickets, a line each; zero between launches
   void *k_cache = nullptr;    // f16 [n_layer][max_ctx][kv_dim]
   void *v_cache = nullptr;
   float *x = nullptr;         // hidden state [n_embd]
@@ -1294,8 +1294,8 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   if (c.n_layer == 0 || c.n_embd == 0 || c.n_head == 0 || c.n_head_kv == 0 || c.n_ff == 0 || c.max_ctx == 0)
     return fail(ctx, OGM_ERR_INVALID, "empty model dimension");
   const uint32_t gq = c.n_head % c.n_head_kv == 0 ? c.n_head / c.n_head_kv : 0;
-  if (gq < 1 || gq > 8)
-    return fail(ctx, OGM_ERR_UNSUPPORTED, "query heads per K/V head must be 1 to 8");
+  if (gq < 1 || ogm_attn_head_parts(gq) == 0)
+    return fail(ctx, OGM_ERR_UNSUPPORTED, "query heads per K/V head must be 1 to 8, or up to 64 in equal parts of at most 8");
   if (c.rope_neox > 1) return fail(ctx, OGM_ERR_INVALID, "rope_neox is 0 (NORM pairs) or 1 (NEOX pairs)");
   if (c.rope_freq_factors)
     for (uint32_t i = 0; i < c.rope_dim / 2; i++)
@@ -1336,7 +1336,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   // positions); a decode step then launches no table kernel
   const size_t rope_all_bytes = (size_t)c.max_ctx * (c.rope_dim / 2) * 8;
   if (c.rope_dim != 0 && rope_all_bytes <= ((size_t)64 << 20)) A((void **)&m->rope_all, rope_all_bytes);
-  A((void **)&m->attn_counters, (size_t)2 * c.n_head_kv * OGM_ATTN_TICKET_STRIDE * 4);
+  A((void **)&m->attn_counters, (size_t)2 * c.n_head_kv * ogm_attn_head_parts(gq) * OGM_ATTN_TICKET_STRIDE * 4);
   A(&m->k_cache, cache_bytes);
   A(&m->v_cache, cache_bytes);
   A((void **)&m->x, (size_t)c.n_embd * 4);
@@ -1389,7 +1389,7 @@ extern "C" int ogm_llama_create(ogm_ctx *ctx, const ogm_llama_config *cfg, const
   hipError_t e = hipMemcpy(m->norms, host.data(), host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->pre, pre_host.data(), pre_host.size() * 4, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(m->freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMemset(m->attn_counters, 0, (size_t)2 * c.n_head_kv * OGM_ATTN_TICKET_STRIDE * 4);
+  if (e == hipSuccess) e = hipMemset(m->attn_counters, 0, (size_t)2 * c.n_head_kv * ogm_attn_head_parts(gq) * OGM_ATTN_TICKET_STRIDE * 4);
   if (e == hipSuccess) e = hipMemset(m->k_cache, 0, cache_bytes);
   if (e == hipSuccess) e = hipMemset(m->v_cache, 0, cache_bytes);
   if (m->rope_all && e == hipSuccess) {

@@ -47,13 +47,17 @@ struct OgmAttnPre {
 //     table `cs`, k and v rounded to f16 into the cache rows of position `pos`;
 //   * causal attention over cache positions 0..pos (engine/attention.rs:426-549): scores =
 //     (q . k) * scale, softmax over positions, out = sum w * v; grouped-query heads share their
-//     K/V head (1 to 8 query heads per K/V head).  Split over chunks of `chunk` positions (64 or
-//     128; 0 = by the size of the launch) and merged;
+//     K/V head (a count ogm_attn_head_parts accepts: up to eight in one workgroup, more in equal parts of at
+//     most eight).  Split over chunks of `chunk` positions (64 or 128; 0 = by the size of the launch) and merged;
 //   * the merged output quantized for the next matmul in `mode`, and stored as f32 when attn_out
 //     is not null.
 // part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch, with
-// max_splits >= pos / chunk + 1; counters: 2 * n_head_kv * OGM_ATTN_TICKET_STRIDE words (one ticket per
+// max_splits >= pos / chunk + 1; counters: 2 * n_head_kv * parts * OGM_ATTN_TICKET_STRIDE words (one ticket per
 // cache line), zero before the first launch (the kernel leaves them zero).
+// ogm_attn_head_parts: the workgroups a K/V head's query heads are dealt to (1 for up to eight heads, else the
+// fewest equal parts of at most eight), or 0 for a count the kernels do not take (none, more than 64, or one that
+// does not divide: 9, 11, 13, ...).
+uint32_t ogm_attn_head_parts(uint32_t heads_per_kv);
 hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
                                   uint32_t rope_dim, const OgmAttnPre &pre, void *k_cache_layer,
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,

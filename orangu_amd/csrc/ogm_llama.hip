@@ -229,13 +229,15 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
   __shared__ float mrg[GROUP != 0 ? 6 : 1][GROUP != 0 ? NT : 1];   // the final merge's slices
   static_assert(!PREFILL || GROUP == 0, "a prefill batch merges in its own launch");
   OGM_STAMP(0);
-  // blockIdx.x: a K/V head and the gq query heads (G head slots) that share it
-  const uint32_t hg = blockIdx.x, split = blockIdx.y, kvh = hg;
+  // blockIdx.x: a K/V head and gq of the query heads (G head slots) that share it -- all of them, or one of
+  // gridDim.x / n_head_kv equal parts of them when the model has more than eight per K/V head (the parts' workgroups
+  // read the same cache rows; in the last chunk each writes the new rows, the same bytes)
+  const uint32_t hg = blockIdx.x, split = blockIdx.y, kvh = hg / (gridDim.x / n_head_kv);
   if constexpr (PREFILL) {
     const uint32_t tok = blockIdx.z;
     pos += tok;
     if (split > pos / (uint32_t)CHUNK) return;   // the whole workgroup: this token has no such chunk
-    const size_t n_head = (size_t)n_head_kv * gq;
+    const size_t n_head = (size_t)gridDim.x * gq;
     q += tok * n_head * HD;
     part_o += tok * n_head * max_splits * HD;
     part_ml += tok * n_head * max_splits * 2;
@@ -574,6 +576,12 @@ __global__ __launch_bounds__(64) void ogm_attn_combine_quant_kernel(const float 
   ogm_quantize_store<GROUP>(o, e0, active, lane, act.q, act.d, act.sums, act.bsum, act.bs16);
 }
 
+uint32_t ogm_attn_head_parts(uint32_t heads_per_kv) {
+  if (heads_per_kv == 0u || heads_per_kv > 64u) return 0u;
+  const uint32_t parts = (heads_per_kv + 7u) / 8u;
+  return heads_per_kv % parts == 0u ? parts : 0u;
+}
+
 hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const float *v_new, const void *cs,
                                   uint32_t rope_dim, const OgmAttnPre &pre, void *k_cache_layer,
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
@@ -594,9 +602,11 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
   if (n_splits > max_splits) return hipErrorInvalidValue;
   const uint32_t n = n_head * head_dim;
   if (n % 32u != 0) return hipErrorInvalidValue;
-  uint32_t gq = n_head / n_head_kv;
-  if (gq > 8u) return hipErrorInvalidValue;
-  const dim3 grid(n_head_kv, n_splits);
+  // more than eight query heads per K/V head: in equal parts of at most eight, a workgroup each
+  const uint32_t parts = ogm_attn_head_parts(n_head / n_head_kv);
+  if (parts == 0u) return hipErrorInvalidValue;
+  const uint32_t gq = n_head / n_head_kv / parts;
+  const dim3 grid(n_head_kv * parts, n_splits);
   const uint32_t G = gq <= 2u ? gq : (gq <= 4u ? 4u : 8u);   // head slots of the kernel
   const uint32_t group = mode == 0 ? 32u : 256u;
   // the merge rides in the attention kernel when every head slot is a head and a K/V head's
@@ -1040,10 +1050,11 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
   if (n_splits > max_splits) return hipErrorInvalidValue;
   const uint32_t n = n_head * head_dim;
   if (n % 4u != 0) return hipErrorInvalidValue;
-  const uint32_t gq = n_head / n_head_kv;
-  if (gq > 8u) return hipErrorInvalidValue;
+  const uint32_t parts = ogm_attn_head_parts(n_head / n_head_kv);
+  if (parts == 0u) return hipErrorInvalidValue;
+  const uint32_t gq = n_head / n_head_kv / parts;
   const uint32_t G = gq <= 2u ? gq : (gq <= 4u ? 4u : 8u);
-  const dim3 grid(n_head_kv, n_splits, n_tokens);
+  const dim3 grid(n_head_kv * parts, n_splits, n_tokens);
   const OgmAttnPre none{nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f, 0u};
   const OgmActDev no_act{};
 #define OGM_ATTN_PREFILL(HD_, G_)                                                                           \
@@ -1360,7 +1371,7 @@ hipError_t ogm_launch_attn_prefill_mfma(const float *q, void *k_cache_layer, voi
                                         float scale, float *attn_out, hipStream_t stream) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0 || n_tokens == 0) return hipErrorInvalidValue;
   const uint32_t gq = n_head / n_head_kv;
-  if (n_head_kv > 65535u || gq > 8u) return hipErrorInvalidValue;
+  if (n_head_kv > 65535u || ogm_attn_head_parts(gq) == 0u) return hipErrorInvalidValue;
   if ((n_tokens + 31u) / 32u > 65535u) return hipErrorInvalidValue;
   const dim3 grid(n_head_kv * ((gq + 3u) / 4u), (n_tokens + 31u) / 32u);
   if (head_dim != 128 && head_dim != 64) return hipErrorInvalidValue;

