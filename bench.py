@@ -209,15 +209,24 @@ def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
     return out
 
 
+DECODE_MODELS = {   # n_layer, n_embd, n_head, n_kv, head_dim, n_ff, n_vocab
+    "8b": (32, 4096, 32, 8, 128, 14336, 128256),
+    # Llama-3.1-405B's layer shapes (16 query heads per K/V head); run on a few of its 126 layers (--decode-layers)
+    "405b": (126, 16384, 128, 8, 128, 53248, 128256),
+}
+
+
 def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool, only_prefill: int = 0,
-               with_prefill: bool = True, only_verify: int = 0, attn_timeline: bool = False) -> dict:
+               with_prefill: bool = True, only_verify: int = 0, attn_timeline: bool = False, model: str = "8b",
+               layers_run: int = 0) -> dict:
     """Batch-1 decode of an 8B-shaped Llama (32 layers: wq, wo 4096x4096, wk, wv 4096->1024, gate, up
     4096->14336 in Q4_K; down 14336->4096 and the 128256-row output in Q6_K; f16 KV cache holding `ctx`
     random positions): tokens per second of ogm_llama_decode_dev with the embedding row, the logits and
     the greedy token resident in HBM.  Every layer has its own device copy of the weights."""
     from orangu_amd import LlamaDecoder, QuantMatrix
     Q6_K = 14
-    n_layer, n_embd, n_head, n_kv, hd, n_ff, n_vocab = 32, 4096, 32, 8, 128, 14336, 128256
+    n_layer_model, n_embd, n_head, n_kv, hd, n_ff, n_vocab = DECODE_MODELS[model]
+    n_layer = layers_run if layers_run > 0 else n_layer_model
     seed = 515
     rng = np.random.default_rng(seed)
     shapes = {"wq": (Q4_K, n_embd, n_embd), "wk": (Q4_K, n_embd, n_kv * hd), "wv": (Q4_K, n_embd, n_kv * hd),
@@ -376,7 +385,9 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     weights = n_layer * sum(o * (i // 256) * (144 if t == Q4_K else 210) for t, i, o in shapes.values()) \
         + n_vocab * (n_embd // 256) * 210
     kv_bytes = 2 * n_layer * ctx * n_kv * hd * 2
-    res = {"workload": f"configs[4]: 8B-shaped Llama Q4_K_M-like, batch-1 greedy decode at context {ctx}",
+    what = "configs[4]: 8B-shaped Llama Q4_K_M-like" if model == "8b" else \
+        f"{n_layer} of the {n_layer_model} layers of a {model.upper()}-shaped Llama Q4_K_M-like (and its output matrix)"
+    res = {"workload": f"{what}, batch-1 greedy decode at context {ctx}",
            "tok_per_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4),
            "generate_tok_per_s": round(1.0 / dt_gen, 1), "generated": [int(t) for t in toks[:4]],
            "prefill_512_ms": round(dt_pre * 1e3, 2) if dt_pre else None,
@@ -484,6 +495,10 @@ def main() -> int:
     ap.add_argument("--decode-steps", type=int, default=64,
                     help="tokens of the 8B-shaped decode leg (config 5); 0 skips it")
     ap.add_argument("--decode-ctx", type=int, default=2048, help="cached positions of the decode leg")
+    ap.add_argument("--decode-model", choices=sorted(DECODE_MODELS), default="8b",
+                    help="with --only-decode: the model whose layer shapes are decoded (405b: give --decode-layers too)")
+    ap.add_argument("--decode-layers", type=int, default=0,
+                    help="with --only-decode: run this many layers of the model instead of all of them")
     ap.add_argument("--only-decode", action="store_true", help="run only the decode leg (for rocprofv3)")
     ap.add_argument("--attn-timeline", action="store_true",
                     help="with --lib of a variant built with -DOGM_ATTN_STAMPS=1: the decode attention kernel's phases")
@@ -558,7 +573,7 @@ def main() -> int:
         return 0
     if args.only_decode:
         print(json.dumps(decode_leg(be, helpers, hiprt, max(1, args.decode_steps), 8, args.decode_ctx, False,
-                                    with_prefill=False)))
+                                    with_prefill=False, model=args.decode_model, layers_run=args.decode_layers)))
         be.close()
         return 0
     if args.wg_waves:

@@ -603,14 +603,29 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
     }
   }
   // Two to sixteen tokens over a K-quant matrix (a speculative-decode verify batch, a decode batch): the GEMV's
-  // distribution with the products on the matrix cores, in either float order.
-  // Measured at the 8B shapes (4096 -> 1024 / 4096 / 14336 Q4_K, 14336 -> 4096 Q6_K): Q6_K from two tokens on
-  // (4 tokens: 18 us against 30), Q4_K / Q5_K from five (up to four the GEMV kernel's per-token dot instructions
-  // are level or ahead: 13 us against 15 at 14336 rows; at eight 16 against 17.5 for the small-batch GEMM).
+  // distribution with the products on the matrix cores, in either float order.  Its workgroups stage all their
+  // tokens' activations of the whole row in LDS, so what it wins depends on the row length and on how many
+  // workgroups the launch has.  Measured on MI355X against what runs otherwise (the GEMV kernel up to five tokens,
+  // the small-batch GEMM from six), whole calls, rows = all matrices of the launch:
+  //   Q4_K, 5 / 8 tokens, us   4096 -> 4096  8.6 / 8.8 against 9.4 / 10.4;  4096 -> 28672  23.8 / 23.4 against 23.3 / 29.6;
+  //     4096 -> 57344  42 / 40 against 46 / 49;  5120 -> 8192  11.7 / 12.2 against 13.9 / 15.9;  5120 -> 16384  20.7 / 23.9
+  //     against 26.8 / 20.8;  8192 -> 4096  10.7 / 11.1 against 12.2 / 16.1;  8192 -> 8192  18.4 / 19.3 against 17.2 /
+  //     18.4;  8192 -> 28672  72 / 78 against 49 / 53 (64 KB of activations a workgroup: one or two to a compute unit)
+  //   Q6_K, 2 / 4 / 8 tokens   14336 -> 4096  18.5 / 18.2 / 21.2 against 15.9 / 20.3 / 23.8;  14336 -> 8192  34 / 36 / 42
+  //     against 26 / 36 / 30;  8192 -> 4096  12.9 / 13.1 / 13.6 against 11.2 / 13.2 / 14.7;  8192 -> 8192  23 / 23.5 / 27
+  //     against 18.6 / 22.5 / 19.4
   // Nine to sixteen tokens need sixteen token slots, whose activations and terms leave one workgroup of four
   // waves to a compute unit (gate and up at 16 tokens: 56 us against 18 for the small-batch GEMM): by default the
   // kernel stops at eight.
-  const uint32_t mma_from = ctx->tune_gemv_mma == 2 ? 2u : t0 == OGM_Q6_K ? 2u : 5u;
+  uint64_t rows_all = 0;
+  for (size_t i = 0; i < n_tg; i++) rows_all += tg[i].w->out_dim;
+  bool mma_pays;
+  if (t0 == OGM_Q6_K)
+    mma_pays = (n_tokens >= 4 && n_tokens < gemm_from && rows_all <= 8192) || (n_tokens >= gemm_from && rows_all <= 4096);
+  else
+    mma_pays = n_tokens >= 5 && (w0->in_dim <= 4096 || (w0->in_dim <= 5120 && (n_tokens == 5 || rows_all <= 8192)) ||
+                                 (w0->in_dim <= 8192 && rows_all <= 4096));
+  const uint32_t mma_from = ctx->tune_gemv_mma == 2 ? 2u : (mma_pays ? 2u : 17u);
   const uint32_t mma_to = ctx->tune_gemv_mma == 2 ? 16u : 8u;
   if (ctx->tune_gemv_mma != 0 && n_tokens >= mma_from && n_tokens <= mma_to && !dump_isum && !dump_imin && !act_base &&
       ogm_gemv_mma_eligible(w0->ggml_type, w0->in_dim, n_tokens, gemm_order)) {
@@ -638,7 +653,13 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
     }
     return OGM_OK;
   }
-  if (gemm_order && !dump_isum && !dump_imin && !act_base && n_tokens >= gemm_from &&
+  // (also below that count when the GEMV kernel's LDS holds fewer tokens of such long rows than the batch has and
+  // it would read the weights once per part: Q6_K 53248 -> 16384 at 4 tokens 450 us against 180, Q4_K 16384 -> 16384
+  // 65 against 52)
+  const uint32_t gemv_chunk = ogm_gemv_max_tokens(w0->ggml_type, w0->in_dim, gemm_order);
+  const bool gemv_rereads = gemv_chunk != 0 && n_tokens > gemv_chunk && ctx->tune_gemm_min_tokens == 0 &&
+                            block_elems_of(w0->ggml_type) == 256;   // (the 32-wide types' GEMM pays from 17 tokens only)
+  if (gemm_order && !dump_isum && !dump_imin && !act_base && (n_tokens >= gemm_from || gemv_rereads) &&
       all_gemm_supported(tg, n_tg, n_tokens)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)
     int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(w0->in_dim, n_tokens));
@@ -684,7 +705,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
     return OGM_OK;
   }
   const uint32_t wg_waves = (uint32_t)ctx->tune_wg_waves;
-  const uint32_t chunk = ogm_gemv_max_tokens(w0->ggml_type, w0->in_dim, gemm_order);
+  const uint32_t chunk = gemv_chunk;
   if (chunk == 0) return fail(ctx, OGM_ERR_UNSUPPORTED, "no kernel for this type");
   const uint32_t blocks_per_row = w0->in_dim / block_elems_of(w0->ggml_type);
   for (size_t g0 = 0; g0 < n_tg; g0 += OGM_GEMV_MAX_MATS) {

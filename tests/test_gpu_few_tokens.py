@@ -138,13 +138,16 @@ def test_row_block_kernel_at_the_8b_shapes(be):
 
 
 def test_default_routing_of_few_token_batches():
-    """Without tuning: Q6_K goes to the row-block kernel from two tokens, Q4_K and Q5_K from five, all up to eight;
-    one token never, nine and more to the small-batch GEMM."""
+    """Without tuning: Q6_K goes to the row-block kernel from four tokens, Q4_K and Q5_K from five, all up to eight;
+    one token never, nine and more to the small-batch GEMM.  Shapes the kernel measured slower on stay off it: from
+    six tokens Q6_K matrices of more than 4096 rows, Q4_K / Q5_K rows of more than 5120 inputs with more than 4096
+    rows.  A batch that the GEMV kernel's LDS cannot hold at once (long rows) goes to the small-batch GEMM however
+    few its tokens, instead of reading the weights once per part.  Same bits everywhere."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
     try:
-        for t, T, want in ((Q6_K, 1, "ogm_gemv_kernel<FmtQ6K,gemv>"), (Q6_K, 2, NAME[Q6_K]), (Q6_K, 8, NAME[Q6_K]),
-                           (Q6_K, 9, "ogm_gemm_sb_q6k_kernel"),
+        for t, T, want in ((Q6_K, 1, "ogm_gemv_kernel<FmtQ6K,gemv>"), (Q6_K, 2, "ogm_gemv_kernel<FmtQ6K,gemm>"),
+                           (Q6_K, 4, NAME[Q6_K]), (Q6_K, 8, NAME[Q6_K]), (Q6_K, 9, "ogm_gemm_sb_q6k_kernel"),
                            (Q4_K, 4, "ogm_gemv_kernel<FmtQ4K,gemm>"), (Q4_K, 5, NAME[Q4_K]), (Q4_K, 8, NAME[Q4_K]),
                            (Q4_K, 16, "ogm_gemm_sb_q4k_kernel"),
                            (Q5_K, 3, "ogm_gemv_kernel<FmtQ5K,gemm>"), (Q5_K, 8, NAME[Q5_K]), (Q5_K, 9, "ogm_gemm_sb_q5k_kernel")):
@@ -153,5 +156,20 @@ def test_default_routing_of_few_token_batches():
             got = b.matmul(x, T, qm(raw, t, 1024, 48))
             assert b.last_kernel() == want, (t, T, b.last_kernel())
             assert_bits(got, oracle.matmul(t, raw, 1024, 48, x, T), f"type {t} at {T} tokens")
+        for t, in_dim, out_dim, T, want in (
+                (Q6_K, 1024, 4100, 5, NAME[Q6_K]), (Q6_K, 1024, 4100, 7, "ogm_gemm_sb_q6k"),       # many rows: to 5 tokens only
+                (Q6_K, 1024, 8200, 4, "ogm_gemv_kernel<FmtQ6K,gemm>"),
+                (Q4_K, 8192, 4096, 6, NAME[Q4_K]), (Q4_K, 8192, 4100, 6, "ogm_gemm_sb_q4k"),        # long rows: few rows only
+                (Q4_K, 5120, 8200, 5, NAME[Q4_K]), (Q4_K, 5120, 8200, 7, "ogm_gemm_sb_q4k"),
+                (Q6_K, 28672, 300, 2, "ogm_gemv_kernel<FmtQ6K,gemm>"), (Q6_K, 28672, 300, 3, "ogm_gemm_sb_q6k"),   # parts of two tokens
+                (Q6_K, 53248, 70, 2, "ogm_gemm_sb_q6k"), (Q4_K, 16384, 200, 3, "ogm_gemv_kernel<FmtQ4K,gemm>"),
+                (Q4_K, 16384, 200, 4, "ogm_gemm_sb_q4k")):
+            raw = synth_weights(t, in_dim, out_dim, seed=T + out_dim)
+            x = synth_x(T, in_dim, seed=T)
+            w = qm(raw, t, in_dim, out_dim)
+            got = b.matmul(x, T, w)
+            assert b.last_kernel().startswith(want), (t, in_dim, out_dim, T, b.last_kernel())
+            assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), f"type {t} {in_dim}->{out_dim} at {T} tokens")
+            b.evict(w)
     finally:
         b.close()
