@@ -450,7 +450,7 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              near zero can differ from the reference's by more than 1e-3 of itself
  *   "gemv_mma"                 2 to 16 tokens over Q4_K / Q5_K / Q6_K rows on the kernel
  *                              that gives a workgroup one row block and multiplies on the matrix cores: 1 =
- *                              default, where it measured faster (Q6_K from two tokens, Q4_K / Q5_K from five, all
+ *                              default, where it measured faster (Q6_K from four tokens, Q4_K / Q5_K from five, all
  *                              up to eight); 2 = wherever it can (two to sixteen); 0 = never.  Same bits as the
  *                              other kernels
  *   "attn_prefill_variant"     attention of a prefill batch: 1 = the decode step's kernel per token and chunk of
