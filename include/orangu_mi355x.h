@@ -451,8 +451,8 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *   "gemv_mma"                 2 to 16 tokens over Q4_K / Q5_K / Q6_K rows on the kernel
  *                              that gives a workgroup one row block and multiplies on the matrix cores: 1 =
  *                              default, where it measured faster (Q6_K from four tokens, Q4_K / Q5_K from five, all
- *                              up to eight); 2 = wherever it can (two to sixteen); 0 = never.  Same bits as the
- *                              other kernels
+ *                              up to eight; rows of up to 4096 inputs, longer ones only in launches of few rows);
+ *                              2 = wherever it can (two to sixteen); 0 = never.  Same bits as the other kernels
  *   "attn_prefill_variant"     attention of a prefill batch: 1 = the decode step's kernel per token and chunk of
  *                              the cache; 2 = the matrix-core kernel; 0 = default: the first for batches of up to
  *                              48 tokens (speculative-decode verify batches), the second above; they agree to
