@@ -417,9 +417,11 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              kernel runs in the GEMM's float order
  *   "gemm_small_max_tokens"    K-quant GEMMs of at most this many tokens take the small-batch kernel, whose
  *                              waves work on different super-blocks of the same rows; 0 = default (64, more
- *                              for matrices of few rows), 1 = never
+ *                              for matrices of few rows, up to 512 for Q4_K / Q5_K matrices of at most 2048; Q6_K
+ *                              launches that "gemm_interleave" sends to its kernel by their size go there
+ *                              first), 1 = never
  *   "gemm_sb_waves"            waves of a small-batch workgroup: 8 or 16; 0 = by the size of the launch
- *   "gemm_medium"              the Q4_K / Q5_K kernel for one or two nearly full tiles of 128 tokens (32 rows x
+ *   "gemm_medium"              the Q4_K / Q5_K kernel for one nearly full tile of 128 tokens, or two (32 rows x
  *                              128 tokens a workgroup, its waves on different super-blocks): 0 = by the size of
  *                              the launch, 1 = never, 2 = whenever the shape allows
  *   "gemm_tile_rows"           feeding-wave GEMMs: 64 = always their 64-row tiles; 0 = by the size of the launch
@@ -437,11 +439,12 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              128 rows x 128 tokens (the feeding-wave kernels unpack otherwise); 2 = whatever
  *                              the grid, from 32 tokens
  *   "gemm_interleave"          the plane kernel with 64-row tiles that adds a super-block up between the next
- *                              one's matrix instructions (Q4_K, Q5_K, Q6_K): 0 = default, on launches of three
- *                              or more token tiles of 128 that leave the 128-row kernel's places under three
- *                              quarters full and have at least 160 tiles of 64 rows (the 8B shapes' q/k/v, wo and
- *                              down projections at 257 to 1024 tokens; their planes are built then); 1 = never;
- *                              2 = wherever the plane kernel runs.  Same bits
+ *                              one's matrix instructions (Q4_K, Q5_K, Q6_K): 0 = default, on launches of at most
+ *                              512 tiles of 64 rows x 128 tokens: Q6_K from 128 such tiles (a lone token tile more
+ *                              than three quarters full) or 96 with at least 192 tokens; Q4_K / Q5_K from three
+ *                              token tiles and 160 tiles, with rows longer than 5120 inputs at most 256 (the 8B
+ *                              shapes' q/k/v, wo and down projections at 257 to 1024 tokens, down from 129; their
+ *                              planes are built then); 1 = never; 2 = wherever the plane kernel runs.  Same bits
  *   "gemm_one_pass"            0 = default.  1: Q4_K and Q5_K on that kernel skip the reference GEMM's separate
  *                              first pass over the mins (vecdot.rs:2229-2240) and add
  *                              ad * (d * isum - dmin * imin) per super-block, the single-token expression of

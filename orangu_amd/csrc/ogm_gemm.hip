@@ -2380,20 +2380,85 @@ hipError_t ogm_gemm_build_planes(uint32_t ggml_type, const uint8_t *wt, uint32_t
   return hipGetLastError();
 }
 
-// Whether a K-quant launch takes the small-batch kernel (workgroups of 32 rows x 32 tokens whose waves take
-// different super-blocks) rather than a tiled one.
-static bool gemm_small_batch(const OgmGemmArgs &a) {
+// Whether a launch over planes takes the kernel with 64-row tiles that adds a super-block up between the next one's
+// matrix instructions (ogm_gemm_dmx_kernel) instead of the one with 128-row tiles (ogm_gemm_dma_kernel).
+// interleave: 0 by the size of the launch, 1 never, 2 whenever the type allows.  Measured on MI355X, whole calls at
+// 512 tokens, us, 64-row interleaved / 128-row / feeding waves: Q6_K 14336 -> 4096 103 / 153 / 126, Q4_K 4096 ->
+// 4096 42 / 64 / 49, 4096 -> 6144 54 / 67 / 64, 14336 -> 4096 130 / 204 / 150; but 4096 -> 14336 115 / 98 / -.
+// Its workgroups (64 rows x 128 tokens) must fit the device in one round, two to a compute unit: beyond 512 of
+// them the 128-row kernel is ahead (Q4_K 4096 -> 14336 at 384 tokens, 672 workgroups: 91 against 87; 5120 -> 13824
+// at 288: 104 against 99; 8192 -> 10240 at 512: 174 against 165).
+//   Q6_K has no first pass to pay for and no medium-batch kernel beside it, so it takes this kernel from 128
+// workgroups on, and from 96 with at least 192 tokens, before the small-batch kernel is asked (against the small-batch
+// and feeding-wave kernels: 14336 -> 4096 at 256 tokens 87 against 101, 4096 -> 4096 at 256 28 against 38, 8192 ->
+// 2048 at 384 50 against 61, 13824 -> 5120 at 160 79 against 93, 28672 -> 8192 at 128 171 against 199; level with
+// them at 160 tokens of the 4096-row matrices; behind with fewer workgroups: 8192 -> 2048 at 256 tokens, 64 of them,
+// 47 against 38).  A lone token tile wants to be nearly full.
+//   Q4_K / Q5_K want three token tiles and 160 workgroups (at 256 tokens it only draws with the medium-batch kernel,
+// which needs no planes: 4096 -> 6144 37 against 37), and with longer rows than 5120 inputs no more workgroups than
+// compute units (8192 -> 8192 at 384 / 512 tokens, 384 / 512 workgroups, 114 / 127 against 101 / 113 for the
+// feeding-wave kernel, 8192 -> 10240 at 384 120 against 108; but 14336 -> 4096 at 384 / 512 tokens, 192 / 256
+// workgroups, 121 / 127 against 135 / 143).
+static bool gemm_interleaved(const OgmGemmArgs &a) {
   const uint32_t nsb = a.in_dim / 256;
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  if (a.interleave == 1u || a.ggml_type == OGM_Q3_K || (q45 && a.one_pass != 0u) || nsb * 512u > GX_TAB || a.n_tokens < 32u)
+    return false;
+  if (a.interleave == 2u) return true;
+  uint32_t tiles64 = 0;
+  for (uint32_t m = 0; m <= a.n_extra; m++) tiles64 += ((m ? a.extra_out_dim[m - 1] : a.out_dim) + 63u) / 64u;
+  const uint32_t tok_tiles = (a.n_tokens + 127u) / 128u;
+  const uint32_t n_wg = tok_tiles * tiles64;
+  if (n_wg > 512u) return false;
+  if (!q45) return (n_wg >= 128u && (tok_tiles >= 2u || a.n_tokens > 96u)) || (n_wg >= 96u && a.n_tokens >= 192u);
+  return tok_tiles >= 3u && n_wg >= 160u && (nsb <= 20u || n_wg <= 256u);
+}
+
+// Whether a tiled launch goes to a kernel whose waves all multiply, given planes.  The one with 128 x 128
+// workgroups wants more of them than there are compute units (two share one, and one alone is slower than the
+// feeding-wave kernels: Q4_K 4096 -> 14336 at 256 tokens 69 us against 57, at 384 tokens 87 against 104), the
+// activations in operand chunks, and everything within 32-bit byte offsets.  (plane_kernel 2: whatever the
+// grid.)
+static bool gemm_dma_eligible(const OgmGemmArgs &a) {
+  const uint32_t nsb = a.in_dim / 256;
+  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
+  if ((q45 && nsb * 512u > GD_TAB) || a.n_tokens < 32u || !a.xh || (uint64_t)t_pad * a.in_dim >= (1ull << 32))
+    return false;
+  uint32_t tiles = 0;
+  for (uint32_t m = 0; m <= a.n_extra; m++) {
+    const uint32_t od = m ? a.extra_out_dim[m - 1] : a.out_dim;
+    if ((uint64_t)((od + 63u) / 64u) * 64u * a.in_dim * 2u >= (1ull << 32)) return false;
+    tiles += (od + GD_ROWS - 1u) / GD_ROWS;
+  }
+  if (a.plane_kernel == 2u || ((a.n_tokens + GD_TOK - 1u) / GD_TOK) * tiles > 256u) return true;
+  return gemm_interleaved(a);
+}
+
+// Whether a K-quant launch takes the small-batch kernel (workgroups of 32 rows x 32 tokens whose waves take
+// different super-blocks) rather than a tiled one.
+// planes_possible: whether the launch has (or, asked before they are built, may get) every matrix's planes.
+static bool gemm_small_batch(const OgmGemmArgs &a, bool planes_possible) {
+  const uint32_t nsb = a.in_dim / 256;
+  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  // Q6_K launches the interleaved plane kernel wants by their size go there (see gemm_interleaved)
+  if (a.ggml_type == OGM_Q6_K && a.small_max_tokens == 0u && a.interleave == 0u && planes_possible &&
+      gemm_dma_eligible(a) && gemm_interleaved(a))
+    return false;
   uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
   for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
   // (measured, Q4_K from 4096 inputs, small-batch against tiled, us: 4096 rows at 192 / 256 / 384 tokens 36 against 45,
   // 39 against 46, 57 against 49; 6144 rows at 128 / 192: 37 against 47, 47 against 47; 14336 rows at 64 / 96: 38 against 44,
   // 51 against 46)
-  // (the last 32 tokens of the two larger limits belong to the medium-batch kernel where that runs: see gemm_medium_batch)
+  // (where the medium-batch kernel runs it takes over earlier: see gemm_medium_batch; 4096 rows at 160 / 192 / 224
+  // tokens 34 / 35 / 37 against its 33 / 33 / 33.  Up to 2048 rows the small batches stay ahead for longer: 2048 ->
+  // 2048 at 256 / 384 / 512 tokens 15 / 20 / 23 against 20 / 21 / 22 medium and 24 / 26 / 26 tiled)
   const bool med = q45 && a.medium != 1u;
   const uint32_t small_max = a.small_max_tokens ? a.small_max_tokens
-                             : (tiles64_all <= 64u ? (med ? 224u : 256u) : tiles64_all <= 128u ? (med ? 96u : 128u) : 64u);
+                             : (tiles64_all <= 32u   ? (q45 ? 512u : 256u)
+                                : tiles64_all <= 64u ? (med ? 160u : 256u)
+                                : tiles64_all <= 128u ? (med ? 96u : 128u)
+                                                      : 64u);
   return a.ggml_type != OGM_Q3_K && a.small_max_tokens != 1u && a.n_tokens <= small_max &&
          (q45 ? 16u : 8u) * 4096u + 128u * nsb <= GM_LDS_MAX;
 }
@@ -2412,8 +2477,10 @@ static bool gemm_medium_batch(const OgmGemmArgs &a) {
   // Measured on MI355X against the kernels it displaces, whole calls, us: 4096 -> 14336 at 128 tokens 42 against 50
   // (feeding waves), at 192 / 256 tokens 78 / 77 against 65 / 65; 4096 -> 4096 at 256 tokens 35 against 39 (small
   // batch), at 128 tokens 33 against 23; 4096 -> 6144 at 128 / 256 tokens 34 / 40 against 36 / 46; 14336 -> 4096 at
-  // 256 tokens 106 against 116.  It wants its token tiles of 128 nearly full, and at two of them matrices of at most
-  // 8192 rows (beyond, the 128-row tiles of the feeding-wave kernels outnumber the compute units' halves).  Its
+  // 256 tokens 106 against 116.  It wants a lone token tile of 128 nearly full (below, the small batches), and at two
+  // of them, full or not, matrices of at most 8192 rows (4096 -> 6144 at 144 / 192 tokens 38 / 37 against 43 / 43 for
+  // the feeding waves, 8192 -> 8192 68 / 69 against 80 / 82; beyond 8192 rows the 128-row tiles of the feeding-wave
+  // kernels outnumber the compute units' halves).  Its
   // workgroups of 32 rows must fit the device in one round, two to a compute unit: gate and up together (28672 rows,
   // 896 workgroups) take 63 us against 56 for the feeding-wave kernel (128-token prefill of the 8B shapes 7.0
   // against 6.65 ms), so at one token tile the launch may have at most 16384 rows.
@@ -2421,52 +2488,7 @@ static bool gemm_medium_batch(const OgmGemmArgs &a) {
   for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
   const uint32_t tok_tiles = (a.n_tokens + SBW_TOK - 1u) / SBW_TOK;
   const bool full_enough = tok_tiles * SBW_TOK - a.n_tokens <= 32u;
-  return full_enough && ((tok_tiles == 1u && tiles64_all <= 256u) || (tok_tiles == 2u && tiles64_all <= 128u));
-}
-
-// Whether a tiled launch goes to the kernel whose waves all multiply, given planes.  It wants more
-// 128 x 128 workgroups than there are compute units (two share one, and one alone is slower than the
-// feeding-wave kernels: Q4_K 4096 -> 14336 at 256 tokens 69 us against 57, at 384 tokens 87 against 104), the
-// activations in operand chunks, and everything within 32-bit byte offsets.  (plane_kernel 2: whatever the
-// grid.)
-// Whether a launch over planes takes the kernel with 64-row tiles that adds a super-block up between the next one's
-// matrix instructions (ogm_gemm_dmx_kernel) instead of the one with 128-row tiles (ogm_gemm_dma_kernel).
-// interleave: 0 by the size of the launch, 1 never, 2 whenever the type allows.  Measured on MI355X, whole calls at
-// 512 tokens, us, 64-row interleaved / 128-row / feeding waves: Q6_K 14336 -> 4096 103 / 153 / 126, Q4_K 4096 ->
-// 4096 42 / 64 / 49, 4096 -> 6144 54 / 67 / 64, 14336 -> 4096 130 / 204 / 150; but 4096 -> 14336 115 / 98 / -, and
-// at 1024 tokens 4096 -> 6144 92 / 89, 4096 -> 4096 64 / 71: the 128-row kernel wants its 512 places (two workgroups
-// a compute unit) three quarters full, the 64-row one at least 160 tiles and three token tiles (at 256 tokens it
-// only draws with the kernels that need no planes: 4096 -> 14336 67 against 70, 4096 -> 6144 39 against 41).
-static bool gemm_interleaved(const OgmGemmArgs &a) {
-  const uint32_t nsb = a.in_dim / 256;
-  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
-  if (a.interleave == 1u || a.ggml_type == OGM_Q3_K || (q45 && a.one_pass != 0u) || nsb * 512u > GX_TAB || a.n_tokens < 32u)
-    return false;
-  if (a.interleave == 2u) return true;
-  uint32_t tiles128 = 0, tiles64 = 0;
-  for (uint32_t m = 0; m <= a.n_extra; m++) {
-    const uint32_t od = m ? a.extra_out_dim[m - 1] : a.out_dim;
-    tiles128 += (od + 127u) / 128u;
-    tiles64 += (od + 63u) / 64u;
-  }
-  const uint32_t tok_tiles = (a.n_tokens + 127u) / 128u;
-  return tok_tiles >= 3u && tok_tiles * tiles128 < 384u && tok_tiles * tiles64 >= 160u;
-}
-
-static bool gemm_dma_eligible(const OgmGemmArgs &a) {
-  const uint32_t nsb = a.in_dim / 256;
-  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
-  const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
-  if ((q45 && nsb * 512u > GD_TAB) || a.n_tokens < 32u || !a.xh || (uint64_t)t_pad * a.in_dim >= (1ull << 32))
-    return false;
-  uint32_t tiles = 0;
-  for (uint32_t m = 0; m <= a.n_extra; m++) {
-    const uint32_t od = m ? a.extra_out_dim[m - 1] : a.out_dim;
-    if ((uint64_t)((od + 63u) / 64u) * 64u * a.in_dim * 2u >= (1ull << 32)) return false;
-    tiles += (od + GD_ROWS - 1u) / GD_ROWS;
-  }
-  if (a.plane_kernel == 2u || ((a.n_tokens + GD_TOK - 1u) / GD_TOK) * tiles > 256u) return true;
-  return gemm_interleaved(a);
+  return (tok_tiles == 1u && full_enough && tiles64_all <= 256u) || (tok_tiles == 2u && tiles64_all <= 128u);
 }
 
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a) {
@@ -2474,7 +2496,7 @@ bool ogm_gemm_uses_planes(const OgmGemmArgs &a) {
   if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return false;
   // (the feeding-wave kernels unpack on every call: reading planes made them no faster -- Q4_K 4096 -> 14336 at 256
   // tokens 66 against 66 us, Q6_K 14336 -> 4096 at 512 tokens 96 against 98)
-  return !gemm_small_batch(a) && gemm_dma_eligible(a);
+  return !gemm_small_batch(a, true) && gemm_dma_eligible(a);
 }
 
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name) {
@@ -2518,7 +2540,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   // (Q4_K 4096 -> 14336: 18 / 35 / 50 us at 32 / 64 / 96 tokens against 42-45 us tiled), and up to 128
   // when the tiled kernel's grid would leave half the CUs idle (4096 -> 4096: 12 / 15 / 21 us at 32 /
   // 64 / 128 tokens against 38-41; 14336 -> 4096: 36 / 39 / 57 against 123-130).
-  if (gemm_small_batch(a)) {
+  bool have_planes = a.planes != nullptr;
+  for (uint32_t m = 0; m < a.n_extra; m++) have_planes = have_planes && a.extra_planes[m] != nullptr;   // every matrix of the launch, or none
+  if (gemm_small_batch(a, have_planes)) {
     GemmSbParams p;
     p.wt = a.wt;
     p.xq = a.act.q;
@@ -2559,8 +2583,6 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
                                                : (w16 ? "ogm_gemm_sb_q5k_w16_kernel" : "ogm_gemm_sb_q5k_kernel");
     return hipGetLastError();
   }
-  bool have_planes = a.planes != nullptr;
-  for (uint32_t m = 0; m < a.n_extra; m++) have_planes = have_planes && a.extra_planes[m] != nullptr;   // every matrix of the launch, or none
   const bool dma = have_planes && gemm_dma_eligible(a);
   if ((!dma || a.medium == 2u) && gemm_medium_batch(a)) {   // (asked for by name, it comes before the planes)
     const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;

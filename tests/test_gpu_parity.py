@@ -599,11 +599,13 @@ def test_medium_batch_kernel_over_several_matrices_and_extreme_ranges(be):
 def test_gemm_threshold_default():
     """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
     float order, 17 through the matrix-core GEMM.  Q4_K: 4 tokens through the GEMV kernel, 5 to 8 through the
-    row-block kernel, 9 to 224
-    through the small-batch kernel (a matrix of few rows), 225 to 256 through the medium-batch kernel, 257
-    through the tiled one; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
+    row-block kernel, then the small-batch kernel: to 512 tokens over a matrix of up to 2048 rows, to 160 over one
+    of up to 4096, where the medium-batch kernel has the rest of the second token tile and a tiled kernel what
+    follows; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
     many that 128 x 128 tiles outnumber the compute units has its planes built and read by the kernel whose
     waves all multiply, while a single nearly full token tile over at most 16384 rows goes to the medium-batch kernel.
+    Q6_K goes to the 64-row plane kernel wherever that has 128 workgroups and a token tile more than three quarters
+    full, or 96 workgroups and 192 tokens, before the small-batch kernel is asked.
     Same bits everywhere."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
@@ -621,14 +623,23 @@ def test_gemm_threshold_default():
         raw = synth_weights(Q4_K, 1024, 70, seed=5)
         w = qm(raw, Q4_K, 1024, 70)
         want = oracle.matmul(Q4_K, raw, 1024, 70, x, 257).reshape(257, 70)
-        # (up to 64 tiles of 64 rows the small-batch kernel keeps batches of up to 224 tokens)
+        # (up to 32 tiles of 64 rows the small-batch kernel keeps batches of up to 512 tokens)
         for n, kernel in ((4, "ogm_gemv_kernel"), (5, "ogm_gemm_fk_kernel<Q4_K>"), (8, "ogm_gemm_fk_kernel<Q4_K>"),
                           (9, "ogm_gemm_sb_q4k_kernel"), (128, "ogm_gemm_sb_q4k_kernel"),
-                          (224, "ogm_gemm_sb_q4k_kernel"), (225, "ogm_gemm_sbw_q4k_kernel"),
-                          (256, "ogm_gemm_sbw_q4k_kernel"), (257, "ogm_gemm_q4k_i8p_r64_kernel")):
+                          (257, "ogm_gemm_sb_q4k_kernel")):
             y = b.matmul(x[:n], n, w)
             assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, want[:n], f"Q4_K, {n} tokens")
+        # (up to 64 tiles, up to 160 tokens; then the medium-batch kernel has the second token tile, full or not)
+        raw = synth_weights(Q4_K, 256, 2100, seed=25)
+        w = qm(raw, Q4_K, 256, 2100)
+        x2 = np.ascontiguousarray(x[:, :256])
+        want = oracle.matmul(Q4_K, raw, 256, 2100, x2, 257).reshape(257, 2100)
+        for n, kernel in ((160, "ogm_gemm_sb_q4k_kernel"), (161, "ogm_gemm_sbw_q4k_kernel"),
+                          (256, "ogm_gemm_sbw_q4k_kernel"), (257, "ogm_gemm_q4k_i8p_r64_kernel")):
+            y = b.matmul(x2[:n], n, w)
+            assert kname(b).startswith(kernel), (n, kname(b))
+            assert_bits(y, want[:n], f"Q4_K of 2100 rows, {n} tokens")
         raw = synth_weights(Q4_K, 768, 70, seed=15)    # three super-blocks a row: tiles of 64 rows, one block wide
         w3 = qm(raw, Q4_K, 768, 70)
         x3 = np.ascontiguousarray(x[:9, :768])
@@ -643,11 +654,21 @@ def test_gemm_threshold_default():
         assert_bits(y, oracle.matmul(Q5_K, raw, 4096, 70, x4, 12), "Q5_K, 12 tokens")
         raw = synth_weights(Q6_K, 256, 8300, seed=6)   # 130 tiles of 64 rows
         w = qm(raw, Q6_K, 256, 8300)
-        want = oracle.matmul(Q6_K, raw, 256, 8300, np.ascontiguousarray(x[:65, :256]), 65).reshape(65, 8300)
-        for n, kernel in ((64, "ogm_gemm_sb_q6k_kernel"), (65, "ogm_gemm_q6k_i8_r64_kernel")):
+        want = oracle.matmul(Q6_K, raw, 256, 8300, np.ascontiguousarray(x[:97, :256]), 97).reshape(97, 8300)
+        # (a token tile of the 64-row plane kernel wants more than 96 tokens; Q6_K takes it from 128 workgroups)
+        for n, kernel in ((64, "ogm_gemm_sb_q6k_kernel"), (65, "ogm_gemm_q6k_i8_r64_kernel"), (97, "ogm_gemm_q6k_dmx_kernel")):
             y = b.matmul(np.ascontiguousarray(x[:n, :256]), n, w)
-            assert kname(b) == kernel, (n, kname(b))
+            assert b.last_kernel() == kernel, (n, b.last_kernel())
             assert_bits(y, want[:n], f"Q6_K, {n} tokens")
+        raw6 = synth_weights(Q6_K, 512, 3100, seed=16)  # 49 tiles of 64 rows: small batches to 256 tokens, unless
+        w6 = qm(raw6, Q6_K, 512, 3100)                   # there are 192 tokens in at least 96 workgroups
+        x6 = np.ascontiguousarray(x[:257, :512])
+        want = oracle.matmul(Q6_K, raw6, 512, 3100, x6, 257).reshape(257, 3100)
+        for n, kernel in ((128, "ogm_gemm_sb_q6k_kernel"), (191, "ogm_gemm_sb_q6k_kernel"), (192, "ogm_gemm_q6k_dmx_kernel"),
+                          (257, "ogm_gemm_q6k_dmx_kernel")):
+            y = b.matmul(x6[:n], n, w6)
+            assert b.last_kernel() == kernel, (n, b.last_kernel())
+            assert_bits(y, want[:n], f"Q6_K of 3100 rows, {n} tokens")
         raw = synth_weights(Q4_K, 256, 16600, seed=9)   # 130 tiles of 128 rows x 2 of 128 tokens
         w = qm(raw, Q4_K, 256, 16600)
         x5 = np.ascontiguousarray(x[:129, :256])
