@@ -192,3 +192,52 @@ def test_default_routing_on_matrices_of_many_rows(be, t, in_dim, out_dim, T, i):
             assert bad.size == 0, f"matmul_decode via {be.last_kernel()}: {bad.size} of {want.size} differ"
     finally:
         be.evict(w)
+
+
+def _medium_grids(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        t = int(rng.choice((11, 12, 13, 14)))
+        in_dim = int(rng.choice((256, 512, 1024, 2048)))
+        out_dim = int(rng.choice((2100, 3100, 4100, 6200, 8300))) + int(rng.integers(-70, 70))
+        T = int(rng.choice((97, 129, 161, 192, 224, 257, 300, 385, 513, 641)))
+        if T * out_dim * in_dim > 3e9:
+            in_dim = 256 * max(1, int(3e9 // (T * out_dim * 256)))
+        out.append(pytest.param(t, in_dim, out_dim, T, i, id=f"{TYPE_NAME[t]}-{in_dim}x{out_dim}-T{T}"))
+    return out
+
+
+MEDIUM_GRID_KERNELS = set()
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim,T,i", _medium_grids(40, 4242))
+def test_default_routing_on_medium_grids(be, t, in_dim, out_dim, T, i):
+    """One to five token tiles of 128 over 33 to 130 row tiles of 64: where, by the size of the launch, the K-quants
+    leave the small-batch kernel for the medium-batch kernel, the plane kernel with 64-row tiles, the feeding-wave
+    kernels or the plane kernel with 128-row tiles.  Every bit of the CPU GEMM's (vecdot.rs:2213-2303, 2352-2398),
+    whichever runs."""
+    from orangu_amd import QuantMatrix
+    raw = synth_weights(t, in_dim, out_dim, seed=9000 + i)
+    x = synth_x(T, in_dim, seed=9500 + i)
+    w = QuantMatrix(np.ascontiguousarray(raw), t, in_dim, out_dim)
+    print("case", TYPE_NAME[t], in_dim, out_dim, T, flush=True)
+    try:
+        got = be.matmul(x, T, w)
+        k1 = be.last_kernel()
+        MEDIUM_GRID_KERNELS.add(k1)
+        want = oracle.matmul(t, raw, in_dim, out_dim, x, T)
+        bad = np.nonzero(bits(got) != bits(want))[0]
+        assert bad.size == 0, f"matmul via {k1}: {bad.size} of {want.size} differ, first {bad[:4]}"
+        print("  via", k1, flush=True)
+    finally:
+        be.evict(w)
+
+
+def test_medium_grids_reached_every_kernel_family():
+    """The walk above is only worth its time if it lands on the kernels it is there for."""
+    if not MEDIUM_GRID_KERNELS:
+        pytest.skip("the walk did not run in this process")
+    names = " ".join(sorted(MEDIUM_GRID_KERNELS))
+    for piece in ("_dmx_kernel", "_dma_kernel", "ogm_gemm_sbw_", "_r64_kernel", "ogm_gemm_sb_"):
+        assert piece in names, (piece, names)
