@@ -217,7 +217,7 @@ DECODE_MODELS = {   # n_layer, n_embd, n_head, n_kv, head_dim, n_ff, n_vocab
 
 
 def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: bool, only_prefill: int = 0,
-               with_prefill: bool = True, only_verify: int = 0, attn_timeline: bool = False, model: str = "8b",
+               with_prefill: bool = True, only_verify: int = 0, attn_timeline: bool = False, attn_chunks_per_wg: int = 0, model: str = "8b",
                layers_run: int = 0) -> dict:
     """Batch-1 decode of an 8B-shaped Llama (32 layers: wq, wo 4096x4096, wk, wv 4096->1024, gate, up
     4096->14336 in Q4_K; down 14336->4096 and the 128256-row output in Q6_K; f16 KV cache holding `ctx`
@@ -292,10 +292,15 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
     if attn_timeline:
         # A variant of the library built with -DOGM_ATTN_STAMPS=1 (`--lib`): the wall-clock stamps of the last
         # layer's attention launch of each of `steps` decode steps, phase by phase, medians over steps.
-        n_wg = n_kv * (ctx // 128 + 1)
+        # (the launcher's rule for the chunks of 128 positions a workgroup takes in a row: ogm_launch_attn_decode)
+        n_chunks = ctx // 128 + 1
+        sub = attn_chunks_per_wg or max(-(-n_chunks * n_kv // 264), 2 if n_chunks * n_kv >= 256 else 1)
+        n_wg = n_kv * -(-n_chunks // min(sub, n_chunks))
         phases = ["start -> q rotated, new K/V row written", "scores of the chunk", "weighted V sum",
                   "partial results stored and acknowledged", "ticket drawn",
                   "merging workgroup: chunks merged", "merging workgroup: row quantized"]
+        if min(sub, n_chunks) > 1:
+            phases[1:3] = ["the workgroup's chunks, one after the other", "its waves' results joined"]
         rows = {k: [] for k in phases}
         spans = []
         for i in range(warmup + steps):
@@ -314,7 +319,8 @@ def decode_leg(be, helpers, hiprt, steps: int, warmup: int, ctx: int, check: boo
         dec.close()
         for h in mats.values():
             be.free_weight(h)
-        return {"workload": f"attention kernel of a decode step at context {ctx}: {n_wg} workgroups, 100 MHz stamps, "
+        return {"workload": f"attention kernel of a decode step at context {ctx}: {n_wg} workgroups of "
+                            f"{min(sub, n_chunks)} chunks, 100 MHz stamps, "
                             f"median over workgroups, then over {steps} steps",
                 "us": {k: round(float(np.median(v)), 2) for k, v in rows.items()},
                 "first start -> last end": round(float(np.median(spans)), 2)}
@@ -564,7 +570,9 @@ def main() -> int:
         be.close()
         return 0
     if args.attn_timeline:
-        print(json.dumps(decode_leg(be, helpers, hiprt, 16, 4, args.decode_ctx, False, attn_timeline=True)))
+        chunks_per_wg = max([int(kv.partition("=")[2]) for kv in args.tune if kv.startswith("attn_decode_chunks=")] + [0])
+        print(json.dumps(decode_leg(be, helpers, hiprt, 16, 4, args.decode_ctx, False, attn_timeline=True,
+                                    attn_chunks_per_wg=chunks_per_wg)))
         be.close()
         return 0
     if args.only_verify:

@@ -409,8 +409,8 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
 
 /* Kernel choices the host makes per shape, exposed so that a benchmark can sweep them and a test can reach
  * every kernel on small shapes.  Unknown keys and values out of range return OGM_ERR_INVALID.  Only
- * "gemm_one_pass" and "attn_prefill_variant" can change a result bit; every other setting selects among
- * kernels that produce the same bits.
+ * "gemm_one_pass", "attn_prefill_variant" and "attn_decode_chunks" can change a result bit; every other
+ * setting selects among kernels that produce the same bits.
  *   "gemv_wg_waves"            waves per workgroup of the GEMV kernel, 1..16; 0 = by the row's tile count
  *   "gemm_min_tokens"          ogm_matmul takes a matrix-core GEMM from this many tokens on; 0 = default (6 for
  *                              Q4_K, Q5_K and Q6_K, 17 for the other types); below it the multi-token GEMV
@@ -456,6 +456,11 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              default, where it measured faster (Q6_K from four tokens, Q4_K / Q5_K from five, all
  *                              up to eight; rows of up to 4096 inputs, longer ones only in launches of few rows);
  *                              2 = wherever it can (two to sixteen); 0 = never.  Same bits as the other kernels
+ *   "attn_decode_chunks"       chunks of 128 cached positions that a workgroup of the decode step's attention
+ *                              takes one after the other, 1..64; 0 = default: one up to about 4000 positions of
+ *                              eight K/V heads (fewer than 256 workgroups), then as many as keep the launch near
+ *                              264 workgroups (2 at 8192 positions, 8 at 32768).  Agrees with one chunk a
+ *                              workgroup to f32 rounding
  *   "attn_prefill_variant"     attention of a prefill batch: 1 = the decode step's kernel per token and chunk of
  *                              the cache; 2 = the matrix-core kernel; 0 = default: the first for batches of up to
  *                              48 tokens (speculative-decode verify batches), the second above; they agree to

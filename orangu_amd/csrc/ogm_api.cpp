@@ -72,6 +72,7 @@ struct ogm_ctx {
   int tune_gemm_interleave = 0;        // the 64-row plane kernel with the f32 step between the matrix instructions: 0 by the launch's size, 1 never, 2 whenever it can
   int tune_gemm_one_pass = 0;          // 1: Q4_K / Q5_K on that kernel fold the min pass into the super-block step (f32 to rounding, not to the bit)
   int tune_prefill_chunk = 2048;       // tokens per prefill pass over the layers (fixed per model at its first prefill)
+  int tune_attn_decode_chunks = 0;     // chunks of the cache a workgroup of the decode step's attention takes in a row; 0: by the context
   int tune_attn_prefill_variant = 0;   // 0: by batch size; 1: the decode kernel per token and chunk; 2: the matrix-core kernel
   // Device memory the prefill planes of all weights may take, in MiB; 0 (the default) = build none.
   // A model's planes are 3.3 times its Q4_K bytes.
@@ -340,6 +341,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
   if (strcmp(key, "gemv_mma") == 0) {
     if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemv_mma must be 0, 1 or 2");
     ctx->tune_gemv_mma = value;
+    return OGM_OK;
+  }
+  if (strcmp(key, "attn_decode_chunks") == 0) {
+    if (value < 0 || value > 64) return fail(ctx, OGM_ERR_INVALID, "attn_decode_chunks must be 0 to 64");
+    ctx->tune_attn_decode_chunks = value;
     return OGM_OK;
   }
   if (strcmp(key, "attn_prefill_variant") == 0) {
@@ -1561,7 +1567,8 @@ static int llama_decode_enqueue(ogm_ctx *ctx, ogm_llama *m, const float *x_dev, 
     const OgmAttnPre pre{L.q_bias, L.k_bias, L.v_bias, L.q_norm, L.k_norm, c.rms_eps, c.rope_neox};
     HIPCHK(ctx, ogm_launch_attn_decode(m->q, m->k, m->v, rope_cs, c.rope_dim, pre, kc, vc, pos, m->max_splits,
                                        c.n_head, c.n_head_kv, c.head_dim, scale, m->part_o, m->part_ml,
-                                       m->attn_counters, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s, 0u));
+                                       m->attn_counters, mode_o, nullptr, act_view(ctx, qd, mode_o, 0), s, 0u,
+                                       (uint32_t)ctx->tune_attn_decode_chunks));
     const int mode_ff = act_mode_for(L.w_gate->ggml_type);
     if (act_mode_for(L.w_up->ggml_type) != mode_ff)
       return fail(ctx, OGM_ERR_UNSUPPORTED, "w_gate and w_up must share an activation mode");

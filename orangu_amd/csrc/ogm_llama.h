@@ -12,6 +12,10 @@
 // of each other, and tickets that share a line queue up behind one another at the memory's atomic unit (136 of
 // them in one line: the last came back 2.9 us after its store; a line each: see the decode step's timeline).
 #define OGM_ATTN_TICKET_STRIDE 32u
+// A decode step over a long context gives a workgroup several chunks in a row, as many as keep the launch near
+// OGM_ATTN_SUB_TARGET workgroups (one to a compute unit and a few), at most OGM_ATTN_SUB_MAX.
+#define OGM_ATTN_SUB_TARGET 264u
+#define OGM_ATTN_SUB_MAX 64u
 #define OGM_ATTN_CHUNK_MIN 64u    // ... or half as many while the launch stays within one round of workgroups;
                                   // the partial-result buffers are sized for this one
 
@@ -48,11 +52,13 @@ struct OgmAttnPre {
 //   * causal attention over cache positions 0..pos (engine/attention.rs:426-549): scores =
 //     (q . k) * scale, softmax over positions, out = sum w * v; grouped-query heads share their
 //     K/V head (a count ogm_attn_head_parts accepts: up to eight in one workgroup, more in equal parts of at
-//     most eight).  Split over chunks of `chunk` positions (64 or 128; 0 = by the size of the launch) and merged;
+//     most eight).  Split over chunks of `chunk` positions (64 or 128; 0 = by the size of the launch), of which a
+//     workgroup takes `chunks_per_wg` in a row (0 = by the size of the launch: one, more on long contexts), and
+//     merged;
 //   * the merged output quantized for the next matmul in `mode`, and stored as f32 when attn_out
 //     is not null.
 // part_o: [n_head][max_splits][head_dim] f32, part_ml: [n_head][max_splits][2] f32 scratch, with
-// max_splits >= pos / chunk + 1; counters: 2 * n_head_kv * parts * OGM_ATTN_TICKET_STRIDE words (one ticket per
+// max_splits >= the number of workgroups per head, at most pos / chunk + 1; counters: 2 * n_head_kv * parts * OGM_ATTN_TICKET_STRIDE words (one ticket per
 // cache line), zero before the first launch (the kernel leaves them zero).
 // ogm_attn_head_parts: the workgroups a K/V head's query heads are dealt to (1 for up to eight heads, else the
 // fewest equal parts of at most eight), or 0 for a count the kernels do not take (none, more than 64, or one that
@@ -63,7 +69,7 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
                                   uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
                                   float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
-                                  hipStream_t stream, uint32_t chunk = 0);
+                                  hipStream_t stream, uint32_t chunk = 0, uint32_t chunks_per_wg = 0);
 
 // h = silu(gate) * up with silu(g) = g / (1 + exp(-g))     (tensor.rs:825-827, arch/mod.rs:1071-1106)
 // quantized for the down projection in `mode`; h (f32) is also stored when not null.  With

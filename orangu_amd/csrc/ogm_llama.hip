@@ -202,8 +202,8 @@ __device__ __forceinline__ AttnPart attn_merge_chunks(const float *part_o, const
 // attends to positions 0 .. pos + t).  q arrives with bias, norm and RoPE applied and every K/V
 // row is in the cache already (ogm_qkv_pre_kernel), workgroups past a token's last chunk leave at
 // once, and nothing is quantized: the next matmul is a GEMM that quantizes its own input.
-template <int HD, int G, int GROUP, bool PREFILL = false, int CHUNK = (int)OGM_ATTN_CHUNK>
-__global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
+template <int HD, int G, int GROUP, bool PREFILL = false, int CHUNK = (int)OGM_ATTN_CHUNK, bool MULTI = false>
+__global__ __launch_bounds__(4 * CHUNK, (MULTI && G <= 4) ? 4 : 1) void ogm_attn_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
                                                        const float *__restrict__ v_new,
                                                        const float2 *__restrict__ cs, uint32_t rope_half,
                                                        OgmAttnPre pre, uint32_t gq,
@@ -211,7 +211,8 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
                                                        uint32_t pos, uint32_t max_splits, uint32_t n_head_kv,
                                                        float scale, float *part_o, float *part_ml,
                                                        uint32_t *counters, float *__restrict__ attn_out,
-                                                       OgmActDev act) {
+                                                       OgmActDev act, uint32_t n_sub) {
+  static_assert(!MULTI || (!PREFILL && CHUNK == 128), "several chunks a workgroup: the decode step, chunks of 128");
   constexpr int NT = 4 * CHUNK, NW = NT / 64;   // four threads per cache position
   constexpr int KU = HD / 32;             // 16-byte pieces of a K row per thread
   constexpr int TPR = HD / 8;             // threads per V row
@@ -242,17 +243,25 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
     part_o += tok * n_head * max_splits * HD;
     part_ml += tok * n_head * max_splits * 2;
   }
-  const uint32_t n_splits = PREFILL ? pos / (uint32_t)CHUNK + 1u : gridDim.y;
+  // MULTI (a decode step over a long context): the workgroup takes n_sub chunks in a row, see below.
+  const uint32_t n_chunks = pos / (uint32_t)CHUNK + 1u;
+  const uint32_t n_splits = PREFILL ? n_chunks : gridDim.y;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t kv_dim = n_head_kv * HD;
   const uint32_t n_pos = pos + 1u;
-  const uint32_t p0 = split * (uint32_t)CHUNK;
+  const uint32_t c_first = MULTI ? split * n_sub : split;                       // the workgroup's first chunk ...
+  const uint32_t c_end = MULTI ? min(c_first + n_sub, n_chunks) : split + 1u;   // ... and the one after its last
+  const uint32_t p0 = c_first * (uint32_t)CHUNK;
   const uint32_t n_here = min((uint32_t)CHUNK, n_pos - p0);
-  const bool is_last = !PREFILL && split == n_splits - 1u;   // holds the current position, not yet cached
-  const uint32_t cur = pos - p0;                 // meaningful in the last chunk only
+  const bool is_last = !PREFILL && c_end == n_chunks;   // holds the current position, not yet cached
+  const uint32_t cur = pos - p0;                 // meaningful in the last chunk only (MULTI: see there)
 
-  const uint32_t r = tid >> 2, c = tid & 3u;              // phase 1: cache row and piece phase
   const uint32_t rr = tid / TPR, dc = tid - rr * TPR;     // phase 2: row slot and 8-dimension chunk
+  // phase 1: cache row and piece phase.  MULTI: a wave scores the sixteen rows whose V rows it sums in phase 2
+  // (64 / TPR of every ROWS), so that the weights stay within the wave
+  constexpr uint32_t R2 = 64u / (uint32_t)TPR;
+  const uint32_t c = tid & 3u;
+  const uint32_t r = MULTI ? (uint32_t)ROWS * ((lane >> 2) / R2) + R2 * wave + ((lane >> 2) % R2) : tid >> 2;
   // rows past the chunk's end read the last row; their scores are discarded (weight 0)
   const __half *krow = kc + (size_t)(p0 + min(r, n_here - 1u)) * kv_dim + kvh * HD;
   uint4 kr[KU];
@@ -345,6 +354,202 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
   __syncthreads();
 
   OGM_STAMP(1);
+  if constexpr (MULTI) {
+    // Several chunks in a row with no workgroup barrier between them: a wave keeps a running maximum per head of
+    // its own sixteen rows of every chunk, its lanes their shares of the softmax sum and of the weighted V sum, and
+    // the eight waves meet once, after the last chunk.  The next chunk's rows travel while this one is worked on,
+    // into the registers this chunk's rows leave: K once the scores' products are formed, V once the weighted
+    // sums are.  (They are requested whether or not the workgroup has a next chunk -- past its last one, the
+    // cache's last chunk: under a condition the compiler keeps twice the registers.)
+    float o[NV], l_lane[NF], m_run[NF];
+#pragma unroll
+    for (int i = 0; i < NV; i++) o[i] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NF; i++) {
+      l_lane[i] = 0.0f;
+      m_run[i] = -INFINITY;
+    }
+    uint32_t g0 = 0;        // first head this lane holds
+    bool owner = true;      // of several lanes holding the same head, the one that stores
+    for (uint32_t chunk_i = c_first; chunk_i < c_end; chunk_i++) {
+      const uint32_t p0c = chunk_i * (uint32_t)CHUNK;
+      const uint32_t n_here_c = min((uint32_t)CHUNK, n_pos - p0c);
+      const bool last_chunk = is_last && chunk_i + 1u == n_chunks;
+      const uint32_t cur_c = pos - p0c;
+      const uint32_t next = min(chunk_i + 1u, n_chunks - 1u);
+      if (chunk_i != c_first) {
+#pragma unroll
+        for (int j = 0; j < KU; j++) asm volatile("" : "+v"(kr[j].x), "+v"(kr[j].y), "+v"(kr[j].z), "+v"(kr[j].w));
+      }
+      if (last_chunk && r == cur_c) {
+#pragma unroll
+        for (int j = 0; j < KU; j++) kr[j] = *(const uint4 *)&kcur[8 * (c + 4 * j)];
+      }
+      float acc[G];
+#pragma unroll
+      for (int g = 0; g < G; g++) acc[g] = 0.0f;
+#pragma unroll
+      for (int j = 0; j < KU; j++) {
+        const __half2 *h2 = (const __half2 *)&kr[j];
+        float kf[8];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float2 f = __half22float2(h2[e]);
+          kf[2 * e] = f.x;
+          kf[2 * e + 1] = f.y;
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+          const float4 qa = *(const float4 *)&qs[g][8 * (c + 4 * j)];
+          const float4 qb = *(const float4 *)&qs[g][8 * (c + 4 * j) + 4];
+          acc[g] = fmaf(qa.x, kf[0], acc[g]); acc[g] = fmaf(qa.y, kf[1], acc[g]);
+          acc[g] = fmaf(qa.z, kf[2], acc[g]); acc[g] = fmaf(qa.w, kf[3], acc[g]);
+          acc[g] = fmaf(qb.x, kf[4], acc[g]); acc[g] = fmaf(qb.y, kf[5], acc[g]);
+          acc[g] = fmaf(qb.z, kf[6], acc[g]); acc[g] = fmaf(qb.w, kf[7], acc[g]);
+        }
+      }
+      {
+        const uint32_t nh_ = min((uint32_t)CHUNK, n_pos - next * (uint32_t)CHUNK);
+        const __half *krow_ = kc + (size_t)(next * (uint32_t)CHUNK + min(r, nh_ - 1u)) * kv_dim + kvh * HD;
+#pragma unroll
+        for (int j = 0; j < KU; j++) kr[j] = *(const uint4 *)(krow_ + 8 * (c + 4 * j));
+      }
+      // sum over the row's four lanes, as in the one-chunk path below
+      g0 = 0;
+      owner = true;
+      {
+        int n = G;
+#pragma unroll
+        for (int b = 1; b < 4; b <<= 1) {
+          const bool up = (lane & b) != 0;
+          if (n >= 2) {
+            n >>= 1;
+#pragma unroll
+            for (int i = 0; i < n; i++) {
+              float lo = acc[i], hi = acc[n + i];
+              asm volatile("" : "+v"(lo), "+v"(hi));   // keeps the selects on values, not on array slots
+              acc[i] = (up ? hi : lo) + (b == 1 ? ogm_quad_xor<1>(up ? lo : hi) : ogm_quad_xor<2>(up ? lo : hi));
+            }
+            g0 += up ? n : 0;
+          } else {
+            acc[0] += b == 1 ? ogm_quad_xor<1>(acc[0]) : ogm_quad_xor<2>(acc[0]);
+            owner = owner && !up;
+          }
+        }
+      }
+      const bool valid = r < n_here_c;
+#pragma unroll
+      for (int i = 0; i < NF; i++) {
+        const float sv = valid ? acc[i] * scale : -INFINITY;
+        // over the wave's sixteen rows of four lanes, lane by lane of the row
+        float m = ogm_row_quads_allreduce(sv, OgmOpMax());
+        m = ogm_butterfly_step<16>(m, OgmOpMax());
+        m = ogm_butterfly_step<32>(m, OgmOpMax());
+        const float m_new = fmaxf(m_run[i], m);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;   // (a wave may have seen no row yet: everything stays zero)
+        const float a = expf(m_run[i] - m_use);
+        const float e = valid ? expf(sv - m_use) : 0.0f;
+        l_lane[i] = l_lane[i] * a + e;
+        m_run[i] = m_new;
+        if (owner) sc[g0 + i][r] = e;
+        if (lane < 4u && owner) red[1][g0 + i][wave] = a;
+      }
+      __builtin_amdgcn_wave_barrier();   // the wave's LDS accesses run in order: its weights and factors are there
+      {
+        float al[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) al[g] = red[1][g][wave];
+#pragma unroll
+        for (int i = 0; i < NV; i++) o[i] *= al[i >> 3];
+      }
+      if (chunk_i != c_first) {
+#pragma unroll
+        for (int st = 0; st < STEPS; st++) asm volatile("" : "+v"(vr[st].x), "+v"(vr[st].y), "+v"(vr[st].z), "+v"(vr[st].w));
+      }
+#pragma unroll
+      for (int st = 0; st < STEPS; st++) {
+        const uint32_t p = st * ROWS + rr;   // past the chunk's end the weight sc is 0
+        if (last_chunk && p >= cur_c) vr[st] = *(const uint4 *)&vcur[8u * dc];   // the cache row is not written yet
+        const __half2 *h2 = (const __half2 *)&vr[st];
+        float vf[8];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const float2 f = __half22float2(h2[j]);
+          vf[2 * j] = f.x;
+          vf[2 * j + 1] = f.y;
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+          const float w = sc[g][p];
+#pragma unroll
+          for (int j = 0; j < 8; j++) o[g * 8 + j] = fmaf(w, vf[j], o[g * 8 + j]);
+        }
+      }
+      {
+        const uint32_t nh_ = min((uint32_t)CHUNK, n_pos - next * (uint32_t)CHUNK);
+        const __half *vbase_ = vc + (size_t)next * (uint32_t)CHUNK * kv_dim + kvh * HD + 8u * dc;
+#pragma unroll
+        for (int st = 0; st < STEPS; st++)
+          vr[st] = *(const uint4 *)(vbase_ + (size_t)min((uint32_t)(st * ROWS) + rr, nh_ - 1u) * kv_dim);
+      }
+      __builtin_amdgcn_wave_barrier();   // before the next chunk's weights replace these
+    }
+    OGM_STAMP(2);
+    // ---- the waves meet: each one's maximum and sum per head, and its weighted V sums
+#pragma unroll
+    for (int i = 0; i < NF; i++) {
+      float l = ogm_row_quads_allreduce(l_lane[i], OgmOpAdd());
+      l = ogm_butterfly_step<16>(l, OgmOpAdd());
+      l = ogm_butterfly_step<32>(l, OgmOpAdd());
+      if (lane < 4u && owner) {
+        red[0][g0 + i][wave] = m_run[i];
+        red[1][g0 + i][wave] = l;
+      }
+    }
+    {
+      uint32_t sel = 0;
+      int n = NV;
+#pragma unroll
+      for (int b = TPR; b < 64; b <<= 1) {
+        const bool up = (lane & b) != 0;
+        n >>= 1;
+#pragma unroll
+        for (int i = 0; i < n; i++) {
+          float lo = o[i], hi = o[n + i];
+          asm volatile("" : "+v"(lo), "+v"(hi));   // keeps the selects on values, not on array slots
+          const float send = up ? lo : hi;
+          o[i] = (up ? hi : lo) + (b == 16 ? ogm_half_xor<16>(send, up) : b == 32 ? ogm_half_xor<32>(send, up)
+                                                                                   : __shfl_xor(send, b, 64));
+        }
+        sel += up ? n : 0;
+      }
+      float *dst = &osum[wave][0][0] + (sel >> 3) * HD + (sel & 7u) + 8u * dc;
+#pragma unroll
+      for (int i = 0; i < n; i++) dst[(i >> 3) * HD + (i & 7)] = o[i];
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < (uint32_t)(G * HD); i += NT) {
+      const uint32_t g = i / HD, d = i - g * HD;
+      float M = red[0][g][0];
+#pragma unroll
+      for (int w = 1; w < NW; w++) M = fmaxf(M, red[0][g][w]);
+      float t = 0.0f, l = 0.0f;
+#pragma unroll
+      for (int w = 0; w < NW; w++) {
+        const float f = expf(red[0][g][w] - M);   // a wave that saw no row: exp(-inf) = 0
+        t += osum[w][g][d] * f;
+        l += red[1][g][w] * f;
+      }
+      if (g < gq) {
+        const uint32_t h = hg * gq + g;
+        st_one<GROUP != 0>(&part_o[((size_t)h * max_splits + split) * HD + d], t);
+        if (d == 0u) {
+          st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2], M);
+          st_one<GROUP != 0>(&part_ml[((size_t)h * max_splits + split) * 2 + 1], l);
+        }
+      }
+    }
+  } else {
   // ---- phase 1: scores
   if (is_last && r == cur) {
 #pragma unroll
@@ -493,6 +698,7 @@ __global__ __launch_bounds__(4 * CHUNK) void ogm_attn_kernel(const float *__rest
       if (g < gq) st_one<GROUP != 0>(&part_o[((size_t)(hg * gq + g) * max_splits + split) * HD + d], t);
     }
   }
+  }   // one chunk
 
   OGM_STAMP(3);
   // ---- the last workgroup of this K/V head merges the chunks and quantizes
@@ -587,7 +793,7 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
                                   void *v_cache_layer, uint32_t pos, uint32_t max_splits, uint32_t n_head,
                                   uint32_t n_head_kv, uint32_t head_dim, float scale, float *part_o,
                                   float *part_ml, uint32_t *counters, int mode, float *attn_out, OgmActDev act,
-                                  hipStream_t stream, uint32_t chunk) {
+                                  hipStream_t stream, uint32_t chunk, uint32_t chunks_per_wg) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0) return hipErrorInvalidValue;
   if (rope_dim > head_dim || rope_dim % 2u != 0) return hipErrorInvalidValue;
   // Cache positions per workgroup: 128; 64 only for short contexts.  The kernel is a chain of
@@ -596,31 +802,50 @@ hipError_t ogm_launch_attn_decode(const float *q, const float *k_new, const floa
   // chunk, while the merge grows with the number of chunks: measured on MI355X with eight K/V heads,
   // 64 against 128 positions per workgroup take 8.4 against 8.9 us at 512 cached positions but 13.6
   // against 10.7 at 2048 and 20.5 against 14.1 at 4096.
-  if (chunk == 0) chunk = (pos / 64u + 1u) * n_head_kv <= 96u ? 64u : 128u;
+  if (chunk == 0) chunk = (chunks_per_wg <= 1u && (pos / 64u + 1u) * n_head_kv <= 96u) ? 64u : 128u;
   if (chunk != 64u && chunk != 128u) return hipErrorInvalidValue;
-  const uint32_t n_splits = pos / chunk + 1u;
-  if (n_splits > max_splits) return hipErrorInvalidValue;
+  const uint32_t n_chunks = pos / chunk + 1u;
   const uint32_t n = n_head * head_dim;
   if (n % 32u != 0) return hipErrorInvalidValue;
   // more than eight query heads per K/V head: in equal parts of at most eight, a workgroup each
   const uint32_t parts = ogm_attn_head_parts(n_head / n_head_kv);
   if (parts == 0u) return hipErrorInvalidValue;
   const uint32_t gq = n_head / n_head_kv / parts;
+  // Chunks a workgroup takes in a row (chunks of 128 only): one while the launch has fewer workgroups than the
+  // device has compute units, then as many as keep it near OGM_ATTN_SUB_TARGET workgroups, at most
+  // OGM_ATTN_SUB_MAX.  A workgroup pays for the rotation of q, the hand-over of its partial results and its
+  // ticket once, its waves work through their chunks without meeting, and the merge at the end has that many
+  // fewer partial results to read.  Measured on MI355X, 8B shapes (eight K/V heads), ms per token at 1 / 2 / 4 / 8 /
+  // 16 chunks a workgroup: 2048 positions 1.80 / 1.86 / 1.97 / 2.18 / 2.60; 4096: 1.95 / 1.90 / 2.00 / 2.21 / 2.63;
+  // 8192: 2.08 / 1.99 / 2.01 / 2.20 / 2.63; 16384: 2.38 / 2.34 / 2.19 / 2.27 / 2.65; 32768: 3.02 / 2.87 / 2.66 /
+  // 2.60 / 2.84.
+  uint32_t n_sub = chunks_per_wg;
+  if (n_sub == 0u) {
+    const uint32_t wgs = n_chunks * n_head_kv * parts;
+    n_sub = (wgs + OGM_ATTN_SUB_TARGET - 1u) / OGM_ATTN_SUB_TARGET;
+    if (wgs >= 256u && n_sub < 2u) n_sub = 2u;
+    if (n_sub > OGM_ATTN_SUB_MAX) n_sub = OGM_ATTN_SUB_MAX;
+  }
+  if (n_sub == 0u || chunk != 128u) n_sub = 1u;   // (chunks of 64 are for contexts of a few hundred positions)
+  if (n_sub > n_chunks) n_sub = n_chunks;
+  const uint32_t n_splits = (n_chunks + n_sub - 1u) / n_sub;
+  if (n_splits > max_splits) return hipErrorInvalidValue;
   const dim3 grid(n_head_kv * parts, n_splits);
   const uint32_t G = gq <= 2u ? gq : (gq <= 4u ? 4u : 8u);   // head slots of the kernel
   const uint32_t group = mode == 0 ? 32u : 256u;
   // the merge rides in the attention kernel when every head slot is a head and a K/V head's
   // outputs are whole quantizer groups
   const uint32_t fused = (G == gq && (G * head_dim) % group == 0) ? group : 0u;
-#define OGM_ATTN_LAUNCH_C(HD_, G_, GR_, CH_)                                                           \
-  hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, GR_, false, CH_>), grid, dim3(4 * CH_), 0, stream, q, k_new, \
+#define OGM_ATTN_LAUNCH_C(HD_, G_, GR_, CH_, MULTI_)                                                    \
+  hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, GR_, false, CH_, MULTI_>), grid, dim3(4 * CH_), 0, stream, q, k_new, \
                      v_new, (const float2 *)cs, rope_dim / 2u, pre, gq, (__half *)k_cache_layer,        \
                      (__half *)v_cache_layer, pos, max_splits, n_head_kv, scale, part_o, part_ml, \
-                     counters, attn_out, act)
+                     counters, attn_out, act, n_sub)
 #define OGM_ATTN_LAUNCH(HD_, G_, GR_)                    \
   do {                                                   \
-    if (chunk == 64u) OGM_ATTN_LAUNCH_C(HD_, G_, GR_, 64); \
-    else OGM_ATTN_LAUNCH_C(HD_, G_, GR_, 128);           \
+    if (chunk == 64u) OGM_ATTN_LAUNCH_C(HD_, G_, GR_, 64, false); \
+    else if (n_sub == 1u) OGM_ATTN_LAUNCH_C(HD_, G_, GR_, 128, false); \
+    else OGM_ATTN_LAUNCH_C(HD_, G_, GR_, 128, true);     \
   } while (0)
 #define OGM_ATTN_GROUPS(HD_, G_)                                \
   do {                                                          \
@@ -1061,7 +1286,7 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
   hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, 0, true>), grid, dim3(512), 0, stream, q, (const float *)nullptr, \
                      (const float *)nullptr, (const float2 *)nullptr, 0u, none, gq, (__half *)k_cache_layer,  \
                      (__half *)v_cache_layer, pos0, max_splits, n_head_kv, scale, part_o, part_ml,            \
-                     (uint32_t *)nullptr, (float *)nullptr, no_act)
+                     (uint32_t *)nullptr, (float *)nullptr, no_act, 1u)
   if (head_dim == 128 && G == 1) OGM_ATTN_PREFILL(128, 1);
   else if (head_dim == 128 && G == 2) OGM_ATTN_PREFILL(128, 2);
   else if (head_dim == 128 && G == 4) OGM_ATTN_PREFILL(128, 4);

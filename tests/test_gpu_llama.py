@@ -241,6 +241,31 @@ def test_decode_at_contexts_whose_chunks_merge_in_several_rounds(be, hd, group, 
         dev.close()
 
 
+@pytest.mark.parametrize("hd,group,n_kv,n_pre,chunks", [
+    (128, 4, 1, 4500, 3), (128, 8, 1, 2200, 2), (64, 4, 2, 8300, 5), (128, 1, 2, 16500, 16), (128, 4, 2, 300, 2),
+    (64, 8, 1, 700, 4), (128, 2, 1, 130, 64), (128, 1, 8, 8300, 0)])
+def test_decode_with_several_chunks_per_workgroup(be, hd, group, n_kv, n_pre, chunks):
+    """On long contexts a workgroup of the decode step's attention takes several chunks of the cache in a row and
+    keeps a running maximum, sum and weighted V sum (by default as many as keep the launch near 512 workgroups:
+    two at 8300 positions of eight K/V heads, the last case; forced here otherwise: 2 to 16 chunks, more than the
+    context has, chunks of 64 positions, two outputs per thread at eight query heads).  Same allowances as with a
+    chunk per workgroup."""
+    n_head = group * n_kv
+    n_embd = 256
+    ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=320, n_layer=1,
+                          types=(Q4_K, Q6_K, Q6_K, Q6_K), max_ctx=n_pre + 4, seed=19, base=500000.0,
+                          attn_norm_scale=TAME[Q4_K])
+    be.set_tuning("attn_decode_chunks", chunks)
+    try:
+        fill_cache_both(ref, dev, rng, 1, n_pre, n_kv * hd)
+        for pos in (n_pre, n_pre + 1):
+            step_both(ref, dev, rng.standard_normal(n_embd).astype(f32), pos, f"context {pos}, {chunks} chunks a workgroup",
+                      attn_rtol=1e-5 * max(n_pre, 250) / 250)
+    finally:
+        be.set_tuning("attn_decode_chunks", 0)
+        dev.close()
+
+
 @contextmanager
 def llama_8b_prefix(be, ctx, dims=(4096, 32, 8, 128, 14336, 128256), n_layer=2):
     """A two-layer prefix of the 8B-shaped Q4_K_M-like model (hidden 4096, 32 query heads over 8 K/V heads
