@@ -1936,7 +1936,8 @@ static int llama_prefill_chunk(ogm_ctx *ctx, ogm_llama *m, uint32_t pos0, uint32
       HIPCHK(ctx, ogm_launch_attn_prefill(P.q + (size_t)t0 * qd, kc, vc, pos0 + t0, nt, m->max_splits, c.n_head,
                                           c.n_head_kv, c.head_dim, scale, P.part_o, P.part_ml,
                                           fused_q ? nullptr : P.attn + (size_t)t0 * qd, s, fused_q ? mode_o : -1,
-                                          fused_q ? act_view(ctx, qd, mode_o, t0) : OgmActDev{}));
+                                          fused_q ? act_view(ctx, qd, mode_o, t0) : OgmActDev{},
+                                          (uint32_t)ctx->tune_attn_decode_chunks));
     }
     const ogm_weight *w1[1] = {L.wo};
     float *y1[1] = {P.proj};

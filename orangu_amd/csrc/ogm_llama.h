@@ -15,6 +15,7 @@
 // A decode step over a long context gives a workgroup several chunks in a row, as many as keep the launch near
 // OGM_ATTN_SUB_TARGET workgroups (one to a compute unit and a few), at most OGM_ATTN_SUB_MAX.
 #define OGM_ATTN_SUB_TARGET 264u
+#define OGM_ATTN_SUB_TARGET_ROWS 528u   // for a batch of tokens (two workgroups to a compute unit)
 #define OGM_ATTN_SUB_MAX 64u
 #define OGM_ATTN_CHUNK_MIN 64u    // ... or half as many while the launch stays within one round of workgroups;
                                   // the partial-result buffers are sized for this one
@@ -108,11 +109,12 @@ hipError_t ogm_launch_qkv_pre(float *q, const float *k, const float *v, const vo
 // 0 .. pos0 + t for token t; attn_out [n_tokens][n_head*head_dim].
 // part_o: [n_tokens][n_head][max_splits][head_dim], part_ml: [n_tokens][n_head][max_splits][2].
 // quant_mode >= 0 (0: per 32, 1: per 256): the merge also quantizes every token's row into row t of `act` for the
-// next matmul, and attn_out may be null.
+// next matmul, and attn_out may be null.  chunks_per_wg: as for ogm_launch_attn_decode (0 = by the size of the launch).
 hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_cache_layer, uint32_t pos0,
                                    uint32_t n_tokens, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
                                    uint32_t head_dim, float scale, float *part_o, float *part_ml, float *attn_out,
-                                   hipStream_t stream, int quant_mode = -1, OgmActDev act = OgmActDev{});
+                                   hipStream_t stream, int quant_mode = -1, OgmActDev act = OgmActDev{},
+                                   uint32_t chunks_per_wg = 0);
 
 // The same on the matrix cores, one launch and no partial results: query tiles of 32 tokens, cache
 // tiles of 64 positions, running softmax.  head_dim 64 or 128, at most 8 query heads per K/V head.

@@ -198,7 +198,7 @@ __device__ __forceinline__ AttnPart attn_merge_chunks(const float *part_o, const
 //     last ticket of its K/V head merges the chunks and quantizes the G * HD outputs; no other
 //     workgroup waits for anything.
 //
-// PREFILL: the same over a batch of query tokens (blockIdx.z; token t sits at position pos + t and
+// PREFILL: the same over a batch of query tokens (blockIdx.y; token t sits at position pos + t and
 // attends to positions 0 .. pos + t).  q arrives with bias, norm and RoPE applied and every K/V
 // row is in the cache already (ogm_qkv_pre_kernel), workgroups past a token's last chunk leave at
 // once, and nothing is quantized: the next matmul is a GEMM that quantizes its own input.
@@ -212,7 +212,7 @@ __global__ __launch_bounds__(4 * CHUNK, (MULTI && G <= 4) ? 4 : 1) void ogm_attn
                                                        float scale, float *part_o, float *part_ml,
                                                        uint32_t *counters, float *__restrict__ attn_out,
                                                        OgmActDev act, uint32_t n_sub) {
-  static_assert(!MULTI || (!PREFILL && CHUNK == 128), "several chunks a workgroup: the decode step, chunks of 128");
+  static_assert(!MULTI || CHUNK == 128, "several chunks a workgroup: chunks of 128");
   constexpr int NT = 4 * CHUNK, NW = NT / 64;   // four threads per cache position
   constexpr int KU = HD / 32;             // 16-byte pieces of a K row per thread
   constexpr int TPR = HD / 8;             // threads per V row
@@ -233,11 +233,14 @@ __global__ __launch_bounds__(4 * CHUNK, (MULTI && G <= 4) ? 4 : 1) void ogm_attn
   // blockIdx.x: a K/V head and gq of the query heads (G head slots) that share it -- all of them, or one of
   // gridDim.x / n_head_kv equal parts of them when the model has more than eight per K/V head (the parts' workgroups
   // read the same cache rows; in the last chunk each writes the new rows, the same bytes)
-  const uint32_t hg = blockIdx.x, split = blockIdx.y, kvh = hg / (gridDim.x / n_head_kv);
+  // (a batch: the tokens on y and the chunks on z, so that the workgroups that read the same cache rows, one per
+  // token, start one after the other -- on the same XCD when the launch has eight workgroups on x -- and all but
+  // the first find the rows in its L2)
+  const uint32_t hg = blockIdx.x, split = PREFILL ? blockIdx.z : blockIdx.y, kvh = hg / (gridDim.x / n_head_kv);
   if constexpr (PREFILL) {
-    const uint32_t tok = blockIdx.z;
+    const uint32_t tok = blockIdx.y;
     pos += tok;
-    if (split > pos / (uint32_t)CHUNK) return;   // the whole workgroup: this token has no such chunk
+    if (split * (MULTI ? n_sub : 1u) > pos / (uint32_t)CHUNK) return;   // the whole workgroup: this token has no such chunk
     const size_t n_head = (size_t)gridDim.x * gq;
     q += tok * n_head * HD;
     part_o += tok * n_head * max_splits * HD;
@@ -245,7 +248,7 @@ __global__ __launch_bounds__(4 * CHUNK, (MULTI && G <= 4) ? 4 : 1) void ogm_attn
   }
   // MULTI (a decode step over a long context): the workgroup takes n_sub chunks in a row, see below.
   const uint32_t n_chunks = pos / (uint32_t)CHUNK + 1u;
-  const uint32_t n_splits = PREFILL ? n_chunks : gridDim.y;
+  const uint32_t n_splits = PREFILL ? (MULTI ? (n_chunks + n_sub - 1u) / n_sub : n_chunks) : gridDim.y;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t kv_dim = n_head_kv * HD;
   const uint32_t n_pos = pos + 1u;
@@ -1239,13 +1242,14 @@ template <int GROUP>
 __global__ __launch_bounds__(64) void ogm_attn_combine_rows_kernel(const float *__restrict__ part_o,
                                                                    const float *__restrict__ part_ml, uint32_t pos0,
                                                                    uint32_t max_splits, uint32_t n, uint32_t head_dim,
-                                                                   float *__restrict__ attn_out, OgmActDev act) {
+                                                                   float *__restrict__ attn_out, OgmActDev act,
+                                                                   uint32_t n_sub) {
   const uint32_t lane = threadIdx.x, tok = blockIdx.y;
   const uint32_t e0 = blockIdx.x * 256u + 4u * lane;
   const bool active = e0 < n;
   if (GROUP == 0 && !active) return;
   const uint32_t n_head = n / head_dim;
-  const uint32_t n_splits = (pos0 + tok) / OGM_ATTN_CHUNK + 1u;
+  const uint32_t n_splits = ((pos0 + tok) / OGM_ATTN_CHUNK + n_sub) / n_sub;   // workgroups of n_sub chunks each
   float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
   if (active) {
     const AttnPart pt = attn_merge_chunks<false>(part_o + (size_t)tok * n_head * max_splits * head_dim,
@@ -1267,7 +1271,7 @@ __global__ __launch_bounds__(64) void ogm_attn_combine_rows_kernel(const float *
 hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_cache_layer, uint32_t pos0,
                                    uint32_t n_tokens, uint32_t max_splits, uint32_t n_head, uint32_t n_head_kv,
                                    uint32_t head_dim, float scale, float *part_o, float *part_ml, float *attn_out,
-                                   hipStream_t stream, int quant_mode, OgmActDev act) {
+                                   hipStream_t stream, int quant_mode, OgmActDev act, uint32_t chunks_per_wg) {
   if (n_head_kv == 0 || n_head % n_head_kv != 0 || n_tokens == 0 || n_tokens > 65535u) return hipErrorInvalidValue;
   if (quant_mode >= 0 && (n_head * head_dim) % (quant_mode == 0 ? 32u : 256u) != 0) return hipErrorInvalidValue;
   if (quant_mode < 0 && attn_out == nullptr) return hipErrorInvalidValue;
@@ -1279,14 +1283,31 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
   if (parts == 0u) return hipErrorInvalidValue;
   const uint32_t gq = n_head / n_head_kv / parts;
   const uint32_t G = gq <= 2u ? gq : (gq <= 4u ? 4u : 8u);
-  const dim3 grid(n_head_kv * parts, n_splits, n_tokens);
+  // Chunks a workgroup takes in a row, as in the decode step (ogm_launch_attn_decode), here to keep the launch near
+  // OGM_ATTN_SUB_TARGET_ROWS workgroups: the time of such a batch over a long context is its workgroups' own, not the
+  // memory's (the tokens' workgroups of a chunk find its rows in L2).
+  uint32_t n_sub = chunks_per_wg;
+  if (n_sub == 0u) {
+    const uint64_t wgs = (uint64_t)n_splits * n_head_kv * parts * n_tokens;
+    n_sub = (uint32_t)((wgs + OGM_ATTN_SUB_TARGET_ROWS - 1u) / OGM_ATTN_SUB_TARGET_ROWS);
+    if (n_sub > OGM_ATTN_SUB_MAX) n_sub = OGM_ATTN_SUB_MAX;
+  }
+  if (n_sub > n_splits) n_sub = n_splits;
+  const uint32_t n_wg_z = (n_splits + n_sub - 1u) / n_sub;
+  if (n_wg_z > 65535u) return hipErrorInvalidValue;
+  const dim3 grid(n_head_kv * parts, n_tokens, n_wg_z);
   const OgmAttnPre none{nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f, 0u};
   const OgmActDev no_act{};
-#define OGM_ATTN_PREFILL(HD_, G_)                                                                           \
-  hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, 0, true>), grid, dim3(512), 0, stream, q, (const float *)nullptr, \
-                     (const float *)nullptr, (const float2 *)nullptr, 0u, none, gq, (__half *)k_cache_layer,  \
-                     (__half *)v_cache_layer, pos0, max_splits, n_head_kv, scale, part_o, part_ml,            \
-                     (uint32_t *)nullptr, (float *)nullptr, no_act, 1u)
+#define OGM_ATTN_PREFILL_M(HD_, G_, MULTI_)                                                                 \
+  hipLaunchKernelGGL((ogm_attn_kernel<HD_, G_, 0, true, 128, MULTI_>), grid, dim3(512), 0, stream, q,       \
+                     (const float *)nullptr, (const float *)nullptr, (const float2 *)nullptr, 0u, none, gq, \
+                     (__half *)k_cache_layer, (__half *)v_cache_layer, pos0, max_splits, n_head_kv, scale,  \
+                     part_o, part_ml, (uint32_t *)nullptr, (float *)nullptr, no_act, n_sub)
+#define OGM_ATTN_PREFILL(HD_, G_)                  \
+  do {                                             \
+    if (n_sub == 1u) OGM_ATTN_PREFILL_M(HD_, G_, false); \
+    else OGM_ATTN_PREFILL_M(HD_, G_, true);        \
+  } while (0)
   if (head_dim == 128 && G == 1) OGM_ATTN_PREFILL(128, 1);
   else if (head_dim == 128 && G == 2) OGM_ATTN_PREFILL(128, 2);
   else if (head_dim == 128 && G == 4) OGM_ATTN_PREFILL(128, 4);
@@ -1297,18 +1318,19 @@ hipError_t ogm_launch_attn_prefill(const float *q, void *k_cache_layer, void *v_
   else if (head_dim == 64 && G == 8) OGM_ATTN_PREFILL(64, 8);
   else return hipErrorInvalidValue;
 #undef OGM_ATTN_PREFILL
+#undef OGM_ATTN_PREFILL_M
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   const dim3 cgrid((n + 255u) / 256u, n_tokens);
   if (quant_mode < 0)
     hipLaunchKernelGGL(ogm_attn_combine_rows_kernel<0>, cgrid, dim3(64), 0, stream, part_o, part_ml, pos0, max_splits, n,
-                       head_dim, attn_out, no_act);
+                       head_dim, attn_out, no_act, n_sub);
   else if (quant_mode == 0)
     hipLaunchKernelGGL(ogm_attn_combine_rows_kernel<32>, cgrid, dim3(64), 0, stream, part_o, part_ml, pos0, max_splits, n,
-                       head_dim, attn_out, act);
+                       head_dim, attn_out, act, n_sub);
   else
     hipLaunchKernelGGL(ogm_attn_combine_rows_kernel<256>, cgrid, dim3(64), 0, stream, part_o, part_ml, pos0, max_splits,
-                       n, head_dim, attn_out, act);
+                       n, head_dim, attn_out, act, n_sub);
   return hipGetLastError();
 }
 

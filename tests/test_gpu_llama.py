@@ -865,6 +865,38 @@ def test_prefill_attention_kernels_agree(be, hd, group, n_kv, n_tokens, pos0):
         assert err <= 2e-5, f"{name}: the two attention kernels differ by {err:.3e}"
 
 
+@pytest.mark.parametrize("hd,group,n_kv,n_tokens,pos0,chunks", [(128, 4, 2, 5, 700, 2), (64, 8, 1, 9, 1300, 3),
+                                                                (128, 2, 2, 4, 517, 64), (128, 1, 8, 6, 1990, 0)])
+def test_batch_attention_with_several_chunks_per_workgroup(be, hd, group, n_kv, n_tokens, pos0, chunks):
+    """A small batch over a longer cache (a verify batch): the per-token kernel whose workgroups take several chunks
+    of the cache in a row (forced: 2, 3, more than there are; the last case by the launch's own rule, 6 tokens x 16
+    chunks x 8 heads) against the matrix-core kernel, as above.  Tokens of a batch that end in different chunks have
+    different numbers of partial results."""
+    n_head = group * n_kv
+    n_embd = n_head * hd
+    wtype = Q4_K if n_embd % 256 == 0 else Q8_0
+    outs = []
+    for variant in (2, 1):
+        ref, dev, rng = build(be, n_embd=n_embd, n_head=n_head, n_kv=n_kv, hd=hd, n_ff=512, n_vocab=256, n_layer=1,
+                              types=(wtype, wtype, wtype, wtype), max_ctx=pos0 + n_tokens, seed=15,
+                              attn_norm_scale=TAME.get(wtype, 1.0))
+        be.set_tuning("attn_prefill_variant", variant)
+        be.set_tuning("attn_decode_chunks", chunks)
+        try:
+            dev.prefill(rng.standard_normal((pos0, n_embd)).astype(f32), 0)
+            be.set_tuning("attn_prefill_variant", variant)
+            logits, _ = dev.prefill(rng.standard_normal((n_tokens, n_embd)).astype(f32), pos0)
+            outs.append((np.asarray(logits, np.float64), np.asarray(dev.hidden(), np.float64)))
+        finally:
+            be.set_tuning("attn_prefill_variant", 0)
+            be.set_tuning("attn_decode_chunks", 0)
+            dev.close()
+    for name, a, b in (("logits", outs[0][0], outs[1][0]), ("hidden state", outs[0][1], outs[1][1])):
+        err = np.abs(a - b).max() / np.abs(b).max()
+        say(f"batch attention, {chunks} chunks a workgroup, hd {hd} group {group} {n_tokens} tokens from {pos0}: {name} differ by {err:.2e}")
+        assert err <= 2e-5, f"{name}: the two attention kernels differ by {err:.3e}"
+
+
 @pytest.mark.parametrize("hd", [128, 64])
 def test_prefill_attention_with_queries_beyond_f16(be, hd):
     """Per-head norms that leave q at magnitudes up to 1.5e5 (an f16 holds 65504) and k around 1e-3:
