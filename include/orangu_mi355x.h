@@ -459,7 +459,8 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *   "attn_decode_chunks"       chunks of 128 cached positions that a workgroup of the decode step's attention
  *                              takes one after the other, 1..64; 0 = default: one up to about 4000 positions of
  *                              eight K/V heads (fewer than 256 workgroups), then as many as keep the launch near
- *                              264 workgroups (2 at 8192 positions, 8 at 32768).  Agrees with one chunk a
+ *                              264 workgroups (2 at 8192 positions, 8 at 32768); the per-token kernel of a
+ *                              small prefill batch likewise, near 528 workgroups.  Agrees with one chunk a
  *                              workgroup to f32 rounding
  *   "attn_prefill_variant"     attention of a prefill batch: 1 = the decode step's kernel per token and chunk of
  *                              the cache; 2 = the matrix-core kernel; 0 = default: the first for batches of up to
