@@ -413,10 +413,14 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  * setting selects among kernels that produce the same bits.
  *   "gemv_wg_waves"            waves per workgroup of the GEMV kernel, 1..16; 0 = by the row's tile count
  *   "gemm_min_tokens"          ogm_matmul takes a matrix-core GEMM from this many tokens on; 0 = default (6 for
- *                              Q4_K, Q5_K and Q6_K, 17 for the other types); below it the multi-token GEMV
- *                              kernel runs in the GEMM's float order
- *   "gemm_small_max_tokens"    K-quant GEMMs of at most this many tokens take the small-batch kernel, whose
- *                              waves work on different super-blocks of the same rows; 0 = default (64, more
+ *                              Q4_K, Q5_K and Q6_K; 9 for Q8_0, Q5_0, Q4_0 and IQ4_NL where their small-batch
+ *                              kernel would run, or as soon as the GEMV kernel would need three passes over
+ *                              the weights; 17 otherwise); below it the multi-token GEMV kernel runs in the
+ *                              GEMM's float order
+ *   "gemm_small_max_tokens"    GEMMs of at most this many tokens take the small-batch kernel of their type, whose
+ *                              waves work on different super-blocks (blocks, for the per-32 types: by default
+ *                              while the launch has at most 1792 workgroups of 32 rows x 32 tokens, 1100 on
+ *                              rows beyond 4096 inputs) of the same rows; 0 = default (K-quants: 64, more
  *                              for matrices of few rows, up to 512 for Q4_K / Q5_K matrices of at most 2048; Q6_K
  *                              launches that "gemm_interleave" sends to its kernel by their size go there
  *                              first), 1 = never

@@ -583,8 +583,14 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   // n_tokens == 1 and every matmul_decode take the GEMV's.
   const int gemm_order = (!decode && n_tokens > 1) ? 1 : 0;
   const uint32_t t0 = w0->ggml_type;
+  // (the per-32 types: from nine tokens, more than a pass of the GEMV kernel holds, where their small-batch GEMM
+  // would run -- Q8_0 2048 -> 2048 at 12 tokens 11 us against the GEMV kernel's 14, at 8 tokens 11 against 9 -- and
+  // from seventeen otherwise)
+  bool flat_small = block_elems_of(t0) == 32 && ctx->tune_gemm_small_max != 1;
+  for (size_t i = 0; flat_small && i < n_tg; i++)
+    flat_small = ogm_gemm_flat_small_batch(tg[i].w->in_dim, tg[i].w->out_dim, n_tokens);
   const uint32_t gemm_from = ctx->tune_gemm_min_tokens ? (uint32_t)ctx->tune_gemm_min_tokens
-                             : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 6u : 17u;
+                             : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 6u : (flat_small ? 9u : 17u);
   // A few tokens over a Q6_K matrix of many rows (the vocabulary projection of a decode batch): one
   // streaming pass on the matrix cores, in either float order.
   if (n_tokens > 1 && !dump_isum && !dump_imin && !act_base && ctx->tune_gemm_ft_min_rows >= 0) {
@@ -661,10 +667,15 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   }
   // (also below that count when the GEMV kernel's LDS holds fewer tokens of such long rows than the batch has and
   // it would read the weights once per part: Q6_K 53248 -> 16384 at 4 tokens 450 us against 180, Q4_K 16384 -> 16384
-  // 65 against 52)
+  // 65 against 52; Q8_0 4096 -> 4096 at 8 / 16 tokens 21 / 31 against 17 / 18, 14336 -> 4096 at 4 / 16 tokens 85 / 330
+  // against 53 / 55 -- the per-32 types where their small-batch GEMM would run)
   const uint32_t gemv_chunk = ogm_gemv_max_tokens(w0->ggml_type, w0->in_dim, gemm_order);
-  const bool gemv_rereads = gemv_chunk != 0 && n_tokens > gemv_chunk && ctx->tune_gemm_min_tokens == 0 &&
-                            block_elems_of(w0->ggml_type) == 256;   // (the 32-wide types' GEMM pays from 17 tokens only)
+  // (the per-32 types from three parts on, or two of rows of up to 8192 inputs: 14336 -> 4096 at 2 tokens, two parts,
+  // 45 us against 53)
+  const uint32_t gemv_parts = gemv_chunk ? (n_tokens + gemv_chunk - 1u) / gemv_chunk : 0u;
+  const bool gemv_rereads = gemv_parts > 1u && ctx->tune_gemm_min_tokens == 0 &&
+                            (block_elems_of(w0->ggml_type) == 256 ||
+                             (flat_small && (gemv_parts > 2u || w0->in_dim <= 8192u)));
   if (gemm_order && !dump_isum && !dump_imin && !act_base && (n_tokens >= gemm_from || gemv_rereads) &&
       all_gemm_supported(tg, n_tg, n_tokens)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)

@@ -2317,12 +2317,144 @@ __global__ __launch_bounds__(768) void ogm_gemm_flat_kernel(GemmFlatParams p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Small batches of the per-32 types: the workgroup above walks a row's blocks one stage after the other, 70 us for
+// 4096 inputs however few the tokens.  Here, as in the K-quants' small-batch kernel, a workgroup owns 32 rows x 32
+// tokens and its eight waves take different blocks at the same time -- a block is one v_mfma_i32_32x32x32_i8, the
+// int8 weights unpacked straight into the operand registers, the activations read from memory as they are -- and
+// leave the blocks' terms (ad * dw) * dot32 (vecdot.rs:2622) in LDS; after every round of sixteen blocks the terms
+// are added in ascending order, one accumulator per output, as dot_flat_pair does (vecdot.rs:2598-2629).
+#define SBF_NB 2u   // blocks a wave takes per round
+
+template <int KIND, uint32_t NW>
+__device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
+  constexpr uint32_t NT = 64u * NW, NACC = 1024u / NT;
+  constexpr uint32_t PIECES = KIND == 3 ? 2u : 1u;
+  constexpr uint32_t TAIL = KIND == 1 ? 6u : 2u;
+  constexpr uint32_t TILE = 64u * (16u * PIECES + TAIL);
+  extern __shared__ __align__(16) uint8_t sb_lds[];
+  float *terms = (float *)sb_lds;                  // [NW * SBF_NB blocks of the round][32 tokens][32 rows]
+  float *ad_l = terms + NW * SBF_NB * 1024u;       // [nblk][32 tokens]
+  const uint32_t nblk = p.nsb;                     // (blocks of 32 here)
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  const uint32_t t0 = blockIdx.x * 32u, r0 = blockIdx.y * 32u;
+  uint32_t tile_row, rr;
+  {
+    const uint32_t row = min(r0 + l32, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+    const uint32_t rb = row >> p.r_shift;
+    rr = row & ((1u << p.r_shift) - 1u);
+    tile_row = rb * p.nct * TILE;
+  }
+  const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + 32 b
+
+  // the tokens' ad of every block: ad_l[b][token]
+  for (uint32_t i = tid; i < 32u * nblk; i += NT) {
+    const uint32_t k = i / nblk, b = i - k * nblk;
+    ad_l[b * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * nblk + b];
+  }
+
+  uint4 wq[SBF_NB];
+  uint32_t tl[SBF_NB], th[SBF_NB];
+#define SBF_LOADW(B0)                                                                                   \
+  do {                                                                                                  \
+    _Pragma("unroll") for (uint32_t j_ = 0; j_ < SBF_NB; j_++) {                                        \
+      const uint32_t b_ = min((uint32_t)(B0) + j_, nblk - 1u); /* past the end: loaded, never used */   \
+      const uint32_t to_ = tile_row + (b_ >> p.c_shift) * TILE;                                         \
+      const uint32_t ln_ = ((b_ & ((1u << p.c_shift) - 1u)) << p.r_shift) + rr;                         \
+      wq[j_] = *(const uint4 *)(p.wt + (to_ + ln_ * 16u + (KIND == 3 ? lh * 1024u : 0u)));              \
+      const uint16_t *tp_ = (const uint16_t *)(p.wt + (to_ + PIECES * 1024u + ln_ * TAIL));             \
+      tl[j_] = tp_[0];                                                                                  \
+      th[j_] = KIND == 1 ? ((uint32_t)tp_[1] | ((uint32_t)tp_[2] << 16)) : 0u;                          \
+    }                                                                                                   \
+  } while (0)
+
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  float acc[NACC];   // outputs (token, row) = (tid / 32 + a NT / 32, tid % 32)
+#pragma unroll
+  for (uint32_t a = 0; a < NACC; a++) acc[a] = 0.0f;
+  SBF_LOADW(wave * SBF_NB);
+  __syncthreads();   // ad_l
+  for (uint32_t s0 = 0; s0 < nblk; s0 += NW * SBF_NB) {
+    const uint32_t b0 = s0 + wave * SBF_NB;
+#pragma unroll
+    for (uint32_t j = 0; j < SBF_NB; j++) {
+      const uint32_t b = b0 + j;
+      if (b < nblk) {   // wave-uniform
+        int4v bw;   // the lane's sixteen weights: k 16 lh .. 16 lh + 15 of its row's block
+        if (KIND == 3) {
+          bw = (int4v){(int)wq[j].x, (int)wq[j].y, (int)wq[j].z, (int)wq[j].w};
+        } else {
+          // byte i of the sixteen: weight i in its low nibble, weight 16 + i in its high one; Q5_0's fifth bits: bit i
+          const uint32_t q_[4] = {wq[j].x, wq[j].y, wq[j].z, wq[j].w};
+          uint32_t w_[4];
+#pragma unroll
+          for (int k_ = 0; k_ < 4; k_++)
+            w_[k_] = ogm_nib32_weights<KIND>((lh ? q_[k_] >> 4 : q_[k_]) & 0x0F0F0F0Fu, (th[j] >> (16u * lh + 4u * k_)) & 0xFu);
+          bw = (int4v){(int)w_[0], (int)w_[1], (int)w_[2], (int)w_[3]};
+        }
+        const int4v xa = *(const int4v *)(p.xq + (xro + 32u * b));
+        const int16v C = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, bw, zi, 0, 0, 0);
+        const float d = gm_f16_bits_to_f32(tl[j]);
+        const float *adp = &ad_l[b * 32u + 4u * lh];
+        float *tp = terms + ((wave * SBF_NB + j) * 32u + 4u * lh) * 32u + l32;   // [block of the round][token][row]
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          const float4 a4 = *(const float4 *)(adp + 8 * q4);
+          const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+          for (int e = 0; e < 4; e++) tp[(8 * q4 + e) * 32] = (a4v[e] * d) * (float)C[4 * q4 + e];
+        }
+      }
+    }
+    SBF_LOADW(b0 + NW * SBF_NB);   // the next round's weights, in flight over the barrier and the additions
+    __syncthreads();
+    {
+      const uint32_t n_here = min(NW * SBF_NB, nblk - s0);
+      for (uint32_t w = 0; w < n_here; w++) {   // ascending blocks, one accumulator per output
+#pragma unroll
+        for (uint32_t a = 0; a < NACC; a++) acc[a] += terms[w * 1024u + a * NT + tid];
+      }
+    }
+    __syncthreads();
+  }
+#undef SBF_LOADW
+  {
+    const uint32_t row = r0 + (tid & 31u);
+#pragma unroll
+    for (uint32_t a = 0; a < NACC; a++) {
+      const uint32_t tok = t0 + (tid >> 5) + a * (NT / 32u);
+      if (row < p.out_dim && tok < p.n_tokens) p.y[(size_t)tok * p.out_dim + row] = acc[a];
+    }
+  }
+}
+
+template <int KIND>
+__global__ __launch_bounds__(512) void ogm_gemm_sb_flat_kernel(GemmSbParams p) { gemm_sb_flat_body<KIND, 8u>(p); }
 
 static const uint32_t GM_LDS_MAX = 160 * 1024;   // LDS of a CU
 
 size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens) {
   // the int8 activations in operand chunks (token count rounded up to 32), for the all-waves-multiply kernel
   return (size_t)in_dim * ((n_tokens + 31u) & ~31u);
+}
+
+// Whether a launch of the per-32 types takes their small-batch kernel: while its workgroups of 32 rows x 32 tokens
+// are few enough -- about seven rounds of the device's compute units where two of them fit one (rows of up to
+// 4096 inputs: 80 KB of LDS), about four where one does.  Measured on MI355X, Q8_0, whole calls, us, small-batch
+// against tiled: 4096 -> 4096 at 32 / 128 / 384 / 512 tokens 19 / 28 / 70 / 91 against 72 / 76 / 82 / 84; 4096 ->
+// 14336 at 32 / 96 / 128 / 192: 27 / 68 / 81 / 125 against 77 / 80 / 82 / 89; 14336 -> 4096 at 32 / 128 / 256 / 384:
+// 56 / 115 / 225 / 322 against 239 / 243 / 252 / 259; 8192 -> 8192 at 32 / 128 / 192: 37 / 131 / 193 against 142 /
+// 147 / 155; 4096 -> 32064 at 32 / 64: 57 / 101 against 86 / 88.  (Q4_0, Q5_0, IQ4_NL within a few per cent.)
+static bool gemm_flat_small(uint32_t n_tokens, uint32_t out_dim, uint32_t lds_bytes) {
+  const uint32_t wgs = ((n_tokens + 31u) / 32u) * ((out_dim + 31u) / 32u);
+  return wgs <= (lds_bytes <= 80u * 1024u ? 1792u : 1100u);
+}
+
+bool ogm_gemm_flat_small_batch(uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
+  const uint32_t lds = 8u * SBF_NB * 4096u + 128u * (in_dim / 32u);
+  return in_dim % 64u == 0 && lds <= GM_LDS_MAX && gemm_flat_small(n_tokens, out_dim, lds);
 }
 
 static bool is_flat32(uint32_t t) { return t == OGM_Q8_0 || t == OGM_Q5_0 || t == OGM_Q4_0 || t == OGM_IQ4_NL; }
@@ -2518,6 +2650,35 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.c_shift = tl.C == 4 ? 2 : 1;   // in_dim % 64 == 0: at least two blocks per tile row
     p.r_shift = 6 - p.c_shift;
     p.nct = tl.nct;
+    // small batches: the kernel whose waves take different blocks (small_max_tokens as for the K-quants: 0 by the
+    // size of the launch, 1 never, otherwise up to that many tokens)
+    const uint32_t sbf_lds = 8u * SBF_NB * 4096u + 128u * p.nblk;
+    const bool sbf = a.small_max_tokens ? a.n_tokens <= a.small_max_tokens : gemm_flat_small(a.n_tokens, a.out_dim, sbf_lds);
+    if (a.small_max_tokens != 1u && sbf && sbf_lds <= GM_LDS_MAX) {
+      GemmSbParams q{};
+      q.wt = a.wt;
+      q.xq = a.act.q;
+      q.ad = a.act.d;
+      q.y = a.y;
+      q.in_dim = a.in_dim;
+      q.out_dim = a.out_dim;
+      q.n_tokens = a.n_tokens;
+      q.nsb = p.nblk;
+      q.c_shift = p.c_shift;
+      q.r_shift = p.r_shift;
+      q.nct = p.nct;
+      const void *fn = a.ggml_type == OGM_Q4_0   ? (const void *)ogm_gemm_sb_flat_kernel<0>
+                       : a.ggml_type == OGM_Q5_0 ? (const void *)ogm_gemm_sb_flat_kernel<1>
+                       : a.ggml_type == OGM_IQ4_NL ? (const void *)ogm_gemm_sb_flat_kernel<2>
+                                                   : (const void *)ogm_gemm_sb_flat_kernel<3>;
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sbf_lds);
+      if (e != hipSuccess) return e;
+      void *kargs[] = {(void *)&q};
+      e = hipLaunchKernel(fn, dim3((a.n_tokens + 31u) / 32u, (a.out_dim + 31u) / 32u), dim3(512), kargs, sbf_lds, stream);
+      if (e != hipSuccess) return e;
+      if (kernel_name) *kernel_name = "ogm_gemm_sb_flat_kernel";
+      return hipGetLastError();
+    }
     const dim3 grid((a.n_tokens + 127u) / 128u, (a.out_dim + 127u) / 128u);
     switch (a.ggml_type) {
       case OGM_Q4_0: hipLaunchKernelGGL(ogm_gemm_flat_kernel<0>, grid, dim3(768), 0, stream, p); break;

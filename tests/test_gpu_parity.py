@@ -597,8 +597,10 @@ def test_medium_batch_kernel_over_several_matrices_and_extreme_ranges(be):
 
 
 def test_gemm_threshold_default():
-    """A context of its own with no tuning.  Q8_0: 16 tokens go through the GEMV kernel in the GEMM's
-    float order, 17 through the matrix-core GEMM.  Q4_K: 4 tokens through the GEMV kernel, 5 to 8 through the
+    """A context of its own with no tuning.  Q8_0: 8 tokens go through the GEMV kernel in the GEMM's
+    float order, 9 through the per-32 types' small-batch GEMM (rows so long that the GEMV kernel would read the
+    weights once per part of the batch: from the first token it cannot hold), a launch of many workgroups through
+    their tiled GEMM.  Q4_K: 4 tokens through the GEMV kernel, 5 to 8 through the
     row-block kernel, then the small-batch kernel: to 512 tokens over a matrix of up to 2048 rows, to 160 over one
     of up to 4096, where the medium-batch kernel has the rest of the second token tile and a tiled kernel what
     follows; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
@@ -614,12 +616,27 @@ def test_gemm_threshold_default():
         x = synth_x(257, 1024, seed=4)
         w = qm(raw, Q8_0, 1024, 70)
         want = oracle.matmul(Q8_0, raw, 1024, 70, x[:17], 17).reshape(17, 70)
-        y16 = b.matmul(x[:16], 16, w)
+        y8 = b.matmul(x[:8], 8, w)
         assert kname(b).startswith("ogm_gemv_kernel")
+        y9 = b.matmul(x[:9], 9, w)
+        assert kname(b) == "ogm_gemm_sb_flat_kernel"
         y17 = b.matmul(x[:17], 17, w)
-        assert kname(b) == "ogm_gemm_flat_kernel"
+        assert kname(b) == "ogm_gemm_sb_flat_kernel"
         assert_bits(y17, want, "Q8_0, 17 tokens")
-        assert_bits(y16, want[:16], "Q8_0, 16 tokens")
+        assert_bits(y9, want[:9], "Q8_0, 9 tokens")
+        assert_bits(y8, want[:8], "Q8_0, 8 tokens")
+        rawl = synth_weights(Q8_0, 14336, 40, seed=23)   # rows of which the GEMV kernel's LDS holds two tokens' worth
+        xl = synth_x(5, 14336, seed=24)
+        y = b.matmul(xl[:2], 2, qm(rawl, Q8_0, 14336, 40))
+        assert kname(b).startswith("ogm_gemv_kernel")
+        y = b.matmul(xl, 5, qm(rawl, Q8_0, 14336, 40))
+        assert kname(b) == "ogm_gemm_sb_flat_kernel"
+        assert_bits(y, oracle.matmul(Q8_0, rawl, 14336, 40, xl, 5), "Q8_0 of 14336 inputs, 5 tokens")
+        rawf = synth_weights(Q8_0, 256, 8300, seed=22)   # 260 row blocks of 32 x 10 token blocks: the tiled kernel
+        xf = np.ascontiguousarray(x[:, :256])
+        y = b.matmul(xf, 257, qm(rawf, Q8_0, 256, 8300))
+        assert kname(b) == "ogm_gemm_flat_kernel"
+        assert_bits(y, oracle.matmul(Q8_0, rawf, 256, 8300, xf, 257), "Q8_0, 257 tokens x 8300 rows")
         raw = synth_weights(Q4_K, 1024, 70, seed=5)
         w = qm(raw, Q4_K, 1024, 70)
         want = oracle.matmul(Q4_K, raw, 1024, 70, x, 257).reshape(257, 70)
@@ -1228,6 +1245,52 @@ def test_mfma_gemm_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T):
     finally:
         be.set_tuning("gemm_min_tokens", GEMM_FROM)
     assert_bits(small, want, "multi-token gemv")
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL])
+@pytest.mark.parametrize("in_dim,out_dim,T", [(64, 5, 9), (128, 130, 17), (896, 64, 40), (4096, 257, 130), (4864, 100, 33),
+                                              (1024, 128, 128), (2048, 129, 70), (14336, 70, 45), (512, 31, 2)])
+def test_small_batch_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T):
+    """The per-32 types' small-batch kernel (32 rows x 32 tokens a workgroup, its waves on different blocks, a block
+    one int8 matrix instruction, the blocks' terms added in ascending order after every round of sixteen): every bit
+    of dot_flat_pair (vecdot.rs:2598-2629), with rows, tokens and blocks that do not fill the last workgroup or the
+    last round."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T + t)
+    x = synth_x(T, in_dim, seed=T + 1)
+    w = qm(raw, t, in_dim, out_dim)
+    be.set_tuning("gemm_small_max_tokens", 1024)
+    be.set_tuning("gemm_min_tokens", 2)
+    try:
+        got = be.matmul(x, T, w)
+        assert kname(be) == "ogm_gemm_sb_flat_kernel"
+    finally:
+        be.set_tuning("gemm_small_max_tokens", 1)
+        be.set_tuning("gemm_min_tokens", GEMM_FROM)
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "small-batch flat gemm")
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL])
+def test_small_batch_flat_extreme_block_sums(be, t):
+    """As test_mfma_gemm_flat_extreme_block_sums, through the small-batch kernel: 32 * 127 * 127 per block in the
+    int8 matrix instruction's 32-bit sums."""
+    bb = BLOCK[t][0]
+    in_dim, out_dim, T = 256, 40, 24
+    blocks = np.zeros((out_dim * 8, bb), np.uint8)
+    blocks[:, 0:2] = np.frombuffer(np.float16(0.0078125).tobytes(), np.uint8)
+    blocks[0::3, 2:] = 0x00 if t != Q8_0 else 0x81
+    blocks[1::3, 2:] = 0xFF if t != Q8_0 else 0x7F
+    blocks[2::3, 2:] = 0xF0 if t != Q8_0 else 0x81
+    raw = blocks.reshape(-1)
+    x = np.full((T, in_dim), 127.0, np.float32)
+    x[1::2] *= -1
+    x[:, 5::11] = -127.0
+    be.set_tuning("gemm_small_max_tokens", 1024)
+    try:
+        got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
+        assert kname(be) == "ogm_gemm_sb_flat_kernel"
+    finally:
+        be.set_tuning("gemm_small_max_tokens", 1)
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "extreme sums, small-batch kernel")
 
 
 @pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL])
