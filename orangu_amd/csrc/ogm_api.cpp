@@ -683,9 +683,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
     if (rc != OGM_OK) return rc;
     // K-quant matrices over the same input (q, k, v; gate, up) share a launch, up to OGM_GEMM_MAX_MATS
     const size_t per_launch = block_elems_of(w0->ggml_type) == 256 ? OGM_GEMM_MAX_MATS : 1;
-    for (size_t i = 0; i < n_tg; i += per_launch) {
-      const size_t ng = n_tg - i < per_launch ? n_tg - i : per_launch;
-      OgmGemmArgs g;
+    auto fill = [&](OgmGemmArgs &g, size_t i, size_t ng) {
       g.ggml_type = w0->ggml_type;
       g.wt = tg[i].w->dev;
       g.in_dim = w0->in_dim;
@@ -708,6 +706,21 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
         g.extra_out_dim[j - 1] = tg[i + j].w->out_dim;
         g.extra_y[j - 1] = tg[i + j].y;
       }
+    };
+    // IQ4_XS has GEMM kernels over its planes only: without them (no room, or shapes beyond the plane kernels'
+    // 32-bit offsets) the batch stays on the GEMV kernel
+    bool planes_or_nothing = true;
+    for (size_t i = 0; w0->ggml_type == OGM_IQ4_XS && planes_or_nothing && i < n_tg; i += per_launch) {
+      const size_t ng = n_tg - i < per_launch ? n_tg - i : per_launch;
+      OgmGemmArgs g;
+      fill(g, i, ng);
+      planes_or_nothing = ogm_gemm_uses_planes(g);
+      for (size_t j = 0; planes_or_nothing && j < ng; j++) planes_or_nothing = ensure_planes(ctx, tg[i + j].w, stream);
+    }
+    for (size_t i = 0; planes_or_nothing && i < n_tg; i += per_launch) {
+      const size_t ng = n_tg - i < per_launch ? n_tg - i : per_launch;
+      OgmGemmArgs g;
+      fill(g, i, ng);
       if (ogm_gemm_uses_planes(g)) {
         // a tiled int8 kernel: over the matrices' planes when all of them have (or now get) theirs
         bool all = true;
@@ -719,7 +732,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
       }
       HIPCHK(ctx, ogm_launch_gemm(g, stream, &ctx->last_kernel));
     }
-    return OGM_OK;
+    if (planes_or_nothing) return OGM_OK;
   }
   const uint32_t wg_waves = (uint32_t)ctx->tune_wg_waves;
   const uint32_t chunk = gemv_chunk;

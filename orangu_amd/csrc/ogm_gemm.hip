@@ -106,6 +106,7 @@ __host__ __device__ inline size_t gp_plane_offset(uint32_t rb, uint32_t nsb, uin
 #define GP_Q3K 1
 #define GP_Q4K 2
 #define GP_Q5K 3
+#define GP_IQ4XS 4   // plane kernels only: the sums of Q6_K's GEMM (a scale per sub-block, no mins), tiles of Q4_K's size, d where Q4_K has it
 // Ablation switches for timing experiments (scratch builds define them; the library never does):
 // each removes one ingredient of the kernel below, results become wrong, and the time that goes
 // away is what that ingredient costs.
@@ -530,6 +531,7 @@ __global__ __launch_bounds__(512) void ogm_gemm_q5k_i8p_r64_kernel(GemmI8pParams
 //   Q6_K: u = sc_g (q - 32) + 128, sc the int8 scale of the group of 16       (vecdot.rs:2119-2143)
 //   Q3_K: one plane, (sc - 32)(4 - q) with the six-bit scale of the group      (vecdot.rs:2100-2117)
 //   Q4_K / Q5_K: u = sc_j q + 128, sc the six-bit scale of the sub-block of 32 (vecdot.rs:2036-2088)
+//   IQ4_XS: u = (ls_j - 32) level + 128, the sub-block's six-bit scale and IQ4_NL's levels  (vecdot.rs:2333-2350)
 // h = u >> 8, l = (u & 255) - 128 as int8: sc * q' = 256 h + l.
 struct GemmPlaneBuildParams {
   const uint8_t *wt;
@@ -539,8 +541,8 @@ struct GemmPlaneBuildParams {
 
 template <int KIND>
 __global__ __launch_bounds__(256) void ogm_gemm_build_planes_kernel(GemmPlaneBuildParams p) {
-  constexpr bool Q3 = KIND == GP_Q3K, Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K;
-  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : KIND == GP_Q4K ? 9216u : Q5 ? 11264u : 13440u;
+  constexpr bool Q3 = KIND == GP_Q3K, Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K, XS = KIND == GP_IQ4XS;
+  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : (KIND == GP_Q4K || XS) ? 9216u : Q5 ? 11264u : 13440u;
   constexpr uint32_t QS_PIECE0 = Q5 ? 3u : 1u;
   constexpr uint32_t NPL = Q3 ? 1u : 2u;
   const uint32_t t16 = threadIdx.x >> 6, r = threadIdx.x & 63u;
@@ -570,6 +572,22 @@ __global__ __launch_bounds__(256) void ogm_gemm_build_planes_kernel(GemmPlaneBui
     hi_shift = 2u * g + (t16 >> 1);
     hi_mask = 0x01010101u;
     hi_lsh = 2;
+  } else if constexpr (XS) {
+    // sub-block ib = 2 g + t16 / 2 of the super-block, its elements 16 (t16 & 1) ..: the low or the high nibbles of
+    // block bytes 8 + 16 ib .. (the upper half of piece ib, the lower half of piece ib + 1), through IQ4_NL's sixteen
+    // levels; the six-bit scale ls - 32 from scales_l / scales_h (vecdot.rs:2333-2350).  The signed level goes in as
+    // the byte level + 128: u = ls (level + 128) + (128 - 128 ls)
+    const uint32_t ib = 2u * g + (t16 >> 1);
+    const uint4 pa = *(const uint4 *)(u0 + ib * 1024u), pb = *(const uint4 *)(u0 + (ib + 1u) * 1024u);
+    const uint4 hd = *(const uint4 *)u0;
+    const uint32_t sh = hd.x >> 16, sl = hd.y, nsh = 4u * (t16 & 1u);
+    ql = make_uint4(ogm_nib32_weights<2>((pa.z >> nsh) & 0x0F0F0F0Fu, 0u) ^ 0x80808080u,
+                    ogm_nib32_weights<2>((pa.w >> nsh) & 0x0F0F0F0Fu, 0u) ^ 0x80808080u,
+                    ogm_nib32_weights<2>((pb.x >> nsh) & 0x0F0F0F0Fu, 0u) ^ 0x80808080u,
+                    ogm_nib32_weights<2>((pb.y >> nsh) & 0x0F0F0F0Fu, 0u) ^ 0x80808080u);
+    sc = (int)(((sl >> (4u * ib)) & 0xFu) | (((sh >> (2u * ib)) & 3u) << 4)) - 32;
+    addc = (short)(128 - 128 * sc);
+    mask_q = 0xFFFFFFFFu;
   } else if constexpr (Q45) {
     ql = *(const uint4 *)(u0 + (QS_PIECE0 + 2u * g + (t16 & 1u)) * 1024u);
     if constexpr (Q5) qh = *(const uint4 *)(u0 + (1u + (t16 & 1u)) * 1024u);
@@ -764,10 +782,11 @@ __global__ __launch_bounds__(256) void ogm_gemm_xtile_kernel(const int8_t *__res
 template <int KIND, bool ONEPASS = false>
 __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaParams p) {
   constexpr bool Q3 = KIND == GP_Q3K, Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K, Q6 = KIND == GP_Q6K;
+  constexpr bool XS = KIND == GP_IQ4XS;   // (no first pass, as Q6_K; its d is the first half of the header word, as Q4_K's)
   static_assert(!ONEPASS || Q45, "only the types with mins have a first pass to fold");
   constexpr uint32_t RING = ONEPASS ? GD_RING_ONEPASS : GD_RING, AHEAD = RING - 1u;
   constexpr uint32_t TAB = RING * GD_SLOT, TAB_SLOT = ONEPASS ? GD_TAB_SLOT_ONEPASS : GD_TAB_SLOT;
-  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : KIND == GP_Q4K ? 9216u : Q5 ? 11264u : 13440u;
+  constexpr uint32_t TILE_BYTES = Q3 ? 7168u : (KIND == GP_Q4K || XS) ? 9216u : Q5 ? 11264u : 13440u;
   constexpr uint32_t NPL = Q3 ? 1u : 2u;
   constexpr int PER = (int)NPL + 1;   // loads a wave issues per step
   extern __shared__ __align__(16) uint8_t lds[];
@@ -1141,9 +1160,9 @@ __global__ __launch_bounds__(64 * GD_NW, 2) void ogm_gemm_dma_kernel(GemmDmaPara
 template <int KIND>
 __global__ __launch_bounds__(64 * GX_NW, 2) void ogm_gemm_dmx_kernel(GemmDmaParams p) {
   constexpr uint32_t NW = GX_NW, ROWS = GX_ROWS, SLOT = GX_SLOT, TAB = GX_TAB, TAB_SLOT = GX_TAB_SLOT;
-  constexpr bool Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K, Q6 = KIND == GP_Q6K;
-  static_assert(Q45 || Q6, "two-plane types only");
-  constexpr uint32_t TILE_BYTES = KIND == GP_Q4K ? 9216u : Q5 ? 11264u : 13440u;
+  constexpr bool Q45 = KIND == GP_Q4K || KIND == GP_Q5K, Q5 = KIND == GP_Q5K, Q6 = KIND == GP_Q6K, XS = KIND == GP_IQ4XS;
+  static_assert(Q45 || Q6 || XS, "two-plane types only");
+  constexpr uint32_t TILE_BYTES = (KIND == GP_Q4K || XS) ? 9216u : Q5 ? 11264u : 13440u;
   constexpr uint32_t AHEAD = GX_AHEAD, PER = 2u;   // loads a wave issues per step
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -2470,19 +2489,26 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
     return (uint64_t)ogm_tiling_for(in_dim / 32u, out_dim).nrb * 64u * (in_dim / 32u) * l.block_bytes <= lim &&
            (uint64_t)in_dim * n_tokens <= lim;
   }
-  if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K && ggml_type != OGM_Q3_K && ggml_type != OGM_Q5_K) ||
+  // (IQ4_XS: only the kernels over prebuilt planes, where its planes can be had; they pay where the GEMV kernel
+  // would need three passes over the weights -- 4096 -> 4096 at 16 / 31 tokens 28 us against 23 / 41, 14336 -> 4096
+  // 77 against 69 / 134)
+  if (ggml_type == OGM_IQ4_XS && n_tokens < 17u) return false;
+  if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K && ggml_type != OGM_Q3_K && ggml_type != OGM_Q5_K &&
+       ggml_type != OGM_IQ4_XS) ||
       in_dim == 0 || in_dim % 256u != 0)
     return false;
   // Q4_K and Q5_K: the first pass of the tiled kernels keeps the tokens' scales of every super-block in LDS
   // (512 bytes a super-block beside 96 KB of stages); longer rows stay on the GEMV kernel, in chunks of tokens
   if ((ggml_type == OGM_Q4_K || ggml_type == OGM_Q5_K) && (size_t)(in_dim / 256u) * 512u + 98304u > GM_LDS_MAX) return false;
-  const uint64_t block = ggml_type == OGM_Q4_K ? 144u : ggml_type == OGM_Q6_K ? 210u : ggml_type == OGM_Q3_K ? 112u : 176u;
+  const uint64_t block = (ggml_type == OGM_Q4_K || ggml_type == OGM_IQ4_XS) ? 144u : ggml_type == OGM_Q6_K ? 210u
+                         : ggml_type == OGM_Q3_K ? 112u : 176u;   // bytes a block takes in the tile-planar copy
   return (uint64_t)ogm_tiling_for(in_dim / 256u, out_dim).nrb * 64u * (in_dim / 256u) * block <= lim &&
          (uint64_t)in_dim * n_tokens * 2u <= lim;
 }
 
 size_t ogm_gemm_plane_bytes(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim) {
-  if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K && ggml_type != OGM_Q3_K && ggml_type != OGM_Q5_K) ||
+  if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K && ggml_type != OGM_Q3_K && ggml_type != OGM_Q5_K &&
+       ggml_type != OGM_IQ4_XS) ||
       in_dim == 0 || in_dim % 256u != 0 || out_dim == 0)
     return 0;
   const uint32_t npl = ggml_type == OGM_Q3_K ? 1u : 2u;
@@ -2507,6 +2533,7 @@ hipError_t ogm_gemm_build_planes(uint32_t ggml_type, const uint8_t *wt, uint32_t
     case OGM_Q6_K: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_Q6K>, grid, dim3(256), 0, stream, p); break;
     case OGM_Q3_K: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_Q3K>, grid, dim3(256), 0, stream, p); break;
     case OGM_Q4_K: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_Q4K>, grid, dim3(256), 0, stream, p); break;
+    case OGM_IQ4_XS: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_IQ4XS>, grid, dim3(256), 0, stream, p); break;
     default: hipLaunchKernelGGL(ogm_gemm_build_planes_kernel<GP_Q5K>, grid, dim3(256), 0, stream, p); break;
   }
   return hipGetLastError();
@@ -2533,8 +2560,9 @@ hipError_t ogm_gemm_build_planes(uint32_t ggml_type, const uint8_t *wt, uint32_t
 // workgroups, 121 / 127 against 135 / 143).
 static bool gemm_interleaved(const OgmGemmArgs &a) {
   const uint32_t nsb = a.in_dim / 256;
-  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
-  if (a.interleave == 1u || a.ggml_type == OGM_Q3_K || (q45 && a.one_pass != 0u) || nsb * 512u > GX_TAB || a.n_tokens < 32u)
+  const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K, xs = a.ggml_type == OGM_IQ4_XS;
+  if (a.interleave == 1u || a.ggml_type == OGM_Q3_K || (q45 && a.one_pass != 0u) || nsb * 512u > GX_TAB ||
+      a.n_tokens < (xs ? 17u : 32u))
     return false;
   if (a.interleave == 2u) return true;
   uint32_t tiles64 = 0;
@@ -2542,6 +2570,9 @@ static bool gemm_interleaved(const OgmGemmArgs &a) {
   const uint32_t tok_tiles = (a.n_tokens + 127u) / 128u;
   const uint32_t n_wg = tok_tiles * tiles64;
   if (n_wg > 512u) return false;
+  // (IQ4_XS has these two kernels only: 4096 -> 4096 at 32 tokens 28 us against 46 on the 128-row tiles, 14336 -> 4096
+  // 77 against 141, 4096 -> 14336 33 against 50)
+  if (xs) return true;
   if (!q45) return (n_wg >= 128u && (tok_tiles >= 2u || a.n_tokens > 96u)) || (n_wg >= 96u && a.n_tokens >= 192u);
   return tok_tiles >= 3u && n_wg >= 160u && (nsb <= 20u || n_wg <= 256u);
 }
@@ -2555,7 +2586,8 @@ static bool gemm_dma_eligible(const OgmGemmArgs &a) {
   const uint32_t nsb = a.in_dim / 256;
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
   const uint32_t t_pad = (a.n_tokens + 31u) & ~31u;
-  if ((q45 && nsb * 512u > GD_TAB) || a.n_tokens < 32u || !a.xh || (uint64_t)t_pad * a.in_dim >= (1ull << 32))
+  if ((q45 && nsb * 512u > GD_TAB) || a.n_tokens < (a.ggml_type == OGM_IQ4_XS ? 17u : 32u) || !a.xh ||
+      (uint64_t)t_pad * a.in_dim >= (1ull << 32))
     return false;
   uint32_t tiles = 0;
   for (uint32_t m = 0; m <= a.n_extra; m++) {
@@ -2563,7 +2595,8 @@ static bool gemm_dma_eligible(const OgmGemmArgs &a) {
     if ((uint64_t)((od + 63u) / 64u) * 64u * a.in_dim * 2u >= (1ull << 32)) return false;
     tiles += (od + GD_ROWS - 1u) / GD_ROWS;
   }
-  if (a.plane_kernel == 2u || ((a.n_tokens + GD_TOK - 1u) / GD_TOK) * tiles > 256u) return true;
+  // (IQ4_XS has no other GEMM kernel)
+  if (a.plane_kernel == 2u || a.ggml_type == OGM_IQ4_XS || ((a.n_tokens + GD_TOK - 1u) / GD_TOK) * tiles > 256u) return true;
   return gemm_interleaved(a);
 }
 
@@ -2573,6 +2606,7 @@ static bool gemm_dma_eligible(const OgmGemmArgs &a) {
 static bool gemm_small_batch(const OgmGemmArgs &a, bool planes_possible) {
   const uint32_t nsb = a.in_dim / 256;
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  if (a.ggml_type == OGM_IQ4_XS) return false;   // (plane kernels only)
   // Q6_K launches the interleaved plane kernel wants by their size go there (see gemm_interleaved)
   if (a.ggml_type == OGM_Q6_K && a.small_max_tokens == 0u && a.interleave == 0u && planes_possible &&
       gemm_dma_eligible(a) && gemm_interleaved(a))
@@ -2816,22 +2850,25 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     if (interleaved) {
       uint32_t tiles_x = (a.out_dim + GX_ROWS - 1u) / GX_ROWS;
       for (uint32_t m = 0; m < a.n_extra; m++) tiles_x += (a.extra_out_dim[m] + GX_ROWS - 1u) / GX_ROWS;
-      const void *fx = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_dmx_kernel<GP_Q6K>
-                       : a.ggml_type == OGM_Q4_K ? (const void *)ogm_gemm_dmx_kernel<GP_Q4K>
-                                                 : (const void *)ogm_gemm_dmx_kernel<GP_Q5K>;
+      const void *fx = a.ggml_type == OGM_Q6_K     ? (const void *)ogm_gemm_dmx_kernel<GP_Q6K>
+                       : a.ggml_type == OGM_IQ4_XS ? (const void *)ogm_gemm_dmx_kernel<GP_IQ4XS>
+                       : a.ggml_type == OGM_Q4_K   ? (const void *)ogm_gemm_dmx_kernel<GP_Q4K>
+                                                   : (const void *)ogm_gemm_dmx_kernel<GP_Q5K>;
       hipError_t ex = hipFuncSetAttribute(fx, hipFuncAttributeMaxDynamicSharedMemorySize, (int)GX_LDS_BYTES);
       if (ex != hipSuccess) return ex;
       void *xargs[] = {(void *)&d};
       ex = hipLaunchKernel(fx, dim3((a.n_tokens + GX_TOK - 1u) / GX_TOK, tiles_x), dim3(64u * GX_NW), xargs, GX_LDS_BYTES, stream);
       if (ex != hipSuccess) return ex;
       if (kernel_name)
-        *kernel_name = a.ggml_type == OGM_Q6_K   ? "ogm_gemm_q6k_dmx_kernel"
-                       : a.ggml_type == OGM_Q4_K ? "ogm_gemm_q4k_dmx_kernel"
-                                                 : "ogm_gemm_q5k_dmx_kernel";
+        *kernel_name = a.ggml_type == OGM_Q6_K     ? "ogm_gemm_q6k_dmx_kernel"
+                       : a.ggml_type == OGM_IQ4_XS ? "ogm_gemm_iq4xs_dmx_kernel"
+                       : a.ggml_type == OGM_Q4_K   ? "ogm_gemm_q4k_dmx_kernel"
+                                                   : "ogm_gemm_q5k_dmx_kernel";
       return hipGetLastError();
     }
     const bool one_pass = q45 && a.one_pass != 0u;
     const void *fn = a.ggml_type == OGM_Q6_K   ? (const void *)ogm_gemm_dma_kernel<GP_Q6K>
+                     : a.ggml_type == OGM_IQ4_XS ? (const void *)ogm_gemm_dma_kernel<GP_IQ4XS>
                      : a.ggml_type == OGM_Q3_K ? (const void *)ogm_gemm_dma_kernel<GP_Q3K>
                      : a.ggml_type == OGM_Q4_K ? (one_pass ? (const void *)ogm_gemm_dma_kernel<GP_Q4K, true>
                                                            : (const void *)ogm_gemm_dma_kernel<GP_Q4K>)
@@ -2845,6 +2882,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     if (e != hipSuccess) return e;
     if (kernel_name)
       *kernel_name = a.ggml_type == OGM_Q6_K   ? "ogm_gemm_q6k_dma_kernel"
+                     : a.ggml_type == OGM_IQ4_XS ? "ogm_gemm_iq4xs_dma_kernel"
                      : a.ggml_type == OGM_Q3_K ? "ogm_gemm_q3k_dma_kernel"
                      : a.ggml_type == OGM_Q4_K ? (one_pass ? "ogm_gemm_q4k_dma_onepass_kernel" : "ogm_gemm_q4k_dma_kernel")
                                                : (one_pass ? "ogm_gemm_q5k_dma_onepass_kernel" : "ogm_gemm_q5k_dma_kernel");
@@ -2852,6 +2890,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   }
   // The feeding-wave kernels: eight (or four) waves unpack the tile-planar bytes into the two planes per call
   // while as many multiply.
+  if (a.ggml_type == OGM_IQ4_XS) return hipErrorInvalidValue;   // (its GEMMs need its planes: ogm_gemm_uses_planes)
   GemmI8pParams p;
   p.wt = a.wt;
   p.xq = a.act.q;

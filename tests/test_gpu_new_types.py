@@ -195,3 +195,67 @@ def test_q2_k_two_step_calls_in_both_activation_modes(be):
         be.free_weight(h)
         xd.free()
         yd.free()
+
+
+@pytest.mark.parametrize("in_dim,out_dim,T,interleave,kernel", [
+    (256, 5, 32, 1, "ogm_gemm_iq4xs_dma_kernel"), (1024, 130, 45, 2, "ogm_gemm_iq4xs_dmx_kernel"),
+    (768, 257, 129, 1, "ogm_gemm_iq4xs_dma_kernel"), (2048, 129, 300, 2, "ogm_gemm_iq4xs_dmx_kernel"),
+    (512, 4200, 513, 0, "ogm_gemm_iq4xs_dmx_kernel"), (256, 16600, 130, 0, "ogm_gemm_iq4xs_dma_kernel"),
+    (14336, 70, 33, 2, "ogm_gemm_iq4xs_dmx_kernel"), (1280, 64, 31, 1, "ogm_gemm_iq4xs_dma_kernel"),
+    (512, 200, 17, 0, "ogm_gemm_iq4xs_dmx_kernel"), (768, 3000, 20, 0, "ogm_gemm_iq4xs_dmx_kernel"),
+    (256, 33000, 23, 0, "ogm_gemm_iq4xs_dma_kernel"), (1280, 64, 16, 0, "ogm_gemv_kernel<FmtIQ4XS,gemm>")])
+def test_iq4_xs_batches_on_the_plane_kernels(be, in_dim, out_dim, T, interleave, kernel):
+    """From seventeen tokens on (three passes of the GEMV kernel) IQ4_XS takes the GEMM kernels over prebuilt int8 planes (the scale of a sub-block of 32
+    folded into IQ4_NL's levels, split by bytes as Q6_K's are; no other GEMM kernel knows the type): every bit of
+    gemm_k_iq4_xs (vecdot.rs:2305-2322), on 128-row tiles and on the 64-row tiles with the f32 step between the
+    matrix instructions (launches of up to 512 workgroups, by default); up to sixteen tokens the GEMV kernel in the same
+    float order."""
+    raw = synth_weights(IQ4_XS, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T)
+    be.set_tuning("gemm_interleave", interleave)
+    try:
+        got = be.matmul(x, T, qm(raw, IQ4_XS, in_dim, out_dim))
+        assert be.last_kernel() == kernel
+    finally:
+        be.set_tuning("gemm_interleave", 0)
+    assert_bits(got, oracle.matmul(IQ4_XS, raw, in_dim, out_dim, x, T), "IQ4_XS over planes")
+
+
+def test_iq4_xs_extreme_sums_on_the_plane_kernels(be):
+    """Levels -127 and 113 under scales -32 and 31 against activations of +-127: the folded weights reach +-4064
+    (planes -16 .. 16 and their low bytes), a super-block's sum 1.3e8."""
+    in_dim, out_dim, T = 1024, 70, 40
+    blocks = np.zeros((out_dim * 4, 136), np.uint8)
+    blocks[:, 0:2] = np.frombuffer(np.float16(0.002).tobytes(), np.uint8)
+    blocks[0::2, 2:4] = 0xFF      # scales_h: the two high bits of every scale set
+    blocks[0::2, 4:8] = 0xFF      # scales_l: 63 - 32 = 31
+    blocks[1::2, 2:8] = 0x00      # 0 - 32 = -32
+    blocks[0::3, 8:] = 0x00       # level -127
+    blocks[1::3, 8:] = 0xFF       # level 113
+    blocks[2::3, 8:] = 0xF0
+    raw = blocks.reshape(-1)
+    x = np.full((T, in_dim), 127.0, np.float32)
+    x[1::2] *= -1
+    x[:, 5::11] = -127.0
+    for interleave in (1, 2):
+        be.set_tuning("gemm_interleave", interleave)
+        try:
+            got = be.matmul(x, T, qm(raw, IQ4_XS, in_dim, out_dim))
+            assert "iq4xs_dm" in be.last_kernel()
+        finally:
+            be.set_tuning("gemm_interleave", 0)
+        assert_bits(got, oracle.matmul(IQ4_XS, raw, in_dim, out_dim, x, T), f"extreme sums, interleave {interleave}")
+
+
+def test_iq4_xs_without_room_for_planes_stays_on_the_gemv_kernel(be):
+    """With no memory allowed for planes the batch runs on the GEMV kernel in the GEMM's float order: same bits."""
+    in_dim, out_dim, T = 512, 300, 70
+    raw = synth_weights(IQ4_XS, in_dim, out_dim, seed=77)
+    x = synth_x(T, in_dim, seed=78)
+    be.set_tuning("gemm_plane_cache_mb", 0)
+    try:
+        got = be.matmul(x, T, qm(raw, IQ4_XS, in_dim, out_dim))
+        assert be.last_kernel().startswith("ogm_gemv_kernel")
+    finally:
+        be.set_tuning("gemm_plane_cache_mb", 32768)
+    assert_bits(got, oracle.matmul(IQ4_XS, raw, in_dim, out_dim, x, T), "IQ4_XS, no planes")
