@@ -588,7 +588,7 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   // from seventeen otherwise)
   bool flat_small = block_elems_of(t0) == 32 && ctx->tune_gemm_small_max != 1;
   for (size_t i = 0; flat_small && i < n_tg; i++)
-    flat_small = ogm_gemm_flat_small_batch(tg[i].w->in_dim, tg[i].w->out_dim, n_tokens);
+    flat_small = ogm_gemm_flat_small_batch(tg[i].w->ggml_type, tg[i].w->in_dim, tg[i].w->out_dim, n_tokens);
   const uint32_t gemm_from = ctx->tune_gemm_min_tokens ? (uint32_t)ctx->tune_gemm_min_tokens
                              : (t0 == OGM_Q4_K || t0 == OGM_Q5_K || t0 == OGM_Q6_K) ? 6u : (flat_small ? 9u : 17u);
   // A few tokens over a Q6_K matrix of many rows (the vocabulary projection of a decode batch): one

@@ -2345,11 +2345,15 @@ __global__ __launch_bounds__(768) void ogm_gemm_flat_kernel(GemmFlatParams p) {
 // are added in ascending order, one accumulator per output, as dot_flat_pair does (vecdot.rs:2598-2629).
 #define SBF_NB 2u   // blocks a wave takes per round
 
+// KIND 0: Q4_0, 1: Q5_0, 2: IQ4_NL, 3: Q8_0, 4: Q5_1 -- whose blocks also have a minimum: the term of a block is
+// ad * (dw * dot32 + m * block_sum) (dot_q5_1, vecdot.rs:2886-2899, which its several-token path equals bit for
+// bit), the block's sum of activations per token from a second matrix instruction against ones.
 template <int KIND, uint32_t NW>
 __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
   constexpr uint32_t NT = 64u * NW, NACC = 1024u / NT;
   constexpr uint32_t PIECES = KIND == 3 ? 2u : 1u;
-  constexpr uint32_t TAIL = KIND == 1 ? 6u : 2u;
+  constexpr uint32_t TAIL = KIND == 1 ? 6u : KIND == 4 ? 8u : 2u;
+  constexpr int NIB = KIND == 4 ? 3 : KIND;   // ogm_nib32_weights' kind
   constexpr uint32_t TILE = 64u * (16u * PIECES + TAIL);
   extern __shared__ __align__(16) uint8_t sb_lds[];
   float *terms = (float *)sb_lds;                  // [NW * SBF_NB blocks of the round][32 tokens][32 rows]
@@ -2384,8 +2388,9 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
       const uint32_t ln_ = ((b_ & ((1u << p.c_shift) - 1u)) << p.r_shift) + rr;                         \
       wq[j_] = *(const uint4 *)(p.wt + (to_ + ln_ * 16u + (KIND == 3 ? lh * 1024u : 0u)));              \
       const uint16_t *tp_ = (const uint16_t *)(p.wt + (to_ + PIECES * 1024u + ln_ * TAIL));             \
-      tl[j_] = tp_[0];                                                                                  \
-      th[j_] = KIND == 1 ? ((uint32_t)tp_[1] | ((uint32_t)tp_[2] << 16)) : 0u;                          \
+      tl[j_] = KIND == 4 ? ((uint32_t)tp_[0] | ((uint32_t)tp_[1] << 16)) : (uint32_t)tp_[0]; /* d (| m) */ \
+      th[j_] = KIND == 1 ? ((uint32_t)tp_[1] | ((uint32_t)tp_[2] << 16))                                \
+               : KIND == 4 ? ((uint32_t)tp_[2] | ((uint32_t)tp_[3] << 16)) : 0u;                        \
     }                                                                                                   \
   } while (0)
 
@@ -2410,12 +2415,17 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
           uint32_t w_[4];
 #pragma unroll
           for (int k_ = 0; k_ < 4; k_++)
-            w_[k_] = ogm_nib32_weights<KIND>((lh ? q_[k_] >> 4 : q_[k_]) & 0x0F0F0F0Fu, (th[j] >> (16u * lh + 4u * k_)) & 0xFu);
+            w_[k_] = ogm_nib32_weights<NIB>((lh ? q_[k_] >> 4 : q_[k_]) & 0x0F0F0F0Fu, (th[j] >> (16u * lh + 4u * k_)) & 0xFu);
           bw = (int4v){(int)w_[0], (int)w_[1], (int)w_[2], (int)w_[3]};
         }
         const int4v xa = *(const int4v *)(p.xq + (xro + 32u * b));
         const int16v C = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, bw, zi, 0, 0, 0);
-        const float d = gm_f16_bits_to_f32(tl[j]);
+        int16v S = zi;   // Q5_1: the tokens' sums of this block's activations, in every column
+        if constexpr (KIND == 4) {
+          const int4v ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+          S = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, ones, zi, 0, 0, 0);
+        }
+        const float d = gm_f16_bits_to_f32(tl[j] & 0xFFFFu), mn = KIND == 4 ? gm_f16_bits_to_f32(tl[j] >> 16) : 0.0f;
         const float *adp = &ad_l[b * 32u + 4u * lh];
         float *tp = terms + ((wave * SBF_NB + j) * 32u + 4u * lh) * 32u + l32;   // [block of the round][token][row]
 #pragma unroll
@@ -2423,7 +2433,12 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
           const float4 a4 = *(const float4 *)(adp + 8 * q4);
           const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
 #pragma unroll
-          for (int e = 0; e < 4; e++) tp[(8 * q4 + e) * 32] = (a4v[e] * d) * (float)C[4 * q4 + e];
+          for (int e = 0; e < 4; e++) {
+            if constexpr (KIND == 4)
+              tp[(8 * q4 + e) * 32] = a4v[e] * (d * (float)C[4 * q4 + e] + mn * (float)S[4 * q4 + e]);
+            else
+              tp[(8 * q4 + e) * 32] = (a4v[e] * d) * (float)C[4 * q4 + e];
+          }
         }
       }
     }
@@ -2471,12 +2486,16 @@ static bool gemm_flat_small(uint32_t n_tokens, uint32_t out_dim, uint32_t lds_by
   return wgs <= (lds_bytes <= 80u * 1024u ? 1792u : 1100u);
 }
 
-bool ogm_gemm_flat_small_batch(uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
+bool ogm_gemm_flat_small_batch(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
   const uint32_t lds = 8u * SBF_NB * 4096u + 128u * (in_dim / 32u);
-  return in_dim % 64u == 0 && lds <= GM_LDS_MAX && gemm_flat_small(n_tokens, out_dim, lds);
+  if (in_dim % 64u != 0 || lds > GM_LDS_MAX) return false;
+  return ggml_type == OGM_Q5_1 || gemm_flat_small(n_tokens, out_dim, lds);   // (Q5_1 has no other GEMM kernel)
 }
 
-static bool is_flat32(uint32_t t) { return t == OGM_Q8_0 || t == OGM_Q5_0 || t == OGM_Q4_0 || t == OGM_IQ4_NL; }
+// The per-32 types with a GEMM kernel: the four symmetric ones (small-batch and tiled), and Q5_1 (small-batch only).
+static bool is_flat32(uint32_t t) {
+  return t == OGM_Q8_0 || t == OGM_Q5_0 || t == OGM_Q4_0 || t == OGM_IQ4_NL || t == OGM_Q5_1;
+}
 
 bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
   // the kernels address weights and activations with 32-bit byte offsets
@@ -2484,6 +2503,7 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
   if (is_flat32(ggml_type)) {
     // two blocks per stage
     if (in_dim == 0 || in_dim % 64u != 0) return false;
+    if (ggml_type == OGM_Q5_1 && 8u * SBF_NB * 4096u + 128u * (in_dim / 32u) > GM_LDS_MAX) return false;
     OgmLayout l;
     ogm_layout_for(ggml_type, &l);
     return (uint64_t)ogm_tiling_for(in_dim / 32u, out_dim).nrb * 64u * (in_dim / 32u) * l.block_bytes <= lim &&
@@ -2687,8 +2707,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     // small batches: the kernel whose waves take different blocks (small_max_tokens as for the K-quants: 0 by the
     // size of the launch, 1 never, otherwise up to that many tokens)
     const uint32_t sbf_lds = 8u * SBF_NB * 4096u + 128u * p.nblk;
-    const bool sbf = a.small_max_tokens ? a.n_tokens <= a.small_max_tokens : gemm_flat_small(a.n_tokens, a.out_dim, sbf_lds);
-    if (a.small_max_tokens != 1u && sbf && sbf_lds <= GM_LDS_MAX) {
+    const bool q51 = a.ggml_type == OGM_Q5_1;   // (this kernel only, whatever the batch)
+    const bool sbf = q51 || (a.small_max_tokens ? a.n_tokens <= a.small_max_tokens : gemm_flat_small(a.n_tokens, a.out_dim, sbf_lds));
+    if ((q51 || a.small_max_tokens != 1u) && sbf && sbf_lds <= GM_LDS_MAX) {
       GemmSbParams q{};
       q.wt = a.wt;
       q.xq = a.act.q;
@@ -2704,6 +2725,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       const void *fn = a.ggml_type == OGM_Q4_0   ? (const void *)ogm_gemm_sb_flat_kernel<0>
                        : a.ggml_type == OGM_Q5_0 ? (const void *)ogm_gemm_sb_flat_kernel<1>
                        : a.ggml_type == OGM_IQ4_NL ? (const void *)ogm_gemm_sb_flat_kernel<2>
+                       : q51                       ? (const void *)ogm_gemm_sb_flat_kernel<4>
                                                    : (const void *)ogm_gemm_sb_flat_kernel<3>;
       hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sbf_lds);
       if (e != hipSuccess) return e;
@@ -2713,6 +2735,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       if (kernel_name) *kernel_name = "ogm_gemm_sb_flat_kernel";
       return hipGetLastError();
     }
+    if (q51) return hipErrorInvalidValue;
     const dim3 grid((a.n_tokens + 127u) / 128u, (a.out_dim + 127u) / 128u);
     switch (a.ggml_type) {
       case OGM_Q4_0: hipLaunchKernelGGL(ogm_gemm_flat_kernel<0>, grid, dim3(768), 0, stream, p); break;

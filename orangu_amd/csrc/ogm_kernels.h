@@ -91,9 +91,9 @@ size_t ogm_gemm_plane_bytes(uint32_t ggml_type, uint32_t in_dim, uint32_t out_di
 hipError_t ogm_gemm_build_planes(uint32_t ggml_type, const uint8_t *wt, uint32_t in_dim, uint32_t out_dim,
                                  uint8_t *planes, hipStream_t stream);
 bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens);
-// Whether a GEMM of a per-32 type (Q8_0, Q5_0, Q4_0, IQ4_NL) of this shape would take their small-batch kernel by
-// the size of the launch: what makes a GEMM pay below seventeen tokens.
-bool ogm_gemm_flat_small_batch(uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens);
+// Whether a GEMM of a per-32 type (Q8_0, Q5_0, Q4_0, IQ4_NL; Q5_1, which has no other) of this shape would take their
+// small-batch kernel by the size of the launch: what makes a GEMM pay below seventeen tokens.
+bool ogm_gemm_flat_small_batch(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens);
 size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens);
 hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char **kernel_name);
 

@@ -259,3 +259,35 @@ def test_iq4_xs_without_room_for_planes_stays_on_the_gemv_kernel(be):
     finally:
         be.set_tuning("gemm_plane_cache_mb", 32768)
     assert_bits(got, oracle.matmul(IQ4_XS, raw, in_dim, out_dim, x, T), "IQ4_XS, no planes")
+
+
+@pytest.mark.parametrize("in_dim,out_dim,T,kernel", [
+    (64, 5, 9, "ogm_gemm_sb_flat_kernel"), (128, 130, 17, "ogm_gemm_sb_flat_kernel"), (896, 64, 40, "ogm_gemm_sb_flat_kernel"),
+    (4864, 100, 33, "ogm_gemm_sb_flat_kernel"), (2048, 129, 300, "ogm_gemm_sb_flat_kernel"),
+    (14336, 70, 45, "ogm_gemm_sb_flat_kernel"), (512, 31, 8, "ogm_gemv_kernel<FmtQ51,gemm>"),
+    (96, 40, 20, "ogm_gemv_kernel<FmtQ51,gemm>")])
+def test_q5_1_batches_on_the_small_batch_kernel(be, in_dim, out_dim, T, kernel):
+    """From nine tokens on (rows of a multiple of 64 inputs) Q5_1 takes the per-32 types' small-batch GEMM, whatever
+    the batch: a block's term is ad * (dw * dot32 + m * block_sum) (dot_q5_1, vecdot.rs:2886-2899), the block sums of
+    the activations from a second matrix instruction against ones; every bit of the CPU path's."""
+    raw = synth_weights(Q5_1, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T)
+    got = be.matmul(x, T, qm(raw, Q5_1, in_dim, out_dim))
+    assert be.last_kernel() == kernel
+    assert_bits(got, oracle.matmul(Q5_1, raw, in_dim, out_dim, x, T), "Q5_1 batch")
+
+
+def test_q5_1_extreme_sums_on_the_small_batch_kernel(be):
+    """All weights 31 (and 0) with the largest minimum against activations of +-127."""
+    in_dim, out_dim, T = 256, 40, 24
+    blocks = np.zeros((out_dim * 8, 24), np.uint8)
+    blocks[:, 0:2] = np.frombuffer(np.float16(0.0078125).tobytes(), np.uint8)
+    blocks[:, 2:4] = np.frombuffer(np.float16(-3.5).tobytes(), np.uint8)
+    blocks[0::2, 4:] = 0xFF
+    raw = blocks.reshape(-1)
+    x = np.full((T, in_dim), 127.0, np.float32)
+    x[1::2] *= -1
+    x[:, 5::11] = -127.0
+    got = be.matmul(x, T, qm(raw, Q5_1, in_dim, out_dim))
+    assert be.last_kernel() == "ogm_gemm_sb_flat_kernel"
+    assert_bits(got, oracle.matmul(Q5_1, raw, in_dim, out_dim, x, T), "Q5_1 extreme sums")
