@@ -148,9 +148,9 @@ def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
     """Kernel timings at the full size of every benchmark configuration: device-resident inputs,
     back-to-back calls over weight copies totalling more than the 256 MB last-level cache, HIP events
     on the launch stream.  Each figure covers the whole call (activation quantizer + matmul kernels)."""
-    Q8_0, Q6_K = 8, 14
-    blk = {Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256)}
-    names = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+    Q8_0, Q6_K, Q5_1, IQ4_XS = 8, 14, 7, 23
+    blk = {Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256), Q5_1: (24, 32), IQ4_XS: (136, 256)}
+    names = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", Q5_1: "Q5_1", IQ4_XS: "IQ4_XS"}
     stream = hiprt.Stream()
     out = {"device": be.device_name(),
            "unit": "us per call (activation quantizer + matmul kernels), median and fastest of 8 batches of "
@@ -203,6 +203,14 @@ def sweep(be, helpers, hiprt, only: str = "", light: bool = False) -> dict:
     run(Q4_K, 4096, 6144, 512, False, "C4 q+k+v-sized GEMM 4096->6144 M=512", n=64)
     run(Q6_K, FFN, HIDDEN, 512, False, "C4 ffn_down GEMM 14336->4096 M=512", n=64)
     run(Q6_K, FFN, HIDDEN, 1, False, "C5 ffn_down GEMV")
+    # the types beside the K-quants at batch sizes of a verify batch and a prompt (C1's matrix, and the FFN's)
+    for T in (16, 32, 128, 512):
+        run(Q8_0, 4096, 4096, T, False, f"C1-type Q8_0 4096->4096 batch {T}", n=64)
+    run(Q8_0, FFN, HIDDEN, 32, False, "Q8_0 ffn_down-sized 14336->4096 batch 32", n=64)
+    run(Q8_0, HIDDEN, FFN, 512, False, "Q8_0 gate-sized 4096->14336 batch 512", n=64)
+    run(IQ4_XS, HIDDEN, FFN, 32, False, "IQ4_XS gate-sized 4096->14336 batch 32", n=64)
+    run(IQ4_XS, HIDDEN, FFN, 512, False, "IQ4_XS gate-sized 4096->14336 batch 512", n=64)
+    run(Q5_1, HIDDEN, FFN, 512, False, "Q5_1 gate-sized 4096->14336 batch 512", n=32)
     for hs in uploaded.values():
         for h in hs:
             be.free_weight(h)
