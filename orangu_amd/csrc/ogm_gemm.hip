@@ -1669,6 +1669,146 @@ __device__ __forceinline__ void gemm_sb_q6k_body(GemmSbParams p) {
 __global__ __launch_bounds__(512) void ogm_gemm_sb_q6k_kernel(GemmSbParams p) { gemm_sb_q6k_body<8u>(p); }
 __global__ __launch_bounds__(1024) void ogm_gemm_sb_q6k_w16_kernel(GemmSbParams p) { gemm_sb_q6k_body<16u>(p); }
 
+// The same for Q3_K, whose GEMM is Q6_K's loop (vecdot.rs:2014-2021) over weights (sc - 32)(q - 4) of seven bits:
+// one operand plane, w' = (sc - 32)(4 - q) as an int8, and isum = -sum.  A unit's seven pieces: hmask (2), qs (4),
+// scales[12] | d | padding (vecdot.rs:2100-2117).
+template <uint32_t NW>
+__device__ __forceinline__ void gemm_sb_q3k_body(GemmSbParams p) {
+  constexpr uint32_t NT = 64u * NW, NACC = 1024u / NT;
+  constexpr uint32_t TILE_BYTES = 7168u;
+  extern __shared__ __align__(16) uint8_t sb_lds[];
+  float *terms = (float *)sb_lds;            // [NW waves][32 tokens][32 rows]
+  float *ad_l = terms + NW * 32u * 32u;      // [nsb][32 tokens]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  uint32_t row_tile = blockIdx.y;
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + 31u) / 32u;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = blockIdx.x * 32u, r0 = row_tile * 32u;
+  uint32_t uo;   // this lane's row: piece 0 of its unit in super-block 0's tile
+  {
+    const uint32_t row = min(r0 + l32, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    uo = rb * p.nct * TILE_BYTES + r * 16u;
+  }
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
+  };
+  const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + 256 s + 32 step
+
+  for (uint32_t i = tid; i < 32u * p.nsb; i += NT) {
+    const uint32_t k = i / p.nsb, s = i - k * p.nsb;
+    ad_l[s * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + s];
+  }
+
+  // the lane's sixteen weights of step 2 g + sub are elements 64 g + 32 sub + 16 lh ..: run t16 = 2 sub + lh of group g.
+  // Their two low bits sit in qs piece 2 (g / 2) + lh at bit 2 (2 (g & 1) + sub), the third in hmask piece lh at bit
+  // 2 g + sub; the group's six-bit scale: four low bits in scales[4 (g & 1) + t16] (the high nibble for g >= 2), two
+  // high bits in scales[8 + t16] at bit 2 g.
+  uint4 wH, wQ0, wQ1, scx;
+#define SB3_LOADW(S)                                                                              \
+  do {                                                                                            \
+    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded, never used */    \
+    const uint32_t so_ = uo + sb_off(s_);                                                         \
+    wH = *(const uint4 *)(p.wt + (so_ + lh * 1024u));                                             \
+    wQ0 = *(const uint4 *)(p.wt + (so_ + (2u + lh) * 1024u));                                     \
+    wQ1 = *(const uint4 *)(p.wt + (so_ + (4u + lh) * 1024u));                                     \
+    scx = *(const uint4 *)(p.wt + (so_ + 6u * 1024u));                                            \
+  } while (0)
+#define SB3_STEP(G, SUB, FIRST)                                                                   \
+  do {                                                                                            \
+    const uint32_t t16_ = 2u * (SUB) + lh;                                                        \
+    const uint32_t lw_ = ((G) & 1u) ? scx.y : scx.x;                                              \
+    const uint32_t low_ = ((lw_ >> (8u * t16_)) >> ((G) >= 2u ? 4u : 0u)) & 0xFu;                 \
+    const uint32_t high_ = ((scx.z >> (8u * t16_)) >> (2u * (G))) & 3u;                           \
+    const int scv_ = (int)(low_ | (high_ << 4)) - 32;                                             \
+    const short2v sc2_ = {(short)-scv_, (short)-scv_};                                            \
+    const short2v c2_ = {(short)(4 * scv_), (short)(4 * scv_)};                                   \
+    const uint4 &Q_ = (G) >= 2u ? wQ1 : wQ0;                                                      \
+    const uint32_t qlw_[4] = {Q_.x, Q_.y, Q_.z, Q_.w}, qhw_[4] = {wH.x, wH.y, wH.z, wH.w};        \
+    uint32_t pw_[4];                                                                              \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      const uint32_t v_ = ((qlw_[w_] >> (2u * (2u * ((G) & 1u) + (SUB)))) & 0x03030303u) |        \
+                          (((qhw_[w_] >> (2u * (G) + (SUB))) & 0x01010101u) << 2);                \
+      union { uint32_t u; short2v s; } e_, f_;                                                    \
+      e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
+      f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
+      e_.s = e_.s * sc2_ + c2_;                                                                   \
+      f_.s = f_.s * sc2_ + c2_;                                                                   \
+      pw_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u);   /* the lanes' low bytes */      \
+    }                                                                                             \
+    const int4v bw_ = {(int)pw_[0], (int)pw_[1], (int)pw_[2], (int)pw_[3]};                       \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 64u * (G) + 32u * (SUB)));                   \
+    H = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bw_, (FIRST) ? zi : H, 0, 0, 0);               \
+  } while (0)
+
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  float acc[NACC];   // outputs (token, row) = (tid / 32 + a NT / 32, tid % 32)
+#pragma unroll
+  for (uint32_t a = 0; a < NACC; a++) acc[a] = 0.0f;
+  SB3_LOADW(wave);
+  __syncthreads();   // ad_l
+  for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
+    const uint32_t s = s0 + wave;
+    if (s < p.nsb) {   // wave-uniform
+      const uint32_t xs_ = xro + 256u * s;
+      int16v H;
+      SB3_STEP(0u, 0u, true);
+      SB3_STEP(0u, 1u, false);
+      SB3_STEP(1u, 0u, false);
+      SB3_STEP(1u, 1u, false);
+      SB3_STEP(2u, 0u, false);
+      SB3_STEP(2u, 1u, false);
+      SB3_STEP(3u, 0u, false);
+      SB3_STEP(3u, 1u, false);
+      const float d = gm_f16_bits_to_f32(scx.w & 0xFFFFu);
+      const float *adp = &ad_l[s * 32u + 4u * lh];
+      float *tp = terms + (wave * 32u + 4u * lh) * 32u + l32;   // [wave][token][row]
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const float4 a4 = *(const float4 *)(adp + 8 * q4);
+        const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) tp[(8 * q4 + e) * 32] = a4v[e] * (d * (float)(-H[4 * q4 + e]));
+      }
+    }
+    SB3_LOADW(s + NW);   // the next round's weights, in flight over the barrier and the additions
+    __syncthreads();
+    {
+      const uint32_t n_here = min(NW, p.nsb - s0);
+      for (uint32_t w = 0; w < n_here; w++) {   // ascending super-blocks, one accumulator per output
+#pragma unroll
+        for (uint32_t a = 0; a < NACC; a++) acc[a] += terms[w * 1024u + a * NT + tid];
+      }
+    }
+    __syncthreads();
+  }
+#undef SB3_LOADW
+#undef SB3_STEP
+  {
+    const uint32_t row = r0 + (tid & 31u);
+#pragma unroll
+    for (uint32_t a = 0; a < NACC; a++) {
+      const uint32_t tok = t0 + (tid >> 5) + a * (NT / 32u);
+      if (row < p.out_dim && tok < p.n_tokens) p.y[(size_t)tok * p.out_dim + row] = acc[a];
+    }
+  }
+}
+
+__global__ __launch_bounds__(512) void ogm_gemm_sb_q3k_kernel(GemmSbParams p) { gemm_sb_q3k_body<8u>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_sb_q3k_w16_kernel(GemmSbParams p) { gemm_sb_q3k_body<16u>(p); }
+
 // The same for Q4_K and Q5_K (gemm_k_q4_k, vecdot.rs:2213-2303): first a sweep over the super-blocks
 // for the terms (ad * dmin) * imin, which the reference subtracts before anything else (rounds of
 // sixteen super-blocks, two per wave: header and the quantizer's sums per 32 only, one f16 matrix
@@ -2645,7 +2785,7 @@ static bool gemm_small_batch(const OgmGemmArgs &a, bool planes_possible) {
                                 : tiles64_all <= 64u ? (med ? 160u : 256u)
                                 : tiles64_all <= 128u ? (med ? 96u : 128u)
                                                       : 64u);
-  return a.ggml_type != OGM_Q3_K && a.small_max_tokens != 1u && a.n_tokens <= small_max &&
+  return a.small_max_tokens != 1u && a.n_tokens <= small_max &&
          (q45 ? 16u : 8u) * 4096u + 128u * nsb <= GM_LDS_MAX;
 }
 
@@ -2789,6 +2929,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
                      16u * 4096u + 128u * nsb <= GM_LDS_MAX;
     const uint32_t lds_bytes = ((q45 || w16) ? 16u : 8u) * 4096u + 128u * nsb;
     const void *fn = a.ggml_type == OGM_Q6_K   ? (w16 ? (const void *)ogm_gemm_sb_q6k_w16_kernel : (const void *)ogm_gemm_sb_q6k_kernel)
+                     : a.ggml_type == OGM_Q3_K ? (w16 ? (const void *)ogm_gemm_sb_q3k_w16_kernel : (const void *)ogm_gemm_sb_q3k_kernel)
                      : a.ggml_type == OGM_Q4_K ? (w16 ? (const void *)ogm_gemm_sb_q45k_w16_kernel<false> : (const void *)ogm_gemm_sb_q45k_kernel<false>)
                                                : (w16 ? (const void *)ogm_gemm_sb_q45k_w16_kernel<true> : (const void *)ogm_gemm_sb_q45k_kernel<true>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -2798,6 +2939,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     if (e != hipSuccess) return e;
     if (kernel_name)
       *kernel_name = a.ggml_type == OGM_Q6_K   ? (w16 ? "ogm_gemm_sb_q6k_w16_kernel" : "ogm_gemm_sb_q6k_kernel")
+                     : a.ggml_type == OGM_Q3_K ? (w16 ? "ogm_gemm_sb_q3k_w16_kernel" : "ogm_gemm_sb_q3k_kernel")
                      : a.ggml_type == OGM_Q4_K ? (w16 ? "ogm_gemm_sb_q4k_w16_kernel" : "ogm_gemm_sb_q4k_kernel")
                                                : (w16 ? "ogm_gemm_sb_q5k_w16_kernel" : "ogm_gemm_sb_q5k_kernel");
     return hipGetLastError();

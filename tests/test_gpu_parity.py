@@ -711,7 +711,7 @@ def test_gemm_threshold_default():
         b.close()
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q3_K, Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("in_dim,out_dim,T", [
     (256, 5, 9), (1024, 100, 17), (768, 64, 32), (1280, 257, 40), (2048, 37, 64), (14336, 96, 33), (1792, 33, 10),
     (4096, 300, 20), (512, 31, 63), (2304, 130, 100), (1024, 70, 128), (256, 1, 1000),
@@ -720,7 +720,8 @@ def test_gemm_threshold_default():
 def test_small_batch_gemm_matches_cpu_gemm(be, t, in_dim, out_dim, T, waves):
     """The small-batch kernel of the K-quants (a workgroup's eight or sixteen waves on different super-blocks of
     32 rows x 32 tokens, terms added in ascending order afterwards): every bit of gemm_k_q4_k /
-    gemm_k_q6_k (vecdot.rs:2213-2303, 2352-2398), at any token count it is asked for."""
+    gemm_k_q6_k (vecdot.rs:2213-2303, 2352-2398; Q3_K through gemm_k_q6_k's loop, :2014-2021), at any token count
+    it is asked for."""
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T + 2)
     be.set_tuning("gemm_small_max_tokens", 1024)
@@ -730,12 +731,13 @@ def test_small_batch_gemm_matches_cpu_gemm(be, t, in_dim, out_dim, T, waves):
     finally:
         be.set_tuning("gemm_small_max_tokens", 1)
         be.set_tuning("gemm_sb_waves", 8)
-    assert kname(be) == {Q4_K: "ogm_gemm_sb_q4k", Q5_K: "ogm_gemm_sb_q5k", Q6_K: "ogm_gemm_sb_q6k"}[t] + \
+    assert kname(be) == {Q3_K: "ogm_gemm_sb_q3k", Q4_K: "ogm_gemm_sb_q4k", Q5_K: "ogm_gemm_sb_q5k", Q6_K: "ogm_gemm_sb_q6k"}[t] + \
         ("_w16_kernel" if waves == 16 else "_kernel")
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "small-batch gemm")
 
 
-@pytest.mark.parametrize("t,block,hi", [(Q4_K, 144, 0xFF), (Q5_K, 176, 0xFF), (Q6_K, 210, 0x7F), (Q6_K, 210, 0x80)])
+@pytest.mark.parametrize("t,block,hi", [(Q4_K, 144, 0xFF), (Q5_K, 176, 0xFF), (Q6_K, 210, 0x7F), (Q6_K, 210, 0x80),
+                                        (Q3_K, 110, 0xFF), (Q3_K, 110, 0x00)])
 @pytest.mark.parametrize("waves", [8, 16])
 def test_small_batch_gemm_extreme_integer_ranges(be, t, block, hi, waves):
     """Every weight bit and scale byte at its extreme (Q6_K: scales +127 and -128), activations +-127."""
@@ -744,6 +746,10 @@ def test_small_batch_gemm_extreme_integer_ranges(be, t, block, hi, waves):
     if t == Q6_K:
         blocks[:, 192:208] = hi
         blocks[:, 208:210] = np.frombuffer(np.float16(0.003).tobytes(), np.uint8)
+    elif t == Q3_K:   # hmask[32] | qs[64] | scales[12] | d: scales 63 - 32 = 31 or 0 - 32 = -32, weights 3 or (hmask 0) -1
+        blocks[:, 96:108] = hi
+        blocks[1::2, 0:32] = 0x00
+        blocks[:, 108:110] = np.frombuffer(np.float16(0.003).tobytes(), np.uint8)
     else:
         blocks[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
         blocks[:, 2:4] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
@@ -789,6 +795,7 @@ def test_mfma_gemm_rows_too_long_for_the_plane_kernel(be):
     (Q4_K, 40, (300, 130, 64), "ogm_gemm_sb_q4k_kernel"),
     (Q5_K, 20, (520, 70, 129), "ogm_gemm_sb_q5k_kernel"),
     (Q6_K, 33, (300, 31), "ogm_gemm_sb_q6k_kernel"),
+    (Q3_K, 33, (128, 300, 70), "ogm_gemm_sb_q3k_kernel"),
 ])
 def test_k_quant_matrices_over_one_input_share_a_gemm_launch(be, t, n_tokens, outs, kernel):
     """q / k / v (llama.rs:730-746) at prefill widths: K-quant matrices of one type over the same
