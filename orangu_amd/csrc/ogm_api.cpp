@@ -707,13 +707,14 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
         g.extra_y[j - 1] = tg[i + j].y;
       }
     };
-    // IQ4_XS has GEMM kernels over its planes only: without them (no room, or shapes beyond the plane kernels'
-    // 32-bit offsets) the batch stays on the GEMV kernel
+    // Beyond its small batches IQ4_XS has GEMM kernels over its planes only: without them (no room, or shapes beyond
+    // the plane kernels' 32-bit offsets) the batch stays on the GEMV kernel
     bool planes_or_nothing = true;
     for (size_t i = 0; w0->ggml_type == OGM_IQ4_XS && planes_or_nothing && i < n_tg; i += per_launch) {
       const size_t ng = n_tg - i < per_launch ? n_tg - i : per_launch;
       OgmGemmArgs g;
       fill(g, i, ng);
+      if (ogm_gemm_takes_small_batch(g)) continue;
       planes_or_nothing = ogm_gemm_uses_planes(g);
       for (size_t j = 0; planes_or_nothing && j < ng; j++) planes_or_nothing = ensure_planes(ctx, tg[i + j].w, stream);
     }

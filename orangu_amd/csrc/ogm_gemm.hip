@@ -1809,6 +1809,143 @@ __device__ __forceinline__ void gemm_sb_q3k_body(GemmSbParams p) {
 __global__ __launch_bounds__(512) void ogm_gemm_sb_q3k_kernel(GemmSbParams p) { gemm_sb_q3k_body<8u>(p); }
 __global__ __launch_bounds__(1024) void ogm_gemm_sb_q3k_w16_kernel(GemmSbParams p) { gemm_sb_q3k_body<16u>(p); }
 
+// The same for IQ4_XS (gemm_k_iq4_xs, vecdot.rs:2305-2322: Q6_K's loop with a scale per sub-block of 32).  A unit's
+// 136 bytes are nine pieces (the last half used): d | scales_h | scales_l, then the eight sub-blocks' sixteen bytes of
+// nibbles from byte 8 on, so sub-block ib is the upper half of piece ib and the lower half of piece ib + 1; both
+// lane halves read the same bytes, the lower one their low nibbles (elements 0..15), the upper one the high ones.
+// Operand planes as the plane builder makes them: u = ls (level + 128) + (128 - 128 ls).
+template <uint32_t NW>
+__device__ __forceinline__ void gemm_sb_iq4xs_body(GemmSbParams p) {
+  constexpr uint32_t NT = 64u * NW, NACC = 1024u / NT;
+  constexpr uint32_t TILE_BYTES = 9216u;
+  extern __shared__ __align__(16) uint8_t sb_lds[];
+  float *terms = (float *)sb_lds;            // [NW waves][32 tokens][32 rows]
+  float *ad_l = terms + NW * 32u * 32u;      // [nsb][32 tokens]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  uint32_t row_tile = blockIdx.y;
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + 31u) / 32u;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = blockIdx.x * 32u, r0 = row_tile * 32u;
+  uint32_t uo;
+  {
+    const uint32_t row = min(r0 + l32, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+    const uint32_t rb = row >> p.r_shift, r = row & ((1u << p.r_shift) - 1u);
+    uo = rb * p.nct * TILE_BYTES + r * 16u;
+  }
+  auto sb_off = [&](uint32_t s) -> uint32_t {
+    return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
+  };
+  const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + 256 s + 32 ib
+  const uint32_t nsh = 4u * lh;
+
+  for (uint32_t i = tid; i < 32u * p.nsb; i += NT) {
+    const uint32_t k = i / p.nsb, s = i - k * p.nsb;
+    ad_l[s * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + s];
+  }
+
+  uint4 pc[9];
+#define SBX_LOADW(S)                                                                              \
+  do {                                                                                            \
+    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded, never used */    \
+    const uint32_t so_ = uo + sb_off(s_);                                                         \
+    _Pragma("unroll") for (int i_ = 0; i_ < 9; i_++) pc[i_] = *(const uint4 *)(p.wt + (so_ + i_ * 1024u)); \
+  } while (0)
+#define SBX_STEP(IB, FIRST)                                                                       \
+  do {                                                                                            \
+    const int ls_ = (int)(((sl_ >> (4u * (IB))) & 0xFu) | (((sh_ >> (2u * (IB))) & 3u) << 4)) - 32; \
+    const short2v sc2_ = {(short)ls_, (short)ls_};                                                \
+    const short2v c2_ = {(short)(128 - 128 * ls_), (short)(128 - 128 * ls_)};                     \
+    const uint32_t qw_[4] = {pc[IB].z, pc[IB].w, pc[(IB) + 1].x, pc[(IB) + 1].y};                 \
+    uint32_t ph_[4], pl_[4];                                                                      \
+    _Pragma("unroll") for (int w_ = 0; w_ < 4; w_++) {                                            \
+      const uint32_t v_ = ogm_nib32_weights<2>((qw_[w_] >> nsh) & 0x0F0F0F0Fu, 0u) ^ 0x80808080u; \
+      union { uint32_t u; short2v s; } e_, f_;                                                    \
+      e_.u = __builtin_amdgcn_perm(0u, v_, 0x0c010c00u);   /* (b0, b1) as 16-bit lanes */         \
+      f_.u = __builtin_amdgcn_perm(0u, v_, 0x0c030c02u);   /* (b2, b3) */                         \
+      e_.s = e_.s * sc2_ + c2_;                                                                   \
+      f_.s = f_.s * sc2_ + c2_;                                                                   \
+      ph_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x07050301u);                                   \
+      pl_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u) ^ 0x80808080u;                     \
+    }                                                                                             \
+    const int4v bh_ = {(int)ph_[0], (int)ph_[1], (int)ph_[2], (int)ph_[3]};                       \
+    const int4v bl_ = {(int)pl_[0], (int)pl_[1], (int)pl_[2], (int)pl_[3]};                       \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 32u * (IB)));                                \
+    H = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bh_, (FIRST) ? zi : H, 0, 0, 0);               \
+    L = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bl_, (FIRST) ? zi : L, 0, 0, 0);               \
+  } while (0)
+
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  float acc[NACC];   // outputs (token, row) = (tid / 32 + a NT / 32, tid % 32)
+#pragma unroll
+  for (uint32_t a = 0; a < NACC; a++) acc[a] = 0.0f;
+  SBX_LOADW(wave);
+  __syncthreads();   // ad_l
+  for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
+    const uint32_t s = s0 + wave;
+    if (s < p.nsb) {   // wave-uniform
+      const uint32_t xs_ = xro + 256u * s;
+      const uint32_t sh_ = pc[0].x >> 16, sl_ = pc[0].y;
+      int16v H, L;
+      SBX_STEP(0, true);
+      SBX_STEP(1, false);
+      SBX_STEP(2, false);
+      SBX_STEP(3, false);
+      SBX_STEP(4, false);
+      SBX_STEP(5, false);
+      SBX_STEP(6, false);
+      SBX_STEP(7, false);
+      const float d = gm_f16_bits_to_f32(pc[0].x & 0xFFFFu);
+      const float *adp = &ad_l[s * 32u + 4u * lh];
+      float *tp = terms + (wave * 32u + 4u * lh) * 32u + l32;   // [wave][token][row]
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const float4 a4 = *(const float4 *)(adp + 8 * q4);
+        const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int is_ = H[4 * q4 + e] * 256 + L[4 * q4 + e];
+          tp[(8 * q4 + e) * 32] = a4v[e] * (d * (float)is_);
+        }
+      }
+    }
+    SBX_LOADW(s + NW);   // the next round's weights, in flight over the barrier and the additions
+    __syncthreads();
+    {
+      const uint32_t n_here = min(NW, p.nsb - s0);
+      for (uint32_t w = 0; w < n_here; w++) {   // ascending super-blocks, one accumulator per output
+#pragma unroll
+        for (uint32_t a = 0; a < NACC; a++) acc[a] += terms[w * 1024u + a * NT + tid];
+      }
+    }
+    __syncthreads();
+  }
+#undef SBX_LOADW
+#undef SBX_STEP
+  {
+    const uint32_t row = r0 + (tid & 31u);
+#pragma unroll
+    for (uint32_t a = 0; a < NACC; a++) {
+      const uint32_t tok = t0 + (tid >> 5) + a * (NT / 32u);
+      if (row < p.out_dim && tok < p.n_tokens) p.y[(size_t)tok * p.out_dim + row] = acc[a];
+    }
+  }
+}
+
+__global__ __launch_bounds__(512) void ogm_gemm_sb_iq4xs_kernel(GemmSbParams p) { gemm_sb_iq4xs_body<8u>(p); }
+__global__ __launch_bounds__(1024) void ogm_gemm_sb_iq4xs_w16_kernel(GemmSbParams p) { gemm_sb_iq4xs_body<16u>(p); }
+
 // The same for Q4_K and Q5_K (gemm_k_q4_k, vecdot.rs:2213-2303): first a sweep over the super-blocks
 // for the terms (ad * dmin) * imin, which the reference subtracts before anything else (rounds of
 // sixteen super-blocks, two per wave: header and the quantizer's sums per 32 only, one f16 matrix
@@ -2649,10 +2786,8 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
     return (uint64_t)ogm_tiling_for(in_dim / 32u, out_dim).nrb * 64u * (in_dim / 32u) * l.block_bytes <= lim &&
            (uint64_t)in_dim * n_tokens <= lim;
   }
-  // (IQ4_XS: only the kernels over prebuilt planes, where its planes can be had; they pay where the GEMV kernel
-  // would need three passes over the weights -- 4096 -> 4096 at 16 / 31 tokens 28 us against 23 / 41, 14336 -> 4096
-  // 77 against 69 / 134)
-  if (ggml_type == OGM_IQ4_XS && n_tokens < 17u) return false;
+  // (IQ4_XS: a small-batch kernel, and beyond the small batches only the kernels over prebuilt planes, where its
+  // planes can be had: see ogm_gemm_takes_small_batch)
   if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K && ggml_type != OGM_Q3_K && ggml_type != OGM_Q5_K &&
        ggml_type != OGM_IQ4_XS) ||
       in_dim == 0 || in_dim % 256u != 0)
@@ -2718,7 +2853,8 @@ hipError_t ogm_gemm_build_planes(uint32_t ggml_type, const uint8_t *wt, uint32_t
 // compute units (8192 -> 8192 at 384 / 512 tokens, 384 / 512 workgroups, 114 / 127 against 101 / 113 for the
 // feeding-wave kernel, 8192 -> 10240 at 384 120 against 108; but 14336 -> 4096 at 384 / 512 tokens, 192 / 256
 // workgroups, 121 / 127 against 135 / 143).
-static bool gemm_interleaved(const OgmGemmArgs &a) {
+// for_small_batch: asked by gemm_small_batch, whether the launch is one this kernel takes ahead of the small batches.
+static bool gemm_interleaved(const OgmGemmArgs &a, bool for_small_batch = false) {
   const uint32_t nsb = a.in_dim / 256;
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K, xs = a.ggml_type == OGM_IQ4_XS;
   if (a.interleave == 1u || a.ggml_type == OGM_Q3_K || (q45 && a.one_pass != 0u) || nsb * 512u > GX_TAB ||
@@ -2730,9 +2866,9 @@ static bool gemm_interleaved(const OgmGemmArgs &a) {
   const uint32_t tok_tiles = (a.n_tokens + 127u) / 128u;
   const uint32_t n_wg = tok_tiles * tiles64;
   if (n_wg > 512u) return false;
-  // (IQ4_XS has these two kernels only: 4096 -> 4096 at 32 tokens 28 us against 46 on the 128-row tiles, 14336 -> 4096
-  // 77 against 141, 4096 -> 14336 33 against 50)
-  if (xs) return true;
+  // (beyond its small batches IQ4_XS has the two plane kernels only: 4096 -> 4096 at 32 tokens 28 us against 46 on the
+  // 128-row tiles, 14336 -> 4096 77 against 141, 4096 -> 14336 33 against 50)
+  if (xs && !for_small_batch) return true;
   if (!q45) return (n_wg >= 128u && (tok_tiles >= 2u || a.n_tokens > 96u)) || (n_wg >= 96u && a.n_tokens >= 192u);
   return tok_tiles >= 3u && n_wg >= 160u && (nsb <= 20u || n_wg <= 256u);
 }
@@ -2766,10 +2902,9 @@ static bool gemm_dma_eligible(const OgmGemmArgs &a) {
 static bool gemm_small_batch(const OgmGemmArgs &a, bool planes_possible) {
   const uint32_t nsb = a.in_dim / 256;
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
-  if (a.ggml_type == OGM_IQ4_XS) return false;   // (plane kernels only)
-  // Q6_K launches the interleaved plane kernel wants by their size go there (see gemm_interleaved)
-  if (a.ggml_type == OGM_Q6_K && a.small_max_tokens == 0u && a.interleave == 0u && planes_possible &&
-      gemm_dma_eligible(a) && gemm_interleaved(a))
+  // Q6_K and IQ4_XS launches the interleaved plane kernel wants by their size go there (see gemm_interleaved)
+  if ((a.ggml_type == OGM_Q6_K || a.ggml_type == OGM_IQ4_XS) && a.small_max_tokens == 0u && a.interleave == 0u &&
+      planes_possible && gemm_dma_eligible(a) && gemm_interleaved(a, true))
     return false;
   uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
   for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
@@ -2816,6 +2951,11 @@ static bool gemm_medium_batch(const OgmGemmArgs &a) {
   const bool full_enough = tok_tiles * SBW_TOK - a.n_tokens <= 32u;
   // (rows of more than 8192 inputs: 16384 -> 16384 at 128 tokens 205 us against 154 for the feeding waves)
   return nsb <= 32u && ((tok_tiles == 1u && full_enough && tiles64_all <= 256u) || (tok_tiles == 2u && tiles64_all <= 128u));
+}
+
+bool ogm_gemm_takes_small_batch(const OgmGemmArgs &a) {
+  if (a.n_tokens == 0 || a.out_dim == 0 || is_flat32(a.ggml_type)) return false;
+  return ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens) && gemm_small_batch(a, true);
 }
 
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a) {
@@ -2930,6 +3070,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     const uint32_t lds_bytes = ((q45 || w16) ? 16u : 8u) * 4096u + 128u * nsb;
     const void *fn = a.ggml_type == OGM_Q6_K   ? (w16 ? (const void *)ogm_gemm_sb_q6k_w16_kernel : (const void *)ogm_gemm_sb_q6k_kernel)
                      : a.ggml_type == OGM_Q3_K ? (w16 ? (const void *)ogm_gemm_sb_q3k_w16_kernel : (const void *)ogm_gemm_sb_q3k_kernel)
+                     : a.ggml_type == OGM_IQ4_XS ? (w16 ? (const void *)ogm_gemm_sb_iq4xs_w16_kernel : (const void *)ogm_gemm_sb_iq4xs_kernel)
                      : a.ggml_type == OGM_Q4_K ? (w16 ? (const void *)ogm_gemm_sb_q45k_w16_kernel<false> : (const void *)ogm_gemm_sb_q45k_kernel<false>)
                                                : (w16 ? (const void *)ogm_gemm_sb_q45k_w16_kernel<true> : (const void *)ogm_gemm_sb_q45k_kernel<true>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -2940,6 +3081,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     if (kernel_name)
       *kernel_name = a.ggml_type == OGM_Q6_K   ? (w16 ? "ogm_gemm_sb_q6k_w16_kernel" : "ogm_gemm_sb_q6k_kernel")
                      : a.ggml_type == OGM_Q3_K ? (w16 ? "ogm_gemm_sb_q3k_w16_kernel" : "ogm_gemm_sb_q3k_kernel")
+                     : a.ggml_type == OGM_IQ4_XS ? (w16 ? "ogm_gemm_sb_iq4xs_w16_kernel" : "ogm_gemm_sb_iq4xs_kernel")
                      : a.ggml_type == OGM_Q4_K ? (w16 ? "ogm_gemm_sb_q4k_w16_kernel" : "ogm_gemm_sb_q4k_kernel")
                                                : (w16 ? "ogm_gemm_sb_q5k_w16_kernel" : "ogm_gemm_sb_q5k_kernel");
     return hipGetLastError();

@@ -85,6 +85,8 @@ struct OgmGemmArgs {
 };
 // Whether this launch would run a tiled int8 plane kernel, i.e. whether planes would be read.
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a);
+// Whether this K-quant or IQ4_XS launch would run the small-batch kernel of its type (which needs no planes).
+bool ogm_gemm_takes_small_batch(const OgmGemmArgs &a);
 // Bytes of a K-quant matrix's planes (0: the type has none), and the kernel that builds them from
 // the tile-planar bytes (2 bytes per weight, 1 for Q3_K; rows padded to a multiple of 64).
 size_t ogm_gemm_plane_bytes(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim);

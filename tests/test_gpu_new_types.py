@@ -213,11 +213,13 @@ def test_iq4_xs_batches_on_the_plane_kernels(be, in_dim, out_dim, T, interleave,
     raw = synth_weights(IQ4_XS, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T)
     be.set_tuning("gemm_interleave", interleave)
+    be.set_tuning("gemm_small_max_tokens", 1)   # (its small-batch kernel has a test of its own)
     try:
         got = be.matmul(x, T, qm(raw, IQ4_XS, in_dim, out_dim))
         assert be.last_kernel() == kernel
     finally:
         be.set_tuning("gemm_interleave", 0)
+        be.set_tuning("gemm_small_max_tokens", 0)
     assert_bits(got, oracle.matmul(IQ4_XS, raw, in_dim, out_dim, x, T), "IQ4_XS over planes")
 
 
@@ -237,19 +239,53 @@ def test_iq4_xs_extreme_sums_on_the_plane_kernels(be):
     x = np.full((T, in_dim), 127.0, np.float32)
     x[1::2] *= -1
     x[:, 5::11] = -127.0
-    for interleave in (1, 2):
+    for interleave, small_max in ((1, 1), (2, 1), (0, 1024)):   # the two plane kernels, the small-batch kernel
         be.set_tuning("gemm_interleave", interleave)
+        be.set_tuning("gemm_small_max_tokens", small_max)
         try:
             got = be.matmul(x, T, qm(raw, IQ4_XS, in_dim, out_dim))
-            assert "iq4xs_dm" in be.last_kernel()
+            assert ("iq4xs_dm" if small_max == 1 else "sb_iq4xs") in be.last_kernel()
         finally:
             be.set_tuning("gemm_interleave", 0)
-        assert_bits(got, oracle.matmul(IQ4_XS, raw, in_dim, out_dim, x, T), f"extreme sums, interleave {interleave}")
+            be.set_tuning("gemm_small_max_tokens", 0)
+        assert_bits(got, oracle.matmul(IQ4_XS, raw, in_dim, out_dim, x, T), f"extreme sums, {be.last_kernel()}")
+
+
+@pytest.mark.parametrize("waves", [8, 16])
+@pytest.mark.parametrize("in_dim,out_dim,T", [(256, 5, 9), (1024, 100, 17), (768, 64, 32), (1280, 257, 40), (14336, 96, 33),
+                                              (2304, 130, 100), (256, 1, 300)])
+def test_iq4_xs_small_batch_kernel(be, in_dim, out_dim, T, waves):
+    """The K-quants' small-batch kernel with IQ4_XS's unpacking (32 rows x 32 tokens, the waves on different
+    super-blocks, terms added in ascending order): every bit of gemm_k_iq4_xs (vecdot.rs:2305-2322)."""
+    raw = synth_weights(IQ4_XS, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T + 2)
+    be.set_tuning("gemm_small_max_tokens", 1024)
+    be.set_tuning("gemm_sb_waves", waves)
+    try:
+        got = be.matmul(x, T, qm(raw, IQ4_XS, in_dim, out_dim))
+        assert be.last_kernel() == ("ogm_gemm_sb_iq4xs_w16_kernel" if waves == 16 else "ogm_gemm_sb_iq4xs_kernel")
+    finally:
+        be.set_tuning("gemm_small_max_tokens", 0)
+        be.set_tuning("gemm_sb_waves", 0)
+    assert_bits(got, oracle.matmul(IQ4_XS, raw, in_dim, out_dim, x, T), "IQ4_XS small batch")
+
+
+def test_iq4_xs_default_routing(be):
+    """Up to eight tokens the GEMV kernel, then the small-batch kernel, and the plane kernels where a launch has
+    enough workgroups for them."""
+    raw = synth_weights(IQ4_XS, 512, 4200, seed=3)
+    x = synth_x(300, 512, seed=4)
+    w = qm(raw, IQ4_XS, 512, 4200)
+    want = oracle.matmul(IQ4_XS, raw, 512, 4200, x, 300).reshape(300, 4200)
+    for T, kernel in ((8, "ogm_gemv_kernel"), (9, "ogm_gemm_sb_iq4xs"), (64, "ogm_gemm_sb_iq4xs"), (300, "ogm_gemm_iq4xs_dmx_kernel")):
+        got = be.matmul(x[:T], T, w)
+        assert be.last_kernel().startswith(kernel), (T, be.last_kernel())
+        assert_bits(got, want[:T], f"IQ4_XS, {T} tokens")
 
 
 def test_iq4_xs_without_room_for_planes_stays_on_the_gemv_kernel(be):
     """With no memory allowed for planes the batch runs on the GEMV kernel in the GEMM's float order: same bits."""
-    in_dim, out_dim, T = 512, 300, 70
+    in_dim, out_dim, T = 512, 300, 700
     raw = synth_weights(IQ4_XS, in_dim, out_dim, seed=77)
     x = synth_x(T, in_dim, seed=78)
     be.set_tuning("gemm_plane_cache_mb", 0)
