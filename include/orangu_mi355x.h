@@ -437,7 +437,7 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              in all (default 32768): on a matrix's first GEMM that would read them its scale-folded
  *                              int8 planes (2 bytes per weight, 1 for Q3_K) are built once and kept; a matrix
  *                              that does not fit, and every matrix at 0, is unpacked on every call (IQ4_XS, whose
- *                              only GEMM kernels read planes, then stays on the GEMV kernel);
+ *                              GEMM kernels beyond its small batches read planes, then stays on the GEMV kernel);
  *                              ogm_weight_download is unaffected
  *   "gemm_plane_kernel"        when the kernel that multiplies the planes (all waves multiply, operands loaded
  *                              straight into LDS) runs: 0 = default, when the launch has more than 256 tiles of
