@@ -1946,6 +1946,124 @@ __device__ __forceinline__ void gemm_sb_iq4xs_body(GemmSbParams p) {
 __global__ __launch_bounds__(512) void ogm_gemm_sb_iq4xs_kernel(GemmSbParams p) { gemm_sb_iq4xs_body<8u>(p); }
 __global__ __launch_bounds__(1024) void ogm_gemm_sb_iq4xs_w16_kernel(GemmSbParams p) { gemm_sb_iq4xs_body<16u>(p); }
 
+// Q2_K at several tokens: the reference's rows-unpacked-once path over per-32 activations (unpack_q2_k +
+// dot_unpacked, vecdot.rs:1144-1164, 420-425, 1722-1728) leaves sixteen f32 terms a super-block, one per group of 16,
+//   act.d[g / 2] * ((d * sc_g) * isum_g - (dmin * mn_g) * sums[g]),
+// added in group order.  A workgroup owns 32 rows x 32 tokens; a round is one super-block, wave w its groups 2 w and
+// 2 w + 1 (the run of 32 two-bit values w): a group is one v_mfma_i32_32x32x16_i8, the activations' sums per 16 a
+// second one against ones, and the sixteen terms of the round are added in ascending order, one accumulator per
+// output.  A unit's 84 bytes: scales[16], qs[64] in four pieces, d | dmin behind the tile's pieces.
+typedef long sbq2_i64;
+
+__global__ __launch_bounds__(512) void ogm_gemm_sb_q2k_kernel(GemmSbParams p) {
+  constexpr uint32_t NW = 8u, NT = 64u * NW, NACC = 1024u / NT;
+  constexpr uint32_t TILE_BYTES = 64u * 84u;
+  extern __shared__ __align__(16) uint8_t sb_lds[];
+  float *terms = (float *)sb_lds;            // [16 groups][32 tokens][32 rows]
+  float *ad_l = terms + 16u * 1024u;         // [in_dim / 32][32 tokens]
+  const uint32_t nblk = p.in_dim / 32u;
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t l32 = lane & 31u, lh = lane >> 5;
+  uint32_t row_tile = blockIdx.y;
+#pragma unroll
+  for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {   // the matrix this row tile belongs to
+    const uint32_t tiles = (p.out_dim + 31u) / 32u;
+    if (m < p.n_extra && row_tile >= tiles) {
+      row_tile -= tiles;
+      p.wt = p.extra_wt[m];
+      p.y = p.extra_y[m];
+      p.out_dim = p.extra_out_dim[m];
+    } else {
+      break;
+    }
+  }
+  const uint32_t t0 = blockIdx.x * 32u, r0 = row_tile * 32u;
+  uint32_t tile_row, rr;
+  {
+    const uint32_t row = min(r0 + l32, p.out_dim - 1u);   // rows past the matrix: clamped, never stored
+    const uint32_t rb = row >> p.r_shift;
+    rr = row & ((1u << p.r_shift) - 1u);
+    tile_row = rb * p.nct * TILE_BYTES;
+  }
+  const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 8u * lh;   // + 256 s + 16 g
+
+  for (uint32_t i = tid; i < 32u * nblk; i += NT) {
+    const uint32_t k = i / nblk, b = i - k * nblk;
+    ad_l[b * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * nblk + b];
+  }
+
+  // the wave's part of a unit: the scales, the two pieces of its run's 32 bytes (bytes 16 h .. of qs[32 (w / 4) ..]),
+  // d | dmin
+  uint4 wsc, wq0, wq1;
+  uint32_t dd;
+  const uint32_t qpiece = 1u + 2u * (wave >> 2), qshift = 2u * (wave & 3u);
+#define SBQ2_LOADW(S)                                                                             \
+  do {                                                                                            \
+    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded, never used */    \
+    const uint32_t to_ = tile_row + (s_ >> p.c_shift) * TILE_BYTES;                               \
+    const uint32_t ln_ = ((s_ & ((1u << p.c_shift) - 1u)) << p.r_shift) + rr;                     \
+    wsc = *(const uint4 *)(p.wt + (to_ + ln_ * 16u));                                             \
+    wq0 = *(const uint4 *)(p.wt + (to_ + ln_ * 16u + qpiece * 1024u));                            \
+    wq1 = *(const uint4 *)(p.wt + (to_ + ln_ * 16u + (qpiece + 1u) * 1024u));                     \
+    dd = *(const uint32_t *)(p.wt + (to_ + 5u * 1024u + ln_ * 4u));                               \
+  } while (0)
+
+  const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  const sbq2_i64 ones = 0x0101010101010101L;
+  float acc[NACC];   // outputs (token, row) = (tid / 32 + a NT / 32, tid % 32)
+#pragma unroll
+  for (uint32_t a = 0; a < NACC; a++) acc[a] = 0.0f;
+  SBQ2_LOADW(0u);
+  __syncthreads();   // ad_l
+  for (uint32_t s = 0; s < p.nsb; s++) {
+    const float d = gm_f16_bits_to_f32(dd & 0xFFFFu), dmin = gm_f16_bits_to_f32(dd >> 16);
+    const uint32_t scw = wave < 2u ? wsc.x : wave < 4u ? wsc.y : wave < 6u ? wsc.z : wsc.w;   // scales[2 w], [2 w + 1] in it
+#pragma unroll
+    for (uint32_t h = 0; h < 2u; h++) {
+      const uint32_t g = 2u * wave + h;
+      const uint4 &Q = h ? wq1 : wq0;
+      union { uint32_t w[2]; sbq2_i64 v; } bw, xa;
+      bw.w[0] = ((lh ? Q.z : Q.x) >> qshift) & 0x03030303u;   // the lane's eight weights: k 8 lh .. of its row's group
+      bw.w[1] = ((lh ? Q.w : Q.y) >> qshift) & 0x03030303u;
+      const uint2 xv = *(const uint2 *)(p.xq + (xro + 256u * s + 16u * g));
+      xa.w[0] = xv.x;
+      xa.w[1] = xv.y;
+      const int16v C = __builtin_amdgcn_mfma_i32_32x32x16_i8(xa.v, bw.v, zi, 0, 0, 0);
+      const int16v S = __builtin_amdgcn_mfma_i32_32x32x16_i8(xa.v, ones, zi, 0, 0, 0);   // the tokens' sums of the group
+      const uint32_t scb = (scw >> (8u * (2u * (wave & 1u) + h))) & 0xFFu;
+      const float scale = d * (float)(scb & 0xFu), mn = dmin * (float)(scb >> 4);
+      const float *adp = &ad_l[(8u * s + wave) * 32u + 4u * lh];
+      float *tp = terms + (g * 32u + 4u * lh) * 32u + l32;   // [group][token][row]
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const float4 a4 = *(const float4 *)(adp + 8 * q4);
+        const float a4v[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          tp[(8 * q4 + e) * 32] = a4v[e] * (scale * (float)C[4 * q4 + e] - mn * (float)S[4 * q4 + e]);
+      }
+    }
+    SBQ2_LOADW(s + 1u);   // the next round's weights, in flight over the barrier and the additions
+    __syncthreads();
+#pragma unroll
+    for (uint32_t g = 0; g < 16u; g++) {   // ascending groups, one accumulator per output
+#pragma unroll
+      for (uint32_t a = 0; a < NACC; a++) acc[a] += terms[g * 1024u + a * NT + tid];
+    }
+    __syncthreads();
+  }
+#undef SBQ2_LOADW
+  {
+    const uint32_t row = r0 + (tid & 31u);
+#pragma unroll
+    for (uint32_t a = 0; a < NACC; a++) {
+      const uint32_t tok = t0 + (tid >> 5) + a * (NT / 32u);
+      if (row < p.out_dim && tok < p.n_tokens) p.y[(size_t)tok * p.out_dim + row] = acc[a];
+    }
+  }
+}
+
 // The same for Q4_K and Q5_K (gemm_k_q4_k, vecdot.rs:2213-2303): first a sweep over the super-blocks
 // for the terms (ad * dmin) * imin, which the reference subtracts before anything else (rounds of
 // sixteen super-blocks, two per wave: header and the quantizer's sums per 32 only, one f16 matrix
@@ -2788,6 +2906,13 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
   }
   // (IQ4_XS: a small-batch kernel, and beyond the small batches only the kernels over prebuilt planes, where its
   // planes can be had: see ogm_gemm_takes_small_batch)
+  // Q2_K (over per-32 activations): one kernel, whose table of the tokens' scales must fit beside its terms; it pays
+  // from about nine tokens (4096 -> 4096 at 4 / 9 / 16 / 512 tokens 35 / 36 / 36 / 186 us against the GEMV kernel's
+  // 20 / 29 / 56 / 1467; 14336 -> 4096 at 4 / 9 / 512: 111 / 109 / 912 against 83 / 184 / 10014)
+  if (ggml_type == OGM_Q2_K)
+    return n_tokens >= 9u && in_dim != 0 && in_dim % 256u == 0 && 16u * 4096u + 128u * (in_dim / 32u) <= GM_LDS_MAX &&
+           (uint64_t)ogm_tiling_for(in_dim / 256u, out_dim).nrb * 64u * (in_dim / 256u) * 84u <= lim &&
+           (uint64_t)in_dim * n_tokens <= lim;
   if ((ggml_type != OGM_Q4_K && ggml_type != OGM_Q6_K && ggml_type != OGM_Q3_K && ggml_type != OGM_Q5_K &&
        ggml_type != OGM_IQ4_XS) ||
       in_dim == 0 || in_dim % 256u != 0)
@@ -2955,11 +3080,12 @@ static bool gemm_medium_batch(const OgmGemmArgs &a) {
 
 bool ogm_gemm_takes_small_batch(const OgmGemmArgs &a) {
   if (a.n_tokens == 0 || a.out_dim == 0 || is_flat32(a.ggml_type)) return false;
-  return ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens) && gemm_small_batch(a, true);
+  if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return false;
+  return a.ggml_type == OGM_Q2_K || gemm_small_batch(a, true);
 }
 
 bool ogm_gemm_uses_planes(const OgmGemmArgs &a) {
-  if (a.n_tokens == 0 || a.out_dim == 0 || is_flat32(a.ggml_type)) return false;
+  if (a.n_tokens == 0 || a.out_dim == 0 || is_flat32(a.ggml_type) || a.ggml_type == OGM_Q2_K) return false;
   if (!ogm_gemm_supported(a.ggml_type, a.in_dim, a.out_dim, a.n_tokens)) return false;
   // (the feeding-wave kernels unpack on every call: reading planes made them no faster -- Q4_K 4096 -> 14336 at 256
   // tokens 66 against 66 us, Q6_K 14336 -> 4096 at 512 tokens 96 against 98)
@@ -3028,6 +3154,39 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   }
   const uint32_t nsb = a.in_dim / 256;
   const bool q45 = a.ggml_type == OGM_Q4_K || a.ggml_type == OGM_Q5_K;
+  if (a.ggml_type == OGM_Q2_K) {   // its one GEMM kernel, whatever the batch
+    GemmSbParams q{};
+    q.wt = a.wt;
+    q.xq = a.act.q;
+    q.ad = a.act.d;   // per 32
+    q.y = a.y;
+    q.in_dim = a.in_dim;
+    q.out_dim = a.out_dim;
+    q.n_tokens = a.n_tokens;
+    q.nsb = nsb;
+    const OgmTiling tl2 = ogm_tiling_for(nsb, a.out_dim);
+    const uint32_t cs2 = tl2.C == 4 ? 2 : (tl2.C == 2 ? 1 : 0);
+    q.c_shift = cs2;
+    q.r_shift = 6 - cs2;
+    q.nct = tl2.nct;
+    q.n_extra = a.n_extra;
+    uint32_t tiles = (a.out_dim + 31u) / 32u;
+    for (uint32_t m = 0; m < OGM_GEMM_MAX_MATS - 1; m++) {
+      q.extra_wt[m] = m < a.n_extra ? a.extra_wt[m] : nullptr;
+      q.extra_y[m] = m < a.n_extra ? a.extra_y[m] : nullptr;
+      q.extra_out_dim[m] = m < a.n_extra ? a.extra_out_dim[m] : 0u;
+      if (m < a.n_extra) tiles += (a.extra_out_dim[m] + 31u) / 32u;
+    }
+    const uint32_t lds_bytes = 16u * 4096u + 128u * (a.in_dim / 32u);
+    const void *fn = (const void *)ogm_gemm_sb_q2k_kernel;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    void *kargs[] = {(void *)&q};
+    e = hipLaunchKernel(fn, dim3((a.n_tokens + 31u) / 32u, tiles), dim3(512), kargs, lds_bytes, stream);
+    if (e != hipSuccess) return e;
+    if (kernel_name) *kernel_name = "ogm_gemm_sb_q2k_kernel";
+    return hipGetLastError();
+  }
   // Q4_K / Q5_K: the first pass's operand, the quantizer's sums per 32 as f16 pairs, comes from the quantizer
   const _Float16 *bs16 = (const _Float16 *)a.act.bs16;
   if (q45 && !bs16) return hipErrorInvalidValue;

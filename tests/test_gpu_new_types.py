@@ -327,3 +327,36 @@ def test_q5_1_extreme_sums_on_the_small_batch_kernel(be):
     got = be.matmul(x, T, qm(raw, Q5_1, in_dim, out_dim))
     assert be.last_kernel() == "ogm_gemm_sb_flat_kernel"
     assert_bits(got, oracle.matmul(Q5_1, raw, in_dim, out_dim, x, T), "Q5_1 extreme sums")
+
+
+@pytest.mark.parametrize("in_dim,out_dim,T,kernel", [
+    (256, 5, 9, "ogm_gemm_sb_q2k_kernel"), (1024, 130, 17, "ogm_gemm_sb_q2k_kernel"), (768, 257, 40, "ogm_gemm_sb_q2k_kernel"),
+    (2048, 129, 300, "ogm_gemm_sb_q2k_kernel"), (14336, 70, 33, "ogm_gemm_sb_q2k_kernel"),
+    (24576, 3, 10, "ogm_gemm_sb_q2k_kernel"), (256, 1, 1000, "ogm_gemm_sb_q2k_kernel"),
+    (512, 31, 8, "ogm_gemv_kernel<FmtQ2KGen,gemm>")])
+def test_q2_k_batches_on_the_matrix_cores(be, in_dim, out_dim, T, kernel):
+    """From nine tokens on Q2_K's several-token arithmetic (unpack_q2_k + dot_unpacked over per-32 activations,
+    vecdot.rs:1144-1164, 420-425, 1722-1728: sixteen terms a super-block, added in group order) runs on a kernel whose
+    waves take the groups of a super-block, a group one K = 16 int8 matrix instruction and a second one against ones
+    for the activations' sum: every bit of the CPU path's."""
+    raw = synth_weights(Q2_K, in_dim, out_dim, seed=in_dim + out_dim + T)
+    x = synth_x(T, in_dim, seed=T)
+    got = be.matmul(x, T, qm(raw, Q2_K, in_dim, out_dim))
+    assert be.last_kernel() == kernel
+    assert_bits(got, oracle.matmul(Q2_K, raw, in_dim, out_dim, x, T), "Q2_K batch")
+
+
+def test_q2_k_extreme_sums_on_the_matrix_cores(be):
+    """All weights 3, scales and minimums 15, against activations of +-127."""
+    in_dim, out_dim, T = 1024, 40, 24
+    blocks = np.full((out_dim * 4, 84), 0xFF, np.uint8)
+    blocks[:, 80:82] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    blocks[:, 82:84] = np.frombuffer(np.float16(0.02).tobytes(), np.uint8)
+    blocks[1::2, 16:80] = 0x00
+    raw = blocks.reshape(-1)
+    x = np.full((T, in_dim), 127.0, np.float32)
+    x[1::2] *= -1
+    x[:, ::7] = 126.0
+    got = be.matmul(x, T, qm(raw, Q2_K, in_dim, out_dim))
+    assert be.last_kernel() == "ogm_gemm_sb_q2k_kernel"
+    assert_bits(got, oracle.matmul(Q2_K, raw, in_dim, out_dim, x, T), "Q2_K extreme sums")

@@ -89,6 +89,7 @@ def test_long_rows_that_outgrow_the_default_lds(be, t, in_dim, out_dim, T, decod
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim)
     x = synth_x(T, in_dim, seed=T)
     w = QuantMatrix(np.ascontiguousarray(raw), t, in_dim, out_dim)
+    be.set_tuning("gemm_min_tokens", 100000)   # (batches of these sizes would take a matrix-core kernel)
     try:
         if decode:
             got, want = be.matmul_decode(x, T, w), oracle.matmul_decode(t, raw, in_dim, out_dim, x, T)
@@ -98,6 +99,7 @@ def test_long_rows_that_outgrow_the_default_lds(be, t, in_dim, out_dim, T, decod
         bad = np.nonzero(bits(got) != bits(want))[0]
         assert bad.size == 0, f"{be.last_kernel()}: {bad.size} of {want.size} differ, first {bad[:4]}"
     finally:
+        be.set_tuning("gemm_min_tokens", 0)
         be.evict(w)
 
 
