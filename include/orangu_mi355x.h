@@ -421,9 +421,15 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              waves work on different super-blocks (blocks, for the per-32 types: by default
  *                              while the launch has at most 1792 workgroups of 32 rows x 32 tokens, 1100 on
  *                              rows beyond 4096 inputs) of the same rows; 0 = default (K-quants: 64, more
- *                              for matrices of few rows, up to 512 for Q4_K / Q5_K matrices of at most 2048; Q6_K
- *                              launches that "gemm_interleave" sends to its kernel by their size go there
- *                              first), 1 = never
+ *                              for matrices of few rows: 128 up to 8192 rows, 256 up to 4096 -- and up to 6144
+ *                              for Q4_K / Q5_K rows of more than 8192 inputs --, 384 up to 2048, 512 there for
+ *                              Q4_K / Q5_K; Q6_K launches that "gemm_interleave" sends to its kernel by their size
+ *                              go there first), 1 = never
+ *   "gemm_act_chunks"          whether a K-quant batch's int8 activations are also written in the operand order
+ *                              of the matrix-core kernels (1 KiB chunks of 32 tokens x 32 inputs; the small-batch
+ *                              kernels then load a chunk in one piece instead of gathering 32 rows, the plane
+ *                              and medium-batch kernels need no relayout launch): 0 = default, from 25 tokens
+ *                              (the forward pass's own producers from 17), 1 = never, 2 = from 9.  Same bits
  *   "gemm_sb_waves"            waves of a small-batch workgroup: 8 or 16; 0 = by the size of the launch
  *   "gemm_medium"              the Q4_K / Q5_K kernel for one nearly full tile of 128 tokens, or two (32 rows x
  *                              128 tokens a workgroup, its waves on different super-blocks): 0 = by the size of
@@ -445,11 +451,12 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              the grid, from 32 tokens
  *   "gemm_interleave"          the plane kernel with 64-row tiles that adds a super-block up between the next
  *                              one's matrix instructions (Q4_K, Q5_K, Q6_K): 0 = default, on launches of at most
- *                              512 tiles of 64 rows x 128 tokens: Q6_K from 128 such tiles (a lone token tile more
- *                              than three quarters full) or 96 with at least 192 tokens; Q4_K / Q5_K from three
- *                              token tiles and 160 tiles, with rows longer than 5120 inputs at most 256 (the 8B
- *                              shapes' q/k/v, wo and down projections at 257 to 1024 tokens, down from 129; their
- *                              planes are built then); 1 = never; 2 = wherever the plane kernel runs.  Same bits
+ *                              512 tiles of 64 rows x 128 tokens: Q6_K from 128 such tiles with the last token
+ *                              tile more than three quarters full or with three token tiles, or from 160 with
+ *                              more than 96 tokens; Q4_K / Q5_K from three token tiles (two over rows of more
+ *                              than 8192 inputs) and 160 tiles, with rows longer than 5120 inputs at most 256 (the
+ *                              8B shapes' q/k/v, wo and down projections at 257 to 1024 tokens; their planes are
+ *                              built then); 1 = never; 2 = wherever the plane kernel runs.  Same bits
  *   "gemm_one_pass"            0 = default.  1: Q4_K and Q5_K on that kernel skip the reference GEMM's separate
  *                              first pass over the mins (vecdot.rs:2229-2240) and add
  *                              ad * (d * isum - dmin * imin) per super-block, the single-token expression of

@@ -69,6 +69,7 @@ struct ogm_ctx {
   bool host_coherent = true;           // the pinned staging buffers are fine-grained (asked for by name); false once the runtime has refused
   int tune_gemv_mma = 1;               // few tokens over Q4_K / Q5_K / Q6_K on the row-block matrix-core kernel: 0 never, 1 where it measured faster, 2 wherever it can
   int tune_gemm_plane_kernel = 0;      // the all-waves-multiply kernel over planes: 0 on large grids, 2 whatever the grid
+  int tune_gemm_act_chunks = 0;       // a K-quant batch's int8 activations also in the matrix-core kernels' operand chunks: 0 from 25 tokens (producers of the forward pass: 17), 1 never, 2 from 9
   int tune_gemm_interleave = 0;        // the 64-row plane kernel with the f32 step between the matrix instructions: 0 by the launch's size, 1 never, 2 whenever it can
   int tune_gemm_one_pass = 0;          // 1: Q4_K / Q5_K on that kernel fold the min pass into the super-block step (f32 to rounding, not to the bit)
   int tune_prefill_chunk = 2048;       // tokens per prefill pass over the layers (fixed per model at its first prefill)
@@ -318,6 +319,11 @@ extern "C" int ogm_set_tuning(ogm_ctx *ctx, const char *key, int value) {
     ctx->tune_gemm_interleave = value;
     return OGM_OK;
   }
+  if (strcmp(key, "gemm_act_chunks") == 0) {
+    if (value < 0 || value > 2) return fail(ctx, OGM_ERR_INVALID, "gemm_act_chunks must be 0, 1 or 2");
+    ctx->tune_gemm_act_chunks = value;
+    return OGM_OK;
+  }
   if (strcmp(key, "gemm_one_pass") == 0) {
     if (value != 0 && value != 1) return fail(ctx, OGM_ERR_INVALID, "gemm_one_pass must be 0 or 1");
     ctx->tune_gemm_one_pass = value;
@@ -485,6 +491,19 @@ extern "C" int ogm_weight_info(const ogm_weight *w, uint32_t *ggml_type, uint32_
 // ------------------------------------------------------------------------------------------
 // matmul
 
+// Whether the int8 activations of a batch over K-quant matrices of this type and width are also laid out in the
+// operand chunks of the matrix-core GEMMs (ogm_xt_row): the plane and medium-batch kernels read nothing else, and the
+// small-batch kernels load a chunk of 32 tokens x 32 k in one piece instead of gathering 32 rows.  from: the batch
+// size from which the caller's producer writes them by default.
+static bool act_chunks_wanted(const ogm_ctx *ctx, uint32_t ggml_type, uint32_t in_dim, uint32_t n_tokens, int decode,
+                              uint32_t from) {
+  if (decode || ctx->tune_gemm_act_chunks == 1 || ogm_gemm_plane_bytes(ggml_type, in_dim, 64u) == 0 ||
+      act_mode_for(ggml_type, n_tokens, decode) != OGM_ACT_PER_256 ||
+      (uint64_t)((n_tokens + 31u) & ~31u) * in_dim >= (1ull << 32))
+    return false;
+  return n_tokens >= (ctx->tune_gemm_act_chunks == 2 ? 9u : from);
+}
+
 // Enqueues the activation quantizer.  Caller holds the lock.
 // with_xt: the int8 activations also go to ctx->xh in the operand chunks of the GEMM whose waves all multiply.
 static int enqueue_quantize(ogm_ctx *ctx, int mode, const float *x_dev, uint32_t in_dim,
@@ -518,11 +537,11 @@ static int enqueue_matmul(ogm_ctx *ctx, const Target *tg, size_t n_tg, const flo
                           int32_t *dump_imin) {
   if (n_tokens == 0 || n_tg == 0) return OGM_OK;
   const ogm_weight *w = tg[0].w;
-  // A batch that may go to the GEMM over prebuilt planes has its activations laid out for it by the quantizer
-  // itself (32 tokens on, K-quants with planes enabled); whether that kernel runs is decided per launch.
-  const bool with_xt = !decode && n_tokens >= 32 && !dump_isum && !dump_imin && ctx->tune_plane_cache_mb > 0 &&
-                       ogm_gemm_plane_bytes(w->ggml_type, w->in_dim, w->out_dim) != 0 &&
-                       (uint64_t)((n_tokens + 31u) & ~31u) * w->in_dim < (1ull << 32);
+  // A batch that may go to a matrix-core GEMM of the K-quants has its activations laid out in that kernel's
+  // operand chunks by the quantizer itself (from 25 tokens: below, the small-batch kernel's loads gather few enough
+  // distinct rows that the plain quantizer's shorter launch decides: 4096 -> 4096 at 24 tokens 11.5 us from rows,
+  // 12.2 from chunks; at 32 tokens 14.3 against 12.5); which kernel runs is decided per launch.
+  const bool with_xt = !dump_isum && !dump_imin && act_chunks_wanted(ctx, w->ggml_type, w->in_dim, n_tokens, decode, 25u);
   int rc = enqueue_quantize(ctx, act_mode_for(w->ggml_type, n_tokens, decode), x_dev, w->in_dim, n_tokens, stream, with_xt);
   if (rc != OGM_OK) return rc;
   return enqueue_gemv(ctx, tg, n_tg, n_tokens, decode, stream, dump_isum, dump_imin);
@@ -970,7 +989,8 @@ static int act_quantize_dev(ogm_ctx *ctx, uint32_t ggml_type, const float *x_dev
   std::lock_guard<std::mutex> lock(ctx->mu);
   HIPCHK(ctx, hipSetDevice(ctx->device));
   hipStream_t s = stream ? (hipStream_t)stream : ctx->stream;
-  return enqueue_quantize(ctx, act_mode_for(ggml_type, n_tokens, decode), x_dev, in_dim, n_tokens, s);
+  return enqueue_quantize(ctx, act_mode_for(ggml_type, n_tokens, decode), x_dev, in_dim, n_tokens, s,
+                          act_chunks_wanted(ctx, ggml_type, in_dim, n_tokens, decode, 25u));
 }
 
 // The activation mode of Backend::matmul (for Q2_K at several tokens: per 32, cpu.rs:113-163) ...
@@ -1875,14 +1895,12 @@ static int llama_matmul_quantized_rows(ogm_ctx *ctx, const ogm_weight *const *ws
 }
 
 // Where a producer kernel of a batch (norm, SwiGLU) should also lay its int8 rows out in the operand chunks of the
-// tiled GEMMs over planes, or null: the same condition as enqueue_matmul's for its quantizer.  Saves the GEMM's own
-// relayout launch (5 us a matmul at 512 tokens of the 8B shapes).
+// matrix-core GEMMs, or null.  Saves the tiled GEMM's own relayout launch (5 us a matmul at 512 tokens of the 8B
+// shapes) and the small-batch kernel its gather of up to 32 rows a load; from 17 tokens, since a producer writes
+// them at no launch of its own.
 static int llama_producer_xt(ogm_ctx *ctx, const ogm_weight *w, int mode, uint32_t in_dim, uint32_t T, int8_t **xt) {
   *xt = nullptr;
-  if (mode != OGM_ACT_PER_256 || T < 32 || in_dim % 256u != 0 || ctx->tune_plane_cache_mb <= 0 ||
-      ogm_gemm_plane_bytes(w->ggml_type, w->in_dim, w->out_dim) == 0 ||
-      (uint64_t)((T + 31u) & ~31u) * in_dim >= (1ull << 32))
-    return OGM_OK;
+  if (mode != OGM_ACT_PER_256 || !act_chunks_wanted(ctx, w->ggml_type, in_dim, T, 0, 17u)) return OGM_OK;
   const int rc = ensure_dev(ctx, ctx->xh, ogm_gemm_xh_bytes(in_dim, T));
   if (rc == OGM_OK) *xt = (int8_t *)ctx->xh.p;
   return rc;

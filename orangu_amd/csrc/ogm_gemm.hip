@@ -1508,6 +1508,7 @@ struct GemmSbParams {
   uint32_t in_dim, out_dim, n_tokens, nsb;
   uint32_t c_shift, r_shift, nct;
   uint32_t n_extra;
+  uint32_t x_chunks;      // xq holds the activations in operand chunks (ogm_xt_row) instead of rows
   const uint8_t *extra_wt[OGM_GEMM_MAX_MATS - 1];
   float *extra_y[OGM_GEMM_MAX_MATS - 1];
   uint32_t extra_out_dim[OGM_GEMM_MAX_MATS - 1];
@@ -1551,7 +1552,11 @@ __device__ __forceinline__ void gemm_sb_q6k_body(GemmSbParams p) {
   auto sb_tail = [&](uint32_t s) -> uint32_t {
     return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 2u;
   };
-  const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + 256 s + 32 sub
+  // a lane's 16 activations of a run of 32: from its token's row, or (x_chunks) from the 1 KiB operand chunk of
+  // the tile's 32 tokens and the run's 32 k, where they lie in the instruction's own order
+  const uint32_t xmul = p.x_chunks ? 32u : 1u;
+  const uint32_t xro = p.x_chunks ? blockIdx.x * p.in_dim * 32u + 16u * lane
+                                  : min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + (256 s + 32 sub) xmul
   const uint32_t sc_shift = 8u * lh;
 
   // the tokens' ad of every super-block: ad_l[s][token]
@@ -1604,7 +1609,7 @@ __device__ __forceinline__ void gemm_sb_q6k_body(GemmSbParams p) {
   do {                                                                                            \
     int4v bh_, bl_;                                                                               \
     SB_UNPACK(bh_, bl_, QL, QH, SCW, G, SUB);                                                     \
-    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 64u * (G) + 32u * (SUB)));                   \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + (64u * (G) + 32u * (SUB)) * xmul));          \
     H = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bh_, (FIRST) ? zi : H, 0, 0, 0);               \
     L = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bl_, (FIRST) ? zi : L, 0, 0, 0);               \
   } while (0)
@@ -1618,7 +1623,7 @@ __device__ __forceinline__ void gemm_sb_q6k_body(GemmSbParams p) {
   for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
     const uint32_t s = s0 + wave;
     if (s < p.nsb) {   // wave-uniform
-      const uint32_t xs_ = xro + 256u * s;
+      const uint32_t xs_ = xro + 256u * s * xmul;
       int16v H, L;
       SB_STEP(wA0, wQ0, scw.x, 0, 0, true);
       SB_STEP(wB0, wQ0, scw.x, 0, 1, false);
@@ -1705,7 +1710,11 @@ __device__ __forceinline__ void gemm_sb_q3k_body(GemmSbParams p) {
   auto sb_off = [&](uint32_t s) -> uint32_t {
     return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
   };
-  const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + 256 s + 32 step
+  // a lane's 16 activations of a run of 32: from its token's row, or (x_chunks) from the 1 KiB operand chunk of
+  // the tile's 32 tokens and the run's 32 k, where they lie in the instruction's own order
+  const uint32_t xmul = p.x_chunks ? 32u : 1u;
+  const uint32_t xro = p.x_chunks ? blockIdx.x * p.in_dim * 32u + 16u * lane
+                                  : min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + (256 s + 32 step) xmul
 
   for (uint32_t i = tid; i < 32u * p.nsb; i += NT) {
     const uint32_t k = i / p.nsb, s = i - k * p.nsb;
@@ -1749,7 +1758,7 @@ __device__ __forceinline__ void gemm_sb_q3k_body(GemmSbParams p) {
       pw_[w_] = __builtin_amdgcn_perm(f_.u, e_.u, 0x06040200u);   /* the lanes' low bytes */      \
     }                                                                                             \
     const int4v bw_ = {(int)pw_[0], (int)pw_[1], (int)pw_[2], (int)pw_[3]};                       \
-    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 64u * (G) + 32u * (SUB)));                   \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + (64u * (G) + 32u * (SUB)) * xmul));          \
     H = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bw_, (FIRST) ? zi : H, 0, 0, 0);               \
   } while (0)
 
@@ -1762,7 +1771,7 @@ __device__ __forceinline__ void gemm_sb_q3k_body(GemmSbParams p) {
   for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
     const uint32_t s = s0 + wave;
     if (s < p.nsb) {   // wave-uniform
-      const uint32_t xs_ = xro + 256u * s;
+      const uint32_t xs_ = xro + 256u * s * xmul;
       int16v H;
       SB3_STEP(0u, 0u, true);
       SB3_STEP(0u, 1u, false);
@@ -1847,7 +1856,11 @@ __device__ __forceinline__ void gemm_sb_iq4xs_body(GemmSbParams p) {
   auto sb_off = [&](uint32_t s) -> uint32_t {
     return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
   };
-  const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + 256 s + 32 ib
+  // a lane's 16 activations of a run of 32: from its token's row, or (x_chunks) from the 1 KiB operand chunk of
+  // the tile's 32 tokens and the run's 32 k, where they lie in the instruction's own order
+  const uint32_t xmul = p.x_chunks ? 32u : 1u;
+  const uint32_t xro = p.x_chunks ? blockIdx.x * p.in_dim * 32u + 16u * lane
+                                  : min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + (256 s + 32 ib) xmul
   const uint32_t nsh = 4u * lh;
 
   for (uint32_t i = tid; i < 32u * p.nsb; i += NT) {
@@ -1881,7 +1894,7 @@ __device__ __forceinline__ void gemm_sb_iq4xs_body(GemmSbParams p) {
     }                                                                                             \
     const int4v bh_ = {(int)ph_[0], (int)ph_[1], (int)ph_[2], (int)ph_[3]};                       \
     const int4v bl_ = {(int)pl_[0], (int)pl_[1], (int)pl_[2], (int)pl_[3]};                       \
-    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 32u * (IB)));                                \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 32u * (IB) * xmul));                         \
     H = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bh_, (FIRST) ? zi : H, 0, 0, 0);               \
     L = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, bl_, (FIRST) ? zi : L, 0, 0, 0);               \
   } while (0)
@@ -1895,7 +1908,7 @@ __device__ __forceinline__ void gemm_sb_iq4xs_body(GemmSbParams p) {
   for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
     const uint32_t s = s0 + wave;
     if (s < p.nsb) {   // wave-uniform
-      const uint32_t xs_ = xro + 256u * s;
+      const uint32_t xs_ = xro + 256u * s * xmul;
       const uint32_t sh_ = pc[0].x >> 16, sl_ = pc[0].y;
       int16v H, L;
       SBX_STEP(0, true);
@@ -2076,8 +2089,8 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
   constexpr uint32_t TILE_BYTES = Q5 ? 11264u : 9216u;
   constexpr uint32_t QS_PIECE0 = Q5 ? 3u : 1u;
   extern __shared__ __align__(16) uint8_t sb_lds[];
-  float *terms = (float *)sb_lds;             // [16 super-blocks][32 tokens][32 rows] (second sweep: NW)
-  float *ad_l = terms + 16u * 32u * 32u;      // [nsb][32 tokens]
+  float *terms = (float *)sb_lds;             // [NW super-blocks][32 tokens][32 rows]
+  float *ad_l = terms + NW * 32u * 32u;       // [nsb][32 tokens]
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t l32 = lane & 31u, lh = lane >> 5;
@@ -2105,9 +2118,25 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
     return (s >> p.c_shift) * TILE_BYTES + ((s & ((1u << p.c_shift) - 1u)) << p.r_shift) * 16u;
   };
   const uint32_t tok = min(t0 + l32, p.n_tokens - 1u);
-  const uint32_t xro = tok * p.in_dim + 16u * lh;   // + 256 s + 32 j
+  // a lane's 16 activations of a sub-block: from its token's row, or (x_chunks) from the 1 KiB operand chunk of
+  // the tile's 32 tokens and the sub-block's 32 k, where they lie in the instruction's own order
+  const uint32_t xmul = p.x_chunks ? 32u : 1u;
+  const uint32_t xro = p.x_chunks ? blockIdx.x * p.in_dim * 32u + 16u * lane : tok * p.in_dim + 16u * lh;   // + (256 s + 32 j) xmul
   const uint32_t tk = tok * p.nsb;
 
+  uint4 hdr, w0, w1, w2, w3, qh5 = make_uint4(0, 0, 0, 0);
+#define SB_LOADW(S)                                                                               \
+  do {                                                                                            \
+    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded, never used */    \
+    const uint32_t so_ = uo + sb_off(s_);                                                         \
+    hdr = *(const uint4 *)(p.wt + so_);                                                           \
+    w0 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 0u + lh) * 1024u));                          \
+    w1 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 2u + lh) * 1024u));                          \
+    w2 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 4u + lh) * 1024u));                          \
+    w3 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 6u + lh) * 1024u));                          \
+    if constexpr (Q5) qh5 = *(const uint4 *)(p.wt + (so_ + (1u + lh) * 1024u));                   \
+  } while (0)
+  SB_LOADW(wave);   // the second sweep's first weights: under way during the first sweep
   for (uint32_t i = tid; i < 32u * p.nsb; i += NT) {
     const uint32_t k = i / p.nsb, s = i - k * p.nsb;
     ad_l[s * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * p.nsb + s];
@@ -2123,10 +2152,9 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
 #pragma unroll
     for (int r = 0; r < 16; r++) zero[r] = 0.0f;
     const float side_scale = lh ? 1.0f : 64.0f;
-    for (uint32_t s0 = 0; s0 < p.nsb; s0 += 16u) {
-#pragma unroll
-      for (uint32_t u = 0; u < 16u / NW; u++) {
-        const uint32_t sl = wave + NW * u, s = s0 + sl;
+    for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
+      {
+        const uint32_t sl = wave, s = s0 + sl;
         if (s < p.nsb) {   // wave-uniform
           const uint4 hd = *(const uint4 *)(p.wt + (uo + sb_off(s)));
           const half8 b2 = *(const half8 *)(p.bs16 + ((tk + s) * 16u + 8u * lh));
@@ -2147,7 +2175,7 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
         }
       }
       __syncthreads();
-      const uint32_t n_here = min(16u, p.nsb - s0);
+      const uint32_t n_here = min(NW, p.nsb - s0);
       for (uint32_t w = 0; w < n_here; w++) {
 #pragma unroll
         for (uint32_t a = 0; a < NACC; a++) acc[a] -= terms[w * 1024u + a * NT + tid];
@@ -2156,18 +2184,6 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
     }
   }
   // ---- second sweep: acc += ad * (d * sum_j sc_j * dot32_j)
-  uint4 hdr, w0, w1, w2, w3, qh5 = make_uint4(0, 0, 0, 0);
-#define SB_LOADW(S)                                                                               \
-  do {                                                                                            \
-    const uint32_t s_ = min((uint32_t)(S), p.nsb - 1u); /* past the end: loaded, never used */    \
-    const uint32_t so_ = uo + sb_off(s_);                                                         \
-    hdr = *(const uint4 *)(p.wt + so_);                                                           \
-    w0 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 0u + lh) * 1024u));                          \
-    w1 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 2u + lh) * 1024u));                          \
-    w2 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 4u + lh) * 1024u));                          \
-    w3 = *(const uint4 *)(p.wt + (so_ + (QS_PIECE0 + 6u + lh) * 1024u));                          \
-    if constexpr (Q5) qh5 = *(const uint4 *)(p.wt + (so_ + (1u + lh) * 1024u));                   \
-  } while (0)
   // One matrix instruction per sub-block on the bare quants (K = 32 is exactly a sub-block; a lane's
   // operand is its row's 16 nibbles, with Q5_K's fifth bit on top), then isum += sc_j * dot_j as
   // 24-bit integer multiply-adds (|dot_j| <= 31 * 127 * 32 < 2^17, sc_j < 64): the same integer.
@@ -2180,7 +2196,7 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
       if constexpr (Q5) v_[w_] |= ((q5w_[w_] >> (J)) & 0x01010101u) << 4;                         \
     }                                                                                             \
     const int4v b_ = {(int)v_[0], (int)v_[1], (int)v_[2], (int)v_[3]};                            \
-    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 32u * (J)));                                 \
+    const int4v xa_ = *(const int4v *)(p.xq + (xs_ + 32u * (J) * xmul));                          \
     D = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa_, b_, zi, 0, 0, 0);                              \
   } while (0)
 #define SB_ACC(D, J, FIRST)                                                                       \
@@ -2190,11 +2206,10 @@ __device__ __forceinline__ void gemm_sb_q45k_body(GemmSbParams p) {
       I[r_] = (FIRST) ? __mul24(sc_, D[r_]) : __mul24(sc_, D[r_]) + I[r_];                        \
   } while (0)
   const int16v zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  SB_LOADW(wave);
   for (uint32_t s0 = 0; s0 < p.nsb; s0 += NW) {
     const uint32_t s = s0 + wave;
     if (s < p.nsb) {   // wave-uniform
-      const uint32_t xs_ = xro + 256u * s;
+      const uint32_t xs_ = xro + 256u * s * xmul;
       uint32_t sca_, scb_;
       q4k_scales(hdr, sca_, scb_);
       int16v I, Da, Db;   // the products of a sub-block are under way while the one before is added
@@ -2994,8 +3009,12 @@ static bool gemm_interleaved(const OgmGemmArgs &a, bool for_small_batch = false)
   // (beyond its small batches IQ4_XS has the two plane kernels only: 4096 -> 4096 at 32 tokens 28 us against 46 on the
   // 128-row tiles, 14336 -> 4096 77 against 141, 4096 -> 14336 33 against 50)
   if (xs && !for_small_batch) return true;
-  if (!q45) return (n_wg >= 128u && (tok_tiles >= 2u || a.n_tokens > 96u)) || (n_wg >= 96u && a.n_tokens >= 192u);
-  return tok_tiles >= 3u && n_wg >= 160u && (nsb <= 20u || n_wg <= 256u);
+  if (!q45) {
+    const uint32_t last = a.n_tokens - (tok_tiles - 1u) * 128u;   // tokens of the last token tile
+    return (n_wg >= 160u && (tok_tiles >= 2u || a.n_tokens > 96u)) || (n_wg >= 128u && last > 96u) ||
+           (n_wg >= 128u && tok_tiles >= 3u);
+  }
+  return (tok_tiles >= 3u || (tok_tiles == 2u && nsb > 32u)) && n_wg >= 160u && (nsb <= 20u || n_wg <= 256u);
 }
 
 // Whether a tiled launch goes to a kernel whose waves all multiply, given planes.  The one with 128 x 128
@@ -3039,14 +3058,15 @@ static bool gemm_small_batch(const OgmGemmArgs &a, bool planes_possible) {
   // (where the medium-batch kernel runs it takes over earlier: see gemm_medium_batch; 4096 rows at 160 / 192 / 224
   // tokens 34 / 35 / 37 against its 33 / 33 / 33.  Up to 2048 rows the small batches stay ahead for longer: 2048 ->
   // 2048 at 256 / 384 / 512 tokens 15 / 20 / 23 against 20 / 21 / 22 medium and 24 / 26 / 26 tiled)
-  const bool med = q45 && a.medium != 1u;
+  const bool long_rows = q45 && nsb > 32u;   // no medium-batch kernel there, and a first pass in the plane kernels
   const uint32_t small_max = a.small_max_tokens ? a.small_max_tokens
-                             : (tiles64_all <= 32u   ? (q45 ? 512u : 256u)
-                                : tiles64_all <= 64u ? (med ? 160u : 256u)
-                                : tiles64_all <= 128u ? (med ? 96u : 128u)
+                             : (tiles64_all <= 32u   ? (q45 ? 512u : 384u)
+                                : tiles64_all <= 64u ? 256u
+                                : tiles64_all <= 96u ? (long_rows ? 256u : 128u)
+                                : tiles64_all <= 128u ? 128u
                                                       : 64u);
   return a.small_max_tokens != 1u && a.n_tokens <= small_max &&
-         (q45 ? 16u : 8u) * 4096u + 128u * nsb <= GM_LDS_MAX;
+         8u * 4096u + 128u * nsb <= GM_LDS_MAX;
 }
 
 // Whether a Q4_K / Q5_K launch beyond the small batches takes the medium-batch kernel (32 rows x 128 tokens per
@@ -3203,7 +3223,8 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   if (gemm_small_batch(a, have_planes)) {
     GemmSbParams p;
     p.wt = a.wt;
-    p.xq = a.act.q;
+    p.x_chunks = (a.xt_ready && a.xh) ? 1u : 0u;   // the operand chunks where a producer wrote them
+    p.xq = p.x_chunks ? (const int8_t *)a.xh : a.act.q;
     p.ad = a.act.d;
     p.bs16 = bs16;
     p.y = a.y;
@@ -3226,7 +3247,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     const uint32_t n_wg = ((a.n_tokens + 31u) / 32u) * tiles;
     const bool w16 = (a.sb_waves ? a.sb_waves == 16u : (n_wg <= 256u && nsb >= 16u)) &&
                      16u * 4096u + 128u * nsb <= GM_LDS_MAX;
-    const uint32_t lds_bytes = ((q45 || w16) ? 16u : 8u) * 4096u + 128u * nsb;
+    const uint32_t lds_bytes = (w16 ? 16u : 8u) * 4096u + 128u * nsb;
     const void *fn = a.ggml_type == OGM_Q6_K   ? (w16 ? (const void *)ogm_gemm_sb_q6k_w16_kernel : (const void *)ogm_gemm_sb_q6k_kernel)
                      : a.ggml_type == OGM_Q3_K ? (w16 ? (const void *)ogm_gemm_sb_q3k_w16_kernel : (const void *)ogm_gemm_sb_q3k_kernel)
                      : a.ggml_type == OGM_IQ4_XS ? (w16 ? (const void *)ogm_gemm_sb_iq4xs_w16_kernel : (const void *)ogm_gemm_sb_iq4xs_kernel)

@@ -5,8 +5,8 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (BLOCK, IQ4_XS, Q2_K, Q5_1, activations_t, pin_scales, pseudo_bytes_fast, row_bytes, synth_weights,
-                     synth_x)
+from helpers import (BLOCK, IQ4_XS, Q2_K, Q3_K, Q4_K, Q5_1, Q5_K, Q6_K, activations_t, pin_scales, pseudo_bytes_fast,
+                     row_bytes, synth_weights, synth_x)
 
 pytestmark = pytest.mark.gpu
 NEW = [Q5_1, Q2_K, IQ4_XS]
@@ -360,3 +360,24 @@ def test_q2_k_extreme_sums_on_the_matrix_cores(be):
     got = be.matmul(x, T, qm(raw, Q2_K, in_dim, out_dim))
     assert be.last_kernel() == "ogm_gemm_sb_q2k_kernel"
     assert_bits(got, oracle.matmul(Q2_K, raw, in_dim, out_dim, x, T), "Q2_K extreme sums")
+
+
+@pytest.mark.parametrize("chunks", [1, 2])
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K, Q3_K, IQ4_XS])
+@pytest.mark.parametrize("in_dim,out_dim,T", [(256, 5, 9), (1024, 100, 33), (4096, 70, 40), (768, 200, 70), (2304, 33, 128)])
+def test_small_batch_kernels_read_rows_or_operand_chunks(be, t, in_dim, out_dim, T, chunks):
+    """The K-quants' small-batch kernels take their int8 activations from the token rows or, where the quantizer
+    also wrote them, from the 1 KiB operand chunks of 32 tokens x 32 inputs (tokens past the batch's last in a chunk
+    are never stored): the same bits either way, on full and ragged token and row tiles (gemm_k_q4_k, gemm_k_q6_k,
+    gemm_k_iq4_xs, vecdot.rs:2213-2398)."""
+    raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T + t)
+    x = synth_x(T, in_dim, seed=T + 3)
+    be.set_tuning("gemm_small_max_tokens", 1024)
+    be.set_tuning("gemm_act_chunks", chunks)
+    try:
+        got = be.matmul(x, T, qm(raw, t, in_dim, out_dim))
+        assert "ogm_gemm_sb_" in be.last_kernel(), be.last_kernel()
+    finally:
+        be.set_tuning("gemm_small_max_tokens", 0)
+        be.set_tuning("gemm_act_chunks", 0)
+    assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), f"type {t}, {T} tokens, act_chunks {chunks}")

@@ -601,13 +601,14 @@ def test_gemm_threshold_default():
     float order, 9 through the per-32 types' small-batch GEMM (rows so long that the GEMV kernel would read the
     weights once per part of the batch: from the first token it cannot hold), a launch of many workgroups through
     their tiled GEMM.  Q4_K: 4 tokens through the GEMV kernel, 5 to 8 through the
-    row-block kernel, then the small-batch kernel: to 512 tokens over a matrix of up to 2048 rows, to 160 over one
-    of up to 4096, where the medium-batch kernel has the rest of the second token tile and a tiled kernel what
-    follows; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
+    row-block kernel, then the small-batch kernel: to 512 tokens over a matrix of up to 2048 rows, to 256 over one
+    of up to 4096, to 128 over one of up to 8192, where the medium-batch kernel has the second token tile and a tiled
+    kernel what follows; a matrix of many rows leaves the small-batch kernel after 64 tokens, and one of so
     many that 128 x 128 tiles outnumber the compute units has its planes built and read by the kernel whose
     waves all multiply, while a single nearly full token tile over at most 16384 rows goes to the medium-batch kernel.
-    Q6_K goes to the 64-row plane kernel wherever that has 128 workgroups and a token tile more than three quarters
-    full, or 96 workgroups and 192 tokens, before the small-batch kernel is asked.
+    Q6_K goes to the 64-row plane kernel wherever that has 128 workgroups and a last token tile more than three
+    quarters full, or three token tiles, or 160 workgroups and more than 96 tokens, before the small-batch kernel is
+    asked.
     Same bits everywhere."""
     from orangu_amd import Mi355xBackend
     b = Mi355xBackend()
@@ -647,16 +648,26 @@ def test_gemm_threshold_default():
             y = b.matmul(x[:n], n, w)
             assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, want[:n], f"Q4_K, {n} tokens")
-        # (up to 64 tiles, up to 160 tokens; then the medium-batch kernel has the second token tile, full or not)
+        # (up to 64 tiles, up to 256 tokens; three token tiles over so few rows are too few workgroups for the planes)
         raw = synth_weights(Q4_K, 256, 2100, seed=25)
         w = qm(raw, Q4_K, 256, 2100)
         x2 = np.ascontiguousarray(x[:, :256])
         want = oracle.matmul(Q4_K, raw, 256, 2100, x2, 257).reshape(257, 2100)
-        for n, kernel in ((160, "ogm_gemm_sb_q4k_kernel"), (161, "ogm_gemm_sbw_q4k_kernel"),
-                          (256, "ogm_gemm_sbw_q4k_kernel"), (257, "ogm_gemm_q4k_i8p_r64_kernel")):
+        for n, kernel in ((160, "ogm_gemm_sb_q4k_kernel"), (256, "ogm_gemm_sb_q4k_kernel"),
+                          (257, "ogm_gemm_q4k_i8p_r64_kernel")):
             y = b.matmul(x2[:n], n, w)
             assert kname(b).startswith(kernel), (n, kname(b))
             assert_bits(y, want[:n], f"Q4_K of 2100 rows, {n} tokens")
+        # (up to 128 tiles, up to 128 tokens; then the medium-batch kernel has the second token tile, full or not,
+        # and the 64-row plane kernel the third)
+        raw = synth_weights(Q4_K, 256, 4200, seed=26)
+        w = qm(raw, Q4_K, 256, 4200)
+        want = oracle.matmul(Q4_K, raw, 256, 4200, x2, 257).reshape(257, 4200)
+        for n, kernel in ((128, "ogm_gemm_sb_q4k_kernel"), (129, "ogm_gemm_sbw_q4k_kernel"),
+                          (256, "ogm_gemm_sbw_q4k_kernel"), (257, "ogm_gemm_q4k_dmx_kernel")):
+            y = b.matmul(x2[:n], n, w)
+            assert b.last_kernel() == kernel, (n, b.last_kernel())
+            assert_bits(y, want[:n], f"Q4_K of 4200 rows, {n} tokens")
         raw = synth_weights(Q4_K, 768, 70, seed=15)    # three super-blocks a row: tiles of 64 rows, one block wide
         w3 = qm(raw, Q4_K, 768, 70)
         x3 = np.ascontiguousarray(x[:9, :768])
@@ -677,11 +688,11 @@ def test_gemm_threshold_default():
             y = b.matmul(np.ascontiguousarray(x[:n, :256]), n, w)
             assert b.last_kernel() == kernel, (n, b.last_kernel())
             assert_bits(y, want[:n], f"Q6_K, {n} tokens")
-        raw6 = synth_weights(Q6_K, 512, 3100, seed=16)  # 49 tiles of 64 rows: small batches to 256 tokens, unless
-        w6 = qm(raw6, Q6_K, 512, 3100)                   # there are 192 tokens in at least 96 workgroups
+        raw6 = synth_weights(Q6_K, 512, 3100, seed=16)  # 49 tiles of 64 rows: small batches to 256 tokens; a third
+        w6 = qm(raw6, Q6_K, 512, 3100)                   # token tile makes 147 workgroups for the plane kernel
         x6 = np.ascontiguousarray(x[:257, :512])
         want = oracle.matmul(Q6_K, raw6, 512, 3100, x6, 257).reshape(257, 3100)
-        for n, kernel in ((128, "ogm_gemm_sb_q6k_kernel"), (191, "ogm_gemm_sb_q6k_kernel"), (192, "ogm_gemm_q6k_dmx_kernel"),
+        for n, kernel in ((128, "ogm_gemm_sb_q6k_kernel"), (192, "ogm_gemm_sb_q6k_kernel"), (256, "ogm_gemm_sb_q6k_kernel"),
                           (257, "ogm_gemm_q6k_dmx_kernel")):
             y = b.matmul(x6[:n], n, w6)
             assert b.last_kernel() == kernel, (n, b.last_kernel())
