@@ -381,3 +381,40 @@ def test_small_batch_kernels_read_rows_or_operand_chunks(be, t, in_dim, out_dim,
         be.set_tuning("gemm_small_max_tokens", 0)
         be.set_tuning("gemm_act_chunks", 0)
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), f"type {t}, {T} tokens, act_chunks {chunks}")
+
+
+@pytest.mark.parametrize("t", [Q4_K, Q6_K, IQ4_XS])
+@pytest.mark.parametrize("T", [12, 40, 130])
+def test_two_step_batches_share_one_quantization(be, t, T):
+    """ogm_act_quantize_dev once, then several weights over the same batch (one by one and in one grouped call), as
+    arch/mod.rs:1082-1096 does for q, k, v: the bits of Backend::matmul on each.  From 25 tokens the quantize step also
+    writes the operand chunks the matrix-core kernels read; the calls that follow must find them, whatever kernel each
+    matrix's size sends it to."""
+    from orangu_amd import hiprt
+    in_dim = 1024
+    outs = (70, 300, 33)
+    raws = [synth_weights(t, in_dim, o, seed=80 + o + T) for o in outs]
+    x = synth_x(T, in_dim, seed=90 + T)
+    hs = [be.upload_raw(r, t, in_dim, o) for r, o in zip(raws, outs)]
+    xd = hiprt.DeviceBuffer.from_numpy(x)
+    yds = [hiprt.DeviceBuffer(4 * T * o) for o in outs]
+    try:
+        want = [oracle.matmul(t, r, in_dim, o, x, T) for r, o in zip(raws, outs)]
+        be.act_quantize_dev(t, xd.ptr, in_dim, T)
+        for h, yd in zip(hs, yds):
+            yd.fill(0xFF)
+            be.matmul_act_dev(h, T, yd.ptr, False)
+        hiprt.device_synchronize()
+        for yd, w, o in zip(yds, want, outs):
+            assert_bits(yd.to_numpy(np.float32, T * o), w, f"two-step, one by one, {o} rows, {be.last_kernel()}")
+            yd.fill(0xFF)
+        be.matmul_multi_act_dev(hs, T, [yd.ptr for yd in yds], False)
+        hiprt.device_synchronize()
+        for yd, w, o in zip(yds, want, outs):
+            assert_bits(yd.to_numpy(np.float32, T * o), w, f"two-step, grouped, {o} rows, {be.last_kernel()}")
+    finally:
+        for h in hs:
+            be.free_weight(h)
+        xd.free()
+        for yd in yds:
+            yd.free()
