@@ -3052,12 +3052,16 @@ static bool gemm_small_batch(const OgmGemmArgs &a, bool planes_possible) {
     return false;
   uint32_t tiles64_all = (a.out_dim + 63u) / 64u;
   for (uint32_t m = 0; m < a.n_extra; m++) tiles64_all += (a.extra_out_dim[m] + 63u) / 64u;
-  // (measured, Q4_K from 4096 inputs, small-batch against tiled, us: 4096 rows at 192 / 256 / 384 tokens 36 against 45,
-  // 39 against 46, 57 against 49; 6144 rows at 128 / 192: 37 against 47, 47 against 47; 14336 rows at 64 / 96: 38 against 44,
-  // 51 against 46)
-  // (where the medium-batch kernel runs it takes over earlier: see gemm_medium_batch; 4096 rows at 160 / 192 / 224
-  // tokens 34 / 35 / 37 against its 33 / 33 / 33.  Up to 2048 rows the small batches stay ahead for longer: 2048 ->
-  // 2048 at 256 / 384 / 512 tokens 15 / 20 / 23 against 20 / 21 / 22 medium and 24 / 26 / 26 tiled)
+  // Measured on MI355X with the activations in operand chunks, whole calls, us, small-batch against the best other
+  // kernel.  Q4_K: 4096 -> 4096 (64 tiles of 64 rows) at 128 / 192 / 256 / 384 tokens 20 / 30 / 32 / 41 against 33 / 33 /
+  // 34 / 40; 4096 -> 6144 (96 tiles) at 128 / 192 / 256: 29 / 38 / 43 against 33 / 37 / 38; 8192 -> 8192 (128 tiles) at
+  // 128 / 192: 54 / 76 against 57 / 70; 4096 -> 14336 (224 tiles) at 64 / 96 / 128: 31 / 42 / 48 against 37 / 38 / 39;
+  // 2048 -> 2048 (32 tiles) at 256 / 512: 14 / 23 against 20 / 22.  Rows of more than 8192 inputs, where the plane
+  // kernels' first pass weighs most and no medium-batch kernel runs: 14336 -> 4096 (64 tiles) at 192 / 256 / 384: 81 /
+  // 90 / 117 against 95 / 95 / 121; 14336 -> 5120 (80 tiles) at 192 / 256 / 384: 87 / 118 / 149 against 116 / 122 / 123;
+  // 14336 -> 8192 (128 tiles) at 128 / 192 / 256: 89 / 127 / 168 against 94 / 126 / 131.  Q6_K: 8192 -> 2048 (32 tiles)
+  // at 256 / 384 / 512: 32 / 48 / 50 against 47 / 50 / 51; 4096 -> 2048 at 384 / 512: 25 / 31 against 29 / 29; the
+  // launches of more tiles leave earlier for the 64-row plane kernel (gemm_interleaved).
   const bool long_rows = q45 && nsb > 32u;   // no medium-batch kernel there, and a first pass in the plane kernels
   const uint32_t small_max = a.small_max_tokens ? a.small_max_tokens
                              : (tiles64_all <= 32u   ? (q45 ? 512u : 384u)
@@ -3080,10 +3084,10 @@ static bool gemm_medium_batch(const OgmGemmArgs &a) {
       (uint64_t)t_pad * a.in_dim >= (1ull << 32))
     return false;
   if (a.medium == 2u) return true;
-  // Measured on MI355X against the kernels it displaces, whole calls, us: 4096 -> 14336 at 128 tokens 42 against 50
-  // (feeding waves), at 192 / 256 tokens 78 / 77 against 65 / 65; 4096 -> 4096 at 256 tokens 35 against 39 (small
-  // batch), at 128 tokens 33 against 23; 4096 -> 6144 at 128 / 256 tokens 34 / 40 against 36 / 46; 14336 -> 4096 at
-  // 256 tokens 106 against 116.  It wants a lone token tile of 128 nearly full (below, the small batches), and at two
+  // Measured on MI355X against the kernels it displaces, whole calls, us: 4096 -> 14336 at 128 tokens 39 against 50
+  // (feeding waves) and 48 (small batch), at 192 / 256 tokens 78 / 77 against 65 / 65; 4096 -> 6144 at 192 / 256 tokens
+  // 38 / 39 against 43 / 46 (feeding waves) and 38 / 43 (small batch); 8192 -> 8192 at 192 / 256: 70 / 71 against 76 / 97
+  // (small batch).  (The small-batch kernel comes first and keeps what gemm_small_batch gives it.)  It wants a lone token tile of 128 nearly full (below, the small batches), and at two
   // of them, full or not, matrices of at most 8192 rows (4096 -> 6144 at 144 / 192 tokens 38 / 37 against 43 / 43 for
   // the feeding waves, 8192 -> 8192 68 / 69 against 80 / 82; beyond 8192 rows the 128-row tiles of the feeding-wave
   // kernels outnumber the compute units' halves).  Its
@@ -3214,10 +3218,8 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
   for (uint32_t m = 0; m < a.n_extra; m++) row_tiles += (a.extra_out_dim[m] + GM_BN - 1) / GM_BN;
   const OgmTiling tl = ogm_tiling_for(nsb, a.out_dim);
   const uint32_t c_shift = tl.C == 4 ? 2 : (tl.C == 2 ? 1 : 0);
-  // Small batches: the kernel whose waves take different super-blocks.  By default up to 64 tokens
-  // (Q4_K 4096 -> 14336: 18 / 35 / 50 us at 32 / 64 / 96 tokens against 42-45 us tiled), and up to 128
-  // when the tiled kernel's grid would leave half the CUs idle (4096 -> 4096: 12 / 15 / 21 us at 32 /
-  // 64 / 128 tokens against 38-41; 14336 -> 4096: 36 / 39 / 57 against 123-130).
+  // Small batches: the kernel whose waves take different super-blocks, up to 64 tokens and longer over matrices of
+  // few rows (gemm_small_batch).
   bool have_planes = a.planes != nullptr;
   for (uint32_t m = 0; m < a.n_extra; m++) have_planes = have_planes && a.extra_planes[m] != nullptr;   // every matrix of the launch, or none
   if (gemm_small_batch(a, have_planes)) {
