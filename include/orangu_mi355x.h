@@ -430,7 +430,8 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              kernels then load a chunk in one piece instead of gathering 32 rows, the plane
  *                              and medium-batch kernels need no relayout launch): 0 = default, from 25 tokens
  *                              (the forward pass's own producers from 17), 1 = never, 2 = from 9.  Same bits
- *   "gemm_sb_waves"            waves of a small-batch workgroup: 8 or 16; 0 = by the size of the launch
+ *   "gemm_sb_waves"            waves of a small-batch workgroup: 8 or 16; 0 = by the size of the launch (sixteen
+ *                              where it has at most 256 workgroups and the rows the blocks for two rounds of them)
  *   "gemm_medium"              the Q4_K / Q5_K kernel for one nearly full tile of 128 tokens, or two (32 rows x
  *                              128 tokens a workgroup, its waves on different super-blocks): 0 = by the size of
  *                              the launch, 1 = never, 2 = whenever the shape allows

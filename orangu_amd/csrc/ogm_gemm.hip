@@ -2876,6 +2876,9 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
 
 template <int KIND>
 __global__ __launch_bounds__(512) void ogm_gemm_sb_flat_kernel(GemmSbParams p) { gemm_sb_flat_body<KIND, 8u>(p); }
+// Sixteen waves: half as many rounds, for launches that leave compute units idle.
+template <int KIND>
+__global__ __launch_bounds__(1024) void ogm_gemm_sb_flat_w16_kernel(GemmSbParams p) { gemm_sb_flat_body<KIND, 16u>(p); }
 
 static const uint32_t GM_LDS_MAX = 160 * 1024;   // LDS of a CU
 
@@ -3152,17 +3155,22 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       q.c_shift = p.c_shift;
       q.r_shift = p.r_shift;
       q.nct = p.nct;
-      const void *fn = a.ggml_type == OGM_Q4_0   ? (const void *)ogm_gemm_sb_flat_kernel<0>
-                       : a.ggml_type == OGM_Q5_0 ? (const void *)ogm_gemm_sb_flat_kernel<1>
-                       : a.ggml_type == OGM_IQ4_NL ? (const void *)ogm_gemm_sb_flat_kernel<2>
-                       : q51                       ? (const void *)ogm_gemm_sb_flat_kernel<4>
-                                                   : (const void *)ogm_gemm_sb_flat_kernel<3>;
-      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sbf_lds);
+      // sixteen waves when the launch leaves compute units idle and the rows have the blocks for two rounds of them
+      const uint32_t n_wg = ((a.n_tokens + 31u) / 32u) * ((a.out_dim + 31u) / 32u);
+      const uint32_t lds16 = 16u * SBF_NB * 4096u + 128u * p.nblk;
+      const bool w16 = (a.sb_waves ? a.sb_waves == 16u : (n_wg <= 256u && p.nblk >= 64u)) && lds16 <= GM_LDS_MAX;
+      const uint32_t lds_here = w16 ? lds16 : sbf_lds;
+      const void *fn = a.ggml_type == OGM_Q4_0   ? (w16 ? (const void *)ogm_gemm_sb_flat_w16_kernel<0> : (const void *)ogm_gemm_sb_flat_kernel<0>)
+                       : a.ggml_type == OGM_Q5_0 ? (w16 ? (const void *)ogm_gemm_sb_flat_w16_kernel<1> : (const void *)ogm_gemm_sb_flat_kernel<1>)
+                       : a.ggml_type == OGM_IQ4_NL ? (w16 ? (const void *)ogm_gemm_sb_flat_w16_kernel<2> : (const void *)ogm_gemm_sb_flat_kernel<2>)
+                       : q51                       ? (w16 ? (const void *)ogm_gemm_sb_flat_w16_kernel<4> : (const void *)ogm_gemm_sb_flat_kernel<4>)
+                                                   : (w16 ? (const void *)ogm_gemm_sb_flat_w16_kernel<3> : (const void *)ogm_gemm_sb_flat_kernel<3>);
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_here);
       if (e != hipSuccess) return e;
       void *kargs[] = {(void *)&q};
-      e = hipLaunchKernel(fn, dim3((a.n_tokens + 31u) / 32u, (a.out_dim + 31u) / 32u), dim3(512), kargs, sbf_lds, stream);
+      e = hipLaunchKernel(fn, dim3((a.n_tokens + 31u) / 32u, (a.out_dim + 31u) / 32u), dim3(w16 ? 1024 : 512), kargs, lds_here, stream);
       if (e != hipSuccess) return e;
-      if (kernel_name) *kernel_name = "ogm_gemm_sb_flat_kernel";
+      if (kernel_name) *kernel_name = w16 ? "ogm_gemm_sb_flat_w16_kernel" : "ogm_gemm_sb_flat_kernel";
       return hipGetLastError();
     }
     if (q51) return hipErrorInvalidValue;

@@ -299,12 +299,12 @@ def test_iq4_xs_without_room_for_planes_stays_on_the_gemv_kernel(be):
 
 @pytest.mark.parametrize("in_dim,out_dim,T,kernel", [
     (64, 5, 9, "ogm_gemm_sb_flat_kernel"), (128, 130, 17, "ogm_gemm_sb_flat_kernel"), (896, 64, 40, "ogm_gemm_sb_flat_kernel"),
-    (4864, 100, 33, "ogm_gemm_sb_flat_kernel"), (2048, 129, 300, "ogm_gemm_sb_flat_kernel"),
+    (4864, 100, 33, "ogm_gemm_sb_flat_w16_kernel"), (2048, 129, 300, "ogm_gemm_sb_flat_w16_kernel"),
     (14336, 70, 45, "ogm_gemm_sb_flat_kernel"), (512, 31, 8, "ogm_gemv_kernel<FmtQ51,gemm>"),
     (96, 40, 20, "ogm_gemv_kernel<FmtQ51,gemm>")])
 def test_q5_1_batches_on_the_small_batch_kernel(be, in_dim, out_dim, T, kernel):
     """From nine tokens on (rows of a multiple of 64 inputs) Q5_1 takes the per-32 types' small-batch GEMM, whatever
-    the batch: a block's term is ad * (dw * dot32 + m * block_sum) (dot_q5_1, vecdot.rs:2886-2899), the block sums of
+    the batch (with sixteen waves where the launch has at most 256 workgroups, the rows 64 blocks and the LDS room): a block's term is ad * (dw * dot32 + m * block_sum) (dot_q5_1, vecdot.rs:2886-2899), the block sums of
     the activations from a second matrix instruction against ones; every bit of the CPU path's."""
     raw = synth_weights(Q5_1, in_dim, out_dim, seed=in_dim + out_dim + T)
     x = synth_x(T, in_dim, seed=T)

@@ -1265,25 +1265,30 @@ def test_mfma_gemm_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T):
     assert_bits(small, want, "multi-token gemv")
 
 
+@pytest.mark.parametrize("waves", [8, 16])
 @pytest.mark.parametrize("t", [Q8_0, Q5_0, Q4_0, IQ4_NL])
 @pytest.mark.parametrize("in_dim,out_dim,T", [(64, 5, 9), (128, 130, 17), (896, 64, 40), (4096, 257, 130), (4864, 100, 33),
                                               (1024, 128, 128), (2048, 129, 70), (14336, 70, 45), (512, 31, 2)])
-def test_small_batch_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T):
-    """The per-32 types' small-batch kernel (32 rows x 32 tokens a workgroup, its waves on different blocks, a block
-    one int8 matrix instruction, the blocks' terms added in ascending order after every round of sixteen): every bit
-    of dot_flat_pair (vecdot.rs:2598-2629), with rows, tokens and blocks that do not fill the last workgroup or the
-    last round."""
+def test_small_batch_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T, waves):
+    """The per-32 types' small-batch kernel (32 rows x 32 tokens a workgroup, its eight or sixteen waves on different
+    blocks, a block one int8 matrix instruction, the blocks' terms added in ascending order after every round of two
+    blocks a wave): every bit of dot_flat_pair (vecdot.rs:2598-2629), with rows, tokens and blocks that do not fill
+    the last workgroup or the last round.  (Sixteen waves' terms need twice the LDS: rows too long for that keep
+    eight.)"""
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T + t)
     x = synth_x(T, in_dim, seed=T + 1)
     w = qm(raw, t, in_dim, out_dim)
     be.set_tuning("gemm_small_max_tokens", 1024)
     be.set_tuning("gemm_min_tokens", 2)
+    be.set_tuning("gemm_sb_waves", waves)
     try:
         got = be.matmul(x, T, w)
-        assert kname(be) == "ogm_gemm_sb_flat_kernel"
+        w16 = waves == 16 and 16 * 2 * 4096 + 128 * (in_dim // 32) <= 160 * 1024
+        assert kname(be) == ("ogm_gemm_sb_flat_w16_kernel" if w16 else "ogm_gemm_sb_flat_kernel")
     finally:
         be.set_tuning("gemm_small_max_tokens", 1)
         be.set_tuning("gemm_min_tokens", GEMM_FROM)
+        be.set_tuning("gemm_sb_waves", 0)
     assert_bits(got, oracle.matmul(t, raw, in_dim, out_dim, x, T), "small-batch flat gemm")
 
 
