@@ -419,8 +419,7 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *                              GEMM's float order
  *   "gemm_small_max_tokens"    GEMMs of at most this many tokens take the small-batch kernel of their type, whose
  *                              waves work on different super-blocks (blocks, for the per-32 types: by default
- *                              while the launch has at most 1792 workgroups of 32 rows x 32 tokens, 1100 on
- *                              rows beyond 4096 inputs) of the same rows; 0 = default (K-quants: 64, more
+ *                              while the launch has at most 1792 workgroups of 32 rows x 32 tokens) of the same rows; 0 = default (K-quants: 64, more
  *                              for matrices of few rows: 128 up to 8192 rows, 256 up to 4096 -- and up to 6144
  *                              for Q4_K / Q5_K rows of more than 8192 inputs --, 384 up to 2048, 512 there for
  *                              Q4_K / Q5_K; Q6_K launches that "gemm_interleave" sends to its kernel by their size

@@ -2766,8 +2766,13 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
   constexpr int NIB = KIND == 4 ? 3 : KIND;   // ogm_nib32_weights' kind
   constexpr uint32_t TILE = 64u * (16u * PIECES + TAIL);
   extern __shared__ __align__(16) uint8_t sb_lds[];
-  float *terms = (float *)sb_lds;                  // [NW * SBF_NB blocks of the round][32 tokens][32 rows]
-  float *ad_l = terms + NW * SBF_NB * 1024u;       // [nblk][32 tokens]
+  // The tokens' ad of one round at a time, in two buffers: every thread fetches one value (block, token) a round
+  // ahead and stores it behind the round's additions, so no pass over all of a row's blocks comes first and the
+  // LDS does not grow with the rows.
+  constexpr uint32_t RB = NW * SBF_NB;             // blocks of a round (NT = 32 RB threads)
+  constexpr uint32_t ADS = 36u;                    // floats between the blocks of a round's ad: 16-byte rows, spread over the banks
+  float *terms = (float *)sb_lds;                  // [RB blocks of the round][32 tokens][32 rows]
+  float *ad_l = terms + RB * 1024u;                // [2][RB blocks][ADS]
   const uint32_t nblk = p.nsb;                     // (blocks of 32 here)
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -2782,11 +2787,9 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
   }
   const uint32_t xro = min(t0 + l32, p.n_tokens - 1u) * p.in_dim + 16u * lh;   // + 32 b
 
-  // the tokens' ad of every block: ad_l[b][token]
-  for (uint32_t i = tid; i < 32u * nblk; i += NT) {
-    const uint32_t k = i / nblk, b = i - k * nblk;
-    ad_l[b * 32u + k] = p.ad[min(t0 + k, p.n_tokens - 1u) * nblk + b];
-  }
+  const uint32_t ad_k = tid / RB, ad_b = tid % RB;   // this thread's token and block of a round
+  const uint32_t ad_src = min(t0 + ad_k, p.n_tokens - 1u) * nblk;
+  ad_l[ad_b * ADS + ad_k] = p.ad[ad_src + min(ad_b, nblk - 1u)];
 
   uint4 wq[SBF_NB];
   uint32_t tl[SBF_NB], th[SBF_NB];
@@ -2810,8 +2813,10 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
   for (uint32_t a = 0; a < NACC; a++) acc[a] = 0.0f;
   SBF_LOADW(wave * SBF_NB);
   __syncthreads();   // ad_l
-  for (uint32_t s0 = 0; s0 < nblk; s0 += NW * SBF_NB) {
+  uint32_t ad_buf = 0;   // the buffer of this round
+  for (uint32_t s0 = 0; s0 < nblk; s0 += RB) {
     const uint32_t b0 = s0 + wave * SBF_NB;
+    const float ad_next = p.ad[ad_src + min(s0 + RB + ad_b, nblk - 1u)];   // (past the end: never used)
 #pragma unroll
     for (uint32_t j = 0; j < SBF_NB; j++) {
       const uint32_t b = b0 + j;
@@ -2836,7 +2841,7 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
           S = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa, ones, zi, 0, 0, 0);
         }
         const float d = gm_f16_bits_to_f32(tl[j] & 0xFFFFu), mn = KIND == 4 ? gm_f16_bits_to_f32(tl[j] >> 16) : 0.0f;
-        const float *adp = &ad_l[b * 32u + 4u * lh];
+        const float *adp = &ad_l[ad_buf * (RB * ADS) + (b - s0) * ADS + 4u * lh];
         float *tp = terms + ((wave * SBF_NB + j) * 32u + 4u * lh) * 32u + l32;   // [block of the round][token][row]
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
@@ -2852,15 +2857,17 @@ __device__ __forceinline__ void gemm_sb_flat_body(GemmSbParams p) {
         }
       }
     }
-    SBF_LOADW(b0 + NW * SBF_NB);   // the next round's weights, in flight over the barrier and the additions
+    SBF_LOADW(b0 + RB);   // the next round's weights, in flight over the barrier and the additions
     __syncthreads();
     {
-      const uint32_t n_here = min(NW * SBF_NB, nblk - s0);
+      const uint32_t n_here = min(RB, nblk - s0);
       for (uint32_t w = 0; w < n_here; w++) {   // ascending blocks, one accumulator per output
 #pragma unroll
         for (uint32_t a = 0; a < NACC; a++) acc[a] += terms[w * 1024u + a * NT + tid];
       }
     }
+    ad_buf ^= 1u;   // the next round's ad into the buffer the round before this one read
+    ad_l[ad_buf * (RB * ADS) + ad_b * ADS + ad_k] = ad_next;
     __syncthreads();
   }
 #undef SBF_LOADW
@@ -2887,22 +2894,23 @@ size_t ogm_gemm_xh_bytes(uint32_t in_dim, uint32_t n_tokens) {
   return (size_t)in_dim * ((n_tokens + 31u) & ~31u);
 }
 
+// LDS of the per-32 types' small-batch kernel with NW waves: a round's terms and two rounds' ad.
+static uint32_t gemm_flat_small_lds(uint32_t nw) { return nw * SBF_NB * 4096u + 2u * nw * SBF_NB * 36u * 4u; }
+
 // Whether a launch of the per-32 types takes their small-batch kernel: while its workgroups of 32 rows x 32 tokens
-// are few enough -- about seven rounds of the device's compute units where two of them fit one (rows of up to
-// 4096 inputs: 80 KB of LDS), about four where one does.  Measured on MI355X, Q8_0, whole calls, us, small-batch
-// against tiled: 4096 -> 4096 at 32 / 128 / 384 / 512 tokens 19 / 28 / 70 / 91 against 72 / 76 / 82 / 84; 4096 ->
-// 14336 at 32 / 96 / 128 / 192: 27 / 68 / 81 / 125 against 77 / 80 / 82 / 89; 14336 -> 4096 at 32 / 128 / 256 / 384:
-// 56 / 115 / 225 / 322 against 239 / 243 / 252 / 259; 8192 -> 8192 at 32 / 128 / 192: 37 / 131 / 193 against 142 /
-// 147 / 155; 4096 -> 32064 at 32 / 64: 57 / 101 against 86 / 88.  (Q4_0, Q5_0, IQ4_NL within a few per cent.)
-static bool gemm_flat_small(uint32_t n_tokens, uint32_t out_dim, uint32_t lds_bytes) {
+// are few enough, about seven rounds of the device's compute units (two workgroups share one).  Measured on MI355X,
+// Q8_0, whole calls, us, small-batch against tiled: 4096 -> 4096 at 32 / 128 / 384 / 512 tokens 14.5 / 24.5 / 62 / 91
+// against 72 / 76 / 82 / 84; 4096 -> 14336 at 32 / 128 / 192: 26 / 73 / 125 against 77 / 82 / 89; 14336 -> 4096 at 32 /
+// 128 / 256: 42 / 73 / 134 against 239 / 243 / 252; 8192 -> 2048 at 128 / 384: 28 / 67.  (Q4_0, Q5_0, IQ4_NL within a
+// few per cent.)
+static bool gemm_flat_small(uint32_t n_tokens, uint32_t out_dim) {
   const uint32_t wgs = ((n_tokens + 31u) / 32u) * ((out_dim + 31u) / 32u);
-  return wgs <= (lds_bytes <= 80u * 1024u ? 1792u : 1100u);
+  return wgs <= 1792u;
 }
 
 bool ogm_gemm_flat_small_batch(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, uint32_t n_tokens) {
-  const uint32_t lds = 8u * SBF_NB * 4096u + 128u * (in_dim / 32u);
-  if (in_dim % 64u != 0 || lds > GM_LDS_MAX) return false;
-  return ggml_type == OGM_Q5_1 || gemm_flat_small(n_tokens, out_dim, lds);   // (Q5_1 has no other GEMM kernel)
+  if (in_dim % 64u != 0) return false;
+  return ggml_type == OGM_Q5_1 || gemm_flat_small(n_tokens, out_dim);   // (Q5_1 has no other GEMM kernel)
 }
 
 // The per-32 types with a GEMM kernel: the four symmetric ones (small-batch and tiled), and Q5_1 (small-batch only).
@@ -2916,7 +2924,6 @@ bool ogm_gemm_supported(uint32_t ggml_type, uint32_t in_dim, uint32_t out_dim, u
   if (is_flat32(ggml_type)) {
     // two blocks per stage
     if (in_dim == 0 || in_dim % 64u != 0) return false;
-    if (ggml_type == OGM_Q5_1 && 8u * SBF_NB * 4096u + 128u * (in_dim / 32u) > GM_LDS_MAX) return false;
     OgmLayout l;
     ogm_layout_for(ggml_type, &l);
     return (uint64_t)ogm_tiling_for(in_dim / 32u, out_dim).nrb * 64u * (in_dim / 32u) * l.block_bytes <= lim &&
@@ -3139,9 +3146,9 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
     p.nct = tl.nct;
     // small batches: the kernel whose waves take different blocks (small_max_tokens as for the K-quants: 0 by the
     // size of the launch, 1 never, otherwise up to that many tokens)
-    const uint32_t sbf_lds = 8u * SBF_NB * 4096u + 128u * p.nblk;
+    const uint32_t sbf_lds = gemm_flat_small_lds(8u);
     const bool q51 = a.ggml_type == OGM_Q5_1;   // (this kernel only, whatever the batch)
-    const bool sbf = q51 || (a.small_max_tokens ? a.n_tokens <= a.small_max_tokens : gemm_flat_small(a.n_tokens, a.out_dim, sbf_lds));
+    const bool sbf = q51 || (a.small_max_tokens ? a.n_tokens <= a.small_max_tokens : gemm_flat_small(a.n_tokens, a.out_dim));
     if ((q51 || a.small_max_tokens != 1u) && sbf && sbf_lds <= GM_LDS_MAX) {
       GemmSbParams q{};
       q.wt = a.wt;
@@ -3157,7 +3164,7 @@ hipError_t ogm_launch_gemm(const OgmGemmArgs &a, hipStream_t stream, const char 
       q.nct = p.nct;
       // sixteen waves when the launch leaves compute units idle and the rows have the blocks for two rounds of them
       const uint32_t n_wg = ((a.n_tokens + 31u) / 32u) * ((a.out_dim + 31u) / 32u);
-      const uint32_t lds16 = 16u * SBF_NB * 4096u + 128u * p.nblk;
+      const uint32_t lds16 = gemm_flat_small_lds(16u);
       const bool w16 = (a.sb_waves ? a.sb_waves == 16u : (n_wg <= 256u && p.nblk >= 64u)) && lds16 <= GM_LDS_MAX;
       const uint32_t lds_here = w16 ? lds16 : sbf_lds;
       const void *fn = a.ggml_type == OGM_Q4_0   ? (w16 ? (const void *)ogm_gemm_sb_flat_w16_kernel<0> : (const void *)ogm_gemm_sb_flat_kernel<0>)

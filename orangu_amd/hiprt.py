@@ -81,7 +81,10 @@ class DeviceBuffer:
         return out
 
     def fill(self, byte: int):
+        """Sets every byte; complete on return (hipMemset runs on the null stream, which a library context's own
+        stream does not wait for)."""
         check(hip().hipMemset(self.ptr, byte, self.nbytes), "hipMemset")
+        device_synchronize()
 
     def free(self):
         if self.ptr:

@@ -184,6 +184,7 @@ def test_q2_k_two_step_calls_in_both_activation_modes(be):
     try:
         for decode, ref in ((True, oracle.matmul_decode), (False, oracle.matmul)):
             yd.fill(0xFF)
+            hiprt.device_synchronize()   # (the fill runs on another stream than the library's)
             be.act_quantize_dev(Q2_K, xd.ptr, in_dim, T, decode=decode)
             be.matmul_act_dev(h, T, yd.ptr, decode)
             hiprt.device_synchronize()
@@ -300,7 +301,7 @@ def test_iq4_xs_without_room_for_planes_stays_on_the_gemv_kernel(be):
 @pytest.mark.parametrize("in_dim,out_dim,T,kernel", [
     (64, 5, 9, "ogm_gemm_sb_flat_kernel"), (128, 130, 17, "ogm_gemm_sb_flat_kernel"), (896, 64, 40, "ogm_gemm_sb_flat_kernel"),
     (4864, 100, 33, "ogm_gemm_sb_flat_w16_kernel"), (2048, 129, 300, "ogm_gemm_sb_flat_w16_kernel"),
-    (14336, 70, 45, "ogm_gemm_sb_flat_kernel"), (512, 31, 8, "ogm_gemv_kernel<FmtQ51,gemm>"),
+    (14336, 70, 45, "ogm_gemm_sb_flat_w16_kernel"), (512, 31, 8, "ogm_gemv_kernel<FmtQ51,gemm>"),
     (96, 40, 20, "ogm_gemv_kernel<FmtQ51,gemm>")])
 def test_q5_1_batches_on_the_small_batch_kernel(be, in_dim, out_dim, T, kernel):
     """From nine tokens on (rows of a multiple of 64 inputs) Q5_1 takes the per-32 types' small-batch GEMM, whatever
@@ -400,14 +401,17 @@ def test_two_step_batches_share_one_quantization(be, t, T):
     yds = [hiprt.DeviceBuffer(4 * T * o) for o in outs]
     try:
         want = [oracle.matmul(t, r, in_dim, o, x, T) for r, o in zip(raws, outs)]
+        for yd in yds:
+            yd.fill(0xFF)
+        hiprt.device_synchronize()   # (the fills run on another stream than the library's)
         be.act_quantize_dev(t, xd.ptr, in_dim, T)
         for h, yd in zip(hs, yds):
-            yd.fill(0xFF)
             be.matmul_act_dev(h, T, yd.ptr, False)
         hiprt.device_synchronize()
         for yd, w, o in zip(yds, want, outs):
             assert_bits(yd.to_numpy(np.float32, T * o), w, f"two-step, one by one, {o} rows, {be.last_kernel()}")
             yd.fill(0xFF)
+        hiprt.device_synchronize()
         be.matmul_multi_act_dev(hs, T, [yd.ptr for yd in yds], False)
         hiprt.device_synchronize()
         for yd, w, o in zip(yds, want, outs):

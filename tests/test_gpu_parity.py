@@ -631,7 +631,7 @@ def test_gemm_threshold_default():
         y = b.matmul(xl[:2], 2, qm(rawl, Q8_0, 14336, 40))
         assert kname(b).startswith("ogm_gemv_kernel")
         y = b.matmul(xl, 5, qm(rawl, Q8_0, 14336, 40))
-        assert kname(b) == "ogm_gemm_sb_flat_kernel"
+        assert kname(b) == "ogm_gemm_sb_flat_w16_kernel"   # (few workgroups, rows of many blocks: sixteen waves)
         assert_bits(y, oracle.matmul(Q8_0, rawl, 14336, 40, xl, 5), "Q8_0 of 14336 inputs, 5 tokens")
         rawf = synth_weights(Q8_0, 256, 8300, seed=22)   # 260 row blocks of 32 x 10 token blocks: the tiled kernel
         xf = np.ascontiguousarray(x[:, :256])
@@ -1273,8 +1273,7 @@ def test_small_batch_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T, waves)
     """The per-32 types' small-batch kernel (32 rows x 32 tokens a workgroup, its eight or sixteen waves on different
     blocks, a block one int8 matrix instruction, the blocks' terms added in ascending order after every round of two
     blocks a wave): every bit of dot_flat_pair (vecdot.rs:2598-2629), with rows, tokens and blocks that do not fill
-    the last workgroup or the last round.  (Sixteen waves' terms need twice the LDS: rows too long for that keep
-    eight.)"""
+    the last workgroup or the last round.  (Sixteen waves keep one round's activation scales in LDS at a time.)"""
     raw = synth_weights(t, in_dim, out_dim, seed=in_dim + out_dim + T + t)
     x = synth_x(T, in_dim, seed=T + 1)
     w = qm(raw, t, in_dim, out_dim)
@@ -1283,7 +1282,7 @@ def test_small_batch_flat_types_match_cpu_gemm(be, t, in_dim, out_dim, T, waves)
     be.set_tuning("gemm_sb_waves", waves)
     try:
         got = be.matmul(x, T, w)
-        w16 = waves == 16 and 16 * 2 * 4096 + 128 * (in_dim // 32) <= 160 * 1024
+        w16 = waves == 16
         assert kname(be) == ("ogm_gemm_sb_flat_w16_kernel" if w16 else "ogm_gemm_sb_flat_kernel")
     finally:
         be.set_tuning("gemm_small_max_tokens", 1)
