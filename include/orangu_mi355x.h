@@ -414,7 +414,7 @@ int ogm_llama_load_gguf(ogm_ctx *ctx, ogm_gguf *g, uint32_t max_ctx, ogm_llama *
  *   "gemv_wg_waves"            waves per workgroup of the GEMV kernel, 1..16; 0 = by the row's tile count
  *   "gemm_min_tokens"          ogm_matmul takes a matrix-core GEMM from this many tokens on; 0 = default (6 for
  *                              Q4_K, Q5_K and Q6_K; 9 for Q8_0, Q5_0, Q4_0 and IQ4_NL where their small-batch
- *                              kernel would run, or as soon as the GEMV kernel would need three passes over
+ *                              kernel would run, or as soon as the GEMV kernel would need two passes over
  *                              the weights; 17 otherwise); below it the multi-token GEMV kernel runs in the
  *                              GEMM's float order
  *   "gemm_small_max_tokens"    GEMMs of at most this many tokens take the small-batch kernel of their type, whose

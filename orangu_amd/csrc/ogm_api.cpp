@@ -689,12 +689,12 @@ static int enqueue_gemv(ogm_ctx *ctx, const Target *tg, size_t n_tg, uint32_t n_
   // 65 against 52; Q8_0 4096 -> 4096 at 8 / 16 tokens 21 / 31 against 17 / 18, 14336 -> 4096 at 4 / 16 tokens 85 / 330
   // against 53 / 55 -- the per-32 types where their small-batch GEMM would run)
   const uint32_t gemv_chunk = ogm_gemv_max_tokens(w0->ggml_type, w0->in_dim, gemm_order);
-  // (the per-32 types from three parts on, or two of rows of up to 8192 inputs: 14336 -> 4096 at 2 tokens, two parts,
-  // 45 us against 53)
+  // (the per-32 types likewise, where their small-batch kernel would run: Q8_0 14336 -> 4096 at 2 tokens, two parts,
+  // 43 us against 40.5; 11008 -> 4096 at 3 / 4 tokens 37 / 39 against 32)
   const uint32_t gemv_parts = gemv_chunk ? (n_tokens + gemv_chunk - 1u) / gemv_chunk : 0u;
   const bool gemv_rereads = gemv_parts > 1u && ctx->tune_gemm_min_tokens == 0 &&
                             (block_elems_of(w0->ggml_type) == 256 ||
-                             (flat_small && (gemv_parts > 2u || w0->in_dim <= 8192u)));
+                             flat_small);
   if (gemm_order && !dump_isum && !dump_imin && !act_base && (n_tokens >= gemm_from || gemv_rereads) &&
       all_gemm_supported(tg, n_tg, n_tokens)) {
     // enough tokens to fill MFMA tiles: the tiled GEMM (same values, weights read once per 128 tokens)

@@ -626,10 +626,13 @@ def test_gemm_threshold_default():
         assert_bits(y17, want, "Q8_0, 17 tokens")
         assert_bits(y9, want[:9], "Q8_0, 9 tokens")
         assert_bits(y8, want[:8], "Q8_0, 8 tokens")
-        rawl = synth_weights(Q8_0, 14336, 40, seed=23)   # rows of which the GEMV kernel's LDS holds two tokens' worth
+        rawl = synth_weights(Q8_0, 14336, 40, seed=23)   # rows of which the GEMV kernel's LDS holds one token's worth
         xl = synth_x(5, 14336, seed=24)
-        y = b.matmul(xl[:2], 2, qm(rawl, Q8_0, 14336, 40))
+        y = b.matmul(xl[:1], 1, qm(rawl, Q8_0, 14336, 40))
         assert kname(b).startswith("ogm_gemv_kernel")
+        y = b.matmul(xl[:2], 2, qm(rawl, Q8_0, 14336, 40))
+        assert kname(b) == "ogm_gemm_sb_flat_w16_kernel"
+        assert_bits(y, oracle.matmul(Q8_0, rawl, 14336, 40, xl[:2], 2), "Q8_0 of 14336 inputs, 2 tokens")
         y = b.matmul(xl, 5, qm(rawl, Q8_0, 14336, 40))
         assert kname(b) == "ogm_gemm_sb_flat_w16_kernel"   # (few workgroups, rows of many blocks: sixteen waves)
         assert_bits(y, oracle.matmul(Q8_0, rawl, 14336, 40, xl, 5), "Q8_0 of 14336 inputs, 5 tokens")
